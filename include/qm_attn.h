@@ -1,0 +1,224 @@
+/*
+ * qm_attn.h — C ABI of the MI355X (gfx950) attention / KV-cache operators.
+ *
+ * Every entry point replaces one private launch wrapper of the reference engine
+ * (devices/rx7900xtx-24g/qwen3_tts_1_7b.cpp, "R17" below).  Conventions kept from
+ * the reference (R17:7968-8020, 17259-17262, 13857-13863):
+ *   - the caller owns all device memory; operators never allocate, free or retain;
+ *   - every operator is enqueued asynchronously on the caller's HIP stream and
+ *     performs no host/device synchronisation, so it can be stream-captured;
+ *   - bf16 tensors travel as uint16_t bit patterns.
+ * Differences: errors are returned as negative codes instead of C++ exceptions
+ * (nothing throws across this ABI; qm_attn.hpp re-throws std::runtime_error to
+ * match R17:7941-7949), and the KV cache is addressed through a page descriptor
+ * of which the reference's flat [kv_head][max_cache][128] buffer (R17:16371-16390)
+ * is the one-page special case.
+ *
+ * All pointers named `*_dev` / documented "device" must be device-accessible.
+ * `hip_stream` is a hipStream_t passed as void* (NULL = the null stream).
+ */
+#ifndef QM_ATTN_H
+#define QM_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- error codes (0 = success) ------------------------------------------- */
+#define QM_OK                 0
+#define QM_ERR_NULL          -1   /* a required pointer is NULL                      */
+#define QM_ERR_GEOMETRY      -2   /* head_dim != 128, q_heads not a supported multiple
+                                     of kv_heads, bad strides / page size           */
+#define QM_ERR_SLOT_RANGE    -3   /* cache position / context beyond page capacity
+                                     (the reference's "cache overflow", R17:16844)  */
+#define QM_ERR_WORKSPACE     -4   /* caller workspace missing or too small           */
+#define QM_ERR_ARGUMENT      -5   /* negative counts, unsupported option             */
+#define QM_ERR_NO_DEVICE     -6   /* no gfx950 device / kernel image unusable        */
+#define QM_ERR_HIP_BASE   -1000   /* -(1000 + hipError_t) for launch failures        */
+
+/* bits OR-ed by kernels into the optional device status word */
+#define QM_STATUS_BAD_PAGE      1u /* page table entry outside [0, n_pages)          */
+#define QM_STATUS_BAD_POSITION  2u /* position / length beyond max_pages*page_size   */
+
+/* ---- paged KV cache descriptor -------------------------------------------- */
+/*
+ * Token t of kv head h of a sequence lives at element offset
+ *     page_table[t / page_size] * stride_page + h * stride_head
+ *       + (t % page_size) * stride_token + d,        d in [0, head_dim)
+ * inside k_pool / v_pool.  The native layout is [page][kv_head][16][128]
+ * (stride_page = kv_heads*16*128, stride_head = 16*128, stride_token = 128), so one
+ * (page, head) block is 4 KiB contiguous.  The reference's LayerCache
+ * [kv_head][max_cache][128] (R17:15505-15522) is page_size = max_cache, n_pages = 1,
+ * stride_head = max_cache*128, page_table = NULL.
+ * Constraints: head_dim == 128, stride_token == 128, page_size % 16 == 0 unless the
+ * sequence has a single page; strides are multiples of 8 elements (16-byte loads).
+ */
+typedef struct qm_kv_cache {
+    uint16_t* k_pool;      /* device */
+    uint16_t* v_pool;      /* device */
+    int64_t   stride_page; /* elements */
+    int64_t   stride_head; /* elements */
+    int64_t   stride_token;/* elements, must be head_dim */
+    int32_t   page_size;   /* tokens per page */
+    int32_t   n_pages;     /* physical pages in the pool */
+    int32_t   kv_heads;
+    int32_t   head_dim;    /* must be 128 */
+} qm_kv_cache;
+
+/* ---- library ----------------------------------------------------------------- */
+/* ABI version of this header; bumped on any signature change. */
+int32_t qm_abi_version(void);
+/* Short static description of an error code. */
+const char* qm_error_string(int32_t code);
+/* Names the architecture the kernels were compiled for ("gfx950"). */
+const char* qm_target_arch(void);
+
+/* ---- (1) fused QK-RMSNorm + RoPE + KV append ------------------------------------- */
+/*
+ * Replaces NativeTalkerEngine::launch_qk_norm_rope_cache_m1 (R17:17569-17606, kernel
+ * talker_qk_norm_rope_cache_fused_kernel R17:15365-15526) and its predictor twin
+ * qk_norm_rope_cache_m1 (R17:13432-13471, kernel R17:12133-12307).
+ * q [q_heads][128], k, v [kv_heads][128], q_norm_w, k_norm_w, cos, sin [128] (device).
+ * Writes q_rotated [q_heads][128]; K (normed, rotated) and V (raw copy) into the cache
+ * slot of token `cache_position`.  page_table: device int32 [max_pages] or NULL
+ * (identity).  Rounding chain: bf16 after normalise, after gamma, after each RoPE
+ * product and after their sum — exactly the reference's.
+ */
+int32_t qm_qk_norm_rope_kv_append(
+    const uint16_t* q, const uint16_t* k, const uint16_t* v,
+    const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+    const uint16_t* cos_row, const uint16_t* sin_row,
+    uint16_t* q_rotated,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    int32_t q_heads, int32_t cache_position, float epsilon,
+    void* hip_stream);
+
+/*
+ * Multi-stream form of the same operator (no reference counterpart: the reference
+ * serves one sequence; R17:17110-17112 computes the single position on the host).
+ * q [n][q_heads][128], k, v [n][kv_heads][128]; positions [n] device int32;
+ * page_table [n][max_pages] device int32; cos/sin: row s if rope_by_position == 0,
+ * row positions[s] otherwise.  A stream whose position or page is out of range is
+ * skipped and the bits above are OR-ed into *status_dev (optional, device uint32).
+ */
+int32_t qm_qk_norm_rope_kv_append_ragged(
+    const uint16_t* q, const uint16_t* k, const uint16_t* v,
+    const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+    const uint16_t* cos_rows, const uint16_t* sin_rows, int32_t rope_by_position,
+    uint16_t* q_rotated,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    const int32_t* positions, int32_t n_streams,
+    int32_t q_heads, float epsilon, uint32_t* status_dev,
+    void* hip_stream);
+
+/* ---- (2) GQA decode attention ------------------------------------------------------ */
+/*
+ * Bytes of caller workspace the split-K decode needs for up to n_streams sequences of
+ * at most max_seq_len tokens.  Pure host arithmetic (capture-safe).
+ */
+size_t qm_decode_workspace_bytes(int32_t n_streams, int32_t q_heads,
+                                 int32_t kv_heads, int32_t max_seq_len);
+
+/*
+ * Replaces NativeTalkerEngine::launch_attention with query_length == 1
+ * (R17:17723-17779, kernel talker_attention_gqa2_m1_locality_kernel R17:16014-16203)
+ * and the predictor's attention_m1 (R17:13473-13497).  query, context_out
+ * [q_heads][128]; keys [key_start, cache_before+1) with key_start from
+ * sliding_window as in R17:16032-16036 (<= 0 disables the window).
+ * Scores are rounded to bf16 before and after scaling like the reference
+ * (R17:16102-16116); softmax and P·V stay in fp32 (online softmax, split-K).
+ */
+int32_t qm_decode_attention(
+    const uint16_t* query,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    uint16_t* context_out,
+    int32_t q_heads, int32_t cache_before, int32_t sliding_window, float scale,
+    void* workspace, size_t workspace_bytes,
+    void* hip_stream);
+
+/*
+ * Ragged multi-stream decode (no reference counterpart; one launch for all streams).
+ * query, context_out [n][q_heads][128]; seq_lens [n] device int32 (context length of
+ * each stream, 0 = produce zeros); page_table [n][max_pages]; max_seq_len: host upper
+ * bound on seq_lens used to size the grid and the workspace.
+ */
+int32_t qm_decode_attention_ragged(
+    const uint16_t* query,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    const int32_t* seq_lens, int32_t n_streams, int32_t max_seq_len,
+    uint16_t* context_out,
+    int32_t q_heads, float scale,
+    void* workspace, size_t workspace_bytes, uint32_t* status_dev,
+    void* hip_stream);
+
+/* ---- (3) prefill ---------------------------------------------------------------------- */
+/*
+ * Per-head RMSNorm (optional) + RoPE over rows.  Replaces rmsnorm_kernel with
+ * rows = S*heads, dim 128 (R17:8276-8338, called R17:16673-16689) followed by
+ * launch_rope_rows (R17:17608-17644, kernel R17:15531-15625).
+ * in/out [rows][heads][128]; cos/sin [rows][128]; norm_w [128] or NULL (RoPE only).
+ */
+int32_t qm_norm_rope_rows(
+    const uint16_t* in, const uint16_t* norm_w,
+    const uint16_t* cos_rows, const uint16_t* sin_rows,
+    uint16_t* out, int32_t rows, int32_t heads, float epsilon,
+    void* hip_stream);
+
+/*
+ * Replaces scatter_prefill_cache (R17:17646-17682, kernel R17:15630-15687) and, with
+ * rows == 1, scatter_decode_cache (R17:17684-17720).  key/value [rows][kv_heads][128]
+ * are copied to tokens first_position .. first_position+rows-1.
+ */
+int32_t qm_scatter_kv(
+    const uint16_t* key, const uint16_t* value,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    int32_t rows, int32_t first_position,
+    void* hip_stream);
+
+/*
+ * Causal GQA prefill on bf16 MFMA.  Replaces launch_attention with query_length > 1,
+ * cache_before == 0 (R17:17782-17813, kernel talker_attention_kernel R17:15744-16006)
+ * fused with scatter_prefill_cache.  query, context_out [batch][seq][q_heads][128];
+ * key, value [batch][seq][kv_heads][128] already normed/rotated; row i attends keys
+ * 0..i of its own batch entry.  If cache != NULL, K/V are also written to the pages of
+ * page_table [batch][max_pages] at tokens 0..seq-1.
+ */
+int32_t qm_prefill_attention_causal(
+    const uint16_t* query, const uint16_t* key, const uint16_t* value,
+    uint16_t* context_out,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads, float scale,
+    uint32_t* status_dev,
+    void* hip_stream);
+
+/* ---- (4) code-predictor attention loop ---------------------------------------------------- */
+/*
+ * One launch for the whole per-frame step loop of the code predictor: replaces, per
+ * (frame, layer) unit, steps x { qk_norm_rope_cache_m1 (R17:13432) + attention_m1
+ * (R17:13473) } and step 0's rope/update_cache/attention (R17:13238-13386), following
+ * the schedule of PersistentPredictor::capture_step (R17:13592-13596).
+ * q [units][rows][16][128], k, v [units][rows][8][128] (rows <= 16, row r at position r);
+ * q_norm_w, k_norm_w [n_layers][128], unit u uses layer u % n_layers;
+ * cos/sin [rows][128]; context_out [units][rows][16][128].
+ * first_rows: 1 or 2 — the number of rows the first step carries (2 = the reference's
+ * causal two-row step 0); it changes the step numbering only, row r always attends keys
+ * 0..r.  k_cache_out / v_cache_out: optional [units][8][16][128] write-back of the
+ * per-unit cache (R17:10711-10737 layout), NULL to skip.
+ * This operator reproduces the reference's full rounding chain, including bf16(P).
+ */
+int32_t qm_predictor_attention_loop(
+    const uint16_t* q, const uint16_t* k, const uint16_t* v,
+    const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+    const uint16_t* cos_rows, const uint16_t* sin_rows,
+    uint16_t* context_out, uint16_t* k_cache_out, uint16_t* v_cache_out,
+    int32_t units, int32_t n_layers, int32_t rows, int32_t first_rows,
+    float epsilon,
+    void* hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QM_ATTN_H */

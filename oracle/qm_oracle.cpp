@@ -1,0 +1,683 @@
+// qm_oracle.cpp — TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+//
+// Scalar CPU restatement (fp32 accumulate, bf16 storage) of the attention / KV-cache
+// operators of the reference engine, devices/rx7900xtx-24g/qwen3_tts_1_7b.cpp ("R17").
+// Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may load this
+// library; the shipped library (libqm_attn.so) never links or calls it.
+//
+// The reference has no CPU implementation and ships no golden vectors for this path,
+// so every function here follows the reference *source text* line by line (cited at
+// each function) and is pinned by the closed forms / invariants / brute-force checks
+// in tests/test_oracle_*.py.  What cannot be pinned here: agreement of the reference's
+// bf16 boundary chain with upstream PyTorch on real weights (claimed in the comments at
+// R17:15446, 15879) — parity unpinned against upstream, inherited as an assumption.
+//
+// Device-specific arithmetic that has no bit-exact CPU twin is restated as follows:
+//   rsqrtf(x)  (R17:15437, 12198, 8309)  ->  1.0f / sqrtf(x), both correctly rounded;
+//   expf(x)    (R17:15933, 12490, 9582)  ->  glibc expf.
+// Wave32 shuffle-tree reductions (R17:15059-15148, 8233-8274, 9358-9364) are simulated
+// lane by lane so that fp32 summation order is the reference's.
+//
+// Attention policies (last argument of the attention functions):
+//   QMO_POLICY_REFERENCE  the reference chain: bf16(QK) -> bf16(*scale) -> fp32 softmax
+//                         -> bf16(P) -> fp32 P.V -> bf16            (R17:15841-16005)
+//   QMO_POLICY_ONLINE     same score roundings; P stays fp32 and is normalised after the
+//                         P.V accumulation (what an online-softmax kernel computes)
+//   QMO_POLICY_FP32       no intermediate rounding at all (plain softmax(QK^T*scale)V)
+
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <thread>
+#include <vector>
+#include <algorithm>
+#include <functional>
+
+#include "../include/qm_attn.h"
+
+#define QMO_POLICY_REFERENCE 0
+#define QMO_POLICY_ONLINE    1
+#define QMO_POLICY_FP32      2
+
+namespace {
+
+constexpr int kDim = 128;
+
+// R17:15024-15031
+inline float bf2f(uint16_t v) {
+    uint32_t bits = static_cast<uint32_t>(v) << 16;
+    float f;
+    std::memcpy(&f, &bits, sizeof f);
+    return f;
+}
+
+// R17:15034-15056 (same as 79-101, 8172-8187, host 21570-21574)
+inline uint16_t f2bf(float value) {
+    uint32_t bits;
+    std::memcpy(&bits, &value, sizeof bits);
+    if ((bits & 0x7fffffffU) > 0x7f800000U) {
+        return static_cast<uint16_t>((bits >> 16) | 0x0040U);
+    }
+    const uint32_t lsb = (bits >> 16) & 1U;
+    bits += 0x7fffU + lsb;
+    return static_cast<uint16_t>(bits >> 16);
+}
+
+// value += __shfl_down(value, offset) for offset 16..1 on a 32-lane wave; a lane whose
+// source is out of range receives its own value (R17:15059-15075, 9358-9364).
+// Returns lane 0.
+inline float wave32_sum(const float* lanes) {
+    // Only the lanes that feed lane 0 matter; all of their sources are in range.
+    float a[16], b[8], c[4], d[2];
+    for (int i = 0; i < 16; ++i) a[i] = lanes[i] + lanes[i + 16];
+    for (int i = 0; i < 8; ++i) b[i] = a[i] + a[i + 8];
+    for (int i = 0; i < 4; ++i) c[i] = b[i] + b[i + 4];
+    for (int i = 0; i < 2; ++i) d[i] = c[i] + c[i + 2];
+    return d[0] + d[1];
+}
+
+// R17:15078-15099: value = value > other ? value : other.
+inline float wave32_max(const float* lanes) {
+    auto mx = [](float v, float o) { return v > o ? v : o; };
+    float a[16], b[8], c[4], d[2];
+    for (int i = 0; i < 16; ++i) a[i] = mx(lanes[i], lanes[i + 16]);
+    for (int i = 0; i < 8; ++i) b[i] = mx(a[i], a[i + 8]);
+    for (int i = 0; i < 4; ++i) c[i] = mx(b[i], b[i + 4]);
+    for (int i = 0; i < 2; ++i) d[i] = mx(c[i], c[i + 2]);
+    return mx(d[0], d[1]);
+}
+
+// talker_block_sum / talker_block_max over `threads` per-thread values
+// (R17:15102-15197): wave trees, then a tree over the per-wave results in wave 0.
+inline float block_sum(const float* per_thread, int threads) {
+    const int waves = (threads + 31) >> 5;
+    float wave_values[32];
+    for (int w = 0; w < 32; ++w) wave_values[w] = 0.0f;
+    for (int w = 0; w < waves; ++w) {
+        float lanes[32];
+        for (int l = 0; l < 32; ++l) {
+            const int t = w * 32 + l;
+            lanes[l] = t < threads ? per_thread[t] : 0.0f;
+        }
+        wave_values[w] = wave32_sum(lanes);
+    }
+    return wave32_sum(wave_values);
+}
+
+inline float block_max(const float* per_thread, int threads) {
+    const int waves = (threads + 31) >> 5;
+    float wave_values[32];
+    for (int w = 0; w < 32; ++w) wave_values[w] = -INFINITY;
+    for (int w = 0; w < waves; ++w) {
+        float lanes[32];
+        for (int l = 0; l < 32; ++l) {
+            const int t = w * 32 + l;
+            lanes[l] = t < threads ? per_thread[t] : -INFINITY;
+        }
+        wave_values[w] = wave32_max(lanes);
+    }
+    return wave32_max(wave_values);
+}
+
+// Sum of squares of one 128-wide head in the reference's order: one thread per
+// dimension, x*x, 32-lane trees, then the tree over the four wave sums
+// (R17:15429-15433 with 128 threads; R17:12178-12194 and 8292-8304 with 256 threads,
+// whose upper four waves contribute exact zeros — same result).
+inline float head_sum_squares(const uint16_t* x) {
+    float sq[kDim];
+    for (int d = 0; d < kDim; ++d) {
+        const float v = bf2f(x[d]);
+        sq[d] = v * v;
+    }
+    return block_sum(sq, kDim);
+}
+
+inline float inverse_rms(float sum, float epsilon) {
+    // R17:15436-15441: rsqrtf(sum / head_dim + epsilon)
+    return 1.0f / std::sqrt(sum / static_cast<float>(kDim) + epsilon);
+}
+
+// RMSNorm of one head: bf16(x*r) then bf16(that * gamma)   (R17:15448-15460, 8321-8336)
+inline void head_rmsnorm(const uint16_t* x, const uint16_t* gamma, float epsilon,
+                         uint16_t* out) {
+    const float r = inverse_rms(head_sum_squares(x), epsilon);
+    for (int d = 0; d < kDim; ++d) {
+        const uint16_t n = f2bf(bf2f(x[d]) * r);
+        out[d] = f2bf(bf2f(n) * bf2f(gamma[d]));
+    }
+}
+
+// RoPE of one head: bf16(bf16(x*cos) + bf16(rotate_half(x)*sin)), rotate_half = (-x2, +x1)
+// (R17:15464-15498, 15571-15624, 8432-8488)
+inline void head_rope(const uint16_t* x, const uint16_t* cosv, const uint16_t* sinv,
+                      uint16_t* out) {
+    uint16_t tmp[kDim];
+    for (int d = 0; d < kDim; ++d) {
+        const int rd = d < kDim / 2 ? d + kDim / 2 : d - kDim / 2;
+        float rotated = bf2f(x[rd]);
+        if (d < kDim / 2) rotated = -rotated;
+        const uint16_t first = f2bf(bf2f(x[d]) * bf2f(cosv[d]));
+        const uint16_t second = f2bf(rotated * bf2f(sinv[d]));
+        tmp[d] = f2bf(bf2f(first) + bf2f(second));
+    }
+    std::memcpy(out, tmp, sizeof tmp);
+}
+
+// Element offset of (token, head) in the paged pool; -1 if out of range.
+inline int64_t slot_offset(const qm_kv_cache* c, const int32_t* page_table,
+                           int32_t max_pages, int64_t token, int head) {
+    if (token < 0) return -1;
+    const int64_t page = token / c->page_size;
+    if (page >= max_pages) return -1;
+    const int64_t phys = page_table ? page_table[page] : page;
+    if (phys < 0 || phys >= c->n_pages) return -1;
+    return phys * c->stride_page + static_cast<int64_t>(head) * c->stride_head
+         + (token % c->page_size) * c->stride_token;
+}
+
+// One score: the reference's wave-per-key dot product — lane l accumulates dims
+// l, l+32, l+64, l+96 with fmaf, then the 32-lane tree (R17:15850-15876, 16080-16100,
+// 9434-9454, 12386-12418).
+inline float qk_dot(const uint16_t* q, const uint16_t* k) {
+    float lanes[32];
+    for (int l = 0; l < 32; ++l) {
+        float acc = 0.0f;
+        for (int d = l; d < kDim; d += 32) acc = std::fmaf(bf2f(q[d]), bf2f(k[d]), acc);
+        lanes[l] = acc;
+    }
+    return wave32_sum(lanes);
+}
+
+inline float score_from_dot(float acc, float scale, int policy) {
+    if (policy == QMO_POLICY_FP32) return acc * scale;
+    // R17:15881-15890: bf16(acc), then bf16(that * scale)
+    const uint16_t raw = f2bf(acc);
+    return bf2f(f2bf(bf2f(raw) * scale));
+}
+
+using RowPtr = std::function<const uint16_t*(int)>;
+
+// Attention of one query head vector over keys [key_start, key_end) in the talker's
+// topology: 256 threads, thread-strided softmax partials, serial P.V
+// (R17:15894-16005 == 16121-16202).
+void attend_talker(const uint16_t* q, const RowPtr& key_row, const RowPtr& value_row,
+                   int key_start, int key_end, float scale, int policy, uint16_t* out) {
+    const int n = key_end - key_start;
+    if (n <= 0) {
+        for (int d = 0; d < kDim; ++d) out[d] = 0;
+        return;
+    }
+    std::vector<float> s(n);
+    for (int i = 0; i < n; ++i) {
+        s[i] = score_from_dot(qk_dot(q, key_row(key_start + i)), scale, policy);
+    }
+    if (policy == QMO_POLICY_REFERENCE) {
+        constexpr int T = 256;
+        float part[T];
+        for (int t = 0; t < T; ++t) {
+            float m = -INFINITY;
+            for (int i = t; i < n; i += T) m = m > s[i] ? m : s[i];
+            part[t] = m;
+        }
+        const float maximum = block_max(part, T);
+        for (int t = 0; t < T; ++t) {
+            float acc = 0.0f;
+            for (int i = t; i < n; i += T) acc += std::exp(s[i] - maximum);
+            part[t] = acc;
+        }
+        const float total = block_sum(part, T);
+        std::vector<float> p(n);
+        for (int i = 0; i < n; ++i) p[i] = bf2f(f2bf(std::exp(s[i] - maximum) / total));
+        float acc[kDim];
+        for (int d = 0; d < kDim; ++d) acc[d] = 0.0f;
+        for (int i = 0; i < n; ++i) {
+            const uint16_t* v = value_row(key_start + i);
+            for (int d = 0; d < kDim; ++d) acc[d] = std::fmaf(p[i], bf2f(v[d]), acc[d]);
+        }
+        for (int d = 0; d < kDim; ++d) out[d] = f2bf(acc[d]);
+        return;
+    }
+    // ONLINE / FP32: fp32 probabilities, normalisation after the accumulation.
+    float maximum = -INFINITY;
+    for (int i = 0; i < n; ++i) maximum = maximum > s[i] ? maximum : s[i];
+    float total = 0.0f;
+    float acc[kDim];
+    for (int d = 0; d < kDim; ++d) acc[d] = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        const float p = std::exp(s[i] - maximum);
+        total += p;
+        const uint16_t* v = value_row(key_start + i);
+        for (int d = 0; d < kDim; ++d) acc[d] = std::fmaf(p, bf2f(v[d]), acc[d]);
+    }
+    for (int d = 0; d < kDim; ++d) out[d] = f2bf(acc[d] / total);
+}
+
+// The predictor's topology for key_length <= 32: one wave per softmax row with lane =
+// key, tree max / tree sum, and P.V as lane-strided fmaf + 32-lane tree
+// (R17:12449-12574 == 9544-9601 + 9666-9697).  `masked_from` >= 0 marks keys that the
+// staged causal mask replaced by bf16 -inf (R17:9516-9523).
+void attend_predictor(const uint16_t* q, const RowPtr& key_row, const RowPtr& value_row,
+                      int key_length, int masked_from, float scale, uint16_t* out) {
+    float s[32];
+    for (int l = 0; l < 32; ++l) s[l] = -INFINITY;
+    for (int i = 0; i < key_length; ++i) {
+        s[i] = score_from_dot(qk_dot(q, key_row(i)), scale, QMO_POLICY_REFERENCE);
+        if (masked_from >= 0 && i >= masked_from) s[i] = bf2f(0xff80);
+    }
+    // max tree; the `lane + offset < 32` guard (R17:12463-12480) only changes lanes that
+    // do not feed lane 0.
+    const float maximum = wave32_max(s);
+    float e[32];
+    for (int l = 0; l < 32; ++l) e[l] = l < key_length ? std::exp(s[l] - maximum) : 0.0f;
+    const float total = wave32_sum(e);
+    float p[32];
+    for (int l = 0; l < 32; ++l) p[l] = l < key_length ? bf2f(f2bf(e[l] / total)) : 0.0f;
+    for (int d = 0; d < kDim; ++d) {
+        float lanes[32];
+        for (int l = 0; l < 32; ++l) {
+            lanes[l] = 0.0f;
+            if (l < key_length) lanes[l] = std::fmaf(p[l], bf2f(value_row(l)[d]), 0.0f);
+        }
+        out[d] = f2bf(wave32_sum(lanes));
+    }
+}
+
+void parallel_for(int64_t n, int n_threads, const std::function<void(int64_t)>& body) {
+    if (n_threads <= 1 || n <= 1) {
+        for (int64_t i = 0; i < n; ++i) body(i);
+        return;
+    }
+    const int workers = static_cast<int>(std::min<int64_t>(n_threads, n));
+    std::vector<std::thread> pool;
+    pool.reserve(workers);
+    for (int w = 0; w < workers; ++w) {
+        pool.emplace_back([&, w]() {
+            for (int64_t i = w; i < n; i += workers) body(i);
+        });
+    }
+    for (auto& t : pool) t.join();
+}
+
+inline uint64_t splitmix_at(uint64_t seed, uint64_t k) {
+    // k-th output (k >= 1) of the SplitMix64 stream seeded with `seed`
+    // (generator of R17:7108-7130: state += golden; mix(state)).
+    uint64_t z = seed + k * 0x9e3779b97f4a7c15ULL;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ULL;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebULL;
+    return z ^ (z >> 31);
+}
+
+bool cache_ok(const qm_kv_cache* c) {
+    return c && c->k_pool && c->v_pool && c->head_dim == kDim && c->stride_token == kDim
+        && c->page_size > 0 && c->n_pages > 0 && c->kv_heads > 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+// ---- scalar helpers ------------------------------------------------------------------
+uint16_t qmo_f32_to_bf16(float v) { return f2bf(v); }
+float qmo_bf16_to_f32(uint16_t v) { return bf2f(v); }
+
+void qmo_f32_to_bf16_array(const float* in, uint16_t* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = f2bf(in[i]);
+}
+void qmo_bf16_to_f32_array(const uint16_t* in, float* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = bf2f(in[i]);
+}
+
+float qmo_head_sum_squares(const uint16_t* x) { return head_sum_squares(x); }
+
+// ---- seeded synthetic inputs (owned by this repo; SplitMix64 -> Box-Muller) ----------
+// Element i uses stream outputs 2i+1 and 2i+2, so the result does not depend on the
+// thread count.
+void qmo_fill_normal_bf16(uint16_t* out, int64_t n, uint64_t seed, float mean, float stdev,
+                          int n_threads) {
+    const int64_t chunk = 1 << 16;
+    const int64_t chunks = (n + chunk - 1) / chunk;
+    parallel_for(chunks, n_threads, [&](int64_t c) {
+        const int64_t lo = c * chunk, hi = std::min(n, lo + chunk);
+        for (int64_t i = lo; i < hi; ++i) {
+            const uint64_t a = splitmix_at(seed, 2 * static_cast<uint64_t>(i) + 1);
+            const uint64_t b = splitmix_at(seed, 2 * static_cast<uint64_t>(i) + 2);
+            const double u1 = (static_cast<double>(a >> 11) + 1.0) * (1.0 / 9007199254740992.0);
+            const double u2 = static_cast<double>(b >> 11) * (1.0 / 9007199254740992.0);
+            const double z = std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586477 * u2);
+            out[i] = f2bf(static_cast<float>(mean + stdev * z));
+        }
+    });
+}
+
+// Integers uniform in [lo, hi] (inclusive).
+void qmo_fill_uniform_int(int32_t* out, int64_t n, uint64_t seed, int32_t lo, int32_t hi) {
+    const uint64_t span = static_cast<uint64_t>(static_cast<int64_t>(hi) - lo + 1);
+    for (int64_t i = 0; i < n; ++i) {
+        out[i] = static_cast<int32_t>(lo + static_cast<int64_t>(
+            splitmix_at(seed, static_cast<uint64_t>(i) + 1) % span));
+    }
+}
+
+// Seeded Fisher-Yates permutation of 0..n-1.
+void qmo_permutation(int32_t* out, int64_t n, uint64_t seed) {
+    for (int64_t i = 0; i < n; ++i) out[i] = static_cast<int32_t>(i);
+    for (int64_t i = n - 1; i > 0; --i) {
+        const uint64_t j = splitmix_at(seed, static_cast<uint64_t>(n - i)) % static_cast<uint64_t>(i + 1);
+        std::swap(out[i], out[j]);
+    }
+}
+
+// ---- RoPE table: make_talker_rope R17:21576-21590, PersistentPredictor::make_rope
+// R17:13161-13197 -------------------------------------------------------------------------
+int32_t qmo_rope_table(int32_t rows, int32_t start, int32_t head_dim, double theta,
+                       uint16_t* cos_out, uint16_t* sin_out) {
+    if (rows < 0 || start < 0 || head_dim <= 0 || (head_dim & 1)) return QM_ERR_GEOMETRY;
+    const int half = head_dim / 2;
+    for (int row = 0; row < rows; ++row) {
+        const double pos = static_cast<double>(start + row);
+        for (int i = 0; i < half; ++i) {
+            const double inv = std::pow(theta, -2.0 * static_cast<double>(i)
+                                                   / static_cast<double>(head_dim));
+            const double a = pos * inv;
+            const uint16_t c = f2bf(static_cast<float>(std::cos(a)));
+            const uint16_t s = f2bf(static_cast<float>(std::sin(a)));
+            const size_t b = static_cast<size_t>(row) * head_dim;
+            cos_out[b + i] = c;
+            cos_out[b + i + half] = c;
+            sin_out[b + i] = s;
+            sin_out[b + i + half] = s;
+        }
+    }
+    return QM_OK;
+}
+
+// ---- (1) fused norm + RoPE + append: R17:15365-15526 (talker), 12133-12307 (predictor) ---
+int32_t qmo_qk_norm_rope_kv_append(
+    const uint16_t* q, const uint16_t* k, const uint16_t* v,
+    const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+    const uint16_t* cos_row, const uint16_t* sin_row,
+    uint16_t* q_rotated,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    int32_t q_heads, int32_t cache_position, float epsilon) {
+    if (!q || !k || !v || !q_norm_w || !k_norm_w || !cos_row || !sin_row || !q_rotated)
+        return QM_ERR_NULL;
+    if (!cache_ok(cache)) return QM_ERR_GEOMETRY;
+    if (slot_offset(cache, page_table, max_pages, cache_position, 0) < 0)
+        return QM_ERR_SLOT_RANGE;
+    uint16_t tmp[kDim];
+    for (int h = 0; h < q_heads; ++h) {
+        head_rmsnorm(q + h * kDim, q_norm_w, epsilon, tmp);
+        head_rope(tmp, cos_row, sin_row, q_rotated + h * kDim);
+    }
+    for (int h = 0; h < cache->kv_heads; ++h) {
+        const int64_t off = slot_offset(cache, page_table, max_pages, cache_position, h);
+        head_rmsnorm(k + h * kDim, k_norm_w, epsilon, tmp);
+        head_rope(tmp, cos_row, sin_row, cache->k_pool + off);
+        // V is appended un-normalised and un-rotated (R17:15515-15524).
+        std::memcpy(cache->v_pool + off, v + h * kDim, kDim * sizeof(uint16_t));
+    }
+    return QM_OK;
+}
+
+int32_t qmo_qk_norm_rope_kv_append_ragged(
+    const uint16_t* q, const uint16_t* k, const uint16_t* v,
+    const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+    const uint16_t* cos_rows, const uint16_t* sin_rows, int32_t rope_by_position,
+    uint16_t* q_rotated,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    const int32_t* positions, int32_t n_streams,
+    int32_t q_heads, float epsilon, uint32_t* status) {
+    if (!positions || !page_table) return QM_ERR_NULL;
+    if (!cache_ok(cache)) return QM_ERR_GEOMETRY;
+    for (int s = 0; s < n_streams; ++s) {
+        const int32_t pos = positions[s];
+        const int32_t* pt = page_table + static_cast<int64_t>(s) * max_pages;
+        if (pos < 0 || pos / cache->page_size >= max_pages) {
+            if (status) *status |= QM_STATUS_BAD_POSITION;
+            continue;
+        }
+        if (slot_offset(cache, pt, max_pages, pos, 0) < 0) {
+            if (status) *status |= QM_STATUS_BAD_PAGE;
+            continue;
+        }
+        const int64_t row = rope_by_position ? pos : s;
+        const int32_t rc = qmo_qk_norm_rope_kv_append(
+            q + static_cast<int64_t>(s) * q_heads * kDim,
+            k + static_cast<int64_t>(s) * cache->kv_heads * kDim,
+            v + static_cast<int64_t>(s) * cache->kv_heads * kDim,
+            q_norm_w, k_norm_w, cos_rows + row * kDim, sin_rows + row * kDim,
+            q_rotated + static_cast<int64_t>(s) * q_heads * kDim,
+            cache, pt, max_pages, q_heads, pos, epsilon);
+        if (rc != QM_OK) return rc;
+    }
+    return QM_OK;
+}
+
+// ---- prefill front half: rmsnorm_kernel rows = S*heads, dim 128 (R17:8276-8338) followed by
+// talker_rope_rows_kernel (R17:15531-15625) -------------------------------------------------
+int32_t qmo_norm_rope_rows(const uint16_t* in, const uint16_t* norm_w,
+                           const uint16_t* cos_rows, const uint16_t* sin_rows,
+                           uint16_t* out, int32_t rows, int32_t heads, float epsilon) {
+    if (!in || !cos_rows || !sin_rows || !out) return QM_ERR_NULL;
+    if (rows < 0 || heads <= 0) return QM_ERR_ARGUMENT;
+    uint16_t tmp[kDim];
+    for (int64_t r = 0; r < rows; ++r) {
+        for (int h = 0; h < heads; ++h) {
+            const uint16_t* x = in + (r * heads + h) * kDim;
+            if (norm_w) {
+                head_rmsnorm(x, norm_w, epsilon, tmp);
+                x = tmp;
+            }
+            head_rope(x, cos_rows + r * kDim, sin_rows + r * kDim, out + (r * heads + h) * kDim);
+        }
+    }
+    return QM_OK;
+}
+
+// scatter_prefill_kv (R17:15630-15687) / scatter_decode_kv (R17:15701-15740)
+int32_t qmo_scatter_kv(const uint16_t* key, const uint16_t* value,
+                       const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+                       int32_t rows, int32_t first_position) {
+    if (!key || !value) return QM_ERR_NULL;
+    if (!cache_ok(cache)) return QM_ERR_GEOMETRY;
+    if (rows < 0 || first_position < 0) return QM_ERR_ARGUMENT;
+    for (int64_t r = 0; r < rows; ++r) {
+        if (slot_offset(cache, page_table, max_pages, first_position + r, 0) < 0)
+            return QM_ERR_SLOT_RANGE;
+    }
+    for (int64_t r = 0; r < rows; ++r) {
+        for (int h = 0; h < cache->kv_heads; ++h) {
+            const int64_t off = slot_offset(cache, page_table, max_pages, first_position + r, h);
+            const int64_t src = (r * cache->kv_heads + h) * kDim;
+            std::memcpy(cache->k_pool + off, key + src, kDim * sizeof(uint16_t));
+            std::memcpy(cache->v_pool + off, value + src, kDim * sizeof(uint16_t));
+        }
+    }
+    return QM_OK;
+}
+
+// ---- attention over a (paged) cache: talker_attention_kernel R17:15744-16006, with
+// query_length == 1 identical to talker_attention_gqa2_m1_locality_kernel R17:16014-16203 ---
+// query, out [query_length][q_heads][128]; row i attends keys [key_start, cache_before+i+1).
+int32_t qmo_attention(
+    const uint16_t* query,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    uint16_t* out,
+    int32_t query_length, int32_t cache_before, int32_t q_heads,
+    int32_t sliding_window, float scale, int32_t policy, int32_t n_threads) {
+    if (!query || !out) return QM_ERR_NULL;
+    if (!cache_ok(cache) || q_heads <= 0 || q_heads % cache->kv_heads) return QM_ERR_GEOMETRY;
+    if (query_length < 0 || cache_before < 0) return QM_ERR_ARGUMENT;
+    if (query_length > 0
+        && slot_offset(cache, page_table, max_pages, cache_before + query_length - 1, 0) < 0)
+        return QM_ERR_SLOT_RANGE;
+    const int group = q_heads / cache->kv_heads;
+    parallel_for(static_cast<int64_t>(query_length) * q_heads, n_threads, [&](int64_t item) {
+        const int qi = static_cast<int>(item / q_heads);
+        const int qh = static_cast<int>(item % q_heads);
+        const int kvh = qh / group;                       // R17:15780-15782
+        const int key_end = cache_before + qi + 1;        // R17:15784-15789
+        const int window_start = key_end - sliding_window;
+        const int key_start = sliding_window > 0 ? (window_start > 0 ? window_start : 0) : 0;
+        RowPtr krow = [&](int t) {
+            return cache->k_pool + slot_offset(cache, page_table, max_pages, t, kvh);
+        };
+        RowPtr vrow = [&](int t) {
+            return cache->v_pool + slot_offset(cache, page_table, max_pages, t, kvh);
+        };
+        const int64_t base = (static_cast<int64_t>(qi) * q_heads + qh) * kDim;
+        attend_talker(query + base, krow, vrow, key_start, key_end, scale, policy, out + base);
+    });
+    return QM_OK;
+}
+
+// Ragged multi-stream decode = qmo_attention(query_length 1) per stream.
+int32_t qmo_decode_attention_ragged(
+    const uint16_t* query,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    const int32_t* seq_lens, int32_t n_streams,
+    uint16_t* out, int32_t q_heads, float scale, int32_t policy, int32_t n_threads) {
+    if (!query || !out || !seq_lens || !page_table) return QM_ERR_NULL;
+    if (!cache_ok(cache) || q_heads <= 0 || q_heads % cache->kv_heads) return QM_ERR_GEOMETRY;
+    int32_t rc_all = QM_OK;
+    parallel_for(n_streams, n_threads, [&](int64_t s) {
+        const int64_t base = s * q_heads * kDim;
+        if (seq_lens[s] <= 0) {
+            std::memset(out + base, 0, sizeof(uint16_t) * q_heads * kDim);
+            return;
+        }
+        const int32_t rc = qmo_attention(query + base, cache, page_table + s * max_pages,
+                                         max_pages, out + base, 1, seq_lens[s] - 1, q_heads,
+                                         -1, scale, policy, 1);
+        if (rc != QM_OK) rc_all = rc;
+    });
+    return rc_all;
+}
+
+// ---- causal prefill over contiguous K/V (+ paged write): talker_attention_kernel with
+// cache_before == 0 after scatter_prefill_cache (R17:16703-16717) --------------------------
+int32_t qmo_prefill_attention_causal(
+    const uint16_t* query, const uint16_t* key, const uint16_t* value, uint16_t* out,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads, float scale,
+    int32_t policy, int32_t n_threads) {
+    if (!query || !key || !value || !out) return QM_ERR_NULL;
+    if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads) return QM_ERR_GEOMETRY;
+    if (batch < 0 || seq < 0) return QM_ERR_ARGUMENT;
+    if (cache) {
+        if (!cache_ok(cache) || cache->kv_heads != kv_heads) return QM_ERR_GEOMETRY;
+        for (int b = 0; b < batch; ++b) {
+            const int32_t rc = qmo_scatter_kv(
+                key + static_cast<int64_t>(b) * seq * kv_heads * kDim,
+                value + static_cast<int64_t>(b) * seq * kv_heads * kDim, cache,
+                page_table ? page_table + static_cast<int64_t>(b) * max_pages : nullptr,
+                max_pages, seq, 0);
+            if (rc != QM_OK) return rc;
+        }
+    }
+    const int group = q_heads / kv_heads;
+    parallel_for(static_cast<int64_t>(batch) * seq * q_heads, n_threads, [&](int64_t item) {
+        const int qh = static_cast<int>(item % q_heads);
+        const int64_t t = item / q_heads;
+        const int qi = static_cast<int>(t % seq);
+        const int b = static_cast<int>(t / seq);
+        const int kvh = qh / group;
+        const uint16_t* kb = key + static_cast<int64_t>(b) * seq * kv_heads * kDim;
+        const uint16_t* vb = value + static_cast<int64_t>(b) * seq * kv_heads * kDim;
+        RowPtr krow = [&](int i) { return kb + (static_cast<int64_t>(i) * kv_heads + kvh) * kDim; };
+        RowPtr vrow = [&](int i) { return vb + (static_cast<int64_t>(i) * kv_heads + kvh) * kDim; };
+        const int64_t base = ((static_cast<int64_t>(b) * seq + qi) * q_heads + qh) * kDim;
+        attend_talker(query + base, krow, vrow, 0, qi + 1, scale, policy, out + base);
+    });
+    return QM_OK;
+}
+
+// ---- predictor -------------------------------------------------------------------------
+// predictor_attention_gqa2_m1_kernel R17:12314-12575 over a flat [8][16][128] cache.
+int32_t qmo_predictor_attention_m1(const uint16_t* query, const uint16_t* key_cache,
+                                   const uint16_t* value_cache, uint16_t* out,
+                                   int32_t key_length) {
+    if (!query || !key_cache || !value_cache || !out) return QM_ERR_NULL;
+    if (key_length < 1 || key_length > 16) return QM_ERR_ARGUMENT;
+    uint32_t sb = 0x3db504f3U;  // kAttentionScaleBits, R17:9354-9356
+    float scale;
+    std::memcpy(&scale, &sb, 4);
+    for (int qh = 0; qh < 16; ++qh) {
+        const int kvh = qh / 2;
+        RowPtr krow = [&](int t) { return key_cache + (static_cast<int64_t>(kvh) * 16 + t) * kDim; };
+        RowPtr vrow = [&](int t) { return value_cache + (static_cast<int64_t>(kvh) * 16 + t) * kDim; };
+        attend_predictor(query + qh * kDim, krow, vrow, key_length, -1, scale, out + qh * kDim);
+    }
+    return QM_OK;
+}
+
+// The staged six-kernel attention of step 0 (R17:9369-9745, dispatch 13300-13386):
+// query in BHSD [16][rows][128], cache [8][16][128], causal mask over key_length keys,
+// output transposed to [rows][16][128].
+int32_t qmo_predictor_attention_staged(const uint16_t* query_bhsd, const uint16_t* key_cache,
+                                       const uint16_t* value_cache, uint16_t* out_bshd,
+                                       int32_t rows, int32_t key_length, int32_t causal) {
+    if (!query_bhsd || !key_cache || !value_cache || !out_bshd) return QM_ERR_NULL;
+    if (rows < 1 || key_length < 1 || key_length > 16) return QM_ERR_ARGUMENT;
+    uint32_t sb = 0x3db504f3U;
+    float scale;
+    std::memcpy(&scale, &sb, 4);
+    for (int qh = 0; qh < 16; ++qh) {
+        const int kvh = qh / 2;
+        RowPtr krow = [&](int t) { return key_cache + (static_cast<int64_t>(kvh) * 16 + t) * kDim; };
+        RowPtr vrow = [&](int t) { return value_cache + (static_cast<int64_t>(kvh) * 16 + t) * kDim; };
+        for (int r = 0; r < rows; ++r) {
+            const int masked_from = causal ? r + 1 : -1;  // key_index > query_index (R17:9517-9520)
+            attend_predictor(query_bhsd + (static_cast<int64_t>(qh) * rows + r) * kDim, krow, vrow,
+                             key_length, masked_from < key_length ? masked_from : -1, scale,
+                             out_bshd + (static_cast<int64_t>(r) * 16 + qh) * kDim);
+        }
+    }
+    return QM_OK;
+}
+
+// The whole step loop of one (frame, layer) unit after another, schedule of
+// PersistentPredictor::capture_step R17:13592-13596: row r is appended at position r and
+// attends keys 0..r.
+int32_t qmo_predictor_attention_loop(
+    const uint16_t* q, const uint16_t* k, const uint16_t* v,
+    const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+    const uint16_t* cos_rows, const uint16_t* sin_rows,
+    uint16_t* context_out, uint16_t* k_cache_out, uint16_t* v_cache_out,
+    int32_t units, int32_t n_layers, int32_t rows, int32_t first_rows,
+    float epsilon, int32_t n_threads) {
+    if (!q || !k || !v || !q_norm_w || !k_norm_w || !cos_rows || !sin_rows || !context_out)
+        return QM_ERR_NULL;
+    if (units < 0 || n_layers <= 0 || rows < 1 || rows > 16) return QM_ERR_ARGUMENT;
+    if (first_rows != 1 && first_rows != 2) return QM_ERR_ARGUMENT;
+    if (first_rows > rows) return QM_ERR_ARGUMENT;
+    parallel_for(units, n_threads, [&](int64_t u) {
+        std::vector<uint16_t> kc(8 * 16 * kDim, 0), vc(8 * 16 * kDim, 0), qrot(16 * kDim);
+        qm_kv_cache cache;
+        cache.k_pool = kc.data();
+        cache.v_pool = vc.data();
+        cache.stride_page = 0;
+        cache.stride_head = 16 * kDim;
+        cache.stride_token = kDim;
+        cache.page_size = 16;
+        cache.n_pages = 1;
+        cache.kv_heads = 8;
+        cache.head_dim = kDim;
+        const int layer = static_cast<int>(u % n_layers);
+        for (int r = 0; r < rows; ++r) {
+            const int64_t row = u * rows + r;
+            qmo_qk_norm_rope_kv_append(
+                q + row * 16 * kDim, k + row * 8 * kDim, v + row * 8 * kDim,
+                q_norm_w + layer * kDim, k_norm_w + layer * kDim,
+                cos_rows + r * kDim, sin_rows + r * kDim, qrot.data(),
+                &cache, nullptr, 1, 16, r, epsilon);
+            qmo_predictor_attention_m1(qrot.data(), kc.data(), vc.data(),
+                                       context_out + row * 16 * kDim, r + 1);
+        }
+        if (k_cache_out) std::memcpy(k_cache_out + u * 8 * 16 * kDim, kc.data(), kc.size() * 2);
+        if (v_cache_out) std::memcpy(v_cache_out + u * 8 * 16 * kDim, vc.data(), vc.size() * 2);
+    });
+    return QM_OK;
+}
+
+}  // extern "C"

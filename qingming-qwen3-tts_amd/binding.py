@@ -1,0 +1,172 @@
+"""ctypes binding of lib/libqm_attn.so.
+
+Arguments are raw device addresses (int) or objects with `.data_ptr()` (torch tensors);
+nothing here touches tensor contents on the host.  There is deliberately no fallback: if
+the library is absent, `lib()` raises.
+"""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(HERE, "lib", "libqm_attn.so")
+
+SCALE_128 = 0.08838834764831845  # 1/sqrt(128), bit pattern 0x3db504f3 (R17:9354-9356)
+
+
+class QmError(RuntimeError):
+    """A C-ABI call returned a negative code (the reference throws std::runtime_error)."""
+
+    def __init__(self, code, what):
+        self.code = code
+        super().__init__(f"{what}: {error_string(code)} ({code})")
+
+
+class KvCache(C.Structure):
+    """Mirror of qm_kv_cache (include/qm_attn.h)."""
+    _fields_ = [
+        ("k_pool", C.c_void_p), ("v_pool", C.c_void_p),
+        ("stride_page", C.c_int64), ("stride_head", C.c_int64), ("stride_token", C.c_int64),
+        ("page_size", C.c_int32), ("n_pages", C.c_int32),
+        ("kv_heads", C.c_int32), ("head_dim", C.c_int32),
+    ]
+
+
+def lib_path():
+    return _LIB_PATH
+
+
+_lib = None
+
+_PTR = C.c_void_p
+_I32 = C.c_int32
+_F32 = C.c_float
+
+_SIGNATURES = {
+    "qm_abi_version": (C.c_int32, []),
+    "qm_error_string": (C.c_char_p, [_I32]),
+    "qm_target_arch": (C.c_char_p, []),
+    "qm_qk_norm_rope_kv_append": (_I32, [_PTR] * 8 + [C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _F32, _PTR]),
+    "qm_qk_norm_rope_kv_append_ragged": (_I32, [_PTR] * 7 + [_I32, _PTR, C.POINTER(KvCache), _PTR, _I32, _PTR,
+                                                 _I32, _I32, _F32, _PTR, _PTR]),
+    "qm_decode_workspace_bytes": (C.c_size_t, [_I32, _I32, _I32, _I32]),
+    "qm_decode_attention": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _I32, _F32,
+                                   _PTR, C.c_size_t, _PTR]),
+    "qm_decode_attention_ragged": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _PTR, _I32,
+                                          _F32, _PTR, C.c_size_t, _PTR, _PTR]),
+    "qm_norm_rope_rows": (_I32, [_PTR] * 5 + [_I32, _I32, _F32, _PTR]),
+    "qm_scatter_kv": (_I32, [_PTR, _PTR, C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _PTR]),
+    "qm_prefill_attention_causal": (_I32, [_PTR] * 4 + [C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _I32, _I32,
+                                           _F32, _PTR, _PTR]),
+    "qm_predictor_attention_loop": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _I32, _F32, _PTR]),
+}
+
+EXPORTS = tuple(_SIGNATURES)
+
+
+def lib():
+    """Loads the shared library (once).  Raises FileNotFoundError if it was not built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise FileNotFoundError(
+                f"{_LIB_PATH} is missing: build it with `python qingming-qwen3-tts_amd/build.py` "
+                "(there is no CPU fallback)")
+        handle = C.CDLL(_LIB_PATH)
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = handle
+    return _lib
+
+
+def error_string(code):
+    return lib().qm_error_string(code).decode()
+
+
+def _addr(x):
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    return x.data_ptr()
+
+
+def _check(code, what):
+    if code != 0:
+        raise QmError(code, what)
+
+
+def paged_cache(k_pool, v_pool, n_pages, kv_heads=8, page_size=16):
+    """Descriptor of the native [page][kv_head][page_size][128] layout."""
+    return KvCache(_addr(k_pool), _addr(v_pool), kv_heads * page_size * 128, page_size * 128, 128,
+                   page_size, n_pages, kv_heads, 128)
+
+
+def flat_cache(key_cache, value_cache, kv_heads, max_cache):
+    """Descriptor of the reference LayerCache [kv_head][max_cache][128] (R17:16371-16390)."""
+    return KvCache(_addr(key_cache), _addr(value_cache), 0, max_cache * 128, 128, max_cache, 1,
+                   kv_heads, 128)
+
+
+def qk_norm_rope_kv_append(q, k, v, gq, gk, cos, sin, q_rot, cache, page_table, max_pages, q_heads,
+                           position, eps=1e-6, stream=0):
+    _check(lib().qm_qk_norm_rope_kv_append(
+        _addr(q), _addr(k), _addr(v), _addr(gq), _addr(gk), _addr(cos), _addr(sin), _addr(q_rot),
+        C.byref(cache), _addr(page_table), max_pages, q_heads, position, eps, stream),
+        "qm_qk_norm_rope_kv_append")
+
+
+def qk_norm_rope_kv_append_ragged(q, k, v, gq, gk, cos, sin, by_position, q_rot, cache, page_table,
+                                  max_pages, positions, n_streams, q_heads, eps=1e-6, status=None,
+                                  stream=0):
+    _check(lib().qm_qk_norm_rope_kv_append_ragged(
+        _addr(q), _addr(k), _addr(v), _addr(gq), _addr(gk), _addr(cos), _addr(sin), int(by_position),
+        _addr(q_rot), C.byref(cache), _addr(page_table), max_pages, _addr(positions), n_streams,
+        q_heads, eps, _addr(status), stream), "qm_qk_norm_rope_kv_append_ragged")
+
+
+def decode_workspace_bytes(n_streams, q_heads, kv_heads, max_seq_len):
+    return lib().qm_decode_workspace_bytes(n_streams, q_heads, kv_heads, max_seq_len)
+
+
+def decode_attention(query, cache, page_table, max_pages, out, q_heads, cache_before,
+                     sliding_window=-1, scale=SCALE_128, workspace=None, workspace_bytes=0, stream=0):
+    _check(lib().qm_decode_attention(
+        _addr(query), C.byref(cache), _addr(page_table), max_pages, _addr(out), q_heads, cache_before,
+        sliding_window, scale, _addr(workspace), workspace_bytes, stream), "qm_decode_attention")
+
+
+def decode_attention_ragged(query, cache, page_table, max_pages, seq_lens, n_streams, max_seq_len, out,
+                            q_heads, scale=SCALE_128, workspace=None, workspace_bytes=0, status=None,
+                            stream=0):
+    _check(lib().qm_decode_attention_ragged(
+        _addr(query), C.byref(cache), _addr(page_table), max_pages, _addr(seq_lens), n_streams,
+        max_seq_len, _addr(out), q_heads, scale, _addr(workspace), workspace_bytes, _addr(status),
+        stream), "qm_decode_attention_ragged")
+
+
+def norm_rope_rows(x, norm_w, cos, sin, out, rows, heads, eps=1e-6, stream=0):
+    _check(lib().qm_norm_rope_rows(_addr(x), _addr(norm_w), _addr(cos), _addr(sin), _addr(out), rows,
+                                   heads, eps, stream), "qm_norm_rope_rows")
+
+
+def scatter_kv(key, value, cache, page_table, max_pages, rows, first_position, stream=0):
+    _check(lib().qm_scatter_kv(_addr(key), _addr(value), C.byref(cache), _addr(page_table), max_pages,
+                               rows, first_position, stream), "qm_scatter_kv")
+
+
+def prefill_attention_causal(query, key, value, out, cache, page_table, max_pages, batch, seq, q_heads,
+                             kv_heads, scale=SCALE_128, status=None, stream=0):
+    _check(lib().qm_prefill_attention_causal(
+        _addr(query), _addr(key), _addr(value), _addr(out),
+        C.byref(cache) if cache is not None else None, _addr(page_table), max_pages, batch, seq,
+        q_heads, kv_heads, scale, _addr(status), stream), "qm_prefill_attention_causal")
+
+
+def predictor_attention_loop(q, k, v, gq, gk, cos, sin, out, k_cache_out, v_cache_out, units, n_layers,
+                             rows, first_rows=1, eps=1e-6, stream=0):
+    _check(lib().qm_predictor_attention_loop(
+        _addr(q), _addr(k), _addr(v), _addr(gq), _addr(gk), _addr(cos), _addr(sin), _addr(out),
+        _addr(k_cache_out), _addr(v_cache_out), units, n_layers, rows, first_rows, eps, stream),
+        "qm_predictor_attention_loop")

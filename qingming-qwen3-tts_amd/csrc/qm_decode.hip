@@ -1,0 +1,429 @@
+// qm_decode.hip — GQA decode attention (single stream and ragged multi-stream) for gfx950.
+//
+// Work decomposition.  The context of one (stream, kv head) is cut into tiles of 16 tokens
+// (= one native page, 4 KiB of K and 4 KiB of V, contiguous).  A block of four waves owns
+// `tiles_per_block` consecutive tiles (split-K); its waves take tiles round-robin.  Inside a
+// wave a tile is fetched by four 128-bit loads per lane for K and four for V: load i covers
+// tokens 4i..4i+3, lane l reads token 4i + l/16, dimensions 8*(l%16)..+7 — one instruction
+// reads 1 KiB contiguous.  All query heads that share the kv head (GQA group G) are served
+// from the same registers, so K and V are read from HBM exactly once.
+//
+// Each 16-lane DPP row is an independent online-softmax stream: its score is completed by a
+// row-rotate all-reduce, and it keeps its own running (max, sum, acc[G][8 dims per lane]).
+// The 16 row-streams of a block are merged through LDS; blocks write fp32 partials
+// (acc, max, sum) to the caller's workspace and a small second kernel merges the splits.
+//
+// Rounding: scores are rounded to bf16 before and after scaling as the reference does
+// (R17:16102-16116); probabilities stay fp32 (the reference's bf16(P) after a full-row
+// softmax, R17:16136-16141, cannot be formed by a single-pass kernel).
+//
+// Algorithmic HBM bytes per token of context: kv_heads * 128 * 2 B * 2 (K and V) = 4096 B
+// at 8 kv heads; the kernel is bound by HBM bandwidth.
+
+#include "qm_device.h"
+#include "qm_host.h"
+
+#include <stdlib.h>
+
+namespace qm {
+
+constexpr int kDecodeThreads = 256;
+constexpr int kDecodeWaves = 4;
+constexpr int kRowStreams = 16;  // 4 waves x 4 DPP rows
+
+struct DecodeParams {
+    const uint16_t* query;        // [n_streams][q_heads][128]
+    uint16_t* out;                // [n_streams][q_heads][128]
+    const int32_t* page_table;    // [n_streams][max_pages] or NULL
+    const int32_t* seq_lens;      // [n_streams] or NULL (single stream: fixed range)
+    float* partial;               // workspace
+    uint32_t* status;
+    PageMap pages;
+    int max_seq_len;
+    int fixed_key_start;
+    int fixed_key_end;
+    int tiles_per_block;
+    int max_splits;
+    int q_heads;
+    float scale;
+};
+
+// Partial record of one (stream, kv head, split): G*128 acc, G max, G sum.
+template <int G>
+__host__ __device__ constexpr int partial_floats() { return G * kDim + 2 * G; }
+
+__device__ __forceinline__ uint4 load_or_zero(const uint16_t* p, bool valid) {
+    uint4 r = make_uint4(0, 0, 0, 0);
+    if (valid) r = *reinterpret_cast<const uint4*>(p);
+    return r;
+}
+
+template <int G>
+__global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodeParams prm, qm_kv_cache cache) {
+    __shared__ float sh_acc[kRowStreams][G][kDim];
+    __shared__ float sh_m[kRowStreams][G];
+    __shared__ float sh_l[kRowStreams][G];
+
+    const int split = blockIdx.x;
+    const int kvh = blockIdx.y;
+    const int stream = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int row = lane >> 4;   // DPP row inside the wave = token slot inside a load
+    const int col = lane & 15;   // 8-dim chunk
+
+    int key_start = prm.fixed_key_start;
+    int key_end = prm.fixed_key_end;
+    if (prm.seq_lens) {
+        key_start = 0;
+        key_end = prm.seq_lens[stream];
+        if (key_end > prm.max_seq_len) {
+            // The grid and the workspace were sized for max_seq_len: attend what fits, flag it.
+            if (tid == 0 && prm.status) atomicOr(prm.status, QM_STATUS_BAD_POSITION);
+            key_end = prm.max_seq_len;
+        }
+    }
+    if (key_end <= key_start) {
+        // Empty context: zeros.  With several splits the merge kernel writes them.
+        if (prm.max_splits == 1 && split == 0) {
+            for (int o = tid; o < G * kDim; o += kDecodeThreads) {
+                prm.out[(static_cast<int64_t>(stream) * prm.q_heads + kvh * G) * kDim + o] = 0;
+            }
+        }
+        return;
+    }
+
+    const int first_tile = key_start / kTile;
+    const int last_tile = (key_end - 1) / kTile;
+    const int tile_lo = first_tile + split * prm.tiles_per_block;
+    if (tile_lo > last_tile) return;
+    const int tile_hi = min(tile_lo + prm.tiles_per_block - 1, last_tile);
+
+    const int32_t* table =
+        prm.page_table ? prm.page_table + static_cast<int64_t>(stream) * prm.pages.max_pages : nullptr;
+
+    // Query chunk of this lane for each head of the group, packed bf16 pairs.
+    uint4 qv[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int qh = kvh * G + g;
+        qv[g] = *reinterpret_cast<const uint4*>(
+            prm.query + (static_cast<int64_t>(stream) * prm.q_heads + qh) * kDim + col * 8);
+    }
+
+    float m[G], l[G], acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m[g] = -INFINITY;
+        l[g] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] = 0.0f;
+    }
+
+    uint4 kreg[4], vreg[4];
+    bool valid[4];
+    auto fetch = [&](int tile, uint4* kr, uint4* vr, bool* ok) {
+        const int first_token = tile * kTile;
+        const int64_t off = tile_offset(cache, prm.pages, table, first_token, kvh, prm.status);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int token = first_token + 4 * i + row;
+            ok[i] = off >= 0 && token >= key_start && token < key_end;
+            const int64_t e = off + static_cast<int64_t>(4 * i + row) * kDim + col * 8;
+            kr[i] = load_or_zero(cache.k_pool + e, ok[i]);
+            vr[i] = load_or_zero(cache.v_pool + e, ok[i]);
+        }
+    };
+
+    int tile = tile_lo + wave;
+    if (tile <= tile_hi) fetch(tile, kreg, vreg, valid);
+
+    while (tile <= tile_hi) {
+        const int next = tile + kDecodeWaves;
+        uint4 knext[4], vnext[4];
+        bool oknext[4];
+        if (next <= tile_hi) fetch(next, knext, vnext, oknext);
+
+        // ---- scores of the 4 tokens this row owns, for every head of the group -------------
+        float s[4][G];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                float d = 0.0f;
+                d = dot2_bf16(qv[g].x, kreg[i].x, d);
+                d = dot2_bf16(qv[g].y, kreg[i].y, d);
+                d = dot2_bf16(qv[g].z, kreg[i].z, d);
+                d = dot2_bf16(qv[g].w, kreg[i].w, d);
+                d = row16_allreduce_sum(d);
+                // bf16(QK) then bf16(* scale), R17:16102-16116
+                d = round_bf16(round_bf16(d) * prm.scale);
+                s[i][g] = valid[i] ? d : -INFINITY;
+            }
+        }
+
+        // ---- online softmax update of this row-stream ------------------------------------------
+        float p[4][G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            float mx = fmaxf(fmaxf(s[0][g], s[1][g]), fmaxf(s[2][g], s[3][g]));
+            const float m_new = fmaxf(m[g], mx);
+            const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
+            const float alpha = fast_exp2((m[g] - m_ref) * kLog2e);
+            float psum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                p[i][g] = fast_exp2((s[i][g] - m_ref) * kLog2e);
+                psum += p[i][g];
+            }
+            l[g] = fmaf(l[g], alpha, psum);
+            m[g] = m_new;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[g][e] *= alpha;
+        }
+
+        // ---- P.V -------------------------------------------------------------------------------
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float v0 = lo_bf16(w[j]);
+                const float v1 = hi_bf16(w[j]);
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    acc[g][2 * j] = fmaf(p[i][g], v0, acc[g][2 * j]);
+                    acc[g][2 * j + 1] = fmaf(p[i][g], v1, acc[g][2 * j + 1]);
+                }
+            }
+        }
+
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            kreg[i] = knext[i];
+            vreg[i] = vnext[i];
+            valid[i] = oknext[i];
+        }
+        tile = next;
+    }
+
+    // ---- merge the 16 row-streams of the block -----------------------------------------------
+    const int rs = wave * 4 + row;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sh_acc[rs][g][col * 8 + e] = acc[g][e];
+        if (col == 0) {
+            sh_m[rs][g] = m[g];
+            sh_l[rs][g] = l[g];
+        }
+    }
+    __syncthreads();
+
+    for (int o = tid; o < G * kDim; o += kDecodeThreads) {
+        const int g = o / kDim;
+        const int d = o % kDim;
+        float mm = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < kRowStreams; ++j) mm = fmaxf(mm, sh_m[j][g]);
+        const float m_ref = mm == -INFINITY ? 0.0f : mm;
+        float ll = 0.0f, aa = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kRowStreams; ++j) {
+            const float w = fast_exp2((sh_m[j][g] - m_ref) * kLog2e);
+            ll = fmaf(sh_l[j][g], w, ll);
+            aa = fmaf(sh_acc[j][g][d], w, aa);
+        }
+        if (prm.max_splits == 1) {
+            const int qh = kvh * G + g;
+            prm.out[(static_cast<int64_t>(stream) * prm.q_heads + qh) * kDim + d] =
+                f2bf(ll > 0.0f ? aa / ll : 0.0f);
+        } else {
+            float* rec = prm.partial
+                + ((static_cast<int64_t>(stream) * gridDim.y + kvh) * prm.max_splits + split)
+                      * partial_floats<G>();
+            rec[g * kDim + d] = aa;
+            if (d == 0) {
+                rec[G * kDim + g] = mm;
+                rec[G * kDim + G + g] = ll;
+            }
+        }
+    }
+}
+
+// Merge of the split partials of one (stream, kv head); also writes zeros for an empty
+// context.  grid (kv_heads, n_streams), block G*128.
+template <int G>
+__global__ void decode_merge_kernel(DecodeParams prm) {
+    const int kvh = blockIdx.x;
+    const int stream = blockIdx.y;
+    const int g = threadIdx.x / kDim;
+    const int d = threadIdx.x % kDim;
+    const int qh = kvh * G + g;
+    uint16_t* dst = prm.out + (static_cast<int64_t>(stream) * prm.q_heads + qh) * kDim + d;
+
+    int key_start = prm.fixed_key_start;
+    int key_end = prm.fixed_key_end;
+    if (prm.seq_lens) {
+        key_start = 0;
+        key_end = min(prm.seq_lens[stream], prm.max_seq_len);
+    }
+    if (key_end <= key_start) {
+        *dst = 0;
+        return;
+    }
+    const int tiles = (key_end - 1) / kTile - key_start / kTile + 1;
+    const int splits = min((tiles + prm.tiles_per_block - 1) / prm.tiles_per_block, prm.max_splits);
+    const float* base = prm.partial
+        + (static_cast<int64_t>(stream) * gridDim.x + kvh) * prm.max_splits * partial_floats<G>();
+
+    float mm = -INFINITY;
+    for (int s = 0; s < splits; ++s) mm = fmaxf(mm, base[s * partial_floats<G>() + G * kDim + g]);
+    const float m_ref = mm == -INFINITY ? 0.0f : mm;
+    float ll = 0.0f, aa = 0.0f;
+    for (int s = 0; s < splits; ++s) {
+        const float* rec = base + s * partial_floats<G>();
+        const float w = fast_exp2((rec[G * kDim + g] - m_ref) * kLog2e);
+        ll = fmaf(rec[G * kDim + G + g], w, ll);
+        aa = fmaf(rec[g * kDim + d], w, aa);
+    }
+    *dst = f2bf(ll > 0.0f ? aa / ll : 0.0f);
+}
+
+// ---- host side -------------------------------------------------------------------------------
+
+// Split plan shared by the workspace query and the launch: pure function of the shape.
+struct DecodePlan {
+    int tiles_per_block;
+    int max_splits;
+};
+
+inline DecodePlan plan_decode(int n_streams, int kv_heads, int max_seq_len) {
+    const int64_t max_tiles = (static_cast<int64_t>(max_seq_len) + kTile - 1) / kTile + 1;
+    int tiles_per_block = 0;
+    if (const char* env = getenv("QM_DECODE_TILES_PER_BLOCK")) tiles_per_block = atoi(env);
+    if (tiles_per_block <= 0) {
+        // Aim for about eight blocks per CU over 256 CUs, at least one tile per wave.
+        const int64_t total = max_tiles * n_streams * kv_heads;
+        int64_t t = total / (256 * 8);
+        t = (t + 3) / 4 * 4;
+        if (t < 4) t = 4;
+        if (t > 16) t = 16;
+        tiles_per_block = static_cast<int>(t);
+    }
+    DecodePlan plan;
+    plan.tiles_per_block = tiles_per_block;
+    plan.max_splits = static_cast<int>((max_tiles + tiles_per_block - 1) / tiles_per_block);
+    return plan;
+}
+
+inline size_t decode_workspace_bytes(int n_streams, int q_heads, int kv_heads, int max_seq_len) {
+    const DecodePlan plan = plan_decode(n_streams, kv_heads, max_seq_len);
+    if (plan.max_splits <= 1) return 0;
+    const int g = q_heads / kv_heads;
+    return static_cast<size_t>(n_streams) * kv_heads * plan.max_splits * (g * kDim + 2 * g)
+         * sizeof(float);
+}
+
+template <int G>
+int32_t launch_decode(const DecodeParams& prm, const qm_kv_cache& cache, int n_streams,
+                      hipStream_t stream) {
+    hipLaunchKernelGGL(decode_split_kernel<G>, dim3(prm.max_splits, cache.kv_heads, n_streams),
+                       dim3(kDecodeThreads), 0, stream, prm, cache);
+    int32_t rc = launch_status();
+    if (rc != QM_OK) return rc;
+    if (prm.max_splits > 1) {
+        hipLaunchKernelGGL(decode_merge_kernel<G>, dim3(cache.kv_heads, n_streams), dim3(G * kDim), 0,
+                           stream, prm);
+        rc = launch_status();
+    }
+    return rc;
+}
+
+int32_t decode_common(const uint16_t* query, const qm_kv_cache* cache, const int32_t* page_table,
+                      int32_t max_pages, const int32_t* seq_lens, int32_t n_streams,
+                      int32_t key_start, int32_t key_end, int32_t max_seq_len, uint16_t* out,
+                      int32_t q_heads, float scale, void* workspace, size_t workspace_bytes,
+                      uint32_t* status_dev, void* hip_stream) {
+    if (!query || !out) return QM_ERR_NULL;
+    int32_t rc = check_cache(cache, max_pages);
+    if (rc != QM_OK) return rc;
+    rc = check_group(q_heads, cache->kv_heads);
+    if (rc != QM_OK) return rc;
+    if ((reinterpret_cast<uintptr_t>(query) & 15)) return QM_ERR_GEOMETRY;
+    if (n_streams < 0 || n_streams > 65535 || cache->kv_heads > 65535) return QM_ERR_ARGUMENT;
+    if (max_seq_len < 0) return QM_ERR_ARGUMENT;
+    if (max_seq_len > cache_capacity(cache, max_pages)) return QM_ERR_SLOT_RANGE;
+    if (n_streams == 0) return QM_OK;
+
+    const DecodePlan plan = plan_decode(n_streams, cache->kv_heads, max_seq_len);
+    const size_t need = decode_workspace_bytes(n_streams, q_heads, cache->kv_heads, max_seq_len);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return QM_ERR_WORKSPACE;
+    if (need > 0 && (reinterpret_cast<uintptr_t>(workspace) & 3)) return QM_ERR_WORKSPACE;
+
+    DecodeParams prm;
+    prm.query = query;
+    prm.out = out;
+    prm.page_table = page_table;
+    prm.seq_lens = seq_lens;
+    prm.partial = static_cast<float*>(workspace);
+    prm.status = status_dev;
+    prm.pages = make_page_map(cache->page_size, max_pages);
+    prm.max_seq_len = max_seq_len;
+    prm.fixed_key_start = key_start;
+    prm.fixed_key_end = key_end;
+    prm.tiles_per_block = plan.tiles_per_block;
+    prm.max_splits = plan.max_splits;
+    prm.q_heads = q_heads;
+    prm.scale = scale;
+
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    switch (q_heads / cache->kv_heads) {
+        case 1: return launch_decode<1>(prm, *cache, n_streams, s);
+        case 2: return launch_decode<2>(prm, *cache, n_streams, s);
+        case 4: return launch_decode<4>(prm, *cache, n_streams, s);
+    }
+    return QM_ERR_GEOMETRY;
+}
+
+}  // namespace qm
+
+extern "C" size_t qm_decode_workspace_bytes(int32_t n_streams, int32_t q_heads, int32_t kv_heads,
+                                            int32_t max_seq_len) {
+    if (n_streams <= 0 || q_heads <= 0 || kv_heads <= 0 || max_seq_len < 0 || q_heads % kv_heads)
+        return 0;
+    return qm::decode_workspace_bytes(n_streams, q_heads, kv_heads, max_seq_len);
+}
+
+extern "C" int32_t qm_decode_attention(
+    const uint16_t* query,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    uint16_t* context_out,
+    int32_t q_heads, int32_t cache_before, int32_t sliding_window, float scale,
+    void* workspace, size_t workspace_bytes, void* hip_stream) {
+    if (cache_before < 0) return QM_ERR_ARGUMENT;
+    // Key range of R17:16032-16036.
+    const int32_t key_end = cache_before + 1;
+    const int32_t window_start = key_end - sliding_window;
+    const int32_t key_start = sliding_window > 0 ? (window_start > 0 ? window_start : 0) : 0;
+    if (cache && !page_table && max_pages > 0 && cache->page_size > 0
+        && cache_before / cache->page_size >= cache->n_pages)
+        return QM_ERR_SLOT_RANGE;
+    return qm::decode_common(query, cache, page_table, max_pages, nullptr, 1, key_start, key_end,
+                             key_end, context_out, q_heads, scale, workspace, workspace_bytes,
+                             nullptr, hip_stream);
+}
+
+extern "C" int32_t qm_decode_attention_ragged(
+    const uint16_t* query,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    const int32_t* seq_lens, int32_t n_streams, int32_t max_seq_len,
+    uint16_t* context_out,
+    int32_t q_heads, float scale,
+    void* workspace, size_t workspace_bytes, uint32_t* status_dev, void* hip_stream) {
+    if (!seq_lens || !page_table) return QM_ERR_NULL;
+    return qm::decode_common(query, cache, page_table, max_pages, seq_lens, n_streams, 0, 0,
+                             max_seq_len, context_out, q_heads, scale, workspace, workspace_bytes,
+                             status_dev, hip_stream);
+}

@@ -1,0 +1,110 @@
+// qm_device.h — device-side helpers shared by the gfx950 kernels (wave64 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/qm_attn.h"
+
+namespace qm {
+
+constexpr int kDim = 128;         // head dimension of every supported model family
+constexpr int kTile = 16;         // tokens per K/V tile = tokens per native page
+constexpr float kLog2e = 1.4426950408889634f;
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+// bf16 <-> f32 exactly as the reference does it (R17:15024-15056): widening is a shift,
+// narrowing is round-to-nearest-even on the bit pattern with NaNs quieted.
+__device__ __forceinline__ float bf2f(uint16_t v) {
+    return __uint_as_float(static_cast<uint32_t>(v) << 16);
+}
+
+__device__ __forceinline__ uint16_t f2bf(float value) {
+    uint32_t bits = __float_as_uint(value);
+    if ((bits & 0x7fffffffU) > 0x7f800000U) {
+        return static_cast<uint16_t>((bits >> 16) | 0x0040U);
+    }
+    bits += 0x7fffU + ((bits >> 16) & 1U);
+    return static_cast<uint16_t>(bits >> 16);
+}
+
+// Round an fp32 value to the nearest bf16 and widen it again (hardware RNE convert).
+__device__ __forceinline__ float round_bf16(float x) {
+    return static_cast<float>(static_cast<__bf16>(x));
+}
+
+__device__ __forceinline__ float lo_bf16(uint32_t packed) { return __uint_as_float(packed << 16); }
+__device__ __forceinline__ float hi_bf16(uint32_t packed) { return __uint_as_float(packed & 0xffff0000U); }
+
+// acc + a.x*b.x + a.y*b.y on packed bf16 pairs (v_dot2c_f32_bf16).
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a),
+                                           __builtin_bit_cast(bf16x2_t, b), acc, false);
+}
+
+// 2^x with the bare v_exp_f32 instruction (inputs here are <= 0 or -inf).
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// DPP row rotate: lane i of each 16-lane row reads lane (i - n) mod 16 of its row.
+template <int N>
+__device__ __forceinline__ float row_ror(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 + N, 0xf, 0xf, false));
+}
+
+// Sum over the 16 lanes of a DPP row; every lane of the row receives the total.
+__device__ __forceinline__ float row16_allreduce_sum(float v) {
+    v += row_ror<8>(v);
+    v += row_ror<4>(v);
+    v += row_ror<2>(v);
+    v += row_ror<1>(v);
+    return v;
+}
+
+// Logical-token -> page mapping precomputed on the host (a shift when page_size is a power
+// of two, page 0 when the sequence has a single page).
+struct PageMap {
+    int page_size;
+    int shift;      // log2(page_size) or -1
+    int max_pages;
+};
+
+__host__ __device__ inline PageMap make_page_map(int page_size, int max_pages) {
+    PageMap m;
+    m.page_size = page_size;
+    m.max_pages = max_pages;
+    m.shift = -1;
+    for (int s = 0; s < 31; ++s) {
+        if ((1 << s) == page_size) m.shift = s;
+    }
+    return m;
+}
+
+__device__ __forceinline__ int page_of(const PageMap& pm, int token) {
+    if (pm.shift >= 0) return token >> pm.shift;
+    if (pm.max_pages == 1) return token < pm.page_size ? 0 : 1;
+    return token / pm.page_size;
+}
+
+// Element offset of token `first_token` of kv head `head` (the addressing rule documented at
+// qm_kv_cache), or -1 with a status bit if the page is out of range.
+__device__ __forceinline__ int64_t tile_offset(const qm_kv_cache& c, const PageMap& pm,
+                                               const int32_t* page_table, int first_token,
+                                               int head, uint32_t* status) {
+    const int page = page_of(pm, first_token);
+    if (page >= pm.max_pages) {
+        if (status) atomicOr(status, QM_STATUS_BAD_POSITION);
+        return -1;
+    }
+    const int phys = page_table ? page_table[page] : page;
+    if (phys < 0 || phys >= c.n_pages) {
+        if (status) atomicOr(status, QM_STATUS_BAD_PAGE);
+        return -1;
+    }
+    return static_cast<int64_t>(phys) * c.stride_page + static_cast<int64_t>(head) * c.stride_head
+         + static_cast<int64_t>(first_token - page * pm.page_size) * kDim;
+}
+
+}  // namespace qm

@@ -1,0 +1,68 @@
+"""Shared builders for the parity tests: seeded inputs, paged pools, host<->device copies."""
+import numpy as np
+
+SCALE = 0.08838834764831845
+
+
+def to_dev(a, dev):
+    """numpy uint16/int32/uint32 -> device tensor with the same bits."""
+    import torch
+    if a.dtype == np.uint16:
+        return torch.from_numpy(a.view(np.int16).copy()).to(dev)
+    if a.dtype == np.uint32:
+        return torch.from_numpy(a.view(np.int32).copy()).to(dev)
+    return torch.from_numpy(a.copy()).to(dev)
+
+
+def to_u16(t):
+    return t.detach().cpu().numpy().view(np.uint16)
+
+
+def max_abs_err(oracle, a_bits, b_bits):
+    a = oracle.bf16_to_f32(a_bits).astype(np.float64)
+    b = oracle.bf16_to_f32(b_bits).astype(np.float64)
+    return float(np.max(np.abs(a - b))) if a.size else 0.0
+
+
+def ulp_distance(a_bits, b_bits):
+    """Distance in bf16 ulps between two arrays of finite same-sign-or-not bf16 bit patterns."""
+    def key(x):
+        x = x.astype(np.int32)
+        return np.where(x & 0x8000, 0x8000 - x, x)
+    return np.abs(key(a_bits) - key(b_bits))
+
+
+class PagedPool:
+    """K/V pools in the native [page][kv_head][16][128] layout plus per-stream page tables
+    built from a seeded permutation of the physical pages (numpy side)."""
+
+    def __init__(self, oracle, seq_lens, seed, kv_heads=8, page_size=16, slack_pages=3, fill="normal",
+                 extra_tokens=0):
+        self.kv_heads = kv_heads
+        self.page_size = page_size
+        seq_lens = np.asarray(seq_lens, dtype=np.int32)
+        self.seq_lens = seq_lens
+        pages_per = (seq_lens + extra_tokens + page_size - 1) // page_size
+        self.max_pages = int(max(1, pages_per.max()))
+        total = int(pages_per.sum())
+        self.n_pages = total + slack_pages
+        perm = oracle.permutation(self.n_pages, seed ^ 0x5151)
+        self.page_table = np.full((len(seq_lens), self.max_pages), -1, dtype=np.int32)
+        cur = 0
+        for s, n in enumerate(pages_per):
+            self.page_table[s, :n] = perm[cur:cur + n]
+            cur += n
+        shape = (self.n_pages, kv_heads, page_size, 128)
+        if fill == "normal":
+            self.k = oracle.normal_bf16(shape, seed + 1)
+            self.v = oracle.normal_bf16(shape, seed + 2)
+        else:
+            self.k = np.full(shape, fill, dtype=np.uint16)
+            self.v = np.full(shape, fill, dtype=np.uint16)
+
+    def descriptor(self, oracle):
+        return oracle.paged_cache(self.k, self.v, self.kv_heads, self.page_size)
+
+    def device(self, qm, dev):
+        kd, vd = to_dev(self.k, dev), to_dev(self.v, dev)
+        return kd, vd, qm.paged_cache(kd, vd, self.n_pages, self.kv_heads, self.page_size), to_dev(self.page_table, dev)
