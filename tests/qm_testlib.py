@@ -37,13 +37,13 @@ class PagedPool:
     built from a seeded permutation of the physical pages (numpy side)."""
 
     def __init__(self, oracle, seq_lens, seed, kv_heads=8, page_size=16, slack_pages=3, fill="normal",
-                 extra_tokens=0):
+                 extra_tokens=0, min_table_pages=0):
         self.kv_heads = kv_heads
         self.page_size = page_size
         seq_lens = np.asarray(seq_lens, dtype=np.int32)
         self.seq_lens = seq_lens
         pages_per = (seq_lens + extra_tokens + page_size - 1) // page_size
-        self.max_pages = int(max(1, pages_per.max()))
+        self.max_pages = int(max(1, pages_per.max(), min_table_pages))
         total = int(pages_per.sum())
         self.n_pages = total + slack_pages
         perm = oracle.permutation(self.n_pages, seed ^ 0x5151)

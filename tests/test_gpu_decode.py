@@ -1,0 +1,179 @@
+"""GPU parity: GQA decode attention (single stream, ragged split-K) through the C ABI.
+
+Tolerance (stated by the task): max abs error <= 1e-2 on bf16 outputs against the scalar fp32
+oracle.  The kernel computes the ONLINE policy (reference score roundings, fp32 softmax); it is
+checked against that policy and against the reference chain (bf16(P) included).
+"""
+import numpy as np
+import pytest
+
+from qm_testlib import SCALE, PagedPool, max_abs_err, to_dev, to_u16
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def _workspace(qm, dev, n_streams, q_heads, kv_heads, max_len):
+    import torch
+    nbytes = qm.decode_workspace_bytes(n_streams, q_heads, kv_heads, max_len)
+    ws = torch.empty(max(nbytes, 4) // 4 + 1, dtype=torch.float32, device=dev)
+    return ws, nbytes
+
+
+def _single_flat(oracle, qm, dev, ctx, max_cache, seed, window=-1, q_heads=16, kv_heads=8):
+    import torch
+    q = oracle.normal_bf16((q_heads, 128), seed)
+    kc = oracle.normal_bf16((kv_heads, max_cache, 128), seed + 1)
+    vc = oracle.normal_bf16((kv_heads, max_cache, 128), seed + 2)
+    # slots at and beyond the context hold NaN: they must never be read into the result
+    kc[:, ctx:] = 0x7fc0
+    vc[:, ctx:] = 0x7fc0
+    want = {}
+    for policy in (0, 1):
+        o = np.zeros_like(q)
+        assert oracle.attention(q, oracle.flat_cache(kc, vc, kv_heads, max_cache), None, 1, o, 1, ctx - 1, q_heads,
+                                window, SCALE, policy, 4) == 0
+        want[policy] = o
+    kd, vd = to_dev(kc, dev), to_dev(vc, dev)
+    out = torch.full((q_heads, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    ws, nbytes = _workspace(qm, dev, 1, q_heads, kv_heads, ctx)
+    qm.decode_attention(to_dev(q, dev), qm.flat_cache(kd, vd, kv_heads, max_cache), None, 1, out, q_heads, ctx - 1,
+                        window, SCALE, ws, nbytes)
+    torch.cuda.synchronize()
+    return to_u16(out), want
+
+
+@pytest.mark.parametrize("ctx,max_cache", [(512, 512), (2048, 2052), (1, 8), (2, 19), (15, 16), (16, 16), (17, 40),
+                                           (63, 64), (65, 100), (1000, 1003), (8192, 8206)])
+def test_decode_single_flat(oracle, qm, dev, ctx, max_cache):
+    got, want = _single_flat(oracle, qm, dev, ctx, max_cache, seed=ctx)
+    assert max_abs_err(oracle, got, want[1]) <= TOL
+    if ctx >= 64:
+        assert max_abs_err(oracle, got, want[0]) <= TOL     # reference chain incl. bf16(P)
+    if ctx == 1:
+        assert np.array_equal(got, want[0])                 # out = V[0] exactly
+
+
+@pytest.mark.parametrize("ctx,window", [(100, 7), (100, 16), (100, 33), (2048, 1024), (50, 1), (50, 500)])
+def test_decode_sliding_window(oracle, qm, dev, ctx, window):
+    got, want = _single_flat(oracle, qm, dev, ctx, ctx + 3, seed=ctx + window, window=window)
+    assert max_abs_err(oracle, got, want[1]) <= TOL
+
+
+@pytest.mark.parametrize("q_heads,kv_heads", [(8, 8), (16, 4), (4, 2)])
+def test_decode_other_gqa_groups(oracle, qm, dev, q_heads, kv_heads):
+    got, want = _single_flat(oracle, qm, dev, 300, 304, seed=q_heads, q_heads=q_heads, kv_heads=kv_heads)
+    assert max_abs_err(oracle, got, want[1]) <= TOL
+
+
+def _ragged(oracle, qm, dev, lens, seed, max_len=None):
+    import torch
+    lens = np.asarray(lens, dtype=np.int32)
+    n = len(lens)
+    pool = PagedPool(oracle, lens, seed=seed, min_table_pages=(max_len or 0) // 16)
+    q = oracle.normal_bf16((n, 16, 128), seed + 10)
+    want = {}
+    for policy in (0, 1):
+        o = np.zeros_like(q)
+        assert oracle.decode_attention_ragged(q, pool.descriptor(oracle), pool.page_table, pool.max_pages, lens, o,
+                                              16, SCALE, policy, 8) == 0
+        want[policy] = o
+    kd, vd, cache_d, table_d = pool.device(qm, dev)
+    max_len = int(lens.max()) if max_len is None else max_len
+    ws, nbytes = _workspace(qm, dev, n, 16, 8, max_len)
+    out = torch.full((n, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    sd = torch.zeros(1, dtype=torch.int32, device=dev)
+    qm.decode_attention_ragged(to_dev(q, dev), cache_d, table_d, pool.max_pages, to_dev(lens, dev), n, max_len, out,
+                               16, SCALE, ws, nbytes, sd)
+    torch.cuda.synchronize()
+    return to_u16(out), want, int(sd.item()), pool
+
+
+def test_decode_ragged_config3_shape(oracle, qm, dev):
+    lens = oracle.uniform_int(64, 2024, 256, 4096)
+    got, want, status, _ = _ragged(oracle, qm, dev, lens, seed=77)
+    assert status == 0
+    assert max_abs_err(oracle, got, want[1]) <= TOL
+    assert max_abs_err(oracle, got, want[0]) <= TOL
+
+
+def test_decode_ragged_edge_lengths(oracle, qm, dev):
+    lens = [0, 1, 2, 15, 16, 17, 31, 32, 33, 255, 256, 257, 4096, 0, 5]
+    got, want, status, _ = _ragged(oracle, qm, dev, lens, seed=5)
+    assert status == 0
+    assert max_abs_err(oracle, got, want[1]) <= TOL
+    assert not got[0].any() and not got[13].any()          # empty streams produce zeros
+    # a larger max_seq_len bound changes the split plan, not the result beyond fp32 merge noise
+    got2, _, _, _ = _ragged(oracle, qm, dev, lens, seed=5, max_len=8192)
+    assert max_abs_err(oracle, got2, want[1]) <= TOL
+
+
+def test_decode_ragged_single_split_path(oracle, qm, dev):
+    lens = [0, 3, 16, 40, 1, 0]
+    got, want, status, _ = _ragged(oracle, qm, dev, lens, seed=15)
+    assert status == 0
+    assert max_abs_err(oracle, got, want[1]) <= TOL
+    assert not got[0].any() and not got[5].any()
+
+
+def test_decode_page_permutation_is_bit_identical(oracle, qm, dev):
+    import torch
+    lens = np.array([700, 33, 1500], dtype=np.int32)
+    got, _, _, pool = _ragged(oracle, qm, dev, lens, seed=31)
+    perm = oracle.permutation(pool.n_pages, 123)
+    k_b, v_b = np.zeros_like(pool.k), np.zeros_like(pool.v)
+    k_b[perm], v_b[perm] = pool.k, pool.v
+    table_b = np.where(pool.page_table >= 0, perm[np.maximum(pool.page_table, 0)], -1).astype(np.int32)
+    q = oracle.normal_bf16((3, 16, 128), 31 + 10)
+    kd, vd = to_dev(k_b, dev), to_dev(v_b, dev)
+    ws, nbytes = _workspace(qm, dev, 3, 16, 8, int(lens.max()))
+    out = torch.zeros((3, 16, 128), dtype=torch.int16, device=dev)
+    qm.decode_attention_ragged(to_dev(q, dev), qm.paged_cache(kd, vd, pool.n_pages), to_dev(table_b, dev),
+                               pool.max_pages, to_dev(lens, dev), 3, int(lens.max()), out, 16, SCALE, ws, nbytes)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_u16(out), got)
+
+
+def test_decode_bad_pages_flagged_not_read(oracle, qm, dev):
+    import torch
+    lens = np.array([100, 100], dtype=np.int32)
+    pool = PagedPool(oracle, lens, seed=2)
+    pool.page_table[1, 3] = 10 ** 6                          # far outside the pool
+    kd, vd, cache_d, table_d = pool.device(qm, dev)
+    q = oracle.normal_bf16((2, 16, 128), 3)
+    ws, nbytes = _workspace(qm, dev, 2, 16, 8, 100)
+    out = torch.zeros((2, 16, 128), dtype=torch.int16, device=dev)
+    sd = torch.zeros(1, dtype=torch.int32, device=dev)
+    qm.decode_attention_ragged(to_dev(q, dev), cache_d, table_d, pool.max_pages, to_dev(lens, dev), 2, 100, out, 16,
+                               SCALE, ws, nbytes, sd)
+    torch.cuda.synchronize()
+    assert int(sd.item()) & 1
+    good = np.zeros((16, 128), dtype=np.uint16)
+    oracle.attention(q[0].copy(), pool.descriptor(oracle), pool.page_table[0], pool.max_pages, good, 1, 99, 16, -1,
+                     SCALE, 1, 1)
+    assert max_abs_err(oracle, to_u16(out)[0], good) <= TOL    # the healthy stream is unaffected
+
+
+def test_decode_argument_errors(oracle, qm, dev):
+    import torch
+    kd = torch.zeros((8, 64, 128), dtype=torch.int16, device=dev)
+    vd = torch.zeros_like(kd)
+    q = torch.zeros((16, 128), dtype=torch.int16, device=dev)
+    out = torch.zeros_like(q)
+    cache = qm.flat_cache(kd, vd, 8, 64)
+    with pytest.raises(qm.QmError) as e:
+        qm.decode_attention(q, cache, None, 1, out, 16, 64)           # context beyond capacity
+    assert e.value.code == -3
+    with pytest.raises(qm.QmError) as e:
+        qm.decode_attention(q, cache, None, 1, out, 12, 10)           # 12 q heads over 8 kv heads
+    assert e.value.code == -2
+    with pytest.raises(qm.QmError) as e:
+        qm.decode_attention(q, cache, None, 1, out, 16, -1)
+    assert e.value.code == -5
+    big = torch.zeros((8, 8192, 128), dtype=torch.int16, device=dev)
+    need = qm.decode_workspace_bytes(1, 16, 8, 8192)
+    assert need > 0
+    with pytest.raises(qm.QmError) as e:
+        qm.decode_attention(q, qm.flat_cache(big, big, 8, 8192), None, 1, out, 16, 8191, -1, SCALE, None, 0)
+    assert e.value.code == -4
