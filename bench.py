@@ -1,0 +1,433 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention / KV-cache hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--all]
+
+A step is one pass of the hot path over one batch of synthetic input that is already resident
+in HBM.  The headline workload is the ragged multi-stream decode (64 streams, context lengths
+uniform in [256, 4096], 16-token pages behind a shuffled page table): the one decode
+configuration whose working set (~0.57 GB) exceeds the caches, so that "HBM GB/s" means HBM.
+The other configurations are timed too (`--all`, default on) and reported under `per_config`.
+One JSON line is printed on stdout.
+
+Inputs are drawn on the device by torch's seeded generator; the CPU baseline leg copies the same
+tensors to the host and times the scalar oracle (oracle/, test infrastructure) on them, and also
+checks the GPU result against it.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+SCALE = 0.08838834764831845
+
+
+def _bits(t):
+    """bf16 tensor -> numpy uint16 bit patterns (host)."""
+    import torch
+    return t.detach().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def _time_steps(fn, steps, warmup):
+    """Average milliseconds per call over `steps` back-to-back calls on torch's current stream
+    (the stream handed to the library), bracketed by device synchronisation."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def _time_graph(fn, reps=20, replays=20):
+    """Average milliseconds per step when `reps` steps are captured into one HIP graph and the graph is
+    replayed `replays` times: device-side time without per-launch host overhead (the reference runs its
+    predictor loop as a HIP graph for the same reason, R17:13856-13896)."""
+    import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        for _ in range(reps):
+            fn()
+    graph.replay()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(replays):
+        graph.replay()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / (reps * replays)
+
+
+class RaggedDecode:
+    """configs[2]: 64 streams, L ~ U{256..4096}, paged KV, split-K decode attention."""
+    name = "ragged_decode_64x[256,4096]_paged16"
+    bound = "hbm"
+
+    def __init__(self, qm, dev, seed=2024, n_streams=64, lo=256, hi=4096):
+        import torch
+        g = torch.Generator(device="cpu").manual_seed(seed)
+        self.qm, self.dev, self.n = qm, dev, n_streams
+        self.lens = torch.randint(lo, hi + 1, (n_streams,), generator=g, dtype=torch.int32)
+        pages_per = (self.lens + 15) // 16
+        self.max_pages = int(pages_per.max())
+        self.n_pages = int(pages_per.sum()) + 7
+        perm = torch.randperm(self.n_pages, generator=g, dtype=torch.int32)
+        table = torch.full((n_streams, self.max_pages), -1, dtype=torch.int32)
+        cur = 0
+        for s in range(n_streams):
+            k = int(pages_per[s])
+            table[s, :k] = perm[cur:cur + k]
+            cur += k
+        gd = torch.Generator(device=dev).manual_seed(seed + 1)
+        shape = (self.n_pages, 8, 16, 128)
+        self.k = torch.randn(shape, generator=gd, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        self.v = torch.randn(shape, generator=gd, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        self.q = torch.randn((n_streams, 16, 128), generator=gd, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        self.out = torch.zeros_like(self.q)
+        self.table = table.to(dev)
+        self.lens_d = self.lens.to(dev)
+        self.max_len = int(self.lens.max())
+        self.ws_bytes = qm.decode_workspace_bytes(n_streams, 16, 8, self.max_len)
+        self.ws = torch.empty(self.ws_bytes // 4 + 1, dtype=torch.float32, device=dev)
+        self.status = torch.zeros(1, dtype=torch.int32, device=dev)
+        self.cache = qm.paged_cache(self.k, self.v, self.n_pages)
+        total = int(self.lens.sum())
+        # K+V of every context token, q + out, page table entries actually used
+        self.bytes = 4096 * total + n_streams * 8192 + 4 * int(pages_per.sum())
+        self.flops = 8192 * total
+        self.tokens = total
+
+    def step(self):
+        import torch
+        self.qm.decode_attention_ragged(self.q, self.cache, self.table, self.max_pages, self.lens_d, self.n,
+                                        self.max_len, self.out, 16, SCALE, self.ws, self.ws_bytes, self.status,
+                                        torch.cuda.current_stream().cuda_stream)
+
+    def cpu_baseline(self, oracle, threads):
+        k, v, q = _bits(self.k), _bits(self.v), _bits(self.q)
+        table = self.table.cpu().numpy()
+        lens = self.lens.numpy()
+        cache = oracle.paged_cache(k, v)
+        out = np.zeros_like(q)
+        res = {}
+        for label, th in (("single", 1), ("all", threads)):
+            t0 = time.perf_counter()
+            rc = oracle.decode_attention_ragged(q, cache, table, self.max_pages, lens, out, 16, SCALE,
+                                                oracle.POLICY_ONLINE, th)
+            res[label] = time.perf_counter() - t0
+            assert rc == 0
+        err = float(np.max(np.abs(oracle.bf16_to_f32(out).astype(np.float64)
+                                  - oracle.bf16_to_f32(_bits(self.out)).astype(np.float64))))
+        return res, err, "whole workload (all 64 streams)"
+
+
+class SingleDecode:
+    """configs[0] / configs[1]: batch-1 decode over a flat [8][max_cache][128] cache; configs[1]
+    also runs the fused norm + RoPE + append at the last position first."""
+    bound = "hbm"
+
+    def __init__(self, qm, dev, ctx, fused_append, seed, copies=1):
+        import torch
+        self.qm, self.dev, self.ctx, self.fused = qm, dev, ctx, fused_append
+        self.name = ("talker_fused_step_ctx%d" if fused_append else "gqa_decode_ctx%d") % ctx
+        gd = torch.Generator(device=dev).manual_seed(seed)
+        self.max_cache = ctx + 4
+        self.copies = copies
+
+        def rnd(shape, std=1.0, mean=0.0):
+            return (torch.randn(shape, generator=gd, device=dev, dtype=torch.float32) * std + mean).to(torch.bfloat16)
+
+        self.k = [rnd((8, self.max_cache, 128)) for _ in range(copies)]
+        self.v = [rnd((8, self.max_cache, 128)) for _ in range(copies)]
+        self.caches = [qm.flat_cache(k, v, 8, self.max_cache) for k, v in zip(self.k, self.v)]
+        self.q = rnd((16, 128))
+        self.out = torch.zeros_like(self.q)
+        if fused_append:
+            # hidden 2048 -> Q [16,128], K/V [8,128] with N(0, 0.02) hidden and weights: the
+            # projection is outside the judged region and done once here with torch.
+            hidden = rnd((2048,), 0.02).float()
+            wq, wk, wv = rnd((2048, 2048), 0.02).float(), rnd((1024, 2048), 0.02).float(), rnd((1024, 2048), 0.02).float()
+            self.q_lin = (wq @ hidden).to(torch.bfloat16).view(16, 128).contiguous()
+            self.k_lin = (wk @ hidden).to(torch.bfloat16).view(8, 128).contiguous()
+            self.v_lin = (wv @ hidden).to(torch.bfloat16).view(8, 128).contiguous()
+            self.gq, self.gk = rnd((128,), 0.1, 1.0), rnd((128,), 0.1, 1.0)
+            pos = ctx - 1
+            inv = 1.0e6 ** (-2.0 * np.arange(64, dtype=np.float64) / 128.0)
+            ang = np.concatenate([pos * inv, pos * inv])
+            self.cos = torch.tensor(np.cos(ang), dtype=torch.float32).to(torch.bfloat16).to(dev)
+            self.sin = torch.tensor(np.sin(ang), dtype=torch.float32).to(torch.bfloat16).to(dev)
+        self.ws_bytes = qm.decode_workspace_bytes(1, 16, 8, ctx)
+        self.ws = torch.empty(self.ws_bytes // 4 + 1, dtype=torch.float32, device=dev)
+        self.bytes = 2 * 8 * ctx * 128 * 2 + 4096 + 4096
+        if fused_append:
+            self.bytes = 2 * 8 * ctx * 128 * 2 + 4096 + 8192 + 1024 + 4096
+        self.flops = 16 * ctx * 128 * 2 * 2
+        self.i = 0
+
+    def step(self):
+        import torch
+        s = torch.cuda.current_stream().cuda_stream
+        c = self.caches[self.i % self.copies]
+        self.i += 1
+        q = self.q
+        if self.fused:
+            self.qm.qk_norm_rope_kv_append(self.q_lin, self.k_lin, self.v_lin, self.gq, self.gk, self.cos, self.sin,
+                                           self.q, c, None, 1, 16, self.ctx - 1, 1e-6, s)
+        self.qm.decode_attention(q, c, None, 1, self.out, 16, self.ctx - 1, -1, SCALE, self.ws, self.ws_bytes, s)
+
+    def cpu_baseline(self, oracle, threads):
+        self.i = 0
+        self.step()
+        import torch
+        torch.cuda.synchronize()
+        k, v = _bits(self.k[0]).copy(), _bits(self.v[0]).copy()
+        cache = oracle.flat_cache(k, v, 8, self.max_cache)
+        q = _bits(self.q).copy()
+        out = np.zeros_like(q)
+        res = {}
+        for label, th in (("single", 1), ("all", threads)):
+            t0 = time.perf_counter()
+            if self.fused:
+                rc = oracle.qk_norm_rope_kv_append(_bits(self.q_lin), _bits(self.k_lin), _bits(self.v_lin),
+                                                   _bits(self.gq), _bits(self.gk), _bits(self.cos), _bits(self.sin),
+                                                   q, cache, None, 1, 16, self.ctx - 1)
+                assert rc == 0
+            rc = oracle.attention(q, cache, None, 1, out, 1, self.ctx - 1, 16, -1, SCALE, oracle.POLICY_ONLINE, th)
+            res[label] = time.perf_counter() - t0
+            assert rc == 0
+        err = float(np.max(np.abs(oracle.bf16_to_f32(out).astype(np.float64)
+                                  - oracle.bf16_to_f32(_bits(self.out)).astype(np.float64))))
+        return res, err, "whole workload"
+
+
+class Prefill:
+    """configs[3]: causal GQA prefill, batch 4 x seq 1024, K/V also written to shuffled 16-token pages."""
+    name = "causal_prefill_b4_s1024_paged16"
+    bound = "mfma"
+
+    def __init__(self, qm, dev, seed=44, batch=4, seq=1024):
+        import torch
+        self.qm, self.batch, self.seq = qm, batch, seq
+        gd = torch.Generator(device=dev).manual_seed(seed)
+        g = torch.Generator(device="cpu").manual_seed(seed)
+
+        def rnd(shape):
+            return torch.randn(shape, generator=gd, device=dev, dtype=torch.float32).to(torch.bfloat16)
+
+        self.q, self.k, self.v = rnd((batch, seq, 16, 128)), rnd((batch, seq, 8, 128)), rnd((batch, seq, 8, 128))
+        self.out = torch.zeros_like(self.q)
+        per = (seq + 15) // 16
+        self.max_pages = per
+        self.n_pages = batch * per + 5
+        perm = torch.randperm(self.n_pages, generator=g, dtype=torch.int32)
+        self.table = perm[:batch * per].view(batch, per).contiguous().to(dev)
+        self.kp = torch.zeros((self.n_pages, 8, 16, 128), dtype=torch.bfloat16, device=dev)
+        self.vp = torch.zeros_like(self.kp)
+        self.cache = qm.paged_cache(self.kp, self.vp, self.n_pages)
+        self.status = torch.zeros(1, dtype=torch.int32, device=dev)
+        self.flops = batch * 16 * (seq * (seq + 1) // 2) * 128 * 2 * 2
+        qo = batch * seq * 16 * 128 * 2
+        kv = batch * seq * 8 * 128 * 2
+        self.bytes = 2 * qo + 2 * kv + 2 * kv      # Q + O, K + V read, K + V written to pages
+
+    def step(self):
+        import torch
+        self.qm.prefill_attention_causal(self.q, self.k, self.v, self.out, self.cache, self.table, self.max_pages,
+                                         self.batch, self.seq, 16, 8, SCALE, self.status,
+                                         torch.cuda.current_stream().cuda_stream)
+
+    def cpu_baseline(self, oracle, threads):
+        """Sample: batch entry 0 (a quarter of the flops)."""
+        q, k, v = _bits(self.q[:1]).copy(), _bits(self.k[:1]).copy(), _bits(self.v[:1]).copy()
+        out = np.zeros_like(q)
+        t0 = time.perf_counter()
+        rc = oracle.prefill_attention_causal(q, k, v, out, None, None, 0, 1, self.seq, 16, 8, SCALE,
+                                             oracle.POLICY_ONLINE, threads)
+        dt = time.perf_counter() - t0
+        assert rc == 0
+        err = float(np.max(np.abs(oracle.bf16_to_f32(out).astype(np.float64)
+                                  - oracle.bf16_to_f32(_bits(self.out[:1])).astype(np.float64))))
+        return {"all": dt * self.batch}, err, "batch entry 0 of %d, time scaled by %d" % (self.batch, self.batch)
+
+
+class PredictorLoop:
+    """configs[4]: 256 frames x 5 layers, 16 steps each (context 1 -> 16), one launch."""
+    name = "predictor_loop_256frames_5layers_16steps"
+    bound = "hbm"
+
+    def __init__(self, qm, dev, seed=55, frames=256, layers=5, rows=16, write_cache=False):
+        import torch
+        self.qm, self.units, self.layers, self.rows, self.frames = qm, frames * layers, layers, rows, frames
+        gd = torch.Generator(device=dev).manual_seed(seed)
+
+        def rnd(shape, std=1.0, mean=0.0):
+            return (torch.randn(shape, generator=gd, device=dev, dtype=torch.float32) * std + mean).to(torch.bfloat16)
+
+        u = self.units
+        self.q, self.k, self.v = rnd((u, rows, 16, 128)), rnd((u, rows, 8, 128)), rnd((u, rows, 8, 128))
+        self.gq, self.gk = rnd((layers, 128), 0.1, 1.0), rnd((layers, 128), 0.1, 1.0)
+        inv = 1.0e6 ** (-2.0 * np.arange(64, dtype=np.float64) / 128.0)
+        ang = np.arange(rows, dtype=np.float64)[:, None] * np.concatenate([inv, inv])[None, :]
+        self.cos = torch.tensor(np.cos(ang), dtype=torch.float32).to(torch.bfloat16).to(dev)
+        self.sin = torch.tensor(np.sin(ang), dtype=torch.float32).to(torch.bfloat16).to(dev)
+        self.out = torch.zeros_like(self.q)
+        self.kc = torch.zeros((u, 8, 16, 128), dtype=torch.bfloat16, device=dev) if write_cache else None
+        self.vc = torch.zeros((u, 8, 16, 128), dtype=torch.bfloat16, device=dev) if write_cache else None
+        per_unit = 3 * 65536 + (65536 if write_cache else 0)
+        self.bytes = per_unit * u
+        self.flops = 1114112 * u
+        if write_cache:
+            self.name += "_cache_writeback"
+
+    def step(self):
+        import torch
+        self.qm.predictor_attention_loop(self.q, self.k, self.v, self.gq, self.gk, self.cos, self.sin, self.out,
+                                         self.kc, self.vc, self.units, self.layers, self.rows, 1, 1e-6,
+                                         torch.cuda.current_stream().cuda_stream)
+
+    def cpu_baseline(self, oracle, threads):
+        """Sample: the first 160 units (32 frames)."""
+        n = min(160, self.units)
+        q, k, v = _bits(self.q[:n]).copy(), _bits(self.k[:n]).copy(), _bits(self.v[:n]).copy()
+        out = np.zeros_like(q)
+        t0 = time.perf_counter()
+        rc = oracle.predictor_attention_loop(q, k, v, _bits(self.gq), _bits(self.gk), _bits(self.cos), _bits(self.sin),
+                                             out, None, None, n, self.layers, self.rows, 1, 1e-6, threads)
+        dt = time.perf_counter() - t0
+        assert rc == 0
+        err = float(np.max(np.abs(oracle.bf16_to_f32(out).astype(np.float64)
+                                  - oracle.bf16_to_f32(_bits(self.out[:n])).astype(np.float64))))
+        return {"all": dt * self.units / n}, err, "first %d of %d units, time scaled" % (n, self.units)
+
+
+def _report(w, ms):
+    rep = {"workload": w.name, "us_per_step": ms * 1e3, "algorithmic_bytes": w.bytes, "algorithmic_flops": w.flops,
+           "GBps": w.bytes / (ms * 1e-3) / 1e9, "TFLOPps": w.flops / (ms * 1e-3) / 1e12}
+    rep["frac_hbm_peak"] = rep["GBps"] / HBM_PEAK_GBPS
+    rep["frac_mfma_peak"] = rep["TFLOPps"] / MFMA_BF16_PEAK_TFLOPS
+    return rep
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one MI355X: this path shards without communication (streams / batch / frames), "
+              "and no multi-GPU figure is produced; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (there is no CPU fallback for the product path)", file=sys.stderr)
+        sys.exit(3)
+    qm = importlib.import_module("qingming-qwen3-tts_amd").binding
+    qm.lib()
+    dev = torch.device("cuda:0")
+    props = torch.cuda.get_device_properties(0)
+
+    head = RaggedDecode(qm, dev)
+    ms = _time_steps(head.step, args.steps, args.warmup)
+    torch.cuda.synchronize()
+    if int(head.status.item()) != 0:
+        raise RuntimeError("device status flagged a bad page/position")
+    rep = _report(head, ms)
+
+    per_config = {}
+    oracle = None
+    threads = min(os.cpu_count() or 1, 16)
+    if not args.no_cpu:
+        from oracle import binding as oracle
+        oracle.build()
+    if not args.headline_only:
+        extra = [
+            ("cfg1_decode_ctx512", lambda: SingleDecode(qm, dev, 512, False, 11)),
+            ("cfg2_talker_fused_step_ctx2048", lambda: SingleDecode(qm, dev, 2048, True, 12)),
+            # the same step over 64 distinct KV caches in rotation (0.54 GB): defeats L2 / MALL
+            # residency, as consecutive layers of a real decode step do
+            ("cfg2_talker_fused_step_ctx2048_rotating64", lambda: SingleDecode(qm, dev, 2048, True, 12, copies=64)),
+            ("cfg4_causal_prefill", lambda: Prefill(qm, dev)),
+            ("cfg5_predictor_loop", lambda: PredictorLoop(qm, dev)),
+            ("cfg5_predictor_loop_cache_writeback", lambda: PredictorLoop(qm, dev, write_cache=True)),
+        ]
+        for key, make in extra:
+            w = make()
+            r = _report(w, _time_steps(w.step, max(args.steps, 100), max(args.warmup, 10)))
+            copies = getattr(w, "copies", 1)
+            r["us_per_step_graph"] = _time_graph(w.step, reps=64 if copies > 1 else 20) * 1e3
+            r["GBps_graph"] = w.bytes / (r["us_per_step_graph"] * 1e-6) / 1e9
+            r["TFLOPps_graph"] = w.flops / (r["us_per_step_graph"] * 1e-6) / 1e12
+            r["bound"] = w.bound
+            r["cache_resident"] = copies == 1 and w.bytes < 256e6
+            if isinstance(w, PredictorLoop):
+                r["us_per_predictor_step"] = r["us_per_step_graph"] / w.rows
+                r["us_per_frame"] = r["us_per_step_graph"] / w.frames
+            if oracle is not None and not (isinstance(w, PredictorLoop) and w.kc is not None) and copies == 1:
+                res, err, sample = w.cpu_baseline(oracle, threads)
+                if err > 1e-2:
+                    raise RuntimeError(f"{key}: GPU result differs from the oracle: max abs err {err}")
+                r["cpu_oracle"] = {"seconds": res["all"], "cores": threads, "sample": sample,
+                                   "gpu_vs_oracle_max_abs_err": err,
+                                   "speedup_vs_cpu": res["all"] / (r["us_per_step_graph"] * 1e-6)}
+            per_config[key] = r
+            del w
+            torch.cuda.empty_cache()
+        rep["us_per_step_graph"] = _time_graph(head.step, reps=5, replays=10) * 1e3
+        per_config["cfg3_ragged_decode"] = dict(rep)
+
+    cpu = None
+    if oracle is not None:
+        res, err, sample = head.cpu_baseline(oracle, threads)
+        if err > 1e-2:
+            raise RuntimeError(f"GPU result differs from the oracle: max abs err {err}")
+        cpu = {"value": head.bytes / res["all"] / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+               "sample": sample, "single_thread_value": head.bytes / res["single"] / 1e9,
+               "seconds": res["all"], "seconds_single_thread": res["single"], "gpu_vs_oracle_max_abs_err": err}
+
+    line = {
+        "metric": "decode_attn_hbm_GBps", "value": rep["GBps"], "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16 storage, f32 accumulate", "data": "synthetic",
+        "config": {"workload": head.name, "streams": head.n, "context_tokens_total": head.tokens,
+                   "q_heads": 16, "kv_heads": 8, "head_dim": 128, "page_size": 16,
+                   "device": props.name, "compute_units": props.multi_processor_count},
+        "roofline": {"bound": "hbm", "achieved": rep["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": rep["GBps"] / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "decode_split_kernel<2> (+ decode_merge_kernel<2>, both inside the timed step)",
+                     "algorithmic_bytes_per_launch": head.bytes, "avg_launch_us": ms * 1e3},
+        "cpu_baseline": cpu,
+        "per_config": per_config,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,6 +1,249 @@
-// placeholder until the loop kernel lands
+// qm_predictor.hip — the code predictor's whole per-frame attention loop in one launch (gfx950).
+//
+// One block owns one (unit, kv head), unit = (frame, layer): it stages the unit's 16 rows of
+// Q (two heads), K and V in LDS (16 KiB), applies QK-RMSNorm + RoPE in place, then evaluates
+// the 16 causal steps (row r attends keys 0..r) and writes the 16 context rows.  K/V never go
+// back to HBM unless the caller asks for the cache.  Launch overhead is paid once for all
+// frames, layers and steps instead of ~150 launches per frame.
+//
+// This operator keeps the reference's complete rounding chain, bf16(P) included, and its fp32
+// summation topology (R17:12386-12418 dot products, 12449-12509 softmax, 12515-12574 P.V), so the
+// result differs from the CPU restatement only where the device expf rounds differently.
+//
+// Algorithmic HBM bytes per (unit, kv head): 8 KiB q + 4 KiB k + 4 KiB v in, 8 KiB context out
+// (+ 8 KiB if the K/V cache is written back) — the loop is bound by HBM bandwidth / latency.
+
+#include "qm_device.h"
 #include "qm_host.h"
+
+namespace qm {
+
+constexpr int kPredRows = 16;     // kMaxCache of the reference (R17:7963)
+constexpr int kPredThreads = 256;
+
+struct PredictorParams {
+    const uint16_t* q;        // [units][rows][16][128]
+    const uint16_t* k;        // [units][rows][8][128]
+    const uint16_t* v;        // [units][rows][8][128]
+    const uint16_t* q_norm_w; // [n_layers][128]
+    const uint16_t* k_norm_w; // [n_layers][128]
+    const uint16_t* cos_rows; // [rows][128]
+    const uint16_t* sin_rows; // [rows][128]
+    uint16_t* out;            // [units][rows][16][128]
+    uint16_t* k_cache_out;    // [units][8][16][128] or NULL
+    uint16_t* v_cache_out;    // [units][8][16][128] or NULL
+    int64_t unit_base;        // index of the first unit of this launch (layer = unit % n_layers)
+    int n_layers;
+    int rows;
+    float epsilon;
+};
+
+// Sum of squares in the reference order for a head held as (x0 = dim lane, x1 = dim lane+64).
+__device__ __forceinline__ float pred_sum_squares(float x0, float x1) {
+    float s0 = x0 * x0;
+    float s1 = x1 * x1;
+#pragma unroll
+    for (int offset = 16; offset > 0; offset >>= 1) {
+        s0 += __shfl_down(s0, offset, 32);
+        s1 += __shfl_down(s1, offset, 32);
+    }
+    const float t = s0 + s1;
+    return __shfl(t, 0) + __shfl(t, 32);
+}
+
+// In-place RMSNorm + RoPE of one 128-wide head in LDS by one wave (same chain as
+// norm_rope_head in qm_norm_rope.hip; R17:12178-12279).
+__device__ __forceinline__ void pred_norm_rope(uint16_t* head, const uint16_t* __restrict__ gamma,
+                                               const uint16_t* __restrict__ cosv,
+                                               const uint16_t* __restrict__ sinv, float epsilon, int lane) {
+    float w0 = bf2f(head[lane]);
+    float w1 = bf2f(head[lane + 64]);
+    const float sum = pred_sum_squares(w0, w1);
+    const float r = 1.0f / sqrtf(sum / 128.0f + epsilon);
+    w0 = bf2f(f2bf(bf2f(f2bf(w0 * r)) * bf2f(gamma[lane])));
+    w1 = bf2f(f2bf(bf2f(f2bf(w1 * r)) * bf2f(gamma[lane + 64])));
+    const float first0 = bf2f(f2bf(w0 * bf2f(cosv[lane])));
+    const float second0 = bf2f(f2bf((-w1) * bf2f(sinv[lane])));
+    const float first1 = bf2f(f2bf(w1 * bf2f(cosv[lane + 64])));
+    const float second1 = bf2f(f2bf(w0 * bf2f(sinv[lane + 64])));
+    head[lane] = f2bf(first0 + second0);
+    head[lane + 64] = f2bf(first1 + second1);
+}
+
+// Fixed reduction tree of the reference's 32-lane shuffle sum restricted to its first 16 leaves
+// (the other 16 are exact zeros): ((x0+x8)+(x4+x12)) + ((x2+x10)+(x6+x14)) + ... as the
+// shfl_down(8), (4), (2), (1) levels produce it.
+__device__ __forceinline__ float tree16(const float* x) {
+    float b[8], c[4], d[2];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) b[i] = x[i] + x[i + 8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) c[i] = b[i] + b[i + 4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) d[i] = c[i] + c[i + 2];
+    return d[0] + d[1];
+}
+
+__global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorParams prm) {
+    __shared__ __attribute__((aligned(16))) uint16_t sh_q[2][kPredRows][kDim];   // [g][row][d]
+    __shared__ __attribute__((aligned(16))) uint16_t sh_k[kPredRows][kDim];
+    __shared__ __attribute__((aligned(16))) uint16_t sh_v[kPredRows][kDim];
+    __shared__ float sh_s[2][kPredRows][kPredRows];                                // scores, then P
+
+    const int kvh = blockIdx.x;
+    const int64_t unit = blockIdx.y;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int rows = prm.rows;
+    const int layer = static_cast<int>((prm.unit_base + unit) % prm.n_layers);
+
+    // ---- stage q (2 heads), k, v of this kv head: 16-byte chunks --------------------------------
+    // q: rows x 2 heads x 16 chunks; k, v: rows x 16 chunks each.
+    for (int c = tid; c < rows * 64; c += kPredThreads) {
+        const int chunk = c & 15;
+        const int which = (c >> 4) & 3;     // 0,1: q head g; 2: k; 3: v
+        const int row = c >> 6;
+        const int64_t r64 = unit * rows + row;
+        if (which < 2) {
+            const uint4 val = *reinterpret_cast<const uint4*>(
+                prm.q + ((r64 * 16 + kvh * 2 + which) * kDim) + chunk * 8);
+            *reinterpret_cast<uint4*>(&sh_q[which][row][chunk * 8]) = val;
+        } else {
+            const uint16_t* src = which == 2 ? prm.k : prm.v;
+            const uint4 val = *reinterpret_cast<const uint4*>(src + ((r64 * 8 + kvh) * kDim) + chunk * 8);
+            *reinterpret_cast<uint4*>(which == 2 ? &sh_k[row][chunk * 8] : &sh_v[row][chunk * 8]) = val;
+        }
+    }
+    __syncthreads();
+
+    // ---- QK-RMSNorm + RoPE in place: 3*rows heads, one wave each ------------------------------------
+    for (int h = wave; h < 3 * rows; h += 4) {
+        const int row = h / 3;
+        const int which = h % 3;            // 0,1: q head g; 2: k
+        uint16_t* head = which < 2 ? sh_q[which][row] : sh_k[row];
+        const uint16_t* gamma = (which < 2 ? prm.q_norm_w : prm.k_norm_w) + layer * kDim;
+        pred_norm_rope(head, gamma, prm.cos_rows + row * kDim, prm.sin_rows + row * kDim, prm.epsilon, lane);
+    }
+    __syncthreads();
+
+    // ---- optional K/V cache write-back, layout [unit][kv head][16][128] (R17:10711-10737) ---------
+    if (prm.k_cache_out) {
+        for (int c = tid; c < kPredRows * 16; c += kPredThreads) {
+            const int row = c >> 4, chunk = c & 15;
+            const int64_t dst = ((unit * 8 + kvh) * kPredRows + row) * kDim + chunk * 8;
+            uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
+            if (row < rows) {
+                kv = *reinterpret_cast<const uint4*>(&sh_k[row][chunk * 8]);
+                vv = *reinterpret_cast<const uint4*>(&sh_v[row][chunk * 8]);
+            }
+            *reinterpret_cast<uint4*>(prm.k_cache_out + dst) = kv;
+            if (prm.v_cache_out) *reinterpret_cast<uint4*>(prm.v_cache_out + dst) = vv;
+        }
+    }
+
+    // ---- scores: one 32-lane half wave per (g, row, key), reference order of operations ------------
+    {
+        const int half = lane >> 5;
+        const int l = lane & 31;
+        const float scale = __uint_as_float(0x3db504f3U);   // kAttentionScaleBits, R17:9354-9356
+        for (int idx = wave * 2 + half; idx < 2 * rows * kPredRows; idx += 8) {
+            const int key = idx & 15;
+            const int row = (idx >> 4) % rows;
+            const int g = (idx >> 4) / rows;
+            if (key > row) continue;                          // uniform per half wave
+            const uint16_t* qh = sh_q[g][row];
+            const uint16_t* kh = sh_k[key];
+            float acc = 0.0f;
+#pragma unroll
+            for (int d = 0; d < kDim; d += 32) acc = fmaf(bf2f(qh[l + d]), bf2f(kh[l + d]), acc);
+#pragma unroll
+            for (int offset = 16; offset > 0; offset >>= 1) acc += __shfl_down(acc, offset, 32);
+            if (l == 0) {
+                const float raw = bf2f(f2bf(acc));
+                sh_s[g][row][key] = bf2f(f2bf(raw * scale));
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- softmax rows: thread t < 2*rows owns row (g, r); probabilities rounded to bf16 --------------
+    if (tid < 2 * rows) {
+        const int g = tid / rows, r = tid % rows;
+        float* s = sh_s[g][r];
+        float maximum = -INFINITY;
+        for (int j = 0; j <= r; ++j) maximum = maximum > s[j] ? maximum : s[j];
+        float e[kPredRows];
+#pragma unroll
+        for (int j = 0; j < kPredRows; ++j) e[j] = j <= r ? expf(s[j] - maximum) : 0.0f;
+        const float total = tree16(e);
+#pragma unroll
+        for (int j = 0; j < kPredRows; ++j) s[j] = j <= r ? bf2f(f2bf(e[j] / total)) : 0.0f;
+    }
+    __syncthreads();
+
+    // ---- P.V: thread (g, d) owns one output column for all rows -------------------------------------
+    {
+        const int g = tid >> 7;
+        const int d = tid & 127;
+        float vcol[kPredRows];
+#pragma unroll
+        for (int j = 0; j < kPredRows; ++j) vcol[j] = j < rows ? bf2f(sh_v[j][d]) : 0.0f;
+        for (int r = 0; r < rows; ++r) {
+            float x[kPredRows];
+#pragma unroll
+            for (int j = 0; j < kPredRows; ++j) x[j] = j <= r ? fmaf(sh_s[g][r][j], vcol[j], 0.0f) : 0.0f;
+            const float o = tree16(x);
+            prm.out[((unit * rows + r) * 16 + kvh * 2 + g) * kDim + d] = f2bf(o);
+        }
+    }
+}
+
+}  // namespace qm
+
 extern "C" int32_t qm_predictor_attention_loop(
-    const uint16_t*, const uint16_t*, const uint16_t*, const uint16_t*, const uint16_t*, const uint16_t*,
-    const uint16_t*, uint16_t*, uint16_t*, uint16_t*, int32_t, int32_t, int32_t, int32_t, float, void*) {
-    return QM_ERR_ARGUMENT; }
+    const uint16_t* q, const uint16_t* k, const uint16_t* v,
+    const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+    const uint16_t* cos_rows, const uint16_t* sin_rows,
+    uint16_t* context_out, uint16_t* k_cache_out, uint16_t* v_cache_out,
+    int32_t units, int32_t n_layers, int32_t rows, int32_t first_rows,
+    float epsilon, void* hip_stream) {
+    if (!q || !k || !v || !q_norm_w || !k_norm_w || !cos_rows || !sin_rows || !context_out)
+        return QM_ERR_NULL;
+    if (units < 0 || units > 65535 * 64 || n_layers <= 0 || rows < 1 || rows > qm::kPredRows)
+        return QM_ERR_ARGUMENT;
+    // first_rows = 2 is the reference's two-row causal step 0 (R17:13593-13596); it renumbers
+    // the steps but row r still attends keys 0..r, so both values run the same kernel.
+    if ((first_rows != 1 && first_rows != 2) || first_rows > rows) return QM_ERR_ARGUMENT;
+    if (v_cache_out && !k_cache_out) return QM_ERR_ARGUMENT;
+    const uintptr_t align = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k)
+                          | reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(k_cache_out)
+                          | reinterpret_cast<uintptr_t>(v_cache_out);
+    if (align & 15) return QM_ERR_GEOMETRY;
+    if (units == 0) return QM_OK;
+    qm::PredictorParams prm;
+    prm.q = q; prm.k = k; prm.v = v;
+    prm.q_norm_w = q_norm_w; prm.k_norm_w = k_norm_w;
+    prm.cos_rows = cos_rows; prm.sin_rows = sin_rows;
+    prm.out = context_out; prm.k_cache_out = k_cache_out; prm.v_cache_out = v_cache_out;
+    prm.unit_base = 0; prm.n_layers = n_layers; prm.rows = rows; prm.epsilon = epsilon;
+    // grid.y is limited to 65535: fold large unit counts into several launches.
+    const int32_t per_launch = 65535;
+    for (int32_t first = 0; first < units; first += per_launch) {
+        const int32_t n = units - first < per_launch ? units - first : per_launch;
+        qm::PredictorParams p = prm;
+        const int64_t row0 = static_cast<int64_t>(first) * rows;
+        p.q = q + row0 * 16 * qm::kDim;
+        p.k = k + row0 * 8 * qm::kDim;
+        p.v = v + row0 * 8 * qm::kDim;
+        p.out = context_out + row0 * 16 * qm::kDim;
+        if (k_cache_out) p.k_cache_out = k_cache_out + static_cast<int64_t>(first) * 8 * 16 * qm::kDim;
+        if (v_cache_out) p.v_cache_out = v_cache_out + static_cast<int64_t>(first) * 8 * 16 * qm::kDim;
+        p.unit_base = first;
+        hipLaunchKernelGGL(qm::predictor_loop_kernel, dim3(8, n), dim3(qm::kPredThreads), 0,
+                           static_cast<hipStream_t>(hip_stream), p);
+        const int32_t rc = qm::launch_status();
+        if (rc != QM_OK) return rc;
+    }
+    return QM_OK;
+}

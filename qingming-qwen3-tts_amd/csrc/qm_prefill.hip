@@ -1,5 +1,368 @@
-// placeholder until the MFMA kernel lands
+// qm_prefill.hip — causal GQA prefill attention on gfx950 bf16 MFMA, fused with the paged K/V write.
+//
+// Tiling.  A block of four waves owns 64 query rows of one (batch, kv head) and both query heads
+// of the GQA pair: a wave's MFMA column dimension is 32 = 16 rows x 2 heads, so every K and V
+// fragment read from LDS feeds both heads.  Keys are streamed in tiles of 64 through two LDS
+// buffers (global loads for tile i+1 are in flight while tile i is multiplied).  The wave
+// computes S^T = K Q^T with v_mfma_f32_32x32x16_bf16 (keys on MFMA rows, query columns on lanes),
+// so that the softmax statistics of a query column live in one lane pair, and the accumulator
+// layout of S^T is directly the B-operand layout of O^T += V^T P^T.  V is transposed on its way
+// into LDS ([dim][key slot], key slots permuted to match the accumulator layout).
+//
+// Scheduling.  Blocks are numbered heaviest query tile first, so that the causal triangle packs
+// onto 256 CUs (two blocks per CU) without a long tail; blocks that share K/V differ by a
+// multiple of batch*kv_heads and therefore land on the same XCD and hit its L2.
+//
+// Rounding.  Scores are rounded to bf16 before and after scaling like the reference
+// (R17:15879-15890); softmax runs online in fp32; P enters the P.V MFMA as bf16 — except in the
+// first query tile, whose rows have so few keys that outputs are large: there P is split into
+// hi + lo bf16 parts (two MFMAs) to stay inside the 1e-2 output tolerance.
+//
+// Causality.  A key after a query row never contributes; keys of later 16-row groups are not
+// read into the product at all.  Inside a wave's own 16-row diagonal group the mask is P = 0
+// times V, so a non-finite V of a later row of the same group would propagate (the reference
+// skips those keys; finite values, the only ones a prefill produces, behave identically).
+//
+// Algorithmic work per (batch, kv head): flops = 2 heads * 2 matmuls * 2 * 128 * S(S+1)/2;
+// HBM bytes = Q + O (2 heads) + K + V read once + K + V written to pages.  Bound: MFMA (with the
+// softmax VALU work — 16 exponentials per lane per 32 keys — as the practical limiter).
+
+#include "qm_device.h"
 #include "qm_host.h"
+
+namespace qm {
+
+constexpr int kPfThreads = 256;
+constexpr int kBM = 64;          // query rows per block
+constexpr int kBN = 64;          // keys per tile
+constexpr int kKS = kDim + 8;    // LDS row stride of the K tile (elements)
+constexpr int kVS = kBN + 8;     // LDS row stride of the V^T tile (elements)
+constexpr int kOS = kDim + 8;    // LDS row stride of the output staging tile
+
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+struct PrefillParams {
+    const uint16_t* q;     // [batch][seq][2*kv_heads][128]
+    const uint16_t* k;     // [batch][seq][kv_heads][128]
+    const uint16_t* v;
+    uint16_t* out;         // [batch][seq][2*kv_heads][128]
+    const int32_t* page_table;   // [batch][max_pages] or NULL
+    uint32_t* status;
+    PageMap pages;
+    int has_cache;
+    int batch;
+    int seq;
+    int kv_heads;
+    int n_qtiles;
+    float scale;
+};
+
+struct PfShared {
+    uint16_t k[2][kBN * kKS];
+    uint16_t vt[2][kDim * kVS];
+};
+
+// LDS slot of key j (0..15) inside a 16-key group: MFMA k index 8*g + e holds the key that the
+// S^T accumulator register e of lane group g belongs to.
+__device__ __forceinline__ int key_slot(int j) {
+    return 8 * ((j & 7) >> 2) + 4 * (j >> 3) + (j & 3);
+}
+
+__device__ __forceinline__ bf16x8_t lds_frag(const uint16_t* p) {
+    return *reinterpret_cast<const bf16x8_t*>(p);
+}
+
+template <bool PRECISE>
+__device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_kv_cache& cache,
+                                             unsigned char* pf_smem, int qt, int pair) {
+    PfShared& sh = *reinterpret_cast<PfShared*>(pf_smem);
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int col = lane & 31;       // MFMA column = (query row % 16, head)
+    const int grp = lane >> 5;       // MFMA k / row group
+
+    const int b = pair / prm.kv_heads;
+    const int kvh = pair % prm.kv_heads;
+    const int S = prm.seq;
+    const int q_heads = 2 * prm.kv_heads;
+
+    const int q0 = qt * kBM;
+    const int my_row = q0 + 16 * wave + (col & 15);   // query row of this lane's column
+    const int my_head = 2 * kvh + (col >> 4);
+
+    // ---- Q fragments (B operand): dims 16*kb + 8*grp .. +7 of this lane's column ----------------
+    bf16x8_t qf[8];
+    {
+        const uint16_t* qp = prm.q + ((static_cast<int64_t>(b) * S + my_row) * q_heads + my_head) * kDim + 8 * grp;
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb) {
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (my_row < S) raw = *reinterpret_cast<const uint4*>(qp + 16 * kb);
+            qf[kb] = __builtin_bit_cast(bf16x8_t, raw);
+        }
+    }
+
+    f32x16_t o[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[dt][r] = 0.0f;
+    float m_run = -INFINITY;
+    float l_run = 0.0f;
+
+    const int64_t kv_base = static_cast<int64_t>(b) * S * prm.kv_heads * kDim + static_cast<int64_t>(kvh) * kDim;
+    const int64_t kv_row = static_cast<int64_t>(prm.kv_heads) * kDim;
+    const int32_t* table = prm.page_table ? prm.page_table + static_cast<int64_t>(b) * prm.pages.max_pages : nullptr;
+
+    // Global -> register staging of one K/V tile.  K: chunk c = tid + 256*i -> key c/16, dims
+    // 8*(c%16).  V: thread (kg = tid/16, dc = tid%16) takes keys 4*kg..4*kg+3, dims 8*dc..+7.
+    uint4 kst[4], vst[4];
+    const int v_kg = tid >> 4, v_dc = tid & 15;
+    auto load_tile = [&](int tile) {
+        const int key0 = tile * kBN;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + kPfThreads * i;
+            const int key = key0 + (c >> 4);
+            kst[i] = make_uint4(0, 0, 0, 0);
+            if (key < S) kst[i] = *reinterpret_cast<const uint4*>(prm.k + kv_base + key * kv_row + 8 * (c & 15));
+            const int vkey = key0 + 4 * v_kg + i;
+            vst[i] = make_uint4(0, 0, 0, 0);
+            if (vkey < S) vst[i] = *reinterpret_cast<const uint4*>(prm.v + kv_base + vkey * kv_row + 8 * v_dc);
+        }
+    };
+    // The block whose query tile equals the key tile also writes those K/V rows to the pages.
+    auto write_pages = [&](int tile) {
+        const int key0 = tile * kBN;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + kPfThreads * i;
+            const int key = key0 + (c >> 4);
+            if (key < S) {
+                const int64_t off = tile_offset(cache, prm.pages, table, key, kvh, prm.status);
+                if (off >= 0) *reinterpret_cast<uint4*>(cache.k_pool + off + 8 * (c & 15)) = kst[i];
+            }
+            const int vkey = key0 + 4 * v_kg + i;
+            if (vkey < S) {
+                const int64_t off = tile_offset(cache, prm.pages, table, vkey, kvh, prm.status);
+                if (off >= 0) *reinterpret_cast<uint4*>(cache.v_pool + off + 8 * v_dc) = vst[i];
+            }
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + kPfThreads * i;
+            *reinterpret_cast<uint4*>(&sh.k[buf][(c >> 4) * kKS + 8 * (c & 15)]) = kst[i];
+        }
+        // transpose 4 keys x 8 dims -> 8 rows of 4 consecutive key slots
+        const int slot0 = 16 * (v_kg >> 2) + key_slot(4 * (v_kg & 3));
+        const uint32_t w[4][4] = {{vst[0].x, vst[0].y, vst[0].z, vst[0].w}, {vst[1].x, vst[1].y, vst[1].z, vst[1].w},
+                                  {vst[2].x, vst[2].y, vst[2].z, vst[2].w}, {vst[3].x, vst[3].y, vst[3].z, vst[3].w}};
+#pragma unroll
+        for (int ee = 0; ee < 8; ++ee) {
+            const int e = (ee + v_dc) & 7;          // rotate to spread LDS banks
+            const int word = e >> 1;
+            uint2 packed;
+            if (e & 1) {
+                packed.x = (w[0][word] >> 16) | (w[1][word] & 0xffff0000U);
+                packed.y = (w[2][word] >> 16) | (w[3][word] & 0xffff0000U);
+            } else {
+                packed.x = (w[0][word] & 0xffffU) | (w[1][word] << 16);
+                packed.y = (w[2][word] & 0xffffU) | (w[3][word] << 16);
+            }
+            *reinterpret_cast<uint2*>(&sh.vt[buf][(8 * v_dc + e) * kVS + slot0]) = packed;
+        }
+    };
+
+    const int n_tiles = qt + 1;
+    load_tile(0);
+    if (prm.has_cache && qt == 0) write_pages(0);   // (qt is 0 only on the split-precision path)
+    store_tile(0);
+    __syncthreads();
+
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        const int buf = tile & 1;
+        const bool more = tile + 1 < n_tiles;
+        if (more) {
+            load_tile(tile + 1);
+            if (prm.has_cache && tile + 1 == qt) write_pages(tile + 1);
+        }
+        const bool diagonal = tile == qt;
+
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int key_base = tile * kBN + 32 * half;
+            // On the diagonal a wave whose last row precedes this half has nothing to do there.
+            if (diagonal && key_base > q0 + 16 * wave + 15) continue;
+
+            // ---- S^T = K Q^T : rows = 32 keys, cols = 32 (row, head) columns ----------------------
+            f32x16_t s;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+            const uint16_t* kp = &sh.k[buf][(32 * half + col) * kKS + 8 * grp];
+#pragma unroll
+            for (int kb = 0; kb < 8; ++kb) {
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(kp + 16 * kb), qf[kb], s, 0, 0, 0);
+            }
+
+            // ---- reference score roundings, causal mask, online softmax ---------------------------
+            float mx = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float x = round_bf16(round_bf16(s[r]) * prm.scale);
+                if (diagonal) {
+                    const int key = key_base + 8 * (r >> 2) + 4 * grp + (r & 3);
+                    if (key > my_row) x = -INFINITY;
+                }
+                s[r] = x;
+                mx = fmaxf(mx, x);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_run, mx);
+            const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
+            if (__builtin_amdgcn_ballot_w64(m_new > m_run)) {
+                const float alpha = fast_exp2((m_run - m_ref) * kLog2e);
+                l_run *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+            }
+            m_run = m_new;
+            const float m_scaled = m_ref * kLog2e;
+            float psum = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                s[r] = fast_exp2(fmaf(s[r], kLog2e, -m_scaled));
+                psum += s[r];
+            }
+            l_run += psum;
+
+            // ---- O^T += V^T P^T : two 16-key groups x four 32-dim tiles ---------------------------
+#pragma unroll
+            for (int kg = 0; kg < 2; ++kg) {
+                // A 16-key group that lies wholly after the wave's last row is masked for every
+                // column: skip it, so that later tokens are not even multiplied by zero.
+                if (diagonal && key_base + 16 * kg > q0 + 16 * wave + 15) continue;
+                bf16x8_t phi, plo;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float pv = s[8 * kg + e];
+                    phi[e] = static_cast<__bf16>(pv);
+                    if (PRECISE) plo[e] = static_cast<__bf16>(pv - static_cast<float>(phi[e]));
+                }
+                const uint16_t* vp = &sh.vt[buf][col * kVS + 32 * half + 16 * kg + 8 * grp];
+#pragma unroll
+                for (int dt = 0; dt < 4; ++dt) {
+                    const bf16x8_t vf = lds_frag(vp + 32 * dt * kVS);
+                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, phi, o[dt], 0, 0, 0);
+                    if (PRECISE) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, plo, o[dt], 0, 0, 0);
+                }
+            }
+        }
+
+        if (more) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- normalise, stage through LDS, write 16 bytes per lane -------------------------------------
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    uint16_t* stage = reinterpret_cast<uint16_t*>(pf_smem) + wave * 32 * kOS;   // 32 columns x 128 dims per wave
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+            const int d0 = 32 * dt + 8 * rq + 4 * grp;
+            uint2 packed;
+            packed.x = static_cast<uint32_t>(f2bf(o[dt][4 * rq + 0] * inv))
+                     | (static_cast<uint32_t>(f2bf(o[dt][4 * rq + 1] * inv)) << 16);
+            packed.y = static_cast<uint32_t>(f2bf(o[dt][4 * rq + 2] * inv))
+                     | (static_cast<uint32_t>(f2bf(o[dt][4 * rq + 3] * inv)) << 16);
+            *reinterpret_cast<uint2*>(&stage[col * kOS + d0]) = packed;
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0);   // the wave reads back only what it wrote itself
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int c = 4 * it + (lane >> 4);
+        const int chunk = lane & 15;
+        const int row = q0 + 16 * wave + (c & 15);
+        const int head = 2 * kvh + (c >> 4);
+        if (row < S) {
+            const uint4 val = *reinterpret_cast<const uint4*>(&stage[c * kOS + 8 * chunk]);
+            *reinterpret_cast<uint4*>(prm.out + ((static_cast<int64_t>(b) * S + row) * q_heads + head) * kDim + 8 * chunk) = val;
+        }
+    }
+}
+
+// grid = batch * kv_heads * n_qtiles blocks, heaviest query tile first; the first query tile
+// (dispatched last) takes the split-precision P path.
+__global__ __launch_bounds__(kPfThreads, 2) void prefill_causal_kernel(PrefillParams prm, qm_kv_cache cache) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char pf_smem[];
+    const int pairs = prm.batch * prm.kv_heads;
+    const int bid = blockIdx.x;
+    const int qt = prm.n_qtiles - 1 - bid / pairs;
+    const int pair = bid % pairs;
+    if (qt == 0) {
+        prefill_body<true>(prm, cache, pf_smem, 0, pair);
+    } else {
+        prefill_body<false>(prm, cache, pf_smem, qt, pair);
+    }
+}
+
+}  // namespace qm
+
 extern "C" int32_t qm_prefill_attention_causal(
-    const uint16_t*, const uint16_t*, const uint16_t*, uint16_t*, const qm_kv_cache*, const int32_t*,
-    int32_t, int32_t, int32_t, int32_t, int32_t, float, uint32_t*, void*) { return QM_ERR_ARGUMENT; }
+    const uint16_t* query, const uint16_t* key, const uint16_t* value,
+    uint16_t* context_out,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads, float scale,
+    uint32_t* status_dev, void* hip_stream) {
+    using namespace qm;
+    if (!query || !key || !value || !context_out) return QM_ERR_NULL;
+    if (batch < 0 || seq < 0) return QM_ERR_ARGUMENT;
+    if (kv_heads <= 0 || q_heads != 2 * kv_heads) return QM_ERR_GEOMETRY;   // GQA pair on the MFMA columns
+    const uintptr_t align = reinterpret_cast<uintptr_t>(query) | reinterpret_cast<uintptr_t>(key)
+                          | reinterpret_cast<uintptr_t>(value) | reinterpret_cast<uintptr_t>(context_out);
+    if (align & 15) return QM_ERR_GEOMETRY;
+    qm_kv_cache desc = {};
+    PageMap pm = make_page_map(16, 1);
+    if (cache) {
+        const int32_t rc = check_cache(cache, max_pages);
+        if (rc != QM_OK) return rc;
+        if (cache->kv_heads != kv_heads) return QM_ERR_GEOMETRY;
+        if (seq > cache_capacity(cache, max_pages)) return QM_ERR_SLOT_RANGE;
+        if (!page_table && (batch > 1 || (seq > 0 && (seq - 1) / cache->page_size >= cache->n_pages)))
+            return QM_ERR_SLOT_RANGE;   // an identity table can serve one sequence only
+        desc = *cache;
+        pm = make_page_map(cache->page_size, max_pages);
+    }
+    if (batch == 0 || seq == 0) return QM_OK;
+    const int n_qtiles = (seq + kBM - 1) / kBM;
+    const int64_t pairs = static_cast<int64_t>(batch) * kv_heads;
+    if (pairs * n_qtiles > 0x7fffffffLL) return QM_ERR_ARGUMENT;
+
+    PrefillParams prm;
+    prm.q = query; prm.k = key; prm.v = value; prm.out = context_out;
+    prm.page_table = page_table; prm.status = status_dev; prm.pages = pm;
+    prm.has_cache = cache ? 1 : 0;
+    prm.batch = batch; prm.seq = seq; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
+
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    const size_t smem = sizeof(PfShared);
+    static bool attr_set = false;
+    if (!attr_set) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_causal_kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+        if (e != hipSuccess) return hip_code(e);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(prefill_causal_kernel, dim3(static_cast<unsigned>(pairs * n_qtiles)), dim3(kPfThreads), smem, s,
+                       prm, desc);
+    return launch_status();
+}

@@ -1,0 +1,74 @@
+"""GPU parity: the code predictor's 16-step attention loop in one launch, through the C ABI.
+
+The kernel keeps the reference's whole rounding chain and summation order, so beyond the stated
+tolerance (max abs error <= 1e-2) nearly every output must be bit-identical to the oracle; the K/V
+cache write-back must be bit-exact.
+"""
+import numpy as np
+import pytest
+
+from qm_testlib import max_abs_err, to_dev, to_u16
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def _run(oracle, qm, dev, units, layers, rows, seed, first_rows=1, write_cache=True):
+    import torch
+    q = oracle.normal_bf16((units, rows, 16, 128), seed)
+    k = oracle.normal_bf16((units, rows, 8, 128), seed + 1)
+    v = oracle.normal_bf16((units, rows, 8, 128), seed + 2)
+    gq = oracle.normal_bf16((layers, 128), seed + 3, 1.0, 0.1)
+    gk = oracle.normal_bf16((layers, 128), seed + 4, 1.0, 0.1)
+    cos, sin = oracle.rope_table(rows, 0)
+    want = np.zeros_like(q)
+    kc = np.zeros((units, 8, 16, 128), dtype=np.uint16)
+    vc = np.zeros_like(kc)
+    assert oracle.predictor_attention_loop(q, k, v, gq, gk, cos, sin, want, kc, vc, units, layers, rows, first_rows,
+                                           1e-6, 16) == 0
+    out = torch.full((units, rows, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    kd = torch.full((units, 8, 16, 128), 0x7fc0, dtype=torch.int16, device=dev) if write_cache else None
+    vd = torch.full((units, 8, 16, 128), 0x7fc0, dtype=torch.int16, device=dev) if write_cache else None
+    qm.predictor_attention_loop(to_dev(q, dev), to_dev(k, dev), to_dev(v, dev), to_dev(gq, dev), to_dev(gk, dev),
+                                to_dev(cos, dev), to_dev(sin, dev), out, kd, vd, units, layers, rows, first_rows)
+    torch.cuda.synchronize()
+    return to_u16(out), want, (to_u16(kd) if write_cache else None, to_u16(vd) if write_cache else None), (kc, vc), v
+
+
+def test_predictor_config5_full_size(oracle, qm, dev):
+    units, layers, rows = 256 * 5, 5, 16
+    got, want, (kd, vd), (kc, vc), v = _run(oracle, qm, dev, units, layers, rows, seed=55)
+    assert max_abs_err(oracle, got, want) <= TOL
+    assert (got != want).mean() < 1e-3                        # only device-expf rounding may differ
+    assert np.array_equal(kd, kc) and np.array_equal(vd, vc)  # cache write-back, bit-exact
+    assert np.array_equal(got[:, 0], np.repeat(v[:, 0], 2, axis=1))   # step 0: context 1 -> out = V
+
+
+@pytest.mark.parametrize("units,layers,rows,first_rows", [(1, 1, 16, 1), (7, 5, 16, 2), (3, 2, 1, 1), (5, 5, 2, 2),
+                                                          (4, 3, 9, 1)])
+def test_predictor_small_and_partial(oracle, qm, dev, units, layers, rows, first_rows):
+    got, want, (kd, vd), (kc, vc), _ = _run(oracle, qm, dev, units, layers, rows, seed=units * 31 + rows,
+                                           first_rows=first_rows)
+    assert max_abs_err(oracle, got, want) <= TOL
+    assert (got != want).mean() < 1e-3
+    assert np.array_equal(kd, kc) and np.array_equal(vd, vc)
+
+
+def test_predictor_without_cache_and_errors(oracle, qm, dev):
+    import torch
+    got, want, _, _, _ = _run(oracle, qm, dev, 6, 5, 16, seed=3, write_cache=False)
+    assert max_abs_err(oracle, got, want) <= TOL
+    z = torch.zeros((1, 16, 16, 128), dtype=torch.int16, device=dev)
+    w = torch.zeros((1, 128), dtype=torch.int16, device=dev)
+    r = torch.zeros((16, 128), dtype=torch.int16, device=dev)
+    for bad in (dict(rows=17), dict(rows=0), dict(first_rows=3), dict(n_layers=0)):
+        args = dict(units=1, n_layers=1, rows=16, first_rows=1)
+        args.update(bad)
+        with pytest.raises(qm.QmError) as e:
+            qm.predictor_attention_loop(z, z, z, w, w, r, r, z, None, None, args["units"], args["n_layers"],
+                                        args["rows"], args["first_rows"])
+        assert e.value.code == -5
+    with pytest.raises(qm.QmError) as e:
+        qm.predictor_attention_loop(None, z, z, w, w, r, r, z, None, None, 1, 1, 16, 1)
+    assert e.value.code == -1

@@ -1,0 +1,111 @@
+"""GPU parity: causal GQA prefill on MFMA with the fused paged K/V write, through the C ABI.
+
+Tolerance (stated by the task): max abs error <= 1e-2 on bf16 outputs against the scalar fp32
+oracle (ONLINE policy: reference score roundings, fp32 softmax); K/V page contents bit-exact.
+"""
+import numpy as np
+import pytest
+
+from qm_testlib import SCALE, PagedPool, max_abs_err, to_dev, to_u16
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def _run(oracle, qm, dev, batch, seq, seed, with_cache=True, threads=16):
+    import torch
+    q = oracle.normal_bf16((batch, seq, 16, 128), seed)
+    k = oracle.normal_bf16((batch, seq, 8, 128), seed + 1)
+    v = oracle.normal_bf16((batch, seq, 8, 128), seed + 2)
+    pool = PagedPool(oracle, [seq] * batch, seed=seed + 3, fill=0x7fc0) if with_cache else None
+    want = {}
+    for policy in (0, 1):
+        o = np.zeros_like(q)
+        rc = oracle.prefill_attention_causal(q, k, v, o, pool.descriptor(oracle) if pool else None,
+                                             pool.page_table if pool else None, pool.max_pages if pool else 0,
+                                             batch, seq, 16, 8, SCALE, policy, threads)
+        assert rc == 0
+        want[policy] = o
+    out = torch.full((batch, seq, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    sd = torch.zeros(1, dtype=torch.int32, device=dev)
+    if pool:
+        fresh = PagedPool(oracle, [seq] * batch, seed=seed + 3, fill=0x7fc0)
+        kd, vd, cache_d, table_d = fresh.device(qm, dev)
+        qm.prefill_attention_causal(to_dev(q, dev), to_dev(k, dev), to_dev(v, dev), out, cache_d, table_d,
+                                    fresh.max_pages, batch, seq, 16, 8, SCALE, sd)
+    else:
+        kd = vd = None
+        qm.prefill_attention_causal(to_dev(q, dev), to_dev(k, dev), to_dev(v, dev), out, None, None, 0, batch, seq,
+                                    16, 8, SCALE, sd)
+    torch.cuda.synchronize()
+    assert int(sd.item()) == 0
+    return to_u16(out), want, pool, kd, vd, (q, k, v)
+
+
+@pytest.mark.parametrize("batch,seq", [(1, 1), (1, 2), (1, 16), (1, 17), (1, 63), (1, 64), (1, 65), (2, 100),
+                                       (1, 128), (3, 130), (1, 257), (2, 512)])
+def test_prefill_small_shapes(oracle, qm, dev, batch, seq):
+    got, want, pool, kd, vd, _ = _run(oracle, qm, dev, batch, seq, seed=1000 + seq, threads=8)
+    assert max_abs_err(oracle, got, want[1]) <= TOL
+    assert np.array_equal(to_u16(kd), pool.k) and np.array_equal(to_u16(vd), pool.v)   # paged write, bit-exact
+    # row 0 of every sequence is V[0] exactly
+    assert np.array_equal(got[:, 0], want[0][:, 0])
+
+
+def test_prefill_config4_full_size(oracle, qm, dev):
+    got, want, pool, kd, vd, _ = _run(oracle, qm, dev, 4, 1024, seed=4)
+    assert max_abs_err(oracle, got, want[1]) <= TOL
+    assert np.array_equal(to_u16(kd), pool.k) and np.array_equal(to_u16(vd), pool.v)
+    # against the reference chain (bf16(P) included): rows with at least 64 keys
+    assert max_abs_err(oracle, got[:, 64:], want[0][:, 64:]) <= TOL
+
+
+def test_prefill_without_cache_and_causality(oracle, qm, dev):
+    import torch
+    got, want, _, _, _, (q, k, v) = _run(oracle, qm, dev, 1, 200, seed=9, with_cache=False)
+    assert max_abs_err(oracle, got, want[1]) <= TOL
+    # Later tokens must not leak into earlier rows: huge finite values anywhere after the row,
+    # NaN from the next 16-row group on (inside a row's own 16-row group the mask is P = 0 times V).
+    for first_bad, poison, rows_ok in ((150, 0x7f7f, 150), (160, 0x7fc0, 160)):
+        k2, v2 = k.copy(), v.copy()
+        k2[0, first_bad:] = poison
+        v2[0, first_bad:] = poison
+        out = torch.zeros((1, 200, 16, 128), dtype=torch.int16, device=dev)
+        qm.prefill_attention_causal(to_dev(q, dev), to_dev(k2, dev), to_dev(v2, dev), out, None, None, 0, 1, 200, 16, 8)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_u16(out)[0, :rows_ok], got[0, :rows_ok])
+
+
+def test_prefill_rows_match_decode_over_written_cache(oracle, qm, dev):
+    """Cross-operator invariant on the GPU: prefill row i == decode attention at position i."""
+    import torch
+    seq = 300
+    got, _, pool, kd, vd, (q, _, _) = _run(oracle, qm, dev, 1, seq, seed=21)
+    cache_d = qm.paged_cache(kd, vd, pool.n_pages)
+    table_d = to_dev(pool.page_table, dev)
+    nb = qm.decode_workspace_bytes(1, 16, 8, seq)
+    ws = torch.empty(nb // 4 + 1, dtype=torch.float32, device=dev)
+    for i in (0, 1, 15, 16, 63, 64, 299):
+        o = torch.zeros((16, 128), dtype=torch.int16, device=dev)
+        qm.decode_attention(to_dev(q[0, i].copy(), dev), cache_d, table_d, pool.max_pages, o, 16, i, -1, SCALE, ws, nb)
+        torch.cuda.synchronize()
+        assert max_abs_err(oracle, to_u16(o), got[0, i]) <= TOL
+
+
+def test_prefill_argument_errors(oracle, qm, dev):
+    import torch
+    x = torch.zeros((1, 64, 16, 128), dtype=torch.int16, device=dev)
+    kv = torch.zeros((1, 64, 8, 128), dtype=torch.int16, device=dev)
+    with pytest.raises(qm.QmError) as e:
+        qm.prefill_attention_causal(x, kv, kv, x, None, None, 0, 1, 64, 16, 4)      # group of 4 unsupported here
+    assert e.value.code == -2
+    with pytest.raises(qm.QmError) as e:
+        qm.prefill_attention_causal(None, kv, kv, x, None, None, 0, 1, 64, 16, 8)
+    assert e.value.code == -1
+    pool_k = torch.zeros((2, 8, 16, 128), dtype=torch.int16, device=dev)
+    cache = qm.paged_cache(pool_k, pool_k, 2)
+    table = torch.zeros((1, 2), dtype=torch.int32, device=dev)
+    with pytest.raises(qm.QmError) as e:
+        qm.prefill_attention_causal(x, kv, kv, x, cache, table, 2, 1, 64, 16, 8)    # 64 tokens > 2 pages
+    assert e.value.code == -3
