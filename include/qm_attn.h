@@ -185,12 +185,20 @@ int32_t qm_scatter_kv(
  * key, value [batch][seq][kv_heads][128] already normed/rotated; row i attends keys
  * 0..i of its own batch entry.  If cache != NULL, K/V are also written to the pages of
  * page_table [batch][max_pages] at tokens 0..seq-1.
+ * kv_stride_token / kv_stride_head / kv_stride_batch: element strides of key and value; all
+ * zero selects the contiguous [batch][seq][kv_heads][128] layout.  The reference's
+ * LayerCache [kv_head][max_cache][128] is read in place with (128, max_cache*128, 0), which
+ * is how launch_attention(query_length > 1, cache_before = 0) is served.
+ * Only q_heads == 2 * kv_heads is supported by this entry point.
+ * Later tokens never contribute to a row; a non-finite V of a later row inside the same
+ * 16-row group would propagate as 0 * inf (the reference skips those keys).
  */
 int32_t qm_prefill_attention_causal(
     const uint16_t* query, const uint16_t* key, const uint16_t* value,
     uint16_t* context_out,
     const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
     int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads, float scale,
+    int64_t kv_stride_token, int64_t kv_stride_head, int64_t kv_stride_batch,
     uint32_t* status_dev,
     void* hip_stream);
 

@@ -1,0 +1,179 @@
+// qm_attn.hpp — C++ host adapters over the C ABI of qm_attn.h.
+//
+// These free functions keep the names, argument order and error behaviour of the reference
+// engine's private launch wrappers (devices/rx7900xtx-24g/qwen3_tts_1_7b.cpp, "R17"), so that an
+// engine written against them needs no other change:
+//   - device pointers are raw, bf16 is uint16_t bit patterns, the KV cache is the flat
+//     [kv_head][max_cache][128] LayerCache (R17:16371-16390);
+//   - every call is asynchronous on the given stream and never synchronises;
+//   - failures throw std::runtime_error with a label, like hip_check / PRED_HIP_CHECK
+//     (R17:7941-7949, 17603-17605) and the host overflow guards (R17:16844-16847).
+// Paged callers use the C ABI (or the *_paged overloads below) directly.
+#ifndef QM_ATTN_HPP
+#define QM_ATTN_HPP
+
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+#include "qm_attn.h"
+
+namespace qm_attn {
+
+inline void check(int32_t code, const char* label) {
+    if (code != QM_OK) {
+        throw std::runtime_error(std::string(label) + ": " + qm_error_string(code) + " ("
+                                 + std::to_string(code) + ")");
+    }
+}
+
+// View of the reference's LayerCache as a one-page qm_kv_cache.
+inline qm_kv_cache flat_cache(std::uint16_t* key_cache, std::uint16_t* value_cache, int kv_heads,
+                              int head_dim, int max_cache) {
+    qm_kv_cache c;
+    c.k_pool = key_cache;
+    c.v_pool = value_cache;
+    c.stride_page = 0;
+    c.stride_head = static_cast<std::int64_t>(max_cache) * head_dim;
+    c.stride_token = head_dim;
+    c.page_size = max_cache;
+    c.n_pages = 1;
+    c.kv_heads = kv_heads;
+    c.head_dim = head_dim;
+    return c;
+}
+
+// Native paged layout [page][kv_head][16][128].
+inline qm_kv_cache paged_cache(std::uint16_t* k_pool, std::uint16_t* v_pool, int n_pages, int kv_heads) {
+    qm_kv_cache c;
+    c.k_pool = k_pool;
+    c.v_pool = v_pool;
+    c.stride_page = static_cast<std::int64_t>(kv_heads) * 16 * 128;
+    c.stride_head = 16 * 128;
+    c.stride_token = 128;
+    c.page_size = 16;
+    c.n_pages = n_pages;
+    c.kv_heads = kv_heads;
+    c.head_dim = 128;
+    return c;
+}
+
+// ≙ NativeTalkerEngine::launch_qk_norm_rope_cache_m1 (R17:17569-17606) with the argument list of
+// talker_qk_norm_rope_cache_fused_kernel (R17:15365-15381); also the predictor's
+// qk_norm_rope_cache_m1 (R17:13432-13471) with q_heads 16, kv_heads 8, max_cache 16.
+inline void launch_qk_norm_rope_cache_m1(
+    const std::uint16_t* q, const std::uint16_t* k, const std::uint16_t* v,
+    const std::uint16_t* q_norm_weight, const std::uint16_t* k_norm_weight,
+    const std::uint16_t* cosine, const std::uint16_t* sine,
+    std::uint16_t* q_rotated, std::uint16_t* key_cache, std::uint16_t* value_cache,
+    int q_heads, int kv_heads, int head_dim, int max_cache, int cache_position, float epsilon,
+    void* stream) {
+    if (cache_position >= max_cache) throw std::runtime_error("Talker decode cache overflow.");
+    const qm_kv_cache c = flat_cache(key_cache, value_cache, kv_heads, head_dim, max_cache);
+    check(qm_qk_norm_rope_kv_append(q, k, v, q_norm_weight, k_norm_weight, cosine, sine, q_rotated, &c,
+                                    nullptr, 1, q_heads, cache_position, epsilon, stream),
+          "Qingming QK norm/RoPE/cache launch");
+}
+
+// Bytes of split-K workspace launch_attention needs for contexts up to max_cache tokens.
+inline std::size_t attention_workspace_bytes(int q_heads, int kv_heads, int max_cache) {
+    return qm_decode_workspace_bytes(1, q_heads, kv_heads, max_cache);
+}
+
+// ≙ NativeTalkerEngine::launch_attention (R17:17723-17814).  query_length == 1 is decode over
+// keys [key_start, cache_before + 1); query_length > 1 is the causal prefill over the rows that
+// scatter_prefill_cache has already placed in the cache, with cache_before == 0 as in
+// NativeTalkerEngine::prefill (R17:16710-16717).  The reference sizes dynamic LDS from the context;
+// here the caller passes a workspace sized by attention_workspace_bytes instead.
+inline void launch_attention(
+    const std::uint16_t* query, std::uint16_t* key_cache, std::uint16_t* value_cache,
+    std::uint16_t* context, int query_length, int cache_before,
+    int q_heads, int kv_heads, int head_dim, int max_cache, int sliding_window, float scale,
+    void* workspace, std::size_t workspace_bytes, void* stream) {
+    const qm_kv_cache c = flat_cache(key_cache, value_cache, kv_heads, head_dim, max_cache);
+    if (query_length == 1) {
+        check(qm_decode_attention(query, &c, nullptr, 1, context, q_heads, cache_before, sliding_window,
+                                  scale, workspace, workspace_bytes, stream),
+              "Talker GQA M1 attention launch");
+        return;
+    }
+    if (cache_before != 0 || sliding_window > 0) {
+        throw std::runtime_error("Talker generic attention launch: only cache_before == 0 without a "
+                                 "sliding window is supported for query_length > 1");
+    }
+    if (query_length > max_cache) throw std::runtime_error("Talker prefill cache overflow.");
+    check(qm_prefill_attention_causal(query, key_cache, value_cache, context, nullptr, nullptr, 0, 1,
+                                      query_length, q_heads, kv_heads, scale, head_dim,
+                                      static_cast<std::int64_t>(max_cache) * head_dim, 0, nullptr, stream),
+          "Talker generic fused attention launch");
+}
+
+// ≙ launch_rope_rows (R17:17608-17644).
+inline void launch_rope_rows(const std::uint16_t* input, const std::uint16_t* cosine,
+                             const std::uint16_t* sine, std::uint16_t* output, int sequence_length,
+                             int heads, int head_dim, void* stream) {
+    if (head_dim != 128) throw std::runtime_error("Talker RoPE rows launch: head_dim must be 128");
+    check(qm_norm_rope_rows(input, nullptr, cosine, sine, output, sequence_length, heads, 0.0f, stream),
+          "Talker RoPE rows launch");
+}
+
+// Per-head RMSNorm over rows = S*heads, dim 128 (rmsnorm_kernel R17:8276, called R17:16673-16689)
+// fused with launch_rope_rows: one launch instead of two plus a global round trip.
+inline void launch_norm_rope_rows(const std::uint16_t* input, const std::uint16_t* norm_weight,
+                                  const std::uint16_t* cosine, const std::uint16_t* sine,
+                                  std::uint16_t* output, int sequence_length, int heads, float epsilon,
+                                  void* stream) {
+    check(qm_norm_rope_rows(input, norm_weight, cosine, sine, output, sequence_length, heads, epsilon,
+                            stream),
+          "Talker norm/RoPE rows launch");
+}
+
+// ≙ scatter_prefill_cache (R17:17646-17682).
+inline void scatter_prefill_cache(const std::uint16_t* key, const std::uint16_t* value,
+                                  std::uint16_t* key_cache, std::uint16_t* value_cache,
+                                  int sequence_length, int kv_heads, int head_dim, int max_cache,
+                                  void* stream) {
+    const qm_kv_cache c = flat_cache(key_cache, value_cache, kv_heads, head_dim, max_cache);
+    check(qm_scatter_kv(key, value, &c, nullptr, 1, sequence_length, 0, stream),
+          "Talker prefill KV scatter launch");
+}
+
+// ≙ scatter_decode_cache (R17:17684-17720).
+inline void scatter_decode_cache(const std::uint16_t* key, const std::uint16_t* value,
+                                 std::uint16_t* key_cache, std::uint16_t* value_cache, int kv_heads,
+                                 int head_dim, int max_cache, int cache_position, void* stream) {
+    if (cache_position >= max_cache) throw std::runtime_error("Talker decode cache overflow.");
+    const qm_kv_cache c = flat_cache(key_cache, value_cache, kv_heads, head_dim, max_cache);
+    check(qm_scatter_kv(key, value, &c, nullptr, 1, 1, cache_position, stream),
+          "Talker decode KV scatter launch");
+}
+
+// ≙ PersistentPredictor::attention_m1 (R17:13473-13497): cache [8][16][128], key_length <= 16.
+inline void predictor_attention_m1(const std::uint16_t* query_rotated, std::uint16_t* key_cache,
+                                   std::uint16_t* value_cache, std::uint16_t* attention_context,
+                                   int key_length, void* stream) {
+    if (key_length < 1 || key_length > 16) throw std::runtime_error("Predictor attention: key_length out of range");
+    const qm_kv_cache c = flat_cache(key_cache, value_cache, 8, 128, 16);
+    check(qm_decode_attention(query_rotated, &c, nullptr, 1, attention_context, 16, key_length - 1, -1,
+                              0.08838834764831845f, nullptr, 0, stream),
+          "Predictor M1 attention launch");
+}
+
+// One launch for all frames x layers x steps of the predictor loop (no reference counterpart as a
+// single call; replaces the attention-path nodes of capture_step R17:13592-13707).
+inline void predictor_attention_loop(
+    const std::uint16_t* q, const std::uint16_t* k, const std::uint16_t* v,
+    const std::uint16_t* q_norm_weight, const std::uint16_t* k_norm_weight,
+    const std::uint16_t* cosine, const std::uint16_t* sine, std::uint16_t* context,
+    std::uint16_t* key_cache_out, std::uint16_t* value_cache_out,
+    int units, int layers, int rows, int first_rows, float epsilon, void* stream) {
+    check(qm_predictor_attention_loop(q, k, v, q_norm_weight, k_norm_weight, cosine, sine, context,
+                                      key_cache_out, value_cache_out, units, layers, rows, first_rows,
+                                      epsilon, stream),
+          "Predictor attention loop launch");
+}
+
+}  // namespace qm_attn
+
+#endif  // QM_ATTN_HPP

@@ -56,7 +56,7 @@ _SIGNATURES = {
     "qm_norm_rope_rows": (_I32, [_PTR] * 5 + [_I32, _I32, _F32, _PTR]),
     "qm_scatter_kv": (_I32, [_PTR, _PTR, C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _PTR]),
     "qm_prefill_attention_causal": (_I32, [_PTR] * 4 + [C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _I32, _I32,
-                                           _F32, _PTR, _PTR]),
+                                           _F32, C.c_int64, C.c_int64, C.c_int64, _PTR, _PTR]),
     "qm_predictor_attention_loop": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _I32, _F32, _PTR]),
 }
 
@@ -157,11 +157,12 @@ def scatter_kv(key, value, cache, page_table, max_pages, rows, first_position, s
 
 
 def prefill_attention_causal(query, key, value, out, cache, page_table, max_pages, batch, seq, q_heads,
-                             kv_heads, scale=SCALE_128, status=None, stream=0):
+                             kv_heads, scale=SCALE_128, status=None, stream=0, kv_strides=(0, 0, 0)):
     _check(lib().qm_prefill_attention_causal(
         _addr(query), _addr(key), _addr(value), _addr(out),
         C.byref(cache) if cache is not None else None, _addr(page_table), max_pages, batch, seq,
-        q_heads, kv_heads, scale, _addr(status), stream), "qm_prefill_attention_causal")
+        q_heads, kv_heads, scale, kv_strides[0], kv_strides[1], kv_strides[2], _addr(status), stream),
+        "qm_prefill_attention_causal")
 
 
 def predictor_attention_loop(q, k, v, gq, gk, cos, sin, out, k_cache_out, v_cache_out, units, n_layers,

@@ -30,6 +30,8 @@ namespace qm {
 constexpr int kDecodeThreads = 256;
 constexpr int kDecodeWaves = 4;
 constexpr int kRowStreams = 16;  // 4 waves x 4 DPP rows
+constexpr int kMaxTilesPerBlock = 64;
+constexpr int kMaxSplitsMerged = 64;   // splits merged per LDS round in the merge kernel
 
 struct DecodeParams {
     const uint16_t* query;        // [n_streams][q_heads][128]
@@ -63,6 +65,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
     __shared__ float sh_acc[kRowStreams][G][kDim];
     __shared__ float sh_m[kRowStreams][G];
     __shared__ float sh_l[kRowStreams][G];
+    __shared__ int64_t sh_off[kMaxTilesPerBlock];   // element offset of each tile of this block, -1 = unreadable
 
     const int split = blockIdx.x;
     const int kvh = blockIdx.y;
@@ -100,8 +103,14 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
     if (tile_lo > last_tile) return;
     const int tile_hi = min(tile_lo + prm.tiles_per_block - 1, last_tile);
 
-    const int32_t* table =
-        prm.page_table ? prm.page_table + static_cast<int64_t>(stream) * prm.pages.max_pages : nullptr;
+    // Page lookups happen once, up front, so that the streaming loop below issues nothing but
+    // K/V loads to the vector memory queue (a page-table load inside the loop would make every
+    // iteration wait for the whole queue to drain).
+    if (tid <= tile_hi - tile_lo) {
+        const int32_t* table =
+            prm.page_table ? prm.page_table + static_cast<int64_t>(stream) * prm.pages.max_pages : nullptr;
+        sh_off[tid] = tile_offset(cache, prm.pages, table, (tile_lo + tid) * kTile, kvh, prm.status);
+    }
 
     // Query chunk of this lane for each head of the group, packed bf16 pairs.
     uint4 qv[G];
@@ -120,31 +129,34 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[g][e] = 0.0f;
     }
+    __syncthreads();
 
+    // Unpredicated fetch: a token outside [key_start, key_end) is redirected to the nearest
+    // token inside (same tile, so the address is valid) and its score is masked afterwards; an
+    // unreadable tile reads pool offset 0 and is masked as a whole.
     uint4 kreg[4], vreg[4];
-    bool valid[4];
-    auto fetch = [&](int tile, uint4* kr, uint4* vr, bool* ok) {
+    int okmask = 0;
+    auto fetch = [&](int tile, uint4* kr, uint4* vr, int& ok) {
         const int first_token = tile * kTile;
-        const int64_t off = tile_offset(cache, prm.pages, table, first_token, kvh, prm.status);
+        int64_t off = sh_off[tile - tile_lo];
+        const bool readable = off >= 0;
+        off = readable ? off : 0;
+        ok = 0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int token = first_token + 4 * i + row;
-            ok[i] = off >= 0 && token >= key_start && token < key_end;
-            const int64_t e = off + static_cast<int64_t>(4 * i + row) * kDim + col * 8;
-            kr[i] = load_or_zero(cache.k_pool + e, ok[i]);
-            vr[i] = load_or_zero(cache.v_pool + e, ok[i]);
+            const bool in_range = readable && token >= key_start && token < key_end;
+            ok |= in_range ? (1 << i) : 0;
+            int safe = min(max(token, key_start), key_end - 1) - first_token;
+            safe = readable ? min(max(safe, 0), kTile - 1) : 0;
+            const int64_t e = off + safe * kDim + col * 8;
+            kr[i] = *reinterpret_cast<const uint4*>(cache.k_pool + e);
+            vr[i] = *reinterpret_cast<const uint4*>(cache.v_pool + e);
         }
     };
 
-    int tile = tile_lo + wave;
-    if (tile <= tile_hi) fetch(tile, kreg, vreg, valid);
-
-    while (tile <= tile_hi) {
-        const int next = tile + kDecodeWaves;
-        uint4 knext[4], vnext[4];
-        bool oknext[4];
-        if (next <= tile_hi) fetch(next, knext, vnext, oknext);
-
+    // One tile of work on a register set: scores, online softmax update, P.V.
+    auto consume = [&](const uint4* kr, const uint4* vr, int ok) {
         // ---- scores of the 4 tokens this row owns, for every head of the group -------------
         float s[4][G];
 #pragma unroll
@@ -152,17 +164,16 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 float d = 0.0f;
-                d = dot2_bf16(qv[g].x, kreg[i].x, d);
-                d = dot2_bf16(qv[g].y, kreg[i].y, d);
-                d = dot2_bf16(qv[g].z, kreg[i].z, d);
-                d = dot2_bf16(qv[g].w, kreg[i].w, d);
+                d = dot2_bf16(qv[g].x, kr[i].x, d);
+                d = dot2_bf16(qv[g].y, kr[i].y, d);
+                d = dot2_bf16(qv[g].z, kr[i].z, d);
+                d = dot2_bf16(qv[g].w, kr[i].w, d);
                 d = row16_allreduce_sum(d);
                 // bf16(QK) then bf16(* scale), R17:16102-16116
                 d = round_bf16(round_bf16(d) * prm.scale);
-                s[i][g] = valid[i] ? d : -INFINITY;
+                s[i][g] = (ok >> i) & 1 ? d : -INFINITY;
             }
         }
-
         // ---- online softmax update of this row-stream ------------------------------------------
         float p[4][G];
 #pragma unroll
@@ -182,15 +193,15 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
 #pragma unroll
             for (int e = 0; e < 8; ++e) acc[g][e] *= alpha;
         }
-
-        // ---- P.V -------------------------------------------------------------------------------
+        // ---- P.V (a masked token has p = 0 and a duplicated, finite row) ---------------------------
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const uint32_t w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
+            const uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
+            const bool live = (ok >> i) & 1;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float v0 = lo_bf16(w[j]);
-                const float v1 = hi_bf16(w[j]);
+                const float v0 = live ? lo_bf16(w[j]) : 0.0f;
+                const float v1 = live ? hi_bf16(w[j]) : 0.0f;
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
                     acc[g][2 * j] = fmaf(p[i][g], v0, acc[g][2 * j]);
@@ -198,14 +209,40 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
                 }
             }
         }
+    };
 
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            kreg[i] = knext[i];
-            vreg[i] = vnext[i];
-            valid[i] = oknext[i];
+    // Two register sets in ping-pong: the loads of one tile are in flight while the other tile
+    // is consumed, with no register copies between iterations.  Every path issues exactly one
+    // fetch between two consumes, so that the in-order load counter lets the consume of a set
+    // start while the eight loads of the other set are still outstanding.
+    uint4 kreg2[4], vreg2[4];
+    int okmask2 = 0;
+    int tile = tile_lo + wave;
+    if (tile <= tile_hi) {
+        fetch(tile, kreg, vreg, okmask);
+        bool last_is_second = false;
+        for (;;) {
+            int next = tile + kDecodeWaves;
+            if (next > tile_hi) break;
+            fetch(next, kreg2, vreg2, okmask2);
+            __builtin_amdgcn_sched_barrier(0);   // issue the loads before waiting on the other set
+            consume(kreg, vreg, okmask);
+            tile = next;
+            next = tile + kDecodeWaves;
+            if (next > tile_hi) {
+                last_is_second = true;
+                break;
+            }
+            fetch(next, kreg, vreg, okmask);
+            __builtin_amdgcn_sched_barrier(0);
+            consume(kreg2, vreg2, okmask2);
+            tile = next;
         }
-        tile = next;
+        if (last_is_second) {
+            consume(kreg2, vreg2, okmask2);
+        } else {
+            consume(kreg, vreg, okmask);
+        }
     }
 
     // ---- merge the 16 row-streams of the block -----------------------------------------------
@@ -278,15 +315,43 @@ __global__ void decode_merge_kernel(DecodeParams prm) {
     const float* base = prm.partial
         + (static_cast<int64_t>(stream) * gridDim.x + kvh) * prm.max_splits * partial_floats<G>();
 
-    float mm = -INFINITY;
-    for (int s = 0; s < splits; ++s) mm = fmaxf(mm, base[s * partial_floats<G>() + G * kDim + g]);
-    const float m_ref = mm == -INFINITY ? 0.0f : mm;
+    // Statistics of all splits go through LDS in one round of loads; the accumulator column of
+    // each thread is then summed with independent (pipelined) loads.
+    __shared__ float sh_w[kMaxSplitsMerged][G];
+    __shared__ float sh_l[kMaxSplitsMerged][G];
     float ll = 0.0f, aa = 0.0f;
-    for (int s = 0; s < splits; ++s) {
-        const float* rec = base + s * partial_floats<G>();
-        const float w = fast_exp2((rec[G * kDim + g] - m_ref) * kLog2e);
-        ll = fmaf(rec[G * kDim + G + g], w, ll);
-        aa = fmaf(rec[g * kDim + d], w, aa);
+    float m_run = -INFINITY;
+    for (int s0 = 0; s0 < splits; s0 += kMaxSplitsMerged) {
+        const int n = min(splits - s0, kMaxSplitsMerged);
+        __syncthreads();
+        for (int i = threadIdx.x; i < n * G; i += blockDim.x) {
+            const float* rec = base + static_cast<int64_t>(s0 + i / G) * partial_floats<G>();
+            sh_w[i / G][i % G] = rec[G * kDim + i % G];
+            sh_l[i / G][i % G] = rec[G * kDim + G + i % G];
+        }
+        __syncthreads();
+        float mm = m_run;
+        for (int s = 0; s < n; ++s) mm = fmaxf(mm, sh_w[s][g]);
+        const float m_ref = mm == -INFINITY ? 0.0f : mm;
+        const float rescale = fast_exp2((m_run - m_ref) * kLog2e);
+        ll *= rescale;
+        aa *= rescale;
+        m_run = mm;
+        float part[8];
+        for (int s = 0; s < n; s += 8) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                part[u] = s + u < n ? base[static_cast<int64_t>(s0 + s + u) * partial_floats<G>() + g * kDim + d] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (s + u < n) {
+                    const float w = fast_exp2((sh_w[s + u][g] - m_ref) * kLog2e);
+                    ll = fmaf(sh_l[s + u][g], w, ll);
+                    aa = fmaf(part[u], w, aa);
+                }
+            }
+        }
     }
     *dst = f2bf(ll > 0.0f ? aa / ll : 0.0f);
 }
@@ -312,6 +377,7 @@ inline DecodePlan plan_decode(int n_streams, int kv_heads, int max_seq_len) {
         if (t > 16) t = 16;
         tiles_per_block = static_cast<int>(t);
     }
+    if (tiles_per_block > kMaxTilesPerBlock) tiles_per_block = kMaxTilesPerBlock;
     DecodePlan plan;
     plan.tiles_per_block = tiles_per_block;
     plan.max_splits = static_cast<int>((max_tiles + tiles_per_block - 1) / tiles_per_block);

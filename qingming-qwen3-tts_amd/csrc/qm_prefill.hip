@@ -48,6 +48,9 @@ struct PrefillParams {
     uint16_t* out;         // [batch][seq][2*kv_heads][128]
     const int32_t* page_table;   // [batch][max_pages] or NULL
     uint32_t* status;
+    int64_t kv_stride_token;     // elements between consecutive keys of one kv head
+    int64_t kv_stride_head;
+    int64_t kv_stride_batch;
     PageMap pages;
     int has_cache;
     int batch;
@@ -112,8 +115,8 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     float m_run = -INFINITY;
     float l_run = 0.0f;
 
-    const int64_t kv_base = static_cast<int64_t>(b) * S * prm.kv_heads * kDim + static_cast<int64_t>(kvh) * kDim;
-    const int64_t kv_row = static_cast<int64_t>(prm.kv_heads) * kDim;
+    const int64_t kv_base = static_cast<int64_t>(b) * prm.kv_stride_batch + static_cast<int64_t>(kvh) * prm.kv_stride_head;
+    const int64_t kv_row = prm.kv_stride_token;
     const int32_t* table = prm.page_table ? prm.page_table + static_cast<int64_t>(b) * prm.pages.max_pages : nullptr;
 
     // Global -> register staging of one K/V tile.  K: chunk c = tid + 256*i -> key c/16, dims
@@ -322,8 +325,17 @@ extern "C" int32_t qm_prefill_attention_causal(
     uint16_t* context_out,
     const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
     int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads, float scale,
+    int64_t kv_stride_token, int64_t kv_stride_head, int64_t kv_stride_batch,
     uint32_t* status_dev, void* hip_stream) {
     using namespace qm;
+    if (kv_stride_token == 0 && kv_stride_head == 0 && kv_stride_batch == 0) {
+        kv_stride_token = static_cast<int64_t>(kv_heads) * kDim;     // [batch][seq][kv_heads][128]
+        kv_stride_head = kDim;
+        kv_stride_batch = static_cast<int64_t>(seq) * kv_heads * kDim;
+    }
+    if (kv_stride_token < kDim || kv_stride_head < 0 || kv_stride_batch < 0
+        || ((kv_stride_token | kv_stride_head | kv_stride_batch) & 7))
+        return QM_ERR_GEOMETRY;
     if (!query || !key || !value || !context_out) return QM_ERR_NULL;
     if (batch < 0 || seq < 0) return QM_ERR_ARGUMENT;
     if (kv_heads <= 0 || q_heads != 2 * kv_heads) return QM_ERR_GEOMETRY;   // GQA pair on the MFMA columns
@@ -351,6 +363,7 @@ extern "C" int32_t qm_prefill_attention_causal(
     prm.q = query; prm.k = key; prm.v = value; prm.out = context_out;
     prm.page_table = page_table; prm.status = status_dev; prm.pages = pm;
     prm.has_cache = cache ? 1 : 0;
+    prm.kv_stride_token = kv_stride_token; prm.kv_stride_head = kv_stride_head; prm.kv_stride_batch = kv_stride_batch;
     prm.batch = batch; prm.seq = seq; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
 
     hipStream_t s = static_cast<hipStream_t>(hip_stream);

@@ -109,3 +109,27 @@ def test_prefill_argument_errors(oracle, qm, dev):
     with pytest.raises(qm.QmError) as e:
         qm.prefill_attention_causal(x, kv, kv, x, cache, table, 2, 1, 64, 16, 8)    # 64 tokens > 2 pages
     assert e.value.code == -3
+
+
+def test_prefill_over_flat_layer_cache_in_place(oracle, qm, dev):
+    """launch_attention(query_length > 1, cache_before = 0) of the reference: K/V are read in place from
+    the flat [kv_head][max_cache][128] LayerCache that scatter_prefill_cache filled (R17:16703-16717)."""
+    import torch
+    seq, max_cache = 150, 163
+    q = oracle.normal_bf16((seq, 16, 128), 1)
+    k = oracle.normal_bf16((seq, 8, 128), 2)
+    v = oracle.normal_bf16((seq, 8, 128), 3)
+    kc = np.full((8, max_cache, 128), 0x7fc0, dtype=np.uint16)     # NaN beyond the sequence
+    vc = np.full((8, max_cache, 128), 0x7fc0, dtype=np.uint16)
+    assert oracle.scatter_kv(k, v, oracle.flat_cache(kc, vc, 8, max_cache), None, 1, seq, 0) == 0
+    want = np.zeros_like(q)
+    assert oracle.attention(q, oracle.flat_cache(kc, vc, 8, max_cache), None, 1, want, seq, 0, 16, -1, SCALE, 1, 8) == 0
+    kd = to_dev(np.full((8, max_cache, 128), 0x7fc0, dtype=np.uint16), dev)
+    vd = to_dev(np.full((8, max_cache, 128), 0x7fc0, dtype=np.uint16), dev)
+    qm.scatter_kv(to_dev(k, dev), to_dev(v, dev), qm.flat_cache(kd, vd, 8, max_cache), None, 1, seq, 0)
+    out = torch.zeros((seq, 16, 128), dtype=torch.int16, device=dev)
+    qm.prefill_attention_causal(to_dev(q, dev), kd, vd, out, None, None, 0, 1, seq, 16, 8, SCALE, None, 0,
+                                (128, max_cache * 128, 0))
+    torch.cuda.synchronize()
+    assert np.array_equal(to_u16(kd), kc)
+    assert max_abs_err(oracle, to_u16(out), want) <= TOL
