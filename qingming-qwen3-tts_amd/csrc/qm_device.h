@@ -36,6 +36,16 @@ __device__ __forceinline__ float round_bf16(float x) {
     return static_cast<float>(static_cast<__bf16>(x));
 }
 
+// Two roundings with one v_cvt_pk_bf16_f32.
+__device__ __forceinline__ void round_bf16_pair(float a, float b, float& ra, float& rb) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t in = {a, b};
+    const bf16x2_t packed = __builtin_convertvector(in, bf16x2_t);
+    const uint32_t bits = __builtin_bit_cast(uint32_t, packed);
+    ra = __uint_as_float(bits << 16);
+    rb = __uint_as_float(bits & 0xffff0000U);
+}
+
 __device__ __forceinline__ float lo_bf16(uint32_t packed) { return __uint_as_float(packed << 16); }
 __device__ __forceinline__ float hi_bf16(uint32_t packed) { return __uint_as_float(packed & 0xffff0000U); }
 

@@ -38,6 +38,10 @@ struct PredictorParams {
     float epsilon;
 };
 
+// bf16 round trip with the hardware converter (round to nearest even; same bits as the integer
+// formula of R17:8172-8187 for every non-NaN input).
+__device__ __forceinline__ float rbf(float x) { return round_bf16(x); }
+
 // Sum of squares in the reference order for a head held as (x0 = dim lane, x1 = dim lane+64).
 __device__ __forceinline__ float pred_sum_squares(float x0, float x1) {
     float s0 = x0 * x0;
@@ -51,55 +55,74 @@ __device__ __forceinline__ float pred_sum_squares(float x0, float x1) {
     return __shfl(t, 0) + __shfl(t, 32);
 }
 
-// In-place RMSNorm + RoPE of one 128-wide head in LDS by one wave (same chain as
-// norm_rope_head in qm_norm_rope.hip; R17:12178-12279).
-__device__ __forceinline__ void pred_norm_rope(uint16_t* head, const uint16_t* __restrict__ gamma,
-                                               const uint16_t* __restrict__ cosv,
-                                               const uint16_t* __restrict__ sinv, float epsilon, int lane) {
+// In-place RMSNorm + RoPE of one 128-wide head in LDS by one wave (chain of R17:12178-12279);
+// gamma, cos and sin come from LDS copies.
+__device__ __forceinline__ void pred_norm_rope(uint16_t* head, const uint16_t* gamma, const uint16_t* cosv,
+                                               const uint16_t* sinv, float epsilon, int lane) {
     float w0 = bf2f(head[lane]);
     float w1 = bf2f(head[lane + 64]);
     const float sum = pred_sum_squares(w0, w1);
     const float r = 1.0f / sqrtf(sum / 128.0f + epsilon);
-    w0 = bf2f(f2bf(bf2f(f2bf(w0 * r)) * bf2f(gamma[lane])));
-    w1 = bf2f(f2bf(bf2f(f2bf(w1 * r)) * bf2f(gamma[lane + 64])));
-    const float first0 = bf2f(f2bf(w0 * bf2f(cosv[lane])));
-    const float second0 = bf2f(f2bf((-w1) * bf2f(sinv[lane])));
-    const float first1 = bf2f(f2bf(w1 * bf2f(cosv[lane + 64])));
-    const float second1 = bf2f(f2bf(w0 * bf2f(sinv[lane + 64])));
+    w0 = rbf(rbf(w0 * r) * bf2f(gamma[lane]));
+    w1 = rbf(rbf(w1 * r) * bf2f(gamma[lane + 64]));
+    const float first0 = rbf(w0 * bf2f(cosv[lane]));
+    const float second0 = rbf((-w1) * bf2f(sinv[lane]));
+    const float first1 = rbf(w1 * bf2f(cosv[lane + 64]));
+    const float second1 = rbf(w0 * bf2f(sinv[lane + 64]));
     head[lane] = f2bf(first0 + second0);
     head[lane + 64] = f2bf(first1 + second1);
 }
 
-// Fixed reduction tree of the reference's 32-lane shuffle sum restricted to its first 16 leaves
-// (the other 16 are exact zeros): ((x0+x8)+(x4+x12)) + ((x2+x10)+(x6+x14)) + ... as the
-// shfl_down(8), (4), (2), (1) levels produce it.
-__device__ __forceinline__ float tree16(const float* x) {
-    float b[8], c[4], d[2];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) b[i] = x[i] + x[i + 8];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) c[i] = b[i] + b[i + 4];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) d[i] = c[i] + c[i + 2];
-    return d[0] + d[1];
+// Sum of x[0..N-1] in the shape of the reference's 32-lane shuffle tree (shfl_down 16, 8, 4, 2, 1)
+// whose leaves N..31 are exact +0: adding +0 to a value that is not -0 is the identity, so absent
+// leaves are dropped instead of added.  X(i) must never be -0 (fmaf(p, v, +0) and exp() are not).
+template <int N, int I, int STRIDE>
+struct TreeSum {
+    template <class X>
+    static __device__ __forceinline__ float eval(const X& x) {
+        if constexpr (STRIDE == 0) {
+            return x(I);
+        } else if constexpr (I + STRIDE < N) {
+            return TreeSum<N, I, STRIDE / 2>::eval(x) + TreeSum<N, I + STRIDE, STRIDE / 2>::eval(x);
+        } else {
+            return TreeSum<N, I, STRIDE / 2>::eval(x);
+        }
+    }
+};
+
+template <int R>
+__device__ __forceinline__ void pv_rows(const float (*p)[kPredRows], const float* vcol, uint16_t* out,
+                                        int64_t row_stride, int rows) {
+    if constexpr (R < kPredRows) {
+        if (R < rows) {
+            const float* pr = p[R];
+            // leaf j = fmaf(P[j], V[j][d], +0), keys 0..R (R17:12523-12549)
+            const float o = TreeSum<R + 1, 0, 8>::eval([&](int j) { return fmaf(pr[j], vcol[j], 0.0f); });
+            out[R * row_stride] = f2bf(o);
+            pv_rows<R + 1>(p, vcol, out, row_stride, rows);
+        }
+    }
 }
 
 __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorParams prm) {
     __shared__ __attribute__((aligned(16))) uint16_t sh_q[2][kPredRows][kDim];   // [g][row][d]
     __shared__ __attribute__((aligned(16))) uint16_t sh_k[kPredRows][kDim];
     __shared__ __attribute__((aligned(16))) uint16_t sh_v[kPredRows][kDim];
+    __shared__ __attribute__((aligned(16))) uint16_t sh_cos[kPredRows][kDim];
+    __shared__ __attribute__((aligned(16))) uint16_t sh_sin[kPredRows][kDim];
+    __shared__ __attribute__((aligned(16))) uint16_t sh_gamma[2][kDim];          // q, k
     __shared__ float sh_s[2][kPredRows][kPredRows];                                // scores, then P
+    __shared__ float sh_e[2][kPredRows][kPredRows];                                // exponentials
 
     const int kvh = blockIdx.x;
     const int64_t unit = blockIdx.y;
     const int tid = threadIdx.x;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int rows = prm.rows;
     const int layer = static_cast<int>((prm.unit_base + unit) % prm.n_layers);
 
-    // ---- stage q (2 heads), k, v of this kv head: 16-byte chunks --------------------------------
-    // q: rows x 2 heads x 16 chunks; k, v: rows x 16 chunks each.
+    // ---- stage q (2 heads), k, v of this kv head, the RoPE rows and the two gammas: 16-byte chunks ---
     for (int c = tid; c < rows * 64; c += kPredThreads) {
         const int chunk = c & 15;
         const int which = (c >> 4) & 3;     // 0,1: q head g; 2: k; 3: v
@@ -115,6 +138,19 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
             *reinterpret_cast<uint4*>(which == 2 ? &sh_k[row][chunk * 8] : &sh_v[row][chunk * 8]) = val;
         }
     }
+    for (int c = tid; c < rows * 32 + 32; c += kPredThreads) {
+        const int chunk = c & 15;
+        if (c < rows * 32) {
+            const int row = c >> 5;
+            const bool is_sin = (c >> 4) & 1;
+            const uint4 val = *reinterpret_cast<const uint4*>((is_sin ? prm.sin_rows : prm.cos_rows) + row * kDim + chunk * 8);
+            *reinterpret_cast<uint4*>(is_sin ? &sh_sin[row][chunk * 8] : &sh_cos[row][chunk * 8]) = val;
+        } else {
+            const int which = (c - rows * 32) >> 4;
+            const uint4 val = *reinterpret_cast<const uint4*>((which ? prm.k_norm_w : prm.q_norm_w) + layer * kDim + chunk * 8);
+            *reinterpret_cast<uint4*>(&sh_gamma[which][chunk * 8]) = val;
+        }
+    }
     __syncthreads();
 
     // ---- QK-RMSNorm + RoPE in place: 3*rows heads, one wave each ------------------------------------
@@ -122,8 +158,7 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
         const int row = h / 3;
         const int which = h % 3;            // 0,1: q head g; 2: k
         uint16_t* head = which < 2 ? sh_q[which][row] : sh_k[row];
-        const uint16_t* gamma = (which < 2 ? prm.q_norm_w : prm.k_norm_w) + layer * kDim;
-        pred_norm_rope(head, gamma, prm.cos_rows + row * kDim, prm.sin_rows + row * kDim, prm.epsilon, lane);
+        pred_norm_rope(head, sh_gamma[which < 2 ? 0 : 1], sh_cos[row], sh_sin[row], prm.epsilon, lane);
     }
     __syncthreads();
 
@@ -142,43 +177,100 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
         }
     }
 
-    // ---- scores: one 32-lane half wave per (g, row, key), reference order of operations ------------
+    // ---- scores ---------------------------------------------------------------------------------------
+    // A 32-lane half wave evaluates one query vector against all 16 keys in the reference's order of
+    // operations (R17:12386-12418): lane hl accumulates dims hl, hl+32, hl+64, hl+96 with fmaf, then the
+    // shuffle tree (hl + hl^16, then ^8, ^4, ^2, ^1).  The tree runs as a reduce-scatter: at every level
+    // a lane keeps half of its remaining keys and adds its partner's values for them, which yields the
+    // same sums (fp addition is commutative) with 16 exchanges instead of 80.  Key j ends in lanes
+    // 2j and 2j+1 of the half wave.
     {
         const int half = lane >> 5;
-        const int l = lane & 31;
+        const int hl = lane & 31;
         const float scale = __uint_as_float(0x3db504f3U);   // kAttentionScaleBits, R17:9354-9356
-        for (int idx = wave * 2 + half; idx < 2 * rows * kPredRows; idx += 8) {
-            const int key = idx & 15;
-            const int row = (idx >> 4) % rows;
-            const int g = (idx >> 4) / rows;
-            if (key > row) continue;                          // uniform per half wave
-            const uint16_t* qh = sh_q[g][row];
-            const uint16_t* kh = sh_k[key];
-            float acc = 0.0f;
+        float kf[kPredRows][4];
 #pragma unroll
-            for (int d = 0; d < kDim; d += 32) acc = fmaf(bf2f(qh[l + d]), bf2f(kh[l + d]), acc);
+        for (int j = 0; j < kPredRows; ++j)
 #pragma unroll
-            for (int offset = 16; offset > 0; offset >>= 1) acc += __shfl_down(acc, offset, 32);
-            if (l == 0) {
-                const float raw = bf2f(f2bf(acc));
-                sh_s[g][row][key] = bf2f(f2bf(raw * scale));
+            for (int c = 0; c < 4; ++c) kf[j][c] = bf2f(sh_k[j][hl + 32 * c]);
+        for (int qi = wave * 2 + half; qi < 2 * rows; qi += 8) {
+            const int g = qi / rows;
+            const int row = qi % rows;
+            float q4[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) q4[c] = bf2f(sh_q[g][row][hl + 32 * c]);
+            float x[kPredRows];
+#pragma unroll
+            for (int j = 0; j < kPredRows; ++j) {
+                float acc = 0.0f;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) acc = fmaf(q4[c], kf[j][c], acc);
+                x[j] = acc;
+            }
+            // level 16 -> 8 keys per lane
+            float y8[8], y4[4], y2[2];
+            {
+                const bool up = hl & 16;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float give = up ? x[j] : x[j + 8];
+                    const float keep = up ? x[j + 8] : x[j];
+                    y8[j] = keep + __shfl_xor(give, 16);
+                }
+            }
+            {
+                const bool up = hl & 8;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float give = up ? y8[j] : y8[j + 4];
+                    const float keep = up ? y8[j + 4] : y8[j];
+                    y4[j] = keep + __shfl_xor(give, 8);
+                }
+            }
+            {
+                const bool up = hl & 4;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const float give = up ? y4[j] : y4[j + 2];
+                    const float keep = up ? y4[j + 2] : y4[j];
+                    y2[j] = keep + __shfl_xor(give, 4);
+                }
+            }
+            float y1;
+            {
+                const bool up = hl & 2;
+                const float give = up ? y2[0] : y2[1];
+                const float keep = up ? y2[1] : y2[0];
+                y1 = keep + __shfl_xor(give, 2);
+            }
+            const float total = y1 + __shfl_xor(y1, 1);
+            if ((hl & 1) == 0) {
+                const float raw = rbf(total);
+                sh_s[g][row][hl >> 1] = rbf(raw * scale);
             }
         }
     }
     __syncthreads();
 
-    // ---- softmax rows: thread t < 2*rows owns row (g, r); probabilities rounded to bf16 --------------
-    if (tid < 2 * rows) {
-        const int g = tid / rows, r = tid % rows;
-        float* s = sh_s[g][r];
+    // ---- softmax, spread over all threads: one (g, row, key) element each ---------------------------------
+    for (int i = tid; i < 2 * rows * kPredRows; i += kPredThreads) {
+        const int j = i & 15;
+        const int r = (i >> 4) % rows;
+        const int g = (i >> 4) / rows;
+        const float* s = sh_s[g][r];
         float maximum = -INFINITY;
-        for (int j = 0; j <= r; ++j) maximum = maximum > s[j] ? maximum : s[j];
-        float e[kPredRows];
-#pragma unroll
-        for (int j = 0; j < kPredRows; ++j) e[j] = j <= r ? expf(s[j] - maximum) : 0.0f;
-        const float total = tree16(e);
-#pragma unroll
-        for (int j = 0; j < kPredRows; ++j) s[j] = j <= r ? bf2f(f2bf(e[j] / total)) : 0.0f;
+        for (int t = 0; t <= r; ++t) maximum = maximum > s[t] ? maximum : s[t];
+        sh_e[g][r][j] = j <= r ? expf(s[j] - maximum) : 0.0f;
+    }
+    __syncthreads();
+    for (int i = tid; i < 2 * rows * kPredRows; i += kPredThreads) {
+        const int j = i & 15;
+        const int r = (i >> 4) % rows;
+        const int g = (i >> 4) / rows;
+        const float* e = sh_e[g][r];
+        // exp() >= +0 and masked entries are +0: the full 16-leaf tree equals the reference's sum
+        const float total = TreeSum<16, 0, 8>::eval([&](int t) { return e[t]; });
+        sh_s[g][r][j] = j <= r ? rbf(e[j] / total) : 0.0f;
     }
     __syncthreads();
 
@@ -188,14 +280,9 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
         const int d = tid & 127;
         float vcol[kPredRows];
 #pragma unroll
-        for (int j = 0; j < kPredRows; ++j) vcol[j] = j < rows ? bf2f(sh_v[j][d]) : 0.0f;
-        for (int r = 0; r < rows; ++r) {
-            float x[kPredRows];
-#pragma unroll
-            for (int j = 0; j < kPredRows; ++j) x[j] = j <= r ? fmaf(sh_s[g][r][j], vcol[j], 0.0f) : 0.0f;
-            const float o = tree16(x);
-            prm.out[((unit * rows + r) * 16 + kvh * 2 + g) * kDim + d] = f2bf(o);
-        }
+        for (int j = 0; j < kPredRows; ++j) vcol[j] = bf2f(sh_v[j][d]);
+        uint16_t* out = prm.out + ((unit * rows) * 16 + kvh * 2 + g) * kDim + d;
+        pv_rows<0>(sh_s[g], vcol, out, 16 * kDim, rows);
     }
 }
 

@@ -9,9 +9,11 @@
 // layout of S^T is directly the B-operand layout of O^T += V^T P^T.  V is transposed on its way
 // into LDS ([dim][key slot], key slots permuted to match the accumulator layout).
 //
-// Scheduling.  Blocks are numbered heaviest query tile first, so that the causal triangle packs
-// onto 256 CUs (two blocks per CU) without a long tail; blocks that share K/V differ by a
-// multiple of batch*kv_heads and therefore land on the same XCD and hit its L2.
+// Scheduling.  Blocks are numbered heaviest query tile first, two blocks per CU, so that light
+// tiles fill in behind heavy ones; blocks that share K/V differ by a multiple of batch*kv_heads
+// and therefore land on the same XCD and hit its L2.  (Folding the causal triangle — one block
+// per query-tile pair (n-1-j, j), QM_PF_FOLD=1 — equalises the blocks but leaves one wave per
+// SIMD, and measured slower: the per-wave instruction stream, not the balance, is the limit.)
 //
 // Rounding.  Scores are rounded to bf16 before and after scaling like the reference
 // (R17:15879-15890); softmax runs online in fp32; P enters the P.V MFMA as bf16 — except in the
@@ -29,6 +31,18 @@
 
 #include "qm_device.h"
 #include "qm_host.h"
+
+// Build-time variants kept for measurement: fold query-tile pairs into one block; how many LDS
+// fragment reads are requested ahead of the MFMAs (0 none, 1 K, 2 K and V^T); waves per SIMD.
+#ifndef QM_PF_FOLD
+#define QM_PF_FOLD 0
+#endif
+#ifndef QM_PF_PREFETCH
+#define QM_PF_PREFETCH 2
+#endif
+#ifndef QM_PF_MINWAVES
+#define QM_PF_MINWAVES 2
+#endif
 
 namespace qm {
 
@@ -123,17 +137,18 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     // 8*(c%16).  V: thread (kg = tid/16, dc = tid%16) takes keys 4*kg..4*kg+3, dims 8*dc..+7.
     uint4 kst[4], vst[4];
     const int v_kg = tid >> 4, v_dc = tid & 15;
+    const uint16_t* k_src = prm.k + kv_base + 8 * (tid & 15);
+    const uint16_t* v_src = prm.v + kv_base + 8 * v_dc;
+    // Unpredicated: a key at or beyond S is redirected to the last key; such keys only occur in the
+    // diagonal tile of the last query tile, where the causal mask removes them (key > row).
     auto load_tile = [&](int tile) {
         const int key0 = tile * kBN;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int c = tid + kPfThreads * i;
-            const int key = key0 + (c >> 4);
-            kst[i] = make_uint4(0, 0, 0, 0);
-            if (key < S) kst[i] = *reinterpret_cast<const uint4*>(prm.k + kv_base + key * kv_row + 8 * (c & 15));
-            const int vkey = key0 + 4 * v_kg + i;
-            vst[i] = make_uint4(0, 0, 0, 0);
-            if (vkey < S) vst[i] = *reinterpret_cast<const uint4*>(prm.v + kv_base + vkey * kv_row + 8 * v_dc);
+            const int key = min(key0 + (tid >> 4) + 16 * i, S - 1);
+            kst[i] = *reinterpret_cast<const uint4*>(k_src + key * kv_row);
+            const int vkey = min(key0 + 4 * v_kg + i, S - 1);
+            vst[i] = *reinterpret_cast<const uint4*>(v_src + vkey * kv_row);
         }
     };
     // The block whose query tile equals the key tile also writes those K/V rows to the pages.
@@ -160,13 +175,15 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
             const int c = tid + kPfThreads * i;
             *reinterpret_cast<uint4*>(&sh.k[buf][(c >> 4) * kKS + 8 * (c & 15)]) = kst[i];
         }
-        // transpose 4 keys x 8 dims -> 8 rows of 4 consecutive key slots
+        // transpose 4 keys x 8 dims -> 8 rows of 4 consecutive key slots.  Row d keeps its 8-slot
+        // blocks XOR-swizzled by (d / 8) % 8 so that the 16 lanes that write the same slots of rows
+        // 8 apart do not all hit one LDS bank.
         const int slot0 = 16 * (v_kg >> 2) + key_slot(4 * (v_kg & 3));
+        const int phys = 8 * ((slot0 >> 3) ^ (v_dc & 7)) + (slot0 & 7);
         const uint32_t w[4][4] = {{vst[0].x, vst[0].y, vst[0].z, vst[0].w}, {vst[1].x, vst[1].y, vst[1].z, vst[1].w},
                                   {vst[2].x, vst[2].y, vst[2].z, vst[2].w}, {vst[3].x, vst[3].y, vst[3].z, vst[3].w}};
 #pragma unroll
-        for (int ee = 0; ee < 8; ++ee) {
-            const int e = (ee + v_dc) & 7;          // rotate to spread LDS banks
+        for (int e = 0; e < 8; ++e) {
             const int word = e >> 1;
             uint2 packed;
             if (e & 1) {
@@ -176,7 +193,7 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
                 packed.x = (w[0][word] & 0xffffU) | (w[1][word] << 16);
                 packed.y = (w[2][word] & 0xffffU) | (w[3][word] << 16);
             }
-            *reinterpret_cast<uint2*>(&sh.vt[buf][(8 * v_dc + e) * kVS + slot0]) = packed;
+            *reinterpret_cast<uint2*>(&sh.vt[buf][(8 * v_dc + e) * kVS + phys]) = packed;
         }
     };
 
@@ -206,22 +223,53 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[r] = 0.0f;
             const uint16_t* kp = &sh.k[buf][(32 * half + col) * kKS + 8 * grp];
+            // All eight K fragments are requested before the first MFMA, and the eight V^T
+            // fragments of this half before the softmax arithmetic, so that LDS latency is paid
+            // once per phase instead of once per MFMA.
+#if QM_PF_PREFETCH >= 1
+            bf16x8_t kfr[8];
+#pragma unroll
+            for (int kb = 0; kb < 8; ++kb) kfr[kb] = lds_frag(kp + 16 * kb);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kb = 0; kb < 8; ++kb) {
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[kb], qf[kb], s, 0, 0, 0);
+            }
+#else
 #pragma unroll
             for (int kb = 0; kb < 8; ++kb) {
                 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(kp + 16 * kb), qf[kb], s, 0, 0, 0);
             }
+#endif
+            bf16x8_t vfr[2][4];
+#if QM_PF_PREFETCH >= 2
+#pragma unroll
+            for (int kg = 0; kg < 2; ++kg) {
+                const int sb = 4 * half + 2 * kg + grp;
+#pragma unroll
+                for (int dt = 0; dt < 4; ++dt) {
+                    const int d = 32 * dt + col;
+                    vfr[kg][dt] = lds_frag(&sh.vt[buf][d * kVS + 8 * (sb ^ ((d >> 3) & 7))]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#endif
 
             // ---- reference score roundings, causal mask, online softmax ---------------------------
             float mx = -INFINITY;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float x = round_bf16(round_bf16(s[r]) * prm.scale);
+            for (int r = 0; r < 16; r += 2) {
+                float x0, x1;
+                round_bf16_pair(s[r], s[r + 1], x0, x1);
+                round_bf16_pair(x0 * prm.scale, x1 * prm.scale, x0, x1);
                 if (diagonal) {
                     const int key = key_base + 8 * (r >> 2) + 4 * grp + (r & 3);
-                    if (key > my_row) x = -INFINITY;
+                    if (key > my_row) x0 = -INFINITY;
+                    if (key + 1 > my_row) x1 = -INFINITY;
                 }
-                s[r] = x;
-                mx = fmaxf(mx, x);
+                s[r] = x0;
+                s[r + 1] = x1;
+                mx = fmaxf(mx, fmaxf(x0, x1));
             }
             mx = fmaxf(mx, __shfl_xor(mx, 32));
             const float m_new = fmaxf(m_run, mx);
@@ -257,12 +305,20 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
                     phi[e] = static_cast<__bf16>(pv);
                     if (PRECISE) plo[e] = static_cast<__bf16>(pv - static_cast<float>(phi[e]));
                 }
-                const uint16_t* vp = &sh.vt[buf][col * kVS + 32 * half + 16 * kg + 8 * grp];
+#if QM_PF_PREFETCH < 2
+                {
+                    const int sb = 4 * half + 2 * kg + grp;
+#pragma unroll
+                    for (int dt = 0; dt < 4; ++dt) {
+                        const int d = 32 * dt + col;
+                        vfr[kg][dt] = lds_frag(&sh.vt[buf][d * kVS + 8 * (sb ^ ((d >> 3) & 7))]);
+                    }
+                }
+#endif
 #pragma unroll
                 for (int dt = 0; dt < 4; ++dt) {
-                    const bf16x8_t vf = lds_frag(vp + 32 * dt * kVS);
-                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, phi, o[dt], 0, 0, 0);
-                    if (PRECISE) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, plo, o[dt], 0, 0, 0);
+                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[kg][dt], phi, o[dt], 0, 0, 0);
+                    if (PRECISE) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[kg][dt], plo, o[dt], 0, 0, 0);
                 }
             }
         }
@@ -303,18 +359,31 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     }
 }
 
-// grid = batch * kv_heads * n_qtiles blocks, heaviest query tile first; the first query tile
-// (dispatched last) takes the split-precision P path.
-__global__ __launch_bounds__(kPfThreads, 2) void prefill_causal_kernel(PrefillParams prm, qm_kv_cache cache) {
+// grid = batch * kv_heads * n_qtiles blocks, heaviest query tile first (or, with QM_PF_FOLD, half
+// as many blocks that each work through query tile n_qtiles-1-j and then query tile j).  The
+// first query tile takes the split-precision P path.
+__global__ __launch_bounds__(kPfThreads, QM_PF_MINWAVES) void prefill_causal_kernel(PrefillParams prm, qm_kv_cache cache) {
     extern __shared__ __attribute__((aligned(16))) unsigned char pf_smem[];
     const int pairs = prm.batch * prm.kv_heads;
     const int bid = blockIdx.x;
-    const int qt = prm.n_qtiles - 1 - bid / pairs;
+    const int j = bid / pairs;
     const int pair = bid % pairs;
-    if (qt == 0) {
-        prefill_body<true>(prm, cache, pf_smem, 0, pair);
-    } else {
-        prefill_body<false>(prm, cache, pf_smem, qt, pair);
+    const int heavy = prm.n_qtiles - 1 - j;
+#if !QM_PF_FOLD
+    if (heavy == 0) prefill_body<true>(prm, cache, pf_smem, 0, pair); else prefill_body<false>(prm, cache, pf_smem, heavy, pair);
+    return;
+#endif
+    for (int pass = 0; pass < 2; ++pass) {
+        const int qt = pass == 0 ? heavy : j;
+        if (pass == 1) {
+            if (qt == heavy) break;
+            __syncthreads();   // the output staging of the first pass aliases the K buffers
+        }
+        if (qt == 0) {
+            prefill_body<true>(prm, cache, pf_smem, 0, pair);
+        } else {
+            prefill_body<false>(prm, cache, pf_smem, qt, pair);
+        }
     }
 }
 
@@ -375,7 +444,7 @@ extern "C" int32_t qm_prefill_attention_causal(
         if (e != hipSuccess) return hip_code(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL(prefill_causal_kernel, dim3(static_cast<unsigned>(pairs * n_qtiles)), dim3(kPfThreads), smem, s,
+    hipLaunchKernelGGL(prefill_causal_kernel, dim3(static_cast<unsigned>(QM_PF_FOLD ? pairs * ((n_qtiles + 1) / 2) : pairs * n_qtiles)), dim3(kPfThreads), smem, s,
                        prm, desc);
     return launch_status();
 }
