@@ -26,6 +26,12 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+# HBM bytes per launch of decode_split_kernel<2> on the headline workload, from rocprofv3 --pmc
+# FETCH_SIZE and WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a
+# plain 512 MiB copy (FETCH_SIZE reads half the copied bytes: factor 2.0; WRITE_SIZE: 1.0).
+# Summary and commands: profiles/decode_split_kernel_ragged64_traffic.txt
+HEADLINE_TRAFFIC_BYTES = int((288788.6 * 2.0 + 9528.9 * 1.0) * 1024)
+
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 SCALE = 0.08838834764831845
@@ -339,6 +345,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain 512 MiB device-to-device copies (for scaling rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE counters against a kernel of known traffic)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one MI355X: this path shards without communication (streams / batch / frames), "
@@ -353,6 +362,15 @@ def main():
     qm.lib()
     dev = torch.device("cuda:0")
     props = torch.cuda.get_device_properties(0)
+
+    if args.calibrate_copy:
+        src = torch.empty(512 * 1024 * 1024 // 4, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     head = RaggedDecode(qm, dev)
     ms = _time_steps(head.step, args.steps, args.warmup)
@@ -420,7 +438,7 @@ def main():
                    "q_heads": 16, "kv_heads": 8, "head_dim": 128, "page_size": 16,
                    "device": props.name, "compute_units": props.multi_processor_count},
         "roofline": {"bound": "hbm", "achieved": rep["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": rep["GBps"] / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": rep["GBps"] / HBM_PEAK_GBPS, "traffic": HEADLINE_TRAFFIC_BYTES,
                      "kernel": "decode_split_kernel<2> (+ decode_merge_kernel<2>, both inside the timed step)",
                      "algorithmic_bytes_per_launch": head.bytes, "avg_launch_us": ms * 1e3},
         "cpu_baseline": cpu,

@@ -46,6 +46,13 @@ __device__ __forceinline__ void round_bf16_pair(float a, float b, float& ra, flo
     rb = __uint_as_float(bits & 0xffff0000U);
 }
 
+// (a, b) -> packed bf16 pair, a in the low half (one v_cvt_pk_bf16_f32, round to nearest even).
+__device__ __forceinline__ uint32_t pack_bf16_pair(float a, float b) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t in = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(in, bf16x2_t));
+}
+
 __device__ __forceinline__ float lo_bf16(uint32_t packed) { return __uint_as_float(packed << 16); }
 __device__ __forceinline__ float hi_bf16(uint32_t packed) { return __uint_as_float(packed & 0xffff0000U); }
 

@@ -42,37 +42,6 @@ struct PredictorParams {
 // formula of R17:8172-8187 for every non-NaN input).
 __device__ __forceinline__ float rbf(float x) { return round_bf16(x); }
 
-// Sum of squares in the reference order for a head held as (x0 = dim lane, x1 = dim lane+64).
-__device__ __forceinline__ float pred_sum_squares(float x0, float x1) {
-    float s0 = x0 * x0;
-    float s1 = x1 * x1;
-#pragma unroll
-    for (int offset = 16; offset > 0; offset >>= 1) {
-        s0 += __shfl_down(s0, offset, 32);
-        s1 += __shfl_down(s1, offset, 32);
-    }
-    const float t = s0 + s1;
-    return __shfl(t, 0) + __shfl(t, 32);
-}
-
-// In-place RMSNorm + RoPE of one 128-wide head in LDS by one wave (chain of R17:12178-12279);
-// gamma, cos and sin come from LDS copies.
-__device__ __forceinline__ void pred_norm_rope(uint16_t* head, const uint16_t* gamma, const uint16_t* cosv,
-                                               const uint16_t* sinv, float epsilon, int lane) {
-    float w0 = bf2f(head[lane]);
-    float w1 = bf2f(head[lane + 64]);
-    const float sum = pred_sum_squares(w0, w1);
-    const float r = 1.0f / sqrtf(sum / 128.0f + epsilon);
-    w0 = rbf(rbf(w0 * r) * bf2f(gamma[lane]));
-    w1 = rbf(rbf(w1 * r) * bf2f(gamma[lane + 64]));
-    const float first0 = rbf(w0 * bf2f(cosv[lane]));
-    const float second0 = rbf((-w1) * bf2f(sinv[lane]));
-    const float first1 = rbf(w1 * bf2f(cosv[lane + 64]));
-    const float second1 = rbf(w0 * bf2f(sinv[lane + 64]));
-    head[lane] = f2bf(first0 + second0);
-    head[lane + 64] = f2bf(first1 + second1);
-}
-
 // Sum of x[0..N-1] in the shape of the reference's 32-lane shuffle tree (shfl_down 16, 8, 4, 2, 1)
 // whose leaves N..31 are exact +0: adding +0 to a value that is not -0 is the identity, so absent
 // leaves are dropped instead of added.  X(i) must never be -0 (fmaf(p, v, +0) and exp() are not).
@@ -113,6 +82,8 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
     __shared__ __attribute__((aligned(16))) uint16_t sh_gamma[2][kDim];          // q, k
     __shared__ float sh_s[2][kPredRows][kPredRows];                                // scores, then P
     __shared__ float sh_e[2][kPredRows][kPredRows];                                // exponentials
+    __shared__ float sh_grp[3 * kPredRows][4];                                     // group sums of squares
+    __shared__ float sh_r[3 * kPredRows];                                          // inverse RMS per vector
 
     const int kvh = blockIdx.x;
     const int64_t unit = blockIdx.y;
@@ -153,12 +124,83 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
     }
     __syncthreads();
 
-    // ---- QK-RMSNorm + RoPE in place: 3*rows heads, one wave each ------------------------------------
-    for (int h = wave; h < 3 * rows; h += 4) {
-        const int row = h / 3;
-        const int which = h % 3;            // 0,1: q head g; 2: k
-        uint16_t* head = which < 2 ? sh_q[which][row] : sh_k[row];
-        pred_norm_rope(head, sh_gamma[which < 2 ? 0 : 1], sh_cos[row], sh_sin[row], prm.epsilon, lane);
+    // ---- QK-RMSNorm + RoPE in place over the 3*rows head vectors (2 q heads + k per row) --------------
+    // (1) One thread per (vector, 32-dim group): the group's sum of squares in the order of the
+    //     reference's 32-lane shuffle tree (R17:8233-8245): x[i] + x[i+16], then +8, +4, +2, +1.
+    const int n_vec = 3 * rows;
+    for (int it = tid; it < n_vec * 4; it += kPredThreads) {
+        const int vec = it >> 2, grp = it & 3;
+        const int vrow = vec / 3, which = vec % 3;
+        const uint16_t* x = (which < 2 ? sh_q[which][vrow] : sh_k[vrow]) + 32 * grp;
+        float sq[32];
+#pragma unroll
+        for (int i = 0; i < 32; i += 8) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(x + i);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float a = lo_bf16(w[j]), b = hi_bf16(w[j]);
+                sq[i + 2 * j] = a * a;
+                sq[i + 2 * j + 1] = b * b;
+            }
+        }
+#pragma unroll
+        for (int stride = 16; stride > 0; stride >>= 1)
+#pragma unroll
+            for (int i = 0; i < stride; ++i) sq[i] = sq[i] + sq[i + stride];
+        sh_grp[vec][grp] = sq[0];
+    }
+    __syncthreads();
+    // (2) One thread per vector: (w0 + w2) + (w1 + w3), the reference's tree over the wave sums
+    //     (R17:8262-8271), then 1 / sqrt(mean + eps).
+    if (tid < n_vec) {
+        const float total = (sh_grp[tid][0] + sh_grp[tid][2]) + (sh_grp[tid][1] + sh_grp[tid][3]);
+        sh_r[tid] = 1.0f / sqrtf(total / 128.0f + prm.epsilon);
+    }
+    __syncthreads();
+    // (3) One thread per (vector, four rotate_half pairs): normalise, gamma, RoPE with every bf16
+    //     rounding of R17:12207-12279.
+    for (int it = tid; it < n_vec * 16; it += kPredThreads) {
+        const int vec = it >> 4, d0 = (it & 15) * 4;
+        const int vrow = vec / 3, which = vec % 3;
+        uint16_t* x = which < 2 ? sh_q[which][vrow] : sh_k[vrow];
+        const uint16_t* gamma = sh_gamma[which < 2 ? 0 : 1];
+        const float r = sh_r[vec];
+        const uint2 xl = *reinterpret_cast<const uint2*>(x + d0), xh = *reinterpret_cast<const uint2*>(x + d0 + 64);
+        const uint2 gl = *reinterpret_cast<const uint2*>(gamma + d0), gh = *reinterpret_cast<const uint2*>(gamma + d0 + 64);
+        const uint2 cl = *reinterpret_cast<const uint2*>(&sh_cos[vrow][d0]), ch = *reinterpret_cast<const uint2*>(&sh_cos[vrow][d0 + 64]);
+        const uint2 sl = *reinterpret_cast<const uint2*>(&sh_sin[vrow][d0]), sh2 = *reinterpret_cast<const uint2*>(&sh_sin[vrow][d0 + 64]);
+        const uint32_t xlw[2] = {xl.x, xl.y}, xhw[2] = {xh.x, xh.y}, glw[2] = {gl.x, gl.y}, ghw[2] = {gh.x, gh.y};
+        const uint32_t clw[2] = {cl.x, cl.y}, chw[2] = {ch.x, ch.y}, slw[2] = {sl.x, sl.y}, shw[2] = {sh2.x, sh2.y};
+        uint32_t out_lo[2], out_hi[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            float res_lo[2], res_hi[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const float x0 = e ? hi_bf16(xlw[j]) : lo_bf16(xlw[j]);
+                const float x1 = e ? hi_bf16(xhw[j]) : lo_bf16(xhw[j]);
+                const float g0 = e ? hi_bf16(glw[j]) : lo_bf16(glw[j]);
+                const float g1 = e ? hi_bf16(ghw[j]) : lo_bf16(ghw[j]);
+                const float c0 = e ? hi_bf16(clw[j]) : lo_bf16(clw[j]);
+                const float c1 = e ? hi_bf16(chw[j]) : lo_bf16(chw[j]);
+                const float s0 = e ? hi_bf16(slw[j]) : lo_bf16(slw[j]);
+                const float s1 = e ? hi_bf16(shw[j]) : lo_bf16(shw[j]);
+                float n0, n1, w0, w1, f0, f1, t0, t1;
+                round_bf16_pair(x0 * r, x1 * r, n0, n1);
+                round_bf16_pair(n0 * g0, n1 * g1, w0, w1);
+                round_bf16_pair(w0 * c0, w1 * c1, f0, f1);
+                round_bf16_pair((-w1) * s0, w0 * s1, t0, t1);
+                res_lo[e] = f0 + t0;
+                res_hi[e] = f1 + t1;
+            }
+            float dummy0, dummy1;
+            (void)dummy0; (void)dummy1;
+            out_lo[j] = pack_bf16_pair(res_lo[0], res_lo[1]);
+            out_hi[j] = pack_bf16_pair(res_hi[0], res_hi[1]);
+        }
+        *reinterpret_cast<uint2*>(x + d0) = make_uint2(out_lo[0], out_lo[1]);
+        *reinterpret_cast<uint2*>(x + d0 + 64) = make_uint2(out_hi[0], out_hi[1]);
     }
     __syncthreads();
 

@@ -136,7 +136,12 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     // Global -> register staging of one K/V tile.  K: chunk c = tid + 256*i -> key c/16, dims
     // 8*(c%16).  V: thread (kg = tid/16, dc = tid%16) takes keys 4*kg..4*kg+3, dims 8*dc..+7.
     uint4 kst[4], vst[4];
-    const int v_kg = tid >> 4, v_dc = tid & 15;
+    // V staging: thread (v_kg, v_dc) takes keys 4*v_kg..+3, dims 8*v_dc..+7.  The bits of tid are dealt
+    // so that 16 consecutive lanes hold 8 dim chunks x 2 key groups whose transposed 8-byte LDS
+    // writes fall on 32 different banks (rows 8 apart are XOR-swizzled, the key groups differ by
+    // four slots).
+    const int v_dc = (tid & 7) | (((tid >> 4) & 1) << 3);
+    const int v_kg = ((tid >> 5) & 1) | (((tid >> 3) & 1) << 1) | (((tid >> 6) & 3) << 2);
     const uint16_t* k_src = prm.k + kv_base + 8 * (tid & 15);
     const uint16_t* v_src = prm.v + kv_base + 8 * v_dc;
     // Unpredicated: a key at or beyond S is redirected to the last key; such keys only occur in the
