@@ -32,6 +32,8 @@
 #include "qm_device.h"
 #include "qm_host.h"
 
+#include <type_traits>
+
 // Build-time variants kept for measurement: fold query-tile pairs into one block; how many LDS
 // fragment reads are requested ahead of the MFMAs (0 none, 1 K, 2 K and V^T); waves per SIMD.
 #ifndef QM_PF_FOLD
@@ -131,75 +133,86 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
 
     const int64_t kv_base = static_cast<int64_t>(b) * prm.kv_stride_batch + static_cast<int64_t>(kvh) * prm.kv_stride_head;
     const int64_t kv_row = prm.kv_stride_token;
+    const int kv_row32 = static_cast<int>(kv_row);
     const int32_t* table = prm.page_table ? prm.page_table + static_cast<int64_t>(b) * prm.pages.max_pages : nullptr;
 
     // Global -> register staging of one K/V tile.  K: chunk c = tid + 256*i -> key c/16, dims
     // 8*(c%16).  V: thread (kg = tid/16, dc = tid%16) takes keys 4*kg..4*kg+3, dims 8*dc..+7.
-    uint4 kst[4], vst[4];
+    // (named registers, not arrays: an array here ends up as a stack object and every load is
+    // followed by a wait and a scratch store)
+    uint4 ks0, ks1, ks2, ks3, vs0, vs1, vs2, vs3;
+    auto each_stage = [&](auto&& f) {
+        f(ks0, vs0, 0);
+        f(ks1, vs1, 1);
+        f(ks2, vs2, 2);
+        f(ks3, vs3, 3);
+    };
     // V staging: thread (v_kg, v_dc) takes keys 4*v_kg..+3, dims 8*v_dc..+7.  The bits of tid are dealt
-    // so that 16 consecutive lanes hold 8 dim chunks x 2 key groups whose transposed 8-byte LDS
-    // writes fall on 32 different banks (rows 8 apart are XOR-swizzled, the key groups differ by
-    // four slots).
-    const int v_dc = (tid & 7) | (((tid >> 4) & 1) << 3);
-    const int v_kg = ((tid >> 5) & 1) | (((tid >> 3) & 1) << 1) | (((tid >> 6) & 3) << 2);
+    // so that 32 consecutive lanes hold 16 dim chunks x 2 key groups whose transposed 8-byte LDS
+    // writes fall on 64 different banks: rows 16 apart have their 8-slot blocks XOR-swizzled (which
+    // leaves the 16-lane fragment reads of 16 consecutive rows conflict-free), rows 8 apart differ by
+    // 32 banks through the row stride, and the two key groups differ by four slots.
+    const int v_dc = tid & 15;
+    const int v_kg = ((tid >> 5) & 1) | (((tid >> 4) & 1) << 1) | (((tid >> 6) & 3) << 2);
     const uint16_t* k_src = prm.k + kv_base + 8 * (tid & 15);
     const uint16_t* v_src = prm.v + kv_base + 8 * v_dc;
     // Unpredicated: a key at or beyond S is redirected to the last key; such keys only occur in the
     // diagonal tile of the last query tile, where the causal mask removes them (key > row).
     auto load_tile = [&](int tile) {
         const int key0 = tile * kBN;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        each_stage([&](uint4& kk, uint4& vv, int i) {
+            // (32-bit element offsets: the host rejects seq * stride >= 2^31)
             const int key = min(key0 + (tid >> 4) + 16 * i, S - 1);
-            kst[i] = *reinterpret_cast<const uint4*>(k_src + key * kv_row);
+            kk = *reinterpret_cast<const uint4*>(k_src + static_cast<uint32_t>(key * kv_row32));
             const int vkey = min(key0 + 4 * v_kg + i, S - 1);
-            vst[i] = *reinterpret_cast<const uint4*>(v_src + vkey * kv_row);
-        }
+            vv = *reinterpret_cast<const uint4*>(v_src + static_cast<uint32_t>(vkey * kv_row32));
+        });
     };
     // The block whose query tile equals the key tile also writes those K/V rows to the pages.
     auto write_pages = [&](int tile) {
         const int key0 = tile * kBN;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int c = tid + kPfThreads * i;
-            const int key = key0 + (c >> 4);
+        each_stage([&](uint4& kk, uint4& vv, int i) {
+            const int key = key0 + (tid >> 4) + 16 * i;
             if (key < S) {
                 const int64_t off = tile_offset(cache, prm.pages, table, key, kvh, prm.status);
-                if (off >= 0) *reinterpret_cast<uint4*>(cache.k_pool + off + 8 * (c & 15)) = kst[i];
+                if (off >= 0) *reinterpret_cast<uint4*>(cache.k_pool + off + 8 * (tid & 15)) = kk;
             }
             const int vkey = key0 + 4 * v_kg + i;
             if (vkey < S) {
                 const int64_t off = tile_offset(cache, prm.pages, table, vkey, kvh, prm.status);
-                if (off >= 0) *reinterpret_cast<uint4*>(cache.v_pool + off + 8 * v_dc) = vst[i];
+                if (off >= 0) *reinterpret_cast<uint4*>(cache.v_pool + off + 8 * v_dc) = vv;
             }
-        }
+        });
     };
     auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int c = tid + kPfThreads * i;
-            *reinterpret_cast<uint4*>(&sh.k[buf][(c >> 4) * kKS + 8 * (c & 15)]) = kst[i];
-        }
-        // transpose 4 keys x 8 dims -> 8 rows of 4 consecutive key slots.  Row d keeps its 8-slot
-        // blocks XOR-swizzled by (d / 8) % 8 so that the 16 lanes that write the same slots of rows
-        // 8 apart do not all hit one LDS bank.
+        each_stage([&](uint4& kk, uint4& vv, int i) {
+            (void)vv;
+            *reinterpret_cast<uint4*>(&sh.k[buf][((tid >> 4) + 16 * i) * kKS + 8 * (tid & 15)]) = kk;
+        });
+        // transpose 4 keys x 8 dims -> 8 rows of 4 consecutive key slots; row d keeps its 8-slot
+        // blocks XOR-swizzled by (d / 16) % 8.
         const int slot0 = 16 * (v_kg >> 2) + key_slot(4 * (v_kg & 3));
-        const int phys = 8 * ((slot0 >> 3) ^ (v_dc & 7)) + (slot0 & 7);
-        const uint32_t w[4][4] = {{vst[0].x, vst[0].y, vst[0].z, vst[0].w}, {vst[1].x, vst[1].y, vst[1].z, vst[1].w},
-                                  {vst[2].x, vst[2].y, vst[2].z, vst[2].w}, {vst[3].x, vst[3].y, vst[3].z, vst[3].w}};
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int word = e >> 1;
+        const int phys = 8 * ((slot0 >> 3) ^ ((v_dc >> 1) & 7)) + (slot0 & 7);
+        uint16_t* dst = &sh.vt[buf][(8 * v_dc) * kVS + phys];
+        auto put = [&](int e, uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
             uint2 packed;
             if (e & 1) {
-                packed.x = (w[0][word] >> 16) | (w[1][word] & 0xffff0000U);
-                packed.y = (w[2][word] >> 16) | (w[3][word] & 0xffff0000U);
+                packed.x = (a >> 16) | (b & 0xffff0000U);
+                packed.y = (c >> 16) | (d & 0xffff0000U);
             } else {
-                packed.x = (w[0][word] & 0xffffU) | (w[1][word] << 16);
-                packed.y = (w[2][word] & 0xffffU) | (w[3][word] << 16);
+                packed.x = (a & 0xffffU) | (b << 16);
+                packed.y = (c & 0xffffU) | (d << 16);
             }
-            *reinterpret_cast<uint2*>(&sh.vt[buf][(8 * v_dc + e) * kVS + phys]) = packed;
-        }
+            *reinterpret_cast<uint2*>(dst + e * kVS) = packed;
+        };
+        put(0, vs0.x, vs1.x, vs2.x, vs3.x);
+        put(1, vs0.x, vs1.x, vs2.x, vs3.x);
+        put(2, vs0.y, vs1.y, vs2.y, vs3.y);
+        put(3, vs0.y, vs1.y, vs2.y, vs3.y);
+        put(4, vs0.z, vs1.z, vs2.z, vs3.z);
+        put(5, vs0.z, vs1.z, vs2.z, vs3.z);
+        put(6, vs0.w, vs1.w, vs2.w, vs3.w);
+        put(7, vs0.w, vs1.w, vs2.w, vs3.w);
     };
 
     const int n_tiles = qt + 1;
@@ -254,7 +267,7 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
 #pragma unroll
                 for (int dt = 0; dt < 4; ++dt) {
                     const int d = 32 * dt + col;
-                    vfr[kg][dt] = lds_frag(&sh.vt[buf][d * kVS + 8 * (sb ^ ((d >> 3) & 7))]);
+                    vfr[kg][dt] = lds_frag(&sh.vt[buf][d * kVS + 8 * (sb ^ ((d >> 4) & 7))]);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -316,7 +329,7 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
 #pragma unroll
                     for (int dt = 0; dt < 4; ++dt) {
                         const int d = 32 * dt + col;
-                        vfr[kg][dt] = lds_frag(&sh.vt[buf][d * kVS + 8 * (sb ^ ((d >> 3) & 7))]);
+                        vfr[kg][dt] = lds_frag(&sh.vt[buf][d * kVS + 8 * (sb ^ ((d >> 4) & 7))]);
                     }
                 }
 #endif
@@ -375,8 +388,15 @@ __global__ __launch_bounds__(kPfThreads, QM_PF_MINWAVES) void prefill_causal_ker
     const int pair = bid % pairs;
     const int heavy = prm.n_qtiles - 1 - j;
 #if !QM_PF_FOLD
-    if (heavy == 0) prefill_body<true>(prm, cache, pf_smem, 0, pair); else prefill_body<false>(prm, cache, pf_smem, heavy, pair);
-    return;
+    {
+        // First half of the grid: query tiles from the heaviest down; second half: from the
+        // lightest up.  With two resident blocks per CU the dispatcher's second block on a CU is
+        // then the light partner of its first, so every CU carries about n_qtiles+1 key tiles.
+        const int top = (prm.n_qtiles + 1) / 2;
+        const int qt = j < top ? heavy : j - top;
+        if (qt == 0) prefill_body<true>(prm, cache, pf_smem, 0, pair); else prefill_body<false>(prm, cache, pf_smem, qt, pair);
+        return;
+    }
 #endif
     for (int pass = 0; pass < 2; ++pass) {
         const int qt = pass == 0 ? heavy : j;
@@ -410,6 +430,7 @@ extern "C" int32_t qm_prefill_attention_causal(
     if (kv_stride_token < kDim || kv_stride_head < 0 || kv_stride_batch < 0
         || ((kv_stride_token | kv_stride_head | kv_stride_batch) & 7))
         return QM_ERR_GEOMETRY;
+    if (static_cast<int64_t>(seq) * kv_stride_token >= (1LL << 31)) return QM_ERR_ARGUMENT;
     if (!query || !key || !value || !context_out) return QM_ERR_NULL;
     if (batch < 0 || seq < 0) return QM_ERR_ARGUMENT;
     if (kv_heads <= 0 || q_heads != 2 * kv_heads) return QM_ERR_GEOMETRY;   // GQA pair on the MFMA columns
