@@ -3,17 +3,18 @@
 // Tiling.  A block of four waves owns 64 query rows of one (batch, kv head) and both query heads
 // of the GQA pair: a wave's MFMA column dimension is 32 = 16 rows x 2 heads, so every K and V
 // fragment read from LDS feeds both heads.  Keys are streamed in tiles of 64 through two LDS
-// buffers (global loads for tile i+1 are in flight while tile i is multiplied).  The wave
-// computes S^T = K Q^T with v_mfma_f32_32x32x16_bf16 (keys on MFMA rows, query columns on lanes),
-// so that the softmax statistics of a query column live in one lane pair, and the accumulator
-// layout of S^T is directly the B-operand layout of O^T += V^T P^T.  V is transposed on its way
-// into LDS ([dim][key slot], key slots permuted to match the accumulator layout).
+// buffers (global loads for the next tile are in flight while the current one is multiplied).
+// A wave computes S^T = K Q^T with v_mfma_f32_32x32x16_bf16 (keys on MFMA rows, query columns on
+// lanes), so that the softmax statistics of a query column live in one lane pair, and the
+// accumulator layout of S^T is directly the B-operand layout of O^T += V^T P^T.  V is transposed
+// on its way into LDS ([dim][key slot], key slots permuted to match the accumulator layout).
+// (QM_PF_KSPLIT=2 builds blocks of two wave groups that take alternate key tiles and merge their
+// softmax states through LDS at the end: it shortens the longest block by 15 % but two waves of
+// one block then share each SIMD, and the batch-4 x 1024 case measured 8 % slower.)
 //
-// Scheduling.  Blocks are numbered heaviest query tile first, two blocks per CU, so that light
-// tiles fill in behind heavy ones; blocks that share K/V differ by a multiple of batch*kv_heads
-// and therefore land on the same XCD and hit its L2.  (Folding the causal triangle — one block
-// per query-tile pair (n-1-j, j), QM_PF_FOLD=1 — equalises the blocks but leaves one wave per
-// SIMD, and measured slower: the per-wave instruction stream, not the balance, is the limit.)
+// Scheduling.  Blocks are numbered heaviest query tile first; the hardware hands the next
+// (lighter) block to whichever CU retires one.  Blocks that share K/V differ by a multiple of
+// batch*kv_heads and therefore land on the same XCD and hit its L2.
 //
 // Rounding.  Scores are rounded to bf16 before and after scaling like the reference
 // (R17:15879-15890); softmax runs online in fp32; P enters the P.V MFMA as bf16 — except in the
@@ -34,10 +35,11 @@
 
 #include <type_traits>
 
-// Build-time variants kept for measurement: fold query-tile pairs into one block; how many LDS
-// fragment reads are requested ahead of the MFMAs (0 none, 1 K, 2 K and V^T); waves per SIMD.
-#ifndef QM_PF_FOLD
-#define QM_PF_FOLD 0
+// Build-time variants kept for measurement: how many wave groups split the key tiles of a block
+// (1 or 2); how many LDS fragment reads are requested ahead of the MFMAs (0 none, 1 K, 2 K and
+// V^T); waves per SIMD.
+#ifndef QM_PF_KSPLIT
+#define QM_PF_KSPLIT 1
 #endif
 #ifndef QM_PF_PREFETCH
 #define QM_PF_PREFETCH 2
@@ -48,7 +50,8 @@
 
 namespace qm {
 
-constexpr int kPfThreads = 256;
+constexpr int kPfGroup = 256;                    // threads of one wave group
+constexpr int kPfThreads = kPfGroup * QM_PF_KSPLIT;
 constexpr int kBM = 64;          // query rows per block
 constexpr int kBN = 64;          // keys per tile
 constexpr int kKS = kDim + 8;    // LDS row stride of the K tile (elements)
@@ -94,9 +97,12 @@ __device__ __forceinline__ bf16x8_t lds_frag(const uint16_t* p) {
 template <bool PRECISE>
 __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_kv_cache& cache,
                                              unsigned char* pf_smem, int qt, int pair) {
-    PfShared& sh = *reinterpret_cast<PfShared*>(pf_smem);
+    // Wave group kp (0 .. KSPLIT-1) owns key tiles kp, kp + KSPLIT, ...; it has its own pair of
+    // LDS tile buffers and its own online-softmax state, merged through LDS at the end.
+    const int kp = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 8);
+    PfShared& sh = reinterpret_cast<PfShared*>(pf_smem)[kp];
 
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x & (kPfGroup - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int col = lane & 31;       // MFMA column = (query row % 16, head)
@@ -215,19 +221,25 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
         put(7, vs0.w, vs1.w, vs2.w, vs3.w);
     };
 
-    const int n_tiles = qt + 1;
-    load_tile(0);
-    if (prm.has_cache && qt == 0) write_pages(0);   // (qt is 0 only on the split-precision path)
-    store_tile(0);
+    // Both groups run the same number of iterations (the barrier is block-wide); a group whose
+    // tile index runs past the diagonal idles through the last one.
+    const int n_iter = qt / QM_PF_KSPLIT + 1;
+    if (kp <= qt) {
+        load_tile(kp);
+        if (prm.has_cache && kp == qt) write_pages(kp);
+        store_tile(0);
+    }
     __syncthreads();
 
-    for (int tile = 0; tile < n_tiles; ++tile) {
-        const int buf = tile & 1;
-        const bool more = tile + 1 < n_tiles;
+    for (int it = 0; it < n_iter; ++it) {
+        const int tile = it * QM_PF_KSPLIT + kp;
+        const int buf = it & 1;
+        const bool more = tile + QM_PF_KSPLIT <= qt;
         if (more) {
-            load_tile(tile + 1);
-            if (prm.has_cache && tile + 1 == qt) write_pages(tile + 1);
+            load_tile(tile + QM_PF_KSPLIT);
+            if (prm.has_cache && tile + QM_PF_KSPLIT == qt) write_pages(tile + QM_PF_KSPLIT);
         }
+        if (tile <= qt) {
         const bool diagonal = tile == qt;
 
 #pragma unroll
@@ -341,14 +353,49 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
             }
         }
 
+        }   // tile <= qt
+
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     }
 
+#if QM_PF_KSPLIT == 2
+    // ---- merge the two key groups: group 1 hands its (O, max, sum) to group 0 through LDS --------
+    {
+        float* xo = reinterpret_cast<float*>(pf_smem);                 // [wave][64 regs][64 lanes]
+        float* xm = xo + 4 * 64 * 64;                                  // [wave][2][64 lanes]
+        if (kp == 1) {
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) xo[(wave * 64 + dt * 16 + r) * 64 + lane] = o[dt][r];
+            xm[(wave * 2 + 0) * 64 + lane] = m_run;
+            xm[(wave * 2 + 1) * 64 + lane] = l_run;
+        }
+        __syncthreads();
+        if (kp == 1) return;
+        const float m1 = xm[(wave * 2 + 0) * 64 + lane];
+        const float l1 = xm[(wave * 2 + 1) * 64 + lane];
+        const float mm = fmaxf(m_run, m1);
+        const float m_ref = mm == -INFINITY ? 0.0f : mm;
+        const float a0 = fast_exp2((m_run - m_ref) * kLog2e);
+        const float a1 = fast_exp2((m1 - m_ref) * kLog2e);
+        l_run = l_run * a0 + l1 * a1;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                o[dt][r] = fmaf(o[dt][r], a0, xo[(wave * 64 + dt * 16 + r) * 64 + lane] * a1);
+    }
+    constexpr int kStageOffset = 4 * 64 * 64 * 4 + 4 * 2 * 64 * 4;   // bytes, behind the exchange area
+#else
+    constexpr int kStageOffset = 0;
+#endif
+
     // ---- normalise, stage through LDS, write 16 bytes per lane -------------------------------------
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-    uint16_t* stage = reinterpret_cast<uint16_t*>(pf_smem) + wave * 32 * kOS;   // 32 columns x 128 dims per wave
+    uint16_t* stage = reinterpret_cast<uint16_t*>(pf_smem + kStageOffset) + wave * 32 * kOS;   // 32 columns x 128 dims per wave
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) {
 #pragma unroll
@@ -377,38 +424,19 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     }
 }
 
-// grid = batch * kv_heads * n_qtiles blocks, heaviest query tile first (or, with QM_PF_FOLD, half
-// as many blocks that each work through query tile n_qtiles-1-j and then query tile j).  The
+// grid = batch * kv_heads * n_qtiles blocks, heaviest query tile first: the hardware hands the
+// next (lighter) block to whichever CU retires one, which pairs heavy with light tiles.  The
 // first query tile takes the split-precision P path.
 __global__ __launch_bounds__(kPfThreads, QM_PF_MINWAVES) void prefill_causal_kernel(PrefillParams prm, qm_kv_cache cache) {
     extern __shared__ __attribute__((aligned(16))) unsigned char pf_smem[];
     const int pairs = prm.batch * prm.kv_heads;
     const int bid = blockIdx.x;
-    const int j = bid / pairs;
+    const int qt = prm.n_qtiles - 1 - bid / pairs;
     const int pair = bid % pairs;
-    const int heavy = prm.n_qtiles - 1 - j;
-#if !QM_PF_FOLD
-    {
-        // First half of the grid: query tiles from the heaviest down; second half: from the
-        // lightest up.  With two resident blocks per CU the dispatcher's second block on a CU is
-        // then the light partner of its first, so every CU carries about n_qtiles+1 key tiles.
-        const int top = (prm.n_qtiles + 1) / 2;
-        const int qt = j < top ? heavy : j - top;
-        if (qt == 0) prefill_body<true>(prm, cache, pf_smem, 0, pair); else prefill_body<false>(prm, cache, pf_smem, qt, pair);
-        return;
-    }
-#endif
-    for (int pass = 0; pass < 2; ++pass) {
-        const int qt = pass == 0 ? heavy : j;
-        if (pass == 1) {
-            if (qt == heavy) break;
-            __syncthreads();   // the output staging of the first pass aliases the K buffers
-        }
-        if (qt == 0) {
-            prefill_body<true>(prm, cache, pf_smem, 0, pair);
-        } else {
-            prefill_body<false>(prm, cache, pf_smem, qt, pair);
-        }
+    if (qt == 0) {
+        prefill_body<true>(prm, cache, pf_smem, 0, pair);
+    } else {
+        prefill_body<false>(prm, cache, pf_smem, qt, pair);
     }
 }
 
@@ -462,7 +490,7 @@ extern "C" int32_t qm_prefill_attention_causal(
     prm.batch = batch; prm.seq = seq; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
 
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
-    const size_t smem = sizeof(PfShared);
+    const size_t smem = sizeof(PfShared) * QM_PF_KSPLIT;
     static bool attr_set = false;
     if (!attr_set) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_causal_kernel),
@@ -470,7 +498,7 @@ extern "C" int32_t qm_prefill_attention_causal(
         if (e != hipSuccess) return hip_code(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL(prefill_causal_kernel, dim3(static_cast<unsigned>(QM_PF_FOLD ? pairs * ((n_qtiles + 1) / 2) : pairs * n_qtiles)), dim3(kPfThreads), smem, s,
+    hipLaunchKernelGGL(prefill_causal_kernel, dim3(static_cast<unsigned>(pairs * n_qtiles)), dim3(kPfThreads), smem, s,
                        prm, desc);
     return launch_status();
 }
