@@ -345,6 +345,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
+    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "predictor"], default=None,
+                    help="time just one of the other configurations and print its record (for profiling one "
+                         "kernel under rocprofv3); the headline line is not produced")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 512 MiB device-to-device copies (for scaling rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters against a kernel of known traffic)")
@@ -371,6 +374,16 @@ def main():
         torch.cuda.synchronize()
         del src, dst
         torch.cuda.empty_cache()
+
+    if args.only:
+        make = {"decode512": lambda: SingleDecode(qm, dev, 512, False, 11),
+                "talker2048": lambda: SingleDecode(qm, dev, 2048, True, 12),
+                "prefill": lambda: Prefill(qm, dev), "predictor": lambda: PredictorLoop(qm, dev)}[args.only]
+        w = make()
+        r = _report(w, _time_steps(w.step, args.steps, args.warmup))
+        r["bound"] = w.bound
+        print(json.dumps(r))
+        return
 
     head = RaggedDecode(qm, dev)
     ms = _time_steps(head.step, args.steps, args.warmup)
