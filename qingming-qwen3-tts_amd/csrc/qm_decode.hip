@@ -35,7 +35,7 @@ constexpr int kDecodeThreads = 256;
 constexpr int kDecodeWaves = 4;
 constexpr int kRowStreams = 16;  // 4 waves x 4 DPP rows
 constexpr int kMaxTilesPerBlock = 64;
-constexpr int kMaxSplitsMerged = 64;   // splits merged per LDS round in the merge kernel
+constexpr int kMergeRound = 32;        // splits merged per round of loads in the merge kernel
 
 struct DecodeParams {
     const uint16_t* query;        // [n_streams][q_heads][128]
@@ -304,34 +304,51 @@ __global__ void decode_merge_kernel(DecodeParams prm) {
     const int qh = kvh * G + g;
     uint16_t* dst = prm.out + (static_cast<int64_t>(stream) * prm.q_heads + qh) * kDim + d;
 
-    int key_start = prm.fixed_key_start;
-    int key_end = prm.fixed_key_end;
-    if (prm.seq_lens) {
-        key_start = 0;
-        key_end = min(prm.seq_lens[stream], prm.max_seq_len);
-    }
-    if (key_end <= key_start) {
-        *dst = 0;
-        return;
-    }
-    const int tiles = (key_end - 1) / kTile - key_start / kTile + 1;
-    const int splits = min((tiles + prm.tiles_per_block - 1) / prm.tiles_per_block, prm.max_splits);
     const float* base = prm.partial
         + (static_cast<int64_t>(stream) * gridDim.x + kvh) * prm.max_splits * partial_floats<G>();
 
-    // Statistics of all splits go through LDS in one round of loads; the accumulator column of
-    // each thread is then summed with independent (pipelined) loads.
-    __shared__ float sh_w[kMaxSplitsMerged][G];
-    __shared__ float sh_l[kMaxSplitsMerged][G];
+    // All loads of a round — the context length, the statistics of up to kMergeRound splits and
+    // this thread's accumulator column of each — are issued before anything is consumed, so the
+    // kernel pays one memory latency per round.  Records of splits that do not exist hold
+    // stale workspace contents; they are read (the addresses are valid) and then ignored.
+    __shared__ float sh_w[kMergeRound][G];
+    __shared__ float sh_l[kMergeRound][G];
     float ll = 0.0f, aa = 0.0f;
     float m_run = -INFINITY;
-    for (int s0 = 0; s0 < splits; s0 += kMaxSplitsMerged) {
-        const int n = min(splits - s0, kMaxSplitsMerged);
+    int splits = 0;
+    for (int s0 = 0; s0 < prm.max_splits; s0 += kMergeRound) {
+        const int cap = min(prm.max_splits - s0, kMergeRound);
+        float stat_m = 0.0f, stat_l = 0.0f;
+        if (static_cast<int>(threadIdx.x) < cap * G) {
+            const float* rec = base + static_cast<int64_t>(s0 + threadIdx.x / G) * partial_floats<G>();
+            stat_m = rec[G * kDim + threadIdx.x % G];
+            stat_l = rec[G * kDim + G + threadIdx.x % G];
+        }
+        float part[kMergeRound];
+#pragma unroll
+        for (int u = 0; u < kMergeRound; ++u) {
+            part[u] = u < cap ? base[static_cast<int64_t>(s0 + u) * partial_floats<G>() + g * kDim + d] : 0.0f;
+        }
+        if (s0 == 0) {
+            int key_start = prm.fixed_key_start;
+            int key_end = prm.fixed_key_end;
+            if (prm.seq_lens) {
+                key_start = 0;
+                key_end = min(prm.seq_lens[stream], prm.max_seq_len);
+            }
+            if (key_end <= key_start) {
+                *dst = 0;
+                return;
+            }
+            const int tiles = (key_end - 1) / kTile - key_start / kTile + 1;
+            splits = min((tiles + prm.tiles_per_block - 1) / prm.tiles_per_block, prm.max_splits);
+        }
+        const int n = min(splits - s0, cap);
+        if (n <= 0) break;
         __syncthreads();
-        for (int i = threadIdx.x; i < n * G; i += blockDim.x) {
-            const float* rec = base + static_cast<int64_t>(s0 + i / G) * partial_floats<G>();
-            sh_w[i / G][i % G] = rec[G * kDim + i % G];
-            sh_l[i / G][i % G] = rec[G * kDim + G + i % G];
+        if (static_cast<int>(threadIdx.x) < cap * G) {
+            sh_w[threadIdx.x / G][threadIdx.x % G] = stat_m;
+            sh_l[threadIdx.x / G][threadIdx.x % G] = stat_l;
         }
         __syncthreads();
         float mm = m_run;
@@ -341,19 +358,12 @@ __global__ void decode_merge_kernel(DecodeParams prm) {
         ll *= rescale;
         aa *= rescale;
         m_run = mm;
-        float part[8];
-        for (int s = 0; s < n; s += 8) {
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                part[u] = s + u < n ? base[static_cast<int64_t>(s0 + s + u) * partial_floats<G>() + g * kDim + d] : 0.0f;
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                if (s + u < n) {
-                    const float w = fast_exp2((sh_w[s + u][g] - m_ref) * kLog2e);
-                    ll = fmaf(sh_l[s + u][g], w, ll);
-                    aa = fmaf(part[u], w, aa);
-                }
+        for (int u = 0; u < kMergeRound; ++u) {
+            if (u < n) {
+                const float w = fast_exp2((sh_w[u][g] - m_ref) * kLog2e);
+                ll = fmaf(sh_l[u][g], w, ll);
+                aa = fmaf(part[u], w, aa);
             }
         }
     }
