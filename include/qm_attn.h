@@ -76,6 +76,22 @@ const char* qm_error_string(int32_t code);
 /* Names the architecture the kernels were compiled for ("gfx950"). */
 const char* qm_target_arch(void);
 
+/* Process-wide tuning options; they have no counterpart in the reference, whose kernels have
+ * one fixed behaviour.  A call reads the options when it is enqueued.
+ *   QM_OPT_PREFILL_SCORE_ROUNDING  1 (default): qm_prefill_attention_causal rounds raw and scaled
+ *       scores to bf16 like the reference (R17:15879-15890); 0: scores stay fp32 (faster; needs
+ *       scale > 0; outputs stay within the 1e-2 tolerance of the fp32 definition).
+ *   QM_OPT_DECODE_TILES_PER_BLOCK  0 (default): the split-K decode picks the 16-token tiles per
+ *       block from the problem size; > 0 forces it (changes qm_decode_workspace_bytes too). */
+enum {
+    QM_OPT_PREFILL_SCORE_ROUNDING = 0,
+    QM_OPT_DECODE_TILES_PER_BLOCK = 1,
+    QM_OPT_COUNT = 2
+};
+/* Returns QM_ERR_ARGUMENT for an unknown option or a negative value. */
+int32_t qm_set_option(int32_t option, int32_t value);
+int32_t qm_get_option(int32_t option, int32_t* value);
+
 /* ---- (1) fused QK-RMSNorm + RoPE + KV append ------------------------------------- */
 /*
  * Replaces NativeTalkerEngine::launch_qk_norm_rope_cache_m1 (R17:17569-17606, kernel

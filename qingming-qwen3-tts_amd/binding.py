@@ -45,6 +45,8 @@ _SIGNATURES = {
     "qm_abi_version": (C.c_int32, []),
     "qm_error_string": (C.c_char_p, [_I32]),
     "qm_target_arch": (C.c_char_p, []),
+    "qm_set_option": (_I32, [_I32, _I32]),
+    "qm_get_option": (_I32, [_I32, C.POINTER(_I32)]),
     "qm_qk_norm_rope_kv_append": (_I32, [_PTR] * 8 + [C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _F32, _PTR]),
     "qm_qk_norm_rope_kv_append_ragged": (_I32, [_PTR] * 7 + [_I32, _PTR, C.POINTER(KvCache), _PTR, _I32, _PTR,
                                                  _I32, _I32, _F32, _PTR, _PTR]),
@@ -95,6 +97,20 @@ def _addr(x):
 def _check(code, what):
     if code != 0:
         raise QmError(code, what)
+
+
+OPT_PREFILL_SCORE_ROUNDING = 0
+OPT_DECODE_TILES_PER_BLOCK = 1
+
+
+def set_option(option, value):
+    _check(lib().qm_set_option(option, value), "qm_set_option")
+
+
+def get_option(option):
+    out = C.c_int32(0)
+    _check(lib().qm_get_option(option, C.byref(out)), "qm_get_option")
+    return out.value
 
 
 def paged_cache(k_pool, v_pool, n_pages, kv_heads=8, page_size=16):

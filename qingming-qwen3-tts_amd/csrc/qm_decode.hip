@@ -380,8 +380,7 @@ struct DecodePlan {
 
 inline DecodePlan plan_decode(int n_streams, int kv_heads, int max_seq_len) {
     const int64_t max_tiles = (static_cast<int64_t>(max_seq_len) + kTile - 1) / kTile + 1;
-    int tiles_per_block = 0;
-    if (const char* env = getenv("QM_DECODE_TILES_PER_BLOCK")) tiles_per_block = atoi(env);
+    int tiles_per_block = option_value(QM_OPT_DECODE_TILES_PER_BLOCK);
     if (tiles_per_block <= 0) {
         // One tile per wave at least; otherwise 8 tiles (128 tokens, 64 KiB of K+V) per block:
         // measured best for ragged batches (short blocks keep the tail of the grid short; the

@@ -39,6 +39,9 @@ inline int32_t check_group(int32_t q_heads, int32_t kv_heads) {
     return QM_OK;
 }
 
+// Process-wide tuning options (qm_set_option); defined with the library's other global entry points.
+int32_t option_value(int32_t option);
+
 inline int32_t launch_status() { return hip_code(hipGetLastError()); }
 
 }  // namespace qm

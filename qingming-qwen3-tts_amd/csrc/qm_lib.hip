@@ -2,6 +2,8 @@
 
 #include "qm_host.h"
 
+#include <atomic>
+
 extern "C" int32_t qm_abi_version(void) { return 1; }
 
 extern "C" const char* qm_target_arch(void) { return "gfx950"; }
@@ -19,4 +21,34 @@ extern "C" const char* qm_error_string(int32_t code) {
     }
     if (code <= QM_ERR_HIP_BASE) return hipGetErrorString(static_cast<hipError_t>(QM_ERR_HIP_BASE - code));
     return "unknown error";
+}
+
+namespace qm {
+
+namespace {
+std::atomic<int32_t> g_options[QM_OPT_COUNT] = {
+    {1},   // QM_OPT_PREFILL_SCORE_ROUNDING
+    {0},   // QM_OPT_DECODE_TILES_PER_BLOCK (0 = chosen from the problem size)
+};
+}  // namespace
+
+int32_t option_value(int32_t option) {
+    return g_options[option].load(std::memory_order_relaxed);
+}
+
+}  // namespace qm
+
+extern "C" int32_t qm_set_option(int32_t option, int32_t value) {
+    if (option < 0 || option >= QM_OPT_COUNT) return QM_ERR_ARGUMENT;
+    if (value < 0) return QM_ERR_ARGUMENT;
+    if (option == QM_OPT_DECODE_TILES_PER_BLOCK && value > 4096) return QM_ERR_ARGUMENT;
+    qm::g_options[option].store(value, std::memory_order_relaxed);
+    return QM_OK;
+}
+
+extern "C" int32_t qm_get_option(int32_t option, int32_t* value) {
+    if (!value) return QM_ERR_NULL;
+    if (option < 0 || option >= QM_OPT_COUNT) return QM_ERR_ARGUMENT;
+    *value = qm::option_value(option);
+    return QM_OK;
 }

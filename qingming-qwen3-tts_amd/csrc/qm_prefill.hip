@@ -3,23 +3,35 @@
 // Tiling.  A block of four waves owns 64 query rows of one (batch, kv head) and both query heads
 // of the GQA pair: a wave's MFMA column dimension is 32 = 16 rows x 2 heads, so every K and V
 // fragment read from LDS feeds both heads.  Keys are streamed in tiles of 64 through two LDS
-// buffers (global loads for the next tile are in flight while the current one is multiplied).
+// stages (global loads for the next tile are in flight while the current one is multiplied).
 // A wave computes S^T = K Q^T with v_mfma_f32_32x32x16_bf16 (keys on MFMA rows, query columns on
 // lanes), so that the softmax statistics of a query column live in one lane pair, and the
 // accumulator layout of S^T is directly the B-operand layout of O^T += V^T P^T.  V is transposed
-// on its way into LDS ([dim][key slot], key slots permuted to match the accumulator layout).
-// (QM_PF_KSPLIT=2 builds blocks of two wave groups that take alternate key tiles and merge their
-// softmax states through LDS at the end: it shortens the longest block by 15 % but two waves of
-// one block then share each SIMD, and the batch-4 x 1024 case measured 8 % slower.)
+// on its way into LDS ([dim][key slot], key slots permuted to match the accumulator layout,
+// 8-slot blocks XOR-swizzled per 16 rows so both the transposing writes and the fragment reads
+// are conflict-free).
+//
+// Occupancy.  A wave cannot issue VALU work in the shadow of its own MFMAs (measured: one MFMA
+// plus eight independent FMAs take the sum of both), so the matrix pipe and the VALU only overlap
+// between waves: the kernel stays within 256 registers and 72 KB of LDS so that two blocks share
+// a CU, and a software pipeline inside the wave (tried, with three LDS stages and 316 registers)
+// brought nothing.
+//
+// Lazy rescale.  The running maximum of a column is only raised when a chunk exceeds it by more
+// than kRescaleSlack (then O and the running sum are rescaled); otherwise probabilities are taken
+// relative to the slightly stale maximum and may reach e^slack, which bf16 P and the fp32
+// accumulators hold without loss of relative precision.
 //
 // Scheduling.  Blocks are numbered heaviest query tile first; the hardware hands the next
 // (lighter) block to whichever CU retires one.  Blocks that share K/V differ by a multiple of
 // batch*kv_heads and therefore land on the same XCD and hit its L2.
 //
-// Rounding.  Scores are rounded to bf16 before and after scaling like the reference
-// (R17:15879-15890); softmax runs online in fp32; P enters the P.V MFMA as bf16 — except in the
-// first query tile, whose rows have so few keys that outputs are large: there P is split into
-// hi + lo bf16 parts (two MFMAs) to stay inside the 1e-2 output tolerance.
+// Rounding.  With score rounding on (the default) scores are rounded to bf16 before and after
+// scaling like the reference (R17:15879-15890); with it off they stay fp32 (8 VALU instructions
+// fewer per score pair).  Softmax runs online in fp32; P enters the P.V MFMA as bf16 and the running
+// sum adds the same rounded values — except in the first query tile, whose rows have so few keys
+// that outputs are large: there P is split into hi + lo bf16 parts (two MFMAs) to stay inside the
+// 1e-2 output tolerance.
 //
 // Causality.  A key after a query row never contributes; keys of later 16-row groups are not
 // read into the product at all.  Inside a wave's own 16-row diagonal group the mask is P = 0
@@ -28,35 +40,24 @@
 //
 // Algorithmic work per (batch, kv head): flops = 2 heads * 2 matmuls * 2 * 128 * S(S+1)/2;
 // HBM bytes = Q + O (2 heads) + K + V read once + K + V written to pages.  Bound: MFMA (with the
-// softmax VALU work — 16 exponentials per lane per 32 keys — as the practical limiter).
+// softmax VALU work — 16 exponentials and two bf16 roundings per lane per 32 keys — as the
+// practical limiter).
 
 #include "qm_device.h"
 #include "qm_host.h"
 
 #include <type_traits>
 
-// Build-time variants kept for measurement: how many wave groups split the key tiles of a block
-// (1 or 2); how many LDS fragment reads are requested ahead of the MFMAs (0 none, 1 K, 2 K and
-// V^T); waves per SIMD.
-#ifndef QM_PF_KSPLIT
-#define QM_PF_KSPLIT 1
-#endif
-#ifndef QM_PF_PREFETCH
-#define QM_PF_PREFETCH 2
-#endif
-#ifndef QM_PF_MINWAVES
-#define QM_PF_MINWAVES 2
-#endif
-
 namespace qm {
 
-constexpr int kPfGroup = 256;                    // threads of one wave group
-constexpr int kPfThreads = kPfGroup * QM_PF_KSPLIT;
+constexpr int kPfThreads = 256;
+constexpr int kPfStages = 2;
 constexpr int kBM = 64;          // query rows per block
 constexpr int kBN = 64;          // keys per tile
 constexpr int kKS = kDim + 8;    // LDS row stride of the K tile (elements)
 constexpr int kVS = kBN + 8;     // LDS row stride of the V^T tile (elements)
 constexpr int kOS = kDim + 8;    // LDS row stride of the output staging tile
+constexpr float kRescaleSlack = 6.0f;
 
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
@@ -79,9 +80,15 @@ struct PrefillParams {
     float scale;
 };
 
-struct PfShared {
-    uint16_t k[2][kBN * kKS];
-    uint16_t vt[2][kDim * kVS];
+struct PfStage {
+    uint16_t k[kBN * kKS];
+    uint16_t vt[kDim * kVS];
+};
+
+// P of one 32-key chunk as MFMA B operands: two 16-key groups; lo only in the split-precision path.
+struct PFrag {
+    bf16x8_t hi[2];
+    bf16x8_t lo[2];
 };
 
 // LDS slot of key j (0..15) inside a 16-key group: MFMA k index 8*g + e holds the key that the
@@ -94,15 +101,25 @@ __device__ __forceinline__ bf16x8_t lds_frag(const uint16_t* p) {
     return *reinterpret_cast<const bf16x8_t*>(p);
 }
 
-template <bool PRECISE>
+// Both 32-lane halves receive max / sum over the two halves (v_permlane32_swap).
+__device__ __forceinline__ float halves_max(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float halves_sum(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+template <int N> using int_c = std::integral_constant<int, N>;
+template <bool B> using bool_c = std::integral_constant<bool, B>;
+
+template <bool PRECISE, bool ROUND>
 __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_kv_cache& cache,
                                              unsigned char* pf_smem, int qt, int pair) {
-    // Wave group kp (0 .. KSPLIT-1) owns key tiles kp, kp + KSPLIT, ...; it has its own pair of
-    // LDS tile buffers and its own online-softmax state, merged through LDS at the end.
-    const int kp = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 8);
-    PfShared& sh = reinterpret_cast<PfShared*>(pf_smem)[kp];
+    PfStage* st = reinterpret_cast<PfStage*>(pf_smem);
 
-    const int tid = threadIdx.x & (kPfGroup - 1);
+    const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int col = lane & 31;       // MFMA column = (query row % 16, head)
@@ -116,6 +133,7 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     const int q0 = qt * kBM;
     const int my_row = q0 + 16 * wave + (col & 15);   // query row of this lane's column
     const int my_head = 2 * kvh + (col >> 4);
+    const int wave_last_row = q0 + 16 * wave + 15;
 
     // ---- Q fragments (B operand): dims 16*kb + 8*grp .. +7 of this lane's column ----------------
     bf16x8_t qf[8];
@@ -138,12 +156,11 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     float l_run = 0.0f;
 
     const int64_t kv_base = static_cast<int64_t>(b) * prm.kv_stride_batch + static_cast<int64_t>(kvh) * prm.kv_stride_head;
-    const int64_t kv_row = prm.kv_stride_token;
-    const int kv_row32 = static_cast<int>(kv_row);
+    const int kv_row32 = static_cast<int>(prm.kv_stride_token);   // (the host rejects seq * stride >= 2^31)
     const int32_t* table = prm.page_table ? prm.page_table + static_cast<int64_t>(b) * prm.pages.max_pages : nullptr;
 
     // Global -> register staging of one K/V tile.  K: chunk c = tid + 256*i -> key c/16, dims
-    // 8*(c%16).  V: thread (kg = tid/16, dc = tid%16) takes keys 4*kg..4*kg+3, dims 8*dc..+7.
+    // 8*(c%16).  V: thread (v_kg, v_dc) takes keys 4*v_kg..+3, dims 8*v_dc..+7.
     // (named registers, not arrays: an array here ends up as a stack object and every load is
     // followed by a wait and a scratch store)
     uint4 ks0, ks1, ks2, ks3, vs0, vs1, vs2, vs3;
@@ -153,26 +170,36 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
         f(ks2, vs2, 2);
         f(ks3, vs3, 3);
     };
-    // V staging: thread (v_kg, v_dc) takes keys 4*v_kg..+3, dims 8*v_dc..+7.  The bits of tid are dealt
-    // so that 32 consecutive lanes hold 16 dim chunks x 2 key groups whose transposed 8-byte LDS
-    // writes fall on 64 different banks: rows 16 apart have their 8-slot blocks XOR-swizzled (which
-    // leaves the 16-lane fragment reads of 16 consecutive rows conflict-free), rows 8 apart differ by
-    // 32 banks through the row stride, and the two key groups differ by four slots.
+    // The bits of tid are dealt so that 32 consecutive lanes hold 16 dim chunks x 2 key groups
+    // whose transposed 8-byte LDS writes fall on 64 different banks: rows 16 apart have their
+    // 8-slot blocks XOR-swizzled (which leaves the 16-lane fragment reads of 16 consecutive rows
+    // conflict-free), rows 8 apart differ by 32 banks through the row stride, and the two key
+    // groups differ by four slots.
     const int v_dc = tid & 15;
     const int v_kg = ((tid >> 5) & 1) | (((tid >> 4) & 1) << 1) | (((tid >> 6) & 3) << 2);
     const uint16_t* k_src = prm.k + kv_base + 8 * (tid & 15);
     const uint16_t* v_src = prm.v + kv_base + 8 * v_dc;
-    // Unpredicated: a key at or beyond S is redirected to the last key; such keys only occur in the
-    // diagonal tile of the last query tile, where the causal mask removes them (key > row).
+    const uint32_t k_lane_off = static_cast<uint32_t>((tid >> 4) * kv_row32);
+    const uint32_t v_lane_off = static_cast<uint32_t>(4 * v_kg * kv_row32);
     auto load_tile = [&](int tile) {
         const int key0 = tile * kBN;
-        each_stage([&](uint4& kk, uint4& vv, int i) {
-            // (32-bit element offsets: the host rejects seq * stride >= 2^31)
-            const int key = min(key0 + (tid >> 4) + 16 * i, S - 1);
-            kk = *reinterpret_cast<const uint4*>(k_src + static_cast<uint32_t>(key * kv_row32));
-            const int vkey = min(key0 + 4 * v_kg + i, S - 1);
-            vv = *reinterpret_cast<const uint4*>(v_src + static_cast<uint32_t>(vkey * kv_row32));
-        });
+        if (key0 + kBN <= S) {
+            const uint16_t* kt = k_src + static_cast<uint32_t>(key0 * kv_row32);
+            const uint16_t* vt = v_src + static_cast<uint32_t>(key0 * kv_row32);
+            each_stage([&](uint4& kk, uint4& vv, int i) {
+                kk = *reinterpret_cast<const uint4*>(kt + (k_lane_off + static_cast<uint32_t>(16 * i * kv_row32)));
+                vv = *reinterpret_cast<const uint4*>(vt + (v_lane_off + static_cast<uint32_t>(i * kv_row32)));
+            });
+        } else {
+            // A key at or beyond S is redirected to the last key; such keys only occur in the
+            // diagonal tile of the last query tile, where the causal mask removes them.
+            each_stage([&](uint4& kk, uint4& vv, int i) {
+                const int key = min(key0 + (tid >> 4) + 16 * i, S - 1);
+                kk = *reinterpret_cast<const uint4*>(k_src + static_cast<uint32_t>(key * kv_row32));
+                const int vkey = min(key0 + 4 * v_kg + i, S - 1);
+                vv = *reinterpret_cast<const uint4*>(v_src + static_cast<uint32_t>(vkey * kv_row32));
+            });
+        }
     };
     // The block whose query tile equals the key tile also writes those K/V rows to the pages.
     auto write_pages = [&](int tile) {
@@ -190,25 +217,27 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
             }
         });
     };
-    auto store_tile = [&](int buf) {
-        each_stage([&](uint4& kk, uint4& vv, int i) {
-            (void)vv;
-            *reinterpret_cast<uint4*>(&sh.k[buf][((tid >> 4) + 16 * i) * kKS + 8 * (tid & 15)]) = kk;
-        });
+    const int k_store = (tid >> 4) * kKS + 8 * (tid & 15);
+    int v_store;
+    {
         // transpose 4 keys x 8 dims -> 8 rows of 4 consecutive key slots; row d keeps its 8-slot
         // blocks XOR-swizzled by (d / 16) % 8.
         const int slot0 = 16 * (v_kg >> 2) + key_slot(4 * (v_kg & 3));
         const int phys = 8 * ((slot0 >> 3) ^ ((v_dc >> 1) & 7)) + (slot0 & 7);
-        uint16_t* dst = &sh.vt[buf][(8 * v_dc) * kVS + phys];
-        auto put = [&](int e, uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+        v_store = (8 * v_dc) * kVS + phys;
+    }
+    auto store_tile = [&](int stage) {
+        uint16_t* kd = st[stage].k + k_store;
+        each_stage([&](uint4& kk, uint4& vv, int i) {
+            (void)vv;
+            *reinterpret_cast<uint4*>(kd + 16 * i * kKS) = kk;
+        });
+        uint16_t* dst = st[stage].vt + v_store;
+        auto put = [&](int e, uint32_t a, uint32_t b2, uint32_t c, uint32_t d) {
+            const uint32_t sel = (e & 1) ? 0x07060302U : 0x05040100U;   // high or low halves of (second, first)
             uint2 packed;
-            if (e & 1) {
-                packed.x = (a >> 16) | (b & 0xffff0000U);
-                packed.y = (c >> 16) | (d & 0xffff0000U);
-            } else {
-                packed.x = (a & 0xffffU) | (b << 16);
-                packed.y = (c & 0xffffU) | (d << 16);
-            }
+            packed.x = __builtin_amdgcn_perm(b2, a, sel);
+            packed.y = __builtin_amdgcn_perm(d, c, sel);
             *reinterpret_cast<uint2*>(dst + e * kVS) = packed;
         };
         put(0, vs0.x, vs1.x, vs2.x, vs3.x);
@@ -221,181 +250,152 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
         put(7, vs0.w, vs1.w, vs2.w, vs3.w);
     };
 
-    // Both groups run the same number of iterations (the barrier is block-wide); a group whose
-    // tile index runs past the diagonal idles through the last one.
-    const int n_iter = qt / QM_PF_KSPLIT + 1;
-    if (kp <= qt) {
-        load_tile(kp);
-        if (prm.has_cache && kp == qt) write_pages(kp);
-        store_tile(0);
-    }
-    __syncthreads();
-
-    for (int it = 0; it < n_iter; ++it) {
-        const int tile = it * QM_PF_KSPLIT + kp;
-        const int buf = it & 1;
-        const bool more = tile + QM_PF_KSPLIT <= qt;
-        if (more) {
-            load_tile(tile + QM_PF_KSPLIT);
-            if (prm.has_cache && tile + QM_PF_KSPLIT == qt) write_pages(tile + QM_PF_KSPLIT);
+    // ---- the pieces of one 32-key chunk --------------------------------------------------------------
+    // S^T = K Q^T of chunk `half` of a stage: rows = 32 keys, cols = 32 (row, head) columns.
+    const int k_lane = col * kKS + 8 * grp;
+    auto qk = [&](int stage, auto half, f32x16_t& s) {
+        const uint16_t* kp = st[stage].k + k_lane + 32 * decltype(half)::value * kKS;
+        bf16x8_t kf[8];
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb) kf[kb] = lds_frag(kp + 16 * kb);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb], qf[kb], s, 0, 0, 0);
+    };
+    // V^T fragment of (chunk half h, group kg, dim tile dt), lane (col, grp): row d = 32*dt + col,
+    // slot block (4h + 2kg + grp) ^ ((d / 16) % 8); the lane part and the constant part of that XOR
+    // touch different bits.
+    const int v_lane = col * kVS + 8 * (grp ^ (col >> 4));
+    auto v_frags = [&](int stage, auto half, bf16x8_t (&vf)[8]) {
+        constexpr int h = decltype(half)::value;
+        const uint16_t* vp = st[stage].vt + v_lane;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            vf[j] = lds_frag(vp + 32 * (j & 3) * kVS + 8 * ((4 * h + 2 * (j >> 2)) ^ (2 * (j & 3))));
+    };
+    // O^T += V^T P^T for one chunk: two 16-key groups x four 32-dim tiles.  On the diagonal a
+    // 16-key group that lies wholly after the wave's last row is masked for every column: it is
+    // skipped, so that later tokens are not even multiplied by zero.
+    auto pv = [&](const bf16x8_t (&vf)[8], const PFrag& p, auto diag, int key_base) {
+#pragma unroll
+        for (int kg = 0; kg < 2; ++kg) {
+            if (decltype(diag)::value && key_base + 16 * kg > wave_last_row) continue;
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) {
+                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * kg + dt], p.hi[kg], o[dt], 0, 0, 0);
+                if (PRECISE) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * kg + dt], p.lo[kg], o[dt], 0, 0, 0);
+            }
         }
-        if (tile <= qt) {
-        const bool diagonal = tile == qt;
-
+    };
+    // Softmax works in `units`: rounded scaled scores (ROUND) or raw fp32 dot products, whose
+    // scale is folded into the exponent's multiplier (the host admits only scale > 0 there).
+    const float coef = ROUND ? kLog2e : prm.scale * kLog2e;
+    const float slack = ROUND ? kRescaleSlack : kRescaleSlack / prm.scale;
+    // Score roundings and causal mask in place; returns the column maximum.
+    auto scores = [&](f32x16_t& s, auto masked, int key_base) -> float {
+        // accumulator register r of lane group grp is key key_base + 8*(r/4) + 4*grp + r%4
+        const int lim = my_row - key_base - 4 * grp;
+        float mx = -INFINITY;
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const int key_base = tile * kBN + 32 * half;
-            // On the diagonal a wave whose last row precedes this half has nothing to do there.
-            if (diagonal && key_base > q0 + 16 * wave + 15) continue;
-
-            // ---- S^T = K Q^T : rows = 32 keys, cols = 32 (row, head) columns ----------------------
-            f32x16_t s;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s[r] = 0.0f;
-            const uint16_t* kp = &sh.k[buf][(32 * half + col) * kKS + 8 * grp];
-            // All eight K fragments are requested before the first MFMA, and the eight V^T
-            // fragments of this half before the softmax arithmetic, so that LDS latency is paid
-            // once per phase instead of once per MFMA.
-#if QM_PF_PREFETCH >= 1
-            bf16x8_t kfr[8];
-#pragma unroll
-            for (int kb = 0; kb < 8; ++kb) kfr[kb] = lds_frag(kp + 16 * kb);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int kb = 0; kb < 8; ++kb) {
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[kb], qf[kb], s, 0, 0, 0);
-            }
-#else
-#pragma unroll
-            for (int kb = 0; kb < 8; ++kb) {
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(kp + 16 * kb), qf[kb], s, 0, 0, 0);
-            }
-#endif
-            bf16x8_t vfr[2][4];
-#if QM_PF_PREFETCH >= 2
-#pragma unroll
-            for (int kg = 0; kg < 2; ++kg) {
-                const int sb = 4 * half + 2 * kg + grp;
-#pragma unroll
-                for (int dt = 0; dt < 4; ++dt) {
-                    const int d = 32 * dt + col;
-                    vfr[kg][dt] = lds_frag(&sh.vt[buf][d * kVS + 8 * (sb ^ ((d >> 4) & 7))]);
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#endif
-
-            // ---- reference score roundings, causal mask, online softmax ---------------------------
-            float mx = -INFINITY;
-#pragma unroll
-            for (int r = 0; r < 16; r += 2) {
-                float x0, x1;
-                round_bf16_pair(s[r], s[r + 1], x0, x1);
+        for (int r = 0; r < 16; r += 2) {
+            float x0 = s[r], x1 = s[r + 1];
+            if (ROUND) {
+                round_bf16_pair(x0, x1, x0, x1);
                 round_bf16_pair(x0 * prm.scale, x1 * prm.scale, x0, x1);
-                if (diagonal) {
-                    const int key = key_base + 8 * (r >> 2) + 4 * grp + (r & 3);
-                    if (key > my_row) x0 = -INFINITY;
-                    if (key + 1 > my_row) x1 = -INFINITY;
-                }
-                s[r] = x0;
-                s[r + 1] = x1;
-                mx = fmaxf(mx, fmaxf(x0, x1));
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            if (decltype(masked)::value) {
+                const int e = 8 * (r >> 2) + (r & 3);
+                if (e > lim) x0 = -INFINITY;
+                if (e + 1 > lim) x1 = -INFINITY;
+            }
+            s[r] = x0;
+            s[r + 1] = x1;
+            mx = fmaxf(mx, fmaxf(x0, x1));
+        }
+        return halves_max(mx);
+    };
+    // Raise the running maximum if some column of the wave exceeds it by more than the slack,
+    // and rescale O and the running sum for it.
+    float m_scaled = 0.0f;
+    auto update_max = [&](float mx) {
+        const bool need = __builtin_amdgcn_ballot_w64(mx > m_run + slack) != 0;
+        if (need) {
             const float m_new = fmaxf(m_run, mx);
             const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
-            if (__builtin_amdgcn_ballot_w64(m_new > m_run)) {
-                const float alpha = fast_exp2((m_run - m_ref) * kLog2e);
-                l_run *= alpha;
-#pragma unroll
-                for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
-            }
+            const float alpha = fast_exp2((m_run - m_ref) * coef);
             m_run = m_new;
-            const float m_scaled = m_ref * kLog2e;
-            float psum = 0.0f;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                s[r] = fast_exp2(fmaf(s[r], kLog2e, -m_scaled));
-                psum += s[r];
-            }
-            l_run += psum;
-
-            // ---- O^T += V^T P^T : two 16-key groups x four 32-dim tiles ---------------------------
-#pragma unroll
-            for (int kg = 0; kg < 2; ++kg) {
-                // A 16-key group that lies wholly after the wave's last row is masked for every
-                // column: skip it, so that later tokens are not even multiplied by zero.
-                if (diagonal && key_base + 16 * kg > q0 + 16 * wave + 15) continue;
-                bf16x8_t phi, plo;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float pv = s[8 * kg + e];
-                    phi[e] = static_cast<__bf16>(pv);
-                    if (PRECISE) plo[e] = static_cast<__bf16>(pv - static_cast<float>(phi[e]));
-                }
-#if QM_PF_PREFETCH < 2
-                {
-                    const int sb = 4 * half + 2 * kg + grp;
-#pragma unroll
-                    for (int dt = 0; dt < 4; ++dt) {
-                        const int d = 32 * dt + col;
-                        vfr[kg][dt] = lds_frag(&sh.vt[buf][d * kVS + 8 * (sb ^ ((d >> 4) & 7))]);
-                    }
-                }
-#endif
-#pragma unroll
-                for (int dt = 0; dt < 4; ++dt) {
-                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[kg][dt], phi, o[dt], 0, 0, 0);
-                    if (PRECISE) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[kg][dt], plo, o[dt], 0, 0, 0);
-                }
-            }
-        }
-
-        }   // tile <= qt
-
-        if (more) store_tile(buf ^ 1);
-        __syncthreads();
-    }
-
-#if QM_PF_KSPLIT == 2
-    // ---- merge the two key groups: group 1 hands its (O, max, sum) to group 0 through LDS --------
-    {
-        float* xo = reinterpret_cast<float*>(pf_smem);                 // [wave][64 regs][64 lanes]
-        float* xm = xo + 4 * 64 * 64;                                  // [wave][2][64 lanes]
-        if (kp == 1) {
+            m_scaled = m_ref * coef;
+            l_run *= alpha;
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) xo[(wave * 64 + dt * 16 + r) * 64 + lane] = o[dt][r];
-            xm[(wave * 2 + 0) * 64 + lane] = m_run;
-            xm[(wave * 2 + 1) * 64 + lane] = l_run;
+                for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
         }
-        __syncthreads();
-        if (kp == 1) return;
-        const float m1 = xm[(wave * 2 + 0) * 64 + lane];
-        const float l1 = xm[(wave * 2 + 1) * 64 + lane];
-        const float mm = fmaxf(m_run, m1);
-        const float m_ref = mm == -INFINITY ? 0.0f : mm;
-        const float a0 = fast_exp2((m_run - m_ref) * kLog2e);
-        const float a1 = fast_exp2((m1 - m_ref) * kLog2e);
-        l_run = l_run * a0 + l1 * a1;
+    };
+    // P = exp(score - max) as bf16 B operands; adds this lane's share of the row sum.
+    auto probs = [&](const f32x16_t& s, PFrag& p) {
+        uint32_t hi[8], lo[8];
+        float psum = 0.0f;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int r = 0; r < 16; r += 2) {
+            const float e0 = fast_exp2(fmaf(s[r], coef, -m_scaled));
+            const float e1 = fast_exp2(fmaf(s[r + 1], coef, -m_scaled));
+            hi[r >> 1] = pack_bf16_pair(e0, e1);
+            if (PRECISE) {
+                lo[r >> 1] = pack_bf16_pair(e0 - lo_bf16(hi[r >> 1]), e1 - hi_bf16(hi[r >> 1]));
+                psum += e0 + e1;
+            } else {
+                psum = dot2_bf16(hi[r >> 1], 0x3f803f80U, psum);   // the sum of what the MFMA multiplies
+            }
+        }
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-                o[dt][r] = fmaf(o[dt][r], a0, xo[(wave * 64 + dt * 16 + r) * 64 + lane] * a1);
+        for (int kg = 0; kg < 2; ++kg) {
+            p.hi[kg] = __builtin_bit_cast(bf16x8_t, make_uint4(hi[4 * kg], hi[4 * kg + 1], hi[4 * kg + 2], hi[4 * kg + 3]));
+            if (PRECISE)
+                p.lo[kg] = __builtin_bit_cast(bf16x8_t, make_uint4(lo[4 * kg], lo[4 * kg + 1], lo[4 * kg + 2], lo[4 * kg + 3]));
+        }
+        l_run += psum;
+    };
+    auto chunk = [&](int stage, auto half, auto diag, int key_base) {
+        // On the diagonal a wave whose last row precedes this chunk has nothing to do in it.
+        if (decltype(diag)::value && key_base > wave_last_row) return;
+        f32x16_t s;
+        bf16x8_t vf[8];
+        PFrag p;
+        qk(stage, half, s);
+        v_frags(stage, half, vf);   // requested before the softmax arithmetic, used after it
+        const float mx = scores(s, diag, key_base);
+        update_max(mx);
+        probs(s, p);
+        pv(vf, p, diag, key_base);
+    };
+
+    // ---- tile 0 into stage 0, then the key tiles up to the diagonal ---------------------------------
+    load_tile(0);
+    if (prm.has_cache && qt == 0) write_pages(0);
+    store_tile(0);
+    __syncthreads();
+
+    if (!PRECISE) {
+        for (int t = 0; t < qt; ++t) {
+            const int stage = t & 1;
+            load_tile(t + 1);
+            chunk(stage, int_c<0>{}, bool_c<false>{}, 0);
+            chunk(stage, int_c<1>{}, bool_c<false>{}, 0);
+            if (prm.has_cache && t + 1 == qt) write_pages(qt);
+            store_tile(stage ^ 1);
+            __syncthreads();
+        }
     }
-    constexpr int kStageOffset = 4 * 64 * 64 * 4 + 4 * 2 * 64 * 4;   // bytes, behind the exchange area
-#else
-    constexpr int kStageOffset = 0;
-#endif
+    chunk(qt & 1, int_c<0>{}, bool_c<true>{}, qt * kBN);
+    chunk(qt & 1, int_c<1>{}, bool_c<true>{}, qt * kBN + 32);
+    __syncthreads();   // the stages become the output staging area
 
     // ---- normalise, stage through LDS, write 16 bytes per lane -------------------------------------
-    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const float l_tot = halves_sum(l_run);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-    uint16_t* stage = reinterpret_cast<uint16_t*>(pf_smem + kStageOffset) + wave * 32 * kOS;   // 32 columns x 128 dims per wave
+    uint16_t* stage = reinterpret_cast<uint16_t*>(pf_smem) + wave * 32 * kOS;   // 32 columns x 128 dims per wave
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) {
 #pragma unroll
@@ -424,19 +424,19 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     }
 }
 
-// grid = batch * kv_heads * n_qtiles blocks, heaviest query tile first: the hardware hands the
-// next (lighter) block to whichever CU retires one, which pairs heavy with light tiles.  The
-// first query tile takes the split-precision P path.
-__global__ __launch_bounds__(kPfThreads, QM_PF_MINWAVES) void prefill_causal_kernel(PrefillParams prm, qm_kv_cache cache) {
+// grid = batch * kv_heads * n_qtiles blocks, heaviest query tile first.  The first query tile
+// takes the split-precision P path.
+template <bool ROUND>
+__global__ __launch_bounds__(kPfThreads, 2) void prefill_causal_kernel(PrefillParams prm, qm_kv_cache cache) {
     extern __shared__ __attribute__((aligned(16))) unsigned char pf_smem[];
     const int pairs = prm.batch * prm.kv_heads;
     const int bid = blockIdx.x;
     const int qt = prm.n_qtiles - 1 - bid / pairs;
     const int pair = bid % pairs;
     if (qt == 0) {
-        prefill_body<true>(prm, cache, pf_smem, 0, pair);
+        prefill_body<true, ROUND>(prm, cache, pf_smem, 0, pair);
     } else {
-        prefill_body<false>(prm, cache, pf_smem, qt, pair);
+        prefill_body<false, ROUND>(prm, cache, pf_smem, qt, pair);
     }
 }
 
@@ -490,15 +490,17 @@ extern "C" int32_t qm_prefill_attention_causal(
     prm.batch = batch; prm.seq = seq; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
 
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
-    const size_t smem = sizeof(PfShared) * QM_PF_KSPLIT;
-    static bool attr_set = false;
-    if (!attr_set) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_causal_kernel),
+    const size_t smem = sizeof(PfStage) * kPfStages;
+    const bool round_scores = option_value(QM_OPT_PREFILL_SCORE_ROUNDING) != 0;
+    if (!round_scores && !(scale > 0.0f)) return QM_ERR_ARGUMENT;   // the scale is folded into the exponent there
+    const auto kernel = round_scores ? prefill_causal_kernel<true> : prefill_causal_kernel<false>;
+    static bool attr_set[2] = {false, false};
+    if (!attr_set[round_scores]) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
         if (e != hipSuccess) return hip_code(e);
-        attr_set = true;
+        attr_set[round_scores] = true;
     }
-    hipLaunchKernelGGL(prefill_causal_kernel, dim3(static_cast<unsigned>(pairs * n_qtiles)), dim3(kPfThreads), smem, s,
-                       prm, desc);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(pairs * n_qtiles)), dim3(kPfThreads), smem, s, prm, desc);
     return launch_status();
 }

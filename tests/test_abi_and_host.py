@@ -78,6 +78,23 @@ def test_host_validation_without_device(qm):
     assert lib.qm_predictor_attention_loop(fake, fake, fake, fake, fake, fake, fake, fake, None, None, 0, 1, 16, 1, 1e-6, None) == 0
 
 
+def test_options_round_trip_and_validation(qm):
+    assert qm.get_option(qm.OPT_PREFILL_SCORE_ROUNDING) == 1      # reference roundings by default
+    assert qm.get_option(qm.OPT_DECODE_TILES_PER_BLOCK) == 0
+    lib = qm.lib()
+    assert lib.qm_set_option(99, 1) == -5 and lib.qm_set_option(-1, 1) == -5
+    assert lib.qm_set_option(qm.OPT_DECODE_TILES_PER_BLOCK, -3) == -5
+    assert lib.qm_get_option(qm.OPT_DECODE_TILES_PER_BLOCK, None) == -1
+    base = qm.decode_workspace_bytes(64, 16, 8, 4096)
+    qm.set_option(qm.OPT_DECODE_TILES_PER_BLOCK, 4)
+    try:
+        assert qm.get_option(qm.OPT_DECODE_TILES_PER_BLOCK) == 4
+        assert qm.decode_workspace_bytes(64, 16, 8, 4096) > base     # more splits, more partial records
+    finally:
+        qm.set_option(qm.OPT_DECODE_TILES_PER_BLOCK, 0)
+    assert qm.decode_workspace_bytes(64, 16, 8, 4096) == base
+
+
 def test_workspace_size_is_monotone_and_pure(qm):
     lib = qm.lib()
     prev = 0
