@@ -11,11 +11,21 @@
 // 8-slot blocks XOR-swizzled per 16 rows so both the transposing writes and the fragment reads
 // are conflict-free).
 //
-// Occupancy.  A wave cannot issue VALU work in the shadow of its own MFMAs (measured: one MFMA
-// plus eight independent FMAs take the sum of both), so the matrix pipe and the VALU only overlap
-// between waves: the kernel stays within 256 registers and 72 KB of LDS so that two blocks share
-// a CU, and a software pipeline inside the wave (tried, with three LDS stages and 316 registers)
-// brought nothing.
+// Occupancy and what bounds the kernel.  A wave cannot issue VALU work in the shadow of its own
+// MFMAs (measured: one MFMA plus eight independent FMAs take the sum of both), so the matrix pipe
+// and the VALU only overlap between waves, and with two waves per SIMD whose phases are long (eight
+// MFMAs, then about 150 VALU instructions, then eight MFMAs) that overlap is small as well: a
+// synthetic pair of such waves takes 2 045 cycles per step against 2 420 serial and 1 216 ideal.
+// The kernel therefore stays within 256 registers and 72 KB of LDS so that two blocks share a CU
+// and fill each other's waits, and otherwise keeps the instruction count per key tile low.
+// Variants that were measured and dropped (batch 4 x 1024 tokens / 4 x 4096 tokens, this one:
+// 42 us / 381 us): a software pipeline inside the wave with three LDS stages and 316 registers,
+// one wave per SIMD (51 us / 467 us); eight-wave blocks whose two wave groups split each key tile
+// and merge through LDS, with phase-skewed groups and each block taking a heavy and a light
+// query tile (41 us / 421 us: the longest block is halved, but the groups meet at a barrier per
+// tile and run in step).  At batch 4 x 1024 tokens the time is the serial length of the blocks
+// that own the last query tiles (16 key tiles at 1.7 us) plus a 4 us start in which every block
+// fetches its first tiles from HBM at once, not chip throughput.
 //
 // Lazy rescale.  The running maximum of a column is only raised when a chunk exceeds it by more
 // than kRescaleSlack (then O and the running sum are rescaled); otherwise probabilities are taken
@@ -202,20 +212,59 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
         }
     };
     // The block whose query tile equals the key tile also writes those K/V rows to the pages.
+    // The eight page-table entries a thread needs for that are requested at the start of the
+    // block (independent loads, long answered when the tile arrives); what is wrong with an
+    // entry is kept as a status bit and reported once.
+    int kp0 = -1, kp1 = -1, kp2 = -1, kp3 = -1, vp0 = -1, vp1 = -1, vp2 = -1, vp3 = -1;
+    uint32_t page_err = 0;
+    auto each_phys = [&](auto&& f) {
+        f(kp0, vp0, 0);
+        f(kp1, vp1, 1);
+        f(kp2, vp2, 2);
+        f(kp3, vp3, 3);
+    };
+    auto fetch_entry = [&](int key) -> int {
+        if (key >= S) return -1;
+        const int page = page_of(prm.pages, key);
+        if (page >= prm.pages.max_pages) {
+            page_err |= QM_STATUS_BAD_POSITION;
+            return -1;
+        }
+        return table ? table[page] : page;
+    };
+    auto fetch_pages = [&]() {
+        each_phys([&](int& kp, int& vp, int i) {
+            kp = fetch_entry(qt * kBN + (tid >> 4) + 16 * i);
+            vp = fetch_entry(qt * kBN + 4 * v_kg + i);
+        });
+    };
+    auto page_store = [&](uint16_t* pool, int phys, int key, int dim0, const uint4& x) {
+        if (key >= S || phys == -1) return;
+        if (phys < 0 || phys >= cache.n_pages) {
+            page_err |= QM_STATUS_BAD_PAGE;
+            return;
+        }
+        const int page = page_of(prm.pages, key);
+        const int64_t off = static_cast<int64_t>(phys) * cache.stride_page + static_cast<int64_t>(kvh) * cache.stride_head
+                          + static_cast<int64_t>(key - page * prm.pages.page_size) * kDim;
+        *reinterpret_cast<uint4*>(pool + off + dim0) = x;
+    };
     auto write_pages = [&](int tile) {
         const int key0 = tile * kBN;
+        uint4 k0, k1, k2, k3, v0, v1, v2, v3;
         each_stage([&](uint4& kk, uint4& vv, int i) {
-            const int key = key0 + (tid >> 4) + 16 * i;
-            if (key < S) {
-                const int64_t off = tile_offset(cache, prm.pages, table, key, kvh, prm.status);
-                if (off >= 0) *reinterpret_cast<uint4*>(cache.k_pool + off + 8 * (tid & 15)) = kk;
-            }
-            const int vkey = key0 + 4 * v_kg + i;
-            if (vkey < S) {
-                const int64_t off = tile_offset(cache, prm.pages, table, vkey, kvh, prm.status);
-                if (off >= 0) *reinterpret_cast<uint4*>(cache.v_pool + off + 8 * v_dc) = vv;
-            }
+            if (i == 0) { k0 = kk; v0 = vv; }
+            if (i == 1) { k1 = kk; v1 = vv; }
+            if (i == 2) { k2 = kk; v2 = vv; }
+            if (i == 3) { k3 = kk; v3 = vv; }
         });
+        each_phys([&](int& kp, int& vp, int i) {
+            const uint4 kk = i == 0 ? k0 : i == 1 ? k1 : i == 2 ? k2 : k3;
+            const uint4 vv = i == 0 ? v0 : i == 1 ? v1 : i == 2 ? v2 : v3;
+            page_store(cache.k_pool, kp, key0 + (tid >> 4) + 16 * i, 8 * (tid & 15), kk);
+            page_store(cache.v_pool, vp, key0 + 4 * v_kg + i, 8 * v_dc, vv);
+        });
+        if (page_err && prm.status) atomicOr(prm.status, page_err);
     };
     const int k_store = (tid >> 4) * kKS + 8 * (tid & 15);
     int v_store;
@@ -373,6 +422,7 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
 
     // ---- tile 0 into stage 0, then the key tiles up to the diagonal ---------------------------------
     load_tile(0);
+    if (prm.has_cache) fetch_pages();
     if (prm.has_cache && qt == 0) write_pages(0);
     store_tile(0);
     __syncthreads();
@@ -402,10 +452,8 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
         for (int rq = 0; rq < 4; ++rq) {
             const int d0 = 32 * dt + 8 * rq + 4 * grp;
             uint2 packed;
-            packed.x = static_cast<uint32_t>(f2bf(o[dt][4 * rq + 0] * inv))
-                     | (static_cast<uint32_t>(f2bf(o[dt][4 * rq + 1] * inv)) << 16);
-            packed.y = static_cast<uint32_t>(f2bf(o[dt][4 * rq + 2] * inv))
-                     | (static_cast<uint32_t>(f2bf(o[dt][4 * rq + 3] * inv)) << 16);
+            packed.x = pack_bf16_pair(o[dt][4 * rq + 0] * inv, o[dt][4 * rq + 1] * inv);
+            packed.y = pack_bf16_pair(o[dt][4 * rq + 2] * inv, o[dt][4 * rq + 3] * inv);
             *reinterpret_cast<uint2*>(&stage[col * kOS + d0]) = packed;
         }
     }
