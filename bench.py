@@ -230,6 +230,55 @@ class SingleDecode:
         return res, err, "whole workload"
 
 
+class QkvGemv:
+    """The next row after the attention path: the fused M = 1 Q/K/V projection that feeds the
+    norm + RoPE + append (hidden 2048 -> q 2048, k 1024, v 1024).  `copies` weight sets are used in
+    rotation (64 sets = 1 GB, as the layers of a real decode step never find their weights cached)."""
+    bound = "hbm"
+
+    def __init__(self, qm, dev, seed=77, copies=1):
+        import torch
+        self.qm, self.copies = qm, copies
+        self.name = "qkv_gemv_m1_hidden2048" + ("_rotating%d" % copies if copies > 1 else "")
+        gd = torch.Generator(device=dev).manual_seed(seed)
+
+        def rnd(shape, std=1.0):
+            return (torch.randn(shape, generator=gd, device=dev, dtype=torch.float32) * std).to(torch.bfloat16)
+
+        self.x = rnd((2048,))
+        self.w = [(rnd((2048, 2048), 0.02), rnd((1024, 2048), 0.02), rnd((1024, 2048), 0.02)) for _ in range(copies)]
+        self.b = (rnd((2048,), 0.1), rnd((1024,), 0.1), rnd((1024,), 0.1))
+        self.q = torch.zeros(2048, dtype=torch.bfloat16, device=dev)
+        self.k = torch.zeros(1024, dtype=torch.bfloat16, device=dev)
+        self.v = torch.zeros(1024, dtype=torch.bfloat16, device=dev)
+        self.bytes = 2 * 4096 * 2048 + 2 * 2048 + 2 * 4096 + 2 * 4096     # weights, input, biases, outputs
+        self.flops = 2 * 4096 * 2048
+        self.i = 0
+
+    def step(self):
+        import torch
+        w = self.w[self.i % self.copies]
+        self.i += 1
+        self.qm.qkv_m1(self.x, w[0], self.b[0], w[1], self.b[1], w[2], self.b[2], self.q, self.k, self.v,
+                       2048, 2048, 1024, torch.cuda.current_stream().cuda_stream)
+
+    def cpu_baseline(self, oracle, threads):
+        import torch
+        self.i = 0
+        self.step()
+        torch.cuda.synchronize()
+        w = [_bits(t).copy() for t in self.w[0]]
+        b = [_bits(t).copy() for t in self.b]
+        outs = [np.zeros(n, dtype=np.uint16) for n in (2048, 1024, 1024)]
+        t0 = time.perf_counter()
+        rc = oracle.qkv_m1(_bits(self.x).copy(), w[0], b[0], w[1], b[1], w[2], b[2], outs[0], outs[1], outs[2],
+                           2048, 2048, 1024, threads)
+        dt = time.perf_counter() - t0
+        assert rc == 0
+        exact = all(np.array_equal(o, _bits(t)) for o, t in zip(outs, (self.q, self.k, self.v)))
+        return {"all": dt}, 0.0 if exact else 1.0, "whole workload (bit-exact comparison)"
+
+
 class Prefill:
     """configs[3]: causal GQA prefill, batch 4 x seq 1024, K/V also written to shuffled 16-token pages."""
     name = "causal_prefill_b4_s1024_paged16"
@@ -345,7 +394,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
-    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "predictor"], default=None,
+    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "predictor", "qkv"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -378,7 +427,8 @@ def main():
     if args.only:
         make = {"decode512": lambda: SingleDecode(qm, dev, 512, False, 11),
                 "talker2048": lambda: SingleDecode(qm, dev, 2048, True, 12),
-                "prefill": lambda: Prefill(qm, dev), "predictor": lambda: PredictorLoop(qm, dev)}[args.only]
+                "prefill": lambda: Prefill(qm, dev), "predictor": lambda: PredictorLoop(qm, dev),
+                "qkv": lambda: QkvGemv(qm, dev, copies=64)}[args.only]
         w = make()
         r = _report(w, _time_steps(w.step, args.steps, args.warmup))
         r["bound"] = w.bound
@@ -408,6 +458,9 @@ def main():
             ("cfg4_causal_prefill", lambda: Prefill(qm, dev)),
             ("cfg5_predictor_loop", lambda: PredictorLoop(qm, dev)),
             ("cfg5_predictor_loop_cache_writeback", lambda: PredictorLoop(qm, dev, write_cache=True)),
+            # beyond the five configurations: the M = 1 projection in front of configuration 2
+            ("next_qkv_gemv_m1", lambda: QkvGemv(qm, dev)),
+            ("next_qkv_gemv_m1_rotating64", lambda: QkvGemv(qm, dev, copies=64)),
         ]
         for key, make in extra:
             w = make()

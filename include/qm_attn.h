@@ -242,6 +242,33 @@ int32_t qm_predictor_attention_loop(
     float epsilon,
     void* hip_stream);
 
+/* --- (5) M = 1 weight-streaming linears around the path ----------------------------------- */
+/*
+ * qm_linear_m1 replaces launch_linear_m1 / talker_linear_fused_kernel (R17:17473-17511,
+ * 15201-15268): output[o] = bf16(sum_k input[k] * weight[o][k] + bias[o]); with a residual the
+ * stored value is bf16(residual[o] + bf16(that)).  weight is [output_columns][reduction_columns]
+ * row-major bf16; bias and residual may be NULL; output must not alias input.
+ * qm_qkv_m1 replaces launch_qkv_m1 / talker_qkv_fused_kernel (R17:17513-17567, 15272-15362):
+ * the three projections of one decode step over one read of the normalised hidden vector;
+ * weights [q_dim][hidden], [kv_dim][hidden], [kv_dim][hidden]; biases may be NULL.
+ * Both reproduce the reference's fp32 summation order (32 strided fmaf chains per output, then
+ * its shuffle tree), so outputs are bit-identical to the reference kernels'.
+ * reduction_columns / hidden must be even and <= 16384 (QM_ERR_GEOMETRY otherwise); weight
+ * pointers 4-byte aligned.
+ */
+int32_t qm_linear_m1(
+    const uint16_t* input, const uint16_t* weight, const uint16_t* bias, const uint16_t* residual,
+    uint16_t* output, int32_t output_columns, int32_t reduction_columns,
+    void* hip_stream);
+int32_t qm_qkv_m1(
+    const uint16_t* input,
+    const uint16_t* q_weight, const uint16_t* q_bias,
+    const uint16_t* k_weight, const uint16_t* k_bias,
+    const uint16_t* v_weight, const uint16_t* v_bias,
+    uint16_t* q_output, uint16_t* k_output, uint16_t* v_output,
+    int32_t hidden, int32_t q_dim, int32_t kv_dim,
+    void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -174,6 +174,28 @@ inline void predictor_attention_loop(
           "Predictor attention loop launch");
 }
 
+// launch_linear_m1 (R17:17473-17511), same argument order and label.
+inline void launch_linear_m1(
+    const std::uint16_t* input, const std::uint16_t* weight, const std::uint16_t* bias,
+    const std::uint16_t* residual, std::uint16_t* output, int output_columns, int reduction_columns,
+    void* stream) {
+    check(qm_linear_m1(input, weight, bias, residual, output, output_columns, reduction_columns, stream),
+          "Qingming M1 linear launch");
+}
+
+// launch_qkv_m1 (R17:17513-17567) with the layer's parameters spelled out.
+inline void launch_qkv_m1(
+    const std::uint16_t* input,
+    const std::uint16_t* q_weight, const std::uint16_t* q_bias,
+    const std::uint16_t* k_weight, const std::uint16_t* k_bias,
+    const std::uint16_t* v_weight, const std::uint16_t* v_bias,
+    std::uint16_t* q, std::uint16_t* k, std::uint16_t* v,
+    int hidden, int q_dim, int kv_dim, void* stream) {
+    check(qm_qkv_m1(input, q_weight, q_bias, k_weight, k_bias, v_weight, v_bias, q, k, v, hidden, q_dim,
+                    kv_dim, stream),
+          "Qingming fused QKV launch");
+}
+
 }  // namespace qm_attn
 
 #endif  // QM_ATTN_HPP

@@ -191,3 +191,14 @@ def predictor_attention_loop(q, k, v, gq, gk, cos, sin, out, k_cache_out, v_cach
         _p(q), _p(k), _p(v), _p(gq), _p(gk), _p(cos), _p(sin), _p(out), _p(k_cache_out),
         _p(v_cache_out), C.c_int32(units), C.c_int32(n_layers), C.c_int32(rows),
         C.c_int32(first_rows), C.c_float(eps), C.c_int32(threads))
+
+
+def linear_m1(x, weight, bias, residual, out, output_columns, reduction_columns, threads=8):
+    return lib().qmo_linear_m1(_p(x), _p(weight), _p(bias), _p(residual), _p(out),
+                               C.c_int32(output_columns), C.c_int32(reduction_columns), C.c_int32(threads))
+
+
+def qkv_m1(x, q_w, q_b, k_w, k_b, v_w, v_b, q_out, k_out, v_out, hidden, q_dim, kv_dim, threads=8):
+    return lib().qmo_qkv_m1(_p(x), _p(q_w), _p(q_b), _p(k_w), _p(k_b), _p(v_w), _p(v_b), _p(q_out),
+                            _p(k_out), _p(v_out), C.c_int32(hidden), C.c_int32(q_dim), C.c_int32(kv_dim),
+                            C.c_int32(threads))

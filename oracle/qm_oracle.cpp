@@ -680,4 +680,60 @@ int32_t qmo_predictor_attention_loop(
     return QM_OK;
 }
 
+// ---- M = 1 weight-streaming linears ------------------------------------------------------------------
+// One output scalar as one 32-lane wave of talker_linear_fused_kernel / talker_qkv_fused_kernel
+// computes it (R17:15239-15266, 15340-15360): lane l accumulates k = l, l+32, ... with fmaf in
+// increasing k, the 32 lane sums go through the shuffle tree, lane 0 adds the bias in fp32 and
+// rounds to bf16; with a residual the stored value is bf16(residual + bf16(result)).
+static uint16_t linear_m1_scalar(const uint16_t* input, const uint16_t* weight_row, const uint16_t* bias,
+                                 const uint16_t* residual, int out, int reduction_columns) {
+    float lanes[32];
+    for (int l = 0; l < 32; ++l) {
+        float acc = 0.0f;
+        for (int k = l; k < reduction_columns; k += 32) acc = std::fmaf(bf2f(input[k]), bf2f(weight_row[k]), acc);
+        lanes[l] = acc;
+    }
+    float a = wave32_sum(lanes);
+    if (bias) a += bf2f(bias[out]);
+    const uint16_t v = f2bf(a);
+    return residual ? f2bf(bf2f(residual[out]) + bf2f(v)) : v;
+}
+
+// talker_linear_fused_kernel + launch_linear_m1 (R17:15201-15268, 17473-17511): weight is
+// [output_columns][reduction_columns] row-major; bias and residual may be NULL.
+int32_t qmo_linear_m1(const uint16_t* input, const uint16_t* weight, const uint16_t* bias,
+                      const uint16_t* residual, uint16_t* output, int32_t output_columns,
+                      int32_t reduction_columns, int32_t n_threads) {
+    if (!input || !weight || !output) return QM_ERR_NULL;
+    if (output_columns < 0 || reduction_columns < 0) return QM_ERR_ARGUMENT;
+    parallel_for(output_columns, n_threads, [&](int64_t o) {
+        output[o] = linear_m1_scalar(input, weight + o * reduction_columns, bias, residual,
+                                     static_cast<int>(o), reduction_columns);
+    });
+    return QM_OK;
+}
+
+// talker_qkv_fused_kernel + launch_qkv_m1 (R17:15272-15362, 17513-17567): three linears over one
+// staged input; output row r of the concatenation q | k | v reads its own weight, bias and output.
+int32_t qmo_qkv_m1(const uint16_t* input, const uint16_t* q_weight, const uint16_t* q_bias,
+                   const uint16_t* k_weight, const uint16_t* k_bias, const uint16_t* v_weight,
+                   const uint16_t* v_bias, uint16_t* q_output, uint16_t* k_output, uint16_t* v_output,
+                   int32_t hidden, int32_t q_dim, int32_t kv_dim, int32_t n_threads) {
+    if (!input || !q_weight || !k_weight || !v_weight || !q_output || !k_output || !v_output) return QM_ERR_NULL;
+    if (hidden < 0 || q_dim < 0 || kv_dim < 0) return QM_ERR_ARGUMENT;
+    parallel_for(static_cast<int64_t>(q_dim) + 2 * kv_dim, n_threads, [&](int64_t first) {
+        if (first < q_dim) {
+            q_output[first] = linear_m1_scalar(input, q_weight + first * hidden, q_bias, nullptr,
+                                               static_cast<int>(first), hidden);
+        } else if (first < q_dim + kv_dim) {
+            const int64_t r = first - q_dim;
+            k_output[r] = linear_m1_scalar(input, k_weight + r * hidden, k_bias, nullptr, static_cast<int>(r), hidden);
+        } else {
+            const int64_t r = first - q_dim - kv_dim;
+            v_output[r] = linear_m1_scalar(input, v_weight + r * hidden, v_bias, nullptr, static_cast<int>(r), hidden);
+        }
+    });
+    return QM_OK;
+}
+
 }  // extern "C"

@@ -60,6 +60,8 @@ _SIGNATURES = {
     "qm_prefill_attention_causal": (_I32, [_PTR] * 4 + [C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _I32, _I32,
                                            _F32, C.c_int64, C.c_int64, C.c_int64, _PTR, _PTR]),
     "qm_predictor_attention_loop": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _I32, _F32, _PTR]),
+    "qm_linear_m1": (_I32, [_PTR] * 5 + [_I32, _I32, _PTR]),
+    "qm_qkv_m1": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _PTR]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
@@ -187,3 +189,14 @@ def predictor_attention_loop(q, k, v, gq, gk, cos, sin, out, k_cache_out, v_cach
         _addr(q), _addr(k), _addr(v), _addr(gq), _addr(gk), _addr(cos), _addr(sin), _addr(out),
         _addr(k_cache_out), _addr(v_cache_out), units, n_layers, rows, first_rows, eps, stream),
         "qm_predictor_attention_loop")
+
+
+def linear_m1(x, weight, bias, residual, out, output_columns, reduction_columns, stream=0):
+    _check(lib().qm_linear_m1(_addr(x), _addr(weight), _addr(bias), _addr(residual), _addr(out),
+                              output_columns, reduction_columns, stream), "qm_linear_m1")
+
+
+def qkv_m1(x, q_w, q_b, k_w, k_b, v_w, v_b, q_out, k_out, v_out, hidden, q_dim, kv_dim, stream=0):
+    _check(lib().qm_qkv_m1(_addr(x), _addr(q_w), _addr(q_b), _addr(k_w), _addr(k_b), _addr(v_w), _addr(v_b),
+                           _addr(q_out), _addr(k_out), _addr(v_out), hidden, q_dim, kv_dim, stream),
+           "qm_qkv_m1")
