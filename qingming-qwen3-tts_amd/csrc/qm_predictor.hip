@@ -16,6 +16,8 @@
 #include "qm_device.h"
 #include "qm_host.h"
 
+#include <type_traits>
+
 namespace qm {
 
 constexpr int kPredRows = 16;     // kMaxCache of the reference (R17:7963)
@@ -67,7 +69,7 @@ __device__ __forceinline__ void pv_rows(const float (*p)[kPredRows], const float
             const float* pr = p[R];
             // leaf j = fmaf(P[j], V[j][d], +0), keys 0..R (R17:12523-12549)
             const float o = TreeSum<R + 1, 0, 8>::eval([&](int j) { return fmaf(pr[j], vcol[j], 0.0f); });
-            out[R * row_stride] = f2bf(o);
+            out[R * row_stride] = __builtin_bit_cast(uint16_t, static_cast<__bf16>(o));   // RNE, one instruction
             pv_rows<R + 1>(p, vcol, out, row_stride, rows);
         }
     }
@@ -80,8 +82,8 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
     __shared__ __attribute__((aligned(16))) uint16_t sh_cos[kPredRows][kDim];
     __shared__ __attribute__((aligned(16))) uint16_t sh_sin[kPredRows][kDim];
     __shared__ __attribute__((aligned(16))) uint16_t sh_gamma[2][kDim];          // q, k
-    __shared__ float sh_s[2][kPredRows][kPredRows];                                // scores, then P
-    __shared__ float sh_e[2][kPredRows][kPredRows];                                // exponentials
+    __shared__ __attribute__((aligned(16))) float sh_s[2][kPredRows][kPredRows];   // scores, then P
+    __shared__ __attribute__((aligned(16))) float sh_kf[kPredRows][kDim];                                       // normed, rotated K as fp32
     __shared__ float sh_grp[3 * kPredRows][4];                                     // group sums of squares
     __shared__ float sh_r[3 * kPredRows];                                          // inverse RMS per vector
 
@@ -201,6 +203,13 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
         }
         *reinterpret_cast<uint2*>(x + d0) = make_uint2(out_lo[0], out_lo[1]);
         *reinterpret_cast<uint2*>(x + d0 + 64) = make_uint2(out_hi[0], out_hi[1]);
+        if (which == 2) {
+            // every wave reads all of K for the scores: widen it once here instead of four times there
+            *reinterpret_cast<float4*>(&sh_kf[vrow][d0]) =
+                make_float4(lo_bf16(out_lo[0]), hi_bf16(out_lo[0]), lo_bf16(out_lo[1]), hi_bf16(out_lo[1]));
+            *reinterpret_cast<float4*>(&sh_kf[vrow][d0 + 64]) =
+                make_float4(lo_bf16(out_hi[0]), hi_bf16(out_hi[0]), lo_bf16(out_hi[1]), hi_bf16(out_hi[1]));
+        }
     }
     __syncthreads();
 
@@ -220,24 +229,37 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
     }
 
     // ---- scores ---------------------------------------------------------------------------------------
-    // A 32-lane half wave evaluates one query vector against all 16 keys in the reference's order of
-    // operations (R17:12386-12418): lane hl accumulates dims hl, hl+32, hl+64, hl+96 with fmaf, then the
-    // shuffle tree (hl + hl^16, then ^8, ^4, ^2, ^1).  The tree runs as a reduce-scatter: at every level
-    // a lane keeps half of its remaining keys and adds its partner's values for them, which yields the
-    // same sums (fp addition is commutative) with 16 exchanges instead of 80.  Key j ends in lanes
-    // 2j and 2j+1 of the half wave.
+    // A 32-lane half wave evaluates one query vector against the keys 0..row in the reference's order
+    // of operations (R17:12386-12418): reference lane v accumulates dims v, v+32, v+64, v+96 with fmaf,
+    // then the shuffle tree (v + v^16, then ^8, ^4, ^2, ^1).  The tree runs as a reduce-scatter: at
+    // every level a lane keeps half of its remaining keys and adds its partner's values for them,
+    // which yields the same sums (fp addition is commutative) with 16 exchanges instead of 80; key j
+    // ends in reference lanes 2j and 2j+1.  Physical lane p plays reference lane v(p), chosen so
+    // that every partner is one cross-lane ALU operand away and nothing goes through LDS:
+    // v = p with bits 1 and 0 flipped where bit 2 is set, which turns v^4 into the DPP
+    // half-row mirror (p^7); v^16 is v_permlane16_swap, v^8 a DPP row rotation, v^2 and v^1 DPP quad
+    // permutations.
     {
         const int half = lane >> 5;
-        const int hl = lane & 31;
+        const int pl = lane & 31;
+        const int hl = pl ^ ((pl & 4) ? 3 : 0);   // the reference lane this lane plays
         const float scale = __uint_as_float(0x3db504f3U);   // kAttentionScaleBits, R17:9354-9356
         float kf[kPredRows][4];
 #pragma unroll
         for (int j = 0; j < kPredRows; ++j)
 #pragma unroll
-            for (int c = 0; c < 4; ++c) kf[j][c] = bf2f(sh_k[j][hl + 32 * c]);
-        for (int qi = wave * 2 + half; qi < 2 * rows; qi += 8) {
-            const int g = qi / rows;
-            const int row = qi % rows;
+            for (int c = 0; c < 4; ++c) kf[j][c] = sh_kf[j][hl + 32 * c];
+        auto dpp = [](float v, auto ctrl) {
+            return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), decltype(ctrl)::value, 0xf, 0xf, false));
+        };
+        constexpr std::integral_constant<int, 0x128> kRowRor8{};        // lane p reads p ^ 8
+        constexpr std::integral_constant<int, 0x141> kHalfMirror{};     // lane p reads p ^ 7
+        constexpr std::integral_constant<int, 0x4e> kQuadXor2{};        // quad_perm [2,3,0,1]
+        constexpr std::integral_constant<int, 0xb1> kQuadXor1{};        // quad_perm [1,0,3,2]
+        // The two halves of a wave take the two heads of the same row, so that the keys after the
+        // row (never read: the softmax masks them) are skipped with a wave-uniform branch.
+        for (int row = wave; row < rows; row += 4) {
+            const int g = half;
             float q4[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) q4[c] = bf2f(sh_q[g][row][hl + 32 * c]);
@@ -245,20 +267,22 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
 #pragma unroll
             for (int j = 0; j < kPredRows; ++j) {
                 float acc = 0.0f;
+                if (j <= row) {
+                    asm volatile("" ::: "memory");   // keeps the branch: the compiler would compute and discard
 #pragma unroll
-                for (int c = 0; c < 4; ++c) acc = fmaf(q4[c], kf[j][c], acc);
+                    for (int c = 0; c < 4; ++c) acc = fmaf(q4[c], kf[j][c], acc);
+                }
                 x[j] = acc;
             }
-            // level 16 -> 8 keys per lane
+            // level 16: reference lanes 0..15 keep keys 0..7, lanes 16..31 keys 8..15.
+            // v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even
+            // rows of its second, so after swapping (x[j], x[j+8]) the two registers hold, in every
+            // lane, its own and its partner's value of the key it keeps.
             float y8[8], y4[4], y2[2];
-            {
-                const bool up = hl & 16;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float give = up ? x[j] : x[j + 8];
-                    const float keep = up ? x[j + 8] : x[j];
-                    y8[j] = keep + __shfl_xor(give, 16);
-                }
+            for (int j = 0; j < 8; ++j) {
+                const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(x[j]), __float_as_uint(x[j + 8]), false, false);
+                y8[j] = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
             }
             {
                 const bool up = hl & 8;
@@ -266,7 +290,7 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
                 for (int j = 0; j < 4; ++j) {
                     const float give = up ? y8[j] : y8[j + 4];
                     const float keep = up ? y8[j + 4] : y8[j];
-                    y4[j] = keep + __shfl_xor(give, 8);
+                    y4[j] = keep + dpp(give, kRowRor8);
                 }
             }
             {
@@ -275,7 +299,7 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
                 for (int j = 0; j < 2; ++j) {
                     const float give = up ? y4[j] : y4[j + 2];
                     const float keep = up ? y4[j + 2] : y4[j];
-                    y2[j] = keep + __shfl_xor(give, 4);
+                    y2[j] = keep + dpp(give, kHalfMirror);
                 }
             }
             float y1;
@@ -283,9 +307,9 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
                 const bool up = hl & 2;
                 const float give = up ? y2[0] : y2[1];
                 const float keep = up ? y2[1] : y2[0];
-                y1 = keep + __shfl_xor(give, 2);
+                y1 = keep + dpp(give, kQuadXor2);
             }
-            const float total = y1 + __shfl_xor(y1, 1);
+            const float total = y1 + dpp(y1, kQuadXor1);
             if ((hl & 1) == 0) {
                 const float raw = rbf(total);
                 sh_s[g][row][hl >> 1] = rbf(raw * scale);
@@ -294,25 +318,40 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
     }
     __syncthreads();
 
-    // ---- softmax, spread over all threads: one (g, row, key) element each ---------------------------------
-    for (int i = tid; i < 2 * rows * kPredRows; i += kPredThreads) {
-        const int j = i & 15;
-        const int r = (i >> 4) % rows;
-        const int g = (i >> 4) / rows;
-        const float* s = sh_s[g][r];
+    // ---- softmax: one thread per (head, row) ----------------------------------------------------------
+    // (an element-per-thread layout recomputes the row maximum and the row sum sixteen times; the
+    // kernel is bound by VALU issue, so the 32 busy lanes of one wave are the cheaper choice)
+    if (tid < 2 * rows) {
+        const int g = tid / rows;
+        const int r = tid % rows;
+        float sc[kPredRows];
+#pragma unroll
+        for (int t = 0; t < kPredRows; t += 4) {
+            const float4 v4 = *reinterpret_cast<const float4*>(&sh_s[g][r][t]);
+            sc[t] = v4.x; sc[t + 1] = v4.y; sc[t + 2] = v4.z; sc[t + 3] = v4.w;
+        }
+        // maximum = maximum > s ? maximum : s over keys 0..r (R17:12449-12470); a masked key enters
+        // as -inf, which never replaces anything
         float maximum = -INFINITY;
-        for (int t = 0; t <= r; ++t) maximum = maximum > s[t] ? maximum : s[t];
-        sh_e[g][r][j] = j <= r ? expf(s[j] - maximum) : 0.0f;
-    }
-    __syncthreads();
-    for (int i = tid; i < 2 * rows * kPredRows; i += kPredThreads) {
-        const int j = i & 15;
-        const int r = (i >> 4) % rows;
-        const int g = (i >> 4) / rows;
-        const float* e = sh_e[g][r];
+#pragma unroll
+        for (int t = 0; t < kPredRows; ++t) {
+            const float cand = t <= r ? sc[t] : -INFINITY;
+            maximum = maximum > cand ? maximum : cand;
+        }
+        float e[kPredRows];
+#pragma unroll
+        for (int t = 0; t < kPredRows; ++t) e[t] = t <= r ? expf(sc[t] - maximum) : 0.0f;
         // exp() >= +0 and masked entries are +0: the full 16-leaf tree equals the reference's sum
         const float total = TreeSum<16, 0, 8>::eval([&](int t) { return e[t]; });
-        sh_s[g][r][j] = j <= r ? rbf(e[j] / total) : 0.0f;
+#pragma unroll
+        for (int t = 0; t < kPredRows; t += 4) {
+            float4 p4;
+            p4.x = t <= r ? rbf(e[t] / total) : 0.0f;
+            p4.y = t + 1 <= r ? rbf(e[t + 1] / total) : 0.0f;
+            p4.z = t + 2 <= r ? rbf(e[t + 2] / total) : 0.0f;
+            p4.w = t + 3 <= r ? rbf(e[t + 3] / total) : 0.0f;
+            *reinterpret_cast<float4*>(&sh_s[g][r][t]) = p4;
+        }
     }
     __syncthreads();
 
