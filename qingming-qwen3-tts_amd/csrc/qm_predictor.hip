@@ -160,55 +160,58 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
         sh_r[tid] = 1.0f / sqrtf(total / 128.0f + prm.epsilon);
     }
     __syncthreads();
-    // (3) One thread per (vector, four rotate_half pairs): normalise, gamma, RoPE with every bf16
-    //     rounding of R17:12207-12279.
-    for (int it = tid; it < n_vec * 16; it += kPredThreads) {
-        const int vec = it >> 4, d0 = (it & 15) * 4;
-        const int vrow = vec / 3, which = vec % 3;
-        uint16_t* x = which < 2 ? sh_q[which][vrow] : sh_k[vrow];
-        const uint16_t* gamma = sh_gamma[which < 2 ? 0 : 1];
-        const float r = sh_r[vec];
-        const uint2 xl = *reinterpret_cast<const uint2*>(x + d0), xh = *reinterpret_cast<const uint2*>(x + d0 + 64);
-        const uint2 gl = *reinterpret_cast<const uint2*>(gamma + d0), gh = *reinterpret_cast<const uint2*>(gamma + d0 + 64);
+    // (3) One thread per (row, four rotate_half pairs) for the row's three vectors, which share the
+    //     RoPE row (and the two q heads their gamma): normalise, gamma, RoPE with every bf16 rounding
+    //     of R17:12207-12279.
+    for (int it = tid; it < rows * 16; it += kPredThreads) {
+        const int vrow = it >> 4, d0 = (it & 15) * 4;
         const uint2 cl = *reinterpret_cast<const uint2*>(&sh_cos[vrow][d0]), ch = *reinterpret_cast<const uint2*>(&sh_cos[vrow][d0 + 64]);
         const uint2 sl = *reinterpret_cast<const uint2*>(&sh_sin[vrow][d0]), sh2 = *reinterpret_cast<const uint2*>(&sh_sin[vrow][d0 + 64]);
-        const uint32_t xlw[2] = {xl.x, xl.y}, xhw[2] = {xh.x, xh.y}, glw[2] = {gl.x, gl.y}, ghw[2] = {gh.x, gh.y};
         const uint32_t clw[2] = {cl.x, cl.y}, chw[2] = {ch.x, ch.y}, slw[2] = {sl.x, sl.y}, shw[2] = {sh2.x, sh2.y};
-        uint32_t out_lo[2], out_hi[2];
+        float c0[4], c1[4], s0[4], s1[4];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            float res_lo[2], res_hi[2];
+            c0[2 * j] = lo_bf16(clw[j]); c0[2 * j + 1] = hi_bf16(clw[j]);
+            c1[2 * j] = lo_bf16(chw[j]); c1[2 * j + 1] = hi_bf16(chw[j]);
+            s0[2 * j] = lo_bf16(slw[j]); s0[2 * j + 1] = hi_bf16(slw[j]);
+            s1[2 * j] = lo_bf16(shw[j]); s1[2 * j + 1] = hi_bf16(shw[j]);
+        }
+        float g0[4], g1[4];
 #pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const float x0 = e ? hi_bf16(xlw[j]) : lo_bf16(xlw[j]);
-                const float x1 = e ? hi_bf16(xhw[j]) : lo_bf16(xhw[j]);
-                const float g0 = e ? hi_bf16(glw[j]) : lo_bf16(glw[j]);
-                const float g1 = e ? hi_bf16(ghw[j]) : lo_bf16(ghw[j]);
-                const float c0 = e ? hi_bf16(clw[j]) : lo_bf16(clw[j]);
-                const float c1 = e ? hi_bf16(chw[j]) : lo_bf16(chw[j]);
-                const float s0 = e ? hi_bf16(slw[j]) : lo_bf16(slw[j]);
-                const float s1 = e ? hi_bf16(shw[j]) : lo_bf16(shw[j]);
+        for (int which = 0; which < 3; ++which) {
+            if (which != 1) {   // head 1 reuses head 0's gamma
+                const uint16_t* gamma = sh_gamma[which < 2 ? 0 : 1];
+                const uint2 gl = *reinterpret_cast<const uint2*>(gamma + d0), gh = *reinterpret_cast<const uint2*>(gamma + d0 + 64);
+                g0[0] = lo_bf16(gl.x); g0[1] = hi_bf16(gl.x); g0[2] = lo_bf16(gl.y); g0[3] = hi_bf16(gl.y);
+                g1[0] = lo_bf16(gh.x); g1[1] = hi_bf16(gh.x); g1[2] = lo_bf16(gh.y); g1[3] = hi_bf16(gh.y);
+            }
+            uint16_t* x = which < 2 ? sh_q[which][vrow] : sh_k[vrow];
+            const float r = sh_r[vrow * 3 + which];
+            const uint2 xl = *reinterpret_cast<const uint2*>(x + d0), xh = *reinterpret_cast<const uint2*>(x + d0 + 64);
+            const float x0[4] = {lo_bf16(xl.x), hi_bf16(xl.x), lo_bf16(xl.y), hi_bf16(xl.y)};
+            const float x1[4] = {lo_bf16(xh.x), hi_bf16(xh.x), lo_bf16(xh.y), hi_bf16(xh.y)};
+            float res_lo[4], res_hi[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
                 float n0, n1, w0, w1, f0, f1, t0, t1;
-                round_bf16_pair(x0 * r, x1 * r, n0, n1);
-                round_bf16_pair(n0 * g0, n1 * g1, w0, w1);
-                round_bf16_pair(w0 * c0, w1 * c1, f0, f1);
-                round_bf16_pair((-w1) * s0, w0 * s1, t0, t1);
+                round_bf16_pair(x0[e] * r, x1[e] * r, n0, n1);
+                round_bf16_pair(n0 * g0[e], n1 * g1[e], w0, w1);
+                round_bf16_pair(w0 * c0[e], w1 * c1[e], f0, f1);
+                round_bf16_pair((-w1) * s0[e], w0 * s1[e], t0, t1);
                 res_lo[e] = f0 + t0;
                 res_hi[e] = f1 + t1;
             }
-            float dummy0, dummy1;
-            (void)dummy0; (void)dummy1;
-            out_lo[j] = pack_bf16_pair(res_lo[0], res_lo[1]);
-            out_hi[j] = pack_bf16_pair(res_hi[0], res_hi[1]);
-        }
-        *reinterpret_cast<uint2*>(x + d0) = make_uint2(out_lo[0], out_lo[1]);
-        *reinterpret_cast<uint2*>(x + d0 + 64) = make_uint2(out_hi[0], out_hi[1]);
-        if (which == 2) {
-            // every wave reads all of K for the scores: widen it once here instead of four times there
-            *reinterpret_cast<float4*>(&sh_kf[vrow][d0]) =
-                make_float4(lo_bf16(out_lo[0]), hi_bf16(out_lo[0]), lo_bf16(out_lo[1]), hi_bf16(out_lo[1]));
-            *reinterpret_cast<float4*>(&sh_kf[vrow][d0 + 64]) =
-                make_float4(lo_bf16(out_hi[0]), hi_bf16(out_hi[0]), lo_bf16(out_hi[1]), hi_bf16(out_hi[1]));
+            const uint32_t out_lo[2] = {pack_bf16_pair(res_lo[0], res_lo[1]), pack_bf16_pair(res_lo[2], res_lo[3])};
+            const uint32_t out_hi[2] = {pack_bf16_pair(res_hi[0], res_hi[1]), pack_bf16_pair(res_hi[2], res_hi[3])};
+            *reinterpret_cast<uint2*>(x + d0) = make_uint2(out_lo[0], out_lo[1]);
+            *reinterpret_cast<uint2*>(x + d0 + 64) = make_uint2(out_hi[0], out_hi[1]);
+            if (which == 2) {
+                // every wave reads all of K for the scores: widen it once here instead of four times there
+                *reinterpret_cast<float4*>(&sh_kf[vrow][d0]) =
+                    make_float4(lo_bf16(out_lo[0]), hi_bf16(out_lo[0]), lo_bf16(out_lo[1]), hi_bf16(out_lo[1]));
+                *reinterpret_cast<float4*>(&sh_kf[vrow][d0 + 64]) =
+                    make_float4(lo_bf16(out_hi[0]), hi_bf16(out_hi[0]), lo_bf16(out_hi[1]), hi_bf16(out_hi[1]));
+            }
         }
     }
     __syncthreads();
