@@ -279,6 +279,110 @@ class QkvGemv:
         return {"all": dt}, 0.0 if exact else 1.0, "whole workload (bit-exact comparison)"
 
 
+class TalkerLayerStep:
+    """Beyond the five configurations: one whole decode step of a talker layer as the reference chains
+    it (R17:17155-17248) — RMSNorm, fused Q/K/V projection, QK-norm + RoPE + append, GQA decode over a
+    2048-token flat cache, o_proj, residual add + post-norm, gate/up/SwiGLU, down_proj + residual —
+    with `layers` distinct weight sets and caches used in rotation (hidden 2048, intermediate 6144 as
+    in Qwen3-1.7B; the reference reads it from the checkpoint, R17:14862)."""
+    bound = "hbm"
+    # the layer's output is a hidden state of magnitude up to ~8, where one bf16 ulp is 0.03-0.06: the
+    # attention's 1e-2 budget surfaces as at most a couple of ulps there
+    tolerance = 0.125
+
+    def __init__(self, qm, dev, layers=28, ctx=2048, seed=91, fused=True):
+        import torch
+        self.qm, self.layers, self.ctx, self.fused = qm, layers, ctx, fused
+        self.name = "talker_layer_decode_step_ctx%d_x%dlayers%s" % (ctx, layers, "" if fused else "_reference_launch_sequence")
+        self.copies = layers
+        gd = torch.Generator(device=dev).manual_seed(seed)
+        H, I = 2048, 6144
+        self.H, self.I = H, I
+
+        def rnd(shape, std=1.0, mean=0.0):
+            return (torch.randn(shape, generator=gd, device=dev, dtype=torch.float32) * std + mean).to(torch.bfloat16)
+
+        self.max_cache = ctx + 4
+        self.w = []
+        for _ in range(layers):
+            k, v = rnd((8, self.max_cache, 128)), rnd((8, self.max_cache, 128))
+            self.w.append(dict(
+                in_norm=rnd((H,), 0.1, 1.0), wq=rnd((H, H), 0.02), wk=rnd((1024, H), 0.02), wv=rnd((1024, H), 0.02),
+                gq=rnd((128,), 0.1, 1.0), gk=rnd((128,), 0.1, 1.0), wo=rnd((H, H), 0.02), post=rnd((H,), 0.1, 1.0),
+                wg=rnd((I, H), 0.02), wu=rnd((I, H), 0.02), wd=rnd((H, I), 0.02), k=k, v=v,
+                cache=qm.flat_cache(k, v, 8, self.max_cache)))
+        pos = ctx - 1
+        inv = 1.0e6 ** (-2.0 * np.arange(64, dtype=np.float64) / 128.0)
+        ang = np.concatenate([pos * inv, pos * inv])
+        self.cos = torch.tensor(np.cos(ang), dtype=torch.float32).to(torch.bfloat16).to(dev)
+        self.sin = torch.tensor(np.sin(ang), dtype=torch.float32).to(torch.bfloat16).to(dev)
+        z = lambda n: torch.zeros(n, dtype=torch.bfloat16, device=dev)
+        self.x = rnd((H,))
+        self.norm, self.q, self.k_, self.v_, self.qrot = z(H), z(H), z(1024), z(1024), z(H)
+        self.ctxv, self.attn, self.res, self.post, self.act, self.out = z(H), z(H), z(H), z(H), z(I), z(H)
+        self.ws_bytes = qm.decode_workspace_bytes(1, 16, 8, ctx)
+        self.ws = torch.empty(self.ws_bytes // 4 + 1, dtype=torch.float32, device=dev)
+        weights = 2 * (H * H + 2 * 1024 * H + H * H + 2 * I * H + H * I)
+        self.bytes = weights + 2 * 8 * ctx * 128 * 2 + 4096 + 2 * (6 * H + 2 * I)   # + KV + append + activations
+        self.flops = weights + 16 * ctx * 128 * 2 * 2
+        self.i = 0
+
+    def step(self):
+        import torch
+        s = torch.cuda.current_stream().cuda_stream
+        L = self.w[self.i % self.layers]
+        self.i += 1
+        qm, H, I = self.qm, self.H, self.I
+        if self.fused:
+            qm.rmsnorm_qkv_m1(self.x, L["in_norm"], L["wq"], None, L["wk"], None, L["wv"], None, self.q, self.k_,
+                              self.v_, H, H, 1024, 1e-6, s)
+        else:
+            qm.rmsnorm_rows(self.x, L["in_norm"], self.norm, 1, H, 1e-6, s)
+            qm.qkv_m1(self.norm, L["wq"], None, L["wk"], None, L["wv"], None, self.q, self.k_, self.v_, H, H, 1024, s)
+        qm.qk_norm_rope_kv_append(self.q, self.k_, self.v_, L["gq"], L["gk"], self.cos, self.sin, self.qrot, L["cache"],
+                                  None, 1, 16, self.ctx - 1, 1e-6, s)
+        qm.decode_attention(self.qrot, L["cache"], None, 1, self.ctxv, 16, self.ctx - 1, -1, SCALE, self.ws,
+                            self.ws_bytes, s)
+        qm.linear_m1(self.ctxv, L["wo"], None, None, self.attn, H, H, s)
+        if self.fused:
+            qm.add_postnorm_gate_up_swiglu_m1(self.x, self.attn, L["post"], self.res, L["wg"], L["wu"], self.act, H, I,
+                                              1e-6, s)
+        else:
+            qm.add_postnorm_m1(self.x, self.attn, L["post"], self.res, self.post, H, 1e-6, s)
+            qm.gate_up_swiglu_m1(self.post, L["wg"], L["wu"], self.act, H, I, s)
+        qm.linear_m1(self.act, L["wd"], None, self.res, self.out, H, I, s)
+
+    def cpu_baseline(self, oracle, threads):
+        """One layer on the host; the comparison is on that layer's output hidden state."""
+        import torch
+        self.i = 0
+        self.step()
+        torch.cuda.synchronize()
+        L = {k: (_bits(v).copy() if hasattr(v, "detach") else v) for k, v in self.w[0].items()}
+        H, I = self.H, self.I
+        x = _bits(self.x).copy()
+        u16 = lambda n: np.zeros(n, dtype=np.uint16)
+        norm, q, k, v, qrot, ctxv, attn, res, post, act, out = (u16(H).reshape(1, H), u16(H), u16(1024), u16(1024),
+                                                                u16(H), u16(H), u16(H), u16(H), u16(H), u16(I), u16(H))
+        # the GPU step already appended position ctx-1 to layer 0's cache: the oracle overwrites it with the same bits
+        cache = oracle.flat_cache(L["k"], L["v"], 8, self.max_cache)
+        t0 = time.perf_counter()
+        assert oracle.rmsnorm_rows(x.reshape(1, H), L["in_norm"], norm, 1, H) == 0
+        assert oracle.qkv_m1(norm[0], L["wq"], None, L["wk"], None, L["wv"], None, q, k, v, H, H, 1024, threads) == 0
+        assert oracle.qk_norm_rope_kv_append(q, k, v, L["gq"], L["gk"], _bits(self.cos), _bits(self.sin), qrot, cache,
+                                             None, 1, 16, self.ctx - 1) == 0
+        assert oracle.attention(qrot, cache, None, 1, ctxv, 1, self.ctx - 1, 16, -1, SCALE, oracle.POLICY_ONLINE,
+                                threads) == 0
+        assert oracle.linear_m1(ctxv, L["wo"], None, None, attn, H, H, threads) == 0
+        assert oracle.add_postnorm_m1(x, attn, L["post"], res, post, H) == 0
+        assert oracle.gate_up_swiglu_m1(post, L["wg"], L["wu"], act, H, I, threads) == 0
+        assert oracle.linear_m1(act, L["wd"], None, res, out, H, I, threads) == 0
+        dt = time.perf_counter() - t0
+        err = float(np.max(np.abs(oracle.bf16_to_f32(out).astype(np.float64)
+                                  - oracle.bf16_to_f32(_bits(self.out)).astype(np.float64))))
+        return {"all": dt}, err, "one layer step"
+
+
 class Prefill:
     """configs[3]: causal GQA prefill, batch 4 x seq 1024, K/V also written to shuffled 16-token pages."""
     name = "causal_prefill_b4_s1024_paged16"
@@ -394,7 +498,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
-    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "predictor", "qkv"], default=None,
+    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "predictor", "qkv", "layer"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -428,7 +532,7 @@ def main():
         make = {"decode512": lambda: SingleDecode(qm, dev, 512, False, 11),
                 "talker2048": lambda: SingleDecode(qm, dev, 2048, True, 12),
                 "prefill": lambda: Prefill(qm, dev), "predictor": lambda: PredictorLoop(qm, dev),
-                "qkv": lambda: QkvGemv(qm, dev, copies=64)}[args.only]
+                "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev)}[args.only]
         w = make()
         r = _report(w, _time_steps(w.step, args.steps, args.warmup))
         r["bound"] = w.bound
@@ -461,6 +565,9 @@ def main():
             # beyond the five configurations: the M = 1 projection in front of configuration 2
             ("next_qkv_gemv_m1", lambda: QkvGemv(qm, dev)),
             ("next_qkv_gemv_m1_rotating64", lambda: QkvGemv(qm, dev, copies=64)),
+            # the whole decode step of one talker layer, 28 layers' weights and caches in rotation (2.8 GB)
+            ("next_talker_layer_decode_step", lambda: TalkerLayerStep(qm, dev)),
+            ("next_talker_layer_decode_step_unfused", lambda: TalkerLayerStep(qm, dev, fused=False)),
         ]
         for key, make in extra:
             w = make()
@@ -474,9 +581,10 @@ def main():
             if isinstance(w, PredictorLoop):
                 r["us_per_predictor_step"] = r["us_per_step_graph"] / w.rows
                 r["us_per_frame"] = r["us_per_step_graph"] / w.frames
-            if oracle is not None and not (isinstance(w, PredictorLoop) and w.kc is not None) and copies == 1:
+            if oracle is not None and not (isinstance(w, PredictorLoop) and w.kc is not None) \
+                    and (copies == 1 or isinstance(w, TalkerLayerStep)):
                 res, err, sample = w.cpu_baseline(oracle, threads)
-                if err > 1e-2:
+                if err > getattr(w, "tolerance", 1e-2):
                     raise RuntimeError(f"{key}: GPU result differs from the oracle: max abs err {err}")
                 r["cpu_oracle"] = {"seconds": res["all"], "cores": threads, "sample": sample,
                                    "gpu_vs_oracle_max_abs_err": err,

@@ -269,6 +269,60 @@ int32_t qm_qkv_m1(
     int32_t hidden, int32_t q_dim, int32_t kv_dim,
     void* hip_stream);
 
+/*
+ * qm_gate_up_swiglu_m1 replaces launch_gate_up_swiglu_m1 / talker_gate_up_swiglu_fused_kernel
+ * (R17:17848-17890, 16289-16362): per channel c, g = bf16(input . gate_weight[c]),
+ * u = bf16(input . up_weight[c]) in the M = 1 linear's summation order,
+ * output[c] = bf16(bf16(g / (1 + expf(-g))) * u).  Weights [intermediate][hidden]; same limits
+ * as qm_linear_m1.  Bit-identical up to the device's expf.
+ */
+int32_t qm_gate_up_swiglu_m1(
+    const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight,
+    uint16_t* output, int32_t hidden, int32_t intermediate,
+    void* hip_stream);
+/*
+ * qm_rmsnorm_rows replaces launch_rmsnorm / rmsnorm_kernel (R17:8908-8929, 8276-8338):
+ * output[r][c] = bf16(bf16(input[r][c] * inverse_rms_r) * weight[c]), the statistic summed in the
+ * reference's 256-thread order.  qm_add_postnorm_m1 replaces launch_add_postnorm_m1 /
+ * talker_add_postnorm_fused_kernel (R17:17817-17846, 16205-16286): residual = bf16(hidden +
+ * attention), normalized = the RMSNorm of that rounded residual.  dimension <= 32768 there.
+ */
+int32_t qm_rmsnorm_rows(
+    const uint16_t* input, const uint16_t* weight, uint16_t* output,
+    int32_t rows, int32_t dimension, float epsilon,
+    void* hip_stream);
+int32_t qm_add_postnorm_m1(
+    const uint16_t* hidden, const uint16_t* attention, const uint16_t* norm_weight,
+    uint16_t* residual, uint16_t* normalized, int32_t dimension, float epsilon,
+    void* hip_stream);
+
+/*
+ * Two fusions of consecutive reference launches of a decode layer; the fused results are
+ * bit-identical to running the two operators one after the other:
+ * qm_rmsnorm_qkv_m1 = launch_rmsnorm(hidden_state, input_norm) (R17:17163-17169) followed by
+ * launch_qkv_m1 (R17:17174-17176): every block normalises the hidden state itself while its
+ * weights are in flight, the normalised vector never goes to memory.
+ * qm_add_postnorm_gate_up_swiglu_m1 = launch_add_postnorm_m1 (R17:17215-17220) followed by
+ * launch_gate_up_swiglu_m1 (R17:17226-17229); `residual` (= bf16(hidden_state + attention), which
+ * down_proj adds later) is written, the post-norm vector is not.
+ * Both need hidden % 8 == 0, hidden <= 16384 and 16-byte aligned weight matrices
+ * (QM_ERR_GEOMETRY otherwise).
+ */
+int32_t qm_rmsnorm_qkv_m1(
+    const uint16_t* hidden_state, const uint16_t* norm_weight, float epsilon,
+    const uint16_t* q_weight, const uint16_t* q_bias,
+    const uint16_t* k_weight, const uint16_t* k_bias,
+    const uint16_t* v_weight, const uint16_t* v_bias,
+    uint16_t* q_output, uint16_t* k_output, uint16_t* v_output,
+    int32_t hidden, int32_t q_dim, int32_t kv_dim,
+    void* hip_stream);
+int32_t qm_add_postnorm_gate_up_swiglu_m1(
+    const uint16_t* hidden_state, const uint16_t* attention, const uint16_t* norm_weight, float epsilon,
+    uint16_t* residual,
+    const uint16_t* gate_weight, const uint16_t* up_weight, uint16_t* output,
+    int32_t hidden, int32_t intermediate,
+    void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

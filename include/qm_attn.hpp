@@ -196,6 +196,29 @@ inline void launch_qkv_m1(
           "Qingming fused QKV launch");
 }
 
+// launch_gate_up_swiglu_m1 (R17:17848-17890).
+inline void launch_gate_up_swiglu_m1(
+    const std::uint16_t* input, const std::uint16_t* gate_weight, const std::uint16_t* up_weight,
+    std::uint16_t* output, int hidden, int intermediate, void* stream) {
+    check(qm_gate_up_swiglu_m1(input, gate_weight, up_weight, output, hidden, intermediate, stream),
+          "Qingming gate/up/SwiGLU launch");
+}
+
+// code_predictor::launch_rmsnorm (R17:8908-8929); epsilon is the reference's kRmsEpsilon.
+inline void launch_rmsnorm(
+    const std::uint16_t* input, const std::uint16_t* weight, std::uint16_t* output, int rows, int dimension,
+    void* stream) {
+    check(qm_rmsnorm_rows(input, weight, output, rows, dimension, 1.0e-6f, stream), "rmsnorm launch");
+}
+
+// launch_add_postnorm_m1 (R17:17817-17846).
+inline void launch_add_postnorm_m1(
+    const std::uint16_t* hidden, const std::uint16_t* attention, const std::uint16_t* norm_weight,
+    std::uint16_t* residual, std::uint16_t* normalized, int dimension, void* stream) {
+    check(qm_add_postnorm_m1(hidden, attention, norm_weight, residual, normalized, dimension, 1.0e-6f, stream),
+          "Qingming add/postnorm launch");
+}
+
 }  // namespace qm_attn
 
 #endif  // QM_ATTN_HPP

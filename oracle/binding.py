@@ -202,3 +202,18 @@ def qkv_m1(x, q_w, q_b, k_w, k_b, v_w, v_b, q_out, k_out, v_out, hidden, q_dim, 
     return lib().qmo_qkv_m1(_p(x), _p(q_w), _p(q_b), _p(k_w), _p(k_b), _p(v_w), _p(v_b), _p(q_out),
                             _p(k_out), _p(v_out), C.c_int32(hidden), C.c_int32(q_dim), C.c_int32(kv_dim),
                             C.c_int32(threads))
+
+
+def rmsnorm_rows(x, weight, out, rows, dimension, eps=1e-6, threads=8):
+    return lib().qmo_rmsnorm_rows(_p(x), _p(weight), _p(out), C.c_int32(rows), C.c_int32(dimension),
+                                  C.c_float(eps), C.c_int32(threads))
+
+
+def add_postnorm_m1(hidden, attention, norm_weight, residual, normalized, dimension, eps=1e-6):
+    return lib().qmo_add_postnorm_m1(_p(hidden), _p(attention), _p(norm_weight), _p(residual), _p(normalized),
+                                     C.c_int32(dimension), C.c_float(eps))
+
+
+def gate_up_swiglu_m1(x, gate_w, up_w, out, hidden, intermediate, threads=8):
+    return lib().qmo_gate_up_swiglu_m1(_p(x), _p(gate_w), _p(up_w), _p(out), C.c_int32(hidden),
+                                       C.c_int32(intermediate), C.c_int32(threads))

@@ -736,4 +736,72 @@ int32_t qmo_qkv_m1(const uint16_t* input, const uint16_t* q_weight, const uint16
     return QM_OK;
 }
 
+// Sum over a 256-thread block of per-thread partial sums, thread t having accumulated the
+// columns t, t+256, ... with fmaf (R17:8291-8301, 16221-16251), reduced by block_reduce_sum /
+// talker_block_sum (eight 32-lane trees, then a tree over the eight results).
+static float strided_sum_squares_256(const uint16_t* x, int dimension) {
+    float per_thread[256];
+    for (int t = 0; t < 256; ++t) {
+        float acc = 0.0f;
+        for (int c = t; c < dimension; c += 256) {
+            const float v = bf2f(x[c]);
+            acc = std::fmaf(v, v, acc);
+        }
+        per_thread[t] = acc;
+    }
+    return block_sum(per_thread, 256);
+}
+
+// rmsnorm_kernel + launch_rmsnorm (R17:8276-8338, 8908-8929; 256 threads per row, epsilon
+// kRmsEpsilon = 1e-6 passed in): out = bf16(bf16(x * inverse_rms) * weight).
+int32_t qmo_rmsnorm_rows(const uint16_t* input, const uint16_t* weight, uint16_t* output, int32_t rows,
+                         int32_t dimension, float epsilon, int32_t n_threads) {
+    if (!input || !weight || !output) return QM_ERR_NULL;
+    if (rows < 0 || dimension <= 0) return QM_ERR_ARGUMENT;
+    parallel_for(rows, n_threads, [&](int64_t r) {
+        const uint16_t* x = input + r * dimension;
+        const float sum = strided_sum_squares_256(x, dimension);
+        const float inv = 1.0f / std::sqrt(sum / static_cast<float>(dimension) + epsilon);
+        for (int c = 0; c < dimension; ++c) {
+            const uint16_t n = f2bf(bf2f(x[c]) * inv);
+            output[r * dimension + c] = f2bf(bf2f(n) * bf2f(weight[c]));
+        }
+    });
+    return QM_OK;
+}
+
+// talker_add_postnorm_fused_kernel + launch_add_postnorm_m1 (R17:16205-16286, 17817-17846):
+// residual = bf16(hidden + attention); normalized = bf16(bf16(residual * inverse_rms) * weight),
+// the statistic taken over the rounded residual.
+int32_t qmo_add_postnorm_m1(const uint16_t* hidden, const uint16_t* attention, const uint16_t* norm_weight,
+                            uint16_t* residual, uint16_t* normalized, int32_t dimension, float epsilon) {
+    if (!hidden || !attention || !norm_weight || !residual || !normalized) return QM_ERR_NULL;
+    if (dimension <= 0) return QM_ERR_ARGUMENT;
+    for (int c = 0; c < dimension; ++c) residual[c] = f2bf(bf2f(hidden[c]) + bf2f(attention[c]));
+    const float sum = strided_sum_squares_256(residual, dimension);
+    const float inv = 1.0f / std::sqrt(sum / static_cast<float>(dimension) + epsilon);
+    for (int c = 0; c < dimension; ++c) {
+        const uint16_t n = f2bf(bf2f(residual[c]) * inv);
+        normalized[c] = f2bf(bf2f(n) * bf2f(norm_weight[c]));
+    }
+    return QM_OK;
+}
+
+// talker_gate_up_swiglu_fused_kernel + launch_gate_up_swiglu_m1 (R17:16289-16362, 17848-17890):
+// per channel two dot products in the M = 1 linear's order (no bias), each rounded to bf16;
+// act = bf16(g / (1 + expf(-g))); out = bf16(act * u).
+int32_t qmo_gate_up_swiglu_m1(const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight,
+                              uint16_t* output, int32_t hidden, int32_t intermediate, int32_t n_threads) {
+    if (!input || !gate_weight || !up_weight || !output) return QM_ERR_NULL;
+    if (hidden < 0 || intermediate < 0) return QM_ERR_ARGUMENT;
+    parallel_for(intermediate, n_threads, [&](int64_t ch) {
+        const uint16_t gb = linear_m1_scalar(input, gate_weight + ch * hidden, nullptr, nullptr, 0, hidden);
+        const uint16_t ub = linear_m1_scalar(input, up_weight + ch * hidden, nullptr, nullptr, 0, hidden);
+        const float gv = bf2f(gb);
+        const uint16_t act = f2bf(gv / (1.0f + std::exp(-gv)));
+        output[ch] = f2bf(bf2f(act) * bf2f(ub));
+    });
+    return QM_OK;
+}
+
 }  // extern "C"

@@ -62,6 +62,11 @@ _SIGNATURES = {
     "qm_predictor_attention_loop": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _I32, _F32, _PTR]),
     "qm_linear_m1": (_I32, [_PTR] * 5 + [_I32, _I32, _PTR]),
     "qm_qkv_m1": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _PTR]),
+    "qm_gate_up_swiglu_m1": (_I32, [_PTR] * 4 + [_I32, _I32, _PTR]),
+    "qm_rmsnorm_rows": (_I32, [_PTR] * 3 + [_I32, _I32, _F32, _PTR]),
+    "qm_add_postnorm_m1": (_I32, [_PTR] * 5 + [_I32, _F32, _PTR]),
+    "qm_rmsnorm_qkv_m1": (_I32, [_PTR, _PTR, _F32] + [_PTR] * 9 + [_I32, _I32, _I32, _PTR]),
+    "qm_add_postnorm_gate_up_swiglu_m1": (_I32, [_PTR, _PTR, _PTR, _F32] + [_PTR] * 4 + [_I32, _I32, _PTR]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
@@ -200,3 +205,31 @@ def qkv_m1(x, q_w, q_b, k_w, k_b, v_w, v_b, q_out, k_out, v_out, hidden, q_dim, 
     _check(lib().qm_qkv_m1(_addr(x), _addr(q_w), _addr(q_b), _addr(k_w), _addr(k_b), _addr(v_w), _addr(v_b),
                            _addr(q_out), _addr(k_out), _addr(v_out), hidden, q_dim, kv_dim, stream),
            "qm_qkv_m1")
+
+
+def gate_up_swiglu_m1(x, gate_w, up_w, out, hidden, intermediate, stream=0):
+    _check(lib().qm_gate_up_swiglu_m1(_addr(x), _addr(gate_w), _addr(up_w), _addr(out), hidden, intermediate, stream),
+           "qm_gate_up_swiglu_m1")
+
+
+def rmsnorm_rows(x, weight, out, rows, dimension, eps=1e-6, stream=0):
+    _check(lib().qm_rmsnorm_rows(_addr(x), _addr(weight), _addr(out), rows, dimension, eps, stream), "qm_rmsnorm_rows")
+
+
+def add_postnorm_m1(hidden, attention, norm_weight, residual, normalized, dimension, eps=1e-6, stream=0):
+    _check(lib().qm_add_postnorm_m1(_addr(hidden), _addr(attention), _addr(norm_weight), _addr(residual),
+                                    _addr(normalized), dimension, eps, stream), "qm_add_postnorm_m1")
+
+
+def rmsnorm_qkv_m1(hidden_state, norm_weight, q_w, q_b, k_w, k_b, v_w, v_b, q_out, k_out, v_out, hidden, q_dim,
+                   kv_dim, eps=1e-6, stream=0):
+    _check(lib().qm_rmsnorm_qkv_m1(_addr(hidden_state), _addr(norm_weight), eps, _addr(q_w), _addr(q_b), _addr(k_w),
+                                   _addr(k_b), _addr(v_w), _addr(v_b), _addr(q_out), _addr(k_out), _addr(v_out),
+                                   hidden, q_dim, kv_dim, stream), "qm_rmsnorm_qkv_m1")
+
+
+def add_postnorm_gate_up_swiglu_m1(hidden_state, attention, norm_weight, residual, gate_w, up_w, out, hidden,
+                                   intermediate, eps=1e-6, stream=0):
+    _check(lib().qm_add_postnorm_gate_up_swiglu_m1(_addr(hidden_state), _addr(attention), _addr(norm_weight), eps,
+                                                   _addr(residual), _addr(gate_w), _addr(up_w), _addr(out), hidden,
+                                                   intermediate, stream), "qm_add_postnorm_gate_up_swiglu_m1")

@@ -124,4 +124,23 @@ __device__ __forceinline__ int64_t tile_offset(const qm_kv_cache& c, const PageM
          + static_cast<int64_t>(first_token - page * pm.page_size) * kDim;
 }
 
+// block_reduce_sum / talker_block_sum of the reference (R17:8233-8274, 15102-15148) for a block of 256
+// threads: eight 32-lane shfl_down trees, then one tree over the eight results.  sh_waves: 8 floats,
+// sh_total: 1 float of LDS; the total is valid in every thread.
+__device__ __forceinline__ float block_sum_256_like_reference(float value, float* sh_waves, float* sh_total) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int offset = 16; offset > 0; offset >>= 1) value += __shfl_down(value, offset, 32);
+    if ((tid & 31) == 0) sh_waves[tid >> 5] = value;
+    __syncthreads();
+    if (tid < 32) {
+        float v = tid < 8 ? sh_waves[tid] : 0.0f;
+#pragma unroll
+        for (int offset = 16; offset > 0; offset >>= 1) v += __shfl_down(v, offset, 32);
+        if (tid == 0) *sh_total = v;
+    }
+    __syncthreads();
+    return *sh_total;
+}
+
 }  // namespace qm

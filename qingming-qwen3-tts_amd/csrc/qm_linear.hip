@@ -1,5 +1,6 @@
 // qm_linear.hip — M = 1 weight-streaming linears (fused Q/K/V projection, o_proj / down_proj with
-// bias and residual) for gfx950, bit-identical to the reference's kernels.
+// bias and residual, gate/up projection with SwiGLU) for gfx950, bit-identical to the reference's
+// kernels.
 //
 // What fixes the design.  The reference computes one output scalar per 32-lane wave: lane l
 // accumulates the products k = l, l+32, l+64, ... with fmaf in increasing k, the 32 lane sums go
@@ -37,10 +38,22 @@ struct LinearParams {
     const uint16_t* residual;     // [rows_0] or NULL (single-matrix form only)
     int rows[3];
     int reduction;
+    // Fused prologue of the staged kernel (pre != 0): the input vector is produced in the block.
+    int pre;                      // 1: RMSNorm(input) * norm_weight; 2: RMSNorm(bf16(input + addend)) * norm_weight
+    const uint16_t* addend;       // pre == 2: the attention output added to the hidden state
+    const uint16_t* norm_weight;  // [reduction]
+    uint16_t* residual_out;       // pre == 2: bf16(input + addend), written by block 0
+    float epsilon;
+    int rows_per_block;           // staged kernel: outputs (channels) per block, 1..8
 };
 
+// DUAL: weight[0] / weight[1] are the gate and up matrices of one SwiGLU channel per output
+// (talker_gate_up_swiglu_fused_kernel, R17:16289-16362): two dot products in the same order, each
+// rounded to bf16, then act = bf16(g / (1 + expf(-g))) and out = bf16(act * u).
+template <bool DUAL>
 __global__ __launch_bounds__(kLinThreads) void linear_m1_kernel(LinearParams prm) {
     extern __shared__ __attribute__((aligned(16))) float lin_x[];   // the input vector, fp32
+    constexpr int kBatch = DUAL ? kLinBatch / 2 : kLinBatch;        // loads per matrix and register batch
 
     const int tid = threadIdx.x;
     const int q = tid & 15;                                         // lane within the output's row
@@ -50,7 +63,7 @@ __global__ __launch_bounds__(kLinThreads) void linear_m1_kernel(LinearParams prm
     // This lane's output: global row index over the concatenation of the (up to) three matrices.
     int row = static_cast<int>(blockIdx.x) * kLinRowsPerBlock + (tid >> 4);
     int m = 0;
-    if (row >= prm.rows[0]) {
+    if (!DUAL && row >= prm.rows[0]) {
         row -= prm.rows[0];
         m = 1;
         if (row >= prm.rows[1]) {
@@ -59,95 +72,315 @@ __global__ __launch_bounds__(kLinThreads) void linear_m1_kernel(LinearParams prm
         }
     }
     const bool live = row < prm.rows[m];
-    const uint16_t* wrow = prm.weight[m] + static_cast<int64_t>(live ? row : 0) * reduction;
+    const int64_t row_off = static_cast<int64_t>(live ? row : 0) * reduction;
+    const uint16_t* wrow = prm.weight[m] + row_off;
+    const uint16_t* urow = prm.weight[1] + row_off;   // DUAL only
 
-    // Steps [j0, j0 + kLinBatch) of this lane's weight row: elements 32j + 2q, 32j + 2q + 1.
+    // Steps [j0, j0 + kBatch) of this lane's weight row(s): elements 32j + 2q, 32j + 2q + 1.
     // Unpredicated: a lane without an output reads row 0, a step past the end the last pair.
-    auto load_batch = [&](uint32_t (&w)[kLinBatch], int j0) {
+    auto load_batch = [&](uint32_t (&w)[kBatch], uint32_t (&u)[kBatch], int j0) {
 #pragma unroll
-        for (int u = 0; u < kLinBatch; ++u) {
-            const int k = min(32 * (j0 + u) + 2 * q, reduction - 2);
-            w[u] = *reinterpret_cast<const uint32_t*>(wrow + k);
+        for (int i = 0; i < kBatch; ++i) {
+            const int k = min(32 * (j0 + i) + 2 * q, reduction - 2);
+            w[i] = *reinterpret_cast<const uint32_t*>(wrow + k);
+            if (DUAL) u[i] = *reinterpret_cast<const uint32_t*>(urow + k);
         }
     };
-    uint32_t wa[kLinBatch], wb[kLinBatch];
-    load_batch(wa, 0);
-    if (kLinBatch < steps) load_batch(wb, kLinBatch);
+    uint32_t wa[kBatch], wb[kBatch], ua[kBatch], ub[kBatch];
+    load_batch(wa, ua, 0);
+    if (kBatch < steps) load_batch(wb, ub, kBatch);
 
     // fp32 input vector, zero-padded to whole steps of 32.
     for (int k = tid; k < 32 * steps; k += kLinThreads) lin_x[k] = k < reduction ? bf2f(prm.input[k]) : 0.0f;
     __syncthreads();
 
-    float acc0 = 0.0f, acc1 = 0.0f;
-    // A whole batch is straight-line code (the LDS reads of its 32 input pairs are requested ahead
-    // of the multiply-adds); a batch cut by the end of the reduction takes the per-step test, and
-    // in a ragged last step the pairs past the end are multiplied as 0 * 0, which leaves the
+    float acc0 = 0.0f, acc1 = 0.0f, up0 = 0.0f, up1 = 0.0f;
+    // A whole batch is straight-line code (the LDS reads of its input pairs are requested ahead of
+    // the multiply-adds); a batch cut by the end of the reduction takes the per-step test, and in
+    // a ragged last step the pairs past the end are multiplied as 0 * 0, which leaves the
     // accumulators (never -0) unchanged.
-    auto consume_batch = [&](const uint32_t (&w)[kLinBatch], int j0) {
+    auto consume_batch = [&](const uint32_t (&w)[kBatch], const uint32_t (&u)[kBatch], int j0) {
         const float* xs = lin_x + 32 * j0 + 2 * q;
-        if (j0 + kLinBatch <= steps && 32 * steps == reduction) {
-            float2 x[kLinBatch];
+        if (j0 + kBatch <= steps && 32 * steps == reduction) {
+            float2 x[kBatch];
 #pragma unroll
-            for (int u = 0; u < kLinBatch; ++u) x[u] = *reinterpret_cast<const float2*>(xs + 32 * u);
+            for (int i = 0; i < kBatch; ++i) x[i] = *reinterpret_cast<const float2*>(xs + 32 * i);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int u = 0; u < kLinBatch; ++u) {
-                acc0 = fmaf(x[u].x, lo_bf16(w[u]), acc0);
-                acc1 = fmaf(x[u].y, hi_bf16(w[u]), acc1);
+            for (int i = 0; i < kBatch; ++i) {
+                acc0 = fmaf(x[i].x, lo_bf16(w[i]), acc0);
+                acc1 = fmaf(x[i].y, hi_bf16(w[i]), acc1);
+                if (DUAL) {
+                    up0 = fmaf(x[i].x, lo_bf16(u[i]), up0);
+                    up1 = fmaf(x[i].y, hi_bf16(u[i]), up1);
+                }
             }
         } else {
 #pragma unroll
-            for (int u = 0; u < kLinBatch; ++u) {
-                if (j0 + u < steps) {
-                    const float2 x = *reinterpret_cast<const float2*>(xs + 32 * u);
-                    const uint32_t wu = 32 * (j0 + u) + 2 * q < reduction ? w[u] : 0u;
-                    acc0 = fmaf(x.x, lo_bf16(wu), acc0);
-                    acc1 = fmaf(x.y, hi_bf16(wu), acc1);
+            for (int i = 0; i < kBatch; ++i) {
+                if (j0 + i < steps) {
+                    const float2 x = *reinterpret_cast<const float2*>(xs + 32 * i);
+                    const bool inside = 32 * (j0 + i) + 2 * q < reduction;
+                    const uint32_t wi = inside ? w[i] : 0u;
+                    acc0 = fmaf(x.x, lo_bf16(wi), acc0);
+                    acc1 = fmaf(x.y, hi_bf16(wi), acc1);
+                    if (DUAL) {
+                        const uint32_t ui = inside ? u[i] : 0u;
+                        up0 = fmaf(x.x, lo_bf16(ui), up0);
+                        up1 = fmaf(x.y, hi_bf16(ui), up1);
+                    }
                 }
             }
         }
     };
-    for (int j0 = 0; j0 < steps; j0 += 2 * kLinBatch) {
-        consume_batch(wa, j0);
-        if (j0 + 2 * kLinBatch < steps) load_batch(wa, j0 + 2 * kLinBatch);
-        if (j0 + kLinBatch < steps) consume_batch(wb, j0 + kLinBatch);
-        if (j0 + 3 * kLinBatch < steps) load_batch(wb, j0 + 3 * kLinBatch);
+    for (int j0 = 0; j0 < steps; j0 += 2 * kBatch) {
+        consume_batch(wa, ua, j0);
+        if (j0 + 2 * kBatch < steps) load_batch(wa, ua, j0 + 2 * kBatch);
+        if (j0 + kBatch < steps) consume_batch(wb, ub, j0 + kBatch);
+        if (j0 + 3 * kBatch < steps) load_batch(wb, ub, j0 + 3 * kBatch);
     }
 
     // The reference's tree over its 32 lanes, v += shfl_down(v, 16 / 8 / 4 / 2 / 1): chain c lives in
     // lane c/2, accumulator c%2, so +16, +8, +4, +2 are lanes q+8, q+4, q+2, q+1 (row_ror by
     // 8, 12, 14, 15 brings lane q+n to lane q) and +1 is the other accumulator of lane 0.
-    acc0 += row_ror<8>(acc0);
-    acc1 += row_ror<8>(acc1);
-    acc0 += row_ror<12>(acc0);
-    acc1 += row_ror<12>(acc1);
-    acc0 += row_ror<14>(acc0);
-    acc1 += row_ror<14>(acc1);
-    acc0 += row_ror<15>(acc0);
-    acc1 += row_ror<15>(acc1);
+    auto tree = [&](float a0, float a1) {
+        a0 += row_ror<8>(a0);
+        a1 += row_ror<8>(a1);
+        a0 += row_ror<12>(a0);
+        a1 += row_ror<12>(a1);
+        a0 += row_ror<14>(a0);
+        a1 += row_ror<14>(a1);
+        a0 += row_ror<15>(a0);
+        a1 += row_ror<15>(a1);
+        return a0 + a1;
+    };
+    const float a = tree(acc0, acc1);
+    const float u_sum = DUAL ? tree(up0, up1) : 0.0f;
     if (q == 0 && live) {
-        float a = acc0 + acc1;
-        if (prm.bias[m]) a += bf2f(prm.bias[m][row]);
-        uint16_t v = f2bf(a);
-        if (prm.residual) v = f2bf(bf2f(prm.residual[row]) + bf2f(v));
-        prm.output[m][row] = v;
+        if (DUAL) {
+            const float gv = bf2f(f2bf(a));
+            const uint16_t act = f2bf(gv / (1.0f + expf(-gv)));
+            prm.output[0][row] = f2bf(bf2f(act) * bf2f(f2bf(u_sum)));
+        } else {
+            float r = a;
+            if (prm.bias[m]) r += bf2f(prm.bias[m][row]);
+            uint16_t v = f2bf(r);
+            if (prm.residual) v = f2bf(bf2f(prm.residual[row]) + bf2f(v));
+            prm.output[m][row] = v;
+        }
     }
 }
 
+template <bool DUAL>
 inline int32_t launch_linear(const LinearParams& prm, hipStream_t s) {
-    const int64_t total = static_cast<int64_t>(prm.rows[0]) + prm.rows[1] + prm.rows[2];
+    const int64_t total = DUAL ? prm.rows[0] : static_cast<int64_t>(prm.rows[0]) + prm.rows[1] + prm.rows[2];
     if (total == 0) return QM_OK;
     const size_t smem = static_cast<size_t>((prm.reduction + 31) / 32 * 32) * sizeof(float);
     static bool attr_set = false;
     if (!attr_set) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(linear_m1_kernel),
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(linear_m1_kernel<DUAL>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize,
                                                  kLinMaxReduction * static_cast<int>(sizeof(float)));
         if (e != hipSuccess) return hip_code(e);
         attr_set = true;
     }
     const unsigned blocks = static_cast<unsigned>((total + kLinRowsPerBlock - 1) / kLinRowsPerBlock);
-    hipLaunchKernelGGL(linear_m1_kernel, dim3(blocks), dim3(kLinThreads), smem, s, prm);
+    hipLaunchKernelGGL(linear_m1_kernel<DUAL>, dim3(blocks), dim3(kLinThreads), smem, s, prm);
+    return launch_status();
+}
+
+// ---- the staged kernel ---------------------------------------------------------------------------------
+// The register path above can keep at most 64 loads of a lane in flight (the hardware's counter
+// of outstanding vector memory instructions), which is 4 KB per output whatever the lane layout, and
+// the order of a chain's additions forbids splitting one output over more lanes: 2 048 outputs of a
+// 6 144-wide reduction moved 1.1 TB/s.  Here the memory traffic is decoupled from the summation
+// order: a block copies the weight rows of its (up to) eight outputs straight from HBM into LDS
+// with 16-byte global_load_lds instructions — every byte of the matrix is requested at once
+// across the chip, no registers held — and only then do 8 x 32 threads walk their chains, one
+// reference lane each, reading 2-byte weights and the fp32 input from LDS.  LDS rows are padded by
+// 64 bytes so the two rows a wave reads in one instruction fall on different banks.
+// The block may also produce its input vector itself (RMSNorm of the hidden state, or residual
+// add + post-norm), in the reference kernels' own thread layout and summation order, while the
+// weights are in flight; that removes two single-block launches from a decode layer.
+constexpr int kStagedThreads = 256;
+constexpr int kStagedMaxRows = 8;
+constexpr int kStagedLdsBudget = 156 * 1024;
+
+__host__ __device__ inline int staged_row_stride(int reduction) { return 2 * reduction + 64; }   // bytes
+__host__ __device__ inline int staged_x_floats(int reduction) { return (reduction + 31) / 32 * 32; }
+
+template <bool DUAL>
+__global__ __launch_bounds__(kStagedThreads) void linear_m1_staged_kernel(LinearParams prm) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char st_smem[];
+    __shared__ float sh_waves[8];
+    __shared__ float sh_total;
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int K = prm.reduction;
+    const int R = prm.rows_per_block;
+    const int row_stride = staged_row_stride(K);
+    float* lin_x = reinterpret_cast<float*>(st_smem);
+    unsigned char* lds_w = st_smem + staged_x_floats(K) * sizeof(float);
+    const int first = static_cast<int>(blockIdx.x) * R;     // first output (channel) of the block
+
+    // ---- request the weight rows: LDS row i of the block <- row (first + i) of its matrix ----------
+    // (DUAL: LDS rows 2c, 2c+1 are the gate and up rows of channel first + c)
+    const int lds_rows = DUAL ? 2 * R : R;
+    const int row_bytes = 2 * K;
+    for (int i = 0; i < lds_rows; ++i) {
+        int out = first + (DUAL ? i >> 1 : i);
+        int m = DUAL ? (i & 1) : 0;
+        if (!DUAL && out >= prm.rows[0]) {
+            out -= prm.rows[0];
+            m = 1;
+            if (out >= prm.rows[1]) {
+                out -= prm.rows[1];
+                m = 2;
+            }
+        }
+        if (out >= prm.rows[DUAL ? 0 : m]) break;           // past the last output (wave-uniform)
+        const unsigned char* src = reinterpret_cast<const unsigned char*>(prm.weight[m] + static_cast<int64_t>(out) * K);
+        unsigned char* dst = lds_w + i * row_stride;
+        for (int off = wave * 1024; off < row_bytes; off += 4 * 1024) {
+            if (off + lane * 16 < row_bytes) {
+                __builtin_amdgcn_global_load_lds(src + off + lane * 16,
+                                                 (__attribute__((address_space(3))) void*)(dst + off),
+                                                 16, 0, 0);
+            }
+        }
+    }
+
+    // ---- the input vector as fp32, zero-padded to whole steps of 32 -----------------------------------
+    const int steps = (K + 31) >> 5;
+    if (prm.pre == 0) {
+        for (int k = tid; k < 32 * steps; k += kStagedThreads) lin_x[k] = k < K ? bf2f(prm.input[k]) : 0.0f;
+    } else {
+        // rmsnorm_kernel (R17:8276-8338) / talker_add_postnorm_fused_kernel (R17:16205-16286): thread t
+        // sums the squares of columns t, t+256, ... with fmaf; block tree; two roundings per element.
+        float local_sum = 0.0f;
+        for (int k = tid; k < K; k += kStagedThreads) {
+            float v = bf2f(prm.input[k]);
+            if (prm.pre == 2) {
+                const uint16_t r = f2bf(v + bf2f(prm.addend[k]));
+                if (blockIdx.x == 0) prm.residual_out[k] = r;
+                v = bf2f(r);
+            }
+            lin_x[k] = v;
+            local_sum = fmaf(v, v, local_sum);
+        }
+        const float total = block_sum_256_like_reference(local_sum, sh_waves, &sh_total);
+        const float inverse_rms = 1.0f / sqrtf(total / static_cast<float>(K) + prm.epsilon);
+        for (int k = tid; k < 32 * steps; k += kStagedThreads) {
+            float y = 0.0f;
+            if (k < K) y = round_bf16(round_bf16(lin_x[k] * inverse_rms) * bf2f(prm.norm_weight[k]));
+            lin_x[k] = y;
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0);      // this wave's global_load_lds writes have landed
+    __syncthreads();
+
+    // ---- 32 chains per output, one thread each: k = l, l+32, ... in increasing k ----------------------
+    const int c = tid >> 5;             // output (channel) within the block
+    const int l = tid & 31;             // reference lane
+    const bool live = c < R && first + c < (DUAL ? prm.rows[0] : prm.rows[0] + prm.rows[1] + prm.rows[2]);
+    const uint16_t* w0 = reinterpret_cast<const uint16_t*>(lds_w + (DUAL ? 2 * c : c) * row_stride) + l;
+    const uint16_t* w1 = reinterpret_cast<const uint16_t*>(lds_w + (2 * c + 1) * row_stride) + l;   // DUAL only
+    const float* xs = lin_x + l;
+    float acc = 0.0f, up = 0.0f;
+    if (live) {
+        const int full = K >> 5;        // steps in which every lane has an element
+        int j = 0;
+        for (; j + 8 <= full; j += 8) {
+            float x[8], a[8], b[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                x[u] = xs[32 * (j + u)];
+                a[u] = bf2f(w0[32 * (j + u)]);
+                if (DUAL) b[u] = bf2f(w1[32 * (j + u)]);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                acc = fmaf(x[u], a[u], acc);
+                if (DUAL) up = fmaf(x[u], b[u], up);
+            }
+        }
+        for (; j < steps; ++j) {
+            if (32 * j + l < K) {
+                acc = fmaf(xs[32 * j], bf2f(w0[32 * j]), acc);
+                if (DUAL) up = fmaf(xs[32 * j], bf2f(w1[32 * j]), up);
+            }
+        }
+    }
+    // the reference's shuffle tree over its 32 lanes; lane 0 holds the sum
+#pragma unroll
+    for (int offset = 16; offset > 0; offset >>= 1) {
+        acc += __shfl_down(acc, offset, 32);
+        if (DUAL) up += __shfl_down(up, offset, 32);
+    }
+    if (l == 0 && live) {
+        int out = first + c;
+        if (DUAL) {
+            const float gv = bf2f(f2bf(acc));
+            const uint16_t act = f2bf(gv / (1.0f + expf(-gv)));
+            prm.output[0][out] = f2bf(bf2f(act) * bf2f(f2bf(up)));
+        } else {
+            int m = 0;
+            if (out >= prm.rows[0]) {
+                out -= prm.rows[0];
+                m = 1;
+                if (out >= prm.rows[1]) {
+                    out -= prm.rows[1];
+                    m = 2;
+                }
+            }
+            float r = acc;
+            if (prm.bias[m]) r += bf2f(prm.bias[m][out]);
+            uint16_t v = f2bf(r);
+            if (prm.residual) v = f2bf(bf2f(prm.residual[out]) + bf2f(v));
+            prm.output[m][out] = v;
+        }
+    }
+}
+
+// Outputs per block of the staged kernel for this reduction length, 0 if even one row does not fit.
+template <bool DUAL>
+inline int staged_rows_per_block(int reduction) {
+    for (int r = kStagedMaxRows; r >= 1; r >>= 1) {
+        const int64_t bytes = static_cast<int64_t>(staged_x_floats(reduction)) * 4
+                            + static_cast<int64_t>(DUAL ? 2 * r : r) * staged_row_stride(reduction);
+        if (bytes <= kStagedLdsBudget) return r;
+    }
+    return 0;
+}
+
+// The staged kernel needs 16-byte pieces: reduction % 8 == 0 and 16-byte aligned weight rows.
+inline bool staged_ok(const LinearParams& prm, bool dual) {
+    if (prm.reduction & 7) return false;
+    const int n = dual ? 2 : 3;
+    for (int i = 0; i < n; ++i)
+        if (reinterpret_cast<uintptr_t>(prm.weight[i]) & 15) return false;
+    return true;
+}
+
+template <bool DUAL>
+inline int32_t launch_staged(LinearParams prm, hipStream_t s) {
+    const int64_t total = DUAL ? prm.rows[0] : static_cast<int64_t>(prm.rows[0]) + prm.rows[1] + prm.rows[2];
+    if (total == 0 && prm.pre != 2) return QM_OK;
+    const int r = staged_rows_per_block<DUAL>(prm.reduction);
+    prm.rows_per_block = r;
+    const size_t smem = static_cast<size_t>(staged_x_floats(prm.reduction)) * 4
+                      + static_cast<size_t>(DUAL ? 2 * r : r) * staged_row_stride(prm.reduction);
+    static bool attr_set = false;
+    if (!attr_set) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(linear_m1_staged_kernel<DUAL>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kStagedLdsBudget);
+        if (e != hipSuccess) return hip_code(e);
+        attr_set = true;
+    }
+    const int64_t blocks = total == 0 ? 1 : (total + r - 1) / r;
+    hipLaunchKernelGGL(linear_m1_staged_kernel<DUAL>, dim3(static_cast<unsigned>(blocks)), dim3(kStagedThreads), smem, s, prm);
     return launch_status();
 }
 
@@ -179,7 +412,9 @@ extern "C" int32_t qm_linear_m1(const uint16_t* input, const uint16_t* weight, c
     prm.reduction = reduction_columns;
     prm.weight[1] = prm.weight[2] = weight;   // never read: rows[1] = rows[2] = 0
     prm.output[1] = prm.output[2] = output;
-    return launch_linear(prm, static_cast<hipStream_t>(hip_stream));
+    if (staged_ok(prm, false) && staged_rows_per_block<false>(prm.reduction) > 0)
+        return launch_staged<false>(prm, static_cast<hipStream_t>(hip_stream));
+    return launch_linear<false>(prm, static_cast<hipStream_t>(hip_stream));
 }
 
 extern "C" int32_t qm_qkv_m1(const uint16_t* input, const uint16_t* q_weight, const uint16_t* q_bias,
@@ -203,5 +438,74 @@ extern "C" int32_t qm_qkv_m1(const uint16_t* input, const uint16_t* q_weight, co
     prm.residual = nullptr;
     prm.rows[0] = q_dim; prm.rows[1] = kv_dim; prm.rows[2] = kv_dim;
     prm.reduction = hidden;
-    return launch_linear(prm, static_cast<hipStream_t>(hip_stream));
+    if (staged_ok(prm, false) && staged_rows_per_block<false>(prm.reduction) > 0)
+        return launch_staged<false>(prm, static_cast<hipStream_t>(hip_stream));
+    return launch_linear<false>(prm, static_cast<hipStream_t>(hip_stream));
+}
+
+extern "C" int32_t qm_gate_up_swiglu_m1(const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight,
+                                        uint16_t* output, int32_t hidden, int32_t intermediate, void* hip_stream) {
+    using namespace qm;
+    if (!input || !gate_weight || !up_weight || !output) return QM_ERR_NULL;
+    if (intermediate < 0) return QM_ERR_ARGUMENT;
+    const int32_t rc = check_reduction(hidden);
+    if (rc != QM_OK) return rc;
+    if ((reinterpret_cast<uintptr_t>(gate_weight) | reinterpret_cast<uintptr_t>(up_weight)) & 3) return QM_ERR_GEOMETRY;
+    LinearParams prm = {};
+    prm.input = input;
+    prm.weight[0] = gate_weight; prm.weight[1] = up_weight; prm.weight[2] = gate_weight;
+    prm.output[0] = prm.output[1] = prm.output[2] = output;
+    prm.rows[0] = intermediate;
+    prm.reduction = hidden;
+    if (staged_ok(prm, true) && staged_rows_per_block<true>(prm.reduction) > 0)
+        return launch_staged<true>(prm, static_cast<hipStream_t>(hip_stream));
+    return launch_linear<true>(prm, static_cast<hipStream_t>(hip_stream));
+}
+
+// ---- fusions of two reference launches each (staged kernel only) -------------------------------------
+extern "C" int32_t qm_rmsnorm_qkv_m1(const uint16_t* hidden_state, const uint16_t* norm_weight, float epsilon,
+                                     const uint16_t* q_weight, const uint16_t* q_bias,
+                                     const uint16_t* k_weight, const uint16_t* k_bias,
+                                     const uint16_t* v_weight, const uint16_t* v_bias,
+                                     uint16_t* q_output, uint16_t* k_output, uint16_t* v_output,
+                                     int32_t hidden, int32_t q_dim, int32_t kv_dim, void* hip_stream) {
+    using namespace qm;
+    if (!hidden_state || !norm_weight || !q_weight || !k_weight || !v_weight || !q_output || !k_output || !v_output)
+        return QM_ERR_NULL;
+    if (q_dim < 0 || kv_dim < 0) return QM_ERR_ARGUMENT;
+    const int32_t rc = check_reduction(hidden);
+    if (rc != QM_OK) return rc;
+    LinearParams prm = {};
+    prm.input = hidden_state;
+    prm.weight[0] = q_weight; prm.weight[1] = k_weight; prm.weight[2] = v_weight;
+    prm.bias[0] = q_bias; prm.bias[1] = k_bias; prm.bias[2] = v_bias;
+    prm.output[0] = q_output; prm.output[1] = k_output; prm.output[2] = v_output;
+    prm.rows[0] = q_dim; prm.rows[1] = kv_dim; prm.rows[2] = kv_dim;
+    prm.reduction = hidden;
+    prm.pre = 1; prm.norm_weight = norm_weight; prm.epsilon = epsilon;
+    if (!staged_ok(prm, false) || staged_rows_per_block<false>(hidden) == 0) return QM_ERR_GEOMETRY;
+    return launch_staged<false>(prm, static_cast<hipStream_t>(hip_stream));
+}
+
+extern "C" int32_t qm_add_postnorm_gate_up_swiglu_m1(const uint16_t* hidden_state, const uint16_t* attention,
+                                                     const uint16_t* norm_weight, float epsilon, uint16_t* residual,
+                                                     const uint16_t* gate_weight, const uint16_t* up_weight,
+                                                     uint16_t* output, int32_t hidden, int32_t intermediate,
+                                                     void* hip_stream) {
+    using namespace qm;
+    if (!hidden_state || !attention || !norm_weight || !residual || !gate_weight || !up_weight || !output)
+        return QM_ERR_NULL;
+    if (intermediate < 0) return QM_ERR_ARGUMENT;
+    const int32_t rc = check_reduction(hidden);
+    if (rc != QM_OK) return rc;
+    LinearParams prm = {};
+    prm.input = hidden_state;
+    prm.weight[0] = gate_weight; prm.weight[1] = up_weight; prm.weight[2] = gate_weight;
+    prm.output[0] = prm.output[1] = prm.output[2] = output;
+    prm.rows[0] = intermediate;
+    prm.reduction = hidden;
+    prm.pre = 2; prm.addend = attention; prm.norm_weight = norm_weight; prm.epsilon = epsilon;
+    prm.residual_out = residual;
+    if (!staged_ok(prm, true) || staged_rows_per_block<true>(hidden) == 0) return QM_ERR_GEOMETRY;
+    return launch_staged<true>(prm, static_cast<hipStream_t>(hip_stream));
 }

@@ -122,3 +122,114 @@ def test_linear_argument_errors(qm, dev):
     assert L.qm_linear_m1(x.data_ptr(), w.data_ptr(), None, None, out.data_ptr(), 0, 64, None) == 0
     assert L.qm_qkv_m1(x.data_ptr(), w.data_ptr(), None, None, None, w.data_ptr(), None, out.data_ptr(),
                        out.data_ptr(), out.data_ptr(), 64, 4, 4, None) == -1
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 2048), (3, 2048), (2, 1024), (5, 130), (1, 16), (2, 6144)])
+def test_rmsnorm_rows_bit_exact(oracle, qm, dev, rows, dim):
+    import torch
+    x = oracle.normal_bf16((rows, dim), 500 + dim)
+    w = oracle.normal_bf16((dim,), 501 + dim, mean=1.0, std=0.1)
+    want = np.zeros_like(x)
+    assert oracle.rmsnorm_rows(x, w, want, rows, dim) == 0
+    out = torch.full((rows, dim), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.rmsnorm_rows(to_dev(x, dev), to_dev(w, dev), out, rows, dim)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_u16(out), want)
+
+
+@pytest.mark.parametrize("dim", [2048, 1024, 130, 6])
+def test_add_postnorm_bit_exact(oracle, qm, dev, dim):
+    import torch
+    h = oracle.normal_bf16((dim,), 600 + dim)
+    a = oracle.normal_bf16((dim,), 601 + dim)
+    w = oracle.normal_bf16((dim,), 602 + dim, mean=1.0, std=0.1)
+    res, nrm = np.zeros(dim, dtype=np.uint16), np.zeros(dim, dtype=np.uint16)
+    assert oracle.add_postnorm_m1(h, a, w, res, nrm, dim) == 0
+    rd = torch.full((dim,), 0x7fc0, dtype=torch.int16, device=dev)
+    nd = torch.full((dim,), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.add_postnorm_m1(to_dev(h, dev), to_dev(a, dev), to_dev(w, dev), rd, nd, dim)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_u16(rd), res) and np.array_equal(to_u16(nd), nrm)
+
+
+@pytest.mark.parametrize("hidden,inter", [(2048, 6144), (2048, 3072), (66, 33), (34, 1)])
+def test_gate_up_swiglu(oracle, qm, dev, hidden, inter):
+    """Bit-identical except where the device's expf and glibc's differ in the last place and the
+    two bf16 roundings behind it do not hide that: at most one bf16 ulp, on well under 0.1 % of outputs."""
+    import torch
+    from qm_testlib import ulp_distance
+    x = oracle.normal_bf16((hidden,), 700 + hidden)
+    gw = oracle.normal_bf16((inter, hidden), 701 + hidden, std=0.03)
+    uw = oracle.normal_bf16((inter, hidden), 702 + hidden, std=0.03)
+    want = np.zeros(inter, dtype=np.uint16)
+    assert oracle.gate_up_swiglu_m1(x, gw, uw, want, hidden, inter, 16) == 0
+    out = torch.full((inter,), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.gate_up_swiglu_m1(to_dev(x, dev), to_dev(gw, dev), to_dev(uw, dev), out, hidden, inter)
+    torch.cuda.synchronize()
+    got = to_u16(out)
+    d = ulp_distance(got, want)
+    assert d.max() <= 1
+    assert np.count_nonzero(d) <= max(1, inter // 1000)
+
+
+@pytest.mark.parametrize("hidden,q_dim,kv_dim", [(2048, 2048, 1024), (512, 40, 24), (1024, 8, 8)])
+def test_fused_rmsnorm_qkv_equals_the_two_operators(oracle, qm, dev, hidden, q_dim, kv_dim):
+    import torch
+    seed = 1100 + hidden
+    x = oracle.normal_bf16((hidden,), seed)
+    nw = oracle.normal_bf16((hidden,), seed + 1, mean=1.0, std=0.1)
+    dims = (q_dim, kv_dim, kv_dim)
+    ws = [oracle.normal_bf16((n, hidden), seed + 2 + i, std=0.02) for i, n in enumerate(dims)]
+    bs = [oracle.normal_bf16((n,), seed + 6 + i, std=0.1) for i, n in enumerate(dims)]
+    normed = np.zeros((1, hidden), dtype=np.uint16)
+    assert oracle.rmsnorm_rows(x.reshape(1, hidden), nw, normed, 1, hidden) == 0
+    want = [np.zeros(n, dtype=np.uint16) for n in dims]
+    assert oracle.qkv_m1(normed[0], ws[0], bs[0], ws[1], bs[1], ws[2], bs[2], want[0], want[1], want[2],
+                         hidden, q_dim, kv_dim, 16) == 0
+    outs = [torch.full((n,), 0x7fc0, dtype=torch.int16, device=dev) for n in dims]
+    wd = [to_dev(w, dev) for w in ws]
+    bd = [to_dev(b, dev) for b in bs]
+    qm.rmsnorm_qkv_m1(to_dev(x, dev), to_dev(nw, dev), wd[0], bd[0], wd[1], bd[1], wd[2], bd[2], outs[0], outs[1],
+                      outs[2], hidden, q_dim, kv_dim)
+    torch.cuda.synchronize()
+    for o, w_ in zip(outs, want):
+        assert np.array_equal(to_u16(o), w_)
+
+
+@pytest.mark.parametrize("hidden,inter", [(2048, 6144), (512, 20), (64, 8)])
+def test_fused_add_postnorm_gate_up_equals_the_two_operators(oracle, qm, dev, hidden, inter):
+    import torch
+    from qm_testlib import ulp_distance
+    seed = 1200 + hidden
+    h = oracle.normal_bf16((hidden,), seed)
+    a = oracle.normal_bf16((hidden,), seed + 1)
+    nw = oracle.normal_bf16((hidden,), seed + 2, mean=1.0, std=0.1)
+    gw = oracle.normal_bf16((inter, hidden), seed + 3, std=0.03)
+    uw = oracle.normal_bf16((inter, hidden), seed + 4, std=0.03)
+    res, nrm = np.zeros(hidden, dtype=np.uint16), np.zeros(hidden, dtype=np.uint16)
+    assert oracle.add_postnorm_m1(h, a, nw, res, nrm, hidden) == 0
+    want = np.zeros(inter, dtype=np.uint16)
+    assert oracle.gate_up_swiglu_m1(nrm, gw, uw, want, hidden, inter, 16) == 0
+    rd = torch.full((hidden,), 0x7fc0, dtype=torch.int16, device=dev)
+    out = torch.full((inter,), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.add_postnorm_gate_up_swiglu_m1(to_dev(h, dev), to_dev(a, dev), to_dev(nw, dev), rd, to_dev(gw, dev),
+                                      to_dev(uw, dev), out, hidden, inter)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_u16(rd), res)
+    d = ulp_distance(to_u16(out), want)
+    assert d.max() <= 1 and np.count_nonzero(d) <= max(1, inter // 1000)
+
+
+def test_fused_entries_reject_what_the_staged_kernel_cannot_take(qm, dev):
+    import torch
+    x = torch.zeros(68, dtype=torch.int16, device=dev)
+    w = torch.zeros((8, 68), dtype=torch.int16, device=dev)
+    o = torch.zeros(8, dtype=torch.int16, device=dev)
+    L = qm.lib()
+    # hidden = 68 is even (fine for qm_qkv_m1) but not a multiple of 8
+    assert L.qm_rmsnorm_qkv_m1(x.data_ptr(), x.data_ptr(), 1e-6, w.data_ptr(), None, w.data_ptr(), None, w.data_ptr(),
+                               None, o.data_ptr(), o.data_ptr(), o.data_ptr(), 68, 8, 8, None) == -2
+    assert L.qm_add_postnorm_gate_up_swiglu_m1(x.data_ptr(), x.data_ptr(), x.data_ptr(), 1e-6, x.data_ptr(),
+                                               w.data_ptr(), w.data_ptr(), o.data_ptr(), 68, 8, None) == -2
+    assert L.qm_rmsnorm_qkv_m1(None, x.data_ptr(), 1e-6, w.data_ptr(), None, w.data_ptr(), None, w.data_ptr(),
+                               None, o.data_ptr(), o.data_ptr(), o.data_ptr(), 64, 8, 8, None) == -1

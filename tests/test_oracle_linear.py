@@ -82,3 +82,69 @@ def test_argument_errors(oracle):
     out = np.zeros(2, dtype=np.uint16)
     assert oracle.linear_m1(None, w, None, None, out, 2, 4) == -1
     assert oracle.linear_m1(x, w, None, None, out, -1, 4) == -5
+
+
+# ---- the other M = 1 pieces of a decode layer ---------------------------------------------------------
+def test_rmsnorm_closed_form_and_rounding_order(oracle):
+    dim = 2048
+    # constant vector c: inverse rms = 1/sqrt(c^2 + eps) exactly (the sum c^2 * dim is exact for c = 2)
+    x = np.full((3, dim), 0x4000, dtype=np.uint16)             # 2.0
+    w = oracle.normal_bf16((dim,), 41, mean=1.0, std=0.1)
+    out = np.zeros_like(x)
+    assert oracle.rmsnorm_rows(x, w, out, 3, dim) == 0
+    inv = np.float32(1.0) / np.sqrt(np.float32(4.0) + np.float32(1e-6), dtype=np.float32)
+    n = oracle.f32_to_bf16(np.array([np.float32(2.0) * inv], dtype=np.float32))[0]            # first rounding
+    want = oracle.f32_to_bf16(oracle.bf16_to_f32(np.full(dim, n, dtype=np.uint16)) * oracle.bf16_to_f32(w))
+    assert np.array_equal(out[0], want) and np.array_equal(out[1], want) and np.array_equal(out[2], want)
+
+
+def test_rmsnorm_random_rows_against_fp64(oracle):
+    rows, dim = 5, 2048
+    x = oracle.normal_bf16((rows, dim), 42)
+    w = oracle.normal_bf16((dim,), 43, mean=1.0, std=0.1)
+    out = np.zeros_like(x)
+    assert oracle.rmsnorm_rows(x, w, out, rows, dim) == 0
+    xf = oracle.bf16_to_f32(x.ravel()).reshape(rows, dim).astype(np.float64)
+    exact = xf / np.sqrt((xf ** 2).mean(axis=1, keepdims=True) + 1e-6) * oracle.bf16_to_f32(w).astype(np.float64)
+    got = oracle.bf16_to_f32(out.ravel()).reshape(rows, dim).astype(np.float64)
+    assert np.all(np.abs(got - exact) <= np.abs(exact) * 2.0 ** -7 + 1e-30)     # two roundings: <= 2 half-ulps
+
+
+def test_add_postnorm_is_rounded_sum_then_rmsnorm(oracle):
+    dim = 2048
+    h = oracle.normal_bf16((dim,), 44)
+    a = oracle.normal_bf16((dim,), 45)
+    w = oracle.normal_bf16((dim,), 46, mean=1.0, std=0.1)
+    res = np.zeros(dim, dtype=np.uint16)
+    nrm = np.zeros(dim, dtype=np.uint16)
+    assert oracle.add_postnorm_m1(h, a, w, res, nrm, dim) == 0
+    assert np.array_equal(res, oracle.f32_to_bf16(oracle.bf16_to_f32(h) + oracle.bf16_to_f32(a)))
+    again = np.zeros((1, dim), dtype=np.uint16)
+    assert oracle.rmsnorm_rows(res.reshape(1, dim), w, again, 1, dim) == 0       # statistic over the rounded residual
+    assert np.array_equal(nrm, again[0])
+
+
+def test_gate_up_swiglu_values(oracle):
+    hidden, inter = 64, 40
+    x = np.zeros(hidden, dtype=np.uint16)
+    x[0] = 0x3f80                                                       # e_0: g = gate[c][0], u = up[c][0]
+    g = oracle.normal_bf16((inter,), 47, std=2.0)
+    u = oracle.normal_bf16((inter,), 48)
+    gw = np.zeros((inter, hidden), dtype=np.uint16)
+    uw = np.zeros((inter, hidden), dtype=np.uint16)
+    gw[:, 0], uw[:, 0] = g, u
+    out = np.zeros(inter, dtype=np.uint16)
+    assert oracle.gate_up_swiglu_m1(x, gw, uw, out, hidden, inter) == 0
+    gf = oracle.bf16_to_f32(g).astype(np.float64)
+    silu = gf / (1.0 + np.exp(-gf))
+    act = oracle.bf16_to_f32(oracle.f32_to_bf16(silu.astype(np.float32))).astype(np.float64)    # bf16(silu)
+    exact = act * oracle.bf16_to_f32(u).astype(np.float64)
+    got = oracle.bf16_to_f32(out).astype(np.float64)
+    assert np.all(np.abs(got - exact) <= np.abs(exact) * 2.0 ** -8 + 1e-30)
+    # g = 0 gives exactly 0 whatever u is; a large negative gate switches the channel off
+    gw[:, 0] = 0
+    assert oracle.gate_up_swiglu_m1(x, gw, uw, out, hidden, inter) == 0
+    assert np.all((out & 0x7fff) == 0)
+    gw[:, 0] = 0xc2c8                                                   # -100
+    assert oracle.gate_up_swiglu_m1(x, gw, uw, out, hidden, inter) == 0
+    assert np.all(np.abs(oracle.bf16_to_f32(out)) < 1e-30)
