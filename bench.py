@@ -156,10 +156,13 @@ class SingleDecode:
     also runs the fused norm + RoPE + append at the last position first."""
     bound = "hbm"
 
-    def __init__(self, qm, dev, ctx, fused_append, seed, copies=1):
+    def __init__(self, qm, dev, ctx, fused_append, seed, copies=1, one_launch=True):
         import torch
         self.qm, self.dev, self.ctx, self.fused = qm, dev, ctx, fused_append
+        self.one_launch = one_launch     # append folded into the attention launch (qm_decode_step_fused)
         self.name = ("talker_fused_step_ctx%d" if fused_append else "gqa_decode_ctx%d") % ctx
+        if fused_append and not one_launch:
+            self.name += "_append_and_decode_launches"
         gd = torch.Generator(device=dev).manual_seed(seed)
         self.max_cache = ctx + 4
         self.copies = copies
@@ -200,6 +203,11 @@ class SingleDecode:
         c = self.caches[self.i % self.copies]
         self.i += 1
         q = self.q
+        if self.fused and self.one_launch:
+            self.qm.decode_step_fused(self.q_lin, self.k_lin, self.v_lin, self.gq, self.gk, self.cos, self.sin, self.q,
+                                      c, None, 1, self.out, 16, self.ctx - 1, -1, SCALE, 1e-6, self.ws, self.ws_bytes,
+                                      None, s)
+            return
         if self.fused:
             self.qm.qk_norm_rope_kv_append(self.q_lin, self.k_lin, self.v_lin, self.gq, self.gk, self.cos, self.sin,
                                            self.q, c, None, 1, 16, self.ctx - 1, 1e-6, s)
@@ -339,10 +347,14 @@ class TalkerLayerStep:
         else:
             qm.rmsnorm_rows(self.x, L["in_norm"], self.norm, 1, H, 1e-6, s)
             qm.qkv_m1(self.norm, L["wq"], None, L["wk"], None, L["wv"], None, self.q, self.k_, self.v_, H, H, 1024, s)
-        qm.qk_norm_rope_kv_append(self.q, self.k_, self.v_, L["gq"], L["gk"], self.cos, self.sin, self.qrot, L["cache"],
-                                  None, 1, 16, self.ctx - 1, 1e-6, s)
-        qm.decode_attention(self.qrot, L["cache"], None, 1, self.ctxv, 16, self.ctx - 1, -1, SCALE, self.ws,
-                            self.ws_bytes, s)
+        if self.fused:
+            qm.decode_step_fused(self.q, self.k_, self.v_, L["gq"], L["gk"], self.cos, self.sin, self.qrot, L["cache"],
+                                 None, 1, self.ctxv, 16, self.ctx - 1, -1, SCALE, 1e-6, self.ws, self.ws_bytes, None, s)
+        else:
+            qm.qk_norm_rope_kv_append(self.q, self.k_, self.v_, L["gq"], L["gk"], self.cos, self.sin, self.qrot,
+                                      L["cache"], None, 1, 16, self.ctx - 1, 1e-6, s)
+            qm.decode_attention(self.qrot, L["cache"], None, 1, self.ctxv, 16, self.ctx - 1, -1, SCALE, self.ws,
+                                self.ws_bytes, s)
         qm.linear_m1(self.ctxv, L["wo"], None, None, self.attn, H, H, s)
         if self.fused:
             qm.add_postnorm_gate_up_swiglu_m1(self.x, self.attn, L["post"], self.res, L["wg"], L["wu"], self.act, H, I,
@@ -559,6 +571,8 @@ def main():
             # the same step over 64 distinct KV caches in rotation (0.54 GB): defeats L2 / MALL
             # residency, as consecutive layers of a real decode step do
             ("cfg2_talker_fused_step_ctx2048_rotating64", lambda: SingleDecode(qm, dev, 2048, True, 12, copies=64)),
+            # the same step as the reference launches it: append kernel, then attention
+            ("cfg2_talker_step_ctx2048_two_operators", lambda: SingleDecode(qm, dev, 2048, True, 12, one_launch=False)),
             ("cfg4_causal_prefill", lambda: Prefill(qm, dev)),
             ("cfg5_predictor_loop", lambda: PredictorLoop(qm, dev)),
             ("cfg5_predictor_loop_cache_writeback", lambda: PredictorLoop(qm, dev, write_cache=True)),

@@ -156,6 +156,28 @@ int32_t qm_decode_attention(
     void* hip_stream);
 
 /*
+ * One decode step of a layer's attention in one call: qm_qk_norm_rope_kv_append at `position`
+ * followed by qm_decode_attention with cache_before = position, i.e. the reference's
+ * launch_qk_norm_rope_cache_m1 + launch_attention pair (R17:17181-17195), with the first folded
+ * into the attention launch (each attention block norms and rotates its own query heads; the
+ * block that owns the new token's tile appends K and V before it reads the tile).
+ * q [q_heads][128], k, v [kv_heads][128] are the raw projections; cos_row, sin_row [128] the RoPE
+ * row of `position`; q_rotated_out [q_heads][128] receives the rotated query (may be NULL).
+ * Results (context, cache contents, q_rotated) are bit-identical to the two separate calls.
+ * Workspace as for qm_decode_attention with max_seq_len = position + 1.
+ */
+int32_t qm_decode_step_fused(
+    const uint16_t* q, const uint16_t* k, const uint16_t* v,
+    const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+    const uint16_t* cos_row, const uint16_t* sin_row,
+    uint16_t* q_rotated_out,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    uint16_t* context_out,
+    int32_t q_heads, int32_t position, int32_t sliding_window, float scale, float epsilon,
+    void* workspace, size_t workspace_bytes, uint32_t* status_dev,
+    void* hip_stream);
+
+/*
  * Ragged multi-stream decode (no reference counterpart; one launch for all streams).
  * query, context_out [n][q_heads][128]; seq_lens [n] device int32 (context length of
  * each stream, 0 = produce zeros); page_table [n][max_pages]; max_seq_len: host upper

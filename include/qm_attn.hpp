@@ -174,6 +174,23 @@ inline void predictor_attention_loop(
           "Predictor attention loop launch");
 }
 
+// launch_qk_norm_rope_cache_m1 + launch_attention of one decode step (R17:17181-17195) in one launch.
+inline void decode_step_m1(
+    const std::uint16_t* q, const std::uint16_t* k, const std::uint16_t* v,
+    const std::uint16_t* q_norm_weight, const std::uint16_t* k_norm_weight,
+    const std::uint16_t* cosine, const std::uint16_t* sine, std::uint16_t* q_rotated,
+    std::uint16_t* key_cache, std::uint16_t* value_cache, std::uint16_t* context,
+    int q_heads, int kv_heads, int head_dim, int max_cache, int cache_position, int sliding_window,
+    float scale, float epsilon, void* workspace, std::size_t workspace_bytes, void* stream) {
+    if (head_dim != 128) throw std::runtime_error("Talker decode step: head_dim must be 128.");
+    if (cache_position < 0 || cache_position >= max_cache) throw std::runtime_error("Talker decode cache overflow.");
+    const qm_kv_cache cache = flat_cache(key_cache, value_cache, kv_heads, head_dim, max_cache);
+    check(qm_decode_step_fused(q, k, v, q_norm_weight, k_norm_weight, cosine, sine, q_rotated, &cache, nullptr, 1,
+                               context, q_heads, cache_position, sliding_window, scale, epsilon, workspace,
+                               workspace_bytes, nullptr, stream),
+          "Talker fused decode step launch");
+}
+
 // launch_linear_m1 (R17:17473-17511), same argument order and label.
 inline void launch_linear_m1(
     const std::uint16_t* input, const std::uint16_t* weight, const std::uint16_t* bias,

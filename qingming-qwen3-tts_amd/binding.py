@@ -53,6 +53,8 @@ _SIGNATURES = {
     "qm_decode_workspace_bytes": (C.c_size_t, [_I32, _I32, _I32, _I32]),
     "qm_decode_attention": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _I32, _F32,
                                    _PTR, C.c_size_t, _PTR]),
+    "qm_decode_step_fused": (_I32, [_PTR] * 8 + [C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _I32, _F32, _F32,
+                                    _PTR, C.c_size_t, _PTR, _PTR]),
     "qm_decode_attention_ragged": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _PTR, _I32,
                                           _F32, _PTR, C.c_size_t, _PTR, _PTR]),
     "qm_norm_rope_rows": (_I32, [_PTR] * 5 + [_I32, _I32, _F32, _PTR]),
@@ -158,6 +160,14 @@ def decode_attention(query, cache, page_table, max_pages, out, q_heads, cache_be
     _check(lib().qm_decode_attention(
         _addr(query), C.byref(cache), _addr(page_table), max_pages, _addr(out), q_heads, cache_before,
         sliding_window, scale, _addr(workspace), workspace_bytes, stream), "qm_decode_attention")
+
+
+def decode_step_fused(q, k, v, gq, gk, cos, sin, q_rot, cache, page_table, max_pages, out, q_heads, position,
+                      sliding_window, scale, eps, workspace, workspace_bytes, status=None, stream=0):
+    _check(lib().qm_decode_step_fused(
+        _addr(q), _addr(k), _addr(v), _addr(gq), _addr(gk), _addr(cos), _addr(sin), _addr(q_rot),
+        C.byref(cache), _addr(page_table), max_pages, _addr(out), q_heads, position, sliding_window, scale, eps,
+        _addr(workspace), workspace_bytes, _addr(status), stream), "qm_decode_step_fused")
 
 
 def decode_attention_ragged(query, cache, page_table, max_pages, seq_lens, n_streams, max_seq_len, out,

@@ -26,6 +26,7 @@
 
 #include "qm_device.h"
 #include "qm_host.h"
+#include "qm_norm_rope_head.h"
 
 #include <stdlib.h>
 
@@ -52,6 +53,18 @@ struct DecodeParams {
     int max_splits;
     int q_heads;
     float scale;
+    // Fused decode step (single stream): the raw projections of the new token; the kernel norms and
+    // rotates q itself and appends k, v at `step_position` before attending.
+    const uint16_t* step_q;       // [q_heads][128]
+    const uint16_t* step_k;       // [kv_heads][128]
+    const uint16_t* step_v;       // [kv_heads][128]
+    const uint16_t* step_q_norm;  // [128]
+    const uint16_t* step_k_norm;  // [128]
+    const uint16_t* step_cos;     // [128]
+    const uint16_t* step_sin;     // [128]
+    uint16_t* step_q_rotated;     // [q_heads][128] or NULL
+    int step_position;
+    float step_epsilon;
 };
 
 // Partial record of one (stream, kv head, split): G*128 acc, G max, G sum.
@@ -64,8 +77,12 @@ __device__ __forceinline__ uint4 load_or_zero(const uint16_t* p, bool valid) {
     return r;
 }
 
-template <int G>
+// STEP: the block first runs the QK-RMSNorm + RoPE of its query heads (and, if it owns the tile of
+// the new token, of the key head, appending K and V to the cache) — the reference's separate
+// launch_qk_norm_rope_cache_m1 (R17:17181) folded into the attention launch.
+template <int G, bool STEP>
 __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodeParams prm, qm_kv_cache cache) {
+    __shared__ __attribute__((aligned(16))) uint16_t sh_qrot[STEP ? G : 1][kDim];
     __shared__ float sh_acc[kRowStreams][G][kDim];
     __shared__ float sh_m[kRowStreams][G];
     __shared__ float sh_l[kRowStreams][G];
@@ -118,11 +135,51 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
 
     // Query chunk of this lane for each head of the group, packed bf16 pairs.
     uint4 qv[G];
+    if (STEP) {
+        // Items: the G query heads; in the block that owns the new token's tile also K and V.
+        // One wave per item, in the arithmetic of the append kernel (bit-identical results).
+        const int position = prm.step_position;
+        const bool owner = tile_lo <= position / kTile && position / kTile <= tile_hi;
+        const int32_t* table = prm.page_table;
+        for (int item = wave; item < G + (owner ? 2 : 0); item += kDecodeWaves) {
+            if (item < G) {
+                const int qh = kvh * G + item;
+                const HeadPair r = norm_rope_head(prm.step_q[qh * kDim + lane], prm.step_q[qh * kDim + lane + 64],
+                                                  prm.step_q_norm, prm.step_cos, prm.step_sin, prm.step_epsilon, lane);
+                sh_qrot[item][lane] = r.lo;
+                sh_qrot[item][lane + 64] = r.hi;
+                if (split == 0 && prm.step_q_rotated) {
+                    prm.step_q_rotated[qh * kDim + lane] = r.lo;
+                    prm.step_q_rotated[qh * kDim + lane + 64] = r.hi;
+                }
+            } else {
+                const int64_t tile_base = tile_offset(cache, prm.pages, table, (position / kTile) * kTile, kvh,
+                                                      lane == 0 ? prm.status : nullptr);
+                if (tile_base >= 0) {
+                    const int64_t dst = tile_base + static_cast<int64_t>(position % kTile) * kDim;
+                    if (item == G) {
+                        const HeadPair r = norm_rope_head(prm.step_k[kvh * kDim + lane], prm.step_k[kvh * kDim + lane + 64],
+                                                          prm.step_k_norm, prm.step_cos, prm.step_sin, prm.step_epsilon, lane);
+                        cache.k_pool[dst + lane] = r.lo;
+                        cache.k_pool[dst + lane + 64] = r.hi;
+                    } else {
+                        // V is appended as it is: no norm, no rotation (R17:15515-15524).
+                        cache.v_pool[dst + lane] = prm.step_v[kvh * kDim + lane];
+                        cache.v_pool[dst + lane + 64] = prm.step_v[kvh * kDim + lane + 64];
+                    }
+                }
+            }
+        }
+        __syncthreads();   // the appended K/V and the rotated q are visible to the whole block
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        const int qh = kvh * G + g;
-        qv[g] = *reinterpret_cast<const uint4*>(
-            prm.query + (static_cast<int64_t>(stream) * prm.q_heads + qh) * kDim + col * 8);
+        for (int g = 0; g < G; ++g) qv[g] = *reinterpret_cast<const uint4*>(&sh_qrot[g][col * 8]);
+    } else {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const int qh = kvh * G + g;
+            qv[g] = *reinterpret_cast<const uint4*>(
+                prm.query + (static_cast<int64_t>(stream) * prm.q_heads + qh) * kDim + col * 8);
+        }
     }
 
     float m[G], l[G], acc[G][8];
@@ -410,8 +467,13 @@ inline size_t decode_workspace_bytes(int n_streams, int q_heads, int kv_heads, i
 template <int G>
 int32_t launch_decode(const DecodeParams& prm, const qm_kv_cache& cache, int n_streams,
                       hipStream_t stream) {
-    hipLaunchKernelGGL(decode_split_kernel<G>, dim3(prm.max_splits, cache.kv_heads, n_streams),
-                       dim3(kDecodeThreads), 0, stream, prm, cache);
+    if (prm.step_q) {
+        hipLaunchKernelGGL((decode_split_kernel<G, true>), dim3(prm.max_splits, cache.kv_heads, n_streams),
+                           dim3(kDecodeThreads), 0, stream, prm, cache);
+    } else {
+        hipLaunchKernelGGL((decode_split_kernel<G, false>), dim3(prm.max_splits, cache.kv_heads, n_streams),
+                           dim3(kDecodeThreads), 0, stream, prm, cache);
+    }
     int32_t rc = launch_status();
     if (rc != QM_OK) return rc;
     if (prm.max_splits > 1) {
@@ -426,8 +488,8 @@ int32_t decode_common(const uint16_t* query, const qm_kv_cache* cache, const int
                       int32_t max_pages, const int32_t* seq_lens, int32_t n_streams,
                       int32_t key_start, int32_t key_end, int32_t max_seq_len, uint16_t* out,
                       int32_t q_heads, float scale, void* workspace, size_t workspace_bytes,
-                      uint32_t* status_dev, void* hip_stream) {
-    if (!query || !out) return QM_ERR_NULL;
+                      uint32_t* status_dev, void* hip_stream, const DecodeParams* step = nullptr) {
+    if ((!query && !step) || !out) return QM_ERR_NULL;
     int32_t rc = check_cache(cache, max_pages);
     if (rc != QM_OK) return rc;
     rc = check_group(q_heads, cache->kv_heads);
@@ -458,6 +520,14 @@ int32_t decode_common(const uint16_t* query, const qm_kv_cache* cache, const int
     prm.max_splits = plan.max_splits;
     prm.q_heads = q_heads;
     prm.scale = scale;
+    prm.step_q = nullptr;
+    if (step) {
+        prm.step_q = step->step_q; prm.step_k = step->step_k; prm.step_v = step->step_v;
+        prm.step_q_norm = step->step_q_norm; prm.step_k_norm = step->step_k_norm;
+        prm.step_cos = step->step_cos; prm.step_sin = step->step_sin;
+        prm.step_q_rotated = step->step_q_rotated;
+        prm.step_position = step->step_position; prm.step_epsilon = step->step_epsilon;
+    }
 
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     switch (q_heads / cache->kv_heads) {
@@ -507,4 +577,32 @@ extern "C" int32_t qm_decode_attention_ragged(
     return qm::decode_common(query, cache, page_table, max_pages, seq_lens, n_streams, 0, 0,
                              max_seq_len, context_out, q_heads, scale, workspace, workspace_bytes,
                              status_dev, hip_stream);
+}
+
+extern "C" int32_t qm_decode_step_fused(
+    const uint16_t* q, const uint16_t* k, const uint16_t* v,
+    const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+    const uint16_t* cos_row, const uint16_t* sin_row,
+    uint16_t* q_rotated_out,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    uint16_t* context_out,
+    int32_t q_heads, int32_t position, int32_t sliding_window, float scale, float epsilon,
+    void* workspace, size_t workspace_bytes, uint32_t* status_dev, void* hip_stream) {
+    if (!q || !k || !v || !q_norm_w || !k_norm_w || !cos_row || !sin_row) return QM_ERR_NULL;
+    if (position < 0) return QM_ERR_SLOT_RANGE;
+    const int32_t key_end = position + 1;
+    const int32_t window_start = key_end - sliding_window;
+    const int32_t key_start = sliding_window > 0 ? (window_start > 0 ? window_start : 0) : 0;
+    if (cache && max_pages > 0 && cache->page_size > 0) {
+        if (position / cache->page_size >= max_pages) return QM_ERR_SLOT_RANGE;
+        if (!page_table && position / cache->page_size >= cache->n_pages) return QM_ERR_SLOT_RANGE;
+    }
+    qm::DecodeParams step = {};
+    step.step_q = q; step.step_k = k; step.step_v = v;
+    step.step_q_norm = q_norm_w; step.step_k_norm = k_norm_w;
+    step.step_cos = cos_row; step.step_sin = sin_row;
+    step.step_q_rotated = q_rotated_out;
+    step.step_position = position; step.step_epsilon = epsilon;
+    return qm::decode_common(nullptr, cache, page_table, max_pages, nullptr, 1, key_start, key_end, key_end,
+                             context_out, q_heads, scale, workspace, workspace_bytes, status_dev, hip_stream, &step);
 }

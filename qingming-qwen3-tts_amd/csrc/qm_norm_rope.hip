@@ -11,56 +11,9 @@
 
 #include "qm_device.h"
 #include "qm_host.h"
+#include "qm_norm_rope_head.h"
 
 namespace qm {
-
-// Sum of squares of the 128 values held as (x0 = dim lane, x1 = dim lane + 64).
-// Groups of 32 dims are reduced by value += shfl_down(value, offset) trees; the four
-// group sums w0..w3 are combined as (w0 + w2) + (w1 + w3), which is what the
-// reference's second-level tree over wave sums evaluates to.
-__device__ __forceinline__ float head_sum_squares(float x0, float x1) {
-    float s0 = x0 * x0;
-    float s1 = x1 * x1;
-#pragma unroll
-    for (int offset = 16; offset > 0; offset >>= 1) {
-        s0 += __shfl_down(s0, offset, 32);
-        s1 += __shfl_down(s1, offset, 32);
-    }
-    const float t = s0 + s1;            // lane 0: w0 + w2, lane 32: w1 + w3
-    return __shfl(t, 0) + __shfl(t, 32);
-}
-
-struct HeadPair {
-    uint16_t lo;  // dimension lane
-    uint16_t hi;  // dimension lane + 64
-};
-
-// RMSNorm (optional) + RoPE of one head; returns the two output bit patterns.
-__device__ __forceinline__ HeadPair norm_rope_head(uint16_t x0b, uint16_t x1b,
-                                                   const uint16_t* __restrict__ gamma,
-                                                   const uint16_t* __restrict__ cosv,
-                                                   const uint16_t* __restrict__ sinv,
-                                                   float epsilon, int lane) {
-    float w0 = bf2f(x0b);
-    float w1 = bf2f(x1b);
-    if (gamma) {
-        const float sum = head_sum_squares(w0, w1);
-        const float r = 1.0f / sqrtf(sum / 128.0f + epsilon);
-        const float n0 = bf2f(f2bf(w0 * r));
-        const float n1 = bf2f(f2bf(w1 * r));
-        w0 = bf2f(f2bf(n0 * bf2f(gamma[lane])));
-        w1 = bf2f(f2bf(n1 * bf2f(gamma[lane + 64])));
-    }
-    // rotate_half(x) = (-x2, +x1): dimension d < 64 pairs with -x[d+64], d >= 64 with +x[d-64].
-    const float first0 = bf2f(f2bf(w0 * bf2f(cosv[lane])));
-    const float second0 = bf2f(f2bf((-w1) * bf2f(sinv[lane])));
-    const float first1 = bf2f(f2bf(w1 * bf2f(cosv[lane + 64])));
-    const float second1 = bf2f(f2bf(w0 * bf2f(sinv[lane + 64])));
-    HeadPair out;
-    out.lo = f2bf(first0 + second0);
-    out.hi = f2bf(first1 + second1);
-    return out;
-}
 
 // grid (q_heads + kv_heads, n_streams), block 64.
 __global__ __launch_bounds__(64) void qk_norm_rope_append_kernel(

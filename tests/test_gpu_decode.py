@@ -177,3 +177,67 @@ def test_decode_argument_errors(oracle, qm, dev):
     with pytest.raises(qm.QmError) as e:
         qm.decode_attention(q, qm.flat_cache(big, big, 8, 8192), None, 1, out, 16, 8191, -1, SCALE, None, 0)
     assert e.value.code == -4
+
+
+@pytest.mark.parametrize("ctx,paged,window", [(1, False, -1), (16, False, -1), (17, True, -1), (512, False, -1),
+                                              (2048, False, -1), (2048, True, -1), (777, True, 100), (4097, True, -1)])
+def test_fused_decode_step_equals_append_then_decode(oracle, qm, dev, ctx, paged, window):
+    """qm_decode_step_fused at position ctx-1 == qm_qk_norm_rope_kv_append + qm_decode_attention:
+    context, rotated query and cache contents bit for bit (same arithmetic, one launch less)."""
+    import torch
+    pos = ctx - 1
+    q = oracle.normal_bf16((16, 128), 3000 + ctx)
+    k = oracle.normal_bf16((8, 128), 3001 + ctx)
+    v = oracle.normal_bf16((8, 128), 3002 + ctx)
+    gq = oracle.normal_bf16((128,), 3003, mean=1.0, std=0.1)
+    gk = oracle.normal_bf16((128,), 3004, mean=1.0, std=0.1)
+    cos, sin = oracle.rope_table(1, pos)
+
+    def make():
+        if paged:
+            pool = PagedPool(oracle, [ctx], seed=3100 + ctx)
+            kd, vd, cache, table = pool.device(qm, dev)
+            return kd, vd, cache, table, pool.max_pages
+        kd = to_dev(oracle.normal_bf16((8, ctx + 3, 128), 3200 + ctx), dev)
+        vd = to_dev(oracle.normal_bf16((8, ctx + 3, 128), 3201 + ctx), dev)
+        return kd, vd, qm.flat_cache(kd, vd, 8, ctx + 3), None, 1
+
+    ws_bytes = qm.decode_workspace_bytes(1, 16, 8, ctx)
+    ws = torch.zeros(ws_bytes // 4 + 1, dtype=torch.float32, device=dev)
+    dq, dk, dv = to_dev(q, dev), to_dev(k, dev), to_dev(v, dev)
+    dgq, dgk, dcos, dsin = to_dev(gq, dev), to_dev(gk, dev), to_dev(cos, dev), to_dev(sin, dev)
+    # two launches
+    kd1, vd1, cache1, table1, mp = make()
+    qrot1 = torch.zeros((16, 128), dtype=torch.int16, device=dev)
+    out1 = torch.zeros((16, 128), dtype=torch.int16, device=dev)
+    qm.qk_norm_rope_kv_append(dq, dk, dv, dgq, dgk, dcos, dsin, qrot1, cache1, table1, mp, 16, pos, 1e-6)
+    qm.decode_attention(qrot1, cache1, table1, mp, out1, 16, pos, window, SCALE, ws, ws_bytes)
+    # one launch
+    kd2, vd2, cache2, table2, _ = make()
+    qrot2 = torch.full((16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    out2 = torch.full((16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    qm.decode_step_fused(dq, dk, dv, dgq, dgk, dcos, dsin, qrot2, cache2, table2, mp, out2, 16, pos, window, SCALE,
+                         1e-6, ws, ws_bytes, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    assert np.array_equal(to_u16(qrot2), to_u16(qrot1))
+    assert np.array_equal(to_u16(kd2), to_u16(kd1)) and np.array_equal(to_u16(vd2), to_u16(vd1))
+    assert np.array_equal(to_u16(out2), to_u16(out1))
+
+
+def test_fused_decode_step_argument_errors(qm, dev):
+    import torch
+    z = torch.zeros((16, 128), dtype=torch.int16, device=dev)
+    kv = torch.zeros((8, 32, 128), dtype=torch.int16, device=dev)
+    cache = qm.flat_cache(kv, kv.clone(), 8, 32)
+    L = qm.lib()
+    import ctypes as C
+    args = lambda pos, q=z.data_ptr(): (q, z.data_ptr(), z.data_ptr(), z.data_ptr(), z.data_ptr(), z.data_ptr(),
+                                        z.data_ptr(), None, C.byref(cache), None, 1, z.data_ptr(), 16, pos, -1,
+                                        SCALE, 1e-6, None, 0, None, None)
+    assert L.qm_decode_step_fused(*args(32)) == -3          # beyond the cache
+    assert L.qm_decode_step_fused(*args(-1)) == -3
+    assert L.qm_decode_step_fused(*args(3, None)) == -1
+    assert L.qm_decode_step_fused(*args(31)) == 0
+    torch.cuda.synchronize()
