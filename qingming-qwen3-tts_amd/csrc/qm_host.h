@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/qm_attn.h"
 
 namespace qm {
@@ -41,6 +43,20 @@ inline int32_t check_group(int32_t q_heads, int32_t kv_heads) {
 
 // Process-wide tuning options (qm_set_option); defined with the library's other global entry points.
 int32_t option_value(int32_t option);
+
+// Raises a kernel's dynamic LDS limit once per (kernel, device); safe to call from several host
+// threads and for several devices of one process.  `done` is the caller's static table.
+constexpr int kMaxDevices = 64;
+inline int32_t ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<bool> (&done)[kMaxDevices]) {
+    int dev = 0;
+    const hipError_t e0 = hipGetDevice(&dev);
+    if (e0 != hipSuccess) return hip_code(e0);
+    if (dev >= 0 && dev < kMaxDevices && done[dev].load(std::memory_order_acquire)) return QM_OK;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return hip_code(e);
+    if (dev >= 0 && dev < kMaxDevices) done[dev].store(true, std::memory_order_release);
+    return QM_OK;
+}
 
 inline int32_t launch_status() { return hip_code(hipGetLastError()); }
 

@@ -176,14 +176,10 @@ inline int32_t launch_linear(const LinearParams& prm, hipStream_t s) {
     const int64_t total = DUAL ? prm.rows[0] : static_cast<int64_t>(prm.rows[0]) + prm.rows[1] + prm.rows[2];
     if (total == 0) return QM_OK;
     const size_t smem = static_cast<size_t>((prm.reduction + 31) / 32 * 32) * sizeof(float);
-    static bool attr_set = false;
-    if (!attr_set) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(linear_m1_kernel<DUAL>),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                 kLinMaxReduction * static_cast<int>(sizeof(float)));
-        if (e != hipSuccess) return hip_code(e);
-        attr_set = true;
-    }
+    static std::atomic<bool> lds_raised[kMaxDevices];
+    const int32_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(linear_m1_kernel<DUAL>),
+                                          kLinMaxReduction * static_cast<int>(sizeof(float)), lds_raised);
+    if (rc != QM_OK) return rc;
     const unsigned blocks = static_cast<unsigned>((total + kLinRowsPerBlock - 1) / kLinRowsPerBlock);
     hipLaunchKernelGGL(linear_m1_kernel<DUAL>, dim3(blocks), dim3(kLinThreads), smem, s, prm);
     return launch_status();
@@ -376,13 +372,10 @@ inline int32_t launch_staged(LinearParams prm, hipStream_t s) {
     prm.rows_per_block = r;
     const size_t smem = static_cast<size_t>(staged_x_floats(prm.reduction)) * 4
                       + static_cast<size_t>(DUAL ? 2 * r : r) * staged_row_stride(prm.reduction);
-    static bool attr_set = false;
-    if (!attr_set) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(linear_m1_staged_kernel<DUAL>),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kStagedLdsBudget);
-        if (e != hipSuccess) return hip_code(e);
-        attr_set = true;
-    }
+    static std::atomic<bool> lds_raised[kMaxDevices];
+    const int32_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(linear_m1_staged_kernel<DUAL>), kStagedLdsBudget,
+                                          lds_raised);
+    if (rc != QM_OK) return rc;
     const int64_t blocks = total == 0 ? 1 : (total + r - 1) / r;
     hipLaunchKernelGGL(linear_m1_staged_kernel<DUAL>, dim3(static_cast<unsigned>(blocks)), dim3(kStagedThreads), smem, s, prm);
     return launch_status();

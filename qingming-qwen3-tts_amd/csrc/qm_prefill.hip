@@ -542,13 +542,10 @@ extern "C" int32_t qm_prefill_attention_causal(
     const bool round_scores = option_value(QM_OPT_PREFILL_SCORE_ROUNDING) != 0;
     if (!round_scores && !(scale > 0.0f)) return QM_ERR_ARGUMENT;   // the scale is folded into the exponent there
     const auto kernel = round_scores ? prefill_causal_kernel<true> : prefill_causal_kernel<false>;
-    static bool attr_set[2] = {false, false};
-    if (!attr_set[round_scores]) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-        if (e != hipSuccess) return hip_code(e);
-        attr_set[round_scores] = true;
-    }
+    static std::atomic<bool> lds_raised[2][kMaxDevices];
+    const int32_t rc_lds = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), static_cast<int>(smem),
+                                              lds_raised[round_scores ? 1 : 0]);
+    if (rc_lds != QM_OK) return rc_lds;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(pairs * n_qtiles)), dim3(kPfThreads), smem, s, prm, desc);
     return launch_status();
 }
