@@ -264,6 +264,19 @@ int32_t qm_predictor_attention_loop(
     float epsilon,
     void* hip_stream);
 
+/*
+ * The predictor's staged attention of step 0: replaces PersistentPredictor::attention and its
+ * six kernels (R17:13300-13386, 9369-9745) — bf16(QK), bf16(*scale), the -inf causal mask
+ * (key > row, R17:9517-9520), softmax rows, bf16(P), P.V and the transpose to [rows][16][128] —
+ * in one launch with the same rounding chain and summation order.
+ * query_bhsd [16][rows][128] (already rotated); key_cache, value_cache [8][16][128];
+ * output [rows][16][128]; rows, key_length in 1..16; causal_prefill as in the reference.
+ */
+int32_t qm_predictor_attention_staged(
+    const uint16_t* query_bhsd, const uint16_t* key_cache, const uint16_t* value_cache,
+    uint16_t* output, int32_t rows, int32_t key_length, int32_t causal_prefill,
+    void* hip_stream);
+
 /* --- (5) M = 1 weight-streaming linears around the path ----------------------------------- */
 /*
  * qm_linear_m1 replaces launch_linear_m1 / talker_linear_fused_kernel (R17:17473-17511,

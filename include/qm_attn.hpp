@@ -174,6 +174,32 @@ inline void predictor_attention_loop(
           "Predictor attention loop launch");
 }
 
+// PersistentPredictor::attention (R17:13300-13386): the staged attention of step 0.
+inline void predictor_attention(
+    const std::uint16_t* query, const std::uint16_t* key_cache, const std::uint16_t* value_cache,
+    std::uint16_t* output, int rows, int key_length, bool causal_prefill, void* stream) {
+    check(qm_predictor_attention_staged(query, key_cache, value_cache, output, rows, key_length,
+                                        causal_prefill ? 1 : 0, stream),
+          "Predictor attention launch");
+}
+
+// PersistentPredictor::rope (R17:13238-13254): RoPE of rows x heads head vectors, no norm.
+inline void predictor_rope(
+    const std::uint16_t* input, const std::uint16_t* cosine, const std::uint16_t* sine, std::uint16_t* output,
+    int rows, int heads, void* stream) {
+    check(qm_norm_rope_rows(input, nullptr, cosine, sine, output, rows, heads, 0.0f, stream), "Predictor rope launch");
+}
+
+// PersistentPredictor::update_cache (R17:13256-13270) for the key and the value cache of a layer
+// ([8][16][128] each): rows of [rows][8][128] go to positions start..start+rows-1.
+inline void predictor_update_cache(
+    const std::uint16_t* key_source, const std::uint16_t* value_source,
+    std::uint16_t* key_cache, std::uint16_t* value_cache, int rows, int start, void* stream) {
+    const qm_kv_cache cache = flat_cache(key_cache, value_cache, 8, 128, 16);
+    check(qm_scatter_kv(key_source, value_source, &cache, nullptr, 1, rows, start, stream),
+          "Predictor update_cache launch");
+}
+
 // launch_qk_norm_rope_cache_m1 + launch_attention of one decode step (R17:17181-17195) in one launch.
 inline void decode_step_m1(
     const std::uint16_t* q, const std::uint16_t* k, const std::uint16_t* v,

@@ -62,6 +62,7 @@ _SIGNATURES = {
     "qm_prefill_attention_causal": (_I32, [_PTR] * 4 + [C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _I32, _I32,
                                            _F32, C.c_int64, C.c_int64, C.c_int64, _PTR, _PTR]),
     "qm_predictor_attention_loop": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _I32, _F32, _PTR]),
+    "qm_predictor_attention_staged": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _PTR]),
     "qm_linear_m1": (_I32, [_PTR] * 5 + [_I32, _I32, _PTR]),
     "qm_qkv_m1": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _PTR]),
     "qm_gate_up_swiglu_m1": (_I32, [_PTR] * 4 + [_I32, _I32, _PTR]),
@@ -243,3 +244,8 @@ def add_postnorm_gate_up_swiglu_m1(hidden_state, attention, norm_weight, residua
     _check(lib().qm_add_postnorm_gate_up_swiglu_m1(_addr(hidden_state), _addr(attention), _addr(norm_weight), eps,
                                                    _addr(residual), _addr(gate_w), _addr(up_w), _addr(out), hidden,
                                                    intermediate, stream), "qm_add_postnorm_gate_up_swiglu_m1")
+
+
+def predictor_attention_staged(query_bhsd, key_cache, value_cache, out, rows, key_length, causal, stream=0):
+    _check(lib().qm_predictor_attention_staged(_addr(query_bhsd), _addr(key_cache), _addr(value_cache), _addr(out),
+                                               rows, key_length, int(causal), stream), "qm_predictor_attention_staged")

@@ -38,6 +38,11 @@ struct PredictorParams {
     int n_layers;
     int rows;
     float epsilon;
+    // STAGED mode (the reference's six-kernel attention, R17:13300-13386): q is already rotated and
+    // laid out [16][rows][128]; k, v point at the [8][16][128] caches; row r sees the keys
+    // j < key_length with (causal ? j <= r : true).
+    int key_length;
+    int causal;
 };
 
 // bf16 round trip with the hardware converter (round to nearest even; same bits as the integer
@@ -75,6 +80,13 @@ __device__ __forceinline__ void pv_rows(const float (*p)[kPredRows], const float
     }
 }
 
+// The same sum for a runtime number of keys: the full 16-leaf tree whose leaves at and beyond
+// `limit` are +0 (never read from V, whose cache slots there may hold anything).
+__device__ __forceinline__ float pv_limited(const float* pr, const float* vcol, int limit) {
+    return TreeSum<kPredRows, 0, 8>::eval([&](int j) { return j < limit ? fmaf(pr[j], vcol[j], 0.0f) : 0.0f; });
+}
+
+template <bool STAGED>
 __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorParams prm) {
     __shared__ __attribute__((aligned(16))) uint16_t sh_q[2][kPredRows][kDim];   // [g][row][d]
     __shared__ __attribute__((aligned(16))) uint16_t sh_k[kPredRows][kDim];
@@ -95,6 +107,31 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
     const int rows = prm.rows;
     const int layer = static_cast<int>((prm.unit_base + unit) % prm.n_layers);
 
+    // keys row r attends: a prefix of the cache
+    auto limit_of = [&](int r) { return STAGED ? (prm.causal ? min(r + 1, prm.key_length) : prm.key_length) : r + 1; };
+    if (STAGED) {
+        // ---- q [16][rows][128] of this head pair, K and V rows 0..key_length-1 of the cache ------------
+        for (int c = tid; c < rows * 32; c += kPredThreads) {
+            const int chunk = c & 15, g = (c >> 4) & 1, row = c >> 5;
+            *reinterpret_cast<uint4*>(&sh_q[g][row][chunk * 8]) = *reinterpret_cast<const uint4*>(
+                prm.q + ((static_cast<int64_t>(kvh * 2 + g) * rows + row) * kDim) + chunk * 8);
+        }
+        for (int c = tid; c < kPredRows * 32; c += kPredThreads) {
+            const int chunk = c & 15, is_v = (c >> 4) & 1, row = c >> 5;
+            uint4 val = make_uint4(0, 0, 0, 0);
+            if (row < prm.key_length)
+                val = *reinterpret_cast<const uint4*>((is_v ? prm.v : prm.k) + (static_cast<int64_t>(kvh) * kPredRows + row) * kDim + chunk * 8);
+            *reinterpret_cast<uint4*>(is_v ? &sh_v[row][chunk * 8] : &sh_k[row][chunk * 8]) = val;
+        }
+        __syncthreads();
+        for (int c = tid; c < kPredRows * 32; c += kPredThreads) {
+            const int row = c >> 5, d0 = (c & 31) * 4;
+            const uint2 kk = *reinterpret_cast<const uint2*>(&sh_k[row][d0]);
+            *reinterpret_cast<float4*>(&sh_kf[row][d0]) = make_float4(lo_bf16(kk.x), hi_bf16(kk.x), lo_bf16(kk.y), hi_bf16(kk.y));
+        }
+        __syncthreads();
+    }
+    if (!STAGED) {
     // ---- stage q (2 heads), k, v of this kv head, the RoPE rows and the two gammas: 16-byte chunks ---
     for (int c = tid; c < rows * 64; c += kPredThreads) {
         const int chunk = c & 15;
@@ -216,8 +253,10 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
     }
     __syncthreads();
 
+    }   // !STAGED
+
     // ---- optional K/V cache write-back, layout [unit][kv head][16][128] (R17:10711-10737) ---------
-    if (prm.k_cache_out) {
+    if (!STAGED && prm.k_cache_out) {
         for (int c = tid; c < kPredRows * 16; c += kPredThreads) {
             const int row = c >> 4, chunk = c & 15;
             const int64_t dst = ((unit * 8 + kvh) * kPredRows + row) * kDim + chunk * 8;
@@ -270,7 +309,7 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
 #pragma unroll
             for (int j = 0; j < kPredRows; ++j) {
                 float acc = 0.0f;
-                if (j <= row) {
+                if (j < limit_of(row)) {
                     asm volatile("" ::: "memory");   // keeps the branch: the compiler would compute and discard
 #pragma unroll
                     for (int c = 0; c < 4; ++c) acc = fmaf(q4[c], kf[j][c], acc);
@@ -327,6 +366,7 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
     if (tid < 2 * rows) {
         const int g = tid / rows;
         const int r = tid % rows;
+        const int limit = limit_of(r);
         float sc[kPredRows];
 #pragma unroll
         for (int t = 0; t < kPredRows; t += 4) {
@@ -338,21 +378,21 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
         float maximum = -INFINITY;
 #pragma unroll
         for (int t = 0; t < kPredRows; ++t) {
-            const float cand = t <= r ? sc[t] : -INFINITY;
+            const float cand = t < limit ? sc[t] : -INFINITY;
             maximum = maximum > cand ? maximum : cand;
         }
         float e[kPredRows];
 #pragma unroll
-        for (int t = 0; t < kPredRows; ++t) e[t] = t <= r ? expf(sc[t] - maximum) : 0.0f;
+        for (int t = 0; t < kPredRows; ++t) e[t] = t < limit ? expf(sc[t] - maximum) : 0.0f;
         // exp() >= +0 and masked entries are +0: the full 16-leaf tree equals the reference's sum
         const float total = TreeSum<16, 0, 8>::eval([&](int t) { return e[t]; });
 #pragma unroll
         for (int t = 0; t < kPredRows; t += 4) {
             float4 p4;
-            p4.x = t <= r ? rbf(e[t] / total) : 0.0f;
-            p4.y = t + 1 <= r ? rbf(e[t + 1] / total) : 0.0f;
-            p4.z = t + 2 <= r ? rbf(e[t + 2] / total) : 0.0f;
-            p4.w = t + 3 <= r ? rbf(e[t + 3] / total) : 0.0f;
+            p4.x = t < limit ? rbf(e[t] / total) : 0.0f;
+            p4.y = t + 1 < limit ? rbf(e[t + 1] / total) : 0.0f;
+            p4.z = t + 2 < limit ? rbf(e[t + 2] / total) : 0.0f;
+            p4.w = t + 3 < limit ? rbf(e[t + 3] / total) : 0.0f;
             *reinterpret_cast<float4*>(&sh_s[g][r][t]) = p4;
         }
     }
@@ -366,7 +406,12 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
 #pragma unroll
         for (int j = 0; j < kPredRows; ++j) vcol[j] = bf2f(sh_v[j][d]);
         uint16_t* out = prm.out + ((unit * rows) * 16 + kvh * 2 + g) * kDim + d;
-        pv_rows<0>(sh_s[g], vcol, out, 16 * kDim, rows);
+        if (STAGED) {
+            for (int r = 0; r < rows; ++r)
+                out[r * 16 * kDim] = __builtin_bit_cast(uint16_t, static_cast<__bf16>(pv_limited(sh_s[g][r], vcol, limit_of(r))));
+        } else {
+            pv_rows<0>(sh_s[g], vcol, out, 16 * kDim, rows);
+        }
     }
 }
 
@@ -398,6 +443,7 @@ extern "C" int32_t qm_predictor_attention_loop(
     prm.cos_rows = cos_rows; prm.sin_rows = sin_rows;
     prm.out = context_out; prm.k_cache_out = k_cache_out; prm.v_cache_out = v_cache_out;
     prm.unit_base = 0; prm.n_layers = n_layers; prm.rows = rows; prm.epsilon = epsilon;
+    prm.key_length = 0; prm.causal = 1;
     // grid.y is limited to 65535: fold large unit counts into several launches.
     const int32_t per_launch = 65535;
     for (int32_t first = 0; first < units; first += per_launch) {
@@ -411,10 +457,28 @@ extern "C" int32_t qm_predictor_attention_loop(
         if (k_cache_out) p.k_cache_out = k_cache_out + static_cast<int64_t>(first) * 8 * 16 * qm::kDim;
         if (v_cache_out) p.v_cache_out = v_cache_out + static_cast<int64_t>(first) * 8 * 16 * qm::kDim;
         p.unit_base = first;
-        hipLaunchKernelGGL(qm::predictor_loop_kernel, dim3(8, n), dim3(qm::kPredThreads), 0,
+        hipLaunchKernelGGL(qm::predictor_loop_kernel<false>, dim3(8, n), dim3(qm::kPredThreads), 0,
                            static_cast<hipStream_t>(hip_stream), p);
         const int32_t rc = qm::launch_status();
         if (rc != QM_OK) return rc;
     }
     return QM_OK;
+}
+
+extern "C" int32_t qm_predictor_attention_staged(const uint16_t* query_bhsd, const uint16_t* key_cache,
+                                                 const uint16_t* value_cache, uint16_t* output, int32_t rows,
+                                                 int32_t key_length, int32_t causal_prefill, void* hip_stream) {
+    if (!query_bhsd || !key_cache || !value_cache || !output) return QM_ERR_NULL;
+    if (rows < 1 || rows > qm::kPredRows || key_length < 1 || key_length > qm::kPredRows) return QM_ERR_ARGUMENT;
+    const uintptr_t align = reinterpret_cast<uintptr_t>(query_bhsd) | reinterpret_cast<uintptr_t>(key_cache)
+                          | reinterpret_cast<uintptr_t>(value_cache);
+    if (align & 15) return QM_ERR_GEOMETRY;
+    qm::PredictorParams prm = {};
+    prm.q = query_bhsd; prm.k = key_cache; prm.v = value_cache;
+    prm.out = output;
+    prm.unit_base = 0; prm.n_layers = 1; prm.rows = rows; prm.epsilon = 0.0f;
+    prm.key_length = key_length; prm.causal = causal_prefill ? 1 : 0;
+    hipLaunchKernelGGL(qm::predictor_loop_kernel<true>, dim3(8, 1), dim3(qm::kPredThreads), 0,
+                       static_cast<hipStream_t>(hip_stream), prm);
+    return qm::launch_status();
 }

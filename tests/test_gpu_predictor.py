@@ -72,3 +72,37 @@ def test_predictor_without_cache_and_errors(oracle, qm, dev):
     with pytest.raises(qm.QmError) as e:
         qm.predictor_attention_loop(None, z, z, w, w, r, r, z, None, None, 1, 1, 16, 1)
     assert e.value.code == -1
+
+
+@pytest.mark.parametrize("rows,key_length,causal", [(2, 2, True), (1, 1, True), (1, 9, False), (1, 16, False),
+                                                    (16, 16, True), (5, 5, True), (3, 7, False)])
+def test_predictor_staged_attention(oracle, qm, dev, rows, key_length, causal):
+    """The reference's six-kernel attention of step 0 (R17:13300-13386) in one launch: every output
+    bit equals the oracle's except where the device's expf differs in the last place (<= 1 bf16 ulp)."""
+    import torch
+    from qm_testlib import to_dev, to_u16, ulp_distance
+    seed = 8000 + 17 * rows + key_length
+    q = oracle.normal_bf16((16, rows, 128), seed)
+    kc = oracle.normal_bf16((8, 16, 128), seed + 1)
+    vc = oracle.normal_bf16((8, 16, 128), seed + 2)
+    kc[:, key_length:] = 0x7fc0          # cache slots beyond key_length hold NaN: never read into the result
+    vc[:, key_length:] = 0x7fc0
+    want = np.zeros((rows, 16, 128), dtype=np.uint16)
+    assert oracle.predictor_attention_staged(q, kc, vc, want, rows, key_length, causal) == 0
+    out = torch.full((rows, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.predictor_attention_staged(to_dev(q, dev), to_dev(kc, dev), to_dev(vc, dev), out, rows, key_length, causal)
+    torch.cuda.synchronize()
+    got = to_u16(out)
+    d = ulp_distance(got, want)
+    assert d.max() <= 1
+    assert np.count_nonzero(d) <= max(1, got.size // 500)
+
+
+def test_predictor_staged_attention_argument_errors(qm, dev):
+    import torch
+    z = torch.zeros((16, 2, 128), dtype=torch.int16, device=dev)
+    c = torch.zeros((8, 16, 128), dtype=torch.int16, device=dev)
+    L = qm.lib()
+    assert L.qm_predictor_attention_staged(z.data_ptr(), c.data_ptr(), c.data_ptr(), z.data_ptr(), 2, 17, 1, None) == -5
+    assert L.qm_predictor_attention_staged(z.data_ptr(), c.data_ptr(), c.data_ptr(), z.data_ptr(), 0, 2, 1, None) == -5
+    assert L.qm_predictor_attention_staged(None, c.data_ptr(), c.data_ptr(), z.data_ptr(), 2, 2, 1, None) == -1
