@@ -82,11 +82,16 @@ const char* qm_target_arch(void);
  *       scores to bf16 like the reference (R17:15879-15890); 0: scores stay fp32 (faster; needs
  *       scale > 0; outputs stay within the 1e-2 tolerance of the fp32 definition).
  *   QM_OPT_DECODE_TILES_PER_BLOCK  0 (default): the split-K decode picks the 16-token tiles per
- *       block from the problem size; > 0 forces it (changes qm_decode_workspace_bytes too). */
+ *       block from the problem size; > 0 forces it (changes qm_decode_workspace_bytes too).
+ *   QM_OPT_PREFILL_KERNEL  0 (default): qm_prefill_attention_causal picks one of its two kernels
+ *       from the grid size; 1: four uniform waves per block; 2: four pairs of a matrix wave and a
+ *       softmax wave per block.  Both give the same bits; other values make the call return
+ *       QM_ERR_ARGUMENT. */
 enum {
     QM_OPT_PREFILL_SCORE_ROUNDING = 0,
     QM_OPT_DECODE_TILES_PER_BLOCK = 1,
-    QM_OPT_COUNT = 2
+    QM_OPT_PREFILL_KERNEL = 2,
+    QM_OPT_COUNT = 3
 };
 /* Returns QM_ERR_ARGUMENT for an unknown option or a negative value. */
 int32_t qm_set_option(int32_t option, int32_t value);
