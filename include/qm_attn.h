@@ -363,6 +363,41 @@ int32_t qm_add_postnorm_gate_up_swiglu_m1(
     int32_t hidden, int32_t intermediate,
     void* hip_stream);
 
+/*
+ * The code predictor's M = 1 linears.  Replace PersistentPredictor::linear_m1 (R17:13499-13533,
+ * kernel predictor_linear_m1_fused_kernel :12579-12654), ::qkv_m1 (R17:13389-13430, kernel
+ * predictor_qkv_m1_fused_kernel :12046-12130) and ::gate_up_swiglu_m1 (R17:13558-13589, kernel
+ * :12736-12815).  Same layouts as the talker's linears above, no bias, and another order of the
+ * sum, reproduced bit for bit: lane l of the row's 32 chains takes the element pairs
+ * k = 2l, 2l + 64, ..., first element of a pair first, each product added with one fmaf
+ * (predictor_bf16_dot2_accumulate in its portable form, R17:8216-8228; the gfx1100 build of the
+ * reference uses that chip's dot2 instruction, whose rounding is not restated here).
+ * qm_predictor_rmsnorm_qkv_m1 and qm_predictor_add_postnorm_gate_up_swiglu_m1 fuse the launch
+ * before (rmsnorm R17:13210-13220; add_postnorm_m1 :13535-13556, kernel :12658-12733, the talker's
+ * arithmetic) like their talker counterparts.  All five need reduction % 8 == 0,
+ * reduction <= 16384 and 16-byte aligned weight matrices (QM_ERR_GEOMETRY otherwise).
+ */
+int32_t qm_predictor_linear_m1(
+    const uint16_t* input, const uint16_t* weight, const uint16_t* residual, uint16_t* output,
+    int32_t output_columns, int32_t reduction_columns, void* hip_stream);
+int32_t qm_predictor_qkv_m1(
+    const uint16_t* input, const uint16_t* q_weight, const uint16_t* k_weight, const uint16_t* v_weight,
+    uint16_t* q_output, uint16_t* k_output, uint16_t* v_output,
+    int32_t hidden, int32_t q_dim, int32_t kv_dim, void* hip_stream);
+int32_t qm_predictor_gate_up_swiglu_m1(
+    const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight, uint16_t* output,
+    int32_t hidden, int32_t intermediate, void* hip_stream);
+int32_t qm_predictor_rmsnorm_qkv_m1(
+    const uint16_t* hidden_state, const uint16_t* norm_weight, float epsilon,
+    const uint16_t* q_weight, const uint16_t* k_weight, const uint16_t* v_weight,
+    uint16_t* q_output, uint16_t* k_output, uint16_t* v_output,
+    int32_t hidden, int32_t q_dim, int32_t kv_dim, void* hip_stream);
+int32_t qm_predictor_add_postnorm_gate_up_swiglu_m1(
+    const uint16_t* hidden_state, const uint16_t* attention, const uint16_t* norm_weight, float epsilon,
+    uint16_t* residual,
+    const uint16_t* gate_weight, const uint16_t* up_weight, uint16_t* output,
+    int32_t hidden, int32_t intermediate, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

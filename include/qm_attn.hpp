@@ -262,6 +262,41 @@ inline void launch_add_postnorm_m1(
           "Qingming add/postnorm launch");
 }
 
+// PersistentPredictor::linear_m1 (R17:13499-13533).
+inline void predictor_linear_m1(
+    const std::uint16_t* input, const std::uint16_t* weight, const std::uint16_t* residual, std::uint16_t* output,
+    int output_columns, int reduction_columns, void* stream) {
+    check(qm_predictor_linear_m1(input, weight, residual, output, output_columns, reduction_columns, stream),
+          "predictor linear_m1 launch");
+}
+
+// PersistentPredictor::qkv_m1 (R17:13389-13430); the geometry the reference bakes in
+// (kHidden 1024, kQueryDim 2048, kKvDim 1024, R17:7951-7959) is passed by the caller.
+inline void predictor_qkv_m1(
+    const std::uint16_t* input, const std::uint16_t* q_weight, const std::uint16_t* k_weight,
+    const std::uint16_t* v_weight, std::uint16_t* q_output, std::uint16_t* k_output, std::uint16_t* v_output,
+    int hidden, int q_dim, int kv_dim, void* stream) {
+    check(qm_predictor_qkv_m1(input, q_weight, k_weight, v_weight, q_output, k_output, v_output, hidden, q_dim,
+                              kv_dim, stream),
+          "predictor qkv_m1 launch");
+}
+
+// PersistentPredictor::gate_up_swiglu_m1 (R17:13558-13589).
+inline void predictor_gate_up_swiglu_m1(
+    const std::uint16_t* input, const std::uint16_t* gate_weight, const std::uint16_t* up_weight,
+    std::uint16_t* output, int hidden, int intermediate, void* stream) {
+    check(qm_predictor_gate_up_swiglu_m1(input, gate_weight, up_weight, output, hidden, intermediate, stream),
+          "predictor gate_up_swiglu_m1 launch");
+}
+
+// PersistentPredictor::add_postnorm_m1 (R17:13535-13556): the talker's arithmetic.
+inline void predictor_add_postnorm_m1(
+    const std::uint16_t* hidden, const std::uint16_t* attention, const std::uint16_t* norm_weight,
+    std::uint16_t* residual, std::uint16_t* normalized, int dimension, void* stream) {
+    check(qm_add_postnorm_m1(hidden, attention, norm_weight, residual, normalized, dimension, 1.0e-6f, stream),
+          "predictor add_postnorm_m1 launch");
+}
+
 }  // namespace qm_attn
 
 #endif  // QM_ATTN_HPP

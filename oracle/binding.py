@@ -217,3 +217,18 @@ def add_postnorm_m1(hidden, attention, norm_weight, residual, normalized, dimens
 def gate_up_swiglu_m1(x, gate_w, up_w, out, hidden, intermediate, threads=8):
     return lib().qmo_gate_up_swiglu_m1(_p(x), _p(gate_w), _p(up_w), _p(out), C.c_int32(hidden),
                                        C.c_int32(intermediate), C.c_int32(threads))
+
+
+def predictor_linear_m1(x, weight, residual, out, output_columns, reduction_columns, threads=8):
+    return lib().qmo_predictor_linear_m1(_p(x), _p(weight), _p(residual), _p(out), C.c_int32(output_columns),
+                                         C.c_int32(reduction_columns), C.c_int32(threads))
+
+
+def predictor_qkv_m1(x, q_w, k_w, v_w, q_out, k_out, v_out, hidden, q_dim, kv_dim, threads=8):
+    return lib().qmo_predictor_qkv_m1(_p(x), _p(q_w), _p(k_w), _p(v_w), _p(q_out), _p(k_out), _p(v_out),
+                                      C.c_int32(hidden), C.c_int32(q_dim), C.c_int32(kv_dim), C.c_int32(threads))
+
+
+def predictor_gate_up_swiglu_m1(x, gate_w, up_w, out, hidden, intermediate, threads=8):
+    return lib().qmo_predictor_gate_up_swiglu_m1(_p(x), _p(gate_w), _p(up_w), _p(out), C.c_int32(hidden),
+                                                 C.c_int32(intermediate), C.c_int32(threads))

@@ -804,4 +804,78 @@ int32_t qmo_gate_up_swiglu_m1(const uint16_t* input, const uint16_t* gate_weight
     return QM_OK;
 }
 
+// ---- the code predictor's M = 1 linears ------------------------------------------------------------
+// predictor_linear_m1_fused_kernel, predictor_qkv_m1_fused_kernel and
+// predictor_gate_up_swiglu_m1_kernel (R17:12579-12654, 12046-12130, 12736-12815) walk a row in
+// another order than the talker's: lane l takes the element pairs k = 2l, 2l + 64, ... (loop
+// condition k + 1 < columns) and adds x[k] w[k] and then x[k+1] w[k+1] to its accumulator
+// (predictor_bf16_dot2_accumulate, R17:8193-8230, in its portable form: two fmaf; the gfx1100 build
+// uses that chip's dot2 instruction instead, whose rounding is the hardware's and is not restated
+// here); a last odd column is added by lane 0 after its pairs; the same shuffle tree; no bias.
+static uint16_t predictor_linear_m1_scalar(const uint16_t* input, const uint16_t* weight_row,
+                                           const uint16_t* residual, int out, int reduction_columns) {
+    float lanes[32];
+    for (int l = 0; l < 32; ++l) {
+        float acc = 0.0f;
+        for (int k = 2 * l; k + 1 < reduction_columns; k += 64) {
+            acc = std::fmaf(bf2f(input[k]), bf2f(weight_row[k]), acc);
+            acc = std::fmaf(bf2f(input[k + 1]), bf2f(weight_row[k + 1]), acc);
+        }
+        lanes[l] = acc;
+    }
+    if (reduction_columns & 1) {
+        const int k = reduction_columns - 1;
+        lanes[0] = std::fmaf(bf2f(input[k]), bf2f(weight_row[k]), lanes[0]);
+    }
+    const uint16_t v = f2bf(wave32_sum(lanes));
+    return residual ? f2bf(bf2f(residual[out]) + bf2f(v)) : v;
+}
+
+int32_t qmo_predictor_linear_m1(const uint16_t* input, const uint16_t* weight, const uint16_t* residual,
+                                uint16_t* output, int32_t output_columns, int32_t reduction_columns,
+                                int32_t n_threads) {
+    if (!input || !weight || !output) return QM_ERR_NULL;
+    if (output_columns < 0 || reduction_columns < 0) return QM_ERR_ARGUMENT;
+    parallel_for(output_columns, n_threads, [&](int64_t o) {
+        output[o] = predictor_linear_m1_scalar(input, weight + o * reduction_columns, residual,
+                                               static_cast<int>(o), reduction_columns);
+    });
+    return QM_OK;
+}
+
+int32_t qmo_predictor_qkv_m1(const uint16_t* input, const uint16_t* q_weight, const uint16_t* k_weight,
+                             const uint16_t* v_weight, uint16_t* q_output, uint16_t* k_output,
+                             uint16_t* v_output, int32_t hidden, int32_t q_dim, int32_t kv_dim,
+                             int32_t n_threads) {
+    if (!input || !q_weight || !k_weight || !v_weight || !q_output || !k_output || !v_output) return QM_ERR_NULL;
+    if (hidden < 0 || q_dim < 0 || kv_dim < 0) return QM_ERR_ARGUMENT;
+    parallel_for(static_cast<int64_t>(q_dim) + 2 * kv_dim, n_threads, [&](int64_t first) {
+        if (first < q_dim) {
+            q_output[first] = predictor_linear_m1_scalar(input, q_weight + first * hidden, nullptr, 0, hidden);
+        } else if (first < q_dim + kv_dim) {
+            const int64_t r = first - q_dim;
+            k_output[r] = predictor_linear_m1_scalar(input, k_weight + r * hidden, nullptr, 0, hidden);
+        } else {
+            const int64_t r = first - q_dim - kv_dim;
+            v_output[r] = predictor_linear_m1_scalar(input, v_weight + r * hidden, nullptr, 0, hidden);
+        }
+    });
+    return QM_OK;
+}
+
+int32_t qmo_predictor_gate_up_swiglu_m1(const uint16_t* input, const uint16_t* gate_weight,
+                                        const uint16_t* up_weight, uint16_t* output, int32_t hidden,
+                                        int32_t intermediate, int32_t n_threads) {
+    if (!input || !gate_weight || !up_weight || !output) return QM_ERR_NULL;
+    if (hidden < 0 || intermediate < 0) return QM_ERR_ARGUMENT;
+    parallel_for(intermediate, n_threads, [&](int64_t ch) {
+        const uint16_t gb = predictor_linear_m1_scalar(input, gate_weight + ch * hidden, nullptr, 0, hidden);
+        const uint16_t ub = predictor_linear_m1_scalar(input, up_weight + ch * hidden, nullptr, 0, hidden);
+        const float gv = bf2f(gb);
+        const uint16_t act = f2bf(gv / (1.0f + std::exp(-gv)));
+        output[ch] = f2bf(bf2f(act) * bf2f(ub));
+    });
+    return QM_OK;
+}
+
 }  // extern "C"

@@ -70,6 +70,11 @@ _SIGNATURES = {
     "qm_add_postnorm_m1": (_I32, [_PTR] * 5 + [_I32, _F32, _PTR]),
     "qm_rmsnorm_qkv_m1": (_I32, [_PTR, _PTR, _F32] + [_PTR] * 9 + [_I32, _I32, _I32, _PTR]),
     "qm_add_postnorm_gate_up_swiglu_m1": (_I32, [_PTR, _PTR, _PTR, _F32] + [_PTR] * 4 + [_I32, _I32, _PTR]),
+    "qm_predictor_linear_m1": (_I32, [_PTR] * 4 + [_I32, _I32, _PTR]),
+    "qm_predictor_qkv_m1": (_I32, [_PTR] * 7 + [_I32, _I32, _I32, _PTR]),
+    "qm_predictor_gate_up_swiglu_m1": (_I32, [_PTR] * 4 + [_I32, _I32, _PTR]),
+    "qm_predictor_rmsnorm_qkv_m1": (_I32, [_PTR, _PTR, _F32] + [_PTR] * 6 + [_I32, _I32, _I32, _PTR]),
+    "qm_predictor_add_postnorm_gate_up_swiglu_m1": (_I32, [_PTR, _PTR, _PTR, _F32] + [_PTR] * 4 + [_I32, _I32, _PTR]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
@@ -245,6 +250,35 @@ def add_postnorm_gate_up_swiglu_m1(hidden_state, attention, norm_weight, residua
     _check(lib().qm_add_postnorm_gate_up_swiglu_m1(_addr(hidden_state), _addr(attention), _addr(norm_weight), eps,
                                                    _addr(residual), _addr(gate_w), _addr(up_w), _addr(out), hidden,
                                                    intermediate, stream), "qm_add_postnorm_gate_up_swiglu_m1")
+
+
+def predictor_linear_m1(x, weight, residual, out, output_columns, reduction_columns, stream=0):
+    _check(lib().qm_predictor_linear_m1(_addr(x), _addr(weight), _addr(residual), _addr(out), output_columns,
+                                        reduction_columns, stream), "qm_predictor_linear_m1")
+
+
+def predictor_qkv_m1(x, q_w, k_w, v_w, q_out, k_out, v_out, hidden, q_dim, kv_dim, stream=0):
+    _check(lib().qm_predictor_qkv_m1(_addr(x), _addr(q_w), _addr(k_w), _addr(v_w), _addr(q_out), _addr(k_out),
+                                     _addr(v_out), hidden, q_dim, kv_dim, stream), "qm_predictor_qkv_m1")
+
+
+def predictor_gate_up_swiglu_m1(x, gate_w, up_w, out, hidden, intermediate, stream=0):
+    _check(lib().qm_predictor_gate_up_swiglu_m1(_addr(x), _addr(gate_w), _addr(up_w), _addr(out), hidden,
+                                                intermediate, stream), "qm_predictor_gate_up_swiglu_m1")
+
+
+def predictor_rmsnorm_qkv_m1(hidden_state, norm_weight, q_w, k_w, v_w, q_out, k_out, v_out, hidden, q_dim, kv_dim,
+                             eps=1e-6, stream=0):
+    _check(lib().qm_predictor_rmsnorm_qkv_m1(_addr(hidden_state), _addr(norm_weight), eps, _addr(q_w), _addr(k_w),
+                                             _addr(v_w), _addr(q_out), _addr(k_out), _addr(v_out), hidden, q_dim,
+                                             kv_dim, stream), "qm_predictor_rmsnorm_qkv_m1")
+
+
+def predictor_add_postnorm_gate_up_swiglu_m1(hidden_state, attention, norm_weight, residual, gate_w, up_w, out,
+                                             hidden, intermediate, eps=1e-6, stream=0):
+    _check(lib().qm_predictor_add_postnorm_gate_up_swiglu_m1(
+        _addr(hidden_state), _addr(attention), _addr(norm_weight), eps, _addr(residual), _addr(gate_w), _addr(up_w),
+        _addr(out), hidden, intermediate, stream), "qm_predictor_add_postnorm_gate_up_swiglu_m1")
 
 
 def predictor_attention_staged(query_bhsd, key_cache, value_cache, out, rows, key_length, causal, stream=0):

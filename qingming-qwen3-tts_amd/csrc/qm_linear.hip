@@ -45,6 +45,11 @@ struct LinearParams {
     uint16_t* residual_out;       // pre == 2: bf16(input + addend), written by block 0
     float epsilon;
     int rows_per_block;           // staged kernel: outputs (channels) per block, 1..8
+    // Order of a row's 32 chains (staged kernel).  0: lane l takes k = l, l + 32, ... (the talker's
+    // kernels).  1: lane l takes the pairs k = 2l, 2l + 1, then 2l + 64, 2l + 65, ..., first
+    // element first (the code predictor's kernels, R17:12110-12120, in their portable form: two
+    // fmaf per pair; the gfx1100 build of the reference uses that chip's dot2 instruction).
+    int pairs;
 };
 
 // DUAL: weight[0] / weight[1] are the gate and up matrices of one SwiGLU channel per output
@@ -289,7 +294,46 @@ __global__ __launch_bounds__(kStagedThreads) void linear_m1_staged_kernel(Linear
     const uint16_t* w1 = reinterpret_cast<const uint16_t*>(lds_w + (2 * c + 1) * row_stride) + l;   // DUAL only
     const float* xs = lin_x + l;
     float acc = 0.0f, up = 0.0f;
-    if (live) {
+    if (live && prm.pairs) {
+        const uint32_t* p0 = reinterpret_cast<const uint32_t*>(lds_w + (DUAL ? 2 * c : c) * row_stride) + l;
+        const uint32_t* p1 = reinterpret_cast<const uint32_t*>(lds_w + (2 * c + 1) * row_stride) + l;   // DUAL only
+        const float2* xp = reinterpret_cast<const float2*>(lin_x) + l;
+        const int full = K >> 6;        // steps of 32 pairs in which every lane has a pair
+        const int pair_steps = (K + 63) >> 6;
+        int j = 0;
+        for (; j + 8 <= full; j += 8) {
+            float2 x[8];
+            uint32_t a[8], b[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                x[u] = xp[32 * (j + u)];
+                a[u] = p0[32 * (j + u)];
+                if (DUAL) b[u] = p1[32 * (j + u)];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                acc = fmaf(x[u].x, lo_bf16(a[u]), acc);
+                acc = fmaf(x[u].y, hi_bf16(a[u]), acc);
+                if (DUAL) {
+                    up = fmaf(x[u].x, lo_bf16(b[u]), up);
+                    up = fmaf(x[u].y, hi_bf16(b[u]), up);
+                }
+            }
+        }
+        for (; j < pair_steps; ++j) {
+            if (64 * j + 2 * l + 1 < K) {
+                const float2 x = xp[32 * j];
+                const uint32_t a = p0[32 * j];
+                acc = fmaf(x.x, lo_bf16(a), acc);
+                acc = fmaf(x.y, hi_bf16(a), acc);
+                if (DUAL) {
+                    const uint32_t b = p1[32 * j];
+                    up = fmaf(x.x, lo_bf16(b), up);
+                    up = fmaf(x.y, hi_bf16(b), up);
+                }
+            }
+        }
+    } else if (live) {
         const int full = K >> 5;        // steps in which every lane has an element
         int j = 0;
         for (; j + 8 <= full; j += 8) {
@@ -388,12 +432,10 @@ inline int32_t check_reduction(int32_t reduction) {
     return QM_OK;
 }
 
-}  // namespace qm
-
-extern "C" int32_t qm_linear_m1(const uint16_t* input, const uint16_t* weight, const uint16_t* bias,
-                                const uint16_t* residual, uint16_t* output, int32_t output_columns,
-                                int32_t reduction_columns, void* hip_stream) {
-    using namespace qm;
+// ---- the entry points' bodies; `pairs` selects the order of the chains (LinearParams::pairs) ------------
+inline int32_t linear_entry(int pairs, const uint16_t* input, const uint16_t* weight, const uint16_t* bias,
+                            const uint16_t* residual, uint16_t* output, int32_t output_columns,
+                            int32_t reduction_columns, void* hip_stream) {
     if (!input || !weight || !output) return QM_ERR_NULL;
     if (output_columns < 0) return QM_ERR_ARGUMENT;
     const int32_t rc = check_reduction(reduction_columns);
@@ -409,18 +451,21 @@ extern "C" int32_t qm_linear_m1(const uint16_t* input, const uint16_t* weight, c
     prm.reduction = reduction_columns;
     prm.weight[1] = prm.weight[2] = weight;   // never read: rows[1] = rows[2] = 0
     prm.output[1] = prm.output[2] = output;
+    prm.pairs = pairs;
     if (staged_ok(prm, false) && staged_rows_per_block<false>(prm.reduction) > 0)
         return launch_staged<false>(prm, static_cast<hipStream_t>(hip_stream));
+    if (pairs) return QM_ERR_GEOMETRY;        // the pair order exists in the staged kernel only
     return launch_linear<false>(prm, static_cast<hipStream_t>(hip_stream));
 }
 
-extern "C" int32_t qm_qkv_m1(const uint16_t* input, const uint16_t* q_weight, const uint16_t* q_bias,
-                             const uint16_t* k_weight, const uint16_t* k_bias, const uint16_t* v_weight,
-                             const uint16_t* v_bias, uint16_t* q_output, uint16_t* k_output,
-                             uint16_t* v_output, int32_t hidden, int32_t q_dim, int32_t kv_dim,
-                             void* hip_stream) {
-    using namespace qm;
+// pre: 0 = the input is given; 1 = RMSNorm(input) * norm_weight is computed in the kernel
+inline int32_t qkv_entry(int pairs, int pre, const uint16_t* input, const uint16_t* norm_weight, float epsilon,
+                         const uint16_t* q_weight, const uint16_t* q_bias, const uint16_t* k_weight,
+                         const uint16_t* k_bias, const uint16_t* v_weight, const uint16_t* v_bias,
+                         uint16_t* q_output, uint16_t* k_output, uint16_t* v_output, int32_t hidden,
+                         int32_t q_dim, int32_t kv_dim, void* hip_stream) {
     if (!input || !q_weight || !k_weight || !v_weight || !q_output || !k_output || !v_output) return QM_ERR_NULL;
+    if (pre && !norm_weight) return QM_ERR_NULL;
     if (q_dim < 0 || kv_dim < 0) return QM_ERR_ARGUMENT;
     const int32_t rc = check_reduction(hidden);
     if (rc != QM_OK) return rc;
@@ -435,15 +480,21 @@ extern "C" int32_t qm_qkv_m1(const uint16_t* input, const uint16_t* q_weight, co
     prm.residual = nullptr;
     prm.rows[0] = q_dim; prm.rows[1] = kv_dim; prm.rows[2] = kv_dim;
     prm.reduction = hidden;
+    prm.pairs = pairs;
+    prm.pre = pre; prm.norm_weight = norm_weight; prm.epsilon = epsilon;
     if (staged_ok(prm, false) && staged_rows_per_block<false>(prm.reduction) > 0)
         return launch_staged<false>(prm, static_cast<hipStream_t>(hip_stream));
+    if (pairs || pre) return QM_ERR_GEOMETRY;  // the pair order and the fused prologue exist in the staged kernel only
     return launch_linear<false>(prm, static_cast<hipStream_t>(hip_stream));
 }
 
-extern "C" int32_t qm_gate_up_swiglu_m1(const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight,
-                                        uint16_t* output, int32_t hidden, int32_t intermediate, void* hip_stream) {
-    using namespace qm;
+// pre: 0 = the input is given; 2 = residual = bf16(input + attention), RMSNorm(residual) * norm_weight
+inline int32_t gate_up_entry(int pairs, int pre, const uint16_t* input, const uint16_t* attention,
+                             const uint16_t* norm_weight, float epsilon, uint16_t* residual,
+                             const uint16_t* gate_weight, const uint16_t* up_weight, uint16_t* output,
+                             int32_t hidden, int32_t intermediate, void* hip_stream) {
     if (!input || !gate_weight || !up_weight || !output) return QM_ERR_NULL;
+    if (pre && (!attention || !norm_weight || !residual)) return QM_ERR_NULL;
     if (intermediate < 0) return QM_ERR_ARGUMENT;
     const int32_t rc = check_reduction(hidden);
     if (rc != QM_OK) return rc;
@@ -454,9 +505,36 @@ extern "C" int32_t qm_gate_up_swiglu_m1(const uint16_t* input, const uint16_t* g
     prm.output[0] = prm.output[1] = prm.output[2] = output;
     prm.rows[0] = intermediate;
     prm.reduction = hidden;
+    prm.pairs = pairs;
+    prm.pre = pre; prm.addend = attention; prm.norm_weight = norm_weight; prm.epsilon = epsilon;
+    prm.residual_out = residual;
     if (staged_ok(prm, true) && staged_rows_per_block<true>(prm.reduction) > 0)
         return launch_staged<true>(prm, static_cast<hipStream_t>(hip_stream));
+    if (pairs || pre) return QM_ERR_GEOMETRY;
     return launch_linear<true>(prm, static_cast<hipStream_t>(hip_stream));
+}
+
+}  // namespace qm
+
+extern "C" int32_t qm_linear_m1(const uint16_t* input, const uint16_t* weight, const uint16_t* bias,
+                                const uint16_t* residual, uint16_t* output, int32_t output_columns,
+                                int32_t reduction_columns, void* hip_stream) {
+    return qm::linear_entry(0, input, weight, bias, residual, output, output_columns, reduction_columns, hip_stream);
+}
+
+extern "C" int32_t qm_qkv_m1(const uint16_t* input, const uint16_t* q_weight, const uint16_t* q_bias,
+                             const uint16_t* k_weight, const uint16_t* k_bias, const uint16_t* v_weight,
+                             const uint16_t* v_bias, uint16_t* q_output, uint16_t* k_output,
+                             uint16_t* v_output, int32_t hidden, int32_t q_dim, int32_t kv_dim,
+                             void* hip_stream) {
+    return qm::qkv_entry(0, 0, input, nullptr, 0.0f, q_weight, q_bias, k_weight, k_bias, v_weight, v_bias,
+                         q_output, k_output, v_output, hidden, q_dim, kv_dim, hip_stream);
+}
+
+extern "C" int32_t qm_gate_up_swiglu_m1(const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight,
+                                        uint16_t* output, int32_t hidden, int32_t intermediate, void* hip_stream) {
+    return qm::gate_up_entry(0, 0, input, nullptr, nullptr, 0.0f, nullptr, gate_weight, up_weight, output, hidden,
+                             intermediate, hip_stream);
 }
 
 // ---- fusions of two reference launches each (staged kernel only) -------------------------------------
@@ -466,22 +544,8 @@ extern "C" int32_t qm_rmsnorm_qkv_m1(const uint16_t* hidden_state, const uint16_
                                      const uint16_t* v_weight, const uint16_t* v_bias,
                                      uint16_t* q_output, uint16_t* k_output, uint16_t* v_output,
                                      int32_t hidden, int32_t q_dim, int32_t kv_dim, void* hip_stream) {
-    using namespace qm;
-    if (!hidden_state || !norm_weight || !q_weight || !k_weight || !v_weight || !q_output || !k_output || !v_output)
-        return QM_ERR_NULL;
-    if (q_dim < 0 || kv_dim < 0) return QM_ERR_ARGUMENT;
-    const int32_t rc = check_reduction(hidden);
-    if (rc != QM_OK) return rc;
-    LinearParams prm = {};
-    prm.input = hidden_state;
-    prm.weight[0] = q_weight; prm.weight[1] = k_weight; prm.weight[2] = v_weight;
-    prm.bias[0] = q_bias; prm.bias[1] = k_bias; prm.bias[2] = v_bias;
-    prm.output[0] = q_output; prm.output[1] = k_output; prm.output[2] = v_output;
-    prm.rows[0] = q_dim; prm.rows[1] = kv_dim; prm.rows[2] = kv_dim;
-    prm.reduction = hidden;
-    prm.pre = 1; prm.norm_weight = norm_weight; prm.epsilon = epsilon;
-    if (!staged_ok(prm, false) || staged_rows_per_block<false>(hidden) == 0) return QM_ERR_GEOMETRY;
-    return launch_staged<false>(prm, static_cast<hipStream_t>(hip_stream));
+    return qm::qkv_entry(0, 1, hidden_state, norm_weight, epsilon, q_weight, q_bias, k_weight, k_bias, v_weight,
+                         v_bias, q_output, k_output, v_output, hidden, q_dim, kv_dim, hip_stream);
 }
 
 extern "C" int32_t qm_add_postnorm_gate_up_swiglu_m1(const uint16_t* hidden_state, const uint16_t* attention,
@@ -489,20 +553,48 @@ extern "C" int32_t qm_add_postnorm_gate_up_swiglu_m1(const uint16_t* hidden_stat
                                                      const uint16_t* gate_weight, const uint16_t* up_weight,
                                                      uint16_t* output, int32_t hidden, int32_t intermediate,
                                                      void* hip_stream) {
-    using namespace qm;
-    if (!hidden_state || !attention || !norm_weight || !residual || !gate_weight || !up_weight || !output)
-        return QM_ERR_NULL;
-    if (intermediate < 0) return QM_ERR_ARGUMENT;
-    const int32_t rc = check_reduction(hidden);
-    if (rc != QM_OK) return rc;
-    LinearParams prm = {};
-    prm.input = hidden_state;
-    prm.weight[0] = gate_weight; prm.weight[1] = up_weight; prm.weight[2] = gate_weight;
-    prm.output[0] = prm.output[1] = prm.output[2] = output;
-    prm.rows[0] = intermediate;
-    prm.reduction = hidden;
-    prm.pre = 2; prm.addend = attention; prm.norm_weight = norm_weight; prm.epsilon = epsilon;
-    prm.residual_out = residual;
-    if (!staged_ok(prm, true) || staged_rows_per_block<true>(hidden) == 0) return QM_ERR_GEOMETRY;
-    return launch_staged<true>(prm, static_cast<hipStream_t>(hip_stream));
+    if (!attention || !norm_weight || !residual) return QM_ERR_NULL;
+    return qm::gate_up_entry(0, 2, hidden_state, attention, norm_weight, epsilon, residual, gate_weight, up_weight,
+                             output, hidden, intermediate, hip_stream);
+}
+
+// ---- the code predictor's twins: the pair order of the chains, no bias ---------------------------------
+extern "C" int32_t qm_predictor_linear_m1(const uint16_t* input, const uint16_t* weight, const uint16_t* residual,
+                                          uint16_t* output, int32_t output_columns, int32_t reduction_columns,
+                                          void* hip_stream) {
+    return qm::linear_entry(1, input, weight, nullptr, residual, output, output_columns, reduction_columns, hip_stream);
+}
+
+extern "C" int32_t qm_predictor_qkv_m1(const uint16_t* input, const uint16_t* q_weight, const uint16_t* k_weight,
+                                       const uint16_t* v_weight, uint16_t* q_output, uint16_t* k_output,
+                                       uint16_t* v_output, int32_t hidden, int32_t q_dim, int32_t kv_dim,
+                                       void* hip_stream) {
+    return qm::qkv_entry(1, 0, input, nullptr, 0.0f, q_weight, nullptr, k_weight, nullptr, v_weight, nullptr,
+                         q_output, k_output, v_output, hidden, q_dim, kv_dim, hip_stream);
+}
+
+extern "C" int32_t qm_predictor_gate_up_swiglu_m1(const uint16_t* input, const uint16_t* gate_weight,
+                                                  const uint16_t* up_weight, uint16_t* output, int32_t hidden,
+                                                  int32_t intermediate, void* hip_stream) {
+    return qm::gate_up_entry(1, 0, input, nullptr, nullptr, 0.0f, nullptr, gate_weight, up_weight, output, hidden,
+                             intermediate, hip_stream);
+}
+
+extern "C" int32_t qm_predictor_rmsnorm_qkv_m1(const uint16_t* hidden_state, const uint16_t* norm_weight, float epsilon,
+                                               const uint16_t* q_weight, const uint16_t* k_weight,
+                                               const uint16_t* v_weight, uint16_t* q_output, uint16_t* k_output,
+                                               uint16_t* v_output, int32_t hidden, int32_t q_dim, int32_t kv_dim,
+                                               void* hip_stream) {
+    return qm::qkv_entry(1, 1, hidden_state, norm_weight, epsilon, q_weight, nullptr, k_weight, nullptr, v_weight,
+                         nullptr, q_output, k_output, v_output, hidden, q_dim, kv_dim, hip_stream);
+}
+
+extern "C" int32_t qm_predictor_add_postnorm_gate_up_swiglu_m1(const uint16_t* hidden_state, const uint16_t* attention,
+                                                               const uint16_t* norm_weight, float epsilon,
+                                                               uint16_t* residual, const uint16_t* gate_weight,
+                                                               const uint16_t* up_weight, uint16_t* output,
+                                                               int32_t hidden, int32_t intermediate, void* hip_stream) {
+    if (!attention || !norm_weight || !residual) return QM_ERR_NULL;
+    return qm::gate_up_entry(1, 2, hidden_state, attention, norm_weight, epsilon, residual, gate_weight, up_weight,
+                             output, hidden, intermediate, hip_stream);
 }

@@ -233,3 +233,117 @@ def test_fused_entries_reject_what_the_staged_kernel_cannot_take(qm, dev):
                                                w.data_ptr(), w.data_ptr(), o.data_ptr(), 68, 8, None) == -2
     assert L.qm_rmsnorm_qkv_m1(None, x.data_ptr(), 1e-6, w.data_ptr(), None, w.data_ptr(), None, w.data_ptr(),
                                None, o.data_ptr(), o.data_ptr(), o.data_ptr(), 64, 8, 8, None) == -1
+
+
+# ---- the code predictor's twins (pair order of the chains, no bias) -----------------------------------
+from linear_cases import predictor_order_cases  # noqa: E402
+
+
+def _gpu_plinear(qm, dev, x, w, residual=None):
+    import torch
+    out = torch.full((w.shape[0],), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.predictor_linear_m1(to_dev(x, dev), to_dev(np.ascontiguousarray(w), dev),
+                           None if residual is None else to_dev(residual, dev), out, w.shape[0], w.shape[1])
+    torch.cuda.synchronize()
+    return to_u16(out)
+
+
+@pytest.mark.parametrize("rows,red,residual", [
+    (1024, 2048, True),       # o_proj + residual of the predictor (kQueryDim -> kHidden)
+    (1024, 3072, True),       # down_proj + residual
+    (2048, 1024, False), (1, 8, False), (5, 72, True), (33, 136, False), (7, 4104, True), (3, 16384, False),
+])
+def test_predictor_linear_m1_bit_exact(oracle, qm, dev, rows, red, residual):
+    seed = 2100 + rows + red
+    x = oracle.normal_bf16((red,), seed)
+    w = oracle.normal_bf16((rows, red), seed + 1, std=0.02)
+    r = oracle.normal_bf16((rows,), seed + 3) if residual else None
+    want = np.zeros(rows, dtype=np.uint16)
+    assert oracle.predictor_linear_m1(x, w, r, want, rows, red, 16) == 0
+    assert np.array_equal(_gpu_plinear(qm, dev, x, w, r), want)
+
+
+@pytest.mark.parametrize("case", [c for c in predictor_order_cases() if c[1].shape[0] % 8 == 0], ids=lambda c: c[0])
+def test_predictor_evaluation_order_on_the_gpu(qm, dev, case):
+    _, wrow, residual, expected = case
+    x = np.full(wrow.shape[0], 0x3f80, dtype=np.uint16)
+    w = np.stack([wrow] * 9)                   # more rows than one block owns
+    r = None if residual is None else np.full(9, residual, dtype=np.uint16)
+    got = _gpu_plinear(qm, dev, x, w, r)
+    assert np.all(got == expected)
+
+
+@pytest.mark.parametrize("hidden,q_dim,kv_dim", [(1024, 2048, 1024), (200, 40, 24), (8, 1, 1)])
+def test_predictor_qkv_m1_bit_exact(oracle, qm, dev, hidden, q_dim, kv_dim):
+    import torch
+    seed = 2300 + hidden
+    x = oracle.normal_bf16((hidden,), seed)
+    nw = oracle.normal_bf16((hidden,), seed + 9, mean=1.0, std=0.1)
+    dims = (q_dim, kv_dim, kv_dim)
+    ws = [oracle.normal_bf16((n, hidden), seed + 1 + i, std=0.02) for i, n in enumerate(dims)]
+    wd = [to_dev(w, dev) for w in ws]
+    want = [np.zeros(n, dtype=np.uint16) for n in dims]
+    assert oracle.predictor_qkv_m1(x, ws[0], ws[1], ws[2], want[0], want[1], want[2], hidden, q_dim, kv_dim, 16) == 0
+    outs = [torch.full((n,), 0x7fc0, dtype=torch.int16, device=dev) for n in dims]
+    qm.predictor_qkv_m1(to_dev(x, dev), wd[0], wd[1], wd[2], outs[0], outs[1], outs[2], hidden, q_dim, kv_dim)
+    torch.cuda.synchronize()
+    for o, w_ in zip(outs, want):
+        assert np.array_equal(to_u16(o), w_)
+    # fused with the RMSNorm in front of it = the two operators
+    normed = np.zeros((1, hidden), dtype=np.uint16)
+    assert oracle.rmsnorm_rows(x.reshape(1, hidden), nw, normed, 1, hidden) == 0
+    assert oracle.predictor_qkv_m1(normed[0], ws[0], ws[1], ws[2], want[0], want[1], want[2], hidden, q_dim, kv_dim,
+                                   16) == 0
+    outs = [torch.full((n,), 0x7fc0, dtype=torch.int16, device=dev) for n in dims]
+    qm.predictor_rmsnorm_qkv_m1(to_dev(x, dev), to_dev(nw, dev), wd[0], wd[1], wd[2], outs[0], outs[1], outs[2],
+                                hidden, q_dim, kv_dim)
+    torch.cuda.synchronize()
+    for o, w_ in zip(outs, want):
+        assert np.array_equal(to_u16(o), w_)
+
+
+@pytest.mark.parametrize("hidden,inter", [(1024, 3072), (200, 33), (8, 1)])
+def test_predictor_gate_up_swiglu(oracle, qm, dev, hidden, inter):
+    """As for the talker's: identical up to the last place of expf (at most one bf16 ulp, rarely)."""
+    import torch
+    from qm_testlib import ulp_distance
+    seed = 2700 + hidden
+    x = oracle.normal_bf16((hidden,), seed)
+    gw = oracle.normal_bf16((inter, hidden), seed + 1, std=0.03)
+    uw = oracle.normal_bf16((inter, hidden), seed + 2, std=0.03)
+    want = np.zeros(inter, dtype=np.uint16)
+    assert oracle.predictor_gate_up_swiglu_m1(x, gw, uw, want, hidden, inter, 16) == 0
+    out = torch.full((inter,), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.predictor_gate_up_swiglu_m1(to_dev(x, dev), to_dev(gw, dev), to_dev(uw, dev), out, hidden, inter)
+    torch.cuda.synchronize()
+    d = ulp_distance(to_u16(out), want)
+    assert d.max() <= 1 and np.count_nonzero(d) <= max(1, inter // 1000)
+    # fused with residual add + post-norm in front of it = the two operators
+    h = oracle.normal_bf16((hidden,), seed + 3)
+    a = oracle.normal_bf16((hidden,), seed + 4)
+    nw = oracle.normal_bf16((hidden,), seed + 5, mean=1.0, std=0.1)
+    res, nrm = np.zeros(hidden, dtype=np.uint16), np.zeros(hidden, dtype=np.uint16)
+    assert oracle.add_postnorm_m1(h, a, nw, res, nrm, hidden) == 0
+    assert oracle.predictor_gate_up_swiglu_m1(nrm, gw, uw, want, hidden, inter, 16) == 0
+    rd = torch.full((hidden,), 0x7fc0, dtype=torch.int16, device=dev)
+    out = torch.full((inter,), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.predictor_add_postnorm_gate_up_swiglu_m1(to_dev(h, dev), to_dev(a, dev), to_dev(nw, dev), rd, to_dev(gw, dev),
+                                                to_dev(uw, dev), out, hidden, inter)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_u16(rd), res)
+    d = ulp_distance(to_u16(out), want)
+    assert d.max() <= 1 and np.count_nonzero(d) <= max(1, inter // 1000)
+
+
+def test_predictor_linears_reject_what_the_staged_kernel_cannot_take(qm, dev):
+    import torch
+    x = torch.zeros(68, dtype=torch.int16, device=dev)
+    w = torch.zeros((8, 68), dtype=torch.int16, device=dev)
+    o = torch.zeros(8, dtype=torch.int16, device=dev)
+    L = qm.lib()
+    assert L.qm_predictor_linear_m1(x.data_ptr(), w.data_ptr(), None, o.data_ptr(), 8, 68, None) == -2   # 68 % 8 != 0
+    assert L.qm_predictor_linear_m1(x.data_ptr(), w.data_ptr(), None, o.data_ptr(), 8, 67, None) == -2   # odd
+    assert L.qm_predictor_linear_m1(None, w.data_ptr(), None, o.data_ptr(), 8, 64, None) == -1
+    assert L.qm_predictor_qkv_m1(x.data_ptr(), w.data_ptr(), w.data_ptr(), w.data_ptr(), o.data_ptr(), o.data_ptr(),
+                                 o.data_ptr(), 68, 8, 8, None) == -2
+    assert L.qm_predictor_gate_up_swiglu_m1(x.data_ptr(), w.data_ptr(), w.data_ptr(), o.data_ptr(), 64, -1, None) == -5

@@ -148,3 +148,58 @@ def test_gate_up_swiglu_values(oracle):
     gw[:, 0] = 0xc2c8                                                   # -100
     assert oracle.gate_up_swiglu_m1(x, gw, uw, out, hidden, inter) == 0
     assert np.all(np.abs(oracle.bf16_to_f32(out)) < 1e-30)
+
+
+# ---- the code predictor's order ----------------------------------------------------------------------
+from linear_cases import predictor_order_cases  # noqa: E402
+
+
+def _plin(oracle, x, w, residual=None):
+    out = np.zeros(w.shape[0], dtype=np.uint16)
+    assert oracle.predictor_linear_m1(x, np.ascontiguousarray(w), residual, out, w.shape[0], w.shape[1]) == 0
+    return out
+
+
+@pytest.mark.parametrize("case", predictor_order_cases(), ids=lambda c: c[0])
+def test_predictor_evaluation_order(oracle, case):
+    _, wrow, residual, expected = case
+    x = np.full(wrow.shape[0], 0x3f80, dtype=np.uint16)
+    w = np.stack([wrow, wrow])
+    r = None if residual is None else np.full(2, residual, dtype=np.uint16)
+    got = _plin(oracle, x, w, r)
+    assert got[0] == expected and got[1] == expected
+
+
+def test_predictor_linear_small_integers_and_fp64(oracle):
+    rng = np.random.default_rng(11)
+    rows, red = 24, 200
+    xi = rng.integers(-8, 9, size=red)
+    wi = rng.integers(-8, 9, size=(rows, red))
+    x = oracle.f32_to_bf16(xi.astype(np.float32))
+    w = oracle.f32_to_bf16(wi.astype(np.float32))
+    want = oracle.f32_to_bf16((wi @ xi).astype(np.float32))          # exact in fp32, any order
+    assert np.array_equal(_plin(oracle, x, w), want)
+    x = oracle.normal_bf16((1024,), 12)
+    w = oracle.normal_bf16((64, 1024), 13, std=0.05)
+    got = oracle.bf16_to_f32(_plin(oracle, x, w)).astype(np.float64)
+    ref = oracle.bf16_to_f32(w).astype(np.float64) @ oracle.bf16_to_f32(x).astype(np.float64)
+    assert np.max(np.abs(got - ref) / (np.abs(ref) + 1.0)) < 1e-2    # one bf16 rounding of a fp32-accurate sum
+
+
+def test_predictor_qkv_and_gate_up_are_built_from_the_linear(oracle):
+    hidden, q_dim, kv_dim, inter = 192, 40, 24, 56
+    x = oracle.normal_bf16((hidden,), 41)
+    ws = [oracle.normal_bf16((n, hidden), 42 + i, std=0.05) for i, n in enumerate((q_dim, kv_dim, kv_dim))]
+    outs = [np.zeros(n, dtype=np.uint16) for n in (q_dim, kv_dim, kv_dim)]
+    assert oracle.predictor_qkv_m1(x, ws[0], ws[1], ws[2], outs[0], outs[1], outs[2], hidden, q_dim, kv_dim) == 0
+    for w, o in zip(ws, outs):
+        assert np.array_equal(o, _plin(oracle, x, w))
+    gate = oracle.normal_bf16((inter, hidden), 51, std=0.08)
+    up = oracle.normal_bf16((inter, hidden), 52, std=0.08)
+    out = np.zeros(inter, dtype=np.uint16)
+    assert oracle.predictor_gate_up_swiglu_m1(x, gate, up, out, hidden, inter) == 0
+    g = oracle.bf16_to_f32(_plin(oracle, x, gate)).astype(np.float64)
+    u = oracle.bf16_to_f32(_plin(oracle, x, up)).astype(np.float64)
+    want = g / (1.0 + np.exp(-g)) * u                                  # SiLU(g) * u
+    got = oracle.bf16_to_f32(out).astype(np.float64)
+    assert np.max(np.abs(got - want) / (np.abs(want) + 1e-3)) < 2e-2   # two bf16 roundings
