@@ -398,6 +398,51 @@ int32_t qm_predictor_add_postnorm_gate_up_swiglu_m1(
     const uint16_t* gate_weight, const uint16_t* up_weight, uint16_t* output,
     int32_t hidden, int32_t intermediate, void* hip_stream);
 
+/* ---- final head: score processing, top-k sampler, history ------------------------ */
+/*
+ * qm_sample_topk replaces gpu_sample_topk_f32_kernel and gpu_sample_topk_bf16_kernel
+ * (R17:7407-7518; callers NativeFinalHead::run_fast_device :14500-14512 and
+ * PersistentPredictor::capture_step :13814-13833): over the `vocab` scores starting at element
+ * `offset` of `logits` (float, or bf16 bit patterns if logits_are_bf16), ordered by score
+ * descending and id ascending, the first keep = min(top_k, vocab) are sampled with probability
+ * proportional to exp(score / temperature) — sums in double in that order, one SplitMix64 draw
+ * from *rng_state (advanced in place, R17:7353-7371), the first index whose running sum exceeds
+ * uniform * total; without a positive total the first id is returned and nothing is drawn.
+ * top_k <= 0 is the arg-max (argmax_final_head R17:14099-14143, argmax_bf16_kernel): highest
+ * score, lowest id among equals; rng_state may then be NULL.
+ * One block; vocab <= 4096 (the reference's sort size), top_k <= 256 (QM_ERR_GEOMETRY beyond),
+ * temperature > 0.  Same chosen id as the reference for scores without NaN.
+ */
+int32_t qm_sample_topk(
+    const void* logits, int32_t logits_are_bf16, int32_t offset, int32_t vocab,
+    int32_t top_k, float temperature, uint64_t* rng_state, int32_t* output_id,
+    void* hip_stream);
+
+/*
+ * qm_final_head_process = cast_final_head_logits + repetition_penalty + suppress_tokens
+ * (R17:14025-14097) in one launch: scores[t] = f32(logits[t]); a token found in
+ * history[0 .. history_count) is multiplied by `penalty` if negative, else by
+ * float(1) / float(penalty) (the reference's constant 0x3f73cf3e for 1.05); token `eos` is -inf
+ * while generation_index < 2; the last `suppressed_tail` tokens other than eos are -inf.
+ * qm_final_head_sample is the device side of NativeFinalHead::run_fast_device after the head
+ * projection (R17:14456-14545) in one launch instead of five: that processing with
+ * history_count = generation_index, then qm_sample_topk over the processed scores, then
+ * history[generation_index] = code (append_sampled_code_history_kernel R17:7530-7543).
+ * `scores_out` (NULL or [vocab] floats) receives the processed scores.  The head projection
+ * itself is qm_linear_m1 (native_ops::linear_bf16 at one row has the talker linear's order,
+ * R17:126-196).  The reference's constants: vocab 3072, eos 2150, suppressed_tail 1024,
+ * penalty 1.05, top_k 50, temperature 0.9 (R17:13958-13961, 7338-7339).
+ */
+int32_t qm_final_head_process(
+    const uint16_t* logits, const int32_t* history, int32_t history_count, int32_t generation_index,
+    int32_t vocab, int32_t eos, int32_t suppressed_tail, float penalty, float* scores,
+    void* hip_stream);
+int32_t qm_final_head_sample(
+    const uint16_t* logits, int32_t* history, int32_t generation_index,
+    int32_t vocab, int32_t eos, int32_t suppressed_tail, float penalty,
+    int32_t top_k, float temperature, uint64_t* rng_state, int32_t* code_out, float* scores_out,
+    void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -297,6 +297,34 @@ inline void predictor_add_postnorm_m1(
           "predictor add_postnorm_m1 launch");
 }
 
+// The sampler launches of NativeFinalHead::run_fast_device (R17:14500-14526) and
+// PersistentPredictor::capture_step (R17:13814-13843): top-k sampling when `sampling_enabled`
+// (the reference's g_sampling_enabled), else the arg-max kernels.
+inline void sample_topk_f32(const float* logits, int vocab, int top_k, float temperature,
+                            std::uint64_t* rng_state, std::int32_t* output_id, bool sampling_enabled, void* stream) {
+    check(qm_sample_topk(logits, 0, 0, vocab, sampling_enabled ? top_k : 0, temperature, rng_state, output_id, stream),
+          "GPU sampler launch");
+}
+inline void sample_topk_bf16(const std::uint16_t* logits, int last_row_offset, int vocab, int top_k, float temperature,
+                             std::uint64_t* rng_state, std::int32_t* output_id, bool sampling_enabled, void* stream) {
+    check(qm_sample_topk(logits, 1, last_row_offset, vocab, sampling_enabled ? top_k : 0, temperature, rng_state,
+                         output_id, stream),
+          "GPU sampler launch");
+}
+
+// The device side of NativeFinalHead::run_fast_device after the head projection
+// (R17:14456-14545; constants R17:13958-13961, 7338-7339): cast, repetition penalty, suppressed
+// tokens, sampling or arg-max, history append — one launch.  The caller keeps the 4-byte
+// read-back and the stream synchronisation (R17:14548-14562), and throws for a generation
+// index beyond its history capacity as the reference does (R17:14433-14440).
+inline void final_head_sample(const std::uint16_t* logits, std::int32_t* history, int generation_index,
+                              std::uint64_t* rng_state, std::int32_t* code, bool sampling_enabled, void* stream) {
+    if (generation_index < 0) throw std::runtime_error("FinalHead generation index exceeds GPU history capacity");
+    check(qm_final_head_sample(logits, history, generation_index, 3072, 2150, 1024, 1.05f, sampling_enabled ? 50 : 0,
+                               0.9f, rng_state, code, nullptr, stream),
+          "FinalHead sample launch");
+}
+
 }  // namespace qm_attn
 
 #endif  // QM_ATTN_HPP

@@ -232,3 +232,31 @@ def predictor_qkv_m1(x, q_w, k_w, v_w, q_out, k_out, v_out, hidden, q_dim, kv_di
 def predictor_gate_up_swiglu_m1(x, gate_w, up_w, out, hidden, intermediate, threads=8):
     return lib().qmo_predictor_gate_up_swiglu_m1(_p(x), _p(gate_w), _p(up_w), _p(out), C.c_int32(hidden),
                                                  C.c_int32(intermediate), C.c_int32(threads))
+
+
+def splitmix64(state, count):
+    """state: numpy uint64 array of one element (advanced in place); returns (raw uint64[count], uniform f64[count])."""
+    import numpy as np
+    raw = np.zeros(count, dtype=np.uint64)
+    uni = np.zeros(count, dtype=np.float64)
+    assert lib().qmo_splitmix64(_p(state), C.c_int32(count), _p(raw), _p(uni)) == 0
+    return raw, uni
+
+
+def sample_topk(logits, is_bf16, offset, vocab, top_k, temperature, rng_state, output_id):
+    return lib().qmo_sample_topk(_p(logits), C.c_int32(int(is_bf16)), C.c_int32(offset), C.c_int32(vocab),
+                                 C.c_int32(top_k), C.c_float(temperature), _p(rng_state), _p(output_id))
+
+
+def final_head_process(logits, history, history_count, generation_index, vocab, eos, suppressed_tail, penalty, scores):
+    return lib().qmo_final_head_process(_p(logits), _p(history), C.c_int32(history_count),
+                                        C.c_int32(generation_index), C.c_int32(vocab), C.c_int32(eos),
+                                        C.c_int32(suppressed_tail), C.c_float(penalty), _p(scores))
+
+
+def final_head_sample(logits, history, generation_index, vocab, eos, suppressed_tail, penalty, top_k, temperature,
+                      rng_state, code_out, scores_out=None):
+    return lib().qmo_final_head_sample(_p(logits), _p(history), C.c_int32(generation_index), C.c_int32(vocab),
+                                       C.c_int32(eos), C.c_int32(suppressed_tail), C.c_float(penalty),
+                                       C.c_int32(top_k), C.c_float(temperature), _p(rng_state), _p(code_out),
+                                       _p(scores_out))

@@ -878,4 +878,116 @@ int32_t qmo_predictor_gate_up_swiglu_m1(const uint16_t* input, const uint16_t* g
     return QM_OK;
 }
 
+// ---- final head: score processing, top-k sampler, history ---------------------------------------------
+// SplitMix64 and the uniform draw of the sampler (R17:7353-7371).
+static uint64_t splitmix64_next(uint64_t* state) {
+    uint64_t z = *state + 0x9e3779b97f4a7c15ULL;
+    *state = z;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ULL;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebULL;
+    return z ^ (z >> 31);
+}
+
+int32_t qmo_splitmix64(uint64_t* state, int32_t count, uint64_t* raw_out, double* uniform_out) {
+    if (!state) return QM_ERR_NULL;
+    for (int i = 0; i < count; ++i) {
+        const uint64_t z = splitmix64_next(state);
+        if (raw_out) raw_out[i] = z;
+        if (uniform_out) uniform_out[i] = static_cast<double>(z >> 11) * (1.0 / 9007199254740992.0);
+    }
+    return QM_OK;
+}
+
+// gpu_sample_topk_f32_kernel / gpu_sample_topk_bf16_kernel (R17:7407-7518): all scores sorted by
+// (score descending, id ascending) (gpu_sampler_better, R17:7347-7351 — a total order for
+// scores without NaN, so the sorting network's result is the sorted sequence); over the first
+// keep = min(top_k, vocab): maximum = score[0] / T, total = sum of exp(score / T - maximum) in
+// double in that order; without a positive total the first id is returned and no number is
+// drawn; else target = uniform * total and the first index whose running sum exceeds it.
+static int32_t sample_sorted(const float* scores, int vocab, int top_k, float temperature, uint64_t* rng_state) {
+    std::vector<int> order(vocab);
+    for (int i = 0; i < vocab; ++i) order[i] = i;
+    std::sort(order.begin(), order.end(), [&](int a, int b) {
+        return scores[a] > scores[b] || (scores[a] == scores[b] && a < b);
+    });
+    const int keep = top_k < vocab ? top_k : vocab;
+    const double inv_t = 1.0 / static_cast<double>(temperature);
+    const double maximum = static_cast<double>(scores[order[0]]) * inv_t;
+    double total = 0.0;
+    for (int i = 0; i < keep; ++i) total += std::exp(static_cast<double>(scores[order[i]]) * inv_t - maximum);
+    if (!(total > 0.0)) return order[0];
+    const double uniform = static_cast<double>(splitmix64_next(rng_state) >> 11) * (1.0 / 9007199254740992.0);
+    const double target = uniform * total;
+    double cumulative = 0.0;
+    for (int i = 0; i < keep; ++i) {
+        cumulative += std::exp(static_cast<double>(scores[order[i]]) * inv_t - maximum);
+        if (target < cumulative) return order[i];
+    }
+    return order[keep - 1];
+}
+
+// logits: float (is_bf16 == 0) or bf16 bit patterns, read from element `offset` on
+// (last_row_offset of the bf16 kernel).  top_k <= 0 selects the arg-max kernels
+// (argmax_final_head R17:14099-14143, argmax_bf16_kernel: highest score, lowest id among equals).
+int32_t qmo_sample_topk(const void* logits, int32_t is_bf16, int32_t offset, int32_t vocab, int32_t top_k,
+                        float temperature, uint64_t* rng_state, int32_t* output_id) {
+    if (!logits || !output_id) return QM_ERR_NULL;
+    if (vocab <= 0 || offset < 0) return QM_ERR_ARGUMENT;
+    std::vector<float> scores(vocab);
+    for (int i = 0; i < vocab; ++i)
+        scores[i] = is_bf16 ? bf2f(static_cast<const uint16_t*>(logits)[offset + i])
+                            : static_cast<const float*>(logits)[offset + i];
+    if (top_k <= 0) {
+        int best = 0;
+        for (int i = 1; i < vocab; ++i)
+            if (scores[i] > scores[best]) best = i;
+        *output_id = best;
+        return QM_OK;
+    }
+    if (!rng_state) return QM_ERR_NULL;
+    *output_id = sample_sorted(scores.data(), vocab, top_k, temperature, rng_state);
+    return QM_OK;
+}
+
+// cast_final_head_logits, repetition_penalty, suppress_tokens (R17:14025-14097), in that order:
+// score = f32(logit); a token found in history[0 .. history_count) is multiplied by the penalty
+// if negative, else by float(1) / float(penalty) (for 1.05: the constant 0x3f73cf3e, R17:14062);
+// the end-of-sequence token is -inf while generation_index < 2; the last `suppressed_tail`
+// tokens other than it are always -inf.
+int32_t qmo_final_head_process(const uint16_t* logits, const int32_t* history, int32_t history_count,
+                               int32_t generation_index, int32_t vocab, int32_t eos, int32_t suppressed_tail,
+                               float penalty, float* scores) {
+    if (!logits || !scores || (history_count > 0 && !history)) return QM_ERR_NULL;
+    if (vocab <= 0 || history_count < 0) return QM_ERR_ARGUMENT;
+    const float reciprocal = 1.0f / penalty;
+    for (int token = 0; token < vocab; ++token) {
+        float score = bf2f(logits[token]);
+        bool repeated = false;
+        for (int i = 0; i < history_count && !repeated; ++i) repeated = history[i] == token;
+        if (repeated) score = score < 0.0f ? score * penalty : score * reciprocal;
+        if (token == eos && generation_index < 2) score = -INFINITY;
+        if (token >= vocab - suppressed_tail && token != eos) score = -INFINITY;
+        scores[token] = score;
+    }
+    return QM_OK;
+}
+
+// The device side of NativeFinalHead::run_fast_device after the head projection
+// (R17:14456-14545): process, sample (or arg-max when top_k <= 0), append the code to the history.
+int32_t qmo_final_head_sample(const uint16_t* logits, int32_t* history, int32_t generation_index, int32_t vocab,
+                              int32_t eos, int32_t suppressed_tail, float penalty, int32_t top_k,
+                              float temperature, uint64_t* rng_state, int32_t* code_out, float* scores_out) {
+    if (!logits || !history || !code_out) return QM_ERR_NULL;
+    if (generation_index < 0) return QM_ERR_ARGUMENT;
+    std::vector<float> scores(vocab > 0 ? vocab : 1);
+    int32_t rc = qmo_final_head_process(logits, history, generation_index, generation_index, vocab, eos,
+                                        suppressed_tail, penalty, scores.data());
+    if (rc != QM_OK) return rc;
+    if (scores_out) std::memcpy(scores_out, scores.data(), sizeof(float) * vocab);
+    rc = qmo_sample_topk(scores.data(), 0, 0, vocab, top_k, temperature, rng_state, code_out);
+    if (rc != QM_OK) return rc;
+    history[generation_index] = *code_out;
+    return QM_OK;
+}
+
 }  // extern "C"

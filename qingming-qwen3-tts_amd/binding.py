@@ -75,6 +75,9 @@ _SIGNATURES = {
     "qm_predictor_gate_up_swiglu_m1": (_I32, [_PTR] * 4 + [_I32, _I32, _PTR]),
     "qm_predictor_rmsnorm_qkv_m1": (_I32, [_PTR, _PTR, _F32] + [_PTR] * 6 + [_I32, _I32, _I32, _PTR]),
     "qm_predictor_add_postnorm_gate_up_swiglu_m1": (_I32, [_PTR, _PTR, _PTR, _F32] + [_PTR] * 4 + [_I32, _I32, _PTR]),
+    "qm_sample_topk": (_I32, [_PTR, _I32, _I32, _I32, _I32, _F32, _PTR, _PTR, _PTR]),
+    "qm_final_head_process": (_I32, [_PTR, _PTR, _I32, _I32, _I32, _I32, _I32, _F32, _PTR, _PTR]),
+    "qm_final_head_sample": (_I32, [_PTR, _PTR, _I32, _I32, _I32, _I32, _F32, _I32, _F32, _PTR, _PTR, _PTR, _PTR]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
@@ -279,6 +282,24 @@ def predictor_add_postnorm_gate_up_swiglu_m1(hidden_state, attention, norm_weigh
     _check(lib().qm_predictor_add_postnorm_gate_up_swiglu_m1(
         _addr(hidden_state), _addr(attention), _addr(norm_weight), eps, _addr(residual), _addr(gate_w), _addr(up_w),
         _addr(out), hidden, intermediate, stream), "qm_predictor_add_postnorm_gate_up_swiglu_m1")
+
+
+def sample_topk(logits, logits_are_bf16, offset, vocab, top_k, temperature, rng_state, output_id, stream=0):
+    _check(lib().qm_sample_topk(_addr(logits), int(logits_are_bf16), offset, vocab, top_k, temperature,
+                                _addr(rng_state), _addr(output_id), stream), "qm_sample_topk")
+
+
+def final_head_process(logits, history, history_count, generation_index, vocab, eos, suppressed_tail, penalty,
+                       scores, stream=0):
+    _check(lib().qm_final_head_process(_addr(logits), _addr(history), history_count, generation_index, vocab, eos,
+                                       suppressed_tail, penalty, _addr(scores), stream), "qm_final_head_process")
+
+
+def final_head_sample(logits, history, generation_index, vocab, eos, suppressed_tail, penalty, top_k, temperature,
+                      rng_state, code_out, scores_out=None, stream=0):
+    _check(lib().qm_final_head_sample(_addr(logits), _addr(history), generation_index, vocab, eos, suppressed_tail,
+                                      penalty, top_k, temperature, _addr(rng_state), _addr(code_out),
+                                      _addr(scores_out), stream), "qm_final_head_sample")
 
 
 def predictor_attention_staged(query_bhsd, key_cache, value_cache, out, rows, key_length, causal, stream=0):
