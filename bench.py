@@ -395,6 +395,156 @@ class TalkerLayerStep:
         return {"all": dt}, err, "one layer step"
 
 
+class PredictorFrameSteps:
+    """Beyond the five configurations: the fourteen M = 1 steps of one code-predictor frame as the
+    reference chains them (PersistentPredictor::capture_step, R17:13592-13854): input projection,
+    five layers (RMSNorm + Q/K/V, QK-norm + RoPE + append + attention over the [8][16][128] cache,
+    o_proj, residual add + post-norm + gate/up/SwiGLU, down_proj + residual), final norm + that
+    step's head, top-k sampler, embedding gather feeding the next step.  29 launches per step with
+    the fused operators (the reference: 46 graph nodes per M = 1 step).  Geometry R17:7951-7962;
+    weights random.  One `step()` is the whole frame."""
+    bound = "hbm"
+    name = "predictor_frame_14_m1_steps_5layers"
+    tolerance = 0.125
+
+    def __init__(self, qm, dev, seed=77):
+        import torch
+        self.qm, self.dev = qm, dev
+        gd = torch.Generator(device=dev).manual_seed(seed)
+        H, Q, KV, I, OUT, V = 1024, 2048, 1024, 3072, 2048, 2048
+        self.dims = (H, Q, KV, I, OUT, V)
+
+        def rnd(shape, std=1.0, mean=0.0):
+            return (torch.randn(shape, generator=gd, device=dev, dtype=torch.float32) * std + mean).to(torch.bfloat16)
+
+        self.proj_w, self.proj_b = rnd((H, OUT), 0.02), rnd((H,), 0.1)
+        self.layers = []
+        for _ in range(5):
+            k, v = rnd((8, 16, 128)), rnd((8, 16, 128))
+            self.layers.append(dict(
+                in_norm=rnd((H,), 0.1, 1.0), wq=rnd((Q, H), 0.03), wk=rnd((KV, H), 0.03), wv=rnd((KV, H), 0.03),
+                gq=rnd((128,), 0.1, 1.0), gk=rnd((128,), 0.1, 1.0), wo=rnd((H, Q), 0.02), post=rnd((H,), 0.1, 1.0),
+                wg=rnd((I, H), 0.03), wu=rnd((I, H), 0.03), wd=rnd((H, I), 0.02), k=k, v=v, k0=k.clone(), v0=v.clone(),
+                cache=qm.flat_cache(k, v, 8, 16)))
+        self.final_norm = rnd((H,), 0.1, 1.0)
+        self.heads = [rnd((V, H), 0.05) for _ in range(14)]
+        self.tables = [rnd((V, OUT)) for _ in range(14)]
+        inv = 1.0e6 ** (-2.0 * np.arange(64, dtype=np.float64) / 128.0)
+        ang = np.arange(16, dtype=np.float64)[:, None] * np.concatenate([inv, inv])[None, :]
+        self.cos = torch.tensor(np.cos(ang), dtype=torch.float32).to(torch.bfloat16).to(dev)
+        self.sin = torch.tensor(np.sin(ang), dtype=torch.float32).to(torch.bfloat16).to(dev)
+        z = lambda n: torch.zeros(n, dtype=torch.bfloat16, device=dev)
+        self.input0 = rnd((OUT,))
+        self.free_input = self.input0.clone()
+        self.hidden = [z(H), z(H)]
+        self.q, self.k_, self.v_, self.qrot, self.ctxv = z(Q), z(KV), z(KV), z(Q), z(Q)
+        self.attn, self.res, self.act, self.logits = z(H), z(H), z(I), z(V)
+        self.first_logits = z(V)
+        self.selected = torch.zeros((16, OUT), dtype=torch.bfloat16, device=dev)
+        self.codes = torch.zeros(16, dtype=torch.int32, device=dev)
+        self.rng = torch.tensor([20240229], dtype=torch.int64, device=dev)
+        self.ws_bytes = qm.decode_workspace_bytes(1, 16, 8, 16)
+        self.ws = torch.empty(self.ws_bytes // 4 + 1, dtype=torch.float32, device=dev)
+        layer_w = 2 * (Q * H + 2 * KV * H + H * Q + 2 * I * H + H * I)
+        self.launches_per_step = 1 + 5 * 5 + 3
+        self.bytes = 14 * (5 * layer_w + 2 * H * OUT + 2 * V * H + 2 * OUT)          # weights streamed once per step
+        self.flops = self.bytes
+        self.copies = 14
+
+    def one_step(self, step, s):
+        qm = self.qm
+        H, Q, KV, I, OUT, V = self.dims
+        position = step + 1                      # cache_before of an M = 1 step (R17:13594-13596)
+        cur, nxt = self.hidden
+        qm.linear_m1(self.free_input, self.proj_w, self.proj_b, None, cur, H, OUT, s)
+        for L in self.layers:
+            qm.predictor_rmsnorm_qkv_m1(cur, L["in_norm"], L["wq"], L["wk"], L["wv"], self.q, self.k_, self.v_, H, Q, KV,
+                                        1e-6, s)
+            qm.decode_step_fused(self.q, self.k_, self.v_, L["gq"], L["gk"], self.cos[position], self.sin[position],
+                                 self.qrot, L["cache"], None, 1, self.ctxv, 16, position, -1, SCALE, 1e-6, self.ws,
+                                 self.ws_bytes, None, s)
+            qm.predictor_linear_m1(self.ctxv, L["wo"], None, self.attn, H, Q, s)
+            qm.predictor_add_postnorm_gate_up_swiglu_m1(cur, self.attn, L["post"], self.res, L["wg"], L["wu"], self.act,
+                                                        H, I, 1e-6, s)
+            qm.predictor_linear_m1(self.act, L["wd"], self.res, nxt, H, I, s)
+            cur, nxt = nxt, cur
+        head = self.heads[step - 1]
+        # final RMSNorm + this step's head (the talker linear's order, no bias): the fused Q/K/V entry with no K/V rows
+        qm.rmsnorm_qkv_m1(cur, self.final_norm, head, None, head, None, head, None, self.logits, self.logits,
+                          self.logits, H, V, 0, 1e-6, s)
+        qm.sample_topk(self.logits, True, 0, V, 50, 0.9, self.rng, self.codes[step + 1:], s)
+        qm.gather_embedding(self.tables[step - 1], V, self.codes, step + 1, OUT, self.selected, self.free_input, s)
+
+    def step(self):
+        import torch
+        s = torch.cuda.current_stream().cuda_stream
+        for step in range(1, 15):
+            self.one_step(step, s)
+
+    def reset(self):
+        self.free_input.copy_(self.input0)
+        self.rng.fill_(20240229)
+        self.codes.zero_()
+        for L in self.layers:
+            L["k"].copy_(L["k0"])
+            L["v"].copy_(L["v0"])
+
+    def cpu_baseline(self, oracle, threads):
+        """The whole frame on the host from the same start state: the fourteen sampled codes."""
+        import torch
+        self.reset()
+        self.step()
+        torch.cuda.synchronize()
+        gpu_codes = self.codes.cpu().numpy().copy()
+        H, Q, KV, I, OUT, V = self.dims
+        u16 = lambda n: np.zeros(n, dtype=np.uint16)
+        B = lambda t: _bits(t).copy()
+        layers = [{k: (B(v) if hasattr(v, "detach") else v) for k, v in L.items() if k != "cache"} for L in self.layers]
+        for L in layers:
+            L["k"], L["v"] = L["k0"].copy(), L["v0"].copy()
+        cos, sin = B(self.cos), B(self.sin)
+        free_input = B(self.input0)
+        rng = np.array([20240229], dtype=np.uint64)
+        codes = np.zeros(16, dtype=np.int32)
+        proj_w, proj_b, final_norm = B(self.proj_w), B(self.proj_b), B(self.final_norm)
+        t0 = time.perf_counter()
+        worst = 0.0
+        for step in range(1, 15):
+            position = step + 1
+            cur = u16(H)
+            assert oracle.linear_m1(free_input, proj_w, proj_b, None, cur, H, OUT, threads) == 0
+            for L in layers:
+                norm, q, k, v, qrot, ctxv, attn, res, post, act, nxt = (u16(H).reshape(1, H), u16(Q), u16(KV), u16(KV),
+                                                                        u16(Q), u16(Q), u16(H), u16(H), u16(H), u16(I),
+                                                                        u16(H))
+                cache = oracle.flat_cache(L["k"], L["v"], 8, 16)
+                assert oracle.rmsnorm_rows(cur.reshape(1, H), L["in_norm"], norm, 1, H) == 0
+                assert oracle.predictor_qkv_m1(norm[0], L["wq"], L["wk"], L["wv"], q, k, v, H, Q, KV, threads) == 0
+                assert oracle.qk_norm_rope_kv_append(q, k, v, L["gq"], L["gk"], cos[position], sin[position], qrot, cache,
+                                                     None, 1, 16, position) == 0
+                assert oracle.attention(qrot, cache, None, 1, ctxv, 1, position, 16, -1, SCALE, oracle.POLICY_ONLINE,
+                                        threads) == 0
+                assert oracle.predictor_linear_m1(ctxv, L["wo"], None, attn, H, Q, threads) == 0
+                assert oracle.add_postnorm_m1(cur, attn, L["post"], res, post, H) == 0
+                assert oracle.predictor_gate_up_swiglu_m1(post, L["wg"], L["wu"], act, H, I, threads) == 0
+                assert oracle.predictor_linear_m1(act, L["wd"], res, nxt, H, I, threads) == 0
+                cur = nxt
+            fin, logits = u16(H).reshape(1, H), u16(V)
+            assert oracle.rmsnorm_rows(cur.reshape(1, H), final_norm, fin, 1, H) == 0
+            assert oracle.linear_m1(fin[0], B(self.heads[step - 1]), None, None, logits, V, H, threads) == 0
+            if step == 14:
+                worst = float(np.max(np.abs(oracle.bf16_to_f32(logits).astype(np.float64)
+                                            - oracle.bf16_to_f32(_bits(self.logits)).astype(np.float64))))
+            out = np.zeros(1, dtype=np.int32)
+            assert oracle.sample_topk(logits, True, 0, V, 50, 0.9, rng, out) == 0
+            codes[step + 1] = out[0]
+            free_input = B(self.tables[step - 1])[out[0]].copy()
+        dt = time.perf_counter() - t0
+        self.codes_match = bool(np.array_equal(codes, gpu_codes))
+        # a code that differs redirects every later step: the logits of the last step are compared only then
+        return {"all": dt}, (worst if self.codes_match else 1.0e9), "one frame (14 steps); all sampled codes equal"
+
+
 class Prefill:
     """configs[3]: causal GQA prefill, batch 4 x seq 1024, K/V also written to shuffled 16-token pages."""
     name = "causal_prefill_b4_s1024_paged16"
@@ -510,7 +660,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
-    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "predictor", "qkv", "layer"], default=None,
+    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "predictor", "qkv", "layer", "frame"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -544,7 +694,8 @@ def main():
         make = {"decode512": lambda: SingleDecode(qm, dev, 512, False, 11),
                 "talker2048": lambda: SingleDecode(qm, dev, 2048, True, 12),
                 "prefill": lambda: Prefill(qm, dev), "predictor": lambda: PredictorLoop(qm, dev),
-                "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev)}[args.only]
+                "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev),
+                "frame": lambda: PredictorFrameSteps(qm, dev)}[args.only]
         w = make()
         r = _report(w, _time_steps(w.step, args.steps, args.warmup))
         r["bound"] = w.bound
@@ -582,12 +733,15 @@ def main():
             # the whole decode step of one talker layer, 28 layers' weights and caches in rotation (2.8 GB)
             ("next_talker_layer_decode_step", lambda: TalkerLayerStep(qm, dev)),
             ("next_talker_layer_decode_step_unfused", lambda: TalkerLayerStep(qm, dev, fused=False)),
+            # the fourteen M = 1 steps of one code-predictor frame, operator by operator (406 launches)
+            ("next_predictor_frame_m1_steps", lambda: PredictorFrameSteps(qm, dev)),
         ]
         for key, make in extra:
             w = make()
             r = _report(w, _time_steps(w.step, max(args.steps, 100), max(args.warmup, 10)))
             copies = getattr(w, "copies", 1)
-            r["us_per_step_graph"] = _time_graph(w.step, reps=64 if copies > 1 else 20) * 1e3
+            r["us_per_step_graph"] = _time_graph(w.step, reps=2 if isinstance(w, PredictorFrameSteps) else
+                                                 64 if copies > 1 else 20) * 1e3
             r["GBps_graph"] = w.bytes / (r["us_per_step_graph"] * 1e-6) / 1e9
             r["TFLOPps_graph"] = w.flops / (r["us_per_step_graph"] * 1e-6) / 1e12
             r["bound"] = w.bound
@@ -595,8 +749,12 @@ def main():
             if isinstance(w, PredictorLoop):
                 r["us_per_predictor_step"] = r["us_per_step_graph"] / w.rows
                 r["us_per_frame"] = r["us_per_step_graph"] / w.frames
+            if isinstance(w, PredictorFrameSteps):
+                r["us_per_frame"] = r["us_per_step_graph"]
+                r["us_per_predictor_step"] = r["us_per_step_graph"] / 14
+                r["launches_per_predictor_step"] = w.launches_per_step
             if oracle is not None and not (isinstance(w, PredictorLoop) and w.kc is not None) \
-                    and (copies == 1 or isinstance(w, TalkerLayerStep)):
+                    and (copies == 1 or isinstance(w, (TalkerLayerStep, PredictorFrameSteps))):
                 res, err, sample = w.cpu_baseline(oracle, threads)
                 if err > getattr(w, "tolerance", 1e-2):
                     raise RuntimeError(f"{key}: GPU result differs from the oracle: max abs err {err}")

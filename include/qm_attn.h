@@ -443,6 +443,17 @@ int32_t qm_final_head_sample(
     int32_t top_k, float temperature, uint64_t* rng_state, int32_t* code_out, float* scores_out,
     void* hip_stream);
 
+/*
+ * Replaces gather_predictor_embedding_kernel (R17:11998-12030; launched in
+ * PersistentPredictor::capture_step :13845-13853): with token = codes[group],
+ * selected_embeddings[group][d] = next_step_input[d] = table[token][d] for d < dimension
+ * (the reference's kOuterHidden = 2048).  A token outside [0, table_rows) moves nothing
+ * (the reference has no such guard).
+ */
+int32_t qm_gather_embedding(
+    const uint16_t* table, int32_t table_rows, const int32_t* codes, int32_t group, int32_t dimension,
+    uint16_t* selected_embeddings, uint16_t* next_step_input, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -78,6 +78,7 @@ _SIGNATURES = {
     "qm_sample_topk": (_I32, [_PTR, _I32, _I32, _I32, _I32, _F32, _PTR, _PTR, _PTR]),
     "qm_final_head_process": (_I32, [_PTR, _PTR, _I32, _I32, _I32, _I32, _I32, _F32, _PTR, _PTR]),
     "qm_final_head_sample": (_I32, [_PTR, _PTR, _I32, _I32, _I32, _I32, _F32, _I32, _F32, _PTR, _PTR, _PTR, _PTR]),
+    "qm_gather_embedding": (_I32, [_PTR, _I32, _PTR, _I32, _I32, _PTR, _PTR, _PTR]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
@@ -300,6 +301,11 @@ def final_head_sample(logits, history, generation_index, vocab, eos, suppressed_
     _check(lib().qm_final_head_sample(_addr(logits), _addr(history), generation_index, vocab, eos, suppressed_tail,
                                       penalty, top_k, temperature, _addr(rng_state), _addr(code_out),
                                       _addr(scores_out), stream), "qm_final_head_sample")
+
+
+def gather_embedding(table, table_rows, codes, group, dimension, selected, next_input, stream=0):
+    _check(lib().qm_gather_embedding(_addr(table), table_rows, _addr(codes), group, dimension, _addr(selected),
+                                     _addr(next_input), stream), "qm_gather_embedding")
 
 
 def predictor_attention_staged(query_bhsd, key_cache, value_cache, out, rows, key_length, causal, stream=0):

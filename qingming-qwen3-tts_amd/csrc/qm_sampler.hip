@@ -80,7 +80,8 @@ __global__ __launch_bounds__(kSmpThreads) void sampler_kernel(SamplerParams prm)
     __shared__ int sh_digit, sh_remaining, sh_count;
     __shared__ unsigned long long sh_cand[kSmpMaxKeep];
     __shared__ unsigned long long sh_sorted[kSmpMaxKeep];
-    __shared__ double sh_exp[kSmpMaxKeep];
+    __shared__ double sh_exp[kSmpMaxKeep];                // the terms, then their running sums
+    __shared__ double sh_target;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -186,28 +187,55 @@ __global__ __launch_bounds__(kSmpThreads) void sampler_kernel(SamplerParams prm)
         sh_exp[tid] = exp(value * inv_t - maximum);
     }
     __syncthreads();
-    if (tid != 0) return;
     auto id_of = [&](int i) { return static_cast<int32_t>(0xffffffffU - static_cast<uint32_t>(sh_sorted[i])); };
-    int32_t chosen = id_of(0);
-    if (prm.top_k > 0) {
-        double total = 0.0;
-        for (int i = 0; i < keep; ++i) total += sh_exp[i];
-        if (total > 0.0) {
-            const double uniform = static_cast<double>(splitmix64_next(prm.rng_state) >> 11) * (1.0 / 9007199254740992.0);
-            const double target = uniform * total;
-            double cumulative = 0.0;
-            chosen = id_of(keep - 1);
-            for (int i = 0; i < keep; ++i) {
-                cumulative += sh_exp[i];
-                if (target < cumulative) {
-                    chosen = id_of(i);
-                    break;
+    // The running sums, added by one thread in the reference's order (its second loop repeats
+    // the partial sums of its first: one pass serves both); the terms are fetched eight at a
+    // time so that the chain waits for additions, not for LDS.
+    if (prm.top_k > 0 && tid == 0) {
+        double running = 0.0;
+        for (int i0 = 0; i0 < keep; i0 += 8) {
+            double term[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) term[u] = i0 + u < keep ? sh_exp[i0 + u] : 0.0;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (i0 + u < keep) {
+                    running += term[u];
+                    sh_exp[i0 + u] = running;
                 }
             }
         }
+        const double total = running;
+        sh_count = -1;                                     // no draw
+        if (total > 0.0) {
+            const double uniform = static_cast<double>(splitmix64_next(prm.rng_state) >> 11) * (1.0 / 9007199254740992.0);
+            sh_target = uniform * total;
+            sh_count = keep - 1;                           // the answer if no running sum exceeds the target
+        }
     }
+    __syncthreads();
+    // first index whose running sum exceeds the target: the smallest such index over all threads
+    if (prm.top_k > 0 && sh_count >= 0 && tid < keep && sh_target < sh_exp[tid]) atomicMin(&sh_count, tid);
+    __syncthreads();
+    if (tid != 0) return;
+    int32_t chosen = id_of(0);
+    if (prm.top_k > 0 && sh_count >= 0) chosen = id_of(sh_count);
     prm.output_id[0] = chosen;
     if (prm.history && prm.append_index >= 0) prm.history[prm.append_index] = chosen;
+}
+
+// gather_predictor_embedding_kernel (R17:11998-12030): the embedding row of the code just sampled
+// becomes the next step's input and is kept for the frame's sum.  A code outside the table
+// (which the reference would read out of bounds) moves nothing.
+__global__ void gather_embedding_kernel(const uint16_t* table, int table_rows, const int32_t* codes, int group,
+                                        int dimension, uint16_t* selected, uint16_t* next_input) {
+    const int d = static_cast<int>(blockIdx.x) * static_cast<int>(blockDim.x) + static_cast<int>(threadIdx.x);
+    if (d >= dimension) return;
+    const int token = codes[group];
+    if (token < 0 || token >= table_rows) return;
+    const uint16_t value = table[static_cast<int64_t>(token) * dimension + d];
+    selected[static_cast<int64_t>(group) * dimension + d] = value;
+    next_input[d] = value;
 }
 
 inline int32_t launch_sampler(const SamplerParams& prm, void* hip_stream) {
@@ -268,4 +296,15 @@ extern "C" int32_t qm_final_head_sample(const uint16_t* logits, int32_t* history
     prm.penalty = penalty; prm.reciprocal = 1.0f / penalty;
     prm.scores_out = scores_out;
     return launch_sampler(prm, hip_stream);
+}
+
+extern "C" int32_t qm_gather_embedding(const uint16_t* table, int32_t table_rows, const int32_t* codes, int32_t group,
+                                       int32_t dimension, uint16_t* selected_embeddings, uint16_t* next_step_input,
+                                       void* hip_stream) {
+    if (!table || !codes || !selected_embeddings || !next_step_input) return QM_ERR_NULL;
+    if (table_rows <= 0 || group < 0 || dimension <= 0) return QM_ERR_ARGUMENT;
+    hipLaunchKernelGGL(qm::gather_embedding_kernel, dim3(static_cast<unsigned>((dimension + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(hip_stream), table, table_rows, codes, group, dimension,
+                       selected_embeddings, next_step_input);
+    return qm::launch_status();
 }
