@@ -13,6 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libqm_attn.so")
+ENGINE_LIB_PATH = os.path.join(LIB_DIR, "libqm_engine.so")
 
 SOURCES = ["qm_lib.hip", "qm_norm_rope.hip", "qm_decode.hip", "qm_prefill.hip", "qm_predictor.hip", "qm_linear.hip", "qm_rmsnorm.hip", "qm_sampler.hip"]
 
@@ -41,7 +42,29 @@ def build(verbose=True, jobs=4):
     if verbose:
         print(" ".join(link), flush=True)
     subprocess.run(link, check=True)
+    build_engine(verbose)
     return LIB_PATH
+
+
+ENGINE_SOURCES = ["engine/qm_safetensors.cpp", "engine/qm_engine.cpp"]
+
+
+def build_engine(verbose=True):
+    """libqm_engine.so: the host-side engine shell (C++ over the HIP runtime and libqm_attn.so, found
+    next to it through an $ORIGIN run path)."""
+    cmd = ["hipcc", "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
+           "-Wno-unused-parameter", "-o", ENGINE_LIB_PATH,
+           *[os.path.join(CSRC, src) for src in ENGINE_SOURCES],
+           "-L" + LIB_DIR, "-lqm_attn", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(line for line in p.stdout.splitlines() if "packed-fp32-ops" not in line and line.strip())
+    if verbose and out:
+        print(out, flush=True)
+    if p.returncode != 0:
+        raise RuntimeError(f"hipcc failed on the engine library:\n{out}")
+    return ENGINE_LIB_PATH
 
 
 def _drain(procs, verbose):

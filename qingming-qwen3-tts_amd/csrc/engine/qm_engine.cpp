@@ -1,0 +1,407 @@
+// qm_engine.cpp — host-side engine shell: talker weights from safetensors, per-layer KV caches,
+// the decode layer loop over the C-ABI operators of libqm_attn, RoPE rows, trajectory hash.
+//
+// Reference: TalkerWeights (R17:14710-15021), NativeTalkerEngine (buffers R17:16392-16470, request
+// reset :16526-16546, decode_device :17097-17262), make_talker_rope (R17:21576-21590), fnv1a64
+// (R17:833-842).  The decode step enqueues five launches per layer where the reference enqueues
+// eight (the fused operators give the same bits) and nothing else: no allocation, no
+// synchronisation, no host read.
+#include "../../../include/qm_engine.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstring>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "../../../include/qm_attn.h"
+#include "qm_safetensors.hpp"
+
+namespace qm_engine {
+
+constexpr int kHidden = 2048;          // R17:14625
+constexpr int kHeadDim = 128;          // kHeadDimRequired, R17:14629
+constexpr float kEpsilon = 1.0e-6f;    // kRmsEpsilon, R17:7965
+constexpr float kScale = 0.08838834764831845f;   // 1 / sqrt(128), R17:7966
+
+struct ApiError : std::runtime_error {
+    int32_t code;
+    ApiError(int32_t c, const std::string& what) : std::runtime_error(what), code(c) {}
+};
+
+thread_local std::string g_last_error;
+
+inline void hip_check(hipError_t e, const char* what) {
+    if (e != hipSuccess) throw ApiError(QM_ERR_HIP_BASE - static_cast<int32_t>(e), std::string(what) + ": " + hipGetErrorString(e));
+}
+inline void op_check(int32_t rc, const char* what) {
+    if (rc != QM_OK) throw ApiError(rc, std::string(what) + ": " + qm_error_string(rc));
+}
+
+// Owner of one device allocation (DeviceBuffer, R17:7968-8020).
+class DeviceBuffer {
+public:
+    DeviceBuffer() = default;
+    explicit DeviceBuffer(size_t bytes) : bytes_(bytes) {
+        if (bytes) hip_check(hipMalloc(&pointer_, bytes), "device allocation");
+    }
+    ~DeviceBuffer() {
+        if (pointer_) (void)hipFree(pointer_);
+    }
+    DeviceBuffer(DeviceBuffer&& o) noexcept : pointer_(o.pointer_), bytes_(o.bytes_) { o.pointer_ = nullptr; o.bytes_ = 0; }
+    DeviceBuffer& operator=(DeviceBuffer&& o) noexcept {
+        if (this != &o) {
+            if (pointer_) (void)hipFree(pointer_);
+            pointer_ = o.pointer_; bytes_ = o.bytes_;
+            o.pointer_ = nullptr; o.bytes_ = 0;
+        }
+        return *this;
+    }
+    DeviceBuffer(const DeviceBuffer&) = delete;
+    DeviceBuffer& operator=(const DeviceBuffer&) = delete;
+    uint16_t* u16() const { return static_cast<uint16_t*>(pointer_); }
+    void* raw() const { return pointer_; }
+    size_t bytes() const { return bytes_; }
+
+private:
+    void* pointer_ = nullptr;
+    size_t bytes_ = 0;
+};
+
+// A BF16 tensor on the device (GpuParam, R17:14639-14683); absent optional tensors give nullptr.
+struct Param {
+    DeviceBuffer buffer;
+    std::vector<int64_t> shape;
+    bool present = false;
+    Param() = default;
+    Param(const TensorView& t, hipStream_t upload) : buffer(static_cast<size_t>(t.elements()) * 2), shape(t.shape), present(true) {
+        if (t.dtype != "BF16") throw TensorError("expected BF16 tensor: " + t.name);
+        hip_check(hipMemcpyAsync(buffer.raw(), t.data, buffer.bytes(), hipMemcpyHostToDevice, upload), "weight upload");
+    }
+    const uint16_t* data() const { return present ? buffer.u16() : nullptr; }
+};
+
+struct Layer {
+    Param input_norm, q_weight, q_bias, k_weight, k_bias, v_weight, v_bias, q_norm, k_norm, o_weight, o_bias, post_norm,
+        gate_weight, up_weight, down_weight;
+    DeviceBuffer key_cache, value_cache;
+};
+
+}  // namespace qm_engine
+
+struct qm_safefile {
+    qm_engine::SafeFile file;
+    std::vector<const qm_engine::TensorView*> order;
+    explicit qm_safefile(const std::string& path) : file(path) {
+        for (const auto& kv : file.tensors()) order.push_back(&kv.second);
+    }
+};
+
+struct qm_talker {
+    std::vector<qm_engine::Layer> layers;
+    qm_engine::Param final_norm;
+    int q_heads = 0, kv_heads = 0, q_dim = 0, kv_dim = 0, intermediate = 0, max_cache = 0, prefill_length = 0;
+    hipStream_t stream = nullptr;
+    bool own_stream = false;
+    qm_engine::DeviceBuffer hidden_a, hidden_b, q, k, v, q_rotated, context, attention, residual, swiglu, final_hidden,
+        cosine, sine, workspace;
+
+    ~qm_talker() {
+        if (own_stream && stream) (void)hipStreamDestroy(stream);
+    }
+};
+
+namespace qm_engine {
+
+static std::string layer_name(int layer, const char* tail) {      // layer_suffix, R17:14633-14638
+    return "talker.model.layers." + std::to_string(layer) + "." + tail;
+}
+
+static void check_layer(int index, const Layer& w) {               // validate_layer, R17:14968-15008
+    const std::vector<int64_t> hidden{kHidden};
+    auto rank2 = [](const Param& p) { return p.shape.size() == 2; };
+    if (w.input_norm.shape != hidden || w.post_norm.shape != hidden || !rank2(w.q_weight) || !rank2(w.k_weight)
+        || !rank2(w.v_weight) || !rank2(w.o_weight) || !rank2(w.gate_weight) || !rank2(w.up_weight) || !rank2(w.down_weight))
+        throw TensorError("talker layer geometry/rank mismatch at layer " + std::to_string(index));
+    if (w.q_weight.shape[1] != kHidden || w.k_weight.shape[1] != kHidden || w.v_weight.shape[1] != kHidden
+        || w.o_weight.shape[0] != kHidden || w.o_weight.shape[1] != w.q_weight.shape[0]
+        || w.k_weight.shape[0] != w.v_weight.shape[0] || w.gate_weight.shape[1] != kHidden
+        || w.up_weight.shape != w.gate_weight.shape || w.down_weight.shape[0] != kHidden
+        || w.down_weight.shape[1] != w.gate_weight.shape[0])
+        throw TensorError("talker projection geometry mismatch at layer " + std::to_string(index));
+    auto bias_ok = [](const Param& bias, const Param& weight) {
+        return !bias.present || (bias.shape.size() == 1 && bias.shape[0] == weight.shape[0]);
+    };
+    if (!bias_ok(w.q_bias, w.q_weight) || !bias_ok(w.k_bias, w.k_weight) || !bias_ok(w.v_bias, w.v_weight)
+        || !bias_ok(w.o_bias, w.o_weight) || w.q_norm.shape != std::vector<int64_t>{kHeadDim}
+        || w.k_norm.shape != std::vector<int64_t>{kHeadDim})
+        throw TensorError("talker bias/norm geometry mismatch at layer " + std::to_string(index));
+}
+
+static std::unique_ptr<qm_talker> create_talker(const std::string& model_dir, int max_cache, hipStream_t stream) {
+    if (max_cache <= 0) throw ApiError(QM_ERR_ARGUMENT, "max_cache must be positive");
+    ModelDirectory host(model_dir);
+    auto engine = std::make_unique<qm_talker>();
+    engine->stream = stream;
+    if (!stream) {
+        hip_check(hipStreamCreateWithFlags(&engine->stream, hipStreamNonBlocking), "generation stream");
+        engine->own_stream = true;
+    }
+    hipStream_t upload = engine->stream;
+    auto optional = [&](const std::string& name) {
+        const TensorView* t = host.maybe_suffix(name);
+        return t ? Param(*t, upload) : Param();
+    };
+    for (int index = 0;; ++index) {
+        const TensorView* input_norm = host.maybe_suffix(layer_name(index, "input_layernorm.weight"));
+        if (!input_norm) break;
+        Layer w;
+        w.input_norm = Param(*input_norm, upload);
+        w.q_weight = Param(host.suffix(layer_name(index, "self_attn.q_proj.weight")), upload);
+        w.q_bias = optional(layer_name(index, "self_attn.q_proj.bias"));
+        w.k_weight = Param(host.suffix(layer_name(index, "self_attn.k_proj.weight")), upload);
+        w.k_bias = optional(layer_name(index, "self_attn.k_proj.bias"));
+        w.v_weight = Param(host.suffix(layer_name(index, "self_attn.v_proj.weight")), upload);
+        w.v_bias = optional(layer_name(index, "self_attn.v_proj.bias"));
+        w.q_norm = Param(host.suffix(layer_name(index, "self_attn.q_norm.weight")), upload);
+        w.k_norm = Param(host.suffix(layer_name(index, "self_attn.k_norm.weight")), upload);
+        w.o_weight = Param(host.suffix(layer_name(index, "self_attn.o_proj.weight")), upload);
+        w.o_bias = optional(layer_name(index, "self_attn.o_proj.bias"));
+        w.post_norm = Param(host.suffix(layer_name(index, "post_attention_layernorm.weight")), upload);
+        w.gate_weight = Param(host.suffix(layer_name(index, "mlp.gate_proj.weight")), upload);
+        w.up_weight = Param(host.suffix(layer_name(index, "mlp.up_proj.weight")), upload);
+        w.down_weight = Param(host.suffix(layer_name(index, "mlp.down_proj.weight")), upload);
+        check_layer(index, w);
+        engine->layers.push_back(std::move(w));
+    }
+    if (engine->layers.empty()) throw TensorError("no talker transformer layers in " + model_dir);
+    engine->final_norm = Param(host.suffix("talker.model.norm.weight"), upload);
+    if (engine->final_norm.shape != std::vector<int64_t>{kHidden}) throw TensorError("talker final norm geometry mismatch");
+
+    const Layer& first = engine->layers.front();
+    engine->q_dim = static_cast<int>(first.q_weight.shape[0]);
+    engine->kv_dim = static_cast<int>(first.k_weight.shape[0]);
+    engine->intermediate = static_cast<int>(first.gate_weight.shape[0]);
+    if (engine->q_dim % kHeadDim || engine->kv_dim % kHeadDim) throw TensorError("invalid talker attention geometry");
+    engine->q_heads = engine->q_dim / kHeadDim;
+    engine->kv_heads = engine->kv_dim / kHeadDim;
+    if (engine->q_heads <= 0 || engine->kv_heads <= 0 || engine->q_heads != 2 * engine->kv_heads)
+        throw TensorError("the attention kernels need q_heads == 2 * kv_heads with head_dim 128");
+    for (size_t i = 1; i < engine->layers.size(); ++i) {
+        const Layer& w = engine->layers[i];
+        if (w.q_weight.shape != first.q_weight.shape || w.k_weight.shape != first.k_weight.shape
+            || w.gate_weight.shape != first.gate_weight.shape)
+            throw TensorError("talker layers differ in geometry at layer " + std::to_string(i));
+    }
+
+    engine->max_cache = max_cache;
+    const size_t cache_bytes = static_cast<size_t>(engine->kv_heads) * max_cache * kHeadDim * 2;
+    for (Layer& w : engine->layers) {
+        w.key_cache = DeviceBuffer(cache_bytes);
+        w.value_cache = DeviceBuffer(cache_bytes);
+    }
+    auto vec = [](int n) { return DeviceBuffer(static_cast<size_t>(n) * 2); };
+    engine->hidden_a = vec(kHidden); engine->hidden_b = vec(kHidden);
+    engine->q = vec(engine->q_dim); engine->k = vec(engine->kv_dim); engine->v = vec(engine->kv_dim);
+    engine->q_rotated = vec(engine->q_dim); engine->context = vec(engine->q_dim);
+    engine->attention = vec(kHidden); engine->residual = vec(kHidden);
+    engine->swiglu = vec(engine->intermediate); engine->final_hidden = vec(kHidden);
+    engine->cosine = vec(kHeadDim); engine->sine = vec(kHeadDim);
+    engine->workspace = DeviceBuffer(qm_decode_workspace_bytes(1, engine->q_heads, engine->kv_heads, max_cache));
+    hip_check(hipStreamSynchronize(upload), "weight upload synchronize");   // the mapped files go away with `host`
+    return engine;
+}
+
+static void reset_talker(qm_talker& e, int prefill_length) {
+    if (prefill_length < 0 || prefill_length > e.max_cache) throw ApiError(QM_ERR_SLOT_RANGE, "prefill length exceeds the cache");
+    for (Layer& w : e.layers) {
+        hip_check(hipMemsetAsync(w.key_cache.raw(), 0, w.key_cache.bytes(), e.stream), "key cache reset");
+        hip_check(hipMemsetAsync(w.value_cache.raw(), 0, w.value_cache.bytes(), e.stream), "value cache reset");
+    }
+    e.prefill_length = prefill_length;
+}
+
+static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const uint16_t* cosine, const uint16_t* sine,
+                              int decode_index) {
+    if (!input_device || !cosine || !sine) throw ApiError(QM_ERR_NULL, "talker device decode input is null");
+    if (decode_index < 0) throw ApiError(QM_ERR_ARGUMENT, "negative decode index");
+    const int position = e.prefill_length + decode_index;
+    if (position >= e.max_cache) throw ApiError(QM_ERR_SLOT_RANGE, "talker device decode cache overflow");
+    hipStream_t s = e.stream;
+    hip_check(hipMemcpyAsync(e.hidden_a.raw(), input_device, kHidden * 2, hipMemcpyDeviceToDevice, s), "decode input copy");
+    hip_check(hipMemcpyAsync(e.cosine.raw(), cosine, kHeadDim * 2, hipMemcpyHostToDevice, s), "decode cosine");
+    hip_check(hipMemcpyAsync(e.sine.raw(), sine, kHeadDim * 2, hipMemcpyHostToDevice, s), "decode sine");
+    DeviceBuffer* current = &e.hidden_a;
+    DeviceBuffer* next = &e.hidden_b;
+    for (Layer& w : e.layers) {
+        qm_kv_cache cache = {};
+        cache.k_pool = w.key_cache.u16();
+        cache.v_pool = w.value_cache.u16();
+        cache.stride_page = 0;
+        cache.stride_head = static_cast<int64_t>(e.max_cache) * kHeadDim;
+        cache.stride_token = kHeadDim;
+        cache.page_size = e.max_cache;
+        cache.n_pages = 1;
+        cache.kv_heads = e.kv_heads;
+        cache.head_dim = kHeadDim;
+        // launch_rmsnorm + launch_qkv_m1 (R17:17163-17176)
+        op_check(qm_rmsnorm_qkv_m1(current->u16(), w.input_norm.data(), kEpsilon, w.q_weight.data(), w.q_bias.data(),
+                                   w.k_weight.data(), w.k_bias.data(), w.v_weight.data(), w.v_bias.data(), e.q.u16(),
+                                   e.k.u16(), e.v.u16(), kHidden, e.q_dim, e.kv_dim, s),
+                 "talker RMSNorm + Q/K/V");
+        // launch_qk_norm_rope_cache_m1 + launch_attention (R17:17181-17195)
+        op_check(qm_decode_step_fused(e.q.u16(), e.k.u16(), e.v.u16(), w.q_norm.data(), w.k_norm.data(), e.cosine.u16(),
+                                      e.sine.u16(), e.q_rotated.u16(), &cache, nullptr, 1, e.context.u16(), e.q_heads,
+                                      position, -1, kScale, kEpsilon, e.workspace.raw(), e.workspace.bytes(), nullptr, s),
+                 "talker norm/RoPE/append + attention");
+        // launch_linear_m1: o_proj (R17:17203-17210)
+        op_check(qm_linear_m1(e.context.u16(), w.o_weight.data(), w.o_bias.data(), nullptr, e.attention.u16(), kHidden,
+                              e.q_dim, s),
+                 "talker o_proj");
+        // launch_add_postnorm_m1 + launch_gate_up_swiglu_m1 (R17:17215-17229)
+        op_check(qm_add_postnorm_gate_up_swiglu_m1(current->u16(), e.attention.u16(), w.post_norm.data(), kEpsilon,
+                                                   e.residual.u16(), w.gate_weight.data(), w.up_weight.data(),
+                                                   e.swiglu.u16(), kHidden, e.intermediate, s),
+                 "talker add + post-norm + gate/up/SwiGLU");
+        // launch_linear_m1: down_proj + residual (R17:17236-17244)
+        op_check(qm_linear_m1(e.swiglu.u16(), w.down_weight.data(), nullptr, e.residual.u16(), next->u16(), kHidden,
+                              e.intermediate, s),
+                 "talker down_proj + residual");
+        std::swap(current, next);
+    }
+    op_check(qm_rmsnorm_rows(current->u16(), e.final_norm.data(), e.final_hidden.u16(), 1, kHidden, kEpsilon, s),
+             "talker final RMSNorm");
+    return e.final_hidden.u16();
+}
+
+// Runs f, turning exceptions into codes.
+template <typename F>
+static int32_t guarded(F&& f) {
+    try {
+        f();
+        return QM_OK;
+    } catch (const ApiError& e) {
+        g_last_error = e.what();
+        return e.code;
+    } catch (const IoError& e) {
+        g_last_error = e.what();
+        return QM_ERR_IO;
+    } catch (const TensorError& e) {
+        g_last_error = e.what();
+        return QM_ERR_TENSOR;
+    } catch (const std::exception& e) {
+        g_last_error = e.what();
+        return QM_ERR_ARGUMENT;
+    }
+}
+
+}  // namespace qm_engine
+
+using namespace qm_engine;
+
+extern "C" const char* qm_engine_last_error(void) { return g_last_error.c_str(); }
+
+extern "C" uint64_t qm_fnv1a64(const void* data, size_t bytes) {
+    const uint8_t* p = static_cast<const uint8_t*>(data);
+    uint64_t value = 1469598103934665603ULL;
+    for (size_t i = 0; i < bytes; ++i) {
+        value ^= p[i];
+        value *= 1099511628211ULL;
+    }
+    return value;
+}
+
+static uint16_t to_bf16(float value) {
+    uint32_t bits;
+    std::memcpy(&bits, &value, sizeof bits);
+    if ((bits & 0x7fffffffU) > 0x7f800000U) return static_cast<uint16_t>((bits >> 16) | 0x0040U);
+    bits += 0x7fffU + ((bits >> 16) & 1U);
+    return static_cast<uint16_t>(bits >> 16);
+}
+
+extern "C" int32_t qm_rope_rows(int32_t rows, int32_t start, int32_t head_dim, double theta, uint16_t* cos_out,
+                                uint16_t* sin_out) {
+    if (!cos_out || !sin_out) return QM_ERR_NULL;
+    if (rows < 0 || start < 0 || head_dim <= 0 || (head_dim & 1)) return QM_ERR_GEOMETRY;
+    const int half = head_dim / 2;
+    for (int row = 0; row < rows; ++row) {
+        const double position = static_cast<double>(start + row);
+        for (int i = 0; i < half; ++i) {
+            const double inverse = std::pow(theta, -2.0 * static_cast<double>(i) / static_cast<double>(head_dim));
+            const double angle = position * inverse;
+            const uint16_t c = to_bf16(static_cast<float>(std::cos(angle)));
+            const uint16_t s = to_bf16(static_cast<float>(std::sin(angle)));
+            const size_t base = static_cast<size_t>(row) * head_dim;
+            cos_out[base + i] = cos_out[base + i + half] = c;
+            sin_out[base + i] = sin_out[base + i + half] = s;
+        }
+    }
+    return QM_OK;
+}
+
+extern "C" int32_t qm_safefile_open(const char* path, qm_safefile** out) {
+    if (!path || !out) return QM_ERR_NULL;
+    *out = nullptr;
+    return guarded([&] { *out = new qm_safefile(path); });
+}
+
+extern "C" void qm_safefile_close(qm_safefile* file) { delete file; }
+
+extern "C" int32_t qm_safefile_count(const qm_safefile* file) { return file ? static_cast<int32_t>(file->order.size()) : 0; }
+
+extern "C" int32_t qm_safefile_tensor(const qm_safefile* file, int32_t index, const char** name, const char** dtype,
+                                      int32_t* rank, int64_t* shape, const void** data, uint64_t* bytes) {
+    if (!file) return QM_ERR_NULL;
+    if (index < 0 || index >= static_cast<int32_t>(file->order.size())) return QM_ERR_ARGUMENT;
+    const TensorView& t = *file->order[static_cast<size_t>(index)];
+    if (t.shape.size() > 8) return QM_ERR_GEOMETRY;
+    if (name) *name = t.name.c_str();
+    if (dtype) *dtype = t.dtype.c_str();
+    if (rank) *rank = static_cast<int32_t>(t.shape.size());
+    if (shape) for (size_t i = 0; i < t.shape.size(); ++i) shape[i] = t.shape[i];
+    if (data) *data = t.data;
+    if (bytes) *bytes = t.bytes;
+    return QM_OK;
+}
+
+extern "C" int32_t qm_talker_create(const char* model_dir, int32_t max_cache, void* hip_stream, qm_talker** out) {
+    if (!model_dir || !out) return QM_ERR_NULL;
+    *out = nullptr;
+    return guarded([&] { *out = create_talker(model_dir, max_cache, static_cast<hipStream_t>(hip_stream)).release(); });
+}
+
+extern "C" void qm_talker_destroy(qm_talker* engine) { delete engine; }
+
+extern "C" int32_t qm_talker_info(const qm_talker* e, int32_t info[7]) {
+    if (!e || !info) return QM_ERR_NULL;
+    info[0] = static_cast<int32_t>(e->layers.size());
+    info[1] = e->q_heads; info[2] = e->kv_heads; info[3] = e->q_dim; info[4] = e->kv_dim;
+    info[5] = e->intermediate; info[6] = e->max_cache;
+    return QM_OK;
+}
+
+extern "C" int32_t qm_talker_reset(qm_talker* engine, int32_t prefill_length) {
+    if (!engine) return QM_ERR_NULL;
+    return guarded([&] { reset_talker(*engine, prefill_length); });
+}
+
+extern "C" int32_t qm_talker_cache(qm_talker* engine, int32_t layer, uint16_t** key_cache, uint16_t** value_cache) {
+    if (!engine || !key_cache || !value_cache) return QM_ERR_NULL;
+    if (layer < 0 || layer >= static_cast<int32_t>(engine->layers.size())) return QM_ERR_ARGUMENT;
+    *key_cache = engine->layers[static_cast<size_t>(layer)].key_cache.u16();
+    *value_cache = engine->layers[static_cast<size_t>(layer)].value_cache.u16();
+    return QM_OK;
+}
+
+extern "C" int32_t qm_talker_decode(qm_talker* engine, const uint16_t* input_device, const uint16_t* cosine,
+                                    const uint16_t* sine, int32_t decode_index, const uint16_t** final_hidden_device) {
+    if (!engine || !final_hidden_device) return QM_ERR_NULL;
+    return guarded([&] { *final_hidden_device = decode(*engine, input_device, cosine, sine, decode_index); });
+}
+
+extern "C" int32_t qm_talker_synchronize(qm_talker* engine) {
+    if (!engine) return QM_ERR_NULL;
+    return guarded([&] { hip_check(hipStreamSynchronize(engine->stream), "generation stream synchronize"); });
+}

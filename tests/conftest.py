@@ -30,6 +30,13 @@ def qm():
 
 
 @pytest.fixture(scope="session")
+def engine():
+    """The engine-shell library binding (libqm_engine.so); no fallback if it is not built."""
+    import importlib
+    return importlib.import_module("qingming-qwen3-tts_amd.engine")
+
+
+@pytest.fixture(scope="session")
 def dev():
     import torch
     if not torch.cuda.is_available():

@@ -1,0 +1,142 @@
+"""GPU parity of the engine shell: a synthetic talker checkpoint (safetensors, written here with
+torch) is loaded by qm_talker_create, a prompt's K/V is placed in the caches, and decode steps run
+through every layer; the final hidden vector of each step is compared with the oracle's chain of
+the same operators (bit-exact, as for the single-layer step), and the trajectory hash of the
+outputs with the hash of the oracle's bytes."""
+import os
+
+import numpy as np
+import pytest
+
+from qm_testlib import SCALE, to_u16
+
+pytestmark = pytest.mark.gpu
+
+H, Q, KV, I, LAYERS, MAX_CACHE, PREFILL = 2048, 2048, 1024, 512, 3, 48, 21
+
+
+def _checkpoint(directory, with_bias):
+    import torch
+    from safetensors.torch import save_file
+    g = torch.Generator().manual_seed(17 + with_bias)
+
+    def rnd(shape, std=1.0, mean=0.0):
+        return (torch.randn(shape, generator=g) * std + mean).to(torch.bfloat16)
+
+    tensors = {"talker.model.norm.weight": rnd((H,), 0.1, 1.0), "talker.model.codec_embedding.weight": rnd((8, 16))}
+    for i in range(LAYERS):
+        p = f"talker.model.layers.{i}."
+        tensors.update({
+            p + "input_layernorm.weight": rnd((H,), 0.1, 1.0), p + "post_attention_layernorm.weight": rnd((H,), 0.1, 1.0),
+            p + "self_attn.q_proj.weight": rnd((Q, H), 0.02), p + "self_attn.k_proj.weight": rnd((KV, H), 0.02),
+            p + "self_attn.v_proj.weight": rnd((KV, H), 0.02), p + "self_attn.o_proj.weight": rnd((H, Q), 0.02),
+            p + "self_attn.q_norm.weight": rnd((128,), 0.1, 1.0), p + "self_attn.k_norm.weight": rnd((128,), 0.1, 1.0),
+            p + "mlp.gate_proj.weight": rnd((I, H), 0.03), p + "mlp.up_proj.weight": rnd((I, H), 0.03),
+            p + "mlp.down_proj.weight": rnd((H, I), 0.03),
+        })
+        if with_bias:
+            tensors.update({p + "self_attn.q_proj.bias": rnd((Q,), 0.1), p + "self_attn.k_proj.bias": rnd((KV,), 0.1),
+                            p + "self_attn.v_proj.bias": rnd((KV,), 0.1), p + "self_attn.o_proj.bias": rnd((H,), 0.1)})
+    # two files, as a sharded checkpoint: the reader takes the union
+    names = sorted(tensors)
+    save_file({n: tensors[n] for n in names[::2]}, os.path.join(directory, "model-00001-of-00002.safetensors"))
+    save_file({n: tensors[n] for n in names[1::2]}, os.path.join(directory, "model-00002-of-00002.safetensors"))
+    return {n: t.view(torch.int16).numpy().view(np.uint16).copy() for n, t in tensors.items()}
+
+
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_engine_decode_steps_match_the_oracle_chain(engine, oracle, qm, dev, tmp_path, with_bias):
+    import torch
+    w = _checkpoint(str(tmp_path), with_bias)
+    talker = engine.Talker(str(tmp_path), MAX_CACHE)
+    assert (talker.layers, talker.q_heads, talker.kv_heads, talker.q_dim, talker.kv_dim, talker.intermediate,
+            talker.max_cache) == (LAYERS, 16, 8, Q, KV, I, MAX_CACHE)
+    talker.reset(PREFILL)
+    # a prompt's K/V, placed as the prefill would leave it: [kv_heads][max_cache][128], zero elsewhere
+    caches = []
+    for layer in range(LAYERS):
+        k = np.zeros((8, MAX_CACHE, 128), dtype=np.uint16)
+        v = np.zeros((8, MAX_CACHE, 128), dtype=np.uint16)
+        k[:, :PREFILL] = oracle.normal_bf16((8, PREFILL, 128), 100 + layer)
+        v[:, :PREFILL] = oracle.normal_bf16((8, PREFILL, 128), 200 + layer)
+        caches.append((k, v))
+    talker.synchronize()
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    for layer, (k, v) in enumerate(caches):
+        ka, va = talker.cache_addresses(layer)
+        assert hip.hipMemcpy(C.c_void_p(ka), k.ctypes.data_as(C.c_void_p), C.c_size_t(k.nbytes), 1) == 0
+        assert hip.hipMemcpy(C.c_void_p(va), v.ctypes.data_as(C.c_void_p), C.c_size_t(v.nbytes), 1) == 0
+
+    def tensor(name):
+        return w.get(name)
+
+    trajectory_gpu, trajectory_cpu = b"", b""
+    for step in range(4):
+        x = oracle.normal_bf16((H,), 900 + step)
+        cos, sin = engine.rope_rows(1, PREFILL + step)
+        xd = torch.from_numpy(x.view(np.int16)).to(dev)
+        address = talker.decode(xd, cos[0], sin[0], step)
+        talker.synchronize()
+        out = torch.empty(H, dtype=torch.int16, device=dev)
+        assert hip.hipMemcpy(C.c_void_p(out.data_ptr()), C.c_void_p(address), C.c_size_t(H * 2), 3) == 0
+        got = to_u16(out)
+        # the oracle's chain (R17:17155-17252)
+        cur = x.copy()
+        u16 = lambda n: np.zeros(n, dtype=np.uint16)
+        for layer in range(LAYERS):
+            p = f"talker.model.layers.{layer}."
+            k, v = caches[layer]
+            cache = oracle.flat_cache(k, v, 8, MAX_CACHE)
+            norm, q, kk, vv, qrot, ctxv, attn, res, post, act, nxt = (u16(H).reshape(1, H), u16(Q), u16(KV), u16(KV),
+                                                                     u16(Q), u16(Q), u16(H), u16(H), u16(H), u16(I), u16(H))
+            assert oracle.rmsnorm_rows(cur.reshape(1, H), tensor(p + "input_layernorm.weight"), norm, 1, H) == 0
+            assert oracle.qkv_m1(norm[0], tensor(p + "self_attn.q_proj.weight"), tensor(p + "self_attn.q_proj.bias"),
+                                 tensor(p + "self_attn.k_proj.weight"), tensor(p + "self_attn.k_proj.bias"),
+                                 tensor(p + "self_attn.v_proj.weight"), tensor(p + "self_attn.v_proj.bias"),
+                                 q, kk, vv, H, Q, KV, 16) == 0
+            assert oracle.qk_norm_rope_kv_append(q, kk, vv, tensor(p + "self_attn.q_norm.weight"),
+                                                 tensor(p + "self_attn.k_norm.weight"), cos[0], sin[0], qrot, cache,
+                                                 None, 1, 16, PREFILL + step) == 0
+            assert oracle.attention(qrot, cache, None, 1, ctxv, 1, PREFILL + step, 16, -1, SCALE, oracle.POLICY_ONLINE,
+                                    16) == 0
+            assert oracle.linear_m1(ctxv, tensor(p + "self_attn.o_proj.weight"), tensor(p + "self_attn.o_proj.bias"),
+                                    None, attn, H, Q, 16) == 0
+            assert oracle.add_postnorm_m1(cur, attn, tensor(p + "post_attention_layernorm.weight"), res, post, H) == 0
+            assert oracle.gate_up_swiglu_m1(post, tensor(p + "mlp.gate_proj.weight"), tensor(p + "mlp.up_proj.weight"),
+                                            act, H, I, 16) == 0
+            assert oracle.linear_m1(act, tensor(p + "mlp.down_proj.weight"), None, res, nxt, H, I, 16) == 0
+            cur = nxt
+        final = u16(H).reshape(1, H)
+        assert oracle.rmsnorm_rows(cur.reshape(1, H), tensor("talker.model.norm.weight"), final, 1, H) == 0
+        err = np.max(np.abs(oracle.bf16_to_f32(final[0]).astype(np.float64) - oracle.bf16_to_f32(got).astype(np.float64)))
+        assert err <= 0.0625, (step, err)          # (the layer step is bit-exact in practice; attention's budget is 1e-2)
+        trajectory_gpu += got.tobytes()
+        trajectory_cpu += final[0].tobytes()
+    if trajectory_gpu == trajectory_cpu:
+        assert engine.fnv1a64(trajectory_gpu) == engine.fnv1a64(trajectory_cpu)
+    # the caches now hold the four appended rows exactly as the oracle's do
+    for layer, (k, v) in enumerate(caches):
+        ka, va = talker.cache_addresses(layer)
+        kd = np.zeros_like(k)
+        assert hip.hipMemcpy(kd.ctypes.data_as(C.c_void_p), C.c_void_p(ka), C.c_size_t(k.nbytes), 2) == 0
+        if layer == 0:
+            assert np.array_equal(kd, k)           # norm, projection and append are bit-exact operators
+        else:
+            # deeper layers see the attention of the layers before them (judged to 1e-2, not to the bit)
+            assert np.max(np.abs(oracle.bf16_to_f32(kd).astype(np.float64) - oracle.bf16_to_f32(k).astype(np.float64))) <= 0.0625
+    # overflow guard (the reference throws "Talker device decode cache overflow")
+    with pytest.raises(engine.EngineError) as err:
+        talker.decode(xd, cos[0], sin[0], MAX_CACHE - PREFILL)
+    assert err.value.code == -3
+    talker.close()
+
+
+def test_engine_rejects_a_checkpoint_with_the_wrong_geometry(engine, dev, tmp_path):
+    import torch
+    from safetensors.torch import save_file
+    bad = {"talker.model.layers.0.input_layernorm.weight": torch.ones(100, dtype=torch.bfloat16)}
+    save_file(bad, os.path.join(str(tmp_path), "m.safetensors"))
+    with pytest.raises(engine.EngineError) as err:
+        engine.Talker(str(tmp_path), 32)
+    assert err.value.code == -8
