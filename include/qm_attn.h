@@ -398,6 +398,25 @@ int32_t qm_predictor_add_postnorm_gate_up_swiglu_m1(
     const uint16_t* gate_weight, const uint16_t* up_weight, uint16_t* output,
     int32_t hidden, int32_t intermediate, void* hip_stream);
 
+/* ---- linears over token rows (the prompt pass) ------------------------------------ */
+/*
+ * qm_linear_rows replaces NativeTalkerEngine::linear_generic -> native_ops::linear_bf16
+ * (R17:17453-17472, 198-245; kernel linear_wave32_bf16_f32acc_kernel :126-196) as the prompt pass
+ * uses it (R17:16646-16790): output[r][n] = bf16(sum_k input[r][k] * weight[n][k] (+ bias[n])), each
+ * sum in the order of qm_linear_m1, so a prompt row and a decode step of the same vector agree to
+ * the bit.  A non-NULL residual [rows][output_columns] folds the launch_add behind it
+ * (add_bf16_kernel R17:8729-8744: bf16(residual + output)).
+ * qm_gate_up_swiglu_rows = the two linear_generic calls on gate and up and launch_swiglu
+ * (R17:16742-16768, swiglu_kernel :8745-8770): qm_gate_up_swiglu_m1 row by row.
+ * reduction % 8 == 0, reduction <= 16384, input and weights 16-byte aligned (QM_ERR_GEOMETRY).
+ */
+int32_t qm_linear_rows(
+    const uint16_t* input, const uint16_t* weight, const uint16_t* bias, const uint16_t* residual,
+    uint16_t* output, int32_t rows, int32_t output_columns, int32_t reduction_columns, void* hip_stream);
+int32_t qm_gate_up_swiglu_rows(
+    const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight, uint16_t* output,
+    int32_t rows, int32_t hidden, int32_t intermediate, void* hip_stream);
+
 /* ---- final head: score processing, top-k sampler, history ------------------------ */
 /*
  * qm_sample_topk replaces gpu_sample_topk_f32_kernel and gpu_sample_topk_bf16_kernel

@@ -84,6 +84,19 @@ int32_t qm_talker_cache(qm_talker* engine, int32_t layer, uint16_t** key_cache, 
  */
 int32_t qm_talker_decode(qm_talker* engine, const uint16_t* input_device, const uint16_t* cosine,
                          const uint16_t* sine, int32_t decode_index, const uint16_t** final_hidden_device);
+/*
+ * NativeTalkerEngine::prefill (R17:16561-16800): zeroes the caches, then sends the prompt's `rows`
+ * token rows through every layer — RMSNorm, q/k/v projections, QK-norm + RoPE, causal attention
+ * that also writes K/V to the layer's cache, o_proj + residual, post-norm, gate/up/SwiGLU,
+ * down_proj + residual — and applies the final RMSNorm to the last row.  Sets the prompt length
+ * that qm_talker_decode continues from.  input_device: [rows][2048] bf16 on the device; cosine,
+ * sine: [rows][128] bf16 on the HOST (positions 0 .. rows-1); *final_hidden_device: the last
+ * row's final hidden vector (engine-owned, [2048]).  Enqueues only.  rows <= max_cache
+ * (QM_ERR_SLOT_RANGE).  Every linear is evaluated in the M = 1 kernels' order, so a token gives
+ * the same K/V whether it was part of the prompt or decoded.
+ */
+int32_t qm_talker_prefill(qm_talker* engine, const uint16_t* input_device, const uint16_t* cosine,
+                          const uint16_t* sine, int32_t rows, const uint16_t** final_hidden_device);
 /* Waits for the engine's stream. */
 int32_t qm_talker_synchronize(qm_talker* engine);
 

@@ -260,3 +260,13 @@ def final_head_sample(logits, history, generation_index, vocab, eos, suppressed_
                                        C.c_int32(eos), C.c_int32(suppressed_tail), C.c_float(penalty),
                                        C.c_int32(top_k), C.c_float(temperature), _p(rng_state), _p(code_out),
                                        _p(scores_out))
+
+
+def linear_rows(x, weight, bias, residual, out, rows, output_columns, reduction_columns, threads=8):
+    return lib().qmo_linear_rows(_p(x), _p(weight), _p(bias), _p(residual), _p(out), C.c_int32(rows),
+                                 C.c_int32(output_columns), C.c_int32(reduction_columns), C.c_int32(threads))
+
+
+def gate_up_swiglu_rows(x, gate_w, up_w, out, rows, hidden, intermediate, threads=8):
+    return lib().qmo_gate_up_swiglu_rows(_p(x), _p(gate_w), _p(up_w), _p(out), C.c_int32(rows), C.c_int32(hidden),
+                                         C.c_int32(intermediate), C.c_int32(threads))

@@ -990,4 +990,37 @@ int32_t qmo_final_head_sample(const uint16_t* logits, int32_t* history, int32_t 
     return QM_OK;
 }
 
+// ---- linears over token rows (the prompt pass) -----------------------------------------------------------
+// native_ops::linear_wave32_bf16_f32acc_kernel (R17:126-196; NativeTalkerEngine::linear_generic
+// :17453-17472): every (row, column) is the M = 1 linear's scalar — same chains, tree, bias.
+// `residual` folds add_bf16_kernel (R17:8729-8744) behind it; the gate/up form folds swiglu_kernel
+// (R17:8745-8770) behind two such linears: exactly the M = 1 SwiGLU arithmetic, row by row.
+int32_t qmo_linear_rows(const uint16_t* input, const uint16_t* weight, const uint16_t* bias,
+                        const uint16_t* residual, uint16_t* output, int32_t rows, int32_t output_columns,
+                        int32_t reduction_columns, int32_t n_threads) {
+    if (!input || !weight || !output) return QM_ERR_NULL;
+    if (rows < 0 || output_columns < 0 || reduction_columns < 0) return QM_ERR_ARGUMENT;
+    parallel_for(static_cast<int64_t>(rows) * output_columns, n_threads, [&](int64_t at) {
+        const int64_t r = at / output_columns;
+        const int o = static_cast<int>(at % output_columns);
+        output[at] = linear_m1_scalar(input + r * reduction_columns, weight + static_cast<int64_t>(o) * reduction_columns,
+                                      bias, residual ? residual + r * output_columns : nullptr, o, reduction_columns);
+    });
+    return QM_OK;
+}
+
+int32_t qmo_gate_up_swiglu_rows(const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight,
+                                uint16_t* output, int32_t rows, int32_t hidden, int32_t intermediate,
+                                int32_t n_threads) {
+    if (!input || !gate_weight || !up_weight || !output) return QM_ERR_NULL;
+    if (rows < 0 || hidden < 0 || intermediate < 0) return QM_ERR_ARGUMENT;
+    for (int r = 0; r < rows; ++r) {
+        const int32_t rc = qmo_gate_up_swiglu_m1(input + static_cast<int64_t>(r) * hidden, gate_weight, up_weight,
+                                                 output + static_cast<int64_t>(r) * intermediate, hidden, intermediate,
+                                                 n_threads);
+        if (rc != QM_OK) return rc;
+    }
+    return QM_OK;
+}
+
 }  // extern "C"

@@ -79,6 +79,8 @@ _SIGNATURES = {
     "qm_final_head_process": (_I32, [_PTR, _PTR, _I32, _I32, _I32, _I32, _I32, _F32, _PTR, _PTR]),
     "qm_final_head_sample": (_I32, [_PTR, _PTR, _I32, _I32, _I32, _I32, _F32, _I32, _F32, _PTR, _PTR, _PTR, _PTR]),
     "qm_gather_embedding": (_I32, [_PTR, _I32, _PTR, _I32, _I32, _PTR, _PTR, _PTR]),
+    "qm_linear_rows": (_I32, [_PTR] * 5 + [_I32, _I32, _I32, _PTR]),
+    "qm_gate_up_swiglu_rows": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _PTR]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
@@ -301,6 +303,16 @@ def final_head_sample(logits, history, generation_index, vocab, eos, suppressed_
     _check(lib().qm_final_head_sample(_addr(logits), _addr(history), generation_index, vocab, eos, suppressed_tail,
                                       penalty, top_k, temperature, _addr(rng_state), _addr(code_out),
                                       _addr(scores_out), stream), "qm_final_head_sample")
+
+
+def linear_rows(x, weight, bias, residual, out, rows, output_columns, reduction_columns, stream=0):
+    _check(lib().qm_linear_rows(_addr(x), _addr(weight), _addr(bias), _addr(residual), _addr(out), rows,
+                                output_columns, reduction_columns, stream), "qm_linear_rows")
+
+
+def gate_up_swiglu_rows(x, gate_w, up_w, out, rows, hidden, intermediate, stream=0):
+    _check(lib().qm_gate_up_swiglu_rows(_addr(x), _addr(gate_w), _addr(up_w), _addr(out), rows, hidden,
+                                        intermediate, stream), "qm_gate_up_swiglu_rows")
 
 
 def gather_embedding(table, table_rows, codes, group, dimension, selected, next_input, stream=0):

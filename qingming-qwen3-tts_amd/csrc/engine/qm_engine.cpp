@@ -107,6 +107,9 @@ struct qm_talker {
     bool own_stream = false;
     qm_engine::DeviceBuffer hidden_a, hidden_b, q, k, v, q_rotated, context, attention, residual, swiglu, final_hidden,
         cosine, sine, workspace;
+    // the prompt pass's row buffers ([rows][...]), allocated by the first prefill for max_cache rows
+    qm_engine::DeviceBuffer p_hidden_a, p_hidden_b, p_norm, p_q, p_k, p_v, p_q_rotated, p_k_rotated, p_context, p_residual,
+        p_swiglu, p_cosine, p_sine;
 
     ~qm_talker() {
         if (own_stream && stream) (void)hipStreamDestroy(stream);
@@ -223,6 +226,20 @@ static void reset_talker(qm_talker& e, int prefill_length) {
     e.prefill_length = prefill_length;
 }
 
+static qm_kv_cache flat_cache_of(const qm_talker& e, const Layer& w) {
+    qm_kv_cache cache = {};
+    cache.k_pool = w.key_cache.u16();
+    cache.v_pool = w.value_cache.u16();
+    cache.stride_page = 0;
+    cache.stride_head = static_cast<int64_t>(e.max_cache) * kHeadDim;
+    cache.stride_token = kHeadDim;
+    cache.page_size = e.max_cache;
+    cache.n_pages = 1;
+    cache.kv_heads = e.kv_heads;
+    cache.head_dim = kHeadDim;
+    return cache;
+}
+
 static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const uint16_t* cosine, const uint16_t* sine,
                               int decode_index) {
     if (!input_device || !cosine || !sine) throw ApiError(QM_ERR_NULL, "talker device decode input is null");
@@ -236,16 +253,7 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
     DeviceBuffer* current = &e.hidden_a;
     DeviceBuffer* next = &e.hidden_b;
     for (Layer& w : e.layers) {
-        qm_kv_cache cache = {};
-        cache.k_pool = w.key_cache.u16();
-        cache.v_pool = w.value_cache.u16();
-        cache.stride_page = 0;
-        cache.stride_head = static_cast<int64_t>(e.max_cache) * kHeadDim;
-        cache.stride_token = kHeadDim;
-        cache.page_size = e.max_cache;
-        cache.n_pages = 1;
-        cache.kv_heads = e.kv_heads;
-        cache.head_dim = kHeadDim;
+        qm_kv_cache cache = flat_cache_of(e, w);
         // launch_rmsnorm + launch_qkv_m1 (R17:17163-17176)
         op_check(qm_rmsnorm_qkv_m1(current->u16(), w.input_norm.data(), kEpsilon, w.q_weight.data(), w.q_bias.data(),
                                    w.k_weight.data(), w.k_bias.data(), w.v_weight.data(), w.v_bias.data(), e.q.u16(),
@@ -273,6 +281,71 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
     }
     op_check(qm_rmsnorm_rows(current->u16(), e.final_norm.data(), e.final_hidden.u16(), 1, kHidden, kEpsilon, s),
              "talker final RMSNorm");
+    return e.final_hidden.u16();
+}
+
+// NativeTalkerEngine::prefill (R17:16561-16800): the prompt's rows through every layer.  The
+// reference's launches per layer and what runs here:
+//   rmsnorm                                   -> qm_rmsnorm_rows
+//   3 x linear_generic (q, k, v)              -> 3 x qm_linear_rows
+//   2 x rmsnorm + 2 x rope_rows               -> 2 x qm_norm_rope_rows
+//   scatter_prefill_cache + attention         -> qm_prefill_attention_causal (writes the cache itself)
+//   linear_generic (o_proj) + add             -> qm_linear_rows with the residual folded in
+//   rmsnorm                                   -> qm_rmsnorm_rows
+//   2 x linear_generic + swiglu               -> qm_gate_up_swiglu_rows
+//   linear_generic (down) + add               -> qm_linear_rows with the residual folded in
+// and the final RMSNorm, of the last row only (the one row the reference reads back).
+static const uint16_t* prefill(qm_talker& e, const uint16_t* input_device, const uint16_t* cosine, const uint16_t* sine,
+                               int rows) {
+    if (!input_device || !cosine || !sine) throw ApiError(QM_ERR_NULL, "talker prefill input is null");
+    if (rows <= 0) throw ApiError(QM_ERR_ARGUMENT, "a prompt has at least one row");
+    if (rows > e.max_cache) throw ApiError(QM_ERR_SLOT_RANGE, "talker prefill exceeds the cache");
+    if (!e.p_hidden_a.raw()) {
+        auto rows_of = [&](int width) { return DeviceBuffer(static_cast<size_t>(e.max_cache) * width * 2); };
+        e.p_hidden_a = rows_of(kHidden); e.p_hidden_b = rows_of(kHidden); e.p_norm = rows_of(kHidden);
+        e.p_q = rows_of(e.q_dim); e.p_k = rows_of(e.kv_dim); e.p_v = rows_of(e.kv_dim);
+        e.p_q_rotated = rows_of(e.q_dim); e.p_k_rotated = rows_of(e.kv_dim); e.p_context = rows_of(e.q_dim);
+        e.p_residual = rows_of(kHidden); e.p_swiglu = rows_of(e.intermediate);
+        e.p_cosine = rows_of(kHeadDim); e.p_sine = rows_of(kHeadDim);
+    }
+    reset_talker(e, rows);
+    hipStream_t s = e.stream;
+    const size_t rope_bytes = static_cast<size_t>(rows) * kHeadDim * 2;
+    hip_check(hipMemcpyAsync(e.p_hidden_a.raw(), input_device, static_cast<size_t>(rows) * kHidden * 2,
+                             hipMemcpyDeviceToDevice, s), "prefill input copy");
+    hip_check(hipMemcpyAsync(e.p_cosine.raw(), cosine, rope_bytes, hipMemcpyHostToDevice, s), "prefill cosine upload");
+    hip_check(hipMemcpyAsync(e.p_sine.raw(), sine, rope_bytes, hipMemcpyHostToDevice, s), "prefill sine upload");
+    DeviceBuffer* current = &e.p_hidden_a;
+    DeviceBuffer* next = &e.p_hidden_b;
+    for (Layer& w : e.layers) {
+        const qm_kv_cache cache = flat_cache_of(e, w);
+        op_check(qm_rmsnorm_rows(current->u16(), w.input_norm.data(), e.p_norm.u16(), rows, kHidden, kEpsilon, s),
+                 "prefill input RMSNorm");
+        op_check(qm_linear_rows(e.p_norm.u16(), w.q_weight.data(), w.q_bias.data(), nullptr, e.p_q.u16(), rows, e.q_dim,
+                                kHidden, s), "prefill q_proj");
+        op_check(qm_linear_rows(e.p_norm.u16(), w.k_weight.data(), w.k_bias.data(), nullptr, e.p_k.u16(), rows, e.kv_dim,
+                                kHidden, s), "prefill k_proj");
+        op_check(qm_linear_rows(e.p_norm.u16(), w.v_weight.data(), w.v_bias.data(), nullptr, e.p_v.u16(), rows, e.kv_dim,
+                                kHidden, s), "prefill v_proj");
+        op_check(qm_norm_rope_rows(e.p_q.u16(), w.q_norm.data(), e.p_cosine.u16(), e.p_sine.u16(), e.p_q_rotated.u16(), rows,
+                                   e.q_heads, kEpsilon, s), "prefill q norm + RoPE");
+        op_check(qm_norm_rope_rows(e.p_k.u16(), w.k_norm.data(), e.p_cosine.u16(), e.p_sine.u16(), e.p_k_rotated.u16(), rows,
+                                   e.kv_heads, kEpsilon, s), "prefill k norm + RoPE");
+        op_check(qm_prefill_attention_causal(e.p_q_rotated.u16(), e.p_k_rotated.u16(), e.p_v.u16(), e.p_context.u16(), &cache,
+                                             nullptr, 1, 1, rows, e.q_heads, e.kv_heads, kScale, 0, 0, 0, nullptr, s),
+                 "prefill attention + cache write");
+        op_check(qm_linear_rows(e.p_context.u16(), w.o_weight.data(), w.o_bias.data(), current->u16(), e.p_residual.u16(),
+                                rows, kHidden, e.q_dim, s), "prefill o_proj + residual");
+        op_check(qm_rmsnorm_rows(e.p_residual.u16(), w.post_norm.data(), e.p_norm.u16(), rows, kHidden, kEpsilon, s),
+                 "prefill post-attention RMSNorm");
+        op_check(qm_gate_up_swiglu_rows(e.p_norm.u16(), w.gate_weight.data(), w.up_weight.data(), e.p_swiglu.u16(), rows,
+                                        kHidden, e.intermediate, s), "prefill gate/up/SwiGLU");
+        op_check(qm_linear_rows(e.p_swiglu.u16(), w.down_weight.data(), nullptr, e.p_residual.u16(), next->u16(), rows,
+                                kHidden, e.intermediate, s), "prefill down_proj + residual");
+        std::swap(current, next);
+    }
+    op_check(qm_rmsnorm_rows(current->u16() + static_cast<size_t>(rows - 1) * kHidden, e.final_norm.data(),
+                             e.final_hidden.u16(), 1, kHidden, kEpsilon, s), "prefill final RMSNorm");
     return e.final_hidden.u16();
 }
 
@@ -399,6 +472,12 @@ extern "C" int32_t qm_talker_decode(qm_talker* engine, const uint16_t* input_dev
                                     const uint16_t* sine, int32_t decode_index, const uint16_t** final_hidden_device) {
     if (!engine || !final_hidden_device) return QM_ERR_NULL;
     return guarded([&] { *final_hidden_device = decode(*engine, input_device, cosine, sine, decode_index); });
+}
+
+extern "C" int32_t qm_talker_prefill(qm_talker* engine, const uint16_t* input_device, const uint16_t* cosine,
+                                     const uint16_t* sine, int32_t rows, const uint16_t** final_hidden_device) {
+    if (!engine || !final_hidden_device) return QM_ERR_NULL;
+    return guarded([&] { *final_hidden_device = prefill(*engine, input_device, cosine, sine, rows); });
 }
 
 extern "C" int32_t qm_talker_synchronize(qm_talker* engine) {

@@ -26,6 +26,7 @@ _SIGNATURES = {
     "qm_talker_reset": (_I32, [_P, _I32]),
     "qm_talker_cache": (_I32, [_P, _I32, C.POINTER(_P), C.POINTER(_P)]),
     "qm_talker_decode": (_I32, [_P, _P, _P, _P, _I32, C.POINTER(_P)]),
+    "qm_talker_prefill": (_I32, [_P, _P, _P, _P, _I32, C.POINTER(_P)]),
     "qm_talker_synchronize": (_I32, [_P]),
 }
 EXPORTS = tuple(_SIGNATURES)
@@ -121,6 +122,17 @@ class Talker:
         out = _P()
         _check(lib().qm_talker_decode(self._handle, address, cosine_host.ctypes.data, sine_host.ctypes.data,
                                       decode_index, C.byref(out)))
+        return out.value
+
+    def prefill(self, input_device, cosine_host, sine_host, rows):
+        """input_device: torch tensor [rows][2048] (or an address); cosine/sine: numpy uint16 [rows][128] on the
+        host.  Returns the device address of the last row's final hidden vector."""
+        address = input_device if isinstance(input_device, int) else input_device.data_ptr()
+        cosine_host = np.ascontiguousarray(cosine_host, dtype=np.uint16)
+        sine_host = np.ascontiguousarray(sine_host, dtype=np.uint16)
+        out = _P()
+        _check(lib().qm_talker_prefill(self._handle, address, cosine_host.ctypes.data, sine_host.ctypes.data, rows,
+                                       C.byref(out)))
         return out.value
 
     def synchronize(self):

@@ -140,3 +140,99 @@ def test_engine_rejects_a_checkpoint_with_the_wrong_geometry(engine, dev, tmp_pa
     with pytest.raises(engine.EngineError) as err:
         engine.Talker(str(tmp_path), 32)
     assert err.value.code == -8
+
+
+def test_engine_prefill_then_decode_matches_the_oracle_chain(engine, oracle, qm, dev, tmp_path):
+    """A 37-token prompt through qm_talker_prefill, then two decoded tokens: last-row hidden vectors,
+    and the caches the prompt leaves behind, against the oracle's chain of the same operators."""
+    import ctypes as C
+    import torch
+    w = _checkpoint(str(tmp_path), True)
+    talker = engine.Talker(str(tmp_path), MAX_CACHE)
+    hip = C.CDLL("libamdhip64.so")
+    S = 37
+    x = oracle.normal_bf16((S, H), 31)
+    cos, sin = engine.rope_rows(S + 2, 0)
+    xd = torch.from_numpy(x.view(np.int16)).to(dev)
+    address = talker.prefill(xd, cos[:S], sin[:S], S)
+    talker.synchronize()
+    out = torch.empty(H, dtype=torch.int16, device=dev)
+    assert hip.hipMemcpy(C.c_void_p(out.data_ptr()), C.c_void_p(address), C.c_size_t(H * 2), 3) == 0
+    got = to_u16(out)
+
+    u16 = lambda *shape: np.zeros(shape, dtype=np.uint16)
+    caches = [(u16(8, MAX_CACHE, 128), u16(8, MAX_CACHE, 128)) for _ in range(LAYERS)]
+    cur = x.copy()
+    for layer in range(LAYERS):
+        p = f"talker.model.layers.{layer}."
+        k_cache, v_cache = caches[layer]
+        cache = oracle.flat_cache(k_cache, v_cache, 8, MAX_CACHE)
+        norm, q, k, v, qrot, krot, ctxv, res, post, act, nxt = (u16(S, H), u16(S, Q), u16(S, KV), u16(S, KV), u16(S, Q),
+                                                               u16(S, KV), u16(S, Q), u16(S, H), u16(S, H), u16(S, I),
+                                                               u16(S, H))
+        assert oracle.rmsnorm_rows(cur, w[p + "input_layernorm.weight"], norm, S, H) == 0
+        for name, dst, n in (("q", q, Q), ("k", k, KV), ("v", v, KV)):
+            assert oracle.linear_rows(norm, w[p + f"self_attn.{name}_proj.weight"], w[p + f"self_attn.{name}_proj.bias"],
+                                      None, dst, S, n, H, 16) == 0
+        assert oracle.norm_rope_rows(q, w[p + "self_attn.q_norm.weight"], cos[:S], sin[:S], qrot, S, 16) == 0
+        assert oracle.norm_rope_rows(k, w[p + "self_attn.k_norm.weight"], cos[:S], sin[:S], krot, S, 8) == 0
+        assert oracle.prefill_attention_causal(qrot, krot, v, ctxv, cache, None, 1, 1, S, 16, 8, SCALE,
+                                               oracle.POLICY_ONLINE, 16) == 0
+        assert oracle.linear_rows(ctxv, w[p + "self_attn.o_proj.weight"], w[p + "self_attn.o_proj.bias"], cur, res, S, H,
+                                  Q, 16) == 0
+        assert oracle.rmsnorm_rows(res, w[p + "post_attention_layernorm.weight"], post, S, H) == 0
+        assert oracle.gate_up_swiglu_rows(post, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], act, S, H, I,
+                                          16) == 0
+        assert oracle.linear_rows(act, w[p + "mlp.down_proj.weight"], None, res, nxt, S, H, I, 16) == 0
+        cur = nxt
+    final = u16(1, H)
+    assert oracle.rmsnorm_rows(cur[S - 1:S], w["talker.model.norm.weight"], final, 1, H) == 0
+    err = np.max(np.abs(oracle.bf16_to_f32(final[0]).astype(np.float64) - oracle.bf16_to_f32(got).astype(np.float64)))
+    assert err <= 0.0625, err
+    # the prompt's K/V in the caches: layer 0 to the bit, deeper layers within the attention budget
+    for layer, (k_cache, v_cache) in enumerate(caches):
+        ka, va = talker.cache_addresses(layer)
+        kd, vd = np.zeros_like(k_cache), np.zeros_like(v_cache)
+        assert hip.hipMemcpy(kd.ctypes.data_as(C.c_void_p), C.c_void_p(ka), C.c_size_t(kd.nbytes), 2) == 0
+        assert hip.hipMemcpy(vd.ctypes.data_as(C.c_void_p), C.c_void_p(va), C.c_size_t(vd.nbytes), 2) == 0
+        assert not kd[:, S:].any() and not vd[:, S:].any()
+        if layer == 0:
+            assert np.array_equal(kd, k_cache) and np.array_equal(vd, v_cache)
+        else:
+            for a, b in ((kd, k_cache), (vd, v_cache)):
+                assert np.max(np.abs(oracle.bf16_to_f32(a).astype(np.float64) - oracle.bf16_to_f32(b).astype(np.float64))) <= 0.0625
+    # decoding continues at position S over those caches
+    for step in range(2):
+        token = oracle.normal_bf16((H,), 77 + step)
+        td = torch.from_numpy(token.view(np.int16)).to(dev)
+        address = talker.decode(td, cos[S + step], sin[S + step], step)
+        talker.synchronize()
+        assert hip.hipMemcpy(C.c_void_p(out.data_ptr()), C.c_void_p(address), C.c_size_t(H * 2), 3) == 0
+        got = to_u16(out)
+        cur1 = token.copy()
+        for layer in range(LAYERS):
+            p = f"talker.model.layers.{layer}."
+            cache = oracle.flat_cache(caches[layer][0], caches[layer][1], 8, MAX_CACHE)
+            norm, q, k, v, qrot, ctxv, attn, res, post, act, nxt = (u16(1, H), u16(Q), u16(KV), u16(KV), u16(Q), u16(Q),
+                                                                    u16(H), u16(H), u16(H), u16(I), u16(H))
+            assert oracle.rmsnorm_rows(cur1.reshape(1, H), w[p + "input_layernorm.weight"], norm, 1, H) == 0
+            assert oracle.qkv_m1(norm[0], w[p + "self_attn.q_proj.weight"], w[p + "self_attn.q_proj.bias"],
+                                 w[p + "self_attn.k_proj.weight"], w[p + "self_attn.k_proj.bias"],
+                                 w[p + "self_attn.v_proj.weight"], w[p + "self_attn.v_proj.bias"], q, k, v, H, Q, KV, 16) == 0
+            assert oracle.qk_norm_rope_kv_append(q, k, v, w[p + "self_attn.q_norm.weight"], w[p + "self_attn.k_norm.weight"],
+                                                 cos[S + step], sin[S + step], qrot, cache, None, 1, 16, S + step) == 0
+            assert oracle.attention(qrot, cache, None, 1, ctxv, 1, S + step, 16, -1, SCALE, oracle.POLICY_ONLINE, 16) == 0
+            assert oracle.linear_m1(ctxv, w[p + "self_attn.o_proj.weight"], w[p + "self_attn.o_proj.bias"], None, attn, H,
+                                    Q, 16) == 0
+            assert oracle.add_postnorm_m1(cur1, attn, w[p + "post_attention_layernorm.weight"], res, post, H) == 0
+            assert oracle.gate_up_swiglu_m1(post, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], act, H, I,
+                                            16) == 0
+            assert oracle.linear_m1(act, w[p + "mlp.down_proj.weight"], None, res, nxt, H, I, 16) == 0
+            cur1 = nxt
+        assert oracle.rmsnorm_rows(cur1.reshape(1, H), w["talker.model.norm.weight"], final, 1, H) == 0
+        err = np.max(np.abs(oracle.bf16_to_f32(final[0]).astype(np.float64) - oracle.bf16_to_f32(got).astype(np.float64)))
+        assert err <= 0.0625, (step, err)
+    with pytest.raises(engine.EngineError) as e:
+        talker.prefill(xd, cos[:S], sin[:S], MAX_CACHE + 1)
+    assert e.value.code == -3
+    talker.close()
