@@ -26,11 +26,11 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# HBM bytes per launch of decode_split_kernel<2> on the headline workload, from rocprofv3 --pmc
+# HBM bytes per launch of decode_split_kernel<2, false, true> on the headline workload, from rocprofv3 --pmc
 # FETCH_SIZE and WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a
 # plain 512 MiB copy (FETCH_SIZE reads half the copied bytes: factor 2.0; WRITE_SIZE: 1.0).
 # Summary and commands: profiles/decode_split_kernel_ragged64_traffic.txt
-HEADLINE_TRAFFIC_BYTES = int((288793.1 * 2.0 + 9528.9 * 1.0) * 1024)
+HEADLINE_TRAFFIC_BYTES = int((288456.9 * 2.0 + 3349.5 * 1.0) * 1024)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
@@ -785,7 +785,7 @@ def main():
                    "device": props.name, "compute_units": props.multi_processor_count},
         "roofline": {"bound": "hbm", "achieved": rep["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": rep["GBps"] / HBM_PEAK_GBPS, "traffic": HEADLINE_TRAFFIC_BYTES,
-                     "kernel": "decode_split_kernel<2> (+ decode_merge_kernel<2>, both inside the timed step)",
+                     "kernel": "decode_split_kernel<2, false, true> (+ decode_merge_kernel<2>, both inside the timed step)",
                      "algorithmic_bytes_per_launch": head.bytes, "avg_launch_us": ms * 1e3},
         "cpu_baseline": cpu,
         "per_config": per_config,

@@ -86,12 +86,18 @@ const char* qm_target_arch(void);
  *   QM_OPT_PREFILL_KERNEL  0 (default): qm_prefill_attention_causal picks one of its two kernels
  *       from the grid size; 1: four uniform waves per block; 2: four pairs of a matrix wave and a
  *       softmax wave per block.  Both give the same bits; other values make the call return
- *       QM_ERR_ARGUMENT. */
+ *       QM_ERR_ARGUMENT.
+ *   QM_OPT_DECODE_STREAMING_LOADS  0 (default): the decode kernels read K and V with the
+ *       non-temporal hint when the contexts of one call may exceed 512 MiB (twice the last-level
+ *       cache: less than that is partly still cached from the step before), and with plain loads
+ *       otherwise; 1: always plain; 2: always
+ *       non-temporal.  Same bits either way; other values make the call return QM_ERR_ARGUMENT. */
 enum {
     QM_OPT_PREFILL_SCORE_ROUNDING = 0,
     QM_OPT_DECODE_TILES_PER_BLOCK = 1,
     QM_OPT_PREFILL_KERNEL = 2,
-    QM_OPT_COUNT = 3
+    QM_OPT_DECODE_STREAMING_LOADS = 3,
+    QM_OPT_COUNT = 4
 };
 /* Returns QM_ERR_ARGUMENT for an unknown option or a negative value. */
 int32_t qm_set_option(int32_t option, int32_t value);

@@ -39,6 +39,13 @@ constexpr int kDecodeWaves = 4;
 constexpr int kRowStreams = 16;  // 4 waves x 4 DPP rows
 constexpr int kMaxTilesPerBlock = 64;
 constexpr int kMergeRound = 32;        // splits merged per round of loads in the merge kernel
+// Calls whose contexts may exceed this many bytes (streams x max_seq_len x bytes per token) read
+// K and V with the non-temporal hint.  Ragged batches of 256..4096 tokens, plain / non-temporal:
+// 16 streams (156 MiB read, bound 256 MiB) 32.5 / 32.8 us, 32 (290, 512) 54.2 / 55.2 us,
+// 48 (429, 768) 89.8 / 78.2 us, 64 (588, 1024) 119.4 / 104.9 us, 128 (1074, 2048) 210.5 / 190.5 us:
+// below about twice the 256 MiB last-level cache part of a context is still cached from the
+// step before and plain loads find it there.
+constexpr int64_t kStreamingContextBytes = 512ll << 20;
 
 struct DecodeParams {
     const uint16_t* query;        // [n_streams][q_heads][128]
@@ -73,6 +80,19 @@ struct DecodeParams {
 template <int G>
 __host__ __device__ constexpr int partial_floats() { return G * kDim + 2 * G; }
 
+// 16 bytes of K or V.  STREAMING adds the non-temporal hint: contexts much larger than the caches
+// are read once per step and should not displace anything on their way (measured on a 600 MB
+// read: 6.7-7.0 TB/s against 6.0-6.5 TB/s with plain loads).
+template <bool STREAMING>
+__device__ __forceinline__ uint4 kv_load(const uint16_t* p) {
+    if (STREAMING) {
+        typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+        const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+        return make_uint4(v.x, v.y, v.z, v.w);
+    }
+    return *reinterpret_cast<const uint4*>(p);
+}
+
 __device__ __forceinline__ uint4 load_or_zero(const uint16_t* p, bool valid) {
     uint4 r = make_uint4(0, 0, 0, 0);
     if (valid) r = *reinterpret_cast<const uint4*>(p);
@@ -82,7 +102,7 @@ __device__ __forceinline__ uint4 load_or_zero(const uint16_t* p, bool valid) {
 // STEP: the block first runs the QK-RMSNorm + RoPE of its query heads (and, if it owns the tile of
 // the new token, of the key head, appending K and V to the cache) — the reference's separate
 // launch_qk_norm_rope_cache_m1 (R17:17181) folded into the attention launch.
-template <int G, bool STEP>
+template <int G, bool STEP, bool STREAMING>
 __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodeParams prm, qm_kv_cache cache) {
     __shared__ __attribute__((aligned(16))) uint16_t sh_qrot[STEP ? G : 1][kDim];
     __shared__ float sh_acc[kRowStreams][G][kDim];
@@ -90,7 +110,11 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
     __shared__ float sh_l[kRowStreams][G];
     __shared__ int64_t sh_off[kMaxTilesPerBlock];   // element offset of each tile of this block, -1 = unreadable
 
-    const int split = blockIdx.x;
+    // Blocks go to the eight XCDs round-robin in linear order (x fastest).  With a power-of-two
+    // number of splits the XCD would be a function of the split index alone, and in a ragged batch
+    // the high splits are mostly empty: rotating the split by (head + stream) gives every XCD
+    // every split index (ragged 64 x 256..4096 at 16 tiles per block: 118 us without, 100 us with).
+    const int split = static_cast<int>((blockIdx.x + blockIdx.y + blockIdx.z) % gridDim.x);
     const int kvh = blockIdx.y;
     const int stream = blockIdx.z;
     const int tid = threadIdx.x;
@@ -213,8 +237,8 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
             int safe = min(max(token, key_start), key_end - 1) - first_token;
             safe = readable ? min(max(safe, 0), kTile - 1) : 0;
             const int64_t e = off + safe * kDim + col * 8;
-            kr[i] = *reinterpret_cast<const uint4*>(cache.k_pool + e);
-            vr[i] = *reinterpret_cast<const uint4*>(cache.v_pool + e);
+            kr[i] = kv_load<STREAMING>(cache.k_pool + e);
+            vr[i] = kv_load<STREAMING>(cache.v_pool + e);
         }
     };
 
@@ -441,14 +465,17 @@ inline DecodePlan plan_decode(int n_streams, int kv_heads, int max_seq_len) {
     const int64_t max_tiles = (static_cast<int64_t>(max_seq_len) + kTile - 1) / kTile + 1;
     int tiles_per_block = option_value(QM_OPT_DECODE_TILES_PER_BLOCK);
     if (tiles_per_block <= 0) {
-        // One tile per wave at least; otherwise 8 tiles (128 tokens, 64 KiB of K+V) per block:
-        // measured best for ragged batches (short blocks keep the tail of the grid short; the
-        // hardware dispatcher balances them), within 5 % of the best for uniform long contexts.
+        // One tile per wave at least; a block should not be shorter than it has to be (its set-up,
+        // the merge of its 16 row-streams and its partial record are fixed costs), yet the grid
+        // must keep a few thousand blocks so that ragged lengths balance: about 8 blocks per CU,
+        // at most 24 tiles (384 tokens, 192 KiB of K+V) per block.  Ragged 64 x 256..4096, three
+        // seeds: 4 tiles 126 / 132 / 111 us, 8: 106 / 113 / 93, 16: 101 / 97 / 88, 24: 100 / 96 / 88,
+        // 32: 100 / 95 / 87, 48: 102 / 99 / 89.
         const int64_t total = max_tiles * n_streams * kv_heads;
         int64_t t = total / (256 * 8);
         t = (t + 3) / 4 * 4;
         if (t < 4) t = 4;
-        if (t > 8) t = 8;
+        if (t > 24) t = 24;
         tiles_per_block = static_cast<int>(t);
     }
     if (tiles_per_block > kMaxTilesPerBlock) tiles_per_block = kMaxTilesPerBlock;
@@ -466,16 +493,21 @@ inline size_t decode_workspace_bytes(int n_streams, int q_heads, int kv_heads, i
          * sizeof(float);
 }
 
-template <int G>
-int32_t launch_decode(const DecodeParams& prm, const qm_kv_cache& cache, int n_streams,
-                      hipStream_t stream) {
+template <int G, bool STREAMING>
+void launch_split(const DecodeParams& prm, const qm_kv_cache& cache, int n_streams, hipStream_t stream) {
+    const dim3 grid(prm.max_splits, cache.kv_heads, n_streams);
     if (prm.step_q) {
-        hipLaunchKernelGGL((decode_split_kernel<G, true>), dim3(prm.max_splits, cache.kv_heads, n_streams),
-                           dim3(kDecodeThreads), 0, stream, prm, cache);
+        hipLaunchKernelGGL((decode_split_kernel<G, true, STREAMING>), grid, dim3(kDecodeThreads), 0, stream, prm, cache);
     } else {
-        hipLaunchKernelGGL((decode_split_kernel<G, false>), dim3(prm.max_splits, cache.kv_heads, n_streams),
-                           dim3(kDecodeThreads), 0, stream, prm, cache);
+        hipLaunchKernelGGL((decode_split_kernel<G, false, STREAMING>), grid, dim3(kDecodeThreads), 0, stream, prm, cache);
     }
+}
+
+template <int G>
+int32_t launch_decode(const DecodeParams& prm, const qm_kv_cache& cache, int n_streams, bool streaming,
+                      hipStream_t stream) {
+    if (streaming) launch_split<G, true>(prm, cache, n_streams, stream);
+    else launch_split<G, false>(prm, cache, n_streams, stream);
     int32_t rc = launch_status();
     if (rc != QM_OK) return rc;
     if (prm.max_splits > 1) {
@@ -500,6 +532,8 @@ int32_t decode_common(const uint16_t* query, const qm_kv_cache* cache, const int
     if (n_streams < 0 || n_streams > 65535 || cache->kv_heads > 65535) return QM_ERR_ARGUMENT;
     if (max_seq_len < 0) return QM_ERR_ARGUMENT;
     if (max_seq_len > cache_capacity(cache, max_pages)) return QM_ERR_SLOT_RANGE;
+    const int loads = option_value(QM_OPT_DECODE_STREAMING_LOADS);
+    if (loads < 0 || loads > 2) return QM_ERR_ARGUMENT;
     if (n_streams == 0) return QM_OK;
 
     const DecodePlan plan = plan_decode(n_streams, cache->kv_heads, max_seq_len);
@@ -531,11 +565,18 @@ int32_t decode_common(const uint16_t* query, const qm_kv_cache* cache, const int
         prm.step_position = step->step_position; prm.step_epsilon = step->step_epsilon;
     }
 
+    // Upper bound of the K and V bytes one call reads.
+    const int64_t context_bytes = static_cast<int64_t>(n_streams) * (seq_lens ? max_seq_len : key_end - key_start)
+                                * cache->kv_heads * kDim * 2 * 2;
+    bool streaming = context_bytes > kStreamingContextBytes;
+    if (loads == 1) streaming = false;
+    if (loads == 2) streaming = true;
+
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     switch (q_heads / cache->kv_heads) {
-        case 1: return launch_decode<1>(prm, *cache, n_streams, s);
-        case 2: return launch_decode<2>(prm, *cache, n_streams, s);
-        case 4: return launch_decode<4>(prm, *cache, n_streams, s);
+        case 1: return launch_decode<1>(prm, *cache, n_streams, streaming, s);
+        case 2: return launch_decode<2>(prm, *cache, n_streams, streaming, s);
+        case 4: return launch_decode<4>(prm, *cache, n_streams, streaming, s);
     }
     return QM_ERR_GEOMETRY;
 }

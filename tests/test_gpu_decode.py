@@ -117,6 +117,40 @@ def test_decode_ragged_single_split_path(oracle, qm, dev):
     assert not got[0].any() and not got[5].any()
 
 
+def test_decode_load_kinds_give_the_same_bits(oracle, qm, dev):
+    """Plain and non-temporal K/V loads differ in cache policy only; an unknown choice is an error."""
+    lens = [0, 1, 17, 255, 256, 257, 4096, 2000, 33]
+    got = {}
+    try:
+        for loads in (1, 2):
+            qm.set_option(qm.OPT_DECODE_STREAMING_LOADS, loads)
+            got[loads], want, status, _ = _ragged(oracle, qm, dev, lens, seed=41)
+            assert status == 0
+            assert max_abs_err(oracle, got[loads], want[1]) <= TOL
+        assert np.array_equal(got[1], got[2])
+        qm.set_option(qm.OPT_DECODE_STREAMING_LOADS, 3)
+        with pytest.raises(qm.QmError) as err:
+            _ragged(oracle, qm, dev, [5, 6], seed=1)
+        assert err.value.code == -5
+    finally:
+        qm.set_option(qm.OPT_DECODE_STREAMING_LOADS, 0)
+
+
+@pytest.mark.parametrize("tiles", [4, 8, 16, 24, 64])
+def test_decode_split_granularities(oracle, qm, dev, tiles):
+    """Every split size (powers of two make the split count one too: the rotated block-to-split
+    mapping must still visit each split exactly once) gives the oracle's result."""
+    lens = [4096, 0, 1, 300, 1024, 4095, 16, 2049]
+    qm.set_option(qm.OPT_DECODE_TILES_PER_BLOCK, tiles)
+    try:
+        got, want, status, _ = _ragged(oracle, qm, dev, lens, seed=52)
+    finally:
+        qm.set_option(qm.OPT_DECODE_TILES_PER_BLOCK, 0)
+    assert status == 0
+    assert max_abs_err(oracle, got, want[1]) <= TOL
+    assert not got[1].any()
+
+
 def test_decode_page_permutation_is_bit_identical(oracle, qm, dev):
     import torch
     lens = np.array([700, 33, 1500], dtype=np.int32)
