@@ -11,21 +11,16 @@
 // 8-slot blocks XOR-swizzled per 16 rows so both the transposing writes and the fragment reads
 // are conflict-free).
 //
-// Occupancy and what bounds the kernel.  A wave cannot issue VALU work in the shadow of its own
-// MFMAs (measured: one MFMA plus eight independent FMAs take the sum of both), so the matrix pipe
-// and the VALU only overlap between waves, and with two waves per SIMD whose phases are long (eight
-// MFMAs, then about 150 VALU instructions, then eight MFMAs) that overlap is small as well: a
-// synthetic pair of such waves takes 2 045 cycles per step against 2 420 serial and 1 216 ideal.
-// The kernel therefore stays within 256 registers and 72 KB of LDS so that two blocks share a CU
-// and fill each other's waits, and otherwise keeps the instruction count per key tile low.
-// Variants that were measured and dropped (batch 4 x 1024 tokens / 4 x 4096 tokens, this one:
-// 42 us / 381 us): a software pipeline inside the wave with three LDS stages and 316 registers,
-// one wave per SIMD (51 us / 467 us); eight-wave blocks whose two wave groups split each key tile
-// and merge through LDS, with phase-skewed groups and each block taking a heavy and a light
-// query tile (41 us / 421 us: the longest block is halved, but the groups meet at a barrier per
-// tile and run in step).  At batch 4 x 1024 tokens the time is the serial length of the blocks
-// that own the last query tiles (16 key tiles at 1.7 us) plus a 4 us start in which every block
-// fetches its first tiles from HBM at once, not chip throughput.
+// Three kernels share this file and give the same bits: the uniform waves described here (the
+// compiler's order inside a wave: all MFMAs of a product, then all of the softmax arithmetic), the
+// wave pairs (matrix waves and softmax waves), and the interleaved waves, which alternate MFMAs
+// and softmax arithmetic instruction by instruction and are the ones the host launches by
+// default; their comments say what was measured.  This kernel stays within 256 registers and
+// 72 KB of LDS so that two blocks share a CU and fill each other's waits.
+// Variants of it that were measured and dropped (batch 4 x 1024 tokens / 4 x 4096 tokens, this
+// one: 42 us / 381 us): three LDS stages with 316 registers, one wave per SIMD (51 us / 467 us);
+// eight-wave blocks whose two wave groups split each key tile and merge through LDS (41 us /
+// 421 us: the longest block is halved, but the groups meet at a barrier per tile and run in step).
 //
 // Lazy rescale.  The running maximum of a column is only raised when a chunk exceeds it by more
 // than kRescaleSlack (then O and the running sum are rescaled); otherwise probabilities are taken
@@ -87,6 +82,7 @@ struct PrefillParams {
     int seq;
     int kv_heads;
     int n_qtiles;
+    int heavy_groups;            // (interleaved kernel) leading groups of blocks, heaviest query tile first; the rest ascend
     float scale;
 };
 
@@ -510,13 +506,10 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_causal_kernel(PrefillPa
 // batch 4 x 1024 tokens, 144.6 against 138.5 for 16 x 1024, 398 against 385 for 4 x 4096; with
 // fp32 scores 37.4 / 147.9 / 409 against 37.4 / 116.4 / 334.  A stage lasts about 1520 cycles
 // in either design.  Counters (4 x 4096): per SIMD and stage the MFMAs are busy for 490 cycles
-// and the VALU for 850, and for only 150 of these both at once: an MFMA of one wave and VALU
-// work of another wave on the same SIMD run one after the other far more than side by side,
-// so the stage costs about the sum of the two whoever issues them.  What the pairs gain is
-// latency (one block per CU needs fewer blocks to fill the chip, and a block's own chain is
-// shorter), which is why they win on the small grid and lose where the chip is full anyway.
-// The host picks by grid size.  What would move both designs is fewer VALU operations per score
-// (now about 13, of which 4 are the quarter-rate exponential and 6 the two bf16 roundings).
+// and the VALU for 850, and for only 150 of these both at once: with phases this long (eight
+// MFMAs, then about 150 VALU instructions) the two kinds of work mostly take turns, whoever
+// issues them, and a stage costs about their sum.  What the pairs gain is latency (one block
+// per CU needs fewer blocks to fill the chip, and a block's own chain is shorter).
 constexpr int kSpThreads = 512;
 constexpr int kKR = kDim * 2;                                    // bytes of a K row in LDS (unpadded, slots swizzled)
 constexpr int kSpKTile = kBN * kKR;
@@ -1035,6 +1028,567 @@ __global__ __launch_bounds__(kSpThreads, 2) void prefill_sp_kernel(PrefillParams
     else prefill_sp_body<false, ROUND>(prm, cache, sp_smem, qt, bid % pairs);
 }
 
+
+// ======================================================================================================
+// The interleaved kernel: each of the four waves of a block runs the matrix and the softmax work
+// of its 16 rows x 2 heads as ONE software-pipelined instruction stream.
+//
+// Independent MFMAs and VALU instructions of the same wave do overlap when they alternate at
+// fine grain (measured: 16 x (one MFMA, eight FMAs) take 684 cycles against 512 + 616 one after
+// the other), and the compiler's own order — all MFMAs of a product, then all of the softmax —
+// leaves that unused.  Stage j of a wave therefore holds three things that do not depend on
+// one another: the P.V MFMAs of chunk j - 1, the softmax arithmetic of chunk j, and the S^T MFMAs
+// of chunk j + 1; the source alternates one MFMA with one slice of the softmax (a score pair) and
+// pins that order with scheduling barriers.  Staging is that of the wave pairs (K and V tiles go
+// straight from global memory into LDS, V is transposed by the LDS read) with two buffers per
+// ring and one block barrier per 64-key tile: 64 KiB of LDS, so that two blocks share a CU.
+// The diagonal tile is finished outside the pipeline, and blocks of the first query tile (one
+// diagonal tile, split-precision P) run the uniform-waves body.
+constexpr int kIlRing = 2 * kSpKTile;                       // two tiles of K, likewise of V
+constexpr int kIlSmemBytes = (2 * kIlRing > static_cast<int>(sizeof(PfStage)) * kPfStages)
+                                 ? 2 * kIlRing : static_cast<int>(sizeof(PfStage)) * kPfStages;
+static_assert(2 * kIlRing >= 4 * 32 * kOS * 2, "the output staging area reuses the rings");
+
+template <bool ROUND>
+__device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const qm_kv_cache& cache,
+                                                unsigned char* il_smem, int qt, int bh) {
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+    unsigned char* lds_k = il_smem;                 // [2][64 rows][256 B]
+    unsigned char* lds_v = il_smem + kIlRing;       // [2][64 rows][256 B]
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int col = lane & 31;
+    const int grp = lane >> 5;
+
+    const int b = bh / prm.kv_heads;
+    const int kvh = bh % prm.kv_heads;
+    const int S = prm.seq;
+    const int q_heads = 2 * prm.kv_heads;
+    const int q0 = qt * kBM;
+    const int my_row = q0 + 16 * wave + (col & 15);
+    const int my_head = 2 * kvh + (col >> 4);
+    const int wave_last_row = q0 + 16 * wave + 15;
+
+    const int64_t kv_base = static_cast<int64_t>(b) * prm.kv_stride_batch + static_cast<int64_t>(kvh) * prm.kv_stride_head;
+    const int kv_row32 = static_cast<int>(prm.kv_stride_token);
+
+    // ---- K/V rows of the diagonal tile for the pages: requested first, written after the first wait ----
+    const bool to_pages = prm.has_cache != 0;
+    int phys[4] = {-1, -1, -1, -1};
+    uint4 kx[4], vx[4];
+    uint32_t page_err = 0;
+    if (to_pages) {
+        const int32_t* table = prm.page_table ? prm.page_table + static_cast<int64_t>(b) * prm.pages.max_pages : nullptr;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int key = qt * kBN + (tid >> 4) + 16 * i;
+            kx[i] = vx[i] = make_uint4(0, 0, 0, 0);
+            if (key < S) {
+                const int page = page_of(prm.pages, key);
+                if (page >= prm.pages.max_pages) page_err |= QM_STATUS_BAD_POSITION;
+                else phys[i] = table ? table[page] : page;
+                const int64_t off = kv_base + static_cast<int64_t>(key) * prm.kv_stride_token + 8 * (tid & 15);
+                kx[i] = *reinterpret_cast<const uint4*>(prm.k + off);
+                vx[i] = *reinterpret_cast<const uint4*>(prm.v + off);
+            }
+        }
+    }
+
+    // ---- staging: as in the wave pairs (slot p of K row r holds piece p ^ (r % 16), of V row r piece
+    // p ^ 4 (r % 4)); wave w fills rows 4 w + l / 16 + 16 j of a tile ----
+    const int k_row = 4 * wave + (lane >> 4);
+    const uint16_t* k_src = prm.k + kv_base + 8 * ((lane & 15) ^ (k_row & 15));
+    const uint16_t* v_src = prm.v + kv_base + 8 * ((lane & 15) ^ (4 * (k_row & 3)));
+    const uint32_t row_bytes = static_cast<uint32_t>(kv_row32) * 2u;
+    // piece j of a tile: one global_load_lds (16 bytes per lane, no registers) fills rows 4 w + 16 j .. + 3; a key
+    // at or beyond S is redirected to the last key (such keys only occur masked)
+    auto load_piece = [&](const uint16_t* src, unsigned char* ring, int tile, int slot, int j) {
+        unsigned char* dst = ring + slot * kSpKTile + (4 * wave + 16 * j) * kKR;
+        const int key = min(tile * kBN + k_row + 16 * j, S - 1);
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned char*>(src)
+                                             + static_cast<uint64_t>(static_cast<uint32_t>(key) * row_bytes),
+                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    };
+    auto load_k = [&](int tile, int slot) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) load_piece(k_src, lds_k, tile, slot, j);
+    };
+    auto load_v = [&](int tile, int slot) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) load_piece(v_src, lds_v, tile, slot, j);
+    };
+
+    load_k(0, 0);
+    load_v(0, 0);
+    load_k(1, 1);                                    // qt >= 1 here: tile 1 exists
+    bf16x8_t qf[8];
+    {
+        const uint16_t* qp = prm.q + ((static_cast<int64_t>(b) * S + my_row) * q_heads + my_head) * kDim + 8 * grp;
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb) {
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (my_row < S) raw = *reinterpret_cast<const uint4*>(qp + 16 * kb);
+            qf[kb] = __builtin_bit_cast(bf16x8_t, raw);
+        }
+    }
+    f32x16_t o[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[dt][r] = 0.0f;
+    wait_vm<0>();
+    if (to_pages) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int key = qt * kBN + (tid >> 4) + 16 * i;
+            if (key >= S || phys[i] == -1) continue;
+            if (phys[i] < 0 || phys[i] >= cache.n_pages) {
+                page_err |= QM_STATUS_BAD_PAGE;
+                continue;
+            }
+            const int page = page_of(prm.pages, key);
+            const int64_t off = static_cast<int64_t>(phys[i]) * cache.stride_page + static_cast<int64_t>(kvh) * cache.stride_head
+                              + static_cast<int64_t>(key - page * prm.pages.page_size) * kDim + 8 * (tid & 15);
+            *reinterpret_cast<uint4*>(cache.k_pool + off) = kx[i];
+            *reinterpret_cast<uint4*>(cache.v_pool + off) = vx[i];
+        }
+        if (page_err && prm.status) atomicOr(prm.status, page_err);
+    }
+    lds_barrier();
+
+    // ---- fragment reads, all as assembly: the compiler would make an LDS read wait for every
+    // global_load_lds in flight, and it must not move them across the barriers either.  Their results
+    // are taken only through k_arrived / v_arrived, which wait for them. ----
+    // K fragment kb of chunk (slot, h): row 32 h + col, slot (2 kb + grp) ^ (col % 16).
+    // V^T fragment (kg, dt): two transposing reads, keys 16 kg + 4 grp + 0..3 and + 8 (see the wave pairs).
+    uint32_t kaddr[8], vaddr[4];
+    {
+        const uint32_t k0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)lds_k))
+                          + col * kKR + 16 * (grp ^ (col & 15));
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb) kaddr[kb] = k0 ^ (32 * kb);
+        const int tr_key = (lane >> 2) & 3;
+        const uint32_t v0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)lds_v))
+                          + (4 * grp + tr_key) * kKR + 16 * (2 * (col >> 4) + ((lane & 3) >> 1)) + 8 * (lane & 1);
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) vaddr[dt] = v0 ^ (64 * (dt ^ tr_key));
+    }
+    struct KRaw { u32x4_t f[8]; };
+    struct VRaw { unsigned long long a[8], c[8]; };
+    // Requests come in halves: K fragments 4 h .. 4 h + 3 (k blocks) and the V^T fragments of 16-key group h.
+    // `dyn`: bytes added at run time (0 in the pipeline, where the buffer is a template constant).
+    auto k_request_half = [&](uint32_t dyn, auto imm, auto half, KRaw& raw) {
+#pragma unroll
+        for (int kb = 4 * decltype(half)::value; kb < 4 * decltype(half)::value + 4; ++kb) {
+            const uint32_t at = kaddr[kb] + dyn;
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(raw.f[kb]) : "v"(at), "n"(decltype(imm)::value));
+        }
+    };
+    auto v_request_half = [&](uint32_t dyn, auto imm, auto half, VRaw& raw) {
+        constexpr int kg = decltype(half)::value;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+            const uint32_t at = vaddr[dt] + dyn;
+            asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(raw.a[4 * kg + dt]) : "v"(at), "n"(decltype(imm)::value + 16 * kg * kKR));
+            asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(raw.c[4 * kg + dt]) : "v"(at), "n"(decltype(imm)::value + (16 * kg + 8) * kKR));
+        }
+    };
+    auto k_request = [&](uint32_t dyn, auto imm, KRaw& raw) {
+        k_request_half(dyn, imm, int_c<0>{}, raw);
+        k_request_half(dyn, imm, int_c<1>{}, raw);
+    };
+    auto v_request = [&](uint32_t dyn, auto imm, VRaw& raw) {
+        v_request_half(dyn, imm, int_c<0>{}, raw);
+        v_request_half(dyn, imm, int_c<1>{}, raw);
+    };
+    auto v_unpack = [&](const VRaw& raw, int j) -> bf16x8_t {
+        const uint4 both_halves = make_uint4(static_cast<uint32_t>(raw.a[j]), static_cast<uint32_t>(raw.a[j] >> 32),
+                                             static_cast<uint32_t>(raw.c[j]), static_cast<uint32_t>(raw.c[j] >> 32));
+        return __builtin_bit_cast(bf16x8_t, both_halves);
+    };
+    // Waits until at most `pending` LDS reads are outstanding, then hands out half h of both sets.
+    auto half_arrived = [&](auto half, auto pending, KRaw& kraw, VRaw& vraw, bf16x8_t (&kf)[8], bf16x8_t (&vf)[8]) {
+        constexpr int h = 4 * decltype(half)::value;
+        asm volatile("s_waitcnt lgkmcnt(%12)"
+                     : "+v"(kraw.f[h]), "+v"(kraw.f[h + 1]), "+v"(kraw.f[h + 2]), "+v"(kraw.f[h + 3]),
+                       "+v"(vraw.a[h]), "+v"(vraw.a[h + 1]), "+v"(vraw.a[h + 2]), "+v"(vraw.a[h + 3]),
+                       "+v"(vraw.c[h]), "+v"(vraw.c[h + 1]), "+v"(vraw.c[h + 2]), "+v"(vraw.c[h + 3])
+                     : "n"(decltype(pending)::value)
+                     : "memory");
+#pragma unroll
+        for (int i = h; i < h + 4; ++i) {
+            kf[i] = __builtin_bit_cast(bf16x8_t, kraw.f[i]);
+            vf[i] = v_unpack(vraw, i);
+        }
+    };
+    auto k_arrived = [&](KRaw& raw, bf16x8_t (&kf)[8]) {
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(raw.f[0]), "+v"(raw.f[1]), "+v"(raw.f[2]), "+v"(raw.f[3]), "+v"(raw.f[4]), "+v"(raw.f[5]),
+                       "+v"(raw.f[6]), "+v"(raw.f[7])
+                     :
+                     : "memory");
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb) kf[kb] = __builtin_bit_cast(bf16x8_t, raw.f[kb]);
+    };
+    auto v_arrived = [&](VRaw& raw, bf16x8_t (&vf)[8]) {
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(raw.a[0]), "+v"(raw.a[1]), "+v"(raw.a[2]), "+v"(raw.a[3]), "+v"(raw.a[4]), "+v"(raw.a[5]),
+                       "+v"(raw.a[6]), "+v"(raw.a[7]), "+v"(raw.c[0]), "+v"(raw.c[1]), "+v"(raw.c[2]), "+v"(raw.c[3]),
+                       "+v"(raw.c[4]), "+v"(raw.c[5]), "+v"(raw.c[6]), "+v"(raw.c[7])
+                     :
+                     : "memory");
+#pragma unroll
+        for (int j = 0; j < 8; ++j) vf[j] = v_unpack(raw, j);
+    };
+
+    // ---- softmax state and slices (the arithmetic of the uniform waves, cut into score pairs) ----
+    const float coef = ROUND ? kLog2e : prm.scale * kLog2e;
+    const float slack = ROUND ? kRescaleSlack : kRescaleSlack / prm.scale;
+    float m_run = -INFINITY, l_run = 0.0f, m_scaled = 0.0f;
+    // roundings (and, on the diagonal, the causal mask) of the score pair r, r + 1 in place
+    auto score_pair = [&](f32x16_t& s, int r, float& mx, auto masked, int lim) {
+        float x0 = s[r], x1 = s[r + 1];
+        if (ROUND) {
+            round_bf16_pair(x0, x1, x0, x1);
+            round_bf16_pair(x0 * prm.scale, x1 * prm.scale, x0, x1);
+        }
+        if (decltype(masked)::value) {
+            const int e = 8 * (r >> 2) + (r & 3);
+            if (e > lim) x0 = -INFINITY;
+            if (e + 1 > lim) x1 = -INFINITY;
+        }
+        s[r] = x0;
+        s[r + 1] = x1;
+        mx = fmaxf(mx, fmaxf(x0, x1));
+    };
+    auto update_max = [&](float mx) {
+        const bool need = __builtin_amdgcn_ballot_w64(mx > m_run + slack) != 0;
+        if (need) {
+            const float m_new = fmaxf(m_run, mx);
+            const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
+            const float alpha = fast_exp2((m_run - m_ref) * coef);
+            m_run = m_new;
+            m_scaled = m_ref * coef;
+            l_run *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+        }
+    };
+    auto prob_pair = [&](const f32x16_t& s, int r, uint32_t& packed, float& psum) {
+        const float e0 = fast_exp2(fmaf(s[r], coef, -m_scaled));
+        const float e1 = fast_exp2(fmaf(s[r + 1], coef, -m_scaled));
+        packed = pack_bf16_pair(e0, e1);
+        psum = dot2_bf16(packed, 0x3f803f80U, psum);          // the sum of what the MFMA multiplies
+    };
+    struct PPair { bf16x8_t g[2]; };
+    auto make_p = [&](const uint32_t (&hi)[8], PPair& p) {
+        p.g[0] = __builtin_bit_cast(bf16x8_t, make_uint4(hi[0], hi[1], hi[2], hi[3]));
+        p.g[1] = __builtin_bit_cast(bf16x8_t, make_uint4(hi[4], hi[5], hi[6], hi[7]));
+    };
+
+    // ---- one stage of the pipeline ----
+    // in:  s_cur = raw S^T of chunk j; p_prev = P of chunk j - 1; vraw = V^T fragments of chunk j - 1 and
+    //      kraw = K fragments of chunk j + 1, both requested (first halves a half stage before the second)
+    // out: s_next = raw S^T of chunk j + 1; p_cur = P of chunk j; vraw = V^T fragments of chunk j (from `v_imm`)
+    //      and kraw = K fragments of chunk j + 2 (from `k_imm`), requested
+    // What the order of the instructions answers to (all measured on this chip):
+    //  - dependent VALU instructions issue 8 cycles apart, independent ones 4 (the exponential takes 12), and
+    //    the arithmetic of one score pair is a single chain six instructions deep: the stage works on two
+    //    pairs at a time, level by level, so that an independent instruction sits between dependent ones;
+    //  - a dependent MFMA waits for the one before it to finish: the S^T MFMAs (one accumulator) alternate
+    //    with the P.V MFMAs (four accumulators), one MFMA per half group of VALU work;
+    //  - eight global_load_lds in a row take 500 cycles to issue: the loads of a tile are handed out one per
+    //    group (`vmem`), and the block barrier of the tile (`sync`) comes after the first group, when the
+    //    LDS reads it has to wait for have long landed;
+    //  - the chain from the maxima to the branch on them is 14 dependent instructions: two MFMAs are issued
+    //    ahead of it.  If the running maximum is raised, O is rescaled at the end of the stage, after the last
+    //    P.V MFMA of chunk j - 1 (whose P is relative to the old maximum).
+    // Scheduling fences pin the order.
+    auto fence = []() { __builtin_amdgcn_sched_barrier(0); };
+    auto stage = [&](f32x16_t& s_cur, f32x16_t& s_next, const PPair& p_prev, PPair& p_cur, KRaw& kraw, VRaw& vraw,
+                     auto k_imm, auto v_imm, auto&& sync, auto&& vmem) {
+        bf16x8_t kf[8], vf[8];
+        auto pv_mfma = [&](int i) {
+            o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i], p_prev.g[i >> 2], o[i & 3], 0, 0, 0);
+        };
+        auto qk_mfma = [&](int i) { s_next = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qf[i], s_next, 0, 0, 0); };
+        half_arrived(int_c<0>{}, int_c<12>{}, kraw, vraw, kf, vf);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s_next[r] = 0.0f;
+        float mx_a = -INFINITY, mx_b = -INFINITY;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int ra = 4 * g, rb = 4 * g + 2;              // pair a = scores ra, ra + 1; pair b = rb, rb + 1
+            pv_mfma(g);
+            fence();
+            if (ROUND) {
+                const float xa0 = s_cur[ra], xa1 = s_cur[ra + 1], xb0 = s_cur[rb], xb1 = s_cur[rb + 1];
+                const uint32_t pa = pack_bf16_pair(xa0, xa1);
+                const uint32_t pb = pack_bf16_pair(xb0, xb1);
+                fence();
+                const float ua0 = lo_bf16(pa), ua1 = hi_bf16(pa), ub0 = lo_bf16(pb), ub1 = hi_bf16(pb);
+                fence();
+                const float ya0 = ua0 * prm.scale, ya1 = ua1 * prm.scale;
+                fence();
+                qk_mfma(g);
+                fence();
+                const float yb0 = ub0 * prm.scale, yb1 = ub1 * prm.scale;
+                fence();
+                const uint32_t qa = pack_bf16_pair(ya0, ya1);
+                const uint32_t qb = pack_bf16_pair(yb0, yb1);
+                fence();
+                float za0 = lo_bf16(qa), za1 = hi_bf16(qa), zb0 = lo_bf16(qb), zb1 = hi_bf16(qb);
+                fence();
+                // The running maxima are taken over the raw scores (the roundings are monotonic and the host
+                // sends a negative scale elsewhere), one v_max3 each: the compiler's fmaxf first quiets every
+                // operand with an instruction of its own.  The rounded values pass through the statements so
+                // that these follow the roundings — whose reads of the MFMA results the compiler guards — and
+                // so that the roundings stay here instead of sinking to where they are used.
+                asm volatile("v_max3_f32 %0, %0, %3, %4" : "+v"(mx_a), "+v"(za0), "+v"(za1) : "v"(xa0), "v"(xa1));
+                asm volatile("v_max3_f32 %0, %0, %3, %4" : "+v"(mx_b), "+v"(zb0), "+v"(zb1) : "v"(xb0), "v"(xb1));
+                s_cur[ra] = za0; s_cur[ra + 1] = za1; s_cur[rb] = zb0; s_cur[rb + 1] = zb1;
+            } else {
+                mx_a = __builtin_fmaxf(mx_a, __builtin_fmaxf(s_cur[ra], s_cur[ra + 1]));
+                fence();
+                qk_mfma(g);
+                fence();
+                mx_b = __builtin_fmaxf(mx_b, __builtin_fmaxf(s_cur[rb], s_cur[rb + 1]));
+            }
+            fence();
+            if (g == 0) sync();
+            vmem(g);
+            fence();
+        }
+        k_request_half(0u, k_imm, int_c<0>{}, kraw);
+        v_request_half(0u, v_imm, int_c<0>{}, vraw);
+        half_arrived(int_c<1>{}, int_c<12>{}, kraw, vraw, kf, vf);
+        qk_mfma(4);
+        pv_mfma(4);
+        fence();
+
+        float mx = __builtin_fmaxf(mx_a, mx_b);
+        if (ROUND) mx = round_bf16(round_bf16(mx) * prm.scale);
+        mx = halves_max(mx);
+        const bool need = __builtin_amdgcn_ballot_w64(mx > m_run + slack) != 0;
+        float alpha = 1.0f;
+        if (need) {
+            const float m_new = fmaxf(m_run, mx);
+            const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
+            alpha = fast_exp2((m_run - m_ref) * coef);
+            m_run = m_new;
+            m_scaled = m_ref * coef;
+            l_run *= alpha;
+        }
+
+        uint32_t hi[8];
+        float psum = 0.0f;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int ra = 4 * g, rb = 4 * g + 2;
+            if (g > 0) pv_mfma(4 + g);
+            fence();
+            const float ta0 = fmaf(s_cur[ra], coef, -m_scaled), ta1 = fmaf(s_cur[ra + 1], coef, -m_scaled);
+            const float tb0 = fmaf(s_cur[rb], coef, -m_scaled), tb1 = fmaf(s_cur[rb + 1], coef, -m_scaled);
+            fence();
+            const float ea0 = fast_exp2(ta0), ea1 = fast_exp2(ta1);
+            fence();
+            if (g < 3) qk_mfma(5 + g);
+            fence();
+            const float eb0 = fast_exp2(tb0), eb1 = fast_exp2(tb1);
+            fence();
+            hi[2 * g] = pack_bf16_pair(ea0, ea1);
+            hi[2 * g + 1] = pack_bf16_pair(eb0, eb1);
+            fence();
+            psum = dot2_bf16(hi[2 * g], 0x3f803f80U, psum);          // the sum of what the MFMA multiplies
+            psum = dot2_bf16(hi[2 * g + 1], 0x3f803f80U, psum);
+            // (an empty statement that keeps this arithmetic here: its results are only used by the next
+            // stage, and the compiler would sink it below the branch at the end of this one)
+            asm volatile("" : "+v"(hi[2 * g]), "+v"(hi[2 * g + 1]), "+v"(psum));
+            fence();
+            vmem(4 + g);
+            fence();
+        }
+        k_request_half(0u, k_imm, int_c<1>{}, kraw);
+        v_request_half(0u, v_imm, int_c<1>{}, vraw);
+        make_p(hi, p_cur);
+        l_run += psum;
+        if (need) {
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+        }
+    };
+
+    // ---- prologue: S^T of chunk (0, 0); K fragments of chunk (0, 1) requested; nothing to multiply yet ----
+    f32x16_t s_a, s_b;
+    PPair p_a, p_b;
+    KRaw kraw;
+    VRaw vraw;
+    {
+        bf16x8_t kf[8];
+        k_request(0u, int_c<0>{}, kraw);
+        k_arrived(kraw, kf);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s_a[r] = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb) s_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb], qf[kb], s_a, 0, 0, 0);
+        k_request(0u, int_c<32 * kKR>{}, kraw);
+        // (the stages count outstanding reads in halves of twelve; these eight are taken here)
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(kraw.f[0]), "+v"(kraw.f[1]), "+v"(kraw.f[2]), "+v"(kraw.f[3]), "+v"(kraw.f[4]), "+v"(kraw.f[5]),
+                       "+v"(kraw.f[6]), "+v"(kraw.f[7])
+                     :
+                     : "memory");
+#pragma unroll
+        for (int j = 0; j < 8; ++j) vraw.a[j] = vraw.c[j] = 0ull;
+        p_b.g[0] = p_b.g[1] = __builtin_bit_cast(bf16x8_t, make_uint4(0, 0, 0, 0));
+    }
+
+    // ---- the tiles before the diagonal: tile t lives in buffer t % 2 of either ring.  During its first stage
+    // (after the tile's barrier: every wave has taken the last fragments of tile t - 1 and of K tile t) the
+    // wave requests K of tile t + 2 into the buffer of K tile t and V of tile t + 1 into the buffer of V tile
+    // t - 1; both are first read during tile t + 1, after its barrier. ----
+    auto tile_body = [&](int t, auto parity) {
+        constexpr int cur = decltype(parity)::value;
+        constexpr int nxt = cur ^ 1;
+        const bool more_k = t + 2 <= qt;
+        // stage (t, 0): P.V of chunk (t - 1, 1), softmax of (t, 0), S^T of (t, 1); requests V(t, 0) and K(t + 1, 0)
+        stage(s_a, s_b, p_b, p_a, kraw, vraw, int_c<nxt * kSpKTile>{}, int_c<cur * kSpKTile>{},
+              [&]() {
+                  wait_vm<0>();
+                  lds_barrier();
+              },
+              [&](int i) {
+                  if (i < 4) {
+                      if (more_k) load_piece(k_src, lds_k, t + 2, cur, i);
+                  } else {
+                      load_piece(v_src, lds_v, t + 1, nxt, i - 4);
+                  }
+              });
+        // stage (t, 1): P.V of chunk (t, 0), softmax of (t, 1), S^T of (t + 1, 0); requests V(t, 1) and K(t + 1, 1)
+        stage(s_b, s_a, p_a, p_b, kraw, vraw, int_c<nxt * kSpKTile + 32 * kKR>{}, int_c<cur * kSpKTile + 32 * kKR>{},
+              []() {}, [](int) {});
+    };
+    for (int t = 0; t < qt; t += 2) {
+        tile_body(t, int_c<0>{});
+        if (t + 1 < qt) tile_body(t + 1, int_c<1>{});
+    }
+    wait_vm<0>();
+    lds_barrier();                                   // V of the diagonal tile has landed for every wave
+
+    // ---- drain: P.V of chunk (qt - 1, 1), then the diagonal tile chunk by chunk ----
+    const uint32_t diag_slot = static_cast<uint32_t>((qt & 1) * kSpKTile);
+    {
+        bf16x8_t vf[8];
+        v_arrived(vraw, vf);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i], p_b.g[i >> 2], o[i & 3], 0, 0, 0);
+    }
+    auto diag_chunk = [&](f32x16_t& s, auto h, int key_base) {
+        VRaw vr;
+        bf16x8_t vf[8];
+        v_request(diag_slot, int_c<decltype(h)::value * 32 * kKR>{}, vr);
+        const int lim = my_row - key_base - 4 * grp;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) score_pair(s, 2 * i, mx, bool_c<true>{}, lim);
+        mx = halves_max(mx);
+        update_max(mx);
+        uint32_t hi[8];
+        float psum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) prob_pair(s, 2 * i, hi[i], psum);
+        l_run += psum;
+        PPair p;
+        make_p(hi, p);
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(vr.a[0]), "+v"(vr.a[1]), "+v"(vr.a[2]), "+v"(vr.a[3]), "+v"(vr.a[4]), "+v"(vr.a[5]),
+                       "+v"(vr.a[6]), "+v"(vr.a[7]), "+v"(vr.c[0]), "+v"(vr.c[1]), "+v"(vr.c[2]), "+v"(vr.c[3]),
+                       "+v"(vr.c[4]), "+v"(vr.c[5]), "+v"(vr.c[6]), "+v"(vr.c[7])
+                     :
+                     : "memory");
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint4 both_halves = make_uint4(static_cast<uint32_t>(vr.a[j]), static_cast<uint32_t>(vr.a[j] >> 32),
+                                                 static_cast<uint32_t>(vr.c[j]), static_cast<uint32_t>(vr.c[j] >> 32));
+            vf[j] = __builtin_bit_cast(bf16x8_t, both_halves);
+        }
+        // a 16-key group wholly after the wave's last row is masked for every column: skipped, so that
+        // later tokens are not even multiplied by zero
+#pragma unroll
+        for (int kg = 0; kg < 2; ++kg) {
+            if (key_base + 16 * kg > wave_last_row) continue;
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * kg + dt], p.g[kg], o[dt], 0, 0, 0);
+        }
+    };
+    // after an even number of stages the raw scores of the diagonal's first chunk are in s_a and the K
+    // fragments of its second chunk have been requested
+    diag_chunk(s_a, int_c<0>{}, qt * kBN);
+    {
+        bf16x8_t kf[8];
+        k_arrived(kraw, kf);                         // (every wave takes them, so that no read is left pending)
+        if (qt * kBN + 32 <= wave_last_row) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_b[r] = 0.0f;
+#pragma unroll
+            for (int kb = 0; kb < 8; ++kb) s_b = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb], qf[kb], s_b, 0, 0, 0);
+            diag_chunk(s_b, int_c<1>{}, qt * kBN + 32);
+        }
+    }
+    lds_barrier();   // every wave is done with the rings: they become the output staging area
+
+    // ---- normalise, stage through LDS, write 16 bytes per lane ----
+    const float l_tot = halves_sum(l_run);
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    uint16_t* stage_out = reinterpret_cast<uint16_t*>(il_smem) + wave * 32 * kOS;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+            const int d0 = 32 * dt + 8 * rq + 4 * grp;
+            uint2 packed;
+            packed.x = pack_bf16_pair(o[dt][4 * rq + 0] * inv, o[dt][4 * rq + 1] * inv);
+            packed.y = pack_bf16_pair(o[dt][4 * rq + 2] * inv, o[dt][4 * rq + 3] * inv);
+            *reinterpret_cast<uint2*>(&stage_out[col * kOS + d0]) = packed;
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0);   // the wave reads back only what it wrote itself
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int c = 4 * it + (lane >> 4);
+        const int piece = lane & 15;
+        const int row = q0 + 16 * wave + (c & 15);
+        const int head = 2 * kvh + (c >> 4);
+        if (row < S) {
+            const uint4 val = *reinterpret_cast<const uint4*>(&stage_out[c * kOS + 8 * piece]);
+            *reinterpret_cast<uint4*>(prm.out + ((static_cast<int64_t>(b) * S + row) * q_heads + head) * kDim + 8 * piece) = val;
+        }
+    }
+}
+
+template <bool ROUND>
+__global__ __launch_bounds__(kPfThreads, 2) void prefill_il_kernel(PrefillParams prm, qm_kv_cache cache) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char il_smem[];
+    const int pairs = prm.batch * prm.kv_heads;
+    const int bid = blockIdx.x;
+    // Heaviest query tile first; when the whole grid is resident at once (at most two blocks per CU,
+    // the second block of a CU being the one CUs later in the grid) the blocks after the first `CUs`
+    // ascend from the lightest tile, so that a CU's two blocks are a heavy and a light one.
+    const int group = bid / pairs;
+    const int qt = group < prm.heavy_groups ? prm.n_qtiles - 1 - group : group - prm.heavy_groups;
+    if (qt == 0) prefill_body<true, ROUND>(prm, cache, il_smem, 0, bid % pairs);
+    else prefill_il_body<ROUND>(prm, cache, il_smem, qt, bid % pairs);
+}
+
 }  // namespace qm
 
 extern "C" int32_t qm_prefill_attention_causal(
@@ -1083,22 +1637,32 @@ extern "C" int32_t qm_prefill_attention_causal(
     prm.has_cache = cache ? 1 : 0;
     prm.kv_stride_token = kv_stride_token; prm.kv_stride_head = kv_stride_head; prm.kv_stride_batch = kv_stride_batch;
     prm.batch = batch; prm.seq = seq; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
+    prm.heavy_groups = n_qtiles;
 
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     const bool round_scores = option_value(QM_OPT_PREFILL_SCORE_ROUNDING) != 0;
     if (!round_scores && !(scale > 0.0f)) return QM_ERR_ARGUMENT;   // the scale is folded into the exponent there
-    // 0: by grid size (the wave pairs while the grid is at most four blocks per CU, else the
-    // uniform waves); 1: uniform waves; 2: wave pairs
+    // 0 and 3: the interleaved waves (fastest at every size measured); 1: uniform waves; 2: wave pairs
     const int which = option_value(QM_OPT_PREFILL_KERNEL);
-    if (which < 0 || which > 2) return QM_ERR_ARGUMENT;
-    bool wave_pairs = which == 2;
-    if (which == 0) {
+    if (which < 0 || which > 3) return QM_ERR_ARGUMENT;
+    // (its running maximum is taken before the scores are scaled: a negative scale goes to the uniform waves)
+    if ((which == 0 || which == 3) && scale >= 0.0f) {
         int device = 0, compute_units = 0;
         hipError_t err = hipGetDevice(&device);
         if (err == hipSuccess) err = hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device);
         if (err != hipSuccess) return hip_code(err);
-        wave_pairs = static_cast<int64_t>(pairs) * n_qtiles <= 4 * static_cast<int64_t>(compute_units) && round_scores;
+        const int64_t blocks = pairs * n_qtiles;
+        if (compute_units % pairs == 0 && blocks > compute_units && blocks <= 2 * static_cast<int64_t>(compute_units))
+            prm.heavy_groups = static_cast<int>(compute_units / pairs);
+        const auto kernel = round_scores ? prefill_il_kernel<true> : prefill_il_kernel<false>;
+        static std::atomic<bool> lds_raised[2][kMaxDevices];
+        const int32_t rc_lds = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), kIlSmemBytes,
+                                                  lds_raised[round_scores ? 1 : 0]);
+        if (rc_lds != QM_OK) return rc_lds;
+        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(pairs * n_qtiles)), dim3(kPfThreads), kIlSmemBytes, s, prm, desc);
+        return launch_status();
     }
+    const bool wave_pairs = which == 2;
     if (wave_pairs) {
         const auto kernel = round_scores ? prefill_sp_kernel<true> : prefill_sp_kernel<false>;
         static std::atomic<bool> lds_raised[2][kMaxDevices];
