@@ -83,11 +83,12 @@ const char* qm_target_arch(void);
  *       scale > 0; outputs stay within the 1e-2 tolerance of the fp32 definition).
  *   QM_OPT_DECODE_TILES_PER_BLOCK  0 (default): the split-K decode picks the 16-token tiles per
  *       block from the problem size; > 0 forces it (changes qm_decode_workspace_bytes too).
- *   QM_OPT_PREFILL_KERNEL  0 (default): qm_prefill_attention_causal runs the fastest of its three
+ *   QM_OPT_PREFILL_KERNEL  0 (default): qm_prefill_attention_causal runs the fastest of its
  *       kernels (now 3); 1: four uniform waves per block; 2: four pairs of a matrix wave and a
  *       softmax wave per block; 3: four waves per block, each one software pipeline that alternates
- *       MFMAs with softmax arithmetic.  All give the same bits (a negative scale always runs
- *       kernel 1 in place of 3); other values make the call return QM_ERR_ARGUMENT.
+ *       MFMAs with softmax arithmetic; 4: as 3 with 32 rows per wave (slower; for measurement).
+ *       All give the same bits (a negative scale always runs kernel 1 in place of 3 and 4); other
+ *       values make the call return QM_ERR_ARGUMENT.
  *   QM_OPT_DECODE_STREAMING_LOADS  0 (default): the decode kernels read K and V with the
  *       non-temporal hint when the contexts of one call may exceed 512 MiB (twice the last-level
  *       cache: less than that is partly still cached from the step before), and with plain loads

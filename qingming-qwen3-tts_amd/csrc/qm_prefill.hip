@@ -1031,25 +1031,40 @@ __global__ __launch_bounds__(kSpThreads, 2) void prefill_sp_kernel(PrefillParams
 
 // ======================================================================================================
 // The interleaved kernel: each of the four waves of a block runs the matrix and the softmax work
-// of its 16 rows x 2 heads as ONE software-pipelined instruction stream.
+// of its NC column groups (16 rows x 2 heads each) as ONE software-pipelined instruction stream.
 //
 // Independent MFMAs and VALU instructions of the same wave do overlap when they alternate at
 // fine grain (measured: 16 x (one MFMA, eight FMAs) take 684 cycles against 512 + 616 one after
-// the other), and the compiler's own order — all MFMAs of a product, then all of the softmax —
-// leaves that unused.  Stage j of a wave therefore holds three things that do not depend on
-// one another: the P.V MFMAs of chunk j - 1, the softmax arithmetic of chunk j, and the S^T MFMAs
-// of chunk j + 1; the source alternates one MFMA with one slice of the softmax (a score pair) and
-// pins that order with scheduling barriers.  Staging is that of the wave pairs (K and V tiles go
-// straight from global memory into LDS, V is transposed by the LDS read) with two buffers per
-// ring and one block barrier per 64-key tile: 64 KiB of LDS, so that two blocks share a CU.
-// The diagonal tile is finished outside the pipeline, and blocks of the first query tile (one
-// diagonal tile, split-precision P) run the uniform-waves body.
+// the other; an MFMA costs the wave about 11 cycles of issue), and the compiler's own order — all
+// MFMAs of a product, then all of the softmax — leaves that unused.  Stage j of a wave therefore
+// holds three things that do not depend on one another: the P.V MFMAs of chunk j - 1, the
+// softmax arithmetic of chunk j, and the S^T MFMAs of chunk j + 1; the source alternates MFMAs
+// with slices of the softmax and pins that order with scheduling fences (see the stage).
+// Staging is that of the wave pairs (K and V tiles go straight from global memory into LDS, V is
+// transposed by the LDS read) with two buffers per ring and one block barrier per 64-key tile:
+// 64 KiB of LDS, so that two blocks share a CU.  The block's own (diagonal) tiles are finished
+// outside the pipeline, and blocks of the first query tile (split-precision P) run the
+// uniform-waves body.
+//
+// Measured (same bits as the other kernels; batch x tokens, uniform waves / this kernel):
+// 4 x 1024: 42.4 / 30.5 us, 16 x 1024: 139 / 106 us, 4 x 4096: 374 / 316 us, 1 x 8192: 366 / 305 us
+// (fp32 scores: 36 / 29, 111 / 100, 339 / 291, 337 / 290).  Where the time goes, from cycle stamps
+// inside the kernel: a stage (32 keys: 16 MFMAs = 512 cycles of the matrix pipe) takes 1100 cycles
+// of a wave that has its SIMD to itself and 1400 on average over a tile (barrier and loads), 1500
+// when two waves share the SIMD, which then completes a stage every 750 cycles (68 % of the matrix
+// pipe).  The whole kernel reaches less than that for two reasons outside the pipeline: under this
+// load the chip clocks at 1.65 GHz (4 x 4096) to 1.9 GHz (4 x 1024) instead of 2.4, and a block
+// spends 16 000 cycles outside its pipeline (7 600 until its first loads have landed, 2 200 on
+// the pages and the first S^T, 5 800 on its own tiles, the last barrier and the output), which is
+// 40 % of the 4 x 1024 case, where the whole grid is resident at once and nothing hides it.
+// Two column groups per wave (NC = 2: half the LDS reads per MFMA, 500 registers, one wave per
+// SIMD) are slower (4 x 1024: 58 us, 4 x 4096: 389 us) and stay selectable for measurement only.
 constexpr int kIlRing = 2 * kSpKTile;                       // two tiles of K, likewise of V
 constexpr int kIlSmemBytes = (2 * kIlRing > static_cast<int>(sizeof(PfStage)) * kPfStages)
                                  ? 2 * kIlRing : static_cast<int>(sizeof(PfStage)) * kPfStages;
-static_assert(2 * kIlRing >= 4 * 32 * kOS * 2, "the output staging area reuses the rings");
+static_assert(kIlSmemBytes >= 2 * 4 * 32 * kOS * 2, "the output staging area (two column groups per wave) reuses the rings");
 
-template <bool ROUND>
+template <bool ROUND, int NC>
 __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const qm_kv_cache& cache,
                                                 unsigned char* il_smem, int qt, int bh) {
     typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -1066,24 +1081,27 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
     const int kvh = bh % prm.kv_heads;
     const int S = prm.seq;
     const int q_heads = 2 * prm.kv_heads;
-    const int q0 = qt * kBM;
-    const int my_row = q0 + 16 * wave + (col & 15);
+    const int q0 = qt * kBM * NC;                    // first query row of the block
+    const int n_full = qt * NC;                      // key tiles wholly before the block's rows: the pipeline's
+    const int last_tile = n_full + NC - 1;           // the block's own rows span the tiles n_full .. last_tile
     const int my_head = 2 * kvh + (col >> 4);
-    const int wave_last_row = q0 + 16 * wave + 15;
+    // column group c of this wave: rows group_row0(c) .. + 15
+    auto group_row0 = [&](int c) { return q0 + 16 * (NC * wave + c); };
 
     const int64_t kv_base = static_cast<int64_t>(b) * prm.kv_stride_batch + static_cast<int64_t>(kvh) * prm.kv_stride_head;
     const int kv_row32 = static_cast<int>(prm.kv_stride_token);
 
-    // ---- K/V rows of the diagonal tile for the pages: requested first, written after the first wait ----
+    // ---- K/V rows of the block's own tiles for the pages: requested first, written after the first wait ----
     const bool to_pages = prm.has_cache != 0;
-    int phys[4] = {-1, -1, -1, -1};
-    uint4 kx[4], vx[4];
+    int phys[4 * NC];
+    uint4 kx[4 * NC], vx[4 * NC];
     uint32_t page_err = 0;
     if (to_pages) {
         const int32_t* table = prm.page_table ? prm.page_table + static_cast<int64_t>(b) * prm.pages.max_pages : nullptr;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int key = qt * kBN + (tid >> 4) + 16 * i;
+        for (int i = 0; i < 4 * NC; ++i) {
+            const int key = q0 + (tid >> 4) + 16 * i;
+            phys[i] = -1;
             kx[i] = vx[i] = make_uint4(0, 0, 0, 0);
             if (key < S) {
                 const int page = page_of(prm.pages, key);
@@ -1123,26 +1141,30 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
     load_k(0, 0);
     load_v(0, 0);
     load_k(1, 1);                                    // qt >= 1 here: tile 1 exists
-    bf16x8_t qf[8];
-    {
-        const uint16_t* qp = prm.q + ((static_cast<int64_t>(b) * S + my_row) * q_heads + my_head) * kDim + 8 * grp;
+    bf16x8_t qf[NC][8];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int row = group_row0(c) + (col & 15);
+        const uint16_t* qp = prm.q + ((static_cast<int64_t>(b) * S + row) * q_heads + my_head) * kDim + 8 * grp;
 #pragma unroll
         for (int kb = 0; kb < 8; ++kb) {
             uint4 raw = make_uint4(0, 0, 0, 0);
-            if (my_row < S) raw = *reinterpret_cast<const uint4*>(qp + 16 * kb);
-            qf[kb] = __builtin_bit_cast(bf16x8_t, raw);
+            if (row < S) raw = *reinterpret_cast<const uint4*>(qp + 16 * kb);
+            qf[c][kb] = __builtin_bit_cast(bf16x8_t, raw);
         }
     }
-    f32x16_t o[4];
+    f32x16_t o[NC][4];
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+    for (int c = 0; c < NC; ++c)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[dt][r] = 0.0f;
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[c][dt][r] = 0.0f;
     wait_vm<0>();
     if (to_pages) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int key = qt * kBN + (tid >> 4) + 16 * i;
+        for (int i = 0; i < 4 * NC; ++i) {
+            const int key = q0 + (tid >> 4) + 16 * i;
             if (key >= S || phys[i] == -1) continue;
             if (phys[i] < 0 || phys[i] >= cache.n_pages) {
                 page_err |= QM_STATUS_BAD_PAGE;
@@ -1160,7 +1182,7 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
 
     // ---- fragment reads, all as assembly: the compiler would make an LDS read wait for every
     // global_load_lds in flight, and it must not move them across the barriers either.  Their results
-    // are taken only through k_arrived / v_arrived, which wait for them. ----
+    // are taken only through the *_arrived statements, which wait for them. ----
     // K fragment kb of chunk (slot, h): row 32 h + col, slot (2 kb + grp) ^ (col % 16).
     // V^T fragment (kg, dt): two transposing reads, keys 16 kg + 4 grp + 0..3 and + 8 (see the wave pairs).
     uint32_t kaddr[8], vaddr[4];
@@ -1177,31 +1199,29 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
     }
     struct KRaw { u32x4_t f[8]; };
     struct VRaw { unsigned long long a[8], c[8]; };
-    // Requests come in halves: K fragments 4 h .. 4 h + 3 (k blocks) and the V^T fragments of 16-key group h.
-    // `dyn`: bytes added at run time (0 in the pipeline, where the buffer is a template constant).
-    auto k_request_half = [&](uint32_t dyn, auto imm, auto half, KRaw& raw) {
-#pragma unroll
-        for (int kb = 4 * decltype(half)::value; kb < 4 * decltype(half)::value + 4; ++kb) {
-            const uint32_t at = kaddr[kb] + dyn;
-            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(raw.f[kb]) : "v"(at), "n"(decltype(imm)::value));
-        }
+    // One K fragment (k block i) / one V^T fragment (i = 4 kg + dt: two reads).  `dyn`: bytes added at run
+    // time (0 in the pipeline, where the buffer is a template constant).
+    auto k_request_one = [&](uint32_t dyn, auto imm, int i, KRaw& raw) {
+        const uint32_t at = kaddr[i] + dyn;
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(raw.f[i]) : "v"(at), "n"(decltype(imm)::value));
     };
-    auto v_request_half = [&](uint32_t dyn, auto imm, auto half, VRaw& raw) {
-        constexpr int kg = decltype(half)::value;
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-            const uint32_t at = vaddr[dt] + dyn;
-            asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(raw.a[4 * kg + dt]) : "v"(at), "n"(decltype(imm)::value + 16 * kg * kKR));
-            asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(raw.c[4 * kg + dt]) : "v"(at), "n"(decltype(imm)::value + (16 * kg + 8) * kKR));
+    auto v_request_one = [&](uint32_t dyn, auto imm, int i, VRaw& raw) {
+        const uint32_t at = vaddr[i & 3] + dyn;
+        if (i < 4) {
+            asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(raw.a[i]) : "v"(at), "n"(decltype(imm)::value));
+            asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(raw.c[i]) : "v"(at), "n"(decltype(imm)::value + 8 * kKR));
+        } else {
+            asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(raw.a[i]) : "v"(at), "n"(decltype(imm)::value + 16 * kKR));
+            asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(raw.c[i]) : "v"(at), "n"(decltype(imm)::value + 24 * kKR));
         }
     };
     auto k_request = [&](uint32_t dyn, auto imm, KRaw& raw) {
-        k_request_half(dyn, imm, int_c<0>{}, raw);
-        k_request_half(dyn, imm, int_c<1>{}, raw);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) k_request_one(dyn, imm, i, raw);
     };
     auto v_request = [&](uint32_t dyn, auto imm, VRaw& raw) {
-        v_request_half(dyn, imm, int_c<0>{}, raw);
-        v_request_half(dyn, imm, int_c<1>{}, raw);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v_request_one(dyn, imm, i, raw);
     };
     auto v_unpack = [&](const VRaw& raw, int j) -> bf16x8_t {
         const uint4 both_halves = make_uint4(static_cast<uint32_t>(raw.a[j]), static_cast<uint32_t>(raw.a[j] >> 32),
@@ -1243,44 +1263,50 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         for (int j = 0; j < 8; ++j) vf[j] = v_unpack(raw, j);
     };
 
-    // ---- softmax state and slices (the arithmetic of the uniform waves, cut into score pairs) ----
+    // ---- softmax state (per column group) and the arithmetic of the uniform waves, cut into score pairs ----
     const float coef = ROUND ? kLog2e : prm.scale * kLog2e;
     const float slack = ROUND ? kRescaleSlack : kRescaleSlack / prm.scale;
-    float m_run = -INFINITY, l_run = 0.0f, m_scaled = 0.0f;
-    // roundings (and, on the diagonal, the causal mask) of the score pair r, r + 1 in place
-    auto score_pair = [&](f32x16_t& s, int r, float& mx, auto masked, int lim) {
+    float m_run[NC], l_run[NC], m_scaled[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        m_run[c] = -INFINITY;
+        l_run[c] = 0.0f;
+        m_scaled[c] = 0.0f;
+    }
+    // roundings and the causal mask of the score pair r, r + 1 in place (the diagonal tiles)
+    auto score_pair_masked = [&](f32x16_t& s, int r, float& mx, int lim) {
         float x0 = s[r], x1 = s[r + 1];
         if (ROUND) {
             round_bf16_pair(x0, x1, x0, x1);
             round_bf16_pair(x0 * prm.scale, x1 * prm.scale, x0, x1);
         }
-        if (decltype(masked)::value) {
-            const int e = 8 * (r >> 2) + (r & 3);
-            if (e > lim) x0 = -INFINITY;
-            if (e + 1 > lim) x1 = -INFINITY;
-        }
+        const int e = 8 * (r >> 2) + (r & 3);
+        if (e > lim) x0 = -INFINITY;
+        if (e + 1 > lim) x1 = -INFINITY;
         s[r] = x0;
         s[r + 1] = x1;
         mx = fmaxf(mx, fmaxf(x0, x1));
     };
-    auto update_max = [&](float mx) {
-        const bool need = __builtin_amdgcn_ballot_w64(mx > m_run + slack) != 0;
+    // raises the running maximum of column group c if some column exceeds it by more than the slack, and
+    // rescales O and the running sum for it (the diagonal tiles; the pipeline defers the rescaling of O)
+    auto update_max = [&](int c, float mx) {
+        const bool need = __builtin_amdgcn_ballot_w64(mx > m_run[c] + slack) != 0;
         if (need) {
-            const float m_new = fmaxf(m_run, mx);
+            const float m_new = fmaxf(m_run[c], mx);
             const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
-            const float alpha = fast_exp2((m_run - m_ref) * coef);
-            m_run = m_new;
-            m_scaled = m_ref * coef;
-            l_run *= alpha;
+            const float alpha = fast_exp2((m_run[c] - m_ref) * coef);
+            m_run[c] = m_new;
+            m_scaled[c] = m_ref * coef;
+            l_run[c] *= alpha;
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+                for (int r = 0; r < 16; ++r) o[c][dt][r] *= alpha;
         }
     };
-    auto prob_pair = [&](const f32x16_t& s, int r, uint32_t& packed, float& psum) {
-        const float e0 = fast_exp2(fmaf(s[r], coef, -m_scaled));
-        const float e1 = fast_exp2(fmaf(s[r + 1], coef, -m_scaled));
+    auto prob_pair = [&](int c, const f32x16_t& s, int r, uint32_t& packed, float& psum) {
+        const float e0 = fast_exp2(fmaf(s[r], coef, -m_scaled[c]));
+        const float e1 = fast_exp2(fmaf(s[r + 1], coef, -m_scaled[c]));
         packed = pack_bf16_pair(e0, e1);
         psum = dot2_bf16(packed, 0x3f803f80U, psum);          // the sum of what the MFMA multiplies
     };
@@ -1296,137 +1322,204 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
     // out: s_next = raw S^T of chunk j + 1; p_cur = P of chunk j; vraw = V^T fragments of chunk j (from `v_imm`)
     //      and kraw = K fragments of chunk j + 2 (from `k_imm`), requested
     // What the order of the instructions answers to (all measured on this chip):
+    //  - a fragment read from LDS feeds the MFMAs of all NC column groups of the wave: with one group (32
+    //    columns) every MFMA needs 1 KiB of LDS, the four SIMDs of a CU together 128 bytes per cycle, which is
+    //    all its LDS delivers; with two groups it is half of that;
     //  - dependent VALU instructions issue 8 cycles apart, independent ones 4 (the exponential takes 12), and
     //    the arithmetic of one score pair is a single chain six instructions deep: the stage works on two
     //    pairs at a time, level by level, so that an independent instruction sits between dependent ones;
-    //  - a dependent MFMA waits for the one before it to finish: the S^T MFMAs (one accumulator) alternate
-    //    with the P.V MFMAs (four accumulators), one MFMA per half group of VALU work;
-    //  - eight global_load_lds in a row take 500 cycles to issue: the loads of a tile are handed out one per
-    //    group (`vmem`), and the block barrier of the tile (`sync`) comes after the first group, when the
-    //    LDS reads it has to wait for have long landed;
-    //  - the chain from the maxima to the branch on them is 14 dependent instructions: two MFMAs are issued
+    //  - a dependent MFMA waits for the one before it to finish: the S^T MFMAs (one accumulator per column
+    //    group) alternate with the P.V MFMAs (four accumulators), one MFMA per half group of VALU work;
+    //  - eight global_load_lds in a row take 500 cycles to issue and twelve LDS reads in a row 200: the loads
+    //    of a tile are handed out one per group (`vmem`), a fragment is requested as soon as the last MFMA
+    //    that uses its registers has been issued, and the block barrier of the tile (`sync`) comes after
+    //    the first group, when the LDS reads it has to wait for have long landed;
+    //  - the chain from the maxima to the branch on them is 14 dependent instructions: MFMAs are issued
     //    ahead of it.  If the running maximum is raised, O is rescaled at the end of the stage, after the last
     //    P.V MFMA of chunk j - 1 (whose P is relative to the old maximum).
     // Scheduling fences pin the order.
     auto fence = []() { __builtin_amdgcn_sched_barrier(0); };
-    auto stage = [&](f32x16_t& s_cur, f32x16_t& s_next, const PPair& p_prev, PPair& p_cur, KRaw& kraw, VRaw& vraw,
-                     auto k_imm, auto v_imm, auto&& sync, auto&& vmem) {
+    auto stage = [&](f32x16_t (&s_cur)[NC], f32x16_t (&s_next)[NC], const PPair (&p_prev)[NC], PPair (&p_cur)[NC],
+                     KRaw& kraw, VRaw& vraw, auto k_imm, auto v_imm, auto&& sync, auto&& vmem) {
         bf16x8_t kf[8], vf[8];
-        auto pv_mfma = [&](int i) {
-            o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i], p_prev.g[i >> 2], o[i & 3], 0, 0, 0);
+        auto pv_mfma = [&](int i, int c) {
+            o[c][i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i], p_prev[c].g[i >> 2], o[c][i & 3], 0, 0, 0);
         };
-        auto qk_mfma = [&](int i) { s_next = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qf[i], s_next, 0, 0, 0); };
+        auto qk_mfma = [&](int i, int c) {
+            s_next[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qf[c][i], s_next[c], 0, 0, 0);
+        };
         half_arrived(int_c<0>{}, int_c<12>{}, kraw, vraw, kf, vf);
+        // (ROUND) the maxima of the raw scores are taken in the first group and then walk, one step per group,
+        // through the roundings (monotonic: the result is the maximum of the rounded scores; the host sends a
+        // negative scale elsewhere) and the exchange between the two halves of the wave, so that the branch
+        // on them after the last group waits for nothing
+        float mx_a[NC], mx_b[NC], mx_step[NC], mx_limit[NC];
+        uint32_t mx_bits[NC];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s_next[r] = 0.0f;
-        float mx_a = -INFINITY, mx_b = -INFINITY;
+        for (int c = 0; c < NC; ++c) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_next[c][r] = 0.0f;
+            mx_a[c] = mx_b[c] = -INFINITY;
+            mx_step[c] = 0.0f;
+            mx_bits[c] = 0;
+            mx_limit[c] = m_run[c] + slack;
+        }
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const int ra = 4 * g, rb = 4 * g + 2;              // pair a = scores ra, ra + 1; pair b = rb, rb + 1
-            pv_mfma(g);
-            fence();
-            if (ROUND) {
-                const float xa0 = s_cur[ra], xa1 = s_cur[ra + 1], xb0 = s_cur[rb], xb1 = s_cur[rb + 1];
-                const uint32_t pa = pack_bf16_pair(xa0, xa1);
-                const uint32_t pb = pack_bf16_pair(xb0, xb1);
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                pv_mfma(g, c);
                 fence();
-                const float ua0 = lo_bf16(pa), ua1 = hi_bf16(pa), ub0 = lo_bf16(pb), ub1 = hi_bf16(pb);
+                if (ROUND) {
+                    const float xa0 = s_cur[c][ra], xa1 = s_cur[c][ra + 1], xb0 = s_cur[c][rb], xb1 = s_cur[c][rb + 1];
+                    uint32_t pa = pack_bf16_pair(xa0, xa1);
+                    const uint32_t pb = pack_bf16_pair(xb0, xb1);
+                    if (g == 0) {
+                        // (assembly: the compiler's fmaxf first quiets every operand with an instruction of its
+                        // own.  `pa` passes through the first statement so that the chain follows a read of the
+                        // MFMA results that the compiler guards; one MFMA wrote all sixteen.)
+                        asm volatile("v_max3_f32 %0, %0, %2, %3" : "+v"(mx_a[c]), "+v"(pa) : "v"(s_cur[c][0]), "v"(s_cur[c][1]));
+                        asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(mx_b[c]) : "v"(s_cur[c][2]), "v"(s_cur[c][3]));
+#pragma unroll
+                        for (int r = 4; r < 16; r += 4) {
+                            asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(mx_a[c]) : "v"(s_cur[c][r]), "v"(s_cur[c][r + 1]));
+                            asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(mx_b[c]) : "v"(s_cur[c][r + 2]), "v"(s_cur[c][r + 3]));
+                        }
+                    }
+                    if (g == 3) {
+                        mx_bits[c] = pack_bf16_pair(mx_step[c], mx_step[c]);
+                        asm volatile("" : "+v"(mx_bits[c]));
+                    }
+                    fence();
+                    const float ua0 = lo_bf16(pa), ua1 = hi_bf16(pa), ub0 = lo_bf16(pb), ub1 = hi_bf16(pb);
+                    if (g == 1) {
+                        asm volatile("v_max_f32 %0, %1, %2" : "=v"(mx_step[c]) : "v"(mx_a[c]), "v"(mx_b[c]));
+                    }
+                    if (g == 3) {
+                        mx_step[c] = lo_bf16(mx_bits[c]);
+                        asm volatile("" : "+v"(mx_step[c]));
+                    }
+                    fence();
+                    const float ya0 = ua0 * prm.scale, ya1 = ua1 * prm.scale;
+                    if (g == 1) {
+                        mx_bits[c] = pack_bf16_pair(mx_step[c], mx_step[c]);
+                        asm volatile("" : "+v"(mx_bits[c]));
+                    }
+                    fence();
+                    qk_mfma(g, c);
+                    fence();
+                    const float yb0 = ub0 * prm.scale, yb1 = ub1 * prm.scale;
+                    if (g == 2) {
+                        mx_step[c] = lo_bf16(mx_bits[c]);
+                        asm volatile("" : "+v"(mx_step[c]));
+                    }
+                    fence();
+                    const uint32_t qa = pack_bf16_pair(ya0, ya1);
+                    const uint32_t qb = pack_bf16_pair(yb0, yb1);
+                    if (g == 2) {
+                        mx_step[c] = mx_step[c] * prm.scale;
+                        asm volatile("" : "+v"(mx_step[c]));
+                    }
+                    fence();
+                    float za0 = lo_bf16(qa), za1 = hi_bf16(qa), zb0 = lo_bf16(qb), zb1 = hi_bf16(qb);
+                    // (an empty statement that keeps the roundings here instead of sinking to where they are used)
+                    asm volatile("" : "+v"(za0), "+v"(za1), "+v"(zb0), "+v"(zb1));
+                    if (g == 3) {
+                        mx_step[c] = halves_max(mx_step[c]);
+                        asm volatile("" : "+v"(mx_step[c]));
+                    }
+                    s_cur[c][ra] = za0; s_cur[c][ra + 1] = za1; s_cur[c][rb] = zb0; s_cur[c][rb + 1] = zb1;
+                } else {
+                    mx_a[c] = __builtin_fmaxf(mx_a[c], __builtin_fmaxf(s_cur[c][ra], s_cur[c][ra + 1]));
+                    fence();
+                    qk_mfma(g, c);
+                    fence();
+                    mx_b[c] = __builtin_fmaxf(mx_b[c], __builtin_fmaxf(s_cur[c][rb], s_cur[c][rb + 1]));
+                }
                 fence();
-                const float ya0 = ua0 * prm.scale, ya1 = ua1 * prm.scale;
-                fence();
-                qk_mfma(g);
-                fence();
-                const float yb0 = ub0 * prm.scale, yb1 = ub1 * prm.scale;
-                fence();
-                const uint32_t qa = pack_bf16_pair(ya0, ya1);
-                const uint32_t qb = pack_bf16_pair(yb0, yb1);
-                fence();
-                float za0 = lo_bf16(qa), za1 = hi_bf16(qa), zb0 = lo_bf16(qb), zb1 = hi_bf16(qb);
-                fence();
-                // The running maxima are taken over the raw scores (the roundings are monotonic and the host
-                // sends a negative scale elsewhere), one v_max3 each: the compiler's fmaxf first quiets every
-                // operand with an instruction of its own.  The rounded values pass through the statements so
-                // that these follow the roundings — whose reads of the MFMA results the compiler guards — and
-                // so that the roundings stay here instead of sinking to where they are used.
-                asm volatile("v_max3_f32 %0, %0, %3, %4" : "+v"(mx_a), "+v"(za0), "+v"(za1) : "v"(xa0), "v"(xa1));
-                asm volatile("v_max3_f32 %0, %0, %3, %4" : "+v"(mx_b), "+v"(zb0), "+v"(zb1) : "v"(xb0), "v"(xb1));
-                s_cur[ra] = za0; s_cur[ra + 1] = za1; s_cur[rb] = zb0; s_cur[rb + 1] = zb1;
-            } else {
-                mx_a = __builtin_fmaxf(mx_a, __builtin_fmaxf(s_cur[ra], s_cur[ra + 1]));
-                fence();
-                qk_mfma(g);
-                fence();
-                mx_b = __builtin_fmaxf(mx_b, __builtin_fmaxf(s_cur[rb], s_cur[rb + 1]));
             }
-            fence();
             if (g == 0) sync();
             vmem(g);
+            k_request_one(0u, k_imm, g, kraw);
+            v_request_one(0u, v_imm, g, vraw);
             fence();
         }
-        k_request_half(0u, k_imm, int_c<0>{}, kraw);
-        v_request_half(0u, v_imm, int_c<0>{}, vraw);
         half_arrived(int_c<1>{}, int_c<12>{}, kraw, vraw, kf, vf);
-        qk_mfma(4);
-        pv_mfma(4);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            qk_mfma(4, c);
+            pv_mfma(4, c);
+        }
         fence();
 
-        float mx = __builtin_fmaxf(mx_a, mx_b);
-        if (ROUND) mx = round_bf16(round_bf16(mx) * prm.scale);
-        mx = halves_max(mx);
-        const bool need = __builtin_amdgcn_ballot_w64(mx > m_run + slack) != 0;
-        float alpha = 1.0f;
-        if (need) {
-            const float m_new = fmaxf(m_run, mx);
-            const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
-            alpha = fast_exp2((m_run - m_ref) * coef);
-            m_run = m_new;
-            m_scaled = m_ref * coef;
-            l_run *= alpha;
+        bool need[NC];
+        float alpha[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const float mx = ROUND ? mx_step[c] : halves_max(__builtin_fmaxf(mx_a[c], mx_b[c]));
+            need[c] = __builtin_amdgcn_ballot_w64(mx > mx_limit[c]) != 0;
+            alpha[c] = 1.0f;
+            if (need[c]) {
+                const float m_new = fmaxf(m_run[c], mx);
+                const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
+                alpha[c] = fast_exp2((m_run[c] - m_ref) * coef);
+                m_run[c] = m_new;
+                m_scaled[c] = m_ref * coef;
+                l_run[c] *= alpha[c];
+            }
         }
-
-        uint32_t hi[8];
-        float psum = 0.0f;
+        uint32_t hi[NC][8];
+        float psum[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) psum[c] = 0.0f;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const int ra = 4 * g, rb = 4 * g + 2;
-            if (g > 0) pv_mfma(4 + g);
-            fence();
-            const float ta0 = fmaf(s_cur[ra], coef, -m_scaled), ta1 = fmaf(s_cur[ra + 1], coef, -m_scaled);
-            const float tb0 = fmaf(s_cur[rb], coef, -m_scaled), tb1 = fmaf(s_cur[rb + 1], coef, -m_scaled);
-            fence();
-            const float ea0 = fast_exp2(ta0), ea1 = fast_exp2(ta1);
-            fence();
-            if (g < 3) qk_mfma(5 + g);
-            fence();
-            const float eb0 = fast_exp2(tb0), eb1 = fast_exp2(tb1);
-            fence();
-            hi[2 * g] = pack_bf16_pair(ea0, ea1);
-            hi[2 * g + 1] = pack_bf16_pair(eb0, eb1);
-            fence();
-            psum = dot2_bf16(hi[2 * g], 0x3f803f80U, psum);          // the sum of what the MFMA multiplies
-            psum = dot2_bf16(hi[2 * g + 1], 0x3f803f80U, psum);
-            // (an empty statement that keeps this arithmetic here: its results are only used by the next
-            // stage, and the compiler would sink it below the branch at the end of this one)
-            asm volatile("" : "+v"(hi[2 * g]), "+v"(hi[2 * g + 1]), "+v"(psum));
-            fence();
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                if (g > 0) pv_mfma(4 + g, c);
+                fence();
+                const float ta0 = fmaf(s_cur[c][ra], coef, -m_scaled[c]), ta1 = fmaf(s_cur[c][ra + 1], coef, -m_scaled[c]);
+                const float tb0 = fmaf(s_cur[c][rb], coef, -m_scaled[c]), tb1 = fmaf(s_cur[c][rb + 1], coef, -m_scaled[c]);
+                fence();
+                const float ea0 = fast_exp2(ta0), ea1 = fast_exp2(ta1);
+                fence();
+                if (g < 3) qk_mfma(5 + g, c);
+                fence();
+                const float eb0 = fast_exp2(tb0), eb1 = fast_exp2(tb1);
+                fence();
+                hi[c][2 * g] = pack_bf16_pair(ea0, ea1);
+                hi[c][2 * g + 1] = pack_bf16_pair(eb0, eb1);
+                fence();
+                psum[c] = dot2_bf16(hi[c][2 * g], 0x3f803f80U, psum[c]);          // the sum of what the MFMA multiplies
+                psum[c] = dot2_bf16(hi[c][2 * g + 1], 0x3f803f80U, psum[c]);
+                // (an empty statement that keeps this arithmetic here: its results are only used by the next
+                // stage, and the compiler would sink it below the branch at the end of this one)
+                asm volatile("" : "+v"(hi[c][2 * g]), "+v"(hi[c][2 * g + 1]), "+v"(psum[c]));
+                fence();
+            }
             vmem(4 + g);
+            k_request_one(0u, k_imm, 4 + g, kraw);
+            v_request_one(0u, v_imm, 4 + g, vraw);
             fence();
         }
-        k_request_half(0u, k_imm, int_c<1>{}, kraw);
-        v_request_half(0u, v_imm, int_c<1>{}, vraw);
-        make_p(hi, p_cur);
-        l_run += psum;
-        if (need) {
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+        for (int c = 0; c < NC; ++c) {
+            make_p(hi[c], p_cur[c]);
+            l_run[c] += psum[c];
+            if (need[c]) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+                for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o[c][dt][r] *= alpha[c];
+            }
         }
     };
 
     // ---- prologue: S^T of chunk (0, 0); K fragments of chunk (0, 1) requested; nothing to multiply yet ----
-    f32x16_t s_a, s_b;
-    PPair p_a, p_b;
+    f32x16_t s_a[NC], s_b[NC];
+    PPair p_a[NC], p_b[NC];
     KRaw kraw;
     VRaw vraw;
     {
@@ -1434,9 +1527,13 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         k_request(0u, int_c<0>{}, kraw);
         k_arrived(kraw, kf);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s_a[r] = 0.0f;
+        for (int c = 0; c < NC; ++c) {
 #pragma unroll
-        for (int kb = 0; kb < 8; ++kb) s_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb], qf[kb], s_a, 0, 0, 0);
+            for (int r = 0; r < 16; ++r) s_a[c][r] = 0.0f;
+#pragma unroll
+            for (int kb = 0; kb < 8; ++kb) s_a[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb], qf[c][kb], s_a[c], 0, 0, 0);
+            p_b[c].g[0] = p_b[c].g[1] = __builtin_bit_cast(bf16x8_t, make_uint4(0, 0, 0, 0));
+        }
         k_request(0u, int_c<32 * kKR>{}, kraw);
         // (the stages count outstanding reads in halves of twelve; these eight are taken here)
         asm volatile("s_waitcnt lgkmcnt(0)"
@@ -1446,17 +1543,16 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
                      : "memory");
 #pragma unroll
         for (int j = 0; j < 8; ++j) vraw.a[j] = vraw.c[j] = 0ull;
-        p_b.g[0] = p_b.g[1] = __builtin_bit_cast(bf16x8_t, make_uint4(0, 0, 0, 0));
     }
 
-    // ---- the tiles before the diagonal: tile t lives in buffer t % 2 of either ring.  During its first stage
+    // ---- the tiles before the block's own: tile t lives in buffer t % 2 of either ring.  During its first stage
     // (after the tile's barrier: every wave has taken the last fragments of tile t - 1 and of K tile t) the
     // wave requests K of tile t + 2 into the buffer of K tile t and V of tile t + 1 into the buffer of V tile
     // t - 1; both are first read during tile t + 1, after its barrier. ----
     auto tile_body = [&](int t, auto parity) {
         constexpr int cur = decltype(parity)::value;
         constexpr int nxt = cur ^ 1;
-        const bool more_k = t + 2 <= qt;
+        const bool more_k = t + 2 <= last_tile;
         // stage (t, 0): P.V of chunk (t - 1, 1), softmax of (t, 0), S^T of (t, 1); requests V(t, 0) and K(t + 1, 0)
         stage(s_a, s_b, p_b, p_a, kraw, vraw, int_c<nxt * kSpKTile>{}, int_c<cur * kSpKTile>{},
               [&]() {
@@ -1474,109 +1570,130 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         stage(s_b, s_a, p_a, p_b, kraw, vraw, int_c<nxt * kSpKTile + 32 * kKR>{}, int_c<cur * kSpKTile + 32 * kKR>{},
               []() {}, [](int) {});
     };
-    for (int t = 0; t < qt; t += 2) {
+    for (int t = 0; t < n_full; t += 2) {
         tile_body(t, int_c<0>{});
-        if (t + 1 < qt) tile_body(t + 1, int_c<1>{});
+        if (t + 1 < n_full) tile_body(t + 1, int_c<1>{});
     }
     wait_vm<0>();
-    lds_barrier();                                   // V of the diagonal tile has landed for every wave
+    lds_barrier();                                   // what has been loaded has landed for every wave, and every
+                                                     // wave has taken its fragments of V tile n_full - 1
+    if (NC == 2) load_v(last_tile, last_tile & 1);   // (the pipeline requested V up to tile n_full only)
 
-    // ---- drain: P.V of chunk (qt - 1, 1), then the diagonal tile chunk by chunk ----
-    const uint32_t diag_slot = static_cast<uint32_t>((qt & 1) * kSpKTile);
+    // ---- drain: P.V of chunk (n_full - 1, 1), then the block's own tiles chunk by chunk ----
     {
         bf16x8_t vf[8];
         v_arrived(vraw, vf);
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i], p_b.g[i >> 2], o[i & 3], 0, 0, 0);
+        for (int c = 0; c < NC; ++c)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                o[c][i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i], p_b[c].g[i >> 2], o[c][i & 3], 0, 0, 0);
     }
-    auto diag_chunk = [&](f32x16_t& s, auto h, int key_base) {
-        VRaw vr;
-        bf16x8_t vf[8];
-        v_request(diag_slot, int_c<decltype(h)::value * 32 * kKR>{}, vr);
-        const int lim = my_row - key_base - 4 * grp;
+    // Chunk d of the block's own tiles (first key key_base) concerns column group c if key_base is not after the
+    // group's last row; it is masked for that group.  A 16-key group wholly after the last row is masked for every
+    // column: skipped, so that later tokens are not even multiplied by zero.
+    auto diag_group = [&](int c, f32x16_t& s, const bf16x8_t (&vf)[8], int key_base) {
+        const int lim = group_row0(c) + (col & 15) - key_base - 4 * grp;
         float mx = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) score_pair(s, 2 * i, mx, bool_c<true>{}, lim);
+        for (int i = 0; i < 8; ++i) score_pair_masked(s, 2 * i, mx, lim);
         mx = halves_max(mx);
-        update_max(mx);
+        update_max(c, mx);
         uint32_t hi[8];
         float psum = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) prob_pair(s, 2 * i, hi[i], psum);
-        l_run += psum;
+        for (int i = 0; i < 8; ++i) prob_pair(c, s, 2 * i, hi[i], psum);
+        l_run[c] += psum;
         PPair p;
         make_p(hi, p);
-        asm volatile("s_waitcnt lgkmcnt(0)"
-                     : "+v"(vr.a[0]), "+v"(vr.a[1]), "+v"(vr.a[2]), "+v"(vr.a[3]), "+v"(vr.a[4]), "+v"(vr.a[5]),
-                       "+v"(vr.a[6]), "+v"(vr.a[7]), "+v"(vr.c[0]), "+v"(vr.c[1]), "+v"(vr.c[2]), "+v"(vr.c[3]),
-                       "+v"(vr.c[4]), "+v"(vr.c[5]), "+v"(vr.c[6]), "+v"(vr.c[7])
-                     :
-                     : "memory");
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const uint4 both_halves = make_uint4(static_cast<uint32_t>(vr.a[j]), static_cast<uint32_t>(vr.a[j] >> 32),
-                                                 static_cast<uint32_t>(vr.c[j]), static_cast<uint32_t>(vr.c[j] >> 32));
-            vf[j] = __builtin_bit_cast(bf16x8_t, both_halves);
-        }
-        // a 16-key group wholly after the wave's last row is masked for every column: skipped, so that
-        // later tokens are not even multiplied by zero
 #pragma unroll
         for (int kg = 0; kg < 2; ++kg) {
-            if (key_base + 16 * kg > wave_last_row) continue;
+            if (key_base + 16 * kg > group_row0(c) + 15) continue;
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)
-                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * kg + dt], p.g[kg], o[dt], 0, 0, 0);
+                o[c][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * kg + dt], p.g[kg], o[c][dt], 0, 0, 0);
         }
     };
-    // after an even number of stages the raw scores of the diagonal's first chunk are in s_a and the K
-    // fragments of its second chunk have been requested
-    diag_chunk(s_a, int_c<0>{}, qt * kBN);
-    {
-        bf16x8_t kf[8];
-        k_arrived(kraw, kf);                         // (every wave takes them, so that no read is left pending)
-        if (qt * kBN + 32 <= wave_last_row) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s_b[r] = 0.0f;
+    for (int d = 0; d < 2 * NC; ++d) {
+        const int tile = n_full + (d >> 1);
+        const int key_base = tile * kBN + 32 * (d & 1);
+        const uint32_t slot_bytes = static_cast<uint32_t>((tile & 1) * kSpKTile);
+        if (d == 2) {
+            wait_vm<0>();
+            lds_barrier();                           // V of the last tile has landed for every wave
+        }
+        const bool any = key_base <= group_row0(NC - 1) + 15;       // (the wave's last column group sees the most)
+        bf16x8_t kf[8], vf[8];
+        if (d >= 1) {
+            // K fragments: those of chunk 1 were requested by the pipeline (every wave takes them, so that no
+            // read is left pending); later ones are requested here
+            if (d >= 2 && any) {
+                if (d & 1) k_request(slot_bytes, int_c<32 * kKR>{}, kraw);
+                else k_request(slot_bytes, int_c<0>{}, kraw);
+            }
+            if (d == 1 || any) k_arrived(kraw, kf);
+        }
+        if (!any) continue;
+        VRaw vr;
+        if (d & 1) v_request(slot_bytes, int_c<32 * kKR>{}, vr);
+        else v_request(slot_bytes, int_c<0>{}, vr);
+        if (d >= 1) {
 #pragma unroll
-            for (int kb = 0; kb < 8; ++kb) s_b = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb], qf[kb], s_b, 0, 0, 0);
-            diag_chunk(s_b, int_c<1>{}, qt * kBN + 32);
+            for (int c = 0; c < NC; ++c) {
+                if (key_base > group_row0(c) + 15) continue;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s_a[c][r] = 0.0f;
+#pragma unroll
+                for (int kb = 0; kb < 8; ++kb) s_a[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb], qf[c][kb], s_a[c], 0, 0, 0);
+            }
+        }
+        v_arrived(vr, vf);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            if (key_base > group_row0(c) + 15) continue;
+            diag_group(c, s_a[c], vf, key_base);
         }
     }
     lds_barrier();   // every wave is done with the rings: they become the output staging area
 
     // ---- normalise, stage through LDS, write 16 bytes per lane ----
-    const float l_tot = halves_sum(l_run);
-    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-    uint16_t* stage_out = reinterpret_cast<uint16_t*>(il_smem) + wave * 32 * kOS;
+    uint16_t* stage_out = reinterpret_cast<uint16_t*>(il_smem) + wave * NC * 32 * kOS;
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt) {
+    for (int c = 0; c < NC; ++c) {
+        const float l_tot = halves_sum(l_run[c]);
+        const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
 #pragma unroll
-        for (int rq = 0; rq < 4; ++rq) {
-            const int d0 = 32 * dt + 8 * rq + 4 * grp;
-            uint2 packed;
-            packed.x = pack_bf16_pair(o[dt][4 * rq + 0] * inv, o[dt][4 * rq + 1] * inv);
-            packed.y = pack_bf16_pair(o[dt][4 * rq + 2] * inv, o[dt][4 * rq + 3] * inv);
-            *reinterpret_cast<uint2*>(&stage_out[col * kOS + d0]) = packed;
+        for (int dt = 0; dt < 4; ++dt) {
+#pragma unroll
+            for (int rq = 0; rq < 4; ++rq) {
+                const int d0 = 32 * dt + 8 * rq + 4 * grp;
+                uint2 packed;
+                packed.x = pack_bf16_pair(o[c][dt][4 * rq + 0] * inv, o[c][dt][4 * rq + 1] * inv);
+                packed.y = pack_bf16_pair(o[c][dt][4 * rq + 2] * inv, o[c][dt][4 * rq + 3] * inv);
+                *reinterpret_cast<uint2*>(&stage_out[(32 * c + col) * kOS + d0]) = packed;
+            }
         }
     }
     __builtin_amdgcn_s_waitcnt(0);   // the wave reads back only what it wrote itself
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
-        const int c = 4 * it + (lane >> 4);
+    for (int it = 0; it < 8 * NC; ++it) {
+        const int cc = 4 * it + (lane >> 4);         // staged column: group cc / 32, head (cc % 32) / 16, row cc % 16
         const int piece = lane & 15;
-        const int row = q0 + 16 * wave + (c & 15);
-        const int head = 2 * kvh + (c >> 4);
+        const int row = group_row0(cc >> 5) + (cc & 15);
+        const int head = 2 * kvh + ((cc & 31) >> 4);
         if (row < S) {
-            const uint4 val = *reinterpret_cast<const uint4*>(&stage_out[c * kOS + 8 * piece]);
+            const uint4 val = *reinterpret_cast<const uint4*>(&stage_out[cc * kOS + 8 * piece]);
             *reinterpret_cast<uint4*>(prm.out + ((static_cast<int64_t>(b) * S + row) * q_heads + head) * kDim + 8 * piece) = val;
         }
     }
 }
 
-template <bool ROUND>
-__global__ __launch_bounds__(kPfThreads, 2) void prefill_il_kernel(PrefillParams prm, qm_kv_cache cache) {
+// grid = batch * kv_heads * ceil(seq / (64 NC)) blocks.  Blocks of the first query tile run the uniform-waves body
+// on its one or two 64-row tiles (split-precision P in the very first).
+template <bool ROUND, int NC>
+__global__ __launch_bounds__(kPfThreads, (NC == 1 ? 2 : 1)) void prefill_il_kernel(PrefillParams prm, qm_kv_cache cache) {
     extern __shared__ __attribute__((aligned(16))) unsigned char il_smem[];
     const int pairs = prm.batch * prm.kv_heads;
     const int bid = blockIdx.x;
@@ -1585,11 +1702,19 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_il_kernel(PrefillParams
     // ascend from the lightest tile, so that a CU's two blocks are a heavy and a light one.
     const int group = bid / pairs;
     const int qt = group < prm.heavy_groups ? prm.n_qtiles - 1 - group : group - prm.heavy_groups;
-    if (qt == 0) prefill_body<true, ROUND>(prm, cache, il_smem, 0, bid % pairs);
-    else prefill_il_body<ROUND>(prm, cache, il_smem, qt, bid % pairs);
+    if (qt == 0) {
+        prefill_body<true, ROUND>(prm, cache, il_smem, 0, bid % pairs);
+        if (NC == 2 && prm.seq > kBM) {
+            __syncthreads();
+            prefill_body<false, ROUND>(prm, cache, il_smem, 1, bid % pairs);
+        }
+    } else {
+        prefill_il_body<ROUND, NC>(prm, cache, il_smem, qt, bid % pairs);
+    }
 }
 
 }  // namespace qm
+
 
 extern "C" int32_t qm_prefill_attention_causal(
     const uint16_t* query, const uint16_t* key, const uint16_t* value,
@@ -1644,22 +1769,33 @@ extern "C" int32_t qm_prefill_attention_causal(
     if (!round_scores && !(scale > 0.0f)) return QM_ERR_ARGUMENT;   // the scale is folded into the exponent there
     // 0 and 3: the interleaved waves (fastest at every size measured); 1: uniform waves; 2: wave pairs
     const int which = option_value(QM_OPT_PREFILL_KERNEL);
-    if (which < 0 || which > 3) return QM_ERR_ARGUMENT;
+    if (which < 0 || which > 4) return QM_ERR_ARGUMENT;
     // (its running maximum is taken before the scores are scaled: a negative scale goes to the uniform waves)
-    if ((which == 0 || which == 3) && scale >= 0.0f) {
+    if ((which == 0 || which >= 3) && scale >= 0.0f) {
+        const int groups = which == 4 ? 2 : 1;                     // column groups (16 rows x 2 heads) per wave
         int device = 0, compute_units = 0;
         hipError_t err = hipGetDevice(&device);
         if (err == hipSuccess) err = hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device);
         if (err != hipSuccess) return hip_code(err);
-        const int64_t blocks = pairs * n_qtiles;
-        if (compute_units % pairs == 0 && blocks > compute_units && blocks <= 2 * static_cast<int64_t>(compute_units))
+        prm.n_qtiles = (seq + kBM * groups - 1) / (kBM * groups);
+        prm.heavy_groups = prm.n_qtiles;
+        const int64_t blocks = pairs * prm.n_qtiles;
+        if (groups == 1 && compute_units % pairs == 0 && blocks > compute_units && blocks <= 2 * static_cast<int64_t>(compute_units))
             prm.heavy_groups = static_cast<int>(compute_units / pairs);
-        const auto kernel = round_scores ? prefill_il_kernel<true> : prefill_il_kernel<false>;
-        static std::atomic<bool> lds_raised[2][kMaxDevices];
-        const int32_t rc_lds = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), kIlSmemBytes,
-                                                  lds_raised[round_scores ? 1 : 0]);
+        static std::atomic<bool> lds_raised[4][kMaxDevices];
+        const void* kernel = groups == 2
+            ? (round_scores ? reinterpret_cast<const void*>(prefill_il_kernel<true, 2>) : reinterpret_cast<const void*>(prefill_il_kernel<false, 2>))
+            : (round_scores ? reinterpret_cast<const void*>(prefill_il_kernel<true, 1>) : reinterpret_cast<const void*>(prefill_il_kernel<false, 1>));
+        const int32_t rc_lds = ensure_dynamic_lds(kernel, kIlSmemBytes, lds_raised[(groups - 1) * 2 + (round_scores ? 1 : 0)]);
         if (rc_lds != QM_OK) return rc_lds;
-        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(pairs * n_qtiles)), dim3(kPfThreads), kIlSmemBytes, s, prm, desc);
+        const dim3 grid(static_cast<unsigned>(blocks));
+        if (groups == 2) {
+            if (round_scores) hipLaunchKernelGGL((prefill_il_kernel<true, 2>), grid, dim3(kPfThreads), kIlSmemBytes, s, prm, desc);
+            else hipLaunchKernelGGL((prefill_il_kernel<false, 2>), grid, dim3(kPfThreads), kIlSmemBytes, s, prm, desc);
+        } else {
+            if (round_scores) hipLaunchKernelGGL((prefill_il_kernel<true, 1>), grid, dim3(kPfThreads), kIlSmemBytes, s, prm, desc);
+            else hipLaunchKernelGGL((prefill_il_kernel<false, 1>), grid, dim3(kPfThreads), kIlSmemBytes, s, prm, desc);
+        }
         return launch_status();
     }
     const bool wave_pairs = which == 2;
