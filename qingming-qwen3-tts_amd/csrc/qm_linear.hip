@@ -209,6 +209,7 @@ inline int32_t launch_linear(const LinearParams& prm, hipStream_t s) {
 // instead of 11 us: a launch here is start + first HBM latency + tail around its streaming time.)
 constexpr int kStagedThreads = 256;
 constexpr int kStagedMaxRows = 8;
+constexpr int kStagedXPerThread = 16;    // input columns a thread can hold in registers (reductions up to 4096)
 constexpr int kStagedLdsBudget = 156 * 1024;
 
 __host__ __device__ inline int staged_row_stride(int reduction) { return 2 * reduction + 64; }   // bytes
@@ -230,23 +231,33 @@ __global__ __launch_bounds__(kStagedThreads) void linear_m1_staged_kernel(Linear
     unsigned char* lds_w = st_smem + staged_x_floats(K) * sizeof(float);
     const int first = static_cast<int>(blockIdx.x) * R;     // first output (channel) of the block
 
-    // ---- request the weight rows: LDS row i of the block <- row (first + i) of its matrix ----------
-    // (DUAL: LDS rows 2c, 2c+1 are the gate and up rows of channel first + c)
-    const int lds_rows = DUAL ? 2 * R : R;
-    const int row_bytes = 2 * K;
-    for (int i = 0; i < lds_rows; ++i) {
-        int out = first + (DUAL ? i >> 1 : i);
-        int m = DUAL ? (i & 1) : 0;
-        if (!DUAL && out >= prm.rows[0]) {
-            out -= prm.rows[0];
+    // Kernel arguments indexed by a run-time matrix number would be fetched again from the argument buffer at
+    // every use (a scalar load and its wait each: 4 500 cycles for the eight rows of a block, measured); the three
+    // entries are picked by selects instead.
+    const int rows0 = prm.rows[0], rows1 = prm.rows[1], rows2 = prm.rows[2];
+    const uint16_t* const weight0 = prm.weight[0];
+    const uint16_t* const weight1 = prm.weight[1];
+    const uint16_t* const weight2 = prm.weight[2];
+    auto matrix_of = [&](int& out) {                        // global output -> (matrix, row in it)
+        int m = 0;
+        if (out >= rows0) {
+            out -= rows0;
             m = 1;
-            if (out >= prm.rows[1]) {
-                out -= prm.rows[1];
+            if (out >= rows1) {
+                out -= rows1;
                 m = 2;
             }
         }
-        if (out >= prm.rows[DUAL ? 0 : m]) break;           // past the last output (wave-uniform)
-        const unsigned char* src = reinterpret_cast<const unsigned char*>(prm.weight[m] + static_cast<int64_t>(out) * K);
+        return m;
+    };
+
+    // ---- request the weight rows: LDS row i of the block <- row (first + i) of its matrix ----------
+    // (DUAL: LDS rows 2c, 2c+1 are the gate and up rows of channel first + c)
+    // The block's rows nearly always lie in one matrix and inside it: then they are requested by straight-line
+    // code (eight rows found one by one, with the matrix looked up per row, took 3 200 cycles of scalar branches
+    // before the first byte was even asked for).
+    const int row_bytes = 2 * K;
+    auto request_row = [&](const unsigned char* src, int i) {
         unsigned char* dst = lds_w + i * row_stride;
         for (int off = wave * 1024; off < row_bytes; off += 4 * 1024) {
             if (off + lane * 16 < row_bytes) {
@@ -255,41 +266,134 @@ __global__ __launch_bounds__(kStagedThreads) void linear_m1_staged_kernel(Linear
                                                  16, 0, 0);
             }
         }
+    };
+    {
+        int first_row = first;
+        const int first_matrix = DUAL ? 0 : matrix_of(first_row);
+        const int matrix_rows = first_matrix == 0 ? rows0 : (first_matrix == 1 ? rows1 : rows2);
+        if (first_row + R <= matrix_rows) {
+            const uint16_t* matrix = first_matrix == 0 ? weight0 : (first_matrix == 1 ? weight1 : weight2);
+            const unsigned char* src = reinterpret_cast<const unsigned char*>(matrix + static_cast<int64_t>(first_row) * K);
+            const unsigned char* src_up = reinterpret_cast<const unsigned char*>(weight1 + static_cast<int64_t>(first_row) * K);
+#pragma unroll
+            for (int i = 0; i < kStagedMaxRows; ++i) {
+                if (i < R) {
+                    if (DUAL) {
+                        request_row(src + static_cast<int64_t>(i) * row_bytes, 2 * i);
+                        request_row(src_up + static_cast<int64_t>(i) * row_bytes, 2 * i + 1);
+                    } else {
+                        request_row(src + static_cast<int64_t>(i) * row_bytes, i);
+                    }
+                }
+            }
+        } else {
+            const int lds_rows = DUAL ? 2 * R : R;
+            for (int i = 0; i < lds_rows; ++i) {
+                int out = first + (DUAL ? i >> 1 : i);
+                const int m = DUAL ? (i & 1) : matrix_of(out);
+                if (out >= (DUAL ? rows0 : (m == 0 ? rows0 : (m == 1 ? rows1 : rows2)))) break;   // past the last output (wave-uniform)
+                const uint16_t* matrix = m == 0 ? weight0 : (m == 1 ? weight1 : weight2);
+                request_row(reinterpret_cast<const unsigned char*>(matrix + static_cast<int64_t>(out) * K), i);
+            }
+        }
+    }
+
+    // ---- the input vector, requested at once: thread t holds columns t, t + 256, ... (up to kStagedXPerThread of
+    // them; longer inputs take the loops below) ----
+    const bool x_in_registers = K <= kStagedThreads * kStagedXPerThread;
+    // (32-bit holders: two 16-bit values sharing a register would make the second load wait for the first)
+    uint32_t x_raw[kStagedXPerThread], add_raw[kStagedXPerThread], norm_raw[kStagedXPerThread];
+    // (a kernel starts with a cold instruction cache, and what it executes before its loads are under way is
+    // paid in fetches: only the loads that are needed are stepped through)
+#pragma unroll
+    for (int i = 0; i < kStagedXPerThread; ++i) x_raw[i] = add_raw[i] = norm_raw[i] = 0u;
+    if (x_in_registers) {
+#pragma unroll
+        for (int i = 0; i < kStagedXPerThread; ++i)
+            if (kStagedThreads * i < K) x_raw[i] = prm.input[min(tid + kStagedThreads * i, K - 1)];
+        if (prm.pre != 0) {
+#pragma unroll
+            for (int i = 0; i < kStagedXPerThread; ++i)
+                if (kStagedThreads * i < K) norm_raw[i] = prm.norm_weight[min(tid + kStagedThreads * i, K - 1)];
+        }
+        if (prm.pre == 2) {
+#pragma unroll
+            for (int i = 0; i < kStagedXPerThread; ++i)
+                if (kStagedThreads * i < K) add_raw[i] = prm.addend[min(tid + kStagedThreads * i, K - 1)];
+        }
+    }
+
+    // ---- what the epilogue adds (bias, residual) is requested now as well, by the lane that will use it ----
+    const int c = tid >> 5;             // output (channel) within the block
+    const int l = tid & 31;             // reference lane
+    const bool live = c < R && first + c < (DUAL ? rows0 : rows0 + rows1 + rows2);
+    int out_row = first + c;
+    int out_matrix = 0;
+    uint32_t bias_raw = 0, residual_raw = 0;
+    bool has_bias = false;
+    if (!DUAL && live && l == 0) {
+        out_matrix = matrix_of(out_row);
+        const uint16_t* bias = out_matrix == 0 ? prm.bias[0] : (out_matrix == 1 ? prm.bias[1] : prm.bias[2]);
+        has_bias = bias != nullptr;
+        if (has_bias) bias_raw = bias[out_row];
+        if (prm.residual) residual_raw = prm.residual[out_row];
     }
 
     // ---- the input vector as fp32, zero-padded to whole steps of 32 -----------------------------------
     const int steps = (K + 31) >> 5;
     if (prm.pre == 0) {
-        for (int k = tid; k < 32 * steps; k += kStagedThreads) lin_x[k] = k < K ? bf2f(prm.input[k]) : 0.0f;
+        if (x_in_registers) {
+#pragma unroll
+            for (int i = 0; i < kStagedXPerThread; ++i) {
+                const int k = tid + kStagedThreads * i;
+                if (k < 32 * steps) lin_x[k] = k < K ? bf2f(static_cast<uint16_t>(x_raw[i])) : 0.0f;
+            }
+        } else {
+            for (int k = tid; k < 32 * steps; k += kStagedThreads) lin_x[k] = k < K ? bf2f(prm.input[k]) : 0.0f;
+        }
     } else {
         // rmsnorm_kernel (R17:8276-8338) / talker_add_postnorm_fused_kernel (R17:16205-16286): thread t
         // sums the squares of columns t, t+256, ... with fmaf; block tree; two roundings per element.
         float local_sum = 0.0f;
-        for (int k = tid; k < K; k += kStagedThreads) {
-            float v = bf2f(prm.input[k]);
+        auto take = [&](int k, uint16_t x_bits, uint16_t add_bits) {
+            float v = bf2f(x_bits);
             if (prm.pre == 2) {
-                const uint16_t r = f2bf(v + bf2f(prm.addend[k]));
+                const uint16_t r = f2bf(v + bf2f(add_bits));
                 if (blockIdx.x == 0) prm.residual_out[k] = r;
                 v = bf2f(r);
             }
             lin_x[k] = v;
             local_sum = fmaf(v, v, local_sum);
+        };
+        if (x_in_registers) {
+#pragma unroll
+            for (int i = 0; i < kStagedXPerThread; ++i) {
+                const int k = tid + kStagedThreads * i;
+                if (k < K) take(k, static_cast<uint16_t>(x_raw[i]), static_cast<uint16_t>(add_raw[i]));
+            }
+        } else {
+            for (int k = tid; k < K; k += kStagedThreads) take(k, prm.input[k], prm.pre == 2 ? prm.addend[k] : static_cast<uint16_t>(0));
         }
         const float total = block_sum_256_like_reference(local_sum, sh_waves, &sh_total);
         const float inverse_rms = 1.0f / sqrtf(total / static_cast<float>(K) + prm.epsilon);
-        for (int k = tid; k < 32 * steps; k += kStagedThreads) {
-            float y = 0.0f;
-            if (k < K) y = round_bf16(round_bf16(lin_x[k] * inverse_rms) * bf2f(prm.norm_weight[k]));
-            lin_x[k] = y;
+        if (x_in_registers) {
+#pragma unroll
+            for (int i = 0; i < kStagedXPerThread; ++i) {
+                const int k = tid + kStagedThreads * i;
+                if (k < 32 * steps) lin_x[k] = k < K ? round_bf16(round_bf16(lin_x[k] * inverse_rms) * bf2f(static_cast<uint16_t>(norm_raw[i]))) : 0.0f;
+            }
+        } else {
+            for (int k = tid; k < 32 * steps; k += kStagedThreads) {
+                float y = 0.0f;
+                if (k < K) y = round_bf16(round_bf16(lin_x[k] * inverse_rms) * bf2f(prm.norm_weight[k]));
+                lin_x[k] = y;
+            }
         }
     }
     __builtin_amdgcn_s_waitcnt(0);      // this wave's global_load_lds writes have landed
     __syncthreads();
 
     // ---- 32 chains per output, one thread each: k = l, l+32, ... in increasing k ----------------------
-    const int c = tid >> 5;             // output (channel) within the block
-    const int l = tid & 31;             // reference lane
-    const bool live = c < R && first + c < (DUAL ? prm.rows[0] : prm.rows[0] + prm.rows[1] + prm.rows[2]);
     const uint16_t* w0 = reinterpret_cast<const uint16_t*>(lds_w + (DUAL ? 2 * c : c) * row_stride) + l;
     const uint16_t* w1 = reinterpret_cast<const uint16_t*>(lds_w + (2 * c + 1) * row_stride) + l;   // DUAL only
     const float* xs = lin_x + l;
@@ -364,26 +468,17 @@ __global__ __launch_bounds__(kStagedThreads) void linear_m1_staged_kernel(Linear
         if (DUAL) up += __shfl_down(up, offset, 32);
     }
     if (l == 0 && live) {
-        int out = first + c;
         if (DUAL) {
             const float gv = bf2f(f2bf(acc));
             const uint16_t act = f2bf(gv / (1.0f + expf(-gv)));
-            prm.output[0][out] = f2bf(bf2f(act) * bf2f(f2bf(up)));
+            prm.output[0][out_row] = f2bf(bf2f(act) * bf2f(f2bf(up)));
         } else {
-            int m = 0;
-            if (out >= prm.rows[0]) {
-                out -= prm.rows[0];
-                m = 1;
-                if (out >= prm.rows[1]) {
-                    out -= prm.rows[1];
-                    m = 2;
-                }
-            }
             float r = acc;
-            if (prm.bias[m]) r += bf2f(prm.bias[m][out]);
+            if (has_bias) r += bf2f(static_cast<uint16_t>(bias_raw));
             uint16_t v = f2bf(r);
-            if (prm.residual) v = f2bf(bf2f(prm.residual[out]) + bf2f(v));
-            prm.output[m][out] = v;
+            if (prm.residual) v = f2bf(bf2f(static_cast<uint16_t>(residual_raw)) + bf2f(v));
+            uint16_t* output = out_matrix == 0 ? prm.output[0] : (out_matrix == 1 ? prm.output[1] : prm.output[2]);
+            output[out_row] = v;
         }
     }
 }
