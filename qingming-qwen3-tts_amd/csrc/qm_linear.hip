@@ -209,7 +209,7 @@ inline int32_t launch_linear(const LinearParams& prm, hipStream_t s) {
 // instead of 11 us: a launch here is start + first HBM latency + tail around its streaming time.)
 constexpr int kStagedThreads = 256;
 constexpr int kStagedMaxRows = 8;
-constexpr int kStagedXPerThread = 16;    // input columns a thread can hold in registers (reductions up to 4096)
+constexpr int kStagedXPerThread = 24;    // input columns a thread can hold in registers (reductions up to 6144)
 constexpr int kStagedLdsBudget = 156 * 1024;
 
 __host__ __device__ inline int staged_row_stride(int reduction) { return 2 * reduction + 64; }   // bytes
@@ -273,18 +273,19 @@ __global__ __launch_bounds__(kStagedThreads) void linear_m1_staged_kernel(Linear
         const int matrix_rows = first_matrix == 0 ? rows0 : (first_matrix == 1 ? rows1 : rows2);
         if (first_row + R <= matrix_rows) {
             const uint16_t* matrix = first_matrix == 0 ? weight0 : (first_matrix == 1 ? weight1 : weight2);
-            const unsigned char* src = reinterpret_cast<const unsigned char*>(matrix + static_cast<int64_t>(first_row) * K);
+            const unsigned char* src = reinterpret_cast<const unsigned char*>(matrix + static_cast<int64_t>(first_row) * K);   // (advances row by row)
             const unsigned char* src_up = reinterpret_cast<const unsigned char*>(weight1 + static_cast<int64_t>(first_row) * K);
-#pragma unroll
-            for (int i = 0; i < kStagedMaxRows; ++i) {
-                if (i < R) {
-                    if (DUAL) {
-                        request_row(src + static_cast<int64_t>(i) * row_bytes, 2 * i);
-                        request_row(src_up + static_cast<int64_t>(i) * row_bytes, 2 * i + 1);
-                    } else {
-                        request_row(src + static_cast<int64_t>(i) * row_bytes, i);
-                    }
+            // (a rolled loop: after its first turn the instructions come from the cache)
+#pragma unroll 1
+            for (int i = 0; i < R; ++i) {
+                if (DUAL) {
+                    request_row(src, 2 * i);
+                    request_row(src_up, 2 * i + 1);
+                    src_up += row_bytes;
+                } else {
+                    request_row(src, i);
                 }
+                src += row_bytes;
             }
         } else {
             const int lds_rows = DUAL ? 2 * R : R;
@@ -349,7 +350,17 @@ __global__ __launch_bounds__(kStagedThreads) void linear_m1_staged_kernel(Linear
                 if (k < 32 * steps) lin_x[k] = k < K ? bf2f(static_cast<uint16_t>(x_raw[i])) : 0.0f;
             }
         } else {
-            for (int k = tid; k < 32 * steps; k += kStagedThreads) lin_x[k] = k < K ? bf2f(prm.input[k]) : 0.0f;
+            // (eight loads at a time: one load per turn would wait for each in turn)
+            for (int k0 = tid; k0 < 32 * steps; k0 += 8 * kStagedThreads) {
+                uint32_t raw[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) raw[u] = prm.input[min(k0 + kStagedThreads * u, K - 1)];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int k = k0 + kStagedThreads * u;
+                    if (k < 32 * steps) lin_x[k] = k < K ? bf2f(static_cast<uint16_t>(raw[u])) : 0.0f;
+                }
+            }
         }
     } else {
         // rmsnorm_kernel (R17:8276-8338) / talker_add_postnorm_fused_kernel (R17:16205-16286): thread t
