@@ -304,24 +304,36 @@ __global__ __launch_bounds__(kStagedThreads) void linear_m1_staged_kernel(Linear
     const bool x_in_registers = K <= kStagedThreads * kStagedXPerThread;
     // (32-bit holders: two 16-bit values sharing a register would make the second load wait for the first)
     uint32_t x_raw[kStagedXPerThread], add_raw[kStagedXPerThread], norm_raw[kStagedXPerThread];
-    // (a kernel starts with a cold instruction cache, and what it executes before its loads are under way is
-    // paid in fetches: only the loads that are needed are stepped through)
+    // A kernel starts with a cold instruction cache: every instruction it executes for the first time costs tens
+    // of cycles of fetch (measured: this kernel's timeline follows the number of distinct instructions on its
+    // path far more than its arithmetic), so the columns are stepped through in batches of four with one test per
+    // batch, nothing is initialised that is not used, and `each_column` below visits exactly what was loaded.
+    auto fetch_columns = [&](const uint16_t* src, uint32_t (&dst)[kStagedXPerThread]) {
 #pragma unroll
-    for (int i = 0; i < kStagedXPerThread; ++i) x_raw[i] = add_raw[i] = norm_raw[i] = 0u;
+        for (int i0 = 0; i0 < kStagedXPerThread; i0 += 4) {
+            if (kStagedThreads * i0 < K) {
+#pragma unroll
+                for (int i = i0; i < i0 + 4; ++i) dst[i] = src[min(tid + kStagedThreads * i, K - 1)];
+            }
+        }
+    };
+    // f(i, k) for this thread's columns k = tid + 256 i < K
+    auto each_column = [&](auto&& f) {
+#pragma unroll
+        for (int i0 = 0; i0 < kStagedXPerThread; i0 += 4) {
+            if (kStagedThreads * i0 < K) {
+#pragma unroll
+                for (int i = i0; i < i0 + 4; ++i) {
+                    const int k = tid + kStagedThreads * i;
+                    if (k < K) f(i, k);
+                }
+            }
+        }
+    };
     if (x_in_registers) {
-#pragma unroll
-        for (int i = 0; i < kStagedXPerThread; ++i)
-            if (kStagedThreads * i < K) x_raw[i] = prm.input[min(tid + kStagedThreads * i, K - 1)];
-        if (prm.pre != 0) {
-#pragma unroll
-            for (int i = 0; i < kStagedXPerThread; ++i)
-                if (kStagedThreads * i < K) norm_raw[i] = prm.norm_weight[min(tid + kStagedThreads * i, K - 1)];
-        }
-        if (prm.pre == 2) {
-#pragma unroll
-            for (int i = 0; i < kStagedXPerThread; ++i)
-                if (kStagedThreads * i < K) add_raw[i] = prm.addend[min(tid + kStagedThreads * i, K - 1)];
-        }
+        fetch_columns(prm.input, x_raw);
+        if (prm.pre != 0) fetch_columns(prm.norm_weight, norm_raw);
+        if (prm.pre == 2) fetch_columns(prm.addend, add_raw);
     }
 
     // ---- what the epilogue adds (bias, residual) is requested now as well, by the lane that will use it ----
@@ -344,11 +356,8 @@ __global__ __launch_bounds__(kStagedThreads) void linear_m1_staged_kernel(Linear
     const int steps = (K + 31) >> 5;
     if (prm.pre == 0) {
         if (x_in_registers) {
-#pragma unroll
-            for (int i = 0; i < kStagedXPerThread; ++i) {
-                const int k = tid + kStagedThreads * i;
-                if (k < 32 * steps) lin_x[k] = k < K ? bf2f(static_cast<uint16_t>(x_raw[i])) : 0.0f;
-            }
+            each_column([&](int i, int k) { lin_x[k] = bf2f(static_cast<uint16_t>(x_raw[i])); });
+            if (tid < 32 * steps - K) lin_x[K + tid] = 0.0f;     // the padding of the last step
         } else {
             // (eight loads at a time: one load per turn would wait for each in turn)
             for (int k0 = tid; k0 < 32 * steps; k0 += 8 * kStagedThreads) {
@@ -377,22 +386,19 @@ __global__ __launch_bounds__(kStagedThreads) void linear_m1_staged_kernel(Linear
             local_sum = fmaf(v, v, local_sum);
         };
         if (x_in_registers) {
-#pragma unroll
-            for (int i = 0; i < kStagedXPerThread; ++i) {
-                const int k = tid + kStagedThreads * i;
-                if (k < K) take(k, static_cast<uint16_t>(x_raw[i]), static_cast<uint16_t>(add_raw[i]));
-            }
+            each_column([&](int i, int k) {
+                take(k, static_cast<uint16_t>(x_raw[i]), prm.pre == 2 ? static_cast<uint16_t>(add_raw[i]) : static_cast<uint16_t>(0));
+            });
         } else {
             for (int k = tid; k < K; k += kStagedThreads) take(k, prm.input[k], prm.pre == 2 ? prm.addend[k] : static_cast<uint16_t>(0));
         }
         const float total = block_sum_256_like_reference(local_sum, sh_waves, &sh_total);
         const float inverse_rms = 1.0f / sqrtf(total / static_cast<float>(K) + prm.epsilon);
         if (x_in_registers) {
-#pragma unroll
-            for (int i = 0; i < kStagedXPerThread; ++i) {
-                const int k = tid + kStagedThreads * i;
-                if (k < 32 * steps) lin_x[k] = k < K ? round_bf16(round_bf16(lin_x[k] * inverse_rms) * bf2f(static_cast<uint16_t>(norm_raw[i]))) : 0.0f;
-            }
+            each_column([&](int i, int k) {
+                lin_x[k] = round_bf16(round_bf16(lin_x[k] * inverse_rms) * bf2f(static_cast<uint16_t>(norm_raw[i])));
+            });
+            if (tid < 32 * steps - K) lin_x[K + tid] = 0.0f;     // the padding of the last step
         } else {
             for (int k = tid; k < 32 * steps; k += kStagedThreads) {
                 float y = 0.0f;
