@@ -550,9 +550,18 @@ class Prefill:
     name = "causal_prefill_b4_s1024_paged16"
     bound = "mfma"
 
-    def __init__(self, qm, dev, seed=44, batch=4, seq=1024):
+    def __init__(self, qm, dev, seed=44, batch=4, seq=1024, split=False):
         import torch
         self.qm, self.batch, self.seq = qm, batch, seq
+        if (batch, seq) != (4, 1024):
+            self.name = "causal_prefill_b%d_s%d_paged16%s" % (batch, seq, "_key_split" if split else "")
+        # key split: a workspace lets up to three blocks share a long query tile (shapes that leave CUs idle)
+        self.workspace, self.workspace_bytes = None, 0
+        if split:
+            self.workspace_bytes = qm.prefill_split_workspace_bytes(batch, seq, 8)
+            self.workspace = torch.zeros(max(self.workspace_bytes, 256) // 4, dtype=torch.int32, device=dev)
+            qm.prefill_split_workspace_init(self.workspace, self.workspace_bytes,
+                                            torch.cuda.current_stream().cuda_stream)
         gd = torch.Generator(device=dev).manual_seed(seed)
         g = torch.Generator(device="cpu").manual_seed(seed)
 
@@ -577,6 +586,12 @@ class Prefill:
 
     def step(self):
         import torch
+        if self.workspace is not None:
+            self.qm.prefill_attention_causal_split(self.q, self.k, self.v, self.out, self.cache, self.table,
+                                                   self.max_pages, self.batch, self.seq, 16, 8, self.workspace,
+                                                   self.workspace_bytes, SCALE, self.status,
+                                                   torch.cuda.current_stream().cuda_stream)
+            return
         self.qm.prefill_attention_causal(self.q, self.k, self.v, self.out, self.cache, self.table, self.max_pages,
                                          self.batch, self.seq, 16, 8, SCALE, self.status,
                                          torch.cuda.current_stream().cuda_stream)
@@ -660,7 +675,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
-    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "predictor", "qkv", "layer", "frame"], default=None,
+    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "predictor", "qkv", "layer",
+                                      "frame"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -693,7 +709,9 @@ def main():
     if args.only:
         make = {"decode512": lambda: SingleDecode(qm, dev, 512, False, 11),
                 "talker2048": lambda: SingleDecode(qm, dev, 2048, True, 12),
-                "prefill": lambda: Prefill(qm, dev), "predictor": lambda: PredictorLoop(qm, dev),
+                "prefill": lambda: Prefill(qm, dev), "prefill1": lambda: Prefill(qm, dev, batch=1),
+                "prefill1split": lambda: Prefill(qm, dev, batch=1, split=True),
+                "predictor": lambda: PredictorLoop(qm, dev),
                 "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev),
                 "frame": lambda: PredictorFrameSteps(qm, dev)}[args.only]
         w = make()
@@ -725,6 +743,9 @@ def main():
             # the same step as the reference launches it: append kernel, then attention
             ("cfg2_talker_step_ctx2048_two_operators", lambda: SingleDecode(qm, dev, 2048, True, 12, one_launch=False)),
             ("cfg4_causal_prefill", lambda: Prefill(qm, dev)),
+            # one prompt, as the talker's prefill runs it: 128 blocks for 256 CUs; the key-split entry fills them
+            ("cfg4b_causal_prefill_one_prompt_1024", lambda: Prefill(qm, dev, batch=1)),
+            ("cfg4b_causal_prefill_one_prompt_1024_key_split", lambda: Prefill(qm, dev, batch=1, split=True)),
             ("cfg5_predictor_loop", lambda: PredictorLoop(qm, dev)),
             ("cfg5_predictor_loop_cache_writeback", lambda: PredictorLoop(qm, dev, write_cache=True)),
             # beyond the five configurations: the M = 1 projection in front of configuration 2

@@ -42,6 +42,7 @@ extern "C" {
 /* bits OR-ed by kernels into the optional device status word */
 #define QM_STATUS_BAD_PAGE      1u /* page table entry outside [0, n_pages)          */
 #define QM_STATUS_BAD_POSITION  2u /* position / length beyond max_pages*page_size   */
+#define QM_STATUS_SPLIT_TIMEOUT 4u /* key-split prefill: a partner's record never came  */
 
 /* ---- paged KV cache descriptor -------------------------------------------- */
 /*
@@ -250,6 +251,39 @@ int32_t qm_prefill_attention_causal(
     const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
     int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads, float scale,
     int64_t kv_stride_token, int64_t kv_stride_head, int64_t kv_stride_batch,
+    uint32_t* status_dev,
+    void* hip_stream);
+
+/*
+ * The same operator with a workspace that lets up to three blocks share the keys of a long query
+ * tile.  No counterpart in the reference (its kernel gives one block a (batch, head, query row)).
+ * A call of qm_prefill_attention_causal whose grid leaves compute units idle (one prompt of 1024
+ * tokens: 128 blocks) lasts as long as the block of the last query tile, which walks over all
+ * keys.  With a workspace the long query tiles are each given to two or three blocks (runs of key
+ * tiles), whose partial results are combined by whichever finishes last.  Results stay within the
+ * operator's tolerance of the unsplit call but are not bit-identical to it (another association
+ * of the sums); they do not depend on the order in which blocks finish.  Rows of query tiles
+ * that are not split, and calls that do not split at all, carry the unsplit call's bits.
+ *   qm_prefill_split_workspace_bytes: bytes needed for (batch, seq, kv_heads) on the current
+ *     device; 0 when the call would not split: fewer than 9 query tiles of 64 rows, or no room
+ *     for the added blocks at two blocks per compute unit (a negative value is an error code).
+ *   qm_prefill_split_workspace_init: once after allocation (a kernel on hip_stream); every call
+ *     leaves the workspace as it found it.  workspace: 256-byte aligned device memory.
+ *   qm_prefill_attention_causal_split: workspace NULL or a shape that does not split: exactly
+ *     qm_prefill_attention_causal; too small for the shape: QM_ERR_WORKSPACE.  Only the default
+ *     kernel (QM_OPT_PREFILL_KERNEL 0 or 3) splits.  Two calls that overlap in time must not share
+ *     a workspace.  QM_STATUS_SPLIT_TIMEOUT in status_dev: a block gave up waiting for a partner's
+ *     record (rows of that query tile are then not written).
+ */
+int64_t qm_prefill_split_workspace_bytes(int32_t batch, int32_t seq, int32_t kv_heads);
+int32_t qm_prefill_split_workspace_init(void* workspace, int64_t workspace_bytes, void* hip_stream);
+int32_t qm_prefill_attention_causal_split(
+    const uint16_t* query, const uint16_t* key, const uint16_t* value,
+    uint16_t* context_out,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads, float scale,
+    int64_t kv_stride_token, int64_t kv_stride_head, int64_t kv_stride_batch,
+    void* workspace, int64_t workspace_bytes,
     uint32_t* status_dev,
     void* hip_stream);
 

@@ -61,6 +61,10 @@ _SIGNATURES = {
     "qm_scatter_kv": (_I32, [_PTR, _PTR, C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _PTR]),
     "qm_prefill_attention_causal": (_I32, [_PTR] * 4 + [C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _I32, _I32,
                                            _F32, C.c_int64, C.c_int64, C.c_int64, _PTR, _PTR]),
+    "qm_prefill_split_workspace_bytes": (C.c_int64, [_I32, _I32, _I32]),
+    "qm_prefill_split_workspace_init": (_I32, [_PTR, C.c_int64, _PTR]),
+    "qm_prefill_attention_causal_split": (_I32, [_PTR] * 4 + [C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _I32, _I32,
+                                                 _F32, C.c_int64, C.c_int64, C.c_int64, _PTR, C.c_int64, _PTR, _PTR]),
     "qm_predictor_attention_loop": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _I32, _F32, _PTR]),
     "qm_predictor_attention_staged": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _PTR]),
     "qm_linear_m1": (_I32, [_PTR] * 5 + [_I32, _I32, _PTR]),
@@ -210,6 +214,31 @@ def prefill_attention_causal(query, key, value, out, cache, page_table, max_page
         C.byref(cache) if cache is not None else None, _addr(page_table), max_pages, batch, seq,
         q_heads, kv_heads, scale, kv_strides[0], kv_strides[1], kv_strides[2], _addr(status), stream),
         "qm_prefill_attention_causal")
+
+
+def prefill_split_workspace_bytes(batch, seq, kv_heads):
+    """Bytes of workspace with which prefill_attention_causal_split shares long query tiles between
+    two blocks on the current device; 0 when that shape would not split."""
+    n = lib().qm_prefill_split_workspace_bytes(batch, seq, kv_heads)
+    if n < 0:
+        _check(int(n), "qm_prefill_split_workspace_bytes")
+    return int(n)
+
+
+def prefill_split_workspace_init(workspace, workspace_bytes, stream=0):
+    _check(lib().qm_prefill_split_workspace_init(_addr(workspace), workspace_bytes, stream),
+           "qm_prefill_split_workspace_init")
+
+
+def prefill_attention_causal_split(query, key, value, out, cache, page_table, max_pages, batch, seq, q_heads,
+                                   kv_heads, workspace, workspace_bytes, scale=SCALE_128, status=None, stream=0,
+                                   kv_strides=(0, 0, 0)):
+    _check(lib().qm_prefill_attention_causal_split(
+        _addr(query), _addr(key), _addr(value), _addr(out),
+        C.byref(cache) if cache is not None else None, _addr(page_table), max_pages, batch, seq,
+        q_heads, kv_heads, scale, kv_strides[0], kv_strides[1], kv_strides[2], _addr(workspace), workspace_bytes,
+        _addr(status), stream),
+        "qm_prefill_attention_causal_split")
 
 
 def predictor_attention_loop(q, k, v, gq, gk, cos, sin, out, k_cache_out, v_cache_out, units, n_layers,

@@ -110,6 +110,8 @@ struct qm_talker {
     // the prompt pass's row buffers ([rows][...]), allocated by the first prefill for max_cache rows
     qm_engine::DeviceBuffer p_hidden_a, p_hidden_b, p_norm, p_q, p_k, p_v, p_q_rotated, p_k_rotated, p_context, p_residual,
         p_swiglu, p_cosine, p_sine;
+    // the prompt pass's key-split workspace (prompts whose attention grid leaves compute units idle), grown on demand
+    qm_engine::DeviceBuffer p_split;
 
     ~qm_talker() {
         if (own_stream && stream) (void)hipStreamDestroy(stream);
@@ -289,7 +291,8 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
 //   rmsnorm                                   -> qm_rmsnorm_rows
 //   3 x linear_generic (q, k, v)              -> 3 x qm_linear_rows
 //   2 x rmsnorm + 2 x rope_rows               -> 2 x qm_norm_rope_rows
-//   scatter_prefill_cache + attention         -> qm_prefill_attention_causal (writes the cache itself)
+//   scatter_prefill_cache + attention         -> qm_prefill_attention_causal_split (writes the cache itself; long
+//                                                query tiles of a prompt are shared by two or three blocks)
 //   linear_generic (o_proj) + add             -> qm_linear_rows with the residual folded in
 //   rmsnorm                                   -> qm_rmsnorm_rows
 //   2 x linear_generic + swiglu               -> qm_gate_up_swiglu_rows
@@ -310,6 +313,13 @@ static const uint16_t* prefill(qm_talker& e, const uint16_t* input_device, const
     }
     reset_talker(e, rows);
     hipStream_t s = e.stream;
+    const int64_t split_bytes = qm_prefill_split_workspace_bytes(1, rows, e.kv_heads);
+    if (split_bytes < 0) op_check(static_cast<int32_t>(split_bytes), "prefill key-split workspace size");
+    if (static_cast<size_t>(split_bytes) > e.p_split.bytes()) {
+        hip_check(hipStreamSynchronize(s), "prefill workspace growth");   // nothing in flight reads the old one
+        e.p_split = DeviceBuffer(static_cast<size_t>(split_bytes));
+        op_check(qm_prefill_split_workspace_init(e.p_split.raw(), split_bytes, s), "prefill key-split workspace init");
+    }
     const size_t rope_bytes = static_cast<size_t>(rows) * kHeadDim * 2;
     hip_check(hipMemcpyAsync(e.p_hidden_a.raw(), input_device, static_cast<size_t>(rows) * kHidden * 2,
                              hipMemcpyDeviceToDevice, s), "prefill input copy");
@@ -331,8 +341,9 @@ static const uint16_t* prefill(qm_talker& e, const uint16_t* input_device, const
                                    e.q_heads, kEpsilon, s), "prefill q norm + RoPE");
         op_check(qm_norm_rope_rows(e.p_k.u16(), w.k_norm.data(), e.p_cosine.u16(), e.p_sine.u16(), e.p_k_rotated.u16(), rows,
                                    e.kv_heads, kEpsilon, s), "prefill k norm + RoPE");
-        op_check(qm_prefill_attention_causal(e.p_q_rotated.u16(), e.p_k_rotated.u16(), e.p_v.u16(), e.p_context.u16(), &cache,
-                                             nullptr, 1, 1, rows, e.q_heads, e.kv_heads, kScale, 0, 0, 0, nullptr, s),
+        op_check(qm_prefill_attention_causal_split(e.p_q_rotated.u16(), e.p_k_rotated.u16(), e.p_v.u16(), e.p_context.u16(),
+                                                   &cache, nullptr, 1, 1, rows, e.q_heads, e.kv_heads, kScale, 0, 0, 0,
+                                                   split_bytes > 0 ? e.p_split.raw() : nullptr, split_bytes, nullptr, s),
                  "prefill attention + cache write");
         op_check(qm_linear_rows(e.p_context.u16(), w.o_weight.data(), w.o_bias.data(), current->u16(), e.p_residual.u16(),
                                 rows, kHidden, e.q_dim, s), "prefill o_proj + residual");

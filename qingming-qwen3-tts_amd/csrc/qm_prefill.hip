@@ -83,6 +83,11 @@ struct PrefillParams {
     int kv_heads;
     int n_qtiles;
     int heavy_groups;            // (interleaved kernel) leading groups of blocks, heaviest query tile first; the rest ascend
+    // (interleaved kernel, key split) a query tile of n key tiles is shared by min(ceil(n / split_chunk), 3) blocks
+    int split_chunk;             // 0: no query tile is split
+    int split_slots;             // query tiles per pair that are split (the last ones)
+    float* split_partials;       // [pair][split query tile][part][kSplitRecordFloats]
+    int* split_tickets;          // [pair][split query tile][8]: arrivals, record of part p published; zero between launches
     float scale;
 };
 
@@ -1064,9 +1069,36 @@ constexpr int kIlSmemBytes = (2 * kIlRing > static_cast<int>(sizeof(PfStage)) * 
                                  ? 2 * kIlRing : static_cast<int>(sizeof(PfStage)) * kPfStages;
 static_assert(kIlSmemBytes >= 2 * 4 * 32 * kOS * 2, "the output staging area (two column groups per wave) reuses the rings");
 
+// Key split: when the whole grid is resident at once and CUs are left over, the kernel lasts as long as the
+// block of the last query tile, a serial chain over all key tiles.  A query tile of many key tiles is then given
+// to up to three blocks, each taking a run of key tiles (the last one also the tile's own, diagonal keys) and
+// ending with an unnormalised O, a reference maximum and a sum per column.  Blocks draw a ticket when they are
+// done: all but the last to arrive publish their record and leave; the last waits for the records of blocks
+// that are already running (bounded), combines  sum over parts of part * w_part  in the order of the parts (the
+// same expression whoever arrives last: the result does not depend on the order of arrival) and writes the
+// output.  Records go through agent-scope atomic stores and loads: they bypass the per-XCD L2s, which are not
+// coherent with one another, and need no fence.
+constexpr int kSplitMaxParts = 3;
+constexpr int kSplitRecordFloats = 66 * kPfThreads;        // per thread: 64 of O, the reference maximum, the sum
+constexpr int kSplitTicketInts = 8;                        // arrivals, one flag per part, padding
+constexpr unsigned kSplitSpinLimit = 1u << 20;
+__host__ __device__ inline int split_parts(int tiles, int chunk) {
+    const int parts = chunk > 0 ? (tiles + chunk - 1) / chunk : 1;
+    return parts > kSplitMaxParts ? kSplitMaxParts : parts;
+}
+// First key tile of part `part` (even: a tile's buffer is its parity); `parts` itself gives the end.  The last part
+// also works through the query tile's own keys outside the pipeline and usually combines the records: it is given
+// about three key tiles fewer than the others, and two at least (one for the pipeline, and the tile's own).
+__host__ __device__ inline int split_first_tile(int tiles, int parts, int part) {
+    const int even_share = 2 * ((part * (tiles + 3)) / (2 * parts));
+    const int latest = 2 * ((tiles - 2) / 2);
+    return even_share < latest ? even_share : latest;
+}
+
 template <bool ROUND, int NC>
 __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const qm_kv_cache& cache,
-                                                unsigned char* il_smem, int qt, int bh) {
+                                                unsigned char* il_smem, int qt, int bh,
+                                                int part = 0, int parts = 1, int split_slot = 0) {
     typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
     unsigned char* lds_k = il_smem;                 // [2][64 rows][256 B]
     unsigned char* lds_v = il_smem + kIlRing;       // [2][64 rows][256 B]
@@ -1084,6 +1116,10 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
     const int q0 = qt * kBM * NC;                    // first query row of the block
     const int n_full = qt * NC;                      // key tiles wholly before the block's rows: the pipeline's
     const int last_tile = n_full + NC - 1;           // the block's own rows span the tiles n_full .. last_tile
+    // the pipeline's tiles of this block: all before the block's own, or one part of them
+    const bool last_part = part == parts - 1;        // the one that also takes the block's own tiles
+    const int t_first = split_first_tile(n_full + 1, parts, part);
+    const int t_end = last_part ? n_full : split_first_tile(n_full + 1, parts, part + 1);
     const int my_head = 2 * kvh + (col >> 4);
     // column group c of this wave: rows group_row0(c) .. + 15
     auto group_row0 = [&](int c) { return q0 + 16 * (NC * wave + c); };
@@ -1092,7 +1128,7 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
     const int kv_row32 = static_cast<int>(prm.kv_stride_token);
 
     // ---- K/V rows of the block's own tiles for the pages: requested first, written after the first wait ----
-    const bool to_pages = prm.has_cache != 0;
+    const bool to_pages = prm.has_cache != 0 && last_part;
     int phys[4 * NC];
     uint4 kx[4 * NC], vx[4 * NC];
     uint32_t page_err = 0;
@@ -1138,9 +1174,9 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         for (int j = 0; j < 4; ++j) load_piece(v_src, lds_v, tile, slot, j);
     };
 
-    load_k(0, 0);
-    load_v(0, 0);
-    load_k(1, 1);                                    // qt >= 1 here: tile 1 exists
+    load_k(t_first, 0);                              // t_first is even: tile t lives in buffer t % 2
+    load_v(t_first, 0);
+    load_k(t_first + 1, 1);                          // qt >= 1, and every part holds two tiles at least: it exists
     bf16x8_t qf[NC][8];
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
@@ -1570,16 +1606,17 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         stage(s_b, s_a, p_a, p_b, kraw, vraw, int_c<nxt * kSpKTile + 32 * kKR>{}, int_c<cur * kSpKTile + 32 * kKR>{},
               []() {}, [](int) {});
     };
-    for (int t = 0; t < n_full; t += 2) {
+    // (a part before the last requests, and multiplies into scores nobody reads, up to two tiles past its end: they exist)
+    for (int t = t_first; t < t_end; t += 2) {
         tile_body(t, int_c<0>{});
-        if (t + 1 < n_full) tile_body(t + 1, int_c<1>{});
+        if (t + 1 < t_end) tile_body(t + 1, int_c<1>{});
     }
     wait_vm<0>();
     lds_barrier();                                   // what has been loaded has landed for every wave, and every
                                                      // wave has taken its fragments of V tile n_full - 1
     if (NC == 2) load_v(last_tile, last_tile & 1);   // (the pipeline requested V up to tile n_full only)
 
-    // ---- drain: P.V of chunk (n_full - 1, 1), then the block's own tiles chunk by chunk ----
+    // ---- drain: P.V of chunk (t_end - 1, 1), then the block's own tiles chunk by chunk ----
     {
         bf16x8_t vf[8];
         v_arrived(vraw, vf);
@@ -1614,6 +1651,7 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
                 o[c][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * kg + dt], p.g[kg], o[c][dt], 0, 0, 0);
         }
     };
+    if (last_part)
 #pragma unroll
     for (int d = 0; d < 2 * NC; ++d) {
         const int tile = n_full + (d >> 1);
@@ -1656,6 +1694,99 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         }
     }
     lds_barrier();   // every wave is done with the rings: they become the output staging area
+
+    // ---- a split query tile: all blocks but the last to arrive publish, the last combines ----
+    if (NC == 1 && parts > 1) {
+        const int64_t slot = static_cast<int64_t>(bh) * prm.split_slots + split_slot;
+        float* records = prm.split_partials + slot * kSplitMaxParts * kSplitRecordFloats + tid;
+        int* tickets = prm.split_tickets + slot * kSplitTicketInts;
+        int* note = reinterpret_cast<int*>(il_smem);
+        if (tid == 0) note[0] = __hip_atomic_fetch_add(&tickets[0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (note[0] < parts - 1) {
+            float* record = records + part * kSplitRecordFloats;
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    __hip_atomic_store(record + (16 * dt + r) * kPfThreads, o[0][dt][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(record + 64 * kPfThreads, m_run[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(record + 65 * kPfThreads, l_run[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            wait_vm<0>();                            // the stores have been acknowledged
+            __syncthreads();
+            if (tid == 0) __hip_atomic_store(&tickets[1 + part], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+        if (tid == 0) {
+            // the publishers drew their tickets before this block and are running: short waits, bounded all the same
+            unsigned spins = 0;
+            for (int p = 0; p < parts; ++p) {
+                if (p == part) continue;
+                while (__hip_atomic_load(&tickets[1 + p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0 && spins < kSplitSpinLimit) {
+                    __builtin_amdgcn_s_sleep(2);
+                    ++spins;
+                }
+            }
+            note[1] = spins < kSplitSpinLimit ? 1 : 0;
+            for (int i = 0; i <= parts; ++i)         // as found, for the next launch
+                __hip_atomic_store(&tickets[i], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (note[1] == 0) {
+            if (tid == 0 && prm.status) atomicOr(prm.status, QM_STATUS_SPLIT_TIMEOUT);
+            return;
+        }
+        float m_part[kSplitMaxParts], w_part[kSplitMaxParts];
+        float m_all = -INFINITY;
+#pragma unroll
+        for (int p = 0; p < kSplitMaxParts; ++p) {
+            m_part[p] = -INFINITY;
+            if (p < parts)
+                m_part[p] = p == part ? m_run[0]
+                          : __hip_atomic_load(records + p * kSplitRecordFloats + 64 * kPfThreads, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            m_all = fmaxf(m_all, m_part[p]);
+        }
+        float l_all = 0.0f;
+#pragma unroll
+        for (int p = 0; p < kSplitMaxParts; ++p) {
+            w_part[p] = m_part[p] == -INFINITY ? 0.0f : fast_exp2((m_part[p] - m_all) * coef);
+            if (p < parts) {
+                const float l_p = p == part ? l_run[0]
+                                : __hip_atomic_load(records + p * kSplitRecordFloats + 65 * kPfThreads, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                l_all = p == 0 ? l_p * w_part[p] : l_all + l_p * w_part[p];
+            }
+        }
+        l_run[0] = l_all;
+        // (two of the four d tiles at a time: every record load of a round is in flight before the first is used;
+        // the other parts' values sit in three slots, part p in slot p or p - 1, whichever skips this block's own)
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            float term[kSplitMaxParts - 1][32];
+#pragma unroll
+            for (int j = 0; j < kSplitMaxParts - 1; ++j) {
+                if (j >= parts - 1) continue;
+                const float* src = records + (j < part ? j : j + 1) * kSplitRecordFloats + 32 * half * kPfThreads;
+#pragma unroll
+                for (int i = 0; i < 32; ++i)
+                    term[j][i] = __hip_atomic_load(src + i * kPfThreads, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                float sum = 0.0f;
+#pragma unroll
+                for (int p = 0; p < kSplitMaxParts; ++p) {
+                    if (p >= parts) continue;
+                    float x = o[0][2 * half + i / 16][i % 16];
+                    if (p < part && p < kSplitMaxParts - 1) x = term[p < kSplitMaxParts - 1 ? p : 0][i];
+                    if (p > part) x = term[p > 0 ? p - 1 : 0][i];
+                    x *= w_part[p];
+                    sum = p == 0 ? x : sum + x;
+                }
+                o[0][2 * half + i / 16][i % 16] = sum;
+            }
+        }
+        __syncthreads();                             // the notes have been read: the area is the staging area again
+    }
 
     // ---- normalise, stage through LDS, write 16 bytes per lane ----
     uint16_t* stage_out = reinterpret_cast<uint16_t*>(il_smem) + wave * NC * 32 * kOS;
@@ -1701,7 +1832,20 @@ __global__ __launch_bounds__(kPfThreads, (NC == 1 ? 2 : 1)) void prefill_il_kern
     // the second block of a CU being the one CUs later in the grid) the blocks after the first `CUs`
     // ascend from the lightest tile, so that a CU's two blocks are a heavy and a light one.
     const int group = bid / pairs;
-    const int qt = group < prm.heavy_groups ? prm.n_qtiles - 1 - group : group - prm.heavy_groups;
+    // key split: the blocks of a query tile's parts follow one another, heaviest query tile first
+    int qt, part = 0, parts = 1;
+    if (NC == 1 && prm.split_chunk > 0) {
+        int left = group;
+        for (qt = prm.n_qtiles - 1; qt > 0; --qt) {
+            parts = split_parts(qt + 1, prm.split_chunk);
+            if (left < parts) break;
+            left -= parts;
+        }
+        part = qt > 0 ? left : 0;
+        parts = qt > 0 ? parts : 1;
+    } else {
+        qt = group < prm.heavy_groups ? prm.n_qtiles - 1 - group : group - prm.heavy_groups;
+    }
     if (qt == 0) {
         prefill_body<true, ROUND>(prm, cache, il_smem, 0, bid % pairs);
         if (NC == 2 && prm.seq > kBM) {
@@ -1709,21 +1853,99 @@ __global__ __launch_bounds__(kPfThreads, (NC == 1 ? 2 : 1)) void prefill_il_kern
             prefill_body<false, ROUND>(prm, cache, il_smem, 1, bid % pairs);
         }
     } else {
-        prefill_il_body<ROUND, NC>(prm, cache, il_smem, qt, bid % pairs);
+        prefill_il_body<ROUND, NC>(prm, cache, il_smem, qt, bid % pairs, part, parts, prm.n_qtiles - 1 - qt);
     }
+}
+
+// Sets the tickets of a key-split workspace to zero (a kernel, not a memset: callers may capture it).
+__global__ void prefill_split_clear_kernel(int* tickets, int64_t count) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < count) tickets[i] = 0;
+}
+
+// The key split of a call: how long a run of key tiles a block takes, and the workspace that takes.
+struct SplitPlan {
+    int chunk = 0;               // 0: no split
+    int slots = 0;               // split query tiles per pair
+    int64_t groups = 0;          // blocks per pair
+    int64_t ticket_bytes = 0;    // rounded up to 256
+    int64_t bytes = 0;           // tickets + records
+};
+
+// Split when the grid stays resident at once with the added blocks: then the kernel lasts as long as the longest
+// chain and the chip has room for more blocks.  The shortest run of key tiles is taken with which every block still
+// has a CU to itself, else the shortest with at most two blocks per CU (beyond that the added blocks would have
+// to wait for a CU and the split loses: a block spends 12 000 to 16 000 cycles outside its pipeline, about six key
+// tiles' worth; measured 4 x 1024: 32 us whole, 41 us in halves).  Publishing, waiting and combining cost about
+// as much as three key tiles (measured: runs of four on 384 tokens 14.2 us against 13.4 us whole): runs are six
+// key tiles at least and the longest chain has to drop by three.
+static SplitPlan plan_split(int64_t pairs, int seq, int compute_units) {
+    SplitPlan plan;
+    const int n_qtiles = (seq + kBM - 1) / kBM;
+    for (int per_cu = 1; per_cu <= 2 && plan.chunk == 0; ++per_cu) {
+        for (int chunk = 6; chunk + 3 <= n_qtiles; ++chunk) {
+            int64_t groups = 0;
+            for (int qt = 0; qt < n_qtiles; ++qt) groups += split_parts(qt + 1, chunk);
+            if (pairs * groups > per_cu * static_cast<int64_t>(compute_units)) continue;
+            plan.chunk = chunk;
+            plan.slots = n_qtiles - chunk;                    // query tiles of more than `chunk` key tiles
+            plan.groups = groups;
+            // (tickets take the same room for every shape, that of the most split query tiles a resident grid can
+            // hold: a workspace that has served one shape holds no record where another shape keeps tickets)
+            const int64_t items = pairs * plan.slots;
+            plan.ticket_bytes = (2 * static_cast<int64_t>(compute_units) * kSplitTicketInts * static_cast<int64_t>(sizeof(int)) + 255) / 256 * 256;
+            plan.bytes = plan.ticket_bytes + items * kSplitMaxParts * kSplitRecordFloats * static_cast<int64_t>(sizeof(float));
+            break;
+        }
+    }
+    return plan;
+}
+
+static int32_t device_compute_units(int* compute_units) {
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err == hipSuccess) err = hipDeviceGetAttribute(compute_units, hipDeviceAttributeMultiprocessorCount, device);
+    return err == hipSuccess ? QM_OK : hip_code(err);
 }
 
 }  // namespace qm
 
 
-extern "C" int32_t qm_prefill_attention_causal(
+extern "C" int64_t qm_prefill_split_workspace_bytes(int32_t batch, int32_t seq, int32_t kv_heads) {
+    using namespace qm;
+    if (batch <= 0 || seq <= 0 || kv_heads <= 0) return 0;
+    int compute_units = 0;
+    const int32_t rc = device_compute_units(&compute_units);
+    if (rc != QM_OK) return rc;
+    return plan_split(static_cast<int64_t>(batch) * kv_heads, seq, compute_units).bytes;
+}
+
+extern "C" int32_t qm_prefill_split_workspace_init(void* workspace, int64_t workspace_bytes, void* hip_stream) {
+    using namespace qm;
+    if (workspace_bytes < 0) return QM_ERR_ARGUMENT;
+    if (workspace_bytes == 0) return QM_OK;
+    if (!workspace) return QM_ERR_NULL;
+    if (reinterpret_cast<uintptr_t>(workspace) & 255) return QM_ERR_GEOMETRY;
+    // tickets lie in front of the records; clearing the whole area is the simple rule that needs no geometry
+    const int64_t count = workspace_bytes / static_cast<int64_t>(sizeof(int));
+    const int64_t blocks = (count + 255) / 256;
+    if (blocks > 0x7fffffffLL) return QM_ERR_ARGUMENT;
+    hipLaunchKernelGGL(prefill_split_clear_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
+                       static_cast<hipStream_t>(hip_stream), static_cast<int*>(workspace), count);
+    return launch_status();
+}
+
+static int32_t prefill_attention_entry(
     const uint16_t* query, const uint16_t* key, const uint16_t* value,
     uint16_t* context_out,
     const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
     int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads, float scale,
     int64_t kv_stride_token, int64_t kv_stride_head, int64_t kv_stride_batch,
+    void* workspace, int64_t workspace_bytes,
     uint32_t* status_dev, void* hip_stream) {
     using namespace qm;
+    if (workspace_bytes < 0 || (workspace_bytes > 0 && !workspace)) return QM_ERR_ARGUMENT;
+    if (reinterpret_cast<uintptr_t>(workspace) & 255) return QM_ERR_GEOMETRY;
     if (kv_stride_token == 0 && kv_stride_head == 0 && kv_stride_batch == 0) {
         kv_stride_token = static_cast<int64_t>(kv_heads) * kDim;     // [batch][seq][kv_heads][128]
         kv_stride_head = kDim;
@@ -1763,6 +1985,7 @@ extern "C" int32_t qm_prefill_attention_causal(
     prm.kv_stride_token = kv_stride_token; prm.kv_stride_head = kv_stride_head; prm.kv_stride_batch = kv_stride_batch;
     prm.batch = batch; prm.seq = seq; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
     prm.heavy_groups = n_qtiles;
+    prm.split_chunk = 0; prm.split_slots = 0; prm.split_partials = nullptr; prm.split_tickets = nullptr;
 
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     const bool round_scores = option_value(QM_OPT_PREFILL_SCORE_ROUNDING) != 0;
@@ -1773,15 +1996,23 @@ extern "C" int32_t qm_prefill_attention_causal(
     // (its running maximum is taken before the scores are scaled: a negative scale goes to the uniform waves)
     if ((which == 0 || which >= 3) && scale >= 0.0f) {
         const int groups = which == 4 ? 2 : 1;                     // column groups (16 rows x 2 heads) per wave
-        int device = 0, compute_units = 0;
-        hipError_t err = hipGetDevice(&device);
-        if (err == hipSuccess) err = hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device);
-        if (err != hipSuccess) return hip_code(err);
+        int compute_units = 0;
+        const int32_t rc_cu = device_compute_units(&compute_units);
+        if (rc_cu != QM_OK) return rc_cu;
         prm.n_qtiles = (seq + kBM * groups - 1) / (kBM * groups);
         prm.heavy_groups = prm.n_qtiles;
-        const int64_t blocks = pairs * prm.n_qtiles;
-        if (groups == 1 && compute_units % pairs == 0 && blocks > compute_units && blocks <= 2 * static_cast<int64_t>(compute_units))
+        int64_t blocks = pairs * prm.n_qtiles;
+        const SplitPlan split = groups == 1 && workspace ? plan_split(pairs, seq, compute_units) : SplitPlan();
+        if (split.chunk > 0) {
+            if (workspace_bytes < split.bytes) return QM_ERR_WORKSPACE;
+            prm.split_chunk = split.chunk;
+            prm.split_slots = split.slots;
+            prm.split_tickets = static_cast<int*>(workspace);
+            prm.split_partials = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + split.ticket_bytes);
+            blocks = pairs * split.groups;
+        } else if (groups == 1 && compute_units % pairs == 0 && blocks > compute_units && blocks <= 2 * static_cast<int64_t>(compute_units)) {
             prm.heavy_groups = static_cast<int>(compute_units / pairs);
+        }
         static std::atomic<bool> lds_raised[4][kMaxDevices];
         const void* kernel = groups == 2
             ? (round_scores ? reinterpret_cast<const void*>(prefill_il_kernel<true, 2>) : reinterpret_cast<const void*>(prefill_il_kernel<false, 2>))
@@ -1816,4 +2047,30 @@ extern "C" int32_t qm_prefill_attention_causal(
     if (rc_lds != QM_OK) return rc_lds;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(pairs * n_qtiles)), dim3(kPfThreads), smem, s, prm, desc);
     return launch_status();
+}
+
+
+extern "C" int32_t qm_prefill_attention_causal(
+    const uint16_t* query, const uint16_t* key, const uint16_t* value,
+    uint16_t* context_out,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads, float scale,
+    int64_t kv_stride_token, int64_t kv_stride_head, int64_t kv_stride_batch,
+    uint32_t* status_dev, void* hip_stream) {
+    return prefill_attention_entry(query, key, value, context_out, cache, page_table, max_pages, batch, seq, q_heads,
+                                   kv_heads, scale, kv_stride_token, kv_stride_head, kv_stride_batch, nullptr, 0,
+                                   status_dev, hip_stream);
+}
+
+extern "C" int32_t qm_prefill_attention_causal_split(
+    const uint16_t* query, const uint16_t* key, const uint16_t* value,
+    uint16_t* context_out,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads, float scale,
+    int64_t kv_stride_token, int64_t kv_stride_head, int64_t kv_stride_batch,
+    void* workspace, int64_t workspace_bytes,
+    uint32_t* status_dev, void* hip_stream) {
+    return prefill_attention_entry(query, key, value, context_out, cache, page_table, max_pages, batch, seq, q_heads,
+                                   kv_heads, scale, kv_stride_token, kv_stride_head, kv_stride_batch, workspace,
+                                   workspace_bytes, status_dev, hip_stream);
 }

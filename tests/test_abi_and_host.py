@@ -70,6 +70,17 @@ def test_host_validation_without_device(qm):
     assert lib.qm_decode_attention(fake, C.byref(c), fake, 4, fake, 16, -2, -1, 0.1, None, 0, None) == -5
     assert lib.qm_norm_rope_rows(fake, fake, fake, fake, fake, -1, 16, 1e-6, None) == -5
     assert lib.qm_prefill_attention_causal(fake, fake, fake, fake, None, None, 0, 1, 64, 16, 4, 0.1, 0, 0, 0, None, None) == -2
+    # the key-split prefill entry checks its workspace arguments before anything else
+    split = lib.qm_prefill_attention_causal_split
+    assert split(fake, fake, fake, fake, None, None, 0, 1, 64, 16, 8, 0.1, 0, 0, 0, None, -1, None, None) == -5
+    assert split(fake, fake, fake, fake, None, None, 0, 1, 64, 16, 8, 0.1, 0, 0, 0, None, 256, None, None) == -5
+    assert split(fake, fake, fake, fake, None, None, 0, 1, 64, 16, 8, 0.1, 0, 0, 0, C.c_void_p(4096 + 16), 256, None, None) == -2
+    assert split(fake, fake, fake, fake, None, None, 0, 1, 64, 16, 4, 0.1, 0, 0, 0, None, 0, None, None) == -2
+    assert split(fake, fake, fake, fake, None, None, 0, 0, 64, 16, 8, 0.1, 0, 0, 0, None, 0, None, None) == 0
+    assert lib.qm_prefill_split_workspace_init(None, 0, None) == 0
+    assert lib.qm_prefill_split_workspace_init(None, 256, None) == -1
+    assert lib.qm_prefill_split_workspace_init(fake, -1, None) == -5
+    assert lib.qm_prefill_split_workspace_bytes(0, 1024, 8) == 0
     assert lib.qm_predictor_attention_loop(fake, fake, fake, fake, fake, fake, fake, fake, None, None, 1, 1, 17, 1, 1e-6, None) == -5
     assert lib.qm_predictor_attention_loop(fake, fake, fake, fake, fake, fake, fake, fake, None, None, 1, 1, 16, 3, 1e-6, None) == -5
     # empty work is a successful no-op

@@ -142,6 +142,59 @@ def test_engine_rejects_a_checkpoint_with_the_wrong_geometry(engine, dev, tmp_pa
     assert err.value.code == -8
 
 
+def test_engine_prefill_of_a_long_prompt_shares_query_tiles_between_blocks(engine, oracle, qm, dev, tmp_path):
+    """A 650-token prompt: qm_talker_prefill hands the attention a key-split workspace (long query tiles are
+    shared by two blocks).  Judged against the same prompt with the uniform-waves prefill kernel chosen, which
+    ignores the workspace: layer 0 caches to the bit, last-row hidden vector and deeper caches within the
+    budget the oracle chain is given below (two association orders of the same sums)."""
+    import ctypes as C
+    import torch
+    _checkpoint(str(tmp_path), True)
+    long_cache, S = 704, 650
+    assert qm.prefill_split_workspace_bytes(1, S, 8) > 0
+    hip = C.CDLL("libamdhip64.so")
+    x = oracle.normal_bf16((S, H), 131)
+    cos, sin = engine.rope_rows(S, 0)
+    xd = torch.from_numpy(x.view(np.int16)).to(dev)
+    runs = {}
+    try:
+        for choice in (0, 1):
+            qm.set_option(qm.OPT_PREFILL_KERNEL, choice)
+            talker = engine.Talker(str(tmp_path), long_cache)
+            hidden = []
+            for _ in range(2):                      # the second prompt finds the workspace as the first left it
+                address = talker.prefill(xd, cos, sin, S)
+                talker.synchronize()
+                out = torch.empty(H, dtype=torch.int16, device=dev)
+                assert hip.hipMemcpy(C.c_void_p(out.data_ptr()), C.c_void_p(address), C.c_size_t(H * 2), 3) == 0
+                hidden.append(to_u16(out))
+            assert np.array_equal(hidden[0], hidden[1])
+            caches = []
+            for layer in range(LAYERS):
+                ka, va = talker.cache_addresses(layer)
+                kd = np.zeros((8, long_cache, 128), dtype=np.uint16)
+                vd = np.zeros_like(kd)
+                assert hip.hipMemcpy(kd.ctypes.data_as(C.c_void_p), C.c_void_p(ka), C.c_size_t(kd.nbytes), 2) == 0
+                assert hip.hipMemcpy(vd.ctypes.data_as(C.c_void_p), C.c_void_p(va), C.c_size_t(vd.nbytes), 2) == 0
+                caches.append((kd, vd))
+            runs[choice] = (hidden[0], caches)
+            del talker
+    finally:
+        qm.set_option(qm.OPT_PREFILL_KERNEL, 0)
+
+    def gap(a, b):
+        return np.max(np.abs(oracle.bf16_to_f32(a).astype(np.float64) - oracle.bf16_to_f32(b).astype(np.float64)))
+
+    assert gap(runs[0][0], runs[1][0]) <= 0.0625
+    for layer in range(LAYERS):
+        for a, b in zip(runs[0][1][layer], runs[1][1][layer]):
+            assert not a[:, S:].any()
+            if layer == 0:
+                assert np.array_equal(a, b)
+            else:
+                assert gap(a, b) <= 0.0625
+
+
 def test_engine_prefill_then_decode_matches_the_oracle_chain(engine, oracle, qm, dev, tmp_path):
     """A 37-token prompt through qm_talker_prefill, then two decoded tokens: last-row hidden vectors,
     and the caches the prompt leaves behind, against the oracle's chain of the same operators."""

@@ -1,0 +1,145 @@
+"""GPU parity: causal prefill with a key-split workspace (qm_prefill_attention_causal_split).
+
+Long query tiles are shared by up to three blocks whose partial results are combined by the last
+block to finish: another association of the sums than the unsplit kernel's, so the bar is the
+operator's tolerance (max abs error <= 1e-2 on bf16 outputs against the scalar fp32 oracle, ONLINE
+policy), not equality of bits with the unsplit call; K/V page contents stay bit-exact, the result
+may not depend on which block finishes last, and the workspace must come back as it was found.
+"""
+import numpy as np
+import pytest
+
+from qm_testlib import SCALE, PagedPool, max_abs_err, to_dev, to_u16
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+POISON = 0x7F7F7F7F      # what the workspace holds before its init call
+
+
+def _workspace(qm, dev, batch, seq, poison=True):
+    import torch
+    n = qm.prefill_split_workspace_bytes(batch, seq, 8)
+    ws = torch.full((max(n, 256) // 4,), POISON if poison else 0, dtype=torch.int32, device=dev)
+    if n:
+        qm.prefill_split_workspace_init(ws, n)
+    return ws, n
+
+
+def _inputs(oracle, batch, seq, seed):
+    return (oracle.normal_bf16((batch, seq, 16, 128), seed), oracle.normal_bf16((batch, seq, 8, 128), seed + 1),
+            oracle.normal_bf16((batch, seq, 8, 128), seed + 2))
+
+
+@pytest.mark.parametrize("batch,seq", [(1, 577), (2, 640), (1, 1024), (3, 700), (1, 1300), (1, 2048)])
+def test_split_prefill_against_oracle_and_unsplit(oracle, qm, dev, batch, seq):
+    import torch
+    q, k, v = _inputs(oracle, batch, seq, 7000 + seq)
+    pool = PagedPool(oracle, [seq] * batch, seed=7003 + seq, fill=0x7fc0)
+    want = np.zeros_like(q)
+    assert oracle.prefill_attention_causal(q, k, v, want, pool.descriptor(oracle), pool.page_table, pool.max_pages,
+                                           batch, seq, 16, 8, SCALE, 1, 16) == 0
+    qd, kd, vd = to_dev(q, dev), to_dev(k, dev), to_dev(v, dev)
+    ws, n = _workspace(qm, dev, batch, seq)
+    assert n > 0, "the case is meant to split"
+    sd = torch.zeros(1, dtype=torch.int32, device=dev)
+    outs = []
+    for _ in range(3):                       # the second and third call find the workspace as the first left it
+        fresh = PagedPool(oracle, [seq] * batch, seed=7003 + seq, fill=0x7fc0)
+        k_pages, v_pages, cache_d, table_d = fresh.device(qm, dev)
+        out = torch.full((batch, seq, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+        qm.prefill_attention_causal_split(qd, kd, vd, out, cache_d, table_d, fresh.max_pages, batch, seq, 16, 8, ws, n,
+                                          SCALE, sd)
+        torch.cuda.synchronize()
+        assert int(sd.item()) == 0
+        assert np.array_equal(to_u16(k_pages), pool.k) and np.array_equal(to_u16(v_pages), pool.v)
+        outs.append(to_u16(out))
+    assert max_abs_err(oracle, outs[0], want) <= TOL
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])   # whoever finishes last
+    whole = torch.full((batch, seq, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.prefill_attention_causal(qd, kd, vd, whole, None, None, 0, batch, seq, 16, 8, SCALE, sd)
+    torch.cuda.synchronize()
+    assert max_abs_err(oracle, outs[0], to_u16(whole)) <= TOL
+    # rows of query tiles that are not split carry the unsplit kernel's bits (the first 384 rows never split)
+    assert np.array_equal(outs[0][:, :384], to_u16(whole)[:, :384])
+    # tickets and flags are back at zero (the workspace starts with eight integers per split query tile)
+    assert int(ws[: 8 * batch * 8].abs().max().item()) == 0
+
+
+def test_split_prefill_fp32_scores_option(oracle, qm, dev):
+    import torch
+    batch, seq = 1, 1024
+    q, k, v = _inputs(oracle, batch, seq, 7100)
+    qd, kd, vd = to_dev(q, dev), to_dev(k, dev), to_dev(v, dev)
+    ws, n = _workspace(qm, dev, batch, seq)
+    sd = torch.zeros(1, dtype=torch.int32, device=dev)
+    qm.set_option(qm.OPT_PREFILL_SCORE_ROUNDING, 0)
+    try:
+        split = torch.zeros((batch, seq, 16, 128), dtype=torch.int16, device=dev)
+        whole = torch.zeros_like(split)
+        qm.prefill_attention_causal_split(qd, kd, vd, split, None, None, 0, batch, seq, 16, 8, ws, n, SCALE, sd)
+        qm.prefill_attention_causal(qd, kd, vd, whole, None, None, 0, batch, seq, 16, 8, SCALE, sd)
+        torch.cuda.synchronize()
+    finally:
+        qm.set_option(qm.OPT_PREFILL_SCORE_ROUNDING, 1)
+    assert int(sd.item()) == 0
+    assert max_abs_err(oracle, to_u16(split), to_u16(whole)) <= TOL
+    assert not np.array_equal(to_u16(split), np.zeros_like(q))
+
+
+def test_split_workspace_rules(oracle, qm, dev):
+    import torch
+    assert qm.prefill_split_workspace_bytes(4, 1024, 8) == 0        # two blocks per CU already: nothing to gain
+    assert qm.prefill_split_workspace_bytes(1, 384, 8) == 0         # chains too short to pay for the exchange
+    assert qm.prefill_split_workspace_bytes(0, 1024, 8) == 0
+    n = qm.prefill_split_workspace_bytes(1, 1024, 8)
+    assert n > 0 and n % 256 == 0
+    q, k, v = _inputs(oracle, 1, 1024, 7200)
+    qd, kd, vd = to_dev(q, dev), to_dev(k, dev), to_dev(v, dev)
+    sd = torch.zeros(1, dtype=torch.int32, device=dev)
+    ws = torch.zeros(n // 4, dtype=torch.int32, device=dev)
+    out = torch.zeros((1, 1024, 16, 128), dtype=torch.int16, device=dev)
+    with pytest.raises(qm.QmError) as e:                            # too small for the shape
+        qm.prefill_attention_causal_split(qd, kd, vd, out, None, None, 0, 1, 1024, 16, 8, ws, n - 256, SCALE, sd)
+    assert e.value.code == -4
+    with pytest.raises(qm.QmError) as e:                            # bytes without a pointer
+        qm.prefill_attention_causal_split(qd, kd, vd, out, None, None, 0, 1, 1024, 16, 8, None, n, SCALE, sd)
+    assert e.value.code == -5
+    with pytest.raises(qm.QmError) as e:                            # not 256-byte aligned
+        qm.prefill_attention_causal_split(qd, kd, vd, out, None, None, 0, 1, 1024, 16, 8, ws[1:], n, SCALE, sd)
+    assert e.value.code == -2
+    # no workspace, and a shape that does not split: the unsplit call, bit for bit
+    whole = torch.zeros_like(out)
+    qm.prefill_attention_causal(qd, kd, vd, whole, None, None, 0, 1, 1024, 16, 8, SCALE, sd)
+    qm.prefill_attention_causal_split(qd, kd, vd, out, None, None, 0, 1, 1024, 16, 8, None, 0, SCALE, sd)
+    torch.cuda.synchronize()
+    assert torch.equal(out, whole)
+    q4, k4, v4 = (to_dev(x, dev) for x in _inputs(oracle, 4, 320, 7300))
+    out4 = torch.zeros((4, 320, 16, 128), dtype=torch.int16, device=dev)
+    whole4 = torch.zeros_like(out4)
+    qm.prefill_attention_causal(q4, k4, v4, whole4, None, None, 0, 4, 320, 16, 8, SCALE, sd)
+    qm.prefill_attention_causal_split(q4, k4, v4, out4, None, None, 0, 4, 320, 16, 8, ws, n, SCALE, sd)
+    torch.cuda.synchronize()
+    assert torch.equal(out4, whole4)
+    assert int(sd.item()) == 0
+
+
+def test_split_prefill_other_kernel_choices_ignore_the_workspace(oracle, qm, dev):
+    """Only the interleaved kernel splits; with another kernel chosen the workspace is left alone."""
+    import torch
+    q, k, v = _inputs(oracle, 1, 1024, 7400)
+    qd, kd, vd = to_dev(q, dev), to_dev(k, dev), to_dev(v, dev)
+    ws, n = _workspace(qm, dev, 1, 1024, poison=False)
+    sd = torch.zeros(1, dtype=torch.int32, device=dev)
+    outs = {}
+    try:
+        for choice in (1, 2, 4):
+            qm.set_option(qm.OPT_PREFILL_KERNEL, choice)
+            out = torch.zeros((1, 1024, 16, 128), dtype=torch.int16, device=dev)
+            qm.prefill_attention_causal_split(qd, kd, vd, out, None, None, 0, 1, 1024, 16, 8, ws, n, SCALE, sd)
+            torch.cuda.synchronize()
+            outs[choice] = out
+    finally:
+        qm.set_option(qm.OPT_PREFILL_KERNEL, 0)
+    assert torch.equal(outs[1], outs[2]) and torch.equal(outs[1], outs[4])
+    assert int(ws.abs().max().item()) == 0 and int(sd.item()) == 0
