@@ -116,6 +116,13 @@ def test_workspace_size_is_monotone_and_pure(qm):
         assert n == lib.qm_decode_workspace_bytes(1, 16, 8, L)
         assert n >= prev
         prev = n
+    # a workspace sized for the longest context serves every shorter one, whatever block length the plan picks
+    for streams in (1, 3, 64, 1000):
+        prev = 0
+        for L in range(1, 70000, 29):
+            n = lib.qm_decode_workspace_bytes(streams, 16, 8, L)
+            assert n >= prev, (streams, L)
+            prev = n
     assert lib.qm_decode_workspace_bytes(64, 16, 8, 4096) >= 64 * 8 * 2 * (2 * 128 + 4) * 4
     assert lib.qm_decode_workspace_bytes(0, 16, 8, 10) == 0
     assert lib.qm_decode_workspace_bytes(1, 16, 5, 10) == 0
