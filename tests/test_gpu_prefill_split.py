@@ -143,3 +143,34 @@ def test_split_prefill_other_kernel_choices_ignore_the_workspace(oracle, qm, dev
         qm.set_option(qm.OPT_PREFILL_KERNEL, 0)
     assert torch.equal(outs[1], outs[2]) and torch.equal(outs[1], outs[4])
     assert int(ws.abs().max().item()) == 0 and int(sd.item()) == 0
+
+
+def test_split_prefill_over_flat_layer_cache_in_place(oracle, qm, dev):
+    """K/V read in place from the flat [kv_head][max_cache][128] cache (strided rows), 700 tokens: the parts of a
+    split query tile start at their own key tiles of the strided layout; against the unsplit call and the oracle."""
+    import torch
+    seq, max_cache = 700, 733
+    q = oracle.normal_bf16((seq, 16, 128), 7501)
+    k = oracle.normal_bf16((seq, 8, 128), 7502)
+    v = oracle.normal_bf16((seq, 8, 128), 7503)
+    kc = np.full((8, max_cache, 128), 0x7fc0, dtype=np.uint16)     # NaN beyond the sequence
+    vc = np.full((8, max_cache, 128), 0x7fc0, dtype=np.uint16)
+    assert oracle.scatter_kv(k, v, oracle.flat_cache(kc, vc, 8, max_cache), None, 1, seq, 0) == 0
+    want = np.zeros_like(q)
+    assert oracle.attention(q, oracle.flat_cache(kc, vc, 8, max_cache), None, 1, want, seq, 0, 16, -1, SCALE, 1, 16) == 0
+    kd, vd = to_dev(kc, dev), to_dev(vc, dev)
+    ws, n = _workspace(qm, dev, 1, seq)
+    assert n > 0
+    sd = torch.zeros(1, dtype=torch.int32, device=dev)
+    split = torch.zeros((seq, 16, 128), dtype=torch.int16, device=dev)
+    whole = torch.zeros_like(split)
+    strides = (128, max_cache * 128, 0)
+    qm.prefill_attention_causal_split(to_dev(q, dev), kd, vd, split, None, None, 0, 1, seq, 16, 8, ws, n, SCALE, sd, 0,
+                                      strides)
+    qm.prefill_attention_causal(to_dev(q, dev), kd, vd, whole, None, None, 0, 1, seq, 16, 8, SCALE, sd, 0, strides)
+    torch.cuda.synchronize()
+    assert int(sd.item()) == 0
+    assert np.array_equal(to_u16(kd), kc)
+    assert max_abs_err(oracle, to_u16(split), want) <= TOL
+    assert max_abs_err(oracle, to_u16(split), to_u16(whole)) <= TOL
+    assert not np.array_equal(to_u16(split)[448:], np.zeros_like(q)[448:])
