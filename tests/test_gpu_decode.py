@@ -275,3 +275,37 @@ def test_fused_decode_step_argument_errors(qm, dev):
     assert L.qm_decode_step_fused(*args(3, None)) == -1
     assert L.qm_decode_step_fused(*args(31)) == 0
     torch.cuda.synchronize()
+
+
+def _double_bf16(bits):
+    """Every finite, normal bf16 value times two: one more in the exponent field, exact."""
+    bits = bits.copy()
+    normal = ((bits & 0x7F80) != 0) & ((bits & 0x7F80) < 0x7F00)
+    bits[normal] += 0x0080
+    return bits
+
+
+def test_decode_is_exactly_linear_in_v_at_config3_size(oracle, qm, dev):
+    """A property that does not depend on the size, at the benchmark's full shape (64 streams of 256..4096
+    tokens, 2.4 M context tokens): doubling every V doubles every output bit for bit — the P.V sums, the
+    rescaling by running maxima, the merge of the row-streams and of the splits and the final rounding all
+    commute with a power of two — while the scores, which do not see V, stay what they were."""
+    import torch
+    lens = np.asarray(oracle.uniform_int(64, 2024, 256, 4096), dtype=np.int32)
+    n, max_len = len(lens), int(lens.max())
+    pool = PagedPool(oracle, lens, seed=78)
+    q = to_dev(oracle.normal_bf16((n, 16, 128), 88), dev)
+    ws, nbytes = _workspace(qm, dev, n, 16, 8, max_len)
+    table_d, lens_d = to_dev(pool.page_table, dev), to_dev(lens, dev)
+    outs = []
+    for v in (pool.v, _double_bf16(pool.v)):
+        kd, vd = to_dev(pool.k, dev), to_dev(v, dev)
+        out = torch.full((n, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+        sd = torch.zeros(1, dtype=torch.int32, device=dev)
+        qm.decode_attention_ragged(q, qm.paged_cache(kd, vd, pool.n_pages), table_d, pool.max_pages, lens_d, n, max_len,
+                                   out, 16, SCALE, ws, nbytes, sd)
+        torch.cuda.synchronize()
+        assert int(sd.item()) == 0
+        outs.append(to_u16(out))
+    assert np.count_nonzero(outs[0] & 0x7F80) > outs[0].size * 0.99      # normal numbers, nearly all
+    assert np.array_equal(outs[1], _double_bf16(outs[0]))

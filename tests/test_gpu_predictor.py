@@ -106,3 +106,34 @@ def test_predictor_staged_attention_argument_errors(qm, dev):
     assert L.qm_predictor_attention_staged(z.data_ptr(), c.data_ptr(), c.data_ptr(), z.data_ptr(), 2, 17, 1, None) == -5
     assert L.qm_predictor_attention_staged(z.data_ptr(), c.data_ptr(), c.data_ptr(), z.data_ptr(), 0, 2, 1, None) == -5
     assert L.qm_predictor_attention_staged(None, c.data_ptr(), c.data_ptr(), z.data_ptr(), 2, 2, 1, None) == -1
+
+
+def test_predictor_loop_is_exactly_linear_in_v_at_config5_size(oracle, qm, dev):
+    """A property that does not depend on the size, at the benchmark's full shape (256 frames x 5 layers x 16
+    steps): doubling every V (one more in the bf16 exponent, exact) doubles every output bit for bit — the
+    probabilities do not see V, and the leaves fmaf(P, V, +0), the tree sums and the final rounding commute with
+    a power of two."""
+    import torch
+    units, layers, rows = 256 * 5, 5, 16
+    q = to_dev(oracle.normal_bf16((units, rows, 16, 128), 91), dev)
+    k = to_dev(oracle.normal_bf16((units, rows, 8, 128), 92), dev)
+    v = oracle.normal_bf16((units, rows, 8, 128), 93)
+    gq = to_dev(oracle.normal_bf16((layers, 128), 94, 1.0, 0.1), dev)
+    gk = to_dev(oracle.normal_bf16((layers, 128), 95, 1.0, 0.1), dev)
+    cos, sin = oracle.rope_table(rows, 0)
+    cos, sin = to_dev(cos, dev), to_dev(sin, dev)
+
+    def doubled(bits):
+        bits = bits.copy()
+        normal = ((bits & 0x7F80) != 0) & ((bits & 0x7F80) < 0x7F00)
+        bits[normal] += 0x0080
+        return bits
+
+    outs = []
+    for vv in (v, doubled(v)):
+        out = torch.full((units, rows, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+        qm.predictor_attention_loop(q, k, to_dev(vv, dev), gq, gk, cos, sin, out, None, None, units, layers, rows, 1)
+        torch.cuda.synchronize()
+        outs.append(to_u16(out))
+    assert np.count_nonzero(outs[0] & 0x7F80) > outs[0].size * 0.99
+    assert np.array_equal(outs[1], doubled(outs[0]))

@@ -174,3 +174,33 @@ def test_split_prefill_over_flat_layer_cache_in_place(oracle, qm, dev):
     assert max_abs_err(oracle, to_u16(split), want) <= TOL
     assert max_abs_err(oracle, to_u16(split), to_u16(whole)) <= TOL
     assert not np.array_equal(to_u16(split)[448:], np.zeros_like(q)[448:])
+
+
+def _double_bf16(bits):
+    """Every finite, normal bf16 value times two: one more in the exponent field, exact."""
+    bits = bits.copy()
+    normal = ((bits & 0x7F80) != 0) & ((bits & 0x7F80) < 0x7F00)
+    bits[normal] += 0x0080
+    return bits
+
+
+@pytest.mark.parametrize("batch,seq,split", [(4, 1024, False), (1, 1024, True), (1, 2048, True)])
+def test_prefill_is_exactly_linear_in_v(oracle, qm, dev, batch, seq, split):
+    """A property that does not depend on the size, at the benchmark's shapes: doubling every V doubles every
+    output bit for bit (P.V on the matrix cores, the rescaling by running maxima, the combination of the parts of
+    a split query tile and the final rounding all commute with a power of two)."""
+    import torch
+    q, k, v = _inputs(oracle, batch, seq, 7600 + seq)
+    qd, kd = to_dev(q, dev), to_dev(k, dev)
+    ws, n = _workspace(qm, dev, batch, seq) if split else (None, 0)
+    assert (n > 0) == split
+    sd = torch.zeros(1, dtype=torch.int32, device=dev)
+    outs = []
+    for vv in (v, _double_bf16(v)):
+        out = torch.zeros((batch, seq, 16, 128), dtype=torch.int16, device=dev)
+        qm.prefill_attention_causal_split(qd, kd, to_dev(vv, dev), out, None, None, 0, batch, seq, 16, 8, ws, n, SCALE, sd)
+        torch.cuda.synchronize()
+        outs.append(to_u16(out))
+    assert int(sd.item()) == 0
+    assert np.count_nonzero(outs[0] & 0x7F80) > outs[0].size * 0.99
+    assert np.array_equal(outs[1], _double_bf16(outs[0]))
