@@ -309,3 +309,24 @@ def test_decode_is_exactly_linear_in_v_at_config3_size(oracle, qm, dev):
         outs.append(to_u16(out))
     assert np.count_nonzero(outs[0] & 0x7F80) > outs[0].size * 0.99      # normal numbers, nearly all
     assert np.array_equal(outs[1], _double_bf16(outs[0]))
+
+
+def test_decode_streams_are_independent_at_config3_size(oracle, qm, dev):
+    """Reversing the order of the 64 streams (queries, lengths, page-table rows) reverses the outputs bit for bit:
+    which block of the grid, which XCD and which split index a stream's tiles land on is no part of the result."""
+    import torch
+    lens = np.asarray(oracle.uniform_int(64, 2025, 256, 4096), dtype=np.int32)
+    n, max_len = len(lens), int(lens.max())
+    pool = PagedPool(oracle, lens, seed=79)
+    q = oracle.normal_bf16((n, 16, 128), 89)
+    ws, nbytes = _workspace(qm, dev, n, 16, 8, max_len)
+    kd, vd = to_dev(pool.k, dev), to_dev(pool.v, dev)
+    cache_d = qm.paged_cache(kd, vd, pool.n_pages)
+    outs = []
+    for order in (np.arange(n), np.arange(n)[::-1].copy()):
+        out = torch.full((n, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+        qm.decode_attention_ragged(to_dev(q[order], dev), cache_d, to_dev(pool.page_table[order], dev), pool.max_pages,
+                                   to_dev(lens[order], dev), n, max_len, out, 16, SCALE, ws, nbytes)
+        torch.cuda.synchronize()
+        outs.append(to_u16(out))
+    assert np.array_equal(outs[1], outs[0][::-1])

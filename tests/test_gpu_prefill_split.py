@@ -204,3 +204,22 @@ def test_prefill_is_exactly_linear_in_v(oracle, qm, dev, batch, seq, split):
     assert int(sd.item()) == 0
     assert np.count_nonzero(outs[0] & 0x7F80) > outs[0].size * 0.99
     assert np.array_equal(outs[1], _double_bf16(outs[0]))
+
+
+def test_prefill_batch_entries_are_independent(oracle, qm, dev):
+    """Every entry of the 4 x 1024 benchmark batch, run alone (another grid, another block order), gives the bits
+    it has inside the batch."""
+    import torch
+    q, k, v = _inputs(oracle, 4, 1024, 7700)
+    sd = torch.zeros(1, dtype=torch.int32, device=dev)
+    whole = torch.zeros((4, 1024, 16, 128), dtype=torch.int16, device=dev)
+    qm.prefill_attention_causal(to_dev(q, dev), to_dev(k, dev), to_dev(v, dev), whole, None, None, 0, 4, 1024, 16, 8,
+                                SCALE, sd)
+    torch.cuda.synchronize()
+    for b in range(4):
+        alone = torch.zeros((1, 1024, 16, 128), dtype=torch.int16, device=dev)
+        qm.prefill_attention_causal(to_dev(q[b:b + 1], dev), to_dev(k[b:b + 1], dev), to_dev(v[b:b + 1], dev), alone, None,
+                                    None, 0, 1, 1024, 16, 8, SCALE, sd)
+        torch.cuda.synchronize()
+        assert torch.equal(alone[0], whole[b]), b
+    assert int(sd.item()) == 0
