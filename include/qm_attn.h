@@ -324,6 +324,28 @@ int32_t qm_predictor_attention_staged(
     uint16_t* output, int32_t rows, int32_t key_length, int32_t causal_prefill,
     void* hip_stream);
 
+/*
+ * The three layout operators in front of the staged attention at the predictor's step 0 (call site
+ * R17:13663-13699), each with the reference wrapper's per-tensor argument list:
+ * qm_predictor_transpose replaces PersistentPredictor::transpose (R17:13222-13236, kernel
+ *   transpose_bshd_to_bhsd_kernel :8366-8400): input [rows][heads][128] -> output [heads][rows][128].
+ * qm_predictor_rope_bhsd replaces PersistentPredictor::rope (R17:13238-13254, kernel apply_rope_kernel
+ *   :8403-8488): input, output [heads][rows][128] (BHSD); head h, row s is rotated with cos/sin row s
+ *   ([rows][128]): bf16(bf16(x*cos) + bf16(rotate_half(x)*sin)), no norm.
+ * qm_predictor_update_cache replaces PersistentPredictor::update_cache (R17:13256-13270, kernel
+ *   update_cache_kernel :8491-8529): source [8][rows][128] (BHSD) is copied to
+ *   cache[(h*16 + start + s)*128 ..] of ONE [8][16][128] cache (the reference calls it once for the
+ *   key and once for the value cache).  start + rows > 16 is QM_ERR_SLOT_RANGE (the reference has no
+ *   guard).  Tensors 16-byte aligned for transpose and update_cache (QM_ERR_GEOMETRY).
+ */
+int32_t qm_predictor_transpose(
+    const uint16_t* input, uint16_t* output, int32_t rows, int32_t heads, void* hip_stream);
+int32_t qm_predictor_rope_bhsd(
+    const uint16_t* input, const uint16_t* cos_rows, const uint16_t* sin_rows, uint16_t* output,
+    int32_t rows, int32_t heads, void* hip_stream);
+int32_t qm_predictor_update_cache(
+    const uint16_t* source, uint16_t* cache, int32_t rows, int32_t start, void* hip_stream);
+
 /* --- (5) M = 1 weight-streaming linears around the path ----------------------------------- */
 /*
  * qm_linear_m1 replaces launch_linear_m1 / talker_linear_fused_kernel (R17:17473-17511,

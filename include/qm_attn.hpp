@@ -183,21 +183,25 @@ inline void predictor_attention(
           "Predictor attention launch");
 }
 
-// PersistentPredictor::rope (R17:13238-13254): RoPE of rows x heads head vectors, no norm.
+// PersistentPredictor::transpose (R17:13222-13236): [rows][heads][128] -> [heads][rows][128].
+inline void predictor_transpose(const std::uint16_t* input, std::uint16_t* output, int rows, int heads,
+                                void* stream) {
+    check(qm_predictor_transpose(input, output, rows, heads, stream), "Predictor transpose launch");
+}
+
+// PersistentPredictor::rope (R17:13238-13254): RoPE of a BHSD tensor [heads][rows][128], head h row s
+// rotated with table row s; no norm.
 inline void predictor_rope(
     const std::uint16_t* input, const std::uint16_t* cosine, const std::uint16_t* sine, std::uint16_t* output,
     int rows, int heads, void* stream) {
-    check(qm_norm_rope_rows(input, nullptr, cosine, sine, output, rows, heads, 0.0f, stream), "Predictor rope launch");
+    check(qm_predictor_rope_bhsd(input, cosine, sine, output, rows, heads, stream), "Predictor rope launch");
 }
 
-// PersistentPredictor::update_cache (R17:13256-13270) for the key and the value cache of a layer
-// ([8][16][128] each): rows of [rows][8][128] go to positions start..start+rows-1.
+// PersistentPredictor::update_cache (R17:13256-13270): BHSD source [8][rows][128] into one
+// [8][16][128] cache at positions start..start+rows-1; called once per cache like the reference.
 inline void predictor_update_cache(
-    const std::uint16_t* key_source, const std::uint16_t* value_source,
-    std::uint16_t* key_cache, std::uint16_t* value_cache, int rows, int start, void* stream) {
-    const qm_kv_cache cache = flat_cache(key_cache, value_cache, 8, 128, 16);
-    check(qm_scatter_kv(key_source, value_source, &cache, nullptr, 1, rows, start, stream),
-          "Predictor update_cache launch");
+    const std::uint16_t* source, std::uint16_t* cache, int rows, int start, void* stream) {
+    check(qm_predictor_update_cache(source, cache, rows, start, stream), "Predictor update_cache launch");
 }
 
 // launch_qk_norm_rope_cache_m1 + launch_attention of one decode step (R17:17181-17195) in one launch.

@@ -185,6 +185,18 @@ def predictor_attention_staged(query_bhsd, key_cache, value_cache, out_bshd, row
                                                 C.c_int32(key_length), C.c_int32(int(causal)))
 
 
+def predictor_transpose(x, out, rows, heads):
+    return lib().qmo_predictor_transpose(_p(x), _p(out), C.c_int32(rows), C.c_int32(heads))
+
+
+def predictor_rope_bhsd(x, cos, sin, out, rows, heads):
+    return lib().qmo_predictor_rope_bhsd(_p(x), _p(cos), _p(sin), _p(out), C.c_int32(rows), C.c_int32(heads))
+
+
+def predictor_update_cache(source, cache, rows, start):
+    return lib().qmo_predictor_update_cache(_p(source), _p(cache), C.c_int32(rows), C.c_int32(start))
+
+
 def predictor_attention_loop(q, k, v, gq, gk, cos, sin, out, k_cache_out, v_cache_out, units,
                              n_layers, rows, first_rows=1, eps=1e-6, threads=8):
     return lib().qmo_predictor_attention_loop(

@@ -636,6 +636,65 @@ int32_t qmo_predictor_attention_staged(const uint16_t* query_bhsd, const uint16_
     return QM_OK;
 }
 
+// The three layout kernels in front of the staged attention of step 0 (call site R17:13663-13699).
+// transpose_bshd_to_bhsd_kernel R17:8366-8400: [rows][heads][128] -> [heads][rows][128].
+int32_t qmo_predictor_transpose(const uint16_t* input, uint16_t* output, int32_t rows, int32_t heads) {
+    if (!input || !output) return QM_ERR_NULL;
+    if (rows < 0 || heads <= 0) return QM_ERR_ARGUMENT;
+    const int64_t count = static_cast<int64_t>(rows) * heads * kDim;
+    for (int64_t index = 0; index < count; ++index) {
+        const int d = static_cast<int>(index % kDim);
+        const int64_t t = index / kDim;
+        const int64_t head = t % heads;
+        const int64_t sequence = t / heads;
+        output[(head * rows + sequence) * kDim + d] = input[index];
+    }
+    return QM_OK;
+}
+
+// apply_rope_kernel R17:8403-8488 on a BHSD tensor [heads][rows][128]: element index ->
+// sequence = (index / 128) % rows, head = (index / 128) / rows; cos/sin row = sequence;
+// bf16(bf16(x * cos) + bf16(+-x[d +- 64] * sin)), the sign negative for d < 64.
+int32_t qmo_predictor_rope_bhsd(const uint16_t* input, const uint16_t* cosine, const uint16_t* sine,
+                                uint16_t* output, int32_t rows, int32_t heads) {
+    if (!input || !cosine || !sine || !output) return QM_ERR_NULL;
+    if (rows < 0 || heads <= 0) return QM_ERR_ARGUMENT;
+    const int64_t count = static_cast<int64_t>(rows) * heads * kDim;
+    for (int64_t index = 0; index < count; ++index) {
+        const int d = static_cast<int>(index % kDim);
+        const int64_t t = index / kDim;
+        const int64_t sequence = t % rows;
+        const int64_t head = t / rows;
+        const int rd = d < kDim / 2 ? d + kDim / 2 : d - kDim / 2;
+        const float sign = d < kDim / 2 ? -1.0f : 1.0f;
+        const int64_t base = (head * rows + sequence) * kDim;
+        const float value = bf2f(input[base + d]);
+        const float rotated = sign * bf2f(input[base + rd]);
+        const uint16_t first = f2bf(value * bf2f(cosine[sequence * kDim + d]));
+        const uint16_t second = f2bf(rotated * bf2f(sine[sequence * kDim + d]));
+        output[index] = f2bf(bf2f(first) + bf2f(second));
+    }
+    return QM_OK;
+}
+
+// update_cache_kernel R17:8491-8529: source [8][rows][128] (BHSD) -> cache [8][16][128] at
+// positions start .. start + rows - 1 of every head.  The reference has no range guard; here a
+// run past the 16 positions is an error and nothing is written.
+int32_t qmo_predictor_update_cache(const uint16_t* source, uint16_t* cache, int32_t rows, int32_t start) {
+    if (!source || !cache) return QM_ERR_NULL;
+    if (rows < 0 || start < 0) return QM_ERR_ARGUMENT;
+    if (start + rows > 16) return QM_ERR_SLOT_RANGE;
+    const int64_t count = static_cast<int64_t>(8) * rows * kDim;
+    for (int64_t index = 0; index < count; ++index) {
+        const int d = static_cast<int>(index % kDim);
+        const int64_t t = index / kDim;
+        const int64_t sequence = t % rows;
+        const int64_t head = t / rows;
+        cache[(head * 16 + start + sequence) * kDim + d] = source[index];
+    }
+    return QM_OK;
+}
+
 // The whole step loop of one (frame, layer) unit after another, schedule of
 // PersistentPredictor::capture_step R17:13592-13596: row r is appended at position r and
 // attends keys 0..r.

@@ -67,6 +67,9 @@ _SIGNATURES = {
                                                  _F32, C.c_int64, C.c_int64, C.c_int64, _PTR, C.c_int64, _PTR, _PTR]),
     "qm_predictor_attention_loop": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _I32, _F32, _PTR]),
     "qm_predictor_attention_staged": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _PTR]),
+    "qm_predictor_transpose": (_I32, [_PTR, _PTR, _I32, _I32, _PTR]),
+    "qm_predictor_rope_bhsd": (_I32, [_PTR] * 4 + [_I32, _I32, _PTR]),
+    "qm_predictor_update_cache": (_I32, [_PTR, _PTR, _I32, _I32, _PTR]),
     "qm_linear_m1": (_I32, [_PTR] * 5 + [_I32, _I32, _PTR]),
     "qm_qkv_m1": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _PTR]),
     "qm_gate_up_swiglu_m1": (_I32, [_PTR] * 4 + [_I32, _I32, _PTR]),
@@ -353,3 +356,17 @@ def gather_embedding(table, table_rows, codes, group, dimension, selected, next_
 def predictor_attention_staged(query_bhsd, key_cache, value_cache, out, rows, key_length, causal, stream=0):
     _check(lib().qm_predictor_attention_staged(_addr(query_bhsd), _addr(key_cache), _addr(value_cache), _addr(out),
                                                rows, key_length, int(causal), stream), "qm_predictor_attention_staged")
+
+
+def predictor_transpose(x, out, rows, heads, stream=0):
+    _check(lib().qm_predictor_transpose(_addr(x), _addr(out), rows, heads, stream), "qm_predictor_transpose")
+
+
+def predictor_rope_bhsd(x, cos, sin, out, rows, heads, stream=0):
+    _check(lib().qm_predictor_rope_bhsd(_addr(x), _addr(cos), _addr(sin), _addr(out), rows, heads, stream),
+           "qm_predictor_rope_bhsd")
+
+
+def predictor_update_cache(source, cache, rows, start, stream=0):
+    _check(lib().qm_predictor_update_cache(_addr(source), _addr(cache), rows, start, stream),
+           "qm_predictor_update_cache")

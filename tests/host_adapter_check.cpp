@@ -63,6 +63,12 @@ int main() {
         qm_attn::predictor_attention_loop(fake, fake, fake, fake, fake, fake, fake, fake, nullptr, nullptr, 1, 5, 17, 1,
                                           1e-6f, nullptr);
     });
+    expect_throw("predictor update_cache overflow", "capacity", [&] {
+        qm_attn::predictor_update_cache(fake, fake, 2, 15, nullptr);
+    });
+    expect_throw("predictor rope null", "pointer is NULL", [&] {
+        qm_attn::predictor_rope(fake, nullptr, fake, fake, 2, 16, nullptr);
+    });
     if (qm_attn::attention_workspace_bytes(16, 8, 8206) == 0) {
         std::printf("FAIL workspace size is zero for a long context\n");
         ++failures;

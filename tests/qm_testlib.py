@@ -66,3 +66,29 @@ class PagedPool:
     def device(self, qm, dev):
         kd, vd = to_dev(self.k, dev), to_dev(self.v, dev)
         return kd, vd, qm.paged_cache(kd, vd, self.n_pages, self.kv_heads, self.page_size), to_dev(self.page_table, dev)
+
+
+def step0_chain(oracle, ops, q, k, v, gq, gk, cos, sin, rows):
+    """The reference's step-0 attention sequence (R17:13650-13705) on numpy arrays: per-head RMSNorm
+    (oracle) -> transpose -> rope -> update_cache -> staged causal attention, the last four through `ops`
+    (the oracle binding, or an object with the same five functions that runs them on the device)."""
+    ones_c, zeros_s = oracle.rope_table(rows, 0)
+    ones_c[:], zeros_s[:] = 0x3F80, 0
+    qn, kn = np.zeros_like(q), np.zeros_like(k)
+    # per-head RMSNorm alone = norm + RoPE with cos 1, sin 0 (x*1 and +0 are exact)
+    assert oracle.norm_rope_rows(q, gq.copy(), ones_c, zeros_s, qn, rows, 16) == 0
+    assert oracle.norm_rope_rows(k, gk.copy(), ones_c, zeros_s, kn, rows, 8) == 0
+    q_bhsd, k_bhsd, v_bhsd = (np.zeros((16, rows, 128), np.uint16), np.zeros((8, rows, 128), np.uint16),
+                              np.zeros((8, rows, 128), np.uint16))
+    assert ops.predictor_transpose(qn, q_bhsd, rows, 16) == 0
+    assert ops.predictor_transpose(kn, k_bhsd, rows, 8) == 0
+    assert ops.predictor_transpose(v, v_bhsd, rows, 8) == 0
+    q_rot, k_rot = np.zeros_like(q_bhsd), np.zeros_like(k_bhsd)
+    assert ops.predictor_rope_bhsd(q_bhsd, cos, sin, q_rot, rows, 16) == 0
+    assert ops.predictor_rope_bhsd(k_bhsd, cos, sin, k_rot, rows, 8) == 0
+    kc, vc = np.zeros((8, 16, 128), np.uint16), np.zeros((8, 16, 128), np.uint16)
+    assert ops.predictor_update_cache(k_rot, kc, rows, 0) == 0
+    assert ops.predictor_update_cache(v_bhsd, vc, rows, 0) == 0
+    out = np.zeros((rows, 16, 128), np.uint16)
+    assert ops.predictor_attention_staged(q_rot, kc, vc, out, rows, rows, True) == 0
+    return out, kc, vc

@@ -137,3 +137,99 @@ def test_predictor_loop_is_exactly_linear_in_v_at_config5_size(oracle, qm, dev):
         outs.append(to_u16(out))
     assert np.count_nonzero(outs[0] & 0x7F80) > outs[0].size * 0.99
     assert np.array_equal(outs[1], doubled(outs[0]))
+
+
+class _DeviceStep0Ops:
+    """The five step-0 operators of the product library behind the oracle binding's numpy signatures."""
+
+    def __init__(self, qm, dev):
+        self.qm, self.dev = qm, dev
+
+    def _call(self, fn, ins, out, *args):
+        import torch
+        d_ins = [to_dev(a, self.dev) for a in ins]
+        d_out = to_dev(out, self.dev)
+        fn(*d_ins, d_out, *args)
+        torch.cuda.synchronize()
+        out[...] = to_u16(d_out).reshape(out.shape)
+        return 0
+
+    def predictor_transpose(self, x, out, rows, heads):
+        return self._call(self.qm.predictor_transpose, [x], out, rows, heads)
+
+    def predictor_rope_bhsd(self, x, cos, sin, out, rows, heads):
+        return self._call(self.qm.predictor_rope_bhsd, [x, cos, sin], out, rows, heads)
+
+    def predictor_update_cache(self, source, cache, rows, start):
+        return self._call(self.qm.predictor_update_cache, [source], cache, rows, start)
+
+    def predictor_attention_staged(self, q, kc, vc, out, rows, key_length, causal):
+        return self._call(self.qm.predictor_attention_staged, [q, kc, vc], out, rows, key_length, causal)
+
+
+@pytest.mark.parametrize("rows,heads", [(2, 16), (2, 8), (1, 16), (16, 8), (5, 3)])
+def test_predictor_transpose_and_rope_bhsd(oracle, qm, dev, rows, heads):
+    """PersistentPredictor::transpose and ::rope (R17:13222-13254) index [head][row][128]: bit-exact."""
+    ops = _DeviceStep0Ops(qm, dev)
+    x = oracle.normal_bf16((rows, heads, 128), 700 + rows * 17 + heads)
+    want_t, got_t = np.zeros((heads, rows, 128), np.uint16), np.full((heads, rows, 128), 0x7fc0, np.uint16)
+    assert oracle.predictor_transpose(x, want_t, rows, heads) == 0
+    ops.predictor_transpose(x, got_t, rows, heads)
+    assert np.array_equal(got_t, want_t)
+    cos, sin = oracle.rope_table(rows, 3)
+    want_r, got_r = np.zeros_like(want_t), np.full_like(want_t, 0x7fc0)
+    assert oracle.predictor_rope_bhsd(want_t, cos, sin, want_r, rows, heads) == 0
+    ops.predictor_rope_bhsd(got_t, cos, sin, got_r, rows, heads)
+    assert np.array_equal(got_r, want_r)
+
+
+@pytest.mark.parametrize("rows,start", [(2, 0), (1, 2), (3, 13), (16, 0), (1, 15)])
+def test_predictor_update_cache(oracle, qm, dev, rows, start):
+    """PersistentPredictor::update_cache (R17:13256-13270): exactly 8*rows*128 elements change, at
+    (h*16 + start + s)*128 — values and slot index bit-exact against the oracle."""
+    ops = _DeviceStep0Ops(qm, dev)
+    src = oracle.normal_bf16((8, rows, 128), 900 + rows + start)
+    src[src == 0xABCD] = 0
+    want, got = np.full((8, 16, 128), 0xABCD, np.uint16), np.full((8, 16, 128), 0xABCD, np.uint16)
+    assert oracle.predictor_update_cache(src, want, rows, start) == 0
+    ops.predictor_update_cache(src, got, rows, start)
+    assert np.array_equal(got, want)
+    assert np.count_nonzero(got != 0xABCD) == 8 * rows * 128
+
+
+def test_predictor_step0_chain_equals_loop_rows(oracle, qm, dev):
+    """transpose -> rope -> update_cache -> staged attention for rows = 2 (the reference's only use,
+    R17:13663-13705) equals the one-launch loop with first_rows = 2 row for row, and its caches."""
+    import torch
+    from qm_testlib import step0_chain, ulp_distance
+    rows = 2
+    q = oracle.normal_bf16((1, rows, 16, 128), 31)
+    k = oracle.normal_bf16((1, rows, 8, 128), 32)
+    v = oracle.normal_bf16((1, rows, 8, 128), 33)
+    gq = oracle.normal_bf16((1, 128), 34, 1.0, 0.1)
+    gk = oracle.normal_bf16((1, 128), 35, 1.0, 0.1)
+    cos, sin = oracle.rope_table(rows, 0)
+    out = torch.full((1, rows, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    kd = torch.full((1, 8, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    vd = torch.full((1, 8, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.predictor_attention_loop(to_dev(q, dev), to_dev(k, dev), to_dev(v, dev), to_dev(gq, dev), to_dev(gk, dev),
+                                to_dev(cos, dev), to_dev(sin, dev), out, kd, vd, 1, 1, rows, 2)
+    torch.cuda.synchronize()
+    got, kc, vc = step0_chain(oracle, _DeviceStep0Ops(qm, dev), q[0], k[0], v[0], gq[0], gk[0], cos, sin, rows)
+    assert np.array_equal(kc, to_u16(kd)[0]) and np.array_equal(vc, to_u16(vd)[0])
+    assert np.array_equal(got, to_u16(out)[0])            # same kernel arithmetic on both routes
+    want, _, _ = step0_chain(oracle, oracle, q[0], k[0], v[0], gq[0], gk[0], cos, sin, rows)
+    assert ulp_distance(got, want).max() <= 1              # device expf
+
+
+def test_predictor_step0_operator_argument_errors(qm, dev):
+    import torch
+    z = torch.zeros((16, 16, 128), dtype=torch.int16, device=dev)
+    L = qm.lib()
+    assert L.qm_predictor_update_cache(z.data_ptr(), z.data_ptr(), 2, 15, None) == -3
+    assert L.qm_predictor_update_cache(z.data_ptr(), z.data_ptr(), -1, 0, None) == -5
+    assert L.qm_predictor_update_cache(None, z.data_ptr(), 1, 0, None) == -1
+    assert L.qm_predictor_rope_bhsd(z.data_ptr(), None, z.data_ptr(), z.data_ptr(), 2, 16, None) == -1
+    assert L.qm_predictor_rope_bhsd(z.data_ptr(), z.data_ptr(), z.data_ptr(), z.data_ptr(), 2, 0, None) == -5
+    assert L.qm_predictor_transpose(z.data_ptr(), z.data_ptr(), 2, 16, None) == -5
+    assert L.qm_predictor_transpose(z.data_ptr(), z.data_ptr() + 2, 2, 16, None) == -2

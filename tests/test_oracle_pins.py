@@ -441,6 +441,80 @@ def test_predictor_staged_step0_equals_m1_rows(oracle):
         assert np.array_equal(o, staged[r])
 
 
+def test_predictor_step0_layout_operators(oracle):
+    """transpose / rope / update_cache of the predictor's step 0 index BHSD [head][row][128]
+    (R17:8366-8529).  Pinned without repeating the oracle's index arithmetic: numpy's own transpose,
+    a rotation whose result is known in closed form per (head, row), and a sentinel-filled cache."""
+    rows, heads = 2, 16
+    x = oracle.normal_bf16((rows, heads, 128), 11)
+    t = np.zeros((heads, rows, 128), dtype=np.uint16)
+    assert oracle.predictor_transpose(x, t, rows, heads) == 0
+    assert np.array_equal(t, x.transpose(1, 0, 2))
+    # rope: head h, row s must use table row s.  Input = unit vector e_0 everywhere, so the rotated
+    # vector is cos_s[0] at dim 0 and +sin_s[64] at dim 64 (rotate_half gives d >= 64 the value +x[d-64]),
+    # whatever the head; table rows differ, so a head/row mix-up shows.
+    cos, sin = oracle.rope_table(rows, 0)
+    cos[1], sin[1] = oracle.rope_table(1, 7)[0][0], oracle.rope_table(1, 7)[1][0]   # row 1 := position 7
+    e0 = np.zeros((heads, rows, 128), dtype=np.uint16)
+    e0[:, :, 0] = 0x3F80
+    out = np.zeros_like(e0)
+    assert oracle.predictor_rope_bhsd(e0, cos, sin, out, rows, heads) == 0
+    for h in range(heads):
+        for s_ in range(rows):
+            assert out[h, s_, 0] == cos[s_, 0] and out[h, s_, 64] == sin[s_, 64]
+            assert not (out[h, s_, 1:64] & 0x7FFF).any() and not (out[h, s_, 65:] & 0x7FFF).any()   # +-0
+    assert out[0, 0, 0] == 0x3F80 and out[0, 0, 64] == 0          # position 0: identity
+    assert out[0, 1, 64] != 0                                      # position 7 rotates
+    # the rotation of a BHSD tensor is the row-wise rotation (pinned elsewhere) of its BSHD transpose
+    y = oracle.normal_bf16((rows, heads, 128), 12)
+    y_bhsd = np.ascontiguousarray(y.transpose(1, 0, 2))
+    got = np.zeros_like(y_bhsd)
+    assert oracle.predictor_rope_bhsd(y_bhsd, cos, sin, got, rows, heads) == 0
+    want = np.zeros_like(y)
+    assert oracle.norm_rope_rows(y, None, cos, sin, want, rows, heads) == 0
+    assert np.array_equal(got, want.transpose(1, 0, 2))
+    # e_64 picks the other sign: out[0] = -sin_s[0], out[64] = cos_s[64]
+    e64 = np.zeros((heads, rows, 128), dtype=np.uint16)
+    e64[:, :, 64] = 0x3F80
+    assert oracle.predictor_rope_bhsd(e64, cos, sin, out, rows, heads) == 0
+    assert out[3, 1, 0] == (sin[1, 0] ^ 0x8000) and out[3, 1, 64] == cos[1, 64]
+    # update_cache: exactly 8 * rows * 128 elements change, head h row s lands at (h*16 + start + s)*128
+    for rows_u, start in ((2, 0), (1, 2), (3, 13), (16, 0)):
+        src = oracle.normal_bf16((8, rows_u, 128), 13 + start)
+        src[src == 0xABCD] = 0
+        cache = np.full((8, 16, 128), 0xABCD, dtype=np.uint16)
+        assert oracle.predictor_update_cache(src, cache, rows_u, start) == 0
+        assert np.count_nonzero(cache != 0xABCD) == 8 * rows_u * 128
+        flat = cache.reshape(-1)
+        for h in (0, 5, 7):
+            for s_ in range(rows_u):
+                at = (h * 16 + start + s_) * 128
+                assert np.array_equal(flat[at:at + 128], src[h, s_])
+    cache = np.full((8, 16, 128), 0xABCD, dtype=np.uint16)
+    assert oracle.predictor_update_cache(src, cache, 2, 15) == -3
+    assert (cache == 0xABCD).all()
+
+
+def test_predictor_step0_chain_equals_loop(oracle):
+    """The reference's step-0 sequence (R17:13663-13705) — transpose, rope, update_cache, staged causal
+    attention — on normed rows gives the loop operator's rows 0 and 1 (first_rows = 2) bit for bit."""
+    rows = 2
+    q = oracle.normal_bf16((1, rows, 16, 128), 21)
+    k = oracle.normal_bf16((1, rows, 8, 128), 22)
+    v = oracle.normal_bf16((1, rows, 8, 128), 23)
+    gq = oracle.normal_bf16((1, 128), 24, 1.0, 0.1)
+    gk = oracle.normal_bf16((1, 128), 25, 1.0, 0.1)
+    cos, sin = oracle.rope_table(rows, 0)
+    want = np.zeros_like(q)
+    kc_want = np.zeros((1, 8, 16, 128), dtype=np.uint16)
+    vc_want = np.zeros_like(kc_want)
+    assert oracle.predictor_attention_loop(q, k, v, gq, gk, cos, sin, want, kc_want, vc_want, 1, 1, rows, 2) == 0
+    from qm_testlib import step0_chain
+    got, kc, vc = step0_chain(oracle, oracle, q[0], k[0], v[0], gq[0], gk[0], cos, sin, rows)
+    assert np.array_equal(kc, kc_want[0]) and np.array_equal(vc, vc_want[0])
+    assert np.array_equal(got, want[0])
+
+
 def test_predictor_loop_properties(oracle):
     units, layers, rows = 4, 2, 16
     q = oracle.normal_bf16((units, rows, 16, 128), 1)
