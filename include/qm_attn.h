@@ -206,6 +206,29 @@ int32_t qm_decode_attention_ragged(
     void* workspace, size_t workspace_bytes, uint32_t* status_dev,
     void* hip_stream);
 
+/*
+ * qm_decode_attention_ragged without a workspace argument and without any allocation.  It has no
+ * counterpart in the reference; it is for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The split records live
+ * in a device array of QM_DECODE_STATIC_SCRATCH_BYTES that the library itself holds on every GPU it
+ * runs on until the process ends (its address on a device is looked up at the first call on that
+ * device).  Same arguments, same kernels and the same bits as qm_decode_attention_ragged.
+ * A shape whose qm_decode_workspace_bytes exceeds the array returns QM_ERR_WORKSPACE and does
+ * nothing (G = 2: n_streams * kv_heads * min(32, max_seq_len/64 + 1) records of 1040 bytes, e.g.
+ * 31 streams of 8 kv heads at any length, 64 streams up to 960 tokens).
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams,
+ * two host threads) race; calls ordered on one stream are safe.  Nothing in the array needs to
+ * start at zero.
+ */
+#define QM_DECODE_STATIC_SCRATCH_BYTES (8u << 20)
+int32_t qm_decode_attention_ragged_static(
+    const uint16_t* query,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    const int32_t* seq_lens, int32_t n_streams, int32_t max_seq_len,
+    uint16_t* context_out,
+    int32_t q_heads, float scale, uint32_t* status_dev,
+    void* hip_stream);
+
 /* ---- (3) prefill ---------------------------------------------------------------------- */
 /*
  * Per-head RMSNorm (optional) + RoPE over rows.  Replaces rmsnorm_kernel with

@@ -57,6 +57,8 @@ _SIGNATURES = {
                                     _PTR, C.c_size_t, _PTR, _PTR]),
     "qm_decode_attention_ragged": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _PTR, _I32,
                                           _F32, _PTR, C.c_size_t, _PTR, _PTR]),
+    "qm_decode_attention_ragged_static": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _PTR, _I32,
+                                                 _F32, _PTR, _PTR]),
     "qm_norm_rope_rows": (_I32, [_PTR] * 5 + [_I32, _I32, _F32, _PTR]),
     "qm_scatter_kv": (_I32, [_PTR, _PTR, C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _PTR]),
     "qm_prefill_attention_causal": (_I32, [_PTR] * 4 + [C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _I32, _I32,
@@ -370,3 +372,13 @@ def predictor_rope_bhsd(x, cos, sin, out, rows, heads, stream=0):
 def predictor_update_cache(source, cache, rows, start, stream=0):
     _check(lib().qm_predictor_update_cache(_addr(source), _addr(cache), rows, start, stream),
            "qm_predictor_update_cache")
+
+
+DECODE_STATIC_SCRATCH_BYTES = 8 << 20
+
+
+def decode_attention_ragged_static(query, cache, page_table, max_pages, seq_lens, n_streams, max_seq_len, out,
+                                   q_heads, scale=SCALE_128, status=None, stream=0):
+    _check(lib().qm_decode_attention_ragged_static(
+        _addr(query), C.byref(cache), _addr(page_table), max_pages, _addr(seq_lens), n_streams,
+        max_seq_len, _addr(out), q_heads, scale, _addr(status), stream), "qm_decode_attention_ragged_static")

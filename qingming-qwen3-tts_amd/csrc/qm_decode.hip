@@ -32,6 +32,8 @@
 
 #include <stdlib.h>
 
+#include <atomic>
+
 namespace qm {
 
 constexpr int kDecodeThreads = 256;
@@ -596,6 +598,32 @@ int32_t decode_common(const uint16_t* query, const qm_kv_cache* cache, const int
     return QM_ERR_GEOMETRY;
 }
 
+// ---- split records in library-owned device memory --------------------------------------------
+// qm_decode_attention_ragged_static keeps the split records in this array instead of a caller's
+// workspace.  Every GPU the library runs on holds its own copy at its own address until the
+// process ends.  In host code the array's name is only a handle for hipGetSymbolAddress: kernels
+// are given the address that call returns for the current device, never the name.
+constexpr size_t kStaticScratchBytes = QM_DECODE_STATIC_SCRATCH_BYTES;
+static __device__ __attribute__((used)) __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on the current device, looked up once per device.
+int32_t static_scratch_address(void** address) {
+    static std::atomic<void*> known[kMaxDevices];
+    int dev = 0;
+    const hipError_t e0 = hipGetDevice(&dev);
+    if (e0 != hipSuccess) return hip_code(e0);
+    if (dev < 0 || dev >= kMaxDevices) return QM_ERR_NO_DEVICE;
+    void* ptr = known[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_code(e);
+        if (!ptr) return QM_ERR_NO_DEVICE;
+        known[dev].store(ptr, std::memory_order_release);
+    }
+    *address = ptr;
+    return QM_OK;
+}
+
 }  // namespace qm
 
 extern "C" size_t qm_decode_workspace_bytes(int32_t n_streams, int32_t q_heads, int32_t kv_heads,
@@ -663,4 +691,23 @@ extern "C" int32_t qm_decode_step_fused(
     step.step_position = position; step.step_epsilon = epsilon;
     return qm::decode_common(nullptr, cache, page_table, max_pages, nullptr, 1, key_start, key_end, key_end,
                              context_out, q_heads, scale, workspace, workspace_bytes, status_dev, hip_stream, &step);
+}
+
+extern "C" int32_t qm_decode_attention_ragged_static(
+    const uint16_t* query,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    const int32_t* seq_lens, int32_t n_streams, int32_t max_seq_len,
+    uint16_t* context_out,
+    int32_t q_heads, float scale, uint32_t* status_dev, void* hip_stream) {
+    if (!seq_lens || !page_table) return QM_ERR_NULL;
+    if (cache && n_streams > 0 && q_heads > 0 && cache->kv_heads > 0 && q_heads % cache->kv_heads == 0 && max_seq_len >= 0
+        && qm::decode_workspace_bytes(n_streams, q_heads, cache->kv_heads, max_seq_len) > qm::kStaticScratchBytes)
+        return QM_ERR_WORKSPACE;   // the shape needs more split records than the array holds
+    void* records = nullptr;
+    const int32_t rc = qm::static_scratch_address(&records);
+    if (rc != QM_OK) return rc;
+    // Nothing in the array has to start at zero: records of splits that do not exist are never used.
+    return qm::decode_common(query, cache, page_table, max_pages, seq_lens, n_streams, 0, 0,
+                             max_seq_len, context_out, q_heads, scale, records, qm::kStaticScratchBytes,
+                             status_dev, hip_stream);
 }
