@@ -94,13 +94,19 @@ const char* qm_target_arch(void);
  *       non-temporal hint when the contexts of one call may exceed 512 MiB (twice the last-level
  *       cache: less than that is partly still cached from the step before), and with plain loads
  *       otherwise; 1: always plain; 2: always
- *       non-temporal.  Same bits either way; other values make the call return QM_ERR_ARGUMENT. */
+ *       non-temporal.  Same bits either way; other values make the call return QM_ERR_ARGUMENT.
+ *   QM_OPT_PREDICTOR_LOOP_KERNEL  0 (default): qm_predictor_attention_loop forms Q.K^T and P.V on the
+ *       matrix cores (fp32 accumulation, fp32 softmax, bf16(QK), bf16(*scale) and bf16(P) as the
+ *       reference); 1: the reference's exact summation chain on the vector ALU (about 2.5x slower).
+ *       The rotated K and the cache write-back are bit-identical in both; contexts agree within the
+ *       operator's tolerance.  Other values make the call return QM_ERR_ARGUMENT. */
 enum {
     QM_OPT_PREFILL_SCORE_ROUNDING = 0,
     QM_OPT_DECODE_TILES_PER_BLOCK = 1,
     QM_OPT_PREFILL_KERNEL = 2,
     QM_OPT_DECODE_STREAMING_LOADS = 3,
-    QM_OPT_COUNT = 4
+    QM_OPT_PREDICTOR_LOOP_KERNEL = 4,
+    QM_OPT_COUNT = 5
 };
 /* Returns QM_ERR_ARGUMENT for an unknown option or a negative value. */
 int32_t qm_set_option(int32_t option, int32_t value);
@@ -323,7 +329,12 @@ int32_t qm_prefill_attention_causal_split(
  * causal two-row step 0); it changes the step numbering only, row r always attends keys
  * 0..r.  k_cache_out / v_cache_out: optional [units][8][16][128] write-back of the
  * per-unit cache (R17:10711-10737 layout), NULL to skip.
- * This operator reproduces the reference's full rounding chain, including bf16(P).
+ * Every bf16 rounding of the reference chain is kept, bf16(P) included.  With
+ * QM_OPT_PREDICTOR_LOOP_KERNEL = 1 the fp32 sums are also taken in the reference's order (results
+ * differ from a CPU restatement only where expf rounds differently); the default kernel takes the
+ * two products on the matrix cores (max abs error <= 1e-2 against the same restatement).  QK-RMSNorm,
+ * RoPE and the cache write-back are bit-exact in both.  The default kernel needs 16-byte aligned
+ * norm weights and RoPE rows as well (QM_ERR_GEOMETRY).
  */
 int32_t qm_predictor_attention_loop(
     const uint16_t* q, const uint16_t* k, const uint16_t* v,

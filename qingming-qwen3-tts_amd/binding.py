@@ -133,6 +133,7 @@ OPT_PREFILL_SCORE_ROUNDING = 0
 OPT_DECODE_TILES_PER_BLOCK = 1
 OPT_PREFILL_KERNEL = 2
 OPT_DECODE_STREAMING_LOADS = 3
+OPT_PREDICTOR_LOOP_KERNEL = 4
 
 
 def set_option(option, value):

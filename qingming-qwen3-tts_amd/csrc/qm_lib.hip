@@ -31,6 +31,7 @@ std::atomic<int32_t> g_options[QM_OPT_COUNT] = {
     {0},   // QM_OPT_DECODE_TILES_PER_BLOCK (0 = chosen from the problem size)
     {0},   // QM_OPT_PREFILL_KERNEL (0 = chosen from the grid size, 1 = four uniform waves, 2 = matrix/softmax wave pairs)
     {0},   // QM_OPT_DECODE_STREAMING_LOADS (0 = chosen from the bytes of context, 1 = plain loads, 2 = non-temporal loads)
+    {0},   // QM_OPT_PREDICTOR_LOOP_KERNEL (0 = matrix cores, 1 = the reference's exact summation chain)
 };
 }  // namespace
 

@@ -15,35 +15,11 @@
 
 #include "qm_device.h"
 #include "qm_host.h"
+#include "qm_predictor_params.h"
 
 #include <type_traits>
 
 namespace qm {
-
-constexpr int kPredRows = 16;     // kMaxCache of the reference (R17:7963)
-constexpr int kPredThreads = 256;
-
-struct PredictorParams {
-    const uint16_t* q;        // [units][rows][16][128]
-    const uint16_t* k;        // [units][rows][8][128]
-    const uint16_t* v;        // [units][rows][8][128]
-    const uint16_t* q_norm_w; // [n_layers][128]
-    const uint16_t* k_norm_w; // [n_layers][128]
-    const uint16_t* cos_rows; // [rows][128]
-    const uint16_t* sin_rows; // [rows][128]
-    uint16_t* out;            // [units][rows][16][128]
-    uint16_t* k_cache_out;    // [units][8][16][128] or NULL
-    uint16_t* v_cache_out;    // [units][8][16][128] or NULL
-    int64_t unit_base;        // index of the first unit of this launch (layer = unit % n_layers)
-    int n_layers;
-    int rows;
-    float epsilon;
-    // STAGED mode (the reference's six-kernel attention, R17:13300-13386): q is already rotated and
-    // laid out [16][rows][128]; k, v point at the [8][16][128] caches; row r sees the keys
-    // j < key_length with (causal ? j <= r : true).
-    int key_length;
-    int causal;
-};
 
 // bf16 round trip with the hardware converter (round to nearest even; same bits as the integer
 // formula of R17:8172-8187 for every non-NaN input).
@@ -437,6 +413,8 @@ extern "C" int32_t qm_predictor_attention_loop(
                           | reinterpret_cast<uintptr_t>(v_cache_out);
     if (align & 15) return QM_ERR_GEOMETRY;
     if (units == 0) return QM_OK;
+    const int32_t kernel = qm::option_value(QM_OPT_PREDICTOR_LOOP_KERNEL);
+    if (kernel < 0 || kernel > 1) return QM_ERR_ARGUMENT;
     qm::PredictorParams prm;
     prm.q = q; prm.k = k; prm.v = v;
     prm.q_norm_w = q_norm_w; prm.k_norm_w = k_norm_w;
@@ -444,6 +422,12 @@ extern "C" int32_t qm_predictor_attention_loop(
     prm.out = context_out; prm.k_cache_out = k_cache_out; prm.v_cache_out = v_cache_out;
     prm.unit_base = 0; prm.n_layers = n_layers; prm.rows = rows; prm.epsilon = epsilon;
     prm.key_length = 0; prm.causal = 1;
+    if (kernel == 0) {
+        const uintptr_t more = reinterpret_cast<uintptr_t>(q_norm_w) | reinterpret_cast<uintptr_t>(k_norm_w)
+                             | reinterpret_cast<uintptr_t>(cos_rows) | reinterpret_cast<uintptr_t>(sin_rows);
+        if (more & 15) return QM_ERR_GEOMETRY;
+        return qm::launch_predictor_loop_mfma(prm, units, static_cast<hipStream_t>(hip_stream));
+    }
     // grid.y is limited to 65535: fold large unit counts into several launches.
     const int32_t per_launch = 65535;
     for (int32_t first = 0; first < units; first += per_launch) {

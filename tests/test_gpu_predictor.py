@@ -1,8 +1,10 @@
 """GPU parity: the code predictor's 16-step attention loop in one launch, through the C ABI.
 
-The kernel keeps the reference's whole rounding chain and summation order, so beyond the stated
-tolerance (max abs error <= 1e-2) nearly every output must be bit-identical to the oracle; the K/V
-cache write-back must be bit-exact.
+Two kernels serve the entry point (QM_OPT_PREDICTOR_LOOP_KERNEL).  The exact-chain kernel (1) keeps the
+reference's whole rounding chain and summation order, so beyond the stated tolerance (max abs error
+<= 1e-2) nearly every output must be bit-identical to the oracle.  The default kernel (0) takes Q.K^T
+and P.V on the matrix cores: outputs within the tolerance.  In both, QK-RMSNorm + RoPE are the
+reference's chain exactly: the K/V cache write-back must be bit-exact.
 """
 import numpy as np
 import pytest
@@ -14,7 +16,19 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-2
 
 
-def _run(oracle, qm, dev, units, layers, rows, seed, first_rows=1, write_cache=True):
+EXACT, MATRIX = 1, 0
+
+
+def _run(oracle, qm, dev, units, layers, rows, seed, first_rows=1, write_cache=True, kernel=EXACT):
+    import torch
+    qm.set_option(qm.OPT_PREDICTOR_LOOP_KERNEL, kernel)
+    try:
+        return _run_selected(oracle, qm, dev, units, layers, rows, seed, first_rows, write_cache)
+    finally:
+        qm.set_option(qm.OPT_PREDICTOR_LOOP_KERNEL, 0)
+
+
+def _run_selected(oracle, qm, dev, units, layers, rows, seed, first_rows, write_cache):
     import torch
     q = oracle.normal_bf16((units, rows, 16, 128), seed)
     k = oracle.normal_bf16((units, rows, 8, 128), seed + 1)
@@ -36,29 +50,41 @@ def _run(oracle, qm, dev, units, layers, rows, seed, first_rows=1, write_cache=T
     return to_u16(out), want, (to_u16(kd) if write_cache else None, to_u16(vd) if write_cache else None), (kc, vc), v
 
 
-def test_predictor_config5_full_size(oracle, qm, dev):
+@pytest.mark.parametrize("kernel", [MATRIX, EXACT])
+def test_predictor_config5_full_size(oracle, qm, dev, kernel):
     units, layers, rows = 256 * 5, 5, 16
-    got, want, (kd, vd), (kc, vc), v = _run(oracle, qm, dev, units, layers, rows, seed=55)
+    got, want, (kd, vd), (kc, vc), v = _run(oracle, qm, dev, units, layers, rows, seed=55, kernel=kernel)
     assert max_abs_err(oracle, got, want) <= TOL
-    assert (got != want).mean() < 1e-3                        # only device-expf rounding may differ
+    if kernel == EXACT:
+        assert (got != want).mean() < 1e-3                    # only device-expf rounding may differ
     assert np.array_equal(kd, kc) and np.array_equal(vd, vc)  # cache write-back, bit-exact
     assert np.array_equal(got[:, 0], np.repeat(v[:, 0], 2, axis=1))   # step 0: context 1 -> out = V
 
 
 @pytest.mark.parametrize("units,layers,rows,first_rows", [(1, 1, 16, 1), (7, 5, 16, 2), (3, 2, 1, 1), (5, 5, 2, 2),
                                                           (4, 3, 9, 1)])
-def test_predictor_small_and_partial(oracle, qm, dev, units, layers, rows, first_rows):
+@pytest.mark.parametrize("kernel", [MATRIX, EXACT])
+def test_predictor_small_and_partial(oracle, qm, dev, units, layers, rows, first_rows, kernel):
     got, want, (kd, vd), (kc, vc), _ = _run(oracle, qm, dev, units, layers, rows, seed=units * 31 + rows,
-                                           first_rows=first_rows)
+                                           first_rows=first_rows, kernel=kernel)
     assert max_abs_err(oracle, got, want) <= TOL
-    assert (got != want).mean() < 1e-3
+    if kernel == EXACT:
+        assert (got != want).mean() < 1e-3
     assert np.array_equal(kd, kc) and np.array_equal(vd, vc)
 
 
 def test_predictor_without_cache_and_errors(oracle, qm, dev):
     import torch
-    got, want, _, _, _ = _run(oracle, qm, dev, 6, 5, 16, seed=3, write_cache=False)
-    assert max_abs_err(oracle, got, want) <= TOL
+    for kernel in (MATRIX, EXACT):
+        got, want, _, _, _ = _run(oracle, qm, dev, 6, 5, 16, seed=3, write_cache=False, kernel=kernel)
+        assert max_abs_err(oracle, got, want) <= TOL
+    qm.set_option(qm.OPT_PREDICTOR_LOOP_KERNEL, 2)
+    try:
+        with pytest.raises(qm.QmError) as e:
+            _run_selected(oracle, qm, dev, 1, 1, 2, 3, 1, False)
+        assert e.value.code == -5
+    finally:
+        qm.set_option(qm.OPT_PREDICTOR_LOOP_KERNEL, 0)
     z = torch.zeros((1, 16, 16, 128), dtype=torch.int16, device=dev)
     w = torch.zeros((1, 128), dtype=torch.int16, device=dev)
     r = torch.zeros((16, 128), dtype=torch.int16, device=dev)
@@ -108,7 +134,8 @@ def test_predictor_staged_attention_argument_errors(qm, dev):
     assert L.qm_predictor_attention_staged(None, c.data_ptr(), c.data_ptr(), z.data_ptr(), 2, 2, 1, None) == -1
 
 
-def test_predictor_loop_is_exactly_linear_in_v_at_config5_size(oracle, qm, dev):
+@pytest.mark.parametrize("kernel", [MATRIX, EXACT])
+def test_predictor_loop_is_exactly_linear_in_v_at_config5_size(oracle, qm, dev, kernel):
     """A property that does not depend on the size, at the benchmark's full shape (256 frames x 5 layers x 16
     steps): doubling every V (one more in the bf16 exponent, exact) doubles every output bit for bit — the
     probabilities do not see V, and the leaves fmaf(P, V, +0), the tree sums and the final rounding commute with
@@ -130,11 +157,15 @@ def test_predictor_loop_is_exactly_linear_in_v_at_config5_size(oracle, qm, dev):
         return bits
 
     outs = []
-    for vv in (v, doubled(v)):
-        out = torch.full((units, rows, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
-        qm.predictor_attention_loop(q, k, to_dev(vv, dev), gq, gk, cos, sin, out, None, None, units, layers, rows, 1)
-        torch.cuda.synchronize()
-        outs.append(to_u16(out))
+    qm.set_option(qm.OPT_PREDICTOR_LOOP_KERNEL, kernel)
+    try:
+        for vv in (v, doubled(v)):
+            out = torch.full((units, rows, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+            qm.predictor_attention_loop(q, k, to_dev(vv, dev), gq, gk, cos, sin, out, None, None, units, layers, rows, 1)
+            torch.cuda.synchronize()
+            outs.append(to_u16(out))
+    finally:
+        qm.set_option(qm.OPT_PREDICTOR_LOOP_KERNEL, 0)
     assert np.count_nonzero(outs[0] & 0x7F80) > outs[0].size * 0.99
     assert np.array_equal(outs[1], doubled(outs[0]))
 
@@ -212,8 +243,12 @@ def test_predictor_step0_chain_equals_loop_rows(oracle, qm, dev):
     out = torch.full((1, rows, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
     kd = torch.full((1, 8, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
     vd = torch.full((1, 8, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
-    qm.predictor_attention_loop(to_dev(q, dev), to_dev(k, dev), to_dev(v, dev), to_dev(gq, dev), to_dev(gk, dev),
-                                to_dev(cos, dev), to_dev(sin, dev), out, kd, vd, 1, 1, rows, 2)
+    qm.set_option(qm.OPT_PREDICTOR_LOOP_KERNEL, EXACT)       # the staged kernel shares the exact chain's arithmetic
+    try:
+        qm.predictor_attention_loop(to_dev(q, dev), to_dev(k, dev), to_dev(v, dev), to_dev(gq, dev), to_dev(gk, dev),
+                                    to_dev(cos, dev), to_dev(sin, dev), out, kd, vd, 1, 1, rows, 2)
+    finally:
+        qm.set_option(qm.OPT_PREDICTOR_LOOP_KERNEL, 0)
     torch.cuda.synchronize()
     got, kc, vc = step0_chain(oracle, _DeviceStep0Ops(qm, dev), q[0], k[0], v[0], gq[0], gk[0], cos, sin, rows)
     assert np.array_equal(kc, to_u16(kd)[0]) and np.array_equal(vc, to_u16(vd)[0])
