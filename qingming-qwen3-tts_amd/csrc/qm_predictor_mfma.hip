@@ -102,13 +102,39 @@ __device__ __forceinline__ float vector_sum_squares(const VecRegs& v) {
 __device__ __forceinline__ uint4 lds_set(const unsigned char* row, int kb, int grp) {
     return *reinterpret_cast<const uint4*>(row + 64 * kb + 16 * grp);
 }
-__device__ __forceinline__ float elem4(const uint4& raw, int e) {
-    const uint32_t w = e < 2 ? raw.x : e < 4 ? raw.y : e < 6 ? raw.z : raw.w;
-    return (e & 1) ? hi_bf16(w) : lo_bf16(w);
+// a.lo * b.lo + a.hi * b.hi of packed bf16 pairs, two or four at a time, in the three-operand encoding with
+// a literal 0 addend (the compiler's own choice, the two-operand form, needs a zeroed accumulator register
+// per use).  The compiler cannot see through an assembly statement, so the wait states this chip wants
+// between a dot-product instruction's write and another instruction's read of it (three) are part of the
+// statement: the results of a group are independent of one another and one s_nop ends the group.
+__device__ __forceinline__ void dot2_pairs_x2(uint32_t a0, uint32_t b0, uint32_t a1, uint32_t b1, float& d0, float& d1) {
+    asm("v_dot2_f32_bf16 %0, %2, %3, 0\n\tv_dot2_f32_bf16 %1, %4, %5, 0\n\ts_nop 2"
+        : "=&v"(d0), "=&v"(d1) : "v"(a0), "v"(b0), "v"(a1), "v"(b1));
+}
+__device__ __forceinline__ void dot2_pairs_x4(uint32_t a0, uint32_t b0, uint32_t a1, uint32_t b1, uint32_t a2, uint32_t b2,
+                                              uint32_t a3, uint32_t b3, float& d0, float& d1, float& d2, float& d3) {
+    asm("v_dot2_f32_bf16 %0, %4, %5, 0\n\tv_dot2_f32_bf16 %1, %6, %7, 0\n\t"
+        "v_dot2_f32_bf16 %2, %8, %9, 0\n\tv_dot2_f32_bf16 %3, %10, %11, 0\n\ts_nop 2"
+        : "=&v"(d0), "=&v"(d1), "=&v"(d2), "=&v"(d3)
+        : "v"(a0), "v"(b0), "v"(a1), "v"(b1), "v"(a2), "v"(b2), "v"(a3), "v"(b3));
+}
+
+__device__ __forceinline__ uint32_t word_of(const uint4& raw, int e) {
+    return e < 2 ? raw.x : e < 4 ? raw.y : e < 6 ? raw.z : raw.w;
+}
+
+// bf16(value) placed in the half of a packed pair that element e occupies (even e: low), the other half +0.
+__device__ __forceinline__ uint32_t round_into_slot(float value, int e) {
+    return (e & 1) ? pack_bf16_pair(0.0f, value) : pack_bf16_pair(value, 0.0f);
 }
 
 // RMSNorm + RoPE of the vector in place (packed bf16), every rounding of R17:12207-12279.
 // gamma, cosv, sinv: LDS rows of 128 bf16 (the norm weight; the RoPE row of this lane's vector).
+// A product of two bf16 values is exact in fp32, so bf16(a) * b is taken as
+// v_dot2_f32_bf16((bf16(a), 0), (b, neighbour)) straight from the packed operands: nothing is
+// unpacked, and the rounding instruction is the conversion itself.  The last step,
+// bf16(w cos) + bf16(rotated w sin), is the same instruction on (1, +-1).  (A product that is an
+// exact zero may come out as +0 where a scalar multiply gives -0.)
 __device__ __forceinline__ void norm_rope_vector(VecRegs& v, const unsigned char* gamma, const unsigned char* cosv,
                                                  const unsigned char* sinv, float epsilon, int grp) {
     const float total = vector_sum_squares(v);
@@ -122,13 +148,13 @@ __device__ __forceinline__ void norm_rope_vector(VecRegs& v, const unsigned char
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const float x0 = elem(v, kb, e), x1 = elem(v, kb + 2, e);
-            float n0, n1, w0, w1, f0, f1, t0, t1;
-            round_bf16_pair(x0 * r, x1 * r, n0, n1);
-            round_bf16_pair(n0 * elem4(g0, e), n1 * elem4(g1, e), w0, w1);
-            round_bf16_pair(w0 * elem4(c0, e), w1 * elem4(c1, e), f0, f1);
-            round_bf16_pair((-w1) * elem4(s0, e), w0 * elem4(s1, e), t0, t1);
-            lo[e] = f0 + t0;
-            hi[e] = f1 + t1;
+            const uint32_t n0 = round_into_slot(x0 * r, e), n1 = round_into_slot(x1 * r, e);
+            float g_0, g_1, f0, f1, t0, t1;
+            dot2_pairs_x2(n0, word_of(g0, e), n1, word_of(g1, e), g_0, g_1);
+            const uint32_t w0 = round_into_slot(g_0, e), w1 = round_into_slot(g_1, e);
+            dot2_pairs_x4(w0, word_of(c0, e), w1, word_of(c1, e), w1, word_of(s0, e), w0, word_of(s1, e), f0, f1, t0, t1);
+            // dimension d < 64: bf16(w0 cos) + bf16(-w1 sin) = bf16(w0 cos) - bf16(w1 sin); d + 64: both added
+            dot2_pairs_x2(pack_bf16_pair(f0, t0), 0xBF803F80U, pack_bf16_pair(f1, t1), 0x3F803F80U, lo[e], hi[e]);
         }
         v.raw[kb] = make_uint4(pack_bf16_pair(lo[0], lo[1]), pack_bf16_pair(lo[2], lo[3]),
                                pack_bf16_pair(lo[4], lo[5]), pack_bf16_pair(lo[6], lo[7]));
