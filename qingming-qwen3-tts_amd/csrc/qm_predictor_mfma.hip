@@ -1,7 +1,7 @@
 // qm_predictor_mfma.hip — the code predictor's per-frame attention loop on the matrix cores (gfx950).
 //
-// One 64-lane wave owns one (unit, kv head) item, unit = (frame, layer), start to end; there is
-// no block-level synchronisation.  Q (two heads), K and the RoPE rows are loaded straight into the
+// One 64-lane wave owns one (unit, kv head) item, unit = (frame, layer), start to end; the four waves of
+// a block share only the RoPE rows and norm weights, staged once in LDS.  Q (two heads), K and the RoPE rows are loaded straight into the
 // MFMA operand layout of v_mfma_f32_16x16x32_bf16 — lane l holds vector (row) l % 16, dimensions
 // 32 kb + 8 (l / 16) + e, kb = 0..3, e = 0..7 — in which
 //   * the reference's 32-dimension groups of the sum of squares are the four kb register sets, and
@@ -20,8 +20,11 @@
 // products are the matrix core's, the exponential is v_exp_f32 and the division a reciprocal —
 // within the operator's tolerance (max abs error <= 1e-2), not bit-identical.
 //
-// Per item: 16 KiB in, 8 KiB out (+ 8 KiB with the cache write-back); about 1 900 wave
-// instructions against 7 000 of the exact-chain kernel, which is bound by VALU issue.
+// Per item: 16 KiB in, 8 KiB out (+ 8 KiB with the cache write-back); about 1 700 vector
+// instructions against 7 000 of the exact-chain kernel, which is bound by VALU issue.  The context
+// rows are staged through the (consumed) V tile so that global stores are 16 bytes per lane:
+// 8-byte stores straight from the accumulator layout cost 59 us instead of 50 us at 256 x 5 x 16.
+// Non-temporal loads and stores were measured and are slower here (52 us).
 
 #include "qm_device.h"
 #include "qm_host.h"
@@ -297,22 +300,40 @@ __global__ __launch_bounds__(kPredThreads, 4) void predictor_loop_mfma_kernel(Pr
     // lane group G reads keys 4 G .. 4 G + 3, the k indices of its MFMA operand.
     const uint32_t v_lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)vt))
                          + (4 * grp + ((lane >> 2) & 3)) * kVRowBytes + 8 * (lane & 3);
-    uint16_t* out0 = prm.out + (row64 * 16 + 2 * kvh) * kDim + 4 * grp;
     __builtin_amdgcn_s_waitcnt(0xc07f);               // lgkmcnt(0): this wave's own LDS writes have landed
     __builtin_amdgcn_wave_barrier();
+    unsigned long long frag[8];
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-        unsigned long long frag;
-        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2\n\ts_waitcnt lgkmcnt(0)" : "=v"(frag) : "v"(v_lds), "n"(32 * t) : "memory");
-        const s16x4_t vf = __builtin_bit_cast(s16x4_t, frag);
-        f32x4_t o0 = {0.0f, 0.0f, 0.0f, 0.0f}, o1 = {0.0f, 0.0f, 0.0f, 0.0f};
-        o0 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, p[0], o0, 0, 0, 0);
-        o1 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, p[1], o1, 0, 0, 0);
-        if (valid) {
+    for (int t = 0; t < 8; ++t)
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(frag[t]) : "v"(v_lds), "n"(32 * t) : "memory");
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(frag[0]), "+v"(frag[1]), "+v"(frag[2]), "+v"(frag[3]), "+v"(frag[4]), "+v"(frag[5]), "+v"(frag[6]), "+v"(frag[7])
+                 :
+                 : "memory");
+    __builtin_amdgcn_wave_barrier();
+    // The V tile has been read: its LDS rows now stage one head's context at a time ([row][128] bf16), so that
+    // the global stores are 16 bytes per lane, 256 contiguous bytes per row.
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            f32x4_t o = {0.0f, 0.0f, 0.0f, 0.0f};
+            o = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, frag[t]), p[g], o, 0, 0, 0);
             // lane: query row `vec`, dimensions 16 t + 4 G + 0..3
-            *reinterpret_cast<uint2*>(out0 + 16 * t) = make_uint2(pack_bf16_pair(o0[0], o0[1]), pack_bf16_pair(o0[2], o0[3]));
-            *reinterpret_cast<uint2*>(out0 + kDim + 16 * t) = make_uint2(pack_bf16_pair(o1[0], o1[1]), pack_bf16_pair(o1[2], o1[3]));
+            *reinterpret_cast<uint2*>(vt + vec * kVRowBytes + 2 * (16 * t + 4 * grp)) =
+                make_uint2(pack_bf16_pair(o[0], o[1]), pack_bf16_pair(o[2], o[3]));
         }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int orow = 4 * j + grp;             // 16 lanes move one row: piece `vec` of row orow
+            const uint4 val = *reinterpret_cast<const uint4*>(vt + orow * kVRowBytes + 16 * vec);
+            if (orow < rows)
+                *reinterpret_cast<uint4*>(prm.out + ((unit * rows + orow) * 16 + 2 * kvh + g) * kDim + 8 * vec) = val;
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);           // the rows have been read before the next head overwrites them
+        __builtin_amdgcn_wave_barrier();
     }
 }
 
