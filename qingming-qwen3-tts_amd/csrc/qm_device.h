@@ -36,6 +36,14 @@ __device__ __forceinline__ float round_bf16(float x) {
     return static_cast<float>(static_cast<__bf16>(x));
 }
 
+// One rounding with one v_cvt_pk_bf16_f32 and nothing to take apart: (0, x) converts to bf16(x) in the
+// upper half of the register over zeros, which is the rounded value as fp32.
+__device__ __forceinline__ float round_bf16_single(float x) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t in = {0.0f, x};
+    return __uint_as_float(__builtin_bit_cast(uint32_t, __builtin_convertvector(in, bf16x2_t)));
+}
+
 // Two roundings with one v_cvt_pk_bf16_f32.
 __device__ __forceinline__ void round_bf16_pair(float a, float b, float& ra, float& rb) {
     typedef float f32x2_t __attribute__((ext_vector_type(2)));

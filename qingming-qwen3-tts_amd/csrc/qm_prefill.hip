@@ -1382,7 +1382,9 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
             o[c][i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i], p_prev[c].g[i >> 2], o[c][i & 3], 0, 0, 0);
         };
         auto qk_mfma = [&](int i, int c) {
-            s_next[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qf[c][i], s_next[c], 0, 0, 0);
+            // (the first product of a chunk starts from a literal zero instead of sixteen zeroed registers)
+            const f32x16_t zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+            s_next[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qf[c][i], i == 0 ? zero : s_next[c], 0, 0, 0);
         };
         half_arrived(int_c<0>{}, int_c<12>{}, kraw, vraw, kf, vf);
         // (ROUND) the maxima of the raw scores are taken in the first group and then walk, one step per group,
@@ -1390,14 +1392,10 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         // negative scale elsewhere) and the exchange between the two halves of the wave, so that the branch
         // on them after the last group waits for nothing
         float mx_a[NC], mx_b[NC], mx_step[NC], mx_limit[NC];
-        uint32_t mx_bits[NC];
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s_next[c][r] = 0.0f;
             mx_a[c] = mx_b[c] = -INFINITY;
             mx_step[c] = 0.0f;
-            mx_bits[c] = 0;
             mx_limit[c] = m_run[c] + slack;
         }
 #pragma unroll
@@ -1408,14 +1406,17 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
                 pv_mfma(g, c);
                 fence();
                 if (ROUND) {
+                    // (a rounding is one instruction per score: v_cvt_pk_bf16_f32 of (0, x) leaves bf16(x) in the
+                    // upper half of the register, which is the rounded value as fp32; rounding two scores into
+                    // one register costs the conversion and two instructions to take them apart again)
                     const float xa0 = s_cur[c][ra], xa1 = s_cur[c][ra + 1], xb0 = s_cur[c][rb], xb1 = s_cur[c][rb + 1];
-                    uint32_t pa = pack_bf16_pair(xa0, xa1);
-                    const uint32_t pb = pack_bf16_pair(xb0, xb1);
+                    float ua0 = round_bf16_single(xa0);
+                    const float ua1 = round_bf16_single(xa1), ub0 = round_bf16_single(xb0), ub1 = round_bf16_single(xb1);
                     if (g == 0) {
                         // (assembly: the compiler's fmaxf first quiets every operand with an instruction of its
-                        // own.  `pa` passes through the first statement so that the chain follows a read of the
+                        // own.  `ua0` passes through the first statement so that the chain follows a read of the
                         // MFMA results that the compiler guards; one MFMA wrote all sixteen.)
-                        asm volatile("v_max3_f32 %0, %0, %2, %3" : "+v"(mx_a[c]), "+v"(pa) : "v"(s_cur[c][0]), "v"(s_cur[c][1]));
+                        asm volatile("v_max3_f32 %0, %0, %2, %3" : "+v"(mx_a[c]), "+v"(ua0) : "v"(s_cur[c][0]), "v"(s_cur[c][1]));
                         asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(mx_b[c]) : "v"(s_cur[c][2]), "v"(s_cur[c][3]));
 #pragma unroll
                         for (int r = 4; r < 16; r += 4) {
@@ -1423,42 +1424,30 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
                             asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(mx_b[c]) : "v"(s_cur[c][r + 2]), "v"(s_cur[c][r + 3]));
                         }
                     }
-                    if (g == 3) {
-                        mx_bits[c] = pack_bf16_pair(mx_step[c], mx_step[c]);
-                        asm volatile("" : "+v"(mx_bits[c]));
-                    }
-                    fence();
-                    const float ua0 = lo_bf16(pa), ua1 = hi_bf16(pa), ub0 = lo_bf16(pb), ub1 = hi_bf16(pb);
                     if (g == 1) {
                         asm volatile("v_max_f32 %0, %1, %2" : "=v"(mx_step[c]) : "v"(mx_a[c]), "v"(mx_b[c]));
                     }
                     if (g == 3) {
-                        mx_step[c] = lo_bf16(mx_bits[c]);
+                        mx_step[c] = round_bf16_single(mx_step[c]);
                         asm volatile("" : "+v"(mx_step[c]));
                     }
                     fence();
                     const float ya0 = ua0 * prm.scale, ya1 = ua1 * prm.scale;
-                    if (g == 1) {
-                        mx_bits[c] = pack_bf16_pair(mx_step[c], mx_step[c]);
-                        asm volatile("" : "+v"(mx_bits[c]));
-                    }
                     fence();
                     qk_mfma(g, c);
                     fence();
                     const float yb0 = ub0 * prm.scale, yb1 = ub1 * prm.scale;
-                    if (g == 2) {
-                        mx_step[c] = lo_bf16(mx_bits[c]);
+                    if (g == 1) {
+                        mx_step[c] = round_bf16_single(mx_step[c]);
                         asm volatile("" : "+v"(mx_step[c]));
                     }
-                    fence();
-                    const uint32_t qa = pack_bf16_pair(ya0, ya1);
-                    const uint32_t qb = pack_bf16_pair(yb0, yb1);
                     if (g == 2) {
                         mx_step[c] = mx_step[c] * prm.scale;
                         asm volatile("" : "+v"(mx_step[c]));
                     }
                     fence();
-                    float za0 = lo_bf16(qa), za1 = hi_bf16(qa), zb0 = lo_bf16(qb), zb1 = hi_bf16(qb);
+                    float za0 = round_bf16_single(ya0), za1 = round_bf16_single(ya1);
+                    float zb0 = round_bf16_single(yb0), zb1 = round_bf16_single(yb1);
                     // (an empty statement that keeps the roundings here instead of sinking to where they are used)
                     asm volatile("" : "+v"(za0), "+v"(za1), "+v"(zb0), "+v"(zb1));
                     if (g == 3) {
