@@ -37,6 +37,7 @@ extern "C" {
 #define QM_ERR_WORKSPACE     -4   /* caller workspace missing or too small           */
 #define QM_ERR_ARGUMENT      -5   /* negative counts, unsupported option             */
 #define QM_ERR_NO_DEVICE     -6   /* no gfx950 device / kernel image unusable        */
+#define QM_ERR_STATUS        -9   /* (engine) a kernel OR-ed QM_STATUS_* bits into the status word   */
 #define QM_ERR_HIP_BASE   -1000   /* -(1000 + hipError_t) for launch failures        */
 
 /* bits OR-ed by kernels into the optional device status word */
@@ -251,12 +252,14 @@ int32_t qm_norm_rope_rows(
 /*
  * Replaces scatter_prefill_cache (R17:17646-17682, kernel R17:15630-15687) and, with
  * rows == 1, scatter_decode_cache (R17:17684-17720).  key/value [rows][kv_heads][128]
- * are copied to tokens first_position .. first_position+rows-1.
+ * are copied to tokens first_position .. first_position+rows-1.  A token whose page table entry is outside
+ * [0, n_pages) is skipped and QM_STATUS_BAD_PAGE is OR-ed into *status_dev (optional, device uint32); the
+ * reference has one flat cache and no such case.
  */
 int32_t qm_scatter_kv(
     const uint16_t* key, const uint16_t* value,
     const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
-    int32_t rows, int32_t first_position,
+    int32_t rows, int32_t first_position, uint32_t* status_dev,
     void* hip_stream);
 
 /*
@@ -296,8 +299,12 @@ int32_t qm_prefill_attention_causal(
  *   qm_prefill_split_workspace_bytes: bytes needed for (batch, seq, kv_heads) on the current
  *     device; 0 when the call would not split: fewer than 9 query tiles of 64 rows, or no room
  *     for the added blocks at two blocks per compute unit (a negative value is an error code).
- *   qm_prefill_split_workspace_init: once after allocation (a kernel on hip_stream); every call
- *     leaves the workspace as it found it.  workspace: 256-byte aligned device memory.
+ *   qm_prefill_split_workspace_init: once after allocation (a kernel on hip_stream).  Every launch
+ *     tags what it writes with a number of its own, so a call never believes what an earlier call
+ *     left behind (also one that ended with QM_STATUS_SPLIT_TIMEOUT) and nothing has to be reset
+ *     between calls.  A launch captured in a HIP graph is replayed with the number it was captured
+ *     with: after QM_STATUS_SPLIT_TIMEOUT initialise the workspace again before the next replay.
+ *     workspace: 256-byte aligned device memory.
  *   qm_prefill_attention_causal_split: workspace NULL or a shape that does not split: exactly
  *     qm_prefill_attention_causal; too small for the shape: QM_ERR_WORKSPACE.  Only the default
  *     kernel (QM_OPT_PREFILL_KERNEL 0 or 3) splits.  Two calls that overlap in time must not share
@@ -570,6 +577,24 @@ int32_t qm_final_head_sample(
 int32_t qm_gather_embedding(
     const uint16_t* table, int32_t table_rows, const int32_t* codes, int32_t group, int32_t dimension,
     uint16_t* selected_embeddings, uint16_t* next_step_input, void* hip_stream);
+
+/*
+ * The two ends of a code-predictor frame (PersistentPredictor::run_frame_device R17:13043-13156, capture_graph
+ * :13856-13896).
+ * qm_predictor_prepare_group0 replaces prepare_group0_input_kernel (R17:11963-11996): with token = code0[0] (the
+ *   talker's code of the frame, on the device), row `token` of the talker's codec embedding table becomes
+ *   selected_embeddings[0][*] and the second row of the two-row input free_input[1][*]; generated_codes[0] =
+ *   token.  A token outside [0, table_rows) stores code 0 and moves nothing, as in the reference.
+ * qm_predictor_next_talker_input replaces sum_codec_embeddings_kernel (R17:8877-8906) and the add behind it
+ *   (R17:13872-13875): embedding_sum = bf16(sum over the `groups` selected embeddings, fp32, in group order),
+ *   next_talker_input = bf16(embedding_sum + context_embedding).  embedding_sum may be NULL.
+ */
+int32_t qm_predictor_prepare_group0(
+    const uint16_t* codec_table, int32_t table_rows, const int32_t* code0, int32_t dimension,
+    uint16_t* free_input, uint16_t* selected_embeddings, int32_t* generated_codes, void* hip_stream);
+int32_t qm_predictor_next_talker_input(
+    const uint16_t* selected_embeddings, int32_t groups, const uint16_t* context_embedding, int32_t dimension,
+    uint16_t* embedding_sum, uint16_t* next_talker_input, void* hip_stream);
 
 #ifdef __cplusplus
 }

@@ -135,7 +135,7 @@ inline void scatter_prefill_cache(const std::uint16_t* key, const std::uint16_t*
                                   int sequence_length, int kv_heads, int head_dim, int max_cache,
                                   void* stream) {
     const qm_kv_cache c = flat_cache(key_cache, value_cache, kv_heads, head_dim, max_cache);
-    check(qm_scatter_kv(key, value, &c, nullptr, 1, sequence_length, 0, stream),
+    check(qm_scatter_kv(key, value, &c, nullptr, 1, sequence_length, 0, nullptr, stream),
           "Talker prefill KV scatter launch");
 }
 
@@ -145,18 +145,21 @@ inline void scatter_decode_cache(const std::uint16_t* key, const std::uint16_t* 
                                  int head_dim, int max_cache, int cache_position, void* stream) {
     if (cache_position >= max_cache) throw std::runtime_error("Talker decode cache overflow.");
     const qm_kv_cache c = flat_cache(key_cache, value_cache, kv_heads, head_dim, max_cache);
-    check(qm_scatter_kv(key, value, &c, nullptr, 1, 1, cache_position, stream),
+    check(qm_scatter_kv(key, value, &c, nullptr, 1, 1, cache_position, nullptr, stream),
           "Talker decode KV scatter launch");
 }
 
 // ≙ PersistentPredictor::attention_m1 (R17:13473-13497): cache [8][16][128], key_length <= 16.
+// Served by the exact-chain kernel (bf16(QK), bf16(* scale), full-row softmax, bf16(P), the reference's
+// summation order): with at most 16 keys an online-softmax result can differ from the reference chain by a
+// bf16 ulp of the output, which is more than the operator's tolerance when outputs exceed 2.
 inline void predictor_attention_m1(const std::uint16_t* query_rotated, std::uint16_t* key_cache,
                                    std::uint16_t* value_cache, std::uint16_t* attention_context,
                                    int key_length, void* stream) {
     if (key_length < 1 || key_length > 16) throw std::runtime_error("Predictor attention: key_length out of range");
-    const qm_kv_cache c = flat_cache(key_cache, value_cache, 8, 128, 16);
-    check(qm_decode_attention(query_rotated, &c, nullptr, 1, attention_context, 16, key_length - 1, -1,
-                              0.08838834764831845f, nullptr, 0, stream),
+    // one query row: [16][1][128] (BHSD) and [1][16][128] are the same bytes as [16][128]
+    check(qm_predictor_attention_staged(query_rotated, key_cache, value_cache, attention_context, 1, key_length, 0,
+                                        stream),
           "Predictor M1 attention launch");
 }
 

@@ -97,8 +97,75 @@ int32_t qm_talker_decode(qm_talker* engine, const uint16_t* input_device, const 
  */
 int32_t qm_talker_prefill(qm_talker* engine, const uint16_t* input_device, const uint16_t* cosine,
                           const uint16_t* sine, int32_t rows, const uint16_t** final_hidden_device);
-/* Waits for the engine's stream. */
+/* Waits for the engine's stream, then reads the device status word the attention kernels OR their
+ * QM_STATUS_* bits into (page or position out of range, a key-split block that gave up waiting): if any is
+ * set the word is cleared, the key-split workspace initialised again and QM_ERR_STATUS returned — what was
+ * computed since the last synchronisation is not to be used. */
 int32_t qm_talker_synchronize(qm_talker* engine);
+
+/* The engine's generation stream (hipStream_t as void*): the final head and the predictor of a generation
+ * loop are created on it. */
+void* qm_talker_stream(qm_talker* engine);
+
+/* ---- final head (NativeFinalHead, R17:14145-14570) ----------------------------------------- */
+typedef struct qm_final_head qm_final_head;
+/*
+ * Uploads talker.codec_head.weight [3072][2048] and allocates the logits, the code history of
+ * `history_capacity` frames, the sampled code and the SplitMix64 generator state (set to `seed`; the
+ * predictor of the same loop draws from the same state, R17:13899).
+ */
+int32_t qm_final_head_create(const char* model_dir, int32_t history_capacity, uint64_t seed, void* hip_stream,
+                             qm_final_head** out);
+void qm_final_head_destroy(qm_final_head* head);
+/* A new request: history cleared, generator state set to `seed`. */
+int32_t qm_final_head_reset(qm_final_head* head, uint64_t seed);
+/*
+ * run_fast_device (R17:14427-14570): codec_head on the (already final-normed) hidden vector, then cast,
+ * repetition penalty over the history of the frames before `frame`, suppressed tokens, top-50 sampling at
+ * temperature 0.9 (arg-max if sampling == 0), history append, and the four-byte read-back with the stream
+ * synchronisation that is the loop's frame boundary.  QM_ERR_SLOT_RANGE beyond the history capacity.
+ */
+int32_t qm_final_head_run(qm_final_head* head, const uint16_t* hidden_device, int32_t frame, int32_t sampling,
+                          int32_t* code_out);
+uint64_t* qm_final_head_rng_state(qm_final_head* head);            /* device */
+const int32_t* qm_final_head_device_code(qm_final_head* head);      /* device: the code of the last run */
+
+/* ---- code predictor frame (PersistentPredictor, R17:12817-13901) ---------------------------- */
+typedef struct qm_predictor qm_predictor;
+/*
+ * PredictorWeights from the model's safetensors (R17:10620-10712): talker.code_predictor.
+ * small_to_mtp_projection.{weight,bias}, model.layers.N.*, model.norm.weight, lm_head.I.weight and
+ * model.codec_embedding.I.weight for I = 0..14, and the talker's codec embedding table
+ * talker.model.codec_embedding.weight; geometry of R17:7951-7964 (hidden 1024, 16/8 heads of 128,
+ * intermediate 3072, vocabulary 2048, 15 steps, 16 code groups).  rng_state_device: the generator state
+ * the samplers advance (qm_final_head_rng_state of the same loop).
+ */
+int32_t qm_predictor_create(const char* model_dir, uint64_t* rng_state_device, void* hip_stream, qm_predictor** out);
+void qm_predictor_destroy(qm_predictor* predictor);
+/*
+ * run_frame_device (R17:13043-13156) with the fifteen steps of capture_step (R17:13592-13854) enqueued
+ * directly: caches, selected embeddings and codes cleared; input rows = (talker hidden, embedding of
+ * code0); step 0 as the reference's two-row staged path, steps 1..14 with the M = 1 operators; then
+ * next talker input = bf16(bf16(sum of the 16 selected embeddings) + context).  context_host: [2048] bf16
+ * on the host.  Synchronises the stream and returns the frame's sixteen codes (codes_out[0] = code0).
+ */
+int32_t qm_predictor_run_frame(qm_predictor* predictor, const uint16_t* talker_hidden_device, const int32_t* code0_device,
+                               const uint16_t* context_host, int32_t sampling, int32_t codes_out[16]);
+const uint16_t* qm_predictor_next_input(qm_predictor* predictor);    /* device [2048] */
+
+/*
+ * The generation loop of generate_codec_sequence (R17:21887-22538) on a prompt whose embedding rows are
+ * already on the device: talker prefill; per frame the final head (stop on the end-of-sequence code 2150
+ * from frame 2 on), the predictor frame conditioned on trailing_text_host[frame] (rows of 2048, first
+ * trailing_rows frames) or tts_pad_host, and the talker's decode step on the predictor's next input at
+ * RoPE position prompt_rows + frame.  codes_out: [maximum_frames][16]; *frames_out: frames emitted;
+ * *hash_out (optional): qm_fnv1a64 of the emitted codes.  The three engines share the talker's stream
+ * (QM_ERR_ARGUMENT otherwise); the caller resets the final head between requests.
+ */
+int32_t qm_generate(qm_talker* talker, qm_final_head* head, qm_predictor* predictor, const uint16_t* prompt_device,
+                    int32_t prompt_rows, int32_t maximum_frames, const uint16_t* tts_pad_host,
+                    const uint16_t* trailing_text_host, int32_t trailing_rows, int32_t sampling, int32_t* codes_out,
+                    int32_t* frames_out, uint64_t* hash_out);
 
 #ifdef __cplusplus
 }

@@ -60,7 +60,7 @@ _SIGNATURES = {
     "qm_decode_attention_ragged_static": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _PTR, _I32,
                                                  _F32, _PTR, _PTR]),
     "qm_norm_rope_rows": (_I32, [_PTR] * 5 + [_I32, _I32, _F32, _PTR]),
-    "qm_scatter_kv": (_I32, [_PTR, _PTR, C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _PTR]),
+    "qm_scatter_kv": (_I32, [_PTR, _PTR, C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _PTR, _PTR]),
     "qm_prefill_attention_causal": (_I32, [_PTR] * 4 + [C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _I32, _I32,
                                            _F32, C.c_int64, C.c_int64, C.c_int64, _PTR, _PTR]),
     "qm_prefill_split_workspace_bytes": (C.c_int64, [_I32, _I32, _I32]),
@@ -88,6 +88,8 @@ _SIGNATURES = {
     "qm_final_head_process": (_I32, [_PTR, _PTR, _I32, _I32, _I32, _I32, _I32, _F32, _PTR, _PTR]),
     "qm_final_head_sample": (_I32, [_PTR, _PTR, _I32, _I32, _I32, _I32, _F32, _I32, _F32, _PTR, _PTR, _PTR, _PTR]),
     "qm_gather_embedding": (_I32, [_PTR, _I32, _PTR, _I32, _I32, _PTR, _PTR, _PTR]),
+    "qm_predictor_prepare_group0": (_I32, [_PTR, _I32, _PTR, _I32, _PTR, _PTR, _PTR, _PTR]),
+    "qm_predictor_next_talker_input": (_I32, [_PTR, _I32, _PTR, _I32, _PTR, _PTR, _PTR]),
     "qm_linear_rows": (_I32, [_PTR] * 5 + [_I32, _I32, _I32, _PTR]),
     "qm_gate_up_swiglu_rows": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _PTR]),
 }
@@ -208,9 +210,9 @@ def norm_rope_rows(x, norm_w, cos, sin, out, rows, heads, eps=1e-6, stream=0):
                                    heads, eps, stream), "qm_norm_rope_rows")
 
 
-def scatter_kv(key, value, cache, page_table, max_pages, rows, first_position, stream=0):
+def scatter_kv(key, value, cache, page_table, max_pages, rows, first_position, status=None, stream=0):
     _check(lib().qm_scatter_kv(_addr(key), _addr(value), C.byref(cache), _addr(page_table), max_pages,
-                               rows, first_position, stream), "qm_scatter_kv")
+                               rows, first_position, _addr(status), stream), "qm_scatter_kv")
 
 
 def prefill_attention_causal(query, key, value, out, cache, page_table, max_pages, batch, seq, q_heads,
@@ -383,3 +385,13 @@ def decode_attention_ragged_static(query, cache, page_table, max_pages, seq_lens
     _check(lib().qm_decode_attention_ragged_static(
         _addr(query), C.byref(cache), _addr(page_table), max_pages, _addr(seq_lens), n_streams,
         max_seq_len, _addr(out), q_heads, scale, _addr(status), stream), "qm_decode_attention_ragged_static")
+
+
+def predictor_prepare_group0(table, table_rows, code0, dimension, free_input, selected, codes, stream=0):
+    _check(lib().qm_predictor_prepare_group0(_addr(table), table_rows, _addr(code0), dimension, _addr(free_input),
+                                             _addr(selected), _addr(codes), stream), "qm_predictor_prepare_group0")
+
+
+def predictor_next_talker_input(selected, groups, context, dimension, embedding_sum, next_input, stream=0):
+    _check(lib().qm_predictor_next_talker_input(_addr(selected), groups, _addr(context), dimension, _addr(embedding_sum),
+                                                _addr(next_input), stream), "qm_predictor_next_talker_input")

@@ -46,7 +46,7 @@ def build(verbose=True, jobs=4):
     return LIB_PATH
 
 
-ENGINE_SOURCES = ["engine/qm_safetensors.cpp", "engine/qm_engine.cpp"]
+ENGINE_SOURCES = ["engine/qm_safetensors.cpp", "engine/qm_engine.cpp", "engine/qm_frame_engine.cpp"]
 
 
 def build_engine(verbose=True):

@@ -16,72 +16,9 @@
 #include <string>
 #include <vector>
 
-#include "../../../include/qm_attn.h"
-#include "qm_safetensors.hpp"
+#include "qm_engine_common.hpp"
 
 namespace qm_engine {
-
-constexpr int kHidden = 2048;          // R17:14625
-constexpr int kHeadDim = 128;          // kHeadDimRequired, R17:14629
-constexpr float kEpsilon = 1.0e-6f;    // kRmsEpsilon, R17:7965
-constexpr float kScale = 0.08838834764831845f;   // 1 / sqrt(128), R17:7966
-
-struct ApiError : std::runtime_error {
-    int32_t code;
-    ApiError(int32_t c, const std::string& what) : std::runtime_error(what), code(c) {}
-};
-
-thread_local std::string g_last_error;
-
-inline void hip_check(hipError_t e, const char* what) {
-    if (e != hipSuccess) throw ApiError(QM_ERR_HIP_BASE - static_cast<int32_t>(e), std::string(what) + ": " + hipGetErrorString(e));
-}
-inline void op_check(int32_t rc, const char* what) {
-    if (rc != QM_OK) throw ApiError(rc, std::string(what) + ": " + qm_error_string(rc));
-}
-
-// Owner of one device allocation (DeviceBuffer, R17:7968-8020).
-class DeviceBuffer {
-public:
-    DeviceBuffer() = default;
-    explicit DeviceBuffer(size_t bytes) : bytes_(bytes) {
-        if (bytes) hip_check(hipMalloc(&pointer_, bytes), "device allocation");
-    }
-    ~DeviceBuffer() {
-        if (pointer_) (void)hipFree(pointer_);
-    }
-    DeviceBuffer(DeviceBuffer&& o) noexcept : pointer_(o.pointer_), bytes_(o.bytes_) { o.pointer_ = nullptr; o.bytes_ = 0; }
-    DeviceBuffer& operator=(DeviceBuffer&& o) noexcept {
-        if (this != &o) {
-            if (pointer_) (void)hipFree(pointer_);
-            pointer_ = o.pointer_; bytes_ = o.bytes_;
-            o.pointer_ = nullptr; o.bytes_ = 0;
-        }
-        return *this;
-    }
-    DeviceBuffer(const DeviceBuffer&) = delete;
-    DeviceBuffer& operator=(const DeviceBuffer&) = delete;
-    uint16_t* u16() const { return static_cast<uint16_t*>(pointer_); }
-    void* raw() const { return pointer_; }
-    size_t bytes() const { return bytes_; }
-
-private:
-    void* pointer_ = nullptr;
-    size_t bytes_ = 0;
-};
-
-// A BF16 tensor on the device (GpuParam, R17:14639-14683); absent optional tensors give nullptr.
-struct Param {
-    DeviceBuffer buffer;
-    std::vector<int64_t> shape;
-    bool present = false;
-    Param() = default;
-    Param(const TensorView& t, hipStream_t upload) : buffer(static_cast<size_t>(t.elements()) * 2), shape(t.shape), present(true) {
-        if (t.dtype != "BF16") throw TensorError("expected BF16 tensor: " + t.name);
-        hip_check(hipMemcpyAsync(buffer.raw(), t.data, buffer.bytes(), hipMemcpyHostToDevice, upload), "weight upload");
-    }
-    const uint16_t* data() const { return present ? buffer.u16() : nullptr; }
-};
 
 struct Layer {
     Param input_norm, q_weight, q_bias, k_weight, k_bias, v_weight, v_bias, q_norm, k_norm, o_weight, o_bias, post_norm,
@@ -112,6 +49,8 @@ struct qm_talker {
         p_swiglu, p_cosine, p_sine;
     // the prompt pass's key-split workspace (prompts whose attention grid leaves compute units idle), grown on demand
     qm_engine::DeviceBuffer p_split;
+    // device status word the attention kernels OR their QM_STATUS_* bits into; read at qm_talker_synchronize
+    qm_engine::DeviceBuffer status;
 
     ~qm_talker() {
         if (own_stream && stream) (void)hipStreamDestroy(stream);
@@ -215,6 +154,8 @@ static std::unique_ptr<qm_talker> create_talker(const std::string& model_dir, in
     engine->swiglu = vec(engine->intermediate); engine->final_hidden = vec(kHidden);
     engine->cosine = vec(kHeadDim); engine->sine = vec(kHeadDim);
     engine->workspace = DeviceBuffer(qm_decode_workspace_bytes(1, engine->q_heads, engine->kv_heads, max_cache));
+    engine->status = DeviceBuffer(256);
+    hip_check(hipMemsetAsync(engine->status.raw(), 0, engine->status.bytes(), engine->stream), "status word reset");
     hip_check(hipStreamSynchronize(upload), "weight upload synchronize");   // the mapped files go away with `host`
     return engine;
 }
@@ -264,7 +205,8 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
         // launch_qk_norm_rope_cache_m1 + launch_attention (R17:17181-17195)
         op_check(qm_decode_step_fused(e.q.u16(), e.k.u16(), e.v.u16(), w.q_norm.data(), w.k_norm.data(), e.cosine.u16(),
                                       e.sine.u16(), e.q_rotated.u16(), &cache, nullptr, 1, e.context.u16(), e.q_heads,
-                                      position, -1, kScale, kEpsilon, e.workspace.raw(), e.workspace.bytes(), nullptr, s),
+                                      position, -1, kScale, kEpsilon, e.workspace.raw(), e.workspace.bytes(),
+                                      static_cast<uint32_t*>(e.status.raw()), s),
                  "talker norm/RoPE/append + attention");
         // launch_linear_m1: o_proj (R17:17203-17210)
         op_check(qm_linear_m1(e.context.u16(), w.o_weight.data(), w.o_bias.data(), nullptr, e.attention.u16(), kHidden,
@@ -343,7 +285,8 @@ static const uint16_t* prefill(qm_talker& e, const uint16_t* input_device, const
                                    e.kv_heads, kEpsilon, s), "prefill k norm + RoPE");
         op_check(qm_prefill_attention_causal_split(e.p_q_rotated.u16(), e.p_k_rotated.u16(), e.p_v.u16(), e.p_context.u16(),
                                                    &cache, nullptr, 1, 1, rows, e.q_heads, e.kv_heads, kScale, 0, 0, 0,
-                                                   split_bytes > 0 ? e.p_split.raw() : nullptr, split_bytes, nullptr, s),
+                                                   split_bytes > 0 ? e.p_split.raw() : nullptr, split_bytes,
+                                                   static_cast<uint32_t*>(e.status.raw()), s),
                  "prefill attention + cache write");
         op_check(qm_linear_rows(e.p_context.u16(), w.o_weight.data(), w.o_bias.data(), current->u16(), e.p_residual.u16(),
                                 rows, kHidden, e.q_dim, s), "prefill o_proj + residual");
@@ -360,32 +303,18 @@ static const uint16_t* prefill(qm_talker& e, const uint16_t* input_device, const
     return e.final_hidden.u16();
 }
 
-// Runs f, turning exceptions into codes.
-template <typename F>
-static int32_t guarded(F&& f) {
-    try {
-        f();
-        return QM_OK;
-    } catch (const ApiError& e) {
-        g_last_error = e.what();
-        return e.code;
-    } catch (const IoError& e) {
-        g_last_error = e.what();
-        return QM_ERR_IO;
-    } catch (const TensorError& e) {
-        g_last_error = e.what();
-        return QM_ERR_TENSOR;
-    } catch (const std::exception& e) {
-        g_last_error = e.what();
-        return QM_ERR_ARGUMENT;
-    }
-}
-
 }  // namespace qm_engine
 
 using namespace qm_engine;
 
-extern "C" const char* qm_engine_last_error(void) { return g_last_error.c_str(); }
+namespace qm_engine {
+std::string& last_error() {
+    thread_local std::string text;
+    return text;
+}
+}  // namespace qm_engine
+
+extern "C" const char* qm_engine_last_error(void) { return qm_engine::last_error().c_str(); }
 
 extern "C" uint64_t qm_fnv1a64(const void* data, size_t bytes) {
     const uint8_t* p = static_cast<const uint8_t*>(data);
@@ -491,7 +420,22 @@ extern "C" int32_t qm_talker_prefill(qm_talker* engine, const uint16_t* input_de
     return guarded([&] { *final_hidden_device = prefill(*engine, input_device, cosine, sine, rows); });
 }
 
+extern "C" void* qm_talker_stream(qm_talker* engine) { return engine ? engine->stream : nullptr; }
+
 extern "C" int32_t qm_talker_synchronize(qm_talker* engine) {
     if (!engine) return QM_ERR_NULL;
-    return guarded([&] { hip_check(hipStreamSynchronize(engine->stream), "generation stream synchronize"); });
+    return guarded([&] {
+        hip_check(hipStreamSynchronize(engine->stream), "generation stream synchronize");
+        // What the kernels flagged since the last synchronisation (a page or position out of range, a key-split
+        // block that gave up waiting for its partner): the results are not to be used.
+        uint32_t bits = 0;
+        hip_check(hipMemcpy(&bits, engine->status.raw(), sizeof bits, hipMemcpyDeviceToHost), "status word read");
+        if (bits != 0) {
+            hip_check(hipMemset(engine->status.raw(), 0, sizeof bits), "status word reset");
+            if ((bits & QM_STATUS_SPLIT_TIMEOUT) && engine->p_split.raw())
+                op_check(qm_prefill_split_workspace_init(engine->p_split.raw(), static_cast<int64_t>(engine->p_split.bytes()),
+                                                         engine->stream), "prefill key-split workspace init");
+            throw ApiError(QM_ERR_STATUS, "talker kernels reported status bits " + std::to_string(bits));
+        }
+    });
 }

@@ -1,0 +1,380 @@
+// qm_frame_engine.cpp — the per-frame generation loop of the engine shell: the final head (codec_head +
+// score processing + sampler + history), the code predictor's 15-step frame, and the loop that alternates
+// talker decode, final head and predictor frame and hashes the codec trajectory.
+//
+// Reference: NativeFinalHead::run_fast_device (R17:14427-14570), PredictorWeights (R17:10411-10712),
+// PersistentPredictor::run_frame_device (R17:13043-13156), capture_step (R17:13592-13854), capture_graph
+// (R17:13856-13896), generate_codec_sequence (R17:21887-22538).  Every device operation is a C-ABI operator of
+// libqm_attn on the talker's generation stream; the host reads back four bytes per frame after the final head
+// and sixty-four after the predictor, as the reference does.
+#include "qm_engine_common.hpp"
+
+#include <array>
+#include <memory>
+
+namespace qm_engine {
+
+constexpr int kOuter = kHidden;            // kOuterHidden, R17:7951: the talker's width
+constexpr int kPredHidden = 1024;          // kHidden, R17:7952
+constexpr int kPredIntermediate = 3072;    // R17:7953
+constexpr int kPredQueryHeads = 16;        // R17:7955
+constexpr int kPredKvHeads = 8;            // R17:7956
+constexpr int kPredQueryDim = kPredQueryHeads * kHeadDim;
+constexpr int kPredKvDim = kPredKvHeads * kHeadDim;
+constexpr int kPredVocab = 2048;           // R17:7960
+constexpr int kPredSteps = 15;             // R17:7961
+constexpr int kCodeGroups = 16;            // R17:7962
+constexpr int kPredMaxCache = 16;          // R17:7964
+constexpr int kHeadVocab = 3072;           // final head, R17:14444
+constexpr int kCodecEos = 2150;            // R17:13958-13961
+constexpr int kSuppressedTail = 1024;
+constexpr float kPenalty = 1.05f;
+constexpr int kTopK = 50;                  // kGpuSamplerTopK, R17:7338
+constexpr float kTemperature = 0.9f;       // kGpuSamplerTemperature, R17:7339
+
+static void expect_shape(const Param& p, std::vector<int64_t> shape, const std::string& what) {
+    if (p.shape != shape) throw TensorError("unexpected shape of " + what);
+}
+
+struct PredictorLayer {
+    Param input_norm, q_weight, k_weight, v_weight, q_norm, k_norm, o_weight, post_norm, gate_weight, up_weight, down_weight;
+    DeviceBuffer key_cache, value_cache;   // [8][16][128]
+};
+
+}  // namespace qm_engine
+
+using namespace qm_engine;
+
+struct qm_final_head {
+    Param weight;                          // talker.codec_head.weight [3072][2048]
+    DeviceBuffer logits, history, code, rng;
+    int capacity = 0;
+    hipStream_t stream = nullptr;
+};
+
+struct qm_predictor {
+    Param projection_weight, projection_bias, final_norm, codec0_table;
+    std::vector<PredictorLayer> layers;
+    std::vector<Param> heads, embeddings;
+    hipStream_t stream = nullptr;
+    uint64_t* rng_state = nullptr;         // device, shared with the final head
+    DeviceBuffer cosine, sine;             // [16][128], positions 0..15
+    DeviceBuffer free_input, context_embedding, hidden_a, hidden_b, norm, q_linear, k_linear, v_linear, q_normed, k_normed,
+        q_bhsd, k_bhsd, v_bhsd, q_rotated, k_rotated, context, attention, residual, post_norm, swiglu, logits,
+        selected, codes, embedding_sum, next_input;
+};
+
+namespace qm_engine {
+
+static std::unique_ptr<qm_final_head> create_final_head(const std::string& model_dir, int capacity, uint64_t seed,
+                                                        hipStream_t stream) {
+    if (capacity <= 0) throw ApiError(QM_ERR_ARGUMENT, "history capacity must be positive");
+    ModelDirectory host(model_dir);
+    auto head = std::make_unique<qm_final_head>();
+    head->stream = stream;
+    head->weight = Param(host.suffix("talker.codec_head.weight"), stream);
+    expect_shape(head->weight, {kHeadVocab, kHidden}, "talker.codec_head.weight");
+    head->logits = DeviceBuffer(kHeadVocab * 2);
+    head->history = DeviceBuffer(static_cast<size_t>(capacity) * sizeof(int32_t));
+    head->code = DeviceBuffer(sizeof(int32_t));
+    head->rng = DeviceBuffer(sizeof(uint64_t));
+    head->capacity = capacity;
+    hip_check(hipMemcpyAsync(head->rng.raw(), &seed, sizeof seed, hipMemcpyHostToDevice, stream), "generator seed upload");
+    hip_check(hipMemsetAsync(head->history.raw(), 0, head->history.bytes(), stream), "history reset");
+    hip_check(hipStreamSynchronize(stream), "final head upload synchronize");
+    return head;
+}
+
+// run_fast_device (R17:14427-14570): codec_head, then cast + repetition penalty + suppressed tokens + sampler (or
+// arg-max) + history append in one launch, then the four-byte read-back that is the frame boundary.
+static int32_t final_head_run(qm_final_head& h, const uint16_t* hidden_device, int frame, bool sampling) {
+    if (frame < 0 || frame >= h.capacity) throw ApiError(QM_ERR_SLOT_RANGE, "FinalHead generation index exceeds GPU history capacity");
+    op_check(qm_linear_m1(hidden_device, h.weight.data(), nullptr, nullptr, h.logits.u16(), kHeadVocab, kHidden, h.stream),
+             "final head projection");
+    op_check(qm_final_head_sample(h.logits.u16(), static_cast<int32_t*>(h.history.raw()), frame, kHeadVocab, kCodecEos,
+                                  kSuppressedTail, kPenalty, sampling ? kTopK : 0, kTemperature,
+                                  static_cast<uint64_t*>(h.rng.raw()), static_cast<int32_t*>(h.code.raw()), nullptr, h.stream),
+             "final head sampler");
+    int32_t code = 0;
+    hip_check(hipMemcpyAsync(&code, h.code.raw(), sizeof code, hipMemcpyDeviceToHost, h.stream), "code read-back");
+    hip_check(hipStreamSynchronize(h.stream), "frame boundary synchronize");
+    return code;
+}
+
+static std::unique_ptr<qm_predictor> create_predictor(const std::string& model_dir, uint64_t* rng_state, hipStream_t stream) {
+    if (!rng_state) throw ApiError(QM_ERR_NULL, "the predictor samples from the final head's generator state");
+    ModelDirectory host(model_dir);
+    auto p = std::make_unique<qm_predictor>();
+    p->stream = stream;
+    p->rng_state = rng_state;
+    const std::string root = "talker.code_predictor.";
+    p->projection_weight = Param(host.suffix(root + "small_to_mtp_projection.weight"), stream);
+    p->projection_bias = Param(host.suffix(root + "small_to_mtp_projection.bias"), stream);
+    expect_shape(p->projection_weight, {kPredHidden, kOuter}, "small_to_mtp_projection.weight");
+    expect_shape(p->projection_bias, {kPredHidden}, "small_to_mtp_projection.bias");
+    for (int index = 0;; ++index) {
+        const std::string lr = root + "model.layers." + std::to_string(index) + ".";
+        const TensorView* first = host.maybe_suffix(lr + "input_layernorm.weight");
+        if (!first) break;
+        PredictorLayer w;
+        w.input_norm = Param(*first, stream);
+        w.q_weight = Param(host.suffix(lr + "self_attn.q_proj.weight"), stream);
+        w.k_weight = Param(host.suffix(lr + "self_attn.k_proj.weight"), stream);
+        w.v_weight = Param(host.suffix(lr + "self_attn.v_proj.weight"), stream);
+        w.o_weight = Param(host.suffix(lr + "self_attn.o_proj.weight"), stream);
+        w.q_norm = Param(host.suffix(lr + "self_attn.q_norm.weight"), stream);
+        w.k_norm = Param(host.suffix(lr + "self_attn.k_norm.weight"), stream);
+        w.post_norm = Param(host.suffix(lr + "post_attention_layernorm.weight"), stream);
+        w.gate_weight = Param(host.suffix(lr + "mlp.gate_proj.weight"), stream);
+        w.up_weight = Param(host.suffix(lr + "mlp.up_proj.weight"), stream);
+        w.down_weight = Param(host.suffix(lr + "mlp.down_proj.weight"), stream);
+        expect_shape(w.input_norm, {kPredHidden}, lr + "input_layernorm.weight");
+        expect_shape(w.q_weight, {kPredQueryDim, kPredHidden}, lr + "self_attn.q_proj.weight");
+        expect_shape(w.k_weight, {kPredKvDim, kPredHidden}, lr + "self_attn.k_proj.weight");
+        expect_shape(w.v_weight, {kPredKvDim, kPredHidden}, lr + "self_attn.v_proj.weight");
+        expect_shape(w.o_weight, {kPredHidden, kPredQueryDim}, lr + "self_attn.o_proj.weight");
+        expect_shape(w.q_norm, {kHeadDim}, lr + "self_attn.q_norm.weight");
+        expect_shape(w.k_norm, {kHeadDim}, lr + "self_attn.k_norm.weight");
+        expect_shape(w.post_norm, {kPredHidden}, lr + "post_attention_layernorm.weight");
+        expect_shape(w.gate_weight, {kPredIntermediate, kPredHidden}, lr + "mlp.gate_proj.weight");
+        expect_shape(w.up_weight, {kPredIntermediate, kPredHidden}, lr + "mlp.up_proj.weight");
+        expect_shape(w.down_weight, {kPredHidden, kPredIntermediate}, lr + "mlp.down_proj.weight");
+        w.key_cache = DeviceBuffer(kPredKvHeads * kPredMaxCache * kHeadDim * 2);
+        w.value_cache = DeviceBuffer(kPredKvHeads * kPredMaxCache * kHeadDim * 2);
+        p->layers.push_back(std::move(w));
+    }
+    if (p->layers.empty()) throw TensorError("no code predictor layers in " + model_dir);
+    p->final_norm = Param(host.suffix(root + "model.norm.weight"), stream);
+    expect_shape(p->final_norm, {kPredHidden}, "code_predictor.model.norm.weight");
+    for (int index = 0; index < kPredSteps; ++index) {
+        p->heads.emplace_back(host.suffix(root + "lm_head." + std::to_string(index) + ".weight"), stream);
+        p->embeddings.emplace_back(host.suffix(root + "model.codec_embedding." + std::to_string(index) + ".weight"), stream);
+        expect_shape(p->heads.back(), {kPredVocab, kPredHidden}, "code_predictor.lm_head weight");
+        expect_shape(p->embeddings.back(), {kPredVocab, kOuter}, "code_predictor.model.codec_embedding weight");
+    }
+    p->codec0_table = Param(host.suffix("talker.model.codec_embedding.weight"), stream);
+    if (p->codec0_table.shape.size() != 2 || p->codec0_table.shape[1] != kOuter || p->codec0_table.shape[0] <= 0
+        || p->codec0_table.shape[0] > 0x7fffffff)
+        throw TensorError("unexpected shape of talker.model.codec_embedding.weight");
+
+    // RoPE rows of positions 0..15 (PersistentPredictor::make_rope, R17:13161-13197: the talker's table rule)
+    std::vector<uint16_t> cos_host(kPredMaxCache * kHeadDim), sin_host(kPredMaxCache * kHeadDim);
+    op_check(qm_rope_rows(kPredMaxCache, 0, kHeadDim, 1000000.0, cos_host.data(), sin_host.data()), "predictor rope rows");
+    p->cosine = DeviceBuffer(cos_host.size() * 2);
+    p->sine = DeviceBuffer(sin_host.size() * 2);
+    hip_check(hipMemcpyAsync(p->cosine.raw(), cos_host.data(), cos_host.size() * 2, hipMemcpyHostToDevice, stream), "rope upload");
+    hip_check(hipMemcpyAsync(p->sine.raw(), sin_host.data(), sin_host.size() * 2, hipMemcpyHostToDevice, stream), "rope upload");
+
+    auto rows2 = [](int width) { return DeviceBuffer(static_cast<size_t>(2) * width * 2); };
+    p->free_input = rows2(kOuter); p->context_embedding = DeviceBuffer(kOuter * 2);
+    p->hidden_a = rows2(kPredHidden); p->hidden_b = rows2(kPredHidden); p->norm = rows2(kPredHidden);
+    p->q_linear = rows2(kPredQueryDim); p->k_linear = rows2(kPredKvDim); p->v_linear = rows2(kPredKvDim);
+    p->q_normed = rows2(kPredQueryDim); p->k_normed = rows2(kPredKvDim);
+    p->q_bhsd = rows2(kPredQueryDim); p->k_bhsd = rows2(kPredKvDim); p->v_bhsd = rows2(kPredKvDim);
+    p->q_rotated = rows2(kPredQueryDim); p->k_rotated = rows2(kPredKvDim); p->context = rows2(kPredQueryDim);
+    p->attention = rows2(kPredHidden); p->residual = rows2(kPredHidden); p->post_norm = rows2(kPredHidden);
+    p->swiglu = rows2(kPredIntermediate); p->logits = rows2(kPredVocab);
+    p->selected = DeviceBuffer(static_cast<size_t>(kCodeGroups) * kOuter * 2);
+    p->codes = DeviceBuffer(kCodeGroups * sizeof(int32_t));
+    p->embedding_sum = DeviceBuffer(kOuter * 2); p->next_input = DeviceBuffer(kOuter * 2);
+    hip_check(hipStreamSynchronize(stream), "predictor upload synchronize");   // the mapped files go away with `host`
+    return p;
+}
+
+// Step 0 of capture_step (R17:13597-13854 with rows = 2): the two-row "staged" path — generic linears in the
+// talker linear's order, per-head RMSNorm over rows * heads vectors, BHSD transpose / RoPE / cache update and the
+// staged causal attention.  o_proj + add and down_proj + add are one launch each (the residual is folded in), gate,
+// up and SwiGLU one.
+static void predictor_step0(qm_predictor& p, bool sampling) {
+    hipStream_t s = p.stream;
+    const int rows = 2;
+    op_check(qm_linear_rows(p.free_input.u16(), p.projection_weight.data(), p.projection_bias.data(), nullptr, p.hidden_a.u16(),
+                            rows, kPredHidden, kOuter, s), "predictor input projection");
+    DeviceBuffer* current = &p.hidden_a;
+    DeviceBuffer* next = &p.hidden_b;
+    for (PredictorLayer& w : p.layers) {
+        op_check(qm_rmsnorm_rows(current->u16(), w.input_norm.data(), p.norm.u16(), rows, kPredHidden, kEpsilon, s), "predictor rmsnorm");
+        op_check(qm_linear_rows(p.norm.u16(), w.q_weight.data(), nullptr, nullptr, p.q_linear.u16(), rows, kPredQueryDim, kPredHidden, s), "predictor q_proj");
+        op_check(qm_linear_rows(p.norm.u16(), w.k_weight.data(), nullptr, nullptr, p.k_linear.u16(), rows, kPredKvDim, kPredHidden, s), "predictor k_proj");
+        op_check(qm_linear_rows(p.norm.u16(), w.v_weight.data(), nullptr, nullptr, p.v_linear.u16(), rows, kPredKvDim, kPredHidden, s), "predictor v_proj");
+        op_check(qm_rmsnorm_rows(p.q_linear.u16(), w.q_norm.data(), p.q_normed.u16(), rows * kPredQueryHeads, kHeadDim, kEpsilon, s), "predictor q_norm");
+        op_check(qm_rmsnorm_rows(p.k_linear.u16(), w.k_norm.data(), p.k_normed.u16(), rows * kPredKvHeads, kHeadDim, kEpsilon, s), "predictor k_norm");
+        op_check(qm_predictor_transpose(p.q_normed.u16(), p.q_bhsd.u16(), rows, kPredQueryHeads, s), "predictor transpose");
+        op_check(qm_predictor_transpose(p.k_normed.u16(), p.k_bhsd.u16(), rows, kPredKvHeads, s), "predictor transpose");
+        op_check(qm_predictor_transpose(p.v_linear.u16(), p.v_bhsd.u16(), rows, kPredKvHeads, s), "predictor transpose");
+        op_check(qm_predictor_rope_bhsd(p.q_bhsd.u16(), p.cosine.u16(), p.sine.u16(), p.q_rotated.u16(), rows, kPredQueryHeads, s), "predictor rope");
+        op_check(qm_predictor_rope_bhsd(p.k_bhsd.u16(), p.cosine.u16(), p.sine.u16(), p.k_rotated.u16(), rows, kPredKvHeads, s), "predictor rope");
+        op_check(qm_predictor_update_cache(p.k_rotated.u16(), w.key_cache.u16(), rows, 0, s), "predictor update_cache");
+        op_check(qm_predictor_update_cache(p.v_bhsd.u16(), w.value_cache.u16(), rows, 0, s), "predictor update_cache");
+        op_check(qm_predictor_attention_staged(p.q_rotated.u16(), w.key_cache.u16(), w.value_cache.u16(), p.context.u16(), rows, 2, 1, s),
+                 "predictor attention");
+        op_check(qm_linear_rows(p.context.u16(), w.o_weight.data(), nullptr, current->u16(), p.residual.u16(), rows, kPredHidden,
+                                kPredQueryDim, s), "predictor o_proj");
+        op_check(qm_rmsnorm_rows(p.residual.u16(), w.post_norm.data(), p.post_norm.u16(), rows, kPredHidden, kEpsilon, s), "predictor post norm");
+        op_check(qm_gate_up_swiglu_rows(p.post_norm.u16(), w.gate_weight.data(), w.up_weight.data(), p.swiglu.u16(), rows, kPredHidden,
+                                        kPredIntermediate, s), "predictor gate/up");
+        op_check(qm_linear_rows(p.swiglu.u16(), w.down_weight.data(), nullptr, p.residual.u16(), next->u16(), rows, kPredHidden,
+                                kPredIntermediate, s), "predictor down_proj");
+        std::swap(current, next);
+    }
+    op_check(qm_rmsnorm_rows(current->u16(), p.final_norm.data(), p.norm.u16(), rows, kPredHidden, kEpsilon, s), "predictor final norm");
+    op_check(qm_linear_rows(p.norm.u16(), p.heads[0].data(), nullptr, nullptr, p.logits.u16(), rows, kPredVocab, kPredHidden, s), "predictor head");
+    int32_t* codes = static_cast<int32_t*>(p.codes.raw());
+    op_check(qm_sample_topk(p.logits.u16(), 1, (rows - 1) * kPredVocab, kPredVocab, sampling ? kTopK : 0, kTemperature, p.rng_state,
+                            codes + 1, s), "predictor sampler");
+    op_check(qm_gather_embedding(p.embeddings[0].data(), kPredVocab, codes, 1, kOuter, p.selected.u16(), p.free_input.u16(), s),
+             "predictor embedding gather");
+}
+
+// Steps 1..14 of capture_step (rows = 1): the M = 1 operators in the predictor's own summation order; the attention
+// over at most 16 keys is the exact-chain kernel (the reference's attention_m1 arithmetic).
+static void predictor_step_m1(qm_predictor& p, int step, bool sampling) {
+    hipStream_t s = p.stream;
+    const int position = step + 1;                     // cache_before, R17:13594-13595
+    const uint16_t* cos_row = p.cosine.u16() + position * kHeadDim;
+    const uint16_t* sin_row = p.sine.u16() + position * kHeadDim;
+    op_check(qm_linear_m1(p.free_input.u16(), p.projection_weight.data(), p.projection_bias.data(), nullptr, p.hidden_a.u16(),
+                          kPredHidden, kOuter, s), "predictor input projection");
+    DeviceBuffer* current = &p.hidden_a;
+    DeviceBuffer* next = &p.hidden_b;
+    for (PredictorLayer& w : p.layers) {
+        qm_kv_cache cache = {};
+        cache.k_pool = w.key_cache.u16(); cache.v_pool = w.value_cache.u16();
+        cache.stride_page = 0; cache.stride_head = kPredMaxCache * kHeadDim; cache.stride_token = kHeadDim;
+        cache.page_size = kPredMaxCache; cache.n_pages = 1; cache.kv_heads = kPredKvHeads; cache.head_dim = kHeadDim;
+        op_check(qm_predictor_rmsnorm_qkv_m1(current->u16(), w.input_norm.data(), kEpsilon, w.q_weight.data(), w.k_weight.data(),
+                                             w.v_weight.data(), p.q_linear.u16(), p.k_linear.u16(), p.v_linear.u16(), kPredHidden,
+                                             kPredQueryDim, kPredKvDim, s), "predictor qkv_m1");
+        op_check(qm_qk_norm_rope_kv_append(p.q_linear.u16(), p.k_linear.u16(), p.v_linear.u16(), w.q_norm.data(), w.k_norm.data(), cos_row,
+                                           sin_row, p.q_rotated.u16(), &cache, nullptr, 1, kPredQueryHeads, position, kEpsilon, s),
+                 "predictor qk_norm_rope_cache_m1");
+        op_check(qm_predictor_attention_staged(p.q_rotated.u16(), w.key_cache.u16(), w.value_cache.u16(), p.context.u16(), 1,
+                                               position + 1, 0, s), "predictor attention_m1");
+        op_check(qm_predictor_linear_m1(p.context.u16(), w.o_weight.data(), nullptr, p.attention.u16(), kPredHidden, kPredQueryDim, s),
+                 "predictor o_proj");
+        op_check(qm_predictor_add_postnorm_gate_up_swiglu_m1(current->u16(), p.attention.u16(), w.post_norm.data(), kEpsilon,
+                                                             p.residual.u16(), w.gate_weight.data(), w.up_weight.data(), p.swiglu.u16(),
+                                                             kPredHidden, kPredIntermediate, s), "predictor gate/up");
+        op_check(qm_predictor_linear_m1(p.swiglu.u16(), w.down_weight.data(), p.residual.u16(), next->u16(), kPredHidden,
+                                        kPredIntermediate, s), "predictor down_proj");
+        std::swap(current, next);
+    }
+    // final RMSNorm + this step's head in the talker linear's order, no bias: the fused norm + Q/K/V entry with no K/V rows
+    const uint16_t* head = p.heads[static_cast<size_t>(step)].data();
+    op_check(qm_rmsnorm_qkv_m1(current->u16(), p.final_norm.data(), kEpsilon, head, nullptr, head, nullptr, head, nullptr, p.logits.u16(),
+                               p.logits.u16(), p.logits.u16(), kPredHidden, kPredVocab, 0, s), "predictor head");
+    int32_t* codes = static_cast<int32_t*>(p.codes.raw());
+    op_check(qm_sample_topk(p.logits.u16(), 1, 0, kPredVocab, sampling ? kTopK : 0, kTemperature, p.rng_state, codes + step + 1, s),
+             "predictor sampler");
+    op_check(qm_gather_embedding(p.embeddings[static_cast<size_t>(step)].data(), kPredVocab, codes, step + 1, kOuter, p.selected.u16(),
+                                 p.free_input.u16(), s), "predictor embedding gather");
+}
+
+// run_frame_device (R17:13043-13156): reset of the caches and of the frame's selected embeddings and codes, the
+// two input rows, the fifteen steps, the next talker input, and the 64-byte read-back of the frame's sixteen codes.
+static void predictor_frame(qm_predictor& p, const uint16_t* talker_hidden_device, const int32_t* code0_device,
+                            const uint16_t* context_host, bool sampling, int32_t codes_out[16]) {
+    if (!talker_hidden_device || !code0_device || !context_host || !codes_out) throw ApiError(QM_ERR_NULL, "predictor frame input is null");
+    hipStream_t s = p.stream;
+    for (PredictorLayer& w : p.layers) {
+        hip_check(hipMemsetAsync(w.key_cache.raw(), 0, w.key_cache.bytes(), s), "predictor key cache reset");
+        hip_check(hipMemsetAsync(w.value_cache.raw(), 0, w.value_cache.bytes(), s), "predictor value cache reset");
+    }
+    hip_check(hipMemsetAsync(p.selected.raw(), 0, p.selected.bytes(), s), "selected embeddings reset");
+    hip_check(hipMemsetAsync(p.codes.raw(), 0, p.codes.bytes(), s), "generated codes reset");
+    hip_check(hipMemcpyAsync(p.free_input.raw(), talker_hidden_device, kOuter * 2, hipMemcpyDeviceToDevice, s), "talker hidden copy");
+    hip_check(hipMemcpyAsync(p.context_embedding.raw(), context_host, kOuter * 2, hipMemcpyHostToDevice, s), "context embedding upload");
+    op_check(qm_predictor_prepare_group0(p.codec0_table.data(), static_cast<int32_t>(p.codec0_table.shape[0]), code0_device, kOuter,
+                                         p.free_input.u16(), p.selected.u16(), static_cast<int32_t*>(p.codes.raw()), s),
+             "predictor group 0 input");
+    predictor_step0(p, sampling);
+    for (int step = 1; step < kPredSteps; ++step) predictor_step_m1(p, step, sampling);
+    op_check(qm_predictor_next_talker_input(p.selected.u16(), kCodeGroups, p.context_embedding.u16(), kOuter, p.embedding_sum.u16(),
+                                            p.next_input.u16(), s), "next talker input");
+    hip_check(hipMemcpyAsync(codes_out, p.codes.raw(), kCodeGroups * sizeof(int32_t), hipMemcpyDeviceToHost, s), "codes read-back");
+    hip_check(hipStreamSynchronize(s), "predictor frame synchronize");
+}
+
+}  // namespace qm_engine
+
+extern "C" int32_t qm_final_head_create(const char* model_dir, int32_t history_capacity, uint64_t seed, void* hip_stream,
+                                        qm_final_head** out) {
+    if (!model_dir || !out) return QM_ERR_NULL;
+    *out = nullptr;
+    return guarded([&] { *out = create_final_head(model_dir, history_capacity, seed, static_cast<hipStream_t>(hip_stream)).release(); });
+}
+
+extern "C" void qm_final_head_destroy(qm_final_head* head) { delete head; }
+
+extern "C" int32_t qm_final_head_reset(qm_final_head* head, uint64_t seed) {
+    if (!head) return QM_ERR_NULL;
+    return guarded([&] {
+        hip_check(hipMemcpyAsync(head->rng.raw(), &seed, sizeof seed, hipMemcpyHostToDevice, head->stream), "generator seed upload");
+        hip_check(hipMemsetAsync(head->history.raw(), 0, head->history.bytes(), head->stream), "history reset");
+        hip_check(hipStreamSynchronize(head->stream), "final head reset synchronize");   // `seed` is a stack variable
+    });
+}
+
+extern "C" int32_t qm_final_head_run(qm_final_head* head, const uint16_t* hidden_device, int32_t frame, int32_t sampling,
+                                     int32_t* code_out) {
+    if (!head || !hidden_device || !code_out) return QM_ERR_NULL;
+    return guarded([&] { *code_out = final_head_run(*head, hidden_device, frame, sampling != 0); });
+}
+
+extern "C" uint64_t* qm_final_head_rng_state(qm_final_head* head) { return head ? static_cast<uint64_t*>(head->rng.raw()) : nullptr; }
+extern "C" const int32_t* qm_final_head_device_code(qm_final_head* head) { return head ? static_cast<const int32_t*>(head->code.raw()) : nullptr; }
+
+extern "C" int32_t qm_predictor_create(const char* model_dir, uint64_t* rng_state_device, void* hip_stream, qm_predictor** out) {
+    if (!model_dir || !out) return QM_ERR_NULL;
+    *out = nullptr;
+    return guarded([&] { *out = create_predictor(model_dir, rng_state_device, static_cast<hipStream_t>(hip_stream)).release(); });
+}
+
+extern "C" void qm_predictor_destroy(qm_predictor* predictor) { delete predictor; }
+
+extern "C" int32_t qm_predictor_run_frame(qm_predictor* predictor, const uint16_t* talker_hidden_device, const int32_t* code0_device,
+                                          const uint16_t* context_host, int32_t sampling, int32_t codes_out[16]) {
+    if (!predictor) return QM_ERR_NULL;
+    return guarded([&] { predictor_frame(*predictor, talker_hidden_device, code0_device, context_host, sampling != 0, codes_out); });
+}
+
+extern "C" const uint16_t* qm_predictor_next_input(qm_predictor* predictor) { return predictor ? predictor->next_input.u16() : nullptr; }
+
+extern "C" int32_t qm_generate(qm_talker* talker, qm_final_head* head, qm_predictor* predictor, const uint16_t* prompt_device,
+                               int32_t prompt_rows, int32_t maximum_frames, const uint16_t* tts_pad_host,
+                               const uint16_t* trailing_text_host, int32_t trailing_rows, int32_t sampling, int32_t* codes_out,
+                               int32_t* frames_out, uint64_t* hash_out) {
+    if (!talker || !head || !predictor || !prompt_device || !tts_pad_host || !codes_out || !frames_out) return QM_ERR_NULL;
+    if (prompt_rows <= 0 || maximum_frames <= 0 || trailing_rows < 0 || (trailing_rows > 0 && !trailing_text_host)) return QM_ERR_ARGUMENT;
+    *frames_out = 0;
+    if (head->stream != qm_talker_stream(talker) || predictor->stream != qm_talker_stream(talker)) return QM_ERR_ARGUMENT;
+    return guarded([&] {
+        // prompt pass (generate_codec_sequence, R17:21887-22538, prefill side): RoPE rows of positions 0..rows-1
+        std::vector<uint16_t> cosine(static_cast<size_t>(prompt_rows) * kHeadDim), sine(cosine.size());
+        op_check(qm_rope_rows(prompt_rows, 0, kHeadDim, 1000000.0, cosine.data(), sine.data()), "prompt rope rows");
+        const uint16_t* hidden = nullptr;
+        op_check(qm_talker_prefill(talker, prompt_device, cosine.data(), sine.data(), prompt_rows, &hidden), "talker prefill");
+        op_check(qm_talker_synchronize(talker), "talker prefill synchronize");     // the rope rows are stack-owned
+        // decode rope rows of positions prompt_rows .. (R17:21762)
+        const int decode_rows = maximum_frames > 1 ? maximum_frames - 1 : 0;
+        std::vector<uint16_t> decode_cos(static_cast<size_t>(decode_rows) * kHeadDim), decode_sin(decode_cos.size());
+        if (decode_rows > 0)
+            op_check(qm_rope_rows(decode_rows, prompt_rows, kHeadDim, 1000000.0, decode_cos.data(), decode_sin.data()), "decode rope rows");
+        int frames = 0;
+        for (int frame = 0; frame < maximum_frames; ++frame) {
+            const int32_t code0 = final_head_run(*head, hidden, frame, sampling != 0);
+            if (code0 == kCodecEos && frame >= 2) break;                           // R17:22222-22232
+            const uint16_t* context = frame < trailing_rows ? trailing_text_host + static_cast<size_t>(frame) * kOuter : tts_pad_host;
+            int32_t* codes = codes_out + static_cast<size_t>(frame) * kCodeGroups;
+            predictor_frame(*predictor, hidden, static_cast<const int32_t*>(head->code.raw()), context, sampling != 0, codes);
+            if (codes[0] != code0) throw ApiError(QM_ERR_ARGUMENT, "native Predictor recurrence output mismatch");
+            ++frames;
+            if (frame + 1 >= maximum_frames) break;
+            op_check(qm_talker_decode(talker, predictor->next_input.u16(), decode_cos.data() + static_cast<size_t>(frame) * kHeadDim,
+                                      decode_sin.data() + static_cast<size_t>(frame) * kHeadDim, frame, &hidden), "talker decode");
+        }
+        op_check(qm_talker_synchronize(talker), "generation synchronize");
+        *frames_out = frames;
+        if (hash_out) *hash_out = qm_fnv1a64(codes_out, static_cast<size_t>(frames) * kCodeGroups * sizeof(int32_t));
+    });
+}

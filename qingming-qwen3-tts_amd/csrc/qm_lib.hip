@@ -4,7 +4,7 @@
 
 #include <atomic>
 
-extern "C" int32_t qm_abi_version(void) { return 1; }
+extern "C" int32_t qm_abi_version(void) { return 2; }
 
 extern "C" const char* qm_target_arch(void) { return "gfx950"; }
 
@@ -17,6 +17,7 @@ extern "C" const char* qm_error_string(int32_t code) {
         case QM_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
         case QM_ERR_ARGUMENT: return "invalid argument";
         case QM_ERR_NO_DEVICE: return "no usable gfx950 device";
+        case QM_ERR_STATUS: return "a kernel reported a status bit (bad page, bad position or key-split timeout)";
         default: break;
     }
     if (code <= QM_ERR_HIP_BASE) return hipGetErrorString(static_cast<hipError_t>(QM_ERR_HIP_BASE - code));

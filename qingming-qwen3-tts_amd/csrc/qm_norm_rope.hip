@@ -90,7 +90,7 @@ __global__ __launch_bounds__(256) void norm_rope_rows_kernel(
 __global__ __launch_bounds__(256) void scatter_kv_kernel(
     const uint16_t* __restrict__ key, const uint16_t* __restrict__ value,
     qm_kv_cache cache, const int32_t* __restrict__ page_table, int max_pages,
-    int64_t total_chunks, int first_position) {
+    int64_t total_chunks, int first_position, uint32_t* status) {
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (idx >= total_chunks) return;
     const int chunk = static_cast<int>(idx & 15);
@@ -99,7 +99,10 @@ __global__ __launch_bounds__(256) void scatter_kv_kernel(
     const int token = first_position + static_cast<int>(t / cache.kv_heads);
     const int page = token / cache.page_size;
     const int phys = page_table ? page_table[page] : page;
-    if (phys < 0 || phys >= cache.n_pages) return;  // validated on the host for NULL tables
+    if (phys < 0 || phys >= cache.n_pages) {        // (validated on the host for NULL tables)
+        if (status && chunk == 0) atomicOr(status, QM_STATUS_BAD_PAGE);
+        return;
+    }
     const int64_t dst = static_cast<int64_t>(phys) * cache.stride_page
                       + static_cast<int64_t>(head) * cache.stride_head
                       + static_cast<int64_t>(token - page * cache.page_size) * kDim + chunk * 8;
@@ -177,7 +180,7 @@ extern "C" int32_t qm_norm_rope_rows(
 extern "C" int32_t qm_scatter_kv(
     const uint16_t* key, const uint16_t* value,
     const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
-    int32_t rows, int32_t first_position, void* hip_stream) {
+    int32_t rows, int32_t first_position, uint32_t* status_dev, void* hip_stream) {
     if (!key || !value) return QM_ERR_NULL;
     int32_t rc = qm::check_cache(cache, max_pages);
     if (rc != QM_OK) return rc;
@@ -195,6 +198,6 @@ extern "C" int32_t qm_scatter_kv(
     if (blocks > 0x7fffffffLL) return QM_ERR_ARGUMENT;
     hipLaunchKernelGGL(qm::scatter_kv_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
                        static_cast<hipStream_t>(hip_stream),
-                       key, value, *cache, page_table, max_pages, chunks, first_position);
+                       key, value, *cache, page_table, max_pages, chunks, first_position, status_dev);
     return qm::launch_status();
 }

@@ -87,7 +87,8 @@ struct PrefillParams {
     int split_chunk;             // 0: no query tile is split
     int split_slots;             // query tiles per pair that are split (the last ones)
     float* split_partials;       // [pair][split query tile][part][kSplitRecordFloats]
-    int* split_tickets;          // [pair][split query tile][8]: arrivals, record of part p published; zero between launches
+    int* split_tickets;          // [pair][split query tile][8]: (epoch << 4 | arrivals), then per part the epoch of its published record
+    int split_epoch;             // 1 .. 2^27 - 1, another value for every launch that splits
     float scale;
 };
 
@@ -1690,7 +1691,19 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         float* records = prm.split_partials + slot * kSplitMaxParts * kSplitRecordFloats + tid;
         int* tickets = prm.split_tickets + slot * kSplitTicketInts;
         int* note = reinterpret_cast<int*>(il_smem);
-        if (tid == 0) note[0] = __hip_atomic_fetch_add(&tickets[0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) {
+            // The ticket word is (epoch << 4) | arrivals of this launch: a word left by another launch (or by one
+            // that gave up waiting) counts as no arrivals, so nothing has to be reset and nothing stale is believed.
+            int seen = __hip_atomic_load(&tickets[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (;;) {
+                const int base = (seen >> 4) == prm.split_epoch ? seen : (prm.split_epoch << 4);
+                if (__hip_atomic_compare_exchange_strong(&tickets[0], &seen, base + 1, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                         __HIP_MEMORY_SCOPE_AGENT)) {
+                    note[0] = base & 15;
+                    break;
+                }
+            }
+        }
         __syncthreads();
         if (note[0] < parts - 1) {
             float* record = records + part * kSplitRecordFloats;
@@ -1703,7 +1716,9 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
             __hip_atomic_store(record + 65 * kPfThreads, l_run[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             wait_vm<0>();                            // the stores have been acknowledged
             __syncthreads();
-            if (tid == 0) __hip_atomic_store(&tickets[1 + part], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // (every store of the record is an agent-scope atomic store that has been acknowledged, for every
+            // wave of the block, before the flag is stored; the flag carries the launch's epoch)
+            if (tid == 0) __hip_atomic_store(&tickets[1 + part], prm.split_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
             return;
         }
         if (tid == 0) {
@@ -1711,13 +1726,18 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
             unsigned spins = 0;
             for (int p = 0; p < parts; ++p) {
                 if (p == part) continue;
-                while (__hip_atomic_load(&tickets[1 + p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0 && spins < kSplitSpinLimit) {
+                while (__hip_atomic_load(&tickets[1 + p], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) != prm.split_epoch
+                       && spins < kSplitSpinLimit) {
                     __builtin_amdgcn_s_sleep(2);
                     ++spins;
                 }
             }
             note[1] = spins < kSplitSpinLimit ? 1 : 0;
-            for (int i = 0; i <= parts; ++i)         // as found, for the next launch
+            // Back to zero: a captured launch is replayed with the epoch it was captured with and must find no
+            // arrivals of its own number.  (After a wait that gave up a late flag may survive this; launches
+            // with another epoch ignore it, a replay of the same captured launch needs the workspace
+            // initialised again, which is what QM_STATUS_SPLIT_TIMEOUT asks for.)
+            for (int i = 0; i <= parts; ++i)
                 __hip_atomic_store(&tickets[i], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         __syncthreads();
@@ -1974,7 +1994,7 @@ static int32_t prefill_attention_entry(
     prm.kv_stride_token = kv_stride_token; prm.kv_stride_head = kv_stride_head; prm.kv_stride_batch = kv_stride_batch;
     prm.batch = batch; prm.seq = seq; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
     prm.heavy_groups = n_qtiles;
-    prm.split_chunk = 0; prm.split_slots = 0; prm.split_partials = nullptr; prm.split_tickets = nullptr;
+    prm.split_chunk = 0; prm.split_slots = 0; prm.split_partials = nullptr; prm.split_tickets = nullptr; prm.split_epoch = 0;
 
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     const bool round_scores = option_value(QM_OPT_PREFILL_SCORE_ROUNDING) != 0;
@@ -1994,6 +2014,8 @@ static int32_t prefill_attention_entry(
         const SplitPlan split = groups == 1 && workspace ? plan_split(pairs, seq, compute_units) : SplitPlan();
         if (split.chunk > 0) {
             if (workspace_bytes < split.bytes) return QM_ERR_WORKSPACE;
+            static std::atomic<uint32_t> launches{0};
+            prm.split_epoch = static_cast<int>(launches.fetch_add(1, std::memory_order_relaxed) % 0x7FFFFFEu) + 1;
             prm.split_chunk = split.chunk;
             prm.split_slots = split.slots;
             prm.split_tickets = static_cast<int*>(workspace);

@@ -320,6 +320,39 @@ __global__ void gather_embedding_kernel(const uint16_t* table, int table_rows, c
     next_input[d] = value;
 }
 
+// prepare_group0_input_kernel (R17:11963-11996): the talker's code of the frame selects a row of the talker's
+// codec embedding table: it is the frame's first selected embedding, the second row of the predictor's two-row
+// input (the first is the talker's hidden vector) and the frame's first code.  A code outside the table
+// stores code 0 and moves nothing, as the reference does.
+__global__ void prepare_group0_kernel(const uint16_t* table, int table_rows, const int32_t* code0, int dimension,
+                                      uint16_t* free_input, uint16_t* selected, int32_t* codes) {
+    const int d = static_cast<int>(blockIdx.x) * static_cast<int>(blockDim.x) + static_cast<int>(threadIdx.x);
+    const int token = code0[0];
+    if (token < 0 || token >= table_rows) {
+        if (d == 0) codes[0] = 0;
+        return;
+    }
+    if (d < dimension) {
+        const uint16_t value = table[static_cast<int64_t>(token) * dimension + d];
+        selected[d] = value;
+        free_input[dimension + d] = value;
+    }
+    if (d == 0) codes[0] = token;
+}
+
+// sum_codec_embeddings_kernel (R17:8877-8906) followed by add (R17:8729-8744) with the context embedding:
+// sum = bf16(e_0 + e_1 + ... in fp32, in group order), next = bf16(sum + context).
+__global__ void next_talker_input_kernel(const uint16_t* selected, int groups, const uint16_t* context, int dimension,
+                                         uint16_t* sum_out, uint16_t* next_out) {
+    const int d = static_cast<int>(blockIdx.x) * static_cast<int>(blockDim.x) + static_cast<int>(threadIdx.x);
+    if (d >= dimension) return;
+    float accumulation = 0.0f;
+    for (int group = 0; group < groups; ++group) accumulation += bf2f(selected[static_cast<int64_t>(group) * dimension + d]);
+    const uint16_t sum = f2bf(accumulation);
+    if (sum_out) sum_out[d] = sum;
+    next_out[d] = f2bf(bf2f(sum) + bf2f(context[d]));
+}
+
 inline int32_t launch_sampler(const SamplerParams& prm, void* hip_stream) {
     if (prm.vocab <= 0 || prm.offset < 0) return QM_ERR_ARGUMENT;
     if (prm.vocab > kSmpMaxVocab || prm.top_k > kSmpMaxKeep) return QM_ERR_GEOMETRY;
@@ -388,5 +421,27 @@ extern "C" int32_t qm_gather_embedding(const uint16_t* table, int32_t table_rows
     hipLaunchKernelGGL(qm::gather_embedding_kernel, dim3(static_cast<unsigned>((dimension + 255) / 256)), dim3(256), 0,
                        static_cast<hipStream_t>(hip_stream), table, table_rows, codes, group, dimension,
                        selected_embeddings, next_step_input);
+    return qm::launch_status();
+}
+
+extern "C" int32_t qm_predictor_prepare_group0(const uint16_t* codec_table, int32_t table_rows, const int32_t* code0,
+                                               int32_t dimension, uint16_t* free_input, uint16_t* selected_embeddings,
+                                               int32_t* generated_codes, void* hip_stream) {
+    if (!codec_table || !code0 || !free_input || !selected_embeddings || !generated_codes) return QM_ERR_NULL;
+    if (table_rows <= 0 || dimension <= 0) return QM_ERR_ARGUMENT;
+    hipLaunchKernelGGL(qm::prepare_group0_kernel, dim3(static_cast<unsigned>((dimension + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(hip_stream), codec_table, table_rows, code0, dimension, free_input,
+                       selected_embeddings, generated_codes);
+    return qm::launch_status();
+}
+
+extern "C" int32_t qm_predictor_next_talker_input(const uint16_t* selected_embeddings, int32_t groups,
+                                                  const uint16_t* context_embedding, int32_t dimension,
+                                                  uint16_t* embedding_sum, uint16_t* next_talker_input, void* hip_stream) {
+    if (!selected_embeddings || !context_embedding || !next_talker_input) return QM_ERR_NULL;
+    if (groups <= 0 || dimension <= 0) return QM_ERR_ARGUMENT;
+    hipLaunchKernelGGL(qm::next_talker_input_kernel, dim3(static_cast<unsigned>((dimension + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(hip_stream), selected_embeddings, groups, context_embedding, dimension,
+                       embedding_sum, next_talker_input);
     return qm::launch_status();
 }

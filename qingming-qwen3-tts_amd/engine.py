@@ -28,6 +28,18 @@ _SIGNATURES = {
     "qm_talker_decode": (_I32, [_P, _P, _P, _P, _I32, C.POINTER(_P)]),
     "qm_talker_prefill": (_I32, [_P, _P, _P, _P, _I32, C.POINTER(_P)]),
     "qm_talker_synchronize": (_I32, [_P]),
+    "qm_talker_stream": (_P, [_P]),
+    "qm_final_head_create": (_I32, [C.c_char_p, _I32, _U64, _P, C.POINTER(_P)]),
+    "qm_final_head_destroy": (None, [_P]),
+    "qm_final_head_reset": (_I32, [_P, _U64]),
+    "qm_final_head_run": (_I32, [_P, _P, _I32, _I32, C.POINTER(_I32)]),
+    "qm_final_head_rng_state": (_P, [_P]),
+    "qm_final_head_device_code": (_P, [_P]),
+    "qm_predictor_create": (_I32, [C.c_char_p, _P, _P, C.POINTER(_P)]),
+    "qm_predictor_destroy": (None, [_P]),
+    "qm_predictor_run_frame": (_I32, [_P, _P, _P, _P, _I32, C.POINTER(_I32)]),
+    "qm_predictor_next_input": (_P, [_P]),
+    "qm_generate": (_I32, [_P, _P, _P, _P, _I32, _I32, _P, _P, _I32, _I32, _P, C.POINTER(_I32), C.POINTER(_U64)]),
 }
 EXPORTS = tuple(_SIGNATURES)
 
@@ -137,3 +149,83 @@ class Talker:
 
     def synchronize(self):
         _check(lib().qm_talker_synchronize(self._handle))
+
+    @property
+    def stream(self):
+        return lib().qm_talker_stream(self._handle)
+
+
+class FinalHead:
+    """qm_final_head: codec_head, score processing, sampler, history and the generator state."""
+
+    def __init__(self, model_dir, history_capacity, seed, stream):
+        self._handle = _P()
+        _check(lib().qm_final_head_create(os.fsencode(model_dir), history_capacity, seed, stream, C.byref(self._handle)))
+
+    def close(self):
+        if self._handle:
+            lib().qm_final_head_destroy(self._handle)
+            self._handle = _P()
+
+    def __del__(self):
+        self.close()
+
+    def reset(self, seed):
+        _check(lib().qm_final_head_reset(self._handle, seed))
+
+    def run(self, hidden_device, frame, sampling=True):
+        address = hidden_device if isinstance(hidden_device, int) else hidden_device.data_ptr()
+        code = _I32()
+        _check(lib().qm_final_head_run(self._handle, address, frame, int(sampling), C.byref(code)))
+        return code.value
+
+    @property
+    def rng_state(self):
+        return lib().qm_final_head_rng_state(self._handle)
+
+    @property
+    def device_code(self):
+        return lib().qm_final_head_device_code(self._handle)
+
+
+class Predictor:
+    """qm_predictor: the code predictor's weights and its fifteen-step frame."""
+
+    def __init__(self, model_dir, rng_state_device, stream):
+        self._handle = _P()
+        _check(lib().qm_predictor_create(os.fsencode(model_dir), rng_state_device, stream, C.byref(self._handle)))
+
+    def close(self):
+        if self._handle:
+            lib().qm_predictor_destroy(self._handle)
+            self._handle = _P()
+
+    def __del__(self):
+        self.close()
+
+    def run_frame(self, talker_hidden_device, code0_device, context_host, sampling=True):
+        hidden = talker_hidden_device if isinstance(talker_hidden_device, int) else talker_hidden_device.data_ptr()
+        code0 = code0_device if isinstance(code0_device, int) else code0_device.data_ptr()
+        context_host = np.ascontiguousarray(context_host, dtype=np.uint16)
+        codes = (_I32 * 16)()
+        _check(lib().qm_predictor_run_frame(self._handle, hidden, code0, context_host.ctypes.data, int(sampling), codes))
+        return list(codes)
+
+    @property
+    def next_input(self):
+        return lib().qm_predictor_next_input(self._handle)
+
+
+def generate(talker, head, predictor, prompt_device, prompt_rows, maximum_frames, tts_pad_host, trailing_text_host=None,
+             sampling=True):
+    """qm_generate: (codes [frames][16] int32, trajectory hash)."""
+    prompt = prompt_device if isinstance(prompt_device, int) else prompt_device.data_ptr()
+    tts_pad_host = np.ascontiguousarray(tts_pad_host, dtype=np.uint16)
+    trailing_rows = 0 if trailing_text_host is None else int(trailing_text_host.shape[0])
+    trailing = None if trailing_text_host is None else np.ascontiguousarray(trailing_text_host, dtype=np.uint16)
+    codes = np.zeros((maximum_frames, 16), dtype=np.int32)
+    frames, digest = _I32(), _U64()
+    _check(lib().qm_generate(talker._handle, head._handle, predictor._handle, prompt, prompt_rows, maximum_frames,
+                             tts_pad_host.ctypes.data, trailing.ctypes.data if trailing is not None else None, trailing_rows,
+                             int(sampling), codes.ctypes.data, C.byref(frames), C.byref(digest)))
+    return codes[:frames.value].copy(), int(digest.value)

@@ -23,7 +23,7 @@ def test_header_symbols_are_exported(qm):
     for name in names:
         assert hasattr(lib, name), f"{name} declared in qm_attn.h but not exported"
     assert sorted(qm.EXPORTS) == names, "binding.py and qm_attn.h disagree on the entry points"
-    assert lib.qm_abi_version() == 1
+    assert lib.qm_abi_version() == 2
     assert lib.qm_target_arch() == b"gfx950"
 
 
@@ -59,7 +59,7 @@ def test_host_validation_without_device(qm):
     assert lib.qm_qk_norm_rope_kv_append(fake, fake, fake, fake, fake, fake, fake, fake, C.byref(c), fake, 4, 16, 64, 1e-6, None) == -3
     assert lib.qm_qk_norm_rope_kv_append(fake, fake, fake, fake, fake, fake, fake, fake, C.byref(c), fake, 4, 16, -1, 1e-6, None) == -3
     assert lib.qm_decode_attention(fake, C.byref(c), fake, 4, fake, 16, 64, -1, 0.1, None, 0, None) == -3
-    assert lib.qm_scatter_kv(fake, fake, C.byref(c), fake, 4, 10, 60, None) == -3
+    assert lib.qm_scatter_kv(fake, fake, C.byref(c), fake, 4, 10, 60, None, None) == -3
     # workspace: long contexts need one
     big = _cache(qm, n_pages=1024)
     need = lib.qm_decode_workspace_bytes(1, 16, 8, 8192)

@@ -162,3 +162,16 @@ def test_scatter_kv_paged_and_flat(oracle, qm, dev):
     with pytest.raises(qm.QmError) as e:
         qm.scatter_kv(to_dev(key, dev), to_dev(val, dev), qm.flat_cache(kf, vf, 8, 91), None, 1, rows, 20)
     assert e.value.code == -3
+    # a page table entry outside the pool: those tokens are skipped and flagged, nothing else changes
+    bad = pool.page_table.copy()
+    bad[0, 2] = pool.n_pages + 5
+    kd2, vd2, cache_d2, _ = pool_fresh = PagedPool(oracle, [first + rows], seed=12, fill=0x1234).device(qm, dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    qm.scatter_kv(to_dev(key, dev), to_dev(val, dev), cache_d2, to_dev(bad, dev), pool.max_pages, rows, first, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 1                                   # QM_STATUS_BAD_PAGE
+    skipped = pool.page_table[0, 2]
+    keep = np.ones(pool.n_pages, dtype=bool)
+    keep[skipped] = False
+    assert np.array_equal(to_u16(kd2)[keep], pool.k[keep]) and np.array_equal(to_u16(vd2)[keep], pool.v[keep])
+    assert (to_u16(kd2)[skipped] == 0x1234).all()

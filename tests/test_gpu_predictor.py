@@ -276,3 +276,27 @@ def test_predictor_step0_operator_argument_errors(qm, dev):
     assert L.qm_predictor_rope_bhsd(z.data_ptr(), z.data_ptr(), z.data_ptr(), z.data_ptr(), 2, 0, None) == -5
     assert L.qm_predictor_transpose(z.data_ptr(), z.data_ptr(), 2, 16, None) == -5
     assert L.qm_predictor_transpose(z.data_ptr(), z.data_ptr() + 2, 2, 16, None) == -2
+
+
+def test_predictor_m1_attention_is_the_exact_chain(oracle, qm, dev):
+    """PersistentPredictor::attention_m1 (R17:13473-13497) is served by the staged kernel with one query row
+    (the [16][1][128] query is the same bytes as [16][128]): against the oracle's M = 1 restatement every
+    context 1..16 agrees to the bit except where the device's expf differs (<= 1 bf16 ulp)."""
+    import torch
+    from qm_testlib import ulp_distance
+    differing = 0
+    for n in range(1, 17):
+        q = oracle.normal_bf16((16, 128), 4100 + n)
+        kc = oracle.normal_bf16((8, 16, 128), 4200 + n)
+        vc = oracle.normal_bf16((8, 16, 128), 4300 + n)
+        kc[:, n:] = 0x7fc0
+        vc[:, n:] = 0x7fc0
+        want = np.zeros_like(q)
+        assert oracle.predictor_attention_m1(q, kc, vc, want, n) == 0
+        out = torch.full((16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+        qm.predictor_attention_staged(to_dev(q, dev), to_dev(kc, dev), to_dev(vc, dev), out, 1, n, False)
+        torch.cuda.synchronize()
+        d = ulp_distance(to_u16(out), want)
+        assert d.max() <= 1
+        differing += int(np.count_nonzero(d))
+    assert differing <= 16 * 2048 // 500

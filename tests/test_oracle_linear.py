@@ -46,6 +46,48 @@ def test_random_rows_agree_with_fp64_dot_products(oracle):
     assert np.mean(got == want) > 0.99
 
 
+def test_linear_rows_against_fp64_and_layout(oracle):
+    """qmo_linear_rows / qmo_gate_up_swiglu_rows pinned on their own, not through the scalar they loop over:
+    every (row, column) against the fp64 dot product (correctly rounded up to an ulp next to a boundary), the
+    bias per column, the residual per (row, column) after the rounding, and the row-major layouts (a
+    transposed or strided index would move values between rows)."""
+    rows, cols, red = 7, 40, 256
+    x = oracle.normal_bf16((rows, red), 21)
+    w = oracle.normal_bf16((cols, red), 22, std=0.05)
+    b = oracle.normal_bf16((cols,), 23, std=0.1)
+    res = oracle.normal_bf16((rows, cols), 24)
+    xf, wf = oracle.bf16_to_f32(x).astype(np.float64), oracle.bf16_to_f32(w).astype(np.float64)
+    exact = xf @ wf.T + oracle.bf16_to_f32(b).astype(np.float64)[None, :]
+    out = np.zeros((rows, cols), dtype=np.uint16)
+    assert oracle.linear_rows(x, w, b, None, out, rows, cols, red) == 0
+    got = oracle.bf16_to_f32(out).astype(np.float64)
+    assert np.all(np.abs(got - exact) <= np.maximum(np.abs(exact), 2.0 ** -126) * 2.0 ** -7)
+    rounded = oracle.f32_to_bf16(exact.astype(np.float32))
+    assert np.mean(out == rounded) > 0.99
+    # residual: bf16(residual + bf16(linear)), per element
+    out_r = np.zeros_like(out)
+    assert oracle.linear_rows(x, w, b, res, out_r, rows, cols, red) == 0
+    want_r = oracle.f32_to_bf16(oracle.bf16_to_f32(res) + oracle.bf16_to_f32(out))
+    assert np.array_equal(out_r, want_r)
+    # one row at a time gives the same rows (no coupling between rows)
+    for r in (0, 3, 6):
+        one = np.zeros((1, cols), dtype=np.uint16)
+        assert oracle.linear_rows(x[r:r + 1].copy(), w, b, None, one, 1, cols, red) == 0
+        assert np.array_equal(one[0], out[r])
+    # gate/up/SwiGLU rows against fp64: g = bf16(x.gate), u = bf16(x.up), bf16(bf16(g*sigmoid(g)) * u)
+    inter = 24
+    gw = oracle.normal_bf16((inter, red), 25, std=0.05)
+    uw = oracle.normal_bf16((inter, red), 26, std=0.05)
+    act = np.zeros((rows, inter), dtype=np.uint16)
+    assert oracle.gate_up_swiglu_rows(x, gw, uw, act, rows, red, inter) == 0
+    g = oracle.bf16_to_f32(oracle.f32_to_bf16((xf @ oracle.bf16_to_f32(gw).astype(np.float64).T).astype(np.float32))).astype(np.float64)
+    u = oracle.bf16_to_f32(oracle.f32_to_bf16((xf @ oracle.bf16_to_f32(uw).astype(np.float64).T).astype(np.float32))).astype(np.float64)
+    silu = oracle.bf16_to_f32(oracle.f32_to_bf16((g / (1.0 + np.exp(-g))).astype(np.float32))).astype(np.float64)
+    want = silu * u
+    got = oracle.bf16_to_f32(act).astype(np.float64)
+    assert np.all(np.abs(got - want) <= np.maximum(np.abs(want), 1e-30) * 2.0 ** -6 + 1e-6)
+
+
 @pytest.mark.parametrize("case", order_cases(), ids=lambda c: c[0])
 def test_evaluation_order(oracle, case):
     _, wrow, bias, residual, expected = case
