@@ -1,0 +1,251 @@
+"""GPU parity of the frame engine (libqm_engine): final head, the code predictor's fifteen-step frame and the
+generation loop, on a synthetic checkpoint written here.
+
+The predictor frame and the final head are compared with the oracle's chain of the same operators from the same
+inputs: the sampled codes must be identical (the linears are bit-exact, the attention over at most 16 keys is the
+exact-chain kernel) and the next talker input with them.  The loop itself is held to the determinism contract of
+the reference (CONTRACT.md:148-158): the same request gives the same codec trajectory and hash, also after a reset,
+and the loop's codes equal a replay of the same engines step by step from Python.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+from qm_testlib import to_u16
+
+pytestmark = pytest.mark.gpu
+
+H, Q, KV, I_T, T_LAYERS = 2048, 2048, 1024, 512, 2           # talker (small intermediate: the test is about the loop)
+PH, PI, P_LAYERS, V, STEPS = 1024, 3072, 2, 2048, 15            # predictor; two layers keep the CPU chain short
+HEAD_V, EOS, TABLE_ROWS = 3072, 2150, 3072
+SEED = 20240229
+
+
+def _checkpoint(directory):
+    import torch
+    from safetensors.torch import save_file
+    g = torch.Generator().manual_seed(99)
+
+    def rnd(shape, std=1.0, mean=0.0):
+        return (torch.randn(shape, generator=g) * std + mean).to(torch.bfloat16)
+
+    t = {"talker.model.norm.weight": rnd((H,), 0.1, 1.0), "talker.model.codec_embedding.weight": rnd((TABLE_ROWS, H), 0.5),
+         "talker.codec_head.weight": rnd((HEAD_V, H), 0.05)}
+    for i in range(T_LAYERS):
+        p = f"talker.model.layers.{i}."
+        t.update({p + "input_layernorm.weight": rnd((H,), 0.1, 1.0), p + "post_attention_layernorm.weight": rnd((H,), 0.1, 1.0),
+                  p + "self_attn.q_proj.weight": rnd((Q, H), 0.02), p + "self_attn.k_proj.weight": rnd((KV, H), 0.02),
+                  p + "self_attn.v_proj.weight": rnd((KV, H), 0.02), p + "self_attn.o_proj.weight": rnd((H, Q), 0.02),
+                  p + "self_attn.q_norm.weight": rnd((128,), 0.1, 1.0), p + "self_attn.k_norm.weight": rnd((128,), 0.1, 1.0),
+                  p + "mlp.gate_proj.weight": rnd((I_T, H), 0.03), p + "mlp.up_proj.weight": rnd((I_T, H), 0.03),
+                  p + "mlp.down_proj.weight": rnd((H, I_T), 0.03)})
+    c = "talker.code_predictor."
+    t.update({c + "small_to_mtp_projection.weight": rnd((PH, H), 0.02), c + "small_to_mtp_projection.bias": rnd((PH,), 0.1),
+              c + "model.norm.weight": rnd((PH,), 0.1, 1.0)})
+    for i in range(P_LAYERS):
+        p = c + f"model.layers.{i}."
+        t.update({p + "input_layernorm.weight": rnd((PH,), 0.1, 1.0), p + "post_attention_layernorm.weight": rnd((PH,), 0.1, 1.0),
+                  p + "self_attn.q_proj.weight": rnd((Q, PH), 0.03), p + "self_attn.k_proj.weight": rnd((KV, PH), 0.03),
+                  p + "self_attn.v_proj.weight": rnd((KV, PH), 0.03), p + "self_attn.o_proj.weight": rnd((PH, Q), 0.02),
+                  p + "self_attn.q_norm.weight": rnd((128,), 0.1, 1.0), p + "self_attn.k_norm.weight": rnd((128,), 0.1, 1.0),
+                  p + "mlp.gate_proj.weight": rnd((PI, PH), 0.03), p + "mlp.up_proj.weight": rnd((PI, PH), 0.03),
+                  p + "mlp.down_proj.weight": rnd((PH, PI), 0.02)})
+    for i in range(STEPS):
+        t[c + f"lm_head.{i}.weight"] = rnd((V, PH), 0.05)
+        t[c + f"model.codec_embedding.{i}.weight"] = rnd((V, H), 0.5)
+    save_file(t, os.path.join(directory, "model.safetensors"))
+    return {n: x.view(torch.int16).numpy().view(np.uint16).copy() for n, x in t.items()}
+
+
+@pytest.fixture(scope="module")
+def model(tmp_path_factory):
+    directory = str(tmp_path_factory.mktemp("frame_model"))
+    return directory, _checkpoint(directory)
+
+
+def _device_bytes(address, nbytes):
+    hip = C.CDLL("libamdhip64.so")
+    out = np.zeros(nbytes // 2, dtype=np.uint16)
+    assert hip.hipMemcpy(out.ctypes.data_as(C.c_void_p), C.c_void_p(address), C.c_size_t(nbytes), 2) == 0
+    return out
+
+
+def _oracle_predictor_frame(oracle, w, hidden, code0, context, rng, sampling=True):
+    """capture_step x 15 and capture_graph's tail (R17:13592-13896) with the oracle's operators."""
+    c = "talker.code_predictor."
+    u16 = lambda *s: np.zeros(s, dtype=np.uint16)
+    cos, sin = oracle.rope_table(16, 0)
+    codes = np.zeros(16, dtype=np.int32)
+    selected = u16(16, H)
+    table = w["talker.model.codec_embedding.weight"]
+    free = u16(2, H)
+    free[0] = hidden
+    codes[0] = code0
+    selected[0] = table[code0]
+    free[1] = table[code0]
+    caches = [(u16(8, 16, 128), u16(8, 16, 128)) for _ in range(P_LAYERS)]
+    top_k = 50 if sampling else 0
+    # ---- step 0: two rows, the staged path ----
+    rows = 2
+    cur = u16(rows, PH)
+    assert oracle.linear_rows(free, w[c + "small_to_mtp_projection.weight"], w[c + "small_to_mtp_projection.bias"], None, cur,
+                              rows, PH, H, 16) == 0
+    for layer in range(P_LAYERS):
+        p = c + f"model.layers.{layer}."
+        kc, vc = caches[layer]
+        norm, q, k, v = u16(rows, PH), u16(rows, Q), u16(rows, KV), u16(rows, KV)
+        assert oracle.rmsnorm_rows(cur, w[p + "input_layernorm.weight"], norm, rows, PH) == 0
+        for name, dst, n in (("q", q, Q), ("k", k, KV), ("v", v, KV)):
+            assert oracle.linear_rows(norm, w[p + f"self_attn.{name}_proj.weight"], None, None, dst, rows, n, PH, 16) == 0
+        qn, kn = u16(rows * 16, 128), u16(rows * 8, 128)
+        assert oracle.rmsnorm_rows(q.reshape(rows * 16, 128), w[p + "self_attn.q_norm.weight"], qn, rows * 16, 128) == 0
+        assert oracle.rmsnorm_rows(k.reshape(rows * 8, 128), w[p + "self_attn.k_norm.weight"], kn, rows * 8, 128) == 0
+        qb, kb, vb = u16(16, rows, 128), u16(8, rows, 128), u16(8, rows, 128)
+        assert oracle.predictor_transpose(qn, qb, rows, 16) == 0
+        assert oracle.predictor_transpose(kn, kb, rows, 8) == 0
+        assert oracle.predictor_transpose(v, vb, rows, 8) == 0
+        qr, kr = u16(16, rows, 128), u16(8, rows, 128)
+        assert oracle.predictor_rope_bhsd(qb, cos, sin, qr, rows, 16) == 0
+        assert oracle.predictor_rope_bhsd(kb, cos, sin, kr, rows, 8) == 0
+        assert oracle.predictor_update_cache(kr, kc, rows, 0) == 0
+        assert oracle.predictor_update_cache(vb, vc, rows, 0) == 0
+        ctx = u16(rows, Q)
+        assert oracle.predictor_attention_staged(qr, kc, vc, ctx.reshape(rows, 16, 128), rows, 2, True) == 0
+        res, post, act, nxt = u16(rows, PH), u16(rows, PH), u16(rows, PI), u16(rows, PH)
+        assert oracle.linear_rows(ctx, w[p + "self_attn.o_proj.weight"], None, cur, res, rows, PH, Q, 16) == 0
+        assert oracle.rmsnorm_rows(res, w[p + "post_attention_layernorm.weight"], post, rows, PH) == 0
+        assert oracle.gate_up_swiglu_rows(post, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], act, rows, PH, PI, 16) == 0
+        assert oracle.linear_rows(act, w[p + "mlp.down_proj.weight"], None, res, nxt, rows, PH, PI, 16) == 0
+        cur = nxt
+    fin, logits = u16(rows, PH), u16(rows, V)
+    assert oracle.rmsnorm_rows(cur, w[c + "model.norm.weight"], fin, rows, PH) == 0
+    assert oracle.linear_rows(fin, w[c + "lm_head.0.weight"], None, None, logits, rows, V, PH, 16) == 0
+    out = np.zeros(1, dtype=np.int32)
+    assert oracle.sample_topk(logits.reshape(-1), True, (rows - 1) * V, V, top_k, 0.9, rng, out) == 0
+    codes[1] = out[0]
+    selected[1] = w[c + "model.codec_embedding.0.weight"][out[0]]
+    free_input = selected[1].copy()
+    # ---- steps 1..14: one row, the M = 1 operators ----
+    for step in range(1, STEPS):
+        position = step + 1
+        cur = u16(PH)
+        assert oracle.linear_m1(free_input, w[c + "small_to_mtp_projection.weight"], w[c + "small_to_mtp_projection.bias"], None,
+                                cur, PH, H, 16) == 0
+        for layer in range(P_LAYERS):
+            p = c + f"model.layers.{layer}."
+            kc, vc = caches[layer]
+            norm, q, k, v, qrot, ctx, attn, res, post, act, nxt = (u16(1, PH), u16(Q), u16(KV), u16(KV), u16(Q), u16(Q),
+                                                                   u16(PH), u16(PH), u16(PH), u16(PI), u16(PH))
+            assert oracle.rmsnorm_rows(cur.reshape(1, PH), w[p + "input_layernorm.weight"], norm, 1, PH) == 0
+            assert oracle.predictor_qkv_m1(norm[0], w[p + "self_attn.q_proj.weight"], w[p + "self_attn.k_proj.weight"],
+                                           w[p + "self_attn.v_proj.weight"], q, k, v, PH, Q, KV, 16) == 0
+            assert oracle.qk_norm_rope_kv_append(q, k, v, w[p + "self_attn.q_norm.weight"], w[p + "self_attn.k_norm.weight"],
+                                                 cos[position], sin[position], qrot, oracle.flat_cache(kc, vc, 8, 16), None, 1,
+                                                 16, position) == 0
+            assert oracle.predictor_attention_m1(qrot, kc, vc, ctx, position + 1) == 0
+            assert oracle.predictor_linear_m1(ctx, w[p + "self_attn.o_proj.weight"], None, attn, PH, Q, 16) == 0
+            assert oracle.add_postnorm_m1(cur, attn, w[p + "post_attention_layernorm.weight"], res, post, PH) == 0
+            assert oracle.predictor_gate_up_swiglu_m1(post, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], act, PH, PI,
+                                                      16) == 0
+            assert oracle.predictor_linear_m1(act, w[p + "mlp.down_proj.weight"], res, nxt, PH, PI, 16) == 0
+            cur = nxt
+        fin, logits = u16(1, PH), u16(V)
+        assert oracle.rmsnorm_rows(cur.reshape(1, PH), w[c + "model.norm.weight"], fin, 1, PH) == 0
+        assert oracle.linear_m1(fin[0], w[c + f"lm_head.{step}.weight"], None, None, logits, V, PH, 16) == 0
+        assert oracle.sample_topk(logits, True, 0, V, top_k, 0.9, rng, out) == 0
+        codes[step + 1] = out[0]
+        selected[step + 1] = w[c + f"model.codec_embedding.{step}.weight"][out[0]]
+        free_input = selected[step + 1].copy()
+    total = oracle.bf16_to_f32(selected).astype(np.float32)
+    acc = np.zeros(H, dtype=np.float32)
+    for group in range(16):
+        acc = (acc + total[group]).astype(np.float32)
+    summed = oracle.f32_to_bf16(acc)
+    nxt_input = oracle.f32_to_bf16(oracle.bf16_to_f32(summed) + oracle.bf16_to_f32(context))
+    return codes, nxt_input
+
+
+def test_final_head_and_predictor_frame_match_the_oracle_chain(engine, oracle, qm, dev, model):
+    import torch
+    directory, w = model
+    talker = engine.Talker(directory, 64)
+    head = engine.FinalHead(directory, 32, SEED, talker.stream)
+    predictor = engine.Predictor(directory, head.rng_state, talker.stream)
+    rng = np.array([SEED], dtype=np.uint64)
+    history = np.zeros(32, dtype=np.int32)
+    for frame, sampling in ((0, True), (1, True), (2, False)):
+        hidden = oracle.normal_bf16((H,), 500 + frame)
+        hd = torch.from_numpy(hidden.view(np.int16)).to(dev)
+        torch.cuda.synchronize()
+        code0 = head.run(hd, frame, sampling)
+        # the oracle's final head: codec_head in the talker linear's order, then the sampler with the history so far
+        logits = np.zeros(HEAD_V, dtype=np.uint16)
+        assert oracle.linear_m1(hidden, w["talker.codec_head.weight"], None, None, logits, HEAD_V, H, 16) == 0
+        want = np.zeros(1, dtype=np.int32)
+        assert oracle.final_head_sample(logits, history, frame, HEAD_V, EOS, 1024, 1.05, 50 if sampling else 0, 0.9, rng, want) == 0
+        assert code0 == int(want[0])
+        context = oracle.normal_bf16((H,), 600 + frame, 0.0, 0.5)
+        codes = predictor.run_frame(hd, head.device_code, context, sampling)
+        want_codes, want_next = _oracle_predictor_frame(oracle, w, hidden, code0, context, rng, sampling)
+        assert codes == want_codes.tolist()
+        assert np.array_equal(_device_bytes(predictor.next_input, H * 2), want_next)
+    predictor.close(); head.close(); talker.close()
+
+
+def _fnv1a64(data):
+    value = 1469598103934665603
+    for b in data:
+        value = ((value ^ b) * 1099511628211) & 0xFFFFFFFFFFFFFFFF
+    return value
+
+
+def test_generation_loop_is_deterministic_and_equals_its_stepwise_replay(engine, oracle, qm, dev, model):
+    import torch
+    directory, w = model
+    prompt_rows, frames = 19, 5
+    talker = engine.Talker(directory, 64)
+    head = engine.FinalHead(directory, 32, SEED, talker.stream)
+    predictor = engine.Predictor(directory, head.rng_state, talker.stream)
+    prompt = oracle.normal_bf16((prompt_rows, H), 41)
+    pd = torch.from_numpy(prompt.view(np.int16)).to(dev)
+    torch.cuda.synchronize()
+    tts_pad = oracle.normal_bf16((H,), 42, 0.0, 0.5)
+    trailing = oracle.normal_bf16((2, H), 43, 0.0, 0.5)
+    codes, digest = engine.generate(talker, head, predictor, pd, prompt_rows, frames, tts_pad, trailing)
+    assert codes.shape == (frames, 16) and digest == _fnv1a64(codes.tobytes()) == engine.fnv1a64(codes.tobytes())
+    assert codes.min() >= 0 and codes[:, 1:].max() < V
+    # the same request again, after a reset: same trajectory, same hash (CONTRACT.md:148-158)
+    for _ in range(2):
+        head.reset(SEED)
+        again, digest2 = engine.generate(talker, head, predictor, pd, prompt_rows, frames, tts_pad, trailing)
+        assert np.array_equal(again, codes) and digest2 == digest
+    # another seed gives another trajectory (the samplers do draw)
+    head.reset(SEED + 1)
+    other, _ = engine.generate(talker, head, predictor, pd, prompt_rows, frames, tts_pad, trailing)
+    assert not np.array_equal(other, codes)
+    # the loop, replayed from Python with the same engines: prefill, then per frame head / predictor / decode
+    head.reset(SEED)
+    cos, sin = engine.rope_rows(prompt_rows, 0)
+    dcos, dsin = engine.rope_rows(frames, prompt_rows)
+    hidden = talker.prefill(pd, cos, sin, prompt_rows)
+    talker.synchronize()
+    replay = []
+    for frame in range(frames):
+        code0 = head.run(hidden, frame)
+        context = trailing[frame] if frame < trailing.shape[0] else tts_pad
+        frame_codes = predictor.run_frame(hidden, head.device_code, context)
+        assert frame_codes[0] == code0
+        replay.append(frame_codes)
+        if frame + 1 < frames:
+            hidden = talker.decode(predictor.next_input, dcos[frame], dsin[frame], frame)
+    talker.synchronize()
+    assert np.array_equal(np.array(replay, dtype=np.int32), codes)
+    # fewer frames: a prefix of the trajectory; argument errors
+    head.reset(SEED)
+    short, _ = engine.generate(talker, head, predictor, pd, prompt_rows, 2, tts_pad, trailing)
+    assert np.array_equal(short, codes[:2])
+    with pytest.raises(engine.EngineError):
+        engine.generate(talker, head, predictor, pd, 0, 2, tts_pad, trailing)
+    predictor.close(); head.close(); talker.close()
