@@ -10,9 +10,9 @@ configuration whose working set (~0.57 GB) exceeds the caches, so that "HBM GB/s
 The other configurations are timed too (`--all`, default on) and reported under `per_config`.
 One JSON line is printed on stdout.
 
-Inputs are drawn on the device by torch's seeded generator; the CPU baseline leg copies the same
-tensors to the host and times the scalar oracle (oracle/, test infrastructure) on them, and also
-checks the GPU result against it.
+Inputs come from the seeded SplitMix64 -> Box-Muller stream that the parity tests use (class Synthetic,
+evaluated on the device); the CPU baseline leg copies the same tensors to the host and times the
+scalar oracle (oracle/, test infrastructure) on them, and also checks the GPU result against it.
 """
 import argparse
 import importlib
@@ -35,6 +35,79 @@ HEADLINE_TRAFFIC_BYTES = int((288456.9 * 2.0 + 3349.5 * 1.0) * 1024)
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 SCALE = 0.08838834764831845
+
+
+_GOLDEN = 0x9E3779B97F4A7C15
+_MIX_A = 0xBF58476D1CE4E5B9
+_MIX_B = 0x94D049BB133111EB
+_MASK64 = (1 << 64) - 1
+
+
+def _signed64(x):
+    x &= _MASK64
+    return x - (1 << 64) if x >> 63 else x
+
+
+def _splitmix_at(seed, k):
+    """k-th output (k >= 1) of the SplitMix64 stream seeded with `seed` (Python integers)."""
+    z = (seed + k * _GOLDEN) & _MASK64
+    z = ((z ^ (z >> 30)) * _MIX_A) & _MASK64
+    z = ((z ^ (z >> 27)) * _MIX_B) & _MASK64
+    return z ^ (z >> 31)
+
+
+class Synthetic:
+    """The seeded inputs of every workload: SplitMix64 -> Box-Muller, element i of a tensor from stream
+    outputs 2i+1 and 2i+2 of that tensor's seed (the generator the parity tests draw from, evaluated here
+    on the device in int64 / float64), and integer draws / Fisher-Yates permutations from the same stream
+    on the host.  Each tensor drawn from one Synthetic takes the next seed."""
+
+    def __init__(self, dev, seed):
+        self.dev, self.seed = dev, seed
+
+    def _next_seed(self):
+        self.seed += 1
+        return self.seed
+
+    @staticmethod
+    def _lsr(z, n):
+        return (z >> n) & ((1 << (64 - n)) - 1)
+
+    def _mix(self, seed, k):
+        z = k * _signed64(_GOLDEN) + _signed64(seed)
+        z = (z ^ self._lsr(z, 30)) * _signed64(_MIX_A)
+        z = (z ^ self._lsr(z, 27)) * _signed64(_MIX_B)
+        return z ^ self._lsr(z, 31)
+
+    def normal(self, shape, std=1.0, mean=0.0):
+        import torch
+        seed = self._next_seed()
+        n = int(np.prod(shape))
+        out = torch.empty(n, dtype=torch.bfloat16, device=self.dev)
+        std64, mean64 = float(np.float32(std)), float(np.float32(mean))
+        chunk = 1 << 24
+        for lo in range(0, n, chunk):
+            i = torch.arange(lo, min(n, lo + chunk), dtype=torch.int64, device=self.dev)
+            a, b = self._mix(seed, 2 * i + 1), self._mix(seed, 2 * i + 2)
+            u1 = (self._lsr(a, 11).double() + 1.0) * (1.0 / 9007199254740992.0)
+            u2 = self._lsr(b, 11).double() * (1.0 / 9007199254740992.0)
+            z = torch.sqrt(-2.0 * torch.log(u1)) * torch.cos(6.283185307179586477 * u2)
+            out[lo:lo + chunk] = (mean64 + std64 * z).float().to(torch.bfloat16)
+        return out.view(shape)
+
+    def integers(self, n, lo, hi):
+        """n integers uniform in [lo, hi] (host, int32)."""
+        seed = self._next_seed()
+        return np.array([lo + _splitmix_at(seed, i + 1) % (hi - lo + 1) for i in range(n)], dtype=np.int32)
+
+    def permutation(self, n):
+        """Seeded Fisher-Yates permutation of 0..n-1 (host, int32)."""
+        seed = self._next_seed()
+        out = list(range(n))
+        for i in range(n - 1, 0, -1):
+            j = _splitmix_at(seed, n - i) % (i + 1)
+            out[i], out[j] = out[j], out[i]
+        return np.array(out, dtype=np.int32)
 
 
 def _bits(t):
@@ -95,24 +168,21 @@ class RaggedDecode:
 
     def __init__(self, qm, dev, seed=2024, n_streams=64, lo=256, hi=4096):
         import torch
-        g = torch.Generator(device="cpu").manual_seed(seed)
+        syn = Synthetic(dev, seed)
         self.qm, self.dev, self.n = qm, dev, n_streams
-        self.lens = torch.randint(lo, hi + 1, (n_streams,), generator=g, dtype=torch.int32)
+        self.lens = torch.from_numpy(syn.integers(n_streams, lo, hi))
         pages_per = (self.lens + 15) // 16
         self.max_pages = int(pages_per.max())
         self.n_pages = int(pages_per.sum()) + 7
-        perm = torch.randperm(self.n_pages, generator=g, dtype=torch.int32)
+        perm = torch.from_numpy(syn.permutation(self.n_pages))
         table = torch.full((n_streams, self.max_pages), -1, dtype=torch.int32)
         cur = 0
         for s in range(n_streams):
             k = int(pages_per[s])
             table[s, :k] = perm[cur:cur + k]
             cur += k
-        gd = torch.Generator(device=dev).manual_seed(seed + 1)
         shape = (self.n_pages, 8, 16, 128)
-        self.k = torch.randn(shape, generator=gd, device=dev, dtype=torch.float32).to(torch.bfloat16)
-        self.v = torch.randn(shape, generator=gd, device=dev, dtype=torch.float32).to(torch.bfloat16)
-        self.q = torch.randn((n_streams, 16, 128), generator=gd, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        self.k, self.v, self.q = syn.normal(shape), syn.normal(shape), syn.normal((n_streams, 16, 128))
         self.out = torch.zeros_like(self.q)
         self.table = table.to(dev)
         self.lens_d = self.lens.to(dev)
@@ -163,12 +233,11 @@ class SingleDecode:
         self.name = ("talker_fused_step_ctx%d" if fused_append else "gqa_decode_ctx%d") % ctx
         if fused_append and not one_launch:
             self.name += "_append_and_decode_launches"
-        gd = torch.Generator(device=dev).manual_seed(seed)
+        syn = Synthetic(dev, seed)
         self.max_cache = ctx + 4
         self.copies = copies
 
-        def rnd(shape, std=1.0, mean=0.0):
-            return (torch.randn(shape, generator=gd, device=dev, dtype=torch.float32) * std + mean).to(torch.bfloat16)
+        rnd = syn.normal
 
         self.k = [rnd((8, self.max_cache, 128)) for _ in range(copies)]
         self.v = [rnd((8, self.max_cache, 128)) for _ in range(copies)]
@@ -248,10 +317,9 @@ class QkvGemv:
         import torch
         self.qm, self.copies = qm, copies
         self.name = "qkv_gemv_m1_hidden2048" + ("_rotating%d" % copies if copies > 1 else "")
-        gd = torch.Generator(device=dev).manual_seed(seed)
+        syn = Synthetic(dev, seed)
 
-        def rnd(shape, std=1.0):
-            return (torch.randn(shape, generator=gd, device=dev, dtype=torch.float32) * std).to(torch.bfloat16)
+        rnd = syn.normal
 
         self.x = rnd((2048,))
         self.w = [(rnd((2048, 2048), 0.02), rnd((1024, 2048), 0.02), rnd((1024, 2048), 0.02)) for _ in range(copies)]
@@ -303,12 +371,11 @@ class TalkerLayerStep:
         self.qm, self.layers, self.ctx, self.fused = qm, layers, ctx, fused
         self.name = "talker_layer_decode_step_ctx%d_x%dlayers%s" % (ctx, layers, "" if fused else "_reference_launch_sequence")
         self.copies = layers
-        gd = torch.Generator(device=dev).manual_seed(seed)
+        syn = Synthetic(dev, seed)
         H, I = 2048, 6144
         self.H, self.I = H, I
 
-        def rnd(shape, std=1.0, mean=0.0):
-            return (torch.randn(shape, generator=gd, device=dev, dtype=torch.float32) * std + mean).to(torch.bfloat16)
+        rnd = syn.normal
 
         self.max_cache = ctx + 4
         self.w = []
@@ -400,7 +467,7 @@ class PredictorFrameSteps:
     reference chains them (PersistentPredictor::capture_step, R17:13592-13854): input projection,
     five layers (RMSNorm + Q/K/V, QK-norm + RoPE + append + attention over the [8][16][128] cache,
     o_proj, residual add + post-norm + gate/up/SwiGLU, down_proj + residual), final norm + that
-    step's head, top-k sampler, embedding gather feeding the next step.  29 launches per step with
+    step's head, top-k sampler, embedding gather feeding the next step.  34 launches per step with
     the fused operators (the reference: 46 graph nodes per M = 1 step).  Geometry R17:7951-7962;
     weights random.  One `step()` is the whole frame."""
     bound = "hbm"
@@ -410,12 +477,11 @@ class PredictorFrameSteps:
     def __init__(self, qm, dev, seed=77):
         import torch
         self.qm, self.dev = qm, dev
-        gd = torch.Generator(device=dev).manual_seed(seed)
+        syn = Synthetic(dev, seed)
         H, Q, KV, I, OUT, V = 1024, 2048, 1024, 3072, 2048, 2048
         self.dims = (H, Q, KV, I, OUT, V)
 
-        def rnd(shape, std=1.0, mean=0.0):
-            return (torch.randn(shape, generator=gd, device=dev, dtype=torch.float32) * std + mean).to(torch.bfloat16)
+        rnd = syn.normal
 
         self.proj_w, self.proj_b = rnd((H, OUT), 0.02), rnd((H,), 0.1)
         self.layers = []
@@ -446,7 +512,7 @@ class PredictorFrameSteps:
         self.ws_bytes = qm.decode_workspace_bytes(1, 16, 8, 16)
         self.ws = torch.empty(self.ws_bytes // 4 + 1, dtype=torch.float32, device=dev)
         layer_w = 2 * (Q * H + 2 * KV * H + H * Q + 2 * I * H + H * I)
-        self.launches_per_step = 1 + 5 * 5 + 3
+        self.launches_per_step = 1 + 5 * 6 + 3
         self.bytes = 14 * (5 * layer_w + 2 * H * OUT + 2 * V * H + 2 * OUT)          # weights streamed once per step
         self.flops = self.bytes
         self.copies = 14
@@ -460,9 +526,12 @@ class PredictorFrameSteps:
         for L in self.layers:
             qm.predictor_rmsnorm_qkv_m1(cur, L["in_norm"], L["wq"], L["wk"], L["wv"], self.q, self.k_, self.v_, H, Q, KV,
                                         1e-6, s)
-            qm.decode_step_fused(self.q, self.k_, self.v_, L["gq"], L["gk"], self.cos[position], self.sin[position],
-                                 self.qrot, L["cache"], None, 1, self.ctxv, 16, position, -1, SCALE, 1e-6, self.ws,
-                                 self.ws_bytes, None, s)
+            # the engine's pair of operators: append at `position`, then attention on the reference's exact chain
+            # (one launch more than the fused decode step, whose sums are ordered differently: a sampled code
+            # must not depend on that)
+            qm.qk_norm_rope_kv_append(self.q, self.k_, self.v_, L["gq"], L["gk"], self.cos[position], self.sin[position],
+                                      self.qrot, L["cache"], None, 1, 16, position, 1e-6, s)
+            qm.predictor_attention_staged(self.qrot, L["k"], L["v"], self.ctxv, 1, position + 1, False, s)
             qm.predictor_linear_m1(self.ctxv, L["wo"], None, self.attn, H, Q, s)
             qm.predictor_add_postnorm_gate_up_swiglu_m1(cur, self.attn, L["post"], self.res, L["wg"], L["wu"], self.act,
                                                         H, I, 1e-6, s)
@@ -522,8 +591,7 @@ class PredictorFrameSteps:
                 assert oracle.predictor_qkv_m1(norm[0], L["wq"], L["wk"], L["wv"], q, k, v, H, Q, KV, threads) == 0
                 assert oracle.qk_norm_rope_kv_append(q, k, v, L["gq"], L["gk"], cos[position], sin[position], qrot, cache,
                                                      None, 1, 16, position) == 0
-                assert oracle.attention(qrot, cache, None, 1, ctxv, 1, position, 16, -1, SCALE, oracle.POLICY_ONLINE,
-                                        threads) == 0
+                assert oracle.predictor_attention_m1(qrot, L["k"], L["v"], ctxv, position + 1) == 0
                 assert oracle.predictor_linear_m1(ctxv, L["wo"], None, attn, H, Q, threads) == 0
                 assert oracle.add_postnorm_m1(cur, attn, L["post"], res, post, H) == 0
                 assert oracle.predictor_gate_up_swiglu_m1(post, L["wg"], L["wu"], act, H, I, threads) == 0
@@ -550,11 +618,15 @@ class Prefill:
     name = "causal_prefill_b4_s1024_paged16"
     bound = "mfma"
 
-    def __init__(self, qm, dev, seed=44, batch=4, seq=1024, split=False):
+    def __init__(self, qm, dev, seed=44, batch=4, seq=1024, split=False, score_rounding=1):
         import torch
-        self.qm, self.batch, self.seq = qm, batch, seq
+        self.qm, self.batch, self.seq, self.score_rounding = qm, batch, seq, score_rounding
         if (batch, seq) != (4, 1024):
             self.name = "causal_prefill_b%d_s%d_paged16%s" % (batch, seq, "_key_split" if split else "")
+        if not score_rounding:
+            # scores stay fp32 between Q.K^T and the softmax (the fp32-accumulate formulation); the default
+            # rounds them to bf16 twice as the reference's operator does
+            self.name += "_fp32_scores"
         # key split: a workspace lets up to three blocks share a long query tile (shapes that leave CUs idle)
         self.workspace, self.workspace_bytes = None, 0
         if split:
@@ -562,18 +634,16 @@ class Prefill:
             self.workspace = torch.zeros(max(self.workspace_bytes, 256) // 4, dtype=torch.int32, device=dev)
             qm.prefill_split_workspace_init(self.workspace, self.workspace_bytes,
                                             torch.cuda.current_stream().cuda_stream)
-        gd = torch.Generator(device=dev).manual_seed(seed)
-        g = torch.Generator(device="cpu").manual_seed(seed)
+        syn = Synthetic(dev, seed)
 
-        def rnd(shape):
-            return torch.randn(shape, generator=gd, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        rnd = syn.normal
 
         self.q, self.k, self.v = rnd((batch, seq, 16, 128)), rnd((batch, seq, 8, 128)), rnd((batch, seq, 8, 128))
         self.out = torch.zeros_like(self.q)
         per = (seq + 15) // 16
         self.max_pages = per
         self.n_pages = batch * per + 5
-        perm = torch.randperm(self.n_pages, generator=g, dtype=torch.int32)
+        perm = torch.from_numpy(syn.permutation(self.n_pages))
         self.table = perm[:batch * per].view(batch, per).contiguous().to(dev)
         self.kp = torch.zeros((self.n_pages, 8, 16, 128), dtype=torch.bfloat16, device=dev)
         self.vp = torch.zeros_like(self.kp)
@@ -586,15 +656,20 @@ class Prefill:
 
     def step(self):
         import torch
+        self.qm.set_option(self.qm.OPT_PREFILL_SCORE_ROUNDING, self.score_rounding)
+        try:
+            self._launch(torch.cuda.current_stream().cuda_stream)
+        finally:
+            self.qm.set_option(self.qm.OPT_PREFILL_SCORE_ROUNDING, 1)
+
+    def _launch(self, stream):
         if self.workspace is not None:
             self.qm.prefill_attention_causal_split(self.q, self.k, self.v, self.out, self.cache, self.table,
                                                    self.max_pages, self.batch, self.seq, 16, 8, self.workspace,
-                                                   self.workspace_bytes, SCALE, self.status,
-                                                   torch.cuda.current_stream().cuda_stream)
+                                                   self.workspace_bytes, SCALE, self.status, stream)
             return
         self.qm.prefill_attention_causal(self.q, self.k, self.v, self.out, self.cache, self.table, self.max_pages,
-                                         self.batch, self.seq, 16, 8, SCALE, self.status,
-                                         torch.cuda.current_stream().cuda_stream)
+                                         self.batch, self.seq, 16, 8, SCALE, self.status, stream)
 
     def cpu_baseline(self, oracle, threads):
         """Sample: batch entry 0 (a quarter of the flops)."""
@@ -602,7 +677,8 @@ class Prefill:
         out = np.zeros_like(q)
         t0 = time.perf_counter()
         rc = oracle.prefill_attention_causal(q, k, v, out, None, None, 0, 1, self.seq, 16, 8, SCALE,
-                                             oracle.POLICY_ONLINE, threads)
+                                             oracle.POLICY_ONLINE if self.score_rounding else oracle.POLICY_FP32,
+                                             threads)
         dt = time.perf_counter() - t0
         assert rc == 0
         err = float(np.max(np.abs(oracle.bf16_to_f32(out).astype(np.float64)
@@ -615,13 +691,16 @@ class PredictorLoop:
     name = "predictor_loop_256frames_5layers_16steps"
     bound = "hbm"
 
-    def __init__(self, qm, dev, seed=55, frames=256, layers=5, rows=16, write_cache=False):
+    def __init__(self, qm, dev, seed=55, frames=256, layers=5, rows=16, write_cache=False, kernel=0):
         import torch
         self.qm, self.units, self.layers, self.rows, self.frames = qm, frames * layers, layers, rows, frames
-        gd = torch.Generator(device=dev).manual_seed(seed)
+        self.kernel = kernel      # 0: products on the matrix cores; 1: every fp32 sum in the reference's order
+        # bf16 outputs of magnitude >= 2 are 0.0156 apart: a sum taken in another order can land one
+        # output spacing away, which is what the gate below allows the matrix-core kernel
+        self.tolerance = 1e-2 if kernel else 2e-2
+        syn = Synthetic(dev, seed)
 
-        def rnd(shape, std=1.0, mean=0.0):
-            return (torch.randn(shape, generator=gd, device=dev, dtype=torch.float32) * std + mean).to(torch.bfloat16)
+        rnd = syn.normal
 
         u = self.units
         self.q, self.k, self.v = rnd((u, rows, 16, 128)), rnd((u, rows, 8, 128)), rnd((u, rows, 8, 128))
@@ -638,12 +717,18 @@ class PredictorLoop:
         self.flops = 1114112 * u
         if write_cache:
             self.name += "_cache_writeback"
+        if kernel:
+            self.name += "_exact_chain"
 
     def step(self):
         import torch
-        self.qm.predictor_attention_loop(self.q, self.k, self.v, self.gq, self.gk, self.cos, self.sin, self.out,
-                                         self.kc, self.vc, self.units, self.layers, self.rows, 1, 1e-6,
-                                         torch.cuda.current_stream().cuda_stream)
+        self.qm.set_option(self.qm.OPT_PREDICTOR_LOOP_KERNEL, self.kernel)
+        try:
+            self.qm.predictor_attention_loop(self.q, self.k, self.v, self.gq, self.gk, self.cos, self.sin, self.out,
+                                             self.kc, self.vc, self.units, self.layers, self.rows, 1, 1e-6,
+                                             torch.cuda.current_stream().cuda_stream)
+        finally:
+            self.qm.set_option(self.qm.OPT_PREDICTOR_LOOP_KERNEL, 0)
 
     def cpu_baseline(self, oracle, threads):
         """Sample: the first 160 units (32 frames)."""
@@ -675,8 +760,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
-    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "predictor", "qkv", "layer",
-                                      "frame"], default=None,
+    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "prefillfp32", "predictor", "predictorexact",
+                                      "qkv", "layer", "frame"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -711,7 +796,9 @@ def main():
                 "talker2048": lambda: SingleDecode(qm, dev, 2048, True, 12),
                 "prefill": lambda: Prefill(qm, dev), "prefill1": lambda: Prefill(qm, dev, batch=1),
                 "prefill1split": lambda: Prefill(qm, dev, batch=1, split=True),
+                "prefillfp32": lambda: Prefill(qm, dev, score_rounding=0),
                 "predictor": lambda: PredictorLoop(qm, dev),
+                "predictorexact": lambda: PredictorLoop(qm, dev, kernel=1),
                 "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev),
                 "frame": lambda: PredictorFrameSteps(qm, dev)}[args.only]
         w = make()
@@ -743,10 +830,12 @@ def main():
             # the same step as the reference launches it: append kernel, then attention
             ("cfg2_talker_step_ctx2048_two_operators", lambda: SingleDecode(qm, dev, 2048, True, 12, one_launch=False)),
             ("cfg4_causal_prefill", lambda: Prefill(qm, dev)),
+            ("cfg4_causal_prefill_fp32_scores", lambda: Prefill(qm, dev, score_rounding=0)),
             # one prompt, as the talker's prefill runs it: 128 blocks for 256 CUs; the key-split entry fills them
             ("cfg4b_causal_prefill_one_prompt_1024", lambda: Prefill(qm, dev, batch=1)),
             ("cfg4b_causal_prefill_one_prompt_1024_key_split", lambda: Prefill(qm, dev, batch=1, split=True)),
             ("cfg5_predictor_loop", lambda: PredictorLoop(qm, dev)),
+            ("cfg5_predictor_loop_exact_chain", lambda: PredictorLoop(qm, dev, kernel=1)),
             ("cfg5_predictor_loop_cache_writeback", lambda: PredictorLoop(qm, dev, write_cache=True)),
             # beyond the five configurations: the M = 1 projection in front of configuration 2
             ("next_qkv_gemv_m1", lambda: QkvGemv(qm, dev)),
@@ -754,7 +843,7 @@ def main():
             # the whole decode step of one talker layer, 28 layers' weights and caches in rotation (2.8 GB)
             ("next_talker_layer_decode_step", lambda: TalkerLayerStep(qm, dev)),
             ("next_talker_layer_decode_step_unfused", lambda: TalkerLayerStep(qm, dev, fused=False)),
-            # the fourteen M = 1 steps of one code-predictor frame, operator by operator (406 launches)
+            # the fourteen M = 1 steps of one code-predictor frame, operator by operator (476 launches)
             ("next_predictor_frame_m1_steps", lambda: PredictorFrameSteps(qm, dev)),
         ]
         for key, make in extra:
@@ -806,6 +895,8 @@ def main():
                    "device": props.name, "compute_units": props.multi_processor_count},
         "roofline": {"bound": "hbm", "achieved": rep["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": rep["GBps"] / HBM_PEAK_GBPS, "traffic": HEADLINE_TRAFFIC_BYTES,
+                     "traffic_source": "profiles/decode_split_kernel_ragged64_traffic.txt (rocprofv3 --pmc FETCH_SIZE / "
+                                       "WRITE_SIZE of this workload; not measured in this run)",
                      "kernel": "decode_split_kernel<2, false, true> (+ decode_merge_kernel<2>, both inside the timed step)",
                      "algorithmic_bytes_per_launch": head.bytes, "avg_launch_us": ms * 1e3},
         "cpu_baseline": cpu,

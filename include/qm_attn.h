@@ -85,12 +85,10 @@ const char* qm_target_arch(void);
  *       scale > 0; outputs stay within the 1e-2 tolerance of the fp32 definition).
  *   QM_OPT_DECODE_TILES_PER_BLOCK  0 (default): the split-K decode picks the 16-token tiles per
  *       block from the problem size; > 0 forces it (changes qm_decode_workspace_bytes too).
- *   QM_OPT_PREFILL_KERNEL  0 (default): qm_prefill_attention_causal runs the fastest of its
- *       kernels (now 3); 1: four uniform waves per block; 2: four pairs of a matrix wave and a
- *       softmax wave per block; 3: four waves per block, each one software pipeline that alternates
- *       MFMAs with softmax arithmetic; 4: as 3 with 32 rows per wave (slower; for measurement).
- *       All give the same bits (a negative scale always runs kernel 1 in place of 3 and 4); other
- *       values make the call return QM_ERR_ARGUMENT.
+ *   QM_OPT_PREFILL_KERNEL  0 (default): qm_prefill_attention_causal runs four waves per block,
+ *       each one software pipeline that alternates MFMAs with softmax arithmetic; 1: four uniform
+ *       waves per block (the compiler's instruction order; also what a negative scale runs).  Same
+ *       bits either way; other values make the call return QM_ERR_ARGUMENT.
  *   QM_OPT_DECODE_STREAMING_LOADS  0 (default): the decode kernels read K and V with the
  *       non-temporal hint when the contexts of one call may exceed 512 MiB (twice the last-level
  *       cache: less than that is partly still cached from the step before), and with plain loads
@@ -307,7 +305,7 @@ int32_t qm_prefill_attention_causal(
  *     workspace: 256-byte aligned device memory.
  *   qm_prefill_attention_causal_split: workspace NULL or a shape that does not split: exactly
  *     qm_prefill_attention_causal; too small for the shape: QM_ERR_WORKSPACE.  Only the default
- *     kernel (QM_OPT_PREFILL_KERNEL 0 or 3) splits.  Two calls that overlap in time must not share
+ *     kernel (QM_OPT_PREFILL_KERNEL 0) splits.  Two calls that overlap in time must not share
  *     a workspace.  QM_STATUS_SPLIT_TIMEOUT in status_dev: a block gave up waiting for a partner's
  *     record (rows of that query tile are then not written).
  */

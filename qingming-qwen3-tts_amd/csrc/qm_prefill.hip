@@ -11,11 +11,15 @@
 // 8-slot blocks XOR-swizzled per 16 rows so both the transposing writes and the fragment reads
 // are conflict-free).
 //
-// Three kernels share this file and give the same bits: the uniform waves described here (the
-// compiler's order inside a wave: all MFMAs of a product, then all of the softmax arithmetic), the
-// wave pairs (matrix waves and softmax waves), and the interleaved waves, which alternate MFMAs
-// and softmax arithmetic instruction by instruction and are the ones the host launches by
-// default; their comments say what was measured.  This kernel stays within 256 registers and
+// Two kernels share this file and give the same bits: the uniform waves described here (the
+// compiler's order inside a wave: all MFMAs of a product, then all of the softmax arithmetic) and
+// the interleaved waves, which alternate MFMAs and softmax arithmetic instruction by instruction
+// and are the ones the host launches by default; their comments say what was measured.  (A third
+// design, blocks of four matrix waves paired with four softmax waves that hand the 32 x 32 chunks
+// over through LDS, gave the same bits at 37.7 us / 398 us for 4 x 1024 / 4 x 4096 tokens against
+// 30.5 / 316 for the interleaved waves: with phases of eight MFMAs and about 150 VALU instructions
+// the two kinds of work mostly took turns on a SIMD whoever issued them.  It is no longer part of
+// this file.)  This kernel stays within 256 registers and
 // 72 KB of LDS so that two blocks share a CU and fill each other's waits.
 // Variants of it that were measured and dropped (batch 4 x 1024 tokens / 4 x 4096 tokens, this
 // one: 42 us / 381 us): three LDS stages with 316 registers, one wave per SIMD (51 us / 467 us);
@@ -491,44 +495,8 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_causal_kernel(PrefillPa
 }
 
 
-// ======================================================================================================
-// The specialised kernel: matrix waves and softmax waves.
-//
-// A block is four pairs of waves, pair i on SIMD i (waves i and i + 4 of a block land on the
-// same SIMD), each pair owning 16 query rows x 2 heads: the matrix wave holds Q and O and runs
-// S^T = K Q^T and O^T += V^T P^T, the softmax wave turns S^T into P.  They hand the 32 x 32 chunk
-// over through LDS as a register image (the matrix wave's accumulator registers lane for lane:
-// no layout change, no bank conflict): in stage k of the block the matrix waves compute S^T of
-// chunk k and the P.V of chunk k - 2 while the softmax waves work on chunk k - 1; one barrier
-// ends a stage.  The softmax wave owns the running maximum and sum; when it raises a maximum
-// (lazily) it publishes the factor with the chunk and the matrix wave rescales O before using
-// that chunk.  The two roundings of the scores are done by the matrix wave, which publishes
-// the scaled scores as bf16.  All staging is the matrix waves' too, and costs them neither
-// registers nor arithmetic: K and V tiles go from global memory straight into rings of three
-// LDS buffers (global_load_lds), two tiles ahead, and V is transposed by the LDS read
-// (ds_read_b64_tr_b16).  The K fragments of a chunk are read during the stage before it.
-//
-// Measured against the kernel above (same results bit for bit): 37.7 us against 42.4 us for
-// batch 4 x 1024 tokens, 144.6 against 138.5 for 16 x 1024, 398 against 385 for 4 x 4096; with
-// fp32 scores 37.4 / 147.9 / 409 against 37.4 / 116.4 / 334.  A stage lasts about 1520 cycles
-// in either design.  Counters (4 x 4096): per SIMD and stage the MFMAs are busy for 490 cycles
-// and the VALU for 850, and for only 150 of these both at once: with phases this long (eight
-// MFMAs, then about 150 VALU instructions) the two kinds of work mostly take turns, whoever
-// issues them, and a stage costs about their sum.  What the pairs gain is latency (one block
-// per CU needs fewer blocks to fill the chip, and a block's own chain is shorter).
-constexpr int kSpThreads = 512;
 constexpr int kKR = kDim * 2;                                    // bytes of a K row in LDS (unpadded, slots swizzled)
-constexpr int kSpKTile = kBN * kKR;
-constexpr int kSpKBytes = 3 * kSpKTile;                          // ring of three K tiles (later the output staging area)
-constexpr int kSpVBytes = 3 * kSpKTile;                          // ring of three V tiles, row-major like K
-constexpr int kSpSxBytes = 4 * 2 * 4 * 64 * 16;                  // [pair][buffer][quarter][lane] 16 bytes
-constexpr int kSpPxBytes = 4 * 2 * 2 * 64 * 16;                  // [pair][buffer][16-key group][lane] 8 bf16
-constexpr int kSpAxBytes = 4 * 2 * 64 * 4;                       // [pair][buffer][lane] rescale factor
-constexpr int kSpFlagBytes = 4 * 2 * 4;                          // [pair][buffer] "O must be rescaled"
-constexpr int kSpLxBytes = 4 * 64 * 4;                           // [pair][lane] final row sums
-constexpr int kSpSmemBytes = kSpKBytes + kSpVBytes + kSpSxBytes + kSpPxBytes + kSpAxBytes + kSpFlagBytes + kSpLxBytes;
-static_assert(kSpKBytes >= 4 * 32 * kOS * 2, "the output staging area reuses the K ring");
-static_assert(kSpKTile >= kSpPxBytes, "the low halves of P of a first query tile live in the third V buffer");
+constexpr int kSpKTile = kBN * kKR;                              // one 64-key tile of K (or V, row-major like K) in LDS
 
 // s_waitcnt that waits until at most N vector-memory operations are outstanding (nothing else).
 template <int N>
@@ -543,498 +511,6 @@ __device__ __forceinline__ void lds_barrier() {
 }
 
 
-template <bool PRECISE, bool ROUND>
-__device__ __forceinline__ void prefill_sp_body(const PrefillParams& prm, const qm_kv_cache& cache,
-                                                unsigned char* sp_smem, int qt, int bh) {
-    unsigned char* lds_k = sp_smem;                                                          // [3][64 rows][256 B]
-    unsigned char* lds_v = sp_smem + kSpKBytes;                                              // [3][64 rows][256 B]
-    uint4* lds_sx = reinterpret_cast<uint4*>(sp_smem + kSpKBytes + kSpVBytes);               // [pair][buf][4][64]
-    uint4* lds_px = reinterpret_cast<uint4*>(sp_smem + kSpKBytes + kSpVBytes + kSpSxBytes);  // [pair][buf][2][64]
-    uint4* lds_plo = reinterpret_cast<uint4*>(lds_v + 2 * kSpKTile);                         // (first query tile only)
-    float* lds_ax = reinterpret_cast<float*>(sp_smem + kSpKBytes + kSpVBytes + kSpSxBytes + kSpPxBytes);
-    int* lds_flag = reinterpret_cast<int*>(sp_smem + kSpKBytes + kSpVBytes + kSpSxBytes + kSpPxBytes + kSpAxBytes);
-    float* lds_lx = reinterpret_cast<float*>(sp_smem + kSpKBytes + kSpVBytes + kSpSxBytes + kSpPxBytes + kSpAxBytes + kSpFlagBytes);
-
-    const int wave8 = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
-    const int pair = wave8 & 3;                              // rows 16*pair .. +15 of the query tile
-    const bool softmax_wave = wave8 >= 4;
-    const int tid = threadIdx.x & 255;                       // thread within its group of four waves
-    const int lane = tid & 63;
-    const int col = lane & 31;
-    const int grp = lane >> 5;
-
-    const int b = bh / prm.kv_heads;
-    const int kvh = bh % prm.kv_heads;
-    const int S = prm.seq;
-    const int q_heads = 2 * prm.kv_heads;
-    const int q0 = qt * kBM;
-    const int my_row = q0 + 16 * pair + (col & 15);
-    const int my_head = 2 * kvh + (col >> 4);
-    const int pair_last_row = q0 + 16 * pair + 15;
-
-    // exchange areas of this pair: scores (fp32: four quarters of four registers; bf16: two
-    // quarters of eight), probabilities, rescale factor, flag
-    uint4* my_sx = lds_sx + pair * 2 * 4 * 64 + lane;        // + (buf * 4 + quarter) * 64
-    uint4* my_px = lds_px + pair * 2 * 2 * 64 + lane;        // + (buf * 2 + kg) * 64
-    uint4* my_plo = lds_plo + pair * 2 * 2 * 64 + lane;      // likewise, the low halves
-    float* my_ax = lds_ax + pair * 2 * 64 + lane;            // + buf * 64
-    int* my_flag = lds_flag + pair * 2;                      // + buf
-
-    // A chunk (tile t, half h) of this pair: its first key, and whether the pair has work in it.
-    auto chunk_key_base = [&](int t, int h) { return t * kBN + 32 * h; };
-    auto chunk_active = [&](int t, int h) { return t < qt || chunk_key_base(t, h) <= pair_last_row; };
-
-    const int64_t kv_base = static_cast<int64_t>(b) * prm.kv_stride_batch + static_cast<int64_t>(kvh) * prm.kv_stride_head;
-    const int kv_row32 = static_cast<int>(prm.kv_stride_token);
-
-    if (!softmax_wave) {
-        // ================================ matrix wave ====================================================
-        // Staging: one global_load_lds instruction of a wave (16 bytes per lane, no registers) fills
-        // four consecutive 256-byte rows of a tile, lane l row l / 16, slot l % 16; which 16-byte
-        // piece of the key the lane fetches into that slot is the swizzle.  K: slot p of key row r
-        // holds piece p ^ (r % 16), so that the fragment reads of 16 consecutive rows fall on 16
-        // different slots.  V stays row-major too (slot p holds piece p ^ 4 (r % 4)) and is
-        // transposed by the LDS read (ds_read_b64_tr_b16).  A key at or beyond S is redirected to
-        // the last key; such keys only occur masked.
-        const int k_row = 4 * pair + (lane >> 4);                       // + 16 j: key row inside the tile
-        const uint16_t* k_src = prm.k + kv_base + 8 * ((lane & 15) ^ (k_row & 15));
-        const uint16_t* v_src = prm.v + kv_base + 8 * ((lane & 15) ^ (4 * (k_row & 3)));
-        // byte offsets of this lane's four rows from the first row of a tile (the host rejects
-        // seq * stride >= 2^31 elements)
-        const uint32_t row_bytes = static_cast<uint32_t>(kv_row32) * 2u;
-        const uint32_t lane_off0 = static_cast<uint32_t>(k_row) * row_bytes;
-        auto load_tile = [&](const uint16_t* src, unsigned char* ring, int tile, int slot) {
-            unsigned char* dst = ring + slot * kSpKTile + 4 * pair * kKR;
-            const unsigned char* base = reinterpret_cast<const unsigned char*>(src);
-            if (tile * kBN + kBN <= S) {
-                const unsigned char* tile_base = base + static_cast<uint64_t>(static_cast<uint32_t>(tile * kBN)) * row_bytes;
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    __builtin_amdgcn_global_load_lds(tile_base + (lane_off0 + 16u * j * row_bytes),
-                                                     (__attribute__((address_space(3))) void*)(dst + 16 * j * kKR), 16, 0, 0);
-            } else {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int key = min(tile * kBN + k_row + 16 * j, S - 1);
-                    __builtin_amdgcn_global_load_lds(base + static_cast<uint64_t>(static_cast<uint32_t>(key)) * row_bytes,
-                                                     (__attribute__((address_space(3))) void*)(dst + 16 * j * kKR), 16, 0, 0);
-                }
-            }
-        };
-        auto load_k = [&](int tile, int slot) { load_tile(k_src, lds_k, tile, slot); };
-        auto load_v = [&](int tile, int slot) { load_tile(v_src, lds_v, tile, slot); };
-
-        load_k(0, 0);
-        load_v(0, 0);
-        if (!PRECISE) load_k(1, 1);
-        bf16x8_t qf[8];
-        {
-            const uint16_t* qp = prm.q + ((static_cast<int64_t>(b) * S + my_row) * q_heads + my_head) * kDim + 8 * grp;
-#pragma unroll
-            for (int kb = 0; kb < 8; ++kb) {
-                uint4 raw = make_uint4(0, 0, 0, 0);
-                if (my_row < S) raw = *reinterpret_cast<const uint4*>(qp + 16 * kb);
-                qf[kb] = __builtin_bit_cast(bf16x8_t, raw);
-            }
-        }
-        f32x16_t o[4];
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o[dt][r] = 0.0f;
-        wait_vm<0>();   // K of tiles 0 and 1 and V of tile 0 have landed in LDS
-        lds_barrier();
-
-        // fragment of K for k block kb: row 32h + col, slot (2kb + grp) ^ (col % 16)
-        const int k_lane = col * kKR + 16 * (grp ^ (col & 15));
-        auto k_frags = [&](int slot, int h, bf16x8_t (&kf)[8]) {
-            const unsigned char* kp = lds_k + slot * kSpKTile + 32 * h * kKR;
-#pragma unroll
-            for (int kb = 0; kb < 8; ++kb) kf[kb] = *reinterpret_cast<const bf16x8_t*>(kp + (k_lane ^ (32 * kb)));
-        };
-        // V^T fragments by transposing reads.  One ds_read_b64_tr_b16 of 16 lanes takes a block of
-        // 4 keys x 16 dims (lane 4 j + q of the 16 addresses dims 4 q .. 4 q + 3 of key j) and gives
-        // lane i the four keys of dim i.  MFMA k index 8 * grp + e of 16-key group kg is key
-        // 16 kg + 8 (e / 4) + 4 grp + e % 4 (the S^T accumulator's order), so the fragment of lane
-        // (dim col, grp) is two such reads, keys 16 kg + 4 grp + 0..3 and + 8.
-        const int tr_key = (lane >> 2) & 3;                              // this lane's key within a block (= key % 4)
-        const int v_lane = (4 * grp + tr_key) * kKR + 16 * (2 * (col >> 4) + ((lane & 3) >> 1)) + 8 * (lane & 1);
-        // The reads are written as assembly: the compiler makes a transposing read wait for every
-        // global_load_lds in flight (it cannot tell that they fill other buffers), which would
-        // expose the whole memory latency once per tile.  It does not see these reads as LDS
-        // traffic, so their results are taken only through v_arrived(), which waits for them.
-        const uint32_t v_addr0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
-                                     (__attribute__((address_space(3))) unsigned char*)lds_v)) + v_lane;
-        struct VRaw { unsigned long long a[8], c[8]; };
-        // fragment j = (group kg = j / 4, dim tile dt = j % 4) of chunk h of the tile in buffer `slot`
-        auto v_request = [&](int slot, auto half, VRaw& raw) {
-            constexpr int h = decltype(half)::value;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int kg = j >> 2, dt = j & 3;
-                const uint32_t at = (v_addr0 + slot * kSpKTile) ^ (64 * (dt ^ tr_key));
-                asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(raw.a[j]) : "v"(at), "n"((32 * h + 16 * kg) * kKR));
-                asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(raw.c[j]) : "v"(at), "n"((32 * h + 16 * kg + 8) * kKR));
-            }
-        };
-        auto v_arrived = [&](VRaw& raw, bf16x8_t (&vf)[8]) {
-            asm volatile("s_waitcnt lgkmcnt(0)"
-                         : "+v"(raw.a[0]), "+v"(raw.a[1]), "+v"(raw.a[2]), "+v"(raw.a[3]), "+v"(raw.a[4]), "+v"(raw.a[5]),
-                           "+v"(raw.a[6]), "+v"(raw.a[7]), "+v"(raw.c[0]), "+v"(raw.c[1]), "+v"(raw.c[2]), "+v"(raw.c[3]),
-                           "+v"(raw.c[4]), "+v"(raw.c[5]), "+v"(raw.c[6]), "+v"(raw.c[7])
-                         :
-                         : "memory");
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint4 both_halves = make_uint4(static_cast<uint32_t>(raw.a[j]), static_cast<uint32_t>(raw.a[j] >> 32),
-                                                     static_cast<uint32_t>(raw.c[j]), static_cast<uint32_t>(raw.c[j] >> 32));
-                vf[j] = __builtin_bit_cast(bf16x8_t, both_halves);
-            }
-        };
-        auto s_mfma = [&](const bf16x8_t (&kf)[8], f32x16_t& s) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s[r] = 0.0f;
-#pragma unroll
-            for (int kb = 0; kb < 8; ++kb) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb], qf[kb], s, 0, 0, 0);
-        };
-        // (assembly for the same reason as the transposing reads: the compiler would drain the
-        // global_load_lds in flight before an LDS write; the stage's barrier waits for the write)
-        typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-        const uint32_t sx_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint4*)my_sx));
-        // (when it stores an MFMA's registers directly, the assembly keeps that instruction's wait states itself)
-        auto sx_write = [&](int quarter, const uint4& value) {
-            const u32x4_t data = {value.x, value.y, value.z, value.w};
-            if (ROUND) asm volatile("ds_write_b128 %0, %1" : : "v"(sx_addr + quarter * 1024), "v"(data) : "memory");
-            else asm volatile("s_nop 15\n\ts_nop 3\n\tds_write_b128 %0, %1" : : "v"(sx_addr + quarter * 1024), "v"(data) : "memory");
-        };
-        // The scores of a chunk for the softmax wave: rounded, scaled and rounded again, as packed
-        // bf16 (ROUND), or the raw dot products.
-        auto s_publish = [&](int h, const f32x16_t& s) {
-            if (ROUND) {
-                uint32_t w[8];
-#pragma unroll
-                for (int r = 0; r < 16; r += 2) {
-                    float x0, x1;
-                    round_bf16_pair(s[r], s[r + 1], x0, x1);
-                    w[r >> 1] = pack_bf16_pair(x0 * prm.scale, x1 * prm.scale);
-                }
-                sx_write(h * 4 + 0, make_uint4(w[0], w[1], w[2], w[3]));
-                sx_write(h * 4 + 1, make_uint4(w[4], w[5], w[6], w[7]));
-            } else {
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4)
-                    sx_write(h * 4 + r4, make_uint4(__float_as_uint(s[4 * r4]), __float_as_uint(s[4 * r4 + 1]),
-                                                    __float_as_uint(s[4 * r4 + 2]), __float_as_uint(s[4 * r4 + 3])));
-            }
-        };
-        auto rescale = [&](float alpha) {
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
-        };
-        // S^T of chunk h of the tile in K buffer `slot` into exchange buffer h
-        auto qk = [&](int slot, int h) {
-            bf16x8_t kf[8];
-            f32x16_t s;
-            k_frags(slot, h, kf);
-            s_mfma(kf, s);
-            s_publish(h, s);
-        };
-        // O^T += V^T P^T of chunk (t, h) from exchange buffer h.  On the diagonal a 16-key group
-        // that lies wholly after the pair's last row is masked for every column: it is skipped,
-        // so that later tokens are not even multiplied by zero.
-        auto pv = [&](int t, int slot, int h) {
-            const bool diag = t == qt;
-            const int key_base = chunk_key_base(t, h);
-            bf16x8_t vf[8];
-            VRaw raw;
-            const int flag = __builtin_amdgcn_readfirstlane(my_flag[h]);
-            const float alpha = my_ax[h * 64];
-            if (h == 0) v_request(slot, int_c<0>{}, raw);
-            else v_request(slot, int_c<1>{}, raw);
-            if (flag) rescale(alpha);
-            v_arrived(raw, vf);
-#pragma unroll
-            for (int kg = 0; kg < 2; ++kg) {
-                if (diag && key_base + 16 * kg > pair_last_row) continue;
-                const bf16x8_t phi = __builtin_bit_cast(bf16x8_t, my_px[(h * 2 + kg) * 64]);
-                if (!PRECISE) {
-#pragma unroll
-                    for (int dt = 0; dt < 4; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * kg + dt], phi, o[dt], 0, 0, 0);
-                } else {
-                    const bf16x8_t plo = __builtin_bit_cast(bf16x8_t, my_plo[(h * 2 + kg) * 64]);
-#pragma unroll
-                    for (int dt = 0; dt < 4; ++dt) {
-                        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * kg + dt], phi, o[dt], 0, 0, 0);
-                        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * kg + dt], plo, o[dt], 0, 0, 0);
-                    }
-                }
-            }
-        };
-        // The steady state: S^T of chunk (t, h) and the P.V of chunk (t - 1, h), which is not on
-        // the diagonal.  Every LDS read is requested before the first MFMA; the scores are
-        // published between the two groups of MFMAs, so that their write is under way while the
-        // second group runs.
-        // `kf` holds the K fragments of this chunk, read during the stage before; `prefetch` reads
-        // those of the next one into it while the P.V MFMAs run.
-        auto both = [&](int slot_before, auto half, bf16x8_t (&kf)[8], auto&& prefetch) {
-            constexpr int h = decltype(half)::value;
-            bf16x8_t vf[8];
-            VRaw raw;
-            f32x16_t s;
-            const int flag = __builtin_amdgcn_readfirstlane(my_flag[h]);
-            const float alpha = my_ax[h * 64];
-            const bf16x8_t p0 = __builtin_bit_cast(bf16x8_t, my_px[(h * 2 + 0) * 64]);
-            const bf16x8_t p1 = __builtin_bit_cast(bf16x8_t, my_px[(h * 2 + 1) * 64]);
-            v_request(slot_before, half, raw);
-            s_mfma(kf, s);
-            s_publish(h, s);
-            if (flag) rescale(alpha);
-            v_arrived(raw, vf);
-            prefetch();
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt], p0, o[dt], 0, 0, 0);
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 + dt], p1, o[dt], 0, 0, 0);
-        };
-
-        // stage 2t + h: S^T of chunk (t, h) and the P.V of chunk (t - 1, h); tile qt + 1 drains.
-        // Tile t lives in buffer t % 3 of either ring.  At the start of tile t this wave requests K
-        // of tile t + 2 (into the buffer of tile t - 1, whose S^T is done) and V of tile t + 1 (into
-        // the buffer of tile t - 2, whose P.V is done); both are first read two tiles later, and
-        // vector-memory operations complete in order, so at the end of a tile everything but
-        // what that tile requested must have landed.
-        if (!PRECISE) {
-            if (qt >= 2) load_k(2, 2);
-            load_v(1, 1);
-        }
-        qk(0, 0);
-        lds_barrier();
-        if (chunk_active(0, 1)) qk(0, 1);
-        lds_barrier();
-        int slot = 0;                                     // buffer of the current tile
-        if (!PRECISE) {
-            int before = 0;                               // buffer of the tile before it
-            slot = 1;
-            bf16x8_t kf[8];                               // K fragments of the coming chunk
-            k_frags(1, 0, kf);
-            for (int t = 1; t < qt; ++t) {
-                const int after = slot == 2 ? 0 : slot + 1;
-                const bool more = t + 2 <= qt;
-                if (more) load_k(t + 2, before);
-                both(before, int_c<0>{}, kf, [&]() { k_frags(slot, 1, kf); });
-                // K of tile t + 1 is read from the second half of this tile on: only V of tile t
-                // and what this half requested may still be on their way
-                if (more) wait_vm<8>();
-                else wait_vm<4>();
-                lds_barrier();
-                load_v(t + 1, after);
-                both(before, int_c<1>{}, kf, [&]() { k_frags(after, 0, kf); });
-                // V of tile t is read from the next tile on
-                if (more) wait_vm<8>();
-                else wait_vm<4>();
-                lds_barrier();
-                before = slot;
-                slot = after;
-            }
-            // the diagonal tile: its first chunk concerns every pair, its second one only some
-            both(before, int_c<0>{}, kf, [&]() { k_frags(slot, 1, kf); });
-            wait_vm<0>();
-            lds_barrier();
-            if (chunk_active(qt, 1)) both(before, int_c<1>{}, kf, []() {});
-            else pv(qt - 1, before, 1);
-            lds_barrier();
-        }
-        pv(qt, slot, 0);
-        lds_barrier();
-        if (chunk_active(qt, 1)) pv(qt, slot, 1);
-        lds_barrier();
-        lds_barrier();   // the softmax waves have published the row sums
-
-        // ---- normalise, stage through LDS (the K ring is free), write 16 bytes per lane ---------------
-        const float l_tot = lds_lx[pair * 64 + lane] + lds_lx[pair * 64 + (lane ^ 32)];
-        const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-        uint16_t* stage = reinterpret_cast<uint16_t*>(sp_smem) + pair * 32 * kOS;
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-#pragma unroll
-            for (int rq = 0; rq < 4; ++rq) {
-                const int d0 = 32 * dt + 8 * rq + 4 * grp;
-                uint2 packed;
-                packed.x = pack_bf16_pair(o[dt][4 * rq + 0] * inv, o[dt][4 * rq + 1] * inv);
-                packed.y = pack_bf16_pair(o[dt][4 * rq + 2] * inv, o[dt][4 * rq + 3] * inv);
-                *reinterpret_cast<uint2*>(&stage[col * kOS + d0]) = packed;
-            }
-        }
-        __builtin_amdgcn_s_waitcnt(0);   // the wave reads back only what it wrote itself
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int it = 0; it < 8; ++it) {
-            const int c = 4 * it + (lane >> 4);
-            const int piece = lane & 15;
-            const int row = q0 + 16 * pair + (c & 15);
-            const int head = 2 * kvh + (c >> 4);
-            if (row < S) {
-                const uint4 val = *reinterpret_cast<const uint4*>(&stage[c * kOS + 8 * piece]);
-                *reinterpret_cast<uint4*>(prm.out + ((static_cast<int64_t>(b) * S + row) * q_heads + head) * kDim + 8 * piece) = val;
-            }
-        }
-    } else {
-        // ================================ softmax wave ===================================================
-        const float coef = ROUND ? kLog2e : prm.scale * kLog2e;
-        const float slack = ROUND ? kRescaleSlack : kRescaleSlack / prm.scale;
-        float m_run = -INFINITY, l_run = 0.0f, m_scaled = 0.0f;
-
-        // These waves have nothing to compute until the first S^T exists: they copy the K/V rows
-        // of the diagonal tile to the pages.  Thread: keys (tid >> 4) + 16 i, dims 8 * (tid % 16);
-        // requested before the first barrier, written after it.
-        const bool to_pages = prm.has_cache != 0;
-        int phys[4] = {-1, -1, -1, -1};
-        uint4 kx[4], vx[4];
-        uint32_t page_err = 0;
-        if (to_pages) {
-            const int32_t* table = prm.page_table ? prm.page_table + static_cast<int64_t>(b) * prm.pages.max_pages : nullptr;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = qt * kBN + (tid >> 4) + 16 * i;
-                kx[i] = vx[i] = make_uint4(0, 0, 0, 0);
-                if (key < S) {
-                    const int page = page_of(prm.pages, key);
-                    if (page >= prm.pages.max_pages) page_err |= QM_STATUS_BAD_POSITION;
-                    else phys[i] = table ? table[page] : page;
-                    const int64_t off = kv_base + static_cast<int64_t>(key) * prm.kv_stride_token + 8 * (tid & 15);
-                    kx[i] = *reinterpret_cast<const uint4*>(prm.k + off);
-                    vx[i] = *reinterpret_cast<const uint4*>(prm.v + off);
-                }
-            }
-        }
-        lds_barrier();   // matches the matrix waves' barrier after tile 0 of K
-        if (to_pages) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = qt * kBN + (tid >> 4) + 16 * i;
-                if (key >= S || phys[i] == -1) continue;
-                if (phys[i] < 0 || phys[i] >= cache.n_pages) {
-                    page_err |= QM_STATUS_BAD_PAGE;
-                    continue;
-                }
-                const int page = page_of(prm.pages, key);
-                const int64_t off = static_cast<int64_t>(phys[i]) * cache.stride_page + static_cast<int64_t>(kvh) * cache.stride_head
-                                  + static_cast<int64_t>(key - page * prm.pages.page_size) * kDim + 8 * (tid & 15);
-                *reinterpret_cast<uint4*>(cache.k_pool + off) = kx[i];
-                *reinterpret_cast<uint4*>(cache.v_pool + off) = vx[i];
-            }
-            if (page_err && prm.status) atomicOr(prm.status, page_err);
-        }
-
-        // scores of chunk (t, h) -> P, from and to exchange buffer h
-        auto softmax = [&](int t, int h, auto masked) {
-            const int key_base = chunk_key_base(t, h);
-            float s[16];
-            if (ROUND) {
-                const uint4 w0 = my_sx[(h * 4 + 0) * 64];
-                const uint4 w1 = my_sx[(h * 4 + 1) * 64];
-                const uint32_t w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-#pragma unroll
-                for (int r = 0; r < 16; r += 2) {
-                    s[r] = lo_bf16(w[r >> 1]);
-                    s[r + 1] = hi_bf16(w[r >> 1]);
-                }
-            } else {
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    const uint4 v4 = my_sx[(h * 4 + r4) * 64];
-                    s[4 * r4] = __uint_as_float(v4.x); s[4 * r4 + 1] = __uint_as_float(v4.y);
-                    s[4 * r4 + 2] = __uint_as_float(v4.z); s[4 * r4 + 3] = __uint_as_float(v4.w);
-                }
-            }
-            // accumulator register r of lane group grp is key key_base + 8*(r/4) + 4*grp + r%4
-            const int lim = my_row - key_base - 4 * grp;
-            float mx = -INFINITY;
-#pragma unroll
-            for (int r = 0; r < 16; r += 2) {
-                if (decltype(masked)::value) {
-                    const int e = 8 * (r >> 2) + (r & 3);
-                    if (e > lim) s[r] = -INFINITY;
-                    if (e + 1 > lim) s[r + 1] = -INFINITY;
-                }
-                mx = fmaxf(mx, fmaxf(s[r], s[r + 1]));
-            }
-            mx = halves_max(mx);
-            // raise the running maximum if some column of the pair exceeds it by more than the slack
-            const bool need = __builtin_amdgcn_ballot_w64(mx > m_run + slack) != 0;
-            if (need) {
-                const float m_new = fmaxf(m_run, mx);
-                const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
-                const float alpha = fast_exp2((m_run - m_ref) * coef);
-                m_run = m_new;
-                m_scaled = m_ref * coef;
-                l_run *= alpha;
-                my_ax[h * 64] = alpha;
-            }
-            if (lane == 0) my_flag[h] = need ? 1 : 0;
-            uint32_t hi[8], lo[8];
-            float psum = 0.0f;
-#pragma unroll
-            for (int r = 0; r < 16; r += 2) {
-                const float e0 = fast_exp2(fmaf(s[r], coef, -m_scaled));
-                const float e1 = fast_exp2(fmaf(s[r + 1], coef, -m_scaled));
-                hi[r >> 1] = pack_bf16_pair(e0, e1);
-                if (PRECISE) {
-                    lo[r >> 1] = pack_bf16_pair(e0 - lo_bf16(hi[r >> 1]), e1 - hi_bf16(hi[r >> 1]));
-                    psum += e0 + e1;
-                } else {
-                    psum = dot2_bf16(hi[r >> 1], 0x3f803f80U, psum);   // the sum of what the MFMA multiplies
-                }
-            }
-            l_run += psum;
-            my_px[(h * 2 + 0) * 64] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-            my_px[(h * 2 + 1) * 64] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
-            if (PRECISE) {
-                my_plo[(h * 2 + 0) * 64] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-                my_plo[(h * 2 + 1) * 64] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
-            }
-        };
-
-        // stage 2t + h: the softmax of the chunk before (t, h)
-        lds_barrier();                                   // stage (0, 0): nothing to do yet
-        if (PRECISE) {
-            softmax(0, 0, bool_c<true>{});
-            lds_barrier();
-        } else {
-            softmax(0, 0, bool_c<false>{});
-            lds_barrier();
-            for (int t = 1; t < qt; ++t) {
-                softmax(t - 1, 1, bool_c<false>{});
-                lds_barrier();
-                softmax(t, 0, bool_c<false>{});
-                lds_barrier();
-            }
-            softmax(qt - 1, 1, bool_c<false>{});
-            lds_barrier();
-            softmax(qt, 0, bool_c<true>{});
-            lds_barrier();
-        }
-        if (chunk_active(qt, 1)) softmax(qt, 1, bool_c<true>{});
-        lds_barrier();
-        lds_barrier();                                   // the matrix waves drain
-        lds_lx[pair * 64 + lane] = l_run;
-        lds_barrier();
-    }
-}
-
-template <bool ROUND>
-__global__ __launch_bounds__(kSpThreads, 2) void prefill_sp_kernel(PrefillParams prm, qm_kv_cache cache) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char sp_smem[];
-    const int pairs = prm.batch * prm.kv_heads;
-    const int bid = blockIdx.x;
-    const int qt = prm.n_qtiles - 1 - bid / pairs;          // heaviest query tile first
-    if (qt == 0) prefill_sp_body<true, ROUND>(prm, cache, sp_smem, 0, bid % pairs);
-    else prefill_sp_body<false, ROUND>(prm, cache, sp_smem, qt, bid % pairs);
-}
-
-
 // ======================================================================================================
 // The interleaved kernel: each of the four waves of a block runs the matrix and the softmax work
 // of its NC column groups (16 rows x 2 heads each) as ONE software-pipelined instruction stream.
@@ -1046,8 +522,8 @@ __global__ __launch_bounds__(kSpThreads, 2) void prefill_sp_kernel(PrefillParams
 // holds three things that do not depend on one another: the P.V MFMAs of chunk j - 1, the
 // softmax arithmetic of chunk j, and the S^T MFMAs of chunk j + 1; the source alternates MFMAs
 // with slices of the softmax and pins that order with scheduling fences (see the stage).
-// Staging is that of the wave pairs (K and V tiles go straight from global memory into LDS, V is
-// transposed by the LDS read) with two buffers per ring and one block barrier per 64-key tile:
+// K and V tiles go straight from global memory into LDS (global_load_lds: no registers, no
+// arithmetic), V is transposed by the LDS read, with two buffers per ring and one block barrier per 64-key tile:
 // 64 KiB of LDS, so that two blocks share a CU.  The block's own (diagonal) tiles are finished
 // outside the pipeline, and blocks of the first query tile (split-precision P) run the
 // uniform-waves body.
@@ -1064,7 +540,7 @@ __global__ __launch_bounds__(kSpThreads, 2) void prefill_sp_kernel(PrefillParams
 // the pages and the first S^T, 5 800 on its own tiles, the last barrier and the output), which is
 // 40 % of the 4 x 1024 case, where the whole grid is resident at once and nothing hides it.
 // Two column groups per wave (NC = 2: half the LDS reads per MFMA, 500 registers, one wave per
-// SIMD) are slower (4 x 1024: 58 us, 4 x 4096: 389 us) and stay selectable for measurement only.
+// SIMD) were slower (4 x 1024: 58 us, 4 x 4096: 389 us); the body keeps NC as a parameter, only NC = 1 is built.
 constexpr int kIlRing = 2 * kSpKTile;                       // two tiles of K, likewise of V
 constexpr int kIlSmemBytes = (2 * kIlRing > static_cast<int>(sizeof(PfStage)) * kPfStages)
                                  ? 2 * kIlRing : static_cast<int>(sizeof(PfStage)) * kPfStages;
@@ -1151,8 +627,12 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         }
     }
 
-    // ---- staging: as in the wave pairs (slot p of K row r holds piece p ^ (r % 16), of V row r piece
-    // p ^ 4 (r % 4)); wave w fills rows 4 w + l / 16 + 16 j of a tile ----
+    // ---- staging: one global_load_lds of a wave (16 bytes per lane) fills four consecutive 256-byte rows of a
+    // tile, lane l row l / 16, slot l % 16; which 16-byte piece of the key the lane fetches into that slot is
+    // the swizzle.  Slot p of K row r holds piece p ^ (r % 16), so that the fragment reads of 16 consecutive
+    // rows fall on 16 different slots; V stays row-major too (slot p of row r holds piece p ^ 4 (r % 4)) and is
+    // transposed by the LDS read.  A key at or beyond S is redirected to the last key; such keys only occur
+    // masked.  Wave w fills rows 4 w + l / 16 + 16 j of a tile ----
     const int k_row = 4 * wave + (lane >> 4);
     const uint16_t* k_src = prm.k + kv_base + 8 * ((lane & 15) ^ (k_row & 15));
     const uint16_t* v_src = prm.v + kv_base + 8 * ((lane & 15) ^ (4 * (k_row & 3)));
@@ -1221,7 +701,10 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
     // global_load_lds in flight, and it must not move them across the barriers either.  Their results
     // are taken only through the *_arrived statements, which wait for them. ----
     // K fragment kb of chunk (slot, h): row 32 h + col, slot (2 kb + grp) ^ (col % 16).
-    // V^T fragment (kg, dt): two transposing reads, keys 16 kg + 4 grp + 0..3 and + 8 (see the wave pairs).
+    // V^T fragment (kg, dt): one ds_read_b64_tr_b16 of 16 lanes takes a block of 4 keys x 16 dims (lane 4 j + q of
+    // the 16 addresses dims 4 q .. 4 q + 3 of key j) and gives lane i the four keys of dim i.  MFMA k index
+    // 8 grp + e of 16-key group kg is key 16 kg + 8 (e / 4) + 4 grp + e % 4 (the S^T accumulator's order), so the
+    // fragment of lane (dim col, grp) is two such reads, keys 16 kg + 4 grp + 0..3 and + 8.
     uint32_t kaddr[8], vaddr[4];
     {
         const uint32_t k0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)lds_k))
@@ -1716,9 +1199,14 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
             __hip_atomic_store(record + 65 * kPfThreads, l_run[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             wait_vm<0>();                            // the stores have been acknowledged
             __syncthreads();
-            // (every store of the record is an agent-scope atomic store that has been acknowledged, for every
-            // wave of the block, before the flag is stored; the flag carries the launch's epoch)
-            if (tid == 0) __hip_atomic_store(&tickets[1 + part], prm.split_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            // Publication order without a release fence: every store of the record is an agent-scope atomic store
+            // (written through to where every XCD of the device reads it), each wave has waited for the
+            // acknowledgement of its own stores (vmcnt 0) before the block barrier above, and the flag, which
+            // carries the launch's epoch, is stored after that barrier.  A release on the flag would add a
+            // write-back of every dirty line of this XCD's L2 (the output rows and cache pages of all the blocks
+            // that run beside this one) in front of it: measured 25.2 us against 20.3 us for one prompt of 1024
+            // tokens, with nothing in the record left for that write-back to publish.
+            if (tid == 0) __hip_atomic_store(&tickets[1 + part], prm.split_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             return;
         }
         if (tid == 0) {
@@ -1999,19 +1487,16 @@ static int32_t prefill_attention_entry(
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     const bool round_scores = option_value(QM_OPT_PREFILL_SCORE_ROUNDING) != 0;
     if (!round_scores && !(scale > 0.0f)) return QM_ERR_ARGUMENT;   // the scale is folded into the exponent there
-    // 0 and 3: the interleaved waves (fastest at every size measured); 1: uniform waves; 2: wave pairs
+    // 0: the interleaved waves (fastest at every size measured); 1: the uniform waves
     const int which = option_value(QM_OPT_PREFILL_KERNEL);
-    if (which < 0 || which > 4) return QM_ERR_ARGUMENT;
+    if (which < 0 || which > 1) return QM_ERR_ARGUMENT;
     // (its running maximum is taken before the scores are scaled: a negative scale goes to the uniform waves)
-    if ((which == 0 || which >= 3) && scale >= 0.0f) {
-        const int groups = which == 4 ? 2 : 1;                     // column groups (16 rows x 2 heads) per wave
+    if (which == 0 && scale >= 0.0f) {
         int compute_units = 0;
         const int32_t rc_cu = device_compute_units(&compute_units);
         if (rc_cu != QM_OK) return rc_cu;
-        prm.n_qtiles = (seq + kBM * groups - 1) / (kBM * groups);
-        prm.heavy_groups = prm.n_qtiles;
         int64_t blocks = pairs * prm.n_qtiles;
-        const SplitPlan split = groups == 1 && workspace ? plan_split(pairs, seq, compute_units) : SplitPlan();
+        const SplitPlan split = workspace ? plan_split(pairs, seq, compute_units) : SplitPlan();
         if (split.chunk > 0) {
             if (workspace_bytes < split.bytes) return QM_ERR_WORKSPACE;
             static std::atomic<uint32_t> launches{0};
@@ -2021,33 +1506,17 @@ static int32_t prefill_attention_entry(
             prm.split_tickets = static_cast<int*>(workspace);
             prm.split_partials = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + split.ticket_bytes);
             blocks = pairs * split.groups;
-        } else if (groups == 1 && compute_units % pairs == 0 && blocks > compute_units && blocks <= 2 * static_cast<int64_t>(compute_units)) {
+        } else if (compute_units % pairs == 0 && blocks > compute_units && blocks <= 2 * static_cast<int64_t>(compute_units)) {
             prm.heavy_groups = static_cast<int>(compute_units / pairs);
         }
-        static std::atomic<bool> lds_raised[4][kMaxDevices];
-        const void* kernel = groups == 2
-            ? (round_scores ? reinterpret_cast<const void*>(prefill_il_kernel<true, 2>) : reinterpret_cast<const void*>(prefill_il_kernel<false, 2>))
-            : (round_scores ? reinterpret_cast<const void*>(prefill_il_kernel<true, 1>) : reinterpret_cast<const void*>(prefill_il_kernel<false, 1>));
-        const int32_t rc_lds = ensure_dynamic_lds(kernel, kIlSmemBytes, lds_raised[(groups - 1) * 2 + (round_scores ? 1 : 0)]);
+        static std::atomic<bool> lds_raised[2][kMaxDevices];
+        const void* kernel = round_scores ? reinterpret_cast<const void*>(prefill_il_kernel<true, 1>)
+                                          : reinterpret_cast<const void*>(prefill_il_kernel<false, 1>);
+        const int32_t rc_lds = ensure_dynamic_lds(kernel, kIlSmemBytes, lds_raised[round_scores ? 1 : 0]);
         if (rc_lds != QM_OK) return rc_lds;
         const dim3 grid(static_cast<unsigned>(blocks));
-        if (groups == 2) {
-            if (round_scores) hipLaunchKernelGGL((prefill_il_kernel<true, 2>), grid, dim3(kPfThreads), kIlSmemBytes, s, prm, desc);
-            else hipLaunchKernelGGL((prefill_il_kernel<false, 2>), grid, dim3(kPfThreads), kIlSmemBytes, s, prm, desc);
-        } else {
-            if (round_scores) hipLaunchKernelGGL((prefill_il_kernel<true, 1>), grid, dim3(kPfThreads), kIlSmemBytes, s, prm, desc);
-            else hipLaunchKernelGGL((prefill_il_kernel<false, 1>), grid, dim3(kPfThreads), kIlSmemBytes, s, prm, desc);
-        }
-        return launch_status();
-    }
-    const bool wave_pairs = which == 2;
-    if (wave_pairs) {
-        const auto kernel = round_scores ? prefill_sp_kernel<true> : prefill_sp_kernel<false>;
-        static std::atomic<bool> lds_raised[2][kMaxDevices];
-        const int32_t rc_lds = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), kSpSmemBytes,
-                                                  lds_raised[round_scores ? 1 : 0]);
-        if (rc_lds != QM_OK) return rc_lds;
-        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(pairs * n_qtiles)), dim3(kSpThreads), kSpSmemBytes, s, prm, desc);
+        if (round_scores) hipLaunchKernelGGL((prefill_il_kernel<true, 1>), grid, dim3(kPfThreads), kIlSmemBytes, s, prm, desc);
+        else hipLaunchKernelGGL((prefill_il_kernel<false, 1>), grid, dim3(kPfThreads), kIlSmemBytes, s, prm, desc);
         return launch_status();
     }
     const size_t smem = sizeof(PfStage) * kPfStages;
