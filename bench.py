@@ -467,7 +467,7 @@ class PredictorFrameSteps:
     reference chains them (PersistentPredictor::capture_step, R17:13592-13854): input projection,
     five layers (RMSNorm + Q/K/V, QK-norm + RoPE + append + attention over the [8][16][128] cache,
     o_proj, residual add + post-norm + gate/up/SwiGLU, down_proj + residual), final norm + that
-    step's head, top-k sampler, embedding gather feeding the next step.  34 launches per step with
+    step's head, top-k sampler, embedding gather feeding the next step.  29 launches per step with
     the fused operators (the reference: 46 graph nodes per M = 1 step).  Geometry R17:7951-7962;
     weights random.  One `step()` is the whole frame."""
     bound = "hbm"
@@ -512,7 +512,7 @@ class PredictorFrameSteps:
         self.ws_bytes = qm.decode_workspace_bytes(1, 16, 8, 16)
         self.ws = torch.empty(self.ws_bytes // 4 + 1, dtype=torch.float32, device=dev)
         layer_w = 2 * (Q * H + 2 * KV * H + H * Q + 2 * I * H + H * I)
-        self.launches_per_step = 1 + 5 * 6 + 3
+        self.launches_per_step = 1 + 5 * 5 + 3
         self.bytes = 14 * (5 * layer_w + 2 * H * OUT + 2 * V * H + 2 * OUT)          # weights streamed once per step
         self.flops = self.bytes
         self.copies = 14
@@ -526,12 +526,10 @@ class PredictorFrameSteps:
         for L in self.layers:
             qm.predictor_rmsnorm_qkv_m1(cur, L["in_norm"], L["wq"], L["wk"], L["wv"], self.q, self.k_, self.v_, H, Q, KV,
                                         1e-6, s)
-            # the engine's pair of operators: append at `position`, then attention on the reference's exact chain
-            # (one launch more than the fused decode step, whose sums are ordered differently: a sampled code
-            # must not depend on that)
-            qm.qk_norm_rope_kv_append(self.q, self.k_, self.v_, L["gq"], L["gk"], self.cos[position], self.sin[position],
-                                      self.qrot, L["cache"], None, 1, 16, position, 1e-6, s)
-            qm.predictor_attention_staged(self.qrot, L["k"], L["v"], self.ctxv, 1, position + 1, False, s)
+            # append at `position` + attention on the reference's exact chain, one launch (the fused decode step
+            # orders its sums differently: a sampled code must not depend on that)
+            qm.predictor_step_attention_m1(self.q, self.k_, self.v_, L["gq"], L["gk"], self.cos[position],
+                                           self.sin[position], L["k"], L["v"], self.ctxv, position, 1e-6, s)
             qm.predictor_linear_m1(self.ctxv, L["wo"], None, self.attn, H, Q, s)
             qm.predictor_add_postnorm_gate_up_swiglu_m1(cur, self.attn, L["post"], self.res, L["wg"], L["wu"], self.act,
                                                         H, I, 1e-6, s)
@@ -843,7 +841,7 @@ def main():
             # the whole decode step of one talker layer, 28 layers' weights and caches in rotation (2.8 GB)
             ("next_talker_layer_decode_step", lambda: TalkerLayerStep(qm, dev)),
             ("next_talker_layer_decode_step_unfused", lambda: TalkerLayerStep(qm, dev, fused=False)),
-            # the fourteen M = 1 steps of one code-predictor frame, operator by operator (476 launches)
+            # the fourteen M = 1 steps of one code-predictor frame, operator by operator (406 launches)
             ("next_predictor_frame_m1_steps", lambda: PredictorFrameSteps(qm, dev)),
         ]
         for key, make in extra:

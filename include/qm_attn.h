@@ -364,6 +364,23 @@ int32_t qm_predictor_attention_staged(
     void* hip_stream);
 
 /*
+ * One M = 1 step of a predictor layer between the Q/K/V projection and o_proj in one launch: replaces the pair
+ * PersistentPredictor::qk_norm_rope_cache_m1 + attention_m1 (R17:13432-13520, call site R17:13633-13645;
+ * kernels R17:12133-12290, 12314-12575) with every rounding and summation order of both.  q [16][128], k, v
+ * [8][128]: the projections' outputs; q_norm_w, k_norm_w [128]; cos_row, sin_row [128]: the RoPE row of
+ * cache_position.  The new K row (normed, rotated) and V row are written to key_cache / value_cache
+ * [8][16][128] at cache_position (0..15; QM_ERR_SLOT_RANGE otherwise) and the rotated query attends the
+ * keys 0..cache_position; context_out [16][128].  Same bits as qm_qk_norm_rope_kv_append followed by
+ * qm_predictor_attention_staged(rows 1, key_length cache_position + 1).  All tensors 16-byte aligned.
+ */
+int32_t qm_predictor_step_attention_m1(
+    const uint16_t* q, const uint16_t* k, const uint16_t* v,
+    const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+    const uint16_t* cos_row, const uint16_t* sin_row,
+    uint16_t* key_cache, uint16_t* value_cache, uint16_t* context_out,
+    int32_t cache_position, float epsilon, void* hip_stream);
+
+/*
  * The three layout operators in front of the staged attention at the predictor's step 0 (call site
  * R17:13663-13699), each with the reference wrapper's per-tensor argument list:
  * qm_predictor_transpose replaces PersistentPredictor::transpose (R17:13222-13236, kernel

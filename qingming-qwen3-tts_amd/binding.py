@@ -69,6 +69,7 @@ _SIGNATURES = {
                                                  _F32, C.c_int64, C.c_int64, C.c_int64, _PTR, C.c_int64, _PTR, _PTR]),
     "qm_predictor_attention_loop": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _I32, _F32, _PTR]),
     "qm_predictor_attention_staged": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _PTR]),
+    "qm_predictor_step_attention_m1": (_I32, [_PTR] * 10 + [_I32, _F32, _PTR]),
     "qm_predictor_transpose": (_I32, [_PTR, _PTR, _I32, _I32, _PTR]),
     "qm_predictor_rope_bhsd": (_I32, [_PTR] * 4 + [_I32, _I32, _PTR]),
     "qm_predictor_update_cache": (_I32, [_PTR, _PTR, _I32, _I32, _PTR]),
@@ -361,6 +362,13 @@ def gather_embedding(table, table_rows, codes, group, dimension, selected, next_
 def predictor_attention_staged(query_bhsd, key_cache, value_cache, out, rows, key_length, causal, stream=0):
     _check(lib().qm_predictor_attention_staged(_addr(query_bhsd), _addr(key_cache), _addr(value_cache), _addr(out),
                                                rows, key_length, int(causal), stream), "qm_predictor_attention_staged")
+
+
+def predictor_step_attention_m1(q, k, v, gq, gk, cos_row, sin_row, key_cache, value_cache, out, position,
+                                eps=1e-6, stream=0):
+    _check(lib().qm_predictor_step_attention_m1(_addr(q), _addr(k), _addr(v), _addr(gq), _addr(gk), _addr(cos_row),
+                                                _addr(sin_row), _addr(key_cache), _addr(value_cache), _addr(out),
+                                                position, eps, stream), "qm_predictor_step_attention_m1")
 
 
 def predictor_transpose(x, out, rows, heads, stream=0):

@@ -238,18 +238,12 @@ static void predictor_step_m1(qm_predictor& p, int step, bool sampling) {
     DeviceBuffer* current = &p.hidden_a;
     DeviceBuffer* next = &p.hidden_b;
     for (PredictorLayer& w : p.layers) {
-        qm_kv_cache cache = {};
-        cache.k_pool = w.key_cache.u16(); cache.v_pool = w.value_cache.u16();
-        cache.stride_page = 0; cache.stride_head = kPredMaxCache * kHeadDim; cache.stride_token = kHeadDim;
-        cache.page_size = kPredMaxCache; cache.n_pages = 1; cache.kv_heads = kPredKvHeads; cache.head_dim = kHeadDim;
         op_check(qm_predictor_rmsnorm_qkv_m1(current->u16(), w.input_norm.data(), kEpsilon, w.q_weight.data(), w.k_weight.data(),
                                              w.v_weight.data(), p.q_linear.u16(), p.k_linear.u16(), p.v_linear.u16(), kPredHidden,
                                              kPredQueryDim, kPredKvDim, s), "predictor qkv_m1");
-        op_check(qm_qk_norm_rope_kv_append(p.q_linear.u16(), p.k_linear.u16(), p.v_linear.u16(), w.q_norm.data(), w.k_norm.data(), cos_row,
-                                           sin_row, p.q_rotated.u16(), &cache, nullptr, 1, kPredQueryHeads, position, kEpsilon, s),
-                 "predictor qk_norm_rope_cache_m1");
-        op_check(qm_predictor_attention_staged(p.q_rotated.u16(), w.key_cache.u16(), w.value_cache.u16(), p.context.u16(), 1,
-                                               position + 1, 0, s), "predictor attention_m1");
+        op_check(qm_predictor_step_attention_m1(p.q_linear.u16(), p.k_linear.u16(), p.v_linear.u16(), w.q_norm.data(), w.k_norm.data(),
+                                                cos_row, sin_row, w.key_cache.u16(), w.value_cache.u16(), p.context.u16(), position,
+                                                kEpsilon, s), "predictor qk_norm_rope_cache_m1 + attention_m1");
         op_check(qm_predictor_linear_m1(p.context.u16(), w.o_weight.data(), nullptr, p.attention.u16(), kPredHidden, kPredQueryDim, s),
                  "predictor o_proj");
         op_check(qm_predictor_add_postnorm_gate_up_swiglu_m1(current->u16(), p.attention.u16(), w.post_norm.data(), kEpsilon,

@@ -16,31 +16,11 @@
 #include "qm_device.h"
 #include "qm_host.h"
 #include "qm_predictor_params.h"
+#include "qm_predictor_chain.h"
 
 #include <type_traits>
 
 namespace qm {
-
-// bf16 round trip with the hardware converter (round to nearest even; same bits as the integer
-// formula of R17:8172-8187 for every non-NaN input).
-__device__ __forceinline__ float rbf(float x) { return round_bf16(x); }
-
-// Sum of x[0..N-1] in the shape of the reference's 32-lane shuffle tree (shfl_down 16, 8, 4, 2, 1)
-// whose leaves N..31 are exact +0: adding +0 to a value that is not -0 is the identity, so absent
-// leaves are dropped instead of added.  X(i) must never be -0 (fmaf(p, v, +0) and exp() are not).
-template <int N, int I, int STRIDE>
-struct TreeSum {
-    template <class X>
-    static __device__ __forceinline__ float eval(const X& x) {
-        if constexpr (STRIDE == 0) {
-            return x(I);
-        } else if constexpr (I + STRIDE < N) {
-            return TreeSum<N, I, STRIDE / 2>::eval(x) + TreeSum<N, I + STRIDE, STRIDE / 2>::eval(x);
-        } else {
-            return TreeSum<N, I, STRIDE / 2>::eval(x);
-        }
-    }
-};
 
 template <int R>
 __device__ __forceinline__ void pv_rows(const float (*p)[kPredRows], const float* vcol, uint16_t* out,
@@ -49,21 +29,22 @@ __device__ __forceinline__ void pv_rows(const float (*p)[kPredRows], const float
         if (R < rows) {
             const float* pr = p[R];
             // leaf j = fmaf(P[j], V[j][d], +0), keys 0..R (R17:12523-12549)
-            const float o = TreeSum<R + 1, 0, 8>::eval([&](int j) { return fmaf(pr[j], vcol[j], 0.0f); });
+            const float o = TreeSum<R + 1, 0, 1>::eval([&](int j) { return fmaf(pr[j], vcol[j], 0.0f); });
             out[R * row_stride] = __builtin_bit_cast(uint16_t, static_cast<__bf16>(o));   // RNE, one instruction
             pv_rows<R + 1>(p, vcol, out, row_stride, rows);
         }
     }
 }
 
-// The same sum for a runtime number of keys: the full 16-leaf tree whose leaves at and beyond
-// `limit` are +0 (never read from V, whose cache slots there may hold anything).
-__device__ __forceinline__ float pv_limited(const float* pr, const float* vcol, int limit) {
-    return TreeSum<kPredRows, 0, 8>::eval([&](int j) { return j < limit ? fmaf(pr[j], vcol[j], 0.0f) : 0.0f; });
-}
-
-template <bool STAGED>
+// MODE 0: the loop (all rows of a unit from the projections' outputs).  MODE 1 (STAGED): attention only, over
+// rotated queries and the caches.  MODE 2 (APPEND): one M = 1 step of a layer in one launch, what the
+// reference runs as qk_norm_rope_cache_m1 + attention_m1 (R17:13700-13760): q [16][128], k, v [8][128] come from
+// the projections, the caches [8][16][128] hold the rows before key_length - 1; the new K row (normed,
+// rotated) and V row are written to the caches at key_length - 1 and the query attends key_length keys.
+template <int MODE>
 __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorParams prm) {
+    constexpr bool STAGED = MODE == 1;
+    constexpr bool APPEND = MODE == 2;
     __shared__ __attribute__((aligned(16))) uint16_t sh_q[2][kPredRows][kDim];   // [g][row][d]
     __shared__ __attribute__((aligned(16))) uint16_t sh_k[kPredRows][kDim];
     __shared__ __attribute__((aligned(16))) uint16_t sh_v[kPredRows][kDim];
@@ -84,7 +65,11 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
     const int layer = static_cast<int>((prm.unit_base + unit) % prm.n_layers);
 
     // keys row r attends: a prefix of the cache
-    auto limit_of = [&](int r) { return STAGED ? (prm.causal ? min(r + 1, prm.key_length) : prm.key_length) : r + 1; };
+    auto limit_of = [&](int r) {
+        return STAGED ? (prm.causal ? min(r + 1, prm.key_length) : prm.key_length) : (APPEND ? prm.key_length : r + 1);
+    };
+    const int new_row = APPEND ? prm.key_length - 1 : 0;                 // APPEND: the cache row this step fills
+    auto key_row_of = [&](int vrow) { return APPEND ? new_row : vrow; };   // where row vrow's K vector lives in sh_k
     if (STAGED) {
         // ---- q [16][rows][128] of this head pair, K and V rows 0..key_length-1 of the cache ------------
         for (int c = tid; c < rows * 32; c += kPredThreads) {
@@ -107,7 +92,38 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
         }
         __syncthreads();
     }
-    if (!STAGED) {
+    if (APPEND) {
+        // ---- the step's q (2 heads), k, v, its RoPE row and the gammas; the cache rows before it ----------
+        for (int c = tid; c < 128; c += kPredThreads) {
+            const int chunk = c & 15, which = c >> 4;     // 0,1: q head g; 2: k; 3: v; 4,5: cos, sin; 6,7: gammas
+            const uint16_t* src = which < 2 ? prm.q + (kvh * 2 + which) * kDim
+                                : which == 2 ? prm.k + kvh * kDim
+                                : which == 3 ? prm.v + kvh * kDim
+                                : which == 4 ? prm.cos_rows : which == 5 ? prm.sin_rows
+                                : which == 6 ? prm.q_norm_w : prm.k_norm_w;
+            uint16_t* dst = which < 2 ? sh_q[which][0] : which == 2 ? sh_k[new_row] : which == 3 ? sh_v[new_row]
+                          : which == 4 ? sh_cos[0] : which == 5 ? sh_sin[0] : sh_gamma[which - 6];
+            *reinterpret_cast<uint4*>(dst + chunk * 8) = *reinterpret_cast<const uint4*>(src + chunk * 8);
+        }
+        for (int c = tid; c < kPredRows * 32; c += kPredThreads) {
+            const int chunk = c & 15, is_v = (c >> 4) & 1, row = c >> 5;
+            if (row == new_row) continue;
+            uint4 val = make_uint4(0, 0, 0, 0);
+            if (row < new_row)
+                val = *reinterpret_cast<const uint4*>((is_v ? prm.v_cache_out : prm.k_cache_out)
+                                                      + (static_cast<int64_t>(kvh) * kPredRows + row) * kDim + chunk * 8);
+            *reinterpret_cast<uint4*>(is_v ? &sh_v[row][chunk * 8] : &sh_k[row][chunk * 8]) = val;
+        }
+        __syncthreads();
+        // (the new row is widened after its rotation, below)
+        for (int c = tid; c < kPredRows * 32; c += kPredThreads) {
+            const int row = c >> 5, d0 = (c & 31) * 4;
+            if (row == new_row) continue;
+            const uint2 kk = *reinterpret_cast<const uint2*>(&sh_k[row][d0]);
+            *reinterpret_cast<float4*>(&sh_kf[row][d0]) = make_float4(lo_bf16(kk.x), hi_bf16(kk.x), lo_bf16(kk.y), hi_bf16(kk.y));
+        }
+    }
+    if (MODE == 0) {
     // ---- stage q (2 heads), k, v of this kv head, the RoPE rows and the two gammas: 16-byte chunks ---
     for (int c = tid; c < rows * 64; c += kPredThreads) {
         const int chunk = c & 15;
@@ -138,6 +154,8 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
         }
     }
     __syncthreads();
+    }   // MODE == 0
+    if (!STAGED) {
 
     // ---- QK-RMSNorm + RoPE in place over the 3*rows head vectors (2 q heads + k per row) --------------
     // (1) One thread per (vector, 32-dim group): the group's sum of squares in the order of the
@@ -146,7 +164,7 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
     for (int it = tid; it < n_vec * 4; it += kPredThreads) {
         const int vec = it >> 2, grp = it & 3;
         const int vrow = vec / 3, which = vec % 3;
-        const uint16_t* x = (which < 2 ? sh_q[which][vrow] : sh_k[vrow]) + 32 * grp;
+        const uint16_t* x = (which < 2 ? sh_q[which][vrow] : sh_k[key_row_of(vrow)]) + 32 * grp;
         float sq[32];
 #pragma unroll
         for (int i = 0; i < 32; i += 8) {
@@ -198,7 +216,7 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
                 g0[0] = lo_bf16(gl.x); g0[1] = hi_bf16(gl.x); g0[2] = lo_bf16(gl.y); g0[3] = hi_bf16(gl.y);
                 g1[0] = lo_bf16(gh.x); g1[1] = hi_bf16(gh.x); g1[2] = lo_bf16(gh.y); g1[3] = hi_bf16(gh.y);
             }
-            uint16_t* x = which < 2 ? sh_q[which][vrow] : sh_k[vrow];
+            uint16_t* x = which < 2 ? sh_q[which][vrow] : sh_k[key_row_of(vrow)];
             const float r = sh_r[vrow * 3 + which];
             const uint2 xl = *reinterpret_cast<const uint2*>(x + d0), xh = *reinterpret_cast<const uint2*>(x + d0 + 64);
             const float x0[4] = {lo_bf16(xl.x), hi_bf16(xl.x), lo_bf16(xl.y), hi_bf16(xl.y)};
@@ -220,9 +238,9 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
             *reinterpret_cast<uint2*>(x + d0 + 64) = make_uint2(out_hi[0], out_hi[1]);
             if (which == 2) {
                 // every wave reads all of K for the scores: widen it once here instead of four times there
-                *reinterpret_cast<float4*>(&sh_kf[vrow][d0]) =
+                *reinterpret_cast<float4*>(&sh_kf[key_row_of(vrow)][d0]) =
                     make_float4(lo_bf16(out_lo[0]), hi_bf16(out_lo[0]), lo_bf16(out_lo[1]), hi_bf16(out_lo[1]));
-                *reinterpret_cast<float4*>(&sh_kf[vrow][d0 + 64]) =
+                *reinterpret_cast<float4*>(&sh_kf[key_row_of(vrow)][d0 + 64]) =
                     make_float4(lo_bf16(out_hi[0]), hi_bf16(out_hi[0]), lo_bf16(out_hi[1]), hi_bf16(out_hi[1]));
             }
         }
@@ -232,7 +250,15 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
     }   // !STAGED
 
     // ---- optional K/V cache write-back, layout [unit][kv head][16][128] (R17:10711-10737) ---------
-    if (!STAGED && prm.k_cache_out) {
+    if (APPEND) {
+        if (tid < 32) {
+            const int chunk = tid & 15, is_v = tid >> 4;
+            *reinterpret_cast<uint4*>((is_v ? prm.v_cache_out : prm.k_cache_out)
+                                      + (static_cast<int64_t>(kvh) * kPredRows + new_row) * kDim + chunk * 8) =
+                *reinterpret_cast<const uint4*>(is_v ? &sh_v[new_row][chunk * 8] : &sh_k[new_row][chunk * 8]);
+        }
+    }
+    if (MODE == 0 && prm.k_cache_out) {
         for (int c = tid; c < kPredRows * 16; c += kPredThreads) {
             const int row = c >> 4, chunk = c & 15;
             const int64_t dst = ((unit * 8 + kvh) * kPredRows + row) * kDim + chunk * 8;
@@ -361,7 +387,7 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
 #pragma unroll
         for (int t = 0; t < kPredRows; ++t) e[t] = t < limit ? expf(sc[t] - maximum) : 0.0f;
         // exp() >= +0 and masked entries are +0: the full 16-leaf tree equals the reference's sum
-        const float total = TreeSum<16, 0, 8>::eval([&](int t) { return e[t]; });
+        const float total = TreeSum<16, 0, 1>::eval([&](int t) { return e[t]; });
 #pragma unroll
         for (int t = 0; t < kPredRows; t += 4) {
             float4 p4;
@@ -382,7 +408,7 @@ __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorP
 #pragma unroll
         for (int j = 0; j < kPredRows; ++j) vcol[j] = bf2f(sh_v[j][d]);
         uint16_t* out = prm.out + ((unit * rows) * 16 + kvh * 2 + g) * kDim + d;
-        if (STAGED) {
+        if (STAGED || APPEND) {
             for (int r = 0; r < rows; ++r)
                 out[r * 16 * kDim] = __builtin_bit_cast(uint16_t, static_cast<__bf16>(pv_limited(sh_s[g][r], vcol, limit_of(r))));
         } else {
@@ -441,7 +467,7 @@ extern "C" int32_t qm_predictor_attention_loop(
         if (k_cache_out) p.k_cache_out = k_cache_out + static_cast<int64_t>(first) * 8 * 16 * qm::kDim;
         if (v_cache_out) p.v_cache_out = v_cache_out + static_cast<int64_t>(first) * 8 * 16 * qm::kDim;
         p.unit_base = first;
-        hipLaunchKernelGGL(qm::predictor_loop_kernel<false>, dim3(8, n), dim3(qm::kPredThreads), 0,
+        hipLaunchKernelGGL(qm::predictor_loop_kernel<0>, dim3(8, n), dim3(qm::kPredThreads), 0,
                            static_cast<hipStream_t>(hip_stream), p);
         const int32_t rc = qm::launch_status();
         if (rc != QM_OK) return rc;
@@ -462,7 +488,32 @@ extern "C" int32_t qm_predictor_attention_staged(const uint16_t* query_bhsd, con
     prm.out = output;
     prm.unit_base = 0; prm.n_layers = 1; prm.rows = rows; prm.epsilon = 0.0f;
     prm.key_length = key_length; prm.causal = causal_prefill ? 1 : 0;
-    hipLaunchKernelGGL(qm::predictor_loop_kernel<true>, dim3(8, 1), dim3(qm::kPredThreads), 0,
+    hipLaunchKernelGGL(qm::predictor_loop_kernel<1>, dim3(8, 1), dim3(qm::kPredThreads), 0,
+                       static_cast<hipStream_t>(hip_stream), prm);
+    return qm::launch_status();
+}
+
+extern "C" int32_t qm_predictor_step_attention_m1(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                                                  const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+                                                  const uint16_t* cos_row, const uint16_t* sin_row,
+                                                  uint16_t* key_cache, uint16_t* value_cache, uint16_t* context_out,
+                                                  int32_t cache_position, float epsilon, void* hip_stream) {
+    if (!q || !k || !v || !q_norm_w || !k_norm_w || !cos_row || !sin_row || !key_cache || !value_cache || !context_out)
+        return QM_ERR_NULL;
+    if (cache_position < 0 || cache_position >= qm::kPredRows) return QM_ERR_SLOT_RANGE;
+    const uintptr_t align = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v)
+                          | reinterpret_cast<uintptr_t>(q_norm_w) | reinterpret_cast<uintptr_t>(k_norm_w)
+                          | reinterpret_cast<uintptr_t>(cos_row) | reinterpret_cast<uintptr_t>(sin_row)
+                          | reinterpret_cast<uintptr_t>(key_cache) | reinterpret_cast<uintptr_t>(value_cache);
+    if (align & 15) return QM_ERR_GEOMETRY;
+    qm::PredictorParams prm = {};
+    prm.q = q; prm.k = k; prm.v = v;
+    prm.q_norm_w = q_norm_w; prm.k_norm_w = k_norm_w;
+    prm.cos_rows = cos_row; prm.sin_rows = sin_row;
+    prm.out = context_out; prm.k_cache_out = key_cache; prm.v_cache_out = value_cache;
+    prm.unit_base = 0; prm.n_layers = 1; prm.rows = 1; prm.epsilon = epsilon;
+    prm.key_length = cache_position + 1; prm.causal = 0;
+    hipLaunchKernelGGL(qm::predictor_loop_kernel<2>, dim3(8, 1), dim3(qm::kPredThreads), 0,
                        static_cast<hipStream_t>(hip_stream), prm);
     return qm::launch_status();
 }

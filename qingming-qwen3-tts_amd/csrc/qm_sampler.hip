@@ -34,88 +34,16 @@
 
 #include "qm_device.h"
 #include "qm_host.h"
+#include "qm_sampler_block.h"
 
 namespace qm {
 
-constexpr int kSmpThreads = 256;
-constexpr int kSmpMaxVocab = 4096;                       // kGpuSamplerSortSize, R17:7336
-constexpr int kSmpPerThread = kSmpMaxVocab / kSmpThreads;
-constexpr int kSmpMaxKeep = 256;
-constexpr int kSmpReplicas = 8;                          // counters per histogram bin (a power of two)
-
-struct SamplerParams {
-    const void* logits;          // float or bf16 bits
-    int is_bf16;
-    int offset;                  // first element (last_row_offset of the bf16 kernel)
-    int vocab;
-    int top_k;                   // <= 0: arg-max
-    float temperature;
-    unsigned long long* rng_state;
-    int32_t* output_id;
-    // final-head processing in front of the selection (process != 0; logits are bf16)
-    int process;
-    int32_t* history;            // read [0, history_count); the code is appended at [append_index] if >= 0
-    int history_count;
-    int append_index;
-    int generation_index;
-    int eos;
-    int suppressed_tail;
-    float penalty;
-    float reciprocal;            // float(1) / float(penalty)
-    float* scores_out;           // processed scores, or NULL
-    int process_only;            // stop after writing scores_out
-};
-
-// Order-preserving image of a float: a > b  <=>  image(a) > image(b)  (-0 counted as +0).
-__device__ __forceinline__ uint32_t ordered_bits(float v) {
-    const uint32_t bits = __float_as_uint(v + 0.0f);
-    return (bits & 0x80000000U) ? ~bits : (bits | 0x80000000U);
-}
-__device__ __forceinline__ float from_ordered_bits(uint32_t image) {
-    return __uint_as_float((image & 0x80000000U) ? (image & 0x7fffffffU) : ~image);
-}
-
-__device__ __forceinline__ unsigned long long splitmix64_next(unsigned long long* state) {
-    unsigned long long z = *state + 0x9e3779b97f4a7c15ULL;
-    *state = z;
-    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ULL;
-    z = (z ^ (z >> 27)) * 0x94d049bb133111ebULL;
-    return z ^ (z >> 31);
-}
-
-// Inclusive prefix sum over the 64 lanes of a wave: four DPP row shifts inside the 16-lane rows, then the
-// three row totals (no LDS traffic; a shuffle-based scan costs an LDS round trip per step).
-__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
-    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);   // row_shr:1
-    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);   // row_shr:2
-    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);   // row_shr:4
-    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);   // row_shr:8
-    const int t0 = __builtin_amdgcn_readlane(v, 15);
-    const int t1 = __builtin_amdgcn_readlane(v, 31);
-    const int t2 = __builtin_amdgcn_readlane(v, 47);
-    if (lane >= 16) v += t0;
-    if (lane >= 32) v += t1;
-    if (lane >= 48) v += t2;
-    return v;
-}
-
 __global__ __launch_bounds__(kSmpThreads) void sampler_kernel(SamplerParams prm) {
-    __shared__ uint32_t sh_seen[kSmpMaxVocab / 32];      // tokens present in the history
-    __shared__ __attribute__((aligned(16))) int sh_hist[256 * kSmpReplicas];   // [bin][replica]
-    __shared__ int sh_wave_total[4], sh_wave_first[4];
-    __shared__ int sh_digit, sh_remaining, sh_done, sh_count;
-    __shared__ unsigned long long sh_cand[kSmpMaxKeep];
-    __shared__ unsigned long long sh_sorted[kSmpMaxKeep];
-    __shared__ __attribute__((aligned(16))) double sh_exp[kSmpMaxKeep];   // the terms, then their running sums
-    __shared__ double sh_target;
-
+    __shared__ SamplerScratch scratch;
     const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
     const int vocab = prm.vocab;
-
     // ---- everything that comes from global memory is requested first, in one go (a load per element
-    // inside the arithmetic below would wait for each one in turn): the scores of ids tid, tid + 256, ...
+    // inside the arithmetic would wait for each one in turn): the scores of ids tid, tid + 256, ...
     // (an id beyond the vocabulary reads the last score and is dropped later), the generator's state ----
     float score[kSmpPerThread];
     if (prm.is_bf16) {
@@ -132,176 +60,10 @@ __global__ __launch_bounds__(kSmpThreads) void sampler_kernel(SamplerParams prm)
     }
     unsigned long long rng = 0;
     if (tid == 0 && prm.top_k > 0 && !prm.process_only) rng = *prm.rng_state;
-#pragma unroll
-    for (int r = 0; r < kSmpReplicas; ++r) sh_hist[tid * kSmpReplicas + r] = 0;   // (a thread only ever reads and clears its own bin)
-
-    // ---- which tokens were generated before (R17:14046-14052, as a bitmap) -----------------------------
-    if (prm.process) {
-        for (int i = tid; i < kSmpMaxVocab / 32; i += kSmpThreads) sh_seen[i] = 0;
-        __syncthreads();
-        for (int i = tid; i < prm.history_count; i += kSmpThreads) {
-            const int token = prm.history[i];
-            if (token >= 0 && token < vocab) atomicOr(&sh_seen[token >> 5], 1U << (token & 31));
-        }
-        __syncthreads();
-    }
-
-    // ---- the scores as keys: larger key = earlier in the order -------------------------------------------
-    unsigned long long key[kSmpPerThread];
-#pragma unroll
-    for (int j = 0; j < kSmpPerThread; ++j) {
-        const int id = tid + kSmpThreads * j;
-        key[j] = 0;                                        // below every real key
-        if (id < vocab) {
-            float value = score[j];
-            if (prm.process) {
-                if ((sh_seen[id >> 5] >> (id & 31)) & 1U) value = value < 0.0f ? value * prm.penalty : value * prm.reciprocal;
-                if (id == prm.eos && prm.generation_index < 2) value = -INFINITY;
-                if (id >= vocab - prm.suppressed_tail && id != prm.eos) value = -INFINITY;
-                if (prm.scores_out) prm.scores_out[id] = value;
-            }
-            key[j] = (static_cast<unsigned long long>(ordered_bits(value)) << 32) | (0xffffffffU - static_cast<uint32_t>(id));
-        }
-    }
-
-    if (prm.process_only) return;
-    const int keep = prm.top_k <= 0 ? 1 : min(prm.top_k, vocab);
-
-    // ---- radix select of the keep-th largest key: digits of 8 bits, most significant first -------------
-    // The significant bits are the 32 of the score and the low 12 of the inverted id (ids < 4096).  A bin of
-    // the histogram has kSmpReplicas counters, a lane adds to counter lane % kSmpReplicas: scores share
-    // their leading bits, and LDS additions to one address take turns.  The passes end as soon as the bin
-    // that holds the keep-th key is wanted whole.
-    unsigned long long prefix = 0, prefix_mask = 0;
-    int remaining = keep;
-    bool whole_bin = false;
-    // (kept as a loop: unrolled, the compiler computes the digits of all passes ahead and runs out of registers)
-#pragma unroll 1
-    for (int pass = 0; pass < 6 && !whole_bin; ++pass) {
-        const int shift = pass < 4 ? 56 - 8 * pass : (pass == 4 ? 4 : 0);       // 56, 48, 40, 32, 4, 0
-        const int width = pass < 5 ? 8 : 4;
-        const unsigned digit_mask = (1U << width) - 1U;
-        __syncthreads();                                   // the bins are clear (and, later, the last pass's results read)
-#pragma unroll
-        for (int j = 0; j < kSmpPerThread; ++j)
-            if (key[j] != 0 && (key[j] & prefix_mask) == prefix)
-                atomicAdd(&sh_hist[(static_cast<unsigned>(key[j] >> shift) & digit_mask) * kSmpReplicas + (lane & (kSmpReplicas - 1))], 1);
-        __syncthreads();
-        // keys in bins above this thread's bin: inside the wave from a prefix sum, then the waves above
-        int own = 0;
-#pragma unroll
-        for (int r = 0; r < kSmpReplicas; ++r) {
-            own += sh_hist[tid * kSmpReplicas + r];
-            sh_hist[tid * kSmpReplicas + r] = 0;
-        }
-        const int upto = wave_inclusive_scan(own, lane);
-        const int wave_sum = __builtin_amdgcn_readlane(upto, 63);
-        if (lane == 0) sh_wave_total[wave] = wave_sum;
-        __syncthreads();
-        int above = wave_sum - upto;
-        for (int w = wave + 1; w < 4; ++w) above += sh_wave_total[w];
-        if (above < remaining && remaining <= above + own) {       // exactly one bin
-            sh_digit = tid;
-            sh_remaining = remaining - above;
-            sh_done = remaining == above + own ? 1 : 0;
-        }
-        __syncthreads();
-        prefix |= static_cast<unsigned long long>(sh_digit) << shift;
-        prefix_mask |= static_cast<unsigned long long>(digit_mask) << shift;
-        remaining = sh_remaining;
-        whole_bin = sh_done != 0;
-    }
-    // The keep-th largest key starts with the digits in `prefix`; the digits of passes not run are free (zero
-    // here), and bits 12..31 of an inverted id, which no pass looks at, are all ones in every key.
-    const unsigned long long threshold = prefix | 0x00000000fffff000ULL;
-
-    // ---- gather the keep keys at or above it, rank them by counting -------------------------------------
-    // (each thread counts its own, a prefix sum over the block gives it its place: no counter to queue at)
-    {
-        int mine = 0;
-#pragma unroll
-        for (int j = 0; j < kSmpPerThread; ++j) mine += (key[j] != 0 && key[j] >= threshold) ? 1 : 0;
-        const int upto = wave_inclusive_scan(mine, lane);
-        __syncthreads();                                   // (the select's last reads of sh_wave_total are done)
-        if (lane == 63) sh_wave_total[wave] = upto;
-        __syncthreads();
-        int at = upto - mine;
-        for (int w = 0; w < wave; ++w) at += sh_wave_total[w];
-#pragma unroll
-        for (int j = 0; j < kSmpPerThread; ++j)
-            if (key[j] != 0 && key[j] >= threshold) sh_cand[at++] = key[j];
-        __syncthreads();
-    }
-    if (tid < keep) {
-        const unsigned long long mine = sh_cand[tid];
-        int rank = 0;
-        for (int j = 0; j < keep; ++j) rank += sh_cand[j] > mine ? 1 : 0;
-        sh_sorted[rank] = mine;
-    }
-    __syncthreads();
-
-    // ---- sample (R17:7431-7460) ----------------------------------------------------------------------------
-    const double inv_t = 1.0 / static_cast<double>(prm.temperature);
-    if (prm.top_k > 0 && tid < keep) {
-        const double maximum = static_cast<double>(from_ordered_bits(static_cast<uint32_t>(sh_sorted[0] >> 32))) * inv_t;
-        const double value = static_cast<double>(from_ordered_bits(static_cast<uint32_t>(sh_sorted[tid] >> 32)));
-        sh_exp[tid] = exp(value * inv_t - maximum);
-    } else if (tid < ((keep + 7) & ~7)) {
-        sh_exp[tid] = 0.0;                                 // (padding of the last batch of eight below: x + 0 is x)
-    }
-    __syncthreads();
-    auto id_of = [&](int i) { return static_cast<int32_t>(0xffffffffU - static_cast<uint32_t>(sh_sorted[i])); };
-    // The running sums, added by one thread in the reference's order (its second loop repeats
-    // the partial sums of its first: one pass serves both); the terms come eight at a time, the next
-    // eight already on their way, so that the chain waits for additions, not for LDS.
-    if (prm.top_k > 0 && tid == 0) {
-        typedef double f64x2_t __attribute__((ext_vector_type(2)));
-        const f64x2_t* terms = reinterpret_cast<const f64x2_t*>(sh_exp);
-        f64x2_t* sums = reinterpret_cast<f64x2_t*>(sh_exp);
-        double running = 0.0;
-        f64x2_t next[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) next[u] = terms[u];
-        for (int i0 = 0; i0 < keep; i0 += 8) {
-            f64x2_t term[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) term[u] = next[u];
-            if (i0 + 8 < keep) {
-#pragma unroll
-                for (int u = 0; u < 4; ++u) next[u] = terms[(i0 + 8) / 2 + u];
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                running += term[u].x;
-                term[u].x = running;
-                running += term[u].y;
-                term[u].y = running;
-                sums[i0 / 2 + u] = term[u];
-            }
-        }
-        const double total = running;
-        sh_count = -1;                                     // no draw
-        if (total > 0.0) {
-            const double uniform = static_cast<double>(splitmix64_next(&rng) >> 11) * (1.0 / 9007199254740992.0);
-            *prm.rng_state = rng;
-            sh_target = uniform * total;
-            sh_count = keep - 1;                           // the answer if no running sum exceeds the target
-        }
-    }
-    __syncthreads();
-    // first index whose running sum exceeds the target: the lowest such lane of each wave, then the lowest wave
-    {
-        const bool beyond = prm.top_k > 0 && sh_count >= 0 && tid < keep && sh_target < sh_exp[tid];
-        const unsigned long long lanes = __builtin_amdgcn_ballot_w64(beyond);
-        if (lane == 0) sh_wave_first[wave] = lanes ? 64 * wave + __builtin_ctzll(lanes) : 0x7fffffff;
-    }
-    __syncthreads();
-    if (tid != 0) return;
-    int32_t chosen = id_of(0);
-    if (prm.top_k > 0 && sh_count >= 0) {
-        const int first = min(min(sh_wave_first[0], sh_wave_first[1]), min(sh_wave_first[2], sh_wave_first[3]));
-        chosen = id_of(min(first, sh_count));              // sh_count = keep - 1: the answer if no sum exceeds the target
-    }
+    const unsigned long long before = rng;
+    const int32_t chosen = sampler_block(prm, scratch, score, rng);
+    if (tid != 0 || chosen == -2) return;
+    if (rng != before) *prm.rng_state = rng;
     prm.output_id[0] = chosen;
     if (prm.history && prm.append_index >= 0) prm.history[prm.append_index] = chosen;
 }

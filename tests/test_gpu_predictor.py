@@ -6,6 +6,8 @@ reference's whole rounding chain and summation order, so beyond the stated toler
 and P.V on the matrix cores: outputs within the tolerance.  In both, QK-RMSNorm + RoPE are the
 reference's chain exactly: the K/V cache write-back must be bit-exact.
 """
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -300,3 +302,121 @@ def test_predictor_m1_attention_is_the_exact_chain(oracle, qm, dev):
         assert d.max() <= 1
         differing += int(np.count_nonzero(d))
     assert differing <= 16 * 2048 // 500
+
+
+def test_predictor_step_attention_m1_equals_the_operator_pair(oracle, qm, dev):
+    """qm_predictor_step_attention_m1 at every cache position 0..15: context and both caches equal, bit for
+    bit, what qm_qk_norm_rope_kv_append followed by qm_predictor_attention_staged leave, and the caches equal
+    the oracle's (norm, RoPE and append are exact); rows after the position are left untouched."""
+    import torch
+    cos, sin = oracle.rope_table(16, 0, 128, 1.0e6)
+    for position in range(16):
+        q = oracle.normal_bf16((16, 128), 5100 + position)
+        k = oracle.normal_bf16((8, 128), 5200 + position)
+        v = oracle.normal_bf16((8, 128), 5300 + position)
+        gq = oracle.normal_bf16((128,), 5400 + position, 1.0, 0.1)
+        gk = oracle.normal_bf16((128,), 5500 + position, 1.0, 0.1)
+        kc = oracle.normal_bf16((8, 16, 128), 5600 + position)
+        vc = oracle.normal_bf16((8, 16, 128), 5700 + position)
+        kc[:, position:] = 0x7fc0            # NaN patterns where nothing has been appended yet
+        vc[:, position:] = 0x7fc0
+        # the pair of operators
+        kd, vd = to_dev(kc, dev), to_dev(vc, dev)
+        qrot = torch.zeros((16, 128), dtype=torch.int16, device=dev)
+        pair = torch.full((16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+        cache = qm.flat_cache(kd, vd, 8, 16)
+        cd, sd = to_dev(cos[position], dev), to_dev(sin[position], dev)
+        qd, kld, vld, gqd, gkd = (to_dev(a, dev) for a in (q, k, v, gq, gk))
+        qm.qk_norm_rope_kv_append(qd, kld, vld, gqd, gkd, cd, sd, qrot, cache, None, 1, 16, position, 1e-6)
+        qm.predictor_attention_staged(qrot, kd, vd, pair, 1, position + 1, False)
+        # the one launch
+        kd2, vd2 = to_dev(kc, dev), to_dev(vc, dev)
+        one = torch.full((16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+        qm.predictor_step_attention_m1(qd, kld, vld, gqd, gkd, cd, sd, kd2, vd2, one, position, 1e-6)
+        torch.cuda.synchronize()
+        assert torch.equal(one, pair), position
+        assert torch.equal(kd2, kd) and torch.equal(vd2, vd), position
+        # the oracle's append on the same inputs
+        ko, vo = kc.copy(), vc.copy()
+        qo = np.zeros_like(q)
+        assert oracle.qk_norm_rope_kv_append(q, k, v, gq, gk, cos[position], sin[position], qo,
+                                             oracle.flat_cache(ko, vo, 8, 16), None, 1, 16, position) == 0
+        assert np.array_equal(to_u16(kd2), ko) and np.array_equal(to_u16(vd2), vo), position
+        want = np.zeros_like(q)
+        assert oracle.predictor_attention_m1(qo, ko, vo, want, position + 1) == 0
+        from qm_testlib import ulp_distance
+        assert ulp_distance(to_u16(one), want).max() <= 1, position
+
+
+def test_predictor_step_attention_m1_argument_errors(qm, dev):
+    import torch
+    z = torch.zeros(8 * 16 * 128, dtype=torch.int16, device=dev)
+    L = qm.lib()
+    p = z.data_ptr()
+    args = lambda position: (p, p, p, p, p, p, p, p, p, p, position, C.c_float(1e-6), None)
+    assert L.qm_predictor_step_attention_m1(*args(16)) == -3
+    assert L.qm_predictor_step_attention_m1(*args(-1)) == -3
+    assert L.qm_predictor_step_attention_m1(None, p, p, p, p, p, p, p, p, p, 0, C.c_float(1e-6), None) == -1
+    assert L.qm_predictor_step_attention_m1(p + 2, p, p, p, p, p, p, p, p, p, 0, C.c_float(1e-6), None) == -2
+
+
+def _cancelling_values(oracle, shape, seed):
+    """bf16 values whose fp32 sum depends on the order of the additions: each run of 16 along axis -2 holds
+    +2^30 and -2^30 at two seeded places among small values (2^30 + 1 is 2^30 in fp32)."""
+    base = oracle.normal_bf16(shape, seed)
+    flat = base.reshape(-1, 16, shape[-1])
+    rng = np.random.default_rng(seed)
+    for g in range(flat.shape[0]):
+        for d in range(shape[-1]):
+            a, b = rng.choice(16, size=2, replace=False)
+            flat[g, a, d] = 0x4e80      # +2^30
+            flat[g, b, d] = 0xce80      # -2^30
+    return flat.reshape(shape)
+
+
+def test_predictor_pv_sum_follows_the_shuffle_tree(oracle, qm, dev):
+    """The fp32 additions of P.V are those of value += shfl_down(value, offset), offset 16 .. 1 (R17:9359-9364):
+    with zero queries every probability is exactly 1 / keys and no exponential differs, so values that cancel
+    only in one order of additions make the outputs of the three exact-chain operators equal the oracle's to the
+    bit, or not at all."""
+    import torch
+    vc = _cancelling_values(oracle, (8, 16, 128), 8101)
+    kc = oracle.normal_bf16((8, 16, 128), 8102)
+    # M = 1 over 16 keys, and 16 causal rows
+    for rows, causal in ((1, False), (16, True)):
+        q = np.zeros((16, rows, 128), dtype=np.uint16)
+        want = np.zeros((rows, 16, 128), dtype=np.uint16)
+        assert oracle.predictor_attention_staged(q, kc, vc, want, rows, 16, causal) == 0
+        out = torch.full((rows, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+        qm.predictor_attention_staged(to_dev(q, dev), to_dev(kc, dev), to_dev(vc, dev), out, rows, 16, causal)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_u16(out), want), (rows, causal)
+    # the fused M = 1 step at the last cache position
+    cos, sin = oracle.rope_table(16, 0, 128, 1.0e6)
+    q1 = np.zeros((16, 128), dtype=np.uint16)
+    k1 = oracle.normal_bf16((8, 128), 8103)
+    gamma = oracle.normal_bf16((128,), 8104, 1.0, 0.1)
+    kd, vd = to_dev(kc, dev), to_dev(vc, dev)
+    one = torch.full((16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.predictor_step_attention_m1(to_dev(q1, dev), to_dev(k1, dev), to_dev(vc[:, 15].copy(), dev), to_dev(gamma, dev),
+                                   to_dev(gamma, dev), to_dev(cos[15], dev), to_dev(sin[15], dev), kd, vd, one, 15, 1e-6)
+    torch.cuda.synchronize()
+    want1 = np.zeros((16, 128), dtype=np.uint16)
+    assert oracle.predictor_attention_m1(q1, to_u16(kd), to_u16(vd), want1, 16) == 0
+    assert np.array_equal(to_u16(one), want1)
+    # the loop's exact-chain kernel: unit of 16 rows, zero queries
+    v = _cancelling_values(oracle, (1, 8, 16, 128), 8105).transpose(0, 2, 1, 3).copy()      # [unit][row][head][128]
+    k = oracle.normal_bf16((1, 16, 8, 128), 8106)
+    q = np.zeros((1, 16, 16, 128), dtype=np.uint16)
+    g2 = oracle.normal_bf16((1, 128), 8107, 1.0, 0.1)
+    want = np.zeros_like(q)
+    assert oracle.predictor_attention_loop(q, k, v, g2, g2, cos, sin, want, None, None, 1, 1, 16, 1, 1e-6, 8) == 0
+    out = torch.full((1, 16, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.set_option(qm.OPT_PREDICTOR_LOOP_KERNEL, 1)
+    try:
+        qm.predictor_attention_loop(to_dev(q, dev), to_dev(k, dev), to_dev(v, dev), to_dev(g2, dev), to_dev(g2, dev),
+                                    to_dev(cos, dev), to_dev(sin, dev), out, None, None, 1, 1, 16, 1, 1e-6)
+    finally:
+        qm.set_option(qm.OPT_PREDICTOR_LOOP_KERNEL, 0)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_u16(out), want)
