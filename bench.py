@@ -474,9 +474,11 @@ class PredictorFrameSteps:
     name = "predictor_frame_14_m1_steps_5layers"
     tolerance = 0.125
 
-    def __init__(self, qm, dev, seed=77):
+    def __init__(self, qm, dev, seed=77, one_launch=False):
         import torch
-        self.qm, self.dev = qm, dev
+        self.qm, self.dev, self.one_launch = qm, dev, one_launch
+        if one_launch:
+            self.name += "_one_launch"
         syn = Synthetic(dev, seed)
         H, Q, KV, I, OUT, V = 1024, 2048, 1024, 3072, 2048, 2048
         self.dims = (H, Q, KV, I, OUT, V)
@@ -513,6 +515,21 @@ class PredictorFrameSteps:
         self.ws = torch.empty(self.ws_bytes // 4 + 1, dtype=torch.float32, device=dev)
         layer_w = 2 * (Q * H + 2 * KV * H + H * Q + 2 * I * H + H * I)
         self.launches_per_step = 1 + 5 * 5 + 3
+        if one_launch:
+            # qm_predictor_frame_steps: 256 resident blocks run all fourteen steps and hand the operators' outputs to
+            # one another through a workspace
+            self.launches_per_step = 1.0 / 14
+            names = dict(in_norm="input_norm", wq="q_weight", wk="k_weight", wv="v_weight", gq="q_norm", gk="k_norm",
+                         wo="o_weight", post="post_norm", wg="gate_weight", wu="up_weight", wd="down_weight", k="key_cache",
+                         v="value_cache")
+            self.frame = qm.predictor_frame([{names[k]: L[k] for k in names} for L in self.layers], self.proj_w, self.proj_b,
+                                            self.final_norm, {s: self.heads[s - 1] for s in range(1, 15)},
+                                            {s: self.tables[s - 1] for s in range(1, 15)}, self.cos, self.sin, self.free_input,
+                                            self.selected, self.codes, self.rng)
+            self.frame_ws_bytes = qm.predictor_frame_workspace_bytes()
+            self.frame_ws = torch.zeros(self.frame_ws_bytes // 4, dtype=torch.int32, device=dev)
+            qm.predictor_frame_workspace_init(self.frame_ws, self.frame_ws_bytes)
+            self.frame_status = torch.zeros(1, dtype=torch.int32, device=dev)
         self.bytes = 14 * (5 * layer_w + 2 * H * OUT + 2 * V * H + 2 * OUT)          # weights streamed once per step
         self.flops = self.bytes
         self.copies = 14
@@ -545,6 +562,9 @@ class PredictorFrameSteps:
     def step(self):
         import torch
         s = torch.cuda.current_stream().cuda_stream
+        if self.one_launch:
+            self.qm.predictor_frame_steps(self.frame, 1, 14, 50, 0.9, self.frame_ws, self.frame_ws_bytes, self.frame_status, s)
+            return
         for step in range(1, 15):
             self.one_step(step, s)
 
@@ -759,7 +779,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
     ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "prefillfp32", "predictor", "predictorexact",
-                                      "qkv", "layer", "frame"], default=None,
+                                      "qkv", "layer", "frame", "frame1"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -798,7 +818,8 @@ def main():
                 "predictor": lambda: PredictorLoop(qm, dev),
                 "predictorexact": lambda: PredictorLoop(qm, dev, kernel=1),
                 "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev),
-                "frame": lambda: PredictorFrameSteps(qm, dev)}[args.only]
+                "frame": lambda: PredictorFrameSteps(qm, dev),
+                "frame1": lambda: PredictorFrameSteps(qm, dev, one_launch=True)}[args.only]
         w = make()
         r = _report(w, _time_steps(w.step, args.steps, args.warmup))
         r["bound"] = w.bound
@@ -843,6 +864,8 @@ def main():
             ("next_talker_layer_decode_step_unfused", lambda: TalkerLayerStep(qm, dev, fused=False)),
             # the fourteen M = 1 steps of one code-predictor frame, operator by operator (406 launches)
             ("next_predictor_frame_m1_steps", lambda: PredictorFrameSteps(qm, dev)),
+            # the same fourteen steps as ONE launch of 256 resident blocks (same codes bit for bit)
+            ("next_predictor_frame_m1_steps_one_launch", lambda: PredictorFrameSteps(qm, dev, one_launch=True)),
         ]
         for key, make in extra:
             w = make()

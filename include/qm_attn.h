@@ -44,6 +44,7 @@ extern "C" {
 #define QM_STATUS_BAD_PAGE      1u /* page table entry outside [0, n_pages)          */
 #define QM_STATUS_BAD_POSITION  2u /* position / length beyond max_pages*page_size   */
 #define QM_STATUS_SPLIT_TIMEOUT 4u /* key-split prefill: a partner's record never came  */
+#define QM_STATUS_FRAME_TIMEOUT 8u /* predictor frame kernel: an operator's input never came */
 
 /* ---- paged KV cache descriptor -------------------------------------------- */
 /*
@@ -98,14 +99,21 @@ const char* qm_target_arch(void);
  *       matrix cores (fp32 accumulation, fp32 softmax, bf16(QK), bf16(*scale) and bf16(P) as the
  *       reference); 1: the reference's exact summation chain on the vector ALU (about 2.5x slower).
  *       The rotated K and the cache write-back are bit-identical in both; contexts agree within the
- *       operator's tolerance.  Other values make the call return QM_ERR_ARGUMENT. */
+ *       operator's tolerance.  Other values make the call return QM_ERR_ARGUMENT.
+ *   QM_OPT_PREDICTOR_FRAME_OPERATORS  0 (default): the engine's predictor frame (qm_engine.h) runs its M = 1
+ *       steps as one launch of qm_predictor_frame_steps; 1: operator by operator.  Same bits either way.
+ *   QM_OPT_PREDICTOR_FRAME_SPIN_LIMIT  0 (default): a block of qm_predictor_frame_steps repeats the request for
+ *       an operator's input up to 131 072 times before it gives up; > 0: that many times (1 makes nearly every
+ *       launch give up at once: for tests of the give-up path, whose every block still returns normally). */
 enum {
     QM_OPT_PREFILL_SCORE_ROUNDING = 0,
     QM_OPT_DECODE_TILES_PER_BLOCK = 1,
     QM_OPT_PREFILL_KERNEL = 2,
     QM_OPT_DECODE_STREAMING_LOADS = 3,
     QM_OPT_PREDICTOR_LOOP_KERNEL = 4,
-    QM_OPT_COUNT = 5
+    QM_OPT_PREDICTOR_FRAME_OPERATORS = 5,
+    QM_OPT_PREDICTOR_FRAME_SPIN_LIMIT = 6,
+    QM_OPT_COUNT = 7
 };
 /* Returns QM_ERR_ARGUMENT for an unknown option or a negative value. */
 int32_t qm_set_option(int32_t option, int32_t value);
@@ -379,6 +387,74 @@ int32_t qm_predictor_step_attention_m1(
     const uint16_t* cos_row, const uint16_t* sin_row,
     uint16_t* key_cache, uint16_t* value_cache, uint16_t* context_out,
     int32_t cache_position, float epsilon, void* hip_stream);
+
+/*
+ * The M = 1 steps first_step .. last_step (1 .. 14) of one code-predictor frame in ONE launch: replaces the graph of
+ * PersistentPredictor::capture_step (R17:13592-13854; 46 nodes per step) for those steps — per step the input
+ * projection (small_to_mtp_projection with bias, R17:13600-13612), five layers of RMSNorm + Q/K/V, QK-norm +
+ * RoPE + cache append + attention at cache position step + 1, o_proj, residual + post-norm + gate/up/SwiGLU,
+ * down_proj + residual (R17:13614-13780), the final norm with that step's head, the top-k sampler (top_k <= 0:
+ * arg-max) and the gather of the sampled code's embedding (R17:13782-13854) — with every rounding and summation
+ * order of the one-operator entry points of this header, whose results it equals bit for bit.
+ *
+ * qm_predictor_frame names the tensors (bf16, 16-byte aligned; geometry of R17:7951-7964: hidden 1024, 16 / 8
+ * heads of 128, intermediate 3072, outer dimension 2048, vocabulary 2048, five layers):
+ *   layers[i]: input_norm, post_norm [1024]; q_weight [2048][1024], k_weight, v_weight [1024][1024]; q_norm,
+ *     k_norm [128]; o_weight [1024][2048]; gate_weight, up_weight [3072][1024]; down_weight [1024][3072];
+ *     key_cache, value_cache [8][16][128] holding the frame's positions 0 .. first_step, appended to in place;
+ *   projection_weight [1024][2048], projection_bias [1024], final_norm [1024]; heads[s] [2048][1024] and
+ *   embeddings[s] [2048][2048] for the steps s run (other entries are not read); cosine, sine [16][128];
+ *   free_input [2048]: in, the input of first_step (the embedding gathered at the end of the step before); out, the
+ *     embedding of the last code sampled;  selected [16][2048]: row s + 1 receives the embedding of step s's code;
+ *   codes [16]: codes[s + 1] receives step s's code;  rng_state: the SplitMix64 state the draws advance.
+ *
+ * The launch is 256 blocks that stay resident and hand each operator's output to one another through
+ * `workspace` (qm_predictor_frame_workspace_bytes() bytes, 256-byte aligned, set up once by
+ * qm_predictor_frame_workspace_init and then carried from call to call: it numbers the operator instances so
+ * that a captured launch can be replayed).  It needs a device with 256 compute units all of which can hold one
+ * of its blocks (QM_ERR_NO_DEVICE otherwise), and two such launches must not overlap in time on one device: each
+ * would wait for blocks of its own that the other keeps out.  Every wait is bounded: if an input never comes the
+ * blocks OR QM_STATUS_FRAME_TIMEOUT into status_dev (optional) and return; the outputs are then not to be used
+ * and the workspace must be initialised again before the next call.
+ */
+typedef struct qm_predictor_frame_layer {
+    const uint16_t* input_norm;
+    const uint16_t* q_weight;
+    const uint16_t* k_weight;
+    const uint16_t* v_weight;
+    const uint16_t* q_norm;
+    const uint16_t* k_norm;
+    const uint16_t* o_weight;
+    const uint16_t* post_norm;
+    const uint16_t* gate_weight;
+    const uint16_t* up_weight;
+    const uint16_t* down_weight;
+    uint16_t* key_cache;
+    uint16_t* value_cache;
+} qm_predictor_frame_layer;
+
+typedef struct qm_predictor_frame {
+    qm_predictor_frame_layer layers[5];
+    const uint16_t* projection_weight;
+    const uint16_t* projection_bias;
+    const uint16_t* final_norm;
+    const uint16_t* heads[15];        /* [step] */
+    const uint16_t* embeddings[15];   /* [step] */
+    const uint16_t* cosine;
+    const uint16_t* sine;
+    uint16_t* free_input;
+    uint16_t* selected;
+    int32_t* codes;
+    uint64_t* rng_state;
+    float epsilon;
+} qm_predictor_frame;
+
+int64_t qm_predictor_frame_workspace_bytes(void);
+int32_t qm_predictor_frame_workspace_init(void* workspace, int64_t workspace_bytes, void* hip_stream);
+int32_t qm_predictor_frame_steps(
+    const qm_predictor_frame* frame, int32_t first_step, int32_t last_step,
+    int32_t top_k, float temperature,
+    void* workspace, int64_t workspace_bytes, uint32_t* status_dev, void* hip_stream);
 
 /*
  * The three layout operators in front of the staged attention at the predictor's step 0 (call site

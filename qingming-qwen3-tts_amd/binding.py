@@ -31,6 +31,25 @@ class KvCache(C.Structure):
     ]
 
 
+class PredictorFrameLayer(C.Structure):
+    """Mirror of qm_predictor_frame_layer (include/qm_attn.h)."""
+    _fields_ = [(name, C.c_void_p) for name in (
+        "input_norm", "q_weight", "k_weight", "v_weight", "q_norm", "k_norm", "o_weight", "post_norm",
+        "gate_weight", "up_weight", "down_weight", "key_cache", "value_cache")]
+
+
+class PredictorFrame(C.Structure):
+    """Mirror of qm_predictor_frame (include/qm_attn.h)."""
+    _fields_ = [
+        ("layers", PredictorFrameLayer * 5),
+        ("projection_weight", C.c_void_p), ("projection_bias", C.c_void_p), ("final_norm", C.c_void_p),
+        ("heads", C.c_void_p * 15), ("embeddings", C.c_void_p * 15),
+        ("cosine", C.c_void_p), ("sine", C.c_void_p),
+        ("free_input", C.c_void_p), ("selected", C.c_void_p), ("codes", C.c_void_p), ("rng_state", C.c_void_p),
+        ("epsilon", C.c_float),
+    ]
+
+
 def lib_path():
     return _LIB_PATH
 
@@ -70,6 +89,9 @@ _SIGNATURES = {
     "qm_predictor_attention_loop": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _I32, _F32, _PTR]),
     "qm_predictor_attention_staged": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _PTR]),
     "qm_predictor_step_attention_m1": (_I32, [_PTR] * 10 + [_I32, _F32, _PTR]),
+    "qm_predictor_frame_workspace_bytes": (C.c_int64, []),
+    "qm_predictor_frame_workspace_init": (_I32, [_PTR, C.c_int64, _PTR]),
+    "qm_predictor_frame_steps": (_I32, [C.POINTER(PredictorFrame), _I32, _I32, _I32, _F32, _PTR, C.c_int64, _PTR, _PTR]),
     "qm_predictor_transpose": (_I32, [_PTR, _PTR, _I32, _I32, _PTR]),
     "qm_predictor_rope_bhsd": (_I32, [_PTR] * 4 + [_I32, _I32, _PTR]),
     "qm_predictor_update_cache": (_I32, [_PTR, _PTR, _I32, _I32, _PTR]),
@@ -137,6 +159,8 @@ OPT_DECODE_TILES_PER_BLOCK = 1
 OPT_PREFILL_KERNEL = 2
 OPT_DECODE_STREAMING_LOADS = 3
 OPT_PREDICTOR_LOOP_KERNEL = 4
+OPT_PREDICTOR_FRAME_OPERATORS = 5
+OPT_PREDICTOR_FRAME_SPIN_LIMIT = 6
 
 
 def set_option(option, value):
@@ -369,6 +393,44 @@ def predictor_step_attention_m1(q, k, v, gq, gk, cos_row, sin_row, key_cache, va
     _check(lib().qm_predictor_step_attention_m1(_addr(q), _addr(k), _addr(v), _addr(gq), _addr(gk), _addr(cos_row),
                                                 _addr(sin_row), _addr(key_cache), _addr(value_cache), _addr(out),
                                                 position, eps, stream), "qm_predictor_step_attention_m1")
+
+
+STATUS_FRAME_TIMEOUT = 8
+
+
+def predictor_frame(layers, projection_weight, projection_bias, final_norm, heads, embeddings, cosine, sine, free_input,
+                    selected, codes, rng_state, epsilon=1e-6):
+    """qm_predictor_frame from tensors: `layers` is five dicts with the field names of qm_predictor_frame_layer,
+    `heads` / `embeddings` map a step (1..14) to its tensor.  The tensors must outlive the descriptor."""
+    frame = PredictorFrame()
+    for i, layer in enumerate(layers):
+        for name, _ in PredictorFrameLayer._fields_:
+            setattr(frame.layers[i], name, _addr(layer[name]))
+    frame.projection_weight, frame.projection_bias, frame.final_norm = (_addr(projection_weight), _addr(projection_bias),
+                                                                        _addr(final_norm))
+    for step, tensor in heads.items():
+        frame.heads[step] = _addr(tensor)
+    for step, tensor in embeddings.items():
+        frame.embeddings[step] = _addr(tensor)
+    frame.cosine, frame.sine = _addr(cosine), _addr(sine)
+    frame.free_input, frame.selected, frame.codes, frame.rng_state = (_addr(free_input), _addr(selected), _addr(codes),
+                                                                      _addr(rng_state))
+    frame.epsilon = epsilon
+    return frame
+
+
+def predictor_frame_workspace_bytes():
+    return lib().qm_predictor_frame_workspace_bytes()
+
+
+def predictor_frame_workspace_init(workspace, workspace_bytes, stream=0):
+    _check(lib().qm_predictor_frame_workspace_init(_addr(workspace), workspace_bytes, stream),
+           "qm_predictor_frame_workspace_init")
+
+
+def predictor_frame_steps(frame, first_step, last_step, top_k, temperature, workspace, workspace_bytes, status=None, stream=0):
+    _check(lib().qm_predictor_frame_steps(C.byref(frame), first_step, last_step, top_k, temperature, _addr(workspace),
+                                          workspace_bytes, _addr(status), stream), "qm_predictor_frame_steps")
 
 
 def predictor_transpose(x, out, rows, heads, stream=0):

@@ -62,6 +62,10 @@ struct qm_predictor {
     DeviceBuffer free_input, context_embedding, hidden_a, hidden_b, norm, q_linear, k_linear, v_linear, q_normed, k_normed,
         q_bhsd, k_bhsd, v_bhsd, q_rotated, k_rotated, context, attention, residual, post_norm, swiglu, logits,
         selected, codes, embedding_sum, next_input;
+    // the M = 1 steps as one launch (qm_predictor_frame_steps): only for the five-layer geometry it is built for
+    bool one_launch = false;
+    qm_predictor_frame frame = {};
+    DeviceBuffer frame_workspace, status;
 };
 
 namespace qm_engine {
@@ -178,6 +182,31 @@ static std::unique_ptr<qm_predictor> create_predictor(const std::string& model_d
     p->codes = DeviceBuffer(kCodeGroups * sizeof(int32_t));
     p->embedding_sum = DeviceBuffer(kOuter * 2); p->next_input = DeviceBuffer(kOuter * 2);
     hip_check(hipStreamSynchronize(stream), "predictor upload synchronize");   // the mapped files go away with `host`
+    p->status = DeviceBuffer(256);
+    hip_check(hipMemsetAsync(p->status.raw(), 0, p->status.bytes(), stream), "predictor status word");
+    if (p->layers.size() == 5) {
+        qm_predictor_frame& f = p->frame;
+        for (size_t i = 0; i < 5; ++i) {
+            PredictorLayer& w = p->layers[i];
+            qm_predictor_frame_layer& d = f.layers[i];
+            d.input_norm = w.input_norm.data(); d.q_weight = w.q_weight.data(); d.k_weight = w.k_weight.data(); d.v_weight = w.v_weight.data();
+            d.q_norm = w.q_norm.data(); d.k_norm = w.k_norm.data(); d.o_weight = w.o_weight.data(); d.post_norm = w.post_norm.data();
+            d.gate_weight = w.gate_weight.data(); d.up_weight = w.up_weight.data(); d.down_weight = w.down_weight.data();
+            d.key_cache = w.key_cache.u16(); d.value_cache = w.value_cache.u16();
+        }
+        f.projection_weight = p->projection_weight.data(); f.projection_bias = p->projection_bias.data(); f.final_norm = p->final_norm.data();
+        for (int step = 1; step < kPredSteps; ++step) {
+            f.heads[step] = p->heads[static_cast<size_t>(step)].data();
+            f.embeddings[step] = p->embeddings[static_cast<size_t>(step)].data();
+        }
+        f.cosine = p->cosine.u16(); f.sine = p->sine.u16();
+        f.free_input = p->free_input.u16(); f.selected = p->selected.u16(); f.codes = static_cast<int32_t*>(p->codes.raw());
+        f.rng_state = rng_state; f.epsilon = kEpsilon;
+        p->frame_workspace = DeviceBuffer(static_cast<size_t>(qm_predictor_frame_workspace_bytes()));
+        op_check(qm_predictor_frame_workspace_init(p->frame_workspace.raw(), static_cast<int64_t>(p->frame_workspace.bytes()), stream),
+                 "predictor frame workspace");
+        p->one_launch = true;
+    }
     return p;
 }
 
@@ -282,11 +311,30 @@ static void predictor_frame(qm_predictor& p, const uint16_t* talker_hidden_devic
                                          p.free_input.u16(), p.selected.u16(), static_cast<int32_t*>(p.codes.raw()), s),
              "predictor group 0 input");
     predictor_step0(p, sampling);
-    for (int step = 1; step < kPredSteps; ++step) predictor_step_m1(p, step, sampling);
+    int32_t by_operators = 0;
+    op_check(qm_get_option(QM_OPT_PREDICTOR_FRAME_OPERATORS, &by_operators), "predictor frame option");
+    const bool one_launch = p.one_launch && by_operators == 0;
+    if (one_launch) {
+        op_check(qm_predictor_frame_steps(&p.frame, 1, kPredSteps - 1, sampling ? kTopK : 0, kTemperature, p.frame_workspace.raw(),
+                                          static_cast<int64_t>(p.frame_workspace.bytes()), static_cast<uint32_t*>(p.status.raw()), s),
+                 "predictor frame steps");
+    } else {
+        for (int step = 1; step < kPredSteps; ++step) predictor_step_m1(p, step, sampling);
+    }
     op_check(qm_predictor_next_talker_input(p.selected.u16(), kCodeGroups, p.context_embedding.u16(), kOuter, p.embedding_sum.u16(),
                                             p.next_input.u16(), s), "next talker input");
     hip_check(hipMemcpyAsync(codes_out, p.codes.raw(), kCodeGroups * sizeof(int32_t), hipMemcpyDeviceToHost, s), "codes read-back");
+    uint32_t status = 0;
+    if (one_launch) hip_check(hipMemcpyAsync(&status, p.status.raw(), sizeof status, hipMemcpyDeviceToHost, s), "status read-back");
     hip_check(hipStreamSynchronize(s), "predictor frame synchronize");
+    if (status != 0) {
+        // the frame kernel gave up waiting: its workspace starts over, the frame's codes are not to be used
+        hip_check(hipMemsetAsync(p.status.raw(), 0, sizeof status, s), "status reset");
+        op_check(qm_predictor_frame_workspace_init(p.frame_workspace.raw(), static_cast<int64_t>(p.frame_workspace.bytes()), s),
+                 "predictor frame workspace");
+        hip_check(hipStreamSynchronize(s), "predictor frame workspace synchronize");
+        throw ApiError(QM_ERR_STATUS, "the predictor frame kernel reported status " + std::to_string(status));
+    }
 }
 
 }  // namespace qm_engine

@@ -17,7 +17,7 @@ extern "C" const char* qm_error_string(int32_t code) {
         case QM_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
         case QM_ERR_ARGUMENT: return "invalid argument";
         case QM_ERR_NO_DEVICE: return "no usable gfx950 device";
-        case QM_ERR_STATUS: return "a kernel reported a status bit (bad page, bad position or key-split timeout)";
+        case QM_ERR_STATUS: return "a kernel reported a status bit (bad page, bad position, key-split or frame timeout)";
         default: break;
     }
     if (code <= QM_ERR_HIP_BASE) return hipGetErrorString(static_cast<hipError_t>(QM_ERR_HIP_BASE - code));
@@ -30,9 +30,11 @@ namespace {
 std::atomic<int32_t> g_options[QM_OPT_COUNT] = {
     {1},   // QM_OPT_PREFILL_SCORE_ROUNDING
     {0},   // QM_OPT_DECODE_TILES_PER_BLOCK (0 = chosen from the problem size)
-    {0},   // QM_OPT_PREFILL_KERNEL (0 = chosen from the grid size, 1 = four uniform waves, 2 = matrix/softmax wave pairs)
+    {0},   // QM_OPT_PREFILL_KERNEL (0 = interleaved waves, 1 = four uniform waves)
     {0},   // QM_OPT_DECODE_STREAMING_LOADS (0 = chosen from the bytes of context, 1 = plain loads, 2 = non-temporal loads)
     {0},   // QM_OPT_PREDICTOR_LOOP_KERNEL (0 = matrix cores, 1 = the reference's exact summation chain)
+    {0},   // QM_OPT_PREDICTOR_FRAME_OPERATORS (0 = the frame's M = 1 steps as one launch, 1 = operator by operator)
+    {0},   // QM_OPT_PREDICTOR_FRAME_SPIN_LIMIT (0 = the kernel's own bound)
 };
 }  // namespace
 

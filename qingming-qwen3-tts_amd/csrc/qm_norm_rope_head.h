@@ -28,31 +28,41 @@ struct HeadPair {
     uint16_t hi;  // dimension lane + 64
 };
 
-// RMSNorm (optional) + RoPE of one head; returns the two output bit patterns.
+// RMSNorm (optional) + RoPE of one head from operands already in registers (gamma, cosine and sine at
+// dimensions lane and lane + 64 as bf16 bits); returns the two output bit patterns.
+__device__ __forceinline__ HeadPair norm_rope_head_values(uint16_t x0b, uint16_t x1b, bool has_gamma,
+                                                          uint16_t gamma0, uint16_t gamma1, uint16_t cos0, uint16_t cos1,
+                                                          uint16_t sin0, uint16_t sin1, float epsilon) {
+    float w0 = bf2f(x0b);
+    float w1 = bf2f(x1b);
+    if (has_gamma) {
+        const float sum = head_sum_squares(w0, w1);
+        const float r = 1.0f / sqrtf(sum / 128.0f + epsilon);
+        const float n0 = bf2f(f2bf(w0 * r));
+        const float n1 = bf2f(f2bf(w1 * r));
+        w0 = bf2f(f2bf(n0 * bf2f(gamma0)));
+        w1 = bf2f(f2bf(n1 * bf2f(gamma1)));
+    }
+    // rotate_half(x) = (-x2, +x1): dimension d < 64 pairs with -x[d+64], d >= 64 with +x[d-64].
+    const float first0 = bf2f(f2bf(w0 * bf2f(cos0)));
+    const float second0 = bf2f(f2bf((-w1) * bf2f(sin0)));
+    const float first1 = bf2f(f2bf(w1 * bf2f(cos1)));
+    const float second1 = bf2f(f2bf(w0 * bf2f(sin1)));
+    HeadPair out;
+    out.lo = f2bf(first0 + second0);
+    out.hi = f2bf(first1 + second1);
+    return out;
+}
+
+// The same with gamma (NULL: no RMSNorm), cosine and sine read from memory.
 __device__ __forceinline__ HeadPair norm_rope_head(uint16_t x0b, uint16_t x1b,
                                                    const uint16_t* __restrict__ gamma,
                                                    const uint16_t* __restrict__ cosv,
                                                    const uint16_t* __restrict__ sinv,
                                                    float epsilon, int lane) {
-    float w0 = bf2f(x0b);
-    float w1 = bf2f(x1b);
-    if (gamma) {
-        const float sum = head_sum_squares(w0, w1);
-        const float r = 1.0f / sqrtf(sum / 128.0f + epsilon);
-        const float n0 = bf2f(f2bf(w0 * r));
-        const float n1 = bf2f(f2bf(w1 * r));
-        w0 = bf2f(f2bf(n0 * bf2f(gamma[lane])));
-        w1 = bf2f(f2bf(n1 * bf2f(gamma[lane + 64])));
-    }
-    // rotate_half(x) = (-x2, +x1): dimension d < 64 pairs with -x[d+64], d >= 64 with +x[d-64].
-    const float first0 = bf2f(f2bf(w0 * bf2f(cosv[lane])));
-    const float second0 = bf2f(f2bf((-w1) * bf2f(sinv[lane])));
-    const float first1 = bf2f(f2bf(w1 * bf2f(cosv[lane + 64])));
-    const float second1 = bf2f(f2bf(w0 * bf2f(sinv[lane + 64])));
-    HeadPair out;
-    out.lo = f2bf(first0 + second0);
-    out.hi = f2bf(first1 + second1);
-    return out;
+    return norm_rope_head_values(x0b, x1b, gamma != nullptr, gamma ? gamma[lane] : static_cast<uint16_t>(0),
+                                 gamma ? gamma[lane + 64] : static_cast<uint16_t>(0), cosv[lane], cosv[lane + 64],
+                                 sinv[lane], sinv[lane + 64], epsilon);
 }
 
 }  // namespace qm

@@ -18,7 +18,7 @@ from qm_testlib import to_u16
 pytestmark = pytest.mark.gpu
 
 H, Q, KV, I_T, T_LAYERS = 2048, 2048, 1024, 512, 2           # talker (small intermediate: the test is about the loop)
-PH, PI, P_LAYERS, V, STEPS = 1024, 3072, 2, 2048, 15            # predictor; two layers keep the CPU chain short
+PH, PI, P_LAYERS, V, STEPS = 1024, 3072, 5, 2048, 15            # predictor: its real geometry (the one-launch frame kernel needs it)
 HEAD_V, EOS, TABLE_ROWS = 3072, 2150, 3072
 SEED = 20240229
 
@@ -167,9 +167,20 @@ def _oracle_predictor_frame(oracle, w, hidden, code0, context, rng, sampling=Tru
     return codes, nxt_input
 
 
-def test_final_head_and_predictor_frame_match_the_oracle_chain(engine, oracle, qm, dev, model):
+@pytest.mark.parametrize("by_operators", [0, 1], ids=["one_launch", "operator_by_operator"])
+def test_final_head_and_predictor_frame_match_the_oracle_chain(engine, oracle, qm, dev, model, by_operators):
+    """Both ways of running the frame's M = 1 steps (QM_OPT_PREDICTOR_FRAME_OPERATORS) against the oracle's chain."""
     import torch
     directory, w = model
+    qm.set_option(qm.OPT_PREDICTOR_FRAME_OPERATORS, by_operators)
+    try:
+        _frames_against_the_oracle(engine, oracle, dev, directory, w)
+    finally:
+        qm.set_option(qm.OPT_PREDICTOR_FRAME_OPERATORS, 0)
+
+
+def _frames_against_the_oracle(engine, oracle, dev, directory, w):
+    import torch
     talker = engine.Talker(directory, 64)
     head = engine.FinalHead(directory, 32, SEED, talker.stream)
     predictor = engine.Predictor(directory, head.rng_state, talker.stream)
@@ -191,6 +202,32 @@ def test_final_head_and_predictor_frame_match_the_oracle_chain(engine, oracle, q
         want_codes, want_next = _oracle_predictor_frame(oracle, w, hidden, code0, context, rng, sampling)
         assert codes == want_codes.tolist()
         assert np.array_equal(_device_bytes(predictor.next_input, H * 2), want_next)
+    predictor.close(); head.close(); talker.close()
+
+
+def test_predictor_frame_that_gives_up_reports_status_and_recovers(engine, oracle, qm, dev, model):
+    """With the frame kernel's waits cut to one attempt (QM_OPT_PREDICTOR_FRAME_SPIN_LIMIT = 1) a frame ends, every block
+    returning normally, with QM_ERR_STATUS; the engine sets its workspace up again and the next frame is right."""
+    import torch
+    directory, w = model
+    talker = engine.Talker(directory, 64)
+    head = engine.FinalHead(directory, 32, SEED, talker.stream)
+    predictor = engine.Predictor(directory, head.rng_state, talker.stream)
+    hidden = oracle.normal_bf16((H,), 700)
+    hd = torch.from_numpy(hidden.view(np.int16)).to(dev)
+    context = oracle.normal_bf16((H,), 701, 0.0, 0.5)
+    torch.cuda.synchronize()
+    code0 = head.run(hd, 0, True)
+    good = predictor.run_frame(hd, head.device_code, context, False)          # arg-max: no generator state involved
+    qm.set_option(qm.OPT_PREDICTOR_FRAME_SPIN_LIMIT, 1)
+    try:
+        with pytest.raises(engine.EngineError) as info:
+            predictor.run_frame(hd, head.device_code, context, False)
+        assert info.value.code == -9
+    finally:
+        qm.set_option(qm.OPT_PREDICTOR_FRAME_SPIN_LIMIT, 0)
+    assert predictor.run_frame(hd, head.device_code, context, False) == good
+    assert good[0] == code0
     predictor.close(); head.close(); talker.close()
 
 
