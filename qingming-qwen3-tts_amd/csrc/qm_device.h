@@ -132,19 +132,32 @@ __device__ __forceinline__ int64_t tile_offset(const qm_kv_cache& c, const PageM
          + static_cast<int64_t>(first_token - page * pm.page_size) * kDim;
 }
 
+// The reference's wave reduction, value += shfl_down(value, offset, 32) for offset 16, 8, 4, 2, 1 (R17:9359-9364,
+// 15059-15075), for the lane whose result is used: lane 0 of each 32-lane half of the wave ends with the sum that
+// loop leaves there, formed by the same additions in the same order (other lanes end with something else).
+// No LDS traffic: the exchange between the two 16-lane rows is v_permlane16_swap, the rest are DPP row shifts,
+// whose lanes beyond the row read zero.
+__device__ __forceinline__ float half_wave_tree_sum(float v) {
+    const auto rows = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(rows[0]) + __uint_as_float(rows[1]);      // every lane: its own value + that of lane ^ 16
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x108, 0xf, 0xf, true));   // row_shl:8
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x104, 0xf, 0xf, true));   // row_shl:4
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x102, 0xf, 0xf, true));   // row_shl:2
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x101, 0xf, 0xf, true));   // row_shl:1
+    return v;
+}
+
 // block_reduce_sum / talker_block_sum of the reference (R17:8233-8274, 15102-15148) for a block of 256
 // threads: eight 32-lane shfl_down trees, then one tree over the eight results.  sh_waves: 8 floats,
 // sh_total: 1 float of LDS; the total is valid in every thread.
 __device__ __forceinline__ float block_sum_256_like_reference(float value, float* sh_waves, float* sh_total) {
     const int tid = threadIdx.x;
-#pragma unroll
-    for (int offset = 16; offset > 0; offset >>= 1) value += __shfl_down(value, offset, 32);
+    value = half_wave_tree_sum(value);
     if ((tid & 31) == 0) sh_waves[tid >> 5] = value;
     __syncthreads();
     if (tid < 32) {
         float v = tid < 8 ? sh_waves[tid] : 0.0f;
-#pragma unroll
-        for (int offset = 16; offset > 0; offset >>= 1) v += __shfl_down(v, offset, 32);
+        v = half_wave_tree_sum(v);
         if (tid == 0) *sh_total = v;
     }
     __syncthreads();

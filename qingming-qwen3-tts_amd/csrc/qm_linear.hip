@@ -479,11 +479,8 @@ __global__ __launch_bounds__(kStagedThreads) void linear_m1_staged_kernel(Linear
         }
     }
     // the reference's shuffle tree over its 32 lanes; lane 0 holds the sum
-#pragma unroll
-    for (int offset = 16; offset > 0; offset >>= 1) {
-        acc += __shfl_down(acc, offset, 32);
-        if (DUAL) up += __shfl_down(up, offset, 32);
-    }
+    acc = half_wave_tree_sum(acc);
+    if (DUAL) up = half_wave_tree_sum(up);
     if (l == 0 && live) {
         if (DUAL) {
             const float gv = bf2f(f2bf(acc));

@@ -167,11 +167,8 @@ __global__ __launch_bounds__(kRowsThreads) void linear_rows_kernel(LinearRowsPar
         // the reference's shuffle tree over its 32 lanes, per token row; lane 0 holds the sums
 #pragma unroll
         for (int r = 0; r < SPAN; ++r) {
-#pragma unroll
-            for (int offset = 16; offset > 0; offset >>= 1) {
-                acc[r] += __shfl_down(acc[r], offset, 32);
-                if (DUAL) up[r] += __shfl_down(up[r], offset, 32);
-            }
+            acc[r] = half_wave_tree_sum(acc[r]);
+            if (DUAL) up[r] = half_wave_tree_sum(up[r]);
         }
         if (l == 0 && live) {
 #pragma unroll

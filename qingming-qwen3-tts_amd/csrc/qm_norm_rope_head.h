@@ -12,15 +12,10 @@ namespace qm {
 // group sums w0..w3 are combined as (w0 + w2) + (w1 + w3), which is what the
 // reference's second-level tree over wave sums evaluates to.
 __device__ __forceinline__ float head_sum_squares(float x0, float x1) {
-    float s0 = x0 * x0;
-    float s1 = x1 * x1;
-#pragma unroll
-    for (int offset = 16; offset > 0; offset >>= 1) {
-        s0 += __shfl_down(s0, offset, 32);
-        s1 += __shfl_down(s1, offset, 32);
-    }
-    const float t = s0 + s1;            // lane 0: w0 + w2, lane 32: w1 + w3
-    return __shfl(t, 0) + __shfl(t, 32);
+    const float s0 = half_wave_tree_sum(x0 * x0);    // lane 0: w0 (dims 0..31), lane 32: w1 (dims 32..63)
+    const float s1 = half_wave_tree_sum(x1 * x1);    // lane 0: w2 (dims 64..95), lane 32: w3
+    const float t = s0 + s1;                         // lane 0: w0 + w2, lane 32: w1 + w3
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(t), 0)) + __int_as_float(__builtin_amdgcn_readlane(__float_as_int(t), 32));
 }
 
 struct HeadPair {

@@ -253,6 +253,20 @@ __device__ __forceinline__ bool linear_phase(FrShared& sh, unsigned char* smem, 
     if (sh.abort) return false;
 
     const int l = tid & 31;             // reference lane
+    // This lane's share of the input vector, read once for all passes; then per output all of its weights are
+    // requested from LDS before the chain starts, so that the chain waits for additions, not for reads.
+    constexpr int kSteps = PAIRS ? K / 64 : K / 32;
+    float2 x_pair[PAIRS ? kSteps : 1];
+    float x_one[PAIRS ? 1 : kSteps];
+    if (PAIRS) {
+        const float2* xp = reinterpret_cast<const float2*>(lin_x) + l;
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j) x_pair[j] = xp[32 * j];
+    } else {
+        const float* xs = lin_x + l;
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j) x_one[j] = xs[32 * j];
+    }
 #pragma unroll 1
     for (int c0 = 0; c0 < R; c0 += 8) {
         const int c = c0 + (tid >> 5);
@@ -260,51 +274,35 @@ __device__ __forceinline__ bool linear_phase(FrShared& sh, unsigned char* smem, 
         const unsigned char* row0 = smem + lds_weights + (live ? (DUAL ? 2 * c : c) : 0) * kStride;
         const unsigned char* row1 = row0 + kStride;                 // DUAL only: the up row
         float acc = 0.0f, up = 0.0f;
-        if (live && PAIRS) {
+        if (PAIRS) {
             const uint32_t* p0 = reinterpret_cast<const uint32_t*>(row0) + l;
             const uint32_t* p1 = reinterpret_cast<const uint32_t*>(row1) + l;
-            const float2* xp = reinterpret_cast<const float2*>(lin_x) + l;
-#pragma unroll 1
-            for (int j = 0; j < K / 64; j += 8) {
-                float2 x[8];
-                uint32_t a[8], b[8];
+            uint32_t a[kSteps], b[DUAL ? kSteps : 1];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    x[u] = xp[32 * (j + u)];
-                    a[u] = p0[32 * (j + u)];
-                    if (DUAL) b[u] = p1[32 * (j + u)];
-                }
+            for (int j = 0; j < kSteps; ++j) {
+                a[j] = p0[32 * j];
+                if (DUAL) b[j] = p1[32 * j];
+            }
 #pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    acc = fmaf(x[u].x, lo_bf16(a[u]), acc);
-                    acc = fmaf(x[u].y, hi_bf16(a[u]), acc);
-                    if (DUAL) {
-                        up = fmaf(x[u].x, lo_bf16(b[u]), up);
-                        up = fmaf(x[u].y, hi_bf16(b[u]), up);
-                    }
+            for (int j = 0; j < kSteps; ++j) {
+                acc = fmaf(x_pair[j].x, lo_bf16(a[j]), acc);
+                acc = fmaf(x_pair[j].y, hi_bf16(a[j]), acc);
+                if (DUAL) {
+                    up = fmaf(x_pair[j].x, lo_bf16(b[j]), up);
+                    up = fmaf(x_pair[j].y, hi_bf16(b[j]), up);
                 }
             }
-        } else if (live) {
+        } else {
             const uint16_t* w0 = reinterpret_cast<const uint16_t*>(row0) + l;
-            const float* xs = lin_x + l;
-#pragma unroll 1
-            for (int j = 0; j < K / 32; j += 8) {
-                float x[8], a[8];
+            uint32_t a[kSteps];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    x[u] = xs[32 * (j + u)];
-                    a[u] = bf2f(w0[32 * (j + u)]);
-                }
+            for (int j = 0; j < kSteps; ++j) a[j] = w0[32 * j];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) acc = fmaf(x[u], a[u], acc);
-            }
+            for (int j = 0; j < kSteps; ++j) acc = fmaf(x_one[j], bf2f(static_cast<uint16_t>(a[j])), acc);
         }
         // the reference's shuffle tree over its 32 lanes; lane 0 holds the sum
-#pragma unroll
-        for (int offset = 16; offset > 0; offset >>= 1) {
-            acc += __shfl_down(acc, offset, 32);
-            if (DUAL) up += __shfl_down(up, offset, 32);
-        }
+        acc = half_wave_tree_sum(acc);
+        if (DUAL) up = half_wave_tree_sum(up);
         if (l == 0 && live) {
             uint16_t bits;
             if (DUAL) {
@@ -397,8 +395,7 @@ __device__ __forceinline__ bool attention_phase(FrShared& sh, unsigned char* sme
             float acc = 0.0f;
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc = fmaf(q4[c], bf2f(kc[j * kDim + l + 32 * c]), acc);
-#pragma unroll
-            for (int offset = 16; offset > 0; offset >>= 1) acc += __shfl_down(acc, offset, 32);
+            acc = half_wave_tree_sum(acc);
             if (l == 0) probs[16 * g + j] = rbf(rbf(acc) * scale);
         }
     }
