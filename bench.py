@@ -462,6 +462,66 @@ class TalkerLayerStep:
         return {"all": dt}, err, "one layer step"
 
 
+class PromptLinears:
+    """Beyond the five configurations: the seven linears of one talker layer over a prompt of `rows` tokens as the
+    prompt pass chains them (NativeTalkerEngine::prefill, R17:16646-16790): q, k, v projections with bias, o_proj +
+    residual, gate/up/SwiGLU, down_proj + residual (hidden 2048, intermediate 6144).  kernel 0: the matrix cores
+    (default); 1: every sum in the reference's order (QM_OPT_LINEAR_ROWS_KERNEL)."""
+    bound = "mfma"
+
+    def __init__(self, qm, dev, rows=1024, kernel=0, seed=313):
+        import torch
+        self.qm, self.rows, self.kernel = qm, rows, kernel
+        self.name = "prompt_linears_%d_tokens_one_talker_layer%s" % (rows, "_exact_chain" if kernel else "")
+        syn = Synthetic(dev, seed)
+        H, KV, I = 2048, 1024, 6144
+        self.H, self.KV, self.I = H, KV, I
+        rnd = syn.normal
+        self.x, self.res = rnd((rows, H)), rnd((rows, H))
+        self.wq, self.wk, self.wv, self.wo = rnd((H, H), 0.02), rnd((KV, H), 0.02), rnd((KV, H), 0.02), rnd((H, H), 0.02)
+        self.bq, self.bk, self.bv = rnd((H,), 0.1), rnd((KV,), 0.1), rnd((KV,), 0.1)
+        self.wg, self.wu, self.wd = rnd((I, H), 0.02), rnd((I, H), 0.02), rnd((H, I), 0.02)
+        z = lambda n: torch.zeros((rows, n), dtype=torch.bfloat16, device=dev)
+        self.q, self.k, self.v, self.o, self.act, self.out = z(H), z(KV), z(KV), z(H), z(I), z(H)
+        self.flops = 2 * rows * (H * H + 2 * KV * H + H * H + 2 * I * H + H * I)
+        self.bytes = 2 * (H * H + 2 * KV * H + H * H + 2 * I * H + H * I) + 2 * rows * (6 * H + 2 * KV + 2 * I)
+        # outputs of magnitude 1 to 4: one bf16 spacing there
+        self.tolerance = 0.0625
+
+    def step(self):
+        import torch
+        qm, s, R, H, KV, I = self.qm, torch.cuda.current_stream().cuda_stream, self.rows, self.H, self.KV, self.I
+        qm.set_option(qm.OPT_LINEAR_ROWS_KERNEL, self.kernel)
+        try:
+            qm.linear_rows(self.x, self.wq, self.bq, None, self.q, R, H, H, s)
+            qm.linear_rows(self.x, self.wk, self.bk, None, self.k, R, KV, H, s)
+            qm.linear_rows(self.x, self.wv, self.bv, None, self.v, R, KV, H, s)
+            qm.linear_rows(self.q, self.wo, None, self.res, self.o, R, H, H, s)
+            qm.gate_up_swiglu_rows(self.o, self.wg, self.wu, self.act, R, H, I, s)
+            qm.linear_rows(self.act, self.wd, None, self.o, self.out, R, H, I, s)
+        finally:
+            qm.set_option(qm.OPT_LINEAR_ROWS_KERNEL, 0)
+
+    def cpu_baseline(self, oracle, threads):
+        """Sample: the first 8 token rows through the same chain."""
+        n = min(8, self.rows)
+        B = lambda t: _bits(t).copy()
+        u16 = lambda c: np.zeros((n, c), dtype=np.uint16)
+        x, res = B(self.x[:n]), B(self.res[:n])
+        q, k, v, o, act, out = u16(self.H), u16(self.KV), u16(self.KV), u16(self.H), u16(self.I), u16(self.H)
+        t0 = time.perf_counter()
+        assert oracle.linear_rows(x, B(self.wq), B(self.bq), None, q, n, self.H, self.H, threads) == 0
+        assert oracle.linear_rows(x, B(self.wk), B(self.bk), None, k, n, self.KV, self.H, threads) == 0
+        assert oracle.linear_rows(x, B(self.wv), B(self.bv), None, v, n, self.KV, self.H, threads) == 0
+        assert oracle.linear_rows(q, B(self.wo), None, res, o, n, self.H, self.H, threads) == 0
+        assert oracle.gate_up_swiglu_rows(o, B(self.wg), B(self.wu), act, n, self.H, self.I, threads) == 0
+        assert oracle.linear_rows(act, B(self.wd), None, o, out, n, self.H, self.I, threads) == 0
+        dt = time.perf_counter() - t0
+        err = float(np.max(np.abs(oracle.bf16_to_f32(out).astype(np.float64)
+                                  - oracle.bf16_to_f32(_bits(self.out[:n])).astype(np.float64))))
+        return {"all": dt * self.rows / n}, err, "first %d of %d token rows, time scaled" % (n, self.rows)
+
+
 class PredictorFrameSteps:
     """Beyond the five configurations: the fourteen M = 1 steps of one code-predictor frame as the
     reference chains them (PersistentPredictor::capture_step, R17:13592-13854): input projection,
@@ -779,7 +839,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
     ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "prefillfp32", "predictor", "predictorexact",
-                                      "qkv", "layer", "frame", "frame1"], default=None,
+                                      "qkv", "layer", "frame", "frame1", "linears", "linearsexact"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -819,7 +879,8 @@ def main():
                 "predictorexact": lambda: PredictorLoop(qm, dev, kernel=1),
                 "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev),
                 "frame": lambda: PredictorFrameSteps(qm, dev),
-                "frame1": lambda: PredictorFrameSteps(qm, dev, one_launch=True)}[args.only]
+                "frame1": lambda: PredictorFrameSteps(qm, dev, one_launch=True),
+                "linears": lambda: PromptLinears(qm, dev), "linearsexact": lambda: PromptLinears(qm, dev, kernel=1)}[args.only]
         w = make()
         r = _report(w, _time_steps(w.step, args.steps, args.warmup))
         r["bound"] = w.bound
@@ -862,6 +923,9 @@ def main():
             # the whole decode step of one talker layer, 28 layers' weights and caches in rotation (2.8 GB)
             ("next_talker_layer_decode_step", lambda: TalkerLayerStep(qm, dev)),
             ("next_talker_layer_decode_step_unfused", lambda: TalkerLayerStep(qm, dev, fused=False)),
+            # the seven linears of a talker layer over a 1024-token prompt: matrix cores, and the exact chain
+            ("next_prompt_linears_1024_tokens", lambda: PromptLinears(qm, dev)),
+            ("next_prompt_linears_1024_tokens_exact_chain", lambda: PromptLinears(qm, dev, kernel=1)),
             # the fourteen M = 1 steps of one code-predictor frame, operator by operator (406 launches)
             ("next_predictor_frame_m1_steps", lambda: PredictorFrameSteps(qm, dev)),
             # the same fourteen steps as ONE launch of 256 resident blocks (same codes bit for bit)

@@ -104,7 +104,11 @@ const char* qm_target_arch(void);
  *       steps as one launch of qm_predictor_frame_steps; 1: operator by operator.  Same bits either way.
  *   QM_OPT_PREDICTOR_FRAME_SPIN_LIMIT  0 (default): a block of qm_predictor_frame_steps repeats the request for
  *       an operator's input up to 131 072 times before it gives up; > 0: that many times (1 makes nearly every
- *       launch give up at once: for tests of the give-up path, whose every block still returns normally). */
+ *       launch give up at once: for tests of the give-up path, whose every block still returns normally).
+ *   QM_OPT_LINEAR_ROWS_KERNEL  0 (default): qm_linear_rows / qm_gate_up_swiglu_rows take the sums of calls with 16 or more
+ *       token rows on the matrix cores where the shape fits their tiles (output columns % 128 == 0, reduction % 128 == 0):
+ *       same roundings after the sum, results within the operators' tolerance of the exact chain; 1: every call in the
+ *       reference's summation order (bit-identical to the M = 1 operators; 20 to 60 times slower on long prompts). */
 enum {
     QM_OPT_PREFILL_SCORE_ROUNDING = 0,
     QM_OPT_DECODE_TILES_PER_BLOCK = 1,
@@ -113,7 +117,8 @@ enum {
     QM_OPT_PREDICTOR_LOOP_KERNEL = 4,
     QM_OPT_PREDICTOR_FRAME_OPERATORS = 5,
     QM_OPT_PREDICTOR_FRAME_SPIN_LIMIT = 6,
-    QM_OPT_COUNT = 7
+    QM_OPT_LINEAR_ROWS_KERNEL = 7,
+    QM_OPT_COUNT = 8
 };
 /* Returns QM_ERR_ARGUMENT for an unknown option or a negative value. */
 int32_t qm_set_option(int32_t option, int32_t value);

@@ -161,6 +161,7 @@ OPT_DECODE_STREAMING_LOADS = 3
 OPT_PREDICTOR_LOOP_KERNEL = 4
 OPT_PREDICTOR_FRAME_OPERATORS = 5
 OPT_PREDICTOR_FRAME_SPIN_LIMIT = 6
+OPT_LINEAR_ROWS_KERNEL = 7
 
 
 def set_option(option, value):

@@ -21,6 +21,7 @@
 
 #include "qm_device.h"
 #include "qm_host.h"
+#include "qm_linear_rows_params.h"
 
 namespace qm {
 
@@ -28,16 +29,6 @@ constexpr int kRowsThreads = 256;
 constexpr int kRowsTile = 8;                   // token rows per pass
 constexpr int kRowsLdsBudget = 156 * 1024;
 constexpr int kRowsMaxReduction = 16384;
-
-struct LinearRowsParams {
-    const uint16_t* input;        // [rows][reduction]
-    const uint16_t* weight[2];    // [columns][reduction]; [1] = the up matrix (DUAL)
-    const uint16_t* bias;         // [columns] or NULL
-    const uint16_t* residual;     // [rows][columns] or NULL
-    uint16_t* output;             // [rows][columns]
-    int rows, columns, reduction;
-    int columns_per_block;        // 8 or 4 (4: the two halves of the block take four token rows each)
-};
 
 __host__ __device__ inline int rows_w_stride(int reduction) { return 2 * reduction + 64; }   // bytes
 
@@ -236,6 +227,18 @@ inline int32_t check_rows(const LinearRowsParams& prm, bool dual) {
     return QM_OK;
 }
 
+// QM_OPT_LINEAR_ROWS_KERNEL: 0 = the matrix cores from kRowsMatrixMinimum token rows on, where the shape fits their tiles
+// (columns % 128 == 0, reduction % 128 == 0, 8-byte aligned rows of bias / residual / output); 1 = always the exact chain.
+constexpr int kRowsMatrixMinimum = 16;
+inline int32_t rows_on_matrix_cores(const LinearRowsParams& prm, int32_t* yes) {
+    const int32_t choice = option_value(QM_OPT_LINEAR_ROWS_KERNEL);
+    if (choice < 0 || choice > 1) return QM_ERR_ARGUMENT;
+    const uintptr_t align = reinterpret_cast<uintptr_t>(prm.bias) | reinterpret_cast<uintptr_t>(prm.residual)
+                          | reinterpret_cast<uintptr_t>(prm.output);
+    *yes = choice == 0 && prm.rows >= kRowsMatrixMinimum && prm.columns % 128 == 0 && prm.reduction % 128 == 0 && (align & 7) == 0;
+    return QM_OK;
+}
+
 }  // namespace qm
 
 extern "C" int32_t qm_linear_rows(const uint16_t* input, const uint16_t* weight, const uint16_t* bias,
@@ -248,6 +251,10 @@ extern "C" int32_t qm_linear_rows(const uint16_t* input, const uint16_t* weight,
     prm.output = output; prm.rows = rows; prm.columns = output_columns; prm.reduction = reduction_columns;
     const int32_t rc = check_rows(prm, false);
     if (rc != QM_OK) return rc;
+    int32_t matrix_cores = 0;
+    const int32_t rc_kernel = rows_on_matrix_cores(prm, &matrix_cores);
+    if (rc_kernel != QM_OK) return rc_kernel;
+    if (matrix_cores) return launch_rows_mfma(prm, false, static_cast<hipStream_t>(hip_stream));
     return launch_rows<false>(prm, static_cast<hipStream_t>(hip_stream));
 }
 
@@ -261,5 +268,9 @@ extern "C" int32_t qm_gate_up_swiglu_rows(const uint16_t* input, const uint16_t*
     prm.output = output; prm.rows = rows; prm.columns = intermediate; prm.reduction = hidden;
     const int32_t rc = check_rows(prm, true);
     if (rc != QM_OK) return rc;
+    int32_t matrix_cores = 0;
+    const int32_t rc_kernel = rows_on_matrix_cores(prm, &matrix_cores);
+    if (rc_kernel != QM_OK) return rc_kernel;
+    if (matrix_cores) return launch_rows_mfma(prm, true, static_cast<hipStream_t>(hip_stream));
     return launch_rows<true>(prm, static_cast<hipStream_t>(hip_stream));
 }

@@ -1,0 +1,23 @@
+// qm_linear_rows_params.h — launch parameters shared by the two kernels behind qm_linear_rows / qm_gate_up_swiglu_rows.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace qm {
+
+struct LinearRowsParams {
+    const uint16_t* input;        // [rows][reduction]
+    const uint16_t* weight[2];    // [columns][reduction]; [1] = the up matrix (DUAL)
+    const uint16_t* bias;         // [columns] or NULL
+    const uint16_t* residual;     // [rows][columns] or NULL
+    uint16_t* output;             // [rows][columns]
+    int rows, columns, reduction;
+    int columns_per_block;        // 8 or 4 (4: the two halves of the block take four token rows each)
+};
+
+// The row linears on the matrix cores (qm_linear_rows_mfma.hip).  `dual`: weight[0] / weight[1] are the gate and up
+// matrices and the epilogue is SwiGLU.  Needs columns % 128 == 0 and reduction % 128 == 0 (checked by the caller).
+int32_t launch_rows_mfma(const LinearRowsParams& prm, bool dual, hipStream_t stream);
+
+}  // namespace qm

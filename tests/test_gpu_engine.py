@@ -195,9 +195,20 @@ def test_engine_prefill_of_a_long_prompt_shares_query_tiles_between_blocks(engin
                 assert gap(a, b) <= 0.0625
 
 
-def test_engine_prefill_then_decode_matches_the_oracle_chain(engine, oracle, qm, dev, tmp_path):
+@pytest.mark.parametrize("rows_kernel", [1, 0], ids=["exact_chain_linears", "matrix_core_linears"])
+def test_engine_prefill_then_decode_matches_the_oracle_chain(engine, oracle, qm, dev, tmp_path, rows_kernel):
     """A 37-token prompt through qm_talker_prefill, then two decoded tokens: last-row hidden vectors,
-    and the caches the prompt leaves behind, against the oracle's chain of the same operators."""
+    and the caches the prompt leaves behind, against the oracle's chain of the same operators.  With the prompt's
+    linears on the exact chain (QM_OPT_LINEAR_ROWS_KERNEL = 1) layer 0's K/V are the oracle's to the bit; on the matrix
+    cores (default) a projection may land on the neighbouring bf16 value, so they are held to the attention budget."""
+    qm.set_option(qm.OPT_LINEAR_ROWS_KERNEL, rows_kernel)
+    try:
+        _prefill_then_decode(engine, oracle, qm, dev, tmp_path, rows_kernel == 1)
+    finally:
+        qm.set_option(qm.OPT_LINEAR_ROWS_KERNEL, 0)
+
+
+def _prefill_then_decode(engine, oracle, qm, dev, tmp_path, exact):
     import ctypes as C
     import torch
     w = _checkpoint(str(tmp_path), True)
@@ -249,7 +260,7 @@ def test_engine_prefill_then_decode_matches_the_oracle_chain(engine, oracle, qm,
         assert hip.hipMemcpy(kd.ctypes.data_as(C.c_void_p), C.c_void_p(ka), C.c_size_t(kd.nbytes), 2) == 0
         assert hip.hipMemcpy(vd.ctypes.data_as(C.c_void_p), C.c_void_p(va), C.c_size_t(vd.nbytes), 2) == 0
         assert not kd[:, S:].any() and not vd[:, S:].any()
-        if layer == 0:
+        if layer == 0 and exact:
             assert np.array_equal(kd, k_cache) and np.array_equal(vd, v_cache)
         else:
             for a, b in ((kd, k_cache), (vd, v_cache)):
