@@ -94,6 +94,7 @@ static std::unique_ptr<qm_talker> create_talker(const std::string& model_dir, in
         engine->own_stream = true;
     }
     hipStream_t upload = engine->stream;
+    StreamDrain drain(upload);             // (uploads read the mapped files: they finish before `host` goes, also on an error)
     auto optional = [&](const std::string& name) {
         const TensorView* t = host.maybe_suffix(name);
         return t ? Param(*t, upload) : Param();

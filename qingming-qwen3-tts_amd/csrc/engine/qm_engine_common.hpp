@@ -78,6 +78,16 @@ struct Param {
     const uint16_t* data() const { return present ? buffer.u16() : nullptr; }
 };
 
+// Declared after the object that owns the mapped checkpoint files and therefore destroyed before it, also when an
+// exception unwinds: the uploads still in flight on the stream read from those mappings.
+struct StreamDrain {
+    hipStream_t stream;
+    explicit StreamDrain(hipStream_t s) : stream(s) {}
+    StreamDrain(const StreamDrain&) = delete;
+    StreamDrain& operator=(const StreamDrain&) = delete;
+    ~StreamDrain() { (void)hipStreamSynchronize(stream); }
+};
+
 // Runs f, turning exceptions into codes.
 template <typename F>
 inline int32_t guarded(F&& f) {

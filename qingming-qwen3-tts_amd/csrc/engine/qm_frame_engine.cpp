@@ -74,6 +74,7 @@ static std::unique_ptr<qm_final_head> create_final_head(const std::string& model
                                                         hipStream_t stream) {
     if (capacity <= 0) throw ApiError(QM_ERR_ARGUMENT, "history capacity must be positive");
     ModelDirectory host(model_dir);
+    StreamDrain drain(stream);             // (uploads read the mapped files: they finish before `host` goes, also on an error)
     auto head = std::make_unique<qm_final_head>();
     head->stream = stream;
     head->weight = Param(host.suffix("talker.codec_head.weight"), stream);
@@ -108,6 +109,7 @@ static int32_t final_head_run(qm_final_head& h, const uint16_t* hidden_device, i
 static std::unique_ptr<qm_predictor> create_predictor(const std::string& model_dir, uint64_t* rng_state, hipStream_t stream) {
     if (!rng_state) throw ApiError(QM_ERR_NULL, "the predictor samples from the final head's generator state");
     ModelDirectory host(model_dir);
+    StreamDrain drain(stream);             // (uploads read the mapped files: they finish before `host` goes, also on an error)
     auto p = std::make_unique<qm_predictor>();
     p->stream = stream;
     p->rng_state = rng_state;

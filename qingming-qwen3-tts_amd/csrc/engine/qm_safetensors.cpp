@@ -240,7 +240,16 @@ SafeFile::SafeFile(const std::string& path) {
             TensorView t;
             t.name = entry.first;
             t.dtype = dtype->text;
-            for (const Json& d : shape->items) t.shape.push_back(static_cast<int64_t>(as_count(d, "an extent")));
+            // every extent fits an int and the element count cannot wrap: a crafted shape must not multiply out to
+            // the byte range of a smaller tensor
+            uint64_t count = 1;
+            for (const Json& d : shape->items) {
+                const uint64_t extent = as_count(d, "an extent");
+                if (extent > 0x7fffffffULL) throw TensorError("tensor extent beyond 2^31 - 1: " + t.name);
+                if (extent != 0 && count > (1ULL << 62) / extent) throw TensorError("tensor element count overflows: " + t.name);
+                count *= extent;
+                t.shape.push_back(static_cast<int64_t>(extent));
+            }
             const uint64_t begin = as_count(offsets->items[0], "an offset");
             const uint64_t end = as_count(offsets->items[1], "an offset");
             if (begin > end || end > data_bytes) throw IoError("tensor out of range: " + t.name);

@@ -112,6 +112,10 @@ def test_reader_rejects_malformed_files(engine, tmp_path):
         "unknown dtype": lambda: _raw_file(tmp, {"t": {"dtype": "Q4", "shape": [8], "data_offsets": [0, 8]}}, b"\0" * 8),
         "reversed offsets": lambda: _raw_file(tmp, {"t": {"dtype": "U8", "shape": [0], "data_offsets": [4, 2]}}, b"\0" * 8),
         "negative extent": lambda: _raw_file(tmp, {"t": {"dtype": "U8", "shape": [-1], "data_offsets": [0, 0]}}, b""),
+        # 2^32 x 2^32 x 2 wraps to 0 elements in 64 bits and would match the empty byte range
+        "element count that wraps": lambda: _raw_file(tmp, {"t": {"dtype": "U8", "shape": [4294967296, 4294967296, 2],
+                                                                  "data_offsets": [0, 0]}}, b""),
+        "extent beyond an int": lambda: _raw_file(tmp, {"t": {"dtype": "U8", "shape": [2147483648, 0], "data_offsets": [0, 0]}}, b""),
         "not JSON": lambda: _raw_file(tmp, b"{\"t\": [1, 2,}", b""),
         "entry without offsets": lambda: _raw_file(tmp, {"t": {"dtype": "U8", "shape": [1]}}, b"\0"),
         "trailing text": lambda: _raw_file(tmp, b"{} x", b""),
