@@ -6,20 +6,26 @@
 // instead of the reference's 32 lane-strided chains: bf16 inputs, fp32 accumulation, the same roundings after the sum,
 // results within the operators' tolerance of the exact-chain kernel (qm_linear_rows.hip), not bit-identical to it.
 //
-// A block of four waves owns 128 token rows x 128 output columns; a wave 64 x 64 as 2 x 2 MFMA tiles.  Both operands
-// are K-contiguous rows (x [m][k], w [n][k]), so one tile layout serves both: 64 k per step, a row of a tile is eight
-// 16-byte pieces in LDS, piece q of row r stored in slot q ^ (r % 8) so that the 32 rows a fragment read touches spread
-// over all banks.  An MFMA takes the weight rows as its A operand and the token rows as B (D = W X^T): a lane then
-// holds, for one token row, runs of four consecutive output columns — 8-byte stores.  The tiles of step t + 2 are
-// requested into registers before step t's MFMAs and written to LDS (three stages) an iteration later: one barrier
-// per step, two steps of arithmetic for a request to come back.  Bound: bf16 MFMA (2.5 PFLOP/s); algorithmic flops 2 m n k (x 2 for the gate/up pair).
+// A block of four waves owns 128 output columns x 128 token rows (waves 2 x 2, each 64 x 64 as 2 x 2 MFMA tiles) or, for
+// calls whose grid would leave CUs empty, x 64 token rows (waves 4 x 1, each 32 columns x 64 rows).  Both operands are
+// K-contiguous rows (x [m][k], w [n][k]), so one tile layout serves both: 64 k per step, a row of a tile is eight 16-byte
+// pieces in LDS, piece q of row r stored in slot q ^ (r % 8) so that the 32 rows a fragment read touches spread over all
+// banks.  An MFMA takes the weight rows as its A operand and the token rows as B (D = W X^T): a lane then holds, for one
+// token row, runs of four consecutive output columns — 8-byte stores.
+// The tiles go from memory straight into a ring of LDS stages (global_load_lds, no registers, the swizzle chosen by which
+// piece a lane fetches), three steps ahead (two for the gate/up pair, whose stage is 48 KiB); a step begins by waiting
+// until its own stage has landed (vmcnt counts the later stages' pieces still in flight), one barrier, then the request
+// for the stage just freed.  The fragment reads are inline assembly: the compiler makes every LDS read of its own wait
+// for all global_load_lds in flight, which would expose the memory latency in every step.
+// Bound: bf16 MFMA (2.5 PFLOP/s); algorithmic flops 2 m n k (x 2 for the gate/up pair).
 
 #include "qm_device.h"
 #include "qm_host.h"
 #include "qm_linear_rows_params.h"
 
+#include <type_traits>
+
 namespace qm {
-namespace {
 
 constexpr int kGmThreads = 256;
 constexpr int kGmTile = 128;                 // token rows and output columns per block
@@ -31,75 +37,74 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 // LDS byte offset of piece `piece` (16 bytes = 8 k) of row `row` inside a tile
 __device__ __forceinline__ int tile_slot(int row, int piece) { return (row * 8 + (piece ^ (row & 7))) * 16; }
 
-// A thread's share of one step's tiles on its way from memory to LDS: four 16-byte pieces per operand, kept as
-// vectors with constant element numbers (arrays carried round the loop end up in scratch memory).
-typedef uint32_t u32x16_t __attribute__((ext_vector_type(16)));
-struct GmStaged {
-    u32x16_t x, w, u;
-};
-__device__ __forceinline__ void gm_take(u32x16_t& to, const uint16_t* const (&src)[4], int k0) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint4 v = *reinterpret_cast<const uint4*>(src[i] + k0);
-        to[4 * i] = v.x; to[4 * i + 1] = v.y; to[4 * i + 2] = v.z; to[4 * i + 3] = v.w;
-    }
-}
-__device__ __forceinline__ void gm_put(const u32x16_t& from, const int (&dst)[4], unsigned char* tile) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-        *reinterpret_cast<uint4*>(tile + dst[i]) = make_uint4(from[4 * i], from[4 * i + 1], from[4 * i + 2], from[4 * i + 3]);
-}
-template <bool DUAL>
-__device__ __forceinline__ void gm_request(GmStaged& st, const uint16_t* const (&sx)[4], const uint16_t* const (&sw)[4],
-                                           const uint16_t* const (&su)[4], int k0) {
-    gm_take(st.x, sx, k0);
-    gm_take(st.w, sw, k0);
-    if (DUAL) gm_take(st.u, su, k0);
-}
-template <bool DUAL>
-__device__ __forceinline__ void gm_deposit(const GmStaged& st, const int (&dst)[4], unsigned char* stage) {
-    gm_put(st.x, dst, stage);
-    gm_put(st.w, dst, stage + kGmTileBytes);
-    if (DUAL) gm_put(st.u, dst, stage + 2 * kGmTileBytes);
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+// s_waitcnt that waits until at most N vector-memory operations are outstanding (nothing else)
+template <int N>
+__device__ __forceinline__ void gm_wait_vm() {
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-template <bool DUAL>
+// One wave's pieces of a stage: piece i goes to LDS bytes [4096 i, 4096 i + 1024) from `first` (the wave's first piece).
+template <int N>
+__device__ __forceinline__ void gm_request(const uint16_t* const (&src)[N], int k0, unsigned char* first) {
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+        __builtin_amdgcn_global_load_lds(src[i] + k0, (__attribute__((address_space(3))) void*)(first + 4096 * i), 16, 0, 0);
+}
+
+template <bool DUAL, int BM>
 __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRowsParams prm) {
     extern __shared__ __attribute__((aligned(16))) unsigned char gm_smem[];
-    constexpr int kOperands = DUAL ? 3 : 2;                      // x, w (, up)
-    constexpr int kStageBytes = kOperands * kGmTileBytes;
+    constexpr int kStages = DUAL ? 3 : 4;
+    constexpr int kXBytes = BM * kGmStep * 2;
+    constexpr int kWeights = DUAL ? 2 : 1;
+    constexpr int kStageBytes = kXBytes + kWeights * kGmTileBytes;
+    constexpr int kTn = BM == 128 ? 2 : 1;                        // MFMA tiles of a wave along the output columns
+    constexpr int kTm = 2;                                        // and along the token rows
+    // pieces of 1 KiB (one instruction of a wave) per stage: x, w (, up); dealt to the four waves in turn
+    constexpr int kPiecesX = kXBytes / 1024, kPiecesW = kGmTileBytes / 1024;
+    constexpr int kPerWave = (kPiecesX + kWeights * kPiecesW) / 4;
+    static_assert((kPiecesX + kWeights * kPiecesW) % 4 == 0, "pieces are dealt evenly to four waves");
+    static_assert(kPerWave * (kStages - 2) <= 63, "the wait counts the later stages' pieces");
+
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wave_n = wave & 1, wave_m = wave >> 1;
+    const int wave_n = BM == 128 ? (wave & 1) : wave;
+    const int wave_m = BM == 128 ? (wave >> 1) : 0;
     const int K = prm.reduction;
     const int n0 = static_cast<int>(blockIdx.x) * kGmTile;
-    const int m0 = static_cast<int>(blockIdx.y) * kGmTile;
+    const int m0 = static_cast<int>(blockIdx.y) * BM;
 
-    // ---- this thread's pieces of a step's tiles: piece index p = tid + 256 i (i < 4) of 1024 per tile; row p / 8,
-    // global piece (p % 8) ^ (row % 8) lands in slot p % 8 ----
-    const uint16_t* src_x[4];
-    const uint16_t* src_w[4];
-    const uint16_t* src_u[4];
-    int dst[4];
+    // ---- this wave's pieces of a stage: instruction q = wave + 4 i covers LDS bytes [1024 q, 1024 q + 1024) of the
+    // stage (x tile, then w, then up); its lane l fills slot l % 8 of tile row 8 (q within the tile) + l / 8 with
+    // global piece slot ^ (row % 8) ----
+    const uint16_t* src[kPerWave];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int p = tid + kGmThreads * i;
-        const int row = p >> 3, slot = p & 7;
+    for (int i = 0; i < kPerWave; ++i) {
+        const int q = wave + 4 * i;
+        const int operand = q < kPiecesX ? 0 : (q < kPiecesX + kPiecesW ? 1 : 2);
+        const int qt = q - (operand == 0 ? 0 : (operand == 1 ? kPiecesX : kPiecesX + kPiecesW));
+        const int row = 8 * qt + (lane >> 3), slot = lane & 7;
         const int piece = slot ^ (row & 7);
-        dst[i] = p * 16;
-        const int m = min(m0 + row, prm.rows - 1);                // rows past the end repeat the last one (never stored)
-        src_x[i] = prm.input + static_cast<int64_t>(m) * K + 8 * piece;
-        src_w[i] = prm.weight[0] + static_cast<int64_t>(n0 + row) * K + 8 * piece;
-        src_u[i] = prm.weight[DUAL ? 1 : 0] + static_cast<int64_t>(n0 + row) * K + 8 * piece;
+        if (operand == 0) {
+            const int m = min(m0 + row, prm.rows - 1);            // rows past the end repeat the last one (never stored)
+            src[i] = prm.input + static_cast<int64_t>(m) * K + 8 * piece;
+        } else {
+            src[i] = prm.weight[operand - 1] + static_cast<int64_t>(n0 + row) * K + 8 * piece;
+        }
     }
-    GmStaged staged_a, staged_b;
+    const int steps = K / kGmStep;
+    // (requests past the last step repeat it and land in a stage nobody reads again: the wait below counts pieces)
+#define QM_GM_REQUEST(step_)                                                                                             \
+    gm_request<kPerWave>(src, min((step_), steps - 1) * kGmStep, gm_smem + ((step_) % kStages) * kStageBytes + 1024 * wave)
 
-    f32x16_t acc[2][2], acc_up[DUAL ? 2 : 1][DUAL ? 2 : 1];
+    f32x16_t acc[kTn][kTm], acc_up[DUAL ? kTn : 1][DUAL ? kTm : 1];
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < kTn; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
+        for (int b = 0; b < kTm; ++b) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 acc[a][b][r] = 0.0f;
@@ -107,73 +112,93 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
             }
         }
 
-    // fragment of tile rows [32 t, 32 t + 32), k block kb (16 k): lane l takes row l % 32, piece 2 kb + l / 32
+    // fragment of tile rows [32 t, 32 t + 32), k block kb (16 k): lane l takes row l % 32, piece 2 kb + l / 32.  The LDS
+    // address of (tile 0 row, k block 0) per lane; tile t adds 32 rows = 4096 bytes, k block kb flips the slot by 2 kb.
     const int frag_row = lane & 31, frag_half = lane >> 5;
-    auto fragment = [&](const unsigned char* tile, int t, int kb) __attribute__((always_inline)) {
-        const int row = 32 * t + frag_row;
-        return *reinterpret_cast<const bf16x8_t*>(tile + tile_slot(row, 2 * kb + frag_half));
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)gm_smem));
+    uint32_t at_kb[4];                                            // byte offset inside a tile for each k block (row part included)
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) at_kb[kb] = static_cast<uint32_t>(frag_row * 128 + (((2 * kb + frag_half) ^ (frag_row & 7)) * 16));
+    struct Frags {
+        u32x4_t w[kTn], x[kTm], u[DUAL ? kTn : 1];
     };
-
-    // Two sets of staging registers: the tiles of step t + 2 are requested while step t is multiplied, and written to
-    // LDS (three stages) an iteration later, so that a request has two steps of arithmetic to come back.
-    const int steps = K / kGmStep;
-    // the MFMAs of k blocks [kb0, kb0 + 2) of a step
-    auto multiply = [&](int step, int kb0) __attribute__((always_inline)) {
-        const unsigned char* stage = gm_smem + (step % 3) * kStageBytes;
-        const unsigned char* x_tile = stage;
-        const unsigned char* w_tile = stage + kGmTileBytes;
-        const unsigned char* u_tile = stage + 2 * kGmTileBytes;
-#pragma unroll
-        for (int kb = kb0; kb < kb0 + 2; ++kb) {
-            bf16x8_t wf[2], xf[2], uf[2];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                wf[t] = fragment(w_tile, 2 * wave_n + t, kb);
-                xf[t] = fragment(x_tile, 2 * wave_m + t, kb);
-                if (DUAL) uf[t] = fragment(u_tile, 2 * wave_n + t, kb);
-            }
-#pragma unroll
-            for (int a = 0; a < 2; ++a)
-#pragma unroll
-                for (int b = 0; b < 2; ++b) {
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[a], xf[b], acc[a][b], 0, 0, 0);
-                    if (DUAL) acc_up[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(uf[a], xf[b], acc_up[a][b], 0, 0, 0);
-                }
+    auto read_frags = [&](Frags& f, uint32_t stage_at, int kb) __attribute__((always_inline)) {
+        const uint32_t x_at = stage_at + at_kb[kb] + static_cast<uint32_t>(wave_m * kTm * 4096);
+        const uint32_t w_at = stage_at + kXBytes + at_kb[kb] + static_cast<uint32_t>(wave_n * kTn * 4096);
+        // (offsets are literal: tile t of an operand lies 32 rows = 4096 bytes further on)
+        asm volatile("ds_read_b128 %0, %1" : "=v"(f.w[0]) : "v"(w_at));
+        if (DUAL) asm volatile("ds_read_b128 %0, %1 offset:16384" : "=v"(f.u[0]) : "v"(w_at));
+        if (kTn == 2) {
+            asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(f.w[kTn - 1]) : "v"(w_at));
+            if (DUAL) asm volatile("ds_read_b128 %0, %1 offset:20480" : "=v"(f.u[kTn - 1]) : "v"(w_at));
+        }
+        asm volatile("ds_read_b128 %0, %1" : "=v"(f.x[0]) : "v"(x_at));
+        asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(f.x[1]) : "v"(x_at));
+    };
+    static_assert(kGmTileBytes == 16384 && kTm == 2, "the literal offsets of the fragment reads");
+    constexpr int kReads = kTn * (DUAL ? 2 : 1) + kTm;            // LDS reads per k block and lane
+    // the results of read_frags(f, ...) may be used once at most `later` reads issued after them are outstanding
+    auto arrived = [&](Frags& f, auto later) __attribute__((always_inline)) {
+        if constexpr (kTn == 2 && DUAL) {
+            asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(f.w[0]), "+v"(f.w[1]), "+v"(f.u[0]), "+v"(f.u[1]), "+v"(f.x[0]), "+v"(f.x[1])
+                         : "n"(decltype(later)::value) : "memory");
+        } else if constexpr (kTn == 2) {
+            asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(f.w[0]), "+v"(f.w[1]), "+v"(f.x[0]), "+v"(f.x[1]) : "n"(decltype(later)::value) : "memory");
+        } else if constexpr (DUAL) {
+            asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(f.w[0]), "+v"(f.u[0]), "+v"(f.x[0]), "+v"(f.x[1]) : "n"(decltype(later)::value) : "memory");
+        } else {
+            asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(f.w[0]), "+v"(f.x[0]), "+v"(f.x[1]) : "n"(decltype(later)::value) : "memory");
         }
     };
-    // (requests past the last step repeat it and their tiles land in a stage nobody reads again: staging that is
-    // conditional on the step makes the compiler keep the staged registers in scratch memory)
-    auto k_of = [&](int step) { return min(step, steps - 1) * kGmStep; };
-    gm_request<DUAL>(staged_a, src_x, src_w, src_u, k_of(0));
-    gm_request<DUAL>(staged_b, src_x, src_w, src_u, k_of(1));
-    gm_deposit<DUAL>(staged_a, dst, gm_smem);
-    __syncthreads();
-    for (int step = 0; step < steps; step += 2) {
-        // (the next step's tiles are written to LDS between the two halves of a step's MFMAs, which hide the writes)
-        gm_request<DUAL>(staged_a, src_x, src_w, src_u, k_of(step + 2));
-        multiply(step, 0);
-        gm_deposit<DUAL>(staged_b, dst, gm_smem + ((step + 1) % 3) * kStageBytes);
-        multiply(step, 2);
-        __syncthreads();
-        gm_request<DUAL>(staged_b, src_x, src_w, src_u, k_of(step + 3));
-        multiply(step + 1, 0);                          // (the number of steps is even: reduction % 128 == 0)
-        gm_deposit<DUAL>(staged_a, dst, gm_smem + ((step + 2) % 3) * kStageBytes);
-        multiply(step + 1, 2);
-        __syncthreads();
+    auto multiply = [&](const Frags& f) __attribute__((always_inline)) {
+#pragma unroll
+        for (int a = 0; a < kTn; ++a)
+#pragma unroll
+            for (int b = 0; b < kTm; ++b) {
+                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, f.w[a]), __builtin_bit_cast(bf16x8_t, f.x[b]),
+                                                                    acc[a][b], 0, 0, 0);
+                if (DUAL)
+                    acc_up[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, f.u[a]),
+                                                                           __builtin_bit_cast(bf16x8_t, f.x[b]), acc_up[a][b], 0, 0, 0);
+            }
+    };
+
+#pragma unroll
+    for (int ahead = 0; ahead < kStages - 1; ++ahead) QM_GM_REQUEST(ahead);
+    for (int step = 0; step < steps; ++step) {
+        gm_wait_vm<kPerWave * (kStages - 2)>();                   // this wave's pieces of the step's stage have landed
+        asm volatile("s_barrier" ::: "memory");                   // everybody's have; and everybody is done with the stage before
+        QM_GM_REQUEST(step + kStages - 1);
+        const uint32_t stage_at = lds_base + static_cast<uint32_t>((step % kStages) * kStageBytes);
+        Frags f0, f1;
+        read_frags(f0, stage_at, 0);
+        read_frags(f1, stage_at, 1);
+        arrived(f0, std::integral_constant<int, kReads>{});
+        multiply(f0);
+        read_frags(f0, stage_at, 2);
+        arrived(f1, std::integral_constant<int, kReads>{});
+        multiply(f1);
+        read_frags(f1, stage_at, 3);
+        arrived(f0, std::integral_constant<int, kReads>{});
+        multiply(f0);
+        arrived(f1, std::integral_constant<int, 0>{});
+        multiply(f1);
     }
+    gm_wait_vm<0>();                                              // (the requests past the last step, before the block's LDS goes)
+#undef QM_GM_REQUEST
 
     // ---- epilogue: accumulator register r of a lane is output column 8 (r / 4) + 4 (lane / 32) + r % 4 of the MFMA
     // tile's 32, token row lane % 32 ----
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
+    for (int a = 0; a < kTn; ++a) {
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            const int m = m0 + 64 * wave_m + 32 * b + (lane & 31);
+        for (int b = 0; b < kTm; ++b) {
+            const int m = m0 + 32 * (kTm * wave_m + b) + (lane & 31);
             const bool inside = m < prm.rows;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 if (!inside) break;
-                const int n = n0 + 64 * wave_n + 32 * a + 8 * g + 4 * (lane >> 5);
+                const int n = n0 + 32 * (kTn * wave_n + a) + 8 * g + 4 * (lane >> 5);
                 uint16_t bits[4];
                 uint2 res = make_uint2(0, 0);
                 if (!DUAL && prm.residual) res = *reinterpret_cast<const uint2*>(prm.residual + static_cast<int64_t>(m) * prm.columns + n);
@@ -202,25 +227,26 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
     }
 }
 
-}  // namespace
+template <bool DUAL, int BM>
+int32_t launch_rows_mfma_as(const LinearRowsParams& prm, hipStream_t stream) {
+    constexpr int kStages = DUAL ? 3 : 4;
+    constexpr int smem = kStages * (BM * kGmStep * 2 + (DUAL ? 2 : 1) * kGmTileBytes);
+    const dim3 grid(static_cast<unsigned>(prm.columns / kGmTile), static_cast<unsigned>((prm.rows + BM - 1) / BM));
+    if (grid.y > 65535u) return QM_ERR_ARGUMENT;
+    static std::atomic<bool> lds_raised[kMaxDevices];
+    const int32_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(linear_rows_mfma_kernel<DUAL, BM>), smem, lds_raised);
+    if (rc != QM_OK) return rc;
+    hipLaunchKernelGGL((linear_rows_mfma_kernel<DUAL, BM>), grid, dim3(kGmThreads), smem, stream, prm);
+    return launch_status();
+}
 
 int32_t launch_rows_mfma(const LinearRowsParams& prm, bool dual, hipStream_t stream) {
     if (prm.rows == 0 || prm.columns == 0) return QM_OK;
-    const dim3 grid(static_cast<unsigned>(prm.columns / kGmTile), static_cast<unsigned>((prm.rows + kGmTile - 1) / kGmTile));
-    if (grid.y > 65535u) return QM_ERR_ARGUMENT;
-    static std::atomic<bool> lds_raised[2][kMaxDevices];
-    if (dual) {
-        const int smem = 3 * 3 * kGmTileBytes;
-        const int32_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(linear_rows_mfma_kernel<true>), smem, lds_raised[1]);
-        if (rc != QM_OK) return rc;
-        hipLaunchKernelGGL(linear_rows_mfma_kernel<true>, grid, dim3(kGmThreads), smem, stream, prm);
-    } else {
-        const int smem = 3 * 2 * kGmTileBytes;
-        const int32_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(linear_rows_mfma_kernel<false>), smem, lds_raised[0]);
-        if (rc != QM_OK) return rc;
-        hipLaunchKernelGGL(linear_rows_mfma_kernel<false>, grid, dim3(kGmThreads), smem, stream, prm);
-    }
-    return launch_status();
+    // blocks of 64 token rows where blocks of 128 would leave CUs without one (one block per CU either way)
+    const int64_t blocks_128 = static_cast<int64_t>(prm.columns / kGmTile) * ((prm.rows + 127) / 128);
+    const bool small = blocks_128 < 200;
+    if (dual) return small ? launch_rows_mfma_as<true, 64>(prm, stream) : launch_rows_mfma_as<true, 128>(prm, stream);
+    return small ? launch_rows_mfma_as<false, 64>(prm, stream) : launch_rows_mfma_as<false, 128>(prm, stream);
 }
 
 }  // namespace qm
