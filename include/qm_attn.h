@@ -462,6 +462,55 @@ int32_t qm_predictor_frame_steps(
     void* workspace, int64_t workspace_bytes, uint32_t* status_dev, void* hip_stream);
 
 /*
+ * Everything between two attentions of the talker's decode step in one launch: the four launches
+ * launch_linear_m1 (o_proj, R17:17203-17210), launch_add_postnorm_m1 + launch_gate_up_swiglu_m1 (R17:17215-17229),
+ * launch_linear_m1 (down_proj + residual, R17:17236-17244) of a layer and launch_rmsnorm + launch_qkv_m1
+ * (R17:17163-17176) of the next one, i.e. qm_linear_m1, qm_add_postnorm_gate_up_swiglu_m1, qm_linear_m1 and
+ * qm_rmsnorm_qkv_m1 of this library, with bit-identical outputs: hidden_out = the layer's output, q_out / k_out /
+ * v_out = the next layer's raw projections (what qm_decode_step_fused takes).  After the last layer the next_* and
+ * *_out pointers are all NULL and the launch ends with hidden_out.  Biases may be NULL.  The talker's geometry only
+ * (hidden 2048, q 2048, kv 1024, intermediate 6144; anything else: QM_ERR_GEOMETRY, take the operators one by one);
+ * weight matrices 16-byte aligned.  256 blocks stay resident and stream the weights through LDS while they hand the
+ * activations to each other through `workspace` (qm_talker_post_attention_workspace_bytes bytes, 256-byte aligned,
+ * set up once with qm_talker_post_attention_workspace_init; launches that share a workspace must not overlap).
+ * QM_ERR_NO_DEVICE if the device cannot hold 256 blocks at once.  Waits are bounded
+ * (QM_OPT_PREDICTOR_FRAME_SPIN_LIMIT applies here too): a launch that gives up ORs QM_STATUS_FRAME_TIMEOUT into
+ * *status_dev, every block returns, outputs are undefined and the workspace must be initialised again.
+ */
+typedef struct qm_talker_post_attention {
+    const uint16_t* context;          /* [q_columns] the layer's attention output */
+    const uint16_t* hidden;           /* [hidden_columns] the layer's input */
+    const uint16_t* o_weight;         /* [hidden_columns][q_columns] */
+    const uint16_t* o_bias;           /* [hidden_columns] or NULL */
+    const uint16_t* post_norm;        /* [hidden_columns] */
+    const uint16_t* gate_weight;      /* [intermediate_columns][hidden_columns] */
+    const uint16_t* up_weight;
+    const uint16_t* down_weight;      /* [hidden_columns][intermediate_columns] */
+    uint16_t* hidden_out;             /* [hidden_columns] */
+    const uint16_t* next_input_norm;  /* [hidden_columns] */
+    const uint16_t* next_q_weight;    /* [q_columns][hidden_columns] */
+    const uint16_t* next_q_bias;
+    const uint16_t* next_k_weight;    /* [kv_columns][hidden_columns] */
+    const uint16_t* next_k_bias;
+    const uint16_t* next_v_weight;
+    const uint16_t* next_v_bias;
+    uint16_t* q_out;                  /* [q_columns] */
+    uint16_t* k_out;                  /* [kv_columns] */
+    uint16_t* v_out;
+    int32_t hidden_columns;
+    int32_t q_columns;
+    int32_t kv_columns;
+    int32_t intermediate_columns;
+    float epsilon;
+} qm_talker_post_attention;
+
+int64_t qm_talker_post_attention_workspace_bytes(void);
+int32_t qm_talker_post_attention_workspace_init(void* workspace, int64_t workspace_bytes, void* hip_stream);
+int32_t qm_talker_post_attention_m1(
+    const qm_talker_post_attention* op,
+    void* workspace, int64_t workspace_bytes, uint32_t* status_dev, void* hip_stream);
+
+/*
  * The three layout operators in front of the staged attention at the predictor's step 0 (call site
  * R17:13663-13699), each with the reference wrapper's per-tensor argument list:
  * qm_predictor_transpose replaces PersistentPredictor::transpose (R17:13222-13236, kernel

@@ -50,6 +50,16 @@ class PredictorFrame(C.Structure):
     ]
 
 
+class TalkerPostAttention(C.Structure):
+    """Mirror of qm_talker_post_attention (include/qm_attn.h)."""
+    _fields_ = [(name, C.c_void_p) for name in (
+        "context", "hidden", "o_weight", "o_bias", "post_norm", "gate_weight", "up_weight", "down_weight", "hidden_out",
+        "next_input_norm", "next_q_weight", "next_q_bias", "next_k_weight", "next_k_bias", "next_v_weight", "next_v_bias",
+        "q_out", "k_out", "v_out")] + [
+        ("hidden_columns", C.c_int32), ("q_columns", C.c_int32), ("kv_columns", C.c_int32),
+        ("intermediate_columns", C.c_int32), ("epsilon", C.c_float)]
+
+
 def lib_path():
     return _LIB_PATH
 
@@ -92,6 +102,9 @@ _SIGNATURES = {
     "qm_predictor_frame_workspace_bytes": (C.c_int64, []),
     "qm_predictor_frame_workspace_init": (_I32, [_PTR, C.c_int64, _PTR]),
     "qm_predictor_frame_steps": (_I32, [C.POINTER(PredictorFrame), _I32, _I32, _I32, _F32, _PTR, C.c_int64, _PTR, _PTR]),
+    "qm_talker_post_attention_workspace_bytes": (C.c_int64, []),
+    "qm_talker_post_attention_workspace_init": (_I32, [_PTR, C.c_int64, _PTR]),
+    "qm_talker_post_attention_m1": (_I32, [C.POINTER(TalkerPostAttention), _PTR, C.c_int64, _PTR, _PTR]),
     "qm_predictor_transpose": (_I32, [_PTR, _PTR, _I32, _I32, _PTR]),
     "qm_predictor_rope_bhsd": (_I32, [_PTR] * 4 + [_I32, _I32, _PTR]),
     "qm_predictor_update_cache": (_I32, [_PTR, _PTR, _I32, _I32, _PTR]),
@@ -432,6 +445,33 @@ def predictor_frame_workspace_init(workspace, workspace_bytes, stream=0):
 def predictor_frame_steps(frame, first_step, last_step, top_k, temperature, workspace, workspace_bytes, status=None, stream=0):
     _check(lib().qm_predictor_frame_steps(C.byref(frame), first_step, last_step, top_k, temperature, _addr(workspace),
                                           workspace_bytes, _addr(status), stream), "qm_predictor_frame_steps")
+
+
+def talker_post_attention(hidden_columns=2048, q_columns=2048, kv_columns=1024, intermediate_columns=6144, epsilon=1e-6,
+                          **tensors):
+    """qm_talker_post_attention from tensors named like its fields (absent ones stay NULL).  The tensors must outlive
+    the descriptor."""
+    op = TalkerPostAttention()
+    for name, tensor in tensors.items():
+        setattr(op, name, _addr(tensor))
+    op.hidden_columns, op.q_columns, op.kv_columns, op.intermediate_columns = (hidden_columns, q_columns, kv_columns,
+                                                                               intermediate_columns)
+    op.epsilon = epsilon
+    return op
+
+
+def talker_post_attention_workspace_bytes():
+    return lib().qm_talker_post_attention_workspace_bytes()
+
+
+def talker_post_attention_workspace_init(workspace, workspace_bytes, stream=0):
+    _check(lib().qm_talker_post_attention_workspace_init(_addr(workspace), workspace_bytes, stream),
+           "qm_talker_post_attention_workspace_init")
+
+
+def talker_post_attention_m1(op, workspace, workspace_bytes, status=None, stream=0):
+    _check(lib().qm_talker_post_attention_m1(C.byref(op), _addr(workspace), workspace_bytes, _addr(status), stream),
+           "qm_talker_post_attention_m1")
 
 
 def predictor_transpose(x, out, rows, heads, stream=0):

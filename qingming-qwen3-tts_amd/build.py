@@ -15,7 +15,7 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libqm_attn.so")
 ENGINE_LIB_PATH = os.path.join(LIB_DIR, "libqm_engine.so")
 
-SOURCES = ["qm_lib.hip", "qm_norm_rope.hip", "qm_decode.hip", "qm_prefill.hip", "qm_predictor.hip", "qm_predictor_layout.hip", "qm_predictor_mfma.hip", "qm_predictor_frame.hip", "qm_linear.hip", "qm_rmsnorm.hip", "qm_sampler.hip", "qm_linear_rows.hip", "qm_linear_rows_mfma.hip"]
+SOURCES = ["qm_lib.hip", "qm_norm_rope.hip", "qm_decode.hip", "qm_prefill.hip", "qm_predictor.hip", "qm_predictor_layout.hip", "qm_predictor_mfma.hip", "qm_predictor_frame.hip", "qm_talker_chain.hip", "qm_linear.hip", "qm_rmsnorm.hip", "qm_sampler.hip", "qm_linear_rows.hip", "qm_linear_rows_mfma.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",

@@ -1,0 +1,172 @@
+"""GPU parity of qm_talker_post_attention_m1: o_proj, residual + post-norm + gate/up/SwiGLU, down_proj + residual of a
+talker layer and the RMSNorm + Q/K/V of the next one in one launch.
+
+The launch must leave exactly what the four one-operator entry points leave (bit for bit); those are held against the
+oracle in test_gpu_linear.py.  Weights are random in the talker's real geometry (R17:7930-7948).
+"""
+import ctypes as C
+
+import pytest
+
+from qm_testlib import to_dev
+
+pytestmark = pytest.mark.gpu
+
+H, Q, KV, I = 2048, 2048, 1024, 6144
+
+
+class _Layer:
+    def __init__(self, oracle, qm, dev, seed, biases):
+        import torch
+        self.qm, self.dev = qm, dev
+        n = [seed]
+
+        def rnd(shape, std=1.0, mean=0.0):
+            n[0] += 1
+            return to_dev(oracle.normal_bf16(shape, n[0], mean, std, threads=16), dev)
+
+        self.context, self.hidden = rnd((Q,)), rnd((H,))
+        self.wo, self.post = rnd((H, Q), 0.02), rnd((H,), 0.1, 1.0)
+        self.wg, self.wu, self.wd = rnd((I, H), 0.03), rnd((I, H), 0.03), rnd((H, I), 0.02)
+        self.in_norm = rnd((H,), 0.1, 1.0)
+        self.wq, self.wk, self.wv = rnd((Q, H), 0.03), rnd((KV, H), 0.03), rnd((KV, H), 0.03)
+        self.bo = rnd((H,), 0.1) if biases else None
+        self.bq, self.bk, self.bv = (rnd((Q,), 0.1), rnd((KV,), 0.1), rnd((KV,), 0.1)) if biases else (None, None, None)
+        z = lambda n_: torch.full((n_,), 0x7fc0, dtype=torch.int16, device=dev)
+        self.attn, self.res, self.act = z(H), z(H), z(I)
+        self.want = dict(hidden=z(H), q=z(Q), k=z(KV), v=z(KV))
+        self.got = dict(hidden=z(H), q=z(Q), k=z(KV), v=z(KV))
+        self.ws_bytes = qm.talker_post_attention_workspace_bytes()
+        self.ws = torch.zeros(self.ws_bytes // 4, dtype=torch.int32, device=dev)
+        qm.talker_post_attention_workspace_init(self.ws, self.ws_bytes)
+        self.status = torch.zeros(1, dtype=torch.int32, device=dev)
+
+    def by_operators(self, with_next=True):
+        qm, w = self.qm, self.want
+        qm.linear_m1(self.context, self.wo, self.bo, None, self.attn, H, Q)
+        qm.add_postnorm_gate_up_swiglu_m1(self.hidden, self.attn, self.post, self.res, self.wg, self.wu, self.act, H, I)
+        qm.linear_m1(self.act, self.wd, None, self.res, w["hidden"], H, I)
+        if with_next:
+            qm.rmsnorm_qkv_m1(w["hidden"], self.in_norm, self.wq, self.bq, self.wk, self.bk, self.wv, self.bv, w["q"], w["k"], w["v"],
+                              H, Q, KV)
+
+    def descriptor(self, with_next=True):
+        g = self.got
+        names = dict(context=self.context, hidden=self.hidden, o_weight=self.wo, o_bias=self.bo, post_norm=self.post,
+                     gate_weight=self.wg, up_weight=self.wu, down_weight=self.wd, hidden_out=g["hidden"])
+        if with_next:
+            names.update(next_input_norm=self.in_norm, next_q_weight=self.wq, next_q_bias=self.bq, next_k_weight=self.wk,
+                         next_k_bias=self.bk, next_v_weight=self.wv, next_v_bias=self.bv, q_out=g["q"], k_out=g["k"], v_out=g["v"])
+        return self.qm.talker_post_attention(**{k: v for k, v in names.items() if v is not None})
+
+    def one_launch(self, with_next=True, stream=0):
+        self.qm.talker_post_attention_m1(self.descriptor(with_next), self.ws, self.ws_bytes, self.status, stream)
+
+    def same(self, names=("hidden", "q", "k", "v")):
+        import torch
+        torch.cuda.synchronize()
+        return all(torch.equal(self.got[name], self.want[name]) for name in names)
+
+
+@pytest.fixture(scope="module", params=[False, True], ids=["no_bias", "biases"])
+def layer(request, oracle, qm, dev):
+    return _Layer(oracle, qm, dev, 7300 + 50 * int(request.param), request.param)
+
+
+def test_one_launch_equals_the_four_operators(layer):
+    import torch
+    layer.by_operators()
+    for _ in range(3):                                     # a later launch finds the workspace as the one before left it
+        for t in layer.got.values():
+            t.fill_(0x7fc0)
+        layer.one_launch()
+        assert layer.same() and int(layer.status.item()) == 0
+    # other inputs, same workspace
+    layer.context.copy_(torch.roll(layer.context, 3))
+    layer.hidden.copy_(torch.roll(layer.hidden, 5))
+    layer.by_operators()
+    layer.one_launch()
+    assert layer.same() and int(layer.status.item()) == 0
+
+
+def test_after_the_last_layer_there_is_no_next(layer):
+    layer.by_operators(with_next=False)
+    for name in ("q", "k", "v"):
+        layer.got[name].fill_(0x1234)
+    layer.one_launch(with_next=False)
+    assert layer.same(("hidden",)) and int(layer.status.item()) == 0
+    assert all(bool((layer.got[name] == 0x1234).all()) for name in ("q", "k", "v"))
+    layer.by_operators()
+    layer.one_launch()
+    assert layer.same()
+
+
+def test_replayed_from_a_graph(layer):
+    import torch
+    layer.by_operators()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=side):
+        layer.one_launch(stream=torch.cuda.current_stream().cuda_stream)
+    for _ in range(3):
+        for t in layer.got.values():
+            t.fill_(0x7fc0)
+        torch.cuda.synchronize()
+        graph.replay()
+        assert layer.same() and int(layer.status.item()) == 0
+    layer.one_launch()                                     # an eager launch after the replays
+    assert layer.same()
+
+
+def test_giving_up_and_argument_errors(layer, qm):
+    import torch
+    layer.by_operators()
+    # a workspace whose abort word is set (a launch gave up before): nothing runs, the status says so
+    for t in layer.got.values():
+        t.fill_(0x7fc0)
+    layer.ws[1] = 1
+    layer.one_launch()
+    torch.cuda.synchronize()
+    assert int(layer.status.item()) == qm.STATUS_FRAME_TIMEOUT
+    assert all(bool((t == 0x7fc0).all()) for t in layer.got.values())
+    layer.status.zero_()
+    qm.talker_post_attention_workspace_init(layer.ws, layer.ws_bytes)
+    layer.one_launch()
+    assert layer.same() and int(layer.status.item()) == 0
+    # waits cut to one attempt: the launch gives up, every block returns, the status says so
+    qm.set_option(qm.OPT_PREDICTOR_FRAME_SPIN_LIMIT, 1)
+    try:
+        layer.one_launch()
+        torch.cuda.synchronize()
+    finally:
+        qm.set_option(qm.OPT_PREDICTOR_FRAME_SPIN_LIMIT, 0)
+    assert int(layer.status.item()) == qm.STATUS_FRAME_TIMEOUT
+    layer.status.zero_()
+    qm.talker_post_attention_workspace_init(layer.ws, layer.ws_bytes)
+    layer.one_launch()
+    assert layer.same() and int(layer.status.item()) == 0
+    # arguments
+    L = qm.lib()
+    op = layer.descriptor()
+    p = layer.ws.data_ptr()
+    call = lambda ws, nbytes: L.qm_talker_post_attention_m1(C.byref(op), ws, nbytes, None, None)
+    assert call(None, layer.ws_bytes) == -1 and call(p, layer.ws_bytes - 256) == -4 and call(p + 64, layer.ws_bytes) == -2
+    op.hidden_columns = 1024
+    assert call(p, layer.ws_bytes) == -2
+    op.hidden_columns = 2048
+    saved = op.post_norm
+    op.post_norm = None
+    assert call(p, layer.ws_bytes) == -1
+    op.post_norm = saved
+    saved = op.next_k_weight
+    op.next_k_weight = None
+    assert call(p, layer.ws_bytes) == -1
+    op.next_k_weight = saved + 2
+    assert call(p, layer.ws_bytes) == -2
+    op.next_k_weight = saved
+    assert call(p, layer.ws_bytes) == 0
+    torch.cuda.synchronize()
+    assert L.qm_talker_post_attention_workspace_init(None, layer.ws_bytes, None) == -1
+    assert L.qm_talker_post_attention_workspace_init(p, layer.ws_bytes - 1, None) == -4
