@@ -366,10 +366,11 @@ class TalkerLayerStep:
     # attention's 1e-2 budget surfaces as at most a couple of ulps there
     tolerance = 0.125
 
-    def __init__(self, qm, dev, layers=28, ctx=2048, seed=91, fused=True):
+    def __init__(self, qm, dev, layers=28, ctx=2048, seed=91, fused=True, chained=False):
         import torch
-        self.qm, self.layers, self.ctx, self.fused = qm, layers, ctx, fused
-        self.name = "talker_layer_decode_step_ctx%d_x%dlayers%s" % (ctx, layers, "" if fused else "_reference_launch_sequence")
+        self.qm, self.layers, self.ctx, self.fused, self.chained = qm, layers, ctx, fused, chained
+        self.name = "talker_layer_decode_step_ctx%d_x%dlayers%s" % (
+            ctx, layers, "_one_launch_between_attentions" if chained else "" if fused else "_reference_launch_sequence")
         self.copies = layers
         syn = Synthetic(dev, seed)
         H, I = 2048, 6144
@@ -401,13 +402,38 @@ class TalkerLayerStep:
         self.bytes = weights + 2 * 8 * ctx * 128 * 2 + 4096 + 2 * (6 * H + 2 * I)   # + KV + append + activations
         self.flops = weights + 16 * ctx * 128 * 2 * 2
         self.i = 0
+        if chained:
+            # o_proj ... down_proj of a layer and the Q/K/V of the layer after it are one launch
+            # (qm_talker_post_attention_m1): a step is the attention of layer i and that launch
+            self.chain_ws_bytes = qm.talker_post_attention_workspace_bytes()
+            self.chain_ws = torch.zeros(self.chain_ws_bytes // 4, dtype=torch.int32, device=dev)
+            qm.talker_post_attention_workspace_init(self.chain_ws, self.chain_ws_bytes)
+            self.status = torch.zeros(1, dtype=torch.int32, device=dev)
+            self.ops = []
+            for i, L in enumerate(self.w):
+                N = self.w[(i + 1) % layers]
+                self.ops.append(qm.talker_post_attention(
+                    context=self.ctxv, hidden=self.x, o_weight=L["wo"], post_norm=L["post"], gate_weight=L["wg"], up_weight=L["wu"],
+                    down_weight=L["wd"], hidden_out=self.out, next_input_norm=N["in_norm"], next_q_weight=N["wq"],
+                    next_k_weight=N["wk"], next_v_weight=N["wv"], q_out=self.q, k_out=self.k_, v_out=self.v_))
+            self.primed = False
 
     def step(self):
         import torch
         s = torch.cuda.current_stream().cuda_stream
         L = self.w[self.i % self.layers]
-        self.i += 1
         qm, H, I = self.qm, self.H, self.I
+        if self.chained:
+            if not self.primed:       # the first layer's Q/K/V (later ones come out of the launch before)
+                qm.rmsnorm_qkv_m1(self.x, L["in_norm"], L["wq"], None, L["wk"], None, L["wv"], None, self.q, self.k_,
+                                  self.v_, H, H, 1024, 1e-6, s)
+                self.primed = True
+            qm.decode_step_fused(self.q, self.k_, self.v_, L["gq"], L["gk"], self.cos, self.sin, self.qrot, L["cache"],
+                                 None, 1, self.ctxv, 16, self.ctx - 1, -1, SCALE, 1e-6, self.ws, self.ws_bytes, None, s)
+            qm.talker_post_attention_m1(self.ops[self.i % self.layers], self.chain_ws, self.chain_ws_bytes, self.status, s)
+            self.i += 1
+            return
+        self.i += 1
         if self.fused:
             qm.rmsnorm_qkv_m1(self.x, L["in_norm"], L["wq"], None, L["wk"], None, L["wv"], None, self.q, self.k_,
                               self.v_, H, H, 1024, 1e-6, s)
@@ -435,8 +461,11 @@ class TalkerLayerStep:
         """One layer on the host; the comparison is on that layer's output hidden state."""
         import torch
         self.i = 0
+        self.primed = False
         self.step()
         torch.cuda.synchronize()
+        if self.chained:
+            assert int(self.status.item()) == 0
         L = {k: (_bits(v).copy() if hasattr(v, "detach") else v) for k, v in self.w[0].items()}
         H, I = self.H, self.I
         x = _bits(self.x).copy()
@@ -839,7 +868,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
     ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "prefillfp32", "predictor", "predictorexact",
-                                      "qkv", "layer", "frame", "frame1", "linears", "linearsexact"], default=None,
+                                      "qkv", "layer", "layer1", "frame", "frame1", "linears", "linearsexact"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -877,7 +906,7 @@ def main():
                 "prefillfp32": lambda: Prefill(qm, dev, score_rounding=0),
                 "predictor": lambda: PredictorLoop(qm, dev),
                 "predictorexact": lambda: PredictorLoop(qm, dev, kernel=1),
-                "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev),
+                "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev), "layer1": lambda: TalkerLayerStep(qm, dev, chained=True),
                 "frame": lambda: PredictorFrameSteps(qm, dev),
                 "frame1": lambda: PredictorFrameSteps(qm, dev, one_launch=True),
                 "linears": lambda: PromptLinears(qm, dev), "linearsexact": lambda: PromptLinears(qm, dev, kernel=1)}[args.only]
@@ -923,6 +952,7 @@ def main():
             # the whole decode step of one talker layer, 28 layers' weights and caches in rotation (2.8 GB)
             ("next_talker_layer_decode_step", lambda: TalkerLayerStep(qm, dev)),
             ("next_talker_layer_decode_step_unfused", lambda: TalkerLayerStep(qm, dev, fused=False)),
+            ("next_talker_layer_decode_step_one_launch", lambda: TalkerLayerStep(qm, dev, chained=True)),
             # the seven linears of a talker layer over a 1024-token prompt: matrix cores, and the exact chain
             ("next_prompt_linears_1024_tokens", lambda: PromptLinears(qm, dev)),
             ("next_prompt_linears_1024_tokens_exact_chain", lambda: PromptLinears(qm, dev, kernel=1)),

@@ -108,7 +108,10 @@ const char* qm_target_arch(void);
  *   QM_OPT_LINEAR_ROWS_KERNEL  0 (default): qm_linear_rows / qm_gate_up_swiglu_rows take the sums of calls with 16 or more
  *       token rows on the matrix cores where the shape fits their tiles (output columns % 128 == 0, reduction % 128 == 0):
  *       same roundings after the sum, results within the operators' tolerance of the exact chain; 1: every call in the
- *       reference's summation order (bit-identical to the M = 1 operators; 20 to 60 times slower on long prompts). */
+ *       reference's summation order (bit-identical to the M = 1 operators; 20 to 60 times slower on long prompts).
+ *   QM_OPT_TALKER_LAYER_OPERATORS  0 (default): the engine's talker decode step (qm_engine.h) runs what lies between two
+ *       attentions as one launch of qm_talker_post_attention_m1 where the checkpoint has the geometry it serves; 1: operator
+ *       by operator.  Same bits either way. */
 enum {
     QM_OPT_PREFILL_SCORE_ROUNDING = 0,
     QM_OPT_DECODE_TILES_PER_BLOCK = 1,
@@ -118,7 +121,8 @@ enum {
     QM_OPT_PREDICTOR_FRAME_OPERATORS = 5,
     QM_OPT_PREDICTOR_FRAME_SPIN_LIMIT = 6,
     QM_OPT_LINEAR_ROWS_KERNEL = 7,
-    QM_OPT_COUNT = 8
+    QM_OPT_TALKER_LAYER_OPERATORS = 8,
+    QM_OPT_COUNT = 9
 };
 /* Returns QM_ERR_ARGUMENT for an unknown option or a negative value. */
 int32_t qm_set_option(int32_t option, int32_t value);

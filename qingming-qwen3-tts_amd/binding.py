@@ -175,6 +175,7 @@ OPT_PREDICTOR_LOOP_KERNEL = 4
 OPT_PREDICTOR_FRAME_OPERATORS = 5
 OPT_PREDICTOR_FRAME_SPIN_LIMIT = 6
 OPT_LINEAR_ROWS_KERNEL = 7
+OPT_TALKER_LAYER_OPERATORS = 8
 
 
 def set_option(option, value):

@@ -51,6 +51,9 @@ struct qm_talker {
     qm_engine::DeviceBuffer p_split;
     // device status word the attention kernels OR their QM_STATUS_* bits into; read at qm_talker_synchronize
     qm_engine::DeviceBuffer status;
+    // hand-off words of qm_talker_post_attention_m1 (checkpoints of the geometry it serves)
+    qm_engine::DeviceBuffer chain_workspace;
+    bool chain_geometry = false;
 
     ~qm_talker() {
         if (own_stream && stream) (void)hipStreamDestroy(stream);
@@ -157,6 +160,12 @@ static std::unique_ptr<qm_talker> create_talker(const std::string& model_dir, in
     engine->workspace = DeviceBuffer(qm_decode_workspace_bytes(1, engine->q_heads, engine->kv_heads, max_cache));
     engine->status = DeviceBuffer(256);
     hip_check(hipMemsetAsync(engine->status.raw(), 0, engine->status.bytes(), engine->stream), "status word reset");
+    engine->chain_geometry = engine->q_dim == 2048 && engine->kv_dim == 1024 && engine->intermediate == 6144 && kHidden == 2048;
+    if (engine->chain_geometry) {
+        engine->chain_workspace = DeviceBuffer(static_cast<size_t>(qm_talker_post_attention_workspace_bytes()));
+        op_check(qm_talker_post_attention_workspace_init(engine->chain_workspace.raw(), static_cast<int64_t>(engine->chain_workspace.bytes()),
+                                                         engine->stream), "talker hand-off workspace init");
+    }
     hip_check(hipStreamSynchronize(upload), "weight upload synchronize");   // the mapped files go away with `host`
     return engine;
 }
@@ -196,19 +205,48 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
     hip_check(hipMemcpyAsync(e.sine.raw(), sine, kHeadDim * 2, hipMemcpyHostToDevice, s), "decode sine");
     DeviceBuffer* current = &e.hidden_a;
     DeviceBuffer* next = &e.hidden_b;
-    for (Layer& w : e.layers) {
+    // What lies between two attentions — o_proj, residual + post-norm + gate/up/SwiGLU, down_proj + residual and the next
+    // layer's RMSNorm + Q/K/V — is one launch where the checkpoint has the geometry that launch serves (same bits).
+    int32_t by_operators = 0;
+    op_check(qm_get_option(QM_OPT_TALKER_LAYER_OPERATORS, &by_operators), "talker layer option");
+    const bool chained = e.chain_geometry && by_operators == 0;
+    for (size_t index = 0; index < e.layers.size(); ++index) {
+        Layer& w = e.layers[index];
         qm_kv_cache cache = flat_cache_of(e, w);
         // launch_rmsnorm + launch_qkv_m1 (R17:17163-17176)
-        op_check(qm_rmsnorm_qkv_m1(current->u16(), w.input_norm.data(), kEpsilon, w.q_weight.data(), w.q_bias.data(),
-                                   w.k_weight.data(), w.k_bias.data(), w.v_weight.data(), w.v_bias.data(), e.q.u16(),
-                                   e.k.u16(), e.v.u16(), kHidden, e.q_dim, e.kv_dim, s),
-                 "talker RMSNorm + Q/K/V");
+        if (!chained || index == 0)
+            op_check(qm_rmsnorm_qkv_m1(current->u16(), w.input_norm.data(), kEpsilon, w.q_weight.data(), w.q_bias.data(),
+                                       w.k_weight.data(), w.k_bias.data(), w.v_weight.data(), w.v_bias.data(), e.q.u16(),
+                                       e.k.u16(), e.v.u16(), kHidden, e.q_dim, e.kv_dim, s),
+                     "talker RMSNorm + Q/K/V");
         // launch_qk_norm_rope_cache_m1 + launch_attention (R17:17181-17195)
         op_check(qm_decode_step_fused(e.q.u16(), e.k.u16(), e.v.u16(), w.q_norm.data(), w.k_norm.data(), e.cosine.u16(),
                                       e.sine.u16(), e.q_rotated.u16(), &cache, nullptr, 1, e.context.u16(), e.q_heads,
                                       position, -1, kScale, kEpsilon, e.workspace.raw(), e.workspace.bytes(),
                                       static_cast<uint32_t*>(e.status.raw()), s),
                  "talker norm/RoPE/append + attention");
+        if (chained) {
+            qm_talker_post_attention op = {};
+            op.context = e.context.u16(); op.hidden = current->u16();
+            op.o_weight = w.o_weight.data(); op.o_bias = w.o_bias.data(); op.post_norm = w.post_norm.data();
+            op.gate_weight = w.gate_weight.data(); op.up_weight = w.up_weight.data(); op.down_weight = w.down_weight.data();
+            op.hidden_out = next->u16();
+            if (index + 1 < e.layers.size()) {
+                Layer& after = e.layers[index + 1];
+                op.next_input_norm = after.input_norm.data();
+                op.next_q_weight = after.q_weight.data(); op.next_q_bias = after.q_bias.data();
+                op.next_k_weight = after.k_weight.data(); op.next_k_bias = after.k_bias.data();
+                op.next_v_weight = after.v_weight.data(); op.next_v_bias = after.v_bias.data();
+                op.q_out = e.q.u16(); op.k_out = e.k.u16(); op.v_out = e.v.u16();
+            }
+            op.hidden_columns = kHidden; op.q_columns = e.q_dim; op.kv_columns = e.kv_dim; op.intermediate_columns = e.intermediate;
+            op.epsilon = kEpsilon;
+            op_check(qm_talker_post_attention_m1(&op, e.chain_workspace.raw(), static_cast<int64_t>(e.chain_workspace.bytes()),
+                                                 static_cast<uint32_t*>(e.status.raw()), s),
+                     "talker o_proj ... next Q/K/V");
+            std::swap(current, next);
+            continue;
+        }
         // launch_linear_m1: o_proj (R17:17203-17210)
         op_check(qm_linear_m1(e.context.u16(), w.o_weight.data(), w.o_bias.data(), nullptr, e.attention.u16(), kHidden,
                               e.q_dim, s),
@@ -436,6 +474,10 @@ extern "C" int32_t qm_talker_synchronize(qm_talker* engine) {
             if ((bits & QM_STATUS_SPLIT_TIMEOUT) && engine->p_split.raw())
                 op_check(qm_prefill_split_workspace_init(engine->p_split.raw(), static_cast<int64_t>(engine->p_split.bytes()),
                                                          engine->stream), "prefill key-split workspace init");
+            if ((bits & QM_STATUS_FRAME_TIMEOUT) && engine->chain_workspace.raw())
+                op_check(qm_talker_post_attention_workspace_init(engine->chain_workspace.raw(),
+                                                                 static_cast<int64_t>(engine->chain_workspace.bytes()), engine->stream),
+                         "talker hand-off workspace init");
             throw ApiError(QM_ERR_STATUS, "talker kernels reported status bits " + std::to_string(bits));
         }
     });

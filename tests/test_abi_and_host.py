@@ -95,7 +95,7 @@ def test_options_round_trip_and_validation(qm):
     assert qm.get_option(qm.OPT_PREFILL_KERNEL) == 0 and qm.get_option(qm.OPT_DECODE_STREAMING_LOADS) == 0
     lib = qm.lib()
     assert lib.qm_set_option(99, 1) == -5 and lib.qm_set_option(-1, 1) == -5
-    assert lib.qm_set_option(qm.OPT_LINEAR_ROWS_KERNEL + 1, 1) == -5      # one past the last option
+    assert lib.qm_set_option(qm.OPT_TALKER_LAYER_OPERATORS + 1, 1) == -5      # one past the last option
     assert qm.get_option(qm.OPT_PREDICTOR_FRAME_OPERATORS) == 0 and qm.get_option(qm.OPT_PREDICTOR_FRAME_SPIN_LIMIT) == 0
     assert lib.qm_set_option(qm.OPT_DECODE_TILES_PER_BLOCK, -3) == -5
     assert lib.qm_get_option(qm.OPT_DECODE_TILES_PER_BLOCK, None) == -1

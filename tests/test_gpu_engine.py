@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 H, Q, KV, I, LAYERS, MAX_CACHE, PREFILL = 2048, 2048, 1024, 512, 3, 48, 21
 
 
-def _checkpoint(directory, with_bias):
+def _checkpoint(directory, with_bias, inter=I, layers=LAYERS):
     import torch
     from safetensors.torch import save_file
     g = torch.Generator().manual_seed(17 + with_bias)
@@ -24,15 +24,15 @@ def _checkpoint(directory, with_bias):
         return (torch.randn(shape, generator=g) * std + mean).to(torch.bfloat16)
 
     tensors = {"talker.model.norm.weight": rnd((H,), 0.1, 1.0), "talker.model.codec_embedding.weight": rnd((8, 16))}
-    for i in range(LAYERS):
+    for i in range(layers):
         p = f"talker.model.layers.{i}."
         tensors.update({
             p + "input_layernorm.weight": rnd((H,), 0.1, 1.0), p + "post_attention_layernorm.weight": rnd((H,), 0.1, 1.0),
             p + "self_attn.q_proj.weight": rnd((Q, H), 0.02), p + "self_attn.k_proj.weight": rnd((KV, H), 0.02),
             p + "self_attn.v_proj.weight": rnd((KV, H), 0.02), p + "self_attn.o_proj.weight": rnd((H, Q), 0.02),
             p + "self_attn.q_norm.weight": rnd((128,), 0.1, 1.0), p + "self_attn.k_norm.weight": rnd((128,), 0.1, 1.0),
-            p + "mlp.gate_proj.weight": rnd((I, H), 0.03), p + "mlp.up_proj.weight": rnd((I, H), 0.03),
-            p + "mlp.down_proj.weight": rnd((H, I), 0.03),
+            p + "mlp.gate_proj.weight": rnd((inter, H), 0.03), p + "mlp.up_proj.weight": rnd((inter, H), 0.03),
+            p + "mlp.down_proj.weight": rnd((H, inter), 0.03),
         })
         if with_bias:
             tensors.update({p + "self_attn.q_proj.bias": rnd((Q,), 0.1), p + "self_attn.k_proj.bias": rnd((KV,), 0.1),
@@ -130,6 +130,55 @@ def test_engine_decode_steps_match_the_oracle_chain(engine, oracle, qm, dev, tmp
         talker.decode(xd, cos[0], sin[0], MAX_CACHE - PREFILL)
     assert err.value.code == -3
     talker.close()
+
+
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_engine_decode_in_the_talkers_geometry_takes_one_launch_between_attentions(engine, qm, dev, tmp_path, with_bias):
+    """With the talker's real intermediate size (6144) the decode step runs qm_talker_post_attention_m1 between two
+    attentions; the final hidden vectors and the caches equal, bit for bit, what the operator-by-operator step (held
+    against the oracle above) leaves."""
+    import ctypes as C
+    import torch
+    layers = 3
+    _checkpoint(str(tmp_path), with_bias, inter=6144, layers=layers)
+    hip = C.CDLL("libamdhip64.so")
+    results = []
+    for by_operators in (1, 0):
+        qm.set_option(qm.OPT_TALKER_LAYER_OPERATORS, by_operators)
+        try:
+            talker = engine.Talker(str(tmp_path), MAX_CACHE)
+            assert talker.intermediate == 6144
+            talker.reset(PREFILL)
+            talker.synchronize()
+            g = torch.Generator().manual_seed(5)
+            for layer in range(layers):
+                ka, va = talker.cache_addresses(layer)
+                for address in (ka, va):
+                    rows = torch.zeros((8, MAX_CACHE, 128), dtype=torch.bfloat16)
+                    rows[:, :PREFILL] = torch.randn((8, PREFILL, 128), generator=g).to(torch.bfloat16)
+                    rows = rows.view(torch.int16).numpy()
+                    assert hip.hipMemcpy(C.c_void_p(address), rows.ctypes.data_as(C.c_void_p), C.c_size_t(rows.nbytes), 1) == 0
+            outputs = []
+            for step in range(3):
+                x = (torch.randn(H, generator=g)).to(torch.bfloat16).view(torch.int16).to(dev)
+                cos, sin = engine.rope_rows(1, PREFILL + step)
+                address = talker.decode(x, cos[0], sin[0], step)
+                talker.synchronize()
+                out = torch.empty(H, dtype=torch.int16, device=dev)
+                assert hip.hipMemcpy(C.c_void_p(out.data_ptr()), C.c_void_p(address), C.c_size_t(H * 2), 3) == 0
+                outputs.append(out.cpu())
+            for layer in range(layers):
+                for address in talker.cache_addresses(layer):
+                    rows = np.zeros((8, MAX_CACHE, 128), dtype=np.uint16)
+                    assert hip.hipMemcpy(rows.ctypes.data_as(C.c_void_p), C.c_void_p(address), C.c_size_t(rows.nbytes), 2) == 0
+                    outputs.append(torch.from_numpy(rows.view(np.int16)))
+            talker.close()
+            results.append(outputs)
+        finally:
+            qm.set_option(qm.OPT_TALKER_LAYER_OPERATORS, 0)
+    assert len(results[0]) == len(results[1]) == 3 + 2 * layers
+    assert all(torch.equal(a, b) for a, b in zip(*results))
+    assert len({bytes(o.numpy().tobytes()) for o in results[0][:3]}) == 3          # (three different steps)
 
 
 def test_engine_rejects_a_checkpoint_with_the_wrong_geometry(engine, dev, tmp_path):
