@@ -64,10 +64,8 @@ constexpr int kTkSlotBytes = 16 * kTkDualStride;
 static_assert(8 * kTkSingleStride <= kTkSlotBytes, "both kinds of unit fit a slot");
 constexpr int kTkSlots = 4;
 constexpr int kTkPieces = 32;                        // 1 KiB pieces per unit (one instruction of a wave each)
-#ifndef QM_TK_WINDOW
-#define QM_TK_WINDOW 12
-#endif
-constexpr int kTkWindow = QM_TK_WINDOW;              // pieces a weight wave has under way at most
+constexpr int kTkFirstHandoffGate = 3;                 // units requested before o_proj's outputs have been exchanged
+constexpr int kTkWindow = 10;                        // pieces a weight wave has under way at most: its share of a unit
 constexpr int kTkLdsX = 0;                           // the operator's input vector, fp32 (down_proj: 6144)
 constexpr int kTkLdsRing = kTkLdsX + kTkInter * 4;
 constexpr int kTkLdsBytes = kTkLdsRing + kTkSlots * kTkSlotBytes;
@@ -116,6 +114,7 @@ struct TkShared {
     __attribute__((aligned(16))) int landed[4];   // units whose pieces of weight wave 0, 1, 2 are in LDS; [3] unused
     __attribute__((aligned(16))) int done[4];     // units each compute wave has read into registers
     int abort;
+    int first_input_seen;       // the compute waves have o_proj's outputs of all blocks
     int arrivals;               // of compute waves at their barrier, counted on
     float groups[8];            // the eight 32-lane sums of a norm
     float residual[8];
@@ -258,6 +257,7 @@ __device__ __forceinline__ int request_unit(const TkParams& p, int v, int b, uns
     // (requests complete in the order they were made: all but the last kTkWindow have landed)
     return issued > kTkWindow ? issued - kTkWindow : 0;
 }
+static_assert(kTkWindow <= kTkPieces / kTkWeightWaves, "a unit is known to have landed when the next has been requested");
 
 __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -274,6 +274,7 @@ __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p)
         sh.landed[0] = sh.landed[1] = sh.landed[2] = sh.landed[3] = 0;
         sh.done[0] = sh.done[1] = sh.done[2] = sh.done[3] = 0;
         sh.arrivals = 0;
+        sh.first_input_seen = 0;
     }
     __syncthreads();
     if (sh.abort) {
@@ -293,6 +294,12 @@ __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p)
         bool alive = true;
 #pragma unroll 1
         for (int r = 0; alive && r < units; ++r) {
+            // While the first hand-off is under way only the first three units are requested: the polls for o_proj's
+            // outputs travel through the same queues as the requests that fill the ring and come back when those have
+            // (gate at unit 1 / 2 / 3 / none: 35.9 / 34.8 / 34.7 / 36.0 us per layer).
+            if (r == kTkFirstHandoffGate) {
+                while (lds_word(&sh.first_input_seen) == 0u && lds_word(&sh.abort) == 0u) __builtin_amdgcn_s_sleep(1);
+            }
             // the slot is free once unit r - kTkSlots has been read by all four compute waves
             if (r >= kTkSlots) {
                 for (;;) {
@@ -308,7 +315,11 @@ __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p)
                 }
                 if (!alive) break;
             }
-            const int landed = request_unit(p, r, b, ring + (r & (kTkSlots - 1)) * kTkSlotBytes, third, issued) / my_pieces;
+            int landed = request_unit(p, r, b, ring + (r & (kTkSlots - 1)) * kTkSlotBytes, third, issued) / my_pieces;
+            if (r == 0) {                                 // the first unit is waited for: say so as soon as it is there
+                wait_vm_at_most<0>();
+                landed = 1;
+            }
             if (landed > published) {
                 published = landed;
                 if (lane == 0) lds_store(&sh.landed[third], static_cast<uint32_t>(published));
@@ -435,6 +446,7 @@ __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p)
                 if (!with_add && qkv_bias && tid < 16) sh.bias[tid] = bf2f(qkv_bias[qkv_row + tid]);
                 alive = poll_words<kPerThread>(with_add ? attn : hidden_words, with_add ? tag(0) : tag(2), abort_word, spin_limit, raw);
                 if (!alive) give_up();
+                if (with_add && tid == 0) lds_store(&sh.first_input_seen, 1u);
                 float value[kPerThread];
 #pragma unroll
                 for (int i = 0; i < kPerThread; ++i) {
