@@ -79,8 +79,9 @@ const char* qm_error_string(int32_t code);
 /* Names the architecture the kernels were compiled for ("gfx950"). */
 const char* qm_target_arch(void);
 
-/* Process-wide tuning options; they have no counterpart in the reference, whose kernels have
- * one fixed behaviour.  A call reads the options when it is enqueued.
+/* Tuning options; they have no counterpart in the reference, whose kernels have one fixed behaviour.  A call
+ * reads the options when it is enqueued: the calling thread's own value where qm_set_thread_option has set one (two
+ * engines driven from two threads can differ), else the process-wide value of qm_set_option.
  *   QM_OPT_PREFILL_SCORE_ROUNDING  1 (default): qm_prefill_attention_causal rounds raw and scaled
  *       scores to bf16 like the reference (R17:15879-15890); 0: scores stay fp32 (faster; needs
  *       scale > 0; outputs stay within the 1e-2 tolerance of the fp32 definition).
@@ -126,6 +127,9 @@ enum {
 };
 /* Returns QM_ERR_ARGUMENT for an unknown option or a negative value. */
 int32_t qm_set_option(int32_t option, int32_t value);
+/* The same for calls enqueued by the calling thread only; value -1 removes the thread's own value. */
+int32_t qm_set_thread_option(int32_t option, int32_t value);
+/* What a call enqueued by the calling thread would read. */
 int32_t qm_get_option(int32_t option, int32_t* value);
 
 /* ---- (1) fused QK-RMSNorm + RoPE + KV append ------------------------------------- */

@@ -99,6 +99,7 @@ _SIGNATURES = {
     "qm_predictor_attention_loop": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _I32, _F32, _PTR]),
     "qm_predictor_attention_staged": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _PTR]),
     "qm_predictor_step_attention_m1": (_I32, [_PTR] * 10 + [_I32, _F32, _PTR]),
+    "qm_set_thread_option": (_I32, [_I32, _I32]),
     "qm_predictor_frame_workspace_bytes": (C.c_int64, []),
     "qm_predictor_frame_workspace_init": (_I32, [_PTR, C.c_int64, _PTR]),
     "qm_predictor_frame_steps": (_I32, [C.POINTER(PredictorFrame), _I32, _I32, _I32, _F32, _PTR, C.c_int64, _PTR, _PTR]),
@@ -180,6 +181,11 @@ OPT_TALKER_LAYER_OPERATORS = 8
 
 def set_option(option, value):
     _check(lib().qm_set_option(option, value), "qm_set_option")
+
+
+def set_thread_option(option, value):
+    """The option for calls made by this thread only; -1 removes the thread's own value."""
+    _check(lib().qm_set_thread_option(option, value), "qm_set_thread_option")
 
 
 def get_option(option):

@@ -38,19 +38,47 @@ std::atomic<int32_t> g_options[QM_OPT_COUNT] = {
     {0},   // QM_OPT_LINEAR_ROWS_KERNEL (0 = matrix cores for 16 or more token rows, 1 = always the exact chain)
     {0},   // QM_OPT_TALKER_LAYER_OPERATORS (0 = one launch between two attentions, 1 = operator by operator)
 };
+
+// a thread's own values: -1 = none, the process-wide value applies
+struct ThreadOptions {
+    int32_t value[QM_OPT_COUNT];
+    ThreadOptions() {
+        for (int32_t& v : value) v = -1;
+    }
+};
+thread_local ThreadOptions t_options;
+
+int32_t check_option(int32_t option, int32_t value) {
+    if (option < 0 || option >= QM_OPT_COUNT) return QM_ERR_ARGUMENT;
+    if (value < 0) return QM_ERR_ARGUMENT;
+    if (option == QM_OPT_DECODE_TILES_PER_BLOCK && value > 4096) return QM_ERR_ARGUMENT;
+    return QM_OK;
+}
 }  // namespace
 
 int32_t option_value(int32_t option) {
-    return g_options[option].load(std::memory_order_relaxed);
+    const int32_t own = t_options.value[option];
+    return own >= 0 ? own : g_options[option].load(std::memory_order_relaxed);
 }
 
 }  // namespace qm
 
 extern "C" int32_t qm_set_option(int32_t option, int32_t value) {
-    if (option < 0 || option >= QM_OPT_COUNT) return QM_ERR_ARGUMENT;
-    if (value < 0) return QM_ERR_ARGUMENT;
-    if (option == QM_OPT_DECODE_TILES_PER_BLOCK && value > 4096) return QM_ERR_ARGUMENT;
+    const int32_t rc = qm::check_option(option, value);
+    if (rc != QM_OK) return rc;
     qm::g_options[option].store(value, std::memory_order_relaxed);
+    return QM_OK;
+}
+
+extern "C" int32_t qm_set_thread_option(int32_t option, int32_t value) {
+    if (value == -1) {                                   // back to the process-wide value
+        if (option < 0 || option >= QM_OPT_COUNT) return QM_ERR_ARGUMENT;
+        qm::t_options.value[option] = -1;
+        return QM_OK;
+    }
+    const int32_t rc = qm::check_option(option, value);
+    if (rc != QM_OK) return rc;
+    qm::t_options.value[option] = value;
     return QM_OK;
 }
 

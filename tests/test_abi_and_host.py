@@ -109,6 +109,39 @@ def test_options_round_trip_and_validation(qm):
     assert qm.decode_workspace_bytes(64, 16, 8, 4096) == base
 
 
+def test_a_threads_own_option_value_is_seen_by_that_thread_only(qm):
+    import threading
+    lib = qm.lib()
+    assert lib.qm_set_thread_option(99, 1) == -5 and lib.qm_set_thread_option(qm.OPT_PREFILL_KERNEL, -2) == -5
+    assert lib.qm_set_thread_option(qm.OPT_DECODE_TILES_PER_BLOCK, 5000) == -5
+    base = qm.decode_workspace_bytes(64, 16, 8, 4096)
+    seen = {}
+
+    def other():
+        # this thread forces 4-tile blocks for its own calls
+        qm.set_thread_option(qm.OPT_DECODE_TILES_PER_BLOCK, 4)
+        seen["value"] = qm.get_option(qm.OPT_DECODE_TILES_PER_BLOCK)
+        seen["bytes"] = qm.decode_workspace_bytes(64, 16, 8, 4096)
+        qm.set_thread_option(qm.OPT_DECODE_TILES_PER_BLOCK, -1)
+        seen["after"] = qm.get_option(qm.OPT_DECODE_TILES_PER_BLOCK)
+
+    worker = threading.Thread(target=other)
+    worker.start()
+    worker.join()
+    assert seen["value"] == 4 and seen["bytes"] > base and seen["after"] == 0
+    assert qm.get_option(qm.OPT_DECODE_TILES_PER_BLOCK) == 0 and qm.decode_workspace_bytes(64, 16, 8, 4096) == base
+    # a thread's own value wins over the process-wide one, and goes away with -1
+    qm.set_option(qm.OPT_PREFILL_KERNEL, 1)
+    try:
+        qm.set_thread_option(qm.OPT_PREFILL_KERNEL, 0)
+        assert qm.get_option(qm.OPT_PREFILL_KERNEL) == 0
+        qm.set_thread_option(qm.OPT_PREFILL_KERNEL, -1)
+        assert qm.get_option(qm.OPT_PREFILL_KERNEL) == 1
+    finally:
+        qm.set_thread_option(qm.OPT_PREFILL_KERNEL, -1)
+        qm.set_option(qm.OPT_PREFILL_KERNEL, 0)
+
+
 def test_workspace_size_is_monotone_and_pure(qm):
     lib = qm.lib()
     prev = 0
