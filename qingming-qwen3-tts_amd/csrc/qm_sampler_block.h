@@ -102,8 +102,10 @@ struct SamplerScratch {
 // only, when a draw happens).  Returns the chosen id in thread 0 (anything in the others), or -2 in every
 // thread when prm.process_only stops after the processed scores.  Nothing is read from prm.logits or
 // prm.rng_state and nothing written to prm.output_id / prm.history / prm.rng_state: that is the caller's.
+// `sync` is the barrier of the kSmpThreads calling threads (the block's barrier where they are the whole block).
+template <class Sync>
 __device__ __forceinline__ int32_t sampler_block(const SamplerParams& prm, SamplerScratch& sh, const float (&score)[kSmpPerThread],
-                                                 unsigned long long& rng) {
+                                                 unsigned long long& rng, Sync&& sync) {
     uint32_t* const sh_seen = sh.seen;
     int* const sh_hist = sh.hist;
     int* const sh_wave_total = sh.wave_total;
@@ -127,12 +129,12 @@ __device__ __forceinline__ int32_t sampler_block(const SamplerParams& prm, Sampl
     // ---- which tokens were generated before (R17:14046-14052, as a bitmap) -----------------------------
     if (prm.process) {
         for (int i = tid; i < kSmpMaxVocab / 32; i += kSmpThreads) sh_seen[i] = 0;
-        __syncthreads();
+        sync();
         for (int i = tid; i < prm.history_count; i += kSmpThreads) {
             const int token = prm.history[i];
             if (token >= 0 && token < vocab) atomicOr(&sh_seen[token >> 5], 1U << (token & 31));
         }
-        __syncthreads();
+        sync();
     }
 
     // ---- the scores as keys: larger key = earlier in the order -------------------------------------------
@@ -170,12 +172,12 @@ __device__ __forceinline__ int32_t sampler_block(const SamplerParams& prm, Sampl
         const int shift = pass < 4 ? 56 - 8 * pass : (pass == 4 ? 4 : 0);       // 56, 48, 40, 32, 4, 0
         const int width = pass < 5 ? 8 : 4;
         const unsigned digit_mask = (1U << width) - 1U;
-        __syncthreads();                                   // the bins are clear (and, later, the last pass's results read)
+        sync();                                   // the bins are clear (and, later, the last pass's results read)
 #pragma unroll
         for (int j = 0; j < kSmpPerThread; ++j)
             if (key[j] != 0 && (key[j] & prefix_mask) == prefix)
                 atomicAdd(&sh_hist[(static_cast<unsigned>(key[j] >> shift) & digit_mask) * kSmpReplicas + (lane & (kSmpReplicas - 1))], 1);
-        __syncthreads();
+        sync();
         // keys in bins above this thread's bin: inside the wave from a prefix sum, then the waves above
         int own = 0;
 #pragma unroll
@@ -186,7 +188,7 @@ __device__ __forceinline__ int32_t sampler_block(const SamplerParams& prm, Sampl
         const int upto = wave_inclusive_scan(own, lane);
         const int wave_sum = __builtin_amdgcn_readlane(upto, 63);
         if (lane == 0) sh_wave_total[wave] = wave_sum;
-        __syncthreads();
+        sync();
         int above = wave_sum - upto;
         for (int w = wave + 1; w < 4; ++w) above += sh_wave_total[w];
         if (above < remaining && remaining <= above + own) {       // exactly one bin
@@ -194,7 +196,7 @@ __device__ __forceinline__ int32_t sampler_block(const SamplerParams& prm, Sampl
             sh_remaining = remaining - above;
             sh_done = remaining == above + own ? 1 : 0;
         }
-        __syncthreads();
+        sync();
         prefix |= static_cast<unsigned long long>(sh_digit) << shift;
         prefix_mask |= static_cast<unsigned long long>(digit_mask) << shift;
         remaining = sh_remaining;
@@ -211,15 +213,15 @@ __device__ __forceinline__ int32_t sampler_block(const SamplerParams& prm, Sampl
 #pragma unroll
         for (int j = 0; j < kSmpPerThread; ++j) mine += (key[j] != 0 && key[j] >= threshold) ? 1 : 0;
         const int upto = wave_inclusive_scan(mine, lane);
-        __syncthreads();                                   // (the select's last reads of sh_wave_total are done)
+        sync();                                   // (the select's last reads of sh_wave_total are done)
         if (lane == 63) sh_wave_total[wave] = upto;
-        __syncthreads();
+        sync();
         int at = upto - mine;
         for (int w = 0; w < wave; ++w) at += sh_wave_total[w];
 #pragma unroll
         for (int j = 0; j < kSmpPerThread; ++j)
             if (key[j] != 0 && key[j] >= threshold) sh_cand[at++] = key[j];
-        __syncthreads();
+        sync();
     }
     if (tid < keep) {
         const unsigned long long mine = sh_cand[tid];
@@ -227,7 +229,7 @@ __device__ __forceinline__ int32_t sampler_block(const SamplerParams& prm, Sampl
         for (int j = 0; j < keep; ++j) rank += sh_cand[j] > mine ? 1 : 0;
         sh_sorted[rank] = mine;
     }
-    __syncthreads();
+    sync();
 
     // ---- sample (R17:7431-7460) ----------------------------------------------------------------------------
     const double inv_t = 1.0 / static_cast<double>(prm.temperature);
@@ -238,7 +240,7 @@ __device__ __forceinline__ int32_t sampler_block(const SamplerParams& prm, Sampl
     } else if (tid < ((keep + 7) & ~7)) {
         sh_exp[tid] = 0.0;                                 // (padding of the last batch of eight below: x + 0 is x)
     }
-    __syncthreads();
+    sync();
     auto id_of = [&](int i) { return static_cast<int32_t>(0xffffffffU - static_cast<uint32_t>(sh_sorted[i])); };
     // The running sums, added by one thread in the reference's order (its second loop repeats
     // the partial sums of its first: one pass serves both); the terms come eight at a time, the next
@@ -276,20 +278,28 @@ __device__ __forceinline__ int32_t sampler_block(const SamplerParams& prm, Sampl
             sh_count = keep - 1;                           // the answer if no running sum exceeds the target
         }
     }
-    __syncthreads();
+    sync();
     // first index whose running sum exceeds the target: the lowest such lane of each wave, then the lowest wave
     {
         const bool beyond = prm.top_k > 0 && sh_count >= 0 && tid < keep && sh_target < sh_exp[tid];
         const unsigned long long lanes = __builtin_amdgcn_ballot_w64(beyond);
         if (lane == 0) sh_wave_first[wave] = lanes ? 64 * wave + __builtin_ctzll(lanes) : 0x7fffffff;
     }
-    __syncthreads();
+    sync();
     int32_t chosen = id_of(0);
     if (tid == 0 && prm.top_k > 0 && sh_count >= 0) {
         const int first = min(min(sh_wave_first[0], sh_wave_first[1]), min(sh_wave_first[2], sh_wave_first[3]));
         chosen = id_of(min(first, sh_count));              // sh_count = keep - 1: the answer if no sum exceeds the target
     }
     return chosen;
+}
+
+struct WholeBlockBarrier {
+    __device__ __forceinline__ void operator()() const { __syncthreads(); }
+};
+__device__ __forceinline__ int32_t sampler_block(const SamplerParams& prm, SamplerScratch& sh, const float (&score)[kSmpPerThread],
+                                                 unsigned long long& rng) {
+    return sampler_block(prm, sh, score, rng, WholeBlockBarrier());
 }
 
 }  // namespace qm

@@ -37,6 +37,7 @@
 
 #include "qm_device.h"
 #include "qm_host.h"
+#include "qm_resident.h"
 
 #include <atomic>
 #include <type_traits>
@@ -121,13 +122,6 @@ struct TkShared {
     float bias[16];
 };
 
-__device__ __forceinline__ uint32_t agent_load(const uint32_t* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void agent_store(uint32_t* p, uint32_t v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // A compute thread's words tid, tid + 256, ... of a tagged vector, all requested at once, again and again until
 // every one carries `tag`.  False when the wait gave up (or another block did).
 template <int N>
@@ -145,68 +139,6 @@ __device__ __forceinline__ bool poll_words(const uint32_t* words, uint32_t tag, 
         if ((spins & 255u) == 255u && agent_load(abort_word) != 0u) return false;
         __builtin_amdgcn_s_sleep(1);
     }
-}
-
-// Waits until at most `later` of this wave's memory operations are outstanding, rounded down to a multiple of four.
-template <int N>
-__device__ __forceinline__ void wait_vm_at_most() {
-    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
-}
-__device__ __forceinline__ void wait_for_all_but(int later) {
-    switch (later >> 2) {
-        case 0: wait_vm_at_most<0>(); break;
-        case 1: wait_vm_at_most<4>(); break;
-        case 2: wait_vm_at_most<8>(); break;
-        case 3: wait_vm_at_most<12>(); break;
-        case 4: wait_vm_at_most<16>(); break;
-        case 5: wait_vm_at_most<20>(); break;
-        case 6: wait_vm_at_most<24>(); break;
-        case 7: wait_vm_at_most<28>(); break;
-        default: wait_vm_at_most<32>(); break;
-    }
-}
-
-// LDS reads the compiler does not see (see the head of the file), with the waits the hardware needs: lds_wait()
-// before the first use, then pin() on every register read into, so that no use is scheduled above the wait.
-__device__ __forceinline__ uint32_t lds_at(const void* p) {
-    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)p));
-}
-template <int J, int N, int STRIDE>
-__device__ __forceinline__ void lds_read_b32(uint32_t at, uint32_t (&v)[N]) {
-    if constexpr (J < N) {
-        asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v[J]) : "v"(at), "n"(J * STRIDE));
-        lds_read_b32<J + 1, N, STRIDE>(at, v);
-    }
-}
-template <int J, int N, int STRIDE>
-__device__ __forceinline__ void lds_read_u16(uint32_t at, uint32_t (&v)[N]) {
-    if constexpr (J < N) {
-        asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(v[J]) : "v"(at), "n"(J * STRIDE));
-        lds_read_u16<J + 1, N, STRIDE>(at, v);
-    }
-}
-__device__ __forceinline__ void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-template <int J, int N>
-__device__ __forceinline__ void pin(uint32_t (&v)[N]) {
-    if constexpr (J < N) {
-        asm volatile("" : "+v"(v[J]));
-        pin<J + 1, N>(v);
-    }
-}
-__device__ __forceinline__ uint32_t lds_word(const void* p) {
-    uint32_t v;
-    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_at(p)) : "memory");
-    return v;
-}
-// the smallest of four (three) counters that lie together, 16-byte aligned
-typedef int tk_int4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ tk_int4 lds_four(const void* p) {
-    tk_int4 v;
-    asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_at(p)) : "memory");
-    return v;
-}
-__device__ __forceinline__ void lds_store(void* p, uint32_t v) {
-    asm volatile("ds_write_b32 %0, %1" : : "v"(lds_at(p)), "v"(v) : "memory");
 }
 
 // A weight wave (`third` = 0, 1, 2): requests its pieces of unit `v` of block `b` into `slot`, one by one, each once
@@ -303,7 +235,7 @@ __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p)
             // the slot is free once unit r - kTkSlots has been read by all four compute waves
             if (r >= kTkSlots) {
                 for (;;) {
-                    const tk_int4 d = lds_four(sh.done);
+                    const lds_int4 d = lds_four(sh.done);
                     if (min(min(d.x, d.y), min(d.z, d.w)) > r - kTkSlots) break;
                     if (lds_word(&sh.abort) != 0u) { alive = false; break; }
                     if (published < r) {                  // nothing to request: see everything requested land, say so
@@ -349,7 +281,7 @@ __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p)
         // it arrived is there for whoever sees its arrival); false when the launch gave up
         auto compute_barrier = [&]() __attribute__((always_inline)) -> bool {
             arrivals += kTkComputeThreads / 64;
-            if (lane == 0) asm volatile("ds_add_u32 %0, %1" : : "v"(lds_at(&sh.arrivals)), "v"(1u) : "memory");
+            if (lane == 0) lds_add_one(&sh.arrivals);
             return wait_for(&sh.arrivals, arrivals);
         };
         auto give_up = [&]() __attribute__((always_inline)) { lds_store(&sh.abort, 1u); };
@@ -360,7 +292,7 @@ __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p)
             constexpr int kSteps = kDual ? kTkDualColumns / 32 : kTkUnitColumns / 32;
             unsigned char* const slot = ring + (unit & (kTkSlots - 1)) * kTkSlotBytes;
             for (;;) {
-                const tk_int4 landed = lds_four(sh.landed);
+                const lds_int4 landed = lds_four(sh.landed);
                 if (min(min(landed.x, landed.y), landed.z) > unit) break;
                 if (lds_word(&sh.abort) != 0u) return false;
                 __builtin_amdgcn_s_sleep(1);
