@@ -33,7 +33,8 @@
 // Arithmetic: the operators of qm_linear.hip (R17:15239-15266, 15340-15360, 16205-16362, 8276-8338) chain for
 // chain, tree for tree and rounding for rounding — the outputs equal the four launches' bit for bit.
 //
-// Geometry is the talker's (R17:7930-7948): hidden 2048, 16 / 8 heads of 128, intermediate 6144.
+// Geometry is that of the 1.7B talker: hidden 2048 (R17:14626), and what its checkpoint gives for the rest
+// (R17:14862, 14993-15003): 16 / 8 heads of 128, intermediate 6144.
 
 #include "qm_device.h"
 #include "qm_host.h"

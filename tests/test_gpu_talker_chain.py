@@ -2,7 +2,8 @@
 talker layer and the RMSNorm + Q/K/V of the next one in one launch.
 
 The launch must leave exactly what the four one-operator entry points leave (bit for bit); those are held against the
-oracle in test_gpu_linear.py.  Weights are random in the talker's real geometry (R17:7930-7948).
+oracle in test_gpu_linear.py.  Weights are random in the 1.7B talker's geometry (hidden 2048, R17:14626; the rest from its
+checkpoint, R17:14993-15003).
 """
 import ctypes as C
 
