@@ -725,6 +725,113 @@ class PredictorFrameSteps:
         return {"all": dt}, (worst if self.codes_match else 1.0e9), "one frame (14 steps); all sampled codes equal"
 
 
+def generate_end_to_end(qm, dev, frames=96, prompt_rows=128, seed=20240229):
+    """Beyond the five configurations: the engine shell's generation loop (prefill of a prompt, then per frame the
+    final head, the code predictor's fifteen steps and the talker's decode step; R17:21887-22538) on a synthetic
+    checkpoint of the 1.7B model's real geometry (28 talker layers of hidden 2048 / intermediate 6144, the code
+    predictor's five layers, fifteen heads and tables), written to a temporary directory as sharded safetensors.
+    Reports the time per generated frame for the default paths and with the talker layers and the predictor frame
+    operator by operator; the codec trajectories of all four must be identical."""
+    import importlib
+    import shutil
+    import tempfile
+    import torch
+    from safetensors.torch import save_file
+    engine = importlib.import_module("qingming-qwen3-tts_amd.engine")
+    H, Q, KV, I, LAYERS = 2048, 2048, 1024, 6144, 28
+    PH, PI, P_LAYERS, V, STEPS = 1024, 3072, 5, 2048, 15
+    HEAD_V, TABLE_ROWS = 3072, 3072
+    g = torch.Generator().manual_seed(7)
+
+    def rnd(shape, std=1.0, mean=0.0):
+        # (host generator: the files are what the engine reads; drawn in fp32 and rounded once)
+        return torch.empty(shape, dtype=torch.float32).normal_(mean, std, generator=g).to(torch.bfloat16)
+
+    directory = tempfile.mkdtemp(prefix="qm_generate_")
+    try:
+        t0 = time.perf_counter()
+        shard = 0
+
+        def write(tensors):
+            nonlocal shard
+            shard += 1
+            save_file(tensors, os.path.join(directory, "model-%05d.safetensors" % shard))
+
+        write({"talker.model.norm.weight": rnd((H,), 0.1, 1.0), "talker.model.codec_embedding.weight": rnd((TABLE_ROWS, H), 0.5),
+               "talker.codec_head.weight": rnd((HEAD_V, H), 0.05)})
+        for i in range(LAYERS):
+            p = "talker.model.layers.%d." % i
+            write({p + "input_layernorm.weight": rnd((H,), 0.1, 1.0), p + "post_attention_layernorm.weight": rnd((H,), 0.1, 1.0),
+                   p + "self_attn.q_proj.weight": rnd((Q, H), 0.02), p + "self_attn.k_proj.weight": rnd((KV, H), 0.02),
+                   p + "self_attn.v_proj.weight": rnd((KV, H), 0.02), p + "self_attn.o_proj.weight": rnd((H, Q), 0.02),
+                   p + "self_attn.q_norm.weight": rnd((128,), 0.1, 1.0), p + "self_attn.k_norm.weight": rnd((128,), 0.1, 1.0),
+                   p + "mlp.gate_proj.weight": rnd((I, H), 0.02), p + "mlp.up_proj.weight": rnd((I, H), 0.02),
+                   p + "mlp.down_proj.weight": rnd((H, I), 0.02)})
+        c = "talker.code_predictor."
+        t = {c + "small_to_mtp_projection.weight": rnd((PH, H), 0.02), c + "small_to_mtp_projection.bias": rnd((PH,), 0.1),
+             c + "model.norm.weight": rnd((PH,), 0.1, 1.0)}
+        for i in range(P_LAYERS):
+            p = c + "model.layers.%d." % i
+            t.update({p + "input_layernorm.weight": rnd((PH,), 0.1, 1.0), p + "post_attention_layernorm.weight": rnd((PH,), 0.1, 1.0),
+                      p + "self_attn.q_proj.weight": rnd((Q, PH), 0.03), p + "self_attn.k_proj.weight": rnd((KV, PH), 0.03),
+                      p + "self_attn.v_proj.weight": rnd((KV, PH), 0.03), p + "self_attn.o_proj.weight": rnd((PH, Q), 0.02),
+                      p + "self_attn.q_norm.weight": rnd((128,), 0.1, 1.0), p + "self_attn.k_norm.weight": rnd((128,), 0.1, 1.0),
+                      p + "mlp.gate_proj.weight": rnd((PI, PH), 0.03), p + "mlp.up_proj.weight": rnd((PI, PH), 0.03),
+                      p + "mlp.down_proj.weight": rnd((PH, PI), 0.02)})
+        for i in range(STEPS):
+            t[c + "lm_head.%d.weight" % i] = rnd((V, PH), 0.05)
+            t[c + "model.codec_embedding.%d.weight" % i] = rnd((V, H), 0.5)
+        write(t)
+        del t
+        wrote = time.perf_counter() - t0
+
+        t0 = time.perf_counter()
+        talker = engine.Talker(directory, prompt_rows + frames + 16)
+        head = engine.FinalHead(directory, frames + 16, seed, talker.stream)
+        predictor = engine.Predictor(directory, head.rng_state, talker.stream)
+        loaded = time.perf_counter() - t0
+        prompt = rnd((prompt_rows, H)).view(torch.int16).to(dev)
+        tts_pad = rnd((H,), 0.5).view(torch.int16).numpy().view(np.uint16)
+        torch.cuda.synchronize()
+        rows = {}
+        reference = None
+        for name, talker_ops, frame_ops in (("default", 0, 0), ("talker_layers_by_operators", 1, 0),
+                                            ("predictor_frame_by_operators", 0, 1), ("both_by_operators", 1, 1)):
+            qm.set_option(qm.OPT_TALKER_LAYER_OPERATORS, talker_ops)
+            qm.set_option(qm.OPT_PREDICTOR_FRAME_OPERATORS, frame_ops)
+            try:
+                best = None
+                for _ in range(3):
+                    head.reset(seed)
+                    # one frame alone = prefill + first frame; the difference to the full run is the steady state
+                    t0 = time.perf_counter()
+                    engine.generate(talker, head, predictor, prompt, prompt_rows, 1, tts_pad)
+                    first = time.perf_counter() - t0
+                    head.reset(seed)
+                    t0 = time.perf_counter()
+                    codes, digest = engine.generate(talker, head, predictor, prompt, prompt_rows, frames, tts_pad)
+                    whole = time.perf_counter() - t0
+                    made = int(codes.shape[0])
+                    per_frame = (whole - first) / max(made - 1, 1)
+                    if best is None or per_frame < best[0]:
+                        best = (per_frame, first, made, digest)
+                if reference is None:
+                    reference = (codes.copy(), digest)
+                elif not (np.array_equal(codes, reference[0]) and digest == reference[1]):
+                    raise RuntimeError("generate: the codec trajectory of '%s' differs from the default paths'" % name)
+                rows[name] = {"ms_per_frame": best[0] * 1e3, "ms_prefill_and_first_frame": best[1] * 1e3, "frames": best[2],
+                              "codec_fnv1a64": "%016x" % best[3]}
+            finally:
+                qm.set_option(qm.OPT_TALKER_LAYER_OPERATORS, 0)
+                qm.set_option(qm.OPT_PREDICTOR_FRAME_OPERATORS, 0)
+        predictor.close(); head.close(); talker.close()
+        return {"workload": "generate_%d_frames_after_a_%d_token_prompt_1p7b_geometry_synthetic_checkpoint" % (frames, prompt_rows),
+                "paths": rows, "seconds_to_write_checkpoint": wrote, "seconds_to_load": loaded,
+                "audio_ms_per_frame": 80.0, "real_time_factor_default": rows["default"]["ms_per_frame"] / 80.0}
+    finally:
+        shutil.rmtree(directory, ignore_errors=True)
+
+
 class Prefill:
     """configs[3]: causal GQA prefill, batch 4 x seq 1024, K/V also written to shuffled 16-token pages."""
     name = "causal_prefill_b4_s1024_paged16"
@@ -873,7 +980,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
     ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "prefillfp32", "predictor", "predictorexact",
-                                      "qkv", "layer", "layer1", "frame", "frame1", "linears", "linearsexact"], default=None,
+                                      "qkv", "layer", "layer1", "frame", "frame1", "linears", "linearsexact", "generate"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -903,6 +1010,9 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
 
+    if args.only == "generate":
+        print(json.dumps(generate_end_to_end(qm, dev)))
+        return
     if args.only:
         make = {"decode512": lambda: SingleDecode(qm, dev, 512, False, 11),
                 "talker2048": lambda: SingleDecode(qm, dev, 2048, True, 12),
@@ -996,6 +1106,12 @@ def main():
             torch.cuda.empty_cache()
         rep["us_per_step_graph"] = _time_graph(head.step, reps=5, replays=10) * 1e3
         per_config["cfg3_ragged_decode"] = dict(rep)
+        # the generation loop end to end on a synthetic checkpoint of the real size (3.2 GB written to a temporary
+        # directory): skipped, with the reason, where that cannot be written
+        try:
+            per_config["next_generate_end_to_end"] = generate_end_to_end(qm, dev)
+        except OSError as e:
+            per_config["next_generate_end_to_end"] = {"skipped": "%s: %s" % (type(e).__name__, e)}
 
     cpu = None
     if oracle is not None:
