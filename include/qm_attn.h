@@ -402,23 +402,30 @@ int32_t qm_predictor_step_attention_m1(
     int32_t cache_position, float epsilon, void* hip_stream);
 
 /*
- * The M = 1 steps first_step .. last_step (1 .. 14) of one code-predictor frame in ONE launch: replaces the graph of
+ * The steps first_step .. last_step (0 .. 14) of one code-predictor frame in ONE launch: replaces the graph of
  * PersistentPredictor::capture_step (R17:13592-13854; 46 nodes per step) for those steps — per step the input
  * projection (small_to_mtp_projection with bias, R17:13600-13612), five layers of RMSNorm + Q/K/V, QK-norm +
  * RoPE + cache append + attention at cache position step + 1, o_proj, residual + post-norm + gate/up/SwiGLU,
  * down_proj + residual (R17:13614-13780), the final norm with that step's head, the top-k sampler (top_k <= 0:
  * arg-max) and the gather of the sampled code's embedding (R17:13782-13854) — with every rounding and summation
- * order of the one-operator entry points of this header, whose results it equals bit for bit.
+ * order of the one-operator entry points of this header, whose results it equals bit for bit.  Step 0 (two rows: the
+ * talker's hidden state and the embedding of the talker's code, R17:13663-13699) is run as two passes at cache
+ * positions 0 and 1 with the chain order of the row operators the reference uses there (qm_linear_rows: every row as
+ * qm_linear_m1 evaluates it), the first pass without head and sampler: the caches' rows 0 and 1, codes[1], selected[1]
+ * and the next input equal, bit for bit, what the reference's step-0 operators leave (qm_linear_rows, qm_rmsnorm_rows,
+ * qm_predictor_transpose / _rope_bhsd / _update_cache, qm_predictor_attention_staged, qm_gate_up_swiglu_rows).
  *
  * qm_predictor_frame names the tensors (bf16, 16-byte aligned; geometry of R17:7951-7964: hidden 1024, 16 / 8
  * heads of 128, intermediate 3072, outer dimension 2048, vocabulary 2048, five layers):
  *   layers[i]: input_norm, post_norm [1024]; q_weight [2048][1024], k_weight, v_weight [1024][1024]; q_norm,
  *     k_norm [128]; o_weight [1024][2048]; gate_weight, up_weight [3072][1024]; down_weight [1024][3072];
- *     key_cache, value_cache [8][16][128] holding the frame's positions 0 .. first_step, appended to in place;
+ *     key_cache, value_cache [8][16][128] holding the frame's positions 0 .. first_step (none when first_step is 0),
+ *     appended to in place;
  *   projection_weight [1024][2048], projection_bias [1024], final_norm [1024]; heads[s] [2048][1024] and
  *   embeddings[s] [2048][2048] for the steps s run (other entries are not read); cosine, sine [16][128];
- *   free_input [2048]: in, the input of first_step (the embedding gathered at the end of the step before); out, the
- *     embedding of the last code sampled;  selected [16][2048]: row s + 1 receives the embedding of step s's code;
+ *   free_input [2048]: in, the input of first_step >= 1 (the embedding gathered at the end of the step before); out, the
+ *     embedding of the last code sampled;  step0_input [2][2048] (read when first_step is 0, else may be NULL): the
+ *     talker's hidden state and the embedding of the talker's code;  selected [16][2048]: row s + 1 receives the embedding of step s's code;
  *   codes [16]: codes[s + 1] receives step s's code;  rng_state: the SplitMix64 state the draws advance.
  *
  * The launch is 256 blocks that stay resident and hand each operator's output to one another through
@@ -460,6 +467,7 @@ typedef struct qm_predictor_frame {
     int32_t* codes;
     uint64_t* rng_state;
     float epsilon;
+    const uint16_t* step0_input;      /* [2][2048], first_step == 0 only */
 } qm_predictor_frame;
 
 int64_t qm_predictor_frame_workspace_bytes(void);

@@ -47,6 +47,7 @@ class PredictorFrame(C.Structure):
         ("cosine", C.c_void_p), ("sine", C.c_void_p),
         ("free_input", C.c_void_p), ("selected", C.c_void_p), ("codes", C.c_void_p), ("rng_state", C.c_void_p),
         ("epsilon", C.c_float),
+        ("step0_input", C.c_void_p),
     ]
 
 
@@ -420,7 +421,7 @@ STATUS_FRAME_TIMEOUT = 8
 
 
 def predictor_frame(layers, projection_weight, projection_bias, final_norm, heads, embeddings, cosine, sine, free_input,
-                    selected, codes, rng_state, epsilon=1e-6):
+                    selected, codes, rng_state, epsilon=1e-6, step0_input=None):
     """qm_predictor_frame from tensors: `layers` is five dicts with the field names of qm_predictor_frame_layer,
     `heads` / `embeddings` map a step (1..14) to its tensor.  The tensors must outlive the descriptor."""
     frame = PredictorFrame()
@@ -437,6 +438,7 @@ def predictor_frame(layers, projection_weight, projection_bias, final_norm, head
     frame.free_input, frame.selected, frame.codes, frame.rng_state = (_addr(free_input), _addr(selected), _addr(codes),
                                                                       _addr(rng_state))
     frame.epsilon = epsilon
+    frame.step0_input = _addr(step0_input)
     return frame
 
 

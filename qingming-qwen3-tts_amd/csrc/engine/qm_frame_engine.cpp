@@ -197,12 +197,13 @@ static std::unique_ptr<qm_predictor> create_predictor(const std::string& model_d
             d.key_cache = w.key_cache.u16(); d.value_cache = w.value_cache.u16();
         }
         f.projection_weight = p->projection_weight.data(); f.projection_bias = p->projection_bias.data(); f.final_norm = p->final_norm.data();
-        for (int step = 1; step < kPredSteps; ++step) {
+        for (int step = 0; step < kPredSteps; ++step) {
             f.heads[step] = p->heads[static_cast<size_t>(step)].data();
             f.embeddings[step] = p->embeddings[static_cast<size_t>(step)].data();
         }
         f.cosine = p->cosine.u16(); f.sine = p->sine.u16();
         f.free_input = p->free_input.u16(); f.selected = p->selected.u16(); f.codes = static_cast<int32_t*>(p->codes.raw());
+        f.step0_input = p->free_input.u16();              // the two rows of step 0 (its first row is also the later steps' input)
         f.rng_state = rng_state; f.epsilon = kEpsilon;
         p->frame_workspace = DeviceBuffer(static_cast<size_t>(qm_predictor_frame_workspace_bytes()));
         op_check(qm_predictor_frame_workspace_init(p->frame_workspace.raw(), static_cast<int64_t>(p->frame_workspace.bytes()), stream),
@@ -312,15 +313,16 @@ static void predictor_frame(qm_predictor& p, const uint16_t* talker_hidden_devic
     op_check(qm_predictor_prepare_group0(p.codec0_table.data(), static_cast<int32_t>(p.codec0_table.shape[0]), code0_device, kOuter,
                                          p.free_input.u16(), p.selected.u16(), static_cast<int32_t*>(p.codes.raw()), s),
              "predictor group 0 input");
-    predictor_step0(p, sampling);
     int32_t by_operators = 0;
     op_check(qm_get_option(QM_OPT_PREDICTOR_FRAME_OPERATORS, &by_operators), "predictor frame option");
     const bool one_launch = p.one_launch && by_operators == 0;
     if (one_launch) {
-        op_check(qm_predictor_frame_steps(&p.frame, 1, kPredSteps - 1, sampling ? kTopK : 0, kTemperature, p.frame_workspace.raw(),
+        // all fifteen steps in one launch (step 0 as two passes of the talker-order chain: same bits as predictor_step0)
+        op_check(qm_predictor_frame_steps(&p.frame, 0, kPredSteps - 1, sampling ? kTopK : 0, kTemperature, p.frame_workspace.raw(),
                                           static_cast<int64_t>(p.frame_workspace.bytes()), static_cast<uint32_t*>(p.status.raw()), s),
                  "predictor frame steps");
     } else {
+        predictor_step0(p, sampling);
         for (int step = 1; step < kPredSteps; ++step) predictor_step_m1(p, step, sampling);
     }
     op_check(qm_predictor_next_talker_input(p.selected.u16(), kCodeGroups, p.context_embedding.u16(), kOuter, p.embedding_sum.u16(),

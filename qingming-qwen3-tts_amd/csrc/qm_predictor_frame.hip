@@ -27,6 +27,11 @@
 // dot products, the same shuffle trees, the same block sums for the norms — the sampled codes are those of the
 // operator-by-operator path bit for bit.
 //
+// Step 0.  The frame's first step has two rows (the talker's hidden state and the embedding of the talker's code) and
+// the reference runs it through its row operators (R17:13663-13699).  Row by row those are the talker-order M = 1
+// operators — lane l takes k = l, l + 32, ... — and the causal two-row attention is the M = 1 attention at positions
+// 0 and 1: step 0 is run here as two more passes of the same loop with that chain order, the first without a head.
+//
 // Geometry is the predictor's (R17:7951-7964): hidden 1024, 16 / 8 heads of 128, intermediate 3072, outer
 // dimension 2048, vocabulary 2048, five layers, cache of 16 positions.
 
@@ -49,8 +54,9 @@ constexpr int kFrInter = 3072;
 constexpr int kFrOuter = 2048;
 constexpr int kFrVocab = 2048;
 constexpr int kFrCache = 16;
-constexpr int kFrFirstStep = 1;
+constexpr int kFrFirstStep = 0;
 constexpr int kFrLastStep = 14;
+constexpr int kFrPositions = 16;                     // passes of a whole frame: positions 0 and 1 are step 0
 constexpr int kFrPhasesPerStep = 32;                 // tags reserved per step (28 used)
 constexpr unsigned kFrSpinLimit = 1u << 17;          // polls of about a microsecond each (FrParams::spin_limit)
 
@@ -120,6 +126,7 @@ struct FrParams {
     const uint16_t* embeddings[kFrLastStep + 1];     // [step]
     const uint16_t* cosine;                          // [16][128]
     const uint16_t* sine;
+    const uint16_t* step0_input;                     // [2][2048] (first_step == 0)
     uint16_t* free_input;                            // [2048]
     uint16_t* selected;                              // [16][2048]
     int32_t* codes;                                  // [16]
@@ -294,11 +301,18 @@ __device__ __forceinline__ bool linear_phase(FrShared& sh, unsigned char* smem, 
             }
         } else {
             const uint16_t* w0 = reinterpret_cast<const uint16_t*>(row0) + l;
-            uint32_t a[kSteps];
+            const uint16_t* w1 = reinterpret_cast<const uint16_t*>(row1) + l;
+            uint32_t a[kSteps], b[DUAL ? kSteps : 1];
 #pragma unroll
-            for (int j = 0; j < kSteps; ++j) a[j] = w0[32 * j];
+            for (int j = 0; j < kSteps; ++j) {
+                a[j] = w0[32 * j];
+                if (DUAL) b[j] = w1[32 * j];
+            }
 #pragma unroll
-            for (int j = 0; j < kSteps; ++j) acc = fmaf(x_one[j], bf2f(static_cast<uint16_t>(a[j])), acc);
+            for (int j = 0; j < kSteps; ++j) {
+                acc = fmaf(x_one[j], bf2f(static_cast<uint16_t>(a[j])), acc);
+                if (DUAL) up = fmaf(x_one[j], bf2f(static_cast<uint16_t>(b[j])), up);
+            }
         }
         // the reference's shuffle tree over its 32 lanes; lane 0 holds the sum
         acc = half_wave_tree_sum(acc);
@@ -444,7 +458,8 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
         return;
     }
 
-    const int first = prm.first_step, last = prm.last_step;
+    // Passes are numbered by the cache position they write: step s >= 1 is position s + 1, step 0 positions 0 and 1.
+    const int first = prm.first_step == 0 ? 0 : prm.first_step + 1, last = prm.last_step + 1;
     const unsigned spin_limit = prm.spin_limit;
     // ---- the weights of the first operators -----------------------------------------------------------------------
     const int qkv_row = kFrRowsQkv * b;                   // this block's Q/K/V rows lie in one matrix
@@ -481,7 +496,7 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
     const int my_layer = b >> 3, my_head = b & 7;
     if (attends) {
         uint16_t* kc = reinterpret_cast<uint16_t*>(smem + kFrLdsCache);
-        const int rows_before = first + 1;                // cache positions 0 .. first
+        const int rows_before = first;                    // cache positions 0 .. first - 1
         for (int c = tid; c < 2 * kFrCache * 16; c += kFrThreads) {
             const int chunk = c & 15, row = (c >> 4) & 15, is_v = c >> 8;
             uint4 value = make_uint4(0, 0, 0, 0);
@@ -506,14 +521,19 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
     uint32_t* const code_words = ws + kFrWsCode;
 
 #pragma unroll 1
-    for (int step = first; step <= last; ++step) {
-        const int position = step + 1;                    // cache_before of an M = 1 step (R17:13594-13596)
-        const uint32_t t0 = base + static_cast<uint32_t>(step - first) * kFrPhasesPerStep;
+    for (int position = first; position <= last; ++position) {
+        const int step = position - 1;                    // of the head and of the table of the code sampled after this pass
+        const bool pairs = position >= 2;                 // the predictor's chain order; step 0 runs the talker's
+        const uint32_t t0 = base + static_cast<uint32_t>(position - first) * kFrPhasesPerStep;
         auto tag = [&](int phase) { return (t0 + static_cast<uint32_t>(phase)) & 0xffffu; };
 
-        // ---- input projection: the first step's input is given, a later one's is the embedding of the code just sampled ----
+        // ---- input projection.  The input of the first pass of a launch is given (step 0: the talker's hidden state,
+        // then the embedding of the talker's code; otherwise the free input); a later one's is the embedding of the code
+        // just sampled ----
         const uint16_t* x_plain = prm.free_input;
-        if (step != first) {
+        if (position < 2) {
+            x_plain = prm.step0_input + position * kFrOuter;
+        } else if (position != first) {
             const uint32_t want = (t0 - kFrPhasesPerStep + 27u) & 0xffffu;
             uint32_t word = 0;
             bool ok = false;
@@ -525,7 +545,7 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
                 __builtin_amdgcn_s_sleep(1);
             }
             if (!ok) sh.abort = 1;
-            x_plain = prm.embeddings[step - 1] + static_cast<int64_t>(word & 0xffffu) * kFrOuter;
+            else x_plain = prm.embeddings[step - 1] + static_cast<int64_t>(word & (kFrVocab - 1)) * kFrOuter;
         }
         if (!linear_phase<false, 0, false, kFrOuter, kFrRowsProj>(sh, smem, kFrLdsOm, nullptr, 0, x_plain, nullptr, 0, nullptr, 0.0f,
                                                                   prm.projection_bias, false, 0, kFrRowsProj * b, hidden, tag(0), abort_word, spin_limit))
@@ -537,38 +557,55 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
 #pragma unroll 1
         for (int layer = 0; layer < kFrLayers; ++layer) {
             const FrLayer& w = prm.layers[layer];
-            const bool more = layer + 1 < kFrLayers || step < last;          // is there a next layer to request weights for
+            const bool more = layer + 1 < kFrLayers || position < last;      // is there a next layer to request weights for
             const FrLayer& next = prm.layers[layer + 1 < kFrLayers ? layer + 1 : 0];
             const int p = 1 + 5 * layer;
-            if (!linear_phase<false, 1, true, kFrHidden, kFrRowsQkv>(sh, smem, kFrLdsQkv, hidden, hidden_tag, nullptr, nullptr, 0, w.input_norm,
-                                                                     prm.epsilon, nullptr, false, 0, qkv_row, qkv, tag(p), abort_word, spin_limit))
-                { alive = false; break; }
+            alive = pairs
+                ? linear_phase<false, 1, true, kFrHidden, kFrRowsQkv>(sh, smem, kFrLdsQkv, hidden, hidden_tag, nullptr, nullptr, 0, w.input_norm,
+                                                                      prm.epsilon, nullptr, false, 0, qkv_row, qkv, tag(p), abort_word, spin_limit)
+                : linear_phase<false, 1, false, kFrHidden, kFrRowsQkv>(sh, smem, kFrLdsQkv, hidden, hidden_tag, nullptr, nullptr, 0, w.input_norm,
+                                                                       prm.epsilon, nullptr, false, 0, qkv_row, qkv, tag(p), abort_word, spin_limit);
+            if (!alive) break;
             if (more) request_qkv(next);
             if (attends && my_layer == layer) {
                 if (!attention_phase(sh, smem, prm, w, my_head, position, qkv, tag(p), ctx, tag(p + 1), abort_word, spin_limit)) { alive = false; break; }
             }
-            if (!linear_phase<false, 0, true, kFrQDim, kFrRowsO>(sh, smem, kFrLdsOm, ctx, tag(p + 1), nullptr, nullptr, 0, nullptr, 0.0f, nullptr,
-                                                                 false, 0, kFrRowsO * b, attn, tag(p + 2), abort_word, spin_limit))
-                { alive = false; break; }
-            if (layer + 1 < kFrLayers) request_o(next); else request_head(step);
-            if (!linear_phase<true, 2, true, kFrHidden, kFrRowsGu>(sh, smem, kFrLdsGu, hidden, hidden_tag, nullptr, attn, tag(p + 2), w.post_norm,
-                                                                   prm.epsilon, nullptr, false, kFrRowsDown * b, kFrRowsGu * b, act, tag(p + 3),
-                                                                   abort_word, spin_limit))
-                { alive = false; break; }
+            alive = pairs
+                ? linear_phase<false, 0, true, kFrQDim, kFrRowsO>(sh, smem, kFrLdsOm, ctx, tag(p + 1), nullptr, nullptr, 0, nullptr, 0.0f, nullptr,
+                                                                  false, 0, kFrRowsO * b, attn, tag(p + 2), abort_word, spin_limit)
+                : linear_phase<false, 0, false, kFrQDim, kFrRowsO>(sh, smem, kFrLdsOm, ctx, tag(p + 1), nullptr, nullptr, 0, nullptr, 0.0f, nullptr,
+                                                                   false, 0, kFrRowsO * b, attn, tag(p + 2), abort_word, spin_limit);
+            if (!alive) break;
+            // (the region after the last o_proj holds the pass's head; the first pass of step 0 has none)
+            if (layer + 1 < kFrLayers) request_o(next);
+            else if (position == 0) request_proj();
+            else request_head(step);
+            alive = pairs
+                ? linear_phase<true, 2, true, kFrHidden, kFrRowsGu>(sh, smem, kFrLdsGu, hidden, hidden_tag, nullptr, attn, tag(p + 2), w.post_norm,
+                                                                    prm.epsilon, nullptr, false, kFrRowsDown * b, kFrRowsGu * b, act, tag(p + 3),
+                                                                    abort_word, spin_limit)
+                : linear_phase<true, 2, false, kFrHidden, kFrRowsGu>(sh, smem, kFrLdsGu, hidden, hidden_tag, nullptr, attn, tag(p + 2), w.post_norm,
+                                                                     prm.epsilon, nullptr, false, kFrRowsDown * b, kFrRowsGu * b, act, tag(p + 3),
+                                                                     abort_word, spin_limit);
+            if (!alive) break;
             if (more) request_gu(next);
-            if (!linear_phase<false, 0, true, kFrInter, kFrRowsDown>(sh, smem, kFrLdsDown, act, tag(p + 3), nullptr, nullptr, 0, nullptr, 0.0f,
-                                                                     nullptr, true, 0, kFrRowsDown * b, hidden, tag(p + 4), abort_word, spin_limit))
-                { alive = false; break; }
+            alive = pairs
+                ? linear_phase<false, 0, true, kFrInter, kFrRowsDown>(sh, smem, kFrLdsDown, act, tag(p + 3), nullptr, nullptr, 0, nullptr, 0.0f,
+                                                                      nullptr, true, 0, kFrRowsDown * b, hidden, tag(p + 4), abort_word, spin_limit)
+                : linear_phase<false, 0, false, kFrInter, kFrRowsDown>(sh, smem, kFrLdsDown, act, tag(p + 3), nullptr, nullptr, 0, nullptr, 0.0f,
+                                                                       nullptr, true, 0, kFrRowsDown * b, hidden, tag(p + 4), abort_word, spin_limit);
+            if (!alive) break;
             if (more) request_down(next);
             hidden_tag = tag(p + 4);
         }
         if (!alive) break;
+        if (position == 0) continue;                      // step 0's first row: its keys and values are what it leaves
 
         // ---- final norm + this step's head ----
         if (!linear_phase<false, 1, false, kFrHidden, kFrRowsHead>(sh, smem, kFrLdsOm, hidden, hidden_tag, nullptr, nullptr, 0, prm.final_norm,
                                                                    prm.epsilon, nullptr, false, 0, kFrRowsHead * b, logits, tag(26), abort_word, spin_limit))
             break;
-        if (step < last) request_proj();
+        if (position < last) request_proj();
 
         // ---- the sampler and the gather of the sampled code's embedding: one block ----
         if (samples) {
@@ -607,7 +644,7 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
     if (tid == 0) {
         if (samples) *prm.rng_state = rng;
         // (every block has read the base before this one could finish its last operator)
-        if (b == 0) agent_store(ws + kFrWsBase, base + static_cast<uint32_t>(kFrLastStep) * kFrPhasesPerStep);
+        if (b == 0) agent_store(ws + kFrWsBase, base + static_cast<uint32_t>(kFrPositions) * kFrPhasesPerStep);
     }
 }
 
@@ -673,6 +710,8 @@ extern "C" int32_t qm_predictor_frame_steps(const qm_predictor_frame* frame, int
     if (!all) return QM_ERR_NULL;
     if (align & 15) return QM_ERR_GEOMETRY;               // 16-byte pieces of weight rows, cache rows and embedding rows
     prm.cosine = frame->cosine; prm.sine = frame->sine;
+    if (first_step == 0 && !frame->step0_input) return QM_ERR_NULL;
+    prm.step0_input = frame->step0_input;
     prm.free_input = frame->free_input; prm.selected = frame->selected; prm.codes = frame->codes;
     prm.rng_state = reinterpret_cast<unsigned long long*>(frame->rng_state);
     prm.workspace = static_cast<uint32_t*>(workspace);

@@ -1,4 +1,4 @@
-"""GPU parity of qm_predictor_frame_steps: the fourteen M = 1 steps of a code-predictor frame in one launch.
+"""GPU parity of qm_predictor_frame_steps: the steps of a code-predictor frame in one launch.
 
 The launch must leave exactly what the operator-by-operator chain of the same C entry points leaves (sampled codes,
 selected embeddings, the next input, the generator state and the appended K/V rows, bit for bit); that chain is held
@@ -43,11 +43,12 @@ class _Frame:
                                     wg=rnd((I, H), 0.03), wu=rnd((I, H), 0.03), wd=rnd((H, I), 0.02), k=k, v=v, k0=k.clone(),
                                     v0=v.clone()))
         self.final_norm = rnd((H,), 0.1, 1.0)
-        self.heads = {s: rnd((V, H), 0.05) for s in range(1, 15)}
-        self.tables = {s: rnd((V, OUT)) for s in range(1, 15)}
+        self.heads = {s: rnd((V, H), 0.05) for s in range(0, 15)}
+        self.tables = {s: rnd((V, OUT)) for s in range(0, 15)}
         cos, sin = oracle.rope_table(16, 0, 128, 1.0e6)
         self.cos, self.sin = to_dev(cos, dev), to_dev(sin, dev)
         self.input0 = rnd((OUT,))
+        self.step0_rows = rnd((2, OUT))                    # the talker's hidden state, the embedding of the talker's code
         z = lambda *shape: torch.zeros(shape, dtype=torch.int16, device=dev)
         self.free_input, self.selected = self.input0.clone(), z(16, OUT)
         self.codes = torch.zeros(16, dtype=torch.int32, device=dev)
@@ -61,7 +62,7 @@ class _Frame:
         self.status = torch.zeros(1, dtype=torch.int32, device=dev)
         layers = [{FIELDS[key]: layer[key] for key in FIELDS} for layer in self.layers]
         self.frame = qm.predictor_frame(layers, self.proj_w, self.proj_b, self.final_norm, self.heads, self.tables, self.cos,
-                                        self.sin, self.free_input, self.selected, self.codes, self.rng)
+                                        self.sin, self.free_input, self.selected, self.codes, self.rng, step0_input=self.step0_rows)
 
     def reset(self):
         self.free_input.copy_(self.input0)
@@ -93,6 +94,30 @@ class _Frame:
                               H, V, 0, 1e-6)
             qm.sample_topk(self.logits, True, 0, V, top_k, 0.9, self.rng, self.codes[step + 1:])
             qm.gather_embedding(self.tables[step], V, self.codes, step + 1, OUT, self.selected, self.free_input)
+
+    def step0_by_operators(self, top_k):
+        """Step 0 row by row with the talker-order M = 1 operators at cache positions 0 and 1 (what the reference's row
+        operators evaluate, row for row); the head, the sampler and the gather after the second row only."""
+        qm = self.qm
+        for layer in self.layers:
+            layer["k"].zero_()
+            layer["v"].zero_()
+        for position in (0, 1):
+            cur, nxt = self.hidden
+            qm.linear_m1(self.step0_rows[position], self.proj_w, self.proj_b, None, cur, H, OUT)
+            for layer in self.layers:
+                qm.rmsnorm_qkv_m1(cur, layer["in_norm"], layer["wq"], None, layer["wk"], None, layer["wv"], None, self.q, self.k_, self.v_,
+                                  H, Q, KV, 1e-6)
+                qm.predictor_step_attention_m1(self.q, self.k_, self.v_, layer["gq"], layer["gk"], self.cos[position],
+                                               self.sin[position], layer["k"], layer["v"], self.ctx, position, 1e-6)
+                qm.linear_m1(self.ctx, layer["wo"], None, None, self.attn, H, Q)
+                qm.add_postnorm_gate_up_swiglu_m1(cur, self.attn, layer["post"], self.res, layer["wg"], layer["wu"], self.act, H, I, 1e-6)
+                qm.linear_m1(self.act, layer["wd"], None, self.res, nxt, H, I)
+                cur, nxt = nxt, cur
+        head = self.heads[0]
+        qm.rmsnorm_qkv_m1(cur, self.final_norm, head, None, head, None, head, None, self.logits, self.logits, self.logits, H, V, 0, 1e-6)
+        qm.sample_topk(self.logits, True, 0, V, top_k, 0.9, self.rng, self.codes[1:])
+        qm.gather_embedding(self.tables[0], V, self.codes, 1, OUT, self.selected, self.free_input)
 
     def one_launch(self, first, last, top_k, stream=0):
         self.qm.predictor_frame_steps(self.frame, first, last, top_k, 0.9, self.ws, self.ws_bytes, self.status, stream)
@@ -127,6 +152,37 @@ def test_frame_steps_equal_the_operator_chain(frame, top_k):
         got = frame.snapshot()
         assert int(frame.status.item()) == 0
         assert _same(got, want)
+
+
+@pytest.mark.parametrize("top_k", [50, 0], ids=["top50", "argmax"])
+def test_step_0_and_the_whole_frame_in_one_launch(frame, top_k):
+    """Step 0 alone leaves what its row-by-row operators leave (caches rows 0 and 1, codes[1], selected[1], the next
+    input, the generator state); steps 0..14 in one launch equal step 0 followed by the operator chain of steps 1..14."""
+    frame.reset()
+    frame.step0_by_operators(top_k)
+    want0 = frame.snapshot()
+    assert 0 <= want0[0].tolist()[1] < V
+    frame.by_operators(1, 14, top_k)
+    want = frame.snapshot()
+    frame.reset()
+    for layer in frame.layers:
+        layer["k"].fill_(0x7fc0)                           # whatever a frame before left: step 0 reads none of it
+        layer["v"].fill_(0x7fc0)
+    frame.one_launch(0, 0, top_k)
+    got0 = frame.snapshot()
+    assert int(frame.status.item()) == 0
+    for layer in frame.layers:                             # (rows 2.. are not step 0's)
+        layer["k"][:, 2:] = 0
+        layer["v"][:, 2:] = 0
+    assert _same(frame.snapshot(), want0) and _same(got0[:4], want0[:4])
+    frame.reset()
+    frame.one_launch(0, 14, top_k)
+    assert _same(frame.snapshot(), want) and int(frame.status.item()) == 0
+    # and step 0 in one launch, the rest in another
+    frame.reset()
+    frame.one_launch(0, 0, top_k)
+    frame.one_launch(1, 14, top_k)
+    assert _same(frame.snapshot(), want)
 
 
 def test_frame_steps_in_several_launches(frame):
@@ -206,7 +262,12 @@ def test_frame_steps_abort_word_and_argument_errors(frame, qm, dev):
     call = lambda first, last, top_k, ws, nbytes: L.qm_predictor_frame_steps(C.byref(frame.frame), first, last, top_k, C.c_float(0.9),
                                                                              ws, nbytes, None, None)
     p = frame.ws.data_ptr()
-    assert call(0, 14, 50, p, frame.ws_bytes) == -5 and call(1, 15, 50, p, frame.ws_bytes) == -5 and call(5, 4, 50, p, frame.ws_bytes) == -5
+    assert call(-1, 14, 50, p, frame.ws_bytes) == -5 and call(1, 15, 50, p, frame.ws_bytes) == -5 and call(5, 4, 50, p, frame.ws_bytes) == -5
+    saved = frame.frame.step0_input
+    frame.frame.step0_input = None                         # step 0 needs its two rows
+    assert call(0, 14, 50, p, frame.ws_bytes) == -1 and call(1, 14, 50, p, frame.ws_bytes) == 0
+    frame.frame.step0_input = saved
+    torch.cuda.synchronize()
     assert call(1, 14, 257, p, frame.ws_bytes) == -5
     assert call(1, 14, 50, p, frame.ws_bytes - 256) == -4 and call(1, 14, 50, p + 64, frame.ws_bytes) == -2
     assert call(1, 14, 50, None, frame.ws_bytes) == -1
