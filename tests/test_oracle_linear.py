@@ -245,3 +245,68 @@ def test_predictor_qkv_and_gate_up_are_built_from_the_linear(oracle):
     want = g / (1.0 + np.exp(-g)) * u                                  # SiLU(g) * u
     got = oracle.bf16_to_f32(out).astype(np.float64)
     assert np.max(np.abs(got - want) / (np.abs(want) + 1e-3)) < 2e-2   # two bf16 roundings
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_the_predictors_step_0_is_two_m1_steps_in_the_talkers_chain_order(oracle, seed):
+    """What lets the frame kernel run step 0 as two more passes of its loop: one predictor layer over the two rows of step 0
+    with the reference's row operators (generic linears, per-head RMSNorm, BHSD transpose / RoPE / cache update, staged
+    causal attention; R17:13663-13699) leaves, bit for bit, what two M = 1 steps at cache positions 0 and 1 leave with the
+    talker-order M = 1 operators (fused Q/K/V, QK-norm + RoPE + append, M = 1 attention, o_proj, add + post-norm,
+    gate/up/SwiGLU, down_proj + residual): the layer's output rows, both caches and the attention's context."""
+    PH, Q, KV, PI, rows = 1024, 2048, 1024, 3072, 2
+    u16 = lambda *s: np.zeros(s, dtype=np.uint16)
+    n = [7000 + 100 * seed]
+
+    def rnd(shape, std=1.0, mean=0.0):
+        n[0] += 1
+        return oracle.normal_bf16(shape, n[0], mean, std, threads=8)
+
+    w = dict(inn=rnd((PH,), 0.1, 1.0), wq=rnd((Q, PH), 0.03), wk=rnd((KV, PH), 0.03), wv=rnd((KV, PH), 0.03),
+             gq=rnd((128,), 0.1, 1.0), gk=rnd((128,), 0.1, 1.0), wo=rnd((PH, Q), 0.02), post=rnd((PH,), 0.1, 1.0),
+             wg=rnd((PI, PH), 0.03), wu=rnd((PI, PH), 0.03), wd=rnd((PH, PI), 0.02))
+    cur = rnd((rows, PH))
+    cos, sin = oracle.rope_table(16, 0)
+    # the row operators
+    kc, vc = u16(8, 16, 128), u16(8, 16, 128)
+    norm, q, k, v = u16(rows, PH), u16(rows, Q), u16(rows, KV), u16(rows, KV)
+    assert oracle.rmsnorm_rows(cur, w["inn"], norm, rows, PH) == 0
+    for name, dst, columns in (("wq", q, Q), ("wk", k, KV), ("wv", v, KV)):
+        assert oracle.linear_rows(norm, w[name], None, None, dst, rows, columns, PH, 8) == 0
+    qn, kn = u16(rows * 16, 128), u16(rows * 8, 128)
+    assert oracle.rmsnorm_rows(q.reshape(rows * 16, 128), w["gq"], qn, rows * 16, 128) == 0
+    assert oracle.rmsnorm_rows(k.reshape(rows * 8, 128), w["gk"], kn, rows * 8, 128) == 0
+    qb, kb, vb = u16(16, rows, 128), u16(8, rows, 128), u16(8, rows, 128)
+    assert oracle.predictor_transpose(qn, qb, rows, 16) == 0
+    assert oracle.predictor_transpose(kn, kb, rows, 8) == 0
+    assert oracle.predictor_transpose(v, vb, rows, 8) == 0
+    qr, kr = u16(16, rows, 128), u16(8, rows, 128)
+    assert oracle.predictor_rope_bhsd(qb, cos, sin, qr, rows, 16) == 0
+    assert oracle.predictor_rope_bhsd(kb, cos, sin, kr, rows, 8) == 0
+    assert oracle.predictor_update_cache(kr, kc, rows, 0) == 0
+    assert oracle.predictor_update_cache(vb, vc, rows, 0) == 0
+    ctx = u16(rows, Q)
+    assert oracle.predictor_attention_staged(qr, kc, vc, ctx.reshape(rows, 16, 128), rows, 2, True) == 0
+    res, post, act, out_rows = u16(rows, PH), u16(rows, PH), u16(rows, PI), u16(rows, PH)
+    assert oracle.linear_rows(ctx, w["wo"], None, cur, res, rows, PH, Q, 8) == 0
+    assert oracle.rmsnorm_rows(res, w["post"], post, rows, PH) == 0
+    assert oracle.gate_up_swiglu_rows(post, w["wg"], w["wu"], act, rows, PH, PI, 8) == 0
+    assert oracle.linear_rows(act, w["wd"], None, res, out_rows, rows, PH, PI, 8) == 0
+    # two M = 1 steps
+    kc2, vc2 = u16(8, 16, 128), u16(8, 16, 128)
+    for r in range(rows):
+        norm1, q1, k1, v1, qrot, ctx1, attn, res1, post1, act1, out1 = (u16(1, PH), u16(Q), u16(KV), u16(KV), u16(Q), u16(Q), u16(PH),
+                                                                        u16(PH), u16(PH), u16(PI), u16(PH))
+        assert oracle.rmsnorm_rows(cur[r].reshape(1, PH), w["inn"], norm1, 1, PH) == 0
+        assert oracle.qkv_m1(norm1[0], w["wq"], None, w["wk"], None, w["wv"], None, q1, k1, v1, PH, Q, KV, 8) == 0
+        assert oracle.qk_norm_rope_kv_append(q1, k1, v1, w["gq"], w["gk"], cos[r], sin[r], qrot, oracle.flat_cache(kc2, vc2, 8, 16),
+                                             None, 1, 16, r) == 0
+        assert oracle.predictor_attention_m1(qrot, kc2, vc2, ctx1, r + 1) == 0
+        assert np.array_equal(ctx1, ctx[r])
+        assert oracle.linear_m1(ctx1, w["wo"], None, None, attn, PH, Q, 8) == 0
+        assert oracle.add_postnorm_m1(cur[r], attn, w["post"], res1, post1, PH) == 0
+        assert oracle.gate_up_swiglu_m1(post1, w["wg"], w["wu"], act1, PH, PI, 8) == 0
+        assert oracle.linear_m1(act1, w["wd"], None, res1, out1, PH, PI, 8) == 0
+        assert np.array_equal(out1, out_rows[r])
+    assert np.array_equal(kc, kc2) and np.array_equal(vc, vc2)
+    assert np.any(kc[:, :2] != 0) and not np.any(kc[:, 2:] != 0)
