@@ -26,7 +26,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# HBM bytes per launch of decode_split_kernel<2, false, true> on the headline workload, from rocprofv3 --pmc
+# HBM bytes per launch of decode_split_kernel<2, false, true, false> on the headline workload, from rocprofv3 --pmc
 # FETCH_SIZE and WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a
 # plain 512 MiB copy (FETCH_SIZE reads half the copied bytes: factor 2.0; WRITE_SIZE: 1.0).
 # Summary and commands: profiles/decode_split_kernel_ragged64_traffic.txt
@@ -1133,7 +1133,7 @@ def main():
                      "frac": rep["GBps"] / HBM_PEAK_GBPS, "traffic": HEADLINE_TRAFFIC_BYTES,
                      "traffic_source": "profiles/decode_split_kernel_ragged64_traffic.txt (rocprofv3 --pmc FETCH_SIZE / "
                                        "WRITE_SIZE of this workload; not measured in this run)",
-                     "kernel": "decode_split_kernel<2, false, true> (+ decode_merge_kernel<2>, both inside the timed step)",
+                     "kernel": "decode_split_kernel<2, false, true, false> (+ decode_merge_kernel<2, false>, both inside the timed step)",
                      "algorithmic_bytes_per_launch": head.bytes, "avg_launch_us": ms * 1e3},
         "cpu_baseline": cpu,
         "per_config": per_config,

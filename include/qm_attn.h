@@ -342,6 +342,33 @@ int32_t qm_prefill_attention_causal_split(
     uint32_t* status_dev,
     void* hip_stream);
 
+/*
+ * Attention of query_length rows of ONE sequence over its cache, for every shape the two entry points
+ * above do not serve: replaces NativeTalkerEngine::launch_attention in its generic branch
+ * (R17:17782-17813, kernel talker_attention_kernel R17:15744-16006) for any cache_before >= 0 (a prompt
+ * continued in chunks), any sliding window and any integral GQA group q_heads / kv_heads.
+ * query, context_out [query_length][q_heads][128]; row i attends keys
+ * [key_start_i, cache_before + i + 1), key_start_i = max(0, cache_before + i + 1 - sliding_window) for
+ * sliding_window > 0, else 0 (R17:15784-15789); query head h reads kv head h / (q_heads / kv_heads)
+ * (R17:15780-15782).  The keys and values of the rows themselves must already be in the cache
+ * (qm_scatter_kv at first_position = cache_before, as scatter_prefill_cache precedes the reference's call).
+ * page_table [max_pages] of that sequence, or NULL for pages in pool order (the flat LayerCache).
+ * Every row runs as one stream of the split-K decode kernels: row i carries the bits
+ * qm_decode_attention gives for cache_before + i, and the rounding is that entry point's.  K and V are
+ * read once per row (from the caches after the first), so for a whole prompt from an empty cache with
+ * group 2 qm_prefill_attention_causal is the faster call by an order of magnitude.
+ * Workspace: qm_attention_rows_workspace_bytes(query_length, q_heads, kv_heads, cache_before + query_length).
+ * query_length <= 65535.  status_dev (optional): QM_STATUS_BAD_PAGE for page-table entries out of range.
+ */
+size_t qm_attention_rows_workspace_bytes(int32_t query_length, int32_t q_heads, int32_t kv_heads, int32_t key_end);
+int32_t qm_attention_rows(
+    const uint16_t* query,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    uint16_t* context_out,
+    int32_t query_length, int32_t cache_before, int32_t q_heads, int32_t sliding_window, float scale,
+    void* workspace, size_t workspace_bytes, uint32_t* status_dev,
+    void* hip_stream);
+
 /* ---- (4) code-predictor attention loop ---------------------------------------------------- */
 /*
  * One launch for the whole per-frame step loop of the code predictor: replaces, per

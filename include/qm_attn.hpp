@@ -76,16 +76,19 @@ inline void launch_qk_norm_rope_cache_m1(
           "Qingming QK norm/RoPE/cache launch");
 }
 
-// Bytes of split-K workspace launch_attention needs for contexts up to max_cache tokens.
-inline std::size_t attention_workspace_bytes(int q_heads, int kv_heads, int max_cache) {
-    return qm_decode_workspace_bytes(1, q_heads, kv_heads, max_cache);
+// Bytes of split-K workspace launch_attention needs for contexts up to max_cache tokens: query_length 1, and
+// query_length > 1 where the call goes to the row-by-row operator (any cache_before, window or group).
+inline std::size_t attention_workspace_bytes(int q_heads, int kv_heads, int max_cache, int query_length = 1) {
+    return qm_attention_rows_workspace_bytes(query_length, q_heads, kv_heads, max_cache);
 }
 
 // ≙ NativeTalkerEngine::launch_attention (R17:17723-17814).  query_length == 1 is decode over
-// keys [key_start, cache_before + 1); query_length > 1 is the causal prefill over the rows that
-// scatter_prefill_cache has already placed in the cache, with cache_before == 0 as in
-// NativeTalkerEngine::prefill (R17:16710-16717).  The reference sizes dynamic LDS from the context;
-// here the caller passes a workspace sized by attention_workspace_bytes instead.
+// keys [key_start, cache_before + 1).  query_length > 1 attends the rows that scatter_prefill_cache has
+// already placed in the cache: a whole prompt from an empty cache with two query heads per kv head, as in
+// NativeTalkerEngine::prefill (R17:16710-16717), runs on the matrix cores; every other case of the
+// reference's generic kernel (cache_before > 0, a sliding window, another group) runs row by row.
+// The reference sizes dynamic LDS from the context; here the caller passes a workspace sized by
+// attention_workspace_bytes instead (the matrix-core case needs none).
 inline void launch_attention(
     const std::uint16_t* query, std::uint16_t* key_cache, std::uint16_t* value_cache,
     std::uint16_t* context, int query_length, int cache_before,
@@ -98,11 +101,13 @@ inline void launch_attention(
               "Talker GQA M1 attention launch");
         return;
     }
-    if (cache_before != 0 || sliding_window > 0) {
-        throw std::runtime_error("Talker generic attention launch: only cache_before == 0 without a "
-                                 "sliding window is supported for query_length > 1");
+    if (cache_before + query_length > max_cache) throw std::runtime_error("Talker prefill cache overflow.");
+    if (cache_before != 0 || sliding_window > 0 || q_heads != 2 * kv_heads) {
+        check(qm_attention_rows(query, &c, nullptr, 1, context, query_length, cache_before, q_heads, sliding_window,
+                                scale, workspace, workspace_bytes, nullptr, stream),
+              "Talker generic fused attention launch");
+        return;
     }
-    if (query_length > max_cache) throw std::runtime_error("Talker prefill cache overflow.");
     check(qm_prefill_attention_causal(query, key_cache, value_cache, context, nullptr, nullptr, 0, 1,
                                       query_length, q_heads, kv_heads, scale, head_dim,
                                       static_cast<std::int64_t>(max_cache) * head_dim, 0, nullptr, stream),

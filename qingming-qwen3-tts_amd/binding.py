@@ -89,6 +89,9 @@ _SIGNATURES = {
                                           _F32, _PTR, C.c_size_t, _PTR, _PTR]),
     "qm_decode_attention_ragged_static": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _PTR, _I32,
                                                  _F32, _PTR, _PTR]),
+    "qm_attention_rows_workspace_bytes": (C.c_size_t, [_I32, _I32, _I32, _I32]),
+    "qm_attention_rows": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _I32, _I32, _F32,
+                                 _PTR, C.c_size_t, _PTR, _PTR]),
     "qm_norm_rope_rows": (_I32, [_PTR] * 5 + [_I32, _I32, _F32, _PTR]),
     "qm_scatter_kv": (_I32, [_PTR, _PTR, C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _PTR, _PTR]),
     "qm_prefill_attention_causal": (_I32, [_PTR] * 4 + [C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _I32, _I32,
@@ -250,6 +253,17 @@ def decode_attention_ragged(query, cache, page_table, max_pages, seq_lens, n_str
         _addr(query), C.byref(cache), _addr(page_table), max_pages, _addr(seq_lens), n_streams,
         max_seq_len, _addr(out), q_heads, scale, _addr(workspace), workspace_bytes, _addr(status),
         stream), "qm_decode_attention_ragged")
+
+
+def attention_rows_workspace_bytes(query_length, q_heads, kv_heads, key_end):
+    return lib().qm_attention_rows_workspace_bytes(query_length, q_heads, kv_heads, key_end)
+
+
+def attention_rows(query, cache, page_table, max_pages, out, query_length, cache_before, q_heads, sliding_window=-1,
+                   scale=SCALE_128, workspace=None, workspace_bytes=0, status=None, stream=0):
+    _check(lib().qm_attention_rows(
+        _addr(query), C.byref(cache), _addr(page_table), max_pages, _addr(out), query_length, cache_before, q_heads,
+        sliding_window, scale, _addr(workspace), workspace_bytes, _addr(status), stream), "qm_attention_rows")
 
 
 def norm_rope_rows(x, norm_w, cos, sin, out, rows, heads, eps=1e-6, stream=0):
@@ -417,7 +431,7 @@ def predictor_step_attention_m1(q, k, v, gq, gk, cos_row, sin_row, key_cache, va
                                                 position, eps, stream), "qm_predictor_step_attention_m1")
 
 
-STATUS_FRAME_TIMEOUT = 8
+STATUS_BAD_PAGE, STATUS_BAD_POSITION, STATUS_SPLIT_TIMEOUT, STATUS_FRAME_TIMEOUT = 1, 2, 4, 8
 
 
 def predictor_frame(layers, projection_weight, projection_bias, final_norm, heads, embeddings, cosine, sine, free_input,

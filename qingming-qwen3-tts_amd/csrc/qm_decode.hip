@@ -76,11 +76,24 @@ struct DecodeParams {
     uint16_t* step_q_rotated;     // [q_heads][128] or NULL
     int step_position;
     float step_epsilon;
+    // Blocks (in y) that share one kv head: 1 when the kernel's G is the whole GQA group; a group the kernels
+    // are not instantiated for runs as several blocks of G heads each on the same K and V.
+    int head_groups_per_kv;
+    // Rows of one sequence as streams (qm_attention_rows): stream i is query row i, all rows share one page
+    // table, row i attends keys [window start, rows_cache_before + i + 1).  -1 = off.
+    int rows_cache_before;
+    int rows_window;
 };
 
 // Partial record of one (stream, kv head, split): G*128 acc, G max, G sum.
 template <int G>
 __host__ __device__ constexpr int partial_floats() { return G * kDim + 2 * G; }
+
+// Key range [start, end) of row `stream` of one sequence (GENERIC kernels, rows_cache_before >= 0): R17:15784-15789.
+__device__ __forceinline__ void row_key_range(const DecodeParams& prm, int stream, int& key_start, int& key_end) {
+    key_end = prm.rows_cache_before + stream + 1;
+    key_start = prm.rows_window > 0 ? max(key_end - prm.rows_window, 0) : 0;
+}
 
 // 16 bytes of K or V.  STREAMING adds the non-temporal hint: contexts much larger than the caches
 // are read once per step and should not displace anything on their way (measured on a 600 MB
@@ -104,7 +117,9 @@ __device__ __forceinline__ uint4 load_or_zero(const uint16_t* p, bool valid) {
 // STEP: the block first runs the QK-RMSNorm + RoPE of its query heads (and, if it owns the tile of
 // the new token, of the key head, appending K and V to the cache) — the reference's separate
 // launch_qk_norm_rope_cache_m1 (R17:17181) folded into the attention launch.
-template <int G, bool STEP, bool STREAMING>
+// GENERIC: what the decode calls of the reference's own shapes never need and therefore do not pay for — a GQA
+// group served by several blocks of G heads per kv head, and the rows of one sequence as streams.
+template <int G, bool STEP, bool STREAMING, bool GENERIC>
 __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodeParams prm, qm_kv_cache cache) {
     __shared__ __attribute__((aligned(16))) uint16_t sh_qrot[STEP ? G : 1][kDim];
     __shared__ float sh_acc[kRowStreams][G][kDim];
@@ -117,7 +132,8 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
     // the high splits are mostly empty: rotating the split by (head + stream) gives every XCD
     // every split index (ragged 64 x 256..4096 at 16 tiles per block: 118 us without, 100 us with).
     const int split = static_cast<int>((blockIdx.x + blockIdx.y + blockIdx.z) % gridDim.x);
-    const int kvh = blockIdx.y;
+    const int hg = blockIdx.y;   // group of G query heads; its kv head:
+    const int kvh = GENERIC ? hg / prm.head_groups_per_kv : hg;
     const int stream = blockIdx.z;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -135,12 +151,14 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
             if (tid == 0 && prm.status) atomicOr(prm.status, QM_STATUS_BAD_POSITION);
             key_end = prm.max_seq_len;
         }
+    } else if (GENERIC && prm.rows_cache_before >= 0) {
+        row_key_range(prm, stream, key_start, key_end);
     }
     if (key_end <= key_start) {
         // Empty context: zeros.  With several splits the merge kernel writes them.
         if (prm.max_splits == 1 && split == 0) {
             for (int o = tid; o < G * kDim; o += kDecodeThreads) {
-                prm.out[(static_cast<int64_t>(stream) * prm.q_heads + kvh * G) * kDim + o] = 0;
+                prm.out[(static_cast<int64_t>(stream) * prm.q_heads + hg * G) * kDim + o] = 0;
             }
         }
         return;
@@ -157,7 +175,9 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
     // iteration wait for the whole queue to drain).
     if (tid <= tile_hi - tile_lo) {
         const int32_t* table =
-            prm.page_table ? prm.page_table + static_cast<int64_t>(stream) * prm.pages.max_pages : nullptr;
+            prm.page_table && !(GENERIC && prm.rows_cache_before >= 0)
+                ? prm.page_table + static_cast<int64_t>(stream) * prm.pages.max_pages
+                : prm.page_table;
         sh_off[tid] = tile_offset(cache, prm.pages, table, (tile_lo + tid) * kTile, kvh, prm.status);
     }
 
@@ -171,7 +191,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
         const int32_t* table = prm.page_table;
         for (int item = wave; item < G + (owner ? 2 : 0); item += kDecodeWaves) {
             if (item < G) {
-                const int qh = kvh * G + item;
+                const int qh = hg * G + item;
                 const HeadPair r = norm_rope_head(prm.step_q[qh * kDim + lane], prm.step_q[qh * kDim + lane + 64],
                                                   prm.step_q_norm, prm.step_cos, prm.step_sin, prm.step_epsilon, lane);
                 sh_qrot[item][lane] = r.lo;
@@ -204,7 +224,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
     } else {
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            const int qh = kvh * G + g;
+            const int qh = hg * G + g;
             qv[g] = *reinterpret_cast<const uint4*>(
                 prm.query + (static_cast<int64_t>(stream) * prm.q_heads + qh) * kDim + col * 8);
         }
@@ -362,12 +382,12 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
             aa = fmaf(sh_acc[j][g][d], w, aa);
         }
         if (prm.max_splits == 1) {
-            const int qh = kvh * G + g;
+            const int qh = hg * G + g;
             prm.out[(static_cast<int64_t>(stream) * prm.q_heads + qh) * kDim + d] =
                 f2bf(ll > 0.0f ? aa / ll : 0.0f);
         } else {
             float* rec = prm.partial
-                + ((static_cast<int64_t>(stream) * gridDim.y + kvh) * prm.max_splits + split)
+                + ((static_cast<int64_t>(stream) * gridDim.y + hg) * prm.max_splits + split)
                       * partial_floats<G>();
             rec[g * kDim + d] = aa;
             if (d == 0) {
@@ -378,19 +398,19 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
     }
 }
 
-// Merge of the split partials of one (stream, kv head); also writes zeros for an empty
-// context.  grid (kv_heads, n_streams), block G*128.
-template <int G>
+// Merge of the split partials of one (stream, group of G heads); also writes zeros for an empty
+// context.  grid (head groups, n_streams), block G*128.
+template <int G, bool GENERIC>
 __global__ void decode_merge_kernel(DecodeParams prm) {
-    const int kvh = blockIdx.x;
+    const int hg = blockIdx.x;
     const int stream = blockIdx.y;
     const int g = threadIdx.x / kDim;
     const int d = threadIdx.x % kDim;
-    const int qh = kvh * G + g;
+    const int qh = hg * G + g;
     uint16_t* dst = prm.out + (static_cast<int64_t>(stream) * prm.q_heads + qh) * kDim + d;
 
     const float* base = prm.partial
-        + (static_cast<int64_t>(stream) * gridDim.x + kvh) * prm.max_splits * partial_floats<G>();
+        + (static_cast<int64_t>(stream) * gridDim.x + hg) * prm.max_splits * partial_floats<G>();
 
     // All loads of a round — the context length, the statistics of up to kMergeRound splits and
     // this thread's accumulator column of each — are issued before anything is consumed, so the
@@ -420,6 +440,8 @@ __global__ void decode_merge_kernel(DecodeParams prm) {
             if (prm.seq_lens) {
                 key_start = 0;
                 key_end = min(prm.seq_lens[stream], prm.max_seq_len);
+            } else if (GENERIC && prm.rows_cache_before >= 0) {
+                row_key_range(prm, stream, key_start, key_end);
             }
             if (key_end <= key_start) {
                 *dst = 0;
@@ -511,42 +533,54 @@ inline size_t decode_workspace_bytes(int n_streams, int q_heads, int kv_heads, i
 }
 
 template <int G, bool STREAMING>
-void launch_split(const DecodeParams& prm, const qm_kv_cache& cache, int n_streams, hipStream_t stream) {
-    const dim3 grid(prm.max_splits, cache.kv_heads, n_streams);
+int32_t launch_split(const DecodeParams& prm, const qm_kv_cache& cache, int n_streams, bool generic, hipStream_t stream) {
+    const dim3 grid(prm.max_splits, cache.kv_heads * prm.head_groups_per_kv, n_streams);
     if (prm.step_q) {
-        hipLaunchKernelGGL((decode_split_kernel<G, true, STREAMING>), grid, dim3(kDecodeThreads), 0, stream, prm, cache);
+        if (generic) return QM_ERR_GEOMETRY;   // the fused step is built for groups of 1, 2 and 4 heads
+        hipLaunchKernelGGL((decode_split_kernel<G, true, STREAMING, false>), grid, dim3(kDecodeThreads), 0, stream, prm, cache);
+    } else if (generic) {
+        hipLaunchKernelGGL((decode_split_kernel<G, false, STREAMING, true>), grid, dim3(kDecodeThreads), 0, stream, prm, cache);
     } else {
-        hipLaunchKernelGGL((decode_split_kernel<G, false, STREAMING>), grid, dim3(kDecodeThreads), 0, stream, prm, cache);
+        hipLaunchKernelGGL((decode_split_kernel<G, false, STREAMING, false>), grid, dim3(kDecodeThreads), 0, stream, prm, cache);
     }
+    return launch_status();
 }
 
 template <int G>
 int32_t launch_decode(const DecodeParams& prm, const qm_kv_cache& cache, int n_streams, bool streaming,
                       hipStream_t stream) {
-    if (streaming) launch_split<G, true>(prm, cache, n_streams, stream);
-    else launch_split<G, false>(prm, cache, n_streams, stream);
-    int32_t rc = launch_status();
+    const bool generic = prm.head_groups_per_kv > 1 || prm.rows_cache_before >= 0;
+    int32_t rc = streaming ? launch_split<G, true>(prm, cache, n_streams, generic, stream)
+                           : launch_split<G, false>(prm, cache, n_streams, generic, stream);
     if (rc != QM_OK) return rc;
     if (prm.max_splits > 1) {
-        hipLaunchKernelGGL(decode_merge_kernel<G>, dim3(cache.kv_heads, n_streams), dim3(G * kDim), 0,
-                           stream, prm);
+        const dim3 grid(cache.kv_heads * prm.head_groups_per_kv, n_streams);
+        if (generic) hipLaunchKernelGGL((decode_merge_kernel<G, true>), grid, dim3(G * kDim), 0, stream, prm);
+        else hipLaunchKernelGGL((decode_merge_kernel<G, false>), grid, dim3(G * kDim), 0, stream, prm);
         rc = launch_status();
     }
     return rc;
 }
 
+// Rows of one sequence as streams: what qm_attention_rows adds to a call.
+struct RowsOfOneSequence {
+    int cache_before;
+    int sliding_window;
+};
+
 int32_t decode_common(const uint16_t* query, const qm_kv_cache* cache, const int32_t* page_table,
                       int32_t max_pages, const int32_t* seq_lens, int32_t n_streams,
                       int32_t key_start, int32_t key_end, int32_t max_seq_len, uint16_t* out,
                       int32_t q_heads, float scale, void* workspace, size_t workspace_bytes,
-                      uint32_t* status_dev, void* hip_stream, const DecodeParams* step = nullptr) {
+                      uint32_t* status_dev, void* hip_stream, const DecodeParams* step = nullptr,
+                      const RowsOfOneSequence* rows = nullptr) {
     if ((!query && !step) || !out) return QM_ERR_NULL;
     int32_t rc = check_cache(cache, max_pages);
     if (rc != QM_OK) return rc;
     rc = check_group(q_heads, cache->kv_heads);
     if (rc != QM_OK) return rc;
     if ((reinterpret_cast<uintptr_t>(query) & 15)) return QM_ERR_GEOMETRY;
-    if (n_streams < 0 || n_streams > 65535 || cache->kv_heads > 65535) return QM_ERR_ARGUMENT;
+    if (n_streams < 0 || n_streams > 65535 || q_heads > 65535) return QM_ERR_ARGUMENT;
     if (max_seq_len < 0) return QM_ERR_ARGUMENT;
     if (max_seq_len > cache_capacity(cache, max_pages)) return QM_ERR_SLOT_RANGE;
     const int loads = option_value(QM_OPT_DECODE_STREAMING_LOADS);
@@ -573,6 +607,12 @@ int32_t decode_common(const uint16_t* query, const qm_kv_cache* cache, const int
     prm.max_splits = plan.max_splits;
     prm.q_heads = q_heads;
     prm.scale = scale;
+    // Heads per block: the largest instantiated G that divides the GQA group.
+    const int group = q_heads / cache->kv_heads;
+    const int heads_per_block = group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
+    prm.head_groups_per_kv = group / heads_per_block;
+    prm.rows_cache_before = rows ? rows->cache_before : -1;
+    prm.rows_window = rows ? rows->sliding_window : 0;
     prm.step_q = nullptr;
     if (step) {
         prm.step_q = step->step_q; prm.step_k = step->step_k; prm.step_v = step->step_v;
@@ -583,14 +623,14 @@ int32_t decode_common(const uint16_t* query, const qm_kv_cache* cache, const int
     }
 
     // Upper bound of the K and V bytes one call reads.
-    const int64_t context_bytes = static_cast<int64_t>(n_streams) * (seq_lens ? max_seq_len : key_end - key_start)
+    const int64_t context_bytes = (rows ? 1 : static_cast<int64_t>(n_streams)) * (seq_lens || rows ? max_seq_len : key_end - key_start)
                                 * cache->kv_heads * kDim * 2 * 2;
     bool streaming = context_bytes > kStreamingContextBytes;
     if (loads == 1) streaming = false;
     if (loads == 2) streaming = true;
 
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
-    switch (q_heads / cache->kv_heads) {
+    switch (heads_per_block) {
         case 1: return launch_decode<1>(prm, *cache, n_streams, streaming, s);
         case 2: return launch_decode<2>(prm, *cache, n_streams, streaming, s);
         case 4: return launch_decode<4>(prm, *cache, n_streams, streaming, s);
@@ -691,6 +731,29 @@ extern "C" int32_t qm_decode_step_fused(
     step.step_position = position; step.step_epsilon = epsilon;
     return qm::decode_common(nullptr, cache, page_table, max_pages, nullptr, 1, key_start, key_end, key_end,
                              context_out, q_heads, scale, workspace, workspace_bytes, status_dev, hip_stream, &step);
+}
+
+extern "C" size_t qm_attention_rows_workspace_bytes(int32_t query_length, int32_t q_heads, int32_t kv_heads,
+                                                    int32_t key_end) {
+    return qm_decode_workspace_bytes(query_length, q_heads, kv_heads, key_end);
+}
+
+extern "C" int32_t qm_attention_rows(
+    const uint16_t* query,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    uint16_t* context_out,
+    int32_t query_length, int32_t cache_before, int32_t q_heads, int32_t sliding_window, float scale,
+    void* workspace, size_t workspace_bytes, uint32_t* status_dev, void* hip_stream) {
+    if (query_length < 0 || cache_before < 0) return QM_ERR_ARGUMENT;
+    if (static_cast<int64_t>(cache_before) + query_length > INT32_MAX) return QM_ERR_SLOT_RANGE;
+    const int32_t key_end = cache_before + query_length;   // of the last row
+    if (cache && !page_table && max_pages > 0 && cache->page_size > 0 && query_length > 0
+        && (key_end - 1) / cache->page_size >= cache->n_pages)
+        return QM_ERR_SLOT_RANGE;
+    const qm::RowsOfOneSequence rows = {cache_before, sliding_window};
+    return qm::decode_common(query, cache, page_table, max_pages, nullptr, query_length, 0, 0, key_end,
+                             context_out, q_heads, scale, workspace, workspace_bytes, status_dev, hip_stream,
+                             nullptr, &rows);
 }
 
 extern "C" int32_t qm_decode_attention_ragged_static(

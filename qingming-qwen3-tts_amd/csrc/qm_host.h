@@ -36,8 +36,6 @@ inline int64_t cache_capacity(const qm_kv_cache* c, int32_t max_pages) {
 
 inline int32_t check_group(int32_t q_heads, int32_t kv_heads) {
     if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads) return QM_ERR_GEOMETRY;
-    const int g = q_heads / kv_heads;
-    if (g != 1 && g != 2 && g != 4) return QM_ERR_GEOMETRY;
     return QM_OK;
 }
 

@@ -42,13 +42,19 @@ int main() {
         qm_attn::launch_attention(fake, fake, fake, fake, 1, 64, 16, 8, 128, 64, -1, 0.088f, nullptr, 0, nullptr);
     });
     expect_throw("attention group", "geometry", [&] {
-        qm_attn::launch_attention(fake, fake, fake, fake, 1, 10, 24, 8, 128, 64, -1, 0.088f, nullptr, 0, nullptr);
+        qm_attn::launch_attention(fake, fake, fake, fake, 1, 10, 20, 8, 128, 64, -1, 0.088f, nullptr, 0, nullptr);
     });
     expect_throw("attention workspace", "workspace", [&] {
         qm_attn::launch_attention(fake, fake, fake, fake, 1, 8000, 16, 8, 128, 8206, -1, 0.088f, nullptr, 0, nullptr);
     });
-    expect_throw("chunked prefill unsupported", "cache_before", [&] {
-        qm_attn::launch_attention(fake, fake, fake, fake, 8, 5, 16, 8, 128, 64, -1, 0.088f, nullptr, 0, nullptr);
+    expect_throw("chunked prefill overflow", "cache overflow", [&] {
+        qm_attn::launch_attention(fake, fake, fake, fake, 8, 60, 16, 8, 128, 64, -1, 0.088f, nullptr, 0, nullptr);
+    });
+    expect_throw("chunked prefill workspace", "workspace", [&] {
+        qm_attn::launch_attention(fake, fake, fake, fake, 8, 1000, 16, 8, 128, 2048, -1, 0.088f, nullptr, 0, nullptr);
+    });
+    expect_throw("chunked prefill group", "geometry", [&] {
+        qm_attn::launch_attention(fake, fake, fake, fake, 8, 5, 20, 8, 128, 64, -1, 0.088f, nullptr, 0, nullptr);
     });
     expect_throw("scatter decode overflow", "cache overflow", [&] {
         qm_attn::scatter_decode_cache(fake, fake, fake, fake, 8, 128, 64, 64, nullptr);

@@ -50,7 +50,6 @@ def test_host_validation_without_device(qm):
     bad = _cache(qm, head_dim=64)
     assert lib.qm_qk_norm_rope_kv_append(fake, fake, fake, fake, fake, fake, fake, fake, C.byref(bad), fake, 4, 16, 0, 1e-6, None) == -2
     assert lib.qm_decode_attention(fake, C.byref(c), fake, 4, fake, 12, 0, -1, 0.1, None, 0, None) == -2
-    assert lib.qm_decode_attention(fake, C.byref(c), fake, 4, fake, 24, 0, -1, 0.1, None, 0, None) == -2   # group 3
     odd = _cache(qm, page_size=24)
     assert lib.qm_decode_attention(fake, C.byref(odd), fake, 4, fake, 16, 0, -1, 0.1, None, 0, None) == -2
     mis = _cache(qm, k=0x1008)

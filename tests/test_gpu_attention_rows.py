@@ -1,0 +1,185 @@
+"""GPU parity of qm_attention_rows: the rows of one sequence over its cache for any cache_before, sliding window and
+GQA group — the reference's generic attention branch (R17:17782-17813, kernel R17:15744-16006).
+
+Against the oracle's restatement of that kernel (online policy: the decode kernels' rounding; tolerance 1e-2 as for decode,
+and the reference chain with bf16(P) from 64 keys on), bit for bit against qm_decode_attention row by row, and against the
+matrix-core prefill where both serve a shape.  Cache slots past the last row hold NaN: they must never be read into a result.
+"""
+import numpy as np
+import pytest
+
+from qm_testlib import SCALE, PagedPool, max_abs_err, to_dev, to_u16
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def _workspace(qm, dev, rows, q_heads, kv_heads, key_end):
+    import torch
+    nbytes = qm.attention_rows_workspace_bytes(rows, q_heads, kv_heads, key_end)
+    return torch.empty(max(nbytes, 4) // 4 + 1, dtype=torch.float32, device=dev), nbytes
+
+
+def _flat(oracle, qm, dev, rows, before, seed, window=-1, q_heads=16, kv_heads=8, slack=3):
+    import torch
+    end = before + rows
+    max_cache = end + slack
+    q = oracle.normal_bf16((rows, q_heads, 128), seed)
+    kc = oracle.normal_bf16((kv_heads, max_cache, 128), seed + 1)
+    vc = oracle.normal_bf16((kv_heads, max_cache, 128), seed + 2)
+    kc[:, end:] = 0x7fc0
+    vc[:, end:] = 0x7fc0
+    want = {}
+    for policy in (0, 1):
+        o = np.zeros_like(q)
+        assert oracle.attention(q, oracle.flat_cache(kc, vc, kv_heads, max_cache), None, 1, o, rows, before, q_heads, window,
+                                SCALE, policy, 8) == 0
+        want[policy] = o
+    kd, vd, qd = to_dev(kc, dev), to_dev(vc, dev), to_dev(q, dev)
+    cache = qm.flat_cache(kd, vd, kv_heads, max_cache)
+    out = torch.full((rows, q_heads, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    ws, nbytes = _workspace(qm, dev, rows, q_heads, kv_heads, end)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    qm.attention_rows(qd, cache, None, 1, out, rows, before, q_heads, window, SCALE, ws, nbytes, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    return to_u16(out), want, (qd, kd, vd, cache, max_cache)
+
+
+@pytest.mark.parametrize("rows,before", [(2, 0), (5, 0), (64, 0), (3, 1), (7, 15), (16, 16), (33, 100), (64, 512), (64, 2048),
+                                         (130, 1000), (256, 37), (1, 300)])
+def test_rows_over_a_flat_cache(oracle, qm, dev, rows, before):
+    got, want, _ = _flat(oracle, qm, dev, rows, before, seed=1000 + rows + before)
+    assert max_abs_err(oracle, got, want[1]) <= TOL
+    first_long = max(0, 64 - before - 1)        # rows with at least 64 keys: also within the tolerance of the reference chain
+    if first_long < rows:
+        assert max_abs_err(oracle, got[first_long:], want[0][first_long:]) <= TOL
+    if before == 0:
+        # the first row attends one key: its output is V[0] exactly
+        assert np.array_equal(got[0], want[0][0])
+
+
+@pytest.mark.parametrize("rows,before,window", [(40, 0, 7), (40, 100, 16), (20, 90, 33), (64, 2048, 1024), (9, 50, 1), (9, 5, 500)])
+def test_rows_with_a_sliding_window(oracle, qm, dev, rows, before, window):
+    got, want, _ = _flat(oracle, qm, dev, rows, before, seed=2000 + rows + window, window=window)
+    assert max_abs_err(oracle, got, want[1]) <= TOL
+
+
+@pytest.mark.parametrize("q_heads,kv_heads", [(8, 8), (16, 4), (4, 2), (24, 8), (12, 2), (16, 2), (5, 1), (28, 4)])
+def test_rows_for_any_integral_group(oracle, qm, dev, q_heads, kv_heads):
+    """Groups 1, 2 and 4 have kernels of their own; 3, 5, 6, 7 and 8 run as several blocks per kv head."""
+    got, want, _ = _flat(oracle, qm, dev, 19, 130, seed=3000 + q_heads, q_heads=q_heads, kv_heads=kv_heads)
+    assert max_abs_err(oracle, got, want[1]) <= TOL
+    assert max_abs_err(oracle, got, want[0]) <= TOL
+
+
+@pytest.mark.parametrize("q_heads,kv_heads", [(24, 8), (16, 2)])
+def test_decode_for_any_integral_group(oracle, qm, dev, q_heads, kv_heads):
+    """The same split of a group over blocks serves the decode entry points."""
+    import torch
+    ctx, max_cache = 700, 704
+    q = oracle.normal_bf16((q_heads, 128), 41)
+    kc = oracle.normal_bf16((kv_heads, max_cache, 128), 42)
+    vc = oracle.normal_bf16((kv_heads, max_cache, 128), 43)
+    want = np.zeros_like(q)
+    assert oracle.attention(q, oracle.flat_cache(kc, vc, kv_heads, max_cache), None, 1, want, 1, ctx - 1, q_heads, -1, SCALE, 1,
+                            4) == 0
+    kd, vd = to_dev(kc, dev), to_dev(vc, dev)
+    out = torch.full((q_heads, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    nbytes = qm.decode_workspace_bytes(1, q_heads, kv_heads, ctx)
+    ws = torch.empty(nbytes // 4 + 1, dtype=torch.float32, device=dev)
+    qm.decode_attention(to_dev(q, dev), qm.flat_cache(kd, vd, kv_heads, max_cache), None, 1, out, q_heads, ctx - 1, -1, SCALE,
+                        ws, nbytes)
+    torch.cuda.synchronize()
+    assert max_abs_err(oracle, to_u16(out), want) <= TOL
+
+
+def test_every_row_carries_the_bits_of_the_decode_call(oracle, qm, dev):
+    import torch
+    rows, before, window = 21, 70, 48
+    got, _, (qd, kd, vd, cache, max_cache) = _flat(oracle, qm, dev, rows, before, seed=77, window=window)
+    nbytes = qm.decode_workspace_bytes(1, 16, 8, before + rows)
+    ws = torch.empty(nbytes // 4 + 1, dtype=torch.float32, device=dev)
+    one = torch.zeros((16, 128), dtype=torch.int16, device=dev)
+    for i in range(rows):
+        qm.decode_attention(qd[i], cache, None, 1, one, 16, before + i, window, SCALE, ws, nbytes)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_u16(one), got[i]), i
+
+
+def test_a_whole_prompt_agrees_with_the_matrix_core_prefill(oracle, qm, dev):
+    """cache_before 0, group 2: both operators serve the shape; they differ in the rounding of the probabilities only."""
+    import torch
+    rows = 200
+    got, want, (qd, kd, vd, cache, max_cache) = _flat(oracle, qm, dev, rows, 0, seed=88)
+    out = torch.full((rows, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.prefill_attention_causal(qd, kd, vd, out, None, None, 0, 1, rows, 16, 8, SCALE, kv_strides=(128, max_cache * 128, 0))
+    torch.cuda.synchronize()
+    assert max_abs_err(oracle, to_u16(out), want[1]) <= TOL
+    # each is within the tolerance of the oracle, so within twice that of the other — except where few keys make
+    # outputs large (the first rows), where one bf16 ulp of the output is what they may differ by
+    a = oracle.bf16_to_f32(got).astype(np.float64)
+    b = oracle.bf16_to_f32(to_u16(out)).astype(np.float64)
+    one_ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(a), 2.0 ** -20))) - 7)
+    assert np.all(np.abs(a - b) <= np.maximum(2 * one_ulp, 2 * TOL))
+
+
+def test_rows_over_a_paged_cache_in_chunks(oracle, qm, dev):
+    """A prompt continued in chunks over shuffled pages: scatter a chunk, attend it, three times; every chunk's rows equal
+    the oracle's over the cache as it stands, and the pages end up holding exactly the prompt."""
+    import torch
+    chunks = [40, 1, 87]
+    total = sum(chunks)
+    pool = PagedPool(oracle, [total], seed=9, fill=0x7fc0)
+    q = oracle.normal_bf16((total, 16, 128), 91)
+    k = oracle.normal_bf16((total, 8, 128), 92)
+    v = oracle.normal_bf16((total, 8, 128), 93)
+    kd, vd, cache_d, table_d = pool.device(qm, dev)
+    cache_o = pool.descriptor(oracle)
+    qd, kin, vin = to_dev(q, dev), to_dev(k, dev), to_dev(v, dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    done = 0
+    for n in chunks:
+        assert oracle.scatter_kv(k[done:done + n], v[done:done + n], cache_o, pool.page_table[0], pool.max_pages, n, done) == 0
+        want = np.zeros((n, 16, 128), dtype=np.uint16)
+        assert oracle.attention(q[done:done + n], cache_o, pool.page_table[0], pool.max_pages, want, n, done, 16, -1, SCALE, 1,
+                                8) == 0
+        qm.scatter_kv(kin[done:done + n], vin[done:done + n], cache_d, table_d, pool.max_pages, n, done, status)
+        ws, nbytes = _workspace(qm, dev, n, 16, 8, done + n)
+        out = torch.full((n, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+        qm.attention_rows(qd[done:done + n], cache_d, table_d, pool.max_pages, out, n, done, 16, -1, SCALE, ws, nbytes, status)
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0
+        assert max_abs_err(oracle, to_u16(out), want) <= TOL
+        done += n
+    assert np.array_equal(to_u16(kd), pool.k) and np.array_equal(to_u16(vd), pool.v)
+
+
+def test_bad_pages_are_flagged_and_arguments_checked(oracle, qm, dev):
+    import ctypes as C
+    import torch
+    pool = PagedPool(oracle, [64], seed=4)
+    kd, vd, cache_d, table_d = pool.device(qm, dev)
+    table = pool.page_table.copy()
+    table[0, 1] = pool.n_pages + 5
+    q = to_dev(oracle.normal_bf16((4, 16, 128), 5), dev)
+    out = torch.zeros((4, 16, 128), dtype=torch.int16, device=dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    ws, nbytes = _workspace(qm, dev, 4, 16, 8, 64)
+    qm.attention_rows(q, cache_d, to_dev(table, dev), pool.max_pages, out, 4, 60, 16, -1, SCALE, ws, nbytes, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) & qm.STATUS_BAD_PAGE
+    L = qm.lib()
+    call = lambda rows, before, heads, ws_ptr, ws_bytes, pages=pool.max_pages: L.qm_attention_rows(
+        q.data_ptr(), C.byref(cache_d), table_d.data_ptr(), pages, out.data_ptr(), rows, before, heads, -1, SCALE, ws_ptr,
+        ws_bytes, None, None)
+    assert call(0, 0, 16, None, 0) == 0                         # no rows: nothing to do
+    assert call(-1, 0, 16, None, 0) == -5 and call(4, -1, 16, None, 0) == -5
+    assert call(4, 61, 16, ws.data_ptr(), nbytes) == -3         # the last row would lie beyond the page table
+    assert call(4, 60, 12, ws.data_ptr(), nbytes) == -2         # 12 query heads over 8 kv heads
+    need = qm.attention_rows_workspace_bytes(4, 16, 8, 1024)
+    big = PagedPool(oracle, [1024], seed=6)
+    _, _, cache_b, table_b = big.device(qm, dev)
+    assert need > 0 and L.qm_attention_rows(q.data_ptr(), C.byref(cache_b), table_b.data_ptr(), big.max_pages, out.data_ptr(), 4,
+                                            1020, 16, -1, SCALE, None, 0, None, None) == -4
