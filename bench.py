@@ -905,6 +905,52 @@ class Prefill:
         return {"all": dt * self.batch}, err, "batch entry 0 of %d, time scaled by %d" % (self.batch, self.batch)
 
 
+class PrefillChunk:
+    """A prompt continued in chunks (the reference's generic attention branch with cache_before > 0): 256 rows at
+    position 2048 of one sequence over the reference's flat LayerCache, on the matrix cores or row by row."""
+    bound = "mfma"
+
+    def __init__(self, qm, dev, seed=46, rows=256, before=2048, by_rows=False):
+        import torch
+        self.qm, self.rows, self.before, self.by_rows = qm, rows, before, by_rows
+        self.name = "prefill_chunk_%d_rows_at_%d_flat_cache%s" % (rows, before, "_row_by_row" if by_rows else "")
+        syn = Synthetic(dev, seed)
+        self.max_cache = before + rows
+        self.q = syn.normal((rows, 16, 128))
+        self.k, self.v = syn.normal((8, self.max_cache, 128)), syn.normal((8, self.max_cache, 128))
+        self.out = torch.zeros_like(self.q)
+        self.cache = qm.flat_cache(self.k, self.v, 8, self.max_cache)
+        self.ws_bytes = qm.attention_rows_workspace_bytes(rows, 16, 8, self.max_cache)
+        self.ws = torch.empty(self.ws_bytes // 4 + 1, dtype=torch.float32, device=dev)
+        keys = sum(before + i + 1 for i in range(rows))
+        self.flops = 16 * keys * 128 * 2 * 2
+        self.bytes = 2 * rows * 16 * 128 * 2 + 2 * self.max_cache * 8 * 128 * 2     # Q + O, K + V read once
+
+    def step(self):
+        import torch
+        stream = torch.cuda.current_stream().cuda_stream
+        if self.by_rows:
+            self.qm.attention_rows(self.q, self.cache, None, 1, self.out, self.rows, self.before, 16, -1, SCALE, self.ws,
+                                   self.ws_bytes, None, stream)
+        else:
+            self.qm.prefill_attention_chunk(self.q, self.k, self.v, self.out, 1, self.rows, self.before, 16, 8, SCALE, stream,
+                                            (128, self.max_cache * 128, 0))
+
+    def cpu_baseline(self, oracle, threads):
+        """Sample: the first 32 rows."""
+        n = 32
+        q, k, v = _bits(self.q[:n]).copy(), _bits(self.k).copy(), _bits(self.v).copy()
+        out = np.zeros_like(q)
+        t0 = time.perf_counter()
+        rc = oracle.attention(q, oracle.flat_cache(k, v, 8, self.max_cache), None, 1, out, n, self.before, 16, -1, SCALE,
+                              oracle.POLICY_ONLINE, threads)
+        dt = time.perf_counter() - t0
+        assert rc == 0
+        err = float(np.max(np.abs(oracle.bf16_to_f32(out).astype(np.float64)
+                                  - oracle.bf16_to_f32(_bits(self.out[:n])).astype(np.float64))))
+        return {"all": dt * self.rows / n}, err, "first %d of %d rows, time scaled" % (n, self.rows)
+
+
 class PredictorLoop:
     """configs[4]: 256 frames x 5 layers, 16 steps each (context 1 -> 16), one launch."""
     name = "predictor_loop_256frames_5layers_16steps"
@@ -979,7 +1025,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
-    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "prefillfp32", "predictor", "predictorexact",
+    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "prefillfp32", "chunk", "chunkrows", "predictor", "predictorexact",
                                       "qkv", "layer", "layer1", "frame", "frame1", "linears", "linearsexact", "generate"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
@@ -1019,6 +1065,7 @@ def main():
                 "prefill": lambda: Prefill(qm, dev), "prefill1": lambda: Prefill(qm, dev, batch=1),
                 "prefill1split": lambda: Prefill(qm, dev, batch=1, split=True),
                 "prefillfp32": lambda: Prefill(qm, dev, score_rounding=0),
+                "chunk": lambda: PrefillChunk(qm, dev), "chunkrows": lambda: PrefillChunk(qm, dev, by_rows=True),
                 "predictor": lambda: PredictorLoop(qm, dev),
                 "predictorexact": lambda: PredictorLoop(qm, dev, kernel=1),
                 "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev), "layer1": lambda: TalkerLayerStep(qm, dev, chained=True),
@@ -1058,6 +1105,10 @@ def main():
             # one prompt, as the talker's prefill runs it: 128 blocks for 256 CUs; the key-split entry fills them
             ("cfg4b_causal_prefill_one_prompt_1024", lambda: Prefill(qm, dev, batch=1)),
             ("cfg4b_causal_prefill_one_prompt_1024_key_split", lambda: Prefill(qm, dev, batch=1, split=True)),
+            # a prompt continued in chunks: 256 rows at position 2048 (matrix cores; and row by row through the decode kernels,
+            # which also serves sliding windows, other GQA groups and paged caches)
+            ("cfg4c_prefill_chunk_256_rows_at_2048", lambda: PrefillChunk(qm, dev)),
+            ("cfg4c_prefill_chunk_256_rows_at_2048_row_by_row", lambda: PrefillChunk(qm, dev, by_rows=True)),
             ("cfg5_predictor_loop", lambda: PredictorLoop(qm, dev)),
             ("cfg5_predictor_loop_exact_chain", lambda: PredictorLoop(qm, dev, kernel=1)),
             ("cfg5_predictor_loop_cache_writeback", lambda: PredictorLoop(qm, dev, write_cache=True)),

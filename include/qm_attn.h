@@ -343,6 +343,27 @@ int32_t qm_prefill_attention_causal_split(
     void* hip_stream);
 
 /*
+ * The causal GQA prefill on bf16 MFMA for rows that CONTINUE a sequence (a prompt fed in chunks): replaces
+ * launch_attention with query_length > 1 and cache_before > 0 (R17:17782-17813, kernel talker_attention_kernel
+ * R17:15744-16006; cache_before == 0 is accepted too).  query, context_out [batch][rows][q_heads][128]; row i stands
+ * at position cache_before + i and attends keys 0 .. cache_before + i of its batch entry.  key, value hold the
+ * cache_before + rows keys of every batch entry — those of the rows themselves included, as after
+ * scatter_prefill_cache — addressed by element strides like qm_prefill_attention_causal's: the reference's LayerCache
+ * [kv_head][max_cache][128] is read in place with (128, max_cache*128, 0); all zero selects contiguous
+ * [batch][cache_before + rows][kv_heads][128].  Only q_heads == 2 * kv_heads, no sliding window, no page table
+ * (qm_attention_rows below serves those).  Rounding as qm_prefill_attention_causal (bf16 scores before and after
+ * scaling unless QM_OPT_PREFILL_SCORE_ROUNDING is 0, fp32 online softmax, bf16 P; P = hi + lo where a query tile's
+ * rows see fewer than 64 keys).  The uniform-waves kernel of qm_prefill_attention_causal with the query rows shifted:
+ * for cache_before == 0 it leaves that entry point's bits.
+ */
+int32_t qm_prefill_attention_chunk(
+    const uint16_t* query, const uint16_t* key, const uint16_t* value,
+    uint16_t* context_out,
+    int32_t batch, int32_t rows, int32_t cache_before, int32_t q_heads, int32_t kv_heads, float scale,
+    int64_t kv_stride_token, int64_t kv_stride_head, int64_t kv_stride_batch,
+    void* hip_stream);
+
+/*
  * Attention of query_length rows of ONE sequence over its cache, for every shape the two entry points
  * above do not serve: replaces NativeTalkerEngine::launch_attention in its generic branch
  * (R17:17782-17813, kernel talker_attention_kernel R17:15744-16006) for any cache_before >= 0 (a prompt
@@ -355,8 +376,8 @@ int32_t qm_prefill_attention_causal_split(
  * page_table [max_pages] of that sequence, or NULL for pages in pool order (the flat LayerCache).
  * Every row runs as one stream of the split-K decode kernels: row i carries the bits
  * qm_decode_attention gives for cache_before + i, and the rounding is that entry point's.  K and V are
- * read once per row (from the caches after the first), so for a whole prompt from an empty cache with
- * group 2 qm_prefill_attention_causal is the faster call by an order of magnitude.
+ * read once per row (from the caches after the first): where they serve the shape (group 2, no window, keys
+ * addressable by strides) qm_prefill_attention_causal and qm_prefill_attention_chunk are faster by an order of magnitude.
  * Workspace: qm_attention_rows_workspace_bytes(query_length, q_heads, kv_heads, cache_before + query_length).
  * query_length <= 65535.  status_dev (optional): QM_STATUS_BAD_PAGE for page-table entries out of range.
  */

@@ -84,11 +84,11 @@ inline std::size_t attention_workspace_bytes(int q_heads, int kv_heads, int max_
 
 // ≙ NativeTalkerEngine::launch_attention (R17:17723-17814).  query_length == 1 is decode over
 // keys [key_start, cache_before + 1).  query_length > 1 attends the rows that scatter_prefill_cache has
-// already placed in the cache: a whole prompt from an empty cache with two query heads per kv head, as in
-// NativeTalkerEngine::prefill (R17:16710-16717), runs on the matrix cores; every other case of the
-// reference's generic kernel (cache_before > 0, a sliding window, another group) runs row by row.
+// already placed in the cache: with two query heads per kv head and no sliding window on the matrix cores (a whole
+// prompt from an empty cache, as in NativeTalkerEngine::prefill R17:16710-16717, or rows that continue a sequence);
+// every other case of the reference's generic kernel (a sliding window, another group) row by row.
 // The reference sizes dynamic LDS from the context; here the caller passes a workspace sized by
-// attention_workspace_bytes instead (the matrix-core case needs none).
+// attention_workspace_bytes instead (the matrix-core cases need none).
 inline void launch_attention(
     const std::uint16_t* query, std::uint16_t* key_cache, std::uint16_t* value_cache,
     std::uint16_t* context, int query_length, int cache_before,
@@ -102,6 +102,12 @@ inline void launch_attention(
         return;
     }
     if (cache_before + query_length > max_cache) throw std::runtime_error("Talker prefill cache overflow.");
+    if (sliding_window <= 0 && q_heads == 2 * kv_heads && cache_before != 0) {
+        check(qm_prefill_attention_chunk(query, key_cache, value_cache, context, 1, query_length, cache_before, q_heads,
+                                         kv_heads, scale, head_dim, static_cast<std::int64_t>(max_cache) * head_dim, 0, stream),
+              "Talker generic fused attention launch");
+        return;
+    }
     if (cache_before != 0 || sliding_window > 0 || q_heads != 2 * kv_heads) {
         check(qm_attention_rows(query, &c, nullptr, 1, context, query_length, cache_before, q_heads, sliding_window,
                                 scale, workspace, workspace_bytes, nullptr, stream),

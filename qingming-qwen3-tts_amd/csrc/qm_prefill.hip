@@ -94,6 +94,10 @@ struct PrefillParams {
     int* split_tickets;          // [pair][split query tile][8]: (epoch << 4 | arrivals), then per part the epoch of its published record
     int split_epoch;             // 1 .. 2^27 - 1, another value for every launch that splits
     float scale;
+    // (chunk kernel) the rows continue a sequence: row i stands at position cache_before + i and attends keys
+    // 0 .. cache_before + i of the key_count = cache_before + seq keys that k and v hold
+    int cache_before;
+    int key_count;
 };
 
 struct PfStage {
@@ -130,7 +134,8 @@ __device__ __forceinline__ float halves_sum(float v) {
 template <int N> using int_c = std::integral_constant<int, N>;
 template <bool B> using bool_c = std::integral_constant<bool, B>;
 
-template <bool PRECISE, bool ROUND>
+// CHUNK: the query rows stand at positions cache_before + row (prefill_chunk_kernel); otherwise at their row.
+template <bool PRECISE, bool ROUND, bool CHUNK = false>
 __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_kv_cache& cache,
                                              unsigned char* pf_smem, int qt, int pair) {
     PfStage* st = reinterpret_cast<PfStage*>(pf_smem);
@@ -144,12 +149,15 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     const int b = pair / prm.kv_heads;
     const int kvh = pair % prm.kv_heads;
     const int S = prm.seq;
+    const int SK = CHUNK ? prm.key_count : S;        // keys that k and v hold
+    const int shift = CHUNK ? prm.cache_before : 0;  // position of query row 0
     const int q_heads = 2 * prm.kv_heads;
 
     const int q0 = qt * kBM;
     const int my_row = q0 + 16 * wave + (col & 15);   // query row of this lane's column
+    const int my_pos = my_row + shift;                // the last key it attends
     const int my_head = 2 * kvh + (col >> 4);
-    const int wave_last_row = q0 + 16 * wave + 15;
+    const int wave_last_row = q0 + 16 * wave + 15 + shift;   // as a position
 
     // ---- Q fragments (B operand): dims 16*kb + 8*grp .. +7 of this lane's column ----------------
     bf16x8_t qf[8];
@@ -199,7 +207,7 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     const uint32_t v_lane_off = static_cast<uint32_t>(4 * v_kg * kv_row32);
     auto load_tile = [&](int tile) {
         const int key0 = tile * kBN;
-        if (key0 + kBN <= S) {
+        if (key0 + kBN <= SK) {
             const uint16_t* kt = k_src + static_cast<uint32_t>(key0 * kv_row32);
             const uint16_t* vt = v_src + static_cast<uint32_t>(key0 * kv_row32);
             each_stage([&](uint4& kk, uint4& vv, int i) {
@@ -210,9 +218,9 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
             // A key at or beyond S is redirected to the last key; such keys only occur in the
             // diagonal tile of the last query tile, where the causal mask removes them.
             each_stage([&](uint4& kk, uint4& vv, int i) {
-                const int key = min(key0 + (tid >> 4) + 16 * i, S - 1);
+                const int key = min(key0 + (tid >> 4) + 16 * i, SK - 1);
                 kk = *reinterpret_cast<const uint4*>(k_src + static_cast<uint32_t>(key * kv_row32));
-                const int vkey = min(key0 + 4 * v_kg + i, S - 1);
+                const int vkey = min(key0 + 4 * v_kg + i, SK - 1);
                 vv = *reinterpret_cast<const uint4*>(v_src + static_cast<uint32_t>(vkey * kv_row32));
             });
         }
@@ -350,7 +358,7 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     // Score roundings and causal mask in place; returns the column maximum.
     auto scores = [&](f32x16_t& s, auto masked, int key_base) -> float {
         // accumulator register r of lane group grp is key key_base + 8*(r/4) + 4*grp + r%4
-        const int lim = my_row - key_base - 4 * grp;
+        const int lim = my_pos - key_base - 4 * grp;
         float mx = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
@@ -433,19 +441,44 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     store_tile(0);
     __syncthreads();
 
-    if (!PRECISE) {
-        for (int t = 0; t < qt; ++t) {
+    if (CHUNK) {
+        // Key tiles every row of the query tile sees whole, then the one or two that the causal mask cuts
+        // (two when the tile's first position is not a multiple of 64); the last tile always takes the masked
+        // path, where keys beyond key_count go.
+        const int last_tile = min(q0 + shift + kBM - 1, SK - 1) / kBN;
+        const int whole = PRECISE ? 0 : min((q0 + shift + 1) / kBN, last_tile);
+        for (int t = 0; t < whole; ++t) {
             const int stage = t & 1;
             load_tile(t + 1);
             chunk(stage, int_c<0>{}, bool_c<false>{}, 0);
             chunk(stage, int_c<1>{}, bool_c<false>{}, 0);
-            if (prm.has_cache && t + 1 == qt) write_pages(qt);
             store_tile(stage ^ 1);
             __syncthreads();
         }
+        for (int t = whole;; ++t) {
+            const int stage = t & 1;
+            if (t < last_tile) load_tile(t + 1);
+            chunk(stage, int_c<0>{}, bool_c<true>{}, t * kBN);
+            chunk(stage, int_c<1>{}, bool_c<true>{}, t * kBN + 32);
+            if (t == last_tile) break;
+            store_tile(stage ^ 1);
+            __syncthreads();
+        }
+    } else {
+        if (!PRECISE) {
+            for (int t = 0; t < qt; ++t) {
+                const int stage = t & 1;
+                load_tile(t + 1);
+                chunk(stage, int_c<0>{}, bool_c<false>{}, 0);
+                chunk(stage, int_c<1>{}, bool_c<false>{}, 0);
+                if (prm.has_cache && t + 1 == qt) write_pages(qt);
+                store_tile(stage ^ 1);
+                __syncthreads();
+            }
+        }
+        chunk(qt & 1, int_c<0>{}, bool_c<true>{}, qt * kBN);
+        chunk(qt & 1, int_c<1>{}, bool_c<true>{}, qt * kBN + 32);
     }
-    chunk(qt & 1, int_c<0>{}, bool_c<true>{}, qt * kBN);
-    chunk(qt & 1, int_c<1>{}, bool_c<true>{}, qt * kBN + 32);
     __syncthreads();   // the stages become the output staging area
 
     // ---- normalise, stage through LDS, write 16 bytes per lane -------------------------------------
@@ -491,6 +524,24 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_causal_kernel(PrefillPa
         prefill_body<true, ROUND>(prm, cache, pf_smem, 0, pair);
     } else {
         prefill_body<false, ROUND>(prm, cache, pf_smem, qt, pair);
+    }
+}
+
+
+// The rows of a sequence continued at position cache_before (R17:17782-17813 with cache_before > 0), over keys
+// and values read in place: grid and blocks as above.  A query tile none of whose rows sees a whole key tile takes
+// the split-precision P path (rows with few keys).
+template <bool ROUND>
+__global__ __launch_bounds__(kPfThreads, 2) void prefill_chunk_kernel(PrefillParams prm, qm_kv_cache cache) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char pf_smem[];
+    const int pairs = prm.batch * prm.kv_heads;
+    const int bid = blockIdx.x;
+    const int qt = prm.n_qtiles - 1 - bid / pairs;
+    const int pair = bid % pairs;
+    if ((qt * kBM + prm.cache_before + 1) / kBN == 0) {
+        prefill_body<true, ROUND, true>(prm, cache, pf_smem, qt, pair);
+    } else {
+        prefill_body<false, ROUND, true>(prm, cache, pf_smem, qt, pair);
     }
 }
 
@@ -1483,6 +1534,7 @@ static int32_t prefill_attention_entry(
     prm.batch = batch; prm.seq = seq; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
     prm.heavy_groups = n_qtiles;
     prm.split_chunk = 0; prm.split_slots = 0; prm.split_partials = nullptr; prm.split_tickets = nullptr; prm.split_epoch = 0;
+    prm.cache_before = 0; prm.key_count = seq;
 
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     const bool round_scores = option_value(QM_OPT_PREFILL_SCORE_ROUNDING) != 0;
@@ -1553,4 +1605,54 @@ extern "C" int32_t qm_prefill_attention_causal_split(
     return prefill_attention_entry(query, key, value, context_out, cache, page_table, max_pages, batch, seq, q_heads,
                                    kv_heads, scale, kv_stride_token, kv_stride_head, kv_stride_batch, workspace,
                                    workspace_bytes, status_dev, hip_stream);
+}
+
+extern "C" int32_t qm_prefill_attention_chunk(
+    const uint16_t* query, const uint16_t* key, const uint16_t* value,
+    uint16_t* context_out,
+    int32_t batch, int32_t rows, int32_t cache_before, int32_t q_heads, int32_t kv_heads, float scale,
+    int64_t kv_stride_token, int64_t kv_stride_head, int64_t kv_stride_batch,
+    void* hip_stream) {
+    using namespace qm;
+    if (batch < 0 || rows < 0 || cache_before < 0) return QM_ERR_ARGUMENT;
+    const int64_t key_count = static_cast<int64_t>(cache_before) + rows;
+    if (kv_stride_token == 0 && kv_stride_head == 0 && kv_stride_batch == 0) {
+        kv_stride_token = static_cast<int64_t>(kv_heads) * kDim;     // [batch][key_count][kv_heads][128]
+        kv_stride_head = kDim;
+        kv_stride_batch = key_count * kv_heads * kDim;
+    }
+    if (kv_stride_token < kDim || kv_stride_head < 0 || kv_stride_batch < 0
+        || ((kv_stride_token | kv_stride_head | kv_stride_batch) & 7))
+        return QM_ERR_GEOMETRY;
+    if (key_count * kv_stride_token >= (1LL << 31)) return QM_ERR_ARGUMENT;
+    if (!query || !key || !value || !context_out) return QM_ERR_NULL;
+    if (kv_heads <= 0 || q_heads != 2 * kv_heads) return QM_ERR_GEOMETRY;   // GQA pair on the MFMA columns
+    const uintptr_t align = reinterpret_cast<uintptr_t>(query) | reinterpret_cast<uintptr_t>(key)
+                          | reinterpret_cast<uintptr_t>(value) | reinterpret_cast<uintptr_t>(context_out);
+    if (align & 15) return QM_ERR_GEOMETRY;
+    if (batch == 0 || rows == 0) return QM_OK;
+    const int n_qtiles = (rows + kBM - 1) / kBM;
+    const int64_t pairs = static_cast<int64_t>(batch) * kv_heads;
+    if (pairs * n_qtiles > 0x7fffffffLL) return QM_ERR_ARGUMENT;
+
+    PrefillParams prm = {};
+    prm.q = query; prm.k = key; prm.v = value; prm.out = context_out;
+    prm.pages = make_page_map(16, 1);
+    prm.kv_stride_token = kv_stride_token; prm.kv_stride_head = kv_stride_head; prm.kv_stride_batch = kv_stride_batch;
+    prm.batch = batch; prm.seq = rows; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
+    prm.heavy_groups = n_qtiles;
+    prm.cache_before = cache_before; prm.key_count = static_cast<int>(key_count);
+
+    const bool round_scores = option_value(QM_OPT_PREFILL_SCORE_ROUNDING) != 0;
+    if (!round_scores && !(scale > 0.0f)) return QM_ERR_ARGUMENT;   // the scale is folded into the exponent there
+    const size_t smem = sizeof(PfStage) * kPfStages;
+    const auto kernel = round_scores ? prefill_chunk_kernel<true> : prefill_chunk_kernel<false>;
+    static std::atomic<bool> lds_raised[2][kMaxDevices];
+    const int32_t rc_lds = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), static_cast<int>(smem),
+                                              lds_raised[round_scores ? 1 : 0]);
+    if (rc_lds != QM_OK) return rc_lds;
+    const qm_kv_cache none = {};
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(pairs * n_qtiles)), dim3(kPfThreads), smem,
+                       static_cast<hipStream_t>(hip_stream), prm, none);
+    return launch_status();
 }

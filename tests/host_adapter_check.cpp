@@ -50,8 +50,8 @@ int main() {
     expect_throw("chunked prefill overflow", "cache overflow", [&] {
         qm_attn::launch_attention(fake, fake, fake, fake, 8, 60, 16, 8, 128, 64, -1, 0.088f, nullptr, 0, nullptr);
     });
-    expect_throw("chunked prefill workspace", "workspace", [&] {
-        qm_attn::launch_attention(fake, fake, fake, fake, 8, 1000, 16, 8, 128, 2048, -1, 0.088f, nullptr, 0, nullptr);
+    expect_throw("windowed rows workspace", "workspace", [&] {
+        qm_attn::launch_attention(fake, fake, fake, fake, 8, 1000, 16, 8, 128, 2048, 512, 0.088f, nullptr, 0, nullptr);
     });
     expect_throw("chunked prefill group", "geometry", [&] {
         qm_attn::launch_attention(fake, fake, fake, fake, 8, 5, 20, 8, 128, 64, -1, 0.088f, nullptr, 0, nullptr);

@@ -183,3 +183,115 @@ def test_bad_pages_are_flagged_and_arguments_checked(oracle, qm, dev):
     _, _, cache_b, table_b = big.device(qm, dev)
     assert need > 0 and L.qm_attention_rows(q.data_ptr(), C.byref(cache_b), table_b.data_ptr(), big.max_pages, out.data_ptr(), 4,
                                             1020, 16, -1, SCALE, None, 0, None, None) == -4
+
+
+# ---- qm_prefill_attention_chunk: the same rows on the matrix cores (group 2, no window, keys addressed by strides) ----
+
+def _chunk(oracle, qm, dev, rows, before, seed, batch=1, slack=5):
+    import torch
+    end = before + rows
+    max_cache = end + slack
+    q = oracle.normal_bf16((batch, rows, 16, 128), seed)
+    kc = oracle.normal_bf16((batch, 8, max_cache, 128), seed + 1)
+    vc = oracle.normal_bf16((batch, 8, max_cache, 128), seed + 2)
+    kc[:, :, end:] = 0x7fc0
+    vc[:, :, end:] = 0x7fc0
+    want = {0: np.zeros_like(q), 1: np.zeros_like(q)}
+    for policy in (0, 1):
+        for b in range(batch):
+            assert oracle.attention(q[b], oracle.flat_cache(kc[b], vc[b], 8, max_cache), None, 1, want[policy][b], rows, before,
+                                    16, -1, SCALE, policy, 8) == 0
+    qd, kd, vd = to_dev(q, dev), to_dev(kc, dev), to_dev(vc, dev)
+    out = torch.full((batch, rows, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    qm.prefill_attention_chunk(qd, kd, vd, out, batch, rows, before, 16, 8, SCALE,
+                               kv_strides=(128, max_cache * 128, 8 * max_cache * 128))
+    torch.cuda.synchronize()
+    return to_u16(out), want, (qd, kd, vd, max_cache)
+
+
+def _within(oracle, got, want, tol=TOL):
+    """Within the tolerance, or — where few keys make an output large — within one bf16 ulp of it."""
+    a = oracle.bf16_to_f32(got).astype(np.float64)
+    b = oracle.bf16_to_f32(want).astype(np.float64)
+    one_ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(b), 2.0 ** -20))) - 7)
+    return bool(np.all(np.abs(a - b) <= np.maximum(one_ulp, tol)))
+
+
+@pytest.mark.parametrize("rows,before", [(1, 0), (5, 0), (64, 0), (200, 0), (1, 1), (3, 1), (7, 15), (64, 63), (64, 64), (65, 65),
+                                         (16, 100), (130, 100), (64, 512), (100, 1000), (64, 2048), (256, 37), (300, 700),
+                                         (2, 62), (63, 1), (1, 127), (1, 128)])
+def test_chunk_on_the_matrix_cores(oracle, qm, dev, rows, before):
+    got, want, _ = _chunk(oracle, qm, dev, rows, before, seed=5000 + 7 * rows + before)
+    assert _within(oracle, got, want[1])
+    first_long = max(0, 64 - before - 1)        # rows with at least 64 keys: also the reference chain with its bf16(P)
+    if first_long < rows:
+        assert max_abs_err(oracle, got[:, first_long:], want[0][:, first_long:]) <= TOL
+    if before == 0:
+        assert np.array_equal(got[0, 0], want[0][0, 0])     # one key: V[0] exactly
+
+
+def test_chunk_of_a_batch_and_contiguous_keys(oracle, qm, dev):
+    import torch
+    got, want, _ = _chunk(oracle, qm, dev, 70, 90, seed=6000, batch=3)
+    assert _within(oracle, got, want[1])
+    # contiguous [batch][keys][kv_heads][128] with all strides zero
+    batch, rows, before = 2, 33, 50
+    end = before + rows
+    q = oracle.normal_bf16((batch, rows, 16, 128), 6100)
+    k = oracle.normal_bf16((batch, end, 8, 128), 6101)
+    v = oracle.normal_bf16((batch, end, 8, 128), 6102)
+    want2 = np.zeros_like(q)
+    for b in range(batch):
+        kc = np.ascontiguousarray(k[b].transpose(1, 0, 2))
+        vc = np.ascontiguousarray(v[b].transpose(1, 0, 2))
+        assert oracle.attention(q[b], oracle.flat_cache(kc, vc, 8, end), None, 1, want2[b], rows, before, 16, -1, SCALE, 1, 8) == 0
+    out = torch.zeros((batch, rows, 16, 128), dtype=torch.int16, device=dev)
+    qm.prefill_attention_chunk(to_dev(q, dev), to_dev(k, dev), to_dev(v, dev), out, batch, rows, before, 16, 8, SCALE)
+    torch.cuda.synchronize()
+    assert _within(oracle, to_u16(out), want2)
+
+
+def test_chunk_from_an_empty_cache_carries_the_prefill_bits(oracle, qm, dev):
+    """cache_before 0 is the whole-prompt prefill: the same bits as qm_prefill_attention_causal, by either of its kernels."""
+    import torch
+    for rows in (1, 64, 100, 333):
+        got, _, (qd, kd, vd, max_cache) = _chunk(oracle, qm, dev, rows, 0, seed=6200 + rows)
+        for kernel in (0, 1):
+            out = torch.zeros((1, rows, 16, 128), dtype=torch.int16, device=dev)
+            qm.set_option(qm.OPT_PREFILL_KERNEL, kernel)
+            try:
+                qm.prefill_attention_causal(qd, kd, vd, out, None, None, 0, 1, rows, 16, 8, SCALE,
+                                            kv_strides=(128, max_cache * 128, 0))
+                torch.cuda.synchronize()
+            finally:
+                qm.set_option(qm.OPT_PREFILL_KERNEL, 0)
+            assert np.array_equal(to_u16(out), got), (rows, kernel)
+
+
+def test_chunk_agrees_with_the_rows_of_the_decode_kernels(oracle, qm, dev):
+    import torch
+    rows, before = 90, 333
+    got, want, (qd, kd, vd, max_cache) = _chunk(oracle, qm, dev, rows, before, seed=6300)
+    cache = qm.flat_cache(kd[0], vd[0], 8, max_cache)
+    ws, nbytes = _workspace(qm, dev, rows, 16, 8, before + rows)
+    out = torch.zeros((rows, 16, 128), dtype=torch.int16, device=dev)
+    qm.attention_rows(qd[0], cache, None, 1, out, rows, before, 16, -1, SCALE, ws, nbytes, None)
+    torch.cuda.synchronize()
+    a = oracle.bf16_to_f32(got[0]).astype(np.float64)
+    b = oracle.bf16_to_f32(to_u16(out)).astype(np.float64)
+    assert np.max(np.abs(a - b)) <= 2 * TOL
+
+
+def test_chunk_argument_errors(qm, dev):
+    import ctypes as C
+    import torch
+    t = torch.zeros(4 * 16 * 128 * 80, dtype=torch.int16, device=dev)
+    p = t.data_ptr()
+    call = lambda rows, before, heads=16, kv=8, st=(0, 0, 0), q=p: qm.lib().qm_prefill_attention_chunk(
+        q, p, p, p, 1, rows, before, heads, kv, SCALE, st[0], st[1], st[2], None)
+    assert call(0, 5) == 0
+    assert call(-1, 0) == -5 and call(4, -1) == -5
+    assert call(4, 5, heads=8) == -2 and call(4, 5, st=(64, 128, 0)) == -2 and call(4, 5, st=(132, 128, 0)) == -2
+    assert call(4, 5, q=p + 2) == -2
+    assert call(4, 2 ** 24, st=(128, 2 ** 31, 0)) == -5           # keys beyond 32-bit element offsets
+    assert qm.lib().qm_prefill_attention_chunk(None, p, p, p, 1, 4, 5, 16, 8, SCALE, 0, 0, 0, None) == -1
