@@ -910,18 +910,20 @@ class PrefillChunk:
     position 2048 of one sequence over the reference's flat LayerCache, on the matrix cores or row by row."""
     bound = "mfma"
 
-    def __init__(self, qm, dev, seed=46, rows=256, before=2048, by_rows=False):
+    def __init__(self, qm, dev, seed=46, rows=256, before=2048, by_rows=False, split=True):
         import torch
         self.qm, self.rows, self.before, self.by_rows = qm, rows, before, by_rows
-        self.name = "prefill_chunk_%d_rows_at_%d_flat_cache%s" % (rows, before, "_row_by_row" if by_rows else "")
+        self.name = "prefill_chunk_%d_rows_at_%d_flat_cache%s" % (rows, before, "_row_by_row" if by_rows else
+                                                                  "" if split else "_one_block_per_query_tile")
         syn = Synthetic(dev, seed)
         self.max_cache = before + rows
         self.q = syn.normal((rows, 16, 128))
         self.k, self.v = syn.normal((8, self.max_cache, 128)), syn.normal((8, self.max_cache, 128))
         self.out = torch.zeros_like(self.q)
         self.cache = qm.flat_cache(self.k, self.v, 8, self.max_cache)
-        self.ws_bytes = qm.attention_rows_workspace_bytes(rows, 16, 8, self.max_cache)
-        self.ws = torch.empty(self.ws_bytes // 4 + 1, dtype=torch.float32, device=dev)
+        self.ws_bytes = qm.attention_rows_workspace_bytes(rows, 16, 8, self.max_cache) if by_rows else \
+            qm.prefill_chunk_workspace_bytes(1, rows, before, 8) if split else 0
+        self.ws = torch.empty(self.ws_bytes // 4 + 64, dtype=torch.float32, device=dev)
         keys = sum(before + i + 1 for i in range(rows))
         self.flops = 16 * keys * 128 * 2 * 2
         self.bytes = 2 * rows * 16 * 128 * 2 + 2 * self.max_cache * 8 * 128 * 2     # Q + O, K + V read once
@@ -934,7 +936,7 @@ class PrefillChunk:
                                    self.ws_bytes, None, stream)
         else:
             self.qm.prefill_attention_chunk(self.q, self.k, self.v, self.out, 1, self.rows, self.before, 16, 8, SCALE, stream,
-                                            (128, self.max_cache * 128, 0))
+                                            (128, self.max_cache * 128, 0), self.ws if self.ws_bytes else None, self.ws_bytes)
 
     def cpu_baseline(self, oracle, threads):
         """Sample: the first 32 rows."""
@@ -1025,7 +1027,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
-    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "prefillfp32", "chunk", "chunkrows", "predictor", "predictorexact",
+    ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "prefillfp32", "chunk", "chunkwhole", "chunkrows", "predictor", "predictorexact",
                                       "qkv", "layer", "layer1", "frame", "frame1", "linears", "linearsexact", "generate"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
@@ -1065,7 +1067,7 @@ def main():
                 "prefill": lambda: Prefill(qm, dev), "prefill1": lambda: Prefill(qm, dev, batch=1),
                 "prefill1split": lambda: Prefill(qm, dev, batch=1, split=True),
                 "prefillfp32": lambda: Prefill(qm, dev, score_rounding=0),
-                "chunk": lambda: PrefillChunk(qm, dev), "chunkrows": lambda: PrefillChunk(qm, dev, by_rows=True),
+                "chunk": lambda: PrefillChunk(qm, dev), "chunkwhole": lambda: PrefillChunk(qm, dev, split=False), "chunkrows": lambda: PrefillChunk(qm, dev, by_rows=True),
                 "predictor": lambda: PredictorLoop(qm, dev),
                 "predictorexact": lambda: PredictorLoop(qm, dev, kernel=1),
                 "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev), "layer1": lambda: TalkerLayerStep(qm, dev, chained=True),
@@ -1108,6 +1110,7 @@ def main():
             # a prompt continued in chunks: 256 rows at position 2048 (matrix cores; and row by row through the decode kernels,
             # which also serves sliding windows, other GQA groups and paged caches)
             ("cfg4c_prefill_chunk_256_rows_at_2048", lambda: PrefillChunk(qm, dev)),
+            ("cfg4c_prefill_chunk_256_rows_at_2048_one_block_per_query_tile", lambda: PrefillChunk(qm, dev, split=False)),
             ("cfg4c_prefill_chunk_256_rows_at_2048_row_by_row", lambda: PrefillChunk(qm, dev, by_rows=True)),
             ("cfg5_predictor_loop", lambda: PredictorLoop(qm, dev)),
             ("cfg5_predictor_loop_exact_chain", lambda: PredictorLoop(qm, dev, kernel=1)),

@@ -354,13 +354,21 @@ int32_t qm_prefill_attention_causal_split(
  * (qm_attention_rows below serves those).  Rounding as qm_prefill_attention_causal (bf16 scores before and after
  * scaling unless QM_OPT_PREFILL_SCORE_ROUNDING is 0, fp32 online softmax, bf16 P; P = hi + lo where a query tile's
  * rows see fewer than 64 keys).  The uniform-waves kernel of qm_prefill_attention_causal with the query rows shifted:
- * for cache_before == 0 it leaves that entry point's bits.
+ * for cache_before == 0 and no workspace it leaves that entry point's bits.
+ * workspace (optional, 256-byte aligned; nothing to initialise): a chunk is few rows over many keys, so its grid of
+ * batch * kv_heads * ceil(rows / 64) blocks can leave most compute units idle.  With a workspace of
+ * qm_prefill_chunk_workspace_bytes (for the current device; 0 when the shape would not split) the key tiles of a query
+ * tile are handed to up to 16 blocks in runs of at least four, whose unnormalised results a second launch combines in
+ * run order: results then differ from the unsplit call in the association of the sums only (within the operator's
+ * tolerance, not bit-identical) and do not depend on timing.  Too small for the shape: QM_ERR_WORKSPACE.
  */
+int64_t qm_prefill_chunk_workspace_bytes(int32_t batch, int32_t rows, int32_t cache_before, int32_t kv_heads);
 int32_t qm_prefill_attention_chunk(
     const uint16_t* query, const uint16_t* key, const uint16_t* value,
     uint16_t* context_out,
     int32_t batch, int32_t rows, int32_t cache_before, int32_t q_heads, int32_t kv_heads, float scale,
     int64_t kv_stride_token, int64_t kv_stride_head, int64_t kv_stride_batch,
+    void* workspace, int64_t workspace_bytes,
     void* hip_stream);
 
 /*

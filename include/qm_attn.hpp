@@ -103,8 +103,13 @@ inline void launch_attention(
     }
     if (cache_before + query_length > max_cache) throw std::runtime_error("Talker prefill cache overflow.");
     if (sliding_window <= 0 && q_heads == 2 * kv_heads && cache_before != 0) {
+        // (the caller's workspace lets the keys be shared between blocks, if it is large enough for that)
+        const std::int64_t split = qm_prefill_chunk_workspace_bytes(1, query_length, cache_before, kv_heads);
+        const bool fits = split > 0 && workspace && static_cast<std::int64_t>(workspace_bytes) >= split
+                       && (reinterpret_cast<std::uintptr_t>(workspace) & 255) == 0;
         check(qm_prefill_attention_chunk(query, key_cache, value_cache, context, 1, query_length, cache_before, q_heads,
-                                         kv_heads, scale, head_dim, static_cast<std::int64_t>(max_cache) * head_dim, 0, stream),
+                                         kv_heads, scale, head_dim, static_cast<std::int64_t>(max_cache) * head_dim, 0,
+                                         fits ? workspace : nullptr, fits ? split : 0, stream),
               "Talker generic fused attention launch");
         return;
     }

@@ -89,7 +89,9 @@ _SIGNATURES = {
                                           _F32, _PTR, C.c_size_t, _PTR, _PTR]),
     "qm_decode_attention_ragged_static": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _PTR, _I32,
                                                  _F32, _PTR, _PTR]),
-    "qm_prefill_attention_chunk": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _I32, _I32, _F32, C.c_int64, C.c_int64, C.c_int64, _PTR]),
+    "qm_prefill_chunk_workspace_bytes": (C.c_int64, [_I32, _I32, _I32, _I32]),
+    "qm_prefill_attention_chunk": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _I32, _I32, _F32, C.c_int64, C.c_int64, C.c_int64,
+                                          _PTR, C.c_int64, _PTR]),
     "qm_attention_rows_workspace_bytes": (C.c_size_t, [_I32, _I32, _I32, _I32]),
     "qm_attention_rows": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _I32, _I32, _F32,
                                  _PTR, C.c_size_t, _PTR, _PTR]),
@@ -256,11 +258,18 @@ def decode_attention_ragged(query, cache, page_table, max_pages, seq_lens, n_str
         stream), "qm_decode_attention_ragged")
 
 
+def prefill_chunk_workspace_bytes(batch, rows, cache_before, kv_heads):
+    n = lib().qm_prefill_chunk_workspace_bytes(batch, rows, cache_before, kv_heads)
+    if n < 0:
+        _check(n, "qm_prefill_chunk_workspace_bytes")
+    return n
+
+
 def prefill_attention_chunk(query, key, value, out, batch, rows, cache_before, q_heads, kv_heads, scale=SCALE_128,
-                            stream=0, kv_strides=(0, 0, 0)):
+                            stream=0, kv_strides=(0, 0, 0), workspace=None, workspace_bytes=0):
     _check(lib().qm_prefill_attention_chunk(
         _addr(query), _addr(key), _addr(value), _addr(out), batch, rows, cache_before, q_heads, kv_heads, scale,
-        kv_strides[0], kv_strides[1], kv_strides[2], stream), "qm_prefill_attention_chunk")
+        kv_strides[0], kv_strides[1], kv_strides[2], _addr(workspace), workspace_bytes, stream), "qm_prefill_attention_chunk")
 
 
 def attention_rows_workspace_bytes(query_length, q_heads, kv_heads, key_end):

@@ -98,7 +98,14 @@ struct PrefillParams {
     // 0 .. cache_before + i of the key_count = cache_before + seq keys that k and v hold
     int cache_before;
     int key_count;
+    // (chunk kernel, key split) the key tiles of a query tile go to blocks in runs of chunk_run; a query tile of more
+    // than one run leaves a record per run and prefill_chunk_merge_kernel combines them
+    int chunk_parts;             // blocks per (pair, query tile) in the grid; 1: no split
+    int chunk_run;
+    float* chunk_records;        // [pair][query tile][part][kChunkRecordFloats]
 };
+
+constexpr int kChunkRecordFloats = 66 * kPfThreads;   // per thread: 64 of O (unnormalised), the reference maximum, the sum
 
 struct PfStage {
     uint16_t k[kBN * kKS];
@@ -137,7 +144,7 @@ template <bool B> using bool_c = std::integral_constant<bool, B>;
 // CHUNK: the query rows stand at positions cache_before + row (prefill_chunk_kernel); otherwise at their row.
 template <bool PRECISE, bool ROUND, bool CHUNK = false>
 __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_kv_cache& cache,
-                                             unsigned char* pf_smem, int qt, int pair) {
+                                             unsigned char* pf_smem, int qt, int pair, int part = 0) {
     PfStage* st = reinterpret_cast<PfStage*>(pf_smem);
 
     const int tid = threadIdx.x;
@@ -435,19 +442,34 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     };
 
     // ---- tile 0 into stage 0, then the key tiles up to the diagonal ---------------------------------
-    load_tile(0);
-    if (prm.has_cache) fetch_pages();
-    if (prm.has_cache && qt == 0) write_pages(0);
-    store_tile(0);
-    __syncthreads();
+    if (!CHUNK) {
+        load_tile(0);
+        if (prm.has_cache) fetch_pages();
+        if (prm.has_cache && qt == 0) write_pages(0);
+        store_tile(0);
+        __syncthreads();
+    }
 
+    bool to_record = false;
     if (CHUNK) {
         // Key tiles every row of the query tile sees whole, then the one or two that the causal mask cuts
         // (two when the tile's first position is not a multiple of 64); the last tile always takes the masked
-        // path, where keys beyond key_count go.
+        // path, where keys beyond key_count go.  With a key split this block takes one run of them.
         const int last_tile = min(q0 + shift + kBM - 1, SK - 1) / kBN;
         const int whole = PRECISE ? 0 : min((q0 + shift + 1) / kBN, last_tile);
-        for (int t = 0; t < whole; ++t) {
+        int t_first = 0, t_last = last_tile;
+        if (!PRECISE && prm.chunk_parts > 1) {
+            t_first = part * prm.chunk_run;
+            if (t_first > last_tile) return;                       // (uniform over the block) no such run
+            t_last = min(t_first + prm.chunk_run - 1, last_tile);
+            to_record = last_tile >= prm.chunk_run;                // the query tile has more than one run
+        }
+        load_tile(t_first);
+        store_tile(t_first & 1);
+        __syncthreads();
+        // (the last tile of a run takes the masked path even where no mask applies: one loop shape for every run)
+        const int unmasked_end = min(whole, t_last);
+        for (int t = t_first; t < unmasked_end; ++t) {
             const int stage = t & 1;
             load_tile(t + 1);
             chunk(stage, int_c<0>{}, bool_c<false>{}, 0);
@@ -455,12 +477,12 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
             store_tile(stage ^ 1);
             __syncthreads();
         }
-        for (int t = whole;; ++t) {
+        for (int t = max(t_first, unmasked_end);; ++t) {
             const int stage = t & 1;
-            if (t < last_tile) load_tile(t + 1);
+            if (t < t_last) load_tile(t + 1);
             chunk(stage, int_c<0>{}, bool_c<true>{}, t * kBN);
             chunk(stage, int_c<1>{}, bool_c<true>{}, t * kBN + 32);
-            if (t == last_tile) break;
+            if (t == t_last) break;
             store_tile(stage ^ 1);
             __syncthreads();
         }
@@ -481,8 +503,22 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     }
     __syncthreads();   // the stages become the output staging area
 
-    // ---- normalise, stage through LDS, write 16 bytes per lane -------------------------------------
     const float l_tot = halves_sum(l_run);
+    if (CHUNK && !PRECISE && to_record) {
+        // One run of several: the unnormalised O, the reference maximum and the sum, as register images (thread t of
+        // the merge kernel takes what thread t leaves here).
+        float* rec = prm.chunk_records
+                   + ((static_cast<int64_t>(pair) * prm.n_qtiles + qt) * prm.chunk_parts + part) * kChunkRecordFloats + tid;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) rec[(16 * dt + r) * kPfThreads] = o[dt][r];
+        rec[64 * kPfThreads] = m_run;
+        rec[65 * kPfThreads] = l_tot;
+        return;
+    }
+
+    // ---- normalise, stage through LDS, write 16 bytes per lane -------------------------------------
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
     uint16_t* stage = reinterpret_cast<uint16_t*>(pf_smem) + wave * 32 * kOS;   // 32 columns x 128 dims per wave
 #pragma unroll
@@ -536,12 +572,70 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_chunk_kernel(PrefillPar
     extern __shared__ __attribute__((aligned(16))) unsigned char pf_smem[];
     const int pairs = prm.batch * prm.kv_heads;
     const int bid = blockIdx.x;
-    const int qt = prm.n_qtiles - 1 - bid / pairs;
+    const int group = bid / pairs;                       // heaviest query tile first, its runs side by side
+    const int qt = prm.n_qtiles - 1 - group / prm.chunk_parts;
+    const int part = group % prm.chunk_parts;
     const int pair = bid % pairs;
     if ((qt * kBM + prm.cache_before + 1) / kBN == 0) {
-        prefill_body<true, ROUND, true>(prm, cache, pf_smem, qt, pair);
+        if (part == 0) prefill_body<true, ROUND, true>(prm, cache, pf_smem, qt, pair);
     } else {
-        prefill_body<false, ROUND, true>(prm, cache, pf_smem, qt, pair);
+        prefill_body<false, ROUND, true>(prm, cache, pf_smem, qt, pair, part);
+    }
+}
+
+// Combines the runs of the query tiles that prefill_chunk_kernel split: sum over runs of O * w over sum of l * w,
+// w = exp(maximum of the run - largest maximum), in run order.  grid = pairs * n_qtiles * 8, 256 threads: thread t
+// holds what thread t of a run's block held (column = (row % 16, head) of a wave), and a block takes eight of the
+// thread's 64 values, all runs' loads in flight at once.
+constexpr int kChunkMaxRuns = 16;
+constexpr int kChunkMergeSlices = 8;
+__global__ __launch_bounds__(kPfThreads) void prefill_chunk_merge_kernel(PrefillParams prm, int round_scores) {
+    const int slice = blockIdx.x % kChunkMergeSlices;
+    const int item = blockIdx.x / kChunkMergeSlices;
+    const int pair = item % (prm.batch * prm.kv_heads);
+    const int qt = item / (prm.batch * prm.kv_heads);
+    const int q0 = qt * kBM;
+    const int last_tile = min(q0 + prm.cache_before + kBM - 1, prm.key_count - 1) / kBN;
+    const int runs = last_tile / prm.chunk_run + 1;
+    if (runs == 1) return;                               // its one block has written the rows itself
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, col = lane & 31, grp = lane >> 5;
+    const float coef = round_scores ? kLog2e : prm.scale * kLog2e;
+    const float* rec = prm.chunk_records + (static_cast<int64_t>(pair) * prm.n_qtiles + qt) * prm.chunk_parts * kChunkRecordFloats + tid;
+    float mv[kChunkMaxRuns], lv[kChunkMaxRuns], ov[kChunkMaxRuns][8];
+#pragma unroll
+    for (int p = 0; p < kChunkMaxRuns; ++p) {
+        const float* r = rec + static_cast<int64_t>(min(p, runs - 1)) * kChunkRecordFloats;
+        mv[p] = r[64 * kPfThreads];
+        lv[p] = r[65 * kPfThreads];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ov[p][i] = r[(8 * slice + i) * kPfThreads];
+    }
+    float m_all = -INFINITY;
+#pragma unroll
+    for (int p = 0; p < kChunkMaxRuns; ++p) m_all = fmaxf(m_all, mv[p]);
+    const float m_ref = m_all == -INFINITY ? 0.0f : m_all;
+    float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    float l = 0.0f;
+#pragma unroll
+    for (int p = 0; p < kChunkMaxRuns; ++p) {
+        const float w = p < runs ? fast_exp2((mv[p] - m_ref) * coef) : 0.0f;
+        l = fmaf(lv[p], w, l);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(ov[p][i], w, acc[i]);
+    }
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    const int b = pair / prm.kv_heads, kvh = pair % prm.kv_heads;
+    const int row = q0 + 16 * wave + (col & 15);
+    if (row >= prm.seq) return;
+    uint16_t* out = prm.out + ((static_cast<int64_t>(b) * prm.seq + row) * (2 * prm.kv_heads) + 2 * kvh + (col >> 4)) * kDim;
+    // value 16 dt + 4 rq + j of a thread is dim 32 dt + 8 rq + 4 grp + j: this slice is dt = slice / 2, rq = 2 (slice % 2), + 1
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        uint2 packed;
+        packed.x = pack_bf16_pair(acc[4 * h + 0] * inv, acc[4 * h + 1] * inv);
+        packed.y = pack_bf16_pair(acc[4 * h + 2] * inv, acc[4 * h + 3] * inv);
+        *reinterpret_cast<uint2*>(out + 32 * (slice >> 1) + 8 * (2 * (slice & 1) + h) + 4 * grp) = packed;
     }
 }
 
@@ -1607,14 +1701,54 @@ extern "C" int32_t qm_prefill_attention_causal_split(
                                    workspace_bytes, status_dev, hip_stream);
 }
 
+namespace qm {
+
+// The key split of a chunk call: with fewer blocks than compute units the key tiles of a query tile are handed out in
+// runs, as many per query tile as fill the chip, of four tiles at least and sixteen runs at most.
+struct ChunkPlan {
+    int parts = 1;       // blocks per (pair, query tile)
+    int run = 0;         // key tiles per block
+    int64_t bytes = 0;   // records
+};
+
+static ChunkPlan plan_chunk(int64_t pairs, int rows, int cache_before, int compute_units) {
+    ChunkPlan plan;
+    const int n_qtiles = (rows + kBM - 1) / kBM;
+    const int64_t blocks = pairs * n_qtiles;
+    const int tiles = (cache_before + rows - 1) / kBN + 1;      // of the last query tile
+    int64_t parts = (compute_units + blocks - 1) / blocks;
+    parts = std::min<int64_t>(parts, std::min(tiles / 4, kChunkMaxRuns));
+    if (parts < 2) return plan;
+    plan.run = static_cast<int>((tiles + parts - 1) / parts);
+    plan.parts = (tiles + plan.run - 1) / plan.run;
+    if (plan.parts < 2) return ChunkPlan();
+    plan.bytes = blocks * plan.parts * kChunkRecordFloats * static_cast<int64_t>(sizeof(float));
+    return plan;
+}
+
+}  // namespace qm
+
+extern "C" int64_t qm_prefill_chunk_workspace_bytes(int32_t batch, int32_t rows, int32_t cache_before, int32_t kv_heads) {
+    using namespace qm;
+    if (batch <= 0 || rows <= 0 || cache_before < 0 || kv_heads <= 0) return 0;
+    if (static_cast<int64_t>(cache_before) + rows > INT32_MAX) return QM_ERR_ARGUMENT;
+    int compute_units = 0;
+    const int32_t rc = device_compute_units(&compute_units);
+    if (rc != QM_OK) return rc;
+    return plan_chunk(static_cast<int64_t>(batch) * kv_heads, rows, cache_before, compute_units).bytes;
+}
+
 extern "C" int32_t qm_prefill_attention_chunk(
     const uint16_t* query, const uint16_t* key, const uint16_t* value,
     uint16_t* context_out,
     int32_t batch, int32_t rows, int32_t cache_before, int32_t q_heads, int32_t kv_heads, float scale,
     int64_t kv_stride_token, int64_t kv_stride_head, int64_t kv_stride_batch,
+    void* workspace, int64_t workspace_bytes,
     void* hip_stream) {
     using namespace qm;
     if (batch < 0 || rows < 0 || cache_before < 0) return QM_ERR_ARGUMENT;
+    if (workspace_bytes < 0 || (workspace_bytes > 0 && !workspace)) return QM_ERR_ARGUMENT;
+    if (reinterpret_cast<uintptr_t>(workspace) & 255) return QM_ERR_GEOMETRY;
     const int64_t key_count = static_cast<int64_t>(cache_before) + rows;
     if (kv_stride_token == 0 && kv_stride_head == 0 && kv_stride_batch == 0) {
         kv_stride_token = static_cast<int64_t>(kv_heads) * kDim;     // [batch][key_count][kv_heads][128]
@@ -1633,7 +1767,7 @@ extern "C" int32_t qm_prefill_attention_chunk(
     if (batch == 0 || rows == 0) return QM_OK;
     const int n_qtiles = (rows + kBM - 1) / kBM;
     const int64_t pairs = static_cast<int64_t>(batch) * kv_heads;
-    if (pairs * n_qtiles > 0x7fffffffLL) return QM_ERR_ARGUMENT;
+    if (pairs * n_qtiles * 16 > 0x7fffffffLL) return QM_ERR_ARGUMENT;
 
     PrefillParams prm = {};
     prm.q = query; prm.k = key; prm.v = value; prm.out = context_out;
@@ -1642,6 +1776,19 @@ extern "C" int32_t qm_prefill_attention_chunk(
     prm.batch = batch; prm.seq = rows; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
     prm.heavy_groups = n_qtiles;
     prm.cache_before = cache_before; prm.key_count = static_cast<int>(key_count);
+    prm.chunk_parts = 1;
+    if (workspace) {
+        int compute_units = 0;
+        const int32_t rc_cu = device_compute_units(&compute_units);
+        if (rc_cu != QM_OK) return rc_cu;
+        const ChunkPlan plan = plan_chunk(pairs, rows, cache_before, compute_units);
+        if (plan.parts > 1) {
+            if (workspace_bytes < plan.bytes) return QM_ERR_WORKSPACE;
+            prm.chunk_parts = plan.parts;
+            prm.chunk_run = plan.run;
+            prm.chunk_records = static_cast<float*>(workspace);
+        }
+    }
 
     const bool round_scores = option_value(QM_OPT_PREFILL_SCORE_ROUNDING) != 0;
     if (!round_scores && !(scale > 0.0f)) return QM_ERR_ARGUMENT;   // the scale is folded into the exponent there
@@ -1652,7 +1799,13 @@ extern "C" int32_t qm_prefill_attention_chunk(
                                               lds_raised[round_scores ? 1 : 0]);
     if (rc_lds != QM_OK) return rc_lds;
     const qm_kv_cache none = {};
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(pairs * n_qtiles)), dim3(kPfThreads), smem,
-                       static_cast<hipStream_t>(hip_stream), prm, none);
-    return launch_status();
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(pairs * n_qtiles * prm.chunk_parts)), dim3(kPfThreads), smem, s, prm, none);
+    int32_t rc = launch_status();
+    if (rc == QM_OK && prm.chunk_parts > 1) {
+        hipLaunchKernelGGL(prefill_chunk_merge_kernel, dim3(static_cast<unsigned>(pairs * n_qtiles * kChunkMergeSlices)), dim3(kPfThreads), 0, s, prm,
+                           round_scores ? 1 : 0);
+        rc = launch_status();
+    }
+    return rc;
 }

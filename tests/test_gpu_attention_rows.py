@@ -282,16 +282,44 @@ def test_chunk_agrees_with_the_rows_of_the_decode_kernels(oracle, qm, dev):
     assert np.max(np.abs(a - b)) <= 2 * TOL
 
 
+@pytest.mark.parametrize("rows,before,batch", [(256, 2048, 1), (64, 2048, 1), (100, 1000, 1), (70, 700, 2), (64, 4000, 1), (1, 8191, 1),
+                                               (130, 515, 1), (20, 500, 1)])
+def test_chunk_with_the_keys_shared_between_blocks(oracle, qm, dev, rows, before, batch):
+    """A workspace lets several blocks share the keys of a query tile; their records are combined in run order: within the
+    tolerance of the oracle, one bf16 ulp (2e-3 near zero) from the unsplit call, and the same bits on every call."""
+    import torch
+    got, want, (qd, kd, vd, max_cache) = _chunk(oracle, qm, dev, rows, before, seed=7000 + rows + before, batch=batch)
+    nbytes = qm.prefill_chunk_workspace_bytes(batch, rows, before, 8)
+    assert nbytes > 0
+    ws = torch.full((nbytes // 4,), 0x7fc00000, dtype=torch.int32, device=dev)      # NaN: nothing stale may be read
+    outs = []
+    for _ in range(3):
+        out = torch.full((batch, rows, 16, 128), 0x7fc0, dtype=torch.int16, device=dev)
+        qm.prefill_attention_chunk(qd, kd, vd, out, batch, rows, before, 16, 8, SCALE,
+                                   kv_strides=(128, max_cache * 128, 8 * max_cache * 128), workspace=ws, workspace_bytes=nbytes)
+        torch.cuda.synchronize()
+        outs.append(to_u16(out))
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    assert max_abs_err(oracle, outs[0], want[1]) <= TOL and max_abs_err(oracle, outs[0], want[0]) <= TOL
+    assert _within(oracle, outs[0], got, tol=2e-3)         # against the unsplit call: one ulp, or 2e-3 near zero
+    # too small a workspace is refused; a shape that would not split needs none
+    assert qm.lib().qm_prefill_attention_chunk(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(), batch, rows, before, 16, 8,
+                                               SCALE, 128, max_cache * 128, 8 * max_cache * 128, ws.data_ptr(), nbytes - 4, None) == -4
+    assert qm.prefill_chunk_workspace_bytes(32, 512, 64, 8) == 0
+
+
 def test_chunk_argument_errors(qm, dev):
     import ctypes as C
     import torch
     t = torch.zeros(4 * 16 * 128 * 80, dtype=torch.int16, device=dev)
     p = t.data_ptr()
     call = lambda rows, before, heads=16, kv=8, st=(0, 0, 0), q=p: qm.lib().qm_prefill_attention_chunk(
-        q, p, p, p, 1, rows, before, heads, kv, SCALE, st[0], st[1], st[2], None)
+        q, p, p, p, 1, rows, before, heads, kv, SCALE, st[0], st[1], st[2], None, 0, None)
     assert call(0, 5) == 0
     assert call(-1, 0) == -5 and call(4, -1) == -5
     assert call(4, 5, heads=8) == -2 and call(4, 5, st=(64, 128, 0)) == -2 and call(4, 5, st=(132, 128, 0)) == -2
     assert call(4, 5, q=p + 2) == -2
     assert call(4, 2 ** 24, st=(128, 2 ** 31, 0)) == -5           # keys beyond 32-bit element offsets
-    assert qm.lib().qm_prefill_attention_chunk(None, p, p, p, 1, 4, 5, 16, 8, SCALE, 0, 0, 0, None) == -1
+    assert qm.lib().qm_prefill_attention_chunk(None, p, p, p, 1, 4, 5, 16, 8, SCALE, 0, 0, 0, None, 0, None) == -1
+    assert qm.lib().qm_prefill_attention_chunk(p, p, p, p, 1, 4, 5, 16, 8, SCALE, 0, 0, 0, None, 64, None) == -5
+    assert qm.lib().qm_prefill_attention_chunk(p, p, p, p, 1, 4, 5, 16, 8, SCALE, 0, 0, 0, p + 16, 64, None) == -2
