@@ -205,6 +205,8 @@ int32_t qm_decode_attention(
  * row of `position`; q_rotated_out [q_heads][128] receives the rotated query (may be NULL).
  * Results (context, cache contents, q_rotated) are bit-identical to the two separate calls.
  * Workspace as for qm_decode_attention with max_seq_len = position + 1.
+ * q_heads / kv_heads must be 1, 2 or 4 here (QM_ERR_GEOMETRY otherwise); qm_decode_attention,
+ * qm_decode_attention_ragged and qm_attention_rows take any integral group.
  */
 int32_t qm_decode_step_fused(
     const uint16_t* q, const uint16_t* k, const uint16_t* v,

@@ -297,6 +297,10 @@ def test_fused_decode_step_argument_errors(qm, dev):
     assert L.qm_decode_step_fused(*args(3, None)) == -1
     assert L.qm_decode_step_fused(*args(31)) == 0
     torch.cuda.synchronize()
+    # the fused step is built for 1, 2 and 4 query heads per kv head (the other decode entry points take any group)
+    wide = list(args(3))
+    wide[12] = 24
+    assert L.qm_decode_step_fused(*wide) == -2
 
 
 def _double_bf16(bits):
