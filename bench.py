@@ -30,7 +30,7 @@ sys.path.insert(0, ROOT)
 # FETCH_SIZE and WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a
 # plain 512 MiB copy (FETCH_SIZE reads half the copied bytes: factor 2.0; WRITE_SIZE: 1.0).
 # Summary and commands: profiles/decode_split_kernel_ragged64_traffic.txt
-HEADLINE_TRAFFIC_BYTES = int((288456.9 * 2.0 + 3349.5 * 1.0) * 1024)
+HEADLINE_TRAFFIC_BYTES = int((289789.3 * 2.0 + 3317.0 * 1.0) * 1024)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
