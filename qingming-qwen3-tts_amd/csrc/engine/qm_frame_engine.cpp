@@ -10,6 +10,7 @@
 #include "qm_engine_common.hpp"
 
 #include <array>
+#include <cstring>
 #include <memory>
 
 namespace qm_engine {
@@ -36,9 +37,18 @@ static void expect_shape(const Param& p, std::vector<int64_t> shape, const std::
     if (p.shape != shape) throw TensorError("unexpected shape of " + what);
 }
 
+// A part of a device allocation that another object owns.
+struct DeviceSlice {
+    void* pointer = nullptr;
+    size_t size = 0;
+    uint16_t* u16() const { return static_cast<uint16_t*>(pointer); }
+    void* raw() const { return pointer; }
+    size_t bytes() const { return size; }
+};
+
 struct PredictorLayer {
     Param input_norm, q_weight, k_weight, v_weight, q_norm, k_norm, o_weight, post_norm, gate_weight, up_weight, down_weight;
-    DeviceBuffer key_cache, value_cache;   // [8][16][128]
+    DeviceSlice key_cache, value_cache;    // [8][16][128], parts of qm_predictor::frame_state
 };
 
 }  // namespace qm_engine
@@ -47,7 +57,7 @@ using namespace qm_engine;
 
 struct qm_final_head {
     Param weight;                          // talker.codec_head.weight [3072][2048]
-    DeviceBuffer logits, history, code, rng;
+    DeviceBuffer logits, history, code, rng, rng_after_head;
     int capacity = 0;
     hipStream_t stream = nullptr;
 };
@@ -61,7 +71,11 @@ struct qm_predictor {
     DeviceBuffer cosine, sine;             // [16][128], positions 0..15
     DeviceBuffer free_input, context_embedding, hidden_a, hidden_b, norm, q_linear, k_linear, v_linear, q_normed, k_normed,
         q_bhsd, k_bhsd, v_bhsd, q_rotated, k_rotated, context, attention, residual, post_norm, swiglu, logits,
-        selected, codes, embedding_sum, next_input;
+        embedding_sum, next_input;
+    // What run_frame_device clears at the start of a frame (R17:13043-13070) — the layers' caches, the selected
+    // embeddings, the codes — lies in one allocation, so that one fill clears it.
+    DeviceBuffer frame_state;
+    DeviceSlice selected, codes;
     // the M = 1 steps as one launch (qm_predictor_frame_steps): only for the five-layer geometry it is built for
     bool one_launch = false;
     qm_predictor_frame frame = {};
@@ -83,6 +97,7 @@ static std::unique_ptr<qm_final_head> create_final_head(const std::string& model
     head->history = DeviceBuffer(static_cast<size_t>(capacity) * sizeof(int32_t));
     head->code = DeviceBuffer(sizeof(int32_t));
     head->rng = DeviceBuffer(sizeof(uint64_t));
+    head->rng_after_head = DeviceBuffer(sizeof(uint64_t));
     head->capacity = capacity;
     hip_check(hipMemcpyAsync(head->rng.raw(), &seed, sizeof seed, hipMemcpyHostToDevice, stream), "generator seed upload");
     hip_check(hipMemsetAsync(head->history.raw(), 0, head->history.bytes(), stream), "history reset");
@@ -92,7 +107,7 @@ static std::unique_ptr<qm_final_head> create_final_head(const std::string& model
 
 // run_fast_device (R17:14427-14570): codec_head, then cast + repetition penalty + suppressed tokens + sampler (or
 // arg-max) + history append in one launch, then the four-byte read-back that is the frame boundary.
-static int32_t final_head_run(qm_final_head& h, const uint16_t* hidden_device, int frame, bool sampling) {
+static void final_head_launch(qm_final_head& h, const uint16_t* hidden_device, int frame, bool sampling) {
     if (frame < 0 || frame >= h.capacity) throw ApiError(QM_ERR_SLOT_RANGE, "FinalHead generation index exceeds GPU history capacity");
     op_check(qm_linear_m1(hidden_device, h.weight.data(), nullptr, nullptr, h.logits.u16(), kHeadVocab, kHidden, h.stream),
              "final head projection");
@@ -100,6 +115,10 @@ static int32_t final_head_run(qm_final_head& h, const uint16_t* hidden_device, i
                                   kSuppressedTail, kPenalty, sampling ? kTopK : 0, kTemperature,
                                   static_cast<uint64_t*>(h.rng.raw()), static_cast<int32_t*>(h.code.raw()), nullptr, h.stream),
              "final head sampler");
+}
+
+static int32_t final_head_run(qm_final_head& h, const uint16_t* hidden_device, int frame, bool sampling) {
+    final_head_launch(h, hidden_device, frame, sampling);
     int32_t code = 0;
     hip_check(hipMemcpyAsync(&code, h.code.raw(), sizeof code, hipMemcpyDeviceToHost, h.stream), "code read-back");
     hip_check(hipStreamSynchronize(h.stream), "frame boundary synchronize");
@@ -145,8 +164,6 @@ static std::unique_ptr<qm_predictor> create_predictor(const std::string& model_d
         expect_shape(w.gate_weight, {kPredIntermediate, kPredHidden}, lr + "mlp.gate_proj.weight");
         expect_shape(w.up_weight, {kPredIntermediate, kPredHidden}, lr + "mlp.up_proj.weight");
         expect_shape(w.down_weight, {kPredHidden, kPredIntermediate}, lr + "mlp.down_proj.weight");
-        w.key_cache = DeviceBuffer(kPredKvHeads * kPredMaxCache * kHeadDim * 2);
-        w.value_cache = DeviceBuffer(kPredKvHeads * kPredMaxCache * kHeadDim * 2);
         p->layers.push_back(std::move(w));
     }
     if (p->layers.empty()) throw TensorError("no code predictor layers in " + model_dir);
@@ -180,8 +197,19 @@ static std::unique_ptr<qm_predictor> create_predictor(const std::string& model_d
     p->q_rotated = rows2(kPredQueryDim); p->k_rotated = rows2(kPredKvDim); p->context = rows2(kPredQueryDim);
     p->attention = rows2(kPredHidden); p->residual = rows2(kPredHidden); p->post_norm = rows2(kPredHidden);
     p->swiglu = rows2(kPredIntermediate); p->logits = rows2(kPredVocab);
-    p->selected = DeviceBuffer(static_cast<size_t>(kCodeGroups) * kOuter * 2);
-    p->codes = DeviceBuffer(kCodeGroups * sizeof(int32_t));
+    {
+        const size_t cache_bytes = static_cast<size_t>(kPredKvHeads) * kPredMaxCache * kHeadDim * 2;     // a multiple of 256
+        const size_t selected_bytes = static_cast<size_t>(kCodeGroups) * kOuter * 2;
+        p->frame_state = DeviceBuffer(2 * cache_bytes * p->layers.size() + selected_bytes + 256);
+        unsigned char* at = static_cast<unsigned char*>(p->frame_state.raw());
+        for (PredictorLayer& w : p->layers) {
+            w.key_cache = DeviceSlice{at, cache_bytes};
+            w.value_cache = DeviceSlice{at + cache_bytes, cache_bytes};
+            at += 2 * cache_bytes;
+        }
+        p->selected = DeviceSlice{at, selected_bytes};
+        p->codes = DeviceSlice{at + selected_bytes, kCodeGroups * sizeof(int32_t)};
+    }
     p->embedding_sum = DeviceBuffer(kOuter * 2); p->next_input = DeviceBuffer(kOuter * 2);
     hip_check(hipStreamSynchronize(stream), "predictor upload synchronize");   // the mapped files go away with `host`
     p->status = DeviceBuffer(256);
@@ -298,16 +326,12 @@ static void predictor_step_m1(qm_predictor& p, int step, bool sampling) {
 
 // run_frame_device (R17:13043-13156): reset of the caches and of the frame's selected embeddings and codes, the
 // two input rows, the fifteen steps, the next talker input, and the 64-byte read-back of the frame's sixteen codes.
+// `code0_out`, if given, receives the code the frame started from with the same synchronize.
 static void predictor_frame(qm_predictor& p, const uint16_t* talker_hidden_device, const int32_t* code0_device,
-                            const uint16_t* context_host, bool sampling, int32_t codes_out[16]) {
+                            const uint16_t* context_host, bool sampling, int32_t codes_out[16], int32_t* code0_out = nullptr) {
     if (!talker_hidden_device || !code0_device || !context_host || !codes_out) throw ApiError(QM_ERR_NULL, "predictor frame input is null");
     hipStream_t s = p.stream;
-    for (PredictorLayer& w : p.layers) {
-        hip_check(hipMemsetAsync(w.key_cache.raw(), 0, w.key_cache.bytes(), s), "predictor key cache reset");
-        hip_check(hipMemsetAsync(w.value_cache.raw(), 0, w.value_cache.bytes(), s), "predictor value cache reset");
-    }
-    hip_check(hipMemsetAsync(p.selected.raw(), 0, p.selected.bytes(), s), "selected embeddings reset");
-    hip_check(hipMemsetAsync(p.codes.raw(), 0, p.codes.bytes(), s), "generated codes reset");
+    hip_check(hipMemsetAsync(p.frame_state.raw(), 0, p.frame_state.bytes(), s), "predictor caches, selected embeddings and codes reset");
     hip_check(hipMemcpyAsync(p.free_input.raw(), talker_hidden_device, kOuter * 2, hipMemcpyDeviceToDevice, s), "talker hidden copy");
     hip_check(hipMemcpyAsync(p.context_embedding.raw(), context_host, kOuter * 2, hipMemcpyHostToDevice, s), "context embedding upload");
     op_check(qm_predictor_prepare_group0(p.codec0_table.data(), static_cast<int32_t>(p.codec0_table.shape[0]), code0_device, kOuter,
@@ -328,6 +352,7 @@ static void predictor_frame(qm_predictor& p, const uint16_t* talker_hidden_devic
     op_check(qm_predictor_next_talker_input(p.selected.u16(), kCodeGroups, p.context_embedding.u16(), kOuter, p.embedding_sum.u16(),
                                             p.next_input.u16(), s), "next talker input");
     hip_check(hipMemcpyAsync(codes_out, p.codes.raw(), kCodeGroups * sizeof(int32_t), hipMemcpyDeviceToHost, s), "codes read-back");
+    if (code0_out) hip_check(hipMemcpyAsync(code0_out, code0_device, sizeof(int32_t), hipMemcpyDeviceToHost, s), "code read-back");
     uint32_t status = 0;
     if (one_launch) hip_check(hipMemcpyAsync(&status, p.status.raw(), sizeof status, hipMemcpyDeviceToHost, s), "status read-back");
     hip_check(hipStreamSynchronize(s), "predictor frame synchronize");
@@ -408,12 +433,25 @@ extern "C" int32_t qm_generate(qm_talker* talker, qm_final_head* head, qm_predic
             op_check(qm_rope_rows(decode_rows, prompt_rows, kHeadDim, 1000000.0, decode_cos.data(), decode_sin.data()), "decode rope rows");
         int frames = 0;
         for (int frame = 0; frame < maximum_frames; ++frame) {
-            const int32_t code0 = final_head_run(*head, hidden, frame, sampling != 0);
-            if (code0 == kCodecEos && frame >= 2) break;                           // R17:22222-22232
+            // The final head's code stays on the device, where the predictor reads it: the host learns it together
+            // with the frame's codes, at ONE synchronize per frame (the reference reads it back first and stops before
+            // the predictor at the end-of-sequence code, R17:22222-22232; here the frame that follows that code has
+            // run when it is seen, its codes are dropped and the generator state is put back to where the final head
+            // left it, so that what a caller finds afterwards is what the reference leaves).
+            final_head_launch(*head, hidden, frame, sampling != 0);
+            hip_check(hipMemcpyAsync(head->rng_after_head.raw(), head->rng.raw(), sizeof(uint64_t), hipMemcpyDeviceToDevice, head->stream),
+                      "generator state snapshot");
             const uint16_t* context = frame < trailing_rows ? trailing_text_host + static_cast<size_t>(frame) * kOuter : tts_pad_host;
-            int32_t* codes = codes_out + static_cast<size_t>(frame) * kCodeGroups;
-            predictor_frame(*predictor, hidden, static_cast<const int32_t*>(head->code.raw()), context, sampling != 0, codes);
-            if (codes[0] != code0) throw ApiError(QM_ERR_ARGUMENT, "native Predictor recurrence output mismatch");
+            int32_t frame_codes[kCodeGroups];
+            int32_t code0 = 0;
+            predictor_frame(*predictor, hidden, static_cast<const int32_t*>(head->code.raw()), context, sampling != 0, frame_codes, &code0);
+            if (code0 == kCodecEos && frame >= 2) {
+                hip_check(hipMemcpyAsync(head->rng.raw(), head->rng_after_head.raw(), sizeof(uint64_t), hipMemcpyDeviceToDevice, head->stream),
+                          "generator state restore");
+                break;
+            }
+            if (frame_codes[0] != code0) throw ApiError(QM_ERR_ARGUMENT, "native Predictor recurrence output mismatch");
+            std::memcpy(codes_out + static_cast<size_t>(frame) * kCodeGroups, frame_codes, sizeof frame_codes);
             ++frames;
             if (frame + 1 >= maximum_frames) break;
             op_check(qm_talker_decode(talker, predictor->next_input.u16(), decode_cos.data() + static_cast<size_t>(frame) * kHeadDim,

@@ -23,7 +23,7 @@ HEAD_V, EOS, TABLE_ROWS = 3072, 2150, 3072
 SEED = 20240229
 
 
-def _checkpoint(directory):
+def _checkpoint(directory, eos_gain=1.0):
     import torch
     from safetensors.torch import save_file
     g = torch.Generator().manual_seed(99)
@@ -55,6 +55,9 @@ def _checkpoint(directory):
     for i in range(STEPS):
         t[c + f"lm_head.{i}.weight"] = rnd((V, PH), 0.05)
         t[c + f"model.codec_embedding.{i}.weight"] = rnd((V, H), 0.5)
+    if eos_gain != 1.0:
+        # the end-of-sequence code wins or loses by a wide margin, depending on the sign of its row's product with the hidden state
+        t["talker.codec_head.weight"][EOS] = (t["talker.codec_head.weight"][EOS].float() * eos_gain).to(torch.bfloat16)
     save_file(t, os.path.join(directory, "model.safetensors"))
     return {n: x.view(torch.int16).numpy().view(np.uint16).copy() for n, x in t.items()}
 
@@ -285,4 +288,47 @@ def test_generation_loop_is_deterministic_and_equals_its_stepwise_replay(engine,
     assert np.array_equal(short, codes[:2])
     with pytest.raises(engine.EngineError):
         engine.generate(talker, head, predictor, pd, 0, 2, tts_pad, trailing)
+    predictor.close(); head.close(); talker.close()
+
+
+def test_generation_stops_at_the_end_of_sequence_code(engine, oracle, qm, dev, tmp_path):
+    """A checkpoint whose final head gives the end-of-sequence code for about every other hidden state: the loop stops at
+    the first such frame from the third on (R17:22222-22232) without counting it, exactly where the stepwise replay — which
+    reads the code before the predictor runs, as the reference does — stops, and leaves the generator state that replay leaves."""
+    import torch
+    directory = str(tmp_path)
+    _checkpoint(directory, eos_gain=60.0)
+    prompt_rows, limit = 11, 24
+    talker = engine.Talker(directory, 64)
+    head = engine.FinalHead(directory, 32, SEED, talker.stream)
+    predictor = engine.Predictor(directory, head.rng_state, talker.stream)
+    pd = torch.from_numpy(oracle.normal_bf16((prompt_rows, H), 51).view(np.int16)).to(dev)
+    torch.cuda.synchronize()
+    tts_pad = oracle.normal_bf16((H,), 52, 0.0, 0.5)
+    codes, digest = engine.generate(talker, head, predictor, pd, prompt_rows, limit, tts_pad, None)
+    state_after_generate = _device_bytes(head.rng_state, 8).copy()
+    assert 2 <= codes.shape[0] < limit, "the checkpoint is meant to end the sequence early, from the third frame on"
+    assert digest == _fnv1a64(codes.tobytes())
+    assert not (codes[2:, 0] == EOS).any()                   # the frame that carries the code is not part of the output
+    # the stepwise replay
+    head.reset(SEED)
+    cos, sin = engine.rope_rows(prompt_rows, 0)
+    dcos, dsin = engine.rope_rows(limit, prompt_rows)
+    hidden = talker.prefill(pd, cos, sin, prompt_rows)
+    talker.synchronize()
+    replay = []
+    for frame in range(limit):
+        code0 = head.run(hidden, frame)
+        if code0 == EOS and frame >= 2:
+            break
+        replay.append(predictor.run_frame(hidden, head.device_code, tts_pad))
+        if frame + 1 < limit:
+            hidden = talker.decode(predictor.next_input, dcos[frame], dsin[frame], frame)
+    talker.synchronize()
+    assert np.array_equal(np.array(replay, dtype=np.int32), codes)
+    assert np.array_equal(_device_bytes(head.rng_state, 8), state_after_generate)
+    # and again through the loop: the same trajectory
+    head.reset(SEED)
+    again, digest2 = engine.generate(talker, head, predictor, pd, prompt_rows, limit, tts_pad, None)
+    assert np.array_equal(again, codes) and digest2 == digest
     predictor.close(); head.close(); talker.close()
