@@ -366,11 +366,13 @@ class TalkerLayerStep:
     # attention's 1e-2 budget surfaces as at most a couple of ulps there
     tolerance = 0.125
 
-    def __init__(self, qm, dev, layers=28, ctx=2048, seed=91, fused=True, chained=False):
+    def __init__(self, qm, dev, layers=28, ctx=2048, seed=91, fused=True, chained=False, two_launches=False):
         import torch
-        self.qm, self.layers, self.ctx, self.fused, self.chained = qm, layers, ctx, fused, chained
+        chained = chained or two_launches
+        self.qm, self.layers, self.ctx, self.fused, self.chained, self.two_launches = qm, layers, ctx, fused, chained, two_launches
         self.name = "talker_layer_decode_step_ctx%d_x%dlayers%s" % (
-            ctx, layers, "_one_launch_between_attentions" if chained else "" if fused else "_reference_launch_sequence")
+            ctx, layers, "_two_launches" if two_launches else "_one_launch_between_attentions" if chained else
+            "" if fused else "_reference_launch_sequence")
         self.copies = layers
         syn = Synthetic(dev, seed)
         H, I = 2048, 6144
@@ -416,6 +418,10 @@ class TalkerLayerStep:
                     context=self.ctxv, hidden=self.x, o_weight=L["wo"], post_norm=L["post"], gate_weight=L["wg"], up_weight=L["wu"],
                     down_weight=L["wd"], hidden_out=self.out, next_input_norm=N["in_norm"], next_q_weight=N["wq"],
                     next_k_weight=N["wk"], next_v_weight=N["wv"], q_out=self.q, k_out=self.k_, v_out=self.v_))
+            # ... and with the attention's merge folded into that launch a layer is two launches (qm_talker_layer_step_m1)
+            self.steps = [qm.talker_layer_step(self.q, self.k_, self.v_, L["gq"], L["gk"], self.cos, self.sin, self.qrot, L["cache"],
+                                               None, 1, self.ctxv, 16, ctx - 1, -1, SCALE, 1e-6, self.ws, self.ws_bytes, op)
+                          for L, op in zip(self.w, self.ops)] if two_launches else None
             self.primed = False
 
     def step(self):
@@ -428,6 +434,10 @@ class TalkerLayerStep:
                 qm.rmsnorm_qkv_m1(self.x, L["in_norm"], L["wq"], None, L["wk"], None, L["wv"], None, self.q, self.k_,
                                   self.v_, H, H, 1024, 1e-6, s)
                 self.primed = True
+            if self.two_launches:
+                qm.talker_layer_step_m1(self.steps[self.i % self.layers], self.chain_ws, self.chain_ws_bytes, self.status, s)
+                self.i += 1
+                return
             qm.decode_step_fused(self.q, self.k_, self.v_, L["gq"], L["gk"], self.cos, self.sin, self.qrot, L["cache"],
                                  None, 1, self.ctxv, 16, self.ctx - 1, -1, SCALE, 1e-6, self.ws, self.ws_bytes, None, s)
             qm.talker_post_attention_m1(self.ops[self.i % self.layers], self.chain_ws, self.chain_ws_bytes, self.status, s)
@@ -795,7 +805,8 @@ def generate_end_to_end(qm, dev, frames=96, prompt_rows=128, seed=20240229):
         torch.cuda.synchronize()
         rows = {}
         reference = None
-        for name, talker_ops, frame_ops in (("default", 0, 0), ("talker_layers_by_operators", 1, 0),
+        for name, talker_ops, frame_ops in (("default", 0, 0), ("talker_layers_in_three_launches", 2, 0),
+                                            ("talker_layers_by_operators", 1, 0),
                                             ("predictor_frame_by_operators", 0, 1), ("both_by_operators", 1, 1)):
             qm.set_option(qm.OPT_TALKER_LAYER_OPERATORS, talker_ops)
             qm.set_option(qm.OPT_PREDICTOR_FRAME_OPERATORS, frame_ops)
@@ -1028,7 +1039,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
     ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "prefillfp32", "chunk", "chunkwhole", "chunkrows", "predictor", "predictorexact",
-                                      "qkv", "layer", "layer1", "frame", "frame1", "linears", "linearsexact", "generate"], default=None,
+                                      "qkv", "layer", "layer1", "layer2", "frame", "frame1", "linears", "linearsexact", "generate"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -1070,7 +1081,7 @@ def main():
                 "chunk": lambda: PrefillChunk(qm, dev), "chunkwhole": lambda: PrefillChunk(qm, dev, split=False), "chunkrows": lambda: PrefillChunk(qm, dev, by_rows=True),
                 "predictor": lambda: PredictorLoop(qm, dev),
                 "predictorexact": lambda: PredictorLoop(qm, dev, kernel=1),
-                "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev), "layer1": lambda: TalkerLayerStep(qm, dev, chained=True),
+                "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev), "layer1": lambda: TalkerLayerStep(qm, dev, chained=True), "layer2": lambda: TalkerLayerStep(qm, dev, two_launches=True),
                 "frame": lambda: PredictorFrameSteps(qm, dev),
                 "frame1": lambda: PredictorFrameSteps(qm, dev, one_launch=True),
                 "linears": lambda: PromptLinears(qm, dev), "linearsexact": lambda: PromptLinears(qm, dev, kernel=1)}[args.only]
@@ -1122,6 +1133,8 @@ def main():
             ("next_talker_layer_decode_step", lambda: TalkerLayerStep(qm, dev)),
             ("next_talker_layer_decode_step_unfused", lambda: TalkerLayerStep(qm, dev, fused=False)),
             ("next_talker_layer_decode_step_one_launch", lambda: TalkerLayerStep(qm, dev, chained=True)),
+            # the attention's merge launch folded into that launch: two launches per layer
+            ("next_talker_layer_decode_step_two_launches", lambda: TalkerLayerStep(qm, dev, two_launches=True)),
             # the seven linears of a talker layer over a 1024-token prompt: matrix cores, and the exact chain
             ("next_prompt_linears_1024_tokens", lambda: PromptLinears(qm, dev)),
             ("next_prompt_linears_1024_tokens_exact_chain", lambda: PromptLinears(qm, dev, kernel=1)),

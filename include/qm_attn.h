@@ -110,9 +110,11 @@ const char* qm_target_arch(void);
  *       token rows on the matrix cores where the shape fits their tiles (output columns % 128 == 0, reduction % 128 == 0):
  *       same roundings after the sum, results within the operators' tolerance of the exact chain; 1: every call in the
  *       reference's summation order (bit-identical to the M = 1 operators; 20 to 60 times slower on long prompts).
- *   QM_OPT_TALKER_LAYER_OPERATORS  0 (default): the engine's talker decode step (qm_engine.h) runs what lies between two
- *       attentions as one launch of qm_talker_post_attention_m1 where the checkpoint has the geometry it serves; 1: operator
- *       by operator.  Same bits either way. */
+ *   QM_OPT_TALKER_LAYER_OPERATORS  how the engine's talker decode step (qm_engine.h) runs a layer where the checkpoint has
+ *       the geometry qm_talker_post_attention_m1 serves.  0 (default): two launches, qm_talker_layer_step_m1 (the attention
+ *       without its merge launch, then everything up to the next layer's Q/K/V, which combines the attention's splits
+ *       first); 2: three launches (qm_decode_step_fused with its merge, qm_talker_post_attention_m1); 1: operator by
+ *       operator.  Same bits every way. */
 enum {
     QM_OPT_PREFILL_SCORE_ROUNDING = 0,
     QM_OPT_DECODE_TILES_PER_BLOCK = 1,
@@ -582,6 +584,44 @@ int64_t qm_talker_post_attention_workspace_bytes(void);
 int32_t qm_talker_post_attention_workspace_init(void* workspace, int64_t workspace_bytes, void* hip_stream);
 int32_t qm_talker_post_attention_m1(
     const qm_talker_post_attention* op,
+    void* workspace, int64_t workspace_bytes, uint32_t* status_dev, void* hip_stream);
+
+/*
+ * A talker layer's decode step after its Q/K/V projections in TWO launches: qm_decode_step_fused without its merge
+ * launch, then qm_talker_post_attention_m1, whose first eight blocks combine the attention's split records (one kv head
+ * each, the statistics, order and bits of the merge launch) and hand the context to all blocks while the weights of
+ * o_proj and gate/up are already on their way into LDS.  Replaces launch_qk_norm_rope_cache_m1 + launch_attention +
+ * the four launches named above (R17:17181-17244, and 17163-17176 of the next layer).  `context` [q_heads][128] receives
+ * the attention's output; `post.context` is ignored.  Results (context, cache, q_rotated, hidden_out, q/k/v_out) are
+ * bit-identical to qm_decode_step_fused followed by qm_talker_post_attention_m1.  The attention's arguments and
+ * attention_workspace are those of qm_decode_step_fused; q_heads 16 over 8 kv heads only (the talker's geometry);
+ * workspace, status word, bounded waits and QM_ERR_* as for qm_talker_post_attention_m1.
+ */
+typedef struct qm_talker_layer_step {
+    const uint16_t* q;                /* [q_heads][128] raw projections of the new token */
+    const uint16_t* k;                /* [kv_heads][128] */
+    const uint16_t* v;
+    const uint16_t* q_norm_w;         /* [128] */
+    const uint16_t* k_norm_w;
+    const uint16_t* cos_row;          /* [128] RoPE row of `position` */
+    const uint16_t* sin_row;
+    uint16_t* q_rotated_out;          /* [q_heads][128] or NULL */
+    const qm_kv_cache* cache;
+    const int32_t* page_table;
+    void* attention_workspace;        /* qm_decode_workspace_bytes(1, q_heads, kv_heads, position + 1) */
+    size_t attention_workspace_bytes;
+    uint16_t* context;                /* [q_heads][128] the attention's output */
+    int32_t max_pages;
+    int32_t q_heads;
+    int32_t position;
+    int32_t sliding_window;
+    float scale;
+    float epsilon;
+    qm_talker_post_attention post;
+} qm_talker_layer_step;
+
+int32_t qm_talker_layer_step_m1(
+    const qm_talker_layer_step* step,
     void* workspace, int64_t workspace_bytes, uint32_t* status_dev, void* hip_stream);
 
 /*

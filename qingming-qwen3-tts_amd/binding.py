@@ -61,6 +61,15 @@ class TalkerPostAttention(C.Structure):
         ("intermediate_columns", C.c_int32), ("epsilon", C.c_float)]
 
 
+class TalkerLayerStep(C.Structure):
+    """Mirror of qm_talker_layer_step (include/qm_attn.h)."""
+    _fields_ = [(name, C.c_void_p) for name in ("q", "k", "v", "q_norm_w", "k_norm_w", "cos_row", "sin_row", "q_rotated_out")] + [
+        ("cache", C.POINTER(KvCache)), ("page_table", C.c_void_p), ("attention_workspace", C.c_void_p),
+        ("attention_workspace_bytes", C.c_size_t), ("context", C.c_void_p),
+        ("max_pages", C.c_int32), ("q_heads", C.c_int32), ("position", C.c_int32), ("sliding_window", C.c_int32),
+        ("scale", C.c_float), ("epsilon", C.c_float), ("post", TalkerPostAttention)]
+
+
 def lib_path():
     return _LIB_PATH
 
@@ -113,6 +122,7 @@ _SIGNATURES = {
     "qm_talker_post_attention_workspace_bytes": (C.c_int64, []),
     "qm_talker_post_attention_workspace_init": (_I32, [_PTR, C.c_int64, _PTR]),
     "qm_talker_post_attention_m1": (_I32, [C.POINTER(TalkerPostAttention), _PTR, C.c_int64, _PTR, _PTR]),
+    "qm_talker_layer_step_m1": (_I32, [C.POINTER(TalkerLayerStep), _PTR, C.c_int64, _PTR, _PTR]),
     "qm_predictor_transpose": (_I32, [_PTR, _PTR, _I32, _I32, _PTR]),
     "qm_predictor_rope_bhsd": (_I32, [_PTR] * 4 + [_I32, _I32, _PTR]),
     "qm_predictor_update_cache": (_I32, [_PTR, _PTR, _I32, _I32, _PTR]),
@@ -512,6 +522,29 @@ def talker_post_attention_workspace_init(workspace, workspace_bytes, stream=0):
 def talker_post_attention_m1(op, workspace, workspace_bytes, status=None, stream=0):
     _check(lib().qm_talker_post_attention_m1(C.byref(op), _addr(workspace), workspace_bytes, _addr(status), stream),
            "qm_talker_post_attention_m1")
+
+
+def talker_layer_step(q, k, v, gq, gk, cos, sin, q_rot, cache, page_table, max_pages, context, q_heads, position, sliding_window,
+                      scale, eps, attention_workspace, attention_workspace_bytes, post):
+    """qm_talker_layer_step: the arguments of decode_step_fused and a TalkerPostAttention.  Everything named must outlive the
+    descriptor (the cache descriptor is kept with it)."""
+    step = TalkerLayerStep()
+    for name, tensor in (("q", q), ("k", k), ("v", v), ("q_norm_w", gq), ("k_norm_w", gk), ("cos_row", cos), ("sin_row", sin),
+                         ("q_rotated_out", q_rot), ("page_table", page_table), ("attention_workspace", attention_workspace),
+                         ("context", context)):
+        setattr(step, name, _addr(tensor))
+    step._cache = cache
+    step.cache = C.pointer(cache)
+    step.attention_workspace_bytes = attention_workspace_bytes
+    step.max_pages, step.q_heads, step.position, step.sliding_window = max_pages, q_heads, position, sliding_window
+    step.scale, step.epsilon = scale, eps
+    step.post = post
+    return step
+
+
+def talker_layer_step_m1(step, workspace, workspace_bytes, status=None, stream=0):
+    _check(lib().qm_talker_layer_step_m1(C.byref(step), _addr(workspace), workspace_bytes, _addr(status), stream),
+           "qm_talker_layer_step_m1")
 
 
 def predictor_transpose(x, out, rows, heads, stream=0):

@@ -209,7 +209,8 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
     // layer's RMSNorm + Q/K/V — is one launch where the checkpoint has the geometry that launch serves (same bits).
     int32_t by_operators = 0;
     op_check(qm_get_option(QM_OPT_TALKER_LAYER_OPERATORS, &by_operators), "talker layer option");
-    const bool chained = e.chain_geometry && by_operators == 0;
+    const bool chained = e.chain_geometry && by_operators != 1;
+    const bool merge_in_chain = chained && by_operators == 0;   // the attention's split records are combined by the launch that follows it
     for (size_t index = 0; index < e.layers.size(); ++index) {
         Layer& w = e.layers[index];
         qm_kv_cache cache = flat_cache_of(e, w);
@@ -220,11 +221,12 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
                                        e.k.u16(), e.v.u16(), kHidden, e.q_dim, e.kv_dim, s),
                      "talker RMSNorm + Q/K/V");
         // launch_qk_norm_rope_cache_m1 + launch_attention (R17:17181-17195)
-        op_check(qm_decode_step_fused(e.q.u16(), e.k.u16(), e.v.u16(), w.q_norm.data(), w.k_norm.data(), e.cosine.u16(),
-                                      e.sine.u16(), e.q_rotated.u16(), &cache, nullptr, 1, e.context.u16(), e.q_heads,
-                                      position, -1, kScale, kEpsilon, e.workspace.raw(), e.workspace.bytes(),
-                                      static_cast<uint32_t*>(e.status.raw()), s),
-                 "talker norm/RoPE/append + attention");
+        if (!merge_in_chain)
+            op_check(qm_decode_step_fused(e.q.u16(), e.k.u16(), e.v.u16(), w.q_norm.data(), w.k_norm.data(), e.cosine.u16(),
+                                          e.sine.u16(), e.q_rotated.u16(), &cache, nullptr, 1, e.context.u16(), e.q_heads,
+                                          position, -1, kScale, kEpsilon, e.workspace.raw(), e.workspace.bytes(),
+                                          static_cast<uint32_t*>(e.status.raw()), s),
+                     "talker norm/RoPE/append + attention");
         if (chained) {
             qm_talker_post_attention op = {};
             op.context = e.context.u16(); op.hidden = current->u16();
@@ -241,9 +243,25 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
             }
             op.hidden_columns = kHidden; op.q_columns = e.q_dim; op.kv_columns = e.kv_dim; op.intermediate_columns = e.intermediate;
             op.epsilon = kEpsilon;
-            op_check(qm_talker_post_attention_m1(&op, e.chain_workspace.raw(), static_cast<int64_t>(e.chain_workspace.bytes()),
+            if (merge_in_chain) {
+                qm_talker_layer_step step = {};
+                step.q = e.q.u16(); step.k = e.k.u16(); step.v = e.v.u16();
+                step.q_norm_w = w.q_norm.data(); step.k_norm_w = w.k_norm.data();
+                step.cos_row = e.cosine.u16(); step.sin_row = e.sine.u16(); step.q_rotated_out = e.q_rotated.u16();
+                step.cache = &cache; step.page_table = nullptr; step.max_pages = 1;
+                step.attention_workspace = e.workspace.raw(); step.attention_workspace_bytes = e.workspace.bytes();
+                step.context = e.context.u16();
+                step.q_heads = e.q_heads; step.position = position; step.sliding_window = -1;
+                step.scale = kScale; step.epsilon = kEpsilon;
+                step.post = op;
+                op_check(qm_talker_layer_step_m1(&step, e.chain_workspace.raw(), static_cast<int64_t>(e.chain_workspace.bytes()),
                                                  static_cast<uint32_t*>(e.status.raw()), s),
-                     "talker o_proj ... next Q/K/V");
+                         "talker norm/RoPE/append + attention ... next Q/K/V");
+            } else {
+                op_check(qm_talker_post_attention_m1(&op, e.chain_workspace.raw(), static_cast<int64_t>(e.chain_workspace.bytes()),
+                                                     static_cast<uint32_t*>(e.status.raw()), s),
+                         "talker o_proj ... next Q/K/V");
+            }
             std::swap(current, next);
             continue;
         }

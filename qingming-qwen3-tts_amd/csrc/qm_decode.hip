@@ -29,6 +29,7 @@
 #include "qm_device.h"
 #include "qm_host.h"
 #include "qm_norm_rope_head.h"
+#include "qm_decode_step.h"
 
 #include <stdlib.h>
 
@@ -40,7 +41,7 @@ constexpr int kDecodeThreads = 256;
 constexpr int kDecodeWaves = 4;
 constexpr int kRowStreams = 16;  // 4 waves x 4 DPP rows
 constexpr int kMaxTilesPerBlock = 64;
-constexpr int kMergeRound = 32;        // splits merged per round of loads in the merge kernel
+constexpr int kMergeRound = kDecodeMergeRound;   // splits merged per round of loads in the merge kernel
 // Calls whose contexts may exceed this many bytes (streams x max_seq_len x bytes per token) read
 // K and V with the non-temporal hint.  Ragged batches of 256..4096 tokens, plain / non-temporal:
 // 16 streams (156 MiB read, bound 256 MiB) 32.5 / 32.8 us, 32 (290, 512) 54.2 / 55.2 us,
@@ -550,12 +551,12 @@ int32_t launch_split(const DecodeParams& prm, const qm_kv_cache& cache, int n_st
 
 template <int G>
 int32_t launch_decode(const DecodeParams& prm, const qm_kv_cache& cache, int n_streams, bool streaming,
-                      hipStream_t stream) {
+                      hipStream_t stream, bool merge) {
     const bool generic = prm.head_groups_per_kv > 1 || prm.rows_cache_before >= 0;
     int32_t rc = streaming ? launch_split<G, true>(prm, cache, n_streams, generic, stream)
                            : launch_split<G, false>(prm, cache, n_streams, generic, stream);
     if (rc != QM_OK) return rc;
-    if (prm.max_splits > 1) {
+    if (merge && prm.max_splits > 1) {
         const dim3 grid(cache.kv_heads * prm.head_groups_per_kv, n_streams);
         if (generic) hipLaunchKernelGGL((decode_merge_kernel<G, true>), grid, dim3(G * kDim), 0, stream, prm);
         else hipLaunchKernelGGL((decode_merge_kernel<G, false>), grid, dim3(G * kDim), 0, stream, prm);
@@ -575,7 +576,7 @@ int32_t decode_common(const uint16_t* query, const qm_kv_cache* cache, const int
                       int32_t key_start, int32_t key_end, int32_t max_seq_len, uint16_t* out,
                       int32_t q_heads, float scale, void* workspace, size_t workspace_bytes,
                       uint32_t* status_dev, void* hip_stream, const DecodeParams* step = nullptr,
-                      const RowsOfOneSequence* rows = nullptr) {
+                      const RowsOfOneSequence* rows = nullptr, DecodeSplitInfo* unmerged = nullptr) {
     if ((!query && !step) || !out) return QM_ERR_NULL;
     int32_t rc = check_cache(cache, max_pages);
     if (rc != QM_OK) return rc;
@@ -633,10 +634,17 @@ int32_t decode_common(const uint16_t* query, const qm_kv_cache* cache, const int
     if (loads == 2) streaming = true;
 
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    if (unmerged) {
+        // the caller combines the records itself (one stream): how many there are, as the merge kernel counts them
+        const int tiles = key_end > key_start ? (key_end - 1) / kTile - key_start / kTile + 1 : 0;
+        unmerged->max_splits = plan.max_splits;
+        unmerged->splits = std::min((tiles + plan.tiles_per_block - 1) / plan.tiles_per_block, plan.max_splits);
+        unmerged->records = plan.max_splits > 1 ? static_cast<const float*>(workspace) : nullptr;
+    }
     switch (heads_per_block) {
-        case 1: return launch_decode<1>(prm, *cache, n_streams, streaming, s);
-        case 2: return launch_decode<2>(prm, *cache, n_streams, streaming, s);
-        case 4: return launch_decode<4>(prm, *cache, n_streams, streaming, s);
+        case 1: return launch_decode<1>(prm, *cache, n_streams, streaming, s, !unmerged);
+        case 2: return launch_decode<2>(prm, *cache, n_streams, streaming, s, !unmerged);
+        case 4: return launch_decode<4>(prm, *cache, n_streams, streaming, s, !unmerged);
     }
     return QM_ERR_GEOMETRY;
 }
@@ -708,7 +716,9 @@ extern "C" int32_t qm_decode_attention_ragged(
                              status_dev, hip_stream);
 }
 
-extern "C" int32_t qm_decode_step_fused(
+namespace qm {
+
+int32_t decode_step(
     const uint16_t* q, const uint16_t* k, const uint16_t* v,
     const uint16_t* q_norm_w, const uint16_t* k_norm_w,
     const uint16_t* cos_row, const uint16_t* sin_row,
@@ -716,7 +726,7 @@ extern "C" int32_t qm_decode_step_fused(
     const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
     uint16_t* context_out,
     int32_t q_heads, int32_t position, int32_t sliding_window, float scale, float epsilon,
-    void* workspace, size_t workspace_bytes, uint32_t* status_dev, void* hip_stream) {
+    void* workspace, size_t workspace_bytes, uint32_t* status_dev, void* hip_stream, DecodeSplitInfo* unmerged) {
     if (!q || !k || !v || !q_norm_w || !k_norm_w || !cos_row || !sin_row) return QM_ERR_NULL;
     if (position < 0) return QM_ERR_SLOT_RANGE;
     const int32_t key_end = position + 1;
@@ -726,14 +736,30 @@ extern "C" int32_t qm_decode_step_fused(
         if (position / cache->page_size >= max_pages) return QM_ERR_SLOT_RANGE;
         if (!page_table && position / cache->page_size >= cache->n_pages) return QM_ERR_SLOT_RANGE;
     }
-    qm::DecodeParams step = {};
+    DecodeParams step = {};
     step.step_q = q; step.step_k = k; step.step_v = v;
     step.step_q_norm = q_norm_w; step.step_k_norm = k_norm_w;
     step.step_cos = cos_row; step.step_sin = sin_row;
     step.step_q_rotated = q_rotated_out;
     step.step_position = position; step.step_epsilon = epsilon;
-    return qm::decode_common(nullptr, cache, page_table, max_pages, nullptr, 1, key_start, key_end, key_end,
-                             context_out, q_heads, scale, workspace, workspace_bytes, status_dev, hip_stream, &step);
+    return decode_common(nullptr, cache, page_table, max_pages, nullptr, 1, key_start, key_end, key_end,
+                         context_out, q_heads, scale, workspace, workspace_bytes, status_dev, hip_stream, &step, nullptr, unmerged);
+}
+
+}  // namespace qm
+
+extern "C" int32_t qm_decode_step_fused(
+    const uint16_t* q, const uint16_t* k, const uint16_t* v,
+    const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+    const uint16_t* cos_row, const uint16_t* sin_row,
+    uint16_t* q_rotated_out,
+    const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    uint16_t* context_out,
+    int32_t q_heads, int32_t position, int32_t sliding_window, float scale, float epsilon,
+    void* workspace, size_t workspace_bytes, uint32_t* status_dev, void* hip_stream) {
+    return qm::decode_step(q, k, v, q_norm_w, k_norm_w, cos_row, sin_row, q_rotated_out, cache, page_table, max_pages, context_out,
+                           q_heads, position, sliding_window, scale, epsilon, workspace, workspace_bytes, status_dev, hip_stream,
+                           nullptr);
 }
 
 extern "C" size_t qm_attention_rows_workspace_bytes(int32_t query_length, int32_t q_heads, int32_t kv_heads,

@@ -36,7 +36,7 @@ std::atomic<int32_t> g_options[QM_OPT_COUNT] = {
     {0},   // QM_OPT_PREDICTOR_FRAME_OPERATORS (0 = the frame's M = 1 steps as one launch, 1 = operator by operator)
     {0},   // QM_OPT_PREDICTOR_FRAME_SPIN_LIMIT (0 = the kernel's own bound)
     {0},   // QM_OPT_LINEAR_ROWS_KERNEL (0 = matrix cores for 16 or more token rows, 1 = always the exact chain)
-    {0},   // QM_OPT_TALKER_LAYER_OPERATORS (0 = one launch between two attentions, 1 = operator by operator)
+    {0},   // QM_OPT_TALKER_LAYER_OPERATORS (0 = two launches per layer, 2 = three, 1 = operator by operator)
 };
 
 // a thread's own values: -1 = none, the process-wide value applies

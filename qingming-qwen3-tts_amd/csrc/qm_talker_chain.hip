@@ -39,6 +39,7 @@
 #include "qm_device.h"
 #include "qm_host.h"
 #include "qm_resident.h"
+#include "qm_decode_step.h"
 
 #include <atomic>
 #include <type_traits>
@@ -86,7 +87,8 @@ constexpr int kTkWsAbort = 1;
 constexpr int kTkWsAttn = 64;
 constexpr int kTkWsAct = kTkWsAttn + kTkHidden;
 constexpr int kTkWsHidden = kTkWsAct + kTkInter;
-constexpr int kTkWsWords = kTkWsHidden + kTkHidden;
+constexpr int kTkWsContext = kTkWsHidden + kTkHidden;   // the attention's output, when this launch combines its splits
+constexpr int kTkWsWords = kTkWsContext + kTkQDim;
 constexpr int64_t kTkWsBytes = (static_cast<int64_t>(kTkWsWords) * 4 + 255) / 256 * 256;
 constexpr uint32_t kTkTagsPerLaunch = 4;
 
@@ -109,6 +111,12 @@ struct TkParams {
     float epsilon;
     unsigned spin_limit;
     int has_next;
+    // The attention ran without its merge launch (qm_talker_layer_step_m1): the first eight blocks combine the split
+    // records of one kv head each and hand the context to everybody; NULL: `context` holds it already.
+    const float* attention_records;
+    int attention_splits;
+    int attention_max_splits;
+    uint16_t* context_out;
 };
 
 struct TkShared {
@@ -351,6 +359,55 @@ __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p)
         if (qkv_row >= kTkQDim + kTkKvDim) { qkv_bias = p.next_bias[2]; qkv_out = p.next_out[2]; qkv_row -= kTkQDim + kTkKvDim; }
         else if (qkv_row >= kTkQDim) { qkv_bias = p.next_bias[1]; qkv_out = p.next_out[1]; qkv_row -= kTkQDim; }
 
+        if (p.attention_records && b < kTkKvDim / 128) {
+            // ---- the attention's splits, combined as decode_merge_kernel<2> combines them (same statistics, same
+            // order, same bits): block h the two query heads of kv head h, thread (g, d) one output ----
+            constexpr int kRecord = 2 * 128 + 4;                 // acc[2][128], max[2], sum[2]
+            const int g = tid >> 7, d = tid & 127;
+            const int n = p.attention_splits;
+            const float* records = p.attention_records + static_cast<int64_t>(b) * p.attention_max_splits * kRecord;
+            float* const stat_m = lin_x;                            // [32][2]: the input vector is not in use yet
+            float* const stat_l = lin_x + 2 * kDecodeMergeRound;
+            // (eight records at a time through one small loop: instructions a block executes once cost tens of cycles
+            // each to fetch, and this runs while the first weights are still on their way)
+            constexpr int kChunk = 8;
+            float part[kChunk];
+            const float* column = records + g * 128 + d;
+#pragma unroll
+            for (int u = 0; u < kChunk; ++u) part[u] = u < n ? column[u * kRecord] : 0.0f;
+            if (tid < 2 * n) {
+                const float* rec = records + (tid >> 1) * kRecord;
+                stat_m[tid] = rec[2 * 128 + (tid & 1)];
+                stat_l[tid] = rec[2 * 128 + 2 + (tid & 1)];
+            }
+            alive = compute_barrier();
+            if (alive) {
+                float mm = -INFINITY;
+                for (int s = 0; s < n; ++s) mm = fmaxf(mm, stat_m[2 * s + g]);
+                const float m_ref = mm == -INFINITY ? 0.0f : mm;
+                float ll = 0.0f, aa = 0.0f;
+#pragma unroll 1
+                for (int first = 0; first < n; first += kChunk) {
+                    if (first > 0) {
+#pragma unroll
+                        for (int u = 0; u < kChunk; ++u) part[u] = first + u < n ? column[(first + u) * kRecord] : 0.0f;
+                    }
+#pragma unroll
+                    for (int u = 0; u < kChunk; ++u) {
+                        if (first + u < n) {
+                            const float w = fast_exp2((stat_m[2 * (first + u) + g] - m_ref) * kLog2e);
+                            ll = fmaf(stat_l[2 * (first + u) + g], w, ll);
+                            aa = fmaf(part[u], w, aa);
+                        }
+                    }
+                }
+                const uint16_t bits = f2bf(ll > 0.0f ? aa / ll : 0.0f);
+                agent_store(ws + kTkWsContext + 256 * b + tid, (tag(3) << 16) | bits);
+                if (p.context_out) p.context_out[256 * b + tid] = bits;
+                alive = compute_barrier();                          // the statistics have been read: the input vector may be written
+            }
+        }
+
         // The units in order, through ONE copy of each piece of code (a kernel's instructions are fetched as they are
         // first executed, tens of cycles each: straight-line code for twelve units ran several times slower than this
         // loop).  Before the first unit of an operator its input vector is formed, after the last the outputs leave.
@@ -359,8 +416,14 @@ __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p)
             if (u == kTkUnitO) {
                 // ---- o_proj (R17:17203-17210): the attention's output is given ----
                 uint32_t raw[kPerThread];
+                if (p.attention_records) {
+                    alive = poll_words<kPerThread>(ws + kTkWsContext, tag(3), abort_word, spin_limit, raw);
+                    if (!alive) give_up();
+                } else {
 #pragma unroll
-                for (int i = 0; i < kPerThread; ++i) raw[i] = p.context[tid + kTkComputeThreads * i];
+                    for (int i = 0; i < kPerThread; ++i) raw[i] = p.context[tid + kTkComputeThreads * i];
+                }
+                if (!alive) break;
                 if (p.o_bias && tid < 8) sh.bias[tid] = bf2f(p.o_bias[8 * b + tid]);
 #pragma unroll
                 for (int i = 0; i < kPerThread; ++i) lin_x[tid + kTkComputeThreads * i] = bf2f(static_cast<uint16_t>(raw[i]));
@@ -478,9 +541,12 @@ extern "C" int32_t qm_talker_post_attention_workspace_init(void* workspace, int6
     return launch_status();
 }
 
-extern "C" int32_t qm_talker_post_attention_m1(const qm_talker_post_attention* op, void* workspace, int64_t workspace_bytes,
-                                               uint32_t* status_dev, void* hip_stream) {
-    using namespace qm;
+namespace qm {
+namespace {
+
+// The launch; with `attention` the kernel first combines that decode step's split records into `context_out`.
+int32_t launch_chain(const qm_talker_post_attention* op, void* workspace, int64_t workspace_bytes, uint32_t* status_dev,
+                     void* hip_stream, const DecodeSplitInfo* attention, uint16_t* context_out) {
     if (!op || !workspace) return QM_ERR_NULL;
     if (workspace_bytes < kTkWsBytes) return QM_ERR_WORKSPACE;
     if (reinterpret_cast<uintptr_t>(workspace) & 255) return QM_ERR_GEOMETRY;
@@ -511,6 +577,13 @@ extern "C" int32_t qm_talker_post_attention_m1(const qm_talker_post_attention* o
     prm.status = status_dev;
     prm.epsilon = op->epsilon;
     prm.has_next = has_next ? 1 : 0;
+    if (attention && attention->records) {
+        if (attention->splits < 1 || attention->splits > kDecodeMergeRound || attention->splits > attention->max_splits) return QM_ERR_ARGUMENT;
+        prm.attention_records = attention->records;
+        prm.attention_splits = attention->splits;
+        prm.attention_max_splits = attention->max_splits;
+        prm.context_out = context_out;
+    }
     const int32_t spin_option = option_value(QM_OPT_PREDICTOR_FRAME_SPIN_LIMIT);
     prm.spin_limit = spin_option > 0 ? static_cast<unsigned>(spin_option) : kTkSpinLimit;
 
@@ -535,4 +608,36 @@ extern "C" int32_t qm_talker_post_attention_m1(const qm_talker_post_attention* o
     if (holds < kTkBlocks) return QM_ERR_NO_DEVICE;
     hipLaunchKernelGGL(talker_chain_kernel, dim3(kTkBlocks), dim3(kTkThreads), kTkLdsBytes, static_cast<hipStream_t>(hip_stream), prm);
     return launch_status();
+}
+
+}  // namespace
+}  // namespace qm
+
+extern "C" int32_t qm_talker_post_attention_m1(const qm_talker_post_attention* op, void* workspace, int64_t workspace_bytes,
+                                               uint32_t* status_dev, void* hip_stream) {
+    return qm::launch_chain(op, workspace, workspace_bytes, status_dev, hip_stream, nullptr, nullptr);
+}
+
+extern "C" int32_t qm_talker_layer_step_m1(const qm_talker_layer_step* step, void* workspace, int64_t workspace_bytes,
+                                           uint32_t* status_dev, void* hip_stream) {
+    using namespace qm;
+    if (!step || !workspace || !step->context) return QM_ERR_NULL;
+    if (step->q_heads != kTkQDim / 128 || !step->cache || step->cache->kv_heads != kTkKvDim / 128) return QM_ERR_GEOMETRY;
+    // validate the second launch's arguments before the first is made: a step is made whole or not at all
+    qm_talker_post_attention post = step->post;
+    post.context = step->context;
+    if (workspace_bytes < kTkWsBytes) return QM_ERR_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(workspace) & 255) return QM_ERR_GEOMETRY;
+    if (post.hidden_columns != kTkHidden || post.q_columns != kTkQDim || post.kv_columns != kTkKvDim
+        || post.intermediate_columns != kTkInter)
+        return QM_ERR_GEOMETRY;
+    if (!post.hidden || !post.o_weight || !post.post_norm || !post.gate_weight || !post.up_weight || !post.down_weight || !post.hidden_out)
+        return QM_ERR_NULL;
+    DecodeSplitInfo info = {};
+    const int32_t rc = decode_step(step->q, step->k, step->v, step->q_norm_w, step->k_norm_w, step->cos_row, step->sin_row,
+                                   step->q_rotated_out, step->cache, step->page_table, step->max_pages, step->context, step->q_heads,
+                                   step->position, step->sliding_window, step->scale, step->epsilon, step->attention_workspace,
+                                   step->attention_workspace_bytes, status_dev, hip_stream, &info);
+    if (rc != QM_OK) return rc;
+    return launch_chain(&post, workspace, workspace_bytes, status_dev, hip_stream, &info, step->context);
 }

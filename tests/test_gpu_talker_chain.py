@@ -171,3 +171,83 @@ def test_giving_up_and_argument_errors(layer, qm):
     torch.cuda.synchronize()
     assert L.qm_talker_post_attention_workspace_init(None, layer.ws_bytes, None) == -1
     assert L.qm_talker_post_attention_workspace_init(p, layer.ws_bytes - 1, None) == -4
+
+
+@pytest.mark.parametrize("ctx,paged", [(1, False), (17, False), (130, True), (300, False), (2048, False), (2048, True), (5000, True)])
+def test_layer_step_in_two_launches_equals_attention_then_the_one_launch(oracle, qm, dev, layer, ctx, paged):
+    """qm_talker_layer_step_m1 — the attention without its merge launch, its split records combined by the first blocks of
+    the launch that follows — leaves what qm_decode_step_fused followed by qm_talker_post_attention_m1 leaves: context,
+    rotated query, cache, hidden state and the next layer's Q/K/V, bit for bit (one split at short contexts, up to 32)."""
+    import numpy as np
+    import torch
+    from qm_testlib import SCALE, PagedPool, to_u16
+    pos = ctx - 1
+    q = to_dev(oracle.normal_bf16((16, 128), 8000 + ctx), dev)
+    k = to_dev(oracle.normal_bf16((8, 128), 8001 + ctx), dev)
+    v = to_dev(oracle.normal_bf16((8, 128), 8002 + ctx), dev)
+    gq = to_dev(oracle.normal_bf16((128,), 8003, mean=1.0, std=0.1), dev)
+    gk = to_dev(oracle.normal_bf16((128,), 8004, mean=1.0, std=0.1), dev)
+    cos_h, sin_h = oracle.rope_table(1, pos)
+    cos, sin = to_dev(cos_h, dev), to_dev(sin_h, dev)
+
+    def make():
+        if paged:
+            pool = PagedPool(oracle, [ctx], seed=8100 + ctx)
+            kd, vd, cache, table = pool.device(qm, dev)
+            return kd, vd, cache, table, pool.max_pages
+        kd = to_dev(oracle.normal_bf16((8, ctx + 3, 128), 8200 + ctx), dev)
+        vd = to_dev(oracle.normal_bf16((8, ctx + 3, 128), 8201 + ctx), dev)
+        return kd, vd, qm.flat_cache(kd, vd, 8, ctx + 3), None, 1
+
+    ws_bytes = qm.decode_workspace_bytes(1, 16, 8, ctx)
+    ws = torch.zeros(ws_bytes // 4 + 1, dtype=torch.float32, device=dev)
+    z = lambda *shape: torch.full(shape, 0x7fc0, dtype=torch.int16, device=dev)
+    # three launches
+    kd1, vd1, cache1, table1, mp = make()
+    qrot1, ctx1 = z(16, 128), z(16, 128)
+    qm.decode_step_fused(q, k, v, gq, gk, cos, sin, qrot1, cache1, table1, mp, ctx1, 16, pos, -1, SCALE, 1e-6, ws, ws_bytes,
+                         layer.status)
+    layer.context.copy_(ctx1.view(-1))
+    for t in layer.want.values():
+        t.fill_(0x7fc0)
+    saved, layer.got = layer.got, layer.want
+    layer.one_launch()
+    layer.got = saved
+    torch.cuda.synchronize()
+    # two launches
+    kd2, vd2, cache2, table2, _ = make()
+    qrot2, ctx2 = z(16, 128), z(16, 128)
+    for t in layer.got.values():
+        t.fill_(0x7fc0)
+    step = qm.talker_layer_step(q, k, v, gq, gk, cos, sin, qrot2, cache2, table2, mp, ctx2, 16, pos, -1, SCALE, 1e-6, ws, ws_bytes,
+                                layer.descriptor())
+    for _ in range(2):                                     # a second step finds the workspaces as the first left them
+        qm.talker_layer_step_m1(step, layer.ws, layer.ws_bytes, layer.status)
+        torch.cuda.synchronize()
+        assert int(layer.status.item()) == 0
+        assert np.array_equal(to_u16(ctx2), to_u16(ctx1)) and np.array_equal(to_u16(qrot2), to_u16(qrot1))
+        assert np.array_equal(to_u16(kd2), to_u16(kd1)) and np.array_equal(to_u16(vd2), to_u16(vd1))
+        assert layer.same()
+
+
+def test_layer_step_argument_errors(oracle, qm, dev, layer):
+    import ctypes as C
+    import torch
+    from qm_testlib import SCALE
+    z = torch.zeros((16, 128), dtype=torch.int16, device=dev)
+    kv = torch.zeros((8, 32, 128), dtype=torch.int16, device=dev)
+    cache = qm.flat_cache(kv, kv.clone(), 8, 32)
+    make = lambda position=3, heads=16: qm.talker_layer_step(z, z, z, z, z, z, z, None, cache, None, 1, z, heads, position, -1, SCALE, 1e-6,
+                                                             None, 0, layer.descriptor())
+    call = lambda step, ws=layer.ws.data_ptr(), nbytes=layer.ws_bytes: qm.lib().qm_talker_layer_step_m1(C.byref(step), ws, nbytes, None, None)
+    assert call(make(32)) == -3 and call(make(heads=8)) == -2
+    assert call(make(), None) == -1 and call(make(), nbytes=layer.ws_bytes - 256) == -4
+    bad = make()
+    bad.post.hidden_columns = 1024
+    assert call(bad) == -2                                 # nothing is launched when the second launch's arguments are wrong
+    bad = make()
+    bad.context = None
+    assert call(bad) == -1
+    assert call(make()) == 0
+    torch.cuda.synchronize()
+    assert qm.lib().qm_talker_layer_step_m1(None, layer.ws.data_ptr(), layer.ws_bytes, None, None) == -1
