@@ -634,17 +634,19 @@ int32_t decode_common(const uint16_t* query, const qm_kv_cache* cache, const int
     if (loads == 2) streaming = true;
 
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    // The caller combines the records itself (one stream) if one round of the merge holds them; a context so long that
+    // it does not is merged here as always and handed over as if it had been a single split.
+    const bool leave_unmerged = unmerged && plan.max_splits > 1 && plan.max_splits <= kMergeRound;
     if (unmerged) {
-        // the caller combines the records itself (one stream): how many there are, as the merge kernel counts them
         const int tiles = key_end > key_start ? (key_end - 1) / kTile - key_start / kTile + 1 : 0;
         unmerged->max_splits = plan.max_splits;
-        unmerged->splits = std::min((tiles + plan.tiles_per_block - 1) / plan.tiles_per_block, plan.max_splits);
-        unmerged->records = plan.max_splits > 1 ? static_cast<const float*>(workspace) : nullptr;
+        unmerged->splits = std::min((tiles + plan.tiles_per_block - 1) / plan.tiles_per_block, plan.max_splits);   // as the merge kernel counts them
+        unmerged->records = leave_unmerged ? static_cast<const float*>(workspace) : nullptr;
     }
     switch (heads_per_block) {
-        case 1: return launch_decode<1>(prm, *cache, n_streams, streaming, s, !unmerged);
-        case 2: return launch_decode<2>(prm, *cache, n_streams, streaming, s, !unmerged);
-        case 4: return launch_decode<4>(prm, *cache, n_streams, streaming, s, !unmerged);
+        case 1: return launch_decode<1>(prm, *cache, n_streams, streaming, s, !leave_unmerged);
+        case 2: return launch_decode<2>(prm, *cache, n_streams, streaming, s, !leave_unmerged);
+        case 4: return launch_decode<4>(prm, *cache, n_streams, streaming, s, !leave_unmerged);
     }
     return QM_ERR_GEOMETRY;
 }

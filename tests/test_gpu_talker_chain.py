@@ -230,6 +230,16 @@ def test_layer_step_in_two_launches_equals_attention_then_the_one_launch(oracle,
         assert layer.same()
 
 
+def test_layer_step_with_more_splits_than_one_merge_round(oracle, qm, dev, layer):
+    """Blocks of four tiles cut a context of 3000 tokens into 47 splits, more than the 32 records one round of the merge takes:
+    the attention then keeps its own merge launch, and the step still leaves the same bits."""
+    qm.set_option(qm.OPT_DECODE_TILES_PER_BLOCK, 4)
+    try:
+        test_layer_step_in_two_launches_equals_attention_then_the_one_launch(oracle, qm, dev, layer, 3000, True)
+    finally:
+        qm.set_option(qm.OPT_DECODE_TILES_PER_BLOCK, 0)
+
+
 def test_layer_step_argument_errors(oracle, qm, dev, layer):
     import ctypes as C
     import torch
