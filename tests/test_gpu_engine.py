@@ -134,16 +134,16 @@ def test_engine_decode_steps_match_the_oracle_chain(engine, oracle, qm, dev, tmp
 
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_engine_decode_in_the_talkers_geometry_takes_one_launch_between_attentions(engine, qm, dev, tmp_path, with_bias):
-    """With the talker's real intermediate size (6144) the decode step runs qm_talker_post_attention_m1 between two
-    attentions; the final hidden vectors and the caches equal, bit for bit, what the operator-by-operator step (held
-    against the oracle above) leaves."""
+    """With the talker's real intermediate size (6144) a layer of the decode step is two launches (qm_talker_layer_step_m1;
+    three with QM_OPT_TALKER_LAYER_OPERATORS = 2: the attention with its merge, then qm_talker_post_attention_m1); the final
+    hidden vectors and the caches equal, bit for bit, what the operator-by-operator step (held against the oracle above) leaves."""
     import ctypes as C
     import torch
     layers = 3
     _checkpoint(str(tmp_path), with_bias, inter=6144, layers=layers)
     hip = C.CDLL("libamdhip64.so")
     results = []
-    for by_operators in (1, 0):
+    for by_operators in (1, 0, 2):
         qm.set_option(qm.OPT_TALKER_LAYER_OPERATORS, by_operators)
         try:
             talker = engine.Talker(str(tmp_path), MAX_CACHE)
@@ -176,8 +176,8 @@ def test_engine_decode_in_the_talkers_geometry_takes_one_launch_between_attentio
             results.append(outputs)
         finally:
             qm.set_option(qm.OPT_TALKER_LAYER_OPERATORS, 0)
-    assert len(results[0]) == len(results[1]) == 3 + 2 * layers
-    assert all(torch.equal(a, b) for a, b in zip(*results))
+    assert len(results[0]) == len(results[1]) == len(results[2]) == 3 + 2 * layers
+    assert all(torch.equal(a, b) and torch.equal(a, c) for a, b, c in zip(*results))
     assert len({bytes(o.numpy().tobytes()) for o in results[0][:3]}) == 3          # (three different steps)
 
 
