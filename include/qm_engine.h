@@ -84,6 +84,12 @@ int32_t qm_talker_cache(qm_talker* engine, int32_t layer, uint16_t** key_cache, 
  */
 int32_t qm_talker_decode(qm_talker* engine, const uint16_t* input_device, const uint16_t* cosine,
                          const uint16_t* sine, int32_t decode_index, const uint16_t** final_hidden_device);
+/* The same with the RoPE row of the step's position on the DEVICE (cosine_device, sine_device [128], valid until the
+ * step has run): for a loop that uploaded the rows of all its positions once, as qm_generate does, instead of two
+ * small host-to-device copies in front of every step. */
+int32_t qm_talker_decode_device_rope(qm_talker* engine, const uint16_t* input_device, const uint16_t* cosine_device,
+                                     const uint16_t* sine_device, int32_t decode_index,
+                                     const uint16_t** final_hidden_device);
 /*
  * NativeTalkerEngine::prefill (R17:16561-16800): zeroes the caches, then sends the prompt's `rows`
  * token rows through every layer — RMSNorm, q/k/v projections, QK-norm + RoPE, causal attention

@@ -193,16 +193,24 @@ static qm_kv_cache flat_cache_of(const qm_talker& e, const Layer& w) {
     return cache;
 }
 
+// `rope_on_device`: cosine and sine are device rows that stay valid until the step has run (a caller that uploaded the
+// rows of all its positions once); else host rows, copied into the engine's own.
 static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const uint16_t* cosine, const uint16_t* sine,
-                              int decode_index) {
+                              int decode_index, bool rope_on_device = false) {
     if (!input_device || !cosine || !sine) throw ApiError(QM_ERR_NULL, "talker device decode input is null");
     if (decode_index < 0) throw ApiError(QM_ERR_ARGUMENT, "negative decode index");
     const int position = e.prefill_length + decode_index;
     if (position >= e.max_cache) throw ApiError(QM_ERR_SLOT_RANGE, "talker device decode cache overflow");
     hipStream_t s = e.stream;
     hip_check(hipMemcpyAsync(e.hidden_a.raw(), input_device, kHidden * 2, hipMemcpyDeviceToDevice, s), "decode input copy");
-    hip_check(hipMemcpyAsync(e.cosine.raw(), cosine, kHeadDim * 2, hipMemcpyHostToDevice, s), "decode cosine");
-    hip_check(hipMemcpyAsync(e.sine.raw(), sine, kHeadDim * 2, hipMemcpyHostToDevice, s), "decode sine");
+    const uint16_t* cos_row = cosine;
+    const uint16_t* sin_row = sine;
+    if (!rope_on_device) {
+        hip_check(hipMemcpyAsync(e.cosine.raw(), cosine, kHeadDim * 2, hipMemcpyHostToDevice, s), "decode cosine");
+        hip_check(hipMemcpyAsync(e.sine.raw(), sine, kHeadDim * 2, hipMemcpyHostToDevice, s), "decode sine");
+        cos_row = e.cosine.u16();
+        sin_row = e.sine.u16();
+    }
     DeviceBuffer* current = &e.hidden_a;
     DeviceBuffer* next = &e.hidden_b;
     // What lies between two attentions — o_proj, residual + post-norm + gate/up/SwiGLU, down_proj + residual and the next
@@ -222,8 +230,8 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
                      "talker RMSNorm + Q/K/V");
         // launch_qk_norm_rope_cache_m1 + launch_attention (R17:17181-17195)
         if (!merge_in_chain)
-            op_check(qm_decode_step_fused(e.q.u16(), e.k.u16(), e.v.u16(), w.q_norm.data(), w.k_norm.data(), e.cosine.u16(),
-                                          e.sine.u16(), e.q_rotated.u16(), &cache, nullptr, 1, e.context.u16(), e.q_heads,
+            op_check(qm_decode_step_fused(e.q.u16(), e.k.u16(), e.v.u16(), w.q_norm.data(), w.k_norm.data(), cos_row,
+                                          sin_row, e.q_rotated.u16(), &cache, nullptr, 1, e.context.u16(), e.q_heads,
                                           position, -1, kScale, kEpsilon, e.workspace.raw(), e.workspace.bytes(),
                                           static_cast<uint32_t*>(e.status.raw()), s),
                      "talker norm/RoPE/append + attention");
@@ -247,7 +255,7 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
                 qm_talker_layer_step step = {};
                 step.q = e.q.u16(); step.k = e.k.u16(); step.v = e.v.u16();
                 step.q_norm_w = w.q_norm.data(); step.k_norm_w = w.k_norm.data();
-                step.cos_row = e.cosine.u16(); step.sin_row = e.sine.u16(); step.q_rotated_out = e.q_rotated.u16();
+                step.cos_row = cos_row; step.sin_row = sin_row; step.q_rotated_out = e.q_rotated.u16();
                 step.cache = &cache; step.page_table = nullptr; step.max_pages = 1;
                 step.attention_workspace = e.workspace.raw(); step.attention_workspace_bytes = e.workspace.bytes();
                 step.context = e.context.u16();
@@ -469,6 +477,13 @@ extern "C" int32_t qm_talker_decode(qm_talker* engine, const uint16_t* input_dev
                                     const uint16_t* sine, int32_t decode_index, const uint16_t** final_hidden_device) {
     if (!engine || !final_hidden_device) return QM_ERR_NULL;
     return guarded([&] { *final_hidden_device = decode(*engine, input_device, cosine, sine, decode_index); });
+}
+
+extern "C" int32_t qm_talker_decode_device_rope(qm_talker* engine, const uint16_t* input_device, const uint16_t* cosine_device,
+                                                const uint16_t* sine_device, int32_t decode_index,
+                                                const uint16_t** final_hidden_device) {
+    if (!engine || !final_hidden_device) return QM_ERR_NULL;
+    return guarded([&] { *final_hidden_device = decode(*engine, input_device, cosine_device, sine_device, decode_index, true); });
 }
 
 extern "C" int32_t qm_talker_prefill(qm_talker* engine, const uint16_t* input_device, const uint16_t* cosine,

@@ -431,6 +431,16 @@ extern "C" int32_t qm_generate(qm_talker* talker, qm_final_head* head, qm_predic
         std::vector<uint16_t> decode_cos(static_cast<size_t>(decode_rows) * kHeadDim), decode_sin(decode_cos.size());
         if (decode_rows > 0)
             op_check(qm_rope_rows(decode_rows, prompt_rows, kHeadDim, 1000000.0, decode_cos.data(), decode_sin.data()), "decode rope rows");
+        // ... uploaded once: a decode step then starts without host-to-device copies in front of it
+        DeviceBuffer rope_device(2 * decode_cos.size() * sizeof(uint16_t) + 256);
+        uint16_t* const cos_device = rope_device.u16();
+        uint16_t* const sin_device = cos_device + decode_cos.size();
+        if (decode_rows > 0) {
+            hipStream_t stream = static_cast<hipStream_t>(qm_talker_stream(talker));
+            hip_check(hipMemcpyAsync(cos_device, decode_cos.data(), decode_cos.size() * 2, hipMemcpyHostToDevice, stream), "decode rope upload");
+            hip_check(hipMemcpyAsync(sin_device, decode_sin.data(), decode_sin.size() * 2, hipMemcpyHostToDevice, stream), "decode rope upload");
+            hip_check(hipStreamSynchronize(stream), "decode rope upload synchronize");
+        }
         int frames = 0;
         for (int frame = 0; frame < maximum_frames; ++frame) {
             // The final head's code stays on the device, where the predictor reads it: the host learns it together
@@ -454,8 +464,8 @@ extern "C" int32_t qm_generate(qm_talker* talker, qm_final_head* head, qm_predic
             std::memcpy(codes_out + static_cast<size_t>(frame) * kCodeGroups, frame_codes, sizeof frame_codes);
             ++frames;
             if (frame + 1 >= maximum_frames) break;
-            op_check(qm_talker_decode(talker, predictor->next_input.u16(), decode_cos.data() + static_cast<size_t>(frame) * kHeadDim,
-                                      decode_sin.data() + static_cast<size_t>(frame) * kHeadDim, frame, &hidden), "talker decode");
+            op_check(qm_talker_decode_device_rope(talker, predictor->next_input.u16(), cos_device + static_cast<size_t>(frame) * kHeadDim,
+                                                  sin_device + static_cast<size_t>(frame) * kHeadDim, frame, &hidden), "talker decode");
         }
         op_check(qm_talker_synchronize(talker), "generation synchronize");
         *frames_out = frames;

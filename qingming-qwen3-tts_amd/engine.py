@@ -26,6 +26,7 @@ _SIGNATURES = {
     "qm_talker_reset": (_I32, [_P, _I32]),
     "qm_talker_cache": (_I32, [_P, _I32, C.POINTER(_P), C.POINTER(_P)]),
     "qm_talker_decode": (_I32, [_P, _P, _P, _P, _I32, C.POINTER(_P)]),
+    "qm_talker_decode_device_rope": (_I32, [_P, _P, _P, _P, _I32, C.POINTER(_P)]),
     "qm_talker_prefill": (_I32, [_P, _P, _P, _P, _I32, C.POINTER(_P)]),
     "qm_talker_synchronize": (_I32, [_P]),
     "qm_talker_stream": (_P, [_P]),
