@@ -326,10 +326,18 @@ static void predictor_step_m1(qm_predictor& p, int step, bool sampling) {
 
 // run_frame_device (R17:13043-13156): reset of the caches and of the frame's selected embeddings and codes, the
 // two input rows, the fifteen steps, the next talker input, and the 64-byte read-back of the frame's sixteen codes.
-// `code0_out`, if given, receives the code the frame started from with the same synchronize.
-static void predictor_frame(qm_predictor& p, const uint16_t* talker_hidden_device, const int32_t* code0_device,
-                            const uint16_t* context_host, bool sampling, int32_t codes_out[16], int32_t* code0_out = nullptr) {
-    if (!talker_hidden_device || !code0_device || !context_host || !codes_out) throw ApiError(QM_ERR_NULL, "predictor frame input is null");
+// What a frame sends back to the host: its codes, the code it started from, the frame kernel's status word.
+struct FrameResult {
+    int32_t codes[kCodeGroups];
+    int32_t code0;
+    uint32_t status;
+};
+
+// Queues a frame; `result` is filled when everything queued here has run (the caller waits for the stream, or — with
+// `result` in pinned memory — for an event it records right after this returns, and may queue more work meanwhile).
+static void predictor_frame_launch(qm_predictor& p, const uint16_t* talker_hidden_device, const int32_t* code0_device,
+                                   const uint16_t* context_host, bool sampling, FrameResult* result) {
+    if (!talker_hidden_device || !code0_device || !context_host || !result) throw ApiError(QM_ERR_NULL, "predictor frame input is null");
     hipStream_t s = p.stream;
     hip_check(hipMemsetAsync(p.frame_state.raw(), 0, p.frame_state.bytes(), s), "predictor caches, selected embeddings and codes reset");
     hip_check(hipMemcpyAsync(p.free_input.raw(), talker_hidden_device, kOuter * 2, hipMemcpyDeviceToDevice, s), "talker hidden copy");
@@ -351,20 +359,52 @@ static void predictor_frame(qm_predictor& p, const uint16_t* talker_hidden_devic
     }
     op_check(qm_predictor_next_talker_input(p.selected.u16(), kCodeGroups, p.context_embedding.u16(), kOuter, p.embedding_sum.u16(),
                                             p.next_input.u16(), s), "next talker input");
-    hip_check(hipMemcpyAsync(codes_out, p.codes.raw(), kCodeGroups * sizeof(int32_t), hipMemcpyDeviceToHost, s), "codes read-back");
-    if (code0_out) hip_check(hipMemcpyAsync(code0_out, code0_device, sizeof(int32_t), hipMemcpyDeviceToHost, s), "code read-back");
-    uint32_t status = 0;
-    if (one_launch) hip_check(hipMemcpyAsync(&status, p.status.raw(), sizeof status, hipMemcpyDeviceToHost, s), "status read-back");
-    hip_check(hipStreamSynchronize(s), "predictor frame synchronize");
-    if (status != 0) {
-        // the frame kernel gave up waiting: its workspace starts over, the frame's codes are not to be used
-        hip_check(hipMemsetAsync(p.status.raw(), 0, sizeof status, s), "status reset");
-        op_check(qm_predictor_frame_workspace_init(p.frame_workspace.raw(), static_cast<int64_t>(p.frame_workspace.bytes()), s),
-                 "predictor frame workspace");
-        hip_check(hipStreamSynchronize(s), "predictor frame workspace synchronize");
-        throw ApiError(QM_ERR_STATUS, "the predictor frame kernel reported status " + std::to_string(status));
-    }
+    hip_check(hipMemcpyAsync(result->codes, p.codes.raw(), kCodeGroups * sizeof(int32_t), hipMemcpyDeviceToHost, s), "codes read-back");
+    hip_check(hipMemcpyAsync(&result->code0, code0_device, sizeof(int32_t), hipMemcpyDeviceToHost, s), "code read-back");
+    // (the status word is zero unless the one launch of the frame's steps gave up)
+    hip_check(hipMemcpyAsync(&result->status, p.status.raw(), sizeof(uint32_t), hipMemcpyDeviceToHost, s), "status read-back");
 }
+
+// After the frame has run: a frame kernel that gave up waiting fails the call, and its workspace starts over.
+static void predictor_frame_finish(qm_predictor& p, const FrameResult& result) {
+    if (result.status == 0) return;
+    hipStream_t s = p.stream;
+    hip_check(hipMemsetAsync(p.status.raw(), 0, sizeof(uint32_t), s), "status reset");
+    op_check(qm_predictor_frame_workspace_init(p.frame_workspace.raw(), static_cast<int64_t>(p.frame_workspace.bytes()), s),
+             "predictor frame workspace");
+    hip_check(hipStreamSynchronize(s), "predictor frame workspace synchronize");
+    throw ApiError(QM_ERR_STATUS, "the predictor frame kernel reported status " + std::to_string(result.status));
+}
+
+static void predictor_frame(qm_predictor& p, const uint16_t* talker_hidden_device, const int32_t* code0_device,
+                            const uint16_t* context_host, bool sampling, int32_t codes_out[16]) {
+    if (!codes_out) throw ApiError(QM_ERR_NULL, "predictor frame input is null");
+    FrameResult result = {};
+    predictor_frame_launch(p, talker_hidden_device, code0_device, context_host, sampling, &result);
+    hip_check(hipStreamSynchronize(p.stream), "predictor frame synchronize");
+    predictor_frame_finish(p, result);
+    std::memcpy(codes_out, result.codes, sizeof result.codes);
+}
+
+// Pinned host memory for what the generation loop reads back while more work is queued, and the event it waits for.
+struct FrameMailbox {
+    FrameResult* result = nullptr;
+    hipEvent_t arrived = nullptr;
+    FrameMailbox() {
+        hip_check(hipHostMalloc(reinterpret_cast<void**>(&result), sizeof(FrameResult), hipHostMallocDefault), "pinned frame result");
+        const hipError_t e = hipEventCreateWithFlags(&arrived, hipEventDisableTiming);
+        if (e != hipSuccess) {
+            (void)hipHostFree(result);
+            hip_check(e, "frame event");
+        }
+    }
+    ~FrameMailbox() {
+        if (arrived) (void)hipEventDestroy(arrived);
+        if (result) (void)hipHostFree(result);
+    }
+    FrameMailbox(const FrameMailbox&) = delete;
+    FrameMailbox& operator=(const FrameMailbox&) = delete;
+};
 
 }  // namespace qm_engine
 
@@ -441,31 +481,37 @@ extern "C" int32_t qm_generate(qm_talker* talker, qm_final_head* head, qm_predic
             hip_check(hipMemcpyAsync(sin_device, decode_sin.data(), decode_sin.size() * 2, hipMemcpyHostToDevice, stream), "decode rope upload");
             hip_check(hipStreamSynchronize(stream), "decode rope upload synchronize");
         }
+        // Per frame the host waits ONCE, and not with an idle GPU: the final head's code stays on the device, where the
+        // predictor reads it; the frame's codes, that code and the status word come back through pinned memory; and the
+        // talker's next step is queued before the host waits for them.  The reference reads the final head's code first
+        // and stops before the predictor at the end-of-sequence code (R17:22222-22232); here the frame that follows that
+        // code — and the talker step after it — have been queued when it is seen: the frame's codes are dropped and the
+        // generator state is put back to where the final head left it, which is what the reference leaves (the extra
+        // cache row lies beyond what any later call reads: a generation starts with a prefill).
+        FrameMailbox mailbox;
+        hipStream_t stream = static_cast<hipStream_t>(qm_talker_stream(talker));
         int frames = 0;
         for (int frame = 0; frame < maximum_frames; ++frame) {
-            // The final head's code stays on the device, where the predictor reads it: the host learns it together
-            // with the frame's codes, at ONE synchronize per frame (the reference reads it back first and stops before
-            // the predictor at the end-of-sequence code, R17:22222-22232; here the frame that follows that code has
-            // run when it is seen, its codes are dropped and the generator state is put back to where the final head
-            // left it, so that what a caller finds afterwards is what the reference leaves).
             final_head_launch(*head, hidden, frame, sampling != 0);
-            hip_check(hipMemcpyAsync(head->rng_after_head.raw(), head->rng.raw(), sizeof(uint64_t), hipMemcpyDeviceToDevice, head->stream),
+            hip_check(hipMemcpyAsync(head->rng_after_head.raw(), head->rng.raw(), sizeof(uint64_t), hipMemcpyDeviceToDevice, stream),
                       "generator state snapshot");
             const uint16_t* context = frame < trailing_rows ? trailing_text_host + static_cast<size_t>(frame) * kOuter : tts_pad_host;
-            int32_t frame_codes[kCodeGroups];
-            int32_t code0 = 0;
-            predictor_frame(*predictor, hidden, static_cast<const int32_t*>(head->code.raw()), context, sampling != 0, frame_codes, &code0);
-            if (code0 == kCodecEos && frame >= 2) {
-                hip_check(hipMemcpyAsync(head->rng.raw(), head->rng_after_head.raw(), sizeof(uint64_t), hipMemcpyDeviceToDevice, head->stream),
+            predictor_frame_launch(*predictor, hidden, static_cast<const int32_t*>(head->code.raw()), context, sampling != 0, mailbox.result);
+            hip_check(hipEventRecord(mailbox.arrived, stream), "frame event record");
+            if (frame + 1 < maximum_frames)
+                op_check(qm_talker_decode_device_rope(talker, predictor->next_input.u16(), cos_device + static_cast<size_t>(frame) * kHeadDim,
+                                                      sin_device + static_cast<size_t>(frame) * kHeadDim, frame, &hidden), "talker decode");
+            hip_check(hipEventSynchronize(mailbox.arrived), "frame boundary synchronize");
+            const FrameResult result = *mailbox.result;
+            predictor_frame_finish(*predictor, result);
+            if (result.code0 == kCodecEos && frame >= 2) {
+                hip_check(hipMemcpyAsync(head->rng.raw(), head->rng_after_head.raw(), sizeof(uint64_t), hipMemcpyDeviceToDevice, stream),
                           "generator state restore");
                 break;
             }
-            if (frame_codes[0] != code0) throw ApiError(QM_ERR_ARGUMENT, "native Predictor recurrence output mismatch");
-            std::memcpy(codes_out + static_cast<size_t>(frame) * kCodeGroups, frame_codes, sizeof frame_codes);
+            if (result.codes[0] != result.code0) throw ApiError(QM_ERR_ARGUMENT, "native Predictor recurrence output mismatch");
+            std::memcpy(codes_out + static_cast<size_t>(frame) * kCodeGroups, result.codes, sizeof result.codes);
             ++frames;
-            if (frame + 1 >= maximum_frames) break;
-            op_check(qm_talker_decode_device_rope(talker, predictor->next_input.u16(), cos_device + static_cast<size_t>(frame) * kHeadDim,
-                                                  sin_device + static_cast<size_t>(frame) * kHeadDim, frame, &hidden), "talker decode");
         }
         op_check(qm_talker_synchronize(talker), "generation synchronize");
         *frames_out = frames;
