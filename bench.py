@@ -508,10 +508,11 @@ class PromptLinears:
     (default); 1: every sum in the reference's order (QM_OPT_LINEAR_ROWS_KERNEL)."""
     bound = "mfma"
 
-    def __init__(self, qm, dev, rows=1024, kernel=0, seed=313):
+    def __init__(self, qm, dev, rows=1024, kernel=0, seed=313, split=False, copies=1):
         import torch
-        self.qm, self.rows, self.kernel = qm, rows, kernel
-        self.name = "prompt_linears_%d_tokens_one_talker_layer%s" % (rows, "_exact_chain" if kernel else "")
+        self.qm, self.rows, self.kernel, self.split = qm, rows, kernel, split
+        self.name = "prompt_linears_%d_tokens_one_talker_layer%s%s" % (rows, "_exact_chain" if kernel else "",
+                                                                      "_reductions_shared_between_blocks" if split else "")
         syn = Synthetic(dev, seed)
         H, KV, I = 2048, 1024, 6144
         self.H, self.KV, self.I = H, KV, I
@@ -526,12 +527,25 @@ class PromptLinears:
         self.bytes = 2 * (H * H + 2 * KV * H + H * H + 2 * I * H + H * I) + 2 * rows * (6 * H + 2 * KV + 2 * I)
         # outputs of magnitude 1 to 4: one bf16 spacing there
         self.tolerance = 0.0625
+        # short prompts: a workspace lets the linears cut their reductions (qm_linear_rows_split)
+        self.ws_bytes = max(qm.linear_rows_split_workspace_bytes(rows, c, r, p) for c, r, p in
+                            ((H, H, False), (KV, H, False), (I, H, True), (H, I, False))) if split else 0
+        self.ws = torch.empty(max(self.ws_bytes, 256) // 4, dtype=torch.float32, device=dev)
 
     def step(self):
         import torch
         qm, s, R, H, KV, I = self.qm, torch.cuda.current_stream().cuda_stream, self.rows, self.H, self.KV, self.I
         qm.set_option(qm.OPT_LINEAR_ROWS_KERNEL, self.kernel)
         try:
+            if self.split:
+                ws, nb = self.ws, self.ws_bytes
+                qm.linear_rows_split(self.x, self.wq, self.bq, None, self.q, R, H, H, ws, nb, s)
+                qm.linear_rows_split(self.x, self.wk, self.bk, None, self.k, R, KV, H, ws, nb, s)
+                qm.linear_rows_split(self.x, self.wv, self.bv, None, self.v, R, KV, H, ws, nb, s)
+                qm.linear_rows_split(self.q, self.wo, None, self.res, self.o, R, H, H, ws, nb, s)
+                qm.gate_up_swiglu_rows_split(self.o, self.wg, self.wu, self.act, R, H, I, ws, nb, s)
+                qm.linear_rows_split(self.act, self.wd, None, self.o, self.out, R, H, I, ws, nb, s)
+                return
             qm.linear_rows(self.x, self.wq, self.bq, None, self.q, R, H, H, s)
             qm.linear_rows(self.x, self.wk, self.bk, None, self.k, R, KV, H, s)
             qm.linear_rows(self.x, self.wv, self.bv, None, self.v, R, KV, H, s)
@@ -1039,7 +1053,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
     ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "prefillfp32", "chunk", "chunkwhole", "chunkrows", "predictor", "predictorexact",
-                                      "qkv", "layer", "layer1", "layer2", "frame", "frame1", "linears", "linearsexact", "generate"], default=None,
+                                      "qkv", "layer", "layer1", "layer2", "frame", "frame1", "linears", "linearsexact", "linears128", "linears128split", "generate"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -1084,7 +1098,8 @@ def main():
                 "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev), "layer1": lambda: TalkerLayerStep(qm, dev, chained=True), "layer2": lambda: TalkerLayerStep(qm, dev, two_launches=True),
                 "frame": lambda: PredictorFrameSteps(qm, dev),
                 "frame1": lambda: PredictorFrameSteps(qm, dev, one_launch=True),
-                "linears": lambda: PromptLinears(qm, dev), "linearsexact": lambda: PromptLinears(qm, dev, kernel=1)}[args.only]
+                "linears": lambda: PromptLinears(qm, dev), "linearsexact": lambda: PromptLinears(qm, dev, kernel=1),
+                "linears128": lambda: PromptLinears(qm, dev, rows=128), "linears128split": lambda: PromptLinears(qm, dev, rows=128, split=True)}[args.only]
         w = make()
         r = _report(w, _time_steps(w.step, args.steps, args.warmup))
         r["bound"] = w.bound
@@ -1138,6 +1153,9 @@ def main():
             # the seven linears of a talker layer over a 1024-token prompt: matrix cores, and the exact chain
             ("next_prompt_linears_1024_tokens", lambda: PromptLinears(qm, dev)),
             ("next_prompt_linears_1024_tokens_exact_chain", lambda: PromptLinears(qm, dev, kernel=1)),
+            # a short prompt (what a sentence of text is): 32 to 96 blocks per linear; with a workspace the reductions are cut
+            ("next_prompt_linears_128_tokens", lambda: PromptLinears(qm, dev, rows=128)),
+            ("next_prompt_linears_128_tokens_reductions_shared", lambda: PromptLinears(qm, dev, rows=128, split=True)),
             # the fourteen M = 1 steps of one code-predictor frame, operator by operator (406 launches)
             ("next_predictor_frame_m1_steps", lambda: PredictorFrameSteps(qm, dev)),
             # the same fourteen steps as ONE launch of 256 resident blocks (same codes bit for bit)

@@ -780,6 +780,25 @@ int32_t qm_linear_rows(
 int32_t qm_gate_up_swiglu_rows(
     const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight, uint16_t* output,
     int32_t rows, int32_t hidden, int32_t intermediate, void* hip_stream);
+/*
+ * The same two operators with a workspace for SHORT prompts (no counterpart in the reference, whose kernel gives every
+ * output its own wave).  On the matrix cores a block owns 128 output columns of 64 or 128 token rows and walks the whole
+ * reduction: 128 rows of a 2048-column linear are 32 blocks on 256 compute units, and the call lasts as long as one
+ * block's chain.  With a workspace of qm_linear_rows_split_workspace_bytes (0 where the shape is not cut: enough blocks
+ * already, or the exact chain) the reduction is cut into 2, 4 or 8 pieces, a block each, whose fp32 sums a second launch
+ * adds in order before the same roundings.  Results differ from the uncut call in the association of the sum only
+ * (within the matrix-core path's tolerance of the exact chain) and are the same on every call.  workspace: 256-byte
+ * aligned, nothing to initialise; NULL: exactly qm_linear_rows / qm_gate_up_swiglu_rows; too small: QM_ERR_WORKSPACE.
+ */
+int64_t qm_linear_rows_split_workspace_bytes(int32_t rows, int32_t output_columns, int32_t reduction_columns, int32_t gate_up_pair);
+int32_t qm_linear_rows_split(
+    const uint16_t* input, const uint16_t* weight, const uint16_t* bias, const uint16_t* residual,
+    uint16_t* output, int32_t rows, int32_t output_columns, int32_t reduction_columns,
+    void* workspace, int64_t workspace_bytes, void* hip_stream);
+int32_t qm_gate_up_swiglu_rows_split(
+    const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight, uint16_t* output,
+    int32_t rows, int32_t hidden, int32_t intermediate,
+    void* workspace, int64_t workspace_bytes, void* hip_stream);
 
 /* ---- final head: score processing, top-k sampler, history ------------------------ */
 /*

@@ -146,6 +146,9 @@ _SIGNATURES = {
     "qm_predictor_next_talker_input": (_I32, [_PTR, _I32, _PTR, _I32, _PTR, _PTR, _PTR]),
     "qm_linear_rows": (_I32, [_PTR] * 5 + [_I32, _I32, _I32, _PTR]),
     "qm_gate_up_swiglu_rows": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _PTR]),
+    "qm_linear_rows_split_workspace_bytes": (C.c_int64, [_I32, _I32, _I32, _I32]),
+    "qm_linear_rows_split": (_I32, [_PTR] * 5 + [_I32, _I32, _I32, _PTR, C.c_int64, _PTR]),
+    "qm_gate_up_swiglu_rows_split": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _PTR, C.c_int64, _PTR]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
@@ -439,6 +442,20 @@ def linear_rows(x, weight, bias, residual, out, rows, output_columns, reduction_
 def gate_up_swiglu_rows(x, gate_w, up_w, out, rows, hidden, intermediate, stream=0):
     _check(lib().qm_gate_up_swiglu_rows(_addr(x), _addr(gate_w), _addr(up_w), _addr(out), rows, hidden,
                                         intermediate, stream), "qm_gate_up_swiglu_rows")
+
+
+def linear_rows_split_workspace_bytes(rows, output_columns, reduction_columns, gate_up_pair=False):
+    return lib().qm_linear_rows_split_workspace_bytes(rows, output_columns, reduction_columns, int(gate_up_pair))
+
+
+def linear_rows_split(x, weight, bias, residual, out, rows, output_columns, reduction_columns, workspace, workspace_bytes, stream=0):
+    _check(lib().qm_linear_rows_split(_addr(x), _addr(weight), _addr(bias), _addr(residual), _addr(out), rows, output_columns,
+                                      reduction_columns, _addr(workspace), workspace_bytes, stream), "qm_linear_rows_split")
+
+
+def gate_up_swiglu_rows_split(x, gate_weight, up_weight, out, rows, hidden, intermediate, workspace, workspace_bytes, stream=0):
+    _check(lib().qm_gate_up_swiglu_rows_split(_addr(x), _addr(gate_weight), _addr(up_weight), _addr(out), rows, hidden, intermediate,
+                                              _addr(workspace), workspace_bytes, stream), "qm_gate_up_swiglu_rows_split")
 
 
 def gather_embedding(table, table_rows, codes, group, dimension, selected, next_input, stream=0):

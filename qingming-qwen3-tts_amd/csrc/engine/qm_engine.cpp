@@ -49,6 +49,7 @@ struct qm_talker {
         p_swiglu, p_cosine, p_sine;
     // the prompt pass's key-split workspace (prompts whose attention grid leaves compute units idle), grown on demand
     qm_engine::DeviceBuffer p_split;
+    qm_engine::DeviceBuffer p_rows_split;   // partial sums of the prompt pass's linears where they cut their reductions
     // device status word the attention kernels OR their QM_STATUS_* bits into; read at qm_talker_synchronize
     qm_engine::DeviceBuffer status;
     // hand-off words of qm_talker_post_attention_m1 (checkpoints of the geometry it serves)
@@ -296,7 +297,7 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
 // NativeTalkerEngine::prefill (R17:16561-16800): the prompt's rows through every layer.  The
 // reference's launches per layer and what runs here:
 //   rmsnorm                                   -> qm_rmsnorm_rows
-//   3 x linear_generic (q, k, v)              -> 3 x qm_linear_rows
+//   3 x linear_generic (q, k, v)              -> 3 x qm_linear_rows (every linear through its _split entry: short prompts)
 //   2 x rmsnorm + 2 x rope_rows               -> 2 x qm_norm_rope_rows
 //   scatter_prefill_cache + attention         -> qm_prefill_attention_causal_split (writes the cache itself; long
 //                                                query tiles of a prompt are shared by two or three blocks)
@@ -327,6 +328,20 @@ static const uint16_t* prefill(qm_talker& e, const uint16_t* input_device, const
         e.p_split = DeviceBuffer(static_cast<size_t>(split_bytes));
         op_check(qm_prefill_split_workspace_init(e.p_split.raw(), split_bytes, s), "prefill key-split workspace init");
     }
+    // A short prompt leaves most compute units without a block of a linear: with this workspace the linears cut their
+    // reductions (qm_linear_rows_split; 0 bytes where a shape is not cut, and then the call is the uncut one).
+    int64_t rows_bytes = 0;
+    for (const int64_t need : {qm_linear_rows_split_workspace_bytes(rows, e.q_dim, kHidden, 0),
+                               qm_linear_rows_split_workspace_bytes(rows, e.kv_dim, kHidden, 0),
+                               qm_linear_rows_split_workspace_bytes(rows, kHidden, e.q_dim, 0),
+                               qm_linear_rows_split_workspace_bytes(rows, e.intermediate, kHidden, 1),
+                               qm_linear_rows_split_workspace_bytes(rows, kHidden, e.intermediate, 0)})
+        rows_bytes = std::max(rows_bytes, need);
+    if (static_cast<size_t>(rows_bytes) > e.p_rows_split.bytes()) {
+        hip_check(hipStreamSynchronize(s), "prefill workspace growth");
+        e.p_rows_split = DeviceBuffer(static_cast<size_t>(rows_bytes));
+    }
+    void* const rows_ws = rows_bytes > 0 ? e.p_rows_split.raw() : nullptr;
     const size_t rope_bytes = static_cast<size_t>(rows) * kHeadDim * 2;
     hip_check(hipMemcpyAsync(e.p_hidden_a.raw(), input_device, static_cast<size_t>(rows) * kHidden * 2,
                              hipMemcpyDeviceToDevice, s), "prefill input copy");
@@ -338,12 +353,12 @@ static const uint16_t* prefill(qm_talker& e, const uint16_t* input_device, const
         const qm_kv_cache cache = flat_cache_of(e, w);
         op_check(qm_rmsnorm_rows(current->u16(), w.input_norm.data(), e.p_norm.u16(), rows, kHidden, kEpsilon, s),
                  "prefill input RMSNorm");
-        op_check(qm_linear_rows(e.p_norm.u16(), w.q_weight.data(), w.q_bias.data(), nullptr, e.p_q.u16(), rows, e.q_dim,
-                                kHidden, s), "prefill q_proj");
-        op_check(qm_linear_rows(e.p_norm.u16(), w.k_weight.data(), w.k_bias.data(), nullptr, e.p_k.u16(), rows, e.kv_dim,
-                                kHidden, s), "prefill k_proj");
-        op_check(qm_linear_rows(e.p_norm.u16(), w.v_weight.data(), w.v_bias.data(), nullptr, e.p_v.u16(), rows, e.kv_dim,
-                                kHidden, s), "prefill v_proj");
+        op_check(qm_linear_rows_split(e.p_norm.u16(), w.q_weight.data(), w.q_bias.data(), nullptr, e.p_q.u16(), rows, e.q_dim,
+                                      kHidden, rows_ws, rows_bytes, s), "prefill q_proj");
+        op_check(qm_linear_rows_split(e.p_norm.u16(), w.k_weight.data(), w.k_bias.data(), nullptr, e.p_k.u16(), rows, e.kv_dim,
+                                      kHidden, rows_ws, rows_bytes, s), "prefill k_proj");
+        op_check(qm_linear_rows_split(e.p_norm.u16(), w.v_weight.data(), w.v_bias.data(), nullptr, e.p_v.u16(), rows, e.kv_dim,
+                                      kHidden, rows_ws, rows_bytes, s), "prefill v_proj");
         op_check(qm_norm_rope_rows(e.p_q.u16(), w.q_norm.data(), e.p_cosine.u16(), e.p_sine.u16(), e.p_q_rotated.u16(), rows,
                                    e.q_heads, kEpsilon, s), "prefill q norm + RoPE");
         op_check(qm_norm_rope_rows(e.p_k.u16(), w.k_norm.data(), e.p_cosine.u16(), e.p_sine.u16(), e.p_k_rotated.u16(), rows,
@@ -353,14 +368,14 @@ static const uint16_t* prefill(qm_talker& e, const uint16_t* input_device, const
                                                    split_bytes > 0 ? e.p_split.raw() : nullptr, split_bytes,
                                                    static_cast<uint32_t*>(e.status.raw()), s),
                  "prefill attention + cache write");
-        op_check(qm_linear_rows(e.p_context.u16(), w.o_weight.data(), w.o_bias.data(), current->u16(), e.p_residual.u16(),
-                                rows, kHidden, e.q_dim, s), "prefill o_proj + residual");
+        op_check(qm_linear_rows_split(e.p_context.u16(), w.o_weight.data(), w.o_bias.data(), current->u16(), e.p_residual.u16(),
+                                      rows, kHidden, e.q_dim, rows_ws, rows_bytes, s), "prefill o_proj + residual");
         op_check(qm_rmsnorm_rows(e.p_residual.u16(), w.post_norm.data(), e.p_norm.u16(), rows, kHidden, kEpsilon, s),
                  "prefill post-attention RMSNorm");
-        op_check(qm_gate_up_swiglu_rows(e.p_norm.u16(), w.gate_weight.data(), w.up_weight.data(), e.p_swiglu.u16(), rows,
-                                        kHidden, e.intermediate, s), "prefill gate/up/SwiGLU");
-        op_check(qm_linear_rows(e.p_swiglu.u16(), w.down_weight.data(), nullptr, e.p_residual.u16(), next->u16(), rows,
-                                kHidden, e.intermediate, s), "prefill down_proj + residual");
+        op_check(qm_gate_up_swiglu_rows_split(e.p_norm.u16(), w.gate_weight.data(), w.up_weight.data(), e.p_swiglu.u16(), rows,
+                                              kHidden, e.intermediate, rows_ws, rows_bytes, s), "prefill gate/up/SwiGLU");
+        op_check(qm_linear_rows_split(e.p_swiglu.u16(), w.down_weight.data(), nullptr, e.p_residual.u16(), next->u16(), rows,
+                                      kHidden, e.intermediate, rows_ws, rows_bytes, s), "prefill down_proj + residual");
         std::swap(current, next);
     }
     op_check(qm_rmsnorm_rows(current->u16() + static_cast<size_t>(rows - 1) * kHidden, e.final_norm.data(),

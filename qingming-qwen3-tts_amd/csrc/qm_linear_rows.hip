@@ -241,36 +241,70 @@ inline int32_t rows_on_matrix_cores(const LinearRowsParams& prm, int32_t* yes) {
 
 }  // namespace qm
 
-extern "C" int32_t qm_linear_rows(const uint16_t* input, const uint16_t* weight, const uint16_t* bias,
-                                  const uint16_t* residual, uint16_t* output, int32_t rows, int32_t output_columns,
-                                  int32_t reduction_columns, void* hip_stream) {
-    using namespace qm;
-    if (!input || !weight || !output) return QM_ERR_NULL;
-    LinearRowsParams prm = {};
-    prm.input = input; prm.weight[0] = weight; prm.weight[1] = weight; prm.bias = bias; prm.residual = residual;
-    prm.output = output; prm.rows = rows; prm.columns = output_columns; prm.reduction = reduction_columns;
-    const int32_t rc = check_rows(prm, false);
+namespace qm {
+
+// With a workspace the matrix-core path may cut the reduction (few token rows); the exact chain never uses it.
+inline int32_t rows_entry(LinearRowsParams prm, bool dual, void* workspace, int64_t workspace_bytes, void* hip_stream) {
+    if (workspace_bytes < 0 || (workspace_bytes > 0 && !workspace)) return QM_ERR_ARGUMENT;
+    if (reinterpret_cast<uintptr_t>(workspace) & 255) return QM_ERR_GEOMETRY;
+    const int32_t rc = check_rows(prm, dual);
     if (rc != QM_OK) return rc;
     int32_t matrix_cores = 0;
     const int32_t rc_kernel = rows_on_matrix_cores(prm, &matrix_cores);
     if (rc_kernel != QM_OK) return rc_kernel;
-    if (matrix_cores) return launch_rows_mfma(prm, false, static_cast<hipStream_t>(hip_stream));
-    return launch_rows<false>(prm, static_cast<hipStream_t>(hip_stream));
+    prm.reduction_parts = 1;
+    prm.partials = nullptr;
+    if (!matrix_cores) return dual ? launch_rows<true>(prm, static_cast<hipStream_t>(hip_stream))
+                                   : launch_rows<false>(prm, static_cast<hipStream_t>(hip_stream));
+    if (workspace) {
+        const size_t need = rows_mfma_workspace_bytes(prm.rows, prm.columns, prm.reduction, dual);
+        if (need > 0) {
+            if (static_cast<size_t>(workspace_bytes) < need) return QM_ERR_WORKSPACE;
+            prm.reduction_parts = rows_mfma_reduction_parts(prm.rows, prm.columns, prm.reduction, dual);
+            prm.partials = static_cast<float*>(workspace);
+        }
+    }
+    return launch_rows_mfma(prm, dual, static_cast<hipStream_t>(hip_stream));
+}
+
+}  // namespace qm
+
+extern "C" int32_t qm_linear_rows(const uint16_t* input, const uint16_t* weight, const uint16_t* bias,
+                                  const uint16_t* residual, uint16_t* output, int32_t rows, int32_t output_columns,
+                                  int32_t reduction_columns, void* hip_stream) {
+    return qm_linear_rows_split(input, weight, bias, residual, output, rows, output_columns, reduction_columns, nullptr, 0, hip_stream);
 }
 
 extern "C" int32_t qm_gate_up_swiglu_rows(const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight,
                                           uint16_t* output, int32_t rows, int32_t hidden, int32_t intermediate,
                                           void* hip_stream) {
+    return qm_gate_up_swiglu_rows_split(input, gate_weight, up_weight, output, rows, hidden, intermediate, nullptr, 0, hip_stream);
+}
+
+extern "C" int64_t qm_linear_rows_split_workspace_bytes(int32_t rows, int32_t output_columns, int32_t reduction_columns, int32_t gate_up_pair) {
+    using namespace qm;
+    if (rows < kRowsMatrixMinimum || output_columns <= 0 || reduction_columns <= 0 || output_columns % 128 || reduction_columns % 128) return 0;
+    return static_cast<int64_t>(rows_mfma_workspace_bytes(rows, output_columns, reduction_columns, gate_up_pair != 0));
+}
+
+extern "C" int32_t qm_linear_rows_split(const uint16_t* input, const uint16_t* weight, const uint16_t* bias,
+                                        const uint16_t* residual, uint16_t* output, int32_t rows, int32_t output_columns,
+                                        int32_t reduction_columns, void* workspace, int64_t workspace_bytes, void* hip_stream) {
+    using namespace qm;
+    if (!input || !weight || !output) return QM_ERR_NULL;
+    LinearRowsParams prm = {};
+    prm.input = input; prm.weight[0] = weight; prm.weight[1] = weight; prm.bias = bias; prm.residual = residual;
+    prm.output = output; prm.rows = rows; prm.columns = output_columns; prm.reduction = reduction_columns;
+    return rows_entry(prm, false, workspace, workspace_bytes, hip_stream);
+}
+
+extern "C" int32_t qm_gate_up_swiglu_rows_split(const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight,
+                                                uint16_t* output, int32_t rows, int32_t hidden, int32_t intermediate,
+                                                void* workspace, int64_t workspace_bytes, void* hip_stream) {
     using namespace qm;
     if (!input || !gate_weight || !up_weight || !output) return QM_ERR_NULL;
     LinearRowsParams prm = {};
     prm.input = input; prm.weight[0] = gate_weight; prm.weight[1] = up_weight;
     prm.output = output; prm.rows = rows; prm.columns = intermediate; prm.reduction = hidden;
-    const int32_t rc = check_rows(prm, true);
-    if (rc != QM_OK) return rc;
-    int32_t matrix_cores = 0;
-    const int32_t rc_kernel = rows_on_matrix_cores(prm, &matrix_cores);
-    if (rc_kernel != QM_OK) return rc_kernel;
-    if (matrix_cores) return launch_rows_mfma(prm, true, static_cast<hipStream_t>(hip_stream));
-    return launch_rows<true>(prm, static_cast<hipStream_t>(hip_stream));
+    return rows_entry(prm, true, workspace, workspace_bytes, hip_stream);
 }

@@ -95,10 +95,12 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
             src[i] = prm.weight[operand - 1] + static_cast<int64_t>(n0 + row) * K + 8 * piece;
         }
     }
-    const int steps = K / kGmStep;
+    // (a block takes piece blockIdx.z of the reduction: all of it unless the launch cut it)
+    const int steps = K / kGmStep / prm.reduction_parts;
+    const int first_step = static_cast<int>(blockIdx.z) * steps;
     // (requests past the last step repeat it and land in a stage nobody reads again: the wait below counts pieces)
 #define QM_GM_REQUEST(step_)                                                                                             \
-    gm_request<kPerWave>(src, min((step_), steps - 1) * kGmStep, gm_smem + ((step_) % kStages) * kStageBytes + 1024 * wave)
+    gm_request<kPerWave>(src, (first_step + min((step_), steps - 1)) * kGmStep, gm_smem + ((step_) % kStages) * kStageBytes + 1024 * wave)
 
     f32x16_t acc[kTn][kTm], acc_up[DUAL ? kTn : 1][DUAL ? kTm : 1];
 #pragma unroll
@@ -189,6 +191,29 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
 
     // ---- epilogue: accumulator register r of a lane is output column 8 (r / 4) + 4 (lane / 32) + r % 4 of the MFMA
     // tile's 32, token row lane % 32 ----
+    if (prm.reduction_parts > 1) {
+        // a piece of the reduction: the sums as they are, for linear_rows_parts_kernel
+        const int64_t plane = static_cast<int64_t>(prm.rows) * prm.columns;
+        float* const part = prm.partials + static_cast<int64_t>(blockIdx.z) * (DUAL ? 2 : 1) * plane;
+#pragma unroll
+        for (int a = 0; a < kTn; ++a) {
+#pragma unroll
+            for (int b = 0; b < kTm; ++b) {
+                const int m = m0 + 32 * (kTm * wave_m + b) + (lane & 31);
+                if (m >= prm.rows) continue;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = n0 + 32 * (kTn * wave_n + a) + 8 * g + 4 * (lane >> 5);
+                    float* at = part + static_cast<int64_t>(m) * prm.columns + n;
+                    *reinterpret_cast<float4*>(at) = make_float4(acc[a][b][4 * g], acc[a][b][4 * g + 1], acc[a][b][4 * g + 2], acc[a][b][4 * g + 3]);
+                    if (DUAL)
+                        *reinterpret_cast<float4*>(at + plane) =
+                            make_float4(acc_up[a][b][4 * g], acc_up[a][b][4 * g + 1], acc_up[a][b][4 * g + 2], acc_up[a][b][4 * g + 3]);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int a = 0; a < kTn; ++a) {
 #pragma unroll
@@ -227,17 +252,86 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
     }
 }
 
+// The pieces of a cut reduction added in order, then what the epilogue above does: thread = four output columns of a row.
+template <bool DUAL>
+__global__ __launch_bounds__(256) void linear_rows_parts_kernel(LinearRowsParams prm) {
+    const int64_t quad = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const int quads_per_row = prm.columns / 4;
+    if (quad >= static_cast<int64_t>(prm.rows) * quads_per_row) return;
+    const int m = static_cast<int>(quad / quads_per_row);
+    const int n = 4 * static_cast<int>(quad % quads_per_row);
+    const int64_t plane = static_cast<int64_t>(prm.rows) * prm.columns;
+    const float* at = prm.partials + static_cast<int64_t>(m) * prm.columns + n;
+    float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f), up = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (int z = 0; z < prm.reduction_parts; ++z) {
+        const float4 v = *reinterpret_cast<const float4*>(at + static_cast<int64_t>(z) * (DUAL ? 2 : 1) * plane);
+        sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+        if (DUAL) {
+            const float4 u = *reinterpret_cast<const float4*>(at + static_cast<int64_t>(z) * 2 * plane + plane);
+            up.x += u.x; up.y += u.y; up.z += u.z; up.w += u.w;
+        }
+    }
+    const float s4[4] = {sum.x, sum.y, sum.z, sum.w}, u4[4] = {up.x, up.y, up.z, up.w};
+    uint16_t bits[4];
+    uint2 res = make_uint2(0, 0), bias = make_uint2(0, 0);
+    if (!DUAL && prm.residual) res = *reinterpret_cast<const uint2*>(prm.residual + static_cast<int64_t>(m) * prm.columns + n);
+    if (!DUAL && prm.bias) bias = *reinterpret_cast<const uint2*>(prm.bias + n);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        if (DUAL) {
+            const float gv = bf2f(f2bf(s4[e]));
+            const uint16_t act = f2bf(gv / (1.0f + expf(-gv)));
+            bits[e] = f2bf(bf2f(act) * bf2f(f2bf(u4[e])));
+        } else {
+            float r = s4[e];
+            if (prm.bias) r += bf2f(static_cast<uint16_t>((e < 2 ? bias.x : bias.y) >> (16 * (e & 1))));
+            uint16_t v = f2bf(r);
+            if (prm.residual) v = f2bf(bf2f(static_cast<uint16_t>((e < 2 ? res.x : res.y) >> (16 * (e & 1)))) + bf2f(v));
+            bits[e] = v;
+        }
+    }
+    *reinterpret_cast<uint2*>(prm.output + static_cast<int64_t>(m) * prm.columns + n) =
+        make_uint2(bits[0] | (static_cast<uint32_t>(bits[1]) << 16), bits[2] | (static_cast<uint32_t>(bits[3]) << 16));
+}
+
 template <bool DUAL, int BM>
 int32_t launch_rows_mfma_as(const LinearRowsParams& prm, hipStream_t stream) {
     constexpr int kStages = DUAL ? 3 : 4;
     constexpr int smem = kStages * (BM * kGmStep * 2 + (DUAL ? 2 : 1) * kGmTileBytes);
-    const dim3 grid(static_cast<unsigned>(prm.columns / kGmTile), static_cast<unsigned>((prm.rows + BM - 1) / BM));
+    const dim3 grid(static_cast<unsigned>(prm.columns / kGmTile), static_cast<unsigned>((prm.rows + BM - 1) / BM),
+                    static_cast<unsigned>(prm.reduction_parts));
     if (grid.y > 65535u) return QM_ERR_ARGUMENT;
     static std::atomic<bool> lds_raised[kMaxDevices];
     const int32_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(linear_rows_mfma_kernel<DUAL, BM>), smem, lds_raised);
     if (rc != QM_OK) return rc;
     hipLaunchKernelGGL((linear_rows_mfma_kernel<DUAL, BM>), grid, dim3(kGmThreads), smem, stream, prm);
-    return launch_status();
+    int32_t status = launch_status();
+    if (status == QM_OK && prm.reduction_parts > 1) {
+        const int64_t quads = static_cast<int64_t>(prm.rows) * (prm.columns / 4);
+        hipLaunchKernelGGL((linear_rows_parts_kernel<DUAL>), dim3(static_cast<unsigned>((quads + 255) / 256)), dim3(256), 0, stream, prm);
+        status = launch_status();
+    }
+    return status;
+}
+
+// Few token rows leave most CUs without a block (128 rows of a 2048-column linear: 32 blocks), and a block's time is its
+// chain of 64-k steps.  With a workspace the reduction is cut so that the grid comes to about one block per CU: pieces of
+// four steps at least, as many as divide the steps evenly, at most eight.
+int rows_mfma_reduction_parts(int rows, int columns, int reduction, bool dual) {
+    (void)dual;
+    if (rows <= 0 || columns < kGmTile || reduction < kGmStep) return 1;
+    const int64_t blocks = static_cast<int64_t>(columns / kGmTile) * ((rows + 63) / 64);
+    const int steps = reduction / kGmStep;
+    int parts = 1;
+    for (int p = 2; p <= 8; p *= 2)
+        if (blocks * p <= 256 && steps % p == 0 && steps / p >= 4) parts = p;
+    return parts;
+}
+
+size_t rows_mfma_workspace_bytes(int rows, int columns, int reduction, bool dual) {
+    const int parts = rows_mfma_reduction_parts(rows, columns, reduction, dual);
+    if (parts <= 1) return 0;
+    return static_cast<size_t>(parts) * (dual ? 2 : 1) * rows * columns * sizeof(float);
 }
 
 int32_t launch_rows_mfma(const LinearRowsParams& prm, bool dual, hipStream_t stream) {

@@ -14,10 +14,20 @@ struct LinearRowsParams {
     uint16_t* output;             // [rows][columns]
     int rows, columns, reduction;
     int columns_per_block;        // 8 or 4 (4: the two halves of the block take four token rows each)
+    // (matrix cores, few token rows) the reduction cut into reduction_parts pieces, one block each: the fp32 sums of
+    // piece z go to partials[z] ([rows][columns]; a gate/up pair: gate plane, then up plane) and a second launch adds the
+    // pieces in order and rounds.  1: every block takes the whole reduction and rounds its sums itself.
+    int reduction_parts;
+    float* partials;
 };
 
 // The row linears on the matrix cores (qm_linear_rows_mfma.hip).  `dual`: weight[0] / weight[1] are the gate and up
 // matrices and the epilogue is SwiGLU.  Needs columns % 128 == 0 and reduction % 128 == 0 (checked by the caller).
 int32_t launch_rows_mfma(const LinearRowsParams& prm, bool dual, hipStream_t stream);
+
+// Into how many pieces launch_rows_mfma cuts the reduction when it is given a workspace for the partial sums (a pure
+// function of the shape), and the bytes that workspace must hold (0: the shape is not cut).
+int rows_mfma_reduction_parts(int rows, int columns, int reduction, bool dual);
+size_t rows_mfma_workspace_bytes(int rows, int columns, int reduction, bool dual);
 
 }  // namespace qm

@@ -113,3 +113,69 @@ def test_linear_rows_argument_errors(qm, dev):
     assert L.qm_linear_rows(x.data_ptr() + 2, w.data_ptr(), None, None, o.data_ptr(), 1, 8, 64, None) == -2
     assert L.qm_linear_rows(x.data_ptr(), w.data_ptr(), None, None, o.data_ptr(), 0, 8, 72, None) == 0
     assert L.qm_gate_up_swiglu_rows(x.data_ptr(), w.data_ptr(), None, o.data_ptr(), 4, 72, 8, None) == -1
+
+
+@pytest.mark.parametrize("rows,cols,red,bias,residual", [
+    (128, 2048, 2048, True, True),      # o_proj of a 128-token prompt: 32 blocks, the reduction in eight pieces
+    (100, 1024, 2048, False, False),    # k_proj: 16 blocks
+    (37, 2048, 6144, False, True),      # down_proj + residual: 96 steps
+    (64, 4096, 2048, True, False),      # 32 blocks: eight pieces
+    (200, 2048, 2048, False, True),     # 64 blocks: four pieces
+])
+def test_linear_rows_with_the_reduction_shared_between_blocks(oracle, qm, dev, rows, cols, red, bias, residual, rows_kernel):
+    """qm_linear_rows_split: few token rows leave most CUs without a block; with a workspace the reduction is cut into pieces
+    whose fp32 sums a second launch adds in order.  Held to the bounds of the uncut matrix-core call; the same bits on every
+    call; on the exact chain the workspace is not used and the result stays bit-exact."""
+    import torch
+    seed = 4500 + rows + cols + red
+    x = oracle.normal_bf16((rows, red), seed)
+    w = oracle.normal_bf16((cols, red), seed + 1, std=0.02)
+    b = oracle.normal_bf16((cols,), seed + 2, std=0.1) if bias else None
+    r = oracle.normal_bf16((rows, cols), seed + 3) if residual else None
+    want = np.zeros((rows, cols), dtype=np.uint16)
+    assert oracle.linear_rows(x, w, b, r, want, rows, cols, red, 16) == 0
+    nbytes = qm.linear_rows_split_workspace_bytes(rows, cols, red)
+    assert nbytes > 0
+    ws = torch.full((nbytes // 4,), float("nan"), dtype=torch.float32, device=dev)
+    xd, wd = to_dev(x, dev), to_dev(w, dev)
+    bd, rd = None if b is None else to_dev(b, dev), None if r is None else to_dev(r, dev)
+    outs = []
+    for _ in range(2):
+        out = torch.full((rows, cols), 0x7fc0, dtype=torch.int16, device=dev)
+        qm.linear_rows_split(xd, wd, bd, rd, out, rows, cols, red, ws, nbytes)
+        torch.cuda.synchronize()
+        outs.append(to_u16(out))
+    assert np.array_equal(outs[0], outs[1])
+    _check(oracle, outs[0], want, rows_kernel == MATRIX, r)
+    if rows_kernel == MATRIX:
+        assert qm.lib().qm_linear_rows_split(xd.data_ptr(), wd.data_ptr(), None, None, out.data_ptr(), rows, cols, red, ws.data_ptr(),
+                                             nbytes - 4, None) == -4
+    assert qm.linear_rows_split_workspace_bytes(1024, 2048, 2048) == 0      # enough blocks already
+
+
+@pytest.mark.parametrize("rows,hidden,inter", [(128, 2048, 6144), (48, 2048, 3072)])
+def test_gate_up_swiglu_rows_with_the_reduction_shared_between_blocks(oracle, qm, dev, rows, hidden, inter, rows_kernel):
+    import torch
+    seed = 5500 + rows + hidden
+    x = oracle.normal_bf16((rows, hidden), seed)
+    gw = oracle.normal_bf16((inter, hidden), seed + 1, std=0.03)
+    uw = oracle.normal_bf16((inter, hidden), seed + 2, std=0.03)
+    want = np.zeros((rows, inter), dtype=np.uint16)
+    assert oracle.gate_up_swiglu_rows(x, gw, uw, want, rows, hidden, inter, 16) == 0
+    nbytes = qm.linear_rows_split_workspace_bytes(rows, inter, hidden, True)
+    assert nbytes > 0
+    ws = torch.full((nbytes // 4,), float("nan"), dtype=torch.float32, device=dev)
+    outs = []
+    for _ in range(2):
+        out = torch.full((rows, inter), 0x7fc0, dtype=torch.int16, device=dev)
+        qm.gate_up_swiglu_rows_split(to_dev(x, dev), to_dev(gw, dev), to_dev(uw, dev), out, rows, hidden, inter, ws, nbytes)
+        torch.cuda.synchronize()
+        outs.append(to_u16(out))
+    assert np.array_equal(outs[0], outs[1])
+    d = ulp_distance(outs[0], want)
+    if rows_kernel == MATRIX:
+        g, w = oracle.bf16_to_f32(outs[0]).astype(np.float64), oracle.bf16_to_f32(want).astype(np.float64)
+        assert np.all(np.abs(g - w) <= 1e-3 + np.abs(w) * 2.0 ** -6), float(np.max(np.abs(g - w)))
+        assert np.count_nonzero(d) <= rows * inter // 100, np.count_nonzero(d)
+    else:
+        assert d.max() <= 1 and np.count_nonzero(d) <= max(1, rows * inter // 1000)
