@@ -188,6 +188,8 @@ size_t qm_decode_workspace_bytes(int32_t n_streams, int32_t q_heads,
  * sliding_window as in R17:16032-16036 (<= 0 disables the window).
  * Scores are rounded to bf16 before and after scaling like the reference
  * (R17:16102-16116); softmax and P·V stay in fp32 (online softmax, split-K).
+ * q_heads: any multiple of the cache's kv_heads (query head h reads kv head h / (q_heads / kv_heads); groups of
+ * 1, 2 and 4 heads have kernels of their own, another group runs as several blocks per kv head).
  */
 int32_t qm_decode_attention(
     const uint16_t* query,
