@@ -20,6 +20,10 @@
 //     its words at once and repeats until every tag is the one it expects: the data is its own flag.  Measured
 //     on this chip, 256 blocks: 2.3 to 2.7 us per hand-off of 1 024 to 4 096 words, against 5.4 to 8.3 us for
 //     store + arrive-counter (or flag array) + load.
+//   * The sampler runs in every block: the step's 2 048 scores reach all blocks as any operator's output does and each
+//     block draws from them with its own copy of the generator state — the same code everywhere, so the code needs no
+//     hand-off of its own on its way into the next step's projection.  The last block alone records the code, gathers
+//     its embedding for the caller and stores the generator state at the end.
 //   * Every wait is bounded; a block that gives up raises the abort word, ORs QM_STATUS_FRAME_TIMEOUT into the
 //     status word and returns, and so does every block that sees the abort word: the grid always drains.
 // Arithmetic.  Every operator keeps the reference's summation order and roundings as the one-operator kernels of
@@ -97,7 +101,7 @@ constexpr int kFrWsCtx = kFrWsQkv + kFrQDim + 2 * kFrKvDim;
 constexpr int kFrWsAttn = kFrWsCtx + kFrQDim;
 constexpr int kFrWsAct = kFrWsAttn + kFrHidden;
 constexpr int kFrWsLogits = kFrWsAct + kFrInter;
-constexpr int kFrWsCode = kFrWsLogits + kFrVocab;
+constexpr int kFrWsCode = kFrWsLogits + kFrVocab;        // 16 spare words (the size is part of the interface)
 constexpr int kFrWsWords = kFrWsCode + 16;
 constexpr int64_t kFrWsBytes = (static_cast<int64_t>(kFrWsWords) * 4 + 255) / 256 * 256;
 
@@ -509,7 +513,7 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
     }
     const bool samples = b == kFrBlocks - 1;
     unsigned long long rng = 0;
-    if (samples && tid == 0) rng = *prm.rng_state;
+    if (tid == 0) rng = *prm.rng_state;        // every block keeps the generator's state: all draw, the last one stores it
     __syncthreads();
 
     uint32_t* const hidden = ws + kFrWsHidden;
@@ -518,7 +522,6 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
     uint32_t* const attn = ws + kFrWsAttn;
     uint32_t* const act = ws + kFrWsAct;
     uint32_t* const logits = ws + kFrWsLogits;
-    uint32_t* const code_words = ws + kFrWsCode;
 
 #pragma unroll 1
     for (int position = first; position <= last; ++position) {
@@ -534,18 +537,8 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
         if (position < 2) {
             x_plain = prm.step0_input + position * kFrOuter;
         } else if (position != first) {
-            const uint32_t want = (t0 - kFrPhasesPerStep + 27u) & 0xffffu;
-            uint32_t word = 0;
-            bool ok = false;
-            for (unsigned spins = 0;; ++spins) {
-                word = agent_load(code_words + (step - 1));
-                if ((word >> 16) == want) { ok = true; break; }
-                if (spins >= spin_limit) break;
-                if ((spins & 255u) == 255u && agent_load(abort_word) != 0u) break;
-                __builtin_amdgcn_s_sleep(1);
-            }
-            if (!ok) sh.abort = 1;
-            else x_plain = prm.embeddings[step - 1] + static_cast<int64_t>(word & (kFrVocab - 1)) * kFrOuter;
+            // (the code of the pass before: every block has drawn it itself, below)
+            x_plain = prm.embeddings[step - 1] + static_cast<int64_t>(sh.code) * kFrOuter;
         }
         if (!linear_phase<false, 0, false, kFrOuter, kFrRowsProj>(sh, smem, kFrLdsOm, nullptr, 0, x_plain, nullptr, 0, nullptr, 0.0f,
                                                                   prm.projection_bias, false, 0, kFrRowsProj * b, hidden, tag(0), abort_word, spin_limit))
@@ -607,8 +600,10 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
             break;
         if (position < last) request_proj();
 
-        // ---- the sampler and the gather of the sampled code's embedding: one block ----
-        if (samples) {
+        // ---- the sampler: EVERY block draws the code, from the same scores and the same generator state — the same code
+        // everywhere, and one hand-off fewer per step than one block that samples and tells the others; the last block
+        // also records the code and gathers its embedding (what the host reads and the next launch starts from) ----
+        {
             uint32_t raw[kFrVocab / kFrThreads];
             if (!poll_words<kFrVocab / kFrThreads>(logits, tag(26), abort_word, spin_limit, raw)) sh.abort = 1;
             float score[kSmpPerThread];
@@ -623,13 +618,14 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
             const int32_t chosen = sampler_block(sp, *reinterpret_cast<SamplerScratch*>(smem + kFrLdsScratch), score, rng);
             if (tid == 0) {
                 sh.code = chosen;
-                prm.codes[step + 1] = chosen;
-                agent_store(code_words + step, (tag(27) << 16) | static_cast<uint32_t>(chosen));
+                if (samples) prm.codes[step + 1] = chosen;
             }
             __syncthreads();
-            const uint4 row = reinterpret_cast<const uint4*>(prm.embeddings[step] + static_cast<int64_t>(sh.code) * kFrOuter)[tid];
-            reinterpret_cast<uint4*>(prm.selected + static_cast<int64_t>(step + 1) * kFrOuter)[tid] = row;
-            reinterpret_cast<uint4*>(prm.free_input)[tid] = row;
+            if (samples) {
+                const uint4 row = reinterpret_cast<const uint4*>(prm.embeddings[step] + static_cast<int64_t>(sh.code) * kFrOuter)[tid];
+                reinterpret_cast<uint4*>(prm.selected + static_cast<int64_t>(step + 1) * kFrOuter)[tid] = row;
+                reinterpret_cast<uint4*>(prm.free_input)[tid] = row;
+            }
             __syncthreads();
         }
     }
