@@ -491,27 +491,33 @@ extern "C" int32_t qm_generate(qm_talker* talker, qm_final_head* head, qm_predic
         FrameMailbox mailbox;
         hipStream_t stream = static_cast<hipStream_t>(qm_talker_stream(talker));
         int frames = 0;
-        for (int frame = 0; frame < maximum_frames; ++frame) {
-            final_head_launch(*head, hidden, frame, sampling != 0);
-            hip_check(hipMemcpyAsync(head->rng_after_head.raw(), head->rng.raw(), sizeof(uint64_t), hipMemcpyDeviceToDevice, stream),
-                      "generator state snapshot");
-            const uint16_t* context = frame < trailing_rows ? trailing_text_host + static_cast<size_t>(frame) * kOuter : tts_pad_host;
-            predictor_frame_launch(*predictor, hidden, static_cast<const int32_t*>(head->code.raw()), context, sampling != 0, mailbox.result);
-            hip_check(hipEventRecord(mailbox.arrived, stream), "frame event record");
-            if (frame + 1 < maximum_frames)
-                op_check(qm_talker_decode_device_rope(talker, predictor->next_input.u16(), cos_device + static_cast<size_t>(frame) * kHeadDim,
-                                                      sin_device + static_cast<size_t>(frame) * kHeadDim, frame, &hidden), "talker decode");
-            hip_check(hipEventSynchronize(mailbox.arrived), "frame boundary synchronize");
-            const FrameResult result = *mailbox.result;
-            predictor_frame_finish(*predictor, result);
-            if (result.code0 == kCodecEos && frame >= 2) {
-                hip_check(hipMemcpyAsync(head->rng.raw(), head->rng_after_head.raw(), sizeof(uint64_t), hipMemcpyDeviceToDevice, stream),
-                          "generator state restore");
-                break;
+        // (work queued ahead reads the rope rows and writes the mailbox: nothing may unwind past them while it runs)
+        try {
+            for (int frame = 0; frame < maximum_frames; ++frame) {
+                final_head_launch(*head, hidden, frame, sampling != 0);
+                hip_check(hipMemcpyAsync(head->rng_after_head.raw(), head->rng.raw(), sizeof(uint64_t), hipMemcpyDeviceToDevice, stream),
+                          "generator state snapshot");
+                const uint16_t* context = frame < trailing_rows ? trailing_text_host + static_cast<size_t>(frame) * kOuter : tts_pad_host;
+                predictor_frame_launch(*predictor, hidden, static_cast<const int32_t*>(head->code.raw()), context, sampling != 0, mailbox.result);
+                hip_check(hipEventRecord(mailbox.arrived, stream), "frame event record");
+                if (frame + 1 < maximum_frames)
+                    op_check(qm_talker_decode_device_rope(talker, predictor->next_input.u16(), cos_device + static_cast<size_t>(frame) * kHeadDim,
+                                                          sin_device + static_cast<size_t>(frame) * kHeadDim, frame, &hidden), "talker decode");
+                hip_check(hipEventSynchronize(mailbox.arrived), "frame boundary synchronize");
+                const FrameResult result = *mailbox.result;
+                predictor_frame_finish(*predictor, result);
+                if (result.code0 == kCodecEos && frame >= 2) {
+                    hip_check(hipMemcpyAsync(head->rng.raw(), head->rng_after_head.raw(), sizeof(uint64_t), hipMemcpyDeviceToDevice, stream),
+                              "generator state restore");
+                    break;
+                }
+                if (result.codes[0] != result.code0) throw ApiError(QM_ERR_ARGUMENT, "native Predictor recurrence output mismatch");
+                std::memcpy(codes_out + static_cast<size_t>(frame) * kCodeGroups, result.codes, sizeof result.codes);
+                ++frames;
             }
-            if (result.codes[0] != result.code0) throw ApiError(QM_ERR_ARGUMENT, "native Predictor recurrence output mismatch");
-            std::memcpy(codes_out + static_cast<size_t>(frame) * kCodeGroups, result.codes, sizeof result.codes);
-            ++frames;
+        } catch (...) {
+            (void)hipStreamSynchronize(stream);
+            throw;
         }
         op_check(qm_talker_synchronize(talker), "generation synchronize");
         *frames_out = frames;

@@ -544,9 +544,8 @@ extern "C" int32_t qm_talker_post_attention_workspace_init(void* workspace, int6
 namespace qm {
 namespace {
 
-// The launch; with `attention` the kernel first combines that decode step's split records into `context_out`.
-int32_t launch_chain(const qm_talker_post_attention* op, void* workspace, int64_t workspace_bytes, uint32_t* status_dev,
-                     void* hip_stream, const DecodeSplitInfo* attention, uint16_t* context_out) {
+// What a launch asks of its arguments (everything that can be seen from the host without a device call).
+int32_t check_chain(const qm_talker_post_attention* op, const void* workspace, int64_t workspace_bytes) {
     if (!op || !workspace) return QM_ERR_NULL;
     if (workspace_bytes < kTkWsBytes) return QM_ERR_WORKSPACE;
     if (reinterpret_cast<uintptr_t>(workspace) & 255) return QM_ERR_GEOMETRY;
@@ -565,6 +564,15 @@ int32_t launch_chain(const qm_talker_post_attention* op, void* workspace, int64_
         align |= reinterpret_cast<uintptr_t>(op->next_q_weight) | reinterpret_cast<uintptr_t>(op->next_k_weight)
                | reinterpret_cast<uintptr_t>(op->next_v_weight);
     if (align & 15) return QM_ERR_GEOMETRY;               // 16-byte pieces of weight rows
+    return QM_OK;
+}
+
+// The launch; with `attention` the kernel first combines that decode step's split records into `context_out`.
+int32_t launch_chain(const qm_talker_post_attention* op, void* workspace, int64_t workspace_bytes, uint32_t* status_dev,
+                     void* hip_stream, const DecodeSplitInfo* attention, uint16_t* context_out) {
+    const int32_t bad = check_chain(op, workspace, workspace_bytes);
+    if (bad != QM_OK) return bad;
+    const bool has_next = op->next_q_weight != nullptr;
     TkParams prm = {};
     prm.context = op->context; prm.hidden = op->hidden; prm.o_weight = op->o_weight; prm.o_bias = op->o_bias;
     prm.post_norm = op->post_norm; prm.gate_weight = op->gate_weight; prm.up_weight = op->up_weight;
@@ -626,13 +634,8 @@ extern "C" int32_t qm_talker_layer_step_m1(const qm_talker_layer_step* step, voi
     // validate the second launch's arguments before the first is made: a step is made whole or not at all
     qm_talker_post_attention post = step->post;
     post.context = step->context;
-    if (workspace_bytes < kTkWsBytes) return QM_ERR_WORKSPACE;
-    if (reinterpret_cast<uintptr_t>(workspace) & 255) return QM_ERR_GEOMETRY;
-    if (post.hidden_columns != kTkHidden || post.q_columns != kTkQDim || post.kv_columns != kTkKvDim
-        || post.intermediate_columns != kTkInter)
-        return QM_ERR_GEOMETRY;
-    if (!post.hidden || !post.o_weight || !post.post_norm || !post.gate_weight || !post.up_weight || !post.down_weight || !post.hidden_out)
-        return QM_ERR_NULL;
+    const int32_t bad = check_chain(&post, workspace, workspace_bytes);
+    if (bad != QM_OK) return bad;
     DecodeSplitInfo info = {};
     const int32_t rc = decode_step(step->q, step->k, step->v, step->q_norm_w, step->k_norm_w, step->cos_row, step->sin_row,
                                    step->q_rotated_out, step->cache, step->page_table, step->max_pages, step->context, step->q_heads,

@@ -258,6 +258,12 @@ def test_layer_step_argument_errors(oracle, qm, dev, layer):
     bad = make()
     bad.context = None
     assert call(bad) == -1
+    bad = make()
+    saved = bad.post.next_v_weight
+    bad.post.next_v_weight = None
+    assert call(bad) == -1                                 # (the next layer's arguments as well)
+    bad.post.next_v_weight = saved + 2
+    assert call(bad) == -2
     assert call(make()) == 0
     torch.cuda.synchronize()
     assert qm.lib().qm_talker_layer_step_m1(None, layer.ws.data_ptr(), layer.ws_bytes, None, None) == -1
