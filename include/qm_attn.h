@@ -471,9 +471,10 @@ int32_t qm_predictor_step_attention_m1(
  * down_proj + residual (R17:13614-13780), the final norm with that step's head, the top-k sampler (top_k <= 0:
  * arg-max) and the gather of the sampled code's embedding (R17:13782-13854) — with every rounding and summation
  * order of the one-operator entry points of this header, whose results it equals bit for bit.  Step 0 (two rows: the
- * talker's hidden state and the embedding of the talker's code, R17:13663-13699) is run as two passes at cache
- * positions 0 and 1 with the chain order of the row operators the reference uses there (qm_linear_rows: every row as
- * qm_linear_m1 evaluates it), the first pass without head and sampler: the caches' rows 0 and 1, codes[1], selected[1]
+ * talker's hidden state and the embedding of the talker's code, R17:13663-13699) is run as one pass that takes both
+ * rows through every operator, at cache positions 0 and 1, with the chain order of the row operators the reference uses
+ * there (qm_linear_rows: every row as qm_linear_m1 evaluates it); head and sampler follow the second row: the caches'
+ * rows 0 and 1, codes[1], selected[1]
  * and the next input equal, bit for bit, what the reference's step-0 operators leave (qm_linear_rows, qm_rmsnorm_rows,
  * qm_predictor_transpose / _rope_bhsd / _update_cache, qm_predictor_attention_staged, qm_gate_up_swiglu_rows).
  *

@@ -34,7 +34,9 @@
 // Step 0.  The frame's first step has two rows (the talker's hidden state and the embedding of the talker's code) and
 // the reference runs it through its row operators (R17:13663-13699).  Row by row those are the talker-order M = 1
 // operators — lane l takes k = l, l + 32, ... — and the causal two-row attention is the M = 1 attention at positions
-// 0 and 1: step 0 is run here as two more passes of the same loop with that chain order, the first without a head.
+// 0 and 1: step 0 is one more pass of the same loop with that chain order in which every operator takes the first
+// row and then the second (each row with its own copy of the handed-over vectors), so it waits for the hand-offs of
+// one row; the head and the sampler follow the second row.
 //
 // Geometry is the predictor's (R17:7951-7964): hidden 1024, 16 / 8 heads of 128, intermediate 3072, outer
 // dimension 2048, vocabulary 2048, five layers, cache of 16 positions.
@@ -101,8 +103,10 @@ constexpr int kFrWsCtx = kFrWsQkv + kFrQDim + 2 * kFrKvDim;
 constexpr int kFrWsAttn = kFrWsCtx + kFrQDim;
 constexpr int kFrWsAct = kFrWsAttn + kFrHidden;
 constexpr int kFrWsLogits = kFrWsAct + kFrInter;
-constexpr int kFrWsCode = kFrWsLogits + kFrVocab;        // 16 spare words (the size is part of the interface)
-constexpr int kFrWsWords = kFrWsCode + 16;
+constexpr int kFrWsCode = kFrWsLogits + kFrVocab;        // 16 spare words
+// step 0's second row: a second copy of the vectors from kFrWsHidden up to kFrWsLogits, kFrWsRowShift words further on
+constexpr int kFrWsRowShift = kFrWsCode + 16 - kFrWsHidden;
+constexpr int kFrWsWords = kFrWsHidden + kFrWsRowShift + (kFrWsLogits - kFrWsHidden);
 constexpr int64_t kFrWsBytes = (static_cast<int64_t>(kFrWsWords) * 4 + 255) / 256 * 256;
 
 struct FrLayer {
@@ -150,7 +154,7 @@ struct FrShared {
     float total;
     int abort;
     int code;
-    float residual[4];
+    float residual[8];              // [row of the pass][the block's four down_proj rows]
 };
 
 __device__ __forceinline__ uint32_t agent_load(const uint32_t* p) {
@@ -210,7 +214,7 @@ __device__ __forceinline__ bool linear_phase(FrShared& sh, unsigned char* smem, 
                                              const uint32_t* add_words, uint32_t add_tag,
                                              const uint16_t* norm_w, float epsilon, const uint16_t* bias, bool add_residual,
                                              int keep_residual_first, int first_out, uint32_t* out_words, uint32_t out_tag,
-                                             const uint32_t* abort_word, unsigned spin_limit) {
+                                             const uint32_t* abort_word, unsigned spin_limit, int row = 0) {
     constexpr int N = K / kFrThreads;                   // input columns per thread: tid, tid + 256, ...
     constexpr int kStride = fr_row_stride(K);
     float* lin_x = reinterpret_cast<float*>(smem + kFrLdsScratch);
@@ -246,7 +250,7 @@ __device__ __forceinline__ bool linear_phase(FrShared& sh, unsigned char* smem, 
             float v = bf2f(static_cast<uint16_t>(x_raw[u]));
             if (PRE == 2) {
                 v = bf2f(f2bf(v + bf2f(static_cast<uint16_t>(add_raw[u]))));
-                if (k >= keep_residual_first && k < keep_residual_first + 4) sh.residual[k - keep_residual_first] = v;
+                if (k >= keep_residual_first && k < keep_residual_first + 4) sh.residual[4 * row + k - keep_residual_first] = v;
             }
             lin_x[k] = v;
             local_sum = fmaf(v, v, local_sum);
@@ -331,7 +335,7 @@ __device__ __forceinline__ bool linear_phase(FrShared& sh, unsigned char* smem, 
                 float r = acc;
                 if (bias) r += bf2f(static_cast<uint16_t>(bias_raw));
                 bits = f2bf(r);
-                if (add_residual) bits = f2bf(sh.residual[c] + bf2f(bits));
+                if (add_residual) bits = f2bf(sh.residual[4 * row + c] + bf2f(bits));
             }
             agent_store(out_words + first_out + c, (out_tag << 16) | bits);
         }
@@ -525,77 +529,109 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
 
 #pragma unroll 1
     for (int position = first; position <= last; ++position) {
-        const int step = position - 1;                    // of the head and of the table of the code sampled after this pass
+        // Step 0's two rows go through every operator one after the other, in ONE pass: an operator's weights are in LDS
+        // for both, and the second row's inputs arrive with the first's (its own copy of every handed-over vector,
+        // kFrWsRowShift words further on), so the pass costs the hand-offs of one row.  It writes cache positions 0 and 1
+        // and ends like position 1: with step 0's head and code.
+        const int rows = position == 0 ? 2 : 1;
+        const int head_position = position + rows - 1;
+        const int step = head_position - 1;               // of the head and of the table of the code sampled after this pass
         const bool pairs = position >= 2;                 // the predictor's chain order; step 0 runs the talker's
         const uint32_t t0 = base + static_cast<uint32_t>(position - first) * kFrPhasesPerStep;
         auto tag = [&](int phase) { return (t0 + static_cast<uint32_t>(phase)) & 0xffffu; };
+        bool alive = true;
 
-        // ---- input projection.  The input of the first pass of a launch is given (step 0: the talker's hidden state,
-        // then the embedding of the talker's code; otherwise the free input); a later one's is the embedding of the code
-        // just sampled ----
-        const uint16_t* x_plain = prm.free_input;
-        if (position < 2) {
-            x_plain = prm.step0_input + position * kFrOuter;
-        } else if (position != first) {
-            // (the code of the pass before: every block has drawn it itself, below)
-            x_plain = prm.embeddings[step - 1] + static_cast<int64_t>(sh.code) * kFrOuter;
+        // ---- input projection.  The input of the first pass of a launch is given (step 0: the talker's hidden state
+        // and the embedding of the talker's code; otherwise the free input); a later one's is the embedding of the code
+        // just sampled (every block has drawn it itself, below) ----
+#pragma unroll 1
+        for (int r = 0; alive && r < rows; ++r) {
+            const uint16_t* x_plain = prm.free_input;
+            if (position < 2) x_plain = prm.step0_input + (position + r) * kFrOuter;
+            else if (position != first) x_plain = prm.embeddings[step - 1] + static_cast<int64_t>(sh.code) * kFrOuter;
+            alive = linear_phase<false, 0, false, kFrOuter, kFrRowsProj>(sh, smem, kFrLdsOm, nullptr, 0, x_plain, nullptr, 0, nullptr, 0.0f,
+                                                                         prm.projection_bias, false, 0, kFrRowsProj * b,
+                                                                         hidden + r * kFrWsRowShift, tag(0), abort_word, spin_limit, r);
         }
-        if (!linear_phase<false, 0, false, kFrOuter, kFrRowsProj>(sh, smem, kFrLdsOm, nullptr, 0, x_plain, nullptr, 0, nullptr, 0.0f,
-                                                                  prm.projection_bias, false, 0, kFrRowsProj * b, hidden, tag(0), abort_word, spin_limit))
-            break;
+        if (!alive) break;
         request_o(prm.layers[0]);
         uint32_t hidden_tag = tag(0);
-        bool alive = true;
 
 #pragma unroll 1
         for (int layer = 0; layer < kFrLayers; ++layer) {
             const FrLayer& w = prm.layers[layer];
-            const bool more = layer + 1 < kFrLayers || position < last;      // is there a next layer to request weights for
+            const bool more = layer + 1 < kFrLayers || head_position < last;      // is there a next layer to request weights for
             const FrLayer& next = prm.layers[layer + 1 < kFrLayers ? layer + 1 : 0];
             const int p = 1 + 5 * layer;
-            alive = pairs
-                ? linear_phase<false, 1, true, kFrHidden, kFrRowsQkv>(sh, smem, kFrLdsQkv, hidden, hidden_tag, nullptr, nullptr, 0, w.input_norm,
-                                                                      prm.epsilon, nullptr, false, 0, qkv_row, qkv, tag(p), abort_word, spin_limit)
-                : linear_phase<false, 1, false, kFrHidden, kFrRowsQkv>(sh, smem, kFrLdsQkv, hidden, hidden_tag, nullptr, nullptr, 0, w.input_norm,
-                                                                       prm.epsilon, nullptr, false, 0, qkv_row, qkv, tag(p), abort_word, spin_limit);
+#pragma unroll 1
+            for (int r = 0; alive && r < rows; ++r) {
+                const int shift = r * kFrWsRowShift;
+                alive = pairs
+                    ? linear_phase<false, 1, true, kFrHidden, kFrRowsQkv>(sh, smem, kFrLdsQkv, hidden + shift, hidden_tag, nullptr, nullptr, 0,
+                                                                          w.input_norm, prm.epsilon, nullptr, false, 0, qkv_row, qkv + shift,
+                                                                          tag(p), abort_word, spin_limit, r)
+                    : linear_phase<false, 1, false, kFrHidden, kFrRowsQkv>(sh, smem, kFrLdsQkv, hidden + shift, hidden_tag, nullptr, nullptr, 0,
+                                                                           w.input_norm, prm.epsilon, nullptr, false, 0, qkv_row, qkv + shift,
+                                                                           tag(p), abort_word, spin_limit, r);
+            }
             if (!alive) break;
             if (more) request_qkv(next);
             if (attends && my_layer == layer) {
-                if (!attention_phase(sh, smem, prm, w, my_head, position, qkv, tag(p), ctx, tag(p + 1), abort_word, spin_limit)) { alive = false; break; }
+#pragma unroll 1
+                for (int r = 0; alive && r < rows; ++r)
+                    alive = attention_phase(sh, smem, prm, w, my_head, position + r, qkv + r * kFrWsRowShift, tag(p), ctx + r * kFrWsRowShift,
+                                            tag(p + 1), abort_word, spin_limit);
+                if (!alive) break;
             }
-            alive = pairs
-                ? linear_phase<false, 0, true, kFrQDim, kFrRowsO>(sh, smem, kFrLdsOm, ctx, tag(p + 1), nullptr, nullptr, 0, nullptr, 0.0f, nullptr,
-                                                                  false, 0, kFrRowsO * b, attn, tag(p + 2), abort_word, spin_limit)
-                : linear_phase<false, 0, false, kFrQDim, kFrRowsO>(sh, smem, kFrLdsOm, ctx, tag(p + 1), nullptr, nullptr, 0, nullptr, 0.0f, nullptr,
-                                                                   false, 0, kFrRowsO * b, attn, tag(p + 2), abort_word, spin_limit);
+#pragma unroll 1
+            for (int r = 0; alive && r < rows; ++r) {
+                const int shift = r * kFrWsRowShift;
+                alive = pairs
+                    ? linear_phase<false, 0, true, kFrQDim, kFrRowsO>(sh, smem, kFrLdsOm, ctx + shift, tag(p + 1), nullptr, nullptr, 0, nullptr, 0.0f,
+                                                                      nullptr, false, 0, kFrRowsO * b, attn + shift, tag(p + 2), abort_word,
+                                                                      spin_limit, r)
+                    : linear_phase<false, 0, false, kFrQDim, kFrRowsO>(sh, smem, kFrLdsOm, ctx + shift, tag(p + 1), nullptr, nullptr, 0, nullptr, 0.0f,
+                                                                       nullptr, false, 0, kFrRowsO * b, attn + shift, tag(p + 2), abort_word,
+                                                                       spin_limit, r);
+            }
             if (!alive) break;
-            // (the region after the last o_proj holds the pass's head; the first pass of step 0 has none)
+            // (the region after the last o_proj holds the pass's head)
             if (layer + 1 < kFrLayers) request_o(next);
-            else if (position == 0) request_proj();
             else request_head(step);
-            alive = pairs
-                ? linear_phase<true, 2, true, kFrHidden, kFrRowsGu>(sh, smem, kFrLdsGu, hidden, hidden_tag, nullptr, attn, tag(p + 2), w.post_norm,
-                                                                    prm.epsilon, nullptr, false, kFrRowsDown * b, kFrRowsGu * b, act, tag(p + 3),
-                                                                    abort_word, spin_limit)
-                : linear_phase<true, 2, false, kFrHidden, kFrRowsGu>(sh, smem, kFrLdsGu, hidden, hidden_tag, nullptr, attn, tag(p + 2), w.post_norm,
-                                                                     prm.epsilon, nullptr, false, kFrRowsDown * b, kFrRowsGu * b, act, tag(p + 3),
-                                                                     abort_word, spin_limit);
+#pragma unroll 1
+            for (int r = 0; alive && r < rows; ++r) {
+                const int shift = r * kFrWsRowShift;
+                alive = pairs
+                    ? linear_phase<true, 2, true, kFrHidden, kFrRowsGu>(sh, smem, kFrLdsGu, hidden + shift, hidden_tag, nullptr, attn + shift,
+                                                                        tag(p + 2), w.post_norm, prm.epsilon, nullptr, false, kFrRowsDown * b,
+                                                                        kFrRowsGu * b, act + shift, tag(p + 3), abort_word, spin_limit, r)
+                    : linear_phase<true, 2, false, kFrHidden, kFrRowsGu>(sh, smem, kFrLdsGu, hidden + shift, hidden_tag, nullptr, attn + shift,
+                                                                         tag(p + 2), w.post_norm, prm.epsilon, nullptr, false, kFrRowsDown * b,
+                                                                         kFrRowsGu * b, act + shift, tag(p + 3), abort_word, spin_limit, r);
+            }
             if (!alive) break;
             if (more) request_gu(next);
-            alive = pairs
-                ? linear_phase<false, 0, true, kFrInter, kFrRowsDown>(sh, smem, kFrLdsDown, act, tag(p + 3), nullptr, nullptr, 0, nullptr, 0.0f,
-                                                                      nullptr, true, 0, kFrRowsDown * b, hidden, tag(p + 4), abort_word, spin_limit)
-                : linear_phase<false, 0, false, kFrInter, kFrRowsDown>(sh, smem, kFrLdsDown, act, tag(p + 3), nullptr, nullptr, 0, nullptr, 0.0f,
-                                                                       nullptr, true, 0, kFrRowsDown * b, hidden, tag(p + 4), abort_word, spin_limit);
+#pragma unroll 1
+            for (int r = 0; alive && r < rows; ++r) {
+                const int shift = r * kFrWsRowShift;
+                alive = pairs
+                    ? linear_phase<false, 0, true, kFrInter, kFrRowsDown>(sh, smem, kFrLdsDown, act + shift, tag(p + 3), nullptr, nullptr, 0, nullptr,
+                                                                          0.0f, nullptr, true, 0, kFrRowsDown * b, hidden + shift, tag(p + 4),
+                                                                          abort_word, spin_limit, r)
+                    : linear_phase<false, 0, false, kFrInter, kFrRowsDown>(sh, smem, kFrLdsDown, act + shift, tag(p + 3), nullptr, nullptr, 0, nullptr,
+                                                                           0.0f, nullptr, true, 0, kFrRowsDown * b, hidden + shift, tag(p + 4),
+                                                                           abort_word, spin_limit, r);
+            }
             if (!alive) break;
             if (more) request_down(next);
             hidden_tag = tag(p + 4);
         }
         if (!alive) break;
-        if (position == 0) continue;                      // step 0's first row: its keys and values are what it leaves
+        uint32_t* const last_hidden = hidden + (rows - 1) * kFrWsRowShift;   // step 0's head reads its second row
+        position = head_position;
 
         // ---- final norm + this step's head ----
-        if (!linear_phase<false, 1, false, kFrHidden, kFrRowsHead>(sh, smem, kFrLdsOm, hidden, hidden_tag, nullptr, nullptr, 0, prm.final_norm,
+        if (!linear_phase<false, 1, false, kFrHidden, kFrRowsHead>(sh, smem, kFrLdsOm, last_hidden, hidden_tag, nullptr, nullptr, 0, prm.final_norm,
                                                                    prm.epsilon, nullptr, false, 0, kFrRowsHead * b, logits, tag(26), abort_word, spin_limit))
             break;
         if (position < last) request_proj();
