@@ -531,6 +531,10 @@ typedef struct qm_predictor_frame {
     uint64_t* rng_state;
     float epsilon;
     const uint16_t* step0_input;      /* [2][2048], first_step == 0 only */
+    /* Optional.  projected[s] [2048][1024]: row c = the input projection (with its bias, as qm_linear_m1 evaluates it)
+     * of row c of embeddings[s].  Where it is given, the step after s starts from that row instead of computing the
+     * projection of the embedding of the code just sampled — one operator fewer per step, same bits.  NULL: computed. */
+    const uint16_t* projected[15];
 } qm_predictor_frame;
 
 int64_t qm_predictor_frame_workspace_bytes(void);

@@ -48,6 +48,7 @@ class PredictorFrame(C.Structure):
         ("free_input", C.c_void_p), ("selected", C.c_void_p), ("codes", C.c_void_p), ("rng_state", C.c_void_p),
         ("epsilon", C.c_float),
         ("step0_input", C.c_void_p),
+        ("projected", C.c_void_p * 15),
     ]
 
 
@@ -479,9 +480,9 @@ STATUS_BAD_PAGE, STATUS_BAD_POSITION, STATUS_SPLIT_TIMEOUT, STATUS_FRAME_TIMEOUT
 
 
 def predictor_frame(layers, projection_weight, projection_bias, final_norm, heads, embeddings, cosine, sine, free_input,
-                    selected, codes, rng_state, epsilon=1e-6, step0_input=None):
+                    selected, codes, rng_state, epsilon=1e-6, step0_input=None, projected=None):
     """qm_predictor_frame from tensors: `layers` is five dicts with the field names of qm_predictor_frame_layer,
-    `heads` / `embeddings` map a step (1..14) to its tensor.  The tensors must outlive the descriptor."""
+    `heads` / `embeddings` (and `projected`, optional) map a step to its tensor.  The tensors must outlive the descriptor."""
     frame = PredictorFrame()
     for i, layer in enumerate(layers):
         for name, _ in PredictorFrameLayer._fields_:
@@ -497,6 +498,8 @@ def predictor_frame(layers, projection_weight, projection_bias, final_norm, head
                                                                       _addr(rng_state))
     frame.epsilon = epsilon
     frame.step0_input = _addr(step0_input)
+    for step, tensor in (projected or {}).items():
+        frame.projected[step] = _addr(tensor)
     return frame
 
 

@@ -132,6 +132,7 @@ struct FrParams {
     const uint16_t* final_norm;
     const uint16_t* heads[kFrLastStep + 1];          // [step]
     const uint16_t* embeddings[kFrLastStep + 1];     // [step]
+    const uint16_t* projected[kFrLastStep + 1];      // [step] optional: the projection of every row of embeddings[step]
     const uint16_t* cosine;                          // [16][128]
     const uint16_t* sine;
     const uint16_t* step0_input;                     // [2][2048] (first_step == 0)
@@ -540,12 +541,15 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
         const uint32_t t0 = base + static_cast<uint32_t>(position - first) * kFrPhasesPerStep;
         auto tag = [&](int phase) { return (t0 + static_cast<uint32_t>(phase)) & 0xffffu; };
         bool alive = true;
+        // the pass's input already projected (a table row of the code just sampled): no projection operator
+        const uint16_t* const projected_row = position >= 2 && position != first && prm.projected[step - 1]
+            ? prm.projected[step - 1] + static_cast<int64_t>(sh.code) * kFrHidden : nullptr;
 
         // ---- input projection.  The input of the first pass of a launch is given (step 0: the talker's hidden state
         // and the embedding of the talker's code; otherwise the free input); a later one's is the embedding of the code
         // just sampled (every block has drawn it itself, below) ----
 #pragma unroll 1
-        for (int r = 0; alive && r < rows; ++r) {
+        for (int r = 0; alive && !projected_row && r < rows; ++r) {
             const uint16_t* x_plain = prm.free_input;
             if (position < 2) x_plain = prm.step0_input + (position + r) * kFrOuter;
             else if (position != first) x_plain = prm.embeddings[step - 1] + static_cast<int64_t>(sh.code) * kFrOuter;
@@ -554,7 +558,7 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
                                                                          hidden + r * kFrWsRowShift, tag(0), abort_word, spin_limit, r);
         }
         if (!alive) break;
-        request_o(prm.layers[0]);
+        if (!projected_row) request_o(prm.layers[0]);       // (else requested when the head had been read)
         uint32_t hidden_tag = tag(0);
 
 #pragma unroll 1
@@ -563,11 +567,12 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
             const bool more = layer + 1 < kFrLayers || head_position < last;      // is there a next layer to request weights for
             const FrLayer& next = prm.layers[layer + 1 < kFrLayers ? layer + 1 : 0];
             const int p = 1 + 5 * layer;
+            const uint16_t* const x_given = layer == 0 ? projected_row : nullptr;   // in place of `hidden` as handed over
 #pragma unroll 1
             for (int r = 0; alive && r < rows; ++r) {
                 const int shift = r * kFrWsRowShift;
                 alive = pairs
-                    ? linear_phase<false, 1, true, kFrHidden, kFrRowsQkv>(sh, smem, kFrLdsQkv, hidden + shift, hidden_tag, nullptr, nullptr, 0,
+                    ? linear_phase<false, 1, true, kFrHidden, kFrRowsQkv>(sh, smem, kFrLdsQkv, hidden + shift, hidden_tag, x_given, nullptr, 0,
                                                                           w.input_norm, prm.epsilon, nullptr, false, 0, qkv_row, qkv + shift,
                                                                           tag(p), abort_word, spin_limit, r)
                     : linear_phase<false, 1, false, kFrHidden, kFrRowsQkv>(sh, smem, kFrLdsQkv, hidden + shift, hidden_tag, nullptr, nullptr, 0,
@@ -602,7 +607,7 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
             for (int r = 0; alive && r < rows; ++r) {
                 const int shift = r * kFrWsRowShift;
                 alive = pairs
-                    ? linear_phase<true, 2, true, kFrHidden, kFrRowsGu>(sh, smem, kFrLdsGu, hidden + shift, hidden_tag, nullptr, attn + shift,
+                    ? linear_phase<true, 2, true, kFrHidden, kFrRowsGu>(sh, smem, kFrLdsGu, hidden + shift, hidden_tag, x_given, attn + shift,
                                                                         tag(p + 2), w.post_norm, prm.epsilon, nullptr, false, kFrRowsDown * b,
                                                                         kFrRowsGu * b, act + shift, tag(p + 3), abort_word, spin_limit, r)
                     : linear_phase<true, 2, false, kFrHidden, kFrRowsGu>(sh, smem, kFrLdsGu, hidden + shift, hidden_tag, nullptr, attn + shift,
@@ -634,7 +639,11 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
         if (!linear_phase<false, 1, false, kFrHidden, kFrRowsHead>(sh, smem, kFrLdsOm, last_hidden, hidden_tag, nullptr, nullptr, 0, prm.final_norm,
                                                                    prm.epsilon, nullptr, false, 0, kFrRowsHead * b, logits, tag(26), abort_word, spin_limit))
             break;
-        if (position < last) request_proj();
+        // the region is free again: the next pass's projection, or — if its input comes projected — its first o_proj
+        if (position < last) {
+            if (prm.projected[step]) request_o(prm.layers[0]);
+            else request_proj();
+        }
 
         // ---- the sampler: EVERY block draws the code, from the same scores and the same generator state — the same code
         // everywhere, and one hand-off fewer per step than one block that samples and tells the others; the last block
@@ -737,6 +746,7 @@ extern "C" int32_t qm_predictor_frame_steps(const qm_predictor_frame* frame, int
     for (int step = first_step; step <= last_step; ++step) {
         prm.heads[step] = frame->heads[step];
         prm.embeddings[step] = frame->embeddings[step];
+        prm.projected[step] = frame->projected[step];
         all = take(frame->heads[step]) && take(frame->embeddings[step]) && all;
     }
     if (!all) return QM_ERR_NULL;

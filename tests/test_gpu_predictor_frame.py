@@ -202,6 +202,47 @@ def test_frame_steps_in_several_launches(frame):
     assert _same(frame.snapshot(), want)
 
 
+def test_frame_steps_from_projected_embedding_tables(frame, qm, dev):
+    """With `projected` tables (the input projection of every embedding row, in qm_linear_m1's chain) a step starts from a
+    table row instead of projecting the sampled code's embedding: same codes, embeddings, caches and generator state —
+    for the whole frame, for launches that start in the middle, and with tables for some steps only."""
+    import torch
+    tables = {}
+    qm.set_option(qm.OPT_LINEAR_ROWS_KERNEL, 1)            # the exact chain: row by row what qm_linear_m1 gives
+    try:
+        for s in range(0, 14):
+            tables[s] = torch.zeros((V, H), dtype=torch.int16, device=dev)
+            qm.linear_rows(frame.tables[s], frame.proj_w, frame.proj_b, None, tables[s], V, H, OUT)
+    finally:
+        qm.set_option(qm.OPT_LINEAR_ROWS_KERNEL, 0)
+    torch.cuda.synchronize()
+    # (one row against the M = 1 operator itself)
+    one = torch.zeros(H, dtype=torch.int16, device=dev)
+    qm.linear_m1(frame.tables[3][77], frame.proj_w, frame.proj_b, None, one, H, OUT)
+    assert torch.equal(one, tables[3][77])
+    saved = {s: frame.frame.projected[s] for s in range(15)}
+    try:
+        for given in (range(0, 14), (2, 3, 9)):
+            for first, last in ((0, 14), (1, 14), (5, 9)):
+                for s in range(15):
+                    frame.frame.projected[s] = None
+                frame.reset()
+                if first > 1:
+                    frame.one_launch(1, first - 1, 50)
+                frame.one_launch(first, last, 50)
+                want = frame.snapshot()
+                for s in given:
+                    frame.frame.projected[s] = tables[s].data_ptr()
+                frame.reset()
+                if first > 1:
+                    frame.one_launch(1, first - 1, 50)
+                frame.one_launch(first, last, 50)
+                assert _same(frame.snapshot(), want) and int(frame.status.item()) == 0
+    finally:
+        for s in range(15):
+            frame.frame.projected[s] = saved[s]
+
+
 def test_frame_steps_replayed_from_a_graph(frame):
     """A captured launch is replayed with the operator numbers the workspace has reached by then: every replay, with the
     program's own eager work in between, gives the eager result."""
