@@ -97,6 +97,7 @@ static_assert(kFrInter * 4 <= kFrLdsScratchBytes, "the longest input vector as f
 // workspace map (32-bit words)
 constexpr int kFrWsBase = 0;          // number of the next launch's first operator instance
 constexpr int kFrWsAbort = 1;
+constexpr int kFrWsLastDual = 2;      // first tag of the last pass that wrote the second row's vectors (step 0)
 constexpr int kFrWsHidden = 64;
 constexpr int kFrWsQkv = kFrWsHidden + kFrHidden;
 constexpr int kFrWsCtx = kFrWsQkv + kFrQDim + 2 * kFrKvDim;
@@ -460,6 +461,8 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
     uint32_t* const ws = prm.workspace;
     const uint32_t* const abort_word = ws + kFrWsAbort;
     const uint32_t base = agent_load(ws + kFrWsBase);
+    const uint32_t last_dual = agent_load(ws + kFrWsLastDual);
+    uint32_t dual_t0 = last_dual;
     if (tid == 0) sh.abort = agent_load(abort_word) != 0u ? 1 : 0;   // a launch gave up and the workspace was not set up again
     __syncthreads();
     if (sh.abort) {
@@ -538,7 +541,14 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
         const int head_position = position + rows - 1;
         const int step = head_position - 1;               // of the head and of the table of the code sampled after this pass
         const bool pairs = position >= 2;                 // the predictor's chain order; step 0 runs the talker's
-        const uint32_t t0 = base + static_cast<uint32_t>(position - first) * kFrPhasesPerStep;
+        uint32_t t0 = base + static_cast<uint32_t>(position - first) * kFrPhasesPerStep;
+        if (rows == 2) {
+            // The second row's vectors are written by step 0 only: what they hold may be any number of launches old, and
+            // tags repeat after 65 536.  If this pass's tags would be those of the pass that wrote them last, it takes
+            // the tags of position 1, which a launch with step 0 does not use otherwise.
+            if (((t0 ^ last_dual) & 0xffffu) == 0u) t0 += kFrPhasesPerStep;
+            dual_t0 = t0;
+        }
         auto tag = [&](int phase) { return (t0 + static_cast<uint32_t>(phase)) & 0xffffu; };
         bool alive = true;
         // the pass's input already projected (a table row of the code just sampled): no projection operator
@@ -685,7 +695,10 @@ __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams
     if (tid == 0) {
         if (samples) *prm.rng_state = rng;
         // (every block has read the base before this one could finish its last operator)
-        if (b == 0) agent_store(ws + kFrWsBase, base + static_cast<uint32_t>(kFrPositions) * kFrPhasesPerStep);
+        if (b == 0) {
+            agent_store(ws + kFrWsBase, base + static_cast<uint32_t>(kFrPositions) * kFrPhasesPerStep);
+            if (dual_t0 != last_dual) agent_store(ws + kFrWsLastDual, dual_t0);
+        }
     }
 }
 

@@ -185,6 +185,35 @@ def test_step_0_and_the_whole_frame_in_one_launch(frame, top_k):
     assert _same(frame.snapshot(), want)
 
 
+def test_step_0_after_the_operator_numbers_wrapped_around(frame):
+    """The vectors of step 0's second row are written by launches with step 0 only, and the 16-bit operator numbers in their
+    words repeat after 128 launches: a launch whose numbers would equal those of the launch that wrote them last takes
+    other numbers for that pass (the words then hold another frame's values, which must not be taken for this frame's)."""
+    import torch
+    frame.reset()
+    frame.one_launch(0, 14, 50)
+    want = frame.snapshot()
+    other = frame.step0_rows.clone()
+    try:
+        frame.step0_rows.copy_(torch.roll(other, 1, dims=1))   # another frame's step 0 leaves its second-row vectors ...
+        frame.reset()
+        frame.one_launch(0, 0, 50)
+        torch.cuda.synchronize()
+        last = int(frame.ws[2].item())                         # (the first operator number of that pass)
+        assert last == int(frame.ws[0].item()) - 512
+        frame.ws[0] = last + 65536                             # ... and 128 launches later the numbers are the same again
+        frame.step0_rows.copy_(other)
+        frame.reset()
+        frame.one_launch(0, 14, 50)
+        assert _same(frame.snapshot(), want) and int(frame.status.item()) == 0
+        assert int(frame.ws[2].item()) == last + 65536 + 32
+    finally:
+        frame.step0_rows.copy_(other)
+        frame.status.zero_()
+        frame.qm.predictor_frame_workspace_init(frame.ws, frame.ws_bytes)
+        torch.cuda.synchronize()
+
+
 def test_frame_steps_in_several_launches(frame):
     """Steps 1..14 as 1..5, 6..6 and 7..14: each launch continues from the caches, the input and the state the one before left."""
     frame.reset()
