@@ -84,13 +84,14 @@ constexpr int kTkUnits = 12;
 // workspace map (32-bit words)
 constexpr int kTkWsBase = 0;                         // number of the next launch's first operator instance
 constexpr int kTkWsAbort = 1;
+constexpr int kTkWsLastContext = 2;                  // operator number in the context words, as the last launch that wrote them left it
 constexpr int kTkWsAttn = 64;
 constexpr int kTkWsAct = kTkWsAttn + kTkHidden;
 constexpr int kTkWsHidden = kTkWsAct + kTkInter;
 constexpr int kTkWsContext = kTkWsHidden + kTkHidden;   // the attention's output, when this launch combines its splits
 constexpr int kTkWsWords = kTkWsContext + kTkQDim;
 constexpr int64_t kTkWsBytes = (static_cast<int64_t>(kTkWsWords) * 4 + 255) / 256 * 256;
-constexpr uint32_t kTkTagsPerLaunch = 4;
+constexpr uint32_t kTkTagsPerLaunch = 8;               // 0..3 used; 5: the context's second choice (below)
 
 struct TkParams {
     const uint16_t* context;
@@ -210,6 +211,12 @@ __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p)
     uint32_t* const ws = p.workspace;
     const uint32_t* const abort_word = ws + kTkWsAbort;
     const uint32_t base = agent_load(ws + kTkWsBase);
+    // The context words are written only by launches that combine the attention's splits: what they hold may be any
+    // number of launches old, and the 16-bit operator numbers repeat.  A launch whose number for them would be the one
+    // they were last written with takes its second choice.
+    const uint32_t last_context = agent_load(ws + kTkWsLastContext);
+    const uint32_t context_number = ((base + 3u) ^ last_context) & 0xffffu ? base + 3u : base + 5u;
+    const uint32_t context_tag = context_number & 0xffffu;
     if (tid == 0) {
         sh.abort = agent_load(abort_word) != 0u ? 1 : 0;   // a launch gave up and the workspace was not set up again
         sh.landed[0] = sh.landed[1] = sh.landed[2] = sh.landed[3] = 0;
@@ -402,7 +409,7 @@ __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p)
                     }
                 }
                 const uint16_t bits = f2bf(ll > 0.0f ? aa / ll : 0.0f);
-                agent_store(ws + kTkWsContext + 256 * b + tid, (tag(3) << 16) | bits);
+                agent_store(ws + kTkWsContext + 256 * b + tid, (context_tag << 16) | bits);
                 if (p.context_out) p.context_out[256 * b + tid] = bits;
                 alive = compute_barrier();                          // the statistics have been read: the input vector may be written
             }
@@ -417,7 +424,7 @@ __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p)
                 // ---- o_proj (R17:17203-17210): the attention's output is given ----
                 uint32_t raw[kPerThread];
                 if (p.attention_records) {
-                    alive = poll_words<kPerThread>(ws + kTkWsContext, tag(3), abort_word, spin_limit, raw);
+                    alive = poll_words<kPerThread>(ws + kTkWsContext, context_tag, abort_word, spin_limit, raw);
                     if (!alive) give_up();
                 } else {
 #pragma unroll
@@ -515,7 +522,10 @@ __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p)
         return;
     }
     // (every block has read the base before this one could finish its last operator)
-    if (tid == 0 && b == 0) agent_store(ws + kTkWsBase, base + kTkTagsPerLaunch);
+    if (tid == 0 && b == 0) {
+        agent_store(ws + kTkWsBase, base + kTkTagsPerLaunch);
+        if (p.attention_records) agent_store(ws + kTkWsLastContext, context_number);
+    }
 }
 
 // Sets a workspace to "nothing produced yet": every tagged word 0, operator numbers from 1 (a kernel, not a

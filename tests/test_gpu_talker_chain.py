@@ -221,13 +221,27 @@ def test_layer_step_in_two_launches_equals_attention_then_the_one_launch(oracle,
         t.fill_(0x7fc0)
     step = qm.talker_layer_step(q, k, v, gq, gk, cos, sin, qrot2, cache2, table2, mp, ctx2, 16, pos, -1, SCALE, 1e-6, ws, ws_bytes,
                                 layer.descriptor())
-    for _ in range(2):                                     # a second step finds the workspaces as the first left them
+    for turn in range(3):                                  # a second step finds the workspaces as the first left them
+        wraps = turn == 2 and int(layer.ws[2].item()) == int(layer.ws[0].item()) - 8 + 3   # (the last launch combined splits)
+        if wraps:
+            # ... and a third whose 16-bit operator number for the context words would be the one they were last written
+            # with (65 536 numbers later) takes its second choice instead of taking the old words for its own: the old
+            # words are made wrong here (their numbers kept), so taking them would show
+            last = int(layer.ws[2].item())
+            layer.ws[0] = last - 3 + 65536
+            words = layer.ws[64 + 2048 + 6144 + 2048:][:2048]      # (the context words follow the three handed-over vectors)
+            words ^= 0x0101
+            for t in layer.got.values():
+                t.fill_(0x7fc0)
         qm.talker_layer_step_m1(step, layer.ws, layer.ws_bytes, layer.status)
         torch.cuda.synchronize()
         assert int(layer.status.item()) == 0
         assert np.array_equal(to_u16(ctx2), to_u16(ctx1)) and np.array_equal(to_u16(qrot2), to_u16(qrot1))
         assert np.array_equal(to_u16(kd2), to_u16(kd1)) and np.array_equal(to_u16(vd2), to_u16(vd1))
         assert layer.same()
+        if wraps:
+            assert int(layer.ws[2].item()) == last + 65536 + 2
+    assert wraps or ctx < 130 or qm.get_option(qm.OPT_DECODE_TILES_PER_BLOCK) != 0   # (the case was exercised where splits are combined)
 
 
 def test_layer_step_with_more_splits_than_one_merge_round(oracle, qm, dev, layer):
