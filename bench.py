@@ -1,14 +1,17 @@
 #!/usr/bin/env python3
 """Benchmark of the attention / KV-cache hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--headline-only] [--all] [--only NAME]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM.  The headline workload is the ragged multi-stream decode (64 streams, context lengths
 uniform in [256, 4096], 16-token pages behind a shuffled page table): the one decode
 configuration whose working set (~0.57 GB) exceeds the caches, so that "HBM GB/s" means HBM.
-The other configurations are timed too (`--all`, default on) and reported under `per_config`.
-One JSON line is printed on stdout.
+The other four configurations and the four widened rows that make up a generated frame are timed too;
+`--all` adds every variant row, `--only NAME` times one row alone (for a profiler).  The full record of
+every row goes to stdout on a line that starts with `per_config ` and to gpurun_out/bench_per_config.json;
+the LAST stdout line is one compact JSON object (metric, value, roofline, cpu_baseline and a
+`summary` of {row: [us per step, fraction of the bounding peak]}), short enough to survive a tail.
 
 Inputs come from the seeded SplitMix64 -> Box-Muller stream that the parity tests use (class Synthetic,
 evaluated on the device); the CPU baseline leg copies the same tensors to the host and times the
@@ -1045,6 +1048,38 @@ def _report(w, ms):
     return rep
 
 
+def _summary(per_config):
+    """{row: [microseconds per step (graph replay where taken), fraction of the peak that bounds the row]}."""
+    out = {}
+    for key, r in per_config.items():
+        if "us_per_step" not in r:
+            if "us_per_frame" in r:
+                out[key] = [round(r["us_per_frame"], 1), None]
+            continue
+        us = r.get("us_per_step_graph", r["us_per_step"])
+        work, peak = (r["algorithmic_flops"], MFMA_BF16_PEAK_TFLOPS * 1e12) if r.get("bound") == "mfma" \
+            else (r["algorithmic_bytes"], HBM_PEAK_GBPS * 1e9)
+        out[key] = [round(us, 2), round(work / (us * 1e-6) / peak, 4)]
+    return out
+
+
+FINAL_LINE_LIMIT = 4000  # bytes; the last stdout line must survive a tail of a few KB
+
+
+def compact_line(line):
+    """The last stdout line: the record as JSON, with the summary's row names shortened and, if still too
+    long, dropped, so that it stays below FINAL_LINE_LIMIT bytes."""
+    text = json.dumps(line, separators=(",", ":"))
+    if len(text) > FINAL_LINE_LIMIT:
+        line = dict(line)
+        line["summary"] = {k: v for k, v in line.get("summary", {}).items() if k.startswith("cfg")}
+        text = json.dumps(line, separators=(",", ":"))
+    if len(text) > FINAL_LINE_LIMIT:
+        line.pop("summary", None)
+        text = json.dumps(line, separators=(",", ":"))
+    return text
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -1052,6 +1087,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="time only the headline workload")
+    ap.add_argument("--all", action="store_true", help="time every variant row, not only the five configurations and "
+                                                       "the four rows of a generated frame")
     ap.add_argument("--only", choices=["decode512", "talker2048", "prefill", "prefill1", "prefill1split", "prefillfp32", "chunk", "chunkwhole", "chunkrows", "predictor", "predictorexact",
                                       "qkv", "layer", "layer1", "layer2", "frame", "frame1", "linears", "linearsexact", "linears128", "linears128split", "generate"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
@@ -1120,47 +1157,50 @@ def main():
         from oracle import binding as oracle
         oracle.build()
     if not args.headline_only:
-        extra = [
-            ("cfg1_decode_ctx512", lambda: SingleDecode(qm, dev, 512, False, 11)),
-            ("cfg2_talker_fused_step_ctx2048", lambda: SingleDecode(qm, dev, 2048, True, 12)),
+        # (row name, constructor, in the default run?)  The default run holds the five configurations and the rows
+        # that make up a generated frame; the variants come with --all.
+        rows = [
+            ("cfg1_decode_ctx512", lambda: SingleDecode(qm, dev, 512, False, 11), True),
+            ("cfg2_talker_fused_step_ctx2048", lambda: SingleDecode(qm, dev, 2048, True, 12), True),
             # the same step over 64 distinct KV caches in rotation (0.54 GB): defeats L2 / MALL
             # residency, as consecutive layers of a real decode step do
-            ("cfg2_talker_fused_step_ctx2048_rotating64", lambda: SingleDecode(qm, dev, 2048, True, 12, copies=64)),
+            ("cfg2_talker_fused_step_ctx2048_rotating64", lambda: SingleDecode(qm, dev, 2048, True, 12, copies=64), False),
             # the same step as the reference launches it: append kernel, then attention
-            ("cfg2_talker_step_ctx2048_two_operators", lambda: SingleDecode(qm, dev, 2048, True, 12, one_launch=False)),
-            ("cfg4_causal_prefill", lambda: Prefill(qm, dev)),
-            ("cfg4_causal_prefill_fp32_scores", lambda: Prefill(qm, dev, score_rounding=0)),
+            ("cfg2_talker_step_ctx2048_two_operators", lambda: SingleDecode(qm, dev, 2048, True, 12, one_launch=False), False),
+            ("cfg4_causal_prefill", lambda: Prefill(qm, dev), True),
+            ("cfg4_causal_prefill_bf16_scores", lambda: Prefill(qm, dev, score_rounding=1), False),
             # one prompt, as the talker's prefill runs it: 128 blocks for 256 CUs; the key-split entry fills them
-            ("cfg4b_causal_prefill_one_prompt_1024", lambda: Prefill(qm, dev, batch=1)),
-            ("cfg4b_causal_prefill_one_prompt_1024_key_split", lambda: Prefill(qm, dev, batch=1, split=True)),
+            ("cfg4b_causal_prefill_one_prompt_1024", lambda: Prefill(qm, dev, batch=1), False),
+            ("cfg4b_causal_prefill_one_prompt_1024_key_split", lambda: Prefill(qm, dev, batch=1, split=True), False),
             # a prompt continued in chunks: 256 rows at position 2048 (matrix cores; and row by row through the decode kernels,
-            # which also serves sliding windows, other GQA groups and paged caches)
-            ("cfg4c_prefill_chunk_256_rows_at_2048", lambda: PrefillChunk(qm, dev)),
-            ("cfg4c_prefill_chunk_256_rows_at_2048_one_block_per_query_tile", lambda: PrefillChunk(qm, dev, split=False)),
-            ("cfg4c_prefill_chunk_256_rows_at_2048_row_by_row", lambda: PrefillChunk(qm, dev, by_rows=True)),
-            ("cfg5_predictor_loop", lambda: PredictorLoop(qm, dev)),
-            ("cfg5_predictor_loop_exact_chain", lambda: PredictorLoop(qm, dev, kernel=1)),
-            ("cfg5_predictor_loop_cache_writeback", lambda: PredictorLoop(qm, dev, write_cache=True)),
+            # which also serves sliding windows)
+            ("cfg4c_prefill_chunk_256_rows_at_2048", lambda: PrefillChunk(qm, dev), False),
+            ("cfg4c_prefill_chunk_256_rows_at_2048_one_block_per_query_tile", lambda: PrefillChunk(qm, dev, split=False), False),
+            ("cfg4c_prefill_chunk_256_rows_at_2048_row_by_row", lambda: PrefillChunk(qm, dev, by_rows=True), False),
+            ("cfg5_predictor_loop", lambda: PredictorLoop(qm, dev), True),
+            ("cfg5_predictor_loop_exact_chain", lambda: PredictorLoop(qm, dev, kernel=1), False),
+            ("cfg5_predictor_loop_cache_writeback", lambda: PredictorLoop(qm, dev, write_cache=True), True),
             # beyond the five configurations: the M = 1 projection in front of configuration 2
-            ("next_qkv_gemv_m1", lambda: QkvGemv(qm, dev)),
-            ("next_qkv_gemv_m1_rotating64", lambda: QkvGemv(qm, dev, copies=64)),
+            ("next_qkv_gemv_m1", lambda: QkvGemv(qm, dev), False),
+            ("next_qkv_gemv_m1_rotating64", lambda: QkvGemv(qm, dev, copies=64), False),
             # the whole decode step of one talker layer, 28 layers' weights and caches in rotation (2.8 GB)
-            ("next_talker_layer_decode_step", lambda: TalkerLayerStep(qm, dev)),
-            ("next_talker_layer_decode_step_unfused", lambda: TalkerLayerStep(qm, dev, fused=False)),
-            ("next_talker_layer_decode_step_one_launch", lambda: TalkerLayerStep(qm, dev, chained=True)),
+            ("next_talker_layer_decode_step", lambda: TalkerLayerStep(qm, dev), False),
+            ("next_talker_layer_decode_step_unfused", lambda: TalkerLayerStep(qm, dev, fused=False), False),
+            ("next_talker_layer_decode_step_one_launch", lambda: TalkerLayerStep(qm, dev, chained=True), False),
             # the attention's merge launch folded into that launch: two launches per layer
-            ("next_talker_layer_decode_step_two_launches", lambda: TalkerLayerStep(qm, dev, two_launches=True)),
+            ("next_talker_layer_decode_step_two_launches", lambda: TalkerLayerStep(qm, dev, two_launches=True), True),
             # the seven linears of a talker layer over a 1024-token prompt: matrix cores, and the exact chain
-            ("next_prompt_linears_1024_tokens", lambda: PromptLinears(qm, dev)),
-            ("next_prompt_linears_1024_tokens_exact_chain", lambda: PromptLinears(qm, dev, kernel=1)),
+            ("next_prompt_linears_1024_tokens", lambda: PromptLinears(qm, dev), True),
+            ("next_prompt_linears_1024_tokens_exact_chain", lambda: PromptLinears(qm, dev, kernel=1), False),
             # a short prompt (what a sentence of text is): 32 to 96 blocks per linear; with a workspace the reductions are cut
-            ("next_prompt_linears_128_tokens", lambda: PromptLinears(qm, dev, rows=128)),
-            ("next_prompt_linears_128_tokens_reductions_shared", lambda: PromptLinears(qm, dev, rows=128, split=True)),
+            ("next_prompt_linears_128_tokens", lambda: PromptLinears(qm, dev, rows=128), False),
+            ("next_prompt_linears_128_tokens_reductions_shared", lambda: PromptLinears(qm, dev, rows=128, split=True), False),
             # the fourteen M = 1 steps of one code-predictor frame, operator by operator (406 launches)
-            ("next_predictor_frame_m1_steps", lambda: PredictorFrameSteps(qm, dev)),
+            ("next_predictor_frame_m1_steps", lambda: PredictorFrameSteps(qm, dev), False),
             # the same fourteen steps as ONE launch of 256 resident blocks (same codes bit for bit)
-            ("next_predictor_frame_m1_steps_one_launch", lambda: PredictorFrameSteps(qm, dev, one_launch=True)),
+            ("next_predictor_frame_m1_steps_one_launch", lambda: PredictorFrameSteps(qm, dev, one_launch=True), True),
         ]
+        extra = [(key, make) for key, make, default in rows if default or args.all]
         for key, make in extra:
             w = make()
             r = _report(w, _time_steps(w.step, max(args.steps, 100), max(args.warmup, 10)))
@@ -1221,9 +1261,19 @@ def main():
                      "kernel": "decode_split_kernel<2, false, true, false> (+ decode_merge_kernel<2, false>, both inside the timed step)",
                      "algorithmic_bytes_per_launch": head.bytes, "avg_launch_us": ms * 1e3},
         "cpu_baseline": cpu,
-        "per_config": per_config,
+        "summary": _summary(per_config),
     }
-    print(json.dumps(line))
+    if per_config:
+        full = json.dumps(per_config)
+        print("per_config " + full, flush=True)
+        try:
+            os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+            with open(os.path.join(ROOT, "gpurun_out", "bench_per_config.json"), "w") as f:
+                f.write(full + "\n")
+            line["per_config_file"] = "gpurun_out/bench_per_config.json"
+        except OSError:
+            pass
+    print(compact_line(line), flush=True)
 
 
 if __name__ == "__main__":
