@@ -87,6 +87,7 @@ struct PrefillParams {
     int kv_heads;
     int n_qtiles;
     int heavy_groups;            // (interleaved kernel) leading groups of blocks, heaviest query tile first; the rest ascend
+    int dealt_pages;             // (interleaved kernel) the whole grid is resident at once: the light blocks write the heavy blocks' pages
     // (interleaved kernel, key split) a query tile of n key tiles is shared by min(ceil(n / split_chunk), 3) blocks
     int split_chunk;             // 0: no query tile is split
     int split_slots;             // query tiles per pair that are split (the last ones)
@@ -717,6 +718,57 @@ __host__ __device__ inline int split_first_tile(int tiles, int parts, int part) 
     return even_share < latest ? even_share : latest;
 }
 
+// Copies the K and V rows of key tile `tile` of (batch b, kv head kvh) to their pages: 256 threads, a thread four
+// rows' 16-byte pieces of either tensor.  The interleaved kernel's blocks of the lighter half of the query tiles copy
+// the heavier half's key tiles with it, kHeavyTilesPerBlock each, the lightest block the last tiles.
+constexpr int kHeavyTilesPerBlock = 3;
+__device__ __forceinline__ void copy_tile_to_pages(const PrefillParams& prm, const qm_kv_cache& cache, int b, int kvh, int tile) {
+    const int tid = threadIdx.x;
+    const int32_t* table = prm.page_table ? prm.page_table + static_cast<int64_t>(b) * prm.pages.max_pages : nullptr;
+    const int64_t kv_base = static_cast<int64_t>(b) * prm.kv_stride_batch + static_cast<int64_t>(kvh) * prm.kv_stride_head;
+    uint32_t page_err = 0;
+    // every load below is unconditional (indices clamped into range), so that all twelve are in flight at once
+    int page[4], phys[4];
+    bool live[4];
+    uint4 kx[4], vx[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int key = tile * kBM + (tid >> 4) + 16 * i;
+        live[i] = key < prm.seq;
+        page[i] = page_of(prm.pages, live[i] ? key : 0);
+        if (live[i] && page[i] >= prm.pages.max_pages) {
+            page_err |= QM_STATUS_BAD_POSITION;
+            live[i] = false;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int entry = live[i] ? page[i] : 0;
+        phys[i] = table ? table[entry] : entry;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int key = min(tile * kBM + (tid >> 4) + 16 * i, prm.seq - 1);
+        const int64_t off = kv_base + static_cast<int64_t>(key) * prm.kv_stride_token + 8 * (tid & 15);
+        kx[i] = *reinterpret_cast<const uint4*>(prm.k + off);
+        vx[i] = *reinterpret_cast<const uint4*>(prm.v + off);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (!live[i]) continue;
+        if (phys[i] < 0 || phys[i] >= cache.n_pages) {
+            page_err |= QM_STATUS_BAD_PAGE;
+            continue;
+        }
+        const int key = tile * kBM + (tid >> 4) + 16 * i;
+        const int64_t off = static_cast<int64_t>(phys[i]) * cache.stride_page + static_cast<int64_t>(kvh) * cache.stride_head
+                          + static_cast<int64_t>(key - page[i] * prm.pages.page_size) * kDim + 8 * (tid & 15);
+        *reinterpret_cast<uint4*>(cache.k_pool + off) = kx[i];
+        *reinterpret_cast<uint4*>(cache.v_pool + off) = vx[i];
+    }
+    if (page_err && prm.status) atomicOr(prm.status, page_err);
+}
+
 template <bool ROUND, int NC>
 __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const qm_kv_cache& cache,
                                                 unsigned char* il_smem, int qt, int bh,
@@ -749,15 +801,33 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
     const int64_t kv_base = static_cast<int64_t>(b) * prm.kv_stride_batch + static_cast<int64_t>(kvh) * prm.kv_stride_head;
     const int kv_row32 = static_cast<int>(prm.kv_stride_token);
 
-    // ---- K/V rows of the block's own tiles for the pages: requested first, written after the first wait ----
-    const bool to_pages = prm.has_cache != 0 && last_part;
-    int phys[4 * NC];
-    uint4 kx[4 * NC], vx[4 * NC];
+    // ---- K/V rows for the pages.  Writing key tile t to the pages is exact and independent of everything else, so
+    // it need not be done by the block of query tile t.
+    // When the whole grid is resident at once (dealt_pages) the kernel lasts as long as the blocks of the heaviest
+    // query tiles, and those write none: every block of the lighter half writes its own tile, and the heavy tiles
+    // are dealt three at a time to the lightest blocks (which have the most time to spare), before anything else
+    // of theirs: their requests join the burst of first requests of the whole grid, and they wait for them while
+    // the heavy blocks already run.
+    // Otherwise blocks queue for the CUs, a block that waits is a CU slot that idles, and every block writes its
+    // own tile: rows requested behind its first tiles, written after its first wait. ----
+    static_assert(NC == 1, "the page write takes key tiles of 64 rows");
+    const int light_tiles = prm.n_qtiles - prm.n_qtiles / 2;
+    if (prm.has_cache != 0 && prm.dealt_pages != 0 && last_part && qt < light_tiles) {
+        copy_tile_to_pages(prm, cache, b, kvh, qt);
+#pragma unroll 1
+        for (int j = 0; j < kHeavyTilesPerBlock; ++j) {
+            const int heavy = prm.n_qtiles - 1 - (kHeavyTilesPerBlock * qt + j);
+            if (heavy >= light_tiles) copy_tile_to_pages(prm, cache, b, kvh, heavy);
+        }
+    }
+    const bool own_pages = prm.has_cache != 0 && prm.dealt_pages == 0 && last_part;
+    int phys[4];
+    uint4 kx[4], vx[4];
     uint32_t page_err = 0;
-    if (to_pages) {
+    auto request_page_rows = [&]() {
         const int32_t* table = prm.page_table ? prm.page_table + static_cast<int64_t>(b) * prm.pages.max_pages : nullptr;
 #pragma unroll
-        for (int i = 0; i < 4 * NC; ++i) {
+        for (int i = 0; i < 4; ++i) {
             const int key = q0 + (tid >> 4) + 16 * i;
             phys[i] = -1;
             kx[i] = vx[i] = make_uint4(0, 0, 0, 0);
@@ -770,62 +840,10 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
                 vx[i] = *reinterpret_cast<const uint4*>(prm.v + off);
             }
         }
-    }
-
-    // ---- staging: one global_load_lds of a wave (16 bytes per lane) fills four consecutive 256-byte rows of a
-    // tile, lane l row l / 16, slot l % 16; which 16-byte piece of the key the lane fetches into that slot is
-    // the swizzle.  Slot p of K row r holds piece p ^ (r % 16), so that the fragment reads of 16 consecutive
-    // rows fall on 16 different slots; V stays row-major too (slot p of row r holds piece p ^ 4 (r % 4)) and is
-    // transposed by the LDS read.  A key at or beyond S is redirected to the last key; such keys only occur
-    // masked.  Wave w fills rows 4 w + l / 16 + 16 j of a tile ----
-    const int k_row = 4 * wave + (lane >> 4);
-    const uint16_t* k_src = prm.k + kv_base + 8 * ((lane & 15) ^ (k_row & 15));
-    const uint16_t* v_src = prm.v + kv_base + 8 * ((lane & 15) ^ (4 * (k_row & 3)));
-    const uint32_t row_bytes = static_cast<uint32_t>(kv_row32) * 2u;
-    // piece j of a tile: one global_load_lds (16 bytes per lane, no registers) fills rows 4 w + 16 j .. + 3; a key
-    // at or beyond S is redirected to the last key (such keys only occur masked)
-    auto load_piece = [&](const uint16_t* src, unsigned char* ring, int tile, int slot, int j) {
-        unsigned char* dst = ring + slot * kSpKTile + (4 * wave + 16 * j) * kKR;
-        const int key = min(tile * kBN + k_row + 16 * j, S - 1);
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned char*>(src)
-                                             + static_cast<uint64_t>(static_cast<uint32_t>(key) * row_bytes),
-                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
     };
-    auto load_k = [&](int tile, int slot) {
+    auto write_page_rows = [&]() {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) load_piece(k_src, lds_k, tile, slot, j);
-    };
-    auto load_v = [&](int tile, int slot) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) load_piece(v_src, lds_v, tile, slot, j);
-    };
-
-    load_k(t_first, 0);                              // t_first is even: tile t lives in buffer t % 2
-    load_v(t_first, 0);
-    load_k(t_first + 1, 1);                          // qt >= 1, and every part holds two tiles at least: it exists
-    bf16x8_t qf[NC][8];
-#pragma unroll
-    for (int c = 0; c < NC; ++c) {
-        const int row = group_row0(c) + (col & 15);
-        const uint16_t* qp = prm.q + ((static_cast<int64_t>(b) * S + row) * q_heads + my_head) * kDim + 8 * grp;
-#pragma unroll
-        for (int kb = 0; kb < 8; ++kb) {
-            uint4 raw = make_uint4(0, 0, 0, 0);
-            if (row < S) raw = *reinterpret_cast<const uint4*>(qp + 16 * kb);
-            qf[c][kb] = __builtin_bit_cast(bf16x8_t, raw);
-        }
-    }
-    f32x16_t o[NC][4];
-#pragma unroll
-    for (int c = 0; c < NC; ++c)
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o[c][dt][r] = 0.0f;
-    wait_vm<0>();
-    if (to_pages) {
-#pragma unroll
-        for (int i = 0; i < 4 * NC; ++i) {
+        for (int i = 0; i < 4; ++i) {
             const int key = q0 + (tid >> 4) + 16 * i;
             if (key >= S || phys[i] == -1) continue;
             if (phys[i] < 0 || phys[i] >= cache.n_pages) {
@@ -839,6 +857,79 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
             *reinterpret_cast<uint4*>(cache.v_pool + off) = vx[i];
         }
         if (page_err && prm.status) atomicOr(prm.status, page_err);
+    };
+
+    // ---- staging: one global_load_lds of a wave (16 bytes per lane) fills four consecutive 256-byte rows of a
+    // tile, lane l row l / 16, slot l % 16; which 16-byte piece of the key the lane fetches into that slot is
+    // the swizzle.  Slot p of K row r holds piece p ^ (r % 16), so that the fragment reads of 16 consecutive
+    // rows fall on 16 different slots; V stays row-major too (slot p of row r holds piece p ^ 4 (r % 4)) and is
+    // transposed by the LDS read.  A key at or beyond S is redirected to the last key; such keys only occur
+    // masked.  Wave w fills rows 4 w + l / 16 + 16 j of a tile ----
+    const int k_row = 4 * wave + (lane >> 4);
+    const uint32_t row_bytes = static_cast<uint32_t>(kv_row32) * 2u;
+    // Requests go through buffer descriptors that cover exactly the S keys of this (batch, kv head): a lane's offset
+    // is the piece's first key (scalar arithmetic) plus a 32-bit value that never changes (its row inside the piece
+    // and the 16-byte piece of the key it fetches), one vector addition per request, and a key at or beyond S is out
+    // of the descriptor's range: it reads as zero and touches no memory (such keys only occur masked).
+    const uint32_t kv_bytes = static_cast<uint32_t>(S - 1) * row_bytes + static_cast<uint32_t>(kKR);
+    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(prm.k + kv_base), 0, static_cast<int>(kv_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(prm.v + kv_base), 0, static_cast<int>(kv_bytes), 0x00020000);
+    const uint32_t k_lane = static_cast<uint32_t>(k_row) * row_bytes + 16u * ((lane & 15) ^ (k_row & 15));
+    const uint32_t v_lane = static_cast<uint32_t>(k_row) * row_bytes + 16u * ((lane & 15) ^ (4 * (k_row & 3)));
+    // piece j of a tile: one request of a wave (16 bytes per lane, no registers) fills rows 4 w + 16 j .. + 3
+    auto load_piece = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lane_off, unsigned char* ring, int tile, int slot, int j) {
+        unsigned char* dst = ring + slot * kSpKTile + (4 * wave + 16 * j) * kKR;
+        const uint32_t piece = static_cast<uint32_t>(tile * kBN + 16 * j) * row_bytes;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16,
+                                                 static_cast<int>(lane_off + piece), 0, 0, 0);
+    };
+    auto load_k_piece = [&](int tile, int slot, int j) { load_piece(k_rsrc, k_lane, lds_k, tile, slot, j); };
+    auto load_v_piece = [&](int tile, int slot, int j) { load_piece(v_rsrc, v_lane, lds_v, tile, slot, j); };
+    auto load_k = [&](int tile, int slot) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) load_k_piece(tile, slot, j);
+    };
+    auto load_v = [&](int tile, int slot) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) load_v_piece(tile, slot, j);
+    };
+
+    // What the first product needs is requested first: K of the first tile and the wave's own Q fragments.  A block
+    // that has no page rows to wait for waits for those alone (loads come back in the order of their requests) and
+    // leaves V of the first tile and K of the second in flight: the first tile's barrier inside the pipeline waits
+    // for them.
+    load_k(t_first, 0);                              // t_first is even: tile t lives in buffer t % 2
+    bf16x8_t qf[NC][8];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int row = group_row0(c) + (col & 15);
+        const uint16_t* qp = prm.q + ((static_cast<int64_t>(b) * S + row) * q_heads + my_head) * kDim + 8 * grp;
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb) {
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (row < S) raw = *reinterpret_cast<const uint4*>(qp + 16 * kb);
+            qf[c][kb] = __builtin_bit_cast(bf16x8_t, raw);
+        }
+    }
+    load_v(t_first, 0);
+    load_k(t_first + 1, 1);                          // qt >= 1, and every part holds two tiles at least: it exists
+    f32x16_t o[NC][4];
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[c][dt][r] = 0.0f;
+    if (own_pages) {
+        request_page_rows();
+        wait_vm<0>();
+        write_page_rows();
+    } else {
+        // (a row at or beyond S requests no Q: then fewer loads are outstanding than the count assumes and the
+        // wait is merely longer)
+        wait_vm<8>();
     }
     lds_barrier();
 
@@ -1021,11 +1112,14 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         // negative scale elsewhere) and the exchange between the two halves of the wave, so that the branch
         // on them after the last group waits for nothing
         float mx_a[NC], mx_b[NC], mx_step[NC], mx_limit[NC];
+        uint32_t hi[NC][8];
+        float psum[NC];
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             mx_a[c] = mx_b[c] = -INFINITY;
             mx_step[c] = 0.0f;
             mx_limit[c] = m_run[c] + slack;
+            psum[c] = 0.0f;
         }
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
@@ -1085,11 +1179,18 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
                     }
                     s_cur[c][ra] = za0; s_cur[c][ra + 1] = za1; s_cur[c][rb] = zb0; s_cur[c][rb + 1] = zb1;
                 } else {
-                    mx_a[c] = __builtin_fmaxf(mx_a[c], __builtin_fmaxf(s_cur[c][ra], s_cur[c][ra + 1]));
+                    // (assembly for the same reason as above.  The first maximum starts from a score through a
+                    // statement the compiler sees, so that it guards the read of the MFMA's results.)
+                    if (g == 0) {
+                        mx_a[c] = s_cur[c][0];
+                        asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(mx_a[c]) : "v"(s_cur[c][1]), "v"(s_cur[c][1]));
+                    } else {
+                        asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(mx_a[c]) : "v"(s_cur[c][ra]), "v"(s_cur[c][ra + 1]));
+                    }
                     fence();
                     qk_mfma(g, c);
                     fence();
-                    mx_b[c] = __builtin_fmaxf(mx_b[c], __builtin_fmaxf(s_cur[c][rb], s_cur[c][rb + 1]));
+                    asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(mx_b[c]) : "v"(s_cur[c][rb]), "v"(s_cur[c][rb + 1]));
                 }
                 fence();
             }
@@ -1111,7 +1212,12 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         float alpha[NC];
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
-            const float mx = ROUND ? mx_step[c] : halves_max(__builtin_fmaxf(mx_a[c], mx_b[c]));
+            float mx = mx_step[c];
+            if (!ROUND) {
+                asm volatile("v_max_f32 %0, %1, %2" : "=v"(mx) : "v"(mx_a[c]), "v"(mx_b[c]));
+                const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+                asm volatile("v_max_f32 %0, %1, %2" : "=v"(mx) : "v"(__uint_as_float(sw[0])), "v"(__uint_as_float(sw[1])));
+            }
             need[c] = __builtin_amdgcn_ballot_w64(mx > mx_limit[c]) != 0;
             alpha[c] = 1.0f;
             if (need[c]) {
@@ -1123,10 +1229,6 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
                 l_run[c] *= alpha[c];
             }
         }
-        uint32_t hi[NC][8];
-        float psum[NC];
-#pragma unroll
-        for (int c = 0; c < NC; ++c) psum[c] = 0.0f;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const int ra = 4 * g, rb = 4 * g + 2;
@@ -1215,9 +1317,9 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
               },
               [&](int i) {
                   if (i < 4) {
-                      if (more_k) load_piece(k_src, lds_k, t + 2, cur, i);
+                      if (more_k) load_k_piece(t + 2, cur, i);
                   } else {
-                      load_piece(v_src, lds_v, t + 1, nxt, i - 4);
+                      load_v_piece(t + 1, nxt, i - 4);
                   }
               });
         // stage (t, 1): P.V of chunk (t, 0), softmax of (t, 1), S^T of (t + 1, 0); requests V(t, 1) and K(t + 1, 1)
@@ -1311,10 +1413,9 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
             diag_group(c, s_a[c], vf, key_base);
         }
     }
-    lds_barrier();   // every wave is done with the rings: they become the output staging area
-
     // ---- a split query tile: all blocks but the last to arrive publish, the last combines ----
     if (NC == 1 && parts > 1) {
+        lds_barrier();   // every wave is done with the rings: their first words carry the notes below
         const int64_t slot = static_cast<int64_t>(bh) * prm.split_slots + split_slot;
         float* records = prm.split_partials + slot * kSplitMaxParts * kSplitRecordFloats + tid;
         int* tickets = prm.split_tickets + slot * kSplitTicketInts;
@@ -1430,35 +1531,31 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         __syncthreads();                             // the notes have been read: the area is the staging area again
     }
 
-    // ---- normalise, stage through LDS, write 16 bytes per lane ----
-    uint16_t* stage_out = reinterpret_cast<uint16_t*>(il_smem) + wave * NC * 32 * kOS;
+    // ---- normalise and write, straight from the registers: no staging area, so a wave that is done does not wait
+    // for the others.  A lane holds dims 32 dt + 8 rq + 4 grp .. + 3 of its column; the two halves of the wave
+    // exchange (v_permlane32_swap) so that the lower half owns the eight dims of even rq and the upper half those of
+    // odd rq: 16 bytes per lane, 32 contiguous bytes per row and request. ----
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
         const float l_tot = halves_sum(l_run[c]);
         const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+        const int row = group_row0(c) + (col & 15);
+        uint16_t* dst = prm.out + ((static_cast<int64_t>(b) * S + row) * q_heads + my_head) * kDim + 8 * grp;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) {
 #pragma unroll
-            for (int rq = 0; rq < 4; ++rq) {
-                const int d0 = 32 * dt + 8 * rq + 4 * grp;
-                uint2 packed;
-                packed.x = pack_bf16_pair(o[c][dt][4 * rq + 0] * inv, o[c][dt][4 * rq + 1] * inv);
-                packed.y = pack_bf16_pair(o[c][dt][4 * rq + 2] * inv, o[c][dt][4 * rq + 3] * inv);
-                *reinterpret_cast<uint2*>(&stage_out[(32 * c + col) * kOS + d0]) = packed;
+            for (int rp = 0; rp < 2; ++rp) {
+                const int re = 8 * rp;               // registers of rq = 2 rp (even) and + 4 (odd)
+                const uint32_t e0 = pack_bf16_pair(o[c][dt][re + 0] * inv, o[c][dt][re + 1] * inv);
+                const uint32_t e1 = pack_bf16_pair(o[c][dt][re + 2] * inv, o[c][dt][re + 3] * inv);
+                const uint32_t o0 = pack_bf16_pair(o[c][dt][re + 4] * inv, o[c][dt][re + 5] * inv);
+                const uint32_t o1 = pack_bf16_pair(o[c][dt][re + 6] * inv, o[c][dt][re + 7] * inv);
+                // lower half: (e, e of the partner); upper half: (o of the partner, o)
+                const auto x = __builtin_amdgcn_permlane32_swap(e0, o0, false, false);
+                const auto y = __builtin_amdgcn_permlane32_swap(e1, o1, false, false);
+                const uint4 val = make_uint4(x[0], y[0], x[1], y[1]);
+                if (row < S) *reinterpret_cast<uint4*>(dst + 32 * dt + 16 * rp) = val;
             }
-        }
-    }
-    __builtin_amdgcn_s_waitcnt(0);   // the wave reads back only what it wrote itself
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int it = 0; it < 8 * NC; ++it) {
-        const int cc = 4 * it + (lane >> 4);         // staged column: group cc / 32, head (cc % 32) / 16, row cc % 16
-        const int piece = lane & 15;
-        const int row = group_row0(cc >> 5) + (cc & 15);
-        const int head = 2 * kvh + ((cc & 31) >> 4);
-        if (row < S) {
-            const uint4 val = *reinterpret_cast<const uint4*>(&stage_out[cc * kOS + 8 * piece]);
-            *reinterpret_cast<uint4*>(prm.out + ((static_cast<int64_t>(b) * S + row) * q_heads + head) * kDim + 8 * piece) = val;
         }
     }
 }
@@ -1489,11 +1586,17 @@ __global__ __launch_bounds__(kPfThreads, (NC == 1 ? 2 : 1)) void prefill_il_kern
         qt = group < prm.heavy_groups ? prm.n_qtiles - 1 - group : group - prm.heavy_groups;
     }
     if (qt == 0) {
-        prefill_body<true, ROUND>(prm, cache, il_smem, 0, bid % pairs);
-        if (NC == 2 && prm.seq > kBM) {
-            __syncthreads();
-            prefill_body<false, ROUND>(prm, cache, il_smem, 1, bid % pairs);
+        const int pair = bid % pairs;
+        // (with the whole grid resident the lightest block also writes the pages of the last key tiles: the blocks
+        // of the heavier half write none)
+        if (prm.has_cache != 0 && prm.dealt_pages != 0) {
+#pragma unroll 1
+            for (int j = 0; j < kHeavyTilesPerBlock; ++j) {
+                const int heavy = prm.n_qtiles - 1 - j;
+                if (heavy >= prm.n_qtiles - prm.n_qtiles / 2) copy_tile_to_pages(prm, cache, pair / prm.kv_heads, pair % prm.kv_heads, heavy);
+            }
         }
+        prefill_body<true, ROUND>(prm, cache, il_smem, 0, pair);
     } else {
         prefill_il_body<ROUND, NC>(prm, cache, il_smem, qt, bid % pairs, part, parts, prm.n_qtiles - 1 - qt);
     }
@@ -1627,6 +1730,7 @@ static int32_t prefill_attention_entry(
     prm.kv_stride_token = kv_stride_token; prm.kv_stride_head = kv_stride_head; prm.kv_stride_batch = kv_stride_batch;
     prm.batch = batch; prm.seq = seq; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
     prm.heavy_groups = n_qtiles;
+    prm.dealt_pages = 0;
     prm.split_chunk = 0; prm.split_slots = 0; prm.split_partials = nullptr; prm.split_tickets = nullptr; prm.split_epoch = 0;
     prm.cache_before = 0; prm.key_count = seq;
 
@@ -1655,6 +1759,7 @@ static int32_t prefill_attention_entry(
         } else if (compute_units % pairs == 0 && blocks > compute_units && blocks <= 2 * static_cast<int64_t>(compute_units)) {
             prm.heavy_groups = static_cast<int>(compute_units / pairs);
         }
+        prm.dealt_pages = blocks <= 2 * static_cast<int64_t>(compute_units) ? 1 : 0;   // two blocks fit a CU
         static std::atomic<bool> lds_raised[2][kMaxDevices];
         const void* kernel = round_scores ? reinterpret_cast<const void*>(prefill_il_kernel<true, 1>)
                                           : reinterpret_cast<const void*>(prefill_il_kernel<false, 1>);
@@ -1775,6 +1880,7 @@ extern "C" int32_t qm_prefill_attention_chunk(
     prm.kv_stride_token = kv_stride_token; prm.kv_stride_head = kv_stride_head; prm.kv_stride_batch = kv_stride_batch;
     prm.batch = batch; prm.seq = rows; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
     prm.heavy_groups = n_qtiles;
+    prm.dealt_pages = 0;
     prm.cache_before = cache_before; prm.key_count = static_cast<int>(key_count);
     prm.chunk_parts = 1;
     if (workspace) {
