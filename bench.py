@@ -992,7 +992,6 @@ class PredictorLoop:
         self.kernel = kernel      # 0: products on the matrix cores; 1: every fp32 sum in the reference's order
         # bf16 outputs of magnitude >= 2 are 0.0156 apart: a sum taken in another order can land one
         # output spacing away, which is what the gate below allows the matrix-core kernel
-        self.tolerance = 1e-2 if kernel else 2e-2
         syn = Synthetic(dev, seed)
 
         rnd = syn.normal
@@ -1035,9 +1034,21 @@ class PredictorLoop:
                                              out, None, None, n, self.layers, self.rows, 1, 1e-6, threads)
         dt = time.perf_counter() - t0
         assert rc == 0
-        err = float(np.max(np.abs(oracle.bf16_to_f32(out).astype(np.float64)
-                                  - oracle.bf16_to_f32(_bits(self.out[:n])).astype(np.float64))))
-        return {"all": dt * self.units / n}, err, "first %d of %d units, time scaled" % (n, self.units)
+        # (the matrix-core kernel's other order of summation moves a bf16-rounded score across a rounding boundary about
+        # once in 10^6 outputs: the same allowance as tests/test_gpu_predictor.py, none for the exact chain)
+        err, outside = _within_rule(oracle, _bits(self.out[:n]), out)
+        ok = outside == 0 if self.kernel else (outside <= 4 and err <= 2e-2)
+        return {"all": dt * self.units / n}, err, "first %d of %d units, time scaled" % (n, self.units), ok
+
+
+def _within_rule(oracle, got_bits, want_bits, tol=1e-2):
+    """The tolerance rule of the parity tests, per element: |got - want| <= max(tol, one bf16 ulp of the oracle's
+    value) (beyond |x| = 2 one bf16 step is 1.56e-2, more than tol).  Returns (max abs error, elements outside the
+    rule)."""
+    want = oracle.bf16_to_f32(want_bits).astype(np.float64)
+    err = np.abs(oracle.bf16_to_f32(got_bits).astype(np.float64) - want)
+    one_ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 2.0 ** -20))) - 7)
+    return float(err.max()) if err.size else 0.0, int(np.count_nonzero(err > np.maximum(one_ulp, tol)))
 
 
 def _report(w, ms):
@@ -1220,8 +1231,8 @@ def main():
                 r["launches_per_predictor_step"] = w.launches_per_step
             if oracle is not None and not (isinstance(w, PredictorLoop) and w.kc is not None) \
                     and (copies == 1 or isinstance(w, (TalkerLayerStep, PredictorFrameSteps))):
-                res, err, sample = w.cpu_baseline(oracle, threads)
-                if err > getattr(w, "tolerance", 1e-2):
+                res, err, sample, *rule = w.cpu_baseline(oracle, threads)
+                if not (rule[0] if rule else err <= getattr(w, "tolerance", 1e-2)):
                     raise RuntimeError(f"{key}: GPU result differs from the oracle: max abs err {err}")
                 r["cpu_oracle"] = {"seconds": res["all"], "cores": threads, "sample": sample,
                                    "gpu_vs_oracle_max_abs_err": err,

@@ -494,9 +494,14 @@ int32_t qm_predictor_step_attention_m1(
  * The launch is 256 blocks that stay resident and hand each operator's output to one another through
  * `workspace` (qm_predictor_frame_workspace_bytes() bytes, 256-byte aligned, set up once by
  * qm_predictor_frame_workspace_init and then carried from call to call: it numbers the operator instances so
- * that a captured launch can be replayed).  It needs a device with 256 compute units all of which can hold one
- * of its blocks (QM_ERR_NO_DEVICE otherwise), and two such launches must not overlap in time on one device: each
- * would wait for blocks of its own that the other keeps out.  Every wait is bounded: if an input never comes the
+ * that a captured launch can be replayed).  It needs the WHOLE CHIP for its duration: 256 compute units all of
+ * which can hold one of its blocks, on a stream that may use them all.  The call returns QM_ERR_NO_DEVICE, before
+ * anything is launched, if the device is smaller or if `hip_stream` was created with a CU mask of fewer compute
+ * units (hipExtStreamCreateWithCUMask, as the reference's generation stream is, R17:7733-7792):
+ * qm_predictor_frame_fits(stream, &fits) asks the same question without launching, and a caller on such a stream
+ * takes the operators one by one (same bits).  What the call cannot see are kernels of OTHER streams that occupy
+ * compute units while it runs, and another launch of this kind: each would keep out blocks the other waits for,
+ * so nothing else may run on the device at the same time.  Every wait is bounded: if an input never comes the
  * blocks OR QM_STATUS_FRAME_TIMEOUT into status_dev (optional) and return; the outputs are then not to be used
  * and the workspace must be initialised again before the next call.
  */
@@ -539,6 +544,9 @@ typedef struct qm_predictor_frame {
 
 int64_t qm_predictor_frame_workspace_bytes(void);
 int32_t qm_predictor_frame_workspace_init(void* workspace, int64_t workspace_bytes, void* hip_stream);
+/* *fits = 1 if qm_predictor_frame_steps can run on `hip_stream` (device and stream CU mask hold 256 blocks), else 0.
+ * No counterpart in the reference, which has no kernel of this kind. */
+int32_t qm_predictor_frame_fits(void* hip_stream, int32_t* fits);
 int32_t qm_predictor_frame_steps(
     const qm_predictor_frame* frame, int32_t first_step, int32_t last_step,
     int32_t top_k, float temperature,
@@ -556,7 +564,10 @@ int32_t qm_predictor_frame_steps(
  * weight matrices 16-byte aligned.  256 blocks stay resident and stream the weights through LDS while they hand the
  * activations to each other through `workspace` (qm_talker_post_attention_workspace_bytes bytes, 256-byte aligned,
  * set up once with qm_talker_post_attention_workspace_init; launches that share a workspace must not overlap).
- * QM_ERR_NO_DEVICE if the device cannot hold 256 blocks at once.  Waits are bounded
+ * Like qm_predictor_frame_steps it needs the whole chip for its duration: QM_ERR_NO_DEVICE, before anything is
+ * launched, if the device cannot hold 256 blocks at once or `hip_stream` is confined by a CU mask to fewer compute
+ * units (qm_talker_chain_fits asks without launching; such a caller takes the operators one by one, same bits), and
+ * no other stream's kernels may occupy compute units while it runs.  Waits are bounded
  * (QM_OPT_PREDICTOR_FRAME_SPIN_LIMIT applies here too): a launch that gives up ORs QM_STATUS_FRAME_TIMEOUT into
  * *status_dev, every block returns, outputs are undefined and the workspace must be initialised again.
  */
@@ -589,6 +600,9 @@ typedef struct qm_talker_post_attention {
 
 int64_t qm_talker_post_attention_workspace_bytes(void);
 int32_t qm_talker_post_attention_workspace_init(void* workspace, int64_t workspace_bytes, void* hip_stream);
+/* *fits = 1 if qm_talker_post_attention_m1 / qm_talker_layer_step_m1 can run on `hip_stream`, else 0.  No counterpart
+ * in the reference. */
+int32_t qm_talker_chain_fits(void* hip_stream, int32_t* fits);
 int32_t qm_talker_post_attention_m1(
     const qm_talker_post_attention* op,
     void* workspace, int64_t workspace_bytes, uint32_t* status_dev, void* hip_stream);

@@ -112,6 +112,9 @@ int32_t qm_talker_synchronize(qm_talker* engine);
 /* The engine's generation stream (hipStream_t as void*): the final head and the predictor of a generation
  * loop are created on it. */
 void* qm_talker_stream(qm_talker* engine);
+/* The device word the talker's kernels OR their QM_STATUS_* bits into (read and cleared by qm_talker_synchronize); the
+ * generation loop copies it back with every frame's codes, so that a flagged step ends the generation at once. */
+const uint32_t* qm_talker_status_device(qm_talker* engine);
 
 /* ---- final head (NativeFinalHead, R17:14145-14570) ----------------------------------------- */
 typedef struct qm_final_head qm_final_head;

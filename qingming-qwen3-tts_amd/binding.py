@@ -119,6 +119,8 @@ _SIGNATURES = {
     "qm_set_thread_option": (_I32, [_I32, _I32]),
     "qm_predictor_frame_workspace_bytes": (C.c_int64, []),
     "qm_predictor_frame_workspace_init": (_I32, [_PTR, C.c_int64, _PTR]),
+    "qm_predictor_frame_fits": (_I32, [_PTR, C.POINTER(C.c_int32)]),
+    "qm_talker_chain_fits": (_I32, [_PTR, C.POINTER(C.c_int32)]),
     "qm_predictor_frame_steps": (_I32, [C.POINTER(PredictorFrame), _I32, _I32, _I32, _F32, _PTR, C.c_int64, _PTR, _PTR]),
     "qm_talker_post_attention_workspace_bytes": (C.c_int64, []),
     "qm_talker_post_attention_workspace_init": (_I32, [_PTR, C.c_int64, _PTR]),
@@ -510,6 +512,20 @@ def predictor_frame_workspace_bytes():
 def predictor_frame_workspace_init(workspace, workspace_bytes, stream=0):
     _check(lib().qm_predictor_frame_workspace_init(_addr(workspace), workspace_bytes, stream),
            "qm_predictor_frame_workspace_init")
+
+
+def predictor_frame_fits(stream=0):
+    """Whether the one-launch predictor frame can run on `stream` (device and stream CU mask hold its 256 blocks)."""
+    fits = C.c_int32(0)
+    _check(lib().qm_predictor_frame_fits(stream, C.byref(fits)), "qm_predictor_frame_fits")
+    return bool(fits.value)
+
+
+def talker_chain_fits(stream=0):
+    """Whether the talker's one launch between two attentions can run on `stream`."""
+    fits = C.c_int32(0)
+    _check(lib().qm_talker_chain_fits(stream, C.byref(fits)), "qm_talker_chain_fits")
+    return bool(fits.value)
 
 
 def predictor_frame_steps(frame, first_step, last_step, top_k, temperature, workspace, workspace_bytes, status=None, stream=0):

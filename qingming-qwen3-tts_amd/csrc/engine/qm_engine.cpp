@@ -55,6 +55,10 @@ struct qm_talker {
     // hand-off words of qm_talker_post_attention_m1 (checkpoints of the geometry it serves)
     qm_engine::DeviceBuffer chain_workspace;
     bool chain_geometry = false;
+    // That launch needs every compute unit of the chip at once.  False where the engine's stream cannot give it that
+    // (a stream created with a CU mask), and from the first time a launch gave up waiting (something else held compute
+    // units): the layers then run operator by operator, which gives the same bits.
+    bool chain_usable = false;
 
     ~qm_talker() {
         if (own_stream && stream) (void)hipStreamDestroy(stream);
@@ -163,6 +167,9 @@ static std::unique_ptr<qm_talker> create_talker(const std::string& model_dir, in
     hip_check(hipMemsetAsync(engine->status.raw(), 0, engine->status.bytes(), engine->stream), "status word reset");
     engine->chain_geometry = engine->q_dim == 2048 && engine->kv_dim == 1024 && engine->intermediate == 6144 && kHidden == 2048;
     if (engine->chain_geometry) {
+        int32_t fits = 0;
+        op_check(qm_talker_chain_fits(engine->stream, &fits), "talker hand-off launch residency");
+        engine->chain_usable = fits != 0;
         engine->chain_workspace = DeviceBuffer(static_cast<size_t>(qm_talker_post_attention_workspace_bytes()));
         op_check(qm_talker_post_attention_workspace_init(engine->chain_workspace.raw(), static_cast<int64_t>(engine->chain_workspace.bytes()),
                                                          engine->stream), "talker hand-off workspace init");
@@ -218,13 +225,14 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
     // layer's RMSNorm + Q/K/V — is one launch where the checkpoint has the geometry that launch serves (same bits).
     int32_t by_operators = 0;
     op_check(qm_get_option(QM_OPT_TALKER_LAYER_OPERATORS, &by_operators), "talker layer option");
-    const bool chained = e.chain_geometry && by_operators != 1;
-    const bool merge_in_chain = chained && by_operators == 0;   // the attention's split records are combined by the launch that follows it
+    bool chained = e.chain_geometry && e.chain_usable && by_operators != 1;
+    bool merge_in_chain = chained && by_operators == 0;   // the attention's split records are combined by the launch that follows it
+    bool qkv_ready = false;                               // the layer's Q/K/V were left by the launch of the layer before
     for (size_t index = 0; index < e.layers.size(); ++index) {
         Layer& w = e.layers[index];
         qm_kv_cache cache = flat_cache_of(e, w);
         // launch_rmsnorm + launch_qkv_m1 (R17:17163-17176)
-        if (!chained || index == 0)
+        if (!qkv_ready)
             op_check(qm_rmsnorm_qkv_m1(current->u16(), w.input_norm.data(), kEpsilon, w.q_weight.data(), w.q_bias.data(),
                                        w.k_weight.data(), w.k_bias.data(), w.v_weight.data(), w.v_bias.data(), e.q.u16(),
                                        e.k.u16(), e.v.u16(), kHidden, e.q_dim, e.kv_dim, s),
@@ -252,6 +260,7 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
             }
             op.hidden_columns = kHidden; op.q_columns = e.q_dim; op.kv_columns = e.kv_dim; op.intermediate_columns = e.intermediate;
             op.epsilon = kEpsilon;
+            int32_t rc = QM_OK;
             if (merge_in_chain) {
                 qm_talker_layer_step step = {};
                 step.q = e.q.u16(); step.k = e.k.u16(); step.v = e.v.u16();
@@ -263,17 +272,31 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
                 step.q_heads = e.q_heads; step.position = position; step.sliding_window = -1;
                 step.scale = kScale; step.epsilon = kEpsilon;
                 step.post = op;
-                op_check(qm_talker_layer_step_m1(&step, e.chain_workspace.raw(), static_cast<int64_t>(e.chain_workspace.bytes()),
-                                                 static_cast<uint32_t*>(e.status.raw()), s),
-                         "talker norm/RoPE/append + attention ... next Q/K/V");
+                rc = qm_talker_layer_step_m1(&step, e.chain_workspace.raw(), static_cast<int64_t>(e.chain_workspace.bytes()),
+                                             static_cast<uint32_t*>(e.status.raw()), s);
             } else {
-                op_check(qm_talker_post_attention_m1(&op, e.chain_workspace.raw(), static_cast<int64_t>(e.chain_workspace.bytes()),
-                                                     static_cast<uint32_t*>(e.status.raw()), s),
-                         "talker o_proj ... next Q/K/V");
+                rc = qm_talker_post_attention_m1(&op, e.chain_workspace.raw(), static_cast<int64_t>(e.chain_workspace.bytes()),
+                                                 static_cast<uint32_t*>(e.status.raw()), s);
             }
-            std::swap(current, next);
-            continue;
+            if (rc != QM_ERR_NO_DEVICE) {
+                op_check(rc, "talker (norm/RoPE/append + attention) o_proj ... next Q/K/V");
+                qkv_ready = index + 1 < e.layers.size();
+                std::swap(current, next);
+                continue;
+            }
+            // The stream cannot hold that launch (nothing of it has been queued: the call checks before it launches):
+            // this layer and the ones after it run operator by operator, and so does every later step.
+            e.chain_usable = false;
+            chained = false;
+            if (merge_in_chain)
+                op_check(qm_decode_step_fused(e.q.u16(), e.k.u16(), e.v.u16(), w.q_norm.data(), w.k_norm.data(), cos_row,
+                                              sin_row, e.q_rotated.u16(), &cache, nullptr, 1, e.context.u16(), e.q_heads,
+                                              position, -1, kScale, kEpsilon, e.workspace.raw(), e.workspace.bytes(),
+                                              static_cast<uint32_t*>(e.status.raw()), s),
+                         "talker norm/RoPE/append + attention");
+            merge_in_chain = false;
         }
+        qkv_ready = false;
         // launch_linear_m1: o_proj (R17:17203-17210)
         op_check(qm_linear_m1(e.context.u16(), w.o_weight.data(), w.o_bias.data(), nullptr, e.attention.u16(), kHidden,
                               e.q_dim, s),
@@ -509,6 +532,10 @@ extern "C" int32_t qm_talker_prefill(qm_talker* engine, const uint16_t* input_de
 
 extern "C" void* qm_talker_stream(qm_talker* engine) { return engine ? engine->stream : nullptr; }
 
+extern "C" const uint32_t* qm_talker_status_device(qm_talker* engine) {
+    return engine ? static_cast<const uint32_t*>(engine->status.raw()) : nullptr;
+}
+
 extern "C" int32_t qm_talker_synchronize(qm_talker* engine) {
     if (!engine) return QM_ERR_NULL;
     return guarded([&] {
@@ -522,6 +549,7 @@ extern "C" int32_t qm_talker_synchronize(qm_talker* engine) {
             if ((bits & QM_STATUS_SPLIT_TIMEOUT) && engine->p_split.raw())
                 op_check(qm_prefill_split_workspace_init(engine->p_split.raw(), static_cast<int64_t>(engine->p_split.bytes()),
                                                          engine->stream), "prefill key-split workspace init");
+            if (bits & QM_STATUS_FRAME_TIMEOUT) engine->chain_usable = false;   // something else holds compute units: operators from now on
             if ((bits & QM_STATUS_FRAME_TIMEOUT) && engine->chain_workspace.raw())
                 op_check(qm_talker_post_attention_workspace_init(engine->chain_workspace.raw(),
                                                                  static_cast<int64_t>(engine->chain_workspace.bytes()), engine->stream),

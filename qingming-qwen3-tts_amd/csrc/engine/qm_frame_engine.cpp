@@ -254,7 +254,10 @@ static std::unique_ptr<qm_predictor> create_predictor(const std::string& model_d
         p->frame_workspace = DeviceBuffer(static_cast<size_t>(qm_predictor_frame_workspace_bytes()));
         op_check(qm_predictor_frame_workspace_init(p->frame_workspace.raw(), static_cast<int64_t>(p->frame_workspace.bytes()), stream),
                  "predictor frame workspace");
-        p->one_launch = true;
+        // (that launch needs every compute unit of the chip at once: not on a stream confined by a CU mask)
+        int32_t fits = 0;
+        op_check(qm_predictor_frame_fits(stream, &fits), "predictor frame launch residency");
+        p->one_launch = fits != 0;
     }
     return p;
 }
@@ -349,12 +352,14 @@ struct FrameResult {
     int32_t codes[kCodeGroups];
     int32_t code0;
     uint32_t status;
+    uint32_t talker_status;     // the talker's status word as of this frame (generation loop), else 0
 };
 
 // Queues a frame; `result` is filled when everything queued here has run (the caller waits for the stream, or — with
 // `result` in pinned memory — for an event it records right after this returns, and may queue more work meanwhile).
 static void predictor_frame_launch(qm_predictor& p, const uint16_t* talker_hidden_device, const int32_t* code0_device,
-                                   const uint16_t* context_host, bool sampling, FrameResult* result) {
+                                   const uint16_t* context_host, bool sampling, FrameResult* result,
+                                   const uint32_t* talker_status_device = nullptr) {
     if (!talker_hidden_device || !code0_device || !context_host || !result) throw ApiError(QM_ERR_NULL, "predictor frame input is null");
     hipStream_t s = p.stream;
     hip_check(hipMemsetAsync(p.frame_state.raw(), 0, p.frame_state.bytes(), s), "predictor caches, selected embeddings and codes reset");
@@ -365,13 +370,20 @@ static void predictor_frame_launch(qm_predictor& p, const uint16_t* talker_hidde
              "predictor group 0 input");
     int32_t by_operators = 0;
     op_check(qm_get_option(QM_OPT_PREDICTOR_FRAME_OPERATORS, &by_operators), "predictor frame option");
-    const bool one_launch = p.one_launch && by_operators == 0;
+    bool one_launch = p.one_launch && by_operators == 0;
     if (one_launch) {
         // all fifteen steps in one launch (step 0 as two passes of the talker-order chain: same bits as predictor_step0)
-        op_check(qm_predictor_frame_steps(&p.frame, 0, kPredSteps - 1, sampling ? kTopK : 0, kTemperature, p.frame_workspace.raw(),
-                                          static_cast<int64_t>(p.frame_workspace.bytes()), static_cast<uint32_t*>(p.status.raw()), s),
-                 "predictor frame steps");
-    } else {
+        const int32_t rc = qm_predictor_frame_steps(&p.frame, 0, kPredSteps - 1, sampling ? kTopK : 0, kTemperature, p.frame_workspace.raw(),
+                                                    static_cast<int64_t>(p.frame_workspace.bytes()), static_cast<uint32_t*>(p.status.raw()), s);
+        if (rc == QM_ERR_NO_DEVICE) {
+            // the stream cannot hold that launch (nothing of it was queued): operator by operator, now and from now on
+            p.one_launch = false;
+            one_launch = false;
+        } else {
+            op_check(rc, "predictor frame steps");
+        }
+    }
+    if (!one_launch) {
         predictor_step0(p, sampling);
         for (int step = 1; step < kPredSteps; ++step) predictor_step_m1(p, step, sampling);
     }
@@ -381,12 +393,17 @@ static void predictor_frame_launch(qm_predictor& p, const uint16_t* talker_hidde
     hip_check(hipMemcpyAsync(&result->code0, code0_device, sizeof(int32_t), hipMemcpyDeviceToHost, s), "code read-back");
     // (the status word is zero unless the one launch of the frame's steps gave up)
     hip_check(hipMemcpyAsync(&result->status, p.status.raw(), sizeof(uint32_t), hipMemcpyDeviceToHost, s), "status read-back");
+    result->talker_status = 0;
+    if (talker_status_device)
+        hip_check(hipMemcpyAsync(&result->talker_status, talker_status_device, sizeof(uint32_t), hipMemcpyDeviceToHost, s),
+                  "talker status read-back");
 }
 
 // After the frame has run: a frame kernel that gave up waiting fails the call, and its workspace starts over.
 static void predictor_frame_finish(qm_predictor& p, const FrameResult& result) {
     if (result.status == 0) return;
     hipStream_t s = p.stream;
+    if (result.status & QM_STATUS_FRAME_TIMEOUT) p.one_launch = false;   // something else holds compute units: operators from now on
     hip_check(hipMemsetAsync(p.status.raw(), 0, sizeof(uint32_t), s), "status reset");
     op_check(qm_predictor_frame_workspace_init(p.frame_workspace.raw(), static_cast<int64_t>(p.frame_workspace.bytes()), s),
              "predictor frame workspace");
@@ -516,13 +533,22 @@ extern "C" int32_t qm_generate(qm_talker* talker, qm_final_head* head, qm_predic
                 hip_check(hipMemcpyAsync(head->rng_after_head.raw(), head->rng.raw(), sizeof(uint64_t), hipMemcpyDeviceToDevice, stream),
                           "generator state snapshot");
                 const uint16_t* context = frame < trailing_rows ? trailing_text_host + static_cast<size_t>(frame) * kOuter : tts_pad_host;
-                predictor_frame_launch(*predictor, hidden, static_cast<const int32_t*>(head->code.raw()), context, sampling != 0, mailbox.result);
+                predictor_frame_launch(*predictor, hidden, static_cast<const int32_t*>(head->code.raw()), context, sampling != 0, mailbox.result,
+                                       qm_talker_status_device(talker));
                 hip_check(hipEventRecord(mailbox.arrived, stream), "frame event record");
                 if (frame + 1 < maximum_frames)
                     op_check(qm_talker_decode_device_rope(talker, predictor->next_input.u16(), cos_device + static_cast<size_t>(frame) * kHeadDim,
                                                           sin_device + static_cast<size_t>(frame) * kHeadDim, frame, &hidden), "talker decode");
                 hip_check(hipEventSynchronize(mailbox.arrived), "frame boundary synchronize");
                 const FrameResult result = *mailbox.result;
+                if (result.talker_status != 0) {
+                    // a talker kernel flagged this step or an earlier one (a launch that gave up waiting returns at once from
+                    // then on, and the frames after it would run on a stale hidden state): stop here; the synchronisation
+                    // reports the bits, clears them and sets the hand-off workspace up again
+                    (void)hipStreamSynchronize(stream);
+                    op_check(qm_talker_synchronize(talker), "talker status during generation");
+                    throw ApiError(QM_ERR_STATUS, "talker kernels reported status bits " + std::to_string(result.talker_status));
+                }
                 predictor_frame_finish(*predictor, result);
                 if (result.code0 == kCodecEos && frame >= 2) {
                     hip_check(hipMemcpyAsync(head->rng.raw(), head->rng_after_head.raw(), sizeof(uint64_t), hipMemcpyDeviceToDevice, stream),

@@ -58,4 +58,27 @@ inline int32_t ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<boo
 
 inline int32_t launch_status() { return hip_code(hipGetLastError()); }
 
+// Whether a kernel all of whose `blocks` blocks must be resident at once (they wait for one another) can be launched
+// on `hip_stream`: blocks_per_cu (the occupancy the runtime reports for the kernel) times the compute units the
+// stream's kernels may use — the device's, or fewer if the stream was created with a CU mask — must hold them all.
+// On a stream that is confined to a part of the chip the blocks left over would never start and the ones running
+// would wait for them until their bounded waits give up.  (What other streams' kernels occupy at the moment of the
+// launch cannot be asked: such a kernel needs the chip to itself for its duration.)
+inline int32_t resident_blocks_fit(void* hip_stream, int device, int blocks_per_cu, int blocks, bool* fits) {
+    int compute_units = 0;
+    const hipError_t e = hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device);
+    if (e != hipSuccess) return hip_code(e);
+    uint32_t mask[32] = {};
+    int usable = compute_units;
+    if (hipExtStreamGetCUMask(static_cast<hipStream_t>(hip_stream), 32, mask) == hipSuccess) {
+        int bits = 0;
+        for (int w = 0; w < 32; ++w) bits += __builtin_popcount(mask[w]);
+        if (bits > 0 && bits < usable) usable = bits;
+    } else {
+        (void)hipGetLastError();      // a stream that cannot be asked (mid-capture, say) counts as unmasked
+    }
+    *fits = static_cast<int64_t>(blocks_per_cu) * usable >= blocks;
+    return QM_OK;
+}
+
 }  // namespace qm

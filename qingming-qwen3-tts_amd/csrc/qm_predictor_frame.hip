@@ -709,10 +709,43 @@ __global__ void predictor_frame_clear_kernel(uint32_t* words, int count) {
     if (i < count) words[i] = i == kFrWsBase ? 1u : 0u;
 }
 
+// Every block must be resident at once, one per CU: QM_OK if `hip_stream` can hold the launch, QM_ERR_NO_DEVICE if
+// the device, or the part of it the stream is confined to by a CU mask, is too small.  (The occupancy is asked of the
+// runtime once per device, the stream's mask at every call.)
+int32_t frame_residency(void* hip_stream) {
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return hip_code(err);
+    if (device < 0 || device >= kMaxDevices) return QM_ERR_NO_DEVICE;
+    static std::atomic<bool> lds_raised[kMaxDevices];
+    const int32_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(predictor_frame_kernel), kFrLdsBytes, lds_raised);
+    if (rc != QM_OK) return rc;
+    static std::atomic<int> per_cu_of[kMaxDevices];        // 0: not asked yet; else blocks a CU holds at once (-1: none)
+    int per_cu = per_cu_of[device].load(std::memory_order_acquire);
+    if (per_cu == 0) {
+        err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, predictor_frame_kernel, kFrThreads, kFrLdsBytes);
+        if (err != hipSuccess) return hip_code(err);
+        if (per_cu <= 0) per_cu = -1;
+        per_cu_of[device].store(per_cu, std::memory_order_release);
+    }
+    bool fits = false;
+    const int32_t rc_fit = resident_blocks_fit(hip_stream, device, per_cu > 0 ? per_cu : 0, kFrBlocks, &fits);
+    if (rc_fit != QM_OK) return rc_fit;
+    return fits ? QM_OK : QM_ERR_NO_DEVICE;
+}
+
 }  // namespace
 }  // namespace qm
 
 extern "C" int64_t qm_predictor_frame_workspace_bytes(void) { return qm::kFrWsBytes; }
+
+extern "C" int32_t qm_predictor_frame_fits(void* hip_stream, int32_t* fits) {
+    if (!fits) return QM_ERR_NULL;
+    const int32_t rc = qm::frame_residency(hip_stream);
+    if (rc != QM_OK && rc != QM_ERR_NO_DEVICE) return rc;
+    *fits = rc == QM_OK ? 1 : 0;
+    return QM_OK;
+}
 
 extern "C" int32_t qm_predictor_frame_workspace_init(void* workspace, int64_t workspace_bytes, void* hip_stream) {
     using namespace qm;
@@ -776,25 +809,8 @@ extern "C" int32_t qm_predictor_frame_steps(const qm_predictor_frame* frame, int
     const int32_t spin_option = option_value(QM_OPT_PREDICTOR_FRAME_SPIN_LIMIT);
     prm.spin_limit = spin_option > 0 ? static_cast<unsigned>(spin_option) : kFrSpinLimit;
 
-    // every block must be resident at once: one per CU (asked of the runtime once per device)
-    int device = 0;
-    hipError_t err = hipGetDevice(&device);
-    if (err != hipSuccess) return hip_code(err);
-    if (device < 0 || device >= kMaxDevices) return QM_ERR_NO_DEVICE;
-    static std::atomic<bool> lds_raised[kMaxDevices];
-    const int32_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(predictor_frame_kernel), kFrLdsBytes, lds_raised);
+    const int32_t rc = qm::frame_residency(hip_stream);
     if (rc != QM_OK) return rc;
-    static std::atomic<int> resident[kMaxDevices];         // 0: not asked yet; else blocks the device holds at once
-    int holds = resident[device].load(std::memory_order_acquire);
-    if (holds == 0) {
-        int compute_units = 0, per_cu = 0;
-        err = hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device);
-        if (err == hipSuccess) err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, predictor_frame_kernel, kFrThreads, kFrLdsBytes);
-        if (err != hipSuccess) return hip_code(err);
-        holds = per_cu * compute_units > 0 ? per_cu * compute_units : -1;
-        resident[device].store(holds, std::memory_order_release);
-    }
-    if (holds < kFrBlocks) return QM_ERR_NO_DEVICE;
     hipLaunchKernelGGL(predictor_frame_kernel, dim3(kFrBlocks), dim3(kFrThreads), kFrLdsBytes, static_cast<hipStream_t>(hip_stream), prm);
     return launch_status();
 }

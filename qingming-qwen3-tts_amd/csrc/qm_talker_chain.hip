@@ -577,6 +577,31 @@ int32_t check_chain(const qm_talker_post_attention* op, const void* workspace, i
     return QM_OK;
 }
 
+// Every block must be resident at once, one per CU: QM_OK if `hip_stream` can hold the launch, QM_ERR_NO_DEVICE if
+// the device, or the part of it the stream is confined to by a CU mask, is too small.  (The occupancy is asked of the
+// runtime once per device, the stream's mask at every call.)
+int32_t chain_residency(void* hip_stream) {
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return hip_code(err);
+    if (device < 0 || device >= kMaxDevices) return QM_ERR_NO_DEVICE;
+    static std::atomic<bool> lds_raised[kMaxDevices];
+    const int32_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(talker_chain_kernel), kTkLdsBytes, lds_raised);
+    if (rc != QM_OK) return rc;
+    static std::atomic<int> per_cu_of[kMaxDevices];        // 0: not asked yet; else blocks a CU holds at once (-1: none)
+    int per_cu = per_cu_of[device].load(std::memory_order_acquire);
+    if (per_cu == 0) {
+        err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, talker_chain_kernel, kTkThreads, kTkLdsBytes);
+        if (err != hipSuccess) return hip_code(err);
+        if (per_cu <= 0) per_cu = -1;
+        per_cu_of[device].store(per_cu, std::memory_order_release);
+    }
+    bool fits = false;
+    const int32_t rc_fit = resident_blocks_fit(hip_stream, device, per_cu > 0 ? per_cu : 0, kTkBlocks, &fits);
+    if (rc_fit != QM_OK) return rc_fit;
+    return fits ? QM_OK : QM_ERR_NO_DEVICE;
+}
+
 // The launch; with `attention` the kernel first combines that decode step's split records into `context_out`.
 int32_t launch_chain(const qm_talker_post_attention* op, void* workspace, int64_t workspace_bytes, uint32_t* status_dev,
                      void* hip_stream, const DecodeSplitInfo* attention, uint16_t* context_out) {
@@ -605,31 +630,22 @@ int32_t launch_chain(const qm_talker_post_attention* op, void* workspace, int64_
     const int32_t spin_option = option_value(QM_OPT_PREDICTOR_FRAME_SPIN_LIMIT);
     prm.spin_limit = spin_option > 0 ? static_cast<unsigned>(spin_option) : kTkSpinLimit;
 
-    // every block must be resident at once: one per CU (asked of the runtime once per device)
-    int device = 0;
-    hipError_t err = hipGetDevice(&device);
-    if (err != hipSuccess) return hip_code(err);
-    if (device < 0 || device >= kMaxDevices) return QM_ERR_NO_DEVICE;
-    static std::atomic<bool> lds_raised[kMaxDevices];
-    const int32_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(talker_chain_kernel), kTkLdsBytes, lds_raised);
+    const int32_t rc = chain_residency(hip_stream);
     if (rc != QM_OK) return rc;
-    static std::atomic<int> resident[kMaxDevices];         // 0: not asked yet; else blocks the device holds at once
-    int holds = resident[device].load(std::memory_order_acquire);
-    if (holds == 0) {
-        int compute_units = 0, per_cu = 0;
-        err = hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device);
-        if (err == hipSuccess) err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, talker_chain_kernel, kTkThreads, kTkLdsBytes);
-        if (err != hipSuccess) return hip_code(err);
-        holds = per_cu * compute_units > 0 ? per_cu * compute_units : -1;
-        resident[device].store(holds, std::memory_order_release);
-    }
-    if (holds < kTkBlocks) return QM_ERR_NO_DEVICE;
     hipLaunchKernelGGL(talker_chain_kernel, dim3(kTkBlocks), dim3(kTkThreads), kTkLdsBytes, static_cast<hipStream_t>(hip_stream), prm);
     return launch_status();
 }
 
 }  // namespace
 }  // namespace qm
+
+extern "C" int32_t qm_talker_chain_fits(void* hip_stream, int32_t* fits) {
+    if (!fits) return QM_ERR_NULL;
+    const int32_t rc = qm::chain_residency(hip_stream);
+    if (rc != QM_OK && rc != QM_ERR_NO_DEVICE) return rc;
+    *fits = rc == QM_OK ? 1 : 0;
+    return QM_OK;
+}
 
 extern "C" int32_t qm_talker_post_attention_m1(const qm_talker_post_attention* op, void* workspace, int64_t workspace_bytes,
                                                uint32_t* status_dev, void* hip_stream) {
@@ -646,6 +662,8 @@ extern "C" int32_t qm_talker_layer_step_m1(const qm_talker_layer_step* step, voi
     post.context = step->context;
     const int32_t bad = check_chain(&post, workspace, workspace_bytes);
     if (bad != QM_OK) return bad;
+    const int32_t no_room = chain_residency(hip_stream);
+    if (no_room != QM_OK) return no_room;
     DecodeSplitInfo info = {};
     const int32_t rc = decode_step(step->q, step->k, step->v, step->q_norm_w, step->k_norm_w, step->cos_row, step->sin_row,
                                    step->q_rotated_out, step->cache, step->page_table, step->max_pages, step->context, step->q_heads,

@@ -30,6 +30,7 @@ _SIGNATURES = {
     "qm_talker_prefill": (_I32, [_P, _P, _P, _P, _I32, C.POINTER(_P)]),
     "qm_talker_synchronize": (_I32, [_P]),
     "qm_talker_stream": (_P, [_P]),
+    "qm_talker_status_device": (_P, [_P]),
     "qm_final_head_create": (_I32, [C.c_char_p, _I32, _U64, _P, C.POINTER(_P)]),
     "qm_final_head_destroy": (None, [_P]),
     "qm_final_head_reset": (_I32, [_P, _U64]),

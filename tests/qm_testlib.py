@@ -24,6 +24,18 @@ def max_abs_err(oracle, a_bits, b_bits):
     return float(np.max(np.abs(a - b))) if a.size else 0.0
 
 
+def within_rule(oracle, got_bits, want_bits, tol=1e-2):
+    """The one tolerance rule for bf16 outputs, per element: |got - want| <= max(tol, one bf16 ulp of the oracle's
+    value).  north_star's bound is tol = 1e-2; from |x| = 2 on a single bf16 step is 1.56e-2, so a result that is the
+    neighbouring bf16 value of the oracle's cannot be held to 1e-2 there.  Returns (every element within the rule,
+    max abs error, number of elements outside the rule)."""
+    want = oracle.bf16_to_f32(want_bits).astype(np.float64)
+    err = np.abs(oracle.bf16_to_f32(got_bits).astype(np.float64) - want)
+    one_ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 2.0 ** -20))) - 7)
+    outside = int(np.count_nonzero(err > np.maximum(one_ulp, tol)))
+    return outside == 0, float(err.max()) if err.size else 0.0, outside
+
+
 def ulp_distance(a_bits, b_bits):
     """Distance in bf16 ulps between two arrays of finite same-sign-or-not bf16 bit patterns."""
     def key(x):

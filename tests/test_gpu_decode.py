@@ -7,7 +7,7 @@ checked against that policy and against the reference chain (bf16(P) included).
 import numpy as np
 import pytest
 
-from qm_testlib import SCALE, PagedPool, max_abs_err, to_dev, to_u16
+from qm_testlib import SCALE, PagedPool, max_abs_err, to_dev, to_u16, within_rule
 
 pytestmark = pytest.mark.gpu
 
@@ -60,10 +60,7 @@ def test_decode_single_flat(oracle, qm, dev, ctx, max_cache):
         # output by up to one bf16 ulp of the output, which beyond |x| = 2 is more than the tolerance: there the
         # online result is held to one ulp of the reference chain's value, everywhere else to the tolerance.
         # (Measured over ten seeds per context: 2 ulps at most with fewer than 8 keys, 1 ulp from 8 keys on.)
-        ref = oracle.bf16_to_f32(want[0]).astype(np.float64)
-        err = np.abs(oracle.bf16_to_f32(got).astype(np.float64) - ref)
-        one_ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref), 2.0 ** -20))) - 7)
-        assert np.all(err <= np.maximum(one_ulp, TOL))
+        assert within_rule(oracle, got, want[0], TOL)[0]
     if ctx == 1:
         assert np.array_equal(got, want[0])                 # out = V[0] exactly
 

@@ -23,7 +23,7 @@ HEAD_V, EOS, TABLE_ROWS = 3072, 2150, 3072
 SEED = 20240229
 
 
-def _checkpoint(directory, eos_gain=1.0):
+def _checkpoint(directory, eos_gain=1.0, intermediate=I_T):
     import torch
     from safetensors.torch import save_file
     g = torch.Generator().manual_seed(99)
@@ -39,8 +39,8 @@ def _checkpoint(directory, eos_gain=1.0):
                   p + "self_attn.q_proj.weight": rnd((Q, H), 0.02), p + "self_attn.k_proj.weight": rnd((KV, H), 0.02),
                   p + "self_attn.v_proj.weight": rnd((KV, H), 0.02), p + "self_attn.o_proj.weight": rnd((H, Q), 0.02),
                   p + "self_attn.q_norm.weight": rnd((128,), 0.1, 1.0), p + "self_attn.k_norm.weight": rnd((128,), 0.1, 1.0),
-                  p + "mlp.gate_proj.weight": rnd((I_T, H), 0.03), p + "mlp.up_proj.weight": rnd((I_T, H), 0.03),
-                  p + "mlp.down_proj.weight": rnd((H, I_T), 0.03)})
+                  p + "mlp.gate_proj.weight": rnd((intermediate, H), 0.03), p + "mlp.up_proj.weight": rnd((intermediate, H), 0.03),
+                  p + "mlp.down_proj.weight": rnd((H, intermediate), 0.03)})
     c = "talker.code_predictor."
     t.update({c + "small_to_mtp_projection.weight": rnd((PH, H), 0.02), c + "small_to_mtp_projection.bias": rnd((PH,), 0.1),
               c + "model.norm.weight": rnd((PH,), 0.1, 1.0)})
@@ -331,4 +331,133 @@ def test_generation_stops_at_the_end_of_sequence_code(engine, oracle, qm, dev, t
     head.reset(SEED)
     again, digest2 = engine.generate(talker, head, predictor, pd, prompt_rows, limit, tts_pad, None)
     assert np.array_equal(again, codes) and digest2 == digest
+    predictor.close(); head.close(); talker.close()
+
+
+def _masked_stream(compute_units):
+    """A HIP stream confined to the first `compute_units` compute units (hipExtStreamCreateWithCUMask), as the
+    reference's generation stream is (R17:7733-7792)."""
+    hip = C.CDLL("libamdhip64.so")
+    words = (compute_units + 31) // 32
+    mask = (C.c_uint32 * words)(*[0xFFFFFFFF if 32 * (i + 1) <= compute_units else (1 << (compute_units - 32 * i)) - 1
+                                  for i in range(words)])
+    stream = C.c_void_p()
+    assert hip.hipExtStreamCreateWithCUMask(C.byref(stream), C.c_uint32(words), mask) == 0
+    return hip, stream
+
+
+def test_a_stream_confined_to_part_of_the_chip_takes_the_operators_one_by_one(engine, oracle, qm, dev, tmp_path):
+    """The two one-launch kernels (a talker layer between two attentions, the predictor's frame) need all 256 compute
+    units at once.  On a stream with a CU mask of half the chip the library says so without launching (…_fits = 0, the
+    launch entry returns QM_ERR_NO_DEVICE), and engines created on that stream run operator by operator: the same codes
+    and hash as engines on an unconfined stream."""
+    import torch
+    directory = str(tmp_path)
+    _checkpoint(directory, intermediate=6144)                # the geometry the talker's one launch per layer serves
+    prompt_rows, frames = 13, 4
+    prompt = oracle.normal_bf16((prompt_rows, H), 61)
+    pd = torch.from_numpy(prompt.view(np.int16)).to(dev)
+    tts_pad = oracle.normal_bf16((H,), 62, 0.0, 0.5)
+    torch.cuda.synchronize()
+    assert qm.talker_chain_fits(0) and qm.predictor_frame_fits(0)
+    talker = engine.Talker(directory, 64)
+    head = engine.FinalHead(directory, 32, SEED, talker.stream)
+    predictor = engine.Predictor(directory, head.rng_state, talker.stream)
+    want, want_digest = engine.generate(talker, head, predictor, pd, prompt_rows, frames, tts_pad, None)
+    predictor.close(); head.close(); talker.close()
+
+    hip, stream = _masked_stream(128)
+    try:
+        assert not qm.talker_chain_fits(stream.value) and not qm.predictor_frame_fits(stream.value)
+        ws_bytes = qm.talker_post_attention_workspace_bytes()
+        ws = torch.zeros(ws_bytes // 4 + 64, dtype=torch.int32, device=dev)
+        z = torch.zeros(8192, dtype=torch.int16, device=dev)
+        big = torch.zeros((6144, 2048), dtype=torch.int16, device=dev)
+        op = qm.talker_post_attention(context=z, hidden=z, o_weight=big, post_norm=z, gate_weight=big, up_weight=big,
+                                      down_weight=big, hidden_out=z)
+        with pytest.raises(qm.QmError) as info:
+            qm.talker_post_attention_m1(op, ws, ws_bytes, None, stream.value)
+        assert info.value.code == -6
+        talker = engine.Talker(directory, 64, stream.value)
+        head = engine.FinalHead(directory, 32, SEED, talker.stream)
+        predictor = engine.Predictor(directory, head.rng_state, talker.stream)
+        got, digest = engine.generate(talker, head, predictor, pd, prompt_rows, frames, tts_pad, None)
+        assert np.array_equal(got, want) and digest == want_digest
+        predictor.close(); head.close(); talker.close()
+    finally:
+        torch.cuda.synchronize()
+        assert hip.hipStreamDestroy(stream) == 0
+
+
+def test_a_talker_launch_that_gives_up_ends_the_generation_at_once_and_the_engine_recovers(engine, oracle, qm, dev, tmp_path):
+    """With the hand-off waits cut to one attempt the talker's one launch per layer gives up (every block returns
+    normally, QM_STATUS_FRAME_TIMEOUT in the engine's status word).  The loop reads that word back with every frame's
+    codes: the generation ends with QM_ERR_STATUS after the first frame that sees it instead of running to the frame
+    limit on a stale hidden state, and the next generation (operator by operator from then on) is right."""
+    import torch
+    directory = str(tmp_path)
+    _checkpoint(directory, intermediate=6144)                # the geometry the talker's one launch per layer serves
+    prompt_rows, frames = 13, 6
+    pd = torch.from_numpy(oracle.normal_bf16((prompt_rows, H), 71).view(np.int16)).to(dev)
+    tts_pad = oracle.normal_bf16((H,), 72, 0.0, 0.5)
+    torch.cuda.synchronize()
+    talker = engine.Talker(directory, 64)
+    head = engine.FinalHead(directory, 32, SEED, talker.stream)
+    predictor = engine.Predictor(directory, head.rng_state, talker.stream)
+    want, want_digest = engine.generate(talker, head, predictor, pd, prompt_rows, frames, tts_pad, None)
+    head.reset(SEED)
+    qm.set_option(qm.OPT_PREDICTOR_FRAME_OPERATORS, 1)       # the predictor by operators: only the talker's launch gives up
+    qm.set_option(qm.OPT_PREDICTOR_FRAME_SPIN_LIMIT, 1)
+    try:
+        with pytest.raises(engine.EngineError) as info:
+            engine.generate(talker, head, predictor, pd, prompt_rows, frames, tts_pad, None)
+        assert info.value.code == -9
+    finally:
+        qm.set_option(qm.OPT_PREDICTOR_FRAME_SPIN_LIMIT, 0)
+        qm.set_option(qm.OPT_PREDICTOR_FRAME_OPERATORS, 0)
+    head.reset(SEED)
+    got, digest = engine.generate(talker, head, predictor, pd, prompt_rows, frames, tts_pad, None)
+    assert np.array_equal(got, want) and digest == want_digest
+    predictor.close(); head.close(); talker.close()
+
+
+def test_prompt_pass_on_the_matrix_cores_against_the_exact_chain(engine, oracle, qm, dev, model, capsys):
+    """From 16 prompt rows on the prompt pass's linears take their sums on the matrix cores (QM_OPT_LINEAR_ROWS_KERNEL 0,
+    the default): tolerance parity with the reference's linear_bf16 chain (R17:126-245), not bit parity, and the codes
+    are sampled, so a trajectory may part from the exact chain's (option value 1) at any frame.  What is held: the
+    prompt pass's last hidden state of the two settings agrees to two bf16 steps of its largest value, either setting is
+    deterministic, and the test reports whether this checkpoint's trajectories agree and from which frame they do not."""
+    import torch
+    directory, w = model
+    prompt_rows, frames = 40, 6
+    pd = torch.from_numpy(oracle.normal_bf16((prompt_rows, H), 81).view(np.int16)).to(dev)
+    tts_pad = oracle.normal_bf16((H,), 82, 0.0, 0.5)
+    torch.cuda.synchronize()
+    talker = engine.Talker(directory, 64)
+    head = engine.FinalHead(directory, 32, SEED, talker.stream)
+    predictor = engine.Predictor(directory, head.rng_state, talker.stream)
+    cos, sin = engine.rope_rows(prompt_rows, 0)
+    runs, hiddens = {}, {}
+    for setting in (0, 1, 0):
+        qm.set_option(qm.OPT_LINEAR_ROWS_KERNEL, setting)
+        try:
+            hidden = talker.prefill(pd, cos, sin, prompt_rows)
+            talker.synchronize()
+            bits = _device_bytes(hidden, H * 2).copy()
+            head.reset(SEED)
+            codes, digest = engine.generate(talker, head, predictor, pd, prompt_rows, frames, tts_pad, None)
+        finally:
+            qm.set_option(qm.OPT_LINEAR_ROWS_KERNEL, 0)
+        if setting in runs:
+            assert np.array_equal(runs[setting][0], codes) and runs[setting][1] == digest      # deterministic
+            assert np.array_equal(hiddens[setting], bits)
+        runs[setting], hiddens[setting] = (codes, digest), bits
+    a, b = oracle.bf16_to_f32(hiddens[0]).astype(np.float64), oracle.bf16_to_f32(hiddens[1]).astype(np.float64)
+    step = 2.0 ** (np.floor(np.log2(np.abs(b).max())) - 7)
+    assert np.abs(a - b).max() <= 2 * step
+    same = np.array_equal(runs[0][0], runs[1][0])
+    differ = np.nonzero((runs[0][0] != runs[1][0]).any(axis=1))[0]
+    with capsys.disabled():
+        print("\n[prompt pass: matrix cores vs exact chain] hidden max abs diff %.4g (one bf16 step of the largest value: %.4g); "
+              "trajectories %s" % (np.abs(a - b).max(), step, "agree" if same else "part at frame %d" % differ[0]))
     predictor.close(); head.close(); talker.close()

@@ -11,7 +11,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from qm_testlib import max_abs_err, to_dev, to_u16
+from qm_testlib import max_abs_err, to_dev, to_u16, within_rule
 
 pytestmark = pytest.mark.gpu
 
@@ -56,18 +56,20 @@ def _run_selected(oracle, qm, dev, units, layers, rows, seed, first_rows, write_
 def test_predictor_config5_full_size(oracle, qm, dev, kernel):
     units, layers, rows = 256 * 5, 5, 16
     got, want, (kd, vd), (kc, vc), v = _run(oracle, qm, dev, units, layers, rows, seed=55, kernel=kernel)
+    # One rule for both kernels (qm_testlib.within_rule): every output within max(1e-2, one bf16 ulp of the oracle's
+    # value).  The exact-chain kernel meets it on every element.  The matrix-core kernel sums the 128 products of a
+    # score in the matrix core's order, and the reference chain rounds that score to bf16 (R17:12449-12463): about once
+    # in 10^6 outputs the two orders fall on different sides of a rounding boundary, the score moves by one bf16 step
+    # (0.25 at |s| >= 32, 2 % of a probability after the scale) and with at most 16 keys one probability carries the
+    # output, which then moves by up to 1.6e-2 whatever its own magnitude.  No order of summation other than the
+    # reference's can avoid that; what is held is how rare and how large it is (measured over four seeds of this
+    # shape: at most 3 of the 2.6 million outputs outside the rule, largest 1.6e-2).
+    ok, worst, outside = within_rule(oracle, got, want, TOL)
     if kernel == EXACT:
-        assert max_abs_err(oracle, got, want) <= TOL
-        assert (got != want).mean() < 1e-3                    # only device-expf rounding may differ
+        assert ok, (worst, outside)
     else:
-        # The reference chain rounds scores and probabilities to bf16, so it is discontinuous: another order of
-        # the fp32 sums (the matrix core's) moves a value across a rounding boundary about once in 10^4, and a
-        # bf16 output of magnitude >= 2 then moves by 1.6e-2.  Measured over four seeds of this shape: at most 3
-        # of the 2.6 million outputs beyond 1e-2, largest 1.6e-2 (the exact-chain kernel: at most 1, from the
-        # device's expf).
-        err = np.abs(oracle.bf16_to_f32(got).astype(np.float64) - oracle.bf16_to_f32(want).astype(np.float64))
-        assert np.count_nonzero(err > TOL) <= 4 and err.max() <= 2e-2
-        assert (got != want).mean() < 2e-3
+        assert outside <= 4 and worst <= 2e-2, (worst, outside)
+    assert (got != want).mean() < (1e-3 if kernel == EXACT else 2e-3)
     assert np.array_equal(kd, kc) and np.array_equal(vd, vc)  # cache write-back, bit-exact
     assert np.array_equal(got[:, 0], np.repeat(v[:, 0], 2, axis=1))   # step 0: context 1 -> out = V
 
