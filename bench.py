@@ -1104,6 +1104,9 @@ def main():
                                       "qkv", "layer", "layer1", "layer2", "frame", "frame1", "linears", "linearsexact", "linears128", "linears128split", "generate"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
+    ap.add_argument("--layers", type=int, default=28,
+                    help="with --only layer / layer1 / layer2: distinct weight sets and caches in rotation (a profiler that "
+                         "records counters for every dispatch is spared most of the input generation with a small number)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 512 MiB device-to-device copies (for scaling rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters against a kernel of known traffic)")
@@ -1143,7 +1146,8 @@ def main():
                 "chunk": lambda: PrefillChunk(qm, dev), "chunkwhole": lambda: PrefillChunk(qm, dev, split=False), "chunkrows": lambda: PrefillChunk(qm, dev, by_rows=True),
                 "predictor": lambda: PredictorLoop(qm, dev),
                 "predictorexact": lambda: PredictorLoop(qm, dev, kernel=1),
-                "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev), "layer1": lambda: TalkerLayerStep(qm, dev, chained=True), "layer2": lambda: TalkerLayerStep(qm, dev, two_launches=True),
+                "qkv": lambda: QkvGemv(qm, dev, copies=64), "layer": lambda: TalkerLayerStep(qm, dev, layers=args.layers), "layer1": lambda: TalkerLayerStep(qm, dev, layers=args.layers, chained=True),
+                "layer2": lambda: TalkerLayerStep(qm, dev, layers=args.layers, two_launches=True),
                 "frame": lambda: PredictorFrameSteps(qm, dev),
                 "frame1": lambda: PredictorFrameSteps(qm, dev, one_launch=True),
                 "linears": lambda: PromptLinears(qm, dev), "linearsexact": lambda: PromptLinears(qm, dev, kernel=1),
