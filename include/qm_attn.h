@@ -299,8 +299,10 @@ int32_t qm_scatter_kv(
  * LayerCache [kv_head][max_cache][128] is read in place with (128, max_cache*128, 0), which
  * is how launch_attention(query_length > 1, cache_before = 0) is served.
  * Only q_heads == 2 * kv_heads is supported by this entry point.
- * Later tokens never contribute to a row; a non-finite V of a later row inside the same
- * 16-row group would propagate as 0 * inf (the reference skips those keys).
+ * Later tokens never contribute to a row, whatever they hold (a non-finite K or V of a later row included: where the
+ * causal mask cuts a 16-key group the matrix core would multiply the masked V by P = 0, so such a group is checked for
+ * non-finite values and, if it holds any, they are taken out of the matrix product and added for the rows that see
+ * them as the reference's fmaf chain adds them, R17:15784-15789, 15947-15990).
  */
 int32_t qm_prefill_attention_causal(
     const uint16_t* query, const uint16_t* key, const uint16_t* value,

@@ -42,10 +42,10 @@
 // that outputs are large: there P is split into hi + lo bf16 parts (two MFMAs) to stay inside the
 // 1e-2 output tolerance.
 //
-// Causality.  A key after a query row never contributes; keys of later 16-row groups are not
-// read into the product at all.  Inside a wave's own 16-row diagonal group the mask is P = 0
-// times V, so a non-finite V of a later row of the same group would propagate (the reference
-// skips those keys; finite values, the only ones a prefill produces, behave identically).
+// Causality.  A key after a query row never contributes, whatever it holds; keys of later 16-row groups are not
+// read into the product at all.  Inside a 16-key group that the mask cuts the mask is P = 0 times V; such a group is
+// checked for non-finite V values, which are then taken out of the matrix product and added for the rows that see
+// them (add_non_finite_products), so that 0 x inf never forms.
 //
 // Algorithmic work per (batch, kv head): flops = 2 heads * 2 matmuls * 2 * 128 * S(S+1)/2;
 // HBM bytes = Q + O (2 heads) + K + V read once + K + V written to pages.  Bound: MFMA (with the
@@ -137,6 +137,80 @@ __device__ __forceinline__ float halves_max(float v) {
 __device__ __forceinline__ float halves_sum(float v) {
     const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// ---- strict causality inside a 16-key group that the mask cuts ----------------------------------------------------
+// The mask is P = 0, and the MFMA still multiplies the masked key's V by it: 0 x (inf or NaN) is NaN, so a non-finite V
+// of a key after a query row would reach that row, which the reference never lets happen (it does not touch keys after
+// the row, R17:15784-15789).  Only a group the mask cuts for some column of the wave is concerned (groups wholly
+// visible are multiplied as the reference multiplies them, groups wholly masked are skipped), and only if it holds a
+// non-finite V at all, which costs three instructions per fragment register to find out.  Then the fragments'
+// non-finite elements are set to zero, so that the MFMA adds the finite products only, and the products of the
+// non-finite elements are added one by one, for the columns that see the key: fmaf(p, v, o) as the reference forms
+// it (p = 0 included: a probability that underflowed gives NaN there too).
+
+// Whether any lane of the wave holds a non-finite bf16 in the four fragments (a half whose exponent bits are all ones
+// carries into bit 15 / 31).
+__device__ __forceinline__ uint32_t exponent_carries(const bf16x8_t& f) {
+    const uint4 w = __builtin_bit_cast(uint4, f);
+    return ((w.x & 0x7f807f80u) + 0x00800080u) | ((w.y & 0x7f807f80u) + 0x00800080u)
+         | ((w.z & 0x7f807f80u) + 0x00800080u) | ((w.w & 0x7f807f80u) + 0x00800080u);
+}
+__device__ __forceinline__ bool any_non_finite(const bf16x8_t& f0, const bf16x8_t& f1, const bf16x8_t& f2, const bf16x8_t& f3) {
+    const uint32_t acc = exponent_carries(f0) | exponent_carries(f1) | exponent_carries(f2) | exponent_carries(f3);
+    return __builtin_amdgcn_ballot_w64((acc & 0x80008000u) != 0) != 0;
+}
+__device__ __forceinline__ uint32_t finite_halves(uint32_t x) {
+    const uint32_t t = (x & 0x7f807f80u) + 0x00800080u;
+    return x & ((t & 0x8000u ? 0u : 0xffffu) | (t & 0x80000000u ? 0u : 0xffff0000u));
+}
+__device__ __forceinline__ void zero_non_finite(bf16x8_t& f) {
+    uint4 w = __builtin_bit_cast(uint4, f);
+    w.x = finite_halves(w.x); w.y = finite_halves(w.y); w.z = finite_halves(w.z); w.w = finite_halves(w.w);
+    f = __builtin_bit_cast(bf16x8_t, w);
+}
+// The products of the non-finite V elements of the 16 keys key0 .. key0 + 15, for the columns that see the key.
+// p_hi (+ p_lo): this lane's eight probabilities of the group as the MFMA takes them (element i = key
+// 8 (i / 4) + 4 grp + i % 4 of the group; the lane of the other half of the wave holds the other eight).
+// v_head: the V rows of this (batch, kv head); a lane's accumulators o[dt][4 rq + c] are dims 32 dt + 8 rq + 4 grp + c.
+template <bool TWO_PARTS>
+__device__ __forceinline__ void add_non_finite_products(f32x16_t (&o)[4], uint4 p_hi, uint4 p_lo, const uint16_t* v_head,
+                                                        int64_t stride_token, int key0, int key_count, int my_pos, int grp) {
+#pragma unroll 1
+    for (int jj = 0; jj < 16; ++jj) {
+        const int key = key0 + jj;
+        if (key >= key_count) break;
+        const int owner = (jj >> 2) & 1;                   // the half of the wave that holds this key's probability
+        const int i = 4 * (jj >> 3) + (jj & 3);
+        const int w = i >> 1;
+        const uint32_t word_hi = w == 0 ? p_hi.x : w == 1 ? p_hi.y : w == 2 ? p_hi.z : p_hi.w;
+        float mine = (i & 1) ? hi_bf16(word_hi) : lo_bf16(word_hi);
+        if (TWO_PARTS) {
+            const uint32_t word_lo = w == 0 ? p_lo.x : w == 1 ? p_lo.y : w == 2 ? p_lo.z : p_lo.w;
+            mine += (i & 1) ? hi_bf16(word_lo) : lo_bf16(word_lo);
+        }
+        const auto both = __builtin_amdgcn_permlane32_swap(__float_as_uint(mine), __float_as_uint(mine), false, false);
+        // (after the swap the first word is the lower half's value in both halves, the second the upper half's)
+        const float prob = __uint_as_float(owner == 0 ? both[0] : both[1]);
+        if (key > my_pos) continue;                        // this column does not see the key (per lane)
+        const uint16_t* row = v_head + static_cast<int64_t>(key) * stride_token + 4 * grp;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+#pragma unroll
+            for (int rq = 0; rq < 4; ++rq) {
+                // (one request at a time: this path is taken for non-finite inputs only and must not cost the
+                // kernel registers)
+                __builtin_amdgcn_sched_barrier(0);
+                const uint2 four = *reinterpret_cast<const uint2*>(row + 32 * dt + 8 * rq);
+                const float v0 = lo_bf16(four.x), v1 = hi_bf16(four.x), v2 = lo_bf16(four.y), v3 = hi_bf16(four.y);
+                if (!(fabsf(v0) <= 3.3895314e38f)) o[dt][4 * rq + 0] = fmaf(prob, v0, o[dt][4 * rq + 0]);
+                if (!(fabsf(v1) <= 3.3895314e38f)) o[dt][4 * rq + 1] = fmaf(prob, v1, o[dt][4 * rq + 1]);
+                if (!(fabsf(v2) <= 3.3895314e38f)) o[dt][4 * rq + 2] = fmaf(prob, v2, o[dt][4 * rq + 2]);
+                if (!(fabsf(v3) <= 3.3895314e38f)) o[dt][4 * rq + 3] = fmaf(prob, v3, o[dt][4 * rq + 3]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
 }
 
 template <int N> using int_c = std::integral_constant<int, N>;
@@ -352,11 +426,24 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
 #pragma unroll
         for (int kg = 0; kg < 2; ++kg) {
             if (decltype(diag)::value && key_base + 16 * kg > wave_last_row) continue;
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt) {
-                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * kg + dt], p.hi[kg], o[dt], 0, 0, 0);
-                if (PRECISE) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * kg + dt], p.lo[kg], o[dt], 0, 0, 0);
+            bf16x8_t v0 = vf[4 * kg], v1 = vf[4 * kg + 1], v2 = vf[4 * kg + 2], v3 = vf[4 * kg + 3];
+            // (a group the mask cuts for some column of the wave — its last key lies after the wave's first row, or
+            // beyond the keys there are — with a non-finite V: see add_non_finite_products)
+            if (decltype(diag)::value && (key_base + 16 * kg + 15 > wave_last_row - 15 || key_base + 16 * kg + 15 >= SK)
+                && any_non_finite(v0, v1, v2, v3)) {
+                zero_non_finite(v0); zero_non_finite(v1); zero_non_finite(v2); zero_non_finite(v3);
+                add_non_finite_products<PRECISE>(o, __builtin_bit_cast(uint4, p.hi[kg]),
+                                                 PRECISE ? __builtin_bit_cast(uint4, p.lo[kg]) : make_uint4(0, 0, 0, 0),
+                                                 prm.v + kv_base, prm.kv_stride_token, key_base + 16 * kg, SK, my_pos, grp);
             }
+            o[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, p.hi[kg], o[0], 0, 0, 0);
+            if (PRECISE) o[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, p.lo[kg], o[0], 0, 0, 0);
+            o[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p.hi[kg], o[1], 0, 0, 0);
+            if (PRECISE) o[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p.lo[kg], o[1], 0, 0, 0);
+            o[2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v2, p.hi[kg], o[2], 0, 0, 0);
+            if (PRECISE) o[2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v2, p.lo[kg], o[2], 0, 0, 0);
+            o[3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v3, p.hi[kg], o[3], 0, 0, 0);
+            if (PRECISE) o[3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v3, p.lo[kg], o[3], 0, 0, 0);
         }
     };
     // Softmax works in `units`: rounded scaled scores (ROUND) or raw fp32 dot products, whose
@@ -727,45 +814,39 @@ __device__ __forceinline__ void copy_tile_to_pages(const PrefillParams& prm, con
     const int32_t* table = prm.page_table ? prm.page_table + static_cast<int64_t>(b) * prm.pages.max_pages : nullptr;
     const int64_t kv_base = static_cast<int64_t>(b) * prm.kv_stride_batch + static_cast<int64_t>(kvh) * prm.kv_stride_head;
     uint32_t page_err = 0;
-    // every load below is unconditional (indices clamped into range), so that all twelve are in flight at once
-    int page[4], phys[4];
-    bool live[4];
-    uint4 kx[4], vx[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    // (named registers, not arrays or structures — those end up as stack objects here — and every load unconditional,
+    // indices clamped into range, so that all twelve are in flight at once; phys < -1 marks a row that is not written)
+    auto request = [&](int i, uint4& kx, uint4& vx, int& page, int& phys) {
         const int key = tile * kBM + (tid >> 4) + 16 * i;
-        live[i] = key < prm.seq;
-        page[i] = page_of(prm.pages, live[i] ? key : 0);
-        if (live[i] && page[i] >= prm.pages.max_pages) {
+        bool live = key < prm.seq;
+        page = page_of(prm.pages, live ? key : 0);
+        if (live && page >= prm.pages.max_pages) {
             page_err |= QM_STATUS_BAD_POSITION;
-            live[i] = false;
+            live = false;
         }
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int entry = live[i] ? page[i] : 0;
-        phys[i] = table ? table[entry] : entry;
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int key = min(tile * kBM + (tid >> 4) + 16 * i, prm.seq - 1);
-        const int64_t off = kv_base + static_cast<int64_t>(key) * prm.kv_stride_token + 8 * (tid & 15);
-        kx[i] = *reinterpret_cast<const uint4*>(prm.k + off);
-        vx[i] = *reinterpret_cast<const uint4*>(prm.v + off);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        if (!live[i]) continue;
-        if (phys[i] < 0 || phys[i] >= cache.n_pages) {
+        const int entry = live ? page : 0;
+        const int found = table ? table[entry] : entry;
+        phys = live ? found : -2;
+        const int64_t off = kv_base + static_cast<int64_t>(min(key, prm.seq - 1)) * prm.kv_stride_token + 8 * (tid & 15);
+        kx = *reinterpret_cast<const uint4*>(prm.k + off);
+        vx = *reinterpret_cast<const uint4*>(prm.v + off);
+    };
+    auto write = [&](int i, const uint4& kx, const uint4& vx, int page, int phys) {
+        if (phys == -2) return;
+        if (phys < 0 || phys >= cache.n_pages) {
             page_err |= QM_STATUS_BAD_PAGE;
-            continue;
+            return;
         }
         const int key = tile * kBM + (tid >> 4) + 16 * i;
-        const int64_t off = static_cast<int64_t>(phys[i]) * cache.stride_page + static_cast<int64_t>(kvh) * cache.stride_head
-                          + static_cast<int64_t>(key - page[i] * prm.pages.page_size) * kDim + 8 * (tid & 15);
-        *reinterpret_cast<uint4*>(cache.k_pool + off) = kx[i];
-        *reinterpret_cast<uint4*>(cache.v_pool + off) = vx[i];
-    }
+        const int64_t off = static_cast<int64_t>(phys) * cache.stride_page + static_cast<int64_t>(kvh) * cache.stride_head
+                          + static_cast<int64_t>(key - page * prm.pages.page_size) * kDim + 8 * (tid & 15);
+        *reinterpret_cast<uint4*>(cache.k_pool + off) = kx;
+        *reinterpret_cast<uint4*>(cache.v_pool + off) = vx;
+    };
+    uint4 k0, k1, k2, k3, v0, v1, v2, v3;
+    int g0, g1, g2, g3, p0, p1, p2, p3;
+    request(0, k0, v0, g0, p0); request(1, k1, v1, g1, p1); request(2, k2, v2, g2, p2); request(3, k3, v3, g3, p3);
+    write(0, k0, v0, g0, p0); write(1, k1, v1, g1, p1); write(2, k2, v2, g2, p2); write(3, k3, v3, g3, p3);
     if (page_err && prm.status) atomicOr(prm.status, page_err);
 }
 
@@ -1366,9 +1447,18 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
 #pragma unroll
         for (int kg = 0; kg < 2; ++kg) {
             if (key_base + 16 * kg > group_row0(c) + 15) continue;
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
-                o[c][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * kg + dt], p.g[kg], o[c][dt], 0, 0, 0);
+            // (the group the mask cuts — the one of the wave's own rows, or one that reaches beyond S — with a
+            // non-finite V: see add_non_finite_products)
+            bf16x8_t v0 = vf[4 * kg], v1 = vf[4 * kg + 1], v2 = vf[4 * kg + 2], v3 = vf[4 * kg + 3];
+            if ((key_base + 16 * kg + 15 > group_row0(c) || key_base + 16 * kg + 15 >= S) && any_non_finite(v0, v1, v2, v3)) {
+                zero_non_finite(v0); zero_non_finite(v1); zero_non_finite(v2); zero_non_finite(v3);
+                add_non_finite_products<false>(o[c], __builtin_bit_cast(uint4, p.g[kg]), make_uint4(0, 0, 0, 0), prm.v + kv_base,
+                                               prm.kv_stride_token, key_base + 16 * kg, S, group_row0(c) + (col & 15), grp);
+            }
+            o[c][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, p.g[kg], o[c][0], 0, 0, 0);
+            o[c][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p.g[kg], o[c][1], 0, 0, 0);
+            o[c][2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v2, p.g[kg], o[c][2], 0, 0, 0);
+            o[c][3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v3, p.g[kg], o[c][3], 0, 0, 0);
         }
     };
     if (last_part)

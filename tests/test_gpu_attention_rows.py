@@ -323,3 +323,21 @@ def test_chunk_argument_errors(qm, dev):
     assert qm.lib().qm_prefill_attention_chunk(None, p, p, p, 1, 4, 5, 16, 8, SCALE, 0, 0, 0, None, 0, None) == -1
     assert qm.lib().qm_prefill_attention_chunk(p, p, p, p, 1, 4, 5, 16, 8, SCALE, 0, 0, 0, None, 64, None) == -5
     assert qm.lib().qm_prefill_attention_chunk(p, p, p, p, 1, 4, 5, 16, 8, SCALE, 0, 0, 0, p + 16, 64, None) == -2
+
+
+@pytest.mark.parametrize("rows,before", [(40, 37), (70, 0), (33, 128)])
+def test_chunk_rows_never_see_the_keys_after_them(oracle, qm, dev, rows, before):
+    """Keys after a row's position may hold anything — NaN included — without reaching the row, also inside the 16-key
+    groups the causal mask cuts (where the matrix core multiplies the masked V by P = 0): the reference does not touch
+    them (R17:15784-15789).  The rows' positions here are not multiples of 16, so a wave's rows cut two key groups."""
+    import torch
+    got, _, (qd, kd, vd, max_cache) = _chunk(oracle, qm, dev, rows, before, seed=7100 + rows)
+    strides = (128, max_cache * 128, 8 * max_cache * 128)
+    for r in list(range(0, min(rows - 1, 34))) + [rows - 2]:
+        k2, v2 = kd.clone(), vd.clone()
+        k2[:, :, before + r + 1:] = 0x7fc0                # NaN
+        v2[:, :, before + r + 1:] = 0x7fc0
+        out = torch.full((1, rows, 16, 128), 0, dtype=torch.int16, device=dev)
+        qm.prefill_attention_chunk(qd, k2, v2, out, 1, rows, before, 16, 8, SCALE, kv_strides=strides)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_u16(out)[0, :r + 1], got[0, :r + 1]), (r,)

@@ -98,16 +98,58 @@ def test_prefill_without_cache_and_causality(oracle, qm, dev):
     import torch
     got, want, _, _, _, (q, k, v) = _run(oracle, qm, dev, 1, 200, seed=9, with_cache=False)
     assert max_abs_err(oracle, got, want[1]) <= TOL
-    # Later tokens must not leak into earlier rows: huge finite values anywhere after the row,
-    # NaN from the next 16-row group on (inside a row's own 16-row group the mask is P = 0 times V).
-    for first_bad, poison, rows_ok in ((150, 0x7f7f, 150), (160, 0x7fc0, 160)):
-        k2, v2 = k.copy(), v.copy()
-        k2[0, first_bad:] = poison
-        v2[0, first_bad:] = poison
-        out = torch.zeros((1, 200, 16, 128), dtype=torch.int16, device=dev)
-        qm.prefill_attention_causal(to_dev(q, dev), to_dev(k2, dev), to_dev(v2, dev), out, None, None, 0, 1, 200, 16, 8)
-        torch.cuda.synchronize()
-        assert np.array_equal(to_u16(out)[0, :rows_ok], got[0, :rows_ok])
+    # Later tokens must not leak into earlier rows, whatever they hold: huge finite values, infinities or NaN from the
+    # very next row on — inside a wave's own 16-row group too, where the mask is P = 0 and 0 x NaN would be NaN
+    # (the reference does not touch keys after the row, R17:15784-15789).  Every position of the boundary inside a
+    # 16-row group is tried for one group, and a few boundaries elsewhere (tile edges, the first and the last rows).
+    for kernel in (0, 1):
+        qm.set_option(qm.OPT_PREFILL_KERNEL, kernel)
+        try:
+            base = torch.zeros((1, 200, 16, 128), dtype=torch.int16, device=dev)
+            qm.prefill_attention_causal(to_dev(q, dev), to_dev(k, dev), to_dev(v, dev), base, None, None, 0, 1, 200, 16, 8)
+            torch.cuda.synchronize()
+            base = to_u16(base)
+            for first_bad, poison in [(150, 0x7f7f), (160, 0x7fc0), (1, 0x7fc0), (17, 0x7f80), (63, 0xff80), (64, 0x7fc0), (65, 0x7fc0),
+                                      (199, 0x7fc0)] + [(r, 0x7fc0) for r in range(129, 145)]:
+                k2, v2 = k.copy(), v.copy()
+                k2[0, first_bad:] = poison
+                v2[0, first_bad:] = poison
+                out = torch.zeros((1, 200, 16, 128), dtype=torch.int16, device=dev)
+                qm.prefill_attention_causal(to_dev(q, dev), to_dev(k2, dev), to_dev(v2, dev), out, None, None, 0, 1, 200, 16, 8)
+                torch.cuda.synchronize()
+                assert np.array_equal(to_u16(out)[0, :first_bad], base[0, :first_bad]), (kernel, first_bad, hex(poison))
+        finally:
+            qm.set_option(qm.OPT_PREFILL_KERNEL, 0)
+
+
+def test_a_non_finite_value_row_reaches_the_rows_that_see_it_as_in_the_reference(oracle, qm, dev):
+    """One V row of infinities and NaN in the middle of the prompt: the rows before it are untouched, and the rows from
+    it on get what the reference's fmaf chain gives them — NaN or an infinity in exactly the dims the poisoned row
+    holds them (the oracle walks the same keys in the same way)."""
+    import torch
+    _, _, _, _, _, (q, k, v) = _run(oracle, qm, dev, 1, 200, seed=19, with_cache=False)
+    bad = 137
+    v2 = v.copy()
+    v2[0, bad, :, 0::4] = 0x7f80         # +inf
+    v2[0, bad, :, 1::4] = 0x7fc0         # NaN
+    want = np.zeros((1, 200, 16, 128), dtype=np.uint16)
+    assert oracle.prefill_attention_causal(q, k, v2, want, None, None, 0, 1, 200, 16, 8, SCALE, 1, 16) == 0
+    wf = oracle.bf16_to_f32(want)
+    for kernel in (0, 1):
+        qm.set_option(qm.OPT_PREFILL_KERNEL, kernel)
+        try:
+            out = torch.zeros((1, 200, 16, 128), dtype=torch.int16, device=dev)
+            qm.prefill_attention_causal(to_dev(q, dev), to_dev(k, dev), to_dev(v2, dev), out, None, None, 0, 1, 200, 16, 8)
+            torch.cuda.synchronize()
+        finally:
+            qm.set_option(qm.OPT_PREFILL_KERNEL, 0)
+        gf = oracle.bf16_to_f32(to_u16(out))
+        assert np.isfinite(gf[0, :bad]).all()
+        assert max_abs_err(oracle, to_u16(out)[0, :bad], want[0, :bad]) <= TOL
+        assert np.array_equal(np.isnan(gf[0, bad:]), np.isnan(wf[0, bad:]))
+        assert np.array_equal(np.isposinf(gf[0, bad:]), np.isposinf(wf[0, bad:]))
+        fin = np.isfinite(wf[0, bad:])
+        assert np.abs(gf[0, bad:][fin] - wf[0, bad:][fin]).max() <= TOL
 
 
 def test_prefill_rows_match_decode_over_written_cache(oracle, qm, dev):
