@@ -938,33 +938,52 @@ class PrefillChunk:
     position 2048 of one sequence over the reference's flat LayerCache, on the matrix cores or row by row."""
     bound = "mfma"
 
-    def __init__(self, qm, dev, seed=46, rows=256, before=2048, by_rows=False, split=True):
+    def __init__(self, qm, dev, seed=46, rows=256, before=2048, by_rows=False, split=True, paged=False, q_heads=16):
         import torch
-        self.qm, self.rows, self.before, self.by_rows = qm, rows, before, by_rows
-        self.name = "prefill_chunk_%d_rows_at_%d_flat_cache%s" % (rows, before, "_row_by_row" if by_rows else
-                                                                  "" if split else "_one_block_per_query_tile")
+        self.qm, self.rows, self.before, self.by_rows, self.paged, self.q_heads = qm, rows, before, by_rows, paged, q_heads
+        self.name = "prefill_chunk_%d_rows_at_%d_%s%s%s" % (
+            rows, before, "paged_cache" if paged else "flat_cache", "" if q_heads == 16 else "_%d_query_heads" % q_heads,
+            "_row_by_row" if by_rows else "" if split else "_one_block_per_query_tile")
         syn = Synthetic(dev, seed)
         self.max_cache = before + rows
-        self.q = syn.normal((rows, 16, 128))
+        self.q = syn.normal((rows, q_heads, 128))
         self.k, self.v = syn.normal((8, self.max_cache, 128)), syn.normal((8, self.max_cache, 128))
         self.out = torch.zeros_like(self.q)
-        self.cache = qm.flat_cache(self.k, self.v, 8, self.max_cache)
-        self.ws_bytes = qm.attention_rows_workspace_bytes(rows, 16, 8, self.max_cache) if by_rows else \
+        if paged:
+            # the same keys behind a shuffled page table: pool [n_pages, 8, 16, 128]
+            self.n_pages = (self.max_cache + 15) // 16
+            order = torch.randperm(self.n_pages, generator=torch.Generator().manual_seed(seed)).to(torch.int32)
+            pad = self.n_pages * 16 - self.max_cache
+            def pool_of(t):
+                t = torch.nn.functional.pad(t, (0, 0, 0, pad)).view(8, self.n_pages, 16, 128).permute(1, 0, 2, 3).contiguous()
+                pool = torch.empty_like(t)
+                pool[order.to(dev).long()] = t
+                return pool
+            self.k_pool, self.v_pool = pool_of(self.k), pool_of(self.v)
+            self.table = order.to(dev)
+            self.cache = qm.paged_cache(self.k_pool, self.v_pool, self.n_pages)
+        else:
+            self.cache = qm.flat_cache(self.k, self.v, 8, self.max_cache)
+        self.ws_bytes = qm.attention_rows_workspace_bytes(rows, q_heads, 8, self.max_cache) if by_rows else \
             qm.prefill_chunk_workspace_bytes(1, rows, before, 8) if split else 0
         self.ws = torch.empty(self.ws_bytes // 4 + 64, dtype=torch.float32, device=dev)
         keys = sum(before + i + 1 for i in range(rows))
-        self.flops = 16 * keys * 128 * 2 * 2
-        self.bytes = 2 * rows * 16 * 128 * 2 + 2 * self.max_cache * 8 * 128 * 2     # Q + O, K + V read once
+        self.flops = q_heads * keys * 128 * 2 * 2
+        self.bytes = 2 * rows * q_heads * 128 * 2 + 2 * self.max_cache * 8 * 128 * 2     # Q + O, K + V read once
 
     def step(self):
         import torch
         stream = torch.cuda.current_stream().cuda_stream
+        ws = self.ws if self.ws_bytes else None
         if self.by_rows:
-            self.qm.attention_rows(self.q, self.cache, None, 1, self.out, self.rows, self.before, 16, -1, SCALE, self.ws,
-                                   self.ws_bytes, None, stream)
+            self.qm.attention_rows(self.q, self.cache, self.table if self.paged else None, self.n_pages if self.paged else 1,
+                                   self.out, self.rows, self.before, self.q_heads, -1, SCALE, self.ws, self.ws_bytes, None, stream)
+        elif self.paged:
+            self.qm.prefill_attention_chunk_paged(self.q, self.cache, self.table, self.n_pages, self.out, 1, self.rows,
+                                                  self.before, self.q_heads, 8, SCALE, ws, self.ws_bytes, None, stream)
         else:
-            self.qm.prefill_attention_chunk(self.q, self.k, self.v, self.out, 1, self.rows, self.before, 16, 8, SCALE, stream,
-                                            (128, self.max_cache * 128, 0), self.ws if self.ws_bytes else None, self.ws_bytes)
+            self.qm.prefill_attention_chunk(self.q, self.k, self.v, self.out, 1, self.rows, self.before, self.q_heads, 8, SCALE,
+                                            stream, (128, self.max_cache * 128, 0), ws, self.ws_bytes)
 
     def cpu_baseline(self, oracle, threads):
         """Sample: the first 32 rows."""
@@ -972,8 +991,8 @@ class PrefillChunk:
         q, k, v = _bits(self.q[:n]).copy(), _bits(self.k).copy(), _bits(self.v).copy()
         out = np.zeros_like(q)
         t0 = time.perf_counter()
-        rc = oracle.attention(q, oracle.flat_cache(k, v, 8, self.max_cache), None, 1, out, n, self.before, 16, -1, SCALE,
-                              oracle.POLICY_ONLINE, threads)
+        rc = oracle.attention(q, oracle.flat_cache(k, v, 8, self.max_cache), None, 1, out, n, self.before, self.q_heads, -1,
+                              SCALE, oracle.POLICY_ONLINE, threads)
         dt = time.perf_counter() - t0
         assert rc == 0
         err = float(np.max(np.abs(oracle.bf16_to_f32(out).astype(np.float64)
@@ -1104,6 +1123,9 @@ def main():
                                       "qkv", "layer", "layer1", "layer2", "frame", "frame1", "linears", "linearsexact", "linears128", "linears128split", "generate"], default=None,
                     help="time just one of the other configurations and print its record (for profiling one "
                          "kernel under rocprofv3); the headline line is not produced")
+    ap.add_argument("--rows", default=None, metavar="TEXT",
+                    help="beside the headline, time exactly the rows whose name contains TEXT (cfg4c, paged, group_4 ...), "
+                         "default or not; the generation loop is left out")
     ap.add_argument("--layers", type=int, default=28,
                     help="with --only layer / layer1 / layer2: distinct weight sets and caches in rotation (a profiler that "
                          "records counters for every dispatch is spared most of the input generation with a small number)")
@@ -1192,6 +1214,11 @@ def main():
             ("cfg4c_prefill_chunk_256_rows_at_2048", lambda: PrefillChunk(qm, dev), False),
             ("cfg4c_prefill_chunk_256_rows_at_2048_one_block_per_query_tile", lambda: PrefillChunk(qm, dev, split=False), False),
             ("cfg4c_prefill_chunk_256_rows_at_2048_row_by_row", lambda: PrefillChunk(qm, dev, by_rows=True), False),
+            ("cfg4c_prefill_chunk_256_rows_at_2048_paged", lambda: PrefillChunk(qm, dev, paged=True), False),
+            ("cfg4c_prefill_chunk_256_rows_at_2048_paged_row_by_row", lambda: PrefillChunk(qm, dev, paged=True, by_rows=True), False),
+            ("cfg4c_prefill_chunk_256_rows_at_2048_group_1", lambda: PrefillChunk(qm, dev, q_heads=8), False),
+            ("cfg4c_prefill_chunk_256_rows_at_2048_group_4", lambda: PrefillChunk(qm, dev, q_heads=32), False),
+            ("cfg4c_prefill_chunk_256_rows_at_2048_group_4_paged", lambda: PrefillChunk(qm, dev, q_heads=32, paged=True), False),
             ("cfg5_predictor_loop", lambda: PredictorLoop(qm, dev), True),
             ("cfg5_predictor_loop_exact_chain", lambda: PredictorLoop(qm, dev, kernel=1), False),
             ("cfg5_predictor_loop_cache_writeback", lambda: PredictorLoop(qm, dev, write_cache=True), True),
@@ -1215,7 +1242,7 @@ def main():
             # the same fourteen steps as ONE launch of 256 resident blocks (same codes bit for bit)
             ("next_predictor_frame_m1_steps_one_launch", lambda: PredictorFrameSteps(qm, dev, one_launch=True), True),
         ]
-        extra = [(key, make) for key, make, default in rows if default or args.all]
+        extra = [(key, make) for key, make, default in rows if (args.rows in key if args.rows else default or args.all)]
         for key, make in extra:
             w = make()
             r = _report(w, _time_steps(w.step, max(args.steps, 100), max(args.warmup, 10)))
@@ -1249,7 +1276,8 @@ def main():
         # the generation loop end to end on a synthetic checkpoint of the real size (3.2 GB written to a temporary
         # directory): skipped, with the reason, where that cannot be written
         try:
-            per_config["next_generate_end_to_end"] = generate_end_to_end(qm, dev)
+            if not args.rows:
+                per_config["next_generate_end_to_end"] = generate_end_to_end(qm, dev)
         except OSError as e:
             per_config["next_generate_end_to_end"] = {"skipped": "%s: %s" % (type(e).__name__, e)}
 

@@ -358,13 +358,16 @@ int32_t qm_prefill_attention_causal_split(
  * cache_before + rows keys of every batch entry — those of the rows themselves included, as after
  * scatter_prefill_cache — addressed by element strides like qm_prefill_attention_causal's: the reference's LayerCache
  * [kv_head][max_cache][128] is read in place with (128, max_cache*128, 0); all zero selects contiguous
- * [batch][cache_before + rows][kv_heads][128].  Only q_heads == 2 * kv_heads, no sliding window, no page table
- * (qm_attention_rows below serves those).  Rounding as qm_prefill_attention_causal (bf16 scores before and after
+ * [batch][cache_before + rows][kv_heads][128].  q_heads / kv_heads = 1, 2 or 4 (the reference's generic kernel serves
+ * any integral group, R17:15780-15782: a wave's 32 matrix columns are 32 / group query rows x group heads, so that
+ * every K and V fragment serves all heads of the group; other groups: qm_attention_rows); no sliding window
+ * (qm_attention_rows).  qm_prefill_attention_chunk_paged below is the same operator over a paged cache.
+ * Rounding as qm_prefill_attention_causal (bf16 scores before and after
  * scaling unless QM_OPT_PREFILL_SCORE_ROUNDING is 0, fp32 online softmax, bf16 P; P = hi + lo where a query tile's
  * rows see fewer than 64 keys).  The uniform-waves kernel of qm_prefill_attention_causal with the query rows shifted:
- * for cache_before == 0 and no workspace it leaves that entry point's bits.
+ * for cache_before == 0, group 2 and no workspace it leaves that entry point's bits.
  * workspace (optional, 256-byte aligned; nothing to initialise): a chunk is few rows over many keys, so its grid of
- * batch * kv_heads * ceil(rows / 64) blocks can leave most compute units idle.  With a workspace of
+ * batch * kv_heads * ceil(rows / (128 / group)) blocks can leave most compute units idle.  With a workspace of
  * qm_prefill_chunk_workspace_bytes (for the current device; 0 when the shape would not split) the key tiles of a query
  * tile are handed to up to 16 blocks in runs of at least four, whose unnormalised results a second launch combines in
  * run order: results then differ from the unsplit call in the association of the sums only (within the operator's
@@ -377,6 +380,21 @@ int32_t qm_prefill_attention_chunk(
     int32_t batch, int32_t rows, int32_t cache_before, int32_t q_heads, int32_t kv_heads, float scale,
     int64_t kv_stride_token, int64_t kv_stride_head, int64_t kv_stride_batch,
     void* workspace, int64_t workspace_bytes,
+    void* hip_stream);
+/*
+ * The same operator over a PAGED cache (this library's native layout; the reference's cache is flat, so this has no
+ * counterpart there): the cache_before + rows keys of batch entry b — those of the rows themselves included, as after
+ * qm_scatter_kv — lie in `cache` at the pages page_table[b][0 ..] names (max_pages entries per batch entry; page_size a
+ * multiple of 16).  Same rounding, groups and workspace as qm_prefill_attention_chunk, and the same bits as that entry
+ * point gives for the same keys in a flat cache.  status_dev (optional): QM_STATUS_BAD_PAGE for a page-table entry
+ * outside the pool (read as page 0: nothing outside the pool is touched; the rows that see it are then wrong).
+ * More keys than max_pages pages hold: QM_ERR_SLOT_RANGE.
+ */
+int32_t qm_prefill_attention_chunk_paged(
+    const uint16_t* query, const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    uint16_t* context_out,
+    int32_t batch, int32_t rows, int32_t cache_before, int32_t q_heads, int32_t kv_heads, float scale,
+    void* workspace, int64_t workspace_bytes, uint32_t* status_dev,
     void* hip_stream);
 
 /*
@@ -392,8 +410,9 @@ int32_t qm_prefill_attention_chunk(
  * page_table [max_pages] of that sequence, or NULL for pages in pool order (the flat LayerCache).
  * Every row runs as one stream of the split-K decode kernels: row i carries the bits
  * qm_decode_attention gives for cache_before + i, and the rounding is that entry point's.  K and V are
- * read once per row (from the caches after the first): where they serve the shape (group 2, no window, keys
- * addressable by strides) qm_prefill_attention_causal and qm_prefill_attention_chunk are faster by an order of magnitude.
+ * read once per row (from the caches after the first): where they serve the shape (group 1, 2 or 4, no window)
+ * qm_prefill_attention_causal, qm_prefill_attention_chunk and qm_prefill_attention_chunk_paged are faster by an order
+ * of magnitude.
  * Workspace: qm_attention_rows_workspace_bytes(query_length, q_heads, kv_heads, cache_before + query_length).
  * query_length <= 65535.  status_dev (optional): QM_STATUS_BAD_PAGE for page-table entries out of range.
  */

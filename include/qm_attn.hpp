@@ -85,8 +85,9 @@ inline std::size_t attention_workspace_bytes(int q_heads, int kv_heads, int max_
 // ≙ NativeTalkerEngine::launch_attention (R17:17723-17814).  query_length == 1 is decode over
 // keys [key_start, cache_before + 1).  query_length > 1 attends the rows that scatter_prefill_cache has
 // already placed in the cache: with two query heads per kv head and no sliding window on the matrix cores (a whole
-// prompt from an empty cache, as in NativeTalkerEngine::prefill R17:16710-16717, or rows that continue a sequence);
-// every other case of the reference's generic kernel (a sliding window, another group) row by row.
+// prompt from an empty cache, as in NativeTalkerEngine::prefill R17:16710-16717, or rows that continue a sequence —
+// those also with one or four query heads per kv head); every other case of the reference's generic kernel (a sliding
+// window, another group) row by row.
 // The reference sizes dynamic LDS from the context; here the caller passes a workspace sized by
 // attention_workspace_bytes instead (the matrix-core cases need none).
 inline void launch_attention(
@@ -102,7 +103,8 @@ inline void launch_attention(
         return;
     }
     if (cache_before + query_length > max_cache) throw std::runtime_error("Talker prefill cache overflow.");
-    if (sliding_window <= 0 && q_heads == 2 * kv_heads && cache_before != 0) {
+    const bool matrix_group = q_heads == kv_heads || q_heads == 2 * kv_heads || q_heads == 4 * kv_heads;
+    if (sliding_window <= 0 && matrix_group && (cache_before != 0 || q_heads != 2 * kv_heads)) {
         // (the caller's workspace lets the keys be shared between blocks, if it is large enough for that)
         const std::int64_t split = qm_prefill_chunk_workspace_bytes(1, query_length, cache_before, kv_heads);
         const bool fits = split > 0 && workspace && static_cast<std::int64_t>(workspace_bytes) >= split
@@ -122,6 +124,35 @@ inline void launch_attention(
     check(qm_prefill_attention_causal(query, key_cache, value_cache, context, nullptr, nullptr, 0, 1,
                                       query_length, q_heads, kv_heads, scale, head_dim,
                                       static_cast<std::int64_t>(max_cache) * head_dim, 0, nullptr, stream),
+          "Talker generic fused attention launch");
+}
+
+// launch_attention over this library's paged cache (no counterpart in the reference, whose cache is flat): the same
+// choice between the decode kernels, the matrix cores and the row-by-row operator.
+inline void launch_attention_paged(
+    const std::uint16_t* query, const qm_kv_cache& cache, const std::int32_t* page_table, int max_pages,
+    std::uint16_t* context, int query_length, int cache_before,
+    int q_heads, int kv_heads, int sliding_window, float scale,
+    void* workspace, std::size_t workspace_bytes, std::uint32_t* status_dev, void* stream) {
+    if (query_length == 1) {
+        check(qm_decode_attention(query, &cache, page_table, max_pages, context, q_heads, cache_before, sliding_window,
+                                  scale, workspace, workspace_bytes, stream),
+              "Talker GQA M1 attention launch");
+        return;
+    }
+    const bool matrix_group = q_heads == kv_heads || q_heads == 2 * kv_heads || q_heads == 4 * kv_heads;
+    if (sliding_window <= 0 && matrix_group && page_table && cache.page_size % 16 == 0) {
+        const std::int64_t split = qm_prefill_chunk_workspace_bytes(1, query_length, cache_before, kv_heads);
+        const bool fits = split > 0 && workspace && static_cast<std::int64_t>(workspace_bytes) >= split
+                       && (reinterpret_cast<std::uintptr_t>(workspace) & 255) == 0;
+        check(qm_prefill_attention_chunk_paged(query, &cache, page_table, max_pages, context, 1, query_length, cache_before,
+                                               q_heads, kv_heads, scale, fits ? workspace : nullptr, fits ? split : 0,
+                                               status_dev, stream),
+              "Talker generic fused attention launch");
+        return;
+    }
+    check(qm_attention_rows(query, &cache, page_table, max_pages, context, query_length, cache_before, q_heads,
+                            sliding_window, scale, workspace, workspace_bytes, status_dev, stream),
           "Talker generic fused attention launch");
 }
 

@@ -102,6 +102,8 @@ _SIGNATURES = {
     "qm_prefill_chunk_workspace_bytes": (C.c_int64, [_I32, _I32, _I32, _I32]),
     "qm_prefill_attention_chunk": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _I32, _I32, _F32, C.c_int64, C.c_int64, C.c_int64,
                                           _PTR, C.c_int64, _PTR]),
+    "qm_prefill_attention_chunk_paged": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _I32, _I32, _I32, _F32,
+                                                _PTR, C.c_int64, _PTR, _PTR]),
     "qm_attention_rows_workspace_bytes": (C.c_size_t, [_I32, _I32, _I32, _I32]),
     "qm_attention_rows": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _I32, _I32, _F32,
                                  _PTR, C.c_size_t, _PTR, _PTR]),
@@ -286,6 +288,13 @@ def prefill_attention_chunk(query, key, value, out, batch, rows, cache_before, q
     _check(lib().qm_prefill_attention_chunk(
         _addr(query), _addr(key), _addr(value), _addr(out), batch, rows, cache_before, q_heads, kv_heads, scale,
         kv_strides[0], kv_strides[1], kv_strides[2], _addr(workspace), workspace_bytes, stream), "qm_prefill_attention_chunk")
+
+
+def prefill_attention_chunk_paged(query, cache, page_table, max_pages, out, batch, rows, cache_before, q_heads, kv_heads,
+                                  scale=SCALE_128, workspace=None, workspace_bytes=0, status=None, stream=0):
+    _check(lib().qm_prefill_attention_chunk_paged(
+        _addr(query), C.byref(cache), _addr(page_table), max_pages, _addr(out), batch, rows, cache_before, q_heads, kv_heads,
+        scale, _addr(workspace), workspace_bytes, _addr(status), stream), "qm_prefill_attention_chunk_paged")
 
 
 def attention_rows_workspace_bytes(query_length, q_heads, kv_heads, key_end):

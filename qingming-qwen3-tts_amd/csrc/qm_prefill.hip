@@ -104,6 +104,10 @@ struct PrefillParams {
     int chunk_parts;             // blocks per (pair, query tile) in the grid; 1: no split
     int chunk_run;
     float* chunk_records;        // [pair][query tile][part][kChunkRecordFloats]
+    // (chunk kernel) keys and values are read from a paged cache: page ids of batch entry b at chunk_table +
+    // b * pages.max_pages, the pool described by the kernel's qm_kv_cache argument; k and v are then unused
+    const int32_t* chunk_table;
+    int chunk_paged;
 };
 
 constexpr int kChunkRecordFloats = 66 * kPfThreads;   // per thread: 64 of O (unnormalised), the reference maximum, the sum
@@ -172,9 +176,10 @@ __device__ __forceinline__ void zero_non_finite(bf16x8_t& f) {
 // The products of the non-finite V elements of the 16 keys key0 .. key0 + 15, for the columns that see the key.
 // p_hi (+ p_lo): this lane's eight probabilities of the group as the MFMA takes them (element i = key
 // 8 (i / 4) + 4 grp + i % 4 of the group; the lane of the other half of the wave holds the other eight).
-// v_head: the V rows of this (batch, kv head); a lane's accumulators o[dt][4 rq + c] are dims 32 dt + 8 rq + 4 grp + c.
+// v_group: the V row of key key0 (the rows of the group follow at stride_token elements); a lane's accumulators
+// o[dt][4 rq + c] are dims 32 dt + 8 rq + 4 grp + c.
 template <bool TWO_PARTS>
-__device__ __forceinline__ void add_non_finite_products(f32x16_t (&o)[4], uint4 p_hi, uint4 p_lo, const uint16_t* v_head,
+__device__ __forceinline__ void add_non_finite_products(f32x16_t (&o)[4], uint4 p_hi, uint4 p_lo, const uint16_t* v_group,
                                                         int64_t stride_token, int key0, int key_count, int my_pos, int grp) {
 #pragma unroll 1
     for (int jj = 0; jj < 16; ++jj) {
@@ -193,7 +198,7 @@ __device__ __forceinline__ void add_non_finite_products(f32x16_t (&o)[4], uint4 
         // (after the swap the first word is the lower half's value in both halves, the second the upper half's)
         const float prob = __uint_as_float(owner == 0 ? both[0] : both[1]);
         if (key > my_pos) continue;                        // this column does not see the key (per lane)
-        const uint16_t* row = v_head + static_cast<int64_t>(key) * stride_token + 4 * grp;
+        const uint16_t* row = v_group + static_cast<int64_t>(jj) * stride_token + 4 * grp;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) {
 #pragma unroll
@@ -217,9 +222,16 @@ template <int N> using int_c = std::integral_constant<int, N>;
 template <bool B> using bool_c = std::integral_constant<bool, B>;
 
 // CHUNK: the query rows stand at positions cache_before + row (prefill_chunk_kernel); otherwise at their row.
-template <bool PRECISE, bool ROUND, bool CHUNK = false>
+// G: query heads per kv head (the GQA group; 1, 2 or 4).  A wave's 32 MFMA columns are 32 / G query rows x G heads,
+// so every K and V fragment serves all G heads, and a block is 4 x 32 / G query rows.  The whole-prompt kernels are
+// built for G = 2 only (their query tiles are as long as a key tile); the chunk kernel for 1, 2 and 4.
+template <bool PRECISE, bool ROUND, bool CHUNK = false, int G = 2>
 __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_kv_cache& cache,
                                              unsigned char* pf_smem, int qt, int pair, int part = 0) {
+    static_assert(G == 1 || G == 2 || G == 4, "the GQA group the MFMA columns are dealt for");
+    static_assert(CHUNK || G == 2, "the whole-prompt kernels index key tiles by query tiles of the same length");
+    constexpr int R = 32 / G;            // query rows of a wave
+    constexpr int BM = 4 * R;            // query rows of a block
     PfStage* st = reinterpret_cast<PfStage*>(pf_smem);
 
     const int tid = threadIdx.x;
@@ -233,13 +245,13 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     const int S = prm.seq;
     const int SK = CHUNK ? prm.key_count : S;        // keys that k and v hold
     const int shift = CHUNK ? prm.cache_before : 0;  // position of query row 0
-    const int q_heads = 2 * prm.kv_heads;
+    const int q_heads = G * prm.kv_heads;
 
-    const int q0 = qt * kBM;
-    const int my_row = q0 + 16 * wave + (col & 15);   // query row of this lane's column
+    const int q0 = qt * BM;
+    const int my_row = q0 + R * wave + (col % R);     // query row of this lane's column
     const int my_pos = my_row + shift;                // the last key it attends
-    const int my_head = 2 * kvh + (col >> 4);
-    const int wave_last_row = q0 + 16 * wave + 15 + shift;   // as a position
+    const int my_head = G * kvh + col / R;
+    const int wave_last_row = q0 + R * wave + R - 1 + shift;   // as a position
 
     // ---- Q fragments (B operand): dims 16*kb + 8*grp .. +7 of this lane's column ----------------
     bf16x8_t qf[8];
@@ -287,9 +299,62 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     const uint16_t* v_src = prm.v + kv_base + 8 * v_dc;
     const uint32_t k_lane_off = static_cast<uint32_t>((tid >> 4) * kv_row32);
     const uint32_t v_lane_off = static_cast<uint32_t>(4 * v_kg * kv_row32);
+    // (chunk kernel over a paged cache) where key `key` of this (batch, kv head) lies in the pool: its page's entry of
+    // the batch entry's table, then page, head and token strides.  An entry outside the pool is flagged and read as
+    // page 0, so that nothing outside the pool is touched.
+    uint32_t chunk_page_err = 0;
+    auto paged_offset = [&](int key) -> int64_t {
+        const int page = page_of(prm.pages, key);
+        int phys = prm.chunk_table[static_cast<int64_t>(b) * prm.pages.max_pages + page];
+        if (phys < 0 || phys >= cache.n_pages) {
+            chunk_page_err |= QM_STATUS_BAD_PAGE;
+            phys = 0;
+        }
+        return static_cast<int64_t>(phys) * cache.stride_page + static_cast<int64_t>(kvh) * cache.stride_head
+             + static_cast<int64_t>(key - page * prm.pages.page_size) * kDim;
+    };
+    // The four 16-key groups of a 64-key tile lie in four pages at most (a page holds a multiple of 16 keys), and
+    // which pages is the same for every lane: four table entries per tile, asked for a tile ahead so that the tile's
+    // own loads do not wait for them.  (A group at or beyond the keys there are names the page of the last key.)
+    int ne0 = 0, ne1 = 0, ne2 = 0, ne3 = 0, ne_tile = -1;
+    auto group_page = [&](int key) -> int { return page_of(prm.pages, min(key, SK - 1)); };
+    auto fetch_tile_entries = [&](int tile) {
+        const int32_t* tab = prm.chunk_table + static_cast<int64_t>(b) * prm.pages.max_pages;
+        ne0 = tab[group_page(tile * kBN)];
+        ne1 = tab[group_page(tile * kBN + 16)];
+        ne2 = tab[group_page(tile * kBN + 32)];
+        ne3 = tab[group_page(tile * kBN + 48)];
+        ne_tile = tile;
+    };
+    auto checked_entry = [&](int phys) -> int {
+        if (phys < 0 || phys >= cache.n_pages) {
+            chunk_page_err |= QM_STATUS_BAD_PAGE;
+            phys = 0;
+        }
+        return phys;
+    };
     auto load_tile = [&](int tile) {
         const int key0 = tile * kBN;
-        if (key0 + kBN <= SK) {
+        if (CHUNK && prm.chunk_paged) {
+            if (ne_tile != tile) fetch_tile_entries(tile);
+            const int e0 = checked_entry(ne0), e1 = checked_entry(ne1), e2 = checked_entry(ne2), e3 = checked_entry(ne3);
+            const int64_t head_off = static_cast<int64_t>(kvh) * cache.stride_head;
+            // (a key at or beyond the keys there are is redirected to the last key, as below)
+            const int vg = v_kg >> 2;                       // the 16-key group of this lane's four V rows
+            const int ve = vg == 0 ? e0 : vg == 1 ? e1 : vg == 2 ? e2 : e3;
+            const int v_first = group_page(key0 + 16 * vg) * prm.pages.page_size;
+            const uint16_t* v_page = cache.v_pool + (static_cast<int64_t>(ve) * cache.stride_page + head_off) + 8 * v_dc;
+            each_stage([&](uint4& kk, uint4& vv, int i) {
+                const int e = i == 0 ? e0 : i == 1 ? e1 : i == 2 ? e2 : e3;
+                const int key = min(key0 + (tid >> 4) + 16 * i, SK - 1);
+                const int k_first = group_page(key0 + 16 * i) * prm.pages.page_size;
+                kk = *reinterpret_cast<const uint4*>(cache.k_pool + (static_cast<int64_t>(e) * cache.stride_page + head_off)
+                                                     + (key - k_first) * kDim + 8 * (tid & 15));
+                const int vkey = min(key0 + 4 * v_kg + i, SK - 1);
+                vv = *reinterpret_cast<const uint4*>(v_page + (vkey - v_first) * kDim);
+            });
+            fetch_tile_entries(tile + 1);
+        } else if (key0 + kBN <= SK) {
             const uint16_t* kt = k_src + static_cast<uint32_t>(key0 * kv_row32);
             const uint16_t* vt = v_src + static_cast<uint32_t>(key0 * kv_row32);
             each_stage([&](uint4& kk, uint4& vv, int i) {
@@ -429,12 +494,17 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
             bf16x8_t v0 = vf[4 * kg], v1 = vf[4 * kg + 1], v2 = vf[4 * kg + 2], v3 = vf[4 * kg + 3];
             // (a group the mask cuts for some column of the wave — its last key lies after the wave's first row, or
             // beyond the keys there are — with a non-finite V: see add_non_finite_products)
-            if (decltype(diag)::value && (key_base + 16 * kg + 15 > wave_last_row - 15 || key_base + 16 * kg + 15 >= SK)
+            if (decltype(diag)::value && (key_base + 16 * kg + 15 > wave_last_row - (R - 1) || key_base + 16 * kg + 15 >= SK)
                 && any_non_finite(v0, v1, v2, v3)) {
                 zero_non_finite(v0); zero_non_finite(v1); zero_non_finite(v2); zero_non_finite(v3);
+                // (a paged cache: the group's sixteen keys lie in one page, pages being multiples of sixteen tokens)
+                const int group_key = key_base + 16 * kg;
+                const bool paged = CHUNK && prm.chunk_paged;
+                const uint16_t* v_group = paged ? cache.v_pool + paged_offset(min(group_key, SK - 1))
+                                                : prm.v + kv_base + static_cast<int64_t>(group_key) * prm.kv_stride_token;
                 add_non_finite_products<PRECISE>(o, __builtin_bit_cast(uint4, p.hi[kg]),
                                                  PRECISE ? __builtin_bit_cast(uint4, p.lo[kg]) : make_uint4(0, 0, 0, 0),
-                                                 prm.v + kv_base, prm.kv_stride_token, key_base + 16 * kg, SK, my_pos, grp);
+                                                 v_group, paged ? kDim : prm.kv_stride_token, group_key, SK, my_pos, grp);
             }
             o[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, p.hi[kg], o[0], 0, 0, 0);
             if (PRECISE) o[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, p.lo[kg], o[0], 0, 0, 0);
@@ -543,7 +613,7 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
         // Key tiles every row of the query tile sees whole, then the one or two that the causal mask cuts
         // (two when the tile's first position is not a multiple of 64); the last tile always takes the masked
         // path, where keys beyond key_count go.  With a key split this block takes one run of them.
-        const int last_tile = min(q0 + shift + kBM - 1, SK - 1) / kBN;
+        const int last_tile = min(q0 + shift + BM - 1, SK - 1) / kBN;
         const int whole = PRECISE ? 0 : min((q0 + shift + 1) / kBN, last_tile);
         int t_first = 0, t_last = last_tile;
         if (!PRECISE && prm.chunk_parts > 1) {
@@ -591,6 +661,7 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     }
     __syncthreads();   // the stages become the output staging area
 
+    if (CHUNK && chunk_page_err && prm.status) atomicOr(prm.status, chunk_page_err);
     const float l_tot = halves_sum(l_run);
     if (CHUNK && !PRECISE && to_record) {
         // One run of several: the unnormalised O, the reference maximum and the sum, as register images (thread t of
@@ -626,8 +697,8 @@ __device__ __forceinline__ void prefill_body(const PrefillParams& prm, const qm_
     for (int it = 0; it < 8; ++it) {
         const int c = 4 * it + (lane >> 4);
         const int chunk = lane & 15;
-        const int row = q0 + 16 * wave + (c & 15);
-        const int head = 2 * kvh + (c >> 4);
+        const int row = q0 + R * wave + (c % R);
+        const int head = G * kvh + c / R;
         if (row < S) {
             const uint4 val = *reinterpret_cast<const uint4*>(&stage[c * kOS + 8 * chunk]);
             *reinterpret_cast<uint4*>(prm.out + ((static_cast<int64_t>(b) * S + row) * q_heads + head) * kDim + 8 * chunk) = val;
@@ -655,7 +726,9 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_causal_kernel(PrefillPa
 // The rows of a sequence continued at position cache_before (R17:17782-17813 with cache_before > 0), over keys
 // and values read in place: grid and blocks as above.  A query tile none of whose rows sees a whole key tile takes
 // the split-precision P path (rows with few keys).
-template <bool ROUND>
+// G query heads per kv head (1, 2 or 4): a block is 128 / G query rows.  Keys and values by strides, or (chunk_paged)
+// from the paged cache `cache` through the page table.
+template <bool ROUND, int G>
 __global__ __launch_bounds__(kPfThreads, 2) void prefill_chunk_kernel(PrefillParams prm, qm_kv_cache cache) {
     extern __shared__ __attribute__((aligned(16))) unsigned char pf_smem[];
     const int pairs = prm.batch * prm.kv_heads;
@@ -664,10 +737,10 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_chunk_kernel(PrefillPar
     const int qt = prm.n_qtiles - 1 - group / prm.chunk_parts;
     const int part = group % prm.chunk_parts;
     const int pair = bid % pairs;
-    if ((qt * kBM + prm.cache_before + 1) / kBN == 0) {
-        if (part == 0) prefill_body<true, ROUND, true>(prm, cache, pf_smem, qt, pair);
+    if ((qt * (128 / G) + prm.cache_before + 1) / kBN == 0) {
+        if (part == 0) prefill_body<true, ROUND, true, G>(prm, cache, pf_smem, qt, pair);
     } else {
-        prefill_body<false, ROUND, true>(prm, cache, pf_smem, qt, pair, part);
+        prefill_body<false, ROUND, true, G>(prm, cache, pf_smem, qt, pair, part);
     }
 }
 
@@ -677,13 +750,14 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_chunk_kernel(PrefillPar
 // thread's 64 values, all runs' loads in flight at once.
 constexpr int kChunkMaxRuns = 16;
 constexpr int kChunkMergeSlices = 8;
-__global__ __launch_bounds__(kPfThreads) void prefill_chunk_merge_kernel(PrefillParams prm, int round_scores) {
+__global__ __launch_bounds__(kPfThreads) void prefill_chunk_merge_kernel(PrefillParams prm, int round_scores, int gqa_group) {
     const int slice = blockIdx.x % kChunkMergeSlices;
     const int item = blockIdx.x / kChunkMergeSlices;
     const int pair = item % (prm.batch * prm.kv_heads);
     const int qt = item / (prm.batch * prm.kv_heads);
-    const int q0 = qt * kBM;
-    const int last_tile = min(q0 + prm.cache_before + kBM - 1, prm.key_count - 1) / kBN;
+    const int wave_rows = 32 / gqa_group, block_rows = 4 * wave_rows;
+    const int q0 = qt * block_rows;
+    const int last_tile = min(q0 + prm.cache_before + block_rows - 1, prm.key_count - 1) / kBN;
     const int runs = last_tile / prm.chunk_run + 1;
     if (runs == 1) return;                               // its one block has written the rows itself
     const int tid = threadIdx.x;
@@ -714,9 +788,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_chunk_merge_kernel(Prefill
     }
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
     const int b = pair / prm.kv_heads, kvh = pair % prm.kv_heads;
-    const int row = q0 + 16 * wave + (col & 15);
+    const int row = q0 + wave_rows * wave + col % wave_rows;
     if (row >= prm.seq) return;
-    uint16_t* out = prm.out + ((static_cast<int64_t>(b) * prm.seq + row) * (2 * prm.kv_heads) + 2 * kvh + (col >> 4)) * kDim;
+    uint16_t* out = prm.out + ((static_cast<int64_t>(b) * prm.seq + row) * (gqa_group * prm.kv_heads) + gqa_group * kvh + col / wave_rows) * kDim;
     // value 16 dt + 4 rq + j of a thread is dim 32 dt + 8 rq + 4 grp + j: this slice is dt = slice / 2, rq = 2 (slice % 2), + 1
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
@@ -1452,7 +1526,8 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
             bf16x8_t v0 = vf[4 * kg], v1 = vf[4 * kg + 1], v2 = vf[4 * kg + 2], v3 = vf[4 * kg + 3];
             if ((key_base + 16 * kg + 15 > group_row0(c) || key_base + 16 * kg + 15 >= S) && any_non_finite(v0, v1, v2, v3)) {
                 zero_non_finite(v0); zero_non_finite(v1); zero_non_finite(v2); zero_non_finite(v3);
-                add_non_finite_products<false>(o[c], __builtin_bit_cast(uint4, p.g[kg]), make_uint4(0, 0, 0, 0), prm.v + kv_base,
+                add_non_finite_products<false>(o[c], __builtin_bit_cast(uint4, p.g[kg]), make_uint4(0, 0, 0, 0),
+                                               prm.v + kv_base + static_cast<int64_t>(key_base + 16 * kg) * prm.kv_stride_token,
                                                prm.kv_stride_token, key_base + 16 * kg, S, group_row0(c) + (col & 15), grp);
             }
             o[c][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, p.g[kg], o[c][0], 0, 0, 0);
@@ -1906,9 +1981,10 @@ struct ChunkPlan {
     int64_t bytes = 0;   // records
 };
 
-static ChunkPlan plan_chunk(int64_t pairs, int rows, int cache_before, int compute_units) {
+static ChunkPlan plan_chunk(int64_t pairs, int rows, int cache_before, int compute_units, int gqa_group) {
     ChunkPlan plan;
-    const int n_qtiles = (rows + kBM - 1) / kBM;
+    const int block_rows = 128 / gqa_group;
+    const int n_qtiles = (rows + block_rows - 1) / block_rows;
     const int64_t blocks = pairs * n_qtiles;
     const int tiles = (cache_before + rows - 1) / kBN + 1;      // of the last query tile
     int64_t parts = (compute_units + blocks - 1) / blocks;
@@ -1921,6 +1997,61 @@ static ChunkPlan plan_chunk(int64_t pairs, int rows, int cache_before, int compu
     return plan;
 }
 
+static bool chunk_group_served(int32_t q_heads, int32_t kv_heads) {
+    return kv_heads > 0 && (q_heads == kv_heads || q_heads == 2 * kv_heads || q_heads == 4 * kv_heads);
+}
+
+template <int G>
+static int32_t launch_chunk_kernels(const PrefillParams& prm, const qm_kv_cache& cache, bool round_scores, int64_t pairs, hipStream_t s) {
+    const size_t smem = sizeof(PfStage) * kPfStages;
+    const auto kernel = round_scores ? prefill_chunk_kernel<true, G> : prefill_chunk_kernel<false, G>;
+    static std::atomic<bool> lds_raised[2][kMaxDevices];
+    const int32_t rc_lds = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), static_cast<int>(smem),
+                                              lds_raised[round_scores ? 1 : 0]);
+    if (rc_lds != QM_OK) return rc_lds;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(pairs * prm.n_qtiles * prm.chunk_parts)), dim3(kPfThreads), smem, s, prm, cache);
+    int32_t rc = launch_status();
+    if (rc == QM_OK && prm.chunk_parts > 1) {
+        hipLaunchKernelGGL(prefill_chunk_merge_kernel, dim3(static_cast<unsigned>(pairs * prm.n_qtiles * kChunkMergeSlices)), dim3(kPfThreads), 0, s,
+                           prm, round_scores ? 1 : 0, G);
+        rc = launch_status();
+    }
+    return rc;
+}
+
+// What the two chunk entry points share once the keys' addressing is settled in `prm` / `cache`.
+static int32_t chunk_entry(PrefillParams& prm, const qm_kv_cache& cache, int32_t batch, int32_t rows, int32_t cache_before,
+                           int32_t q_heads, int32_t kv_heads, float scale, void* workspace, int64_t workspace_bytes, void* hip_stream) {
+    const int gqa_group = q_heads / kv_heads;
+    const int block_rows = 128 / gqa_group;
+    const int n_qtiles = (rows + block_rows - 1) / block_rows;
+    const int64_t pairs = static_cast<int64_t>(batch) * kv_heads;
+    if (pairs * n_qtiles * 16 > 0x7fffffffLL) return QM_ERR_ARGUMENT;
+    prm.batch = batch; prm.seq = rows; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
+    prm.heavy_groups = n_qtiles;
+    prm.dealt_pages = 0;
+    prm.cache_before = cache_before; prm.key_count = cache_before + rows;
+    prm.chunk_parts = 1;
+    if (workspace) {
+        int compute_units = 0;
+        const int32_t rc_cu = device_compute_units(&compute_units);
+        if (rc_cu != QM_OK) return rc_cu;
+        const ChunkPlan plan = plan_chunk(pairs, rows, cache_before, compute_units, gqa_group);
+        if (plan.parts > 1) {
+            if (workspace_bytes < plan.bytes) return QM_ERR_WORKSPACE;
+            prm.chunk_parts = plan.parts;
+            prm.chunk_run = plan.run;
+            prm.chunk_records = static_cast<float*>(workspace);
+        }
+    }
+    const bool round_scores = option_value(QM_OPT_PREFILL_SCORE_ROUNDING) != 0;
+    if (!round_scores && !(scale > 0.0f)) return QM_ERR_ARGUMENT;   // the scale is folded into the exponent there
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    if (gqa_group == 1) return launch_chunk_kernels<1>(prm, cache, round_scores, pairs, s);
+    if (gqa_group == 2) return launch_chunk_kernels<2>(prm, cache, round_scores, pairs, s);
+    return launch_chunk_kernels<4>(prm, cache, round_scores, pairs, s);
+}
+
 }  // namespace qm
 
 extern "C" int64_t qm_prefill_chunk_workspace_bytes(int32_t batch, int32_t rows, int32_t cache_before, int32_t kv_heads) {
@@ -1930,7 +2061,11 @@ extern "C" int64_t qm_prefill_chunk_workspace_bytes(int32_t batch, int32_t rows,
     int compute_units = 0;
     const int32_t rc = device_compute_units(&compute_units);
     if (rc != QM_OK) return rc;
-    return plan_chunk(static_cast<int64_t>(batch) * kv_heads, rows, cache_before, compute_units).bytes;
+    // (enough for any of the groups served: the smaller the group, the fewer and longer the query tiles)
+    int64_t bytes = 0;
+    for (int g = 1; g <= 4; g *= 2)
+        bytes = std::max(bytes, plan_chunk(static_cast<int64_t>(batch) * kv_heads, rows, cache_before, compute_units, g).bytes);
+    return bytes;
 }
 
 extern "C" int32_t qm_prefill_attention_chunk(
@@ -1955,53 +2090,44 @@ extern "C" int32_t qm_prefill_attention_chunk(
         return QM_ERR_GEOMETRY;
     if (key_count * kv_stride_token >= (1LL << 31)) return QM_ERR_ARGUMENT;
     if (!query || !key || !value || !context_out) return QM_ERR_NULL;
-    if (kv_heads <= 0 || q_heads != 2 * kv_heads) return QM_ERR_GEOMETRY;   // GQA pair on the MFMA columns
+    if (!chunk_group_served(q_heads, kv_heads)) return QM_ERR_GEOMETRY;     // 32 / G query rows x G heads on the MFMA columns
     const uintptr_t align = reinterpret_cast<uintptr_t>(query) | reinterpret_cast<uintptr_t>(key)
                           | reinterpret_cast<uintptr_t>(value) | reinterpret_cast<uintptr_t>(context_out);
     if (align & 15) return QM_ERR_GEOMETRY;
     if (batch == 0 || rows == 0) return QM_OK;
-    const int n_qtiles = (rows + kBM - 1) / kBM;
-    const int64_t pairs = static_cast<int64_t>(batch) * kv_heads;
-    if (pairs * n_qtiles * 16 > 0x7fffffffLL) return QM_ERR_ARGUMENT;
-
     PrefillParams prm = {};
     prm.q = query; prm.k = key; prm.v = value; prm.out = context_out;
     prm.pages = make_page_map(16, 1);
     prm.kv_stride_token = kv_stride_token; prm.kv_stride_head = kv_stride_head; prm.kv_stride_batch = kv_stride_batch;
-    prm.batch = batch; prm.seq = rows; prm.kv_heads = kv_heads; prm.n_qtiles = n_qtiles; prm.scale = scale;
-    prm.heavy_groups = n_qtiles;
-    prm.dealt_pages = 0;
-    prm.cache_before = cache_before; prm.key_count = static_cast<int>(key_count);
-    prm.chunk_parts = 1;
-    if (workspace) {
-        int compute_units = 0;
-        const int32_t rc_cu = device_compute_units(&compute_units);
-        if (rc_cu != QM_OK) return rc_cu;
-        const ChunkPlan plan = plan_chunk(pairs, rows, cache_before, compute_units);
-        if (plan.parts > 1) {
-            if (workspace_bytes < plan.bytes) return QM_ERR_WORKSPACE;
-            prm.chunk_parts = plan.parts;
-            prm.chunk_run = plan.run;
-            prm.chunk_records = static_cast<float*>(workspace);
-        }
-    }
-
-    const bool round_scores = option_value(QM_OPT_PREFILL_SCORE_ROUNDING) != 0;
-    if (!round_scores && !(scale > 0.0f)) return QM_ERR_ARGUMENT;   // the scale is folded into the exponent there
-    const size_t smem = sizeof(PfStage) * kPfStages;
-    const auto kernel = round_scores ? prefill_chunk_kernel<true> : prefill_chunk_kernel<false>;
-    static std::atomic<bool> lds_raised[2][kMaxDevices];
-    const int32_t rc_lds = ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), static_cast<int>(smem),
-                                              lds_raised[round_scores ? 1 : 0]);
-    if (rc_lds != QM_OK) return rc_lds;
     const qm_kv_cache none = {};
-    hipStream_t s = static_cast<hipStream_t>(hip_stream);
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(pairs * n_qtiles * prm.chunk_parts)), dim3(kPfThreads), smem, s, prm, none);
-    int32_t rc = launch_status();
-    if (rc == QM_OK && prm.chunk_parts > 1) {
-        hipLaunchKernelGGL(prefill_chunk_merge_kernel, dim3(static_cast<unsigned>(pairs * n_qtiles * kChunkMergeSlices)), dim3(kPfThreads), 0, s, prm,
-                           round_scores ? 1 : 0);
-        rc = launch_status();
-    }
-    return rc;
+    return chunk_entry(prm, none, batch, rows, cache_before, q_heads, kv_heads, scale, workspace, workspace_bytes, hip_stream);
+}
+
+extern "C" int32_t qm_prefill_attention_chunk_paged(
+    const uint16_t* query, const qm_kv_cache* cache, const int32_t* page_table, int32_t max_pages,
+    uint16_t* context_out,
+    int32_t batch, int32_t rows, int32_t cache_before, int32_t q_heads, int32_t kv_heads, float scale,
+    void* workspace, int64_t workspace_bytes, uint32_t* status_dev,
+    void* hip_stream) {
+    using namespace qm;
+    if (batch < 0 || rows < 0 || cache_before < 0) return QM_ERR_ARGUMENT;
+    if (workspace_bytes < 0 || (workspace_bytes > 0 && !workspace)) return QM_ERR_ARGUMENT;
+    if (reinterpret_cast<uintptr_t>(workspace) & 255) return QM_ERR_GEOMETRY;
+    if (!query || !context_out || !page_table) return QM_ERR_NULL;
+    const int32_t rc = check_cache(cache, max_pages);
+    if (rc != QM_OK) return rc;
+    if (cache->kv_heads != kv_heads || !chunk_group_served(q_heads, kv_heads)) return QM_ERR_GEOMETRY;
+    if (cache->page_size % 16) return QM_ERR_GEOMETRY;              // a 16-key group lies in one page
+    const int64_t key_count = static_cast<int64_t>(cache_before) + rows;
+    if (key_count > cache_capacity(cache, max_pages) || key_count > INT32_MAX) return QM_ERR_SLOT_RANGE;
+    if ((reinterpret_cast<uintptr_t>(query) | reinterpret_cast<uintptr_t>(context_out)) & 15) return QM_ERR_GEOMETRY;
+    if (batch == 0 || rows == 0) return QM_OK;
+    PrefillParams prm = {};
+    prm.q = query; prm.out = context_out;
+    prm.k = cache->k_pool; prm.v = cache->v_pool;                   // (not read: the tiles come through the page table)
+    prm.pages = make_page_map(cache->page_size, max_pages);
+    prm.kv_stride_token = kDim; prm.kv_stride_head = 0; prm.kv_stride_batch = 0;
+    prm.chunk_table = page_table; prm.chunk_paged = 1;
+    prm.status = status_dev;
+    return chunk_entry(prm, *cache, batch, rows, cache_before, q_heads, kv_heads, scale, workspace, workspace_bytes, hip_stream);
 }

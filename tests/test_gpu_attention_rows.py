@@ -304,7 +304,7 @@ def test_chunk_with_the_keys_shared_between_blocks(oracle, qm, dev, rows, before
     assert _within(oracle, outs[0], got, tol=2e-3)         # against the unsplit call: one ulp, or 2e-3 near zero
     # too small a workspace is refused; a shape that would not split needs none
     assert qm.lib().qm_prefill_attention_chunk(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(), batch, rows, before, 16, 8,
-                                               SCALE, 128, max_cache * 128, 8 * max_cache * 128, ws.data_ptr(), nbytes - 4, None) == -4
+                                               SCALE, 128, max_cache * 128, 8 * max_cache * 128, ws.data_ptr(), 4096, None) == -4
     assert qm.prefill_chunk_workspace_bytes(32, 512, 64, 8) == 0
 
 
@@ -317,7 +317,7 @@ def test_chunk_argument_errors(qm, dev):
         q, p, p, p, 1, rows, before, heads, kv, SCALE, st[0], st[1], st[2], None, 0, None)
     assert call(0, 5) == 0
     assert call(-1, 0) == -5 and call(4, -1) == -5
-    assert call(4, 5, heads=8) == -2 and call(4, 5, st=(64, 128, 0)) == -2 and call(4, 5, st=(132, 128, 0)) == -2
+    assert call(4, 5, heads=24) == -2 and call(4, 5, st=(64, 128, 0)) == -2 and call(4, 5, st=(132, 128, 0)) == -2
     assert call(4, 5, q=p + 2) == -2
     assert call(4, 2 ** 24, st=(128, 2 ** 31, 0)) == -5           # keys beyond 32-bit element offsets
     assert qm.lib().qm_prefill_attention_chunk(None, p, p, p, 1, 4, 5, 16, 8, SCALE, 0, 0, 0, None, 0, None) == -1
@@ -341,3 +341,97 @@ def test_chunk_rows_never_see_the_keys_after_them(oracle, qm, dev, rows, before)
         qm.prefill_attention_chunk(qd, k2, v2, out, 1, rows, before, 16, 8, SCALE, kv_strides=strides)
         torch.cuda.synchronize()
         assert np.array_equal(to_u16(out)[0, :r + 1], got[0, :r + 1]), (r,)
+
+
+# ---- the chunk operator for GQA groups 1, 2 and 4, and over a paged cache ----
+
+def _chunk_any(oracle, qm, dev, rows, before, seed, q_heads, kv_heads, paged, split=False):
+    """Rows [before, before + rows) of one sequence, by qm_prefill_attention_chunk over a flat cache or by
+    qm_prefill_attention_chunk_paged over a PagedPool with a shuffled page table; the oracle's answers by policy."""
+    import torch
+    end = before + rows
+    q = oracle.normal_bf16((rows, q_heads, 128), seed)
+    out = torch.full((rows, q_heads, 128), 0x7fc0, dtype=torch.int16, device=dev)
+    want = {0: np.zeros_like(q), 1: np.zeros_like(q)}
+    nb = qm.prefill_chunk_workspace_bytes(1, rows, before, kv_heads) if split else 0
+    ws = torch.empty(nb // 4 + 64, dtype=torch.float32, device=dev) if nb else None
+    if paged:
+        pool = PagedPool(oracle, [end], seed + 1, kv_heads=kv_heads, extra_tokens=5)
+        desc = pool.descriptor(oracle)
+        for policy in (0, 1):
+            assert oracle.attention(q, desc, pool.page_table[0], pool.max_pages, want[policy], rows, before, q_heads, -1, SCALE,
+                                    policy, 8) == 0
+        kd, vd, cache_d, table_d = pool.device(qm, dev)
+        status = torch.zeros(1, dtype=torch.int32, device=dev)
+        qm.prefill_attention_chunk_paged(to_dev(q, dev), cache_d, table_d, pool.max_pages, out, 1, rows, before, q_heads, kv_heads,
+                                         SCALE, ws, nb, status)
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0
+    else:
+        max_cache = end + 3
+        kc = oracle.normal_bf16((kv_heads, max_cache, 128), seed + 1)
+        vc = oracle.normal_bf16((kv_heads, max_cache, 128), seed + 2)
+        kc[:, end:] = 0x7fc0
+        vc[:, end:] = 0x7fc0
+        for policy in (0, 1):
+            assert oracle.attention(q, oracle.flat_cache(kc, vc, kv_heads, max_cache), None, 1, want[policy], rows, before, q_heads,
+                                    -1, SCALE, policy, 8) == 0
+        qm.prefill_attention_chunk(to_dev(q, dev), to_dev(kc, dev), to_dev(vc, dev), out, 1, rows, before, q_heads, kv_heads, SCALE,
+                                   kv_strides=(128, max_cache * 128, 0), workspace=ws, workspace_bytes=nb)
+        torch.cuda.synchronize()
+    return to_u16(out), want
+
+
+@pytest.mark.parametrize("paged", [False, True], ids=["flat", "paged"])
+@pytest.mark.parametrize("q_heads,kv_heads", [(8, 8), (16, 8), (16, 4), (4, 4), (8, 2)])
+@pytest.mark.parametrize("rows,before", [(1, 0), (40, 0), (130, 0), (7, 15), (64, 63), (100, 100), (33, 128), (256, 37), (200, 700)])
+def test_chunk_for_groups_and_pages(oracle, qm, dev, rows, before, q_heads, kv_heads, paged):
+    got, want = _chunk_any(oracle, qm, dev, rows, before, 9000 + 13 * rows + before + q_heads, q_heads, kv_heads, paged)
+    assert _within(oracle, got, want[1])
+    first_long = max(0, 64 - before - 1)        # rows with at least 64 keys: also the reference chain with its bf16(P)
+    if first_long < rows:
+        assert max_abs_err(oracle, got[first_long:], want[0][first_long:]) <= TOL
+
+
+@pytest.mark.parametrize("q_heads,kv_heads", [(8, 8), (16, 8), (16, 4)])
+def test_paged_chunk_carries_the_bits_of_the_flat_one_and_shares_its_keys(oracle, qm, dev, q_heads, kv_heads):
+    """The same keys in a flat cache and behind a shuffled page table give the same bits, with and without the keys
+    shared between blocks (workspace); a page-table entry outside the pool is flagged."""
+    import torch
+    rows, before = 96, 1500
+    end = before + rows
+    pool = PagedPool(oracle, [end], 9900 + q_heads, kv_heads=kv_heads)
+    q = oracle.normal_bf16((rows, q_heads, 128), 9901)
+    # the same keys, flat
+    max_cache = end
+    kc = np.zeros((kv_heads, max_cache, 128), dtype=np.uint16)
+    vc = np.zeros_like(kc)
+    for t in range(end):
+        page, inside = pool.page_table[0, t // 16], t % 16
+        kc[:, t] = pool.k[page, :, inside]
+        vc[:, t] = pool.v[page, :, inside]
+    kd, vd, cache_d, table_d = pool.device(qm, dev)
+    for split in (False, True):
+        nb = qm.prefill_chunk_workspace_bytes(1, rows, before, kv_heads) if split else 0
+        assert (nb > 0) == split
+        ws = torch.empty(nb // 4 + 64, dtype=torch.float32, device=dev) if nb else None
+        flat = torch.zeros((rows, q_heads, 128), dtype=torch.int16, device=dev)
+        qm.prefill_attention_chunk(to_dev(q, dev), to_dev(kc, dev), to_dev(vc, dev), flat, 1, rows, before, q_heads, kv_heads, SCALE,
+                                   kv_strides=(128, max_cache * 128, 0), workspace=ws, workspace_bytes=nb)
+        paged = torch.zeros_like(flat)
+        status = torch.zeros(1, dtype=torch.int32, device=dev)
+        qm.prefill_attention_chunk_paged(to_dev(q, dev), cache_d, table_d, pool.max_pages, paged, 1, rows, before, q_heads, kv_heads,
+                                         SCALE, ws, nb, status)
+        torch.cuda.synchronize()
+        assert int(status.item()) == 0 and torch.equal(flat, paged), split
+    bad = pool.page_table.copy()
+    bad[0, 3] = pool.n_pages + 7
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    out = torch.zeros((rows, q_heads, 128), dtype=torch.int16, device=dev)
+    qm.prefill_attention_chunk_paged(to_dev(q, dev), cache_d, to_dev(bad, dev), pool.max_pages, out, 1, rows, before, q_heads, kv_heads,
+                                     SCALE, None, 0, status)
+    torch.cuda.synchronize()
+    assert int(status.item()) & 1          # QM_STATUS_BAD_PAGE
+    with pytest.raises(qm.QmError) as e:
+        qm.prefill_attention_chunk_paged(to_dev(q, dev), cache_d, table_d, 3, out, 1, rows, before, q_heads, kv_heads)
+    assert e.value.code == -3              # more keys than three pages hold
