@@ -9,13 +9,16 @@
 // A block of four waves owns 128 output columns x 128 token rows (waves 2 x 2, each 64 x 64 as 2 x 2 MFMA tiles) or, for
 // calls whose grid would leave CUs empty, x 64 token rows (waves 4 x 1, each 32 columns x 64 rows).  Both operands are
 // K-contiguous rows (x [m][k], w [n][k]), so one tile layout serves both: 64 k per step, a row of a tile is eight 16-byte
-// pieces in LDS, piece q of row r stored in slot q ^ (r % 8) so that the 32 rows a fragment read touches spread over all
-// banks.  An MFMA takes the weight rows as its A operand and the token rows as B (D = W X^T): a lane then holds, for one
+// pieces in LDS, piece q of row r stored in slot q ^ ((r / 2) % 8) so that the sixteen rows a fragment read touches in a
+// cycle spread over all 64 banks.  An MFMA takes the weight rows as its A operand and the token rows as B (D = W X^T): a lane then holds, for one
 // token row, runs of four consecutive output columns — 8-byte stores.
 // The tiles go from memory straight into a ring of LDS stages (global_load_lds, no registers, the swizzle chosen by which
-// piece a lane fetches), three steps ahead (two for the gate/up pair, whose stage is 48 KiB); a step begins by waiting
-// until its own stage has landed (vmcnt counts the later stages' pieces still in flight), one barrier, then the request
-// for the stage just freed.  The fragment reads are inline assembly: the compiler makes every LDS read of its own wait
+// piece a lane fetches), up to four steps ahead (three for the gate/up pair, whose stage is 48 KiB).  A step's one barrier
+// stands between the MFMAs of its last two k blocks, where a wave has read all it needs of the step's stage and waits
+// (vmcnt counts the later stages' pieces still in flight) for its own pieces of the next; the requests for the stage
+// just freed go out a piece at a time between the MFMAs that follow (issued in a bunch, the four waves' requests keep
+// the CU's address path and the waves busy for 700 cycles of a 1024-cycle step), and the next step's first fragments
+// are read behind the barrier while the last k block's MFMAs run.  The fragment reads are inline assembly: the compiler makes every LDS read of its own wait
 // for all global_load_lds in flight, which would expose the memory latency in every step.
 // Bound: bf16 MFMA (2.5 PFLOP/s); algorithmic flops 2 m n k (x 2 for the gate/up pair).
 
@@ -35,7 +38,9 @@ constexpr int kGmTileBytes = kGmTile * kGmStep * 2;   // 16 KiB per operand tile
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 // LDS byte offset of piece `piece` (16 bytes = 8 k) of row `row` inside a tile
-__device__ __forceinline__ int tile_slot(int row, int piece) { return (row * 8 + (piece ^ (row & 7))) * 16; }
+// (the LDS has 64 banks of four bytes: a row of 128 bytes covers half of them, which half by the row's parity, and the
+// sixteen lanes served in a cycle read sixteen consecutive rows: the eight rows of one parity take eight different slots)
+__device__ __forceinline__ int slot_key(int row) { return (row >> 1) & 7; }
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
@@ -45,12 +50,31 @@ __device__ __forceinline__ void gm_wait_vm() {
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-// One wave's pieces of a stage: piece i goes to LDS bytes [4096 i, 4096 i + 1024) from `first` (the wave's first piece).
-template <int N>
-__device__ __forceinline__ void gm_request(const uint16_t* const (&src)[N], int k0, unsigned char* first) {
-#pragma unroll
-    for (int i = 0; i < N; ++i)
-        __builtin_amdgcn_global_load_lds(src[i] + k0, (__attribute__((address_space(3))) void*)(first + 4096 * i), 16, 0, 0);
+// What follows the fp32 sums of two neighbouring output columns, as a packed bf16 pair.  Every rounding is one half of a
+// v_cvt_pk_bf16_f32 (round to nearest even, a NaN quieted with its payload kept: the bits f2bf gives for every fp32 input).
+// Linear: bf16(sum + bias), then bf16(residual + that) (linear_bf16 and add_bf16, R17:126-245, 8772-8790).
+__device__ __forceinline__ uint32_t finish_pair(float s0, float s1, bool has_bias, uint32_t bias, bool has_residual, uint32_t residual) {
+    if (has_bias) {
+        s0 += lo_bf16(bias);
+        s1 += hi_bf16(bias);
+    }
+    uint32_t v = pack_bf16_pair(s0, s1);
+    if (has_residual) v = pack_bf16_pair(lo_bf16(residual) + lo_bf16(v), hi_bf16(residual) + hi_bf16(v));
+    return v;
+}
+
+// Gate/up: swiglu_kernel (R17:8746-8770) on the rounded gate and up values.
+__device__ __forceinline__ uint32_t swiglu_pair(float g0, float g1, float u0, float u1) {
+    float gv0, gv1, uv0, uv1, a0, a1;
+    round_bf16_pair(g0, g1, gv0, gv1);
+    round_bf16_pair(u0, u1, uv0, uv1);
+    round_bf16_pair(gv0 / (1.0f + expf(-gv0)), gv1 / (1.0f + expf(-gv1)), a0, a1);
+    return pack_bf16_pair(a0 * uv0, a1 * uv1);
+}
+
+// 16 bytes per lane from `from` to LDS: lane l's land at `to` + 16 l
+__device__ __forceinline__ void gm_to_lds(const uint16_t* from, unsigned char* to) {
+    __builtin_amdgcn_global_load_lds(from, (__attribute__((address_space(3))) void*)to, 16, 0, 0);
 }
 
 template <bool DUAL, int BM>
@@ -66,7 +90,7 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
     constexpr int kPiecesX = kXBytes / 1024, kPiecesW = kGmTileBytes / 1024;
     constexpr int kPerWave = (kPiecesX + kWeights * kPiecesW) / 4;
     static_assert((kPiecesX + kWeights * kPiecesW) % 4 == 0, "pieces are dealt evenly to four waves");
-    static_assert(kPerWave * (kStages - 2) <= 63, "the wait counts the later stages' pieces");
+    static_assert(kPerWave * (kStages - 1) <= 63, "the waits count the later stages' pieces");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -79,7 +103,7 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
 
     // ---- this wave's pieces of a stage: instruction q = wave + 4 i covers LDS bytes [1024 q, 1024 q + 1024) of the
     // stage (x tile, then w, then up); its lane l fills slot l % 8 of tile row 8 (q within the tile) + l / 8 with
-    // global piece slot ^ (row % 8) ----
+    // global piece slot ^ slot_key(row) ----
     const uint16_t* src[kPerWave];
 #pragma unroll
     for (int i = 0; i < kPerWave; ++i) {
@@ -87,7 +111,7 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
         const int operand = q < kPiecesX ? 0 : (q < kPiecesX + kPiecesW ? 1 : 2);
         const int qt = q - (operand == 0 ? 0 : (operand == 1 ? kPiecesX : kPiecesX + kPiecesW));
         const int row = 8 * qt + (lane >> 3), slot = lane & 7;
-        const int piece = slot ^ (row & 7);
+        const int piece = slot ^ slot_key(row);
         if (operand == 0) {
             const int m = min(m0 + row, prm.rows - 1);            // rows past the end repeat the last one (never stored)
             src[i] = prm.input + static_cast<int64_t>(m) * K + 8 * piece;
@@ -98,9 +122,12 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
     // (a block takes piece blockIdx.z of the reduction: all of it unless the launch cut it)
     const int steps = K / kGmStep / prm.reduction_parts;
     const int first_step = static_cast<int>(blockIdx.z) * steps;
-    // (requests past the last step repeat it and land in a stage nobody reads again: the wait below counts pieces)
-#define QM_GM_REQUEST(step_)                                                                                             \
-    gm_request<kPerWave>(src, (first_step + min((step_), steps - 1)) * kGmStep, gm_smem + ((step_) % kStages) * kStageBytes + 1024 * wave)
+    // Piece `i` of this wave's pieces of step `step_`, into stage step_ % kStages.  (Requests past the last step repeat it
+    // and land in a stage nobody reads again: the wait before the barrier counts pieces.)
+    auto request_piece = [&](int step_, int i) __attribute__((always_inline)) {
+        const int k0 = (first_step + min(step_, steps - 1)) * kGmStep;
+        gm_to_lds(src[i] + k0, gm_smem + (step_ % kStages) * kStageBytes + 1024 * wave + 4096 * i);
+    };
 
     f32x16_t acc[kTn][kTm], acc_up[DUAL ? kTn : 1][DUAL ? kTm : 1];
 #pragma unroll
@@ -120,7 +147,7 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)gm_smem));
     uint32_t at_kb[4];                                            // byte offset inside a tile for each k block (row part included)
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) at_kb[kb] = static_cast<uint32_t>(frag_row * 128 + (((2 * kb + frag_half) ^ (frag_row & 7)) * 16));
+    for (int kb = 0; kb < 4; ++kb) at_kb[kb] = static_cast<uint32_t>(frag_row * 128 + (((2 * kb + frag_half) ^ slot_key(frag_row)) * 16));
     struct Frags {
         u32x4_t w[kTn], x[kTm], u[DUAL ? kTn : 1];
     };
@@ -152,7 +179,14 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
             asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(f.w[0]), "+v"(f.x[0]), "+v"(f.x[1]) : "n"(decltype(later)::value) : "memory");
         }
     };
-    auto multiply = [&](const Frags& f) __attribute__((always_inline)) {
+    // The MFMAs of one k block, with this wave's pieces [P0, P1) of step `req_step` requested between them: a request
+    // takes the CU's one address path about 16 cycles a piece (64 bytes a cycle), and issued in a bunch by four waves at
+    // once they leave the matrix cores idle for that long; between MFMAs they are issued in the shadow of the 32 cycles
+    // each MFMA takes.
+    constexpr int kMfmas = kTn * kTm * (DUAL ? 2 : 1);
+    auto multiply = [&](const Frags& f, int req_step, auto p0, auto p1) __attribute__((always_inline)) {
+        constexpr int P0 = decltype(p0)::value, P1 = decltype(p1)::value;
+        int done = 0, piece = P0;
 #pragma unroll
         for (int a = 0; a < kTn; ++a)
 #pragma unroll
@@ -162,32 +196,53 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
                 if (DUAL)
                     acc_up[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, f.u[a]),
                                                                            __builtin_bit_cast(bf16x8_t, f.x[b]), acc_up[a][b], 0, 0, 0);
+                done += DUAL ? 2 : 1;
+                // (as many pieces behind this MFMA as keep them evenly spread over the k block's MFMAs)
+                while (piece < P1 && (piece - P0 + 1) * kMfmas <= done * (P1 - P0)) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    request_piece(req_step, piece);
+                    __builtin_amdgcn_sched_barrier(0);
+                    ++piece;
+                }
             }
     };
+    using std::integral_constant;
+    constexpr int kQ1 = kPerWave / 4, kQ2 = kPerWave / 2, kQ3 = 3 * kPerWave / 4;
 
+    // A step's schedule.  The stage of step s is complete for everybody at the barrier of step s - 1; k blocks 0 and 1 of
+    // it are read right behind that barrier, while the MFMAs of the last k block of step s - 1 run.  The barrier of step s
+    // stands between the MFMAs of k blocks 2 and 3, at a point where this wave has read all it needs of stage s (its last
+    // reads have landed): behind it stage s is free, and the pieces of step s + kStages are requested into it, spread over
+    // the four k blocks that follow.  The wait in front of the barrier lets the pieces of the steps after s + 1 be in flight.
 #pragma unroll
-    for (int ahead = 0; ahead < kStages - 1; ++ahead) QM_GM_REQUEST(ahead);
+    for (int ahead = 0; ahead < kStages; ++ahead)
+#pragma unroll
+        for (int i = 0; i < (ahead == kStages - 1 ? kQ1 : kPerWave); ++i) request_piece(ahead, i);
+    gm_wait_vm<kPerWave * (kStages - 2) + kQ1>();
+    asm volatile("s_barrier" ::: "memory");
+    Frags f0, f1;
+    read_frags(f0, lds_base, 0);
+    read_frags(f1, lds_base, 1);
     for (int step = 0; step < steps; ++step) {
-        gm_wait_vm<kPerWave * (kStages - 2)>();                   // this wave's pieces of the step's stage have landed
-        asm volatile("s_barrier" ::: "memory");                   // everybody's have; and everybody is done with the stage before
-        QM_GM_REQUEST(step + kStages - 1);
         const uint32_t stage_at = lds_base + static_cast<uint32_t>((step % kStages) * kStageBytes);
-        Frags f0, f1;
-        read_frags(f0, stage_at, 0);
-        read_frags(f1, stage_at, 1);
-        arrived(f0, std::integral_constant<int, kReads>{});
-        multiply(f0);
+        const uint32_t next_at = lds_base + static_cast<uint32_t>(((step + 1) % kStages) * kStageBytes);
+        const int req = step - 1 + kStages;                       // (its first quarter went out behind the last barrier)
+        arrived(f0, integral_constant<int, kReads>{});
+        multiply(f0, req, integral_constant<int, kQ1>{}, integral_constant<int, kQ2>{});
         read_frags(f0, stage_at, 2);
-        arrived(f1, std::integral_constant<int, kReads>{});
-        multiply(f1);
+        arrived(f1, integral_constant<int, kReads>{});
+        multiply(f1, req, integral_constant<int, kQ2>{}, integral_constant<int, kQ3>{});
         read_frags(f1, stage_at, 3);
-        arrived(f0, std::integral_constant<int, kReads>{});
-        multiply(f0);
-        arrived(f1, std::integral_constant<int, 0>{});
-        multiply(f1);
+        arrived(f0, integral_constant<int, kReads>{});
+        multiply(f0, req, integral_constant<int, kQ3>{}, integral_constant<int, kPerWave>{});
+        arrived(f1, integral_constant<int, 0>{});
+        gm_wait_vm<kPerWave * (kStages - 2)>();                   // this wave's pieces of the next step's stage have landed
+        asm volatile("s_barrier" ::: "memory");                   // everybody's have; and everybody has read this step's stage
+        if (step + 1 < steps) read_frags(f0, next_at, 0);
+        multiply(f1, step + kStages, integral_constant<int, 0>{}, integral_constant<int, kQ1>{});
+        if (step + 1 < steps) read_frags(f1, next_at, 1);
     }
     gm_wait_vm<0>();                                              // (the requests past the last step, before the block's LDS goes)
-#undef QM_GM_REQUEST
 
     // ---- epilogue: accumulator register r of a lane is output column 8 (r / 4) + 4 (lane / 32) + r % 4 of the MFMA
     // tile's 32, token row lane % 32 ----
@@ -224,29 +279,22 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
             for (int g = 0; g < 4; ++g) {
                 if (!inside) break;
                 const int n = n0 + 32 * (kTn * wave_n + a) + 8 * g + 4 * (lane >> 5);
-                uint16_t bits[4];
                 uint2 res = make_uint2(0, 0);
                 if (!DUAL && prm.residual) res = *reinterpret_cast<const uint2*>(prm.residual + static_cast<int64_t>(m) * prm.columns + n);
                 uint2 bias = make_uint2(0, 0);
                 if (!DUAL && prm.bias) bias = *reinterpret_cast<const uint2*>(prm.bias + n);
+                uint32_t packed[2];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float sum = acc[a][b][4 * g + e];
+                for (int e = 0; e < 2; ++e) {
+                    const float s0 = acc[a][b][4 * g + 2 * e], s1 = acc[a][b][4 * g + 2 * e + 1];
                     if (DUAL) {
-                        // swiglu_kernel (R17:8746-8770) on the rounded gate and up values
-                        const float gv = bf2f(f2bf(sum));
-                        const uint16_t act = f2bf(gv / (1.0f + expf(-gv)));
-                        bits[e] = f2bf(bf2f(act) * bf2f(f2bf(acc_up[a][b][4 * g + e])));
+                        packed[e] = swiglu_pair(s0, s1, acc_up[a][b][4 * g + 2 * e], acc_up[a][b][4 * g + 2 * e + 1]);
                     } else {
-                        float r = sum;
-                        if (prm.bias) r += bf2f(static_cast<uint16_t>((e < 2 ? bias.x : bias.y) >> (16 * (e & 1))));
-                        uint16_t v = f2bf(r);
-                        if (prm.residual) v = f2bf(bf2f(static_cast<uint16_t>((e < 2 ? res.x : res.y) >> (16 * (e & 1)))) + bf2f(v));
-                        bits[e] = v;
+                        packed[e] = finish_pair(s0, s1, prm.bias != nullptr, e == 0 ? bias.x : bias.y, prm.residual != nullptr,
+                                                e == 0 ? res.x : res.y);
                     }
                 }
-                *reinterpret_cast<uint2*>(prm.output + static_cast<int64_t>(m) * prm.columns + n) =
-                    make_uint2(bits[0] | (static_cast<uint32_t>(bits[1]) << 16), bits[2] | (static_cast<uint32_t>(bits[3]) << 16));
+                *reinterpret_cast<uint2*>(prm.output + static_cast<int64_t>(m) * prm.columns + n) = make_uint2(packed[0], packed[1]);
             }
         }
     }
@@ -271,27 +319,18 @@ __global__ __launch_bounds__(256) void linear_rows_parts_kernel(LinearRowsParams
             up.x += u.x; up.y += u.y; up.z += u.z; up.w += u.w;
         }
     }
-    const float s4[4] = {sum.x, sum.y, sum.z, sum.w}, u4[4] = {up.x, up.y, up.z, up.w};
-    uint16_t bits[4];
     uint2 res = make_uint2(0, 0), bias = make_uint2(0, 0);
     if (!DUAL && prm.residual) res = *reinterpret_cast<const uint2*>(prm.residual + static_cast<int64_t>(m) * prm.columns + n);
     if (!DUAL && prm.bias) bias = *reinterpret_cast<const uint2*>(prm.bias + n);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        if (DUAL) {
-            const float gv = bf2f(f2bf(s4[e]));
-            const uint16_t act = f2bf(gv / (1.0f + expf(-gv)));
-            bits[e] = f2bf(bf2f(act) * bf2f(f2bf(u4[e])));
-        } else {
-            float r = s4[e];
-            if (prm.bias) r += bf2f(static_cast<uint16_t>((e < 2 ? bias.x : bias.y) >> (16 * (e & 1))));
-            uint16_t v = f2bf(r);
-            if (prm.residual) v = f2bf(bf2f(static_cast<uint16_t>((e < 2 ? res.x : res.y) >> (16 * (e & 1)))) + bf2f(v));
-            bits[e] = v;
-        }
+    uint2 packed;
+    if (DUAL) {
+        packed.x = swiglu_pair(sum.x, sum.y, up.x, up.y);
+        packed.y = swiglu_pair(sum.z, sum.w, up.z, up.w);
+    } else {
+        packed.x = finish_pair(sum.x, sum.y, prm.bias != nullptr, bias.x, prm.residual != nullptr, res.x);
+        packed.y = finish_pair(sum.z, sum.w, prm.bias != nullptr, bias.y, prm.residual != nullptr, res.y);
     }
-    *reinterpret_cast<uint2*>(prm.output + static_cast<int64_t>(m) * prm.columns + n) =
-        make_uint2(bits[0] | (static_cast<uint32_t>(bits[1]) << 16), bits[2] | (static_cast<uint32_t>(bits[3]) << 16));
+    *reinterpret_cast<uint2*>(prm.output + static_cast<int64_t>(m) * prm.columns + n) = packed;
 }
 
 template <bool DUAL, int BM>
