@@ -72,10 +72,45 @@ __device__ __forceinline__ uint32_t swiglu_pair(float g0, float g1, float u0, fl
     return pack_bf16_pair(a0 * uv0, a1 * uv1);
 }
 
-// 16 bytes per lane from `from` to LDS: lane l's land at `to` + 16 l
-__device__ __forceinline__ void gm_to_lds(const uint16_t* from, unsigned char* to) {
-    __builtin_amdgcn_global_load_lds(from, (__attribute__((address_space(3))) void*)to, 16, 0, 0);
-}
+// Where the side operations of a k block stand among its MFMAs.  The MFMAs of a k block run over the wave's tiles (a, b),
+// a the weight tile and b the token tile, b fastest, and for a gate/up pair the gate MFMA before the up MFMA; MFMA number i
+// is followed by slot i.  A matrix-core instruction takes 32 cycles and the wave issues in order, so whatever else the wave
+// has to issue (LDS reads, requests to memory) goes one or two to a slot, in the shadow of the MFMA before it.
+template <bool DUAL, int TN, int TM>
+struct GmSchedule {
+    static constexpr int kD = DUAL ? 2 : 1;
+    static constexpr int kMfmas = TN * TM * kD;
+    static constexpr int kReads = TN * kD + TM;                   // fragments (LDS reads) of a k block
+    // the slot behind the last MFMA that takes a fragment: from there on its registers can be read into again
+    static constexpr int w_slot(int a) { return (a * TM + TM - 1) * kD; }
+    static constexpr int u_slot(int a) { return (a * TM + TM - 1) * kD + 1; }
+    static constexpr int x_slot(int b) { return ((TN - 1) * TM + b) * kD + kD - 1; }
+    static constexpr int own_at(int slot) {
+        int n = 0;
+        for (int a = 0; a < TN; ++a) n += (w_slot(a) == slot) + (DUAL && u_slot(a) == slot);
+        for (int b = 0; b < TM; ++b) n += x_slot(b) == slot;
+        return n;
+    }
+    static constexpr int own_from(int slot) {
+        int n = 0;
+        for (int s = slot; s < kMfmas; ++s) n += own_at(s);
+        return n;
+    }
+    // the other buffer's fragments, read ahead of their k block: from slot 0 on, this many to a slot
+    static constexpr int kEarlyPerSlot = (kReads + kMfmas - 1) / kMfmas;
+    static constexpr int kLastEarlySlot = (kReads - 1) / kEarlyPerSlot;
+    // `pieces` requests over the slots: one more to a slot at a time, the slots with fewer reads of their own first
+    static constexpr int requests_at(int slot, int pieces) {
+        int given[kMfmas] = {};
+        for (int p = 0; p < pieces; ++p) {
+            int best = 0;
+            for (int s = 1; s < kMfmas; ++s)
+                if (own_at(s) + given[s] < own_at(best) + given[best]) best = s;
+            ++given[best];
+        }
+        return given[slot];
+    }
+};
 
 template <bool DUAL, int BM>
 __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRowsParams prm) {
@@ -86,11 +121,12 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
     constexpr int kStageBytes = kXBytes + kWeights * kGmTileBytes;
     constexpr int kTn = BM == 128 ? 2 : 1;                        // MFMA tiles of a wave along the output columns
     constexpr int kTm = 2;                                        // and along the token rows
+    using Schedule = GmSchedule<DUAL, kTn, kTm>;
     // pieces of 1 KiB (one instruction of a wave) per stage: x, w (, up); dealt to the four waves in turn
     constexpr int kPiecesX = kXBytes / 1024, kPiecesW = kGmTileBytes / 1024;
     constexpr int kPerWave = (kPiecesX + kWeights * kPiecesW) / 4;
-    static_assert((kPiecesX + kWeights * kPiecesW) % 4 == 0, "pieces are dealt evenly to four waves");
-    static_assert(kPerWave * (kStages - 1) <= 63, "the waits count the later stages' pieces");
+    static_assert(kPiecesX % 4 == 0 && kPiecesW % 4 == 0, "a wave's piece i is of the same operand in every wave");
+    static_assert(kPerWave * (kStages - 2) <= 63, "the waits count the later stages' pieces");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -103,30 +139,33 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
 
     // ---- this wave's pieces of a stage: instruction q = wave + 4 i covers LDS bytes [1024 q, 1024 q + 1024) of the
     // stage (x tile, then w, then up); its lane l fills slot l % 8 of tile row 8 (q within the tile) + l / 8 with
-    // global piece slot ^ slot_key(row) ----
-    const uint16_t* src[kPerWave];
-#pragma unroll
-    for (int i = 0; i < kPerWave; ++i) {
-        const int q = wave + 4 * i;
-        const int operand = q < kPiecesX ? 0 : (q < kPiecesX + kPiecesW ? 1 : 2);
-        const int qt = q - (operand == 0 ? 0 : (operand == 1 ? kPiecesX : kPiecesX + kPiecesW));
-        const int row = 8 * qt + (lane >> 3), slot = lane & 7;
-        const int piece = slot ^ slot_key(row);
-        if (operand == 0) {
-            const int m = min(m0 + row, prm.rows - 1);            // rows past the end repeat the last one (never stored)
-            src[i] = prm.input + static_cast<int64_t>(m) * K + 8 * piece;
-        } else {
-            src[i] = prm.weight[operand - 1] + static_cast<int64_t>(n0 + row) * K + 8 * piece;
-        }
-    }
+    // global piece slot ^ slot_key(row).  The tiles are read through buffer descriptors that begin at the block's first
+    // row of each operand: a lane's offset is the same for every piece (32 rows further on, the key of a row is the
+    // same), what changes from piece to piece and step to step is a scalar; token rows past the last are out of the
+    // descriptor's range and read as zero without touching memory (their results are never stored). ----
+    const uint32_t row_bytes = static_cast<uint32_t>(K) * 2u;
+    const int x_rows = min(prm.rows - m0, BM);
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(prm.input + static_cast<int64_t>(m0) * K), 0, static_cast<int>(x_rows * row_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(prm.weight[0] + static_cast<int64_t>(n0) * K), 0, static_cast<int>(kGmTile * row_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t u_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(prm.weight[DUAL ? 1 : 0] + static_cast<int64_t>(n0) * K), 0, static_cast<int>(kGmTile * row_bytes), 0x00020000);
+    const int lane_row = 8 * wave + (lane >> 3);
+    const uint32_t lane_off = static_cast<uint32_t>(lane_row) * row_bytes + 16u * static_cast<uint32_t>((lane & 7) ^ slot_key(lane_row));
     // (a block takes piece blockIdx.z of the reduction: all of it unless the launch cut it)
     const int steps = K / kGmStep / prm.reduction_parts;
     const int first_step = static_cast<int>(blockIdx.z) * steps;
     // Piece `i` of this wave's pieces of step `step_`, into stage step_ % kStages.  (Requests past the last step repeat it
     // and land in a stage nobody reads again: the wait before the barrier counts pieces.)
     auto request_piece = [&](int step_, int i) __attribute__((always_inline)) {
-        const int k0 = (first_step + min(step_, steps - 1)) * kGmStep;
-        gm_to_lds(src[i] + k0, gm_smem + (step_ % kStages) * kStageBytes + 1024 * wave + 4096 * i);
+        constexpr int kX = kPiecesX / 4, kW = kPiecesW / 4;
+        const int j = i < kX ? i : (i < kX + kW ? i - kX : i - kX - kW);                  // 32 rows further on per piece
+        const uint32_t k_bytes = static_cast<uint32_t>((first_step + min(step_, steps - 1)) * kGmStep * 2);
+        const int scalar = static_cast<int>(k_bytes + static_cast<uint32_t>(32 * j) * row_bytes);
+        auto* to = (__attribute__((address_space(3))) void*)(gm_smem + (step_ % kStages) * kStageBytes + 1024 * wave + 4096 * i);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(i < kX ? x_rsrc : (i < kX + kW ? w_rsrc : u_rsrc), to, 16, static_cast<int>(lane_off),
+                                                 scalar, 0, 0);
     };
 
     f32x16_t acc[kTn][kTm], acc_up[DUAL ? kTn : 1][DUAL ? kTm : 1];
@@ -145,28 +184,55 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
     // address of (tile 0 row, k block 0) per lane; tile t adds 32 rows = 4096 bytes, k block kb flips the slot by 2 kb.
     const int frag_row = lane & 31, frag_half = lane >> 5;
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)gm_smem));
-    uint32_t at_kb[4];                                            // byte offset inside a tile for each k block (row part included)
+    uint32_t x_kb[4], w_kb[4];                                    // this wave's first x / w tile, row and k block included
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) at_kb[kb] = static_cast<uint32_t>(frag_row * 128 + (((2 * kb + frag_half) ^ slot_key(frag_row)) * 16));
+    for (int kb = 0; kb < 4; ++kb) {
+        const uint32_t at = static_cast<uint32_t>(frag_row * 128 + (((2 * kb + frag_half) ^ slot_key(frag_row)) * 16));
+        x_kb[kb] = at + static_cast<uint32_t>(wave_m * kTm * 4096);
+        w_kb[kb] = at + static_cast<uint32_t>(kXBytes + wave_n * kTn * 4096);
+    }
     struct Frags {
         u32x4_t w[kTn], x[kTm], u[DUAL ? kTn : 1];
     };
-    auto read_frags = [&](Frags& f, uint32_t stage_at, int kb) __attribute__((always_inline)) {
-        const uint32_t x_at = stage_at + at_kb[kb] + static_cast<uint32_t>(wave_m * kTm * 4096);
-        const uint32_t w_at = stage_at + kXBytes + at_kb[kb] + static_cast<uint32_t>(wave_n * kTn * 4096);
-        // (offsets are literal: tile t of an operand lies 32 rows = 4096 bytes further on)
-        asm volatile("ds_read_b128 %0, %1" : "=v"(f.w[0]) : "v"(w_at));
-        if (DUAL) asm volatile("ds_read_b128 %0, %1 offset:16384" : "=v"(f.u[0]) : "v"(w_at));
-        if (kTn == 2) {
-            asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(f.w[kTn - 1]) : "v"(w_at));
-            if (DUAL) asm volatile("ds_read_b128 %0, %1 offset:20480" : "=v"(f.u[kTn - 1]) : "v"(w_at));
-        }
-        asm volatile("ds_read_b128 %0, %1" : "=v"(f.x[0]) : "v"(x_at));
-        asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(f.x[1]) : "v"(x_at));
+    static_assert(kGmTileBytes == 16384, "the up tile lies 16384 bytes behind the gate tile");
+    // (the reads are inline assembly: the compiler makes every LDS read of its own wait for all requests in flight,
+    // which would expose the memory latency in every step; tile t of an operand lies 32 rows = 4096 bytes further on)
+    auto read_w = [&](Frags& f, uint32_t stage_at, int kb, auto a) __attribute__((always_inline)) {
+        const uint32_t at = stage_at + w_kb[kb];
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.w[decltype(a)::value]) : "v"(at), "n"(4096 * decltype(a)::value));
     };
-    static_assert(kGmTileBytes == 16384 && kTm == 2, "the literal offsets of the fragment reads");
-    constexpr int kReads = kTn * (DUAL ? 2 : 1) + kTm;            // LDS reads per k block and lane
-    // the results of read_frags(f, ...) may be used once at most `later` reads issued after them are outstanding
+    auto read_u = [&](Frags& f, uint32_t stage_at, int kb, auto a) __attribute__((always_inline)) {
+        const uint32_t at = stage_at + w_kb[kb];
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.u[decltype(a)::value]) : "v"(at), "n"(16384 + 4096 * decltype(a)::value));
+    };
+    auto read_x = [&](Frags& f, uint32_t stage_at, int kb, auto b) __attribute__((always_inline)) {
+        const uint32_t at = stage_at + x_kb[kb];
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.x[decltype(b)::value]) : "v"(at), "n"(4096 * decltype(b)::value));
+    };
+    using std::integral_constant;
+    // fragment number `n` of a k block in the order of first use: w0, x0, (u0,) x1 .., then the later weight tiles
+    auto read_nth = [&](Frags& f, uint32_t stage_at, int kb, auto n) __attribute__((always_inline)) {
+        constexpr int N = decltype(n)::value, kD = DUAL ? 2 : 1;
+        if constexpr (N == 0) read_w(f, stage_at, kb, integral_constant<int, 0>{});
+        else if constexpr (N == 1) read_x(f, stage_at, kb, integral_constant<int, 0>{});
+        else if constexpr (DUAL && N == 2) read_u(f, stage_at, kb, integral_constant<int, 0>{});
+        else if constexpr (N < kD + kTm) read_x(f, stage_at, kb, integral_constant<int, N - kD>{});
+        else if constexpr (DUAL && (N - kD - kTm) % 2 == 1) read_u(f, stage_at, kb, integral_constant<int, 1 + (N - kD - kTm) / 2>{});
+        else read_w(f, stage_at, kb, integral_constant<int, 1 + (N - kD - kTm) / kD>{});
+    };
+    auto read_all = [&](Frags& f, uint32_t stage_at, int kb) __attribute__((always_inline)) {
+        read_nth(f, stage_at, kb, integral_constant<int, 0>{});
+        read_nth(f, stage_at, kb, integral_constant<int, 1>{});
+        read_nth(f, stage_at, kb, integral_constant<int, 2>{});
+        if constexpr (Schedule::kReads > 3) read_nth(f, stage_at, kb, integral_constant<int, 3>{});
+        if constexpr (Schedule::kReads > 4) {
+            read_nth(f, stage_at, kb, integral_constant<int, 4>{});
+            read_nth(f, stage_at, kb, integral_constant<int, 5>{});
+        }
+    };
+    static_assert(Schedule::kReads == 3 || Schedule::kReads == 4 || Schedule::kReads == 6, "read_all lists them");
+    constexpr int kReads = Schedule::kReads;
+    // the fragments of f may be used once at most `later` reads issued after them are outstanding
     auto arrived = [&](Frags& f, auto later) __attribute__((always_inline)) {
         if constexpr (kTn == 2 && DUAL) {
             asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(f.w[0]), "+v"(f.w[1]), "+v"(f.u[0]), "+v"(f.u[1]), "+v"(f.x[0]), "+v"(f.x[1])
@@ -179,68 +245,87 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
             asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(f.w[0]), "+v"(f.x[0]), "+v"(f.x[1]) : "n"(decltype(later)::value) : "memory");
         }
     };
-    // The MFMAs of one k block, with this wave's pieces [P0, P1) of step `req_step` requested between them: a request
-    // takes the CU's one address path about 16 cycles a piece (64 bytes a cycle), and issued in a bunch by four waves at
-    // once they leave the matrix cores idle for that long; between MFMAs they are issued in the shadow of the 32 cycles
-    // each MFMA takes.
-    constexpr int kMfmas = kTn * kTm * (DUAL ? 2 : 1);
-    auto multiply = [&](const Frags& f, int req_step, auto p0, auto p1) __attribute__((always_inline)) {
-        constexpr int P0 = decltype(p0)::value, P1 = decltype(p1)::value;
-        int done = 0, piece = P0;
-#pragma unroll
-        for (int a = 0; a < kTn; ++a)
-#pragma unroll
-            for (int b = 0; b < kTm; ++b) {
-                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, f.w[a]), __builtin_bit_cast(bf16x8_t, f.x[b]),
-                                                                    acc[a][b], 0, 0, 0);
-                if (DUAL)
-                    acc_up[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, f.u[a]),
-                                                                           __builtin_bit_cast(bf16x8_t, f.x[b]), acc_up[a][b], 0, 0, 0);
-                done += DUAL ? 2 : 1;
-                // (as many pieces behind this MFMA as keep them evenly spread over the k block's MFMAs)
-                while (piece < P1 && (piece - P0 + 1) * kMfmas <= done * (P1 - P0)) {
-                    __builtin_amdgcn_sched_barrier(0);
-                    request_piece(req_step, piece);
-                    __builtin_amdgcn_sched_barrier(0);
-                    ++piece;
-                }
-            }
-    };
-    using std::integral_constant;
-    constexpr int kQ1 = kPerWave / 4, kQ2 = kPerWave / 2, kQ3 = 3 * kPerWave / 4;
 
-    // A step's schedule.  The stage of step s is complete for everybody at the barrier of step s - 1; k blocks 0 and 1 of
-    // it are read right behind that barrier, while the MFMAs of the last k block of step s - 1 run.  The barrier of step s
-    // stands between the MFMAs of k blocks 2 and 3, at a point where this wave has read all it needs of stage s (its last
-    // reads have landed): behind it stage s is free, and the pieces of step s + kStages are requested into it, spread over
-    // the four k blocks that follow.  The wait in front of the barrier lets the pieces of the steps after s + 1 be in flight.
+    // The MFMAs of one k block from the fragments f, and in the slots between them:
+    //  OWN    a fragment of f that has served its last MFMA is read again, for k block own_kb of the stage at own_at;
+    //  EARLY  the fragments of g are read for k block 0 of the stage at early_at, from the first slot on;
+    //  PIECES this wave's pieces [P0, P0 + PIECES) of step req_step are requested, the emptier slots first.
+    auto multiply = [&](Frags& f, Frags& g, auto own, uint32_t own_at, int own_kb, auto early, uint32_t early_at, int req_step, auto p0,
+                        auto pieces) __attribute__((always_inline)) {
+        constexpr bool OWN = decltype(own)::value, EARLY = decltype(early)::value;
+        constexpr int P0 = decltype(p0)::value, PIECES = decltype(pieces)::value;
+        int piece = P0;
+        auto slot = [&](auto number) __attribute__((always_inline)) {
+            constexpr int S = decltype(number)::value;
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (EARLY) {
+                if constexpr (S * Schedule::kEarlyPerSlot < kReads) read_nth(g, early_at, 0, integral_constant<int, S * Schedule::kEarlyPerSlot>{});
+                if constexpr (Schedule::kEarlyPerSlot == 2 && S * 2 + 1 < kReads) read_nth(g, early_at, 0, integral_constant<int, S * 2 + 1>{});
+            }
+            if constexpr (OWN) {
+                constexpr int kD = Schedule::kD, unit = S / kD, a = unit / kTm, b = unit % kTm;
+                if constexpr (Schedule::w_slot(a) == S) read_w(f, own_at, own_kb, integral_constant<int, a>{});
+                if constexpr (DUAL && Schedule::u_slot(a) == S) read_u(f, own_at, own_kb, integral_constant<int, a>{});
+                if constexpr (Schedule::x_slot(b) == S && a == kTn - 1) read_x(f, own_at, own_kb, integral_constant<int, b>{});
+            }
 #pragma unroll
-    for (int ahead = 0; ahead < kStages; ++ahead)
+            for (int r = 0; r < Schedule::requests_at(S, PIECES); ++r) request_piece(req_step, piece++);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto unit = [&](auto a_, auto b_) __attribute__((always_inline)) {
+            constexpr int a = decltype(a_)::value, b = decltype(b_)::value, first = (a * kTm + b) * Schedule::kD;
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, f.w[a]), __builtin_bit_cast(bf16x8_t, f.x[b]),
+                                                                acc[a][b], 0, 0, 0);
+            slot(integral_constant<int, first>{});
+            if constexpr (DUAL) {
+                acc_up[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, f.u[a]), __builtin_bit_cast(bf16x8_t, f.x[b]),
+                                                                       acc_up[a][b], 0, 0, 0);
+                slot(integral_constant<int, first + 1>{});
+            }
+        };
+        unit(integral_constant<int, 0>{}, integral_constant<int, 0>{});
+        unit(integral_constant<int, 0>{}, integral_constant<int, 1>{});
+        if constexpr (kTn == 2) {
+            unit(integral_constant<int, 1>{}, integral_constant<int, 0>{});
+            unit(integral_constant<int, 1>{}, integral_constant<int, 1>{});
+        }
+    };
+    static_assert(kTm == 2 && kTn <= 2, "multiply lists the units");
+    constexpr int kThird1 = kPerWave / 3, kThird2 = (kPerWave - kThird1) / 2, kThird3 = kPerWave - kThird1 - kThird2;
+    using yes = std::true_type;
+    using no = std::false_type;
+
+    // A step's schedule.  f0 holds k blocks 0 and 2 of a stage in turn, f1 k blocks 1 and 3.  While the MFMAs of a k block
+    // run, its fragments are read again as they fall free, for the k block two further on: f0 during k block 0 (for 2), f1
+    // during 1 (for 3) and during 3 (for 1 of the next step).  The step's one barrier stands behind the MFMAs of k block 2:
+    // there this wave's reads of the stage have all landed and its own pieces of the next step's stage have (the wait lets
+    // the pieces of the steps after that be in flight); behind it the next stage is complete for everybody and this one
+    // free.  f0's fragments for k block 0 of the next step are read in the first slots of k block 3; the pieces of step
+    // s + kStages - 1 are requested into the stage freed at the barrier before, spread over k blocks 0 to 2.
 #pragma unroll
-        for (int i = 0; i < (ahead == kStages - 1 ? kQ1 : kPerWave); ++i) request_piece(ahead, i);
-    gm_wait_vm<kPerWave * (kStages - 2) + kQ1>();
+    for (int ahead = 0; ahead < kStages - 1; ++ahead)
+#pragma unroll
+        for (int i = 0; i < kPerWave; ++i) request_piece(ahead, i);
+    gm_wait_vm<kPerWave * (kStages - 2)>();
     asm volatile("s_barrier" ::: "memory");
     Frags f0, f1;
-    read_frags(f0, lds_base, 0);
-    read_frags(f1, lds_base, 1);
+    read_all(f0, lds_base, 0);
+    read_all(f1, lds_base, 1);
     for (int step = 0; step < steps; ++step) {
         const uint32_t stage_at = lds_base + static_cast<uint32_t>((step % kStages) * kStageBytes);
         const uint32_t next_at = lds_base + static_cast<uint32_t>(((step + 1) % kStages) * kStageBytes);
-        const int req = step - 1 + kStages;                       // (its first quarter went out behind the last barrier)
-        arrived(f0, integral_constant<int, kReads>{});
-        multiply(f0, req, integral_constant<int, kQ1>{}, integral_constant<int, kQ2>{});
-        read_frags(f0, stage_at, 2);
+        const int req = step + kStages - 1;
+        // (f0's last read was issued in slot kLastEarlySlot of the k block before, f1's own reads of that slot and later behind it)
+        arrived(f0, integral_constant<int, Schedule::own_from(Schedule::kLastEarlySlot)>{});
+        multiply(f0, f1, yes{}, stage_at, 2, no{}, 0u, req, integral_constant<int, 0>{}, integral_constant<int, kThird1>{});
         arrived(f1, integral_constant<int, kReads>{});
-        multiply(f1, req, integral_constant<int, kQ2>{}, integral_constant<int, kQ3>{});
-        read_frags(f1, stage_at, 3);
+        multiply(f1, f0, yes{}, stage_at, 3, no{}, 0u, req, integral_constant<int, kThird1>{}, integral_constant<int, kThird2>{});
         arrived(f0, integral_constant<int, kReads>{});
-        multiply(f0, req, integral_constant<int, kQ3>{}, integral_constant<int, kPerWave>{});
+        multiply(f0, f1, no{}, 0u, 0, no{}, 0u, req, integral_constant<int, kThird1 + kThird2>{}, integral_constant<int, kThird3>{});
         arrived(f1, integral_constant<int, 0>{});
         gm_wait_vm<kPerWave * (kStages - 2)>();                   // this wave's pieces of the next step's stage have landed
         asm volatile("s_barrier" ::: "memory");                   // everybody's have; and everybody has read this step's stage
-        if (step + 1 < steps) read_frags(f0, next_at, 0);
-        multiply(f1, step + kStages, integral_constant<int, 0>{}, integral_constant<int, kQ1>{});
-        if (step + 1 < steps) read_frags(f1, next_at, 1);
+        multiply(f1, f0, yes{}, next_at, 1, yes{}, next_at, req, integral_constant<int, 0>{}, integral_constant<int, 0>{});
     }
     gm_wait_vm<0>();                                              // (the requests past the last step, before the block's LDS goes)
 
