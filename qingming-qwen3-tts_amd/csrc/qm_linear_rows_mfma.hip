@@ -31,16 +31,17 @@
 namespace qm {
 
 constexpr int kGmThreads = 256;
-constexpr int kGmTile = 128;                 // token rows and output columns per block
-constexpr int kGmStep = 64;                  // k per step
-constexpr int kGmTileBytes = kGmTile * kGmStep * 2;   // 16 KiB per operand tile
+constexpr int kGmTile = 128;                 // output columns per block (192 for a gate/up pair that it divides), token rows 128 or 64
+constexpr int kGmStep = 64;                  // k per step (32 with the 192-column tile)
 
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 // LDS byte offset of piece `piece` (16 bytes = 8 k) of row `row` inside a tile
-// (the LDS has 64 banks of four bytes: a row of 128 bytes covers half of them, which half by the row's parity, and the
-// sixteen lanes served in a cycle read sixteen consecutive rows: the eight rows of one parity take eight different slots)
-__device__ __forceinline__ int slot_key(int row) { return (row >> 1) & 7; }
+// The LDS has 64 banks of four bytes, and the sixteen lanes served in a cycle read the same piece of sixteen consecutive
+// rows.  A row of ROW_BYTES covers ROW_BYTES / 4 banks, which of them by the row's number within 256 bytes; the rows that
+// share banks take different slots for the same piece: slot = piece ^ key(row).
+template <int ROW_BYTES>
+__device__ __forceinline__ int slot_key(int row) { return (row / (256 / ROW_BYTES)) & (ROW_BYTES / 16 - 1); }
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
@@ -71,6 +72,14 @@ __device__ __forceinline__ uint32_t swiglu_pair(float g0, float g1, float u0, fl
     round_bf16_pair(gv0 / (1.0f + expf(-gv0)), gv1 / (1.0f + expf(-gv1)), a0, a1);
     return pack_bf16_pair(a0 * uv0, a1 * uv1);
 }
+
+// A block's tile: BM token rows x BN output columns (x 2 for a gate/up pair), KSTEP k per step, a ring of kStages stages.
+template <bool DUAL, int BM, int BN, int KSTEP>
+struct GmShape {
+    static constexpr int kStageBytes = (BM + (DUAL ? 2 : 1) * BN) * KSTEP * 2;
+    static constexpr int kStages = kStageBytes * 4 <= 128 * 1024 ? 4 : (kStageBytes * 3 <= 144 * 1024 ? 3 : 2);
+    static_assert(kStageBytes * kStages <= 160 * 1024 - 1024, "the CU's LDS");
+};
 
 // Where the side operations of a k block stand among its MFMAs.  The MFMAs of a k block run over the wave's tiles (a, b),
 // a the weight tile and b the token tile, b fastest, and for a gate/up pair the gate MFMA before the up MFMA; MFMA number i
@@ -110,23 +119,33 @@ struct GmSchedule {
         }
         return given[slot];
     }
+    static constexpr int requests_before(int slot, int pieces) {
+        int n = 0;
+        for (int s = 0; s < slot; ++s) n += requests_at(s, pieces);
+        return n;
+    }
 };
 
-template <bool DUAL, int BM>
+template <bool DUAL, int BM, int BN, int KSTEP>
 __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRowsParams prm) {
     extern __shared__ __attribute__((aligned(16))) unsigned char gm_smem[];
-    constexpr int kStages = DUAL ? 3 : 4;
-    constexpr int kXBytes = BM * kGmStep * 2;
+    constexpr int kStages = GmShape<DUAL, BM, BN, KSTEP>::kStages;
+    constexpr int kRowBytes = KSTEP * 2, kSlots = kRowBytes / 16, kKb = KSTEP / 16;
+    constexpr int kRowsPerPiece = 64 / kSlots;                    // tile rows one instruction of a wave fills
+    constexpr int kXBytes = BM * kRowBytes, kWBytes = BN * kRowBytes;
     constexpr int kWeights = DUAL ? 2 : 1;
-    constexpr int kStageBytes = kXBytes + kWeights * kGmTileBytes;
-    constexpr int kTn = BM == 128 ? 2 : 1;                        // MFMA tiles of a wave along the output columns
+    constexpr int kStageBytes = kXBytes + kWeights * kWBytes;
+    static_assert(kStageBytes == GmShape<DUAL, BM, BN, KSTEP>::kStageBytes, "");
+    constexpr int kTn = BM == 128 ? BN / 64 : BN / 128;           // MFMA tiles of a wave along the output columns
     constexpr int kTm = 2;                                        // and along the token rows
+    constexpr int kFragTile = 32 * kRowBytes;                     // LDS bytes from an operand's MFMA tile to its next
     using Schedule = GmSchedule<DUAL, kTn, kTm>;
     // pieces of 1 KiB (one instruction of a wave) per stage: x, w (, up); dealt to the four waves in turn
-    constexpr int kPiecesX = kXBytes / 1024, kPiecesW = kGmTileBytes / 1024;
+    constexpr int kPiecesX = kXBytes / 1024, kPiecesW = kWBytes / 1024;
     constexpr int kPerWave = (kPiecesX + kWeights * kPiecesW) / 4;
     static_assert(kPiecesX % 4 == 0 && kPiecesW % 4 == 0, "a wave's piece i is of the same operand in every wave");
-    static_assert(kPerWave * (kStages - 2) <= 63, "the waits count the later stages' pieces");
+    static_assert(kPerWave * (kStages - 2) <= 63 && kStages >= 2, "the waits count the later stages' pieces");
+    static_assert(kKb == 4 || kKb == 2, "the two step schedules");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -134,35 +153,37 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
     const int wave_n = BM == 128 ? (wave & 1) : wave;
     const int wave_m = BM == 128 ? (wave >> 1) : 0;
     const int K = prm.reduction;
-    const int n0 = static_cast<int>(blockIdx.x) * kGmTile;
+    const int n0 = static_cast<int>(blockIdx.x) * BN;
     const int m0 = static_cast<int>(blockIdx.y) * BM;
 
     // ---- this wave's pieces of a stage: instruction q = wave + 4 i covers LDS bytes [1024 q, 1024 q + 1024) of the
-    // stage (x tile, then w, then up); its lane l fills slot l % 8 of tile row 8 (q within the tile) + l / 8 with
-    // global piece slot ^ slot_key(row).  The tiles are read through buffer descriptors that begin at the block's first
-    // row of each operand: a lane's offset is the same for every piece (32 rows further on, the key of a row is the
-    // same), what changes from piece to piece and step to step is a scalar; token rows past the last are out of the
-    // descriptor's range and read as zero without touching memory (their results are never stored). ----
+    // stage (x tile, then w, then up); its lane l fills slot l % kSlots of tile row kRowsPerPiece (q within the tile) +
+    // l / kSlots with global piece slot ^ slot_key(row).  The tiles are read through buffer descriptors that begin at the
+    // block's first row of each operand: a lane's offset is the same for every piece (4 kRowsPerPiece rows further on,
+    // the key of a row is the same), what changes from piece to piece and step to step is a scalar; token rows past the
+    // last are out of the descriptor's range and read as zero without touching memory (their results are never stored).
     const uint32_t row_bytes = static_cast<uint32_t>(K) * 2u;
     const int x_rows = min(prm.rows - m0, BM);
     const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(prm.input + static_cast<int64_t>(m0) * K), 0, static_cast<int>(x_rows * row_bytes), 0x00020000);
     const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t*>(prm.weight[0] + static_cast<int64_t>(n0) * K), 0, static_cast<int>(kGmTile * row_bytes), 0x00020000);
+        const_cast<uint16_t*>(prm.weight[0] + static_cast<int64_t>(n0) * K), 0, static_cast<int>(BN * row_bytes), 0x00020000);
     const __amdgpu_buffer_rsrc_t u_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t*>(prm.weight[DUAL ? 1 : 0] + static_cast<int64_t>(n0) * K), 0, static_cast<int>(kGmTile * row_bytes), 0x00020000);
-    const int lane_row = 8 * wave + (lane >> 3);
-    const uint32_t lane_off = static_cast<uint32_t>(lane_row) * row_bytes + 16u * static_cast<uint32_t>((lane & 7) ^ slot_key(lane_row));
+        const_cast<uint16_t*>(prm.weight[DUAL ? 1 : 0] + static_cast<int64_t>(n0) * K), 0, static_cast<int>(BN * row_bytes), 0x00020000);
+    const int lane_row = kRowsPerPiece * wave + lane / kSlots;
+    const uint32_t lane_off = static_cast<uint32_t>(lane_row) * row_bytes
+                            + 16u * static_cast<uint32_t>((lane % kSlots) ^ slot_key<kRowBytes>(lane_row));
+    static_assert((4 * kRowsPerPiece) % (256 / kRowBytes * kSlots) == 0, "a piece further on, a row's key is the same");
     // (a block takes piece blockIdx.z of the reduction: all of it unless the launch cut it)
-    const int steps = K / kGmStep / prm.reduction_parts;
+    const int steps = K / KSTEP / prm.reduction_parts;
     const int first_step = static_cast<int>(blockIdx.z) * steps;
     // Piece `i` of this wave's pieces of step `step_`, into stage step_ % kStages.  (Requests past the last step repeat it
     // and land in a stage nobody reads again: the wait before the barrier counts pieces.)
     auto request_piece = [&](int step_, int i) __attribute__((always_inline)) {
         constexpr int kX = kPiecesX / 4, kW = kPiecesW / 4;
-        const int j = i < kX ? i : (i < kX + kW ? i - kX : i - kX - kW);                  // 32 rows further on per piece
-        const uint32_t k_bytes = static_cast<uint32_t>((first_step + min(step_, steps - 1)) * kGmStep * 2);
-        const int scalar = static_cast<int>(k_bytes + static_cast<uint32_t>(32 * j) * row_bytes);
+        const int j = i < kX ? i : (i < kX + kW ? i - kX : i - kX - kW);
+        const uint32_t k_bytes = static_cast<uint32_t>((first_step + min(step_, steps - 1)) * KSTEP * 2);
+        const int scalar = static_cast<int>(k_bytes + static_cast<uint32_t>(4 * kRowsPerPiece * j) * row_bytes);
         auto* to = (__attribute__((address_space(3))) void*)(gm_smem + (step_ % kStages) * kStageBytes + 1024 * wave + 4096 * i);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(i < kX ? x_rsrc : (i < kX + kW ? w_rsrc : u_rsrc), to, 16, static_cast<int>(lane_off),
                                                  scalar, 0, 0);
@@ -181,34 +202,35 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
         }
 
     // fragment of tile rows [32 t, 32 t + 32), k block kb (16 k): lane l takes row l % 32, piece 2 kb + l / 32.  The LDS
-    // address of (tile 0 row, k block 0) per lane; tile t adds 32 rows = 4096 bytes, k block kb flips the slot by 2 kb.
+    // address of (tile 0 row, k block 0) per lane; tile t adds 32 rows, k block kb flips the slot by 2 kb.
     const int frag_row = lane & 31, frag_half = lane >> 5;
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)gm_smem));
-    uint32_t x_kb[4], w_kb[4];                                    // this wave's first x / w tile, row and k block included
+    uint32_t x_kb[kKb], w_kb[kKb];                                // this wave's first x / w tile, row and k block included
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-        const uint32_t at = static_cast<uint32_t>(frag_row * 128 + (((2 * kb + frag_half) ^ slot_key(frag_row)) * 16));
-        x_kb[kb] = at + static_cast<uint32_t>(wave_m * kTm * 4096);
-        w_kb[kb] = at + static_cast<uint32_t>(kXBytes + wave_n * kTn * 4096);
+    for (int kb = 0; kb < kKb; ++kb) {
+        const uint32_t at = static_cast<uint32_t>(frag_row * kRowBytes + (((2 * kb + frag_half) ^ slot_key<kRowBytes>(frag_row)) * 16));
+        x_kb[kb] = at + static_cast<uint32_t>(wave_m * kTm * kFragTile);
+        w_kb[kb] = at + static_cast<uint32_t>(kXBytes + wave_n * kTn * kFragTile);
     }
     struct Frags {
         u32x4_t w[kTn], x[kTm], u[DUAL ? kTn : 1];
     };
-    static_assert(kGmTileBytes == 16384, "the up tile lies 16384 bytes behind the gate tile");
     // (the reads are inline assembly: the compiler makes every LDS read of its own wait for all requests in flight,
-    // which would expose the memory latency in every step; tile t of an operand lies 32 rows = 4096 bytes further on)
+    // which would expose the memory latency in every step; tile t of an operand lies kFragTile bytes further on, the up
+    // tile kWBytes behind the gate tile)
     auto read_w = [&](Frags& f, uint32_t stage_at, int kb, auto a) __attribute__((always_inline)) {
         const uint32_t at = stage_at + w_kb[kb];
-        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.w[decltype(a)::value]) : "v"(at), "n"(4096 * decltype(a)::value));
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.w[decltype(a)::value]) : "v"(at), "n"(kFragTile * decltype(a)::value));
     };
     auto read_u = [&](Frags& f, uint32_t stage_at, int kb, auto a) __attribute__((always_inline)) {
         const uint32_t at = stage_at + w_kb[kb];
-        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.u[decltype(a)::value]) : "v"(at), "n"(16384 + 4096 * decltype(a)::value));
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.u[decltype(a)::value]) : "v"(at), "n"(kWBytes + kFragTile * decltype(a)::value));
     };
     auto read_x = [&](Frags& f, uint32_t stage_at, int kb, auto b) __attribute__((always_inline)) {
         const uint32_t at = stage_at + x_kb[kb];
-        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.x[decltype(b)::value]) : "v"(at), "n"(4096 * decltype(b)::value));
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.x[decltype(b)::value]) : "v"(at), "n"(kFragTile * decltype(b)::value));
     };
+    static_assert(kWBytes + kFragTile * kTn <= 65535, "the literal offsets of the fragment reads");
     using std::integral_constant;
     // fragment number `n` of a k block in the order of first use: w0, x0, (u0,) x1 .., then the later weight tiles
     auto read_nth = [&](Frags& f, uint32_t stage_at, int kb, auto n) __attribute__((always_inline)) {
@@ -229,12 +251,19 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
             read_nth(f, stage_at, kb, integral_constant<int, 4>{});
             read_nth(f, stage_at, kb, integral_constant<int, 5>{});
         }
+        if constexpr (Schedule::kReads > 6) {
+            read_nth(f, stage_at, kb, integral_constant<int, 6>{});
+            read_nth(f, stage_at, kb, integral_constant<int, 7>{});
+        }
     };
-    static_assert(Schedule::kReads == 3 || Schedule::kReads == 4 || Schedule::kReads == 6, "read_all lists them");
+    static_assert(Schedule::kReads == 3 || Schedule::kReads == 4 || Schedule::kReads == 6 || Schedule::kReads == 8, "read_all lists them");
     constexpr int kReads = Schedule::kReads;
     // the fragments of f may be used once at most `later` reads issued after them are outstanding
     auto arrived = [&](Frags& f, auto later) __attribute__((always_inline)) {
-        if constexpr (kTn == 2 && DUAL) {
+        if constexpr (kTn == 3 && DUAL) {
+            asm volatile("s_waitcnt lgkmcnt(%8)" : "+v"(f.w[0]), "+v"(f.w[1]), "+v"(f.w[kTn - 1]), "+v"(f.u[0]), "+v"(f.u[1]), "+v"(f.u[kTn - 1]),
+                         "+v"(f.x[0]), "+v"(f.x[1]) : "n"(decltype(later)::value) : "memory");
+        } else if constexpr (kTn == 2 && DUAL) {
             asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(f.w[0]), "+v"(f.w[1]), "+v"(f.u[0]), "+v"(f.u[1]), "+v"(f.x[0]), "+v"(f.x[1])
                          : "n"(decltype(later)::value) : "memory");
         } else if constexpr (kTn == 2) {
@@ -242,6 +271,7 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
         } else if constexpr (DUAL) {
             asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(f.w[0]), "+v"(f.u[0]), "+v"(f.x[0]), "+v"(f.x[1]) : "n"(decltype(later)::value) : "memory");
         } else {
+            static_assert(kTn <= 2 || DUAL, "");
             asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(f.w[0]), "+v"(f.x[0]), "+v"(f.x[1]) : "n"(decltype(later)::value) : "memory");
         }
     };
@@ -254,7 +284,6 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
                         auto pieces) __attribute__((always_inline)) {
         constexpr bool OWN = decltype(own)::value, EARLY = decltype(early)::value;
         constexpr int P0 = decltype(p0)::value, PIECES = decltype(pieces)::value;
-        int piece = P0;
         auto slot = [&](auto number) __attribute__((always_inline)) {
             constexpr int S = decltype(number)::value;
             __builtin_amdgcn_sched_barrier(0);
@@ -268,8 +297,12 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
                 if constexpr (DUAL && Schedule::u_slot(a) == S) read_u(f, own_at, own_kb, integral_constant<int, a>{});
                 if constexpr (Schedule::x_slot(b) == S && a == kTn - 1) read_x(f, own_at, own_kb, integral_constant<int, b>{});
             }
-#pragma unroll
-            for (int r = 0; r < Schedule::requests_at(S, PIECES); ++r) request_piece(req_step, piece++);
+            constexpr int kHere = Schedule::requests_at(S, PIECES), kFirst = P0 + Schedule::requests_before(S, PIECES);
+            static_assert(kHere <= 4, "listed below");
+            if constexpr (kHere > 0) request_piece(req_step, kFirst);
+            if constexpr (kHere > 1) request_piece(req_step, kFirst + 1);
+            if constexpr (kHere > 2) request_piece(req_step, kFirst + 2);
+            if constexpr (kHere > 3) request_piece(req_step, kFirst + 3);
             __builtin_amdgcn_sched_barrier(0);
         };
         auto unit = [&](auto a_, auto b_) __attribute__((always_inline)) {
@@ -285,13 +318,20 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
         };
         unit(integral_constant<int, 0>{}, integral_constant<int, 0>{});
         unit(integral_constant<int, 0>{}, integral_constant<int, 1>{});
-        if constexpr (kTn == 2) {
+        if constexpr (kTn >= 2) {
             unit(integral_constant<int, 1>{}, integral_constant<int, 0>{});
             unit(integral_constant<int, 1>{}, integral_constant<int, 1>{});
         }
+        if constexpr (kTn == 3) {
+            unit(integral_constant<int, 2>{}, integral_constant<int, 0>{});
+            unit(integral_constant<int, 2>{}, integral_constant<int, 1>{});
+        }
     };
-    static_assert(kTm == 2 && kTn <= 2, "multiply lists the units");
-    constexpr int kThird1 = kPerWave / 3, kThird2 = (kPerWave - kThird1) / 2, kThird3 = kPerWave - kThird1 - kThird2;
+    static_assert(kTm == 2 && kTn <= 3, "multiply lists the units");
+    // (a step's requests over its first three k blocks; with two stages they must have landed at the step's own barrier
+    // and go out as early as one to a slot allows)
+    constexpr int kThird1 = kStages == 2 ? (kPerWave > Schedule::kMfmas ? Schedule::kMfmas : kPerWave) : kPerWave / 3;
+    constexpr int kThird2 = kStages == 2 ? kPerWave - kThird1 : (kPerWave - kThird1) / 2, kThird3 = kPerWave - kThird1 - kThird2;
     using yes = std::true_type;
     using no = std::false_type;
 
@@ -317,11 +357,16 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
         const int req = step + kStages - 1;
         // (f0's last read was issued in slot kLastEarlySlot of the k block before, f1's own reads of that slot and later behind it)
         arrived(f0, integral_constant<int, Schedule::own_from(Schedule::kLastEarlySlot)>{});
-        multiply(f0, f1, yes{}, stage_at, 2, no{}, 0u, req, integral_constant<int, 0>{}, integral_constant<int, kThird1>{});
-        arrived(f1, integral_constant<int, kReads>{});
-        multiply(f1, f0, yes{}, stage_at, 3, no{}, 0u, req, integral_constant<int, kThird1>{}, integral_constant<int, kThird2>{});
-        arrived(f0, integral_constant<int, kReads>{});
-        multiply(f0, f1, no{}, 0u, 0, no{}, 0u, req, integral_constant<int, kThird1 + kThird2>{}, integral_constant<int, kThird3>{});
+        if constexpr (kKb == 4) {
+            multiply(f0, f1, yes{}, stage_at, 2, no{}, 0u, req, integral_constant<int, 0>{}, integral_constant<int, kThird1>{});
+            arrived(f1, integral_constant<int, kReads>{});
+            multiply(f1, f0, yes{}, stage_at, 3, no{}, 0u, req, integral_constant<int, kThird1>{}, integral_constant<int, kThird2>{});
+            arrived(f0, integral_constant<int, kReads>{});
+            multiply(f0, f1, no{}, 0u, 0, no{}, 0u, req, integral_constant<int, kThird1 + kThird2>{}, integral_constant<int, kThird3>{});
+        } else {
+            // (a step of two k blocks: f0 holds the first, f1 the second; all of the step's requests go out during the first)
+            multiply(f0, f1, no{}, 0u, 0, no{}, 0u, req, integral_constant<int, 0>{}, integral_constant<int, kPerWave>{});
+        }
         arrived(f1, integral_constant<int, 0>{});
         gm_wait_vm<kPerWave * (kStages - 2)>();                   // this wave's pieces of the next step's stage have landed
         asm volatile("s_barrier" ::: "memory");                   // everybody's have; and everybody has read this step's stage
@@ -418,17 +463,17 @@ __global__ __launch_bounds__(256) void linear_rows_parts_kernel(LinearRowsParams
     *reinterpret_cast<uint2*>(prm.output + static_cast<int64_t>(m) * prm.columns + n) = packed;
 }
 
-template <bool DUAL, int BM>
+template <bool DUAL, int BM, int BN, int KSTEP>
 int32_t launch_rows_mfma_as(const LinearRowsParams& prm, hipStream_t stream) {
-    constexpr int kStages = DUAL ? 3 : 4;
-    constexpr int smem = kStages * (BM * kGmStep * 2 + (DUAL ? 2 : 1) * kGmTileBytes);
-    const dim3 grid(static_cast<unsigned>(prm.columns / kGmTile), static_cast<unsigned>((prm.rows + BM - 1) / BM),
+    using Shape = GmShape<DUAL, BM, BN, KSTEP>;
+    constexpr int smem = Shape::kStages * Shape::kStageBytes;
+    const dim3 grid(static_cast<unsigned>(prm.columns / BN), static_cast<unsigned>((prm.rows + BM - 1) / BM),
                     static_cast<unsigned>(prm.reduction_parts));
     if (grid.y > 65535u) return QM_ERR_ARGUMENT;
     static std::atomic<bool> lds_raised[kMaxDevices];
-    const int32_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(linear_rows_mfma_kernel<DUAL, BM>), smem, lds_raised);
+    const int32_t rc = ensure_dynamic_lds(reinterpret_cast<const void*>(linear_rows_mfma_kernel<DUAL, BM, BN, KSTEP>), smem, lds_raised);
     if (rc != QM_OK) return rc;
-    hipLaunchKernelGGL((linear_rows_mfma_kernel<DUAL, BM>), grid, dim3(kGmThreads), smem, stream, prm);
+    hipLaunchKernelGGL((linear_rows_mfma_kernel<DUAL, BM, BN, KSTEP>), grid, dim3(kGmThreads), smem, stream, prm);
     int32_t status = launch_status();
     if (status == QM_OK && prm.reduction_parts > 1) {
         const int64_t quads = static_cast<int64_t>(prm.rows) * (prm.columns / 4);
@@ -461,10 +506,18 @@ size_t rows_mfma_workspace_bytes(int rows, int columns, int reduction, bool dual
 int32_t launch_rows_mfma(const LinearRowsParams& prm, bool dual, hipStream_t stream) {
     if (prm.rows == 0 || prm.columns == 0) return QM_OK;
     // blocks of 64 token rows where blocks of 128 would leave CUs without one (one block per CU either way)
-    const int64_t blocks_128 = static_cast<int64_t>(prm.columns / kGmTile) * ((prm.rows + 127) / 128);
+    const int64_t row_tiles = (prm.rows + 127) / 128;
+    const int64_t blocks_128 = static_cast<int64_t>(prm.columns / kGmTile) * row_tiles;
     const bool small = blocks_128 < 200;
-    if (dual) return small ? launch_rows_mfma_as<true, 64>(prm, stream) : launch_rows_mfma_as<true, 128>(prm, stream);
-    return small ? launch_rows_mfma_as<false, 64>(prm, stream) : launch_rows_mfma_as<false, 128>(prm, stream);
+    if (dual) {
+        // a gate/up pair whose grid of 128-column tiles is more than the CUs take at once and less than twice that: tiles
+        // of 192 columns, if those fit in one round (1024 tokens x 6144 channels: 384 blocks of 128, 256 of 192)
+        const int64_t blocks_192 = static_cast<int64_t>(prm.columns / 192) * row_tiles;
+        if (prm.reduction_parts == 1 && prm.columns % 192 == 0 && blocks_128 > 256 && blocks_128 < 512 && blocks_192 <= 256)
+            return launch_rows_mfma_as<true, 128, 192, 64>(prm, stream);
+        return small ? launch_rows_mfma_as<true, 64, 128, 64>(prm, stream) : launch_rows_mfma_as<true, 128, 128, 64>(prm, stream);
+    }
+    return small ? launch_rows_mfma_as<false, 64, 128, 64>(prm, stream) : launch_rows_mfma_as<false, 128, 128, 64>(prm, stream);
 }
 
 }  // namespace qm
