@@ -506,7 +506,7 @@ class TalkerLayerStep:
 
 class PromptLinears:
     """Beyond the five configurations: the seven linears of one talker layer over a prompt of `rows` tokens as the
-    prompt pass chains them (NativeTalkerEngine::prefill, R17:16646-16790): q, k, v projections with bias, o_proj +
+    prompt pass chains them (NativeTalkerEngine::prefill, R17:16646-16790): q, k, v projections with bias (one call), o_proj +
     residual, gate/up/SwiGLU, down_proj + residual (hidden 2048, intermediate 6144).  kernel 0: the matrix cores
     (default); 1: every sum in the reference's order (QM_OPT_LINEAR_ROWS_KERNEL)."""
     bound = "mfma"
@@ -542,16 +542,14 @@ class PromptLinears:
         try:
             if self.split:
                 ws, nb = self.ws, self.ws_bytes
-                qm.linear_rows_split(self.x, self.wq, self.bq, None, self.q, R, H, H, ws, nb, s)
-                qm.linear_rows_split(self.x, self.wk, self.bk, None, self.k, R, KV, H, ws, nb, s)
-                qm.linear_rows_split(self.x, self.wv, self.bv, None, self.v, R, KV, H, ws, nb, s)
+                qm.qkv_rows(self.x, (self.wq, self.wk, self.wv), (self.bq, self.bk, self.bv), (self.q, self.k, self.v), R, H, KV, H,
+                            ws, nb, s)
                 qm.linear_rows_split(self.q, self.wo, None, self.res, self.o, R, H, H, ws, nb, s)
                 qm.gate_up_swiglu_rows_split(self.o, self.wg, self.wu, self.act, R, H, I, ws, nb, s)
                 qm.linear_rows_split(self.act, self.wd, None, self.o, self.out, R, H, I, ws, nb, s)
                 return
-            qm.linear_rows(self.x, self.wq, self.bq, None, self.q, R, H, H, s)
-            qm.linear_rows(self.x, self.wk, self.bk, None, self.k, R, KV, H, s)
-            qm.linear_rows(self.x, self.wv, self.bv, None, self.v, R, KV, H, s)
+            qm.qkv_rows(self.x, (self.wq, self.wk, self.wv), (self.bq, self.bk, self.bv), (self.q, self.k, self.v), R, H, KV, H,
+                        None, 0, s)
             qm.linear_rows(self.q, self.wo, None, self.res, self.o, R, H, H, s)
             qm.gate_up_swiglu_rows(self.o, self.wg, self.wu, self.act, R, H, I, s)
             qm.linear_rows(self.act, self.wd, None, self.o, self.out, R, H, I, s)

@@ -841,6 +841,24 @@ int32_t qm_gate_up_swiglu_rows_split(
     const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight, uint16_t* output,
     int32_t rows, int32_t hidden, int32_t intermediate,
     void* workspace, int64_t workspace_bytes, void* hip_stream);
+/*
+ * The q, k and v projections of the prompt pass (the first three linear_generic calls of a layer, R17:16646-16672) as one
+ * call: output for output what three qm_linear_rows calls on the same input give, bit for bit (on the matrix cores an
+ * output's sum does not depend on the tile it is computed in).  Where all three run uncut on the matrix cores they share
+ * one grid (1024 tokens: 256 blocks, one per compute unit, instead of 256 + 128 + 128 in three launches); otherwise the
+ * call is the three calls.  _split: the workspace of qm_linear_rows_split (the larger of the two shapes' sizes).
+ */
+int32_t qm_qkv_rows(
+    const uint16_t* input, const uint16_t* q_weight, const uint16_t* k_weight, const uint16_t* v_weight,
+    const uint16_t* q_bias, const uint16_t* k_bias, const uint16_t* v_bias,
+    uint16_t* q_output, uint16_t* k_output, uint16_t* v_output,
+    int32_t rows, int32_t q_columns, int32_t kv_columns, int32_t reduction_columns, void* hip_stream);
+int32_t qm_qkv_rows_split(
+    const uint16_t* input, const uint16_t* q_weight, const uint16_t* k_weight, const uint16_t* v_weight,
+    const uint16_t* q_bias, const uint16_t* k_bias, const uint16_t* v_bias,
+    uint16_t* q_output, uint16_t* k_output, uint16_t* v_output,
+    int32_t rows, int32_t q_columns, int32_t kv_columns, int32_t reduction_columns,
+    void* workspace, int64_t workspace_bytes, void* hip_stream);
 
 /* ---- final head: score processing, top-k sampler, history ------------------------ */
 /*

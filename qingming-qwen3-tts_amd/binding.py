@@ -154,6 +154,8 @@ _SIGNATURES = {
     "qm_linear_rows_split_workspace_bytes": (C.c_int64, [_I32, _I32, _I32, _I32]),
     "qm_linear_rows_split": (_I32, [_PTR] * 5 + [_I32, _I32, _I32, _PTR, C.c_int64, _PTR]),
     "qm_gate_up_swiglu_rows_split": (_I32, [_PTR] * 4 + [_I32, _I32, _I32, _PTR, C.c_int64, _PTR]),
+    "qm_qkv_rows": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _I32, _PTR]),
+    "qm_qkv_rows_split": (_I32, [_PTR] * 10 + [_I32, _I32, _I32, _I32, _PTR, C.c_int64, _PTR]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
@@ -463,6 +465,13 @@ def linear_rows_split_workspace_bytes(rows, output_columns, reduction_columns, g
 def linear_rows_split(x, weight, bias, residual, out, rows, output_columns, reduction_columns, workspace, workspace_bytes, stream=0):
     _check(lib().qm_linear_rows_split(_addr(x), _addr(weight), _addr(bias), _addr(residual), _addr(out), rows, output_columns,
                                       reduction_columns, _addr(workspace), workspace_bytes, stream), "qm_linear_rows_split")
+
+
+def qkv_rows(x, weights, biases, outs, rows, q_columns, kv_columns, reduction_columns, workspace=None, workspace_bytes=0, stream=0):
+    """weights / biases / outs: (q, k, v) triples; a bias may be None."""
+    _check(lib().qm_qkv_rows_split(_addr(x), *[_addr(w) for w in weights], *[_addr(b) for b in biases], *[_addr(o) for o in outs],
+                                   rows, q_columns, kv_columns, reduction_columns, _addr(workspace), workspace_bytes, stream),
+           "qm_qkv_rows_split")
 
 
 def gate_up_swiglu_rows_split(x, gate_weight, up_weight, out, rows, hidden, intermediate, workspace, workspace_bytes, stream=0):

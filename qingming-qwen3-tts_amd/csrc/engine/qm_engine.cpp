@@ -320,7 +320,7 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
 // NativeTalkerEngine::prefill (R17:16561-16800): the prompt's rows through every layer.  The
 // reference's launches per layer and what runs here:
 //   rmsnorm                                   -> qm_rmsnorm_rows
-//   3 x linear_generic (q, k, v)              -> 3 x qm_linear_rows (every linear through its _split entry: short prompts)
+//   3 x linear_generic (q, k, v)              -> qm_qkv_rows (every linear through its _split entry: short prompts)
 //   2 x rmsnorm + 2 x rope_rows               -> 2 x qm_norm_rope_rows
 //   scatter_prefill_cache + attention         -> qm_prefill_attention_causal_split (writes the cache itself; long
 //                                                query tiles of a prompt are shared by two or three blocks)
@@ -376,12 +376,9 @@ static const uint16_t* prefill(qm_talker& e, const uint16_t* input_device, const
         const qm_kv_cache cache = flat_cache_of(e, w);
         op_check(qm_rmsnorm_rows(current->u16(), w.input_norm.data(), e.p_norm.u16(), rows, kHidden, kEpsilon, s),
                  "prefill input RMSNorm");
-        op_check(qm_linear_rows_split(e.p_norm.u16(), w.q_weight.data(), w.q_bias.data(), nullptr, e.p_q.u16(), rows, e.q_dim,
-                                      kHidden, rows_ws, rows_bytes, s), "prefill q_proj");
-        op_check(qm_linear_rows_split(e.p_norm.u16(), w.k_weight.data(), w.k_bias.data(), nullptr, e.p_k.u16(), rows, e.kv_dim,
-                                      kHidden, rows_ws, rows_bytes, s), "prefill k_proj");
-        op_check(qm_linear_rows_split(e.p_norm.u16(), w.v_weight.data(), w.v_bias.data(), nullptr, e.p_v.u16(), rows, e.kv_dim,
-                                      kHidden, rows_ws, rows_bytes, s), "prefill v_proj");
+        op_check(qm_qkv_rows_split(e.p_norm.u16(), w.q_weight.data(), w.k_weight.data(), w.v_weight.data(), w.q_bias.data(),
+                                   w.k_bias.data(), w.v_bias.data(), e.p_q.u16(), e.p_k.u16(), e.p_v.u16(), rows, e.q_dim, e.kv_dim,
+                                   kHidden, rows_ws, rows_bytes, s), "prefill q/k/v_proj");
         op_check(qm_norm_rope_rows(e.p_q.u16(), w.q_norm.data(), e.p_cosine.u16(), e.p_sine.u16(), e.p_q_rotated.u16(), rows,
                                    e.q_heads, kEpsilon, s), "prefill q norm + RoPE");
         op_check(qm_norm_rope_rows(e.p_k.u16(), w.k_norm.data(), e.p_cosine.u16(), e.p_sine.u16(), e.p_k_rotated.u16(), rows,

@@ -254,6 +254,7 @@ inline int32_t rows_entry(LinearRowsParams prm, bool dual, void* workspace, int6
     if (rc_kernel != QM_OK) return rc_kernel;
     prm.reduction_parts = 1;
     prm.partials = nullptr;
+    prm.groups = 1;
     if (!matrix_cores) return dual ? launch_rows<true>(prm, static_cast<hipStream_t>(hip_stream))
                                    : launch_rows<false>(prm, static_cast<hipStream_t>(hip_stream));
     if (workspace) {
@@ -296,6 +297,55 @@ extern "C" int32_t qm_linear_rows_split(const uint16_t* input, const uint16_t* w
     prm.input = input; prm.weight[0] = weight; prm.weight[1] = weight; prm.bias = bias; prm.residual = residual;
     prm.output = output; prm.rows = rows; prm.columns = output_columns; prm.reduction = reduction_columns;
     return rows_entry(prm, false, workspace, workspace_bytes, hip_stream);
+}
+
+// Three linears of one input.  On the matrix cores, uncut: one grid over the column tiles of all three (the same sums and
+// roundings as three calls: an output's k blocks are added in the same order whatever the tile); otherwise three calls.
+extern "C" int32_t qm_qkv_rows_split(const uint16_t* input, const uint16_t* q_weight, const uint16_t* k_weight, const uint16_t* v_weight,
+                                     const uint16_t* q_bias, const uint16_t* k_bias, const uint16_t* v_bias,
+                                     uint16_t* q_output, uint16_t* k_output, uint16_t* v_output, int32_t rows, int32_t q_columns,
+                                     int32_t kv_columns, int32_t reduction_columns, void* workspace, int64_t workspace_bytes,
+                                     void* hip_stream) {
+    using namespace qm;
+    if (!input || !q_weight || !k_weight || !v_weight || !q_output || !k_output || !v_output) return QM_ERR_NULL;
+    if (workspace_bytes < 0 || (workspace_bytes > 0 && !workspace)) return QM_ERR_ARGUMENT;
+    LinearRowsParams prm = {};
+    prm.input = input; prm.weight[0] = q_weight; prm.weight[1] = q_weight; prm.bias = q_bias; prm.output = q_output;
+    prm.rows = rows; prm.columns = q_columns; prm.reduction = reduction_columns;
+    LinearRowsParams other = prm;
+    other.weight[0] = other.weight[1] = k_weight; other.bias = k_bias; other.output = k_output; other.columns = kv_columns;
+    int32_t fused = 0, fused_other = 0;
+    int32_t rc = check_rows(prm, false);
+    if (rc == QM_OK) rc = check_rows(other, false);
+    if (rc == QM_OK) rc = rows_on_matrix_cores(prm, &fused);
+    if (rc == QM_OK) rc = rows_on_matrix_cores(other, &fused_other);
+    if (rc != QM_OK) return rc;
+    const uintptr_t align = reinterpret_cast<uintptr_t>(v_weight) | reinterpret_cast<uintptr_t>(v_bias) | reinterpret_cast<uintptr_t>(v_output);
+    const bool cut = workspace && (rows_mfma_workspace_bytes(rows, q_columns, reduction_columns, false) > 0
+                                   || rows_mfma_workspace_bytes(rows, kv_columns, reduction_columns, false) > 0);
+    if (!fused || !fused_other || (align & 15) || cut) {
+        rc = qm_linear_rows_split(input, q_weight, q_bias, nullptr, q_output, rows, q_columns, reduction_columns, workspace, workspace_bytes, hip_stream);
+        if (rc == QM_OK)
+            rc = qm_linear_rows_split(input, k_weight, k_bias, nullptr, k_output, rows, kv_columns, reduction_columns, workspace, workspace_bytes, hip_stream);
+        if (rc == QM_OK)
+            rc = qm_linear_rows_split(input, v_weight, v_bias, nullptr, v_output, rows, kv_columns, reduction_columns, workspace, workspace_bytes, hip_stream);
+        return rc;
+    }
+    prm.reduction_parts = 1;
+    prm.groups = 3;
+    prm.group_first_tile[0] = q_columns / 128;
+    prm.group_first_tile[1] = (q_columns + kv_columns) / 128;
+    prm.group_weight[0] = k_weight; prm.group_bias[0] = k_bias; prm.group_output[0] = k_output; prm.group_columns[0] = kv_columns;
+    prm.group_weight[1] = v_weight; prm.group_bias[1] = v_bias; prm.group_output[1] = v_output; prm.group_columns[1] = kv_columns;
+    return launch_rows_mfma(prm, false, static_cast<hipStream_t>(hip_stream));
+}
+
+extern "C" int32_t qm_qkv_rows(const uint16_t* input, const uint16_t* q_weight, const uint16_t* k_weight, const uint16_t* v_weight,
+                               const uint16_t* q_bias, const uint16_t* k_bias, const uint16_t* v_bias,
+                               uint16_t* q_output, uint16_t* k_output, uint16_t* v_output, int32_t rows, int32_t q_columns,
+                               int32_t kv_columns, int32_t reduction_columns, void* hip_stream) {
+    return qm_qkv_rows_split(input, q_weight, k_weight, v_weight, q_bias, k_bias, v_bias, q_output, k_output, v_output, rows, q_columns,
+                             kv_columns, reduction_columns, nullptr, 0, hip_stream);
 }
 
 extern "C" int32_t qm_gate_up_swiglu_rows_split(const uint16_t* input, const uint16_t* gate_weight, const uint16_t* up_weight,

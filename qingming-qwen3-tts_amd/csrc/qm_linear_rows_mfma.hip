@@ -6,21 +6,27 @@
 // instead of the reference's 32 lane-strided chains: bf16 inputs, fp32 accumulation, the same roundings after the sum,
 // results within the operators' tolerance of the exact-chain kernel (qm_linear_rows.hip), not bit-identical to it.
 //
-// A block of four waves owns 128 output columns x 128 token rows (waves 2 x 2, each 64 x 64 as 2 x 2 MFMA tiles) or, for
-// calls whose grid would leave CUs empty, x 64 token rows (waves 4 x 1, each 32 columns x 64 rows).  Both operands are
-// K-contiguous rows (x [m][k], w [n][k]), so one tile layout serves both: 64 k per step, a row of a tile is eight 16-byte
-// pieces in LDS, piece q of row r stored in slot q ^ ((r / 2) % 8) so that the sixteen rows a fragment read touches in a
-// cycle spread over all 64 banks.  An MFMA takes the weight rows as its A operand and the token rows as B (D = W X^T): a lane then holds, for one
-// token row, runs of four consecutive output columns — 8-byte stores.
-// The tiles go from memory straight into a ring of LDS stages (global_load_lds, no registers, the swizzle chosen by which
-// piece a lane fetches), up to four steps ahead (three for the gate/up pair, whose stage is 48 KiB).  A step's one barrier
-// stands between the MFMAs of its last two k blocks, where a wave has read all it needs of the step's stage and waits
-// (vmcnt counts the later stages' pieces still in flight) for its own pieces of the next; the requests for the stage
-// just freed go out a piece at a time between the MFMAs that follow (issued in a bunch, the four waves' requests keep
-// the CU's address path and the waves busy for 700 cycles of a 1024-cycle step), and the next step's first fragments
-// are read behind the barrier while the last k block's MFMAs run.  The fragment reads are inline assembly: the compiler makes every LDS read of its own wait
-// for all global_load_lds in flight, which would expose the memory latency in every step.
-// Bound: bf16 MFMA (2.5 PFLOP/s); algorithmic flops 2 m n k (x 2 for the gate/up pair).
+// A block of four waves owns a tile of BM token rows x BN output columns: 128 x 128 (waves 2 x 2, each 64 x 64 as 2 x 2
+// MFMA tiles); 64 x 128 for calls whose grid of 128-row tiles would leave CUs empty (waves 4 x 1, each 32 columns x 64
+// rows); 128 x 192 for a gate/up pair whose 128-column tiles come to between one and two rounds of the CUs and whose
+// 192-column tiles fit in one (1024 tokens x 6144 channels: 256 blocks).  Several linears of one input (q, k, v) share a
+// grid: a column tile's number says which of them it belongs to.  Both operands are K-contiguous rows (x [m][k],
+// w [n][k]), so one tile layout serves both: KSTEP (64, or 128 for 64-row tiles with a long reduction) k per step, a row
+// of a tile is KSTEP / 8 16-byte pieces in LDS, piece q of row r stored in slot q ^ key(r), the key chosen so that the
+// sixteen rows a fragment read touches in a cycle spread over all 64 banks.  An MFMA takes the weight rows as its A
+// operand and the token rows as B (D = W X^T): a lane then holds, for one token row, runs of four consecutive output
+// columns — 8-byte stores.
+// The tiles go from memory straight into a ring of LDS stages (buffer_load ... lds, no registers, the swizzle chosen by
+// which piece a lane fetches): four stages where they fit in 128 KiB, else three, two for the 192-column tile (64 KiB a
+// stage).  A step's one barrier stands between the MFMAs of its last two k blocks, where a wave has read all it needs of
+// the step's stage and waits (vmcnt counts the later stages' pieces still in flight) for its own pieces of the next.
+// Nothing but MFMAs is issued in a bunch: a k block's LDS reads and the requests for the stage just freed stand one or
+// two to a slot between its MFMAs (GmSchedule), because the wave issues in order and an MFMA hides 32 cycles of other
+// issue and no more — bunched, the four waves' requests of a step keep the CU's one address path (64 bytes a cycle) and
+// with it the waves busy for 700 cycles of a 1024-cycle step.  The fragment reads are inline assembly: the compiler makes
+// every LDS read of its own wait for all requests in flight, which would expose the memory latency in every step.
+// Bound: bf16 MFMA (2.5 PFLOP/s at 2.4 GHz; under these kernels the clock settles at 1.8 to 1.9 GHz); algorithmic flops
+// 2 m n k (x 2 for the gate/up pair).
 
 #include "qm_device.h"
 #include "qm_host.h"
@@ -145,7 +151,7 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
     constexpr int kPerWave = (kPiecesX + kWeights * kPiecesW) / 4;
     static_assert(kPiecesX % 4 == 0 && kPiecesW % 4 == 0, "a wave's piece i is of the same operand in every wave");
     static_assert(kPerWave * (kStages - 2) <= 63 && kStages >= 2, "the waits count the later stages' pieces");
-    static_assert(kKb == 4 || kKb == 2, "the two step schedules");
+    static_assert(kKb == 4 || kKb == 8, "the step schedule lists the k blocks");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -153,8 +159,24 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
     const int wave_n = BM == 128 ? (wave & 1) : wave;
     const int wave_m = BM == 128 ? (wave >> 1) : 0;
     const int K = prm.reduction;
-    const int n0 = static_cast<int>(blockIdx.x) * BN;
     const int m0 = static_cast<int>(blockIdx.y) * BM;
+    // (several linears of one input in one grid: which of them this block's column tile belongs to)
+    int tile = static_cast<int>(blockIdx.x);
+    const uint16_t* weight0 = prm.weight[0];
+    const uint16_t* bias = prm.bias;
+    uint16_t* output = prm.output;
+    int columns = prm.columns;
+    if (!DUAL && prm.groups > 1) {
+        const int g = (tile >= prm.group_first_tile[0]) + (prm.groups > 2 && tile >= prm.group_first_tile[1]);
+        if (g > 0) {
+            tile -= prm.group_first_tile[g - 1];
+            weight0 = prm.group_weight[g - 1];
+            bias = prm.group_bias[g - 1];
+            output = prm.group_output[g - 1];
+            columns = prm.group_columns[g - 1];
+        }
+    }
+    const int n0 = tile * BN;
 
     // ---- this wave's pieces of a stage: instruction q = wave + 4 i covers LDS bytes [1024 q, 1024 q + 1024) of the
     // stage (x tile, then w, then up); its lane l fills slot l % kSlots of tile row kRowsPerPiece (q within the tile) +
@@ -167,9 +189,9 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
     const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(prm.input + static_cast<int64_t>(m0) * K), 0, static_cast<int>(x_rows * row_bytes), 0x00020000);
     const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t*>(prm.weight[0] + static_cast<int64_t>(n0) * K), 0, static_cast<int>(BN * row_bytes), 0x00020000);
+        const_cast<uint16_t*>(weight0 + static_cast<int64_t>(n0) * K), 0, static_cast<int>(BN * row_bytes), 0x00020000);
     const __amdgpu_buffer_rsrc_t u_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t*>(prm.weight[DUAL ? 1 : 0] + static_cast<int64_t>(n0) * K), 0, static_cast<int>(BN * row_bytes), 0x00020000);
+        const_cast<uint16_t*>((DUAL ? prm.weight[1] : weight0) + static_cast<int64_t>(n0) * K), 0, static_cast<int>(BN * row_bytes), 0x00020000);
     const int lane_row = kRowsPerPiece * wave + lane / kSlots;
     const uint32_t lane_off = static_cast<uint32_t>(lane_row) * row_bytes
                             + 16u * static_cast<uint32_t>((lane % kSlots) ^ slot_key<kRowBytes>(lane_row));
@@ -328,20 +350,22 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
         }
     };
     static_assert(kTm == 2 && kTn <= 3, "multiply lists the units");
-    // (a step's requests over its first three k blocks; with two stages they must have landed at the step's own barrier
-    // and go out as early as one to a slot allows)
-    constexpr int kThird1 = kStages == 2 ? (kPerWave > Schedule::kMfmas ? Schedule::kMfmas : kPerWave) : kPerWave / 3;
-    constexpr int kThird2 = kStages == 2 ? kPerWave - kThird1 : (kPerWave - kThird1) / 2, kThird3 = kPerWave - kThird1 - kThird2;
     using yes = std::true_type;
     using no = std::false_type;
 
-    // A step's schedule.  f0 holds k blocks 0 and 2 of a stage in turn, f1 k blocks 1 and 3.  While the MFMAs of a k block
-    // run, its fragments are read again as they fall free, for the k block two further on: f0 during k block 0 (for 2), f1
-    // during 1 (for 3) and during 3 (for 1 of the next step).  The step's one barrier stands behind the MFMAs of k block 2:
-    // there this wave's reads of the stage have all landed and its own pieces of the next step's stage have (the wait lets
-    // the pieces of the steps after that be in flight); behind it the next stage is complete for everybody and this one
-    // free.  f0's fragments for k block 0 of the next step are read in the first slots of k block 3; the pieces of step
-    // s + kStages - 1 are requested into the stage freed at the barrier before, spread over k blocks 0 to 2.
+    // A step's schedule.  f0 holds the even k blocks of a stage in turn, f1 the odd ones.  While the MFMAs of a k block
+    // run, its fragments are read again as they fall free, for the k block two further on; the last k block's (f1) are
+    // read for k block 1 of the next step.  The step's one barrier stands behind the MFMAs of the last k block but one:
+    // there this wave's reads of the stage have all landed and its own pieces of the next step's stage have (the wait
+    // lets the pieces of the steps after that be in flight); behind it the next stage is complete for everybody and
+    // this one free.  f0's fragments for k block 0 of the next step are read in the first slots of the last k block; the
+    // pieces of step s + kStages - 1 are requested into the stage freed at the barrier before, spread over the k blocks in
+    // front of the barrier (with two stages they must have landed at the step's own barrier and go out as early as one
+    // to a slot allows).
+    auto piece_begin = [](int j) constexpr {
+        if (kStages == 2) return j == 0 ? 0 : (j == 1 ? (kPerWave > Schedule::kMfmas ? Schedule::kMfmas : kPerWave) : kPerWave);
+        return j * kPerWave / (kKb - 1);
+    };
 #pragma unroll
     for (int ahead = 0; ahead < kStages - 1; ++ahead)
 #pragma unroll
@@ -355,17 +379,30 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
         const uint32_t stage_at = lds_base + static_cast<uint32_t>((step % kStages) * kStageBytes);
         const uint32_t next_at = lds_base + static_cast<uint32_t>(((step + 1) % kStages) * kStageBytes);
         const int req = step + kStages - 1;
-        // (f0's last read was issued in slot kLastEarlySlot of the k block before, f1's own reads of that slot and later behind it)
-        arrived(f0, integral_constant<int, Schedule::own_from(Schedule::kLastEarlySlot)>{});
-        if constexpr (kKb == 4) {
-            multiply(f0, f1, yes{}, stage_at, 2, no{}, 0u, req, integral_constant<int, 0>{}, integral_constant<int, kThird1>{});
-            arrived(f1, integral_constant<int, kReads>{});
-            multiply(f1, f0, yes{}, stage_at, 3, no{}, 0u, req, integral_constant<int, kThird1>{}, integral_constant<int, kThird2>{});
-            arrived(f0, integral_constant<int, kReads>{});
-            multiply(f0, f1, no{}, 0u, 0, no{}, 0u, req, integral_constant<int, kThird1 + kThird2>{}, integral_constant<int, kThird3>{});
-        } else {
-            // (a step of two k blocks: f0 holds the first, f1 the second; all of the step's requests go out during the first)
-            multiply(f0, f1, no{}, 0u, 0, no{}, 0u, req, integral_constant<int, 0>{}, integral_constant<int, kPerWave>{});
+        // k block j in front of the barrier: its own fragments go on to k block j + 2 (the last of them reads nothing)
+        auto k_block = [&](auto j_) __attribute__((always_inline)) {
+            constexpr int j = decltype(j_)::value;
+            constexpr int p0 = piece_begin(j), count = piece_begin(j + 1) - p0;
+            // (f0's last read for k block 0 was issued in slot kLastEarlySlot of the k block before, f1's own reads of
+            // that slot and later behind it)
+            constexpr int later = j == 0 ? Schedule::own_from(Schedule::kLastEarlySlot) : kReads;
+            using own = std::integral_constant<bool, (j + 2 < kKb)>;
+            if constexpr (j % 2 == 0) {
+                arrived(f0, integral_constant<int, later>{});
+                multiply(f0, f1, own{}, stage_at, j + 2, no{}, 0u, req, integral_constant<int, p0>{}, integral_constant<int, count>{});
+            } else {
+                arrived(f1, integral_constant<int, later>{});
+                multiply(f1, f0, own{}, stage_at, j + 2, no{}, 0u, req, integral_constant<int, p0>{}, integral_constant<int, count>{});
+            }
+        };
+        k_block(integral_constant<int, 0>{});
+        k_block(integral_constant<int, 1>{});
+        k_block(integral_constant<int, 2>{});
+        if constexpr (kKb == 8) {
+            k_block(integral_constant<int, 3>{});
+            k_block(integral_constant<int, 4>{});
+            k_block(integral_constant<int, 5>{});
+            k_block(integral_constant<int, 6>{});
         }
         arrived(f1, integral_constant<int, 0>{});
         gm_wait_vm<kPerWave * (kStages - 2)>();                   // this wave's pieces of the next step's stage have landed
@@ -410,9 +447,9 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
                 if (!inside) break;
                 const int n = n0 + 32 * (kTn * wave_n + a) + 8 * g + 4 * (lane >> 5);
                 uint2 res = make_uint2(0, 0);
-                if (!DUAL && prm.residual) res = *reinterpret_cast<const uint2*>(prm.residual + static_cast<int64_t>(m) * prm.columns + n);
-                uint2 bias = make_uint2(0, 0);
-                if (!DUAL && prm.bias) bias = *reinterpret_cast<const uint2*>(prm.bias + n);
+                if (!DUAL && prm.residual) res = *reinterpret_cast<const uint2*>(prm.residual + static_cast<int64_t>(m) * columns + n);
+                uint2 bias_pair = make_uint2(0, 0);
+                if (!DUAL && bias) bias_pair = *reinterpret_cast<const uint2*>(bias + n);
                 uint32_t packed[2];
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
@@ -420,11 +457,11 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
                     if (DUAL) {
                         packed[e] = swiglu_pair(s0, s1, acc_up[a][b][4 * g + 2 * e], acc_up[a][b][4 * g + 2 * e + 1]);
                     } else {
-                        packed[e] = finish_pair(s0, s1, prm.bias != nullptr, e == 0 ? bias.x : bias.y, prm.residual != nullptr,
+                        packed[e] = finish_pair(s0, s1, bias != nullptr, e == 0 ? bias_pair.x : bias_pair.y, prm.residual != nullptr,
                                                 e == 0 ? res.x : res.y);
                     }
                 }
-                *reinterpret_cast<uint2*>(prm.output + static_cast<int64_t>(m) * prm.columns + n) = make_uint2(packed[0], packed[1]);
+                *reinterpret_cast<uint2*>(output + static_cast<int64_t>(m) * columns + n) = make_uint2(packed[0], packed[1]);
             }
         }
     }
@@ -467,7 +504,9 @@ template <bool DUAL, int BM, int BN, int KSTEP>
 int32_t launch_rows_mfma_as(const LinearRowsParams& prm, hipStream_t stream) {
     using Shape = GmShape<DUAL, BM, BN, KSTEP>;
     constexpr int smem = Shape::kStages * Shape::kStageBytes;
-    const dim3 grid(static_cast<unsigned>(prm.columns / BN), static_cast<unsigned>((prm.rows + BM - 1) / BM),
+    int column_tiles = prm.columns / BN;
+    for (int g = 1; g < prm.groups; ++g) column_tiles += prm.group_columns[g - 1] / BN;
+    const dim3 grid(static_cast<unsigned>(column_tiles), static_cast<unsigned>((prm.rows + BM - 1) / BM),
                     static_cast<unsigned>(prm.reduction_parts));
     if (grid.y > 65535u) return QM_ERR_ARGUMENT;
     static std::atomic<bool> lds_raised[kMaxDevices];
@@ -507,7 +546,9 @@ int32_t launch_rows_mfma(const LinearRowsParams& prm, bool dual, hipStream_t str
     if (prm.rows == 0 || prm.columns == 0) return QM_OK;
     // blocks of 64 token rows where blocks of 128 would leave CUs without one (one block per CU either way)
     const int64_t row_tiles = (prm.rows + 127) / 128;
-    const int64_t blocks_128 = static_cast<int64_t>(prm.columns / kGmTile) * row_tiles;
+    int64_t columns = prm.columns;
+    for (int g = 1; g < prm.groups; ++g) columns += prm.group_columns[g - 1];
+    const int64_t blocks_128 = columns / kGmTile * row_tiles;
     const bool small = blocks_128 < 200;
     if (dual) {
         // a gate/up pair whose grid of 128-column tiles is more than the CUs take at once and less than twice that: tiles
@@ -517,6 +558,9 @@ int32_t launch_rows_mfma(const LinearRowsParams& prm, bool dual, hipStream_t str
             return launch_rows_mfma_as<true, 128, 192, 64>(prm, stream);
         return small ? launch_rows_mfma_as<true, 64, 128, 64>(prm, stream) : launch_rows_mfma_as<true, 128, 128, 64>(prm, stream);
     }
+    // (64 token rows and a long uncut reduction: steps of 128 k, half as many barriers for the same MFMAs; a short one
+    // loses more to the larger first stages than it gains)
+    if (small && prm.reduction_parts == 1 && prm.reduction >= 4096) return launch_rows_mfma_as<false, 64, 128, 128>(prm, stream);
     return small ? launch_rows_mfma_as<false, 64, 128, 64>(prm, stream) : launch_rows_mfma_as<false, 128, 128, 64>(prm, stream);
 }
 

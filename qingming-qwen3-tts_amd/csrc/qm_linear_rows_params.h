@@ -19,6 +19,15 @@ struct LinearRowsParams {
     // pieces in order and rounds.  1: every block takes the whole reduction and rounds its sums itself.
     int reduction_parts;
     float* partials;
+    // (matrix cores, no gate/up pair) up to three linears of the same input in one grid: the column tiles of linear g
+    // start at tile group_first_tile[g] (group 0 at 0), and a block of group g > 0 takes weight / bias / output / columns
+    // from group_*[g - 1] instead of the fields above.  groups = 1: one linear.
+    int groups;
+    int group_first_tile[2];
+    const uint16_t* group_weight[2];
+    const uint16_t* group_bias[2];
+    uint16_t* group_output[2];
+    int group_columns[2];
 };
 
 // The row linears on the matrix cores (qm_linear_rows_mfma.hip).  `dual`: weight[0] / weight[1] are the gate and up

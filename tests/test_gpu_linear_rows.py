@@ -182,3 +182,46 @@ def test_gate_up_swiglu_rows_with_the_reduction_shared_between_blocks(oracle, qm
         assert np.count_nonzero(d) <= rows * inter // 100, np.count_nonzero(d)
     else:
         assert d.max() <= 1 and np.count_nonzero(d) <= max(1, rows * inter // 1000)
+
+
+@pytest.mark.parametrize("rows,q_cols,kv_cols,red", [(1024, 2048, 1024, 2048), (300, 512, 256, 384), (128, 2048, 1024, 2048), (7, 256, 128, 256)])
+def test_qkv_rows_is_three_linear_rows(qm, dev, oracle, rows, q_cols, kv_cols, red):
+    """qm_qkv_rows: bit for bit what three qm_linear_rows calls give (one grid on the matrix cores where the shapes are
+    served uncut; three calls below sixteen rows or with a workspace that cuts the reduction)."""
+    import torch
+    x = to_dev(oracle.normal_bf16((rows, red), 77), dev)
+    ws = [to_dev(oracle.normal_bf16((c, red), 78 + i, std=0.03), dev) for i, c in enumerate((q_cols, kv_cols, kv_cols))]
+    bs = [to_dev(oracle.normal_bf16((c,), 88 + i, std=0.1), dev) for i, c in enumerate((q_cols, kv_cols, kv_cols))]
+    for biases in (bs, [bs[0], None, bs[2]]):
+        want = [torch.full((rows, c), 0x7fc0, dtype=torch.int16, device=dev) for c in (q_cols, kv_cols, kv_cols)]
+        got = [torch.full((rows, c), 0x7fc0, dtype=torch.int16, device=dev) for c in (q_cols, kv_cols, kv_cols)]
+        for w, b, o, c in zip(ws, biases, want, (q_cols, kv_cols, kv_cols)):
+            qm.linear_rows(x, w, b, None, o, rows, c, red)
+        qm.qkv_rows(x, ws, biases, got, rows, q_cols, kv_cols, red)
+        torch.cuda.synchronize()
+        for g, w in zip(got, want):
+            assert torch.equal(g, w)
+    # with the workspace of the short-prompt entries: the three calls with that workspace
+    nbytes = max(qm.linear_rows_split_workspace_bytes(rows, c, red, False) for c in (q_cols, kv_cols))
+    if nbytes:
+        wsp = torch.empty(nbytes // 4, dtype=torch.float32, device=dev)
+        want = [torch.full((rows, c), 0x7fc0, dtype=torch.int16, device=dev) for c in (q_cols, kv_cols, kv_cols)]
+        got = [torch.full((rows, c), 0x7fc0, dtype=torch.int16, device=dev) for c in (q_cols, kv_cols, kv_cols)]
+        for w, b, o, c in zip(ws, bs, want, (q_cols, kv_cols, kv_cols)):
+            qm.linear_rows_split(x, w, b, None, o, rows, c, red, wsp, nbytes)
+        qm.qkv_rows(x, ws, bs, got, rows, q_cols, kv_cols, red, wsp, nbytes)
+        torch.cuda.synchronize()
+        for g, w in zip(got, want):
+            assert torch.equal(g, w)
+
+
+def test_qkv_rows_argument_errors(qm, dev):
+    import torch
+    x = torch.zeros((16, 128), dtype=torch.int16, device=dev)
+    w = torch.zeros((128, 128), dtype=torch.int16, device=dev)
+    o = torch.zeros((16, 128), dtype=torch.int16, device=dev)
+    f = qm.lib().qm_qkv_rows
+    assert f(None, w.data_ptr(), w.data_ptr(), w.data_ptr(), None, None, None, o.data_ptr(), o.data_ptr(), o.data_ptr(), 16, 128, 128, 128, None) == -1
+    assert f(x.data_ptr(), w.data_ptr(), w.data_ptr(), w.data_ptr(), None, None, None, o.data_ptr(), o.data_ptr(), None, 16, 128, 128, 128, None) == -1
+    assert f(x.data_ptr(), w.data_ptr(), w.data_ptr(), w.data_ptr(), None, None, None, o.data_ptr(), o.data_ptr(), o.data_ptr(), 16, 128, 128, 124, None) == -2
+    assert f(x.data_ptr(), w.data_ptr(), w.data_ptr(), w.data_ptr(), None, None, None, o.data_ptr(), o.data_ptr(), o.data_ptr(), -1, 128, 128, 128, None) == -5
