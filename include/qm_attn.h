@@ -827,8 +827,8 @@ int32_t qm_gate_up_swiglu_rows(
  * output its own wave).  On the matrix cores a block owns 128 output columns of 64 or 128 token rows and walks the whole
  * reduction: 128 rows of a 2048-column linear are 32 blocks on 256 compute units, and the call lasts as long as one
  * block's chain.  With a workspace of qm_linear_rows_split_workspace_bytes (0 where the shape is not cut: enough blocks
- * already, or the exact chain) the reduction is cut into 2, 4 or 8 pieces, a block each, whose fp32 sums a second launch
- * adds in order before the same roundings.  Results differ from the uncut call in the association of the sum only
+ * already, a reduction below 4096, or the exact chain) the reduction is cut into 2, 4 or 8 pieces, a block each, whose
+ * fp32 sums a second launch adds in order before the same roundings.  Results differ from the uncut call in the association of the sum only
  * (within the matrix-core path's tolerance of the exact chain) and are the same on every call.  workspace: 256-byte
  * aligned, nothing to initialise; NULL: exactly qm_linear_rows / qm_gate_up_swiglu_rows; too small: QM_ERR_WORKSPACE.
  */
@@ -844,9 +844,10 @@ int32_t qm_gate_up_swiglu_rows_split(
 /*
  * The q, k and v projections of the prompt pass (the first three linear_generic calls of a layer, R17:16646-16672) as one
  * call: output for output what three qm_linear_rows calls on the same input give, bit for bit (on the matrix cores an
- * output's sum does not depend on the tile it is computed in).  Where all three run uncut on the matrix cores they share
- * one grid (1024 tokens: 256 blocks, one per compute unit, instead of 256 + 128 + 128 in three launches); otherwise the
- * call is the three calls.  _split: the workspace of qm_linear_rows_split (the larger of the two shapes' sizes).
+ * output's sum does not depend on the tile it is computed in).  Where all three run on the matrix cores they share
+ * one grid (1024 tokens: 256 blocks, one per compute unit, instead of 256 + 128 + 128 in three launches) and no
+ * reduction is cut; otherwise the call is the three calls.  _split: the workspace of qm_linear_rows_split (the larger of
+ * the two shapes' sizes), used by the three calls only.
  */
 int32_t qm_qkv_rows(
     const uint16_t* input, const uint16_t* q_weight, const uint16_t* k_weight, const uint16_t* v_weight,

@@ -523,16 +523,19 @@ int32_t launch_rows_mfma_as(const LinearRowsParams& prm, hipStream_t stream) {
 }
 
 // Few token rows leave most CUs without a block (128 rows of a 2048-column linear: 32 blocks), and a block's time is its
-// chain of 64-k steps.  With a workspace the reduction is cut so that the grid comes to about one block per CU: pieces of
-// four steps at least, as many as divide the steps evenly, at most eight.
+// chain of 64-k steps.  With a workspace a long reduction (64 steps or more: the down projection's 6144) is cut so that
+// the grid comes to about one block per CU: as many pieces as divide the steps evenly, at most eight.  A reduction of
+// 2048 stays whole: the uncut call takes 10 to 11 us at any number of rows up to 512, and the second launch that adds
+// the pieces costs what the shorter chains save (measured: 8 us cut at 16 rows, 12 at 128, 14 at 512).
 int rows_mfma_reduction_parts(int rows, int columns, int reduction, bool dual) {
     (void)dual;
     if (rows <= 0 || columns < kGmTile || reduction < kGmStep) return 1;
     const int64_t blocks = static_cast<int64_t>(columns / kGmTile) * ((rows + 63) / 64);
     const int steps = reduction / kGmStep;
+    if (steps < 64) return 1;
     int parts = 1;
     for (int p = 2; p <= 8; p *= 2)
-        if (blocks * p <= 256 && steps % p == 0 && steps / p >= 4) parts = p;
+        if (blocks * p <= 256 && steps % p == 0) parts = p;
     return parts;
 }
 

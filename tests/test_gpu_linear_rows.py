@@ -119,11 +119,11 @@ def test_linear_rows_argument_errors(qm, dev):
 
 
 @pytest.mark.parametrize("rows,cols,red,bias,residual", [
-    (128, 2048, 2048, True, True),      # o_proj of a 128-token prompt: 32 blocks, the reduction in eight pieces
-    (100, 1024, 2048, False, False),    # k_proj: 16 blocks
-    (37, 2048, 6144, False, True),      # down_proj + residual: 96 steps
-    (64, 4096, 2048, True, False),      # 32 blocks: eight pieces
-    (200, 2048, 2048, False, True),     # 64 blocks: four pieces
+    (128, 2048, 4096, True, True),      # 32 blocks, 64 steps: eight pieces
+    (100, 1024, 4096, False, False),    # 16 blocks
+    (37, 2048, 6144, False, True),      # down_proj + residual of a short prompt: 96 steps
+    (64, 4096, 4096, True, False),      # 32 blocks: eight pieces
+    (200, 1024, 4096, False, True),     # 32 blocks: eight pieces
 ])
 def test_linear_rows_with_the_reduction_shared_between_blocks(oracle, qm, dev, rows, cols, red, bias, residual, rows_kernel):
     """qm_linear_rows_split: few token rows leave most CUs without a block; with a workspace the reduction is cut into pieces
@@ -153,10 +153,11 @@ def test_linear_rows_with_the_reduction_shared_between_blocks(oracle, qm, dev, r
     if rows_kernel == MATRIX:
         assert qm.lib().qm_linear_rows_split(xd.data_ptr(), wd.data_ptr(), None, None, out.data_ptr(), rows, cols, red, ws.data_ptr(),
                                              nbytes - 4, None) == -4
-    assert qm.linear_rows_split_workspace_bytes(1024, 2048, 2048) == 0      # enough blocks already
+    assert qm.linear_rows_split_workspace_bytes(1024, 2048, 6144) == 0      # enough blocks already
+    assert qm.linear_rows_split_workspace_bytes(128, 2048, 2048) == 0       # a reduction of 2048 stays whole
 
 
-@pytest.mark.parametrize("rows,hidden,inter", [(128, 2048, 6144), (48, 2048, 3072)])
+@pytest.mark.parametrize("rows,hidden,inter", [(128, 4096, 3072), (48, 4096, 1536)])
 def test_gate_up_swiglu_rows_with_the_reduction_shared_between_blocks(oracle, qm, dev, rows, hidden, inter, rows_kernel):
     import torch
     seed = 5500 + rows + hidden
@@ -187,7 +188,7 @@ def test_gate_up_swiglu_rows_with_the_reduction_shared_between_blocks(oracle, qm
 @pytest.mark.parametrize("rows,q_cols,kv_cols,red", [(1024, 2048, 1024, 2048), (300, 512, 256, 384), (128, 2048, 1024, 2048), (7, 256, 128, 256)])
 def test_qkv_rows_is_three_linear_rows(qm, dev, oracle, rows, q_cols, kv_cols, red):
     """qm_qkv_rows: bit for bit what three qm_linear_rows calls give (one grid on the matrix cores where the shapes are
-    served uncut; three calls below sixteen rows or with a workspace that cuts the reduction)."""
+    served; three calls below sixteen rows)."""
     import torch
     x = to_dev(oracle.normal_bf16((rows, red), 77), dev)
     ws = [to_dev(oracle.normal_bf16((c, red), 78 + i, std=0.03), dev) for i, c in enumerate((q_cols, kv_cols, kv_cols))]
@@ -201,18 +202,16 @@ def test_qkv_rows_is_three_linear_rows(qm, dev, oracle, rows, q_cols, kv_cols, r
         torch.cuda.synchronize()
         for g, w in zip(got, want):
             assert torch.equal(g, w)
-    # with the workspace of the short-prompt entries: the three calls with that workspace
-    nbytes = max(qm.linear_rows_split_workspace_bytes(rows, c, red, False) for c in (q_cols, kv_cols))
-    if nbytes:
-        wsp = torch.empty(nbytes // 4, dtype=torch.float32, device=dev)
-        want = [torch.full((rows, c), 0x7fc0, dtype=torch.int16, device=dev) for c in (q_cols, kv_cols, kv_cols)]
-        got = [torch.full((rows, c), 0x7fc0, dtype=torch.int16, device=dev) for c in (q_cols, kv_cols, kv_cols)]
-        for w, b, o, c in zip(ws, bs, want, (q_cols, kv_cols, kv_cols)):
-            qm.linear_rows_split(x, w, b, None, o, rows, c, red, wsp, nbytes)
-        qm.qkv_rows(x, ws, bs, got, rows, q_cols, kv_cols, red, wsp, nbytes)
+    # with a workspace (of whatever size: the one grid never cuts a reduction) the same bits
+    wsp = torch.empty(1 << 20, dtype=torch.float32, device=dev)
+    got = [torch.full((rows, c), 0x7fc0, dtype=torch.int16, device=dev) for c in (q_cols, kv_cols, kv_cols)]
+    qm.qkv_rows(x, ws, bs, got, rows, q_cols, kv_cols, red, wsp, 4 << 20)
+    torch.cuda.synchronize()
+    for g, w, b, c in zip(got, ws, bs, (q_cols, kv_cols, kv_cols)):
+        want = torch.full((rows, c), 0x7fc0, dtype=torch.int16, device=dev)
+        qm.linear_rows(x, w, b, None, want, rows, c, red)
         torch.cuda.synchronize()
-        for g, w in zip(got, want):
-            assert torch.equal(g, w)
+        assert torch.equal(g, want)
 
 
 def test_qkv_rows_argument_errors(qm, dev):
