@@ -1,14 +1,15 @@
 #!/usr/bin/env python3
 """Benchmark of the attention / KV-cache hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--headline-only] [--all] [--only NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--headline-only] [--all] [--rows TEXT] [--only NAME [--layers N]]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM.  The headline workload is the ragged multi-stream decode (64 streams, context lengths
 uniform in [256, 4096], 16-token pages behind a shuffled page table): the one decode
 configuration whose working set (~0.57 GB) exceeds the caches, so that "HBM GB/s" means HBM.
 The other four configurations and the four widened rows that make up a generated frame are timed too;
-`--all` adds every variant row, `--only NAME` times one row alone (for a profiler).  The full record of
+`--all` adds every variant row, `--rows TEXT` times exactly the rows whose name contains TEXT, `--only NAME` times one row
+alone (for a profiler).  The full record of
 every row goes to stdout on a line that starts with `per_config ` and to gpurun_out/bench_per_config.json;
 the LAST stdout line is one compact JSON object (metric, value, roofline, cpu_baseline and a
 `summary` of {row: [us per step, fraction of the bounding peak]}), short enough to survive a tail.
