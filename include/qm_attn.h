@@ -78,6 +78,13 @@ int32_t qm_abi_version(void);
 const char* qm_error_string(int32_t code);
 /* Names the architecture the kernels were compiled for ("gfx950"). */
 const char* qm_target_arch(void);
+/*
+ * Self-test of the library's fp32 -> bf16 rounding (no counterpart in the reference): the kernels round with the
+ * hardware's v_cvt_pk_bf16_f32 where the reference's float_to_bf16 (R17:15040-15056) is an integer sequence; this
+ * compares the two on the device for the `count` fp32 bit patterns from `first_bits` on and ADDS the number of
+ * mismatches to *mismatches_dev (device memory, cleared by the caller).  The tests sweep all 2^32 patterns.
+ */
+int32_t qm_selftest_bf16_rounding(uint32_t first_bits, uint32_t count, uint64_t* mismatches_dev, void* hip_stream);
 
 /* Tuning options; they have no counterpart in the reference, whose kernels have one fixed behaviour.  A call
  * reads the options when it is enqueued: the calling thread's own value where qm_set_thread_option has set one (two

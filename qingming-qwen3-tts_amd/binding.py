@@ -83,6 +83,7 @@ _F32 = C.c_float
 
 _SIGNATURES = {
     "qm_abi_version": (C.c_int32, []),
+    "qm_selftest_bf16_rounding": (C.c_int32, [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]),
     "qm_error_string": (C.c_char_p, [_I32]),
     "qm_target_arch": (C.c_char_p, []),
     "qm_set_option": (_I32, [_I32, _I32]),

@@ -23,12 +23,12 @@ __device__ __forceinline__ float bf2f(uint16_t v) {
 }
 
 __device__ __forceinline__ uint16_t f2bf(float value) {
-    uint32_t bits = __float_as_uint(value);
-    if ((bits & 0x7fffffffU) > 0x7f800000U) {
-        return static_cast<uint16_t>((bits >> 16) | 0x0040U);
-    }
-    bits += 0x7fffU + ((bits >> 16) & 1U);
-    return static_cast<uint16_t>(bits >> 16);
+    // v_cvt_pk_bf16_f32 gives, for every one of the 2^32 fp32 bit patterns, the bits of the reference's integer
+    // sequence (add 0x7fff + the lowest kept bit, shift; a NaN quieted with its payload kept): compared exhaustively
+    // on the device.  One instruction instead of six and a branch.
+    uint32_t packed;
+    asm("v_cvt_pk_bf16_f32 %0, %1, %1" : "=v"(packed) : "v"(value));
+    return static_cast<uint16_t>(packed);
 }
 
 // Round an fp32 value to the nearest bf16 and widen it again (hardware RNE convert).

@@ -1,8 +1,40 @@
 // qm_lib.hip — library identification and error strings of the C ABI.
 
+#include "qm_device.h"
 #include "qm_host.h"
 
 #include <atomic>
+
+namespace qm {
+
+// f2bf (one v_cvt_pk_bf16_f32) against the reference's integer sequence (R17:15040-15056: NaNs quieted, else add 0x7fff +
+// the lowest kept bit and shift) for the `count` bit patterns from `first` on; mismatches are counted.
+__global__ void bf16_rounding_check_kernel(uint32_t first, uint32_t count, unsigned long long* mismatches) {
+    unsigned long long bad = 0;
+    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < count;
+         i += static_cast<uint64_t>(gridDim.x) * blockDim.x) {
+        const uint32_t bits = first + static_cast<uint32_t>(i);
+        uint32_t want = bits;
+        if ((bits & 0x7fffffffU) > 0x7f800000U) {
+            want = (bits >> 16) | 0x0040U;
+        } else {
+            want += 0x7fffU + ((bits >> 16) & 1U);
+            want >>= 16;
+        }
+        bad += f2bf(__uint_as_float(bits)) != static_cast<uint16_t>(want);
+    }
+    if (bad) atomicAdd(mismatches, bad);
+}
+
+}  // namespace qm
+
+extern "C" int32_t qm_selftest_bf16_rounding(uint32_t first_bits, uint32_t count, uint64_t* mismatches_dev, void* hip_stream) {
+    if (!mismatches_dev) return QM_ERR_NULL;
+    if (count == 0) return QM_OK;
+    hipLaunchKernelGGL(qm::bf16_rounding_check_kernel, dim3(2048), dim3(256), 0, static_cast<hipStream_t>(hip_stream), first_bits, count,
+                       reinterpret_cast<unsigned long long*>(mismatches_dev));
+    return qm::launch_status();
+}
 
 extern "C" int32_t qm_abi_version(void) { return 2; }
 

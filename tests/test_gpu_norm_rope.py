@@ -175,3 +175,15 @@ def test_scatter_kv_paged_and_flat(oracle, qm, dev):
     keep[skipped] = False
     assert np.array_equal(to_u16(kd2)[keep], pool.k[keep]) and np.array_equal(to_u16(vd2)[keep], pool.v[keep])
     assert (to_u16(kd2)[skipped] == 0x1234).all()
+
+
+def test_hardware_bf16_rounding_equals_the_reference_sequence_for_every_float(qm, dev):
+    """The kernels round fp32 to bf16 with v_cvt_pk_bf16_f32; the reference (and the oracle) with an integer sequence.  All
+    2^32 bit patterns, NaN payloads and denormals included, must give the same bits (compared on the device)."""
+    import torch
+    bad = torch.zeros(1, dtype=torch.int64, device=dev)
+    for quarter in range(4):
+        assert qm.lib().qm_selftest_bf16_rounding(quarter << 30, 1 << 30, bad.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert int(bad.item()) == 0
+    assert qm.lib().qm_selftest_bf16_rounding(0, 16, None, None) == -1
