@@ -322,7 +322,7 @@ extern "C" int32_t qm_qkv_rows_split(const uint16_t* input, const uint16_t* q_we
     if (rc != QM_OK) return rc;
     const uintptr_t align = reinterpret_cast<uintptr_t>(v_weight) | reinterpret_cast<uintptr_t>(v_bias) | reinterpret_cast<uintptr_t>(v_output);
     // (the one grid is never cut: at 128 rows it takes 11 us where three cut calls take 31)
-    if (!fused || !fused_other || (align & 15)) {
+    if (!fused || !fused_other || q_columns == 0 || kv_columns == 0 || (align & 15)) {
         rc = qm_linear_rows_split(input, q_weight, q_bias, nullptr, q_output, rows, q_columns, reduction_columns, workspace, workspace_bytes, hip_stream);
         if (rc == QM_OK)
             rc = qm_linear_rows_split(input, k_weight, k_bias, nullptr, k_output, rows, kv_columns, reduction_columns, workspace, workspace_bytes, hip_stream);

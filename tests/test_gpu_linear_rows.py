@@ -224,3 +224,23 @@ def test_qkv_rows_argument_errors(qm, dev):
     assert f(x.data_ptr(), w.data_ptr(), w.data_ptr(), w.data_ptr(), None, None, None, o.data_ptr(), o.data_ptr(), None, 16, 128, 128, 128, None) == -1
     assert f(x.data_ptr(), w.data_ptr(), w.data_ptr(), w.data_ptr(), None, None, None, o.data_ptr(), o.data_ptr(), o.data_ptr(), 16, 128, 128, 124, None) == -2
     assert f(x.data_ptr(), w.data_ptr(), w.data_ptr(), w.data_ptr(), None, None, None, o.data_ptr(), o.data_ptr(), o.data_ptr(), -1, 128, 128, 128, None) == -5
+
+
+def test_qkv_rows_with_an_empty_member(qm, dev, oracle):
+    """A linear of no columns among the three leaves the other two as they are alone (the shapes that would share one
+    grid: 64 rows, widths in 128s)."""
+    import torch
+    rows, red = 64, 256
+    x = to_dev(oracle.normal_bf16((rows, red), 5), dev)
+    for q_cols, kv_cols in ((0, 128), (256, 0)):
+        widths = (q_cols, kv_cols, kv_cols)
+        ws = [to_dev(oracle.normal_bf16((max(c, 1), red), 6 + i, std=0.03), dev) for i, c in enumerate(widths)]
+        got = [torch.full((rows, max(c, 1)), 0x7fc0, dtype=torch.int16, device=dev) for c in widths]
+        want = [torch.full((rows, max(c, 1)), 0x7fc0, dtype=torch.int16, device=dev) for c in widths]
+        for w, o, c in zip(ws, want, widths):
+            qm.linear_rows(x, w, None, None, o, rows, c, red)
+        qm.qkv_rows(x, ws, [None, None, None], got, rows, q_cols, kv_cols, red)
+        torch.cuda.synchronize()
+        for g, w in zip(got, want):
+            assert torch.equal(g, w)
+
