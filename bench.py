@@ -1205,7 +1205,8 @@ def main():
             # the same step as the reference launches it: append kernel, then attention
             ("cfg2_talker_step_ctx2048_two_operators", lambda: SingleDecode(qm, dev, 2048, True, 12, one_launch=False), False),
             ("cfg4_causal_prefill", lambda: Prefill(qm, dev), True),
-            ("cfg4_causal_prefill_fp32_scores", lambda: Prefill(qm, dev, score_rounding=0), False),
+            # scores kept fp32 between Q.K^T and the softmax (the fp32-accumulate formulation; not the reference's two roundings)
+            ("cfg4_causal_prefill_fp32_scores", lambda: Prefill(qm, dev, score_rounding=0), True),
             # one prompt, as the talker's prefill runs it: 128 blocks for 256 CUs; the key-split entry fills them
             ("cfg4b_causal_prefill_one_prompt_1024", lambda: Prefill(qm, dev, batch=1), False),
             ("cfg4b_causal_prefill_one_prompt_1024_key_split", lambda: Prefill(qm, dev, batch=1, split=True), False),
