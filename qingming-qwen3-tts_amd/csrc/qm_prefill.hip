@@ -1023,8 +1023,8 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
     const int k_row = 4 * wave + (lane >> 4);
     const uint32_t row_bytes = static_cast<uint32_t>(kv_row32) * 2u;
     // Requests go through buffer descriptors that cover exactly the S keys of this (batch, kv head): a lane's offset
-    // is the piece's first key (scalar arithmetic) plus a 32-bit value that never changes (its row inside the piece
-    // and the 16-byte piece of the key it fetches), one vector addition per request, and a key at or beyond S is out
+    // is the piece's first key (the instruction's scalar offset) plus a 32-bit value that never changes (its row inside
+    // the piece and the 16-byte piece of the key it fetches: the vector offset), and a key at or beyond S is out
     // of the descriptor's range: it reads as zero and touches no memory (such keys only occur masked).
     const uint32_t kv_bytes = static_cast<uint32_t>(S - 1) * row_bytes + static_cast<uint32_t>(kKR);
     const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -1034,13 +1034,18 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
     const uint32_t k_lane = static_cast<uint32_t>(k_row) * row_bytes + 16u * ((lane & 15) ^ (k_row & 15));
     const uint32_t v_lane = static_cast<uint32_t>(k_row) * row_bytes + 16u * ((lane & 15) ^ (4 * (k_row & 3)));
     // piece j of a tile: one request of a wave (16 bytes per lane, no registers) fills rows 4 w + 16 j .. + 3
-    auto load_piece = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lane_off, unsigned char* ring, int tile, int slot, int j) {
+    // (`wanted` false: the request stays in the instruction stream, which a branch around it would cut in two, and
+    // asks for the bytes that follow the descriptor's range: zeros into a buffer nobody reads, no memory touched)
+    auto load_piece = [&](const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lane_off, unsigned char* ring, int tile, int slot, int j,
+                          bool wanted = true) {
         unsigned char* dst = ring + slot * kSpKTile + (4 * wave + 16 * j) * kKR;
-        const uint32_t piece = static_cast<uint32_t>(tile * kBN + 16 * j) * row_bytes;
+        const uint32_t piece = wanted ? static_cast<uint32_t>(tile * kBN + 16 * j) * row_bytes : kv_bytes;
+        // (the piece's offset travels as the instruction's scalar offset, which takes part in the range check like the
+        // vector offset: no vector addition)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16,
-                                                 static_cast<int>(lane_off + piece), 0, 0, 0);
+                                                 static_cast<int>(lane_off), static_cast<int>(piece), 0, 0);
     };
-    auto load_k_piece = [&](int tile, int slot, int j) { load_piece(k_rsrc, k_lane, lds_k, tile, slot, j); };
+    auto load_k_piece = [&](int tile, int slot, int j, bool wanted = true) { load_piece(k_rsrc, k_lane, lds_k, tile, slot, j, wanted); };
     auto load_v_piece = [&](int tile, int slot, int j) { load_piece(v_rsrc, v_lane, lds_v, tile, slot, j); };
     auto load_k = [&](int tile, int slot) {
 #pragma unroll
@@ -1177,12 +1182,15 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
     // ---- softmax state (per column group) and the arithmetic of the uniform waves, cut into score pairs ----
     const float coef = ROUND ? kLog2e : prm.scale * kLog2e;
     const float slack = ROUND ? kRescaleSlack : kRescaleSlack / prm.scale;
-    float m_run[NC], l_run[NC], m_scaled[NC];
+    // (m_limit: what a stage's maximum must exceed for the running maximum to be raised, m_run + slack; kept by the
+    // pipeline's stages only, which are the first to change m_run)
+    float m_run[NC], l_run[NC], m_scaled_neg[NC], m_limit[NC];   // (m_scaled_neg: minus the reference maximum times the exponent's factor)
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
         m_run[c] = -INFINITY;
         l_run[c] = 0.0f;
-        m_scaled[c] = 0.0f;
+        m_scaled_neg[c] = 0.0f;
+        m_limit[c] = -INFINITY;
     }
     // roundings and the causal mask of the score pair r, r + 1 in place (the diagonal tiles)
     auto score_pair_masked = [&](f32x16_t& s, int r, float& mx, int lim) {
@@ -1207,7 +1215,7 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
             const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
             const float alpha = fast_exp2((m_run[c] - m_ref) * coef);
             m_run[c] = m_new;
-            m_scaled[c] = m_ref * coef;
+            m_scaled_neg[c] = -(m_ref * coef);
             l_run[c] *= alpha;
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)
@@ -1216,8 +1224,8 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         }
     };
     auto prob_pair = [&](int c, const f32x16_t& s, int r, uint32_t& packed, float& psum) {
-        const float e0 = fast_exp2(fmaf(s[r], coef, -m_scaled[c]));
-        const float e1 = fast_exp2(fmaf(s[r + 1], coef, -m_scaled[c]));
+        const float e0 = fast_exp2(fmaf(s[r], coef, m_scaled_neg[c]));
+        const float e1 = fast_exp2(fmaf(s[r + 1], coef, m_scaled_neg[c]));
         packed = pack_bf16_pair(e0, e1);
         psum = dot2_bf16(packed, 0x3f803f80U, psum);          // the sum of what the MFMA multiplies
     };
@@ -1266,14 +1274,13 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         // through the roundings (monotonic: the result is the maximum of the rounded scores; the host sends a
         // negative scale elsewhere) and the exchange between the two halves of the wave, so that the branch
         // on them after the last group waits for nothing
-        float mx_a[NC], mx_b[NC], mx_step[NC], mx_limit[NC];
+        float mx_a[NC], mx_b[NC], mx_step[NC];
         uint32_t hi[NC][8];
         float psum[NC];
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             mx_a[c] = mx_b[c] = -INFINITY;
             mx_step[c] = 0.0f;
-            mx_limit[c] = m_run[c] + slack;
             psum[c] = 0.0f;
         }
 #pragma unroll
@@ -1294,8 +1301,8 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
                         // (assembly: the compiler's fmaxf first quiets every operand with an instruction of its
                         // own.  `ua0` passes through the first statement so that the chain follows a read of the
                         // MFMA results that the compiler guards; one MFMA wrote all sixteen.)
-                        asm volatile("v_max3_f32 %0, %0, %2, %3" : "+v"(mx_a[c]), "+v"(ua0) : "v"(s_cur[c][0]), "v"(s_cur[c][1]));
-                        asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(mx_b[c]) : "v"(s_cur[c][2]), "v"(s_cur[c][3]));
+                        asm volatile("v_max_f32 %0, %2, %3" : "=v"(mx_a[c]), "+v"(ua0) : "v"(s_cur[c][0]), "v"(s_cur[c][1]));
+                        asm volatile("v_max_f32 %0, %1, %2" : "=v"(mx_b[c]) : "v"(s_cur[c][2]), "v"(s_cur[c][3]));
 #pragma unroll
                         for (int r = 4; r < 16; r += 4) {
                             asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(mx_a[c]) : "v"(s_cur[c][r]), "v"(s_cur[c][r + 1]));
@@ -1329,8 +1336,8 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
                     // (an empty statement that keeps the roundings here instead of sinking to where they are used)
                     asm volatile("" : "+v"(za0), "+v"(za1), "+v"(zb0), "+v"(zb1));
                     if (g == 3) {
-                        mx_step[c] = halves_max(mx_step[c]);
-                        asm volatile("" : "+v"(mx_step[c]));
+                        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx_step[c]), __float_as_uint(mx_step[c]), false, false);
+                        asm volatile("v_max_f32 %0, %1, %2" : "=v"(mx_step[c]) : "v"(__uint_as_float(sw[0])), "v"(__uint_as_float(sw[1])));
                     }
                     s_cur[c][ra] = za0; s_cur[c][ra + 1] = za1; s_cur[c][rb] = zb0; s_cur[c][rb + 1] = zb1;
                 } else {
@@ -1363,8 +1370,10 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
         }
         fence();
 
+        // (a raised maximum: the new reference is needed at once, for the probabilities; the factor that O and the
+        // running sum shrink by is formed where it is used, at the end of the stage, from the exponent kept here)
         bool need[NC];
-        float alpha[NC];
+        float shrink[NC];
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             float mx = mx_step[c];
@@ -1373,15 +1382,15 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
                 const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
                 asm volatile("v_max_f32 %0, %1, %2" : "=v"(mx) : "v"(__uint_as_float(sw[0])), "v"(__uint_as_float(sw[1])));
             }
-            need[c] = __builtin_amdgcn_ballot_w64(mx > mx_limit[c]) != 0;
-            alpha[c] = 1.0f;
+            need[c] = __builtin_amdgcn_ballot_w64(mx > m_limit[c]) != 0;
+            asm volatile("" : "=v"(shrink[c]));        // (read only where need[c]: a register, no instruction)
             if (need[c]) {
                 const float m_new = fmaxf(m_run[c], mx);
                 const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
-                alpha[c] = fast_exp2((m_run[c] - m_ref) * coef);
+                shrink[c] = (m_run[c] - m_ref) * coef;
                 m_run[c] = m_new;
-                m_scaled[c] = m_ref * coef;
-                l_run[c] *= alpha[c];
+                m_limit[c] = m_new + slack;
+                m_scaled_neg[c] = -(m_ref * coef);
             }
         }
 #pragma unroll
@@ -1391,8 +1400,8 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
             for (int c = 0; c < NC; ++c) {
                 if (g > 0) pv_mfma(4 + g, c);
                 fence();
-                const float ta0 = fmaf(s_cur[c][ra], coef, -m_scaled[c]), ta1 = fmaf(s_cur[c][ra + 1], coef, -m_scaled[c]);
-                const float tb0 = fmaf(s_cur[c][rb], coef, -m_scaled[c]), tb1 = fmaf(s_cur[c][rb + 1], coef, -m_scaled[c]);
+                const float ta0 = fmaf(s_cur[c][ra], coef, m_scaled_neg[c]), ta1 = fmaf(s_cur[c][ra + 1], coef, m_scaled_neg[c]);
+                const float tb0 = fmaf(s_cur[c][rb], coef, m_scaled_neg[c]), tb1 = fmaf(s_cur[c][rb + 1], coef, m_scaled_neg[c]);
                 fence();
                 const float ea0 = fast_exp2(ta0), ea1 = fast_exp2(ta1);
                 fence();
@@ -1418,13 +1427,15 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             make_p(hi[c], p_cur[c]);
-            l_run[c] += psum[c];
             if (need[c]) {
+                const float alpha = fast_exp2(shrink[c]);
+                l_run[c] *= alpha;
 #pragma unroll
                 for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) o[c][dt][r] *= alpha[c];
+                    for (int r = 0; r < 16; ++r) o[c][dt][r] *= alpha;
             }
+            l_run[c] += psum[c];
         }
     };
 
@@ -1472,7 +1483,7 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
               },
               [&](int i) {
                   if (i < 4) {
-                      if (more_k) load_k_piece(t + 2, cur, i);
+                      load_k_piece(t + 2, cur, i, more_k);
                   } else {
                       load_v_piece(t + 1, nxt, i - 4);
                   }
