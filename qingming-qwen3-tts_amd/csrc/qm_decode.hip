@@ -122,6 +122,7 @@ __device__ __forceinline__ uint4 load_or_zero(const uint16_t* p, bool valid) {
 // group served by several blocks of G heads per kv head, and the rows of one sequence as streams.
 template <int G, bool STEP, bool STREAMING, bool GENERIC>
 __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodeParams prm, qm_kv_cache cache) {
+    request_arguments(prm, cache);
     __shared__ __attribute__((aligned(16))) uint16_t sh_qrot[STEP ? G : 1][kDim];
     __shared__ float sh_acc[kRowStreams][G][kDim];
     __shared__ float sh_m[kRowStreams][G];
@@ -405,6 +406,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_split_kernel(DecodePara
 // context.  grid (head groups, n_streams), block G*128.
 template <int G, bool GENERIC>
 __global__ void decode_merge_kernel(DecodeParams prm) {
+    request_arguments(prm);
     const int hg = blockIdx.x;
     const int stream = blockIdx.y;
     const int g = threadIdx.x / kDim;

@@ -57,6 +57,7 @@ struct LinearParams {
 // rounded to bf16, then act = bf16(g / (1 + expf(-g))) and out = bf16(act * u).
 template <bool DUAL>
 __global__ __launch_bounds__(kLinThreads) void linear_m1_kernel(LinearParams prm) {
+    request_arguments(prm);
     extern __shared__ __attribute__((aligned(16))) float lin_x[];   // the input vector, fp32
     constexpr int kBatch = DUAL ? kLinBatch / 2 : kLinBatch;        // loads per matrix and register batch
 
@@ -217,6 +218,7 @@ __host__ __device__ inline int staged_x_floats(int reduction) { return (reductio
 
 template <bool DUAL>
 __global__ __launch_bounds__(kStagedThreads) void linear_m1_staged_kernel(LinearParams prm) {
+    request_arguments(prm);
     extern __shared__ __attribute__((aligned(16))) unsigned char st_smem[];
     __shared__ float sh_waves[8];
     __shared__ float sh_total;

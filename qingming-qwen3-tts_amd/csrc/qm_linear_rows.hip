@@ -35,6 +35,7 @@ __host__ __device__ inline int rows_w_stride(int reduction) { return 2 * reducti
 // SPAN: token rows per thread and pass (8 with eight columns per block, 4 with four)
 template <bool DUAL, int SPAN>
 __global__ __launch_bounds__(kRowsThreads) void linear_rows_kernel(LinearRowsParams prm) {
+    request_arguments(prm);
     extern __shared__ __attribute__((aligned(16))) unsigned char lr_smem[];
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

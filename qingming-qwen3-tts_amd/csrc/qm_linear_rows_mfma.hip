@@ -134,6 +134,7 @@ struct GmSchedule {
 
 template <bool DUAL, int BM, int BN, int KSTEP>
 __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRowsParams prm) {
+    request_arguments(prm);
     extern __shared__ __attribute__((aligned(16))) unsigned char gm_smem[];
     constexpr int kStages = GmShape<DUAL, BM, BN, KSTEP>::kStages;
     constexpr int kRowBytes = KSTEP * 2, kSlots = kRowBytes / 16, kKb = KSTEP / 16;
@@ -470,6 +471,7 @@ __global__ __launch_bounds__(kGmThreads) void linear_rows_mfma_kernel(LinearRows
 // The pieces of a cut reduction added in order, then what the epilogue above does: thread = four output columns of a row.
 template <bool DUAL>
 __global__ __launch_bounds__(256) void linear_rows_parts_kernel(LinearRowsParams prm) {
+    request_arguments(prm);
     const int64_t quad = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     const int quads_per_row = prm.columns / 4;
     if (quad >= static_cast<int64_t>(prm.rows) * quads_per_row) return;

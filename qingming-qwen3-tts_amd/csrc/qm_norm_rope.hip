@@ -24,6 +24,8 @@ __global__ __launch_bounds__(64) void qk_norm_rope_append_kernel(
     qm_kv_cache cache, const int32_t* __restrict__ page_table, int max_pages,
     const int32_t* __restrict__ positions, int fixed_position,
     int q_heads, float epsilon, uint32_t* status) {
+    request_arguments(q, k, v, q_norm_w, k_norm_w, cos_rows, sin_rows, rope_by_position, q_rotated, cache, page_table, max_pages,
+                      positions, fixed_position, q_heads, epsilon, status);
     const int lane = threadIdx.x;
     const int slot = blockIdx.x;
     const int stream = blockIdx.y;
@@ -75,6 +77,7 @@ __global__ __launch_bounds__(256) void norm_rope_rows_kernel(
     const uint16_t* __restrict__ in, const uint16_t* __restrict__ norm_w,
     const uint16_t* __restrict__ cos_rows, const uint16_t* __restrict__ sin_rows,
     uint16_t* __restrict__ out, int64_t total_heads, int heads, float epsilon) {
+    request_arguments(in, norm_w, cos_rows, sin_rows, out, total_heads, heads, epsilon);
     const int lane = threadIdx.x & 63;
     const int64_t item = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
     if (item >= total_heads) return;
@@ -91,6 +94,7 @@ __global__ __launch_bounds__(256) void scatter_kv_kernel(
     const uint16_t* __restrict__ key, const uint16_t* __restrict__ value,
     qm_kv_cache cache, const int32_t* __restrict__ page_table, int max_pages,
     int64_t total_chunks, int first_position, uint32_t* status) {
+    request_arguments(key, value, cache, page_table, max_pages, total_chunks, first_position, status);
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (idx >= total_chunks) return;
     const int chunk = static_cast<int>(idx & 15);

@@ -43,6 +43,7 @@ __device__ __forceinline__ void pv_rows(const float (*p)[kPredRows], const float
 // rotated) and V row are written to the caches at key_length - 1 and the query attends key_length keys.
 template <int MODE>
 __global__ __launch_bounds__(kPredThreads) void predictor_loop_kernel(PredictorParams prm) {
+    request_arguments(prm);
     constexpr bool STAGED = MODE == 1;
     constexpr bool APPEND = MODE == 2;
     __shared__ __attribute__((aligned(16))) uint16_t sh_q[2][kPredRows][kDim];   // [g][row][d]

@@ -454,6 +454,7 @@ __device__ __forceinline__ bool attention_phase(FrShared& sh, unsigned char* sme
 }
 
 __global__ __launch_bounds__(kFrThreads, 1) void predictor_frame_kernel(FrParams prm) {
+    request_arguments(prm);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     __shared__ FrShared sh;
     const int tid = threadIdx.x;

@@ -181,6 +181,7 @@ __device__ __forceinline__ VecRegs load_vector(const uint16_t* base, bool valid)
 // grid: ceil(units * 8 / 4) blocks of 256 threads; wave w of block b owns item 4 b + w,
 // item = unit * 8 + kv head.
 __global__ __launch_bounds__(kPredThreads, 4) void predictor_loop_mfma_kernel(PredictorParams prm, int64_t items) {
+    request_arguments(prm, items);
     __shared__ __attribute__((aligned(16))) unsigned char sh_v[4][kVTileBytes];
     __shared__ __attribute__((aligned(16))) unsigned char sh_cos[kVTileBytes];      // [row][128] bf16, padded rows
     __shared__ __attribute__((aligned(16))) unsigned char sh_sin[kVTileBytes];

@@ -751,6 +751,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_chunk_kernel(PrefillPar
 constexpr int kChunkMaxRuns = 16;
 constexpr int kChunkMergeSlices = 8;
 __global__ __launch_bounds__(kPfThreads) void prefill_chunk_merge_kernel(PrefillParams prm, int round_scores, int gqa_group) {
+    request_arguments(prm, round_scores, gqa_group);
     const int slice = blockIdx.x % kChunkMergeSlices;
     const int item = blockIdx.x / kChunkMergeSlices;
     const int pair = item % (prm.batch * prm.kv_heads);
@@ -1741,6 +1742,7 @@ __device__ __forceinline__ void prefill_il_body(const PrefillParams& prm, const 
 template <bool ROUND, int NC>
 __global__ __launch_bounds__(kPfThreads, (NC == 1 ? 2 : 1)) void prefill_il_kernel(PrefillParams prm, qm_kv_cache cache) {
     extern __shared__ __attribute__((aligned(16))) unsigned char il_smem[];
+    request_arguments(prm, cache);
     const int pairs = prm.batch * prm.kv_heads;
     const int bid = blockIdx.x;
     // Heaviest query tile first; when the whole grid is resident at once (at most two blocks per CU,

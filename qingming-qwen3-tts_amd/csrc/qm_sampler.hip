@@ -39,6 +39,7 @@
 namespace qm {
 
 __global__ __launch_bounds__(kSmpThreads) void sampler_kernel(SamplerParams prm) {
+    request_arguments(prm);
     __shared__ SamplerScratch scratch;
     const int tid = threadIdx.x;
     const int vocab = prm.vocab;

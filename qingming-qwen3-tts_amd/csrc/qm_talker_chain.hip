@@ -202,6 +202,7 @@ __device__ __forceinline__ int request_unit(const TkParams& p, int v, int b, uns
 static_assert(kTkWindow <= kTkPieces / kTkWeightWaves, "a unit is known to have landed when the next has been requested");
 
 __global__ __launch_bounds__(kTkThreads, 1) void talker_chain_kernel(TkParams p) {
+    request_arguments(p);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     __shared__ TkShared sh;
     const int tid = threadIdx.x;
