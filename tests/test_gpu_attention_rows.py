@@ -435,3 +435,27 @@ def test_paged_chunk_carries_the_bits_of_the_flat_one_and_shares_its_keys(oracle
     with pytest.raises(qm.QmError) as e:
         qm.prefill_attention_chunk_paged(to_dev(q, dev), cache_d, table_d, 3, out, 1, rows, before, q_heads, kv_heads)
     assert e.value.code == -3              # more keys than three pages hold
+
+
+def test_a_score_on_a_bf16_rounding_boundary_moves_only_its_own_row(oracle, qm, dev):
+    """The reference rounds every raw score to bf16 (R17:15862-15880), and the matrix core adds a score's 128 products in
+    another order than the reference's chain: a score whose exact value lies within a few fp32 ulps of the midpoint of two
+    bf16 values can round to the other neighbour.  Found by a randomized run over 7 000 shapes (this one case): row 19, head 9
+    of a 32-row chunk at position 207 has its largest score, 47.625007, two fp32 ulps above the midpoint 47.625 of 47.5 and
+    47.75; the key carries 16 % of the row, so the row's outputs move by up to 1.6e-2.  What is held: the witness exists (fp64
+    dot products), every other (row, head) is within the rule, and the moved row is within the step's effect."""
+    rows, before, q_heads, kv_heads, seed = 32, 207, 32, 8, 87910
+    got, want = _chunk_any(oracle, qm, dev, rows, before, seed, q_heads, kv_heads, paged=False)
+    q = oracle.bf16_to_f32(oracle.normal_bf16((rows, q_heads, 128), seed)).astype(np.float64)
+    keys = oracle.bf16_to_f32(oracle.normal_bf16((kv_heads, before + rows + 3, 128), seed + 1)).astype(np.float64)
+    row, head = 19, 9
+    scores = (keys[head // (q_heads // kv_heads), :before + row + 1] @ q[row, head]).astype(np.float32)
+    from_midpoint = np.abs((scores.view(np.uint32) & 0xffff).astype(np.int64) - 0x8000)      # in fp32 ulps
+    assert from_midpoint.min() <= 4 and int(np.argmin(from_midpoint)) == int(np.argmax(scores))
+    a = oracle.bf16_to_f32(got).astype(np.float64)
+    b = oracle.bf16_to_f32(want[1]).astype(np.float64)
+    others = np.ones((rows, q_heads), dtype=bool)
+    others[row, head] = False
+    assert _within(oracle, got[others], want[1][others])
+    assert np.abs(a[row, head] - b[row, head]).max() <= 2e-2
+
