@@ -821,7 +821,10 @@ int32_t qm_predictor_add_postnorm_gate_up_swiglu_m1(
  * (add_bf16_kernel R17:8729-8744: bf16(residual + output)).
  * qm_gate_up_swiglu_rows = the two linear_generic calls on gate and up and launch_swiglu
  * (R17:16742-16768, swiglu_kernel :8745-8770): qm_gate_up_swiglu_m1 row by row.
- * reduction % 8 == 0, reduction <= 16384, input and weights 16-byte aligned (QM_ERR_GEOMETRY).
+ * reduction % 8 == 0, reduction <= 16384, input and weights 16-byte aligned (QM_ERR_GEOMETRY).  The exact chain
+ * (calls of fewer than 16 rows, shapes off the 128-wide matrix tiles, QM_OPT_LINEAR_ROWS_KERNEL = 1) keeps eight token
+ * rows and its weight rows in LDS: there reduction <= 6640 for a linear and hidden <= 4976 for a gate/up pair
+ * (QM_ERR_GEOMETRY beyond; the talker's largest are 6144 and 2048).
  */
 int32_t qm_linear_rows(
     const uint16_t* input, const uint16_t* weight, const uint16_t* bias, const uint16_t* residual,
