@@ -280,6 +280,15 @@ int32_t qm_norm_rope_rows(
     const uint16_t* cos_rows, const uint16_t* sin_rows,
     uint16_t* out, int32_t rows, int32_t heads, float epsilon,
     void* hip_stream);
+/*
+ * The same for the prompt pass's query and key tensors in ONE launch (the two rmsnorm + two launch_rope_rows calls of
+ * NativeTalkerEngine::prefill, R17:16673-16712): q_in/q_out [rows][q_heads][128], k_in/k_out [rows][kv_heads][128], one
+ * norm weight each (or NULL), the same cos/sin rows.  Bit for bit two qm_norm_rope_rows calls.
+ */
+int32_t qm_qk_norm_rope_rows(
+    const uint16_t* q_in, const uint16_t* k_in, const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+    const uint16_t* cos_rows, const uint16_t* sin_rows, uint16_t* q_out, uint16_t* k_out,
+    int32_t rows, int32_t q_heads, int32_t kv_heads, float epsilon, void* hip_stream);
 
 /*
  * Replaces scatter_prefill_cache (R17:17646-17682, kernel R17:15630-15687) and, with

@@ -109,6 +109,7 @@ _SIGNATURES = {
     "qm_attention_rows": (_I32, [_PTR, C.POINTER(KvCache), _PTR, _I32, _PTR, _I32, _I32, _I32, _I32, _F32,
                                  _PTR, C.c_size_t, _PTR, _PTR]),
     "qm_norm_rope_rows": (_I32, [_PTR] * 5 + [_I32, _I32, _F32, _PTR]),
+    "qm_qk_norm_rope_rows": (_I32, [_PTR] * 8 + [_I32, _I32, _I32, _F32, _PTR]),
     "qm_scatter_kv": (_I32, [_PTR, _PTR, C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _PTR, _PTR]),
     "qm_prefill_attention_causal": (_I32, [_PTR] * 4 + [C.POINTER(KvCache), _PTR, _I32, _I32, _I32, _I32, _I32,
                                            _F32, C.c_int64, C.c_int64, C.c_int64, _PTR, _PTR]),
@@ -314,6 +315,11 @@ def attention_rows(query, cache, page_table, max_pages, out, query_length, cache
 def norm_rope_rows(x, norm_w, cos, sin, out, rows, heads, eps=1e-6, stream=0):
     _check(lib().qm_norm_rope_rows(_addr(x), _addr(norm_w), _addr(cos), _addr(sin), _addr(out), rows,
                                    heads, eps, stream), "qm_norm_rope_rows")
+
+
+def qk_norm_rope_rows(q, k, q_norm_w, k_norm_w, cos, sin, q_out, k_out, rows, q_heads, kv_heads, eps=1e-6, stream=0):
+    _check(lib().qm_qk_norm_rope_rows(_addr(q), _addr(k), _addr(q_norm_w), _addr(k_norm_w), _addr(cos), _addr(sin), _addr(q_out),
+                                      _addr(k_out), rows, q_heads, kv_heads, eps, stream), "qm_qk_norm_rope_rows")
 
 
 def scatter_kv(key, value, cache, page_table, max_pages, rows, first_position, status=None, stream=0):

@@ -321,7 +321,7 @@ static const uint16_t* decode(qm_talker& e, const uint16_t* input_device, const 
 // reference's launches per layer and what runs here:
 //   rmsnorm                                   -> qm_rmsnorm_rows
 //   3 x linear_generic (q, k, v)              -> qm_qkv_rows (every linear through its _split entry: short prompts)
-//   2 x rmsnorm + 2 x rope_rows               -> 2 x qm_norm_rope_rows
+//   2 x rmsnorm + 2 x rope_rows               -> qm_qk_norm_rope_rows (one launch)
 //   scatter_prefill_cache + attention         -> qm_prefill_attention_causal_split (writes the cache itself; long
 //                                                query tiles of a prompt are shared by two or three blocks)
 //   linear_generic (o_proj) + add             -> qm_linear_rows with the residual folded in
@@ -379,10 +379,9 @@ static const uint16_t* prefill(qm_talker& e, const uint16_t* input_device, const
         op_check(qm_qkv_rows_split(e.p_norm.u16(), w.q_weight.data(), w.k_weight.data(), w.v_weight.data(), w.q_bias.data(),
                                    w.k_bias.data(), w.v_bias.data(), e.p_q.u16(), e.p_k.u16(), e.p_v.u16(), rows, e.q_dim, e.kv_dim,
                                    kHidden, rows_ws, rows_bytes, s), "prefill q/k/v_proj");
-        op_check(qm_norm_rope_rows(e.p_q.u16(), w.q_norm.data(), e.p_cosine.u16(), e.p_sine.u16(), e.p_q_rotated.u16(), rows,
-                                   e.q_heads, kEpsilon, s), "prefill q norm + RoPE");
-        op_check(qm_norm_rope_rows(e.p_k.u16(), w.k_norm.data(), e.p_cosine.u16(), e.p_sine.u16(), e.p_k_rotated.u16(), rows,
-                                   e.kv_heads, kEpsilon, s), "prefill k norm + RoPE");
+        op_check(qm_qk_norm_rope_rows(e.p_q.u16(), e.p_k.u16(), w.q_norm.data(), w.k_norm.data(), e.p_cosine.u16(), e.p_sine.u16(),
+                                      e.p_q_rotated.u16(), e.p_k_rotated.u16(), rows, e.q_heads, e.kv_heads, kEpsilon, s),
+                 "prefill q and k norm + RoPE");
         op_check(qm_prefill_attention_causal_split(e.p_q_rotated.u16(), e.p_k_rotated.u16(), e.p_v.u16(), e.p_context.u16(),
                                                    &cache, nullptr, 1, 1, rows, e.q_heads, e.kv_heads, kScale, 0, 0, 0,
                                                    split_bytes > 0 ? e.p_split.raw() : nullptr, split_bytes,

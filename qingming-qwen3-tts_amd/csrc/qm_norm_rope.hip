@@ -89,6 +89,29 @@ __global__ __launch_bounds__(256) void norm_rope_rows_kernel(
     out[base + lane + 64] = r.hi;
 }
 
+// The prompt pass's query and key heads in one grid: item = row * (q_heads + kv_heads) + head, the first q_heads of a
+// row its query heads; every head as norm_rope_rows_kernel forms it.
+__global__ __launch_bounds__(256) void qk_norm_rope_rows_kernel(
+    const uint16_t* __restrict__ q_in, const uint16_t* __restrict__ k_in, const uint16_t* __restrict__ q_norm_w,
+    const uint16_t* __restrict__ k_norm_w, const uint16_t* __restrict__ cos_rows, const uint16_t* __restrict__ sin_rows,
+    uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_out, int64_t total_heads, int q_heads, int kv_heads, float epsilon) {
+    request_arguments(q_in, k_in, q_norm_w, k_norm_w, cos_rows, sin_rows, q_out, k_out, total_heads, q_heads, kv_heads, epsilon);
+    const int lane = threadIdx.x & 63;
+    const int64_t item = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (item >= total_heads) return;
+    const int per_row = q_heads + kv_heads;
+    const int64_t row = item / per_row;
+    const int head = static_cast<int>(item - row * per_row);
+    const bool is_query = head < q_heads;
+    const uint16_t* in = is_query ? q_in : k_in;
+    uint16_t* out = is_query ? q_out : k_out;
+    const int64_t base = is_query ? (row * q_heads + head) * kDim : (row * kv_heads + (head - q_heads)) * kDim;
+    const HeadPair r = norm_rope_head(in[base + lane], in[base + lane + 64], is_query ? q_norm_w : k_norm_w,
+                                      cos_rows + row * kDim, sin_rows + row * kDim, epsilon, lane);
+    out[base + lane] = r.lo;
+    out[base + lane + 64] = r.hi;
+}
+
 // [rows][kv_heads][128] -> pages; one thread moves 16 bytes of K and 16 bytes of V.
 __global__ __launch_bounds__(256) void scatter_kv_kernel(
     const uint16_t* __restrict__ key, const uint16_t* __restrict__ value,
@@ -178,6 +201,22 @@ extern "C" int32_t qm_norm_rope_rows(
     hipLaunchKernelGGL(qm::norm_rope_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
                        static_cast<hipStream_t>(hip_stream),
                        in, norm_w, cos_rows, sin_rows, out, total, heads, epsilon);
+    return qm::launch_status();
+}
+
+extern "C" int32_t qm_qk_norm_rope_rows(
+    const uint16_t* q_in, const uint16_t* k_in, const uint16_t* q_norm_w, const uint16_t* k_norm_w,
+    const uint16_t* cos_rows, const uint16_t* sin_rows, uint16_t* q_out, uint16_t* k_out,
+    int32_t rows, int32_t q_heads, int32_t kv_heads, float epsilon, void* hip_stream) {
+    if (!q_in || !k_in || !cos_rows || !sin_rows || !q_out || !k_out) return QM_ERR_NULL;
+    if (rows < 0 || q_heads <= 0 || kv_heads <= 0) return QM_ERR_ARGUMENT;
+    if (rows == 0) return QM_OK;
+    const int64_t total = static_cast<int64_t>(rows) * (static_cast<int64_t>(q_heads) + kv_heads);
+    const int64_t blocks = (total + 3) / 4;
+    if (blocks > 0x7fffffffLL) return QM_ERR_ARGUMENT;
+    hipLaunchKernelGGL(qm::qk_norm_rope_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
+                       static_cast<hipStream_t>(hip_stream),
+                       q_in, k_in, q_norm_w, k_norm_w, cos_rows, sin_rows, q_out, k_out, total, q_heads, kv_heads, epsilon);
     return qm::launch_status();
 }
 

@@ -140,6 +140,27 @@ def test_norm_rope_rows_bit_exact(oracle, qm, dev, rows, heads, with_norm):
     assert np.array_equal(to_u16(out), want)
 
 
+@pytest.mark.parametrize("rows,q_heads,kv_heads,with_norm", [(1, 16, 8, True), (33, 16, 8, True), (130, 8, 8, False), (7, 3, 1, True)])
+def test_query_and_key_rows_in_one_launch_are_the_two_calls(oracle, qm, dev, rows, q_heads, kv_heads, with_norm):
+    import torch
+    q = to_dev(oracle.normal_bf16((rows, q_heads, 128), 600 + rows), dev)
+    k = to_dev(oracle.normal_bf16((rows, kv_heads, 128), 601 + rows), dev)
+    gq = to_dev(oracle.normal_bf16((128,), 602, 1.0, 0.1), dev) if with_norm else None
+    gk = to_dev(oracle.normal_bf16((128,), 603, 1.0, 0.1), dev) if with_norm else None
+    cos, sin = (to_dev(a, dev) for a in oracle.rope_table(rows, 5))
+    want_q, want_k, got_q, got_k = (torch.full(t.shape, 0x7fc0, dtype=torch.int16, device=dev) for t in (q, k, q, k))
+    qm.norm_rope_rows(q, gq, cos, sin, want_q, rows, q_heads)
+    qm.norm_rope_rows(k, gk, cos, sin, want_k, rows, kv_heads)
+    qm.qk_norm_rope_rows(q, k, gq, gk, cos, sin, got_q, got_k, rows, q_heads, kv_heads)
+    torch.cuda.synchronize()
+    assert torch.equal(got_q, want_q) and torch.equal(got_k, want_k)
+    f = qm.lib().qm_qk_norm_rope_rows
+    a = [t.data_ptr() for t in (q, k)] + [None, None] + [cos.data_ptr(), sin.data_ptr(), got_q.data_ptr(), got_k.data_ptr()]
+    assert f(*a, -1, q_heads, kv_heads, 1e-6, None) == -5 and f(*a, rows, 0, kv_heads, 1e-6, None) == -5
+    assert f(*(a[:1] + [None] + a[2:]), rows, q_heads, kv_heads, 1e-6, None) == -1
+    assert f(*a, 0, q_heads, kv_heads, 1e-6, None) == 0
+
+
 def test_scatter_kv_paged_and_flat(oracle, qm, dev):
     import torch
     rows, first = 75, 9
