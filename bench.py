@@ -828,12 +828,14 @@ def generate_end_to_end(qm, dev, frames=96, prompt_rows=128, seed=20240229):
             qm.set_option(qm.OPT_PREDICTOR_FRAME_OPERATORS, frame_ops)
             try:
                 best = None
+                quickest_first = None      # (the first run of the first path also loads code objects: each figure is its best of three)
                 for _ in range(3):
                     head.reset(seed)
                     # one frame alone = prefill + first frame; the difference to the full run is the steady state
                     t0 = time.perf_counter()
                     engine.generate(talker, head, predictor, prompt, prompt_rows, 1, tts_pad)
                     first = time.perf_counter() - t0
+                    quickest_first = first if quickest_first is None else min(quickest_first, first)
                     head.reset(seed)
                     t0 = time.perf_counter()
                     codes, digest = engine.generate(talker, head, predictor, prompt, prompt_rows, frames, tts_pad)
@@ -846,7 +848,7 @@ def generate_end_to_end(qm, dev, frames=96, prompt_rows=128, seed=20240229):
                     reference = (codes.copy(), digest)
                 elif not (np.array_equal(codes, reference[0]) and digest == reference[1]):
                     raise RuntimeError("generate: the codec trajectory of '%s' differs from the default paths'" % name)
-                rows[name] = {"ms_per_frame": best[0] * 1e3, "ms_prefill_and_first_frame": best[1] * 1e3, "frames": best[2],
+                rows[name] = {"ms_per_frame": best[0] * 1e3, "ms_prefill_and_first_frame": quickest_first * 1e3, "frames": best[2],
                               "codec_fnv1a64": "%016x" % best[3]}
             finally:
                 qm.set_option(qm.OPT_TALKER_LAYER_OPERATORS, 0)
