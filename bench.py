@@ -10,7 +10,7 @@ configuration whose working set (~0.57 GB) exceeds the caches, so that "HBM GB/s
 The other four configurations and the four widened rows that make up a generated frame are timed too;
 `--all` adds every variant row, `--rows TEXT` times exactly the rows whose name contains TEXT, `--only NAME` times one row
 alone (for a profiler).  The full record of
-every row goes to stdout on a line that starts with `per_config ` and to gpurun_out/bench_per_config.json;
+every row goes to stdout on a line that starts with `per_config ` and to the file PER_CONFIG_FILE names;
 the LAST stdout line is one compact JSON object (metric, value, roofline, cpu_baseline and a
 `summary` of {row: [us per step, fraction of the bounding peak]}), short enough to survive a tail.
 
@@ -1096,6 +1096,7 @@ def _summary(per_config):
 
 
 FINAL_LINE_LIMIT = 4000  # bytes; the last stdout line must survive a tail of a few KB
+PER_CONFIG_FILE = "gpurun_out/bench_per_config.json"   # the full per-row record, relative to the repository root
 
 
 def compact_line(line):
@@ -1313,10 +1314,10 @@ def main():
         full = json.dumps(per_config)
         print("per_config " + full, flush=True)
         try:
-            os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-            with open(os.path.join(ROOT, "gpurun_out", "bench_per_config.json"), "w") as f:
+            os.makedirs(os.path.dirname(os.path.join(ROOT, PER_CONFIG_FILE)), exist_ok=True)
+            with open(os.path.join(ROOT, PER_CONFIG_FILE), "w") as f:
                 f.write(full + "\n")
-            line["per_config_file"] = "gpurun_out/bench_per_config.json"
+            line["per_config_file"] = PER_CONFIG_FILE
         except OSError:
             pass
     print(compact_line(line), flush=True)
